@@ -1,0 +1,439 @@
+/*
+ * TEST INFRASTRUCTURE - not part of the shipped library. See oracle.h.
+ *
+ * Build: gcc -std=c99 -O2 -fopenmp -ffp-contract=off -fPIC -shared oracle.c -lm
+ * (-ffp-contract=off matters: the reference never fuses a*b+c, and bit-exact
+ * parity of the elementwise map depends on it.)
+ *
+ * Parity pins (what fixes each function besides reading the reference):
+ *   map            brute-force parenthesised scalar loop; guide/basic.cpp:25-30 values
+ *   reductions     test/test.cu:9-18,35,47 closed forms; doc/README.md:162-185; all-ones counts
+ *   softmax        uniform logits -> 1/n exactly; shift invariance; float64 brute force.
+ *                  Absolute values depend on libm expf: parity unpinned at the ulp level
+ *                  (the reference's tests only compare CPU with GPU at 1e-4).
+ *   softmax grad   -1 at the label column, identical copy elsewhere
+ *   pool / unpool  test/pool.cu:29-48, test/pairtest.cu:29-77 closed forms
+ *   patch2col      test/unpack.cu:29-59 closed form; index-valued images
+ *   col2patch      coverage counts 4/6/9; adjoint identity with patch2col
+ *   half           exhaustive round trip; F16C agreement where the host has it
+ * and, where /root/reference is present, bit-for-bit agreement with the reference's
+ * own headers compiled into oracle/_ref (see oracle/Makefile).
+ */
+#include "oracle.h"
+
+#include <float.h>
+#include <math.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#include "../mshadow_amd/cases/portable_math.h"
+
+int orc_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+/* ------------------------------------------------------------------ half */
+
+/* mshadow/half.h:197-242 (software path) and :321-330 (F16C, rounding mode 0):
+   round to nearest, ties to even; overflow to infinity; gradual underflow. */
+uint16_t orc_float2half(float v) {
+  uint32_t x;
+  memcpy(&x, &v, 4);
+  uint32_t sign = (x >> 16) & 0x8000u;
+  uint32_t a = x & 0x7fffffffu;
+  if (a > 0x7f800000u) { /* NaN: quiet, keep the top payload bits */
+    return (uint16_t)(sign | 0x7e00u | ((a >> 13) & 0x1ffu));
+  }
+  if (a >= 0x38800000u) { /* normal half range or above */
+    uint32_t r = a + 0xfffu + ((a >> 13) & 1u);
+    uint32_t h = (r - 0x38000000u) >> 13;
+    if (h >= 0x7c00u) h = 0x7c00u;
+    return (uint16_t)(sign | h);
+  }
+  /* result is a half subnormal (unit 2^-24) or zero */
+  uint32_t e = a >> 23;
+  if (e < 102u) return (uint16_t)sign; /* below 2^-25: rounds to zero */
+  uint32_t m = (a & 0x7fffffu) | 0x800000u;
+  uint32_t shift = 126u - e; /* 14..24 */
+  uint32_t q = m >> shift;
+  uint32_t rem = m & ((1u << shift) - 1u);
+  uint32_t half = 1u << (shift - 1u);
+  if (rem > half || (rem == half && (q & 1u))) ++q;
+  return (uint16_t)(sign | q);
+}
+
+/* mshadow/half.h:244-283: exact widening */
+float orc_half2float(uint16_t h) {
+  uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+  uint32_t e = (h >> 10) & 0x1fu;
+  uint32_t m = h & 0x3ffu;
+  uint32_t x;
+  if (e == 0) {
+    if (m == 0) {
+      x = sign;
+    } else {
+      float f = (float)m * 5.9604644775390625e-08f; /* m * 2^-24, exact */
+      memcpy(&x, &f, 4);
+      x |= sign;
+    }
+  } else if (e == 31) {
+    x = sign | 0x7f800000u | (m << 13);
+  } else {
+    x = sign | ((e + 112u) << 23) | (m << 13);
+  }
+  float f;
+  memcpy(&f, &x, 4);
+  return f;
+}
+
+void orc_float2half_n(uint16_t *dst, const float *src, int64_t n) {
+#pragma omp parallel for
+  for (int64_t i = 0; i < n; ++i) dst[i] = orc_float2half(src[i]);
+}
+
+void orc_half2float_n(float *dst, const uint16_t *src, int64_t n) {
+#pragma omp parallel for
+  for (int64_t i = 0; i < n; ++i) dst[i] = orc_half2float(src[i]);
+}
+
+/* half_t arithmetic: every operator widens, computes in float and rounds back
+   (mshadow/half.h:45-66); operator+= rounds after each step (:58-62) */
+static inline uint16_t half_add(uint16_t a, uint16_t b) {
+  return orc_float2half(orc_half2float(a) + orc_half2float(b));
+}
+
+/* ------------------------------------------------------------------ savers / reducers */
+
+/* mshadow/base.h:539-602 */
+static inline void save_f32(float *dst, float v, int saver) {
+  switch (saver) {
+    case ORC_SAVETO: *dst = v; break;
+    case ORC_PLUSTO: *dst += v; break;
+    case ORC_MINUSTO: *dst -= v; break;
+    case ORC_MULTO: *dst *= v; break;
+    default: *dst /= v; break;
+  }
+}
+
+/* mshadow/base.h:676-680 (sum), :752-761 (maximum = std::max(dst, src)),
+   :822-831 (minimum = std::min(dst, src)) */
+static inline void reduce_f32(float *dst, float src, int reducer) {
+  switch (reducer) {
+    case ORC_SUM: *dst += src; break;
+    case ORC_MAX: *dst = (*dst < src) ? src : *dst; break;
+    default: *dst = (src < *dst) ? src : *dst; break;
+  }
+}
+
+/* mshadow/base.h:716-719, :794-797, :858-861 */
+static inline float init_f32(int reducer) {
+  switch (reducer) {
+    case ORC_SUM: return 0.0f;
+    case ORC_MAX: return -FLT_MAX;
+    default: return FLT_MAX;
+  }
+}
+
+/* mshadow/base.h:711-714 (sum: 1), :787-790 and :851-854 (equality) */
+static inline float partial_grad_f32(float redres, float redsrc, int reducer) {
+  if (reducer == ORC_SUM) return 1.0f;
+  return redres == redsrc ? 1.0f : 0.0f;
+}
+
+/* ------------------------------------------------------------------ elementwise map */
+
+/* MapPlan, mshadow/tensor_cpu-inl.h:143-159: one thread per row y, x ascending,
+   Saver::Save(dst(y,x), plan.Eval(y,x)). The expression tree
+   A*B + 0.5f*F<sigmoid>(C) - D evaluates as ((a*b) + (0.5f*sig(c))) - d
+   (mshadow/expression.h:353-374, expr_engine-inl.h:116-131). */
+void orc_map_fused_f32(float *dst, int dstride, const float *a, int astride, const float *b,
+                       int bstride, const float *c, int cstride, const float *d, int dstride_d,
+                       int rows, int cols, int saver) {
+#pragma omp parallel for
+  for (int y = 0; y < rows; ++y) {
+    for (int x = 0; x < cols; ++x) {
+      float ab = a[(int64_t)y * astride + x] * b[(int64_t)y * bstride + x];
+      float hs = 0.5f * pmath_sigmoid(c[(int64_t)y * cstride + x]);
+      float v = (ab + hs) - d[(int64_t)y * dstride_d + x];
+      save_f32(&dst[(int64_t)y * dstride + x], v, saver);
+    }
+  }
+}
+
+/* scalar right-hand side: Plan<ScalarExp>, mshadow/expr_engine-inl.h:83-93 */
+void orc_map_scalar_f32(float *dst, int dstride, int rows, int cols, float scalar, int saver) {
+#pragma omp parallel for
+  for (int y = 0; y < rows; ++y) {
+    for (int x = 0; x < cols; ++x) save_f32(&dst[(int64_t)y * dstride + x], scalar, saver);
+  }
+}
+
+/* ((a + s1) / s2) + s3, the expression of guide/basic.cpp:27 */
+void orc_map_axpb_f32(float *dst, int dstride, const float *a, int astride, int rows, int cols,
+                      float s1, float s2, float s3, int saver) {
+#pragma omp parallel for
+  for (int y = 0; y < rows; ++y) {
+    for (int x = 0; x < cols; ++x) {
+      float v = ((a[(int64_t)y * astride + x] + s1) / s2) + s3;
+      save_f32(&dst[(int64_t)y * dstride + x], v, saver);
+    }
+  }
+}
+
+/* ------------------------------------------------------------------ reductions */
+
+/* MapReduceKeepLowest, mshadow/tensor_cpu-inl.h:203-228: one thread per column,
+   res = src(0,x), then rows 1.. in order, Save(dst[x], res * scale). */
+void orc_reduce_keep_lowest_f32(float *dst, const float *src, int sstride, int rows, int cols,
+                                int reducer, int saver, float scale) {
+#pragma omp parallel for
+  for (int x = 0; x < cols; ++x) {
+    float res = src[x];
+    for (int y = 1; y < rows; ++y) reduce_f32(&res, src[(int64_t)y * sstride + x], reducer);
+    save_f32(&dst[x], res * scale, saver);
+  }
+}
+
+/* MapReduceKeepHighDim, mshadow/tensor_cpu-inl.h:230-268: shape viewed as
+   (n, c, y, x); per kept index c: for each n an inner reduction over (y, x) from the
+   reducer's initial value, merged in n order into the outer accumulator. */
+void orc_reduce_keep_highdim_f32(float *dst, const float *src, int sstride, int n, int c, int y,
+                                 int x, int reducer, int saver, float scale) {
+#pragma omp parallel for
+  for (int ci = 0; ci < c; ++ci) {
+    float res = init_f32(reducer);
+    for (int ni = 0; ni < n; ++ni) {
+      float tres = init_f32(reducer);
+      for (int yi = 0; yi < y; ++yi) {
+        const float *row = src + (int64_t)((ni * c + ci) * y + yi) * sstride;
+        for (int xi = 0; xi < x; ++xi) reduce_f32(&tres, row[xi], reducer);
+      }
+      reduce_f32(&res, tres, reducer);
+    }
+    save_f32(&dst[ci], res * scale, saver);
+  }
+}
+
+/* ------------------------------------------------------------------ softmax */
+
+/* Softmax, mshadow/tensor_cpu-inl.h:270-285 (one row) and :464-472 (rows in
+   parallel): max with a strict '<' update, exp(x - max) written to dst and summed
+   left to right in float, then a true division per element. In-place is allowed
+   because each element of the row is read before it is written. */
+void orc_softmax_f32(float *dst, int dstride, const float *src, int sstride, int rows, int cols) {
+#pragma omp parallel for
+  for (int y = 0; y < rows; ++y) {
+    const float *e = src + (int64_t)y * sstride;
+    float *o = dst + (int64_t)y * dstride;
+    float mmax = e[0];
+    for (int x = 1; x < cols; ++x) {
+      if (mmax < e[x]) mmax = e[x];
+    }
+    float sum = 0.0f;
+    for (int x = 0; x < cols; ++x) {
+      o[x] = expf(e[x] - mmax);
+      sum += o[x];
+    }
+    for (int x = 0; x < cols; ++x) o[x] /= sum;
+  }
+}
+
+/* SoftmaxGrad, mshadow/tensor_cpu-inl.h:287-302: label is stored in the data
+   type and truncated with static_cast<int>; a label outside [0, cols) leaves a copy. */
+void orc_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride,
+                          const float *label, int rows, int cols) {
+#pragma omp parallel for
+  for (int y = 0; y < rows; ++y) {
+    const int k = (int)label[y];
+    const float *s = src + (int64_t)y * sstride;
+    float *o = dst + (int64_t)y * dstride;
+    for (int x = 0; x < cols; ++x) {
+      if (x == k) {
+        o[k] = s[k] - 1.0f;
+      } else {
+        o[x] = s[x];
+      }
+    }
+  }
+}
+
+/* ------------------------------------------------------------------ pool / unpool */
+
+static inline int imin(int a, int b) { return a < b ? a : b; }
+
+/* Plan<PoolingExp>::Eval, mshadow/extension/spatial_pool.h:125-142, driven by the
+   MapPlan loop over the flattened output (rows = planes * ph, cols = pw). */
+void orc_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes, int h, int w,
+                  int ph, int pw, int ky, int kx, int sy, int sx, int reducer) {
+  const int out_rows = planes * ph;
+#pragma omp parallel for
+  for (int i = 0; i < out_rows; ++i) {
+    const int py = i % ph;
+    const int c = i / ph;
+    const int y_start = py * sy;
+    const int y_end = imin(y_start + ky, h);
+    for (int j = 0; j < pw; ++j) {
+      const int x_start = j * sx;
+      const int x_end = imin(x_start + kx, w);
+      float res = init_f32(reducer);
+      for (int y = y_start; y < y_end; ++y) {
+        for (int x = x_start; x < x_end; ++x) {
+          reduce_f32(&res, src[(int64_t)(c * h + y) * sstride + x], reducer);
+        }
+      }
+      dst[(int64_t)i * dstride + j] = res;
+    }
+  }
+}
+
+/* Plan<UnPoolingExp>::Eval, mshadow/extension/spatial_unpool.h:102-125: every
+   source pixel sums grad over the windows that cover it, weighted by
+   PartialGrad(src, pooled) (equality for max / min), py then px ascending. */
+void orc_unpool_f32(float *dst, int dstride, const float *src, int sstride, const float *pooled,
+                    int pstride, const float *grad, int gstride, int planes, int h, int w, int ph,
+                    int pw, int ky, int kx, int sy, int sx, int reducer) {
+  const int out_rows = planes * h;
+#pragma omp parallel for
+  for (int i = 0; i < out_rows; ++i) {
+    const int y = i % h;
+    const int c = i / h;
+    const int py_min = y < ky ? 0 : (y - ky + sy) / sy;
+    const int py_max = imin((y + sy) / sy, ph);
+    for (int x = 0; x < w; ++x) {
+      const float vsrc = src[(int64_t)i * sstride + x];
+      const int px_min = x < kx ? 0 : (x - kx + sx) / sx;
+      const int px_max = imin((x + sx) / sx, pw);
+      float val = 0.0f;
+      for (int py = py_min; py < py_max; ++py) {
+        for (int px = px_min; px < px_max; ++px) {
+          const float p = pooled[(int64_t)(c * ph + py) * pstride + px];
+          const float g = grad[(int64_t)(c * ph + py) * gstride + px];
+          val += partial_grad_f32(vsrc, p, reducer) * g;
+        }
+      }
+      dst[(int64_t)i * dstride + x] = val;
+    }
+  }
+}
+
+/* ------------------------------------------------------------------ patch2col / col2patch */
+
+/* The index math below is shared by the f16 and f32 entry points through macros so
+   that both follow the same lines of the reference.
+
+   Plan<PaddingExp>::Eval, mshadow/extension/pad.h:87-99, over a source with
+   (hs, ws) rows / cols per plane: value at padded row i (= plane * (hs + 2 pad_y) + y)
+   and column j. */
+#define PAD_EVAL(T, ZERO, img, istride, hs, ws, pad_y, pad_x, i, j, out)              \
+  do {                                                                                \
+    const int new_h_ = (hs) + 2 * (pad_y);                                            \
+    const int y_ = (i) % new_h_;                                                      \
+    const int c_ = (i) / new_h_;                                                      \
+    if (y_ < (pad_y) || (j) < (pad_x)) {                                              \
+      (out) = (ZERO);                                                                 \
+    } else {                                                                          \
+      const int h_ = y_ - (pad_y);                                                    \
+      const int w_ = (j) - (pad_x);                                                   \
+      if (h_ < (hs) && w_ < (ws)) {                                                   \
+        (out) = (img)[(int64_t)(c_ * (hs) + h_) * (istride) + w_];                    \
+      } else {                                                                        \
+        (out) = (ZERO);                                                               \
+      }                                                                               \
+    }                                                                                 \
+  } while (0)
+
+/* Plan<UnpackPatchToColXExp>::Eval, mshadow/extension/unpack_patch2col.h:126-141,
+   with the padded image (pad.h) as its source; output shape per :43-67. */
+#define IM2COL_BODY(T, ZERO)                                                          \
+  const int hp = h + 2 * pad_y, wp = w + 2 * pad_x;                                   \
+  const int o_height = (hp - (dy * (ky - 1) + 1)) / sy + 1;                           \
+  const int o_width = (wp - (dx * (kx - 1) + 1)) / sx + 1;                            \
+  const int out_rows = ky * kx * c;                                                   \
+  const int out_cols = o_height * o_width * n;                                        \
+  _Pragma("omp parallel for") for (int i = 0; i < out_rows; ++i) {                    \
+    const int x_offset = i % kx * dx;                                                 \
+    const int idivp = i / kx;                                                         \
+    const int y_offset = idivp % ky * dy;                                             \
+    const int ch = idivp / ky;                                                        \
+    for (int j = 0; j < out_cols; ++j) {                                              \
+      const int x = (j % o_width) * sx + x_offset;                                    \
+      const int jdivw = j / o_width;                                                  \
+      const int y = (jdivw % o_height) * sy + y_offset;                               \
+      const int ni = jdivw / o_height;                                                \
+      T v;                                                                            \
+      if (x < wp && y < hp) {                                                         \
+        PAD_EVAL(T, ZERO, img, istride, h, w, pad_y, pad_x, (ni * c + ch) * hp + y, x, v); \
+      } else {                                                                        \
+        v = (ZERO);                                                                   \
+      }                                                                               \
+      col[(int64_t)i * cstride + j] = v;                                              \
+    }                                                                                 \
+  }
+
+void orc_im2col_f16(uint16_t *col, int cstride, const uint16_t *img, int istride, int n, int c,
+                    int h, int w, int ky, int kx, int sy, int sx, int dy, int dx, int pad_y,
+                    int pad_x) {
+  IM2COL_BODY(uint16_t, (uint16_t)0)
+}
+
+void orc_im2col_f32(float *col, int cstride, const float *img, int istride, int n, int c, int h,
+                    int w, int ky, int kx, int sy, int sx, int dy, int dx, int pad_y, int pad_x) {
+  IM2COL_BODY(float, 0.0f)
+}
+
+/* Plan<CroppingExp>::Eval (mshadow/extension/crop.h:103-110, offsets pad_y / pad_x)
+   over Plan<PackColToPatchXExp>::Eval (mshadow/extension/pack_col2patch.h:118-144)
+   for an image of (n, c, h + 2 pad_y, w + 2 pad_x): patches are visited py then px
+   ascending and accumulated in the element type, so half rounds after every add. */
+#define COL2IM_BODY(T, ZERO, ADD)                                                     \
+  const int hp = h + 2 * pad_y, wp = w + 2 * pad_x;                                   \
+  const int o_height = (hp - (dy * (ky - 1) + 1)) / sy + 1;                           \
+  const int o_width = (wp - (dx * (kx - 1) + 1)) / sx + 1;                            \
+  const int psize_y_dilate = dy * (ky - 1) + 1;                                       \
+  const int psize_x_dilate = dx * (kx - 1) + 1;                                       \
+  const int out_rows = n * c * h;                                                     \
+  _Pragma("omp parallel for") for (int oi = 0; oi < out_rows; ++oi) {                 \
+    /* crop: output row oi -> source row of the padded image */                       \
+    const int cy = oi % h;                                                            \
+    const int cc = oi / h;                                                            \
+    const int i = cc * hp + cy + pad_y;                                               \
+    const int y = i % hp;                                                             \
+    const int idivh = i / hp;                                                         \
+    const int ch = idivh % c;                                                         \
+    const int ni = idivh / c;                                                         \
+    const int py_min = y < psize_y_dilate ? y % dy : (y - psize_y_dilate + sy) / sy;  \
+    const int py_max = imin((y + sy) / sy, o_height);                                 \
+    for (int oj = 0; oj < w; ++oj) {                                                  \
+      const int x = oj + pad_x;                                                       \
+      const int px_min = x < psize_x_dilate ? x % dx : (x - psize_x_dilate + sx) / sx; \
+      const int px_max = imin((x + sx) / sx, o_width);                                \
+      T res = (ZERO);                                                                 \
+      for (int py = py_min; py < py_max; py += dy) {                                  \
+        for (int px = px_min; px < px_max; px += dx) {                                \
+          const int r = (ch * ky + (y - py * sy) / dy) * kx + (x - px * sx) / dx;     \
+          const int q = (ni * o_height + py) * o_width + px;                          \
+          res = ADD(res, col[(int64_t)r * cstride + q]);                              \
+        }                                                                             \
+      }                                                                               \
+      img[(int64_t)oi * istride + oj] = res;                                          \
+    }                                                                                 \
+  }
+
+#define ADD_F32(a, b) ((a) + (b))
+
+void orc_col2im_f16(uint16_t *img, int istride, const uint16_t *col, int cstride, int n, int c,
+                    int h, int w, int ky, int kx, int sy, int sx, int dy, int dx, int pad_y,
+                    int pad_x) {
+  COL2IM_BODY(uint16_t, (uint16_t)0, half_add)
+}
+
+void orc_col2im_f32(float *img, int istride, const float *col, int cstride, int n, int c, int h,
+                    int w, int ky, int kx, int sy, int sx, int dy, int dx, int pad_y, int pad_x) {
+  COL2IM_BODY(float, 0.0f, ADD_F32)
+}

@@ -1,0 +1,80 @@
+/*
+ * TEST INFRASTRUCTURE - not part of the shipped library.
+ *
+ * Plain-C restatement of the CPU path of dmlc/mshadow for the nine hot-path
+ * operations (elementwise map, two reduce-to-1D forms, softmax forward and
+ * gradient, pool / unpool, patch2col / col2patch with pad / crop). Every
+ * function follows the loop order and the rounding points of the reference
+ * file:line it cites, so that results are bit-identical to the reference built
+ * with -ffp-contract=off. Only tests, the smoke check and the benchmark's CPU
+ * baseline may call into this file; the GPU library never does.
+ *
+ * All sizes and indices are 32-bit signed like the reference's index_t
+ * (mshadow/base.h:288-292). Strides are row pitches in elements
+ * (mshadow/tensor.h:419-423).
+ */
+#ifndef MSHADOW_ORACLE_H_
+#define MSHADOW_ORACLE_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* savers, mshadow/base.h:539-602 */
+enum { ORC_SAVETO = 0, ORC_PLUSTO = 1, ORC_MINUSTO = 2, ORC_MULTO = 3, ORC_DIVTO = 4 };
+/* reducers, mshadow/base.h:604-862 */
+enum { ORC_SUM = 0, ORC_MAX = 1, ORC_MIN = 2 };
+
+/* number of OpenMP threads the loops below will use */
+int orc_num_threads(void);
+
+/* half <-> float, mshadow/half.h:197-242 (round to nearest even) and :285-330 */
+uint16_t orc_float2half(float v);
+float orc_half2float(uint16_t h);
+void orc_float2half_n(uint16_t *dst, const float *src, int64_t n);
+void orc_half2float_n(float *dst, const uint16_t *src, int64_t n);
+
+/* dst <saver>= a*b + 0.5f*sigmoid(c) - d, sigmoid = pmath_sigmoid (caller functor) */
+void orc_map_fused_f32(float *dst, int dstride, const float *a, int astride,
+                       const float *b, int bstride, const float *c, int cstride,
+                       const float *d, int dstride_d, int rows, int cols, int saver);
+/* dst <saver>= scalar */
+void orc_map_scalar_f32(float *dst, int dstride, int rows, int cols, float scalar, int saver);
+/* dst <saver>= (a + s1) / s2 + s3   (guide/basic.cpp:25-30 shape of expression) */
+void orc_map_axpb_f32(float *dst, int dstride, const float *a, int astride, int rows, int cols,
+                      float s1, float s2, float s3, int saver);
+
+void orc_reduce_keep_lowest_f32(float *dst, const float *src, int sstride, int rows, int cols,
+                                int reducer, int saver, float scale);
+void orc_reduce_keep_highdim_f32(float *dst, const float *src, int sstride, int n, int c, int y,
+                                 int x, int reducer, int saver, float scale);
+
+void orc_softmax_f32(float *dst, int dstride, const float *src, int sstride, int rows, int cols);
+void orc_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride,
+                          const float *label, int rows, int cols);
+
+void orc_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes, int h, int w,
+                  int ph, int pw, int ky, int kx, int sy, int sx, int reducer);
+void orc_unpool_f32(float *dst, int dstride, const float *src, int sstride, const float *pooled,
+                    int pstride, const float *grad, int gstride, int planes, int h, int w, int ph,
+                    int pw, int ky, int kx, int sy, int sx, int reducer);
+
+/* col = unpack_patch2col(pad(img, pad_y, pad_x), ky, kx, sy, sx, dy, dx) */
+void orc_im2col_f16(uint16_t *col, int cstride, const uint16_t *img, int istride, int n, int c,
+                    int h, int w, int ky, int kx, int sy, int sx, int dy, int dx, int pad_y,
+                    int pad_x);
+void orc_im2col_f32(float *col, int cstride, const float *img, int istride, int n, int c, int h,
+                    int w, int ky, int kx, int sy, int sx, int dy, int dx, int pad_y, int pad_x);
+/* img = crop(pack_col2patch(col, (n,c,h+2pad_y,w+2pad_x), ...), (h,w), pad_y, pad_x) */
+void orc_col2im_f16(uint16_t *img, int istride, const uint16_t *col, int cstride, int n, int c,
+                    int h, int w, int ky, int kx, int sy, int sx, int dy, int dx, int pad_y,
+                    int pad_x);
+void orc_col2im_f32(float *img, int istride, const float *col, int cstride, int n, int c, int h,
+                    int w, int ky, int kx, int sy, int sx, int dy, int dx, int pad_y, int pad_x);
+
+#ifdef __cplusplus
+}
+#endif
+#endif  /* MSHADOW_ORACLE_H_ */

@@ -1,0 +1,180 @@
+/*
+ * TEST INFRASTRUCTURE - not part of the shipped library.
+ *
+ * Thin C entry points around the *real* dmlc/mshadow headers (included from
+ * /root/reference through -I, never copied): each function wraps the caller's
+ * buffers in Tensor<cpu> handles and evaluates the same expression a user of the
+ * reference would write. The resulting library (oracle/_ref/libmshadow_ref.so)
+ * checks the C restatement in oracle.c bit for bit and serves as the timed CPU
+ * baseline. Signatures mirror oracle.h with the prefix ref_.
+ */
+#include <mshadow/tensor.h>
+
+#include <omp.h>
+#include <stdint.h>
+
+#include "../mshadow_amd/cases/portable_math.h"
+
+using namespace mshadow;
+using namespace mshadow::expr;
+
+namespace {
+
+/* caller-side functor, same shape as guide/neuralnet/nnet.cu:14-18 */
+struct sigmoid {
+  MSHADOW_XINLINE static float Map(float a) { return pmath_sigmoid(a); }
+};
+
+template <typename T>
+Tensor<cpu, 2, T> T2(const T *p, int rows, int cols, int stride) {
+  return Tensor<cpu, 2, T>(const_cast<T *>(p), Shape2(rows, cols), stride, NULL);
+}
+template <typename T>
+Tensor<cpu, 4, T> T4(const T *p, int n, int c, int h, int w, int stride) {
+  return Tensor<cpu, 4, T>(const_cast<T *>(p), Shape4(n, c, h, w), stride, NULL);
+}
+template <typename T>
+Tensor<cpu, 3, T> T3(const T *p, int a, int b, int c, int stride) {
+  return Tensor<cpu, 3, T>(const_cast<T *>(p), Shape3(a, b, c), stride, NULL);
+}
+template <typename T>
+Tensor<cpu, 1, T> T1(const T *p, int n) {
+  return Tensor<cpu, 1, T>(const_cast<T *>(p), Shape1(n));
+}
+
+template <typename Dst, typename E>
+void Assign(Dst dst, const E &e, int saver) {
+  switch (saver) {
+    case 0: dst = e; break;
+    case 1: dst += e; break;
+    case 2: dst -= e; break;
+    case 3: dst *= e; break;
+    default: dst /= e; break;
+  }
+}
+
+template <typename Reducer, typename Src>
+void ReduceHigh(Tensor<cpu, 1, float> dst, const Src &src, int saver, float scale) {
+  switch (saver) {
+    case 0: dst = scale * reduce_except_dim<1, Reducer>(src); break;
+    case 1: dst += scale * reduce_except_dim<1, Reducer>(src); break;
+    case 2: dst -= scale * reduce_except_dim<1, Reducer>(src); break;
+    case 3: dst *= scale * reduce_except_dim<1, Reducer>(src); break;
+    default: dst /= scale * reduce_except_dim<1, Reducer>(src); break;
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int ref_num_threads(void) { return omp_get_max_threads(); }
+
+void ref_float2half_n(uint16_t *dst, const float *src, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) dst[i] = half::half_t(src[i]).half_;
+}
+void ref_half2float_n(float *dst, const uint16_t *src, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) dst[i] = static_cast<float>(half::half_t::Binary(src[i]));
+}
+
+void ref_map_fused_f32(float *dst, int dstride, const float *a, int astride, const float *b,
+                       int bstride, const float *c, int cstride, const float *d, int dstride_d,
+                       int rows, int cols, int saver) {
+  Tensor<cpu, 2, float> A = T2(a, rows, cols, astride), B = T2(b, rows, cols, bstride),
+                        C = T2(c, rows, cols, cstride), D = T2(d, rows, cols, dstride_d);
+  Assign(T2(dst, rows, cols, dstride), A * B + 0.5f * F<sigmoid>(C) - D, saver);
+}
+
+void ref_map_scalar_f32(float *dst, int dstride, int rows, int cols, float scalar, int saver) {
+  Tensor<cpu, 2, float> o = T2(dst, rows, cols, dstride);
+  switch (saver) {
+    case 0: o = scalar; break;
+    case 1: o += scalar; break;
+    case 2: o -= scalar; break;
+    case 3: o *= scalar; break;
+    default: o /= scalar; break;
+  }
+}
+
+void ref_map_axpb_f32(float *dst, int dstride, const float *a, int astride, int rows, int cols,
+                      float s1, float s2, float s3, int saver) {
+  Tensor<cpu, 2, float> A = T2(a, rows, cols, astride);
+  Assign(T2(dst, rows, cols, dstride), (A + s1) / s2 + s3, saver);
+}
+
+void ref_reduce_keep_lowest_f32(float *dst, const float *src, int sstride, int rows, int cols,
+                                int reducer, int saver, float scale) {
+  Tensor<cpu, 2, float> S = T2(src, rows, cols, sstride);
+  Tensor<cpu, 1, float> o = T1(dst, cols);
+  /* reduce_except_dim<1> of a 2-D source keeps the lowest dimension
+     (reduceto1d.h:92-100), the same engine sum_rows uses */
+  if (reducer == 0) ReduceHigh<red::sum>(o, S, saver, scale);
+  else if (reducer == 1) ReduceHigh<red::maximum>(o, S, saver, scale);
+  else ReduceHigh<red::minimum>(o, S, saver, scale);
+}
+
+void ref_reduce_keep_highdim_f32(float *dst, const float *src, int sstride, int n, int c, int y,
+                                 int x, int reducer, int saver, float scale) {
+  Tensor<cpu, 4, float> S = T4(src, n, c, y, x, sstride);
+  Tensor<cpu, 1, float> o = T1(dst, c);
+  if (reducer == 0) ReduceHigh<red::sum>(o, S, saver, scale);
+  else if (reducer == 1) ReduceHigh<red::maximum>(o, S, saver, scale);
+  else ReduceHigh<red::minimum>(o, S, saver, scale);
+}
+
+void ref_softmax_f32(float *dst, int dstride, const float *src, int sstride, int rows, int cols) {
+  Softmax(T2(dst, rows, cols, dstride), T2(src, rows, cols, sstride));
+}
+
+void ref_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride,
+                          const float *label, int rows, int cols) {
+  SoftmaxGrad(T2(dst, rows, cols, dstride), T2(src, rows, cols, sstride), T1(label, rows));
+}
+
+void ref_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes, int h, int w,
+                  int ph, int pw, int ky, int kx, int sy, int sx, int reducer) {
+  Tensor<cpu, 3, float> S = T3(src, planes, h, w, sstride);
+  Tensor<cpu, 3, float> o = T3(dst, planes, ph, pw, dstride);
+  if (reducer == 0) o = pool<red::sum>(S, Shape2(ph, pw), ky, kx, sy, sx);
+  else if (reducer == 1) o = pool<red::maximum>(S, Shape2(ph, pw), ky, kx, sy, sx);
+  else o = pool<red::minimum>(S, Shape2(ph, pw), ky, kx, sy, sx);
+}
+
+void ref_unpool_f32(float *dst, int dstride, const float *src, int sstride, const float *pooled,
+                    int pstride, const float *grad, int gstride, int planes, int h, int w, int ph,
+                    int pw, int ky, int kx, int sy, int sx, int reducer) {
+  Tensor<cpu, 3, float> S = T3(src, planes, h, w, sstride);
+  Tensor<cpu, 3, float> P = T3(pooled, planes, ph, pw, pstride);
+  Tensor<cpu, 3, float> G = T3(grad, planes, ph, pw, gstride);
+  Tensor<cpu, 3, float> o = T3(dst, planes, h, w, dstride);
+  if (reducer == 0) o = unpool<red::sum>(S, P, G, ky, kx, sy, sx);
+  else if (reducer == 1) o = unpool<red::maximum>(S, P, G, ky, kx, sy, sx);
+  else o = unpool<red::minimum>(S, P, G, ky, kx, sy, sx);
+}
+
+#define REF_IM2COL(NAME, CT, MT)                                                              \
+  void NAME(CT *col, int cstride, const CT *img, int istride, int n, int c, int h, int w,     \
+            int ky, int kx, int sy, int sx, int dy, int dx, int pad_y, int pad_x) {           \
+    const int hp = h + 2 * pad_y, wp = w + 2 * pad_x;                                         \
+    const int oh = (hp - (dy * (ky - 1) + 1)) / sy + 1, ow = (wp - (dx * (kx - 1) + 1)) / sx + 1; \
+    Tensor<cpu, 4, MT> I = T4(reinterpret_cast<const MT *>(img), n, c, h, w, istride);        \
+    Tensor<cpu, 2, MT> O = T2(reinterpret_cast<MT *>(col), ky * kx * c, oh * ow * n, cstride); \
+    O = unpack_patch2col(pad(I, pad_y, pad_x), ky, kx, sy, sx, dy, dx);                       \
+  }
+REF_IM2COL(ref_im2col_f16, uint16_t, half::half_t)
+REF_IM2COL(ref_im2col_f32, float, float)
+
+#define REF_COL2IM(NAME, CT, MT)                                                              \
+  void NAME(CT *img, int istride, const CT *col, int cstride, int n, int c, int h, int w,     \
+            int ky, int kx, int sy, int sx, int dy, int dx, int pad_y, int pad_x) {           \
+    const int hp = h + 2 * pad_y, wp = w + 2 * pad_x;                                         \
+    const int oh = (hp - (dy * (ky - 1) + 1)) / sy + 1, ow = (wp - (dx * (kx - 1) + 1)) / sx + 1; \
+    Tensor<cpu, 4, MT> I = T4(reinterpret_cast<MT *>(img), n, c, h, w, istride);              \
+    Tensor<cpu, 2, MT> C = T2(reinterpret_cast<const MT *>(col), ky * kx * c, oh * ow * n, cstride); \
+    I = crop(pack_col2patch(C, Shape4(n, c, hp, wp), ky, kx, sy, sx, dy, dx), Shape2(h, w),   \
+             pad_y, pad_x);                                                                   \
+  }
+REF_COL2IM(ref_col2im_f16, uint16_t, half::half_t)
+REF_COL2IM(ref_col2im_f32, float, float)
+
+}  // extern "C"
