@@ -1,0 +1,188 @@
+/*
+ * libmshadow_hip - C ABI of the gfx950 (MI355X) device layer behind mshadow's
+ * Tensor<gpu> / Stream<gpu> API.
+ *
+ * The reference has no FFI: its GPU device is a set of C++ templates that call the
+ * CUDA runtime and launch CUDA kernels (mshadow/tensor_gpu-inl.h,
+ * mshadow/stream_gpu-inl.h, mshadow/cuda/tensor_gpu-inl.cuh). This header is the
+ * boundary that replaces those call sites. Each entry names the reference code it
+ * stands in for. Three groups:
+ *   1. runtime      device, stream, event, memory, copy
+ *   2. launch       start a kernel instantiated in the caller's translation unit
+ *                   (expression templates compile there, not in this library)
+ *   3. fixed ops    whole operations on plain (pointer, pitch, shape) arguments
+ *
+ * Conventions: every function returns 0 on success and a non-zero code otherwise,
+ * with a thread-local message available from mshadow_hip_last_error(); no exception
+ * crosses the boundary. Pointers are device pointers unless named host. `stream` is
+ * the opaque handle from mshadow_hip_stream_create, or NULL for the device's default
+ * stream. Pitches ("stride") are in ELEMENTS, as in mshadow's Tensor::stride_; sizes
+ * and indices are 32-bit like mshadow's index_t. Kernels are asynchronous: a call
+ * returns once the work is queued on `stream`. The library never allocates device
+ * memory on its own; the caller owns every buffer.
+ */
+#ifndef MSHADOW_HIP_H_
+#define MSHADOW_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MSHADOW_HIP_ABI_VERSION 1
+
+/* status codes */
+enum {
+  MSHADOW_HIP_OK = 0,
+  MSHADOW_HIP_ERR_RUNTIME = 1,  /* a HIP runtime call failed; text in last_error */
+  MSHADOW_HIP_ERR_ARGUMENT = 2, /* shapes / pointers / enums rejected before launch */
+  MSHADOW_HIP_ERR_UNSUPPORTED = 3
+};
+
+/* saver: how a result is combined into dst (mshadow/base.h:539-602, sv::) */
+enum { MSHADOW_HIP_SAVETO = 0, MSHADOW_HIP_PLUSTO = 1, MSHADOW_HIP_MINUSTO = 2,
+       MSHADOW_HIP_MULTO = 3, MSHADOW_HIP_DIVTO = 4 };
+/* reducer (mshadow/base.h:604-862, red::) */
+enum { MSHADOW_HIP_SUM = 0, MSHADOW_HIP_MAX = 1, MSHADOW_HIP_MIN = 2 };
+/* copy direction for mshadow_hip_memcpy2d_async */
+enum { MSHADOW_HIP_H2D = 1, MSHADOW_HIP_D2H = 2, MSHADOW_HIP_D2D = 3, MSHADOW_HIP_H2H = 0 };
+
+/* message of the last failure on the calling thread ("" if none) */
+const char *mshadow_hip_last_error(void);
+int mshadow_hip_abi_version(void);
+
+/* ------------------------------------------------------------------ 1. runtime */
+
+typedef struct mshadow_hip_props {
+  char name[256];
+  char arch[64];             /* e.g. "gfx950:sramecc+:xnack-" */
+  int compute_units;
+  int wavefront_size;
+  int max_threads_per_block;
+  int clock_khz;
+  int memory_clock_khz;
+  int memory_bus_bits;
+  int l2_bytes;
+  size_t lds_bytes_per_block;
+  size_t total_global_mem;
+} mshadow_hip_props;
+
+/* InitTensorEngine<gpu> / SetDevice<gpu>: mshadow/tensor_gpu-inl.h:14-36
+   (cudaGetDeviceCount, cudaSetDevice, cudaGetDeviceProperties) */
+int mshadow_hip_device_count(int *count);
+int mshadow_hip_set_device(int device);
+int mshadow_hip_get_device(int *device);
+int mshadow_hip_get_props(int device, mshadow_hip_props *out);
+int mshadow_hip_device_sync(void);
+
+/* Stream<gpu>: mshadow/stream_gpu-inl.h:61-74 (Wait, CheckIdle), :181-211
+   (NewStream / DeleteStream -> cudaStreamCreate / cudaStreamDestroy) */
+int mshadow_hip_stream_create(void **stream);
+int mshadow_hip_stream_destroy(void *stream);
+int mshadow_hip_stream_sync(void *stream);
+int mshadow_hip_stream_query(void *stream, int *idle);
+
+/* timing (the reference has none; used by the benchmark harness) */
+int mshadow_hip_event_create(void **event);
+int mshadow_hip_event_destroy(void *event);
+int mshadow_hip_event_record(void *event, void *stream);
+int mshadow_hip_event_sync(void *event);
+int mshadow_hip_event_elapsed_ms(void *start, void *stop, float *ms);
+
+/* AllocSpace / FreeSpace<gpu>: mshadow/tensor_gpu-inl.h:37-56 (cudaMallocPitch,
+   cudaFree). pitch_bytes is a multiple of 256 when rows > 1. */
+int mshadow_hip_malloc_pitch(void **ptr, size_t *pitch_bytes, size_t width_bytes, size_t rows);
+int mshadow_hip_malloc(void **ptr, size_t bytes);
+int mshadow_hip_free(void *ptr);
+/* AllocHost_ / FreeHost_<gpu>: mshadow/tensor_cpu-inl.h:58-69 (pinned host memory) */
+int mshadow_hip_malloc_host(void **host_ptr, size_t bytes);
+int mshadow_hip_free_host(void *host_ptr);
+/* Copy cpu<->gpu, gpu<->gpu: mshadow/tensor_gpu-inl.h:57-92 (cudaMemcpy2DAsync).
+   Pitches and width in BYTES here, like the runtime call it replaces. */
+int mshadow_hip_memcpy2d_async(void *dst, size_t dpitch_bytes, const void *src,
+                               size_t spitch_bytes, size_t width_bytes, size_t rows, int kind,
+                               void *stream);
+int mshadow_hip_memset_async(void *dst, int byte_value, size_t bytes, void *stream);
+
+/* ------------------------------------------------------------------ 2. launch */
+
+/* The <<<grid, block, lds, stream>>> launch plus cudaPeekAtLastError of
+   mshadow/cuda/tensor_gpu-inl.cuh:16-21 and :95-120: `kernel` is the host-side
+   address of a __global__ function compiled by hipcc in the caller's own
+   translation unit (an instantiation of the kernel templates shipped in
+   mshadow/hip/); `args` is the array of pointers to its arguments. */
+int mshadow_hip_launch(const void *kernel, const uint32_t grid[3], const uint32_t block[3],
+                       void **args, size_t lds_bytes, void *stream);
+int mshadow_hip_peek_last_error(void);
+/* Grid size for `work_items` items at `items_per_block` per block: enough blocks to
+   cover the work, capped at `max_waves` resident rounds of the device's CUs
+   (replaces the kBaseGridNum / kMaxGridNum heuristics of tensor_gpu-inl.cuh:25-45). */
+int mshadow_hip_suggest_grid(size_t work_items, size_t items_per_block, int max_waves,
+                             uint32_t *grid_x);
+
+/* ------------------------------------------------------------------ 3. fixed ops */
+
+/* Softmax(dst, energy): mshadow/tensor_gpu-inl.h:157-161 -> cuda::Softmax,
+   tensor_gpu-inl.cuh:330-393. Row-wise; dst may alias src. The row sum is taken in
+   the CPU path's left-to-right order (tensor_cpu-inl.h:277-281). */
+int mshadow_hip_softmax_f32(float *dst, int dstride, const float *src, int sstride, int rows,
+                            int cols, void *stream);
+/* SoftmaxGrad(dst, src, label): mshadow/tensor_gpu-inl.h:169-174 ->
+   tensor_gpu-inl.cuh:239-256, :395-412. label holds `rows` floats, truncated to int. */
+int mshadow_hip_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride,
+                                 const float *label, int rows, int cols, void *stream);
+
+/* MapReduceKeepLowest<Saver, Reducer>(dst, src, scale): mshadow/tensor_gpu-inl.h:118-133
+   -> MapRedKeepLowestKernel, tensor_gpu-inl.cuh:122-168. dst[x] <saver>= scale *
+   reduce_y src[y][x], rows >= 1, reduced top to bottom like tensor_cpu-inl.h:221-227. */
+int mshadow_hip_reduce_keep_lowest_f32(float *dst, const float *src, int sstride, int rows,
+                                       int cols, int reducer, int saver, float scale,
+                                       void *stream);
+/* MapReduceKeepHighDim<Saver, Reducer, dimkeep>: mshadow/tensor_gpu-inl.h:135-156 ->
+   MapReduceKeepDim1Kernel, tensor_gpu-inl.cuh:170-215, on the equivalent 4-D view
+   (n, c, y, x) with row pitch sstride: dst[c] <saver>= scale * reduce_n(reduce_{y,x}
+   src[n][c][y][x]) in the two-level order of tensor_cpu-inl.h:254-267. */
+int mshadow_hip_reduce_keep_highdim_f32(float *dst, const float *src, int sstride, int n, int c,
+                                        int y, int x, int reducer, int saver, float scale,
+                                        void *stream);
+
+/* dst = pool<Reducer>(src, Shape2(ph, pw), ky, kx, sy, sx): the MapPlanKernel launch of
+   tensor_gpu-inl.cuh:67-120 with Plan<PoolingExp>::Eval (extension/spatial_pool.h:125-142)
+   as its body. src is planes x h x w with row pitch sstride, dst planes x ph x pw. */
+int mshadow_hip_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes,
+                         int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,
+                         int reducer, void *stream);
+/* dst = unpool<Reducer>(src, pooled, grad, ky, kx, sy, sx): same launch with
+   Plan<UnPoolingExp>::Eval (extension/spatial_unpool.h:102-125). */
+int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstride,
+                           const float *pooled, int pstride, const float *grad, int gstride,
+                           int planes, int h, int w, int ph, int pw, int ky, int kx, int sy,
+                           int sx, int reducer, void *stream);
+
+/* col = unpack_patch2col(pad(img, pad_y, pad_x), ky, kx, sy, sx, dy, dx): MapPlanKernel
+   with Plan<UnpackPatchToColXExp>::Eval (extension/unpack_patch2col.h:126-141) over
+   Plan<PaddingExp>::Eval (extension/pad.h:87-99). img is (n, c, h, w) with row pitch
+   istride; col is (ky*kx*c) x (oh*ow*n) with row pitch cstride. f16 = raw binary16 bits. */
+int mshadow_hip_im2col_f16(uint16_t *col, int cstride, const uint16_t *img, int istride, int n,
+                           int c, int h, int w, int ky, int kx, int sy, int sx, int dy, int dx,
+                           int pad_y, int pad_x, void *stream);
+int mshadow_hip_im2col_f32(float *col, int cstride, const float *img, int istride, int n, int c,
+                           int h, int w, int ky, int kx, int sy, int sx, int dy, int dx,
+                           int pad_y, int pad_x, void *stream);
+/* img = crop(pack_col2patch(col, (n, c, h+2*pad_y, w+2*pad_x), ky, kx, sy, sx, dy, dx),
+   (h, w), pad_y, pad_x): MapPlanKernel with Plan<CroppingExp>::Eval (extension/crop.h:
+   103-110) over Plan<PackColToPatchXExp>::Eval (extension/pack_col2patch.h:118-144);
+   overlapping patches are added in (py, px) order in the element type. */
+int mshadow_hip_col2im_f16(uint16_t *img, int istride, const uint16_t *col, int cstride, int n,
+                           int c, int h, int w, int ky, int kx, int sy, int sx, int dy, int dx,
+                           int pad_y, int pad_x, void *stream);
+int mshadow_hip_col2im_f32(float *img, int istride, const float *col, int cstride, int n, int c,
+                           int h, int w, int ky, int kx, int sy, int sx, int dy, int dx,
+                           int pad_y, int pad_x, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MSHADOW_HIP_H_ */

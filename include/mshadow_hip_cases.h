@@ -1,0 +1,89 @@
+/*
+ * libmshadow_cases - caller-style programs written against <mshadow/tensor.h>
+ * (Tensor<gpu>, Stream<gpu>, expression templates), compiled by hipcc and exported as
+ * C functions so that tests and the benchmark can drive the C++ expression API from
+ * any language. They play the role of the reference's guide/ and test/ programs
+ * (guide/neuralnet/convnet.cu:81-122 calls every one of these operations); each body
+ * is the line of mshadow code quoted in its comment.
+ *
+ * All pointers are DEVICE pointers owned by the caller; pitches in elements; `stream`
+ * is a handle from mshadow_hip_stream_create. `variant` 0 writes the expression on
+ * plain tensors (the library recognises it and runs the tuned kernel); variant 1 wraps
+ * the source in F<op::identity>() so that the same operation runs through the generic
+ * expression kernel instead. Return value: 0, or non-zero with the text available from
+ * mshadow_case_last_error() when a CHECK failed (DMLC_LOG_FATAL_THROW build).
+ */
+#ifndef MSHADOW_HIP_CASES_H_
+#define MSHADOW_HIP_CASES_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char *mshadow_case_last_error(void);
+
+/* dst <saver>= A * B + 0.5f * F<sigmoid>(C) - D        (saver: 0 = 1 += 2 -= 3 *= 4 /=) */
+int mshadow_case_map_fused_f32(float *dst, int dstride, const float *a, int astride,
+                               const float *b, int bstride, const float *c, int cstride,
+                               const float *d, int dstride_d, int rows, int cols, int saver,
+                               void *stream);
+/* dst <saver>= scalar */
+int mshadow_case_map_scalar_f32(float *dst, int dstride, int rows, int cols, float scalar,
+                                int saver, void *stream);
+/* dst <saver>= (A + s1) / s2 + s3 */
+int mshadow_case_map_axpb_f32(float *dst, int dstride, const float *a, int astride, int rows,
+                              int cols, float s1, float s2, float s3, int saver, void *stream);
+
+/* dst <saver>= scale * reduce_except_dim<1, Reducer>(src2d)   (sum_rows when Reducer = sum) */
+int mshadow_case_reduce_keep_lowest_f32(float *dst, const float *src, int sstride, int rows,
+                                        int cols, int reducer, int saver, float scale,
+                                        int variant, void *stream);
+/* dst <saver>= scale * reduce_except_dim<1, Reducer>(src4d)   (sumall_except_dim<1>) */
+int mshadow_case_reduce_keep_highdim_f32(float *dst, const float *src, int sstride, int n, int c,
+                                         int y, int x, int reducer, int saver, float scale,
+                                         int variant, void *stream);
+
+/* Softmax(dst, src) and SoftmaxGrad(dst, src, label) */
+int mshadow_case_softmax_f32(float *dst, int dstride, const float *src, int sstride, int rows,
+                             int cols, void *stream);
+int mshadow_case_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride,
+                                  const float *label, int rows, int cols, void *stream);
+
+/* dst = pool<Reducer>(src, Shape2(ph, pw), ky, kx, sy, sx) */
+int mshadow_case_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes,
+                          int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,
+                          int reducer, int variant, void *stream);
+/* dst = unpool<Reducer>(src, pooled, grad, ky, kx, sy, sx) */
+int mshadow_case_unpool_f32(float *dst, int dstride, const float *src, int sstride,
+                            const float *pooled, int pstride, const float *grad, int gstride,
+                            int planes, int h, int w, int ph, int pw, int ky, int kx, int sy,
+                            int sx, int reducer, int variant, void *stream);
+
+/* col = unpack_patch2col(pad(img, pad_y, pad_x), ky, kx, sy, sx, dy, dx) */
+int mshadow_case_im2col_f16(uint16_t *col, int cstride, const uint16_t *img, int istride, int n,
+                            int c, int h, int w, int ky, int kx, int sy, int sx, int dy, int dx,
+                            int pad_y, int pad_x, int variant, void *stream);
+int mshadow_case_im2col_f32(float *col, int cstride, const float *img, int istride, int n, int c,
+                            int h, int w, int ky, int kx, int sy, int sx, int dy, int dx,
+                            int pad_y, int pad_x, int variant, void *stream);
+/* img = crop(pack_col2patch(col, Shape4(n, c, h+2*pad_y, w+2*pad_x), ky, kx, sy, sx, dy, dx),
+              Shape2(h, w), pad_y, pad_x) */
+int mshadow_case_col2im_f16(uint16_t *img, int istride, const uint16_t *col, int cstride, int n,
+                            int c, int h, int w, int ky, int kx, int sy, int sx, int dy, int dx,
+                            int pad_y, int pad_x, int variant, void *stream);
+int mshadow_case_col2im_f32(float *img, int istride, const float *col, int cstride, int n, int c,
+                            int h, int w, int ky, int kx, int sy, int sx, int dy, int dx,
+                            int pad_y, int pad_x, int variant, void *stream);
+
+/* InitTensorEngine / NewStream / TensorContainer<gpu> / Copy (host -> device -> device ->
+   host) / DeleteStream on host buffers of rows x cols floats; *device_stride receives the
+   pitch AllocSpace chose with pad on or off. */
+int mshadow_case_copy_roundtrip_f32(float *host_out, const float *host_in, int rows, int cols,
+                                    int pad, int *device_stride);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MSHADOW_HIP_CASES_H_ */

@@ -1,0 +1,382 @@
+"""ctypes bindings of libmshadow_hip.so (include/mshadow_hip.h) and libmshadow_cases.so
+(include/mshadow_hip_cases.h).
+
+Nothing here computes: every operation is a call into the native library. Loading fails
+loudly when the library has not been built (run `python -c "import __graft_entry__ as g;
+g.build()"` or `python -m mshadow_amd.build`).
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+HIP_SO = os.path.join(HERE, "lib", "libmshadow_hip.so")
+CASES_SO = os.path.join(HERE, "lib", "libmshadow_cases.so")
+
+SAVETO, PLUSTO, MINUSTO, MULTO, DIVTO = range(5)
+SUM, MAX, MIN = range(3)
+H2D, D2H, D2D = 1, 2, 3
+
+_i, _f, _p, _sz = C.c_int, C.c_float, C.c_void_p, C.c_size_t
+
+
+class HipError(RuntimeError):
+    pass
+
+
+class Props(C.Structure):
+    _fields_ = [("name", C.c_char * 256), ("arch", C.c_char * 64), ("compute_units", _i),
+                ("wavefront_size", _i), ("max_threads_per_block", _i), ("clock_khz", _i),
+                ("memory_clock_khz", _i), ("memory_bus_bits", _i), ("l2_bytes", _i),
+                ("lds_bytes_per_block", _sz), ("total_global_mem", _sz)]
+
+
+# name -> argtypes, for every symbol include/mshadow_hip.h declares
+HIP_SYMBOLS = {
+    "mshadow_hip_last_error": ([], C.c_char_p),
+    "mshadow_hip_abi_version": ([], _i),
+    "mshadow_hip_device_count": ([C.POINTER(_i)], _i),
+    "mshadow_hip_set_device": ([_i], _i),
+    "mshadow_hip_get_device": ([C.POINTER(_i)], _i),
+    "mshadow_hip_get_props": ([_i, C.POINTER(Props)], _i),
+    "mshadow_hip_device_sync": ([], _i),
+    "mshadow_hip_stream_create": ([C.POINTER(_p)], _i),
+    "mshadow_hip_stream_destroy": ([_p], _i),
+    "mshadow_hip_stream_sync": ([_p], _i),
+    "mshadow_hip_stream_query": ([_p, C.POINTER(_i)], _i),
+    "mshadow_hip_event_create": ([C.POINTER(_p)], _i),
+    "mshadow_hip_event_destroy": ([_p], _i),
+    "mshadow_hip_event_record": ([_p, _p], _i),
+    "mshadow_hip_event_sync": ([_p], _i),
+    "mshadow_hip_event_elapsed_ms": ([_p, _p, C.POINTER(_f)], _i),
+    "mshadow_hip_malloc_pitch": ([C.POINTER(_p), C.POINTER(_sz), _sz, _sz], _i),
+    "mshadow_hip_malloc": ([C.POINTER(_p), _sz], _i),
+    "mshadow_hip_free": ([_p], _i),
+    "mshadow_hip_malloc_host": ([C.POINTER(_p), _sz], _i),
+    "mshadow_hip_free_host": ([_p], _i),
+    "mshadow_hip_memcpy2d_async": ([_p, _sz, _p, _sz, _sz, _sz, _i, _p], _i),
+    "mshadow_hip_memset_async": ([_p, _i, _sz, _p], _i),
+    "mshadow_hip_launch": ([_p, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(_p), _sz,
+                            _p], _i),
+    "mshadow_hip_peek_last_error": ([], _i),
+    "mshadow_hip_suggest_grid": ([_sz, _sz, _i, C.POINTER(C.c_uint32)], _i),
+    "mshadow_hip_softmax_f32": ([_p, _i, _p, _i, _i, _i, _p], _i),
+    "mshadow_hip_softmax_grad_f32": ([_p, _i, _p, _i, _p, _i, _i, _p], _i),
+    "mshadow_hip_reduce_keep_lowest_f32": ([_p, _p, _i, _i, _i, _i, _i, _f, _p], _i),
+    "mshadow_hip_reduce_keep_highdim_f32": ([_p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p], _i),
+    "mshadow_hip_pool_f32": ([_p, _i, _p, _i] + [_i] * 10 + [_p], _i),
+    "mshadow_hip_unpool_f32": ([_p, _i, _p, _i, _p, _i, _p, _i] + [_i] * 10 + [_p], _i),
+    "mshadow_hip_im2col_f16": ([_p, _i, _p, _i] + [_i] * 12 + [_p], _i),
+    "mshadow_hip_im2col_f32": ([_p, _i, _p, _i] + [_i] * 12 + [_p], _i),
+    "mshadow_hip_col2im_f16": ([_p, _i, _p, _i] + [_i] * 12 + [_p], _i),
+    "mshadow_hip_col2im_f32": ([_p, _i, _p, _i] + [_i] * 12 + [_p], _i),
+}
+
+CASES_SYMBOLS = {
+    "mshadow_case_last_error": ([], C.c_char_p),
+    "mshadow_case_map_fused_f32": ([_p, _i, _p, _i, _p, _i, _p, _i, _p, _i, _i, _i, _i, _p], _i),
+    "mshadow_case_map_scalar_f32": ([_p, _i, _i, _i, _f, _i, _p], _i),
+    "mshadow_case_map_axpb_f32": ([_p, _i, _p, _i, _i, _i, _f, _f, _f, _i, _p], _i),
+    "mshadow_case_reduce_keep_lowest_f32": ([_p, _p, _i, _i, _i, _i, _i, _f, _i, _p], _i),
+    "mshadow_case_reduce_keep_highdim_f32": ([_p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _i, _p], _i),
+    "mshadow_case_softmax_f32": ([_p, _i, _p, _i, _i, _i, _p], _i),
+    "mshadow_case_softmax_grad_f32": ([_p, _i, _p, _i, _p, _i, _i, _p], _i),
+    "mshadow_case_pool_f32": ([_p, _i, _p, _i] + [_i] * 11 + [_p], _i),
+    "mshadow_case_unpool_f32": ([_p, _i, _p, _i, _p, _i, _p, _i] + [_i] * 11 + [_p], _i),
+    "mshadow_case_im2col_f16": ([_p, _i, _p, _i] + [_i] * 13 + [_p], _i),
+    "mshadow_case_im2col_f32": ([_p, _i, _p, _i] + [_i] * 13 + [_p], _i),
+    "mshadow_case_col2im_f16": ([_p, _i, _p, _i] + [_i] * 13 + [_p], _i),
+    "mshadow_case_col2im_f32": ([_p, _i, _p, _i] + [_i] * 13 + [_p], _i),
+    "mshadow_case_copy_roundtrip_f32": ([_p, _p, _i, _i, _i, C.POINTER(_i)], _i),
+}
+
+
+def _bind(path, table):
+    if not os.path.exists(path):
+        raise HipError(f"{path} is not built; run `python -m mshadow_amd.build`")
+    dll = C.CDLL(path, mode=C.RTLD_GLOBAL)
+    for name, (argtypes, restype) in table.items():
+        fn = getattr(dll, name)  # AttributeError if the symbol is not exported
+        fn.argtypes = argtypes
+        fn.restype = restype
+    return dll
+
+
+class DeviceBuffer:
+    """A pitched 2-D allocation on the GPU holding an N-d array (rows = leading dims).
+
+    `pad` adds that many unused elements to every row (stride = cols + pad), which is how
+    tests exercise stride != cols. Uploads / downloads go through
+    mshadow_hip_memcpy2d_async on the given stream.
+    """
+
+    def __init__(self, library, shape, dtype, pad=0, fill=None):
+        self.lib = library
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = np.dtype(dtype)
+        self.cols = self.shape[-1] if self.shape else 1
+        self.rows = int(np.prod(self.shape[:-1])) if len(self.shape) > 1 else 1
+        self.stride = self.cols + int(pad)
+        self.nbytes = max(self.rows * self.stride * self.dtype.itemsize, 256)
+        ptr = _p()
+        library.check(library.dll.mshadow_hip_malloc(C.byref(ptr), self.nbytes))
+        self.ptr = ptr.value
+        if fill is not None:
+            library.check(library.dll.mshadow_hip_memset_async(self.ptr, fill, self.nbytes, None))
+            library.check(library.dll.mshadow_hip_stream_sync(None))
+
+    @classmethod
+    def from_array(cls, library, arr, pad=0, stream=None):
+        buf = cls(library, arr.shape, arr.dtype, pad)
+        buf.upload(arr, stream)
+        return buf
+
+    def upload(self, arr, stream=None):
+        arr = np.ascontiguousarray(arr, dtype=self.dtype)
+        assert arr.shape == self.shape, (arr.shape, self.shape)
+        it = self.dtype.itemsize
+        self.lib.check(self.lib.dll.mshadow_hip_memcpy2d_async(
+            self.ptr, self.stride * it, arr.ctypes.data, self.cols * it, self.cols * it,
+            self.rows, H2D, stream))
+        self.lib.check(self.lib.dll.mshadow_hip_stream_sync(stream))
+
+    def download(self, stream=None):
+        out = np.empty(self.shape, dtype=self.dtype)
+        it = self.dtype.itemsize
+        self.lib.check(self.lib.dll.mshadow_hip_memcpy2d_async(
+            out.ctypes.data, self.cols * it, self.ptr, self.stride * it, self.cols * it,
+            self.rows, D2H, stream))
+        self.lib.check(self.lib.dll.mshadow_hip_stream_sync(stream))
+        return out
+
+    def free(self):
+        if self.ptr:
+            self.lib.check(self.lib.dll.mshadow_hip_free(self.ptr))
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Library:
+    """Loaded libmshadow_hip.so (+ optionally libmshadow_cases.so) with error checking."""
+
+    def __init__(self, with_cases=False):
+        self.dll = _bind(HIP_SO, HIP_SYMBOLS)
+        self.cases = _bind(CASES_SO, CASES_SYMBOLS) if with_cases else None
+
+    # -- status handling
+    def check(self, status):
+        if status != 0:
+            raise HipError(self.dll.mshadow_hip_last_error().decode(errors="replace"))
+
+    def check_case(self, status):
+        if status != 0:
+            raise HipError(self.cases.mshadow_case_last_error().decode(errors="replace"))
+
+    # -- runtime
+    def device_count(self):
+        n = _i(0)
+        self.check(self.dll.mshadow_hip_device_count(C.byref(n)))
+        return n.value
+
+    def set_device(self, dev):
+        self.check(self.dll.mshadow_hip_set_device(dev))
+
+    def props(self, dev=0):
+        p = Props()
+        self.check(self.dll.mshadow_hip_get_props(dev, C.byref(p)))
+        return p
+
+    def stream_create(self):
+        s = _p()
+        self.check(self.dll.mshadow_hip_stream_create(C.byref(s)))
+        return s.value
+
+    def stream_destroy(self, s):
+        self.check(self.dll.mshadow_hip_stream_destroy(s))
+
+    def stream_sync(self, s=None):
+        self.check(self.dll.mshadow_hip_stream_sync(s))
+
+    def device_sync(self):
+        self.check(self.dll.mshadow_hip_device_sync())
+
+    def event_create(self):
+        e = _p()
+        self.check(self.dll.mshadow_hip_event_create(C.byref(e)))
+        return e.value
+
+    def event_destroy(self, e):
+        self.check(self.dll.mshadow_hip_event_destroy(e))
+
+    def event_record(self, e, s):
+        self.check(self.dll.mshadow_hip_event_record(e, s))
+
+    def event_sync(self, e):
+        self.check(self.dll.mshadow_hip_event_sync(e))
+
+    def elapsed_ms(self, start, stop):
+        ms = _f(0)
+        self.check(self.dll.mshadow_hip_event_elapsed_ms(start, stop, C.byref(ms)))
+        return ms.value
+
+    def buffer(self, shape, dtype, pad=0, fill=None):
+        return DeviceBuffer(self, shape, dtype, pad, fill)
+
+    def to_device(self, arr, pad=0, stream=None):
+        return DeviceBuffer.from_array(self, arr, pad, stream)
+
+    # -- fixed-function ops (DeviceBuffer arguments)
+    def softmax(self, dst, src, stream=None):
+        rows, cols = src.rows, src.cols
+        self.check(self.dll.mshadow_hip_softmax_f32(dst.ptr, dst.stride, src.ptr, src.stride, rows,
+                                                    cols, stream))
+
+    def softmax_grad(self, dst, src, label, stream=None):
+        self.check(self.dll.mshadow_hip_softmax_grad_f32(dst.ptr, dst.stride, src.ptr, src.stride,
+                                                         label.ptr, src.rows, src.cols, stream))
+
+    def reduce_keep_lowest(self, dst, src, reducer=SUM, saver=SAVETO, scale=1.0, stream=None):
+        self.check(self.dll.mshadow_hip_reduce_keep_lowest_f32(
+            dst.ptr, src.ptr, src.stride, src.rows, src.cols, reducer, saver, scale, stream))
+
+    def reduce_keep_highdim(self, dst, src, reducer=SUM, saver=SAVETO, scale=1.0, stream=None):
+        n, c, y, x = src.shape
+        self.check(self.dll.mshadow_hip_reduce_keep_highdim_f32(
+            dst.ptr, src.ptr, src.stride, n, c, y, x, reducer, saver, scale, stream))
+
+    def pool(self, dst, src, ky, kx, sy, sx, reducer=MAX, stream=None):
+        h, w = src.shape[-2:]
+        ph, pw = dst.shape[-2:]
+        planes = int(np.prod(src.shape[:-2]))
+        self.check(self.dll.mshadow_hip_pool_f32(dst.ptr, dst.stride, src.ptr, src.stride, planes,
+                                                 h, w, ph, pw, ky, kx, sy, sx, reducer, stream))
+
+    def unpool(self, dst, src, pooled, grad, ky, kx, sy, sx, reducer=MAX, stream=None):
+        h, w = src.shape[-2:]
+        ph, pw = pooled.shape[-2:]
+        planes = int(np.prod(src.shape[:-2]))
+        self.check(self.dll.mshadow_hip_unpool_f32(
+            dst.ptr, dst.stride, src.ptr, src.stride, pooled.ptr, pooled.stride, grad.ptr,
+            grad.stride, planes, h, w, ph, pw, ky, kx, sy, sx, reducer, stream))
+
+    def im2col(self, col, img, ky, kx, sy, sx, dy=1, dx=1, pad_y=0, pad_x=0, stream=None):
+        n, c, h, w = img.shape
+        fn = self.dll.mshadow_hip_im2col_f16 if img.dtype == np.uint16 else \
+            self.dll.mshadow_hip_im2col_f32
+        self.check(fn(col.ptr, col.stride, img.ptr, img.stride, n, c, h, w, ky, kx, sy, sx, dy, dx,
+                      pad_y, pad_x, stream))
+
+    def col2im(self, img, col, ky, kx, sy, sx, dy=1, dx=1, pad_y=0, pad_x=0, stream=None):
+        n, c, h, w = img.shape
+        fn = self.dll.mshadow_hip_col2im_f16 if img.dtype == np.uint16 else \
+            self.dll.mshadow_hip_col2im_f32
+        self.check(fn(img.ptr, img.stride, col.ptr, col.stride, n, c, h, w, ky, kx, sy, sx, dy, dx,
+                      pad_y, pad_x, stream))
+
+    # -- caller-style programs through the C++ expression API (libmshadow_cases)
+    def case_map_fused(self, dst, a, b, c, d, saver=SAVETO, stream=None):
+        self.check_case(self.cases.mshadow_case_map_fused_f32(
+            dst.ptr, dst.stride, a.ptr, a.stride, b.ptr, b.stride, c.ptr, c.stride, d.ptr,
+            d.stride, dst.rows, dst.cols, saver, stream))
+
+    def case_map_scalar(self, dst, scalar, saver=SAVETO, stream=None):
+        self.check_case(self.cases.mshadow_case_map_scalar_f32(dst.ptr, dst.stride, dst.rows,
+                                                               dst.cols, scalar, saver, stream))
+
+    def case_map_axpb(self, dst, a, s1, s2, s3, saver=SAVETO, stream=None):
+        self.check_case(self.cases.mshadow_case_map_axpb_f32(
+            dst.ptr, dst.stride, a.ptr, a.stride, dst.rows, dst.cols, s1, s2, s3, saver, stream))
+
+    def case_reduce_keep_lowest(self, dst, src, reducer=SUM, saver=SAVETO, scale=1.0, variant=0,
+                                stream=None):
+        self.check_case(self.cases.mshadow_case_reduce_keep_lowest_f32(
+            dst.ptr, src.ptr, src.stride, src.rows, src.cols, reducer, saver, scale, variant,
+            stream))
+
+    def case_reduce_keep_highdim(self, dst, src, reducer=SUM, saver=SAVETO, scale=1.0, variant=0,
+                                 stream=None):
+        n, c, y, x = src.shape
+        self.check_case(self.cases.mshadow_case_reduce_keep_highdim_f32(
+            dst.ptr, src.ptr, src.stride, n, c, y, x, reducer, saver, scale, variant, stream))
+
+    def case_softmax(self, dst, src, stream=None):
+        self.check_case(self.cases.mshadow_case_softmax_f32(dst.ptr, dst.stride, src.ptr,
+                                                            src.stride, src.rows, src.cols, stream))
+
+    def case_softmax_grad(self, dst, src, label, stream=None):
+        self.check_case(self.cases.mshadow_case_softmax_grad_f32(
+            dst.ptr, dst.stride, src.ptr, src.stride, label.ptr, src.rows, src.cols, stream))
+
+    def case_pool(self, dst, src, ky, kx, sy, sx, reducer=MAX, variant=0, stream=None):
+        h, w = src.shape[-2:]
+        ph, pw = dst.shape[-2:]
+        planes = int(np.prod(src.shape[:-2]))
+        self.check_case(self.cases.mshadow_case_pool_f32(
+            dst.ptr, dst.stride, src.ptr, src.stride, planes, h, w, ph, pw, ky, kx, sy, sx,
+            reducer, variant, stream))
+
+    def case_unpool(self, dst, src, pooled, grad, ky, kx, sy, sx, reducer=MAX, variant=0,
+                    stream=None):
+        h, w = src.shape[-2:]
+        ph, pw = pooled.shape[-2:]
+        planes = int(np.prod(src.shape[:-2]))
+        self.check_case(self.cases.mshadow_case_unpool_f32(
+            dst.ptr, dst.stride, src.ptr, src.stride, pooled.ptr, pooled.stride, grad.ptr,
+            grad.stride, planes, h, w, ph, pw, ky, kx, sy, sx, reducer, variant, stream))
+
+    def case_im2col(self, col, img, ky, kx, sy, sx, dy=1, dx=1, pad_y=0, pad_x=0, variant=0,
+                    stream=None):
+        n, c, h, w = img.shape
+        fn = self.cases.mshadow_case_im2col_f16 if img.dtype == np.uint16 else \
+            self.cases.mshadow_case_im2col_f32
+        self.check_case(fn(col.ptr, col.stride, img.ptr, img.stride, n, c, h, w, ky, kx, sy, sx,
+                           dy, dx, pad_y, pad_x, variant, stream))
+
+    def case_col2im(self, img, col, ky, kx, sy, sx, dy=1, dx=1, pad_y=0, pad_x=0, variant=0,
+                    stream=None):
+        n, c, h, w = img.shape
+        fn = self.cases.mshadow_case_col2im_f16 if img.dtype == np.uint16 else \
+            self.cases.mshadow_case_col2im_f32
+        self.check_case(fn(img.ptr, img.stride, col.ptr, col.stride, n, c, h, w, ky, kx, sy, sx,
+                           dy, dx, pad_y, pad_x, variant, stream))
+
+    def case_copy_roundtrip(self, arr, pad):
+        arr = np.ascontiguousarray(arr, dtype=np.float32)
+        out = np.empty_like(arr)
+        stride = _i(0)
+        self.check_case(self.cases.mshadow_case_copy_roundtrip_f32(
+            out.ctypes.data, arr.ctypes.data, arr.shape[0], arr.shape[1], int(pad),
+            C.byref(stride)))
+        return out, stride.value
+
+
+_lib = None
+_cases = None
+
+
+def load_lib():
+    global _lib
+    if _lib is None:
+        _lib = Library(with_cases=False)
+    return _lib
+
+
+def load_cases():
+    global _cases
+    if _cases is None:
+        _cases = Library(with_cases=True)
+    return _cases
+
+
+def lib():
+    return load_lib()
+
+
+def cases():
+    return load_cases()

@@ -1,0 +1,283 @@
+/*
+ * Caller-style programs against <mshadow/tensor.h>, exported as C (see
+ * include/mshadow_hip_cases.h). Everything below is ordinary mshadow user code: handles
+ * around existing memory, expressions, assignment. Built with DMLC_LOG_FATAL_THROW so a
+ * failed CHECK comes back as an error code instead of aborting the test process.
+ */
+#define DMLC_LOG_FATAL_THROW 1
+#include <mshadow/tensor.h>
+#include <mshadow_hip_cases.h>
+
+#include <string>
+
+#include "portable_math.h"
+
+using namespace mshadow;
+using namespace mshadow::expr;
+
+namespace {
+
+/* user functor, same shape as guide/neuralnet/nnet.cu:14-18 of the reference */
+struct sigmoid {
+  MSHADOW_XINLINE static float Map(float a) { return pmath_sigmoid(a); }
+};
+
+std::string &CaseError() {
+  static thread_local std::string msg;
+  return msg;
+}
+
+/* a Stream<gpu> object around a raw handle the caller owns */
+struct BorrowedStream {
+  Stream<gpu> s;
+  explicit BorrowedStream(void *handle) { s.stream_ = handle; }
+  Stream<gpu> *get() { return &s; }
+};
+
+template <typename T>
+Tensor<gpu, 2, T> G2(const T *p, int rows, int cols, int stride, Stream<gpu> *s) {
+  return Tensor<gpu, 2, T>(const_cast<T *>(p), Shape2(rows, cols), stride, s);
+}
+template <typename T>
+Tensor<gpu, 3, T> G3(const T *p, int a, int b, int c, int stride, Stream<gpu> *s) {
+  return Tensor<gpu, 3, T>(const_cast<T *>(p), Shape3(a, b, c), stride, s);
+}
+template <typename T>
+Tensor<gpu, 4, T> G4(const T *p, int n, int c, int h, int w, int stride, Stream<gpu> *s) {
+  return Tensor<gpu, 4, T>(const_cast<T *>(p), Shape4(n, c, h, w), stride, s);
+}
+template <typename T>
+Tensor<gpu, 1, T> G1(const T *p, int n, Stream<gpu> *s) {
+  return Tensor<gpu, 1, T>(const_cast<T *>(p), Shape1(n), s);
+}
+
+template <typename Dst, typename E>
+void Assign(Dst dst, const E &e, int saver) {
+  switch (saver) {
+    case 0: dst = e; break;
+    case 1: dst += e; break;
+    case 2: dst -= e; break;
+    case 3: dst *= e; break;
+    default: dst /= e; break;
+  }
+}
+
+template <typename Reducer, typename Src>
+void ReduceInto(Tensor<gpu, 1, float> dst, const Src &src, int saver, float scale) {
+  Assign(dst, scale * reduce_except_dim<1, Reducer>(src), saver);
+}
+template <typename Src>
+void ReduceDispatch(Tensor<gpu, 1, float> dst, const Src &src, int reducer, int saver,
+                    float scale) {
+  if (reducer == 0) ReduceInto<red::sum>(dst, src, saver, scale);
+  else if (reducer == 1) ReduceInto<red::maximum>(dst, src, saver, scale);
+  else ReduceInto<red::minimum>(dst, src, saver, scale);
+}
+
+}  // namespace
+
+#define CASE_BEGIN try {
+#define CASE_END                          \
+  }                                       \
+  catch (const std::exception &e) {       \
+    CaseError() = e.what();               \
+    return 1;                             \
+  }                                       \
+  return 0;
+
+extern "C" {
+
+const char *mshadow_case_last_error(void) { return CaseError().c_str(); }
+
+int mshadow_case_map_fused_f32(float *dst, int dstride, const float *a, int astride,
+                               const float *b, int bstride, const float *c, int cstride,
+                               const float *d, int dstride_d, int rows, int cols, int saver,
+                               void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Tensor<gpu, 2, float> A = G2(a, rows, cols, astride, st.get()),
+                        B = G2(b, rows, cols, bstride, st.get()),
+                        C = G2(c, rows, cols, cstride, st.get()),
+                        D = G2(d, rows, cols, dstride_d, st.get());
+  Assign(G2(dst, rows, cols, dstride, st.get()), A * B + 0.5f * F<sigmoid>(C) - D, saver);
+  CASE_END
+}
+
+int mshadow_case_map_scalar_f32(float *dst, int dstride, int rows, int cols, float scalar,
+                                int saver, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Tensor<gpu, 2, float> o = G2(dst, rows, cols, dstride, st.get());
+  switch (saver) {
+    case 0: o = scalar; break;
+    case 1: o += scalar; break;
+    case 2: o -= scalar; break;
+    case 3: o *= scalar; break;
+    default: o /= scalar; break;
+  }
+  CASE_END
+}
+
+int mshadow_case_map_axpb_f32(float *dst, int dstride, const float *a, int astride, int rows,
+                              int cols, float s1, float s2, float s3, int saver, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Tensor<gpu, 2, float> A = G2(a, rows, cols, astride, st.get());
+  Assign(G2(dst, rows, cols, dstride, st.get()), (A + s1) / s2 + s3, saver);
+  CASE_END
+}
+
+int mshadow_case_reduce_keep_lowest_f32(float *dst, const float *src, int sstride, int rows,
+                                        int cols, int reducer, int saver, float scale,
+                                        int variant, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Tensor<gpu, 2, float> S = G2(src, rows, cols, sstride, st.get());
+  Tensor<gpu, 1, float> o = G1(dst, cols, st.get());
+  if (variant == 0) ReduceDispatch(o, S, reducer, saver, scale);
+  else ReduceDispatch(o, F<op::identity>(S), reducer, saver, scale);
+  CASE_END
+}
+
+int mshadow_case_reduce_keep_highdim_f32(float *dst, const float *src, int sstride, int n, int c,
+                                         int y, int x, int reducer, int saver, float scale,
+                                         int variant, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Tensor<gpu, 4, float> S = G4(src, n, c, y, x, sstride, st.get());
+  Tensor<gpu, 1, float> o = G1(dst, c, st.get());
+  if (variant == 0) ReduceDispatch(o, S, reducer, saver, scale);
+  else ReduceDispatch(o, F<op::identity>(S), reducer, saver, scale);
+  CASE_END
+}
+
+int mshadow_case_softmax_f32(float *dst, int dstride, const float *src, int sstride, int rows,
+                             int cols, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Softmax(G2(dst, rows, cols, dstride, st.get()), G2(src, rows, cols, sstride, st.get()));
+  CASE_END
+}
+
+int mshadow_case_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride,
+                                  const float *label, int rows, int cols, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  SoftmaxGrad(G2(dst, rows, cols, dstride, st.get()), G2(src, rows, cols, sstride, st.get()),
+              G1(label, rows, st.get()));
+  CASE_END
+}
+
+int mshadow_case_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes,
+                          int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,
+                          int reducer, int variant, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Tensor<gpu, 3, float> S = G3(src, planes, h, w, sstride, st.get());
+  Tensor<gpu, 3, float> o = G3(dst, planes, ph, pw, dstride, st.get());
+  const Shape<2> ps = Shape2(ph, pw);
+  if (variant == 0) {
+    if (reducer == 0) o = pool<red::sum>(S, ps, ky, kx, sy, sx);
+    else if (reducer == 1) o = pool<red::maximum>(S, ps, ky, kx, sy, sx);
+    else o = pool<red::minimum>(S, ps, ky, kx, sy, sx);
+  } else {
+    if (reducer == 0) o = pool<red::sum>(F<op::identity>(S), ps, ky, kx, sy, sx);
+    else if (reducer == 1) o = pool<red::maximum>(F<op::identity>(S), ps, ky, kx, sy, sx);
+    else o = pool<red::minimum>(F<op::identity>(S), ps, ky, kx, sy, sx);
+  }
+  CASE_END
+}
+
+int mshadow_case_unpool_f32(float *dst, int dstride, const float *src, int sstride,
+                            const float *pooled, int pstride, const float *grad, int gstride,
+                            int planes, int h, int w, int ph, int pw, int ky, int kx, int sy,
+                            int sx, int reducer, int variant, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Tensor<gpu, 3, float> S = G3(src, planes, h, w, sstride, st.get());
+  Tensor<gpu, 3, float> P = G3(pooled, planes, ph, pw, pstride, st.get());
+  Tensor<gpu, 3, float> Gd = G3(grad, planes, ph, pw, gstride, st.get());
+  Tensor<gpu, 3, float> o = G3(dst, planes, h, w, dstride, st.get());
+  if (variant == 0) {
+    if (reducer == 0) o = unpool<red::sum>(S, P, Gd, ky, kx, sy, sx);
+    else if (reducer == 1) o = unpool<red::maximum>(S, P, Gd, ky, kx, sy, sx);
+    else o = unpool<red::minimum>(S, P, Gd, ky, kx, sy, sx);
+  } else {
+    if (reducer == 0) {
+      o = unpool<red::sum>(F<op::identity>(S), F<op::identity>(P), F<op::identity>(Gd), ky, kx, sy, sx);
+    } else if (reducer == 1) {
+      o = unpool<red::maximum>(F<op::identity>(S), F<op::identity>(P), F<op::identity>(Gd), ky, kx, sy, sx);
+    } else {
+      o = unpool<red::minimum>(F<op::identity>(S), F<op::identity>(P), F<op::identity>(Gd), ky, kx, sy, sx);
+    }
+  }
+  CASE_END
+}
+
+#define CASE_IM2COL(NAME, CT, MT)                                                                \
+  int NAME(CT *col, int cstride, const CT *img, int istride, int n, int c, int h, int w, int ky, \
+           int kx, int sy, int sx, int dy, int dx, int pad_y, int pad_x, int variant,            \
+           void *stream) {                                                                       \
+    CASE_BEGIN                                                                                   \
+    BorrowedStream st(stream);                                                                   \
+    const int hp = h + 2 * pad_y, wp = w + 2 * pad_x;                                            \
+    const int oh = (hp - (dy * (ky - 1) + 1)) / sy + 1, ow = (wp - (dx * (kx - 1) + 1)) / sx + 1; \
+    Tensor<gpu, 4, MT> I = G4(reinterpret_cast<const MT *>(img), n, c, h, w, istride, st.get()); \
+    Tensor<gpu, 2, MT> O =                                                                       \
+        G2(reinterpret_cast<MT *>(col), ky * kx * c, oh * ow * n, cstride, st.get());            \
+    if (variant == 0) O = unpack_patch2col(pad(I, pad_y, pad_x), ky, kx, sy, sx, dy, dx);        \
+    else O = unpack_patch2col(pad(F<op::identity>(I), pad_y, pad_x), ky, kx, sy, sx, dy, dx);    \
+    CASE_END                                                                                     \
+  }
+CASE_IM2COL(mshadow_case_im2col_f16, uint16_t, half::half_t)
+CASE_IM2COL(mshadow_case_im2col_f32, float, float)
+
+#define CASE_COL2IM(NAME, CT, MT)                                                                \
+  int NAME(CT *img, int istride, const CT *col, int cstride, int n, int c, int h, int w, int ky, \
+           int kx, int sy, int sx, int dy, int dx, int pad_y, int pad_x, int variant,            \
+           void *stream) {                                                                       \
+    CASE_BEGIN                                                                                   \
+    BorrowedStream st(stream);                                                                   \
+    const int hp = h + 2 * pad_y, wp = w + 2 * pad_x;                                            \
+    const int oh = (hp - (dy * (ky - 1) + 1)) / sy + 1, ow = (wp - (dx * (kx - 1) + 1)) / sx + 1; \
+    Tensor<gpu, 4, MT> I = G4(reinterpret_cast<MT *>(img), n, c, h, w, istride, st.get());       \
+    Tensor<gpu, 2, MT> C =                                                                       \
+        G2(reinterpret_cast<const MT *>(col), ky * kx * c, oh * ow * n, cstride, st.get());      \
+    if (variant == 0) {                                                                          \
+      I = crop(pack_col2patch(C, Shape4(n, c, hp, wp), ky, kx, sy, sx, dy, dx), Shape2(h, w),    \
+               pad_y, pad_x);                                                                    \
+    } else {                                                                                     \
+      I = crop(pack_col2patch(F<op::identity>(C), Shape4(n, c, hp, wp), ky, kx, sy, sx, dy, dx), \
+               Shape2(h, w), pad_y, pad_x);                                                      \
+    }                                                                                            \
+    CASE_END                                                                                     \
+  }
+CASE_COL2IM(mshadow_case_col2im_f16, uint16_t, half::half_t)
+CASE_COL2IM(mshadow_case_col2im_f32, float, float)
+
+int mshadow_case_copy_roundtrip_f32(float *host_out, const float *host_in, int rows, int cols,
+                                    int pad, int *device_stride) {
+  CASE_BEGIN
+  InitTensorEngine<gpu>(0);
+  Stream<gpu> *stream = NewStream<gpu>(0);
+  {
+    Tensor<cpu, 2, float> hin(const_cast<float *>(host_in), Shape2(rows, cols));
+    Tensor<cpu, 2, float> hout(host_out, Shape2(rows, cols));
+    TensorContainer<gpu, 2, float> a(pad != 0), b(pad != 0);
+    a.set_stream(stream);
+    b.set_stream(stream);
+    a.Resize(Shape2(rows, cols));
+    b.Resize(Shape2(rows, cols));
+    if (device_stride != NULL) *device_stride = a.stride_;
+    Copy(a, hin, stream);
+    Copy(b, a, stream);
+    b += 0.0f;  // an expression on a possibly pitched container
+    Copy(hout, b, stream);
+    stream->Wait();
+  }
+  DeleteStream(stream);
+  ShutdownTensorEngine<gpu>();
+  CASE_END
+}
+
+}  // extern "C"

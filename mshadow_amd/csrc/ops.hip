@@ -1,0 +1,359 @@
+/*
+ * C ABI, group 3: fixed-function operations on plain (pointer, pitch, shape) arguments.
+ * Each entry validates its arguments on the host (a kernel is never launched on shapes
+ * it does not cover), picks the kernel variant from shape and alignment, queues it on
+ * the caller's stream and reports launch errors. See include/mshadow_hip.h.
+ */
+#include "abi_common.h"
+
+#include <mshadow/hip/kernels/reduce.h>
+
+#include "patch_kernels.h"
+#include "pool_kernels.h"
+#include "softmax_kernels.h"
+
+using namespace mshadow_abi;
+using namespace mshadow_hipk;
+
+namespace {
+
+/* minimal evaluators with the Plan interface the kernel templates expect */
+template <typename T>
+struct RawPlan2D {
+  T *p;
+  int stride;
+  __device__ T &REval(unsigned y, unsigned x) { return p[static_cast<size_t>(y) * stride + x]; }
+  __device__ const T &Eval(unsigned y, unsigned x) const {
+    return p[static_cast<size_t>(y) * stride + x];
+  }
+};
+template <typename T>
+struct RawPlan1D {
+  T *p;
+  __device__ T &REval(unsigned, unsigned x) { return p[x]; }
+  __device__ const T &Eval(unsigned, unsigned x) const { return p[x]; }
+};
+
+inline bool Aligned16(const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
+template <typename F>
+int DispatchSaver(int saver, F f) {
+  switch (saver) {
+    case MSHADOW_HIP_SAVETO: return f(mshadow::sv::saveto());
+    case MSHADOW_HIP_PLUSTO: return f(mshadow::sv::plusto());
+    case MSHADOW_HIP_MINUSTO: return f(mshadow::sv::minusto());
+    case MSHADOW_HIP_MULTO: return f(mshadow::sv::multo());
+    case MSHADOW_HIP_DIVTO: return f(mshadow::sv::divto());
+    default: return Fail(MSHADOW_HIP_ERR_ARGUMENT, "unknown saver");
+  }
+}
+template <typename F>
+int DispatchReducer(int reducer, F f) {
+  switch (reducer) {
+    case MSHADOW_HIP_SUM: return f(mshadow::red::sum());
+    case MSHADOW_HIP_MAX: return f(mshadow::red::maximum());
+    case MSHADOW_HIP_MIN: return f(mshadow::red::minimum());
+    default: return Fail(MSHADOW_HIP_ERR_ARGUMENT, "unknown reducer");
+  }
+}
+
+}  // namespace
+
+namespace {
+int MakePatchGeom(PatchGeom *g, int n, int c, int h, int w, int ky, int kx, int sy, int sx,
+                  int dy, int dx, int pad_y, int pad_x) {
+  if (n < 0 || c < 0 || h < 0 || w < 0) return Fail(MSHADOW_HIP_ERR_ARGUMENT, "negative shape");
+  if (ky < 1 || kx < 1 || sy < 1 || sx < 1 || dy < 1 || dx < 1 || pad_y < 0 || pad_x < 0) {
+    return Fail(MSHADOW_HIP_ERR_ARGUMENT, "kernel, stride, dilation must be >= 1, pad >= 0");
+  }
+  const int hp = h + 2 * pad_y, wp = w + 2 * pad_x;
+  if (hp < ky || wp < kx || hp < dy * (ky - 1) + 1 || wp < dx * (kx - 1) + 1) {
+    return Fail(MSHADOW_HIP_ERR_ARGUMENT, "image shape smaller than patch size");
+  }
+  g->n = n; g->c = c; g->h = h; g->w = w;
+  g->ky = ky; g->kx = kx; g->sy = sy; g->sx = sx; g->dy = dy; g->dx = dx;
+  g->pad_y = pad_y; g->pad_x = pad_x; g->hp = hp; g->wp = wp;
+  g->oh = (hp - (dy * (ky - 1) + 1)) / sy + 1;
+  g->ow = (wp - (dx * (kx - 1) + 1)) / sx + 1;
+  const long long rows = static_cast<long long>(ky) * kx * c;
+  const long long cols = static_cast<long long>(n) * g->oh * g->ow;
+  if (rows >= (1ll << 31) || cols >= (1ll << 31) ||
+      static_cast<long long>(n) * c * h >= (1ll << 31) ||
+      static_cast<long long>(n) * c * h * w >= (1ll << 32)) {
+    return Fail(MSHADOW_HIP_ERR_ARGUMENT, "too large for 32-bit indices");
+  }
+  return MSHADOW_HIP_OK;
+}
+
+template <typename T>
+int Im2Col(T *col, int cstride, const T *img, int istride, const PatchGeom &g, void *stream) {
+  const long long rows = static_cast<long long>(g.ky) * g.kx * g.c;
+  const long long cols = static_cast<long long>(g.n) * g.oh * g.ow;
+  if (rows == 0 || cols == 0) return MSHADOW_HIP_OK;
+  if (col == NULL || img == NULL) return Fail(MSHADOW_HIP_ERR_ARGUMENT, "im2col: NULL tensor");
+  if (cstride < cols || istride < g.w) {
+    return Fail(MSHADOW_HIP_ERR_ARGUMENT, "im2col: pitch smaller than the row");
+  }
+  const int EPT = 16 / sizeof(T);
+  const unsigned chunks = static_cast<unsigned>((cols + kPatchBlock * EPT - 1) / (kPatchBlock * EPT));
+  const long long blocks = rows * chunks;
+  if (blocks >= (1ll << 31)) return Fail(MSHADOW_HIP_ERR_ARGUMENT, "im2col: too many workgroups");
+  hipLaunchKernelGGL((Im2ColKernel<T, EPT>), dim3(static_cast<unsigned>(blocks)),
+                     dim3(kPatchBlock), 0, AsStream(stream), col, cstride, img, istride, g, chunks);
+  return AfterLaunch("im2col");
+}
+
+template <typename T>
+int Col2Im(T *img, int istride, const T *col, int cstride, const PatchGeom &g, void *stream) {
+  const long long cols = static_cast<long long>(g.n) * g.oh * g.ow;
+  const long long total = static_cast<long long>(g.n) * g.c * g.h * g.w;
+  if (total == 0) return MSHADOW_HIP_OK;
+  if (col == NULL || img == NULL) return Fail(MSHADOW_HIP_ERR_ARGUMENT, "col2im: NULL tensor");
+  if (cstride < cols || istride < g.w) {
+    return Fail(MSHADOW_HIP_ERR_ARGUMENT, "col2im: pitch smaller than the row");
+  }
+  unsigned grid = 0;
+  int st = mshadow_hip_suggest_grid(static_cast<size_t>(total), kPatchBlock, 8, &grid);
+  if (st != MSHADOW_HIP_OK) return st;
+  hipLaunchKernelGGL((Col2ImKernel<T>), dim3(grid), dim3(kPatchBlock), 0, AsStream(stream), img,
+                     istride, col, cstride, g, static_cast<unsigned>(total));
+  return AfterLaunch("col2im");
+}
+}  // namespace
+
+
+extern "C" {
+
+/* ------------------------------------------------------------------ softmax */
+
+int mshadow_hip_softmax_f32(float *dst, int dstride, const float *src, int sstride, int rows,
+                            int cols, void *stream) {
+  ABI_REQUIRE(rows >= 0 && cols >= 0, "negative shape");
+  if (rows == 0 || cols == 0) return MSHADOW_HIP_OK;
+  ABI_REQUIRE(dst != NULL && src != NULL, "NULL tensor");
+  ABI_REQUIRE(dstride >= cols && sstride >= cols, "pitch smaller than the row");
+  hipStream_t s = AsStream(stream);
+  const bool vec = Aligned16(dst) && Aligned16(src) && dstride % 4 == 0 && sstride % 4 == 0;
+#define SOFTMAX_LAUNCH(T, S, V) \
+  hipLaunchKernelGGL((SoftmaxRowKernel<T, S, V>), dim3(rows), dim3(T), 0, s, dst, dstride, src, \
+                     sstride, cols)
+  if (vec) {
+    if (cols <= 1024) SOFTMAX_LAUNCH(256, 1, 4);
+    else if (cols <= 2048) SOFTMAX_LAUNCH(256, 2, 4);
+    else if (cols <= 4096) SOFTMAX_LAUNCH(256, 4, 4);
+    else if (cols <= 8192) SOFTMAX_LAUNCH(256, 8, 4);
+    else if (cols <= 16384) SOFTMAX_LAUNCH(512, 8, 4);
+    else if (cols <= 32768) SOFTMAX_LAUNCH(512, 16, 4);
+    else if (cols <= 65536) SOFTMAX_LAUNCH(1024, 16, 4);
+    else hipLaunchKernelGGL((SoftmaxLongRowKernel<1024>), dim3(rows), dim3(1024), 0, s, dst,
+                            dstride, src, sstride, cols);
+  } else {
+    if (cols <= 1024) SOFTMAX_LAUNCH(256, 4, 1);
+    else if (cols <= 4096) SOFTMAX_LAUNCH(256, 16, 1);
+    else if (cols <= 16384) SOFTMAX_LAUNCH(1024, 16, 1);
+    else hipLaunchKernelGGL((SoftmaxLongRowKernel<1024>), dim3(rows), dim3(1024), 0, s, dst,
+                            dstride, src, sstride, cols);
+  }
+#undef SOFTMAX_LAUNCH
+  return AfterLaunch("softmax");
+}
+
+int mshadow_hip_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride,
+                                 const float *label, int rows, int cols, void *stream) {
+  ABI_REQUIRE(rows >= 0 && cols >= 0, "negative shape");
+  if (rows == 0 || cols == 0) return MSHADOW_HIP_OK;
+  ABI_REQUIRE(dst != NULL && src != NULL && label != NULL, "NULL tensor");
+  ABI_REQUIRE(dstride >= cols && sstride >= cols, "pitch smaller than the row");
+  const int per_block = kGradBlock * kGradPacks * 4;
+  const unsigned chunks = (cols + per_block - 1) / per_block;
+  ABI_REQUIRE(chunks <= 65535u, "row too long");
+  const bool vec = Aligned16(dst) && Aligned16(src) && dstride % 4 == 0 && sstride % 4 == 0;
+  if (vec) {
+    hipLaunchKernelGGL((SoftmaxGradKernel<true>), dim3(rows, chunks), dim3(kGradBlock), 0,
+                       AsStream(stream), dst, dstride, src, sstride, label, cols);
+  } else {
+    hipLaunchKernelGGL((SoftmaxGradKernel<false>), dim3(rows, chunks), dim3(kGradBlock), 0,
+                       AsStream(stream), dst, dstride, src, sstride, label, cols);
+  }
+  return AfterLaunch("softmax_grad");
+}
+
+/* ------------------------------------------------------------------ reductions */
+
+int mshadow_hip_reduce_keep_lowest_f32(float *dst, const float *src, int sstride, int rows,
+                                       int cols, int reducer, int saver, float scale,
+                                       void *stream) {
+  ABI_REQUIRE(rows >= 1, "can not reduce over empty tensor");
+  ABI_REQUIRE(cols >= 0, "negative shape");
+  if (cols == 0) return MSHADOW_HIP_OK;
+  ABI_REQUIRE(dst != NULL && src != NULL, "NULL tensor");
+  ABI_REQUIRE(sstride >= cols, "pitch smaller than the row");
+  RawPlan1D<float> d = {dst};
+  RawPlan2D<const float> sp = {src, sstride};
+  const unsigned grid = (cols + mshadow::hip::kLowestCols - 1) / mshadow::hip::kLowestCols;
+  hipStream_t s = AsStream(stream);
+  int st = DispatchReducer(reducer, [&](auto red) {
+    return DispatchSaver(saver, [&](auto sv) {
+      typedef decltype(red) R;
+      typedef decltype(sv) S;
+      hipLaunchKernelGGL((mshadow::hip::ReduceKeepLowestKernel<S, R, float, RawPlan1D<float>,
+                                                               RawPlan2D<const float> >),
+                         dim3(grid), dim3(mshadow::hip::kRedBlock), 0, s, d, sp,
+                         static_cast<uint32_t>(rows), static_cast<uint32_t>(cols), scale);
+      return MSHADOW_HIP_OK;
+    });
+  });
+  if (st != MSHADOW_HIP_OK) return st;
+  return AfterLaunch("reduce_keep_lowest");
+}
+
+int mshadow_hip_reduce_keep_highdim_f32(float *dst, const float *src, int sstride, int n, int c,
+                                        int y, int x, int reducer, int saver, float scale,
+                                        void *stream) {
+  ABI_REQUIRE(n >= 0 && c >= 0 && y >= 0 && x >= 0, "negative shape");
+  if (c == 0) return MSHADOW_HIP_OK;
+  ABI_REQUIRE(dst != NULL, "NULL tensor");
+  ABI_REQUIRE(src != NULL || static_cast<long long>(n) * y * x == 0, "NULL tensor");
+  ABI_REQUIRE(sstride >= x, "pitch smaller than the row");
+  ABI_REQUIRE(static_cast<long long>(n) * c * y < (1ll << 31), "too many rows for 32-bit indices");
+  RawPlan1D<float> d = {dst};
+  RawPlan2D<const float> sp = {src, sstride};
+  hipStream_t s = AsStream(stream);
+  int st = DispatchReducer(reducer, [&](auto red) {
+    return DispatchSaver(saver, [&](auto sv) {
+      typedef decltype(red) R;
+      typedef decltype(sv) S;
+#define HIGHDIM_LAUNCH(SEGS)                                                                   \
+  hipLaunchKernelGGL((mshadow::hip::ReduceKeepHighDimKernel<S, R, float, SEGS, RawPlan1D<float>, \
+                                                            RawPlan2D<const float> >),         \
+                     dim3(c), dim3(mshadow::hip::kRedBlock), 0, s, d, sp,                      \
+                     static_cast<uint32_t>(n), static_cast<uint32_t>(c),                       \
+                     static_cast<uint32_t>(y), static_cast<uint32_t>(x), scale)
+      if (n > 16) HIGHDIM_LAUNCH(64);
+      else if (n > 4) HIGHDIM_LAUNCH(16);
+      else if (n > 1) HIGHDIM_LAUNCH(4);
+      else HIGHDIM_LAUNCH(1);
+#undef HIGHDIM_LAUNCH
+      return MSHADOW_HIP_OK;
+    });
+  });
+  if (st != MSHADOW_HIP_OK) return st;
+  return AfterLaunch("reduce_keep_highdim");
+}
+
+/* ------------------------------------------------------------------ pool / unpool */
+
+static const size_t kPoolLdsBudget = 48 * 1024;  // per workgroup: three resident per CU
+
+int mshadow_hip_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes,
+                         int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,
+                         int reducer, void *stream) {
+  ABI_REQUIRE(planes >= 0 && h >= 0 && w >= 0 && ph >= 0 && pw >= 0, "negative shape");
+  ABI_REQUIRE(ky >= 1 && kx >= 1 && sy >= 1 && sx >= 1, "kernel and stride must be positive");
+  ABI_REQUIRE(h >= ky && w >= kx, "kernel must be smaller than image");
+  ABI_REQUIRE(reducer >= MSHADOW_HIP_SUM && reducer <= MSHADOW_HIP_MIN, "unknown reducer");
+  if (planes == 0 || ph == 0 || pw == 0) return MSHADOW_HIP_OK;
+  ABI_REQUIRE(dst != NULL && src != NULL, "NULL tensor");
+  ABI_REQUIRE(dstride >= pw && sstride >= w, "pitch smaller than the row");
+  ABI_REQUIRE(static_cast<long long>(planes) * h < (1ll << 31) &&
+                  static_cast<long long>(planes) * ph * pw < (1ll << 32),
+              "too large for 32-bit indices");
+  PoolGeom g = {h, w, ph, pw, ky, kx, sy, sx, 0, 0, w + 1};
+  hipStream_t s = AsStream(stream);
+  const size_t row_bytes = static_cast<size_t>(g.lds_pitch) * sizeof(float);
+  /* output rows per band so that (band - 1) * sy + ky input rows fit the budget */
+  long long max_in_rows = static_cast<long long>(kPoolLdsBudget / row_bytes);
+  long long band = max_in_rows >= ky ? (max_in_rows - ky) / sy + 1 : 0;
+  if (band > ph) band = ph;
+  /* keep at least ~4 workgroups per CU in flight when planes are few */
+  while (band > 8 && static_cast<long long>(planes) * ((ph + band - 1) / band) < 1024) {
+    band = (band + 1) / 2;
+  }
+#define POOL_SWITCH(KERNEL, ...)                                                               \
+  switch (reducer) {                                                                           \
+    case MSHADOW_HIP_SUM: hipLaunchKernelGGL((KERNEL<MSHADOW_HIP_SUM>), __VA_ARGS__); break;    \
+    case MSHADOW_HIP_MAX: hipLaunchKernelGGL((KERNEL<MSHADOW_HIP_MAX>), __VA_ARGS__); break;    \
+    default: hipLaunchKernelGGL((KERNEL<MSHADOW_HIP_MIN>), __VA_ARGS__); break;                 \
+  }
+  if (band >= 1) {
+    g.band = static_cast<int>(band);
+    g.bands = (ph + g.band - 1) / g.band;
+    const size_t lds = (static_cast<size_t>(g.band - 1) * sy + ky) * row_bytes;
+    const long long blocks = static_cast<long long>(planes) * g.bands;
+    ABI_REQUIRE(blocks < (1ll << 31), "too many workgroups");
+    POOL_SWITCH(PoolKernel, dim3(static_cast<unsigned>(blocks)), dim3(kPoolBlock), lds, s, dst,
+                dstride, src, sstride, g)
+  } else {
+    const unsigned total = static_cast<unsigned>(planes) * ph * pw;
+    unsigned grid = 0;
+    int st = mshadow_hip_suggest_grid(total, kPoolBlock, 4, &grid);
+    if (st != MSHADOW_HIP_OK) return st;
+    POOL_SWITCH(PoolDirectKernel, dim3(grid), dim3(kPoolBlock), 0, s, dst, dstride, src, sstride,
+                g, total)
+  }
+  return AfterLaunch("pool");
+}
+
+int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstride,
+                           const float *pooled, int pstride, const float *grad, int gstride,
+                           int planes, int h, int w, int ph, int pw, int ky, int kx, int sy,
+                           int sx, int reducer, void *stream) {
+  ABI_REQUIRE(planes >= 0 && h >= 0 && w >= 0 && ph >= 0 && pw >= 0, "negative shape");
+  ABI_REQUIRE(ky >= 1 && kx >= 1 && sy >= 1 && sx >= 1, "kernel and stride must be positive");
+  ABI_REQUIRE(reducer >= MSHADOW_HIP_SUM && reducer <= MSHADOW_HIP_MIN, "unknown reducer");
+  if (planes == 0 || h == 0 || w == 0) return MSHADOW_HIP_OK;
+  ABI_REQUIRE(dst != NULL && src != NULL, "NULL tensor");
+  ABI_REQUIRE((pooled != NULL && grad != NULL) || ph == 0 || pw == 0, "NULL tensor");
+  ABI_REQUIRE(dstride >= w && sstride >= w && pstride >= pw && gstride >= pw,
+              "pitch smaller than the row");
+  ABI_REQUIRE(static_cast<long long>(planes) * h * w < (1ll << 32) &&
+                  static_cast<long long>(planes) * h < (1ll << 31),
+              "too large for 32-bit indices");
+  PoolGeom g = {h, w, ph, pw, ky, kx, sy, sx, 0, 0, pw + 1};
+  hipStream_t s = AsStream(stream);
+  const size_t row_bytes = static_cast<size_t>(g.lds_pitch) * sizeof(float) * 2;  // pooled + grad
+  /* source rows per band: prow_max = (band + ky - 2) / sy + 2 pooled rows must fit */
+  long long max_prow = static_cast<long long>(kPoolLdsBudget / row_bytes);
+  long long band = (max_prow - 2) * sy - ky + 2;
+  if (band > h) band = h;
+  while (band > 8 && static_cast<long long>(planes) * ((h + band - 1) / band) < 1024) {
+    band = (band + 1) / 2;
+  }
+  if (band >= 1 && max_prow >= 3) {
+    g.band = static_cast<int>(band);
+    g.bands = (h + g.band - 1) / g.band;
+    const int prow_max = (g.band + ky - 2) / sy + 2;
+    const size_t lds = static_cast<size_t>(prow_max) * row_bytes;
+    const long long blocks = static_cast<long long>(planes) * g.bands;
+    ABI_REQUIRE(blocks < (1ll << 31), "too many workgroups");
+    POOL_SWITCH(UnpoolKernel, dim3(static_cast<unsigned>(blocks)), dim3(kPoolBlock), lds, s, dst,
+                dstride, src, sstride, pooled, pstride, grad, gstride, g, prow_max)
+  } else {
+    const unsigned total = static_cast<unsigned>(planes) * h * w;
+    unsigned grid = 0;
+    int st = mshadow_hip_suggest_grid(total, kPoolBlock, 4, &grid);
+    if (st != MSHADOW_HIP_OK) return st;
+    POOL_SWITCH(UnpoolDirectKernel, dim3(grid), dim3(kPoolBlock), 0, s, dst, dstride, src,
+                sstride, pooled, pstride, grad, gstride, g, total)
+  }
+#undef POOL_SWITCH
+  return AfterLaunch("unpool");
+}
+
+/* ------------------------------------------------------------------ im2col / col2im */
+
+#define PATCH_ENTRY(NAME, T, FN, A, AS, B, BS)                                                 \
+  int NAME(T *A, int AS, const T *B, int BS, int n, int c, int h, int w, int ky, int kx, int sy, \
+           int sx, int dy, int dx, int pad_y, int pad_x, void *stream) {                        \
+    PatchGeom g;                                                                               \
+    int st = MakePatchGeom(&g, n, c, h, w, ky, kx, sy, sx, dy, dx, pad_y, pad_x);              \
+    if (st != MSHADOW_HIP_OK) return st;                                                       \
+    return FN<T>(A, AS, B, BS, g, stream);                                                     \
+  }
+PATCH_ENTRY(mshadow_hip_im2col_f16, uint16_t, Im2Col, col, cstride, img, istride)
+PATCH_ENTRY(mshadow_hip_im2col_f32, float, Im2Col, col, cstride, img, istride)
+PATCH_ENTRY(mshadow_hip_col2im_f16, uint16_t, Col2Im, img, istride, col, cstride)
+PATCH_ENTRY(mshadow_hip_col2im_f32, float, Col2Im, img, istride, col, cstride)
+#undef PATCH_ENTRY
+
+}  // extern "C"

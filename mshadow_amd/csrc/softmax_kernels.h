@@ -1,0 +1,253 @@
+/*
+ * Row softmax and its gradient for gfx950.
+ *
+ * SoftmaxRowKernel: one workgroup per row, the whole row held in registers, so HBM
+ * sees one read of src and one write of dst (2 * 4 bytes per element; the reference
+ * kernel, mshadow/cuda/tensor_gpu-inl.cuh:330-393, moves 5). Steps per row:
+ *   1. 128-bit loads, row maximum by wave shuffles + one LDS exchange;
+ *   2. p = expf(x - max) in registers;
+ *   3. the row sum in the CPU path's left-to-right order (ordered_sum.h), so that the
+ *      result matches mshadow/tensor_cpu-inl.h:270-285 to the last bit of the sum;
+ *   4. p / sum with IEEE division, 128-bit stores.
+ * dst may alias src (every element is read before the row is written).
+ * SoftmaxLongRowKernel covers rows too long for registers with the same arithmetic,
+ * staging p through dst. SoftmaxGradKernel is a 128-bit copy with one element per row
+ * decremented (mshadow/tensor_cpu-inl.h:287-302).
+ */
+#ifndef MSHADOW_AMD_CSRC_SOFTMAX_KERNELS_H_
+#define MSHADOW_AMD_CSRC_SOFTMAX_KERNELS_H_
+
+#include <hip/hip_runtime.h>
+
+#include <mshadow/hip/kernels/common.h>
+
+#include "ordered_sum.h"
+
+namespace mshadow_hipk {
+
+using mshadow::hip::kWave;
+using mshadow::hip::LaneId;
+using mshadow::hip::ReadLaneF32;
+using mshadow::hip::ReadLaneU32;
+using mshadow::hip::WaveId;
+using mshadow::hip::WaveInclusiveScanU32;
+using mshadow::hip::WaveMaxF32;
+using mshadow::hip::WaveSumU32;
+
+/*! \brief LDS scratch of the ordered sum: two alternating sets of per-wave totals and
+ *  the hand-over slot for the running sum */
+template <int WAVES>
+struct OrderedSumLds {
+  uint32_t q[2][WAVES];
+  float s;
+  float wmax[WAVES];
+};
+
+/*! \brief one wave adds its 64 * N terms (lane order, then element order) to s exactly
+ *  as a serial loop would; called only for the wave in which a chunk was rejected */
+template <int N>
+__device__ inline float WaveResolve(float s, const float (&t)[N]) {
+  using namespace ordered_sum;
+  const int lane = LaneId();
+  int start = 0;
+  while (true) {
+    const Binade b = BinadeOf(s);
+    const uint32_t q = (lane >= start) ? LaneQuant<N>(t, b) : 0u;
+    const uint32_t incl = WaveInclusiveScanU32(q);  // <= 64 * 2^24, no overflow
+    const bool fail = (lane >= start) && (b.m + incl >= kBig);
+    const unsigned long long mask = __ballot(fail);
+    if (mask == 0ull) return Accept(s, b, ReadLaneU32(incl, kWave - 1));
+    const int first = __ffsll(mask) - 1;
+    /* lanes before `first` are exact integer adds */
+    s = Accept(s, b, ReadLaneU32(incl - q, first));
+    /* lane `first` does real float adds; every lane computes, one result is taken */
+    s = ReadLaneF32(TrueAdd<N>(s, t), first);
+    start = first + 1;
+    if (start == kWave) return s;
+  }
+}
+
+/*! \brief block-wide: add one slab (THREADS * N consecutive terms, thread-major) to s.
+ *  s is uniform over the block on entry and on exit. `buf` alternates the LDS slot. */
+template <int THREADS, int N>
+__device__ inline float BlockOrderedAdd(float s, const float (&t)[N],
+                                        OrderedSumLds<THREADS / kWave> *lds, int *buf) {
+  using namespace ordered_sum;
+  const int W = THREADS / kWave;
+  const int wave = WaveId();
+  const int lane = LaneId();
+  int pos = 0;  // waves before pos are already in s
+  while (true) {
+    const Binade b = BinadeOf(s);
+    if (wave >= pos) {
+      uint32_t q = WaveSumU32(LaneQuant<N>(t, b));
+      if (lane == 0) lds->q[*buf][wave] = q < kBig ? q : kBig;
+    }
+    __syncthreads();
+    uint32_t acc = 0;
+    int failw = W;
+    for (int w = pos; w < W; ++w) {
+      const uint32_t qw = lds->q[*buf][w];
+      if (b.m + acc + qw >= kBig) {
+        failw = w;
+        break;
+      }
+      acc += qw;
+    }
+    *buf ^= 1;
+    s = Accept(s, b, acc);
+    if (failw == W) return s;
+    if (wave == failw) {
+      const float r = WaveResolve<N>(s, t);
+      if (lane == 0) lds->s = r;
+    }
+    __syncthreads();
+    s = lds->s;
+    pos = failw + 1;
+    if (pos == W) return s;
+  }
+}
+
+template <int THREADS>
+__device__ inline float BlockMax(float v, OrderedSumLds<THREADS / kWave> *lds) {
+  const int W = THREADS / kWave;
+  v = WaveMaxF32(v);
+  if (LaneId() == 0) lds->wmax[WaveId()] = v;
+  __syncthreads();
+  float m = lds->wmax[0];
+#pragma unroll
+  for (int w = 1; w < W; ++w) {
+    const float o = lds->wmax[w];
+    m = (m < o) ? o : m;
+  }
+  return m;
+}
+
+/*! \brief THREADS * SLABS * VEC >= cols. VEC == 4 needs 16-byte aligned rows. */
+template <int THREADS, int SLABS, int VEC>
+__global__ void __launch_bounds__(THREADS)
+    SoftmaxRowKernel(float *dst, int dstride, const float *src, int sstride, int cols) {
+  __shared__ OrderedSumLds<THREADS / kWave> lds;
+  const int tid = threadIdx.x;
+  const float *in = src + static_cast<size_t>(blockIdx.x) * sstride;
+  float *out = dst + static_cast<size_t>(blockIdx.x) * dstride;
+  const float kNegInf = -__builtin_huge_valf();
+
+  float v[SLABS][VEC];
+  float mx = kNegInf;
+#pragma unroll
+  for (int j = 0; j < SLABS; ++j) {
+    const int base = (j * THREADS + tid) * VEC;
+    if (VEC == 4 && base + 4 <= cols) {
+      const float4 q = *reinterpret_cast<const float4 *>(in + base);
+      v[j][0] = q.x; v[j][1 % VEC] = q.y; v[j][2 % VEC] = q.z; v[j][3 % VEC] = q.w;
+    } else {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) v[j][i] = (base + i < cols) ? in[base + i] : kNegInf;
+    }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) mx = (mx < v[j][i]) ? v[j][i] : mx;
+  }
+  mx = BlockMax<THREADS>(mx, &lds);
+
+#pragma unroll
+  for (int j = 0; j < SLABS; ++j) {
+    const int base = (j * THREADS + tid) * VEC;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[j][i] = (base + i < cols) ? expf(v[j][i] - mx) : 0.0f;
+  }
+
+  float s = 0.0f;
+  int buf = 0;
+#pragma unroll
+  for (int j = 0; j < SLABS; ++j) {
+    if (j * THREADS * VEC < cols) s = BlockOrderedAdd<THREADS, VEC>(s, v[j], &lds, &buf);
+  }
+
+#pragma unroll
+  for (int j = 0; j < SLABS; ++j) {
+    const int base = (j * THREADS + tid) * VEC;
+    if (VEC == 4 && base + 4 <= cols) {
+      float4 q;
+      q.x = v[j][0] / s; q.y = v[j][1 % VEC] / s; q.z = v[j][2 % VEC] / s; q.w = v[j][3 % VEC] / s;
+      *reinterpret_cast<float4 *>(out + base) = q;
+    } else {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        if (base + i < cols) out[base + i] = v[j][i] / s;
+      }
+    }
+  }
+}
+
+/*! \brief any row length: three passes, exp(x - max) parked in dst between them */
+template <int THREADS>
+__global__ void __launch_bounds__(THREADS)
+    SoftmaxLongRowKernel(float *dst, int dstride, const float *src, int sstride, int cols) {
+  __shared__ OrderedSumLds<THREADS / kWave> lds;
+  const int tid = threadIdx.x;
+  const float *in = src + static_cast<size_t>(blockIdx.x) * sstride;
+  float *out = dst + static_cast<size_t>(blockIdx.x) * dstride;
+  const float kNegInf = -__builtin_huge_valf();
+  float mx = kNegInf;
+  for (int x = tid; x < cols; x += THREADS) {
+    const float e = in[x];
+    mx = (mx < e) ? e : mx;
+  }
+  mx = BlockMax<THREADS>(mx, &lds);
+  float s = 0.0f;
+  int buf = 0;
+  for (int x0 = 0; x0 < cols; x0 += THREADS) {
+    const int x = x0 + tid;
+    float p[1];
+    p[0] = (x < cols) ? expf(in[x] - mx) : 0.0f;
+    if (x < cols) out[x] = p[0];
+    s = BlockOrderedAdd<THREADS, 1>(s, p, &lds, &buf);
+  }
+  for (int x = tid; x < cols; x += THREADS) out[x] = out[x] / s;
+}
+
+const int kGradBlock = 256;
+const int kGradPacks = 4;  // 128-bit packs per thread
+
+/*! \brief grid.x = rows, grid.y = column chunks of kGradBlock * kGradPacks * 4 elements */
+template <bool VEC4>
+__global__ void __launch_bounds__(kGradBlock)
+    SoftmaxGradKernel(float *dst, int dstride, const float *src, int sstride, const float *label,
+                      int cols) {
+  const int y = blockIdx.x;
+  const int k = static_cast<int>(label[y]);
+  const float *in = src + static_cast<size_t>(y) * sstride;
+  float *out = dst + static_cast<size_t>(y) * dstride;
+  const int chunk0 = blockIdx.y * (kGradBlock * kGradPacks * 4);
+  if (VEC4) {
+    float4 q[kGradPacks];
+#pragma unroll
+    for (int u = 0; u < kGradPacks; ++u) {
+      const int x = chunk0 + (u * kGradBlock + threadIdx.x) * 4;
+      if (x + 4 <= cols) q[u] = *reinterpret_cast<const float4 *>(in + x);
+    }
+#pragma unroll
+    for (int u = 0; u < kGradPacks; ++u) {
+      const int x = chunk0 + (u * kGradBlock + threadIdx.x) * 4;
+      if (x + 4 <= cols) {
+        if (k == x) q[u].x = q[u].x - 1.0f;
+        if (k == x + 1) q[u].y = q[u].y - 1.0f;
+        if (k == x + 2) q[u].z = q[u].z - 1.0f;
+        if (k == x + 3) q[u].w = q[u].w - 1.0f;
+        *reinterpret_cast<float4 *>(out + x) = q[u];
+      } else {
+        for (int i = x; i < cols; ++i) out[i] = (i == k) ? in[i] - 1.0f : in[i];
+      }
+    }
+  } else {
+#pragma unroll
+    for (int u = 0; u < kGradPacks * 4; ++u) {
+      const int x = chunk0 + u * kGradBlock + threadIdx.x;
+      if (x < cols) out[x] = (x == k) ? in[x] - 1.0f : in[x];
+    }
+  }
+}
+
+}  // namespace mshadow_hipk
+#endif  // MSHADOW_AMD_CSRC_SOFTMAX_KERNELS_H_

@@ -1,0 +1,293 @@
+/*
+ * Plan<Exp, DType>: the by-value, device-copyable evaluator of an expression tree.
+ *
+ * MakePlan(tree) flattens the reference-linked tree into nested Plan objects holding
+ * raw pointers, pitches and scalars; `plan.Eval(y, x)` yields the element of the 2-D
+ * view at row y, column x. This is the contract of mshadow/expr_engine-inl.h:39-232
+ * in the reference (Plan / MakePlan are extension points: callers specialise Plan for
+ * their own nodes and only need Eval).
+ *
+ * Added for gfx950: plans made only of tensors, scalars and elementwise maps also
+ * evaluate N adjacent columns at once (EvalPack<N>) from one 128-bit global load per
+ * tensor leaf. A plan advertises that with `kPackable`; PackReady() checks at run
+ * time that every leaf pointer and pitch is aligned for N-wide access. Plans without
+ * these members (caller-defined ones) simply take the scalar path.
+ */
+#ifndef MSHADOW_EXPR_PLAN_H_
+#define MSHADOW_EXPR_PLAN_H_
+
+#include <stdint.h>
+
+#include "../core/tensor_types.h"
+
+namespace mshadow {
+namespace expr {
+
+/*! \brief N adjacent elements of a row, aligned so that one memory instruction moves them */
+template <typename DType, int N>
+struct MSHADOW_ALIGNED(sizeof(DType) * N) Pack {
+  DType v[N];
+};
+
+/*! \brief base of the chainer nodes: a node that knows its own output shape */
+template <typename SubType, typename SrcExp, int dim, typename DType>
+struct MakeTensorExp : public Exp<MakeTensorExp<SubType, SrcExp, dim, DType>, DType, type::kChainer> {
+  /*! \brief shape of the output */
+  Shape<dim> shape_;
+  inline const SubType &real_self(void) const { return *static_cast<const SubType *>(this); }
+};
+
+template <typename ExpType, typename DType>
+class Plan {
+ public:
+  /*! \brief value at row y, column x of the flattened 2-D view */
+  MSHADOW_XINLINE DType Eval(index_t y, index_t x) const;
+};
+
+/* ---- leaves ---- */
+template <typename Device, int dim, typename DType>
+class Plan<Tensor<Device, dim, DType>, DType> {
+ public:
+  static const bool kPackable = true;
+  explicit Plan(const Tensor<Device, dim, DType> &t) : dptr_(t.dptr_), stride_(t.stride_) {}
+  MSHADOW_XINLINE DType &REval(index_t y, index_t x) { return dptr_[y * stride_ + x]; }
+  MSHADOW_XINLINE const DType &Eval(index_t y, index_t x) const { return dptr_[y * stride_ + x]; }
+  template <int N>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t x) const {
+    return *reinterpret_cast<const Pack<DType, N> *>(dptr_ + y * stride_ + x);
+  }
+  template <int N>
+  MSHADOW_XINLINE void StorePack(index_t y, index_t x, const Pack<DType, N> &p) {
+    *reinterpret_cast<Pack<DType, N> *>(dptr_ + y * stride_ + x) = p;
+  }
+  /*! \brief host check: pointer and pitch allow n-wide access; *flat stays true only
+   *  while rows are dense (pitch == cols) so that the 2-D view can be walked linearly */
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    if (stride_ != cols) *flat = false;
+    return reinterpret_cast<uintptr_t>(dptr_) % (sizeof(DType) * n) == 0 && stride_ % n == 0;
+  }
+
+ private:
+  DType *dptr_;
+  index_t stride_;
+};
+
+template <typename Device, typename DType>
+class Plan<Tensor<Device, 1, DType>, DType> {
+ public:
+  static const bool kPackable = true;
+  explicit Plan(const Tensor<Device, 1, DType> &t) : dptr_(t.dptr_) {}
+  MSHADOW_XINLINE DType &REval(index_t y, index_t x) { return dptr_[x]; }
+  MSHADOW_XINLINE const DType &Eval(index_t y, index_t x) const { return dptr_[x]; }
+  template <int N>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t x) const {
+    return *reinterpret_cast<const Pack<DType, N> *>(dptr_ + x);
+  }
+  template <int N>
+  MSHADOW_XINLINE void StorePack(index_t y, index_t x, const Pack<DType, N> &p) {
+    *reinterpret_cast<Pack<DType, N> *>(dptr_ + x) = p;
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    return reinterpret_cast<uintptr_t>(dptr_) % (sizeof(DType) * n) == 0;
+  }
+
+ private:
+  DType *dptr_;
+};
+
+template <typename DType>
+class Plan<ScalarExp<DType>, DType> {
+ public:
+  static const bool kPackable = true;
+  explicit Plan(DType scalar) : scalar_(scalar) {}
+  MSHADOW_XINLINE DType Eval(index_t y, index_t x) const { return scalar_; }
+  template <int N>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t x) const {
+    Pack<DType, N> p;
+#pragma unroll
+    for (int i = 0; i < N; ++i) p.v[i] = scalar_;
+    return p;
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const { return true; }
+
+ private:
+  DType scalar_;
+};
+
+/* ---- interior nodes ---- */
+template <typename DstDType, typename SrcDType, typename EType, int etype>
+class Plan<TypecastExp<DstDType, SrcDType, EType, etype>, DstDType> {
+ public:
+  explicit Plan(const Plan<EType, SrcDType> &src) : src_(src) {}
+  MSHADOW_XINLINE DstDType Eval(index_t y, index_t x) const {
+    return DstDType(src_.Eval(y, x));  // NOLINT(*)
+  }
+
+ private:
+  Plan<EType, SrcDType> src_;
+};
+
+namespace plan_detail {
+/*! \brief P::kPackable if the plan type declares it, false otherwise */
+template <typename P>
+struct Packable {
+  template <typename Q>
+  static char Test(int (*)[Q::kPackable ? 1 : -1]);
+  template <typename Q>
+  static long Test(...);  // NOLINT(*)
+  static const bool value = sizeof(Test<P>(0)) == sizeof(char);
+};
+}  // namespace plan_detail
+
+template <typename OP, typename TA, typename TB, typename TC, int etype, typename DType>
+class Plan<TernaryMapExp<OP, TA, TB, TC, DType, etype>, DType> {
+ public:
+  static const bool kPackable = plan_detail::Packable<Plan<TA, DType> >::value &&
+                                plan_detail::Packable<Plan<TB, DType> >::value &&
+                                plan_detail::Packable<Plan<TC, DType> >::value;
+  explicit Plan(const Plan<TA, DType> &item1, const Plan<TB, DType> &item2,
+                const Plan<TC, DType> &item3)
+      : item1_(item1), item2_(item2), item3_(item3) {}
+  MSHADOW_XINLINE DType Eval(index_t y, index_t x) const {
+    return OP::Map(item1_.Eval(y, x), item2_.Eval(y, x), item3_.Eval(y, x));
+  }
+  template <int N>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t x) const {
+    const Pack<DType, N> a = item1_.template EvalPack<N>(y, x);
+    const Pack<DType, N> b = item2_.template EvalPack<N>(y, x);
+    const Pack<DType, N> c = item3_.template EvalPack<N>(y, x);
+    Pack<DType, N> r;
+#pragma unroll
+    for (int i = 0; i < N; ++i) r.v[i] = OP::Map(a.v[i], b.v[i], c.v[i]);
+    return r;
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    return item1_.PackReady(n, cols, flat) && item2_.PackReady(n, cols, flat) &&
+           item3_.PackReady(n, cols, flat);
+  }
+
+ private:
+  Plan<TA, DType> item1_;
+  Plan<TB, DType> item2_;
+  Plan<TC, DType> item3_;
+};
+
+template <typename OP, typename TA, typename TB, int etype, typename DType>
+class Plan<BinaryMapExp<OP, TA, TB, DType, etype>, DType> {
+ public:
+  static const bool kPackable = plan_detail::Packable<Plan<TA, DType> >::value &&
+                                plan_detail::Packable<Plan<TB, DType> >::value;
+  explicit Plan(const Plan<TA, DType> &lhs, const Plan<TB, DType> &rhs) : lhs_(lhs), rhs_(rhs) {}
+  MSHADOW_XINLINE DType Eval(index_t y, index_t x) const {
+    return OP::Map(lhs_.Eval(y, x), rhs_.Eval(y, x));
+  }
+  template <int N>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t x) const {
+    const Pack<DType, N> a = lhs_.template EvalPack<N>(y, x);
+    const Pack<DType, N> b = rhs_.template EvalPack<N>(y, x);
+    Pack<DType, N> r;
+#pragma unroll
+    for (int i = 0; i < N; ++i) r.v[i] = OP::Map(a.v[i], b.v[i]);
+    return r;
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    return lhs_.PackReady(n, cols, flat) && rhs_.PackReady(n, cols, flat);
+  }
+
+ private:
+  Plan<TA, DType> lhs_;
+  Plan<TB, DType> rhs_;
+};
+
+template <typename OP, typename TA, int etype, typename DType>
+class Plan<UnaryMapExp<OP, TA, DType, etype>, DType> {
+ public:
+  static const bool kPackable = plan_detail::Packable<Plan<TA, DType> >::value;
+  explicit Plan(const Plan<TA, DType> &src) : src_(src) {}
+  MSHADOW_XINLINE DType Eval(index_t y, index_t x) const { return OP::Map(src_.Eval(y, x)); }
+  template <int N>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t x) const {
+    const Pack<DType, N> a = src_.template EvalPack<N>(y, x);
+    Pack<DType, N> r;
+#pragma unroll
+    for (int i = 0; i < N; ++i) r.v[i] = OP::Map(a.v[i]);
+    return r;
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    return src_.PackReady(n, cols, flat);
+  }
+
+ private:
+  Plan<TA, DType> src_;
+};
+
+/*! \brief a chainer node evaluates through the plan of its concrete type */
+template <typename SubType, typename SrcExp, int dim, typename DType>
+struct Plan<MakeTensorExp<SubType, SrcExp, dim, DType>, DType> {
+ public:
+  Plan(const Plan<SubType, DType> &src) : src_(src) {}  // NOLINT(*)
+  MSHADOW_XINLINE DType Eval(index_t y, index_t x) const { return src_.Eval(y, x); }
+
+ private:
+  Plan<SubType, DType> src_;
+};
+
+template <typename EType, typename DType>
+class Plan<TransposeExp<EType, DType>, DType> {
+ public:
+  explicit Plan(const Plan<EType, DType> &src) : src_(src) {}
+  MSHADOW_XINLINE DType Eval(index_t y, index_t x) const { return src_.Eval(x, y); }
+
+ private:
+  Plan<EType, DType> src_;
+};
+
+/* ---- MakePlan: tree -> plan (mshadow/expr_engine-inl.h:175-232) ---- */
+template <typename OP, typename TA, typename TB, typename DType, int etype>
+inline Plan<BinaryMapExp<OP, TA, TB, DType, etype>, DType> MakePlan(
+    const BinaryMapExp<OP, TA, TB, DType, etype> &e);
+template <typename OP, typename TA, typename TB, typename TC, typename DType, int etype>
+inline Plan<TernaryMapExp<OP, TA, TB, TC, DType, etype>, DType> MakePlan(
+    const TernaryMapExp<OP, TA, TB, TC, DType, etype> &e);
+
+template <typename DType>
+inline Plan<ScalarExp<DType>, DType> MakePlan(const ScalarExp<DType> &e) {
+  return Plan<ScalarExp<DType>, DType>(e.scalar_);
+}
+template <typename DstDType, typename SrcDType, typename EType, int etype>
+inline Plan<TypecastExp<DstDType, SrcDType, EType, etype>, DstDType> MakePlan(
+    const TypecastExp<DstDType, SrcDType, EType, etype> &e) {
+  return Plan<TypecastExp<DstDType, SrcDType, EType, etype>, DstDType>(MakePlan(e.exp));
+}
+template <typename T, typename DType>
+inline Plan<T, DType> MakePlan(const RValueExp<T, DType> &e) {
+  return Plan<T, DType>(e.self());
+}
+template <typename T, typename DType>
+inline Plan<TransposeExp<T, DType>, DType> MakePlan(const TransposeExp<T, DType> &e) {
+  return Plan<TransposeExp<T, DType>, DType>(MakePlan(e.exp));
+}
+template <typename T, typename SrcExp, int dim, typename DType>
+inline Plan<T, DType> MakePlan(const MakeTensorExp<T, SrcExp, dim, DType> &e) {
+  return Plan<T, DType>(e.real_self());
+}
+template <typename OP, typename TA, typename DType, int etype>
+inline Plan<UnaryMapExp<OP, TA, DType, etype>, DType> MakePlan(
+    const UnaryMapExp<OP, TA, DType, etype> &e) {
+  return Plan<UnaryMapExp<OP, TA, DType, etype>, DType>(MakePlan(e.src_));
+}
+template <typename OP, typename TA, typename TB, typename DType, int etype>
+inline Plan<BinaryMapExp<OP, TA, TB, DType, etype>, DType> MakePlan(
+    const BinaryMapExp<OP, TA, TB, DType, etype> &e) {
+  return Plan<BinaryMapExp<OP, TA, TB, DType, etype>, DType>(MakePlan(e.lhs_), MakePlan(e.rhs_));
+}
+template <typename OP, typename TA, typename TB, typename TC, typename DType, int etype>
+inline Plan<TernaryMapExp<OP, TA, TB, TC, DType, etype>, DType> MakePlan(
+    const TernaryMapExp<OP, TA, TB, TC, DType, etype> &e) {
+  return Plan<TernaryMapExp<OP, TA, TB, TC, DType, etype>, DType>(
+      MakePlan(e.item1_), MakePlan(e.item2_), MakePlan(e.item3_));
+}
+
+}  // namespace expr
+}  // namespace mshadow
+#endif  // MSHADOW_EXPR_PLAN_H_

@@ -1,0 +1,8 @@
+/*! \file extension.h  the expression extensions this backend provides */
+#ifndef MSHADOW_EXTENSION_H_
+#define MSHADOW_EXTENSION_H_
+#include "./tensor.h"
+#include "./ext/reduceto1d.h"
+#include "./ext/pooling.h"
+#include "./ext/patches.h"
+#endif  // MSHADOW_EXTENSION_H_

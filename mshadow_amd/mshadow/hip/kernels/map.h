@@ -1,0 +1,79 @@
+/*
+ * Elementwise evaluation kernels: Saver::Save(dst(y, x), plan.Eval(y, x)) for every
+ * element of the destination's 2-D view. They replace MapPlanKernel /
+ * MapPlanLargeKernel of the reference (mshadow/cuda/tensor_gpu-inl.cuh:67-120), which
+ * handle one element per thread with a division per element and 4-byte accesses.
+ *
+ * MapPackKernel  every leaf is a tensor or scalar and all pointers / pitches are
+ *                16-byte aligned: each thread moves kPackUnroll packs of N = 16 /
+ *                sizeof(DType) elements with one 128-bit global access per leaf. When
+ *                all rows are dense the 2-D view is walked linearly and no division
+ *                is executed at all; otherwise there is one per pack.
+ *                Algorithmic traffic: (leaves + 1) * sizeof(DType) bytes per element,
+ *                HBM-bound (5 * 4 B for dst = A*B + 0.5f*F<sigmoid>(C) - D).
+ * MapScalarKernel any plan (chainers, transposes, caller-defined plans, unaligned or
+ *                ragged rows): one element per thread-iteration, grid-stride.
+ */
+#ifndef MSHADOW_HIP_KERNELS_MAP_H_
+#define MSHADOW_HIP_KERNELS_MAP_H_
+
+#include "../../expr/plan.h"
+#include "./common.h"
+
+namespace mshadow {
+namespace hip {
+
+const int kMapBlock = 256;
+/*! \brief packs per thread; the loads of all of them are issued before the first use */
+const int kPackUnroll = 4;
+
+template <typename Saver, typename DType, typename DPlan, typename SPlan>
+__global__ void __launch_bounds__(kMapBlock)
+    MapScalarKernel(DPlan dplan, SPlan splan, uint32_t rows, uint32_t cols) {
+  const uint32_t total = rows * cols;
+  const uint32_t step = gridDim.x * kMapBlock;
+  for (uint32_t i = blockIdx.x * kMapBlock + threadIdx.x; i < total; i += step) {
+    const uint32_t y = i / cols;
+    const uint32_t x = i - y * cols;
+    Saver::template Save<DType>(dplan.REval(y, x), splan.Eval(y, x));
+  }
+}
+
+template <typename Saver, typename DType, int N, bool kFlat, typename DPlan, typename SPlan>
+__global__ void __launch_bounds__(kMapBlock)
+    MapPackKernel(DPlan dplan, SPlan splan, uint32_t total_packs, uint32_t packs_per_row) {
+  typedef expr::Pack<DType, N> P;
+  const uint32_t base = blockIdx.x * (kMapBlock * kPackUnroll) + threadIdx.x;
+  uint32_t y[kPackUnroll], x[kPackUnroll];
+  P val[kPackUnroll];
+#pragma unroll
+  for (int u = 0; u < kPackUnroll; ++u) {
+    const uint32_t p = base + u * kMapBlock;
+    if (kFlat) {
+      y[u] = 0;
+      x[u] = p * N;
+    } else {
+      y[u] = p / packs_per_row;
+      x[u] = (p - y[u] * packs_per_row) * N;
+    }
+    if (p < total_packs) val[u] = splan.template EvalPack<N>(y[u], x[u]);
+  }
+#pragma unroll
+  for (int u = 0; u < kPackUnroll; ++u) {
+    const uint32_t p = base + u * kMapBlock;
+    if (p < total_packs) {
+      if (SaverReadsDst<Saver>::value) {
+        P old = dplan.template EvalPack<N>(y[u], x[u]);
+#pragma unroll
+        for (int i = 0; i < N; ++i) Saver::template Save<DType>(old.v[i], val[u].v[i]);
+        dplan.template StorePack<N>(y[u], x[u], old);
+      } else {
+        dplan.template StorePack<N>(y[u], x[u], val[u]);
+      }
+    }
+  }
+}
+
+}  // namespace hip
+}  // namespace mshadow
+#endif  // MSHADOW_HIP_KERNELS_MAP_H_

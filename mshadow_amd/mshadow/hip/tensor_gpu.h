@@ -1,0 +1,466 @@
+/*
+ * Tensor<gpu>: the gfx950 device of the API.
+ *
+ * Host-side definitions that replace mshadow/tensor_gpu-inl.h:14-214 of the reference.
+ * Memory, copies, streams and the fixed-function operations go through the C ABI of
+ * libmshadow_hip (include/mshadow_hip.h) and are available to any translation unit.
+ * Evaluating an arbitrary expression into a Tensor<gpu> instantiates a kernel template
+ * from mshadow/hip/kernels/ for the caller's expression type and starts it through
+ * mshadow_hip_launch; that part needs hipcc, exactly as the reference needs nvcc for
+ * it (tensor_gpu-inl.h:96-98). Expressions whose shape the library knows - pool /
+ * unpool of float tensors, unpack_patch2col(pad(tensor)), crop(pack_col2patch(tensor)),
+ * reductions of plain float tensors - are routed to the tuned fixed-function kernels
+ * first (FastPath below).
+ */
+#ifndef MSHADOW_HIP_TENSOR_GPU_H_
+#define MSHADOW_HIP_TENSOR_GPU_H_
+
+#include <mshadow_hip.h>
+
+#include "../tensor.h"
+#include "./stream.h"
+
+#if defined(__HIPCC__)
+#include "./kernels/map.h"
+#include "./kernels/reduce.h"
+#endif
+
+namespace mshadow {
+
+template <>
+inline void InitTensorEngine<gpu>(int dev_id) {
+  int device_count = 0;
+  MSHADOW_HIP_CALL(mshadow_hip_device_count(&device_count));
+  CHECK_GT(device_count, 0) << "Cannot find a HIP device. Please check the ROCm installation";
+  const int device_id = dev_id < 0 ? 0 : dev_id;
+  CHECK_LT(device_id, device_count) << "Incorrect Device ID";
+  MSHADOW_HIP_CALL(mshadow_hip_set_device(device_id));
+  mshadow_hip_props prop;
+  MSHADOW_HIP_CALL(mshadow_hip_get_props(device_id, &prop));
+}
+template <>
+inline void ShutdownTensorEngine<gpu>(void) {}
+template <>
+inline void SetDevice<gpu>(int devid) {
+  MSHADOW_HIP_CALL(mshadow_hip_set_device(devid));
+}
+
+/*! \brief pinned host memory for transfers */
+template <>
+inline void *AllocHost_<gpu>(size_t size) {
+  void *dptr;
+  MSHADOW_HIP_CALL(mshadow_hip_malloc_host(&dptr, size));
+  return dptr;
+}
+template <>
+inline void FreeHost_<gpu>(void *dptr) {
+  MSHADOW_HIP_CALL(mshadow_hip_free_host(dptr));
+}
+
+/*! \brief rows get a 256-byte-aligned pitch when padding is on and the last dimension
+ *  is at least MSHADOW_MIN_PAD_RATIO * 32 elements (rule of tensor_gpu-inl.h:37-51) */
+template <int dim, typename DType>
+inline void AllocSpace(Tensor<gpu, dim, DType> *obj, bool pad) {
+  size_t pitch;
+  void *p = NULL;
+  if (pad && obj->size(dim - 1) >= MSHADOW_MIN_PAD_RATIO * 32) {
+    MSHADOW_HIP_CALL(mshadow_hip_malloc_pitch(&p, &pitch, obj->size(dim - 1) * sizeof(DType),
+                                              obj->shape_.FlatTo2D()[0]));
+    obj->stride_ = static_cast<index_t>(pitch / sizeof(DType));
+  } else {
+    obj->stride_ = obj->size(dim - 1);
+    MSHADOW_HIP_CALL(mshadow_hip_malloc_pitch(&p, &pitch, obj->shape_.Size() * sizeof(DType), 1));
+  }
+  obj->dptr_ = reinterpret_cast<DType *>(p);
+}
+template <int dim, typename DType>
+inline void FreeSpace(Tensor<gpu, dim, DType> *obj) {
+  MSHADOW_HIP_CALL(mshadow_hip_free(obj->dptr_));
+  obj->dptr_ = NULL;
+}
+
+namespace gpu_detail {
+template <typename A, typename B, int dim, typename DType>
+inline void Copy2D(Tensor<A, dim, DType> _dst, Tensor<B, dim, DType> _src, int kind,
+                   Stream<gpu> *stream) {
+  CHECK_EQ(_dst.shape_, _src.shape_) << "Copy:shape mismatch";
+  Tensor<A, 2, DType> dst = _dst.FlatTo2D();
+  Tensor<B, 2, DType> src = _src.FlatTo2D();
+  MSHADOW_HIP_CALL(mshadow_hip_memcpy2d_async(
+      dst.dptr_, dst.stride_ * sizeof(DType), src.dptr_, src.stride_ * sizeof(DType),
+      dst.size(1) * sizeof(DType), dst.size(0), kind, Stream<gpu>::GetStream(stream)));
+  if (stream == NULL) {  // only reachable with MSHADOW_FORCE_STREAM off
+    MSHADOW_HIP_CALL(mshadow_hip_stream_sync(NULL));
+  }
+}
+}  // namespace gpu_detail
+
+template <int dim, typename DType>
+inline void Copy(Tensor<cpu, dim, DType> dst, const Tensor<gpu, dim, DType> &src,
+                 Stream<gpu> *stream) {
+  gpu_detail::Copy2D(dst, src, MSHADOW_HIP_D2H, stream);
+}
+template <int dim, typename DType>
+inline void Copy(Tensor<gpu, dim, DType> dst, const Tensor<gpu, dim, DType> &src,
+                 Stream<gpu> *stream) {
+  gpu_detail::Copy2D(dst, src, MSHADOW_HIP_D2D, stream);
+}
+template <int dim, typename DType>
+inline void Copy(Tensor<gpu, dim, DType> dst, const Tensor<cpu, dim, DType> &src,
+                 Stream<gpu> *stream) {
+  gpu_detail::Copy2D(dst, src, MSHADOW_HIP_H2D, stream);
+}
+
+/* ------------------------------------------------------------------ fixed-function ops */
+namespace gpu_detail {
+template <typename Saver>
+struct SaverCode {
+  static const int value = -1;
+};
+template <>
+struct SaverCode<sv::saveto> { static const int value = MSHADOW_HIP_SAVETO; };
+template <>
+struct SaverCode<sv::plusto> { static const int value = MSHADOW_HIP_PLUSTO; };
+template <>
+struct SaverCode<sv::minusto> { static const int value = MSHADOW_HIP_MINUSTO; };
+template <>
+struct SaverCode<sv::multo> { static const int value = MSHADOW_HIP_MULTO; };
+template <>
+struct SaverCode<sv::divto> { static const int value = MSHADOW_HIP_DIVTO; };
+template <typename Reducer>
+struct ReducerCode {
+  static const int value = -1;
+};
+template <>
+struct ReducerCode<red::sum> { static const int value = MSHADOW_HIP_SUM; };
+template <>
+struct ReducerCode<red::maximum> { static const int value = MSHADOW_HIP_MAX; };
+template <>
+struct ReducerCode<red::minimum> { static const int value = MSHADOW_HIP_MIN; };
+
+inline const uint16_t *Bits(const half::half_t *p) { return reinterpret_cast<const uint16_t *>(p); }
+inline uint16_t *Bits(half::half_t *p) { return reinterpret_cast<uint16_t *>(p); }
+}  // namespace gpu_detail
+
+inline void Softmax(Tensor<gpu, 2, float> dst, const Tensor<gpu, 2, float> &src) {
+  CHECK_EQ(dst.shape_, src.shape_) << "Softmax: shape mismatch";
+  MSHADOW_HIP_CALL(mshadow_hip_softmax_f32(dst.dptr_, dst.stride_, src.dptr_, src.stride_,
+                                           dst.size(0), dst.size(1),
+                                           Stream<gpu>::GetStream(dst.stream_)));
+}
+inline void SoftmaxGrad(const Tensor<gpu, 2, float> &dst, const Tensor<gpu, 2, float> &src,
+                        const Tensor<gpu, 1, float> &label) {
+  CHECK_EQ(dst.shape_, src.shape_) << "SoftmaxGrad: shape mismatch";
+  CHECK_EQ(dst.size(0), label.size(0)) << "SoftmaxGrad: label shape mismatch";
+  MSHADOW_HIP_CALL(mshadow_hip_softmax_grad_f32(dst.dptr_, dst.stride_, src.dptr_, src.stride_,
+                                                label.dptr_, dst.size(0), dst.size(1),
+                                                Stream<gpu>::GetStream(dst.stream_)));
+}
+/* the templates declared in tensor.h forward to the float implementations above; other
+   element types have no fixed-function softmax in this backend */
+template <typename DType>
+inline void Softmax(Tensor<gpu, 2, DType> dst, const Tensor<gpu, 2, DType> &src) {
+  LOG(FATAL) << "Softmax<gpu>: only float is provided by this backend";
+}
+template <typename DType>
+inline void SoftmaxGrad(const Tensor<gpu, 2, DType> &dst, const Tensor<gpu, 2, DType> &src,
+                        const Tensor<gpu, 1, DType> &label) {
+  LOG(FATAL) << "SoftmaxGrad<gpu>: only float is provided by this backend";
+}
+
+/* ------------------------------------------------------------------ expression routing */
+namespace gpu_detail {
+
+/*! \brief FastPath<Saver, dim, DType, E>::Run(dst, exp) returns true if it queued a
+ *  fixed-function kernel for the whole assignment; the primary template matches nothing */
+template <typename Saver, int dim, typename DType, typename E>
+struct FastPath {
+  inline static bool Run(Tensor<gpu, dim, DType> *dst, const E &exp) { return false; }
+};
+
+/* dst = pool<Reducer>(float tensor, ...) */
+template <typename Reducer, int dim>
+struct FastPath<sv::saveto, dim, float,
+                expr::PoolingExp<Reducer, Tensor<gpu, dim, float>, float, dim> > {
+  typedef expr::PoolingExp<Reducer, Tensor<gpu, dim, float>, float, dim> E;
+  inline static bool Run(Tensor<gpu, dim, float> *dst, const E &e) {
+    if (ReducerCode<Reducer>::value < 0) return false;
+    const Tensor<gpu, dim, float> &s = e.src_;
+    MSHADOW_HIP_CALL(mshadow_hip_pool_f32(
+        dst->dptr_, dst->stride_, s.dptr_, s.stride_, s.shape_.ProdShape(0, dim - 2),
+        e.src_height_, e.src_width_, e.shape_[dim - 2], e.shape_[dim - 1], e.ksize_y_, e.ksize_x_,
+        e.kstride_y_, e.kstride_x_, ReducerCode<Reducer>::value,
+        Stream<gpu>::GetStream(dst->stream_)));
+    return true;
+  }
+};
+/* dst = unpool<Reducer>(float tensors, ...) */
+template <typename Reducer, int dim>
+struct FastPath<sv::saveto, dim, float,
+                expr::UnPoolingExp<Reducer, Tensor<gpu, dim, float>, float, dim> > {
+  typedef expr::UnPoolingExp<Reducer, Tensor<gpu, dim, float>, float, dim> E;
+  inline static bool Run(Tensor<gpu, dim, float> *dst, const E &e) {
+    if (ReducerCode<Reducer>::value < 0) return false;
+    const Tensor<gpu, dim, float> &s = e.data_src_, &p = e.data_pooled_, &g = e.grad_pooled_;
+    MSHADOW_HIP_CALL(mshadow_hip_unpool_f32(
+        dst->dptr_, dst->stride_, s.dptr_, s.stride_, p.dptr_, p.stride_, g.dptr_, g.stride_,
+        s.shape_.ProdShape(0, dim - 2), e.shape_[dim - 2], e.shape_[dim - 1], e.pshape_y_,
+        e.pshape_x_, e.ksize_y_, e.ksize_x_, e.kstride_y_, e.kstride_x_,
+        ReducerCode<Reducer>::value, Stream<gpu>::GetStream(dst->stream_)));
+    return true;
+  }
+};
+
+template <typename DType>
+struct PatchAbi;
+template <>
+struct PatchAbi<float> {
+  template <typename... A>
+  static int Im2Col(float *col, int cs, const float *img, A... a) {
+    return mshadow_hip_im2col_f32(col, cs, img, a...);
+  }
+  template <typename... A>
+  static int Col2Im(float *img, int is, const float *col, A... a) {
+    return mshadow_hip_col2im_f32(img, is, col, a...);
+  }
+};
+template <>
+struct PatchAbi<half::half_t> {
+  template <typename... A>
+  static int Im2Col(half::half_t *col, int cs, const half::half_t *img, A... a) {
+    return mshadow_hip_im2col_f16(Bits(col), cs, Bits(img), a...);
+  }
+  template <typename... A>
+  static int Col2Im(half::half_t *img, int is, const half::half_t *col, A... a) {
+    return mshadow_hip_col2im_f16(Bits(img), is, Bits(col), a...);
+  }
+};
+template <typename DType>
+struct HasPatchAbi {
+  static const bool value = false;
+};
+template <>
+struct HasPatchAbi<float> { static const bool value = true; };
+template <>
+struct HasPatchAbi<half::half_t> { static const bool value = true; };
+
+/* col = unpack_patch2col(pad(tensor, py, px), ...) and col = unpack_patch2col(tensor, ...) */
+template <typename DType, int sdim>
+struct FastPath<sv::saveto, 2, DType,
+                expr::UnpackPatchToColXExp<
+                    expr::PaddingExp<Tensor<gpu, sdim, DType>, DType, sdim>, DType, sdim> > {
+  typedef expr::UnpackPatchToColXExp<expr::PaddingExp<Tensor<gpu, sdim, DType>, DType, sdim>,
+                                     DType, sdim> E;
+  inline static bool Run(Tensor<gpu, 2, DType> *dst, const E &e) {
+    if (!HasPatchAbi<DType>::value) return false;
+    const expr::PaddingExp<Tensor<gpu, sdim, DType>, DType, sdim> &p = e.img_;
+    const Tensor<gpu, sdim, DType> &img = p.src_;
+    MSHADOW_HIP_CALL(PatchAbi<DType>::Im2Col(
+        dst->dptr_, dst->stride_, img.dptr_, img.stride_, img.shape_.ProdShape(0, sdim - 3),
+        img.shape_[sdim - 3], img.shape_[sdim - 2], img.shape_[sdim - 1], e.psize_y_, e.psize_x_,
+        e.pstride_y_, e.pstride_x_, e.pdilate_y_, e.pdilate_x_, p.pad_y_, p.pad_x_,
+        Stream<gpu>::GetStream(dst->stream_)));
+    return true;
+  }
+};
+template <typename DType, int sdim>
+struct FastPath<sv::saveto, 2, DType,
+                expr::UnpackPatchToColXExp<Tensor<gpu, sdim, DType>, DType, sdim> > {
+  typedef expr::UnpackPatchToColXExp<Tensor<gpu, sdim, DType>, DType, sdim> E;
+  inline static bool Run(Tensor<gpu, 2, DType> *dst, const E &e) {
+    if (!HasPatchAbi<DType>::value) return false;
+    const Tensor<gpu, sdim, DType> &img = e.img_;
+    MSHADOW_HIP_CALL(PatchAbi<DType>::Im2Col(
+        dst->dptr_, dst->stride_, img.dptr_, img.stride_, img.shape_.ProdShape(0, sdim - 3),
+        img.shape_[sdim - 3], img.shape_[sdim - 2], img.shape_[sdim - 1], e.psize_y_, e.psize_x_,
+        e.pstride_y_, e.pstride_x_, e.pdilate_y_, e.pdilate_x_, 0, 0,
+        Stream<gpu>::GetStream(dst->stream_)));
+    return true;
+  }
+};
+/* img = crop(pack_col2patch(col, padded shape, ...), (h, w), py, px) */
+template <typename DType, int ddim>
+struct FastPath<sv::saveto, ddim, DType,
+                expr::CroppingExp<expr::PackColToPatchXExp<Tensor<gpu, 2, DType>, DType, ddim>,
+                                  DType, ddim> > {
+  typedef expr::PackColToPatchXExp<Tensor<gpu, 2, DType>, DType, ddim> Pack;
+  typedef expr::CroppingExp<Pack, DType, ddim> E;
+  inline static bool Run(Tensor<gpu, ddim, DType> *dst, const E &e) {
+    if (!HasPatchAbi<DType>::value) return false;
+    const Pack &p = e.src_;
+    const index_t h = e.shape_[ddim - 2], w = e.shape_[ddim - 1];
+    /* the fixed-function kernel handles symmetric padding: the crop must sit pad_y / pad_x
+       inside an image that is exactly 2 * pad larger */
+    if (p.shape_[ddim - 2] != h + 2 * e.pad_height_ || p.shape_[ddim - 1] != w + 2 * e.pad_width_) {
+      return false;
+    }
+    const Tensor<gpu, 2, DType> &col = p.src_;
+    MSHADOW_HIP_CALL(PatchAbi<DType>::Col2Im(
+        dst->dptr_, dst->stride_, col.dptr_, col.stride_, e.shape_.ProdShape(0, ddim - 3),
+        e.shape_[ddim - 3], h, w, p.psize_y_, p.psize_x_, p.pstride_y_, p.pstride_x_,
+        p.pdilate_y_, p.pdilate_x_, e.pad_height_, e.pad_width_,
+        Stream<gpu>::GetStream(dst->stream_)));
+    return true;
+  }
+};
+/* img = pack_col2patch(col, shape, ...) without padding */
+template <typename DType, int ddim>
+struct FastPath<sv::saveto, ddim, DType,
+                expr::PackColToPatchXExp<Tensor<gpu, 2, DType>, DType, ddim> > {
+  typedef expr::PackColToPatchXExp<Tensor<gpu, 2, DType>, DType, ddim> E;
+  inline static bool Run(Tensor<gpu, ddim, DType> *dst, const E &p) {
+    if (!HasPatchAbi<DType>::value) return false;
+    const Tensor<gpu, 2, DType> &col = p.src_;
+    MSHADOW_HIP_CALL(PatchAbi<DType>::Col2Im(
+        dst->dptr_, dst->stride_, col.dptr_, col.stride_, p.shape_.ProdShape(0, ddim - 3),
+        p.shape_[ddim - 3], p.shape_[ddim - 2], p.shape_[ddim - 1], p.psize_y_, p.psize_x_,
+        p.pstride_y_, p.pstride_x_, p.pdilate_y_, p.pdilate_x_, 0, 0,
+        Stream<gpu>::GetStream(dst->stream_)));
+    return true;
+  }
+};
+
+#if defined(__HIPCC__)
+template <typename K>
+inline void Launch(K kernel, uint32_t grid_x, uint32_t block_x, void **args, void *stream) {
+  const uint32_t grid[3] = {grid_x, 1, 1};
+  const uint32_t block[3] = {block_x, 1, 1};
+  MSHADOW_HIP_CALL(mshadow_hip_launch(reinterpret_cast<const void *>(kernel), grid, block, args, 0,
+                                      stream));
+}
+
+/*! \brief generic elementwise evaluation: pack kernel when the plan allows, else scalar */
+template <typename Saver, typename DType, typename DPlan, typename SPlan, bool kPackable>
+struct MapLauncher {
+  inline static void Run(DPlan dplan, SPlan splan, Shape<2> shape, void *stream) {
+    uint32_t rows = shape[0], cols = shape[1];
+    if (rows == 0 || cols == 0) return;
+    uint32_t grid = 0;
+    MSHADOW_HIP_CALL(mshadow_hip_suggest_grid(static_cast<size_t>(rows) * cols, hip::kMapBlock,
+                                              32, &grid));
+    void *args[] = {&dplan, &splan, &rows, &cols};
+    Launch(hip::MapScalarKernel<Saver, DType, DPlan, SPlan>, grid, hip::kMapBlock, args, stream);
+  }
+};
+template <typename Saver, typename DType, typename DPlan, typename SPlan>
+struct MapLauncher<Saver, DType, DPlan, SPlan, true> {
+  inline static void Run(DPlan dplan, SPlan splan, Shape<2> shape, void *stream) {
+    const int N = 16 / sizeof(DType);
+    uint32_t rows = shape[0], cols = shape[1];
+    if (rows == 0 || cols == 0) return;
+    bool flat = true;
+    const bool aligned = cols % N == 0 && dplan.PackReady(N, cols, &flat) &&
+                         splan.PackReady(N, cols, &flat);
+    if (!aligned) {
+      MapLauncher<Saver, DType, DPlan, SPlan, false>::Run(dplan, splan, shape, stream);
+      return;
+    }
+    uint32_t ppr = cols / N;
+    uint32_t total = rows * ppr;
+    const uint32_t per_block = hip::kMapBlock * hip::kPackUnroll;
+    const uint32_t grid = (total + per_block - 1) / per_block;
+    void *args[] = {&dplan, &splan, &total, &ppr};
+    if (flat || rows == 1) {
+      Launch(hip::MapPackKernel<Saver, DType, N, true, DPlan, SPlan>, grid, hip::kMapBlock, args,
+             stream);
+    } else {
+      Launch(hip::MapPackKernel<Saver, DType, N, false, DPlan, SPlan>, grid, hip::kMapBlock, args,
+             stream);
+    }
+  }
+};
+#endif  // __HIPCC__
+
+}  // namespace gpu_detail
+
+template <typename Saver, typename R, int dim, typename DType, typename E, int etype>
+inline void MapExp(TRValue<R, gpu, dim, DType> *dst, const expr::Exp<E, DType, etype> &exp) {
+  expr::TypeCheckPass<expr::TypeCheck<gpu, dim, DType, E>::kMapPass>::
+      Error_All_Tensor_in_Exp_Must_Have_Same_Type();
+  Shape<dim> eshape = expr::ShapeCheck<dim, E>::Check(exp.self());
+  Shape<dim> dshape = expr::ShapeCheck<dim, R>::Check(dst->self());
+  CHECK(eshape[0] == 0 || eshape == dshape)
+      << "Assignment: Shape of Tensors are not consistent with target, "
+      << "eshape: " << eshape << " dshape:" << dshape;
+  if (gpu_detail::FastPath<Saver, dim, DType, E>::Run(dst->ptrself(), exp.self())) return;
+#if defined(__HIPCC__)
+  typedef expr::Plan<R, DType> DPlan;
+  typedef expr::Plan<E, DType> SPlan;
+  gpu_detail::MapLauncher<Saver, DType, DPlan, SPlan,
+                          expr::plan_detail::Packable<DPlan>::value &&
+                              expr::plan_detail::Packable<SPlan>::value>::
+      Run(expr::MakePlan(dst->self()), expr::MakePlan(exp.self()), dshape.FlatTo2D(),
+          Stream<gpu>::GetStream(expr::StreamInfo<gpu, R>::Get(dst->self())));
+#else
+  LOG(FATAL) << "MapExp<gpu>: this expression has no fixed-function kernel; compile the "
+                "calling translation unit with hipcc so that its kernel can be instantiated";
+#endif
+}
+
+template <typename Saver, typename Reducer, typename R, typename DType, typename E, int etype>
+inline void MapReduceKeepLowest(TRValue<R, gpu, 1, DType> *dst,
+                                const expr::Exp<E, DType, etype> &exp, DType scale) {
+  expr::TypeCheckPass<expr::TypeCheck<gpu, 1, DType, E>::kRedPass>::
+      Error_TypeCheck_Not_Pass_For_Reduce_Exp();
+  Shape<2> eshape = expr::ShapeCheck<expr::ExpInfo<E>::kDim, E>::Check(exp.self()).FlatTo2D();
+  Shape<1> dshape = expr::ShapeCheck<1, R>::Check(dst->self());
+  CHECK_EQ(eshape[1], dshape[0]) << "MapReduceKeepLowest::reduction dimension do not match";
+  CHECK_NE(eshape[0], 0U) << "can not reduce over empty tensor";
+#if defined(__HIPCC__)
+  typedef expr::Plan<R, DType> DPlan;
+  typedef expr::Plan<E, DType> SPlan;
+  DPlan dplan = expr::MakePlan(dst->self());
+  SPlan splan = expr::MakePlan(exp.self());
+  uint32_t rows = eshape[0], cols = eshape[1];
+  if (cols == 0) return;
+  void *args[] = {&dplan, &splan, &rows, &cols, &scale};
+  gpu_detail::Launch(hip::ReduceKeepLowestKernel<Saver, Reducer, DType, DPlan, SPlan>,
+                     (cols + hip::kLowestCols - 1) / hip::kLowestCols, hip::kRedBlock, args,
+                     Stream<gpu>::GetStream(expr::StreamInfo<gpu, R>::Get(dst->self())));
+#else
+  LOG(FATAL) << "MapReduceKeepLowest<gpu>: compile the calling translation unit with hipcc";
+#endif
+}
+
+template <typename Saver, typename Reducer, int dimkeep, typename R, typename DType, typename E,
+          int etype>
+inline void MapReduceKeepHighDim(TRValue<R, gpu, 1, DType> *dst,
+                                 const expr::Exp<E, DType, etype> &exp, DType scale) {
+  expr::TypeCheckPass<expr::TypeCheck<gpu, dimkeep, DType, E>::kRedPass>::
+      Error_TypeCheck_Not_Pass_For_Reduce_Exp();
+  typedef Shape<expr::ExpInfo<E>::kDim> EShape;
+  EShape eshape = expr::ShapeCheck<expr::ExpInfo<E>::kDim, E>::Check(exp.self());
+  Shape<1> dshape = expr::ShapeCheck<1, R>::Check(dst->self());
+  CHECK_EQ(eshape[dimkeep], dshape[0]) << "MapReduceKeepHighDim::reduction dimension do not match";
+#if defined(__HIPCC__)
+  typedef expr::Plan<R, DType> DPlan;
+  typedef expr::Plan<E, DType> SPlan;
+  DPlan dplan = expr::MakePlan(dst->self());
+  SPlan splan = expr::MakePlan(exp.self());
+  uint32_t n_out = eshape.ProdShape(0, dimkeep), n_keep = eshape[dimkeep];
+  uint32_t n_y = eshape.ProdShape(dimkeep + 1, EShape::kSubdim), n_x = eshape[EShape::kSubdim];
+  if (n_keep == 0) return;
+  void *args[] = {&dplan, &splan, &n_out, &n_keep, &n_y, &n_x, &scale};
+  void *stream = Stream<gpu>::GetStream(expr::StreamInfo<gpu, R>::Get(dst->self()));
+  /* segments staged side by side = chain lanes in use; fewer, longer pieces when the
+     outer extent is small */
+  if (n_out > 16) {
+    gpu_detail::Launch(hip::ReduceKeepHighDimKernel<Saver, Reducer, DType, 64, DPlan, SPlan>,
+                       n_keep, hip::kRedBlock, args, stream);
+  } else if (n_out > 4) {
+    gpu_detail::Launch(hip::ReduceKeepHighDimKernel<Saver, Reducer, DType, 16, DPlan, SPlan>,
+                       n_keep, hip::kRedBlock, args, stream);
+  } else if (n_out > 1) {
+    gpu_detail::Launch(hip::ReduceKeepHighDimKernel<Saver, Reducer, DType, 4, DPlan, SPlan>,
+                       n_keep, hip::kRedBlock, args, stream);
+  } else {
+    gpu_detail::Launch(hip::ReduceKeepHighDimKernel<Saver, Reducer, DType, 1, DPlan, SPlan>,
+                       n_keep, hip::kRedBlock, args, stream);
+  }
+#else
+  LOG(FATAL) << "MapReduceKeepHighDim<gpu>: compile the calling translation unit with hipcc";
+#endif
+}
+
+}  // namespace mshadow
+#endif  // MSHADOW_HIP_TENSOR_GPU_H_

@@ -1,0 +1,125 @@
+/*
+ * mshadow for gfx950: the one header callers include.
+ *
+ *   #include <mshadow/tensor.h>
+ *   Tensor<gpu, 2> dst = ..., a = ..., b = ...;
+ *   dst = a * b + 0.5f * F<sigmoid>(c) - d;     // one HIP kernel, 128-bit accesses
+ *   v   = sumall_except_dim<1>(x4d);            // order-faithful wave64 reduction
+ *   Softmax(p, logits);
+ *
+ * Declarations of the device functions follow mshadow/tensor.h:616-1050 of the
+ * reference (names, template parameter order, default arguments). Definitions:
+ * cpu/tensor_cpu.h for Tensor<cpu>, hip/tensor_gpu.h for Tensor<gpu>. A translation
+ * unit compiled by a host compiler gets memory, copy, stream and the fixed-function
+ * operations for Tensor<gpu> (they live behind the C ABI of libmshadow_hip);
+ * evaluating arbitrary expressions into a Tensor<gpu> needs hipcc, because the
+ * kernel is instantiated from the caller's expression type.
+ */
+#ifndef MSHADOW_TENSOR_H_
+#define MSHADOW_TENSOR_H_
+
+#include <iostream>
+#include <string>
+
+#include "./base.h"
+#include "./core/tensor_types.h"
+#include "./expr/traits.h"
+#include "./expression.h"
+
+namespace mshadow {
+
+/*! \brief select and initialise a device; needed before any GPU tensor operation */
+template <typename Device>
+inline void InitTensorEngine(int device_id = 0);
+/*! \brief counterpart of InitTensorEngine */
+template <typename Device>
+inline void ShutdownTensorEngine(void);
+/*! \brief make devid the calling thread's current device */
+template <typename Device>
+inline void SetDevice(int devid);
+/*! \brief create a computation stream; the two flags ask for BLAS / DNN handles, which
+ *  this backend does not provide (they are accepted and ignored) */
+template <typename Device>
+inline Stream<Device> *NewStream(bool create_blas_handle, bool create_dnn_handle, int dev_id = -1);
+template <typename Device>
+inline Stream<Device> *NewStream(int dev_id) {
+  return NewStream<Device>(true, false, dev_id);
+}
+template <typename Device>
+inline void DeleteStream(Stream<Device> *stream);
+
+/*! \brief allocate obj->dptr_ for obj->shape_; with pad, rows get an aligned pitch */
+template <int dim, typename DType>
+inline void AllocSpace(Tensor<cpu, dim, DType> *obj, bool pad = MSHADOW_ALLOC_PAD);
+template <int dim, typename DType>
+inline void AllocSpace(Tensor<gpu, dim, DType> *obj, bool pad = MSHADOW_ALLOC_PAD);
+template <int dim, typename DType>
+inline void FreeSpace(Tensor<cpu, dim, DType> *obj);
+template <int dim, typename DType>
+inline void FreeSpace(Tensor<gpu, dim, DType> *obj);
+/*! \brief allocate and fill with initv */
+template <typename Device, typename DType, int dim>
+inline Tensor<Device, dim, DType> NewTensor(const Shape<dim> &shape, DType initv,
+                                            bool pad = MSHADOW_ALLOC_PAD,
+                                            Stream<Device> *stream = NULL);
+
+/*! \brief pitch-aware copy between tensors of equal shape, asynchronous on stream for
+ *  the GPU forms (synchronous if stream is NULL and MSHADOW_FORCE_STREAM is 0) */
+template <int dim, typename DType>
+inline void Copy(Tensor<cpu, dim, DType> dst, const Tensor<cpu, dim, DType> &src,
+                 Stream<cpu> *stream = NULL);
+template <int dim, typename DType>
+inline void Copy(Tensor<cpu, dim, DType> dst, const Tensor<gpu, dim, DType> &src,
+                 Stream<gpu> *stream = NULL);
+template <int dim, typename DType>
+inline void Copy(Tensor<gpu, dim, DType> dst, const Tensor<cpu, dim, DType> &src,
+                 Stream<gpu> *stream = NULL);
+template <int dim, typename DType>
+inline void Copy(Tensor<gpu, dim, DType> dst, const Tensor<gpu, dim, DType> &src,
+                 Stream<gpu> *stream = NULL);
+
+/*! \brief dst[y] = softmax(energy[y]) for every row */
+template <typename DType>
+inline void Softmax(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 2, DType> &energy);
+template <typename DType>
+inline void Softmax(Tensor<gpu, 2, DType> dst, const Tensor<gpu, 2, DType> &energy);
+/*! \brief dst = src with 1 subtracted at column label[y] of each row */
+template <typename DType>
+inline void SoftmaxGrad(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 2, DType> &src,
+                        const Tensor<cpu, 1, DType> &label);
+template <typename DType>
+inline void SoftmaxGrad(const Tensor<gpu, 2, DType> &dst, const Tensor<gpu, 2, DType> &src,
+                        const Tensor<gpu, 1, DType> &label);
+
+/*! \brief Saver::Save(dst(y,x), exp(y,x)) for every element */
+template <typename Saver, typename R, int dim, typename DType, typename E, int etype>
+inline void MapExp(TRValue<R, cpu, dim, DType> *dst, const expr::Exp<E, DType, etype> &exp);
+template <typename Saver, typename R, int dim, typename DType, typename E, int etype>
+inline void MapExp(TRValue<R, gpu, dim, DType> *dst, const expr::Exp<E, DType, etype> &exp);
+/*! \brief dst[x] <saver>= scale * reduce over rows of exp(y, x) */
+template <typename Saver, typename Reducer, typename R, typename DType, typename E, int etype>
+inline void MapReduceKeepLowest(TRValue<R, cpu, 1, DType> *dst,
+                                const expr::Exp<E, DType, etype> &exp, DType scale = 1);
+template <typename Saver, typename Reducer, typename R, typename DType, typename E, int etype>
+inline void MapReduceKeepLowest(TRValue<R, gpu, 1, DType> *dst,
+                                const expr::Exp<E, DType, etype> &exp, DType scale = 1);
+/*! \brief dst[c] <saver>= scale * reduce over every dimension but dimkeep */
+template <typename Saver, typename Reducer, int dimkeep, typename R, typename DType, typename E,
+          int etype>
+inline void MapReduceKeepHighDim(TRValue<R, cpu, 1, DType> *dst,
+                                 const expr::Exp<E, DType, etype> &exp, DType scale = 1);
+template <typename Saver, typename Reducer, int dimkeep, typename R, typename DType, typename E,
+          int etype>
+inline void MapReduceKeepHighDim(TRValue<R, gpu, 1, DType> *dst,
+                                 const expr::Exp<E, DType, etype> &exp, DType scale = 1);
+
+}  // namespace mshadow
+
+#include "./expr/engine.h"
+#include "./extension.h"
+#include "./expr/scalar_ops.h"
+#include "./cpu/tensor_cpu.h"
+#include "./hip/tensor_gpu.h"
+#include "./tensor_container.h"
+
+#endif  // MSHADOW_TENSOR_H_

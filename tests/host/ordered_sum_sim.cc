@@ -1,0 +1,174 @@
+// Host check of the order-faithful sum used by the softmax kernel.
+//
+// Emulates one workgroup (W waves x 64 lanes x N terms per lane, slab after slab) with
+// the same decisions the device code takes - per-lane quantisation from
+// mshadow_amd/csrc/ordered_sum.h, wave totals, the block scan for the first rejected
+// wave, the lane scan inside it, real float adds for the rejected lane - and compares the
+// result with a plain serial float loop, bit for bit, on rows built to hit every branch:
+// softmax-like terms, ties, huge dynamic range, leading zeros, subnormals, inf / NaN.
+// Prints "OK <cases>" and exits 0 on success.
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <random>
+#include <vector>
+
+#include "../../mshadow_amd/csrc/ordered_sum.h"
+
+using namespace ordered_sum;
+
+static float Serial(const std::vector<float> &t) {
+  volatile float s = 0.0f;
+  for (float v : t) s = s + v;
+  return s;
+}
+
+template <int N>
+static float WaveResolveSim(float s, const float (*t)[N]) {  // t[64][N]
+  int start = 0;
+  while (true) {
+    Binade b = BinadeOf(s);
+    uint32_t q[64], incl[64];
+    uint32_t run = 0;
+    for (int l = 0; l < 64; ++l) {
+      q[l] = (l >= start) ? LaneQuant<N>(t[l], b) : 0u;
+      run += q[l];
+      incl[l] = run;
+    }
+    int first = -1;
+    for (int l = start; l < 64; ++l) {
+      if (b.m + incl[l] >= kBig) { first = l; break; }
+    }
+    if (first < 0) return Accept(s, b, incl[63]);
+    s = Accept(s, b, incl[first] - q[first]);
+    s = TrueAdd<N>(s, t[first]);
+    start = first + 1;
+    if (start == 64) return s;
+  }
+}
+
+template <int W, int N>
+static float BlockAddSim(float s, const float (*t)[N], long *resolves) {  // t[W*64][N]
+  int pos = 0;
+  while (true) {
+    Binade b = BinadeOf(s);
+    uint32_t qw[W];
+    for (int w = pos; w < W; ++w) {
+      uint32_t q = 0;
+      for (int l = 0; l < 64; ++l) q += LaneQuant<N>(t[w * 64 + l], b);
+      qw[w] = q < kBig ? q : kBig;
+    }
+    uint32_t acc = 0;
+    int failw = W;
+    for (int w = pos; w < W; ++w) {
+      if (b.m + acc + qw[w] >= kBig) { failw = w; break; }
+      acc += qw[w];
+    }
+    s = Accept(s, b, acc);
+    if (failw == W) return s;
+    s = WaveResolveSim<N>(s, t + failw * 64);
+    ++*resolves;
+    pos = failw + 1;
+    if (pos == W) return s;
+  }
+}
+
+template <int W, int N>
+static bool Check(const std::vector<float> &row, const char *name, long *resolves) {
+  const int slab = W * 64 * N;
+  std::vector<float> padded(row);
+  while (padded.size() % slab) padded.push_back(0.0f);
+  float s = 0.0f;
+  for (size_t off = 0; off < padded.size(); off += slab) {
+    s = BlockAddSim<W, N>(s, reinterpret_cast<const float(*)[N]>(padded.data() + off), resolves);
+  }
+  const float want = Serial(row);
+  if (BitsOf(s) != BitsOf(want) && !(std::isnan(s) && std::isnan(want))) {
+    fprintf(stderr, "MISMATCH %s W=%d N=%d n=%zu got %a want %a\n", name, W, N, row.size(), s, want);
+    return false;
+  }
+  return true;
+}
+
+static bool CheckAll(const std::vector<float> &row, const char *name, long *resolves) {
+  return Check<8, 4>(row, name, resolves) && Check<4, 4>(row, name, resolves) &&
+         Check<16, 4>(row, name, resolves) && Check<4, 1>(row, name, resolves) &&
+         Check<1, 4>(row, name, resolves);
+}
+
+int main() {
+  std::mt19937 rng(1234);
+  std::normal_distribution<float> normal(0.0f, 1.0f);
+  std::uniform_real_distribution<float> uni(0.0f, 1.0f);
+  long cases = 0, resolves = 0;
+  bool ok = true;
+  // 1. softmax-like rows: exp(x - max), x ~ N(0, sigma)
+  for (float sigma : {0.1f, 1.0f, 3.0f, 10.0f, 40.0f}) {
+    for (int n : {1, 3, 64, 257, 1000, 4096, 32000}) {
+      for (int rep = 0; rep < 6; ++rep) {
+        std::vector<float> x(n);
+        float mx = -INFINITY;
+        for (auto &v : x) { v = normal(rng) * sigma; mx = std::fmax(mx, v); }
+        for (auto &v : x) v = expf(v - mx);
+        ok = CheckAll(x, "softmax", &resolves) && ok;
+        ++cases;
+      }
+    }
+  }
+  // 2. grids that produce exact ties: multiples of 2^-k around a sum near powers of two
+  for (int rep = 0; rep < 200; ++rep) {
+    int n = 1 + rng() % 3000;
+    std::vector<float> x(n);
+    for (auto &v : x) v = std::ldexp(static_cast<float>(rng() % 64), -static_cast<int>(rng() % 30));
+    ok = CheckAll(x, "ties", &resolves) && ok;
+    ++cases;
+  }
+  // 3. all equal (sum of ones is exact below 2^24, then sticks), and constants
+  for (float c : {1.0f, 0.5f, 3.0f, 1e-3f, 0.1f}) {
+    std::vector<float> x(40000, c);
+    ok = CheckAll(x, "const", &resolves) && ok;
+    ++cases;
+  }
+  // 4. leading zeros / subnormals / tiny then large; ascending and descending magnitudes
+  for (int rep = 0; rep < 60; ++rep) {
+    int n = 500 + rng() % 5000;
+    std::vector<float> x(n);
+    for (int i = 0; i < n; ++i) {
+      float e = -140.0f + 150.0f * i / n;  // 2^-140 .. 2^10
+      x[i] = std::ldexp(1.0f + uni(rng), static_cast<int>(e));
+      if (rng() % 7 == 0) x[i] = 0.0f;
+    }
+    if (rep % 3 == 1) std::reverse(x.begin(), x.end());
+    if (rep % 3 == 2) std::shuffle(x.begin(), x.end(), rng);
+    ok = CheckAll(x, "range", &resolves) && ok;
+    ++cases;
+  }
+  {
+    std::vector<float> x(3000, 0.0f);
+    ok = CheckAll(x, "zeros", &resolves) && ok;
+    x[2999] = 1e-40f;
+    ok = CheckAll(x, "zeros+denorm", &resolves) && ok;
+    x[10] = 3e-42f;
+    ok = CheckAll(x, "denorms", &resolves) && ok;
+    x[1500] = INFINITY;
+    ok = CheckAll(x, "inf", &resolves) && ok;
+    x[100] = NAN;
+    ok = CheckAll(x, "nan", &resolves) && ok;
+    x.assign(5000, 3.0e38f);  // overflow to inf on the way
+    ok = CheckAll(x, "overflow", &resolves) && ok;
+    cases += 6;
+  }
+  // 5. uniform magnitudes (binade crossings spread over the whole row)
+  for (int rep = 0; rep < 40; ++rep) {
+    int n = 20000 + rng() % 20000;
+    std::vector<float> x(n);
+    for (auto &v : x) v = uni(rng);
+    ok = CheckAll(x, "uniform", &resolves) && ok;
+    ++cases;
+  }
+  if (!ok) return 1;
+  printf("OK %ld cases, %ld wave resolves\n", cases, resolves);
+  return 0;
+}

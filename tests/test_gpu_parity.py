@@ -1,0 +1,408 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle.
+
+Every test feeds the same seeded arrays to the oracle (oracle/liboracle.so, and the
+reference-built library where it is present) and to the GPU. Two GPU routes are checked:
+the fixed-function entry points of libmshadow_hip.so (include/mshadow_hip.h) and the C++
+expression API (Tensor<gpu> expressions compiled in libmshadow_cases.so), the latter both
+on the recognised fast path (variant 0) and through the generic expression kernel
+(variant 1).
+
+Bars: bit-exact for the elementwise map, pool / unpool, patch2col / col2patch, the
+softmax gradient and - because the kernels keep the CPU path's order of additions - the
+reductions. Softmax forward is compared at relative 1e-5 (the tolerance of the task);
+its only source of difference is expf (libm on the host, the device math library here).
+"""
+import numpy as np
+import pytest
+
+from checkers import DIVTO, MAX, MIN, MINUSTO, MULTO, PLUSTO, SAVETO, SUM, Checker, have_ref
+from gpu_util import assert_bits_equal, f32, host_padded, normal, uniform
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def G():
+    import mshadow_amd
+    g = mshadow_amd.load_cases()
+    assert g.device_count() >= 1, "no GPU visible"
+    g.set_device(0)
+    return g
+
+
+@pytest.fixture(scope="module")
+def stream(G):
+    s = G.stream_create()
+    yield s
+    G.stream_destroy(s)
+
+
+@pytest.fixture(scope="module")
+def O():
+    return Checker("orc")
+
+
+def test_device_is_gfx950(G):
+    p = G.props(0)
+    assert b"gfx950" in p.arch, p.arch
+    assert p.wavefront_size == 64
+    print("device:", p.name.decode(), p.arch.decode(), "CUs", p.compute_units, "LDS/block",
+          p.lds_bytes_per_block)
+
+
+def test_reference_library_agrees_with_oracle_on_this_host(O):
+    """The reference-built checker travels as a binary; make sure it still matches here."""
+    if not have_ref():
+        pytest.skip("oracle/_ref not present")
+    R = Checker("ref")
+    a, b, c, d = (uniform(100 + i, (64, 257)) for i in range(4))
+    o1, o2 = np.empty_like(a), np.empty_like(a)
+    O.map_fused(o1, a, b, c, d)
+    R.map_fused(o2, a, b, c, d)
+    assert_bits_equal(o1, o2, "ref vs oracle map")
+    x = normal(104, (16, 4000), 3.0)
+    s1, s2 = np.empty_like(x), np.empty_like(x)
+    O.softmax(s1, x)
+    R.softmax(s2, x)
+    assert_bits_equal(s1, s2, "ref vs oracle softmax")
+
+
+# ------------------------------------------------------------------ copy / alloc
+@pytest.mark.parametrize("shape,pad", [((7, 55), 0), ((7, 55), 1), ((33, 64), 1), ((3, 1000), 1),
+                                       ((1, 5), 1)])
+def test_copy_roundtrip_and_pitch(G, shape, pad):
+    a = uniform(1, shape)
+    out, stride = G.case_copy_roundtrip(a, pad)
+    assert_bits_equal(out, a, "copy round trip")
+    if pad and shape[1] >= 64:
+        assert stride % 64 == 0 and stride >= shape[1]  # 256-byte pitch
+    else:
+        assert stride == shape[1]
+
+
+# ------------------------------------------------------------------ elementwise map
+MAP_SHAPES = [((4096 // 8, 4096 // 8), 0), ((257, 515), 0), ((257, 516), 4), ((33, 7), 1),
+              ((1, 1), 0), ((5, 1024), 0), ((129, 260), 12)]
+
+
+@pytest.mark.parametrize("shape,pad", MAP_SHAPES)
+@pytest.mark.parametrize("saver", [SAVETO, PLUSTO, MINUSTO, MULTO, DIVTO])
+def test_map_fused(G, O, stream, shape, pad, saver):
+    a, b, c, d = (uniform(10 + i, shape) for i in range(4))
+    start = np.random.default_rng(14).uniform(1, 2, shape).astype(f32)
+    want = host_padded(start, pad)
+    O.map_fused(want, host_padded(a, pad), host_padded(b, pad), host_padded(c, pad),
+                host_padded(d, pad), saver)
+    da, db, dc, dd = (G.to_device(t, pad) for t in (a, b, c, d))
+    dst = G.to_device(start, pad)
+    G.case_map_fused(dst, da, db, dc, dd, saver, stream)
+    assert_bits_equal(dst.download(stream), want, f"map {shape} pad {pad} saver {saver}")
+
+
+def test_map_mixed_strides_and_misaligned_pointer(G, O, stream):
+    """Leaves with different pitches (pack kernel, row-indexed) and an odd column count
+    (scalar kernel)."""
+    for shape, pads in (((64, 256), (0, 4, 8, 12, 16)), ((64, 255), (0, 1, 2, 3, 0))):
+        a, b, c, d = (uniform(20 + i, shape) for i in range(4))
+        want = np.empty(shape, f32)
+        O.map_fused(want, a, b, c, d)
+        bufs = [G.to_device(t, p) for t, p in zip((a, b, c, d), pads[:4])]
+        dst = G.buffer(shape, f32, pads[4])
+        G.case_map_fused(dst, *bufs, SAVETO, stream)
+        assert_bits_equal(dst.download(stream), want, f"mixed strides {shape}")
+
+
+@pytest.mark.parametrize("saver", [SAVETO, PLUSTO, MULTO, DIVTO])
+def test_map_scalar_and_axpb(G, O, stream, saver):
+    shape = (37, 300)
+    start = uniform(30, shape) + f32(2)
+    a = uniform(31, shape)
+    want = start.copy()
+    O.map_scalar(want, 1.7, saver)
+    dst = G.to_device(start, 4)
+    G.case_map_scalar(dst, 1.7, saver, stream)
+    assert_bits_equal(dst.download(stream), want, "scalar rhs")
+    want = start.copy()
+    O.map_axpb(want, a, 10.0, 3.0, 2.0, saver)
+    dst = G.to_device(start, 0)
+    G.case_map_axpb(dst, G.to_device(a), 10.0, 3.0, 2.0, saver, stream)
+    assert_bits_equal(dst.download(stream), want, "axpb")
+
+
+def test_map_shape_mismatch_is_an_error(G, stream):
+    from mshadow_amd import HipError
+    a = G.to_device(uniform(1, (4, 8)))
+    dst = G.buffer((4, 8), f32)
+    # lie about the shape of dst through the raw entry: rows differ between dst and sources
+    import ctypes as C
+    st = G.cases.mshadow_case_softmax_f32(dst.ptr, 8, a.ptr, 8, 4, 8, stream)
+    assert st == 0
+    with pytest.raises(HipError):
+        G.check(G.dll.mshadow_hip_softmax_f32(dst.ptr, 4, a.ptr, 8, 4, 8, stream))  # pitch < cols
+
+
+# ------------------------------------------------------------------ reductions
+LOWEST_SHAPES = [((16384 // 8, 4096 // 8), 0), ((1000, 37), 3), ((1, 130), 0), ((257, 16), 0),
+                 ((255, 1), 1), ((4097, 48), 0)]
+
+
+@pytest.mark.parametrize("shape,pad", LOWEST_SHAPES)
+@pytest.mark.parametrize("reducer", [SUM, MAX, MIN])
+@pytest.mark.parametrize("route", ["abi", "expr", "expr_generic"])
+def test_reduce_keep_lowest(G, O, stream, shape, pad, reducer, route):
+    m = normal(40, shape)
+    for saver, scale in ((SAVETO, 1.0), (PLUSTO, 0.75)):
+        start = uniform(41, (shape[1],)) + f32(2)
+        want = start.copy()
+        O.reduce_keep_lowest(want, host_padded(m, pad), reducer, saver, scale)
+        dst = G.to_device(start)
+        src = G.to_device(m, pad)
+        if route == "abi":
+            G.reduce_keep_lowest(dst, src, reducer, saver, scale, stream)
+        else:
+            G.case_reduce_keep_lowest(dst, src, reducer, saver, scale,
+                                      1 if route == "expr_generic" else 0, stream)
+        assert_bits_equal(dst.download(stream), want, f"keep_lowest {shape} {route}")
+
+
+HIGH_SHAPES = [((8, 32, 56, 56), 0), ((64, 5, 7, 9), 2), ((3, 4, 5, 6), 0), ((1, 3, 2, 4), 0),
+               ((70, 3, 1, 1), 0), ((17, 2, 33, 65), 3), ((2, 2, 70, 70), 0)]
+
+
+@pytest.mark.parametrize("shape,pad", HIGH_SHAPES)
+@pytest.mark.parametrize("reducer", [SUM, MAX, MIN])
+@pytest.mark.parametrize("route", ["abi", "expr", "expr_generic"])
+def test_reduce_keep_highdim(G, O, stream, shape, pad, reducer, route):
+    x = normal(50, shape)
+    for saver, scale in ((SAVETO, 1.0), (MINUSTO, 1.25)):
+        start = uniform(51, (shape[1],)) + f32(2)
+        want = start.copy()
+        O.reduce_keep_highdim(want, host_padded(x, pad), reducer, saver, scale)
+        dst = G.to_device(start)
+        src = G.to_device(x, pad)
+        if route == "abi":
+            G.reduce_keep_highdim(dst, src, reducer, saver, scale, stream)
+        else:
+            G.case_reduce_keep_highdim(dst, src, reducer, saver, scale,
+                                       1 if route == "expr_generic" else 0, stream)
+        assert_bits_equal(dst.download(stream), want, f"keep_highdim {shape} {route}")
+
+
+def test_reduce_reference_known_answers(G, stream):
+    # test/test.cu:9-18,35,47 of the reference
+    i, j, k = np.meshgrid(np.arange(3), np.arange(2), np.arange(4), indexing="ij")
+    tc = (f32(0.1) * i.astype(f32) + f32(0.2) * j.astype(f32) + f32(0.1) * k.astype(f32))
+    out = G.buffer((4,), f32)
+    G.case_reduce_keep_lowest(out, G.to_device(tc[0]), SUM, SAVETO, 1.0, 0, stream)
+    assert np.allclose(out.download(stream), [0.2, 0.4, 0.6, 0.8], atol=1e-4)
+    out3 = G.buffer((3,), f32)
+    G.case_reduce_keep_highdim(out3, G.to_device(tc.reshape(1, 3, 2, 4)), SUM, SAVETO, 1.0, 0,
+                               stream)
+    assert np.allclose(out3.download(stream), [2.0, 2.8, 3.6], atol=1e-4)
+
+
+# ------------------------------------------------------------------ softmax
+SOFTMAX_SHAPES = [((64, 32000), 0), ((5, 1000), 0), ((5, 1001), 0), ((3, 7), 1), ((9, 2048), 4),
+                  ((4, 8192), 0), ((3, 16384), 0), ((2, 40000), 0), ((2, 70001), 0), ((7, 1), 0),
+                  ((3, 5000), 3), ((2, 20000), 1)]
+
+
+def _softmax_check(got, want, src):
+    rel = np.abs(got.astype(np.float64) - want) / np.maximum(want, np.finfo(f32).tiny)
+    mask = want > 0
+    assert np.all(got[~mask] == 0) or np.allclose(got[~mask], want[~mask], atol=1e-44)
+    worst = rel[mask].max() if mask.any() else 0.0
+    assert worst <= 1e-5, f"softmax relative error {worst:.3e} > 1e-5 (tolerance of the task)"
+    return worst
+
+
+@pytest.mark.parametrize("shape,pad", SOFTMAX_SHAPES)
+def test_softmax_forward(G, O, stream, shape, pad):
+    x = normal(60, shape, 3.0)
+    want = np.empty(shape, f32)
+    O.softmax(want, x)
+    src = G.to_device(x, pad)
+    dst = G.buffer(shape, f32, pad)
+    G.softmax(dst, src, stream)
+    got = dst.download(stream)
+    worst = _softmax_check(got, want, x)
+    # through Softmax(Tensor<gpu,2>, Tensor<gpu,2>) and in place
+    G.case_softmax(src, src, stream)
+    assert_bits_equal(src.download(stream), got, "in-place softmax via the C++ API")
+    print(f"softmax {shape} pad {pad}: worst relative difference to the CPU path {worst:.2e}")
+
+
+def test_softmax_exact_cases(G, stream):
+    # uniform logits: exp(0) = 1 exactly, the sum of n ones is exact, so every output is 1/n
+    for n in (4, 7, 1000, 32000):
+        x = np.full((3, n), 0.37, f32)
+        dst = G.buffer(x.shape, f32)
+        G.softmax(dst, G.to_device(x), stream)
+        assert np.all(dst.download(stream) == f32(1.0) / f32(n))
+    # a row of distinct powers of two in exp-space is too contrived; instead: the row sum
+    # the kernel used must be the left-to-right float sum of ITS OWN exponentials.
+    x = normal(61, (8, 32000), 3.0)
+    dst = G.buffer(x.shape, f32)
+    G.softmax(dst, G.to_device(x), stream)
+    got = dst.download(stream)
+    for y in range(8):
+        k = int(np.argmax(x[y]))
+        s = f32(1.0) / got[y, k]          # exp(0) / sum
+        # reconstruct p_i = got_i * s only approximately; the check is on the order effect:
+        p = np.exp((x[y] - x[y].max()).astype(np.float64))
+        exact = p.sum()
+        seq_bias = (float(s) - exact) / exact
+        # the sequential float sum sits ~2.6e-5 below the exact sum on this distribution;
+        # a tree sum would sit within 1e-6 of it
+        assert -6e-5 < seq_bias < -5e-6, seq_bias
+
+
+def test_softmax_extreme_rows(G, O, stream):
+    rows = [
+        np.linspace(-200, 0, 5000),          # long underflowing head (leading zeros)
+        np.linspace(0, -200, 5000),
+        np.concatenate([np.full(10, -1e30), [0.0], np.full(300, -90.0)]),  # denormal terms
+        np.full(777, -3.0e38),               # all equal, huge magnitude
+        np.r_[np.zeros(4000), 50.0],         # sum dominated by the last term
+    ]
+    for r in rows:
+        x = np.asarray(r, dtype=f32)[None, :]
+        want = np.empty_like(x)
+        O.softmax(want, x)
+        dst = G.buffer(x.shape, f32)
+        G.softmax(dst, G.to_device(x), stream)
+        got = dst.download(stream)
+        big = want > 1e-30
+        rel = np.abs(got[big].astype(np.float64) - want[big]) / want[big]
+        assert rel.max() <= 1e-5
+        assert np.all(np.abs(got[~big].astype(np.float64) - want[~big]) <= 1e-35)
+
+
+@pytest.mark.parametrize("shape,pad", [((64, 32000), 0), ((9, 1001), 0), ((9, 1000), 4),
+                                       ((5, 7), 1), ((3, 20000), 0)])
+def test_softmax_grad(G, O, stream, shape, pad):
+    rng = np.random.default_rng(62)
+    p = rng.uniform(0, 1, shape).astype(f32)
+    label = rng.integers(0, shape[1], shape[0]).astype(f32)
+    if shape[0] > 4:
+        label[1], label[2], label[3] = shape[1] + 5, -3.0, 0.9
+    want = np.empty(shape, f32)
+    O.softmax_grad(want, p, label)
+    for route in ("abi", "expr"):
+        dst = G.buffer(shape, f32, pad)
+        args = (dst, G.to_device(p, pad), G.to_device(label))
+        (G.softmax_grad if route == "abi" else G.case_softmax_grad)(*args, stream)
+        assert_bits_equal(dst.download(stream), want, f"softmax_grad {shape} {route}")
+
+
+# ------------------------------------------------------------------ pool / unpool
+POOL_CASES = [  # planes, h, w, ky, kx, sy, sx, pad
+    (16, 112, 112, 3, 3, 2, 2, 0), (6, 37, 41, 3, 3, 2, 2, 2), (6, 37, 41, 2, 2, 2, 2, 0),
+    (3, 9, 11, 3, 2, 1, 3, 1), (2, 30, 30, 5, 5, 3, 2, 0), (4, 6, 6, 1, 1, 1, 1, 0),
+    (2, 7, 300, 7, 3, 1, 2, 0), (1, 3, 20000, 2, 2, 1, 2, 0),
+]
+
+
+@pytest.mark.parametrize("case", POOL_CASES)
+@pytest.mark.parametrize("reducer", [MAX, MIN, SUM])
+@pytest.mark.parametrize("variant", [0, 1])
+def test_pool_unpool(G, O, stream, case, reducer, variant):
+    planes, h, w, ky, kx, sy, sx, pad = case
+    if variant == 1 and w > 1000:
+        pytest.skip("generic route covered by the smaller shapes")
+    rng = np.random.default_rng(70 + h + w)
+    # a coarse value grid makes duplicated maxima common, which equality routing must honour
+    src = (rng.integers(-8, 9, (planes, h, w)).astype(f32) / f32(8)) if h < 100 else \
+        uniform(71, (planes, h, w))
+    ph, pw = (h - ky) // sy + 1, (w - kx) // sx + 1
+    want = np.empty((planes, ph, pw), f32)
+    O.pool(want, host_padded(src, pad), ky, kx, sy, sx, reducer)
+    dsrc = G.to_device(src, pad)
+    dpool = G.buffer((planes, ph, pw), f32, pad)
+    G.case_pool(dpool, dsrc, ky, kx, sy, sx, reducer, variant, stream)
+    assert_bits_equal(dpool.download(stream), want, f"pool {case}")
+    grad = normal(72, (planes, ph, pw))
+    wantu = np.empty((planes, h, w), f32)
+    O.unpool(wantu, src, want, grad, ky, kx, sy, sx, reducer)
+    dgrad = G.to_device(grad, pad)
+    dun = G.buffer((planes, h, w), f32, pad)
+    G.case_unpool(dun, dsrc, dpool, dgrad, ky, kx, sy, sx, reducer, variant, stream)
+    assert_bits_equal(dun.download(stream), wantu, f"unpool {case}")
+    if variant == 0:  # and straight through the C ABI
+        d2 = G.buffer((planes, ph, pw), f32)
+        G.pool(d2, dsrc, ky, kx, sy, sx, reducer, stream)
+        assert_bits_equal(d2.download(stream), want, "pool abi")
+        u2 = G.buffer((planes, h, w), f32)
+        G.unpool(u2, dsrc, dpool, dgrad, ky, kx, sy, sx, reducer, stream)
+        assert_bits_equal(u2.download(stream), wantu, "unpool abi")
+
+
+def test_pool_reference_known_answers(G, stream):
+    # test/pool.cu:29-48 of the reference: 6x6 0.1i+0.1j, 2x2 stride 2 -> src[2a+1][2b+1]
+    i, j = np.meshgrid(np.arange(6), np.arange(6), indexing="ij")
+    src = (i.astype(f32) * f32(0.1) + j.astype(f32) * f32(0.1)).reshape(1, 6, 6)
+    out = G.buffer((1, 3, 3), f32)
+    G.case_pool(out, G.to_device(src), 2, 2, 2, 2, MAX, 0, stream)
+    assert np.array_equal(out.download(stream)[0], src[0, 1::2, 1::2])
+    # explicit pooled shape larger than natural: windows past the edge keep -FLT_MAX
+    out = G.buffer((1, 4, 4), f32)
+    G.pool(out, G.to_device(src), 2, 2, 2, 2, MAX, stream)
+    got = out.download(stream)
+    assert np.array_equal(got[0, :3, :3], src[0, 1::2, 1::2])
+    assert np.all(got[0, 3, :] == -np.finfo(f32).max) and np.all(got[0, :, 3] == -np.finfo(f32).max)
+
+
+# ------------------------------------------------------------------ im2col / col2im
+CONV = [  # n, c, h, w, ky, kx, sy, sx, dy, dx, py, px
+    (2, 16, 56, 56, 3, 3, 1, 1, 1, 1, 1, 1), (3, 5, 19, 23, 3, 3, 2, 2, 1, 1, 0, 0),
+    (3, 5, 19, 23, 5, 3, 2, 1, 1, 1, 2, 1), (2, 3, 19, 23, 3, 3, 1, 1, 2, 2, 2, 2),
+    (2, 3, 9, 8, 2, 3, 1, 2, 2, 2, 1, 0), (1, 1, 6, 6, 3, 3, 2, 2, 1, 1, 0, 0),
+    (2, 4, 7, 7, 1, 1, 1, 1, 1, 1, 0, 0), (1, 2, 30, 31, 7, 7, 3, 3, 1, 1, 3, 3),
+]
+
+
+@pytest.mark.parametrize("cfg", CONV)
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("variant", [0, 1])
+def test_im2col_col2im(G, O, stream, cfg, dtype, variant):
+    n, c, h, w, ky, kx, sy, sx, dy, dx, py, px = cfg
+    shape = Checker.col_shape(n, c, h, w, ky, kx, sy, sx, dy, dx, py, px)
+    imgf = uniform(80, (n, c, h, w))
+    colf = normal(81, shape)
+    if dtype == "f16":
+        img, colin, dt = O.float2half(imgf), O.float2half(colf), np.uint16
+    else:
+        img, colin, dt = imgf, colf, f32
+    for pad in (0, 3):
+        want = np.empty(shape, dt)
+        O.im2col(want, img, ky, kx, sy, sx, dy, dx, py, px)
+        dcol = G.buffer(shape, dt, pad)
+        G.case_im2col(dcol, G.to_device(img, pad), ky, kx, sy, sx, dy, dx, py, px, variant, stream)
+        assert_bits_equal(dcol.download(stream), want, f"im2col {cfg} {dtype} pad {pad}")
+        wanti = np.empty((n, c, h, w), dt)
+        O.col2im(wanti, colin, ky, kx, sy, sx, dy, dx, py, px)
+        dimg = G.buffer((n, c, h, w), dt, pad)
+        G.case_col2im(dimg, G.to_device(colin, pad), ky, kx, sy, sx, dy, dx, py, px, variant,
+                      stream)
+        assert_bits_equal(dimg.download(stream), wanti, f"col2im {cfg} {dtype} pad {pad}")
+    if variant == 0:
+        dcol = G.buffer(shape, dt)
+        G.im2col(dcol, G.to_device(img), ky, kx, sy, sx, dy, dx, py, px, stream)
+        assert_bits_equal(dcol.download(stream), want, "im2col abi")
+        dimg = G.buffer((n, c, h, w), dt)
+        G.col2im(dimg, G.to_device(colin), ky, kx, sy, sx, dy, dx, py, px, stream)
+        assert_bits_equal(dimg.download(stream), wanti, "col2im abi")
+
+
+def test_im2col_reference_known_answer(G, stream):
+    # test/unpack.cu:29-59 of the reference
+    i, j = np.meshgrid(np.arange(6), np.arange(6), indexing="ij")
+    img = (i.astype(f32) * f32(0.1) + j.astype(f32) * f32(0.2)).reshape(1, 1, 6, 6)
+    col = G.buffer((9, 4), f32)
+    G.case_im2col(col, G.to_device(img), 3, 3, 2, 2, 1, 1, 0, 0, 0, stream)
+    got = col.download(stream)
+    for ky in range(3):
+        for kx in range(3):
+            for oy in range(2):
+                for ox in range(2):
+                    assert got[ky * 3 + kx, oy * 2 + ox] == img[0, 0, 2 * oy + ky, 2 * ox + kx]
