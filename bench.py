@@ -1,0 +1,277 @@
+#!/usr/bin/env python3
+"""Benchmark of the mshadow hot path on one MI355X.
+
+A step is one pass of the nine hot-path operations over one batch of synthetic inputs of
+the shapes named in BASELINE.json (configs 1-5): fused elementwise map, the two
+reduce-to-1D forms, softmax forward and gradient, max-pool and its backward, im2col and
+col2im. Inputs are generated once from fixed seeds and are resident in HBM before the
+timed region; every operation is queued on one stream through the C ABI (the elementwise
+map through the C++ expression API compiled in libmshadow_cases.so).
+
+Output: one JSON line. `value` is the whole-step effective bandwidth: algorithmic bytes
+(each tensor counted once, table in BASELINE.md) of all nine operations divided by the
+step time. `per_op` lists each operation's own GB/s, fraction of the 8 TB/s HBM peak and
+GElem/s from HIP events recorded around it on the same stream. `roofline` describes the
+kernel that takes the largest share of the step. `cpu_baseline` times the reference CPU
+path (oracle/_ref, the reference's own headers) or, where that library is absent, the C
+restatement, on the host cores of the same machine over the same inputs.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+f32 = np.float32
+
+
+def algorithmic_bytes():
+    """Compulsory traffic per operation: every tensor once."""
+    e = 4
+    return {
+        "map_fused": 5 * e * 4096 * 4096,
+        "sumall_except_dim1": e * 64 * 256 * 56 * 56 + e * 256,
+        "sum_rows": e * 16384 * 4096 + e * 4096,
+        "softmax": 2 * e * 8192 * 32000,
+        "softmax_grad": 2 * e * 8192 * 32000 + e * 8192,
+        "pool_max": e * 128 * 64 * 112 * 112 + e * 128 * 64 * 55 * 55,
+        "unpool_max": 2 * e * 128 * 64 * 112 * 112 + 2 * e * 128 * 64 * 55 * 55,
+        "im2col_f16": 2 * 32 * 256 * 56 * 56 + 2 * 2304 * 100352,
+        "col2im_f16": 2 * 32 * 256 * 56 * 56 + 2 * 2304 * 100352,
+    }
+
+
+def work_elements():
+    return {
+        "map_fused": 4096 * 4096, "sumall_except_dim1": 64 * 256 * 56 * 56,
+        "sum_rows": 16384 * 4096, "softmax": 8192 * 32000, "softmax_grad": 8192 * 32000,
+        "pool_max": 128 * 64 * 55 * 55, "unpool_max": 128 * 64 * 112 * 112,
+        "im2col_f16": 2304 * 100352, "col2im_f16": 2304 * 100352,
+    }
+
+
+OPS = list(algorithmic_bytes().keys())
+
+
+def make_inputs(scale=1):
+    """Seeded synthetic inputs of the BASELINE shapes (scale > 1 shrinks the leading
+    dimension for quick functional runs; the reported benchmark uses scale 1)."""
+    def rng(seed):
+        return np.random.default_rng(seed)
+    s = scale
+    d = {}
+    d["A"], d["B"], d["C"], d["D"] = (rng(i).uniform(-1, 1, (4096 // s, 4096)).astype(f32)
+                                      for i in (1, 2, 3, 4))
+    d["X2a"] = rng(5).standard_normal((64 // s, 256, 56, 56), dtype=f32)
+    d["M2b"] = rng(6).standard_normal((16384 // s, 4096), dtype=f32)
+    d["L"] = rng(7).standard_normal((8192 // s, 32000), dtype=f32) * f32(3)
+    d["labels"] = rng(8).integers(0, 32000, 8192 // s).astype(f32)
+    d["X4"] = rng(9).uniform(-1, 1, (128 // s, 64, 112, 112)).astype(f32)
+    d["G4"] = rng(10).standard_normal((128 // s, 64, 55, 55), dtype=f32)
+    return d
+
+
+def half_inputs(orc, scale=1):
+    s = scale
+    img = orc.float2half(np.random.default_rng(11).uniform(-1, 1, (32 // s, 256, 56, 56)).astype(f32))
+    colshape = (2304, (32 // s) * 56 * 56)
+    col = orc.float2half(np.random.default_rng(12).standard_normal(colshape, dtype=f32))
+    return img, col
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--scale", type=int, default=1, help="shrink leading dims (functional runs)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-reps", type=int, default=3)
+    ap.add_argument("--only", default="", help="comma list of ops to run (profiling aid)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU; every operation of the path runs at its "
+                 "full shape on one MI355X and nothing is sharded (--gpus must be 1)")
+
+    import mshadow_amd
+    from checkers import Checker, have_ref
+    G = mshadow_amd.load_cases()
+    if G.device_count() < 1:
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+    G.set_device(0)
+    props = G.props(0)
+    orc = Checker("orc")
+    only = [o for o in args.only.split(",") if o] or OPS
+
+    t0 = time.time()
+    H = make_inputs(args.scale)
+    img_h, col_h = half_inputs(orc, args.scale)
+    gen_s = time.time() - t0
+
+    s = G.stream_create()
+    dev = {k: G.to_device(v) for k, v in H.items()}
+    dimg, dcol_in = G.to_device(img_h), G.to_device(col_h)
+    out_map = G.buffer(H["A"].shape, f32)
+    out_2a = G.buffer((256,), f32)
+    out_2b = G.buffer((4096,), f32)
+    out_p = G.buffer(H["L"].shape, f32)
+    out_g = G.buffer(H["L"].shape, f32)
+    out_pool = G.buffer(H["G4"].shape, f32)
+    out_unpool = G.buffer(H["X4"].shape, f32)
+    out_col = G.buffer(col_h.shape, np.uint16)
+    out_img = G.buffer(img_h.shape, np.uint16)
+
+    def run_op(name):
+        if name == "map_fused":
+            G.case_map_fused(out_map, dev["A"], dev["B"], dev["C"], dev["D"], 0, s)
+        elif name == "sumall_except_dim1":
+            G.reduce_keep_highdim(out_2a, dev["X2a"], stream=s)
+        elif name == "sum_rows":
+            G.reduce_keep_lowest(out_2b, dev["M2b"], stream=s)
+        elif name == "softmax":
+            G.softmax(out_p, dev["L"], s)
+        elif name == "softmax_grad":
+            G.softmax_grad(out_g, out_p, dev["labels"], s)
+        elif name == "pool_max":
+            G.pool(out_pool, dev["X4"], 3, 3, 2, 2, stream=s)
+        elif name == "unpool_max":
+            G.unpool(out_unpool, dev["X4"], out_pool, dev["G4"], 3, 3, 2, 2, stream=s)
+        elif name == "im2col_f16":
+            G.im2col(out_col, dimg, 3, 3, 1, 1, 1, 1, 1, 1, s)
+        elif name == "col2im_f16":
+            G.col2im(out_img, dcol_in, 3, 3, 1, 1, 1, 1, 1, 1, s)
+
+    # softmax_grad / unpool consume the outputs of softmax / pool: make them valid first
+    G.softmax(out_p, dev["L"], s)
+    G.pool(out_pool, dev["X4"], 3, 3, 2, 2, stream=s)
+    for _ in range(args.warmup):
+        for name in only:
+            run_op(name)
+    G.stream_sync(s)
+    G.device_sync()
+
+    nev = len(only) + 1
+    events = [[G.event_create() for _ in range(nev)] for _ in range(args.steps)]
+    G.device_sync()
+    wall0 = time.perf_counter()
+    for k in range(args.steps):
+        G.event_record(events[k][0], s)
+        for i, name in enumerate(only):
+            run_op(name)
+            G.event_record(events[k][i + 1], s)
+    G.stream_sync(s)
+    G.device_sync()
+    wall = time.perf_counter() - wall0
+
+    abytes = algorithmic_bytes()
+    elems = work_elements()
+    scale_fix = 1.0 / args.scale
+    per_op = []
+    op_ms = {}
+    for i, name in enumerate(only):
+        ms = np.array([G.elapsed_ms(events[k][i], events[k][i + 1]) for k in range(args.steps)])
+        op_ms[name] = float(ms.mean())
+        gbs = abytes[name] * scale_fix / (ms.mean() * 1e-3) / 1e9
+        per_op.append({"op": name, "ms": round(float(ms.mean()), 4), "ms_min": round(float(ms.min()), 4),
+                       "GBps": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+                       "GElemps": round(elems[name] * scale_fix / (ms.mean() * 1e-3) / 1e9, 2)})
+    step_ms = wall / args.steps * 1e3
+    total_bytes = sum(abytes[n] for n in only) * scale_fix
+    value = total_bytes / (step_ms * 1e-3) / 1e9
+    dominant = max(op_ms, key=op_ms.get)
+    dom_gbs = abytes[dominant] * scale_fix / (op_ms[dominant] * 1e-3) / 1e9
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(orc, have_ref, Checker, H, img_h, col_h, only, abytes, scale_fix,
+                           args.cpu_reps)
+        for row in per_op:
+            c = cpu["per_op_ms"].get(row["op"])
+            if c:
+                row["cpu_ms"] = round(c, 2)
+                row["speedup_vs_cpu"] = round(c / row["ms"], 1)
+
+    out = {
+        "metric": "effective HBM GB/s (algorithmic bytes / time) over the nine hot-path ops",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(step_ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32 (f16 storage for im2col/col2im)",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE configs 1-5 at full shape, one pass each per step: "
+                               "map 4096x4096 f32; sumall_except_dim<1> (64,256,56,56); sum_rows "
+                               "16384x4096; Softmax+SoftmaxGrad 8192x32000; pool/unpool max 3x3 s2 "
+                               "(128,64,112,112); im2col/col2im 3x3 s1 p1 (32,256,56,56) f16"
+                               + ("" if args.scale == 1 else f" [leading dims / {args.scale}]"),
+                   "ops": only, "device": props.name.decode() or props.arch.decode(),
+                   "arch": props.arch.decode(), "compute_units": props.compute_units},
+        "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(dom_gbs, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
+                     "traffic": None},
+        "per_op": per_op,
+        "input_generation_s": round(gen_s, 1),
+    }
+    if cpu is not None:
+        out["cpu_baseline"] = {k: v for k, v in cpu.items() if k != "per_op_ms"}
+    print(json.dumps(out))
+
+
+def cpu_baseline(orc, have_ref, Checker, H, img_h, col_h, only, abytes, scale_fix, reps):
+    """The same nine operations on the host: the reference's own headers where the
+    reference-built library is present ("reference"), the C restatement otherwise
+    ("port"). One warm-up pass, then `reps` timed passes over the full inputs."""
+    kind = "reference" if have_ref() else "port"
+    cpu = Checker("ref") if kind == "reference" else orc
+    o_map = np.empty_like(H["A"])
+    o_2a, o_2b = np.empty(256, f32), np.empty(4096, f32)
+    o_p, o_g = np.empty_like(H["L"]), np.empty_like(H["L"])
+    o_pool, o_un = np.empty_like(H["G4"]), np.empty_like(H["X4"])
+    o_col, o_img = np.empty_like(col_h), np.empty_like(img_h)
+    fns = {
+        "map_fused": lambda: cpu.map_fused(o_map, H["A"], H["B"], H["C"], H["D"]),
+        "sumall_except_dim1": lambda: cpu.reduce_keep_highdim(o_2a, H["X2a"]),
+        "sum_rows": lambda: cpu.reduce_keep_lowest(o_2b, H["M2b"]),
+        "softmax": lambda: cpu.softmax(o_p, H["L"]),
+        "softmax_grad": lambda: cpu.softmax_grad(o_g, o_p, H["labels"]),
+        "pool_max": lambda: cpu.pool(o_pool, H["X4"], 3, 3, 2, 2),
+        "unpool_max": lambda: cpu.unpool(o_un, H["X4"], o_pool, H["G4"], 3, 3, 2, 2),
+        "im2col_f16": lambda: cpu.im2col(o_col, img_h, 3, 3, 1, 1, 1, 1, 1, 1),
+        "col2im_f16": lambda: cpu.col2im(o_img, col_h, 3, 3, 1, 1, 1, 1, 1, 1),
+    }
+    cpu.softmax(o_p, H["L"])
+    cpu.pool(o_pool, H["X4"], 3, 3, 2, 2)
+    per = {}
+    for name in only:
+        fns[name]()  # warm-up
+        t = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fns[name]()
+            t.append(time.perf_counter() - t0)
+        per[name] = float(np.mean(t)) * 1e3
+    total_ms = sum(per.values())
+    total_bytes = sum(abytes[n] for n in only) * scale_fix
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"value": round(total_bytes / (total_ms * 1e-3) / 1e9, 2), "unit": "GB/s",
+            "cores": cpu.num_threads(), "kind": kind,
+            "sample": f"all ops of the step at full shape, mean of {reps} passes after 1 warm-up "
+                      f"({total_ms:.0f} ms per pass)",
+            "cpu_model": model, "per_op_ms": per}
+
+
+if __name__ == "__main__":
+    main()
