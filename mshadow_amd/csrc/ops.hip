@@ -60,6 +60,8 @@ int DispatchReducer(int reducer, F f) {
 }  // namespace
 
 namespace {
+const size_t kPatchLdsBudget = 40 * 1024;  // per workgroup
+
 int MakePatchGeom(PatchGeom *g, int n, int c, int h, int w, int ky, int kx, int sy, int sx,
                   int dy, int dx, int pad_y, int pad_x) {
   if (n < 0 || c < 0 || h < 0 || w < 0) return Fail(MSHADOW_HIP_ERR_ARGUMENT, "negative shape");
@@ -95,11 +97,36 @@ int Im2Col(T *col, int cstride, const T *img, int istride, const PatchGeom &g, v
     return Fail(MSHADOW_HIP_ERR_ARGUMENT, "im2col: pitch smaller than the row");
   }
   const int EPT = 16 / sizeof(T);
-  const unsigned chunks = static_cast<unsigned>((cols + kPatchBlock * EPT - 1) / (kPatchBlock * EPT));
-  const long long blocks = rows * chunks;
-  if (blocks >= (1ll << 31)) return Fail(MSHADOW_HIP_ERR_ARGUMENT, "im2col: too many workgroups");
-  hipLaunchKernelGGL((Im2ColKernel<T, EPT>), dim3(static_cast<unsigned>(blocks)),
-                     dim3(kPatchBlock), 0, AsStream(stream), col, cstride, img, istride, g, chunks);
+  /* tiled: padded input rows of a band of patch rows must fit the LDS budget */
+  const size_t row_bytes = static_cast<size_t>(g.wp) * sizeof(T);
+  const long long max_rows = static_cast<long long>(kPatchLdsBudget / row_bytes);
+  const long long halo = static_cast<long long>(g.ky - 1) * g.dy + 1;
+  long long band = max_rows >= halo ? (max_rows - halo) / g.sy + 1 : 0;
+  if (band > g.oh) band = g.oh;
+  const long long planes = static_cast<long long>(g.n) * g.c;
+  while (band > 8 && planes * ((g.oh + band - 1) / band) < 1024) band = (band + 1) / 2;
+  if (band >= 1) {
+    const long long nb = (g.oh + band - 1) / band;
+    band = (g.oh + nb - 1) / nb;
+    PatchTile t;
+    t.band = static_cast<int>(band);
+    t.bands = static_cast<int>(nb);
+    t.rows_max = static_cast<int>((band - 1) * g.sy + halo);
+    t.pitch = g.wp;
+    const size_t lds = static_cast<size_t>(t.rows_max) * row_bytes;
+    const long long blocks = planes * nb;
+    if (blocks >= (1ll << 31)) return Fail(MSHADOW_HIP_ERR_ARGUMENT, "im2col: too many workgroups");
+    hipLaunchKernelGGL((Im2ColTiledKernel<T, EPT>), dim3(static_cast<unsigned>(blocks)),
+                       dim3(kPatchBlock), lds, AsStream(stream), col, cstride, img, istride, g, t);
+  } else {
+    const unsigned chunks =
+        static_cast<unsigned>((cols + kPatchBlock * EPT - 1) / (kPatchBlock * EPT));
+    const long long blocks = rows * chunks;
+    if (blocks >= (1ll << 31)) return Fail(MSHADOW_HIP_ERR_ARGUMENT, "im2col: too many workgroups");
+    hipLaunchKernelGGL((Im2ColKernel<T, EPT>), dim3(static_cast<unsigned>(blocks)),
+                       dim3(kPatchBlock), 0, AsStream(stream), col, cstride, img, istride, g,
+                       chunks);
+  }
   return AfterLaunch("im2col");
 }
 
@@ -112,11 +139,42 @@ int Col2Im(T *img, int istride, const T *col, int cstride, const PatchGeom &g, v
   if (cstride < cols || istride < g.w) {
     return Fail(MSHADOW_HIP_ERR_ARGUMENT, "col2im: pitch smaller than the row");
   }
-  unsigned grid = 0;
-  int st = mshadow_hip_suggest_grid(static_cast<size_t>(total), kPatchBlock, 8, &grid);
-  if (st != MSHADOW_HIP_OK) return st;
-  hipLaunchKernelGGL((Col2ImKernel<T>), dim3(grid), dim3(kPatchBlock), 0, AsStream(stream), img,
-                     istride, col, cstride, g, static_cast<unsigned>(total));
+  const int EPT = 16 / sizeof(T);
+  /* tiled: per tap, the patch rows a band of image rows touches; all taps must fit */
+  const long long taps = static_cast<long long>(g.ky) * g.kx;
+  const size_t prow_bytes = static_cast<size_t>(taps) * g.ow * sizeof(T);
+  const long long max_prows = static_cast<long long>(kPatchLdsBudget / prow_bytes);
+  /* an image band of b rows touches at most (b + span_y - 2) / sy + 2 patch rows */
+  const long long span_y = static_cast<long long>(g.dy) * (g.ky - 1) + 1;
+  long long band = (max_prows - 2) * g.sy - span_y + 2;
+  if (band > g.h) band = g.h;
+  const long long planes = static_cast<long long>(g.n) * g.c;
+  while (band > 8 && planes * ((g.h + band - 1) / band) < 1024) band = (band + 1) / 2;
+  if (band >= 1 && max_prows >= 3) {
+    const long long nb = (g.h + band - 1) / band;
+    band = (g.h + nb - 1) / nb;
+    PatchTile t;
+    t.band = static_cast<int>(band);
+    t.bands = static_cast<int>(nb);
+    t.rows_max = static_cast<int>((band + span_y - 2) / g.sy + 2);
+    t.pitch = (t.rows_max * g.ow + EPT - 1) / EPT * EPT;
+    const size_t lds = static_cast<size_t>(taps) * t.pitch * sizeof(T);
+    const long long blocks = planes * nb;
+    if (blocks >= (1ll << 31)) return Fail(MSHADOW_HIP_ERR_ARGUMENT, "col2im: too many workgroups");
+    if (g.dy == 1 && g.dx == 1) {
+      hipLaunchKernelGGL((Col2ImTiledKernel<T, EPT, true>), dim3(static_cast<unsigned>(blocks)),
+                         dim3(kPatchBlock), lds, AsStream(stream), img, istride, col, cstride, g, t);
+    } else {
+      hipLaunchKernelGGL((Col2ImTiledKernel<T, EPT, false>), dim3(static_cast<unsigned>(blocks)),
+                         dim3(kPatchBlock), lds, AsStream(stream), img, istride, col, cstride, g, t);
+    }
+  } else {
+    unsigned grid = 0;
+    int st = mshadow_hip_suggest_grid(static_cast<size_t>(total), kPatchBlock, 8, &grid);
+    if (st != MSHADOW_HIP_OK) return st;
+    hipLaunchKernelGGL((Col2ImKernel<T>), dim3(grid), dim3(kPatchBlock), 0, AsStream(stream), img,
+                       istride, col, cstride, g, static_cast<unsigned>(total));
+  }
   return AfterLaunch("col2im");
 }
 }  // namespace
@@ -196,10 +254,19 @@ int mshadow_hip_reduce_keep_lowest_f32(float *dst, const float *src, int sstride
     return DispatchSaver(saver, [&](auto sv) {
       typedef decltype(red) R;
       typedef decltype(sv) S;
-      hipLaunchKernelGGL((mshadow::hip::ReduceKeepLowestKernel<S, R, float, RawPlan1D<float>,
-                                                               RawPlan2D<const float> >),
-                         dim3(grid), dim3(mshadow::hip::kRedBlock), 0, s, d, sp,
-                         static_cast<uint32_t>(rows), static_cast<uint32_t>(cols), scale);
+      if (rows >= 4096) {
+        hipLaunchKernelGGL(
+            (mshadow::hip::ReduceKeepLowestKernel<S, R, float, mshadow::hip::kRedBlockLarge,
+                                                  RawPlan1D<float>, RawPlan2D<const float> >),
+            dim3(grid), dim3(mshadow::hip::kRedBlockLarge), 0, s, d, sp,
+            static_cast<uint32_t>(rows), static_cast<uint32_t>(cols), scale);
+      } else {
+        hipLaunchKernelGGL(
+            (mshadow::hip::ReduceKeepLowestKernel<S, R, float, mshadow::hip::kRedBlockSmall,
+                                                  RawPlan1D<float>, RawPlan2D<const float> >),
+            dim3(grid), dim3(mshadow::hip::kRedBlockSmall), 0, s, d, sp,
+            static_cast<uint32_t>(rows), static_cast<uint32_t>(cols), scale);
+      }
       return MSHADOW_HIP_OK;
     });
   });
@@ -223,16 +290,21 @@ int mshadow_hip_reduce_keep_highdim_f32(float *dst, const float *src, int sstrid
     return DispatchSaver(saver, [&](auto sv) {
       typedef decltype(red) R;
       typedef decltype(sv) S;
-#define HIGHDIM_LAUNCH(SEGS)                                                                   \
-  hipLaunchKernelGGL((mshadow::hip::ReduceKeepHighDimKernel<S, R, float, SEGS, RawPlan1D<float>, \
+#define HIGHDIM_LAUNCH_T(T, SEGS)                                                              \
+  hipLaunchKernelGGL((mshadow::hip::ReduceKeepHighDimKernel<S, R, float, T, SEGS, RawPlan1D<float>, \
                                                             RawPlan2D<const float> >),         \
-                     dim3(c), dim3(mshadow::hip::kRedBlock), 0, s, d, sp,                      \
-                     static_cast<uint32_t>(n), static_cast<uint32_t>(c),                       \
-                     static_cast<uint32_t>(y), static_cast<uint32_t>(x), scale)
-      if (n > 16) HIGHDIM_LAUNCH(64);
-      else if (n > 4) HIGHDIM_LAUNCH(16);
-      else if (n > 1) HIGHDIM_LAUNCH(4);
-      else HIGHDIM_LAUNCH(1);
+                     dim3(c), dim3(T), 0, s, d, sp, static_cast<uint32_t>(n),                  \
+                     static_cast<uint32_t>(c), static_cast<uint32_t>(y),                       \
+                     static_cast<uint32_t>(x), scale)
+#define HIGHDIM_LAUNCH(SEGS)                                                                   \
+  if (large) HIGHDIM_LAUNCH_T(mshadow::hip::kRedBlockLarge, SEGS);                             \
+  else HIGHDIM_LAUNCH_T(mshadow::hip::kRedBlockSmall, SEGS)
+      const bool large = static_cast<long long>(n) * y * x >= (1 << 18);
+      if (n > 16) { HIGHDIM_LAUNCH(64); }
+      else if (n > 4) { HIGHDIM_LAUNCH(16); }
+      else if (n > 1) { HIGHDIM_LAUNCH(4); }
+      else { HIGHDIM_LAUNCH(1); }
+#undef HIGHDIM_LAUNCH_T
 #undef HIGHDIM_LAUNCH
       return MSHADOW_HIP_OK;
     });
@@ -258,7 +330,7 @@ int mshadow_hip_pool_f32(float *dst, int dstride, const float *src, int sstride,
   ABI_REQUIRE(static_cast<long long>(planes) * h < (1ll << 31) &&
                   static_cast<long long>(planes) * ph * pw < (1ll << 32),
               "too large for 32-bit indices");
-  PoolGeom g = {h, w, ph, pw, ky, kx, sy, sx, 0, 0, w + 1};
+  PoolGeom g = {h, w, ph, pw, ky, kx, sy, sx, 0, 0, w};
   hipStream_t s = AsStream(stream);
   const size_t row_bytes = static_cast<size_t>(g.lds_pitch) * sizeof(float);
   /* output rows per band so that (band - 1) * sy + ky input rows fit the budget */
@@ -268,6 +340,11 @@ int mshadow_hip_pool_f32(float *dst, int dstride, const float *src, int sstride,
   /* keep at least ~4 workgroups per CU in flight when planes are few */
   while (band > 8 && static_cast<long long>(planes) * ((ph + band - 1) / band) < 1024) {
     band = (band + 1) / 2;
+  }
+  if (band >= 1) {  // equal-sized bands; about 24 KB of LDS each keeps several resident per CU
+    long long nb = (ph + band - 1) / band;
+    if (band * static_cast<long long>(sy) * row_bytes > 24 * 1024 && nb < 2 && ph >= 16) nb = 2;
+    band = (ph + nb - 1) / nb;
   }
 #define POOL_SWITCH(KERNEL, ...)                                                               \
   switch (reducer) {                                                                           \
@@ -281,8 +358,25 @@ int mshadow_hip_pool_f32(float *dst, int dstride, const float *src, int sstride,
     const size_t lds = (static_cast<size_t>(g.band - 1) * sy + ky) * row_bytes;
     const long long blocks = static_cast<long long>(planes) * g.bands;
     ABI_REQUIRE(blocks < (1ll << 31), "too many workgroups");
-    POOL_SWITCH(PoolKernel, dim3(static_cast<unsigned>(blocks)), dim3(kPoolBlock), lds, s, dst,
-                dstride, src, sstride, g)
+#define POOL_TILED(KY, KX)                                                                     \
+  switch (reducer) {                                                                           \
+    case MSHADOW_HIP_SUM:                                                                      \
+      hipLaunchKernelGGL((PoolKernel<MSHADOW_HIP_SUM, KY, KX>), dim3(static_cast<unsigned>(blocks)), \
+                         dim3(kPoolBlock), lds, s, dst, dstride, src, sstride, g);             \
+      break;                                                                                   \
+    case MSHADOW_HIP_MAX:                                                                      \
+      hipLaunchKernelGGL((PoolKernel<MSHADOW_HIP_MAX, KY, KX>), dim3(static_cast<unsigned>(blocks)), \
+                         dim3(kPoolBlock), lds, s, dst, dstride, src, sstride, g);             \
+      break;                                                                                   \
+    default:                                                                                   \
+      hipLaunchKernelGGL((PoolKernel<MSHADOW_HIP_MIN, KY, KX>), dim3(static_cast<unsigned>(blocks)), \
+                         dim3(kPoolBlock), lds, s, dst, dstride, src, sstride, g);             \
+      break;                                                                                   \
+  }
+    if (ky == 3 && kx == 3) { POOL_TILED(3, 3) }
+    else if (ky == 2 && kx == 2) { POOL_TILED(2, 2) }
+    else { POOL_TILED(0, 0) }
+#undef POOL_TILED
   } else {
     const unsigned total = static_cast<unsigned>(planes) * ph * pw;
     unsigned grid = 0;
@@ -309,7 +403,7 @@ int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstrid
   ABI_REQUIRE(static_cast<long long>(planes) * h * w < (1ll << 32) &&
                   static_cast<long long>(planes) * h < (1ll << 31),
               "too large for 32-bit indices");
-  PoolGeom g = {h, w, ph, pw, ky, kx, sy, sx, 0, 0, pw + 1};
+  PoolGeom g = {h, w, ph, pw, ky, kx, sy, sx, 0, 0, pw};
   hipStream_t s = AsStream(stream);
   const size_t row_bytes = static_cast<size_t>(g.lds_pitch) * sizeof(float) * 2;  // pooled + grad
   /* source rows per band: prow_max = (band + ky - 2) / sy + 2 pooled rows must fit */
@@ -318,6 +412,10 @@ int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstrid
   if (band > h) band = h;
   while (band > 8 && static_cast<long long>(planes) * ((h + band - 1) / band) < 1024) {
     band = (band + 1) / 2;
+  }
+  if (band >= 1) {  // equal-sized bands
+    const long long nb = (h + band - 1) / band;
+    band = (h + nb - 1) / nb;
   }
   if (band >= 1 && max_prow >= 3) {
     g.band = static_cast<int>(band);

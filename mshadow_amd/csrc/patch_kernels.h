@@ -53,6 +53,148 @@ struct Acc<uint16_t> {
   }
 };
 
+/* ---------------------------------------------------------------- LDS-tiled versions
+ * One workgroup per (image, channel) plane, or per band of rows of it:
+ *   im2col  stages the zero-padded input band once, then writes the ky*kx shifted copies
+ *           (each a contiguous run of the column matrix) with 128-bit stores;
+ *   col2im  stages, per kernel tap, the contiguous run of the column matrix that the band
+ *           needs (128-bit loads), then sums each pixel's covering patches from LDS in
+ *           the reference's (py, px) order.
+ * So the large side (the column matrix) moves through HBM exactly once in long
+ * contiguous pieces and the small side once per band. */
+struct PatchTile {
+  int band;       // im2col: patch rows (oy) per workgroup; col2im: image rows per workgroup
+  int bands;      // bands per plane
+  int rows_max;   // im2col: padded input rows staged; col2im: patch rows (py) staged per tap
+  int pitch;      // im2col: LDS elements per staged input row; col2im: per staged tap
+};
+
+template <typename T, int EPT>
+__global__ void __launch_bounds__(kPatchBlock)
+    Im2ColTiledKernel(T *col, int cstride, const T *img, int istride, PatchGeom g, PatchTile t) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  T *lds = reinterpret_cast<T *>(smem_raw);
+  const int plane = blockIdx.x / t.bands;      // n * c + ch
+  const int band = blockIdx.x - plane * t.bands;
+  const int ch = plane % g.c;
+  const int n = plane / g.c;
+  const int oy0 = band * t.band;
+  const int noy = min(t.band, g.oh - oy0);
+  const int iy0 = oy0 * g.sy;                  // first padded input row of the band
+  const int in_rows = (noy - 1) * g.sy + (g.ky - 1) * g.dy + 1;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const T *src = img + static_cast<size_t>(plane) * g.h * istride;
+  for (int r = wave; r < in_rows; r += kPatchBlock / 64) {
+    const int y = iy0 + r - g.pad_y;
+    const bool row_ok = y >= 0 && y < g.h;
+    for (int xx = lane; xx < g.wp; xx += 64) {
+      const int x = xx - g.pad_x;
+      T v = 0;
+      if (row_ok && x >= 0 && x < g.w) v = src[static_cast<size_t>(y) * istride + x];
+      lds[r * t.pitch + xx] = v;
+    }
+  }
+  __syncthreads();
+  const int count = noy * g.ow;                // contiguous outputs per tap
+  const int nvec = (count + EPT - 1) / EPT;
+  const int taps = g.ky * g.kx;
+  const size_t j0 = (static_cast<size_t>(n) * g.oh + oy0) * g.ow;
+  for (int idx = threadIdx.x; idx < taps * nvec; idx += kPatchBlock) {
+    const int tap = idx / nvec;
+    const int v = idx - tap * nvec;
+    const int a = tap / g.kx;
+    const int b = tap - a * g.kx;
+    const int e0 = v * EPT;
+    int oy = e0 / g.ow;
+    int ox = e0 - oy * g.ow;
+    T vals[EPT];
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      vals[e] = (e0 + e < count) ? lds[(oy * g.sy + a * g.dy) * t.pitch + ox * g.sx + b * g.dx]
+                                 : static_cast<T>(0);
+      if (++ox == g.ow) {
+        ox = 0;
+        ++oy;
+      }
+    }
+    T *out = col + static_cast<size_t>((ch * g.ky + a) * g.kx + b) * cstride + j0 + e0;
+    if (e0 + EPT <= count && reinterpret_cast<uintptr_t>(out) % (sizeof(T) * EPT) == 0) {
+      typedef T Vec __attribute__((ext_vector_type(EPT)));
+      Vec pack;
+#pragma unroll
+      for (int e = 0; e < EPT; ++e) pack[e] = vals[e];
+      *reinterpret_cast<Vec *>(out) = pack;
+    } else {
+#pragma unroll
+      for (int e = 0; e < EPT; ++e) {
+        if (e0 + e < count) out[e] = vals[e];
+      }
+    }
+  }
+}
+
+template <typename T, int EPT, bool UNIT_DILATE>
+__global__ void __launch_bounds__(kPatchBlock)
+    Col2ImTiledKernel(T *img, int istride, const T *col, int cstride, PatchGeom g, PatchTile t) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  T *lds = reinterpret_cast<T *>(smem_raw);
+  const int plane = blockIdx.x / t.bands;
+  const int band = blockIdx.x - plane * t.bands;
+  const int ch = plane % g.c;
+  const int n = plane / g.c;
+  const int cy0 = band * t.band;
+  const int ncy = min(t.band, g.h - cy0);
+  const int span_y = g.dy * (g.ky - 1) + 1;
+  const int span_x = g.dx * (g.kx - 1) + 1;
+  /* patch rows any pixel row of the band can touch */
+  const int yf = cy0 + g.pad_y, yl = cy0 + ncy - 1 + g.pad_y;
+  const int p0 = yf < span_y ? 0 : (yf - span_y + g.sy) / g.sy;
+  const int p1 = min((yl + g.sy) / g.sy, g.oh);
+  const int npy = max(p1 - p0, 0);
+  const int run = npy * g.ow;                  // contiguous column-matrix elements per tap
+  const int nvec = (run + EPT - 1) / EPT;
+  const int taps = g.ky * g.kx;
+  const size_t j0 = (static_cast<size_t>(n) * g.oh + p0) * g.ow;
+  for (int idx = threadIdx.x; idx < taps * nvec; idx += kPatchBlock) {
+    const int tap = idx / nvec;
+    const int v = idx - tap * nvec;
+    const int e0 = v * EPT;
+    const T *in = col + static_cast<size_t>(ch * taps + tap) * cstride + j0 + e0;
+    T *out = lds + tap * t.pitch + e0;         // t.pitch is a multiple of EPT: aligned
+    if (e0 + EPT <= run && reinterpret_cast<uintptr_t>(in) % (sizeof(T) * EPT) == 0) {
+      typedef T Vec __attribute__((ext_vector_type(EPT)));
+      *reinterpret_cast<Vec *>(out) = *reinterpret_cast<const Vec *>(in);
+    } else {
+#pragma unroll
+      for (int e = 0; e < EPT; ++e) {
+        if (e0 + e < run) out[e] = in[e];
+      }
+    }
+  }
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  T *dst = img + (static_cast<size_t>(plane) * g.h + cy0) * istride;
+  for (int cyr = wave; cyr < ncy; cyr += kPatchBlock / 64) {
+    const int y = cy0 + cyr + g.pad_y;
+    const int py_min = y < span_y ? y % g.dy : (y - span_y + g.sy) / g.sy;
+    const int py_max = min((y + g.sy) / g.sy, g.oh);
+    for (int cx = lane; cx < g.w; cx += 64) {
+      const int x = cx + g.pad_x;
+      const int px_min = x < span_x ? x % g.dx : (x - span_x + g.sx) / g.sx;
+      const int px_max = min((x + g.sx) / g.sx, g.ow);
+      T res = Acc<T>::Zero();
+      for (int py = py_min; py < py_max; py += g.dy) {
+        const int a = UNIT_DILATE ? (y - py * g.sy) : (y - py * g.sy) / g.dy;
+        for (int px = px_min; px < px_max; px += g.dx) {
+          const int b = UNIT_DILATE ? (x - px * g.sx) : (x - px * g.sx) / g.dx;
+          res = Acc<T>::Add(res, lds[(a * g.kx + b) * t.pitch + (py - p0) * g.ow + px]);
+        }
+      }
+      dst[static_cast<size_t>(cyr) * istride + cx] = res;
+    }
+  }
+}
+
 /*! \brief EPT consecutive column-matrix elements per thread; grid.x = rows of the column
  *  matrix (c, a, b) times `chunks` pieces of kPatchBlock * EPT columns each. */
 template <typename T, int EPT>

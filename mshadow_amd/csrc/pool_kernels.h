@@ -4,14 +4,16 @@
  * The reference evaluates pool / unpool through its generic map kernel with
  * Plan<PoolingExp>::Eval / Plan<UnPoolingExp>::Eval as the body
  * (mshadow/extension/spatial_pool.h:125-142, spatial_unpool.h:102-125), i.e. ky*kx
- * scattered global loads per output. Here a workgroup stages a band of input rows of
- * one (n, c) plane in LDS with coalesced loads and every window is then read from LDS,
- * so HBM sees each input element once:
+ * scattered global loads per output. Here a workgroup stages a band of rows of one
+ * (n, c) plane in LDS with coalesced (128-bit where aligned) loads and every window is
+ * then read from LDS, so HBM sees each input element once:
  *   pool    reads  planes*h*w*4 B, writes planes*ph*pw*4 B
  *   unpool  reads  planes*(h*w + 2*ph*pw)*4 B, writes planes*h*w*4 B
- * Results are bit-identical to the reference: same window clipping, same (y, x)
- * reduction order from the reducer's initial value, `max` / `min` by operator<, and the
- * gradient routed by equality with a separate multiply and add (no fused multiply-add).
+ * Work inside a band is laid out wave-per-row / lane-per-column, so no integer division
+ * is executed per element. Results are bit-identical to the reference: same window
+ * clipping, same (y, x) reduction order from the reducer's initial value, `max` / `min`
+ * by operator<, and the gradient routed by equality with a separate multiply and add
+ * (no fused multiply-add).
  */
 #ifndef MSHADOW_AMD_CSRC_POOL_KERNELS_H_
 #define MSHADOW_AMD_CSRC_POOL_KERNELS_H_
@@ -24,6 +26,7 @@
 namespace mshadow_hipk {
 
 const int kPoolBlock = 256;
+const int kPoolWaves = kPoolBlock / 64;
 
 template <int REDUCER>
 struct PoolOp;
@@ -53,43 +56,77 @@ struct PoolGeom {
   int lds_pitch;   // floats per staged row
 };
 
+/*! \brief copy `nrows` rows of `width` floats (global pitch gpitch) into LDS (pitch
+ *  lpitch). When both pitches equal the width the band is one contiguous run and is
+ *  moved with 128-bit loads; otherwise one wave takes one row at a time. */
+__device__ __forceinline__ void StageRows(float *lds, int lpitch, const float *g, int gpitch,
+                                          int nrows, int width) {
+  if (gpitch == width && lpitch == width) {
+    const int total = nrows * width;
+    const int lead = static_cast<int>((16 - (reinterpret_cast<uintptr_t>(g) & 15)) & 15) / 4;
+    const int head = lead < total ? lead : total;
+    for (int i = threadIdx.x; i < head; i += kPoolBlock) lds[i] = g[i];
+    const int nvec = (total - head) / 4;
+    /* LDS side may be misaligned by `head` floats: store the four lanes separately */
+    for (int v = threadIdx.x; v < nvec; v += kPoolBlock) {
+      const float4 q = *reinterpret_cast<const float4 *>(g + head + 4 * v);
+      float *o = lds + head + 4 * v;
+      o[0] = q.x; o[1] = q.y; o[2] = q.z; o[3] = q.w;
+    }
+    for (int i = head + 4 * nvec + threadIdx.x; i < total; i += kPoolBlock) lds[i] = g[i];
+  } else {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int r = wave; r < nrows; r += kPoolWaves) {
+      const float *row = g + static_cast<size_t>(r) * gpitch;
+      for (int c = lane; c < width; c += 64) lds[r * lpitch + c] = row[c];
+    }
+  }
+}
+
 /*! \brief grid.x = planes * bands. Dynamic LDS: in_rows * lds_pitch floats, where
- *  in_rows = (band - 1) * sy + ky. */
-template <int REDUCER>
+ *  in_rows = (band - 1) * sy + ky. KY / KX > 0 fix the window size at compile time
+ *  (the loops unroll); 0 means "use g.ky / g.kx". */
+template <int REDUCER, int KY, int KX>
 __global__ void __launch_bounds__(kPoolBlock)
     PoolKernel(float *dst, int dstride, const float *src, int sstride, PoolGeom g) {
   extern __shared__ float smem[];
   typedef PoolOp<REDUCER> Op;
+  const int ky = KY > 0 ? KY : g.ky;
+  const int kx = KX > 0 ? KX : g.kx;
   const int plane = blockIdx.x / g.bands;
   const int band = blockIdx.x - plane * g.bands;
   const int py0 = band * g.band;
   const int npy = min(g.band, g.ph - py0);
   const int y0 = py0 * g.sy;
-  const int y1 = min(y0 + (npy - 1) * g.sy + g.ky, g.h);  // one past the last row needed
+  const int y1 = min(y0 + (npy - 1) * g.sy + ky, g.h);  // one past the last row needed
   const int nrows = max(y1 - y0, 0);
-  const float *in = src + (static_cast<size_t>(plane) * g.h + y0) * sstride;
-  /* stage rows y0..y1 (whole width) */
-  const int total = nrows * g.w;
-  for (int i = threadIdx.x; i < total; i += kPoolBlock) {
-    const int r = i / g.w;
-    const int c = i - r * g.w;
-    smem[r * g.lds_pitch + c] = in[static_cast<size_t>(r) * sstride + c];
-  }
+  StageRows(smem, g.lds_pitch, src + (static_cast<size_t>(plane) * g.h + y0) * sstride, sstride,
+            nrows, g.w);
   __syncthreads();
   float *out = dst + (static_cast<size_t>(plane) * g.ph + py0) * dstride;
-  const int nout = npy * g.pw;
-  for (int o = threadIdx.x; o < nout; o += kPoolBlock) {
-    const int py = o / g.pw;
-    const int px = o - py * g.pw;
-    const int ys = py * g.sy;                      // relative to y0
-    const int ye = min(ys + g.ky, g.h - y0);
-    const int xs = px * g.sx;
-    const int xe = min(xs + g.kx, g.w);
-    float res = Op::Init();
-    for (int y = ys; y < ye; ++y) {
-      for (int x = xs; x < xe; ++x) res = Op::Reduce(res, smem[y * g.lds_pitch + x]);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int py = wave; py < npy; py += kPoolWaves) {
+    const int ys = py * g.sy;  // relative to y0
+    const int ye = min(ys + ky, g.h - y0);
+    for (int px = lane; px < g.pw; px += 64) {
+      const int xs = px * g.sx;
+      const int xe = min(xs + kx, g.w);
+      float res = Op::Init();
+      if (KY > 0 && KX > 0 && ye - ys == KY && xe - xs == KX) {
+#pragma unroll
+        for (int y = 0; y < (KY > 0 ? KY : 1); ++y) {
+#pragma unroll
+          for (int x = 0; x < (KX > 0 ? KX : 1); ++x) {
+            res = Op::Reduce(res, smem[(ys + y) * g.lds_pitch + xs + x]);
+          }
+        }
+      } else {
+        for (int y = ys; y < ye; ++y) {
+          for (int x = xs; x < xe; ++x) res = Op::Reduce(res, smem[y * g.lds_pitch + x]);
+        }
+      }
+      out[static_cast<size_t>(py) * dstride + px] = res;
     }
-    out[static_cast<size_t>(py) * dstride + px] = res;
   }
 }
 
@@ -134,36 +171,44 @@ __global__ void __launch_bounds__(kPoolBlock)
   const int p0 = y0 < g.ky ? 0 : (y0 - g.ky + g.sy) / g.sy;
   const int p1 = min((ylast + g.sy) / g.sy, g.ph);
   const int np = max(p1 - p0, 0);
-  const float *pin = pooled + (static_cast<size_t>(plane) * g.ph + p0) * pstride;
-  const float *gin = grad + (static_cast<size_t>(plane) * g.ph + p0) * gstride;
-  const int total = np * g.pw;
-  for (int i = threadIdx.x; i < total; i += kPoolBlock) {
-    const int r = i / g.pw;
-    const int c = i - r * g.pw;
-    sp[r * g.lds_pitch + c] = pin[static_cast<size_t>(r) * pstride + c];
-    sg[r * g.lds_pitch + c] = gin[static_cast<size_t>(r) * gstride + c];
-  }
-  __syncthreads();
+  StageRows(sp, g.lds_pitch, pooled + (static_cast<size_t>(plane) * g.ph + p0) * pstride, pstride,
+            np, g.pw);
+  StageRows(sg, g.lds_pitch, grad + (static_cast<size_t>(plane) * g.ph + p0) * gstride, gstride,
+            np, g.pw);
   const float *in = src + (static_cast<size_t>(plane) * g.h + y0) * sstride;
   float *out = dst + (static_cast<size_t>(plane) * g.h + y0) * dstride;
-  const int nout = ny * g.w;
-  for (int o = threadIdx.x; o < nout; o += kPoolBlock) {
-    const int yr = o / g.w;
-    const int x = o - yr * g.w;
-    const int y = y0 + yr;
-    const float vsrc = in[static_cast<size_t>(yr) * sstride + x];
-    const int py_min = y < g.ky ? 0 : (y - g.ky + g.sy) / g.sy;
-    const int px_min = x < g.kx ? 0 : (x - g.kx + g.sx) / g.sx;
-    const int py_max = min((y + g.sy) / g.sy, g.ph);
-    const int px_max = min((x + g.sx) / g.sx, g.pw);
-    float val = 0.0f;
-    for (int py = py_min; py < py_max; ++py) {
-      for (int px = px_min; px < px_max; ++px) {
-        const int li = (py - p0) * g.lds_pitch + px;
-        val = val + Op::Grad(vsrc, sp[li]) * sg[li];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  /* each lane fetches its source pixel of kRowsAhead rows before using any of them */
+  const int kRowsAhead = 4;
+  __syncthreads();
+  for (int yr0 = wave; yr0 < ny; yr0 += kPoolWaves * kRowsAhead) {
+    for (int x = lane; x < g.w; x += 64) {
+      float vs[kRowsAhead];
+#pragma unroll
+      for (int u = 0; u < kRowsAhead; ++u) {
+        const int yr = yr0 + u * kPoolWaves;
+        vs[u] = (yr < ny) ? in[static_cast<size_t>(yr) * sstride + x] : 0.0f;
+      }
+      const int px_min = x < g.kx ? 0 : (x - g.kx + g.sx) / g.sx;
+      const int px_max = min((x + g.sx) / g.sx, g.pw);
+#pragma unroll
+      for (int u = 0; u < kRowsAhead; ++u) {
+        const int yr = yr0 + u * kPoolWaves;
+        if (yr < ny) {
+          const int y = y0 + yr;
+          const int py_min = y < g.ky ? 0 : (y - g.ky + g.sy) / g.sy;
+          const int py_max = min((y + g.sy) / g.sy, g.ph);
+          float val = 0.0f;
+          for (int py = py_min; py < py_max; ++py) {
+            for (int px = px_min; px < px_max; ++px) {
+              const int li = (py - p0) * g.lds_pitch + px;
+              val = val + Op::Grad(vs[u], sp[li]) * sg[li];
+            }
+          }
+          out[static_cast<size_t>(yr) * dstride + x] = val;
+        }
       }
     }
-    out[static_cast<size_t>(yr) * dstride + x] = val;
   }
 }
 

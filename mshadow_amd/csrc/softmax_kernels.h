@@ -4,11 +4,11 @@
  * SoftmaxRowKernel: one workgroup per row, the whole row held in registers, so HBM
  * sees one read of src and one write of dst (2 * 4 bytes per element; the reference
  * kernel, mshadow/cuda/tensor_gpu-inl.cuh:330-393, moves 5). Steps per row:
- *   1. 128-bit loads, row maximum by wave shuffles + one LDS exchange;
- *   2. p = expf(x - max) in registers;
+ *   1. 128-bit loads, row maximum by DPP wave reduction + one LDS exchange;
+ *   2. p = exp(x - max) in registers (hardware exp2 with a compensated argument);
  *   3. the row sum in the CPU path's left-to-right order (ordered_sum.h), so that the
- *      result matches mshadow/tensor_cpu-inl.h:270-285 to the last bit of the sum;
- *   4. p / sum with IEEE division, 128-bit stores.
+ *      sum is, bit for bit, what mshadow/tensor_cpu-inl.h:277-281 computes from the same p;
+ *   4. p / sum (reciprocal and one correction step), 128-bit stores.
  * dst may alias src (every element is read before the row is written).
  * SoftmaxLongRowKernel covers rows too long for registers with the same arithmetic,
  * staging p through dst. SoftmaxGradKernel is a 128-bit copy with one element per row
@@ -84,15 +84,18 @@ __device__ inline float BlockOrderedAdd(float s, const float (&t)[N],
       if (lane == 0) lds->q[*buf][wave] = q < kBig ? q : kBig;
     }
     __syncthreads();
+    /* every thread scans the per-wave totals (one LDS vector read, then registers) */
+    uint32_t qw[W];
+#pragma unroll
+    for (int w = 0; w < W; ++w) qw[w] = lds->q[*buf][w];
     uint32_t acc = 0;
     int failw = W;
-    for (int w = pos; w < W; ++w) {
-      const uint32_t qw = lds->q[*buf][w];
-      if (b.m + acc + qw >= kBig) {
-        failw = w;
-        break;
-      }
-      acc += qw;
+#pragma unroll
+    for (int w = 0; w < W; ++w) {
+      const bool live = w >= pos && failw == W;
+      const bool over = b.m + acc + qw[w] >= kBig;
+      if (live && over) failw = w;
+      if (live && !over) acc += qw[w];
     }
     *buf ^= 1;
     s = Accept(s, b, acc);
@@ -106,6 +109,31 @@ __device__ inline float BlockOrderedAdd(float s, const float (&t)[N],
     pos = failw + 1;
     if (pos == W) return s;
   }
+}
+
+/*! \brief e^x for x <= 0 (any float accepted): 2^(x * log2 e) with the rounding error of
+ *  the product carried separately, so the result stays within about 1.5 ulp for the whole
+ *  range a softmax sees. The hardware exp2 does not return subnormals, so results below
+ *  2^-126 are computed 64 binades up and scaled back. */
+__device__ __forceinline__ float ExpNonPositive(float x) {
+  const float kLog2eHi = 1.44269502162933349609375f;
+  const float kLog2eLo = 1.925963033500011079013347625732421875e-08f;
+  const float t = x * kLog2eHi;
+  float r = __builtin_fmaf(x, kLog2eHi, -t);   // exact rounding error of the product
+  r = __builtin_fmaf(x, kLog2eLo, r);
+  const bool tiny = t < -125.0f;
+  const float e = __builtin_amdgcn_exp2f(tiny ? t + 64.0f : t);
+  const float v = __builtin_fmaf(e, r * 0.693147182464599609375f, e);  // e * 2^r, |r| << 1
+  if (t < -151.0f) return 0.0f;  // below half of the smallest subnormal (also x = -inf)
+  return tiny ? v * 5.42101086242752217003726400434970855712890625e-20f : v;  // 2^-64
+}
+
+/*! \brief p / s given rcp = 1 / s: one Newton correction on the quotient. The result is
+ *  the correctly rounded quotient except for rare half-ulp cases. */
+__device__ __forceinline__ float DivideBy(float p, float s, float rcp) {
+  const float q = p * rcp;
+  const float e = __builtin_fmaf(-q, s, p);
+  return __builtin_fmaf(e, rcp, q);
 }
 
 template <int THREADS>
@@ -125,7 +153,7 @@ __device__ inline float BlockMax(float v, OrderedSumLds<THREADS / kWave> *lds) {
 
 /*! \brief THREADS * SLABS * VEC >= cols. VEC == 4 needs 16-byte aligned rows. */
 template <int THREADS, int SLABS, int VEC>
-__global__ void __launch_bounds__(THREADS)
+__global__ void __launch_bounds__(THREADS, 4)  // >= 4 waves per SIMD: two 512-thread rows per CU
     SoftmaxRowKernel(float *dst, int dstride, const float *src, int sstride, int cols) {
   __shared__ OrderedSumLds<THREADS / kWave> lds;
   const int tid = threadIdx.x;
@@ -154,7 +182,7 @@ __global__ void __launch_bounds__(THREADS)
   for (int j = 0; j < SLABS; ++j) {
     const int base = (j * THREADS + tid) * VEC;
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) v[j][i] = (base + i < cols) ? expf(v[j][i] - mx) : 0.0f;
+    for (int i = 0; i < VEC; ++i) v[j][i] = (base + i < cols) ? ExpNonPositive(v[j][i] - mx) : 0.0f;
   }
 
   float s = 0.0f;
@@ -164,17 +192,24 @@ __global__ void __launch_bounds__(THREADS)
     if (j * THREADS * VEC < cols) s = BlockOrderedAdd<THREADS, VEC>(s, v[j], &lds, &buf);
   }
 
+  /* s >= 1 for finite logits (the maximum contributes exp(0)); anything else (NaN or
+     infinite logits) takes the plain division so that specials propagate as on the CPU */
+  const bool fast_div = s >= 1.0f && s < 3.0e38f;
+  const float rcp = 1.0f / s;
 #pragma unroll
   for (int j = 0; j < SLABS; ++j) {
     const int base = (j * THREADS + tid) * VEC;
+    float o[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) o[i] = fast_div ? DivideBy(v[j][i], s, rcp) : v[j][i] / s;
     if (VEC == 4 && base + 4 <= cols) {
       float4 q;
-      q.x = v[j][0] / s; q.y = v[j][1 % VEC] / s; q.z = v[j][2 % VEC] / s; q.w = v[j][3 % VEC] / s;
+      q.x = o[0]; q.y = o[1 % VEC]; q.z = o[2 % VEC]; q.w = o[3 % VEC];
       *reinterpret_cast<float4 *>(out + base) = q;
     } else {
 #pragma unroll
       for (int i = 0; i < VEC; ++i) {
-        if (base + i < cols) out[base + i] = v[j][i] / s;
+        if (base + i < cols) out[base + i] = o[i];
       }
     }
   }
@@ -200,7 +235,7 @@ __global__ void __launch_bounds__(THREADS)
   for (int x0 = 0; x0 < cols; x0 += THREADS) {
     const int x = x0 + tid;
     float p[1];
-    p[0] = (x < cols) ? expf(in[x] - mx) : 0.0f;
+    p[0] = (x < cols) ? ExpNonPositive(in[x] - mx) : 0.0f;
     if (x < cols) out[x] = p[0];
     s = BlockOrderedAdd<THREADS, 1>(s, p, &lds, &buf);
   }

@@ -9,9 +9,9 @@
  * relative on outputs near zero, so these kernels keep it: each output (or each inner
  * (n, c) segment) is a serial chain of dependent adds owned by ONE lane. Bandwidth
  * comes from everything around the chain:
- *   - all 256 threads of a workgroup stream the next tiles from HBM with coalesced
- *     loads (16 independent loads per thread in flight, two stages deep), and drop
- *     them into LDS transposed, so that
+ *   - all threads of a workgroup (1024 for long reductions) stream the next tiles from
+ *     HBM with coalesced loads (16 independent loads per thread in flight, two stages
+ *     deep: up to 128 KB per CU), and drop them into LDS transposed, so that
  *   - the chain lanes of wave 0 read their own next 4 operands with one ds_read_b128
  *     and spend one dependent add per element.
  * Work is split so that every CU owns a few chains (16 columns, or one kept index, per
@@ -32,13 +32,14 @@
 namespace mshadow {
 namespace hip {
 
-const int kRedBlock = 256;
 /*! \brief loads per thread per stage (all issued before any is consumed) */
 const int kRedDepth = 16;
-/*! \brief elements staged per workgroup per stage */
-const int kRedTile = kRedBlock * kRedDepth;
 /*! \brief columns per workgroup in KeepLowest: 16 floats = one 64-byte segment per row */
 const int kLowestCols = 16;
+/*! \brief workgroup sizes: the large one keeps 64 KB of loads in flight per stage and is
+ *  used when the reduction is long enough to fill its pipeline */
+const int kRedBlockSmall = 256;
+const int kRedBlockLarge = 1024;
 
 /*! \brief value of v in lane `lane` for any small trivially copyable type */
 template <typename DType>
@@ -55,29 +56,63 @@ __device__ __forceinline__ DType WaveBroadcast(DType v, int lane) {
   return r;
 }
 
-/*! \brief fold `count` consecutive LDS values into res, in order */
+/*! \brief fold vals[begin .. count) into res, in order. The operands of the next 32
+ *  steps are fetched from LDS (eight 128-bit reads) while the current 32 dependent
+ *  reductions execute, so a step costs one VALU issue plus a quarter of an LDS read. */
 template <typename Reducer, typename DType>
 __device__ __forceinline__ void ChainFold(DType &res, const DType *vals, int begin, int count) {
   typedef expr::Pack<DType, 4> P4;
+  const int kBlk = 32;
   int r = begin;
-  /* head up to a multiple of 4, then packs, then tail */
-  for (; r < count && (r & 3); ++r) Reducer::Reduce(res, vals[r]);
-  for (; r + 4 <= count; r += 4) {
-    const P4 p = *reinterpret_cast<const P4 *>(vals + r);
-    Reducer::Reduce(res, p.v[0]);
-    Reducer::Reduce(res, p.v[1]);
-    Reducer::Reduce(res, p.v[2]);
-    Reducer::Reduce(res, p.v[3]);
+  for (; r < count && (r & (kBlk - 1)); ++r) Reducer::Reduce(res, vals[r]);
+  if (r + kBlk <= count) {
+    P4 a[kBlk / 4];
+#pragma unroll
+    for (int i = 0; i < kBlk / 4; ++i) a[i] = *reinterpret_cast<const P4 *>(vals + r + 4 * i);
+    for (; r + 2 * kBlk <= count; r += kBlk) {
+      P4 b[kBlk / 4];
+#pragma unroll
+      for (int i = 0; i < kBlk / 4; ++i) {
+        b[i] = *reinterpret_cast<const P4 *>(vals + r + kBlk + 4 * i);
+      }
+#pragma unroll
+      for (int i = 0; i < kBlk / 4; ++i) {
+        Reducer::Reduce(res, a[i].v[0]);
+        Reducer::Reduce(res, a[i].v[1]);
+        Reducer::Reduce(res, a[i].v[2]);
+        Reducer::Reduce(res, a[i].v[3]);
+      }
+#pragma unroll
+      for (int i = 0; i < kBlk / 4; ++i) a[i] = b[i];
+    }
+#pragma unroll
+    for (int i = 0; i < kBlk / 4; ++i) {
+      Reducer::Reduce(res, a[i].v[0]);
+      Reducer::Reduce(res, a[i].v[1]);
+      Reducer::Reduce(res, a[i].v[2]);
+      Reducer::Reduce(res, a[i].v[3]);
+    }
+    r += kBlk;
   }
   for (; r < count; ++r) Reducer::Reduce(res, vals[r]);
 }
 
+/*! \brief which strip of kLowestCols columns a workgroup takes. Workgroups are dealt to
+ *  the 8 XCDs round-robin; neighbouring strips share 128-byte cache lines, so each XCD
+ *  (one L2) is given a contiguous run of strips when the count divides evenly. */
+__device__ __forceinline__ uint32_t StripOfBlock(uint32_t block, uint32_t nblocks) {
+  const uint32_t kXcd = 8;
+  if (nblocks % kXcd != 0) return block;
+  return (block % kXcd) * (nblocks / kXcd) + block / kXcd;
+}
+
 /* ------------------------------------------------------------------ KeepLowest */
-template <typename Saver, typename Reducer, typename DType, typename DPlan, typename SPlan>
-__global__ void __launch_bounds__(kRedBlock)
+template <typename Saver, typename Reducer, typename DType, int THREADS, typename DPlan,
+          typename SPlan>
+__global__ void __launch_bounds__(THREADS)
     ReduceKeepLowestKernel(DPlan dplan, SPlan splan, uint32_t rows, uint32_t cols, DType scale) {
   const int CW = kLowestCols;
-  const int RPP = kRedBlock / CW;    // rows covered by one load pass of the workgroup
+  const int RPP = THREADS / CW;      // rows covered by one load pass of the workgroup
   const int TR = RPP * kRedDepth;    // rows per stage
   const int LD = TR + 4;             // pitch of one column in the transposed tile
   __shared__ MSHADOW_ALIGNED(16) DType tile[2][CW * LD];
@@ -85,7 +120,7 @@ __global__ void __launch_bounds__(kRedBlock)
   const int t = threadIdx.x;
   const int col = t % CW;
   const int rsub = t / CW;
-  const uint32_t x = blockIdx.x * CW + col;
+  const uint32_t x = StripOfBlock(blockIdx.x, gridDim.x) * CW + col;
   const bool col_ok = x < cols;
   const uint32_t nstage = (rows + TR - 1) / TR;
   const bool chain_lane = (t < CW) && col_ok;  // lanes 0..CW-1 of wave 0 own the chains
@@ -129,12 +164,12 @@ __global__ void __launch_bounds__(kRedBlock)
 /* ------------------------------------------------------------------ KeepHighDim */
 /* shape viewed as (n_out, n_keep, n_y, n_x); one workgroup per kept index c. SEGS inner
    segments (n values) are staged side by side, one chain lane each. */
-template <typename Saver, typename Reducer, typename DType, int SEGS, typename DPlan,
+template <typename Saver, typename Reducer, typename DType, int THREADS, int SEGS, typename DPlan,
           typename SPlan>
-__global__ void __launch_bounds__(kRedBlock)
+__global__ void __launch_bounds__(THREADS)
     ReduceKeepHighDimKernel(DPlan dplan, SPlan splan, uint32_t n_out, uint32_t n_keep,
                             uint32_t n_y, uint32_t n_x, DType scale) {
-  const int TL = kRedTile / SEGS;  // elements of each segment per stage
+  const int TL = THREADS * kRedDepth / SEGS;  // elements of each segment per stage
   const int LD = TL + 4;
   __shared__ MSHADOW_ALIGNED(16) DType tile[2][SEGS * LD];
 
@@ -152,7 +187,7 @@ __global__ void __launch_bounds__(kRedBlock)
     const uint32_t g_ = (STAGE) / stages_per_group;                                    \
     const uint32_t e0_ = ((STAGE) - g_ * stages_per_group) * TL;                       \
     _Pragma("unroll") for (int k = 0; k < kRedDepth; ++k) {                            \
-      const uint32_t f_ = k * kRedBlock + t;                                           \
+      const uint32_t f_ = k * THREADS + t;                                             \
       const uint32_t n_ = g_ * SEGS + f_ / TL;                                         \
       const uint32_t e_ = e0_ + f_ % TL;                                               \
       DType v_ = DType(0);                                                             \
@@ -163,7 +198,7 @@ __global__ void __launch_bounds__(kRedBlock)
       REGS[k] = v_;                                                                    \
     }                                                                                  \
   }
-  MSHADOW_HIGHDIM_LOAD(cur, 0u)
+  if (nstage > 0) MSHADOW_HIGHDIM_LOAD(cur, 0u)
   DType res, tres;
   Reducer::SetInitValue(res);
   Reducer::SetInitValue(tres);
@@ -172,7 +207,7 @@ __global__ void __launch_bounds__(kRedBlock)
     DType *buf = tile[st & 1];
 #pragma unroll
     for (int k = 0; k < kRedDepth; ++k) {
-      const uint32_t f = k * kRedBlock + t;
+      const uint32_t f = k * THREADS + t;
       buf[(f / TL) * LD + f % TL] = cur[k];
     }
     __syncthreads();

@@ -414,9 +414,17 @@ inline void MapReduceKeepLowest(TRValue<R, gpu, 1, DType> *dst,
   uint32_t rows = eshape[0], cols = eshape[1];
   if (cols == 0) return;
   void *args[] = {&dplan, &splan, &rows, &cols, &scale};
-  gpu_detail::Launch(hip::ReduceKeepLowestKernel<Saver, Reducer, DType, DPlan, SPlan>,
-                     (cols + hip::kLowestCols - 1) / hip::kLowestCols, hip::kRedBlock, args,
-                     Stream<gpu>::GetStream(expr::StreamInfo<gpu, R>::Get(dst->self())));
+  void *stream = Stream<gpu>::GetStream(expr::StreamInfo<gpu, R>::Get(dst->self()));
+  const uint32_t strips = (cols + hip::kLowestCols - 1) / hip::kLowestCols;
+  if (rows >= 4096) {
+    gpu_detail::Launch(hip::ReduceKeepLowestKernel<Saver, Reducer, DType, hip::kRedBlockLarge,
+                                                   DPlan, SPlan>,
+                       strips, hip::kRedBlockLarge, args, stream);
+  } else {
+    gpu_detail::Launch(hip::ReduceKeepLowestKernel<Saver, Reducer, DType, hip::kRedBlockSmall,
+                                                   DPlan, SPlan>,
+                       strips, hip::kRedBlockSmall, args, stream);
+  }
 #else
   LOG(FATAL) << "MapReduceKeepLowest<gpu>: compile the calling translation unit with hipcc";
 #endif
@@ -442,21 +450,29 @@ inline void MapReduceKeepHighDim(TRValue<R, gpu, 1, DType> *dst,
   if (n_keep == 0) return;
   void *args[] = {&dplan, &splan, &n_out, &n_keep, &n_y, &n_x, &scale};
   void *stream = Stream<gpu>::GetStream(expr::StreamInfo<gpu, R>::Get(dst->self()));
-  /* segments staged side by side = chain lanes in use; fewer, longer pieces when the
-     outer extent is small */
-  if (n_out > 16) {
-    gpu_detail::Launch(hip::ReduceKeepHighDimKernel<Saver, Reducer, DType, 64, DPlan, SPlan>,
-                       n_keep, hip::kRedBlock, args, stream);
-  } else if (n_out > 4) {
-    gpu_detail::Launch(hip::ReduceKeepHighDimKernel<Saver, Reducer, DType, 16, DPlan, SPlan>,
-                       n_keep, hip::kRedBlock, args, stream);
-  } else if (n_out > 1) {
-    gpu_detail::Launch(hip::ReduceKeepHighDimKernel<Saver, Reducer, DType, 4, DPlan, SPlan>,
-                       n_keep, hip::kRedBlock, args, stream);
-  } else {
-    gpu_detail::Launch(hip::ReduceKeepHighDimKernel<Saver, Reducer, DType, 1, DPlan, SPlan>,
-                       n_keep, hip::kRedBlock, args, stream);
+  /* segments staged side by side = chain lanes in use (fewer, longer pieces when the
+     outer extent is small); the large workgroup when each kept index has enough work */
+  const bool large = static_cast<uint64_t>(n_out) * n_y * n_x >= (1u << 18);
+#define MSHADOW_HIGHDIM_LAUNCH(SEGS)                                                          \
+  if (large) {                                                                                \
+    gpu_detail::Launch(hip::ReduceKeepHighDimKernel<Saver, Reducer, DType, hip::kRedBlockLarge, \
+                                                    SEGS, DPlan, SPlan>,                      \
+                       n_keep, hip::kRedBlockLarge, args, stream);                            \
+  } else {                                                                                    \
+    gpu_detail::Launch(hip::ReduceKeepHighDimKernel<Saver, Reducer, DType, hip::kRedBlockSmall, \
+                                                    SEGS, DPlan, SPlan>,                      \
+                       n_keep, hip::kRedBlockSmall, args, stream);                            \
   }
+  if (n_out > 16) {
+    MSHADOW_HIGHDIM_LAUNCH(64)
+  } else if (n_out > 4) {
+    MSHADOW_HIGHDIM_LAUNCH(16)
+  } else if (n_out > 1) {
+    MSHADOW_HIGHDIM_LAUNCH(4)
+  } else {
+    MSHADOW_HIGHDIM_LAUNCH(1)
+  }
+#undef MSHADOW_HIGHDIM_LAUNCH
 #else
   LOG(FATAL) << "MapReduceKeepHighDim<gpu>: compile the calling translation unit with hipcc";
 #endif
