@@ -161,7 +161,7 @@ int Col2Im(T *img, int istride, const T *col, int cstride, const PatchGeom &g, v
     const size_t lds = static_cast<size_t>(taps) * t.pitch * sizeof(T);
     const long long blocks = planes * nb;
     if (blocks >= (1ll << 31)) return Fail(MSHADOW_HIP_ERR_ARGUMENT, "col2im: too many workgroups");
-    if (g.dy == 1 && g.dx == 1) {
+    if (g.dy == 1 && g.dx == 1 && g.sy == 1 && g.sx == 1) {
       hipLaunchKernelGGL((Col2ImTiledKernel<T, EPT, true>), dim3(static_cast<unsigned>(blocks)),
                          dim3(kPatchBlock), lds, AsStream(stream), img, istride, col, cstride, g, t);
     } else {
@@ -191,7 +191,9 @@ int mshadow_hip_softmax_f32(float *dst, int dstride, const float *src, int sstri
   ABI_REQUIRE(dst != NULL && src != NULL, "NULL tensor");
   ABI_REQUIRE(dstride >= cols && sstride >= cols, "pitch smaller than the row");
   hipStream_t s = AsStream(stream);
-  const bool vec = Aligned16(dst) && Aligned16(src) && dstride % 4 == 0 && sstride % 4 == 0;
+  /* 128-bit path: aligned rows made of whole packs */
+  const bool vec = Aligned16(dst) && Aligned16(src) && dstride % 4 == 0 && sstride % 4 == 0 &&
+                   cols % 4 == 0;
 #define SOFTMAX_LAUNCH(T, S, V) \
   hipLaunchKernelGGL((SoftmaxRowKernel<T, S, V>), dim3(rows), dim3(T), 0, s, dst, dstride, src, \
                      sstride, cols)
@@ -209,6 +211,7 @@ int mshadow_hip_softmax_f32(float *dst, int dstride, const float *src, int sstri
     if (cols <= 1024) SOFTMAX_LAUNCH(256, 4, 1);
     else if (cols <= 4096) SOFTMAX_LAUNCH(256, 16, 1);
     else if (cols <= 16384) SOFTMAX_LAUNCH(1024, 16, 1);
+    else if (cols <= 32768) SOFTMAX_LAUNCH(1024, 32, 1);
     else hipLaunchKernelGGL((SoftmaxLongRowKernel<1024>), dim3(rows), dim3(1024), 0, s, dst,
                             dstride, src, sstride, cols);
   }
@@ -355,7 +358,7 @@ int mshadow_hip_pool_f32(float *dst, int dstride, const float *src, int sstride,
   if (band >= 1) {
     g.band = static_cast<int>(band);
     g.bands = (ph + g.band - 1) / g.band;
-    const size_t lds = (static_cast<size_t>(g.band - 1) * sy + ky) * row_bytes;
+    const size_t lds = (static_cast<size_t>(g.band - 1) * sy + ky) * row_bytes + 16;
     const long long blocks = static_cast<long long>(planes) * g.bands;
     ABI_REQUIRE(blocks < (1ll << 31), "too many workgroups");
 #define POOL_TILED(KY, KX)                                                                     \
@@ -421,11 +424,32 @@ int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstrid
     g.band = static_cast<int>(band);
     g.bands = (h + g.band - 1) / g.band;
     const int prow_max = (g.band + ky - 2) / sy + 2;
-    const size_t lds = static_cast<size_t>(prow_max) * row_bytes;
+    const size_t lds = static_cast<size_t>(prow_max) * row_bytes + 32;
     const long long blocks = static_cast<long long>(planes) * g.bands;
     ABI_REQUIRE(blocks < (1ll << 31), "too many workgroups");
-    POOL_SWITCH(UnpoolKernel, dim3(static_cast<unsigned>(blocks)), dim3(kPoolBlock), lds, s, dst,
-                dstride, src, sstride, pooled, pstride, grad, gstride, g, prow_max)
+#define UNPOOL_TILED(SY, SX)                                                                   \
+  switch (reducer) {                                                                           \
+    case MSHADOW_HIP_SUM:                                                                      \
+      hipLaunchKernelGGL((UnpoolKernel<MSHADOW_HIP_SUM, SY, SX>),                              \
+                         dim3(static_cast<unsigned>(blocks)), dim3(kPoolBlock), lds, s, dst,   \
+                         dstride, src, sstride, pooled, pstride, grad, gstride, g, prow_max);  \
+      break;                                                                                   \
+    case MSHADOW_HIP_MAX:                                                                      \
+      hipLaunchKernelGGL((UnpoolKernel<MSHADOW_HIP_MAX, SY, SX>),                              \
+                         dim3(static_cast<unsigned>(blocks)), dim3(kPoolBlock), lds, s, dst,   \
+                         dstride, src, sstride, pooled, pstride, grad, gstride, g, prow_max);  \
+      break;                                                                                   \
+    default:                                                                                   \
+      hipLaunchKernelGGL((UnpoolKernel<MSHADOW_HIP_MIN, SY, SX>),                              \
+                         dim3(static_cast<unsigned>(blocks)), dim3(kPoolBlock), lds, s, dst,   \
+                         dstride, src, sstride, pooled, pstride, grad, gstride, g, prow_max);  \
+      break;                                                                                   \
+  }
+    if (sy == 2 && sx == 2) { UNPOOL_TILED(2, 2) }
+    else if (sy == 1 && sx == 1) { UNPOOL_TILED(1, 1) }
+    else if (sy == 3 && sx == 3) { UNPOOL_TILED(3, 3) }
+    else { UNPOOL_TILED(0, 0) }
+#undef UNPOOL_TILED
   } else {
     const unsigned total = static_cast<unsigned>(planes) * h * w;
     unsigned grid = 0;

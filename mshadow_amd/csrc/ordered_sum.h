@@ -13,8 +13,9 @@
  *   half way between two integers (then the tie-break depends on the parity of m).
  *
  * So inside a binade the float adds are exact INTEGER adds of q = rne(t/u), which are
- * associative: lanes quantise their terms, a wave/block sums the integers, and the
- * chunk is accepted if m + sum(q) stays below 2^24 and no term was a tie. Otherwise
+ * associative: lanes quantise their terms, a wave/block sums the integers (held in
+ * floats, exact below 2^24), and the chunk is accepted if m + sum(q) stays below 2^24
+ * and no term was a tie. Otherwise
  * the first offending position is located by prefix sums; everything before it is
  * accepted, the offending lane performs its (at most 4) additions as real float adds,
  * and the remainder is re-quantised against the new binade. A row of N(0,3) logits
@@ -39,8 +40,12 @@
 
 namespace ordered_sum {
 
-/*! \brief a quantised contribution this large means "do not accept me as an integer" */
-const uint32_t kBig = 1u << 24;
+/*! \brief quantised contributions are carried as floats holding integers: sums below
+ *  2^24 are exact, and a sum that reaches 2^24 in exact arithmetic can never round to
+ *  less, so "not below kLimit" is a faithful overflow test. A lane that must not be
+ *  accepted as integers (tie, inf, NaN, unusable binade) contributes kReject. */
+const float kLimit = 16777216.0f;  // 2^24
+const float kReject = 33554432.0f;  // 2^25
 
 OSUM_HD uint32_t BitsOf(float f) {
   uint32_t u;
@@ -57,7 +62,7 @@ OSUM_HD float FloatOf(uint32_t u) {
 struct Binade {
   float u;        //!< ulp of S: 2^(k-23)
   float inv_u;    //!< 2^(23-k)
-  uint32_t m;     //!< S / u, an integer in [2^23, 2^24)
+  float m;        //!< S / u, an integer in [2^23, 2^24), as a float
   bool usable;    //!< S is a positive normal number large enough for u and inv_u to be normal
 };
 
@@ -69,37 +74,40 @@ OSUM_HD Binade BinadeOf(float s) {
   r.usable = (b >> 31) == 0 && e >= 27u && e < 255u;
   r.u = r.usable ? FloatOf((e - 23u) << 23) : 0.0f;
   r.inv_u = r.usable ? FloatOf((277u - e) << 23) : 0.0f;
-  r.m = r.usable ? ((b & 0x7fffffu) | 0x800000u) : 0u;
+  r.m = r.usable ? s * r.inv_u : 0.0f;  /* exact: scaling by a power of two */
   return r;
 }
 
-/*! \brief rne(t / u) of one term, or kBig if the term is a tie, too large, inf or NaN */
-OSUM_HD uint32_t QuantOne(float t, float inv_u) {
-  const float scaled = t * inv_u;  /* exact: inv_u is a power of two */
-  if (!(scaled < 16777216.0f)) return kBig;
-  const float q = rintf(scaled);   /* round to nearest even */
-  if (fabsf(scaled - q) == 0.5f) return kBig;
-  return static_cast<uint32_t>(q);
-}
-
-/*! \brief contribution of one lane's N consecutive terms, saturated at kBig.
- *  When the binade is not usable (S is 0, subnormal-small, inf or NaN) only all-zero
- *  lanes can be accepted: adding +0 never changes S. */
+/*! \brief contribution of one lane's N consecutive terms: sum of rne(t / u), or kReject
+ *  if any term is a tie (or NaN). Terms too large for the binade simply make the sum
+ *  reach kLimit. When the binade is not usable (S is 0, subnormal-small, inf or NaN)
+ *  only all-zero lanes can be accepted: adding +0 never changes S. */
 template <int N>
-OSUM_HD uint32_t LaneQuant(const float (&t)[N], const Binade &b) {
+OSUM_HD float LaneQuant(const float (&t)[N], const Binade &b) {
   if (!b.usable) {
     bool any = false;
     for (int i = 0; i < N; ++i) any = any || !(t[i] == 0.0f);
-    return any ? kBig : 0u;
+    return any ? kReject : 0.0f;
   }
-  uint32_t s = 0;
-  for (int i = 0; i < N; ++i) s += QuantOne(t[i], b.inv_u);
-  return s < kBig ? s : kBig;
+  float sum = 0.0f;
+  bool tie = false;
+  for (int i = 0; i < N; ++i) {
+    const float scaled = t[i] * b.inv_u;  /* exact: inv_u is a power of two */
+    const float q = rintf(scaled);        /* round to nearest even */
+    /* |scaled - q| == 0.5 exactly when the term sits half way; NaN also lands here */
+    tie = tie || !(fabsf(scaled - q) < 0.5f);
+    sum += q;
+  }
+  return tie ? kReject : sum;
 }
 
-/*! \brief S after accepting integer contributions summing to q (m + q < 2^24) */
-OSUM_HD float Accept(float s, const Binade &b, uint32_t q) {
-  return b.usable ? static_cast<float>(b.m + q) * b.u : s;
+/*! \brief true if integer contributions totalling q can be added without leaving the
+ *  binade (written so that NaN fails) */
+OSUM_HD bool Fits(const Binade &b, float q) { return b.m + q < kLimit; }
+
+/*! \brief S after accepting integer contributions summing to q (Fits(b, q) holds) */
+OSUM_HD float Accept(float s, const Binade &b, float q) {
+  return b.usable ? (b.m + q) * b.u : s;
 }
 
 /*! \brief the real thing: N float additions in order */

@@ -95,49 +95,73 @@ __global__ void __launch_bounds__(kPatchBlock)
     }
   }
   __syncthreads();
-  const int count = noy * g.ow;                // contiguous outputs per tap
-  const int nvec = (count + EPT - 1) / EPT;
-  const int taps = g.ky * g.kx;
+  /* each tap (a, b) owns one row of the column matrix and, inside it, the band is one
+     contiguous run of `count` elements. A thread walks that run in packs of EPT; its
+     (oy, ox) position advances by a fixed step, so the only division is the one below. */
+  const int count = noy * g.ow;
+  const int step = kPatchBlock * EPT;
+  const int step_oy = step / g.ow;
+  const int step_ox = step - step_oy * g.ow;
+  const int first = threadIdx.x * EPT;
+  const int first_oy = first / g.ow;
+  const int first_ox = first - first_oy * g.ow;
   const size_t j0 = (static_cast<size_t>(n) * g.oh + oy0) * g.ow;
-  for (int idx = threadIdx.x; idx < taps * nvec; idx += kPatchBlock) {
-    const int tap = idx / nvec;
-    const int v = idx - tap * nvec;
-    const int a = tap / g.kx;
-    const int b = tap - a * g.kx;
-    const int e0 = v * EPT;
-    int oy = e0 / g.ow;
-    int ox = e0 - oy * g.ow;
-    T vals[EPT];
+  for (int a = 0; a < g.ky; ++a) {
+    for (int b = 0; b < g.kx; ++b) {
+      T *row = col + static_cast<size_t>((ch * g.ky + a) * g.kx + b) * cstride + j0;
+      const T *tap = lds + a * g.dy * t.pitch + b * g.dx;
+      int oy = first_oy, ox = first_ox;
+      for (int e0 = first; e0 < count; e0 += step) {
+        T vals[EPT];
+        if (ox + EPT <= g.ow) {  // the pack stays inside one patch row
+          const T *p = tap + oy * g.sy * t.pitch + ox * g.sx;
 #pragma unroll
-    for (int e = 0; e < EPT; ++e) {
-      vals[e] = (e0 + e < count) ? lds[(oy * g.sy + a * g.dy) * t.pitch + ox * g.sx + b * g.dx]
-                                 : static_cast<T>(0);
-      if (++ox == g.ow) {
-        ox = 0;
-        ++oy;
-      }
-    }
-    T *out = col + static_cast<size_t>((ch * g.ky + a) * g.kx + b) * cstride + j0 + e0;
-    if (e0 + EPT <= count && reinterpret_cast<uintptr_t>(out) % (sizeof(T) * EPT) == 0) {
-      typedef T Vec __attribute__((ext_vector_type(EPT)));
-      Vec pack;
+          for (int e = 0; e < EPT; ++e) vals[e] = p[e * g.sx];
+        } else {
+          int yy = oy, xx = ox;
 #pragma unroll
-      for (int e = 0; e < EPT; ++e) pack[e] = vals[e];
-      *reinterpret_cast<Vec *>(out) = pack;
-    } else {
+          for (int e = 0; e < EPT; ++e) {
+            vals[e] = (e0 + e < count) ? tap[yy * g.sy * t.pitch + xx * g.sx] : static_cast<T>(0);
+            if (++xx == g.ow) {
+              xx = 0;
+              ++yy;
+            }
+          }
+        }
+        T *out = row + e0;
+        if (e0 + EPT <= count && reinterpret_cast<uintptr_t>(out) % (sizeof(T) * EPT) == 0) {
+          typedef T Vec __attribute__((ext_vector_type(EPT)));
+          Vec pack;
 #pragma unroll
-      for (int e = 0; e < EPT; ++e) {
-        if (e0 + e < count) out[e] = vals[e];
+          for (int e = 0; e < EPT; ++e) pack[e] = vals[e];
+          *reinterpret_cast<Vec *>(out) = pack;
+        } else {
+#pragma unroll
+          for (int e = 0; e < EPT; ++e) {
+            if (e0 + e < count) out[e] = vals[e];
+          }
+        }
+        ox += step_ox;
+        oy += step_oy;
+        if (ox >= g.ow) {
+          ox -= g.ow;
+          ++oy;
+        }
       }
     }
   }
 }
 
-template <typename T, int EPT, bool UNIT_DILATE>
+/*! \brief FAST: stride 1 and dilation 1 in both directions (the common convolution case):
+ *  every patch-range bound is then a subtraction instead of a division. */
+template <typename T, int EPT, bool FAST>
 __global__ void __launch_bounds__(kPatchBlock)
     Col2ImTiledKernel(T *img, int istride, const T *col, int cstride, PatchGeom g, PatchTile t) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   T *lds = reinterpret_cast<T *>(smem_raw);
+  if (FAST) {
+    g.sy = g.sx = g.dy = g.dx = 1;
+  }
   const int plane = blockIdx.x / t.bands;
   const int band = blockIdx.x - plane * t.bands;
   const int ch = plane % g.c;
@@ -152,22 +176,21 @@ __global__ void __launch_bounds__(kPatchBlock)
   const int p1 = min((yl + g.sy) / g.sy, g.oh);
   const int npy = max(p1 - p0, 0);
   const int run = npy * g.ow;                  // contiguous column-matrix elements per tap
-  const int nvec = (run + EPT - 1) / EPT;
   const int taps = g.ky * g.kx;
   const size_t j0 = (static_cast<size_t>(n) * g.oh + p0) * g.ow;
-  for (int idx = threadIdx.x; idx < taps * nvec; idx += kPatchBlock) {
-    const int tap = idx / nvec;
-    const int v = idx - tap * nvec;
-    const int e0 = v * EPT;
-    const T *in = col + static_cast<size_t>(ch * taps + tap) * cstride + j0 + e0;
-    T *out = lds + tap * t.pitch + e0;         // t.pitch is a multiple of EPT: aligned
-    if (e0 + EPT <= run && reinterpret_cast<uintptr_t>(in) % (sizeof(T) * EPT) == 0) {
-      typedef T Vec __attribute__((ext_vector_type(EPT)));
-      *reinterpret_cast<Vec *>(out) = *reinterpret_cast<const Vec *>(in);
-    } else {
+  for (int tap = 0; tap < taps; ++tap) {
+    const T *in = col + static_cast<size_t>(ch * taps + tap) * cstride + j0;
+    T *out = lds + tap * t.pitch;              // t.pitch is a multiple of EPT: aligned
+    const bool vec_ok = reinterpret_cast<uintptr_t>(in) % (sizeof(T) * EPT) == 0;
+    for (int e0 = threadIdx.x * EPT; e0 < run; e0 += kPatchBlock * EPT) {
+      if (vec_ok && e0 + EPT <= run) {
+        typedef T Vec __attribute__((ext_vector_type(EPT)));
+        *reinterpret_cast<Vec *>(out + e0) = *reinterpret_cast<const Vec *>(in + e0);
+      } else {
 #pragma unroll
-      for (int e = 0; e < EPT; ++e) {
-        if (e0 + e < run) out[e] = in[e];
+        for (int e = 0; e < EPT; ++e) {
+          if (e0 + e < run) out[e0 + e] = in[e0 + e];
+        }
       }
     }
   }
@@ -184,9 +207,9 @@ __global__ void __launch_bounds__(kPatchBlock)
       const int px_max = min((x + g.sx) / g.sx, g.ow);
       T res = Acc<T>::Zero();
       for (int py = py_min; py < py_max; py += g.dy) {
-        const int a = UNIT_DILATE ? (y - py * g.sy) : (y - py * g.sy) / g.dy;
+        const int a = (y - py * g.sy) / g.dy;
         for (int px = px_min; px < px_max; px += g.dx) {
-          const int b = UNIT_DILATE ? (x - px * g.sx) : (x - px * g.sx) / g.dx;
+          const int b = (x - px * g.sx) / g.dx;
           res = Acc<T>::Add(res, lds[(a * g.kx + b) * t.pitch + (py - p0) * g.ow + px]);
         }
       }

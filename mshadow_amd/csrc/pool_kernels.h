@@ -56,24 +56,43 @@ struct PoolGeom {
   int lds_pitch;   // floats per staged row
 };
 
+/*! \brief LDS images are shifted by 0..3 floats so that LDS addresses have the same
+ *  16-byte phase as the global addresses they mirror: both sides of the staging copy can
+ *  then use 128-bit accesses. Callers allocate 4 extra floats per staged array. */
+__device__ __forceinline__ int LdsPhase(const float *g) {
+  return static_cast<int>((reinterpret_cast<uintptr_t>(g) >> 2) & 3);
+}
+
 /*! \brief copy `nrows` rows of `width` floats (global pitch gpitch) into LDS (pitch
- *  lpitch). When both pitches equal the width the band is one contiguous run and is
- *  moved with 128-bit loads; otherwise one wave takes one row at a time. */
+ *  lpitch); `lds` already includes the phase shift of LdsPhase(g). When both pitches equal
+ *  the width the band is one contiguous run and moves as 128-bit packs, eight loads in
+ *  flight per thread; otherwise one wave takes one row at a time. */
 __device__ __forceinline__ void StageRows(float *lds, int lpitch, const float *g, int gpitch,
                                           int nrows, int width) {
   if (gpitch == width && lpitch == width) {
     const int total = nrows * width;
-    const int lead = static_cast<int>((16 - (reinterpret_cast<uintptr_t>(g) & 15)) & 15) / 4;
+    const int lead = (4 - LdsPhase(g)) & 3;
     const int head = lead < total ? lead : total;
-    for (int i = threadIdx.x; i < head; i += kPoolBlock) lds[i] = g[i];
+    if (static_cast<int>(threadIdx.x) < head) lds[threadIdx.x] = g[threadIdx.x];
     const int nvec = (total - head) / 4;
-    /* LDS side may be misaligned by `head` floats: store the four lanes separately */
-    for (int v = threadIdx.x; v < nvec; v += kPoolBlock) {
-      const float4 q = *reinterpret_cast<const float4 *>(g + head + 4 * v);
-      float *o = lds + head + 4 * v;
-      o[0] = q.x; o[1] = q.y; o[2] = q.z; o[3] = q.w;
+    const float4 *gv = reinterpret_cast<const float4 *>(g + head);
+    float4 *lv = reinterpret_cast<float4 *>(lds + head);
+    const int kUnroll = 8;
+    for (int v0 = threadIdx.x; v0 < nvec; v0 += kPoolBlock * kUnroll) {
+      float4 q[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {  // unpredicated: past the end re-reads the last pack
+        const int v = v0 + u * kPoolBlock;
+        q[u] = gv[v < nvec ? v : nvec - 1];
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int v = v0 + u * kPoolBlock;
+        if (v < nvec) lv[v] = q[u];
+      }
     }
-    for (int i = head + 4 * nvec + threadIdx.x; i < total; i += kPoolBlock) lds[i] = g[i];
+    const int tail = head + 4 * nvec + threadIdx.x;
+    if (tail < total) lds[tail] = g[tail];
   } else {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     for (int r = wave; r < nrows; r += kPoolWaves) {
@@ -83,7 +102,7 @@ __device__ __forceinline__ void StageRows(float *lds, int lpitch, const float *g
   }
 }
 
-/*! \brief grid.x = planes * bands. Dynamic LDS: in_rows * lds_pitch floats, where
+/*! \brief grid.x = planes * bands. Dynamic LDS: in_rows * lds_pitch + 4 floats, where
  *  in_rows = (band - 1) * sy + ky. KY / KX > 0 fix the window size at compile time
  *  (the loops unroll); 0 means "use g.ky / g.kx". */
 template <int REDUCER, int KY, int KX>
@@ -100,8 +119,9 @@ __global__ void __launch_bounds__(kPoolBlock)
   const int y0 = py0 * g.sy;
   const int y1 = min(y0 + (npy - 1) * g.sy + ky, g.h);  // one past the last row needed
   const int nrows = max(y1 - y0, 0);
-  StageRows(smem, g.lds_pitch, src + (static_cast<size_t>(plane) * g.h + y0) * sstride, sstride,
-            nrows, g.w);
+  const float *in = src + (static_cast<size_t>(plane) * g.h + y0) * sstride;
+  float *tile = smem + LdsPhase(in);
+  StageRows(tile, g.lds_pitch, in, sstride, nrows, g.w);
   __syncthreads();
   float *out = dst + (static_cast<size_t>(plane) * g.ph + py0) * dstride;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -117,12 +137,12 @@ __global__ void __launch_bounds__(kPoolBlock)
         for (int y = 0; y < (KY > 0 ? KY : 1); ++y) {
 #pragma unroll
           for (int x = 0; x < (KX > 0 ? KX : 1); ++x) {
-            res = Op::Reduce(res, smem[(ys + y) * g.lds_pitch + xs + x]);
+            res = Op::Reduce(res, tile[(ys + y) * g.lds_pitch + xs + x]);
           }
         }
       } else {
         for (int y = ys; y < ye; ++y) {
-          for (int x = xs; x < xe; ++x) res = Op::Reduce(res, smem[y * g.lds_pitch + x]);
+          for (int x = xs; x < xe; ++x) res = Op::Reduce(res, tile[y * g.lds_pitch + x]);
         }
       }
       out[static_cast<size_t>(py) * dstride + px] = res;
@@ -153,15 +173,17 @@ __global__ void __launch_bounds__(kPoolBlock)
 }
 
 /*! \brief grid.x = planes * bands over SOURCE rows. Dynamic LDS: two arrays (pooled,
- *  grad) of prow_max * lds_pitch floats, prow_max = (band + ky - 2) / sy + 2. */
-template <int REDUCER>
+ *  grad) of prow_max * lds_pitch + 4 floats, prow_max = (band + ky - 2) / sy + 2.
+ *  SY / SX > 0 fix the strides at compile time so that the divisions below become
+ *  multiplications; 0 means "use g.sy / g.sx". */
+template <int REDUCER, int SY, int SX>
 __global__ void __launch_bounds__(kPoolBlock)
     UnpoolKernel(float *dst, int dstride, const float *src, int sstride, const float *pooled,
                  int pstride, const float *grad, int gstride, PoolGeom g, int prow_max) {
   extern __shared__ float smem[];
   typedef PoolOp<REDUCER> Op;
-  float *sp = smem;
-  float *sg = smem + prow_max * g.lds_pitch;
+  if (SY > 0) g.sy = SY;
+  if (SX > 0) g.sx = SX;
   const int plane = blockIdx.x / g.bands;
   const int band = blockIdx.x - plane * g.bands;
   const int y0 = band * g.band;
@@ -171,10 +193,12 @@ __global__ void __launch_bounds__(kPoolBlock)
   const int p0 = y0 < g.ky ? 0 : (y0 - g.ky + g.sy) / g.sy;
   const int p1 = min((ylast + g.sy) / g.sy, g.ph);
   const int np = max(p1 - p0, 0);
-  StageRows(sp, g.lds_pitch, pooled + (static_cast<size_t>(plane) * g.ph + p0) * pstride, pstride,
-            np, g.pw);
-  StageRows(sg, g.lds_pitch, grad + (static_cast<size_t>(plane) * g.ph + p0) * gstride, gstride,
-            np, g.pw);
+  const float *pin = pooled + (static_cast<size_t>(plane) * g.ph + p0) * pstride;
+  const float *gin = grad + (static_cast<size_t>(plane) * g.ph + p0) * gstride;
+  float *sp = smem + LdsPhase(pin);
+  float *sg = smem + prow_max * g.lds_pitch + 4 + LdsPhase(gin);
+  StageRows(sp, g.lds_pitch, pin, pstride, np, g.pw);
+  StageRows(sg, g.lds_pitch, gin, gstride, np, g.pw);
   const float *in = src + (static_cast<size_t>(plane) * g.h + y0) * sstride;
   float *out = dst + (static_cast<size_t>(plane) * g.h + y0) * dstride;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;

@@ -28,17 +28,15 @@ namespace mshadow_hipk {
 using mshadow::hip::kWave;
 using mshadow::hip::LaneId;
 using mshadow::hip::ReadLaneF32;
-using mshadow::hip::ReadLaneU32;
 using mshadow::hip::WaveId;
-using mshadow::hip::WaveInclusiveScanU32;
+using mshadow::hip::WaveInclusiveScanF32;
 using mshadow::hip::WaveMaxF32;
-using mshadow::hip::WaveSumU32;
 
 /*! \brief LDS scratch of the ordered sum: two alternating sets of per-wave totals and
  *  the hand-over slot for the running sum */
 template <int WAVES>
 struct OrderedSumLds {
-  uint32_t q[2][WAVES];
+  float q[2][WAVES];
   float s;
   float wmax[WAVES];
 };
@@ -52,14 +50,14 @@ __device__ inline float WaveResolve(float s, const float (&t)[N]) {
   int start = 0;
   while (true) {
     const Binade b = BinadeOf(s);
-    const uint32_t q = (lane >= start) ? LaneQuant<N>(t, b) : 0u;
-    const uint32_t incl = WaveInclusiveScanU32(q);  // <= 64 * 2^24, no overflow
-    const bool fail = (lane >= start) && (b.m + incl >= kBig);
+    const float q = (lane >= start) ? LaneQuant<N>(t, b) : 0.0f;
+    const float incl = WaveInclusiveScanF32(q);
+    const bool fail = (lane >= start) && !Fits(b, incl);
     const unsigned long long mask = __ballot(fail);
-    if (mask == 0ull) return Accept(s, b, ReadLaneU32(incl, kWave - 1));
+    if (mask == 0ull) return Accept(s, b, ReadLaneF32(incl, kWave - 1));
     const int first = __ffsll(mask) - 1;
-    /* lanes before `first` are exact integer adds */
-    s = Accept(s, b, ReadLaneU32(incl - q, first));
+    /* lanes before `first` are exact integer adds (their inclusive prefix is exact) */
+    s = Accept(s, b, first > 0 ? ReadLaneF32(incl, first - 1) : 0.0f);
     /* lane `first` does real float adds; every lane computes, one result is taken */
     s = ReadLaneF32(TrueAdd<N>(s, t), first);
     start = first + 1;
@@ -80,23 +78,18 @@ __device__ inline float BlockOrderedAdd(float s, const float (&t)[N],
   while (true) {
     const Binade b = BinadeOf(s);
     if (wave >= pos) {
-      uint32_t q = WaveSumU32(LaneQuant<N>(t, b));
-      if (lane == 0) lds->q[*buf][wave] = q < kBig ? q : kBig;
+      const float q = ReadLaneF32(WaveInclusiveScanF32(LaneQuant<N>(t, b)), kWave - 1);
+      if (lane == 0) lds->q[*buf][wave] = q;
     }
     __syncthreads();
-    /* every thread scans the per-wave totals (one LDS vector read, then registers) */
-    uint32_t qw[W];
-#pragma unroll
-    for (int w = 0; w < W; ++w) qw[w] = lds->q[*buf][w];
-    uint32_t acc = 0;
-    int failw = W;
-#pragma unroll
-    for (int w = 0; w < W; ++w) {
-      const bool live = w >= pos && failw == W;
-      const bool over = b.m + acc + qw[w] >= kBig;
-      if (live && over) failw = w;
-      if (live && !over) acc += qw[w];
-    }
+    /* the per-wave totals are scanned across lanes (lane w holds wave w's total): the
+       first wave whose inclusive prefix leaves the binade is the one to resolve */
+    const float qv = (lane < W && lane >= pos) ? lds->q[*buf][lane] : 0.0f;
+    const float incl = WaveInclusiveScanF32(qv);
+    const bool over = lane < W && lane >= pos && !Fits(b, incl);
+    const unsigned long long mask = __ballot(over);
+    const int failw = mask ? __ffsll(mask) - 1 : W;
+    const float acc = failw > 0 ? ReadLaneF32(incl, failw - 1) : 0.0f;
     *buf ^= 1;
     s = Accept(s, b, acc);
     if (failw == W) return s;
@@ -121,11 +114,14 @@ __device__ __forceinline__ float ExpNonPositive(float x) {
   const float t = x * kLog2eHi;
   float r = __builtin_fmaf(x, kLog2eHi, -t);   // exact rounding error of the product
   r = __builtin_fmaf(x, kLog2eLo, r);
-  const bool tiny = t < -125.0f;
-  const float e = __builtin_amdgcn_exp2f(tiny ? t + 64.0f : t);
-  const float v = __builtin_fmaf(e, r * 0.693147182464599609375f, e);  // e * 2^r, |r| << 1
-  if (t < -151.0f) return 0.0f;  // below half of the smallest subnormal (also x = -inf)
-  return tiny ? v * 5.42101086242752217003726400434970855712890625e-20f : v;  // 2^-64
+  if (__builtin_expect(!(t >= -125.0f), 0)) {   // subnormal / zero result, -inf, NaN
+    if (t < -151.0f) return 0.0f;               // below half of the smallest subnormal
+    const float e = __builtin_amdgcn_exp2f(t + 64.0f);
+    const float v = __builtin_fmaf(e, r * 0.693147182464599609375f, e);
+    return v * 5.42101086242752217003726400434970855712890625e-20f;  // 2^-64
+  }
+  const float e = __builtin_amdgcn_exp2f(t);
+  return __builtin_fmaf(e, r * 0.693147182464599609375f, e);  // e * 2^r, |r| << 1
 }
 
 /*! \brief p / s given rcp = 1 / s: one Newton correction on the quotient. The result is
@@ -151,7 +147,8 @@ __device__ inline float BlockMax(float v, OrderedSumLds<THREADS / kWave> *lds) {
   return m;
 }
 
-/*! \brief THREADS * SLABS * VEC >= cols. VEC == 4 needs 16-byte aligned rows. */
+/*! \brief THREADS * SLABS * VEC >= cols. VEC == 4 needs 16-byte aligned rows and
+ *  cols % 4 == 0. */
 template <int THREADS, int SLABS, int VEC>
 __global__ void __launch_bounds__(THREADS, 4)  // >= 4 waves per SIMD: two 512-thread rows per CU
     SoftmaxRowKernel(float *dst, int dstride, const float *src, int sstride, int cols) {
@@ -166,8 +163,9 @@ __global__ void __launch_bounds__(THREADS, 4)  // >= 4 waves per SIMD: two 512-t
 #pragma unroll
   for (int j = 0; j < SLABS; ++j) {
     const int base = (j * THREADS + tid) * VEC;
-    if (VEC == 4 && base + 4 <= cols) {
-      const float4 q = *reinterpret_cast<const float4 *>(in + base);
+    if (VEC == 4) {  // cols % 4 == 0: a pack is either whole or absent
+      float4 q = make_float4(kNegInf, kNegInf, kNegInf, kNegInf);
+      if (base < cols) q = *reinterpret_cast<const float4 *>(in + base);
       v[j][0] = q.x; v[j][1 % VEC] = q.y; v[j][2 % VEC] = q.z; v[j][3 % VEC] = q.w;
     } else {
 #pragma unroll
@@ -202,10 +200,10 @@ __global__ void __launch_bounds__(THREADS, 4)  // >= 4 waves per SIMD: two 512-t
     float o[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) o[i] = fast_div ? DivideBy(v[j][i], s, rcp) : v[j][i] / s;
-    if (VEC == 4 && base + 4 <= cols) {
+    if (VEC == 4) {
       float4 q;
       q.x = o[0]; q.y = o[1 % VEC]; q.z = o[2 % VEC]; q.w = o[3 % VEC];
-      *reinterpret_cast<float4 *>(out + base) = q;
+      if (base < cols) *reinterpret_cast<float4 *>(out + base) = q;
     } else {
 #pragma unroll
       for (int i = 0; i < VEC; ++i) {

@@ -60,6 +60,19 @@ __device__ __forceinline__ uint32_t WaveInclusiveScanU32(uint32_t v) {
   v += DppU32<MSHADOW_DPP_ROW_BCAST31, 0xc>(0u, v);
   return v;
 }
+/*! \brief the same for floats (used on integer-valued floats, where it is exact below 2^24) */
+__device__ __forceinline__ float WaveInclusiveScanF32(float v) {
+#define MSHADOW_FSCAN_STEP(CTRL, MASK) \
+  v += __uint_as_float(DppU32<CTRL, MASK>(0u, __float_as_uint(v)));
+  MSHADOW_FSCAN_STEP(MSHADOW_DPP_ROW_SHR(1), 0xf)
+  MSHADOW_FSCAN_STEP(MSHADOW_DPP_ROW_SHR(2), 0xf)
+  MSHADOW_FSCAN_STEP(MSHADOW_DPP_ROW_SHR(4), 0xf)
+  MSHADOW_FSCAN_STEP(MSHADOW_DPP_ROW_SHR(8), 0xf)
+  MSHADOW_FSCAN_STEP(MSHADOW_DPP_ROW_BCAST15, 0xa)
+  MSHADOW_FSCAN_STEP(MSHADOW_DPP_ROW_BCAST31, 0xc)
+#undef MSHADOW_FSCAN_STEP
+  return v;
+}
 /*! \brief sum over the 64 lanes; result in every lane (as a scalar) */
 __device__ __forceinline__ uint32_t WaveSumU32(uint32_t v) {
   return ReadLaneU32(WaveInclusiveScanU32(v), kWave - 1);

@@ -59,40 +59,53 @@ __device__ __forceinline__ DType WaveBroadcast(DType v, int lane) {
 /*! \brief fold vals[begin .. count) into res, in order. The operands of the next 32
  *  steps are fetched from LDS (eight 128-bit reads) while the current 32 dependent
  *  reductions execute, so a step costs one VALU issue plus a quarter of an LDS read. */
+template <typename Reducer, typename DType, int PACKS>
+__device__ __forceinline__ void ChainLoad(expr::Pack<DType, 4> (&dst)[PACKS], const DType *src) {
+#pragma unroll
+  for (int i = 0; i < PACKS; ++i) {
+    dst[i] = *reinterpret_cast<const expr::Pack<DType, 4> *>(src + 4 * i);
+  }
+}
+template <typename Reducer, typename DType, int PACKS>
+__device__ __forceinline__ void ChainApply(DType &res, const expr::Pack<DType, 4> (&p)[PACKS]) {
+#pragma unroll
+  for (int i = 0; i < PACKS; ++i) {
+    Reducer::Reduce(res, p[i].v[0]);
+    Reducer::Reduce(res, p[i].v[1]);
+    Reducer::Reduce(res, p[i].v[2]);
+    Reducer::Reduce(res, p[i].v[3]);
+  }
+}
+
 template <typename Reducer, typename DType>
 __device__ __forceinline__ void ChainFold(DType &res, const DType *vals, int begin, int count) {
   typedef expr::Pack<DType, 4> P4;
   const int kBlk = 32;
+  const int kPacks = kBlk / 4;
   int r = begin;
   for (; r < count && (r & (kBlk - 1)); ++r) Reducer::Reduce(res, vals[r]);
   if (r + kBlk <= count) {
-    P4 a[kBlk / 4];
-#pragma unroll
-    for (int i = 0; i < kBlk / 4; ++i) a[i] = *reinterpret_cast<const P4 *>(vals + r + 4 * i);
-    for (; r + 2 * kBlk <= count; r += kBlk) {
-      P4 b[kBlk / 4];
-#pragma unroll
-      for (int i = 0; i < kBlk / 4; ++i) {
-        b[i] = *reinterpret_cast<const P4 *>(vals + r + kBlk + 4 * i);
-      }
-#pragma unroll
-      for (int i = 0; i < kBlk / 4; ++i) {
-        Reducer::Reduce(res, a[i].v[0]);
-        Reducer::Reduce(res, a[i].v[1]);
-        Reducer::Reduce(res, a[i].v[2]);
-        Reducer::Reduce(res, a[i].v[3]);
-      }
-#pragma unroll
-      for (int i = 0; i < kBlk / 4; ++i) a[i] = b[i];
+    /* two register sets alternate: while one is being folded the other is in flight */
+    P4 a[kPacks], b[kPacks];
+    ChainLoad<Reducer, DType, kPacks>(a, vals + r);
+    for (; r + 3 * kBlk <= count; r += 2 * kBlk) {
+      ChainLoad<Reducer, DType, kPacks>(b, vals + r + kBlk);
+      __builtin_amdgcn_sched_barrier(0);
+      ChainApply<Reducer, DType, kPacks>(res, a);
+      ChainLoad<Reducer, DType, kPacks>(a, vals + r + 2 * kBlk);
+      __builtin_amdgcn_sched_barrier(0);
+      ChainApply<Reducer, DType, kPacks>(res, b);
     }
-#pragma unroll
-    for (int i = 0; i < kBlk / 4; ++i) {
-      Reducer::Reduce(res, a[i].v[0]);
-      Reducer::Reduce(res, a[i].v[1]);
-      Reducer::Reduce(res, a[i].v[2]);
-      Reducer::Reduce(res, a[i].v[3]);
+    if (r + 2 * kBlk <= count) {
+      ChainLoad<Reducer, DType, kPacks>(b, vals + r + kBlk);
+      __builtin_amdgcn_sched_barrier(0);
+      ChainApply<Reducer, DType, kPacks>(res, a);
+      ChainApply<Reducer, DType, kPacks>(res, b);
+      r += 2 * kBlk;
+    } else {
+      ChainApply<Reducer, DType, kPacks>(res, a);
+      r += kBlk;
     }
-    r += kBlk;
   }
   for (; r < count; ++r) Reducer::Reduce(res, vals[r]);
 }
@@ -125,20 +138,29 @@ __global__ void __launch_bounds__(THREADS)
   const uint32_t nstage = (rows + TR - 1) / TR;
   const bool chain_lane = (t < CW) && col_ok;  // lanes 0..CW-1 of wave 0 own the chains
 
+  /* loads are never predicated: out-of-range rows / columns re-read the last valid one
+     (their values are not consumed), so every stage issues exactly kRedDepth loads and
+     the wait before the LDS write can leave the next stage's loads in flight */
+  const uint32_t xc = col_ok ? x : cols - 1;
+  const uint32_t last_row = rows - 1;
   DType cur[kRedDepth], nxt[kRedDepth];
 #pragma unroll
   for (int k = 0; k < kRedDepth; ++k) {
     const uint32_t r = rsub + RPP * k;
-    cur[k] = (col_ok && r < rows) ? splan.Eval(r, x) : DType(0);
+    nxt[k] = splan.Eval(r < rows ? r : last_row, xc);
   }
   DType res = DType(0);
   for (uint32_t st = 0; st < nstage; ++st) {
     const uint32_t row0 = st * TR;
+    /* take delivery of this stage's loads, then put the next stage's in flight; they
+       travel while wave 0 runs the chain below */
+#pragma unroll
+    for (int k = 0; k < kRedDepth; ++k) cur[k] = nxt[k];
     if (st + 1 < nstage) {
 #pragma unroll
       for (int k = 0; k < kRedDepth; ++k) {
         const uint32_t r = row0 + TR + rsub + RPP * k;
-        nxt[k] = (col_ok && r < rows) ? splan.Eval(r, x) : DType(0);
+        nxt[k] = splan.Eval(r < rows ? r : last_row, xc);
       }
     }
     DType *buf = tile[st & 1];
@@ -155,8 +177,6 @@ __global__ void __launch_bounds__(THREADS)
       }
       ChainFold<Reducer>(res, mine, begin, count);
     }
-#pragma unroll
-    for (int k = 0; k < kRedDepth; ++k) cur[k] = nxt[k];
   }
   if (chain_lane) Saver::template Save<DType>(dplan.REval(0, x), res * scale);
 }
@@ -188,21 +208,22 @@ __global__ void __launch_bounds__(THREADS)
     const uint32_t e0_ = ((STAGE) - g_ * stages_per_group) * TL;                       \
     _Pragma("unroll") for (int k = 0; k < kRedDepth; ++k) {                            \
       const uint32_t f_ = k * THREADS + t;                                             \
-      const uint32_t n_ = g_ * SEGS + f_ / TL;                                         \
-      const uint32_t e_ = e0_ + f_ % TL;                                               \
-      DType v_ = DType(0);                                                             \
-      if (n_ < n_out && e_ < seg_len) {                                                \
-        const uint32_t y_ = e_ / n_x;                                                  \
-        v_ = splan.Eval((n_ * n_keep + c) * n_y + y_, e_ - y_ * n_x);                  \
-      }                                                                                \
-      REGS[k] = v_;                                                                    \
+      uint32_t n_ = g_ * SEGS + f_ / TL;                                               \
+      uint32_t e_ = e0_ + f_ % TL;                                                     \
+      /* never predicated (see KeepLowest): clamp to the last valid element */         \
+      n_ = n_ < n_out ? n_ : n_out - 1;                                                \
+      e_ = e_ < seg_len ? e_ : seg_len - 1;                                            \
+      const uint32_t y_ = e_ / n_x;                                                    \
+      REGS[k] = splan.Eval((n_ * n_keep + c) * n_y + y_, e_ - y_ * n_x);               \
     }                                                                                  \
   }
-  if (nstage > 0) MSHADOW_HIGHDIM_LOAD(cur, 0u)
+  if (nstage > 0) MSHADOW_HIGHDIM_LOAD(nxt, 0u)
   DType res, tres;
   Reducer::SetInitValue(res);
   Reducer::SetInitValue(tres);
   for (uint32_t st = 0; st < nstage; ++st) {
+#pragma unroll
+    for (int k = 0; k < kRedDepth; ++k) cur[k] = nxt[k];
     if (st + 1 < nstage) MSHADOW_HIGHDIM_LOAD(nxt, st + 1)
     DType *buf = tile[st & 1];
 #pragma unroll
@@ -229,8 +250,6 @@ __global__ void __launch_bounds__(THREADS)
         Reducer::SetInitValue(tres);
       }
     }
-#pragma unroll
-    for (int k = 0; k < kRedDepth; ++k) cur[k] = nxt[k];
   }
 #undef MSHADOW_HIGHDIM_LOAD
   if (t == 0) Saver::template Save<DType>(dplan.REval(0, c), DType(res * scale));

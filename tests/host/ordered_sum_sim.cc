@@ -30,19 +30,18 @@ static float WaveResolveSim(float s, const float (*t)[N]) {  // t[64][N]
   int start = 0;
   while (true) {
     Binade b = BinadeOf(s);
-    uint32_t q[64], incl[64];
-    uint32_t run = 0;
+    float incl[64];
+    float run = 0.0f;
     for (int l = 0; l < 64; ++l) {
-      q[l] = (l >= start) ? LaneQuant<N>(t[l], b) : 0u;
-      run += q[l];
+      run += (l >= start) ? LaneQuant<N>(t[l], b) : 0.0f;  // lane order, like the DPP scan
       incl[l] = run;
     }
     int first = -1;
     for (int l = start; l < 64; ++l) {
-      if (b.m + incl[l] >= kBig) { first = l; break; }
+      if (!Fits(b, incl[l])) { first = l; break; }
     }
     if (first < 0) return Accept(s, b, incl[63]);
-    s = Accept(s, b, incl[first] - q[first]);
+    s = Accept(s, b, first > 0 ? incl[first - 1] : 0.0f);
     s = TrueAdd<N>(s, t[first]);
     start = first + 1;
     if (start == 64) return s;
@@ -54,19 +53,20 @@ static float BlockAddSim(float s, const float (*t)[N], long *resolves) {  // t[W
   int pos = 0;
   while (true) {
     Binade b = BinadeOf(s);
-    uint32_t qw[W];
+    float qw[W];
     for (int w = pos; w < W; ++w) {
-      uint32_t q = 0;
+      float q = 0.0f;
       for (int l = 0; l < 64; ++l) q += LaneQuant<N>(t[w * 64 + l], b);
-      qw[w] = q < kBig ? q : kBig;
+      qw[w] = q;
     }
-    uint32_t acc = 0;
+    float acc = 0.0f, prev = 0.0f;
     int failw = W;
     for (int w = pos; w < W; ++w) {
-      if (b.m + acc + qw[w] >= kBig) { failw = w; break; }
       acc += qw[w];
+      if (!Fits(b, acc)) { failw = w; break; }
+      prev = acc;
     }
-    s = Accept(s, b, acc);
+    s = Accept(s, b, prev);
     if (failw == W) return s;
     s = WaveResolveSim<N>(s, t + failw * 64);
     ++*resolves;
