@@ -227,14 +227,17 @@ int mshadow_hip_softmax_grad_f32(float *dst, int dstride, const float *src, int 
   ABI_REQUIRE(dstride >= cols && sstride >= cols, "pitch smaller than the row");
   const int per_block = kGradBlock * kGradPacks * 4;
   const unsigned chunks = (cols + per_block - 1) / per_block;
-  ABI_REQUIRE(chunks <= 65535u, "row too long");
+  const unsigned long long blocks = static_cast<unsigned long long>(rows) * chunks;
+  ABI_REQUIRE(blocks < (1ull << 31), "too many workgroups");
   const bool vec = Aligned16(dst) && Aligned16(src) && dstride % 4 == 0 && sstride % 4 == 0;
   if (vec) {
-    hipLaunchKernelGGL((SoftmaxGradKernel<true>), dim3(rows, chunks), dim3(kGradBlock), 0,
-                       AsStream(stream), dst, dstride, src, sstride, label, cols);
+    hipLaunchKernelGGL((SoftmaxGradKernel<true>), dim3(static_cast<unsigned>(blocks)),
+                       dim3(kGradBlock), 0, AsStream(stream), dst, dstride, src, sstride, label,
+                       cols, chunks);
   } else {
-    hipLaunchKernelGGL((SoftmaxGradKernel<false>), dim3(rows, chunks), dim3(kGradBlock), 0,
-                       AsStream(stream), dst, dstride, src, sstride, label, cols);
+    hipLaunchKernelGGL((SoftmaxGradKernel<false>), dim3(static_cast<unsigned>(blocks)),
+                       dim3(kGradBlock), 0, AsStream(stream), dst, dstride, src, sstride, label,
+                       cols, chunks);
   }
   return AfterLaunch("softmax_grad");
 }
@@ -427,28 +430,28 @@ int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstrid
     const size_t lds = static_cast<size_t>(prow_max) * row_bytes + 32;
     const long long blocks = static_cast<long long>(planes) * g.bands;
     ABI_REQUIRE(blocks < (1ll << 31), "too many workgroups");
-#define UNPOOL_TILED(SY, SX)                                                                   \
+#define UNPOOL_TILED(KY, KX, SY, SX)                                                                   \
   switch (reducer) {                                                                           \
     case MSHADOW_HIP_SUM:                                                                      \
-      hipLaunchKernelGGL((UnpoolKernel<MSHADOW_HIP_SUM, SY, SX>),                              \
+      hipLaunchKernelGGL((UnpoolKernel<MSHADOW_HIP_SUM, KY, KX, SY, SX>),                              \
                          dim3(static_cast<unsigned>(blocks)), dim3(kPoolBlock), lds, s, dst,   \
                          dstride, src, sstride, pooled, pstride, grad, gstride, g, prow_max);  \
       break;                                                                                   \
     case MSHADOW_HIP_MAX:                                                                      \
-      hipLaunchKernelGGL((UnpoolKernel<MSHADOW_HIP_MAX, SY, SX>),                              \
+      hipLaunchKernelGGL((UnpoolKernel<MSHADOW_HIP_MAX, KY, KX, SY, SX>),                              \
                          dim3(static_cast<unsigned>(blocks)), dim3(kPoolBlock), lds, s, dst,   \
                          dstride, src, sstride, pooled, pstride, grad, gstride, g, prow_max);  \
       break;                                                                                   \
     default:                                                                                   \
-      hipLaunchKernelGGL((UnpoolKernel<MSHADOW_HIP_MIN, SY, SX>),                              \
+      hipLaunchKernelGGL((UnpoolKernel<MSHADOW_HIP_MIN, KY, KX, SY, SX>),                              \
                          dim3(static_cast<unsigned>(blocks)), dim3(kPoolBlock), lds, s, dst,   \
                          dstride, src, sstride, pooled, pstride, grad, gstride, g, prow_max);  \
       break;                                                                                   \
   }
-    if (sy == 2 && sx == 2) { UNPOOL_TILED(2, 2) }
-    else if (sy == 1 && sx == 1) { UNPOOL_TILED(1, 1) }
-    else if (sy == 3 && sx == 3) { UNPOOL_TILED(3, 3) }
-    else { UNPOOL_TILED(0, 0) }
+    if (ky == 3 && kx == 3 && sy == 2 && sx == 2) { UNPOOL_TILED(3, 3, 2, 2) }
+    else if (ky == 2 && kx == 2 && sy == 2 && sx == 2) { UNPOOL_TILED(2, 2, 2, 2) }
+    else if (ky == 3 && kx == 3 && sy == 1 && sx == 1) { UNPOOL_TILED(3, 3, 1, 1) }
+    else { UNPOOL_TILED(0, 0, 0, 0) }
 #undef UNPOOL_TILED
   } else {
     const unsigned total = static_cast<unsigned>(planes) * h * w;

@@ -19,6 +19,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "stream_access.h"
+
 namespace mshadow_hipk {
 
 const int kPatchBlock = 256;
@@ -129,12 +131,10 @@ __global__ void __launch_bounds__(kPatchBlock)
           }
         }
         T *out = row + e0;
-        if (e0 + EPT <= count && reinterpret_cast<uintptr_t>(out) % (sizeof(T) * EPT) == 0) {
-          typedef T Vec __attribute__((ext_vector_type(EPT)));
-          Vec pack;
-#pragma unroll
-          for (int e = 0; e < EPT; ++e) pack[e] = vals[e];
-          *reinterpret_cast<Vec *>(out) = pack;
+        if (e0 + EPT <= count && reinterpret_cast<uintptr_t>(out) % 16 == 0) {
+          U4 pack;  // EPT elements are exactly 16 bytes
+          __builtin_memcpy(&pack, vals, 16);
+          StreamStore16(out, pack);
         } else {
 #pragma unroll
           for (int e = 0; e < EPT; ++e) {
@@ -184,8 +184,7 @@ __global__ void __launch_bounds__(kPatchBlock)
     const bool vec_ok = reinterpret_cast<uintptr_t>(in) % (sizeof(T) * EPT) == 0;
     for (int e0 = threadIdx.x * EPT; e0 < run; e0 += kPatchBlock * EPT) {
       if (vec_ok && e0 + EPT <= run) {
-        typedef T Vec __attribute__((ext_vector_type(EPT)));
-        *reinterpret_cast<Vec *>(out + e0) = *reinterpret_cast<const Vec *>(in + e0);
+        *reinterpret_cast<U4 *>(out + e0) = StreamLoad16(in + e0);
       } else {
 #pragma unroll
         for (int e = 0; e < EPT; ++e) {

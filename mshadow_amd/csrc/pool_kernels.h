@@ -23,6 +23,8 @@
 
 #include <cfloat>
 
+#include "stream_access.h"
+
 namespace mshadow_hipk {
 
 const int kPoolBlock = 256;
@@ -75,15 +77,15 @@ __device__ __forceinline__ void StageRows(float *lds, int lpitch, const float *g
     const int head = lead < total ? lead : total;
     if (static_cast<int>(threadIdx.x) < head) lds[threadIdx.x] = g[threadIdx.x];
     const int nvec = (total - head) / 4;
-    const float4 *gv = reinterpret_cast<const float4 *>(g + head);
-    float4 *lv = reinterpret_cast<float4 *>(lds + head);
+    const float *gv = g + head;
+    F4 *lv = reinterpret_cast<F4 *>(lds + head);
     const int kUnroll = 8;
     for (int v0 = threadIdx.x; v0 < nvec; v0 += kPoolBlock * kUnroll) {
-      float4 q[kUnroll];
+      F4 q[kUnroll];
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {  // unpredicated: past the end re-reads the last pack
         const int v = v0 + u * kPoolBlock;
-        q[u] = gv[v < nvec ? v : nvec - 1];
+        q[u] = StreamLoadF4(gv + 4 * (v < nvec ? v : nvec - 1));
       }
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
@@ -145,7 +147,7 @@ __global__ void __launch_bounds__(kPoolBlock)
           for (int x = xs; x < xe; ++x) res = Op::Reduce(res, tile[y * g.lds_pitch + x]);
         }
       }
-      out[static_cast<size_t>(py) * dstride + px] = res;
+      StreamStore(out + static_cast<size_t>(py) * dstride + px, res);
     }
   }
 }
@@ -174,16 +176,21 @@ __global__ void __launch_bounds__(kPoolBlock)
 
 /*! \brief grid.x = planes * bands over SOURCE rows. Dynamic LDS: two arrays (pooled,
  *  grad) of prow_max * lds_pitch + 4 floats, prow_max = (band + ky - 2) / sy + 2.
- *  SY / SX > 0 fix the strides at compile time so that the divisions below become
- *  multiplications; 0 means "use g.sy / g.sx". */
-template <int REDUCER, int SY, int SX>
+ *  KY, KX, SY, SX > 0 fix the window and stride at compile time: the number of windows
+ *  that can cover a pixel, ceil(K / S) per direction, is then a constant, the loops unroll
+ *  and the range divisions become shifts. 0 means "use the run-time value". A candidate
+ *  window that does not exist is skipped with a select, which leaves `val` untouched
+ *  exactly like the reference's loop bounds do. */
+template <int REDUCER, int KY, int KX, int SY, int SX>
 __global__ void __launch_bounds__(kPoolBlock)
     UnpoolKernel(float *dst, int dstride, const float *src, int sstride, const float *pooled,
                  int pstride, const float *grad, int gstride, PoolGeom g, int prow_max) {
   extern __shared__ float smem[];
   typedef PoolOp<REDUCER> Op;
-  if (SY > 0) g.sy = SY;
-  if (SX > 0) g.sx = SX;
+  const bool kFixed = KY > 0 && KX > 0 && SY > 0 && SX > 0;
+  if (kFixed) {
+    g.ky = KY; g.kx = KX; g.sy = SY; g.sx = SX;
+  }
   const int plane = blockIdx.x / g.bands;
   const int band = blockIdx.x - plane * g.bands;
   const int y0 = band * g.band;
@@ -201,9 +208,11 @@ __global__ void __launch_bounds__(kPoolBlock)
   StageRows(sg, g.lds_pitch, gin, gstride, np, g.pw);
   const float *in = src + (static_cast<size_t>(plane) * g.h + y0) * sstride;
   float *out = dst + (static_cast<size_t>(plane) * g.h + y0) * dstride;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   /* each lane fetches its source pixel of kRowsAhead rows before using any of them */
   const int kRowsAhead = 4;
+  const int kCandY = kFixed ? (KY + SY - 1) / (SY > 0 ? SY : 1) : 1;
+  const int kCandX = kFixed ? (KX + SX - 1) / (SX > 0 ? SX : 1) : 1;
   __syncthreads();
   for (int yr0 = wave; yr0 < ny; yr0 += kPoolWaves * kRowsAhead) {
     for (int x = lane; x < g.w; x += 64) {
@@ -211,7 +220,7 @@ __global__ void __launch_bounds__(kPoolBlock)
 #pragma unroll
       for (int u = 0; u < kRowsAhead; ++u) {
         const int yr = yr0 + u * kPoolWaves;
-        vs[u] = (yr < ny) ? in[static_cast<size_t>(yr) * sstride + x] : 0.0f;
+        vs[u] = (yr < ny) ? StreamLoad(in + static_cast<size_t>(yr) * sstride + x) : 0.0f;
       }
       const int px_min = x < g.kx ? 0 : (x - g.kx + g.sx) / g.sx;
       const int px_max = min((x + g.sx) / g.sx, g.pw);
@@ -223,13 +232,29 @@ __global__ void __launch_bounds__(kPoolBlock)
           const int py_min = y < g.ky ? 0 : (y - g.ky + g.sy) / g.sy;
           const int py_max = min((y + g.sy) / g.sy, g.ph);
           float val = 0.0f;
-          for (int py = py_min; py < py_max; ++py) {
-            for (int px = px_min; px < px_max; ++px) {
-              const int li = (py - p0) * g.lds_pitch + px;
-              val = val + Op::Grad(vs[u], sp[li]) * sg[li];
+          if (kFixed) {
+#pragma unroll
+            for (int iy = 0; iy < kCandY; ++iy) {
+              const int py = py_min + iy;
+#pragma unroll
+              for (int ix = 0; ix < kCandX; ++ix) {
+                const int px = px_min + ix;
+                const bool live = py < py_max && px < px_max;
+                /* clamp the LDS index of a missing candidate into the staged area */
+                const int li = live ? (py - p0) * g.lds_pitch + px : 0;
+                const float t = val + Op::Grad(vs[u], sp[li]) * sg[li];
+                val = live ? t : val;
+              }
+            }
+          } else {
+            for (int py = py_min; py < py_max; ++py) {
+              for (int px = px_min; px < px_max; ++px) {
+                const int li = (py - p0) * g.lds_pitch + px;
+                val = val + Op::Grad(vs[u], sp[li]) * sg[li];
+              }
             }
           }
-          out[static_cast<size_t>(yr) * dstride + x] = val;
+          StreamStore(out + static_cast<size_t>(yr) * dstride + x, val);
         }
       }
     }

@@ -22,6 +22,7 @@
 #include <mshadow/hip/kernels/common.h>
 
 #include "ordered_sum.h"
+#include "stream_access.h"
 
 namespace mshadow_hipk {
 
@@ -164,8 +165,8 @@ __global__ void __launch_bounds__(THREADS, 4)  // >= 4 waves per SIMD: two 512-t
   for (int j = 0; j < SLABS; ++j) {
     const int base = (j * THREADS + tid) * VEC;
     if (VEC == 4) {  // cols % 4 == 0: a pack is either whole or absent
-      float4 q = make_float4(kNegInf, kNegInf, kNegInf, kNegInf);
-      if (base < cols) q = *reinterpret_cast<const float4 *>(in + base);
+      F4 q = {kNegInf, kNegInf, kNegInf, kNegInf};
+      if (base < cols) q = StreamLoadF4(in + base);
       v[j][0] = q.x; v[j][1 % VEC] = q.y; v[j][2 % VEC] = q.z; v[j][3 % VEC] = q.w;
     } else {
 #pragma unroll
@@ -201,9 +202,9 @@ __global__ void __launch_bounds__(THREADS, 4)  // >= 4 waves per SIMD: two 512-t
 #pragma unroll
     for (int i = 0; i < VEC; ++i) o[i] = fast_div ? DivideBy(v[j][i], s, rcp) : v[j][i] / s;
     if (VEC == 4) {
-      float4 q;
+      F4 q;
       q.x = o[0]; q.y = o[1 % VEC]; q.z = o[2 % VEC]; q.w = o[3 % VEC];
-      if (base < cols) *reinterpret_cast<float4 *>(out + base) = q;
+      if (base < cols) StreamStoreF4(out + base, q);
     } else {
 #pragma unroll
       for (int i = 0; i < VEC; ++i) {
@@ -241,24 +242,27 @@ __global__ void __launch_bounds__(THREADS)
 }
 
 const int kGradBlock = 256;
-const int kGradPacks = 4;  // 128-bit packs per thread
+const int kGradPacks = 2;  // 128-bit packs per thread
 
-/*! \brief grid.x = rows, grid.y = column chunks of kGradBlock * kGradPacks * 4 elements */
+/*! \brief grid.x = rows * chunks, a chunk being kGradBlock * kGradPacks * 4 columns.
+ *  Consecutive workgroups walk along a row, so the workgroups in flight at any moment
+ *  stream one contiguous region of memory. */
 template <bool VEC4>
 __global__ void __launch_bounds__(kGradBlock)
     SoftmaxGradKernel(float *dst, int dstride, const float *src, int sstride, const float *label,
-                      int cols) {
-  const int y = blockIdx.x;
+                      int cols, unsigned chunks) {
+  const int y = blockIdx.x / chunks;
+  const int chunk = blockIdx.x - y * chunks;
   const int k = static_cast<int>(label[y]);
   const float *in = src + static_cast<size_t>(y) * sstride;
   float *out = dst + static_cast<size_t>(y) * dstride;
-  const int chunk0 = blockIdx.y * (kGradBlock * kGradPacks * 4);
+  const int chunk0 = chunk * (kGradBlock * kGradPacks * 4);
   if (VEC4) {
-    float4 q[kGradPacks];
+    F4 q[kGradPacks];
 #pragma unroll
     for (int u = 0; u < kGradPacks; ++u) {
       const int x = chunk0 + (u * kGradBlock + threadIdx.x) * 4;
-      if (x + 4 <= cols) q[u] = *reinterpret_cast<const float4 *>(in + x);
+      if (x + 4 <= cols) q[u] = StreamLoadF4(in + x);
     }
 #pragma unroll
     for (int u = 0; u < kGradPacks; ++u) {
@@ -268,7 +272,7 @@ __global__ void __launch_bounds__(kGradBlock)
         if (k == x + 1) q[u].y = q[u].y - 1.0f;
         if (k == x + 2) q[u].z = q[u].z - 1.0f;
         if (k == x + 3) q[u].w = q[u].w - 1.0f;
-        *reinterpret_cast<float4 *>(out + x) = q[u];
+        StreamStoreF4(out + x, q[u]);
       } else {
         for (int i = x; i < cols; ++i) out[i] = (i == k) ? in[i] - 1.0f : in[i];
       }

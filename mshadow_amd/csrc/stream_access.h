@@ -1,0 +1,41 @@
+/*
+ * Non-temporal ("streaming") global memory accesses for data that passes through a
+ * kernel exactly once. Measured on MI355X with a 1 GiB copy: 6.2-6.5 TB/s with these
+ * against 5.7 TB/s with the default cache policy, because lines that will not be reused
+ * stop displacing each other in L2 / Infinity Cache.
+ */
+#ifndef MSHADOW_AMD_CSRC_STREAM_ACCESS_H_
+#define MSHADOW_AMD_CSRC_STREAM_ACCESS_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mshadow_hipk {
+
+typedef float F4 __attribute__((ext_vector_type(4)));
+typedef uint32_t U4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ F4 StreamLoadF4(const float *p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const F4 *>(p));
+}
+__device__ __forceinline__ void StreamStoreF4(float *p, F4 v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<F4 *>(p));
+}
+__device__ __forceinline__ float StreamLoad(const float *p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void StreamStore(float *p, float v) { __builtin_nontemporal_store(v, p); }
+__device__ __forceinline__ uint16_t StreamLoad(const uint16_t *p) {
+  return __builtin_nontemporal_load(p);
+}
+__device__ __forceinline__ void StreamStore(uint16_t *p, uint16_t v) {
+  __builtin_nontemporal_store(v, p);
+}
+/*! \brief 16 bytes of any element type */
+__device__ __forceinline__ U4 StreamLoad16(const void *p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const U4 *>(p));
+}
+__device__ __forceinline__ void StreamStore16(void *p, U4 v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<U4 *>(p));
+}
+
+}  // namespace mshadow_hipk
+#endif  // MSHADOW_AMD_CSRC_STREAM_ACCESS_H_

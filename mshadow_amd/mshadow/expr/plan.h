@@ -10,7 +10,8 @@
  * Added for gfx950: plans made only of tensors, scalars and elementwise maps also
  * evaluate N adjacent columns at once (EvalPack<N>) from one 128-bit global load per
  * tensor leaf. A plan advertises that with `kPackable`; PackReady() checks at run
- * time that every leaf pointer and pitch is aligned for N-wide access. Plans without
+ * time that every leaf pointer and pitch is aligned for N-wide access. EvalPack's second
+ * template argument asks the leaves for non-temporal (streaming) accesses. Plans without
  * these members (caller-defined ones) simply take the scalar path.
  */
 #ifndef MSHADOW_EXPR_PLAN_H_
@@ -28,6 +29,54 @@ template <typename DType, int N>
 struct MSHADOW_ALIGNED(sizeof(DType) * N) Pack {
   DType v[N];
 };
+
+namespace plan_detail {
+/*! \brief raw 128/64/32-bit vector used to move a Pack with one memory instruction */
+template <int BYTES>
+struct RawVec {
+  typedef uint32_t type __attribute__((ext_vector_type(BYTES / 4)));
+};
+template <>
+struct RawVec<4> {
+  typedef uint32_t type;
+};
+template <>
+struct RawVec<2> {
+  typedef uint16_t type;
+};
+template <>
+struct RawVec<1> {
+  typedef uint8_t type;
+};
+/*! \brief load / store one Pack. STREAM marks the access non-temporal: the data passes
+ *  through once and should not displace other lines in the caches (device code only). */
+template <typename DType, int N, bool STREAM>
+MSHADOW_XINLINE Pack<DType, N> LoadPack(const DType *p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  if (STREAM) {
+    typedef typename RawVec<sizeof(DType) * N>::type Raw;
+    const Raw raw = __builtin_nontemporal_load(reinterpret_cast<const Raw *>(p));
+    Pack<DType, N> out;
+    __builtin_memcpy(&out, &raw, sizeof(out));
+    return out;
+  }
+#endif
+  return *reinterpret_cast<const Pack<DType, N> *>(p);
+}
+template <typename DType, int N, bool STREAM>
+MSHADOW_XINLINE void StorePackTo(DType *p, const Pack<DType, N> &v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  if (STREAM) {
+    typedef typename RawVec<sizeof(DType) * N>::type Raw;
+    Raw raw;
+    __builtin_memcpy(&raw, &v, sizeof(raw));
+    __builtin_nontemporal_store(raw, reinterpret_cast<Raw *>(p));
+    return;
+  }
+#endif
+  *reinterpret_cast<Pack<DType, N> *>(p) = v;
+}
+}  // namespace plan_detail
 
 /*! \brief base of the chainer nodes: a node that knows its own output shape */
 template <typename SubType, typename SrcExp, int dim, typename DType>
@@ -52,13 +101,13 @@ class Plan<Tensor<Device, dim, DType>, DType> {
   explicit Plan(const Tensor<Device, dim, DType> &t) : dptr_(t.dptr_), stride_(t.stride_) {}
   MSHADOW_XINLINE DType &REval(index_t y, index_t x) { return dptr_[y * stride_ + x]; }
   MSHADOW_XINLINE const DType &Eval(index_t y, index_t x) const { return dptr_[y * stride_ + x]; }
-  template <int N>
+  template <int N, bool STREAM = false>
   MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t x) const {
-    return *reinterpret_cast<const Pack<DType, N> *>(dptr_ + y * stride_ + x);
+    return plan_detail::LoadPack<DType, N, STREAM>(dptr_ + y * stride_ + x);
   }
-  template <int N>
+  template <int N, bool STREAM = false>
   MSHADOW_XINLINE void StorePack(index_t y, index_t x, const Pack<DType, N> &p) {
-    *reinterpret_cast<Pack<DType, N> *>(dptr_ + y * stride_ + x) = p;
+    plan_detail::StorePackTo<DType, N, STREAM>(dptr_ + y * stride_ + x, p);
   }
   /*! \brief host check: pointer and pitch allow n-wide access; *flat stays true only
    *  while rows are dense (pitch == cols) so that the 2-D view can be walked linearly */
@@ -79,13 +128,13 @@ class Plan<Tensor<Device, 1, DType>, DType> {
   explicit Plan(const Tensor<Device, 1, DType> &t) : dptr_(t.dptr_) {}
   MSHADOW_XINLINE DType &REval(index_t y, index_t x) { return dptr_[x]; }
   MSHADOW_XINLINE const DType &Eval(index_t y, index_t x) const { return dptr_[x]; }
-  template <int N>
+  template <int N, bool STREAM = false>
   MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t x) const {
-    return *reinterpret_cast<const Pack<DType, N> *>(dptr_ + x);
+    return plan_detail::LoadPack<DType, N, STREAM>(dptr_ + x);
   }
-  template <int N>
+  template <int N, bool STREAM = false>
   MSHADOW_XINLINE void StorePack(index_t y, index_t x, const Pack<DType, N> &p) {
-    *reinterpret_cast<Pack<DType, N> *>(dptr_ + x) = p;
+    plan_detail::StorePackTo<DType, N, STREAM>(dptr_ + x, p);
   }
   inline bool PackReady(int n, index_t cols, bool *flat) const {
     return reinterpret_cast<uintptr_t>(dptr_) % (sizeof(DType) * n) == 0;
@@ -101,7 +150,7 @@ class Plan<ScalarExp<DType>, DType> {
   static const bool kPackable = true;
   explicit Plan(DType scalar) : scalar_(scalar) {}
   MSHADOW_XINLINE DType Eval(index_t y, index_t x) const { return scalar_; }
-  template <int N>
+  template <int N, bool STREAM = false>
   MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t x) const {
     Pack<DType, N> p;
 #pragma unroll
@@ -151,11 +200,11 @@ class Plan<TernaryMapExp<OP, TA, TB, TC, DType, etype>, DType> {
   MSHADOW_XINLINE DType Eval(index_t y, index_t x) const {
     return OP::Map(item1_.Eval(y, x), item2_.Eval(y, x), item3_.Eval(y, x));
   }
-  template <int N>
+  template <int N, bool STREAM = false>
   MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t x) const {
-    const Pack<DType, N> a = item1_.template EvalPack<N>(y, x);
-    const Pack<DType, N> b = item2_.template EvalPack<N>(y, x);
-    const Pack<DType, N> c = item3_.template EvalPack<N>(y, x);
+    const Pack<DType, N> a = item1_.template EvalPack<N, STREAM>(y, x);
+    const Pack<DType, N> b = item2_.template EvalPack<N, STREAM>(y, x);
+    const Pack<DType, N> c = item3_.template EvalPack<N, STREAM>(y, x);
     Pack<DType, N> r;
 #pragma unroll
     for (int i = 0; i < N; ++i) r.v[i] = OP::Map(a.v[i], b.v[i], c.v[i]);
@@ -181,10 +230,10 @@ class Plan<BinaryMapExp<OP, TA, TB, DType, etype>, DType> {
   MSHADOW_XINLINE DType Eval(index_t y, index_t x) const {
     return OP::Map(lhs_.Eval(y, x), rhs_.Eval(y, x));
   }
-  template <int N>
+  template <int N, bool STREAM = false>
   MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t x) const {
-    const Pack<DType, N> a = lhs_.template EvalPack<N>(y, x);
-    const Pack<DType, N> b = rhs_.template EvalPack<N>(y, x);
+    const Pack<DType, N> a = lhs_.template EvalPack<N, STREAM>(y, x);
+    const Pack<DType, N> b = rhs_.template EvalPack<N, STREAM>(y, x);
     Pack<DType, N> r;
 #pragma unroll
     for (int i = 0; i < N; ++i) r.v[i] = OP::Map(a.v[i], b.v[i]);
@@ -205,9 +254,9 @@ class Plan<UnaryMapExp<OP, TA, DType, etype>, DType> {
   static const bool kPackable = plan_detail::Packable<Plan<TA, DType> >::value;
   explicit Plan(const Plan<TA, DType> &src) : src_(src) {}
   MSHADOW_XINLINE DType Eval(index_t y, index_t x) const { return OP::Map(src_.Eval(y, x)); }
-  template <int N>
+  template <int N, bool STREAM = false>
   MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t x) const {
-    const Pack<DType, N> a = src_.template EvalPack<N>(y, x);
+    const Pack<DType, N> a = src_.template EvalPack<N, STREAM>(y, x);
     Pack<DType, N> r;
 #pragma unroll
     for (int i = 0; i < N; ++i) r.v[i] = OP::Map(a.v[i]);

@@ -360,13 +360,22 @@ struct MapLauncher<Saver, DType, DPlan, SPlan, true> {
     const uint32_t per_block = hip::kMapBlock * hip::kPackUnroll;
     const uint32_t grid = (total + per_block - 1) / per_block;
     void *args[] = {&dplan, &splan, &total, &ppr};
-    if (flat || rows == 1) {
-      Launch(hip::MapPackKernel<Saver, DType, N, true, DPlan, SPlan>, grid, hip::kMapBlock, args,
-             stream);
+    /* streaming (non-temporal) accesses once a tensor no longer fits the caches anyway */
+    const bool stream_hint = static_cast<size_t>(rows) * cols * sizeof(DType) >= (8u << 20);
+    const bool is_flat = flat || rows == 1;
+#define MSHADOW_MAP_LAUNCH(FLAT, STREAM)                                                   \
+  Launch(hip::MapPackKernel<Saver, DType, N, FLAT, STREAM, DPlan, SPlan>, grid, hip::kMapBlock, \
+         args, stream)
+    if (is_flat && stream_hint) {
+      MSHADOW_MAP_LAUNCH(true, true);
+    } else if (is_flat) {
+      MSHADOW_MAP_LAUNCH(true, false);
+    } else if (stream_hint) {
+      MSHADOW_MAP_LAUNCH(false, true);
     } else {
-      Launch(hip::MapPackKernel<Saver, DType, N, false, DPlan, SPlan>, grid, hip::kMapBlock, args,
-             stream);
+      MSHADOW_MAP_LAUNCH(false, false);
     }
+#undef MSHADOW_MAP_LAUNCH
   }
 };
 #endif  // __HIPCC__
