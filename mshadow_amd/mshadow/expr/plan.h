@@ -34,7 +34,11 @@ namespace plan_detail {
 /*! \brief raw 128/64/32-bit vector used to move a Pack with one memory instruction */
 template <int BYTES>
 struct RawVec {
+#if defined(__clang__)
   typedef uint32_t type __attribute__((ext_vector_type(BYTES / 4)));
+#else
+  struct type { uint32_t w[BYTES / 4]; };  // host compilers never issue the streaming forms
+#endif
 };
 template <>
 struct RawVec<4> {
