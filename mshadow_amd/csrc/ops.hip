@@ -7,6 +7,7 @@
 #include "abi_common.h"
 
 #include <mshadow/hip/kernels/reduce.h>
+#include <mshadow/hip/kernels/reduce_dma.h>
 
 #include "patch_kernels.h"
 #include "pool_kernels.h"
@@ -61,6 +62,10 @@ int DispatchReducer(int reducer, F f) {
 
 namespace {
 const size_t kPatchLdsBudget = 40 * 1024;  // per workgroup
+/* reductions long enough to fill the LDS ring of the direct-to-LDS kernels (which hold
+   a whole CU's LDS); shorter ones run the register-staged kernels, several per CU */
+const int kDmaMinRows = 2048;
+const long long kDmaMinPerKept = 1ll << 16;
 
 int MakePatchGeom(PatchGeom *g, int n, int c, int h, int w, int ky, int kx, int sy, int sx,
                   int dy, int dx, int pad_y, int pad_x) {
@@ -260,7 +265,12 @@ int mshadow_hip_reduce_keep_lowest_f32(float *dst, const float *src, int sstride
     return DispatchSaver(saver, [&](auto sv) {
       typedef decltype(red) R;
       typedef decltype(sv) S;
-      if (rows >= 4096) {
+      if (rows >= kDmaMinRows) {
+        hipLaunchKernelGGL((mshadow::hip::ReduceKeepLowestDmaKernel<S, R>), dim3(grid),
+                           dim3(mshadow::hip::kDmaThreads), 0, s, dst, src,
+                           static_cast<uint32_t>(sstride), static_cast<uint32_t>(rows),
+                           static_cast<uint32_t>(cols), scale);
+      } else if (rows >= 4096) {
         hipLaunchKernelGGL(
             (mshadow::hip::ReduceKeepLowestKernel<S, R, float, mshadow::hip::kRedBlockLarge,
                                                   RawPlan1D<float>, RawPlan2D<const float> >),
@@ -289,8 +299,10 @@ int mshadow_hip_reduce_keep_highdim_f32(float *dst, const float *src, int sstrid
   ABI_REQUIRE(src != NULL || static_cast<long long>(n) * y * x == 0, "NULL tensor");
   ABI_REQUIRE(sstride >= x, "pitch smaller than the row");
   ABI_REQUIRE(static_cast<long long>(n) * c * y < (1ll << 31), "too many rows for 32-bit indices");
+  ABI_REQUIRE(static_cast<long long>(y) * x < (1ll << 31), "inner extent too large for 32-bit indices");
   RawPlan1D<float> d = {dst};
   RawPlan2D<const float> sp = {src, sstride};
+  const mshadow::FastDivU32 div_x(static_cast<uint32_t>(x > 0 ? x : 1));
   hipStream_t s = AsStream(stream);
   int st = DispatchReducer(reducer, [&](auto red) {
     return DispatchSaver(saver, [&](auto sv) {
@@ -301,11 +313,16 @@ int mshadow_hip_reduce_keep_highdim_f32(float *dst, const float *src, int sstrid
                                                             RawPlan2D<const float> >),         \
                      dim3(c), dim3(T), 0, s, d, sp, static_cast<uint32_t>(n),                  \
                      static_cast<uint32_t>(c), static_cast<uint32_t>(y),                       \
-                     static_cast<uint32_t>(x), scale)
+                     static_cast<uint32_t>(x), div_x, scale)
 #define HIGHDIM_LAUNCH(SEGS)                                                                   \
-  if (large) HIGHDIM_LAUNCH_T(mshadow::hip::kRedBlockLarge, SEGS);                             \
+  if (large)                                                                                   \
+    hipLaunchKernelGGL((mshadow::hip::ReduceKeepHighDimDmaKernel<S, R, SEGS>), dim3(c),        \
+                       dim3(mshadow::hip::kDmaThreads), 0, s, dst, src,                        \
+                       static_cast<uint32_t>(sstride), static_cast<uint32_t>(n),               \
+                       static_cast<uint32_t>(c), static_cast<uint32_t>(y),                     \
+                       static_cast<uint32_t>(x), div_x, scale);                                \
   else HIGHDIM_LAUNCH_T(mshadow::hip::kRedBlockSmall, SEGS)
-      const bool large = static_cast<long long>(n) * y * x >= (1 << 18);
+      const bool large = static_cast<long long>(n) * y * x >= kDmaMinPerKept;
       if (n > 16) { HIGHDIM_LAUNCH(64); }
       else if (n > 4) { HIGHDIM_LAUNCH(16); }
       else if (n > 1) { HIGHDIM_LAUNCH(4); }

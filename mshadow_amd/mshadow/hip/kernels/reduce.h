@@ -26,6 +26,7 @@
 #ifndef MSHADOW_HIP_KERNELS_REDUCE_H_
 #define MSHADOW_HIP_KERNELS_REDUCE_H_
 
+#include "../../core/fastdiv.h"
 #include "../../expr/plan.h"
 #include "./common.h"
 
@@ -56,14 +57,17 @@ __device__ __forceinline__ DType WaveBroadcast(DType v, int lane) {
   return r;
 }
 
-/*! \brief fold vals[begin .. count) into res, in order. The operands of the next 32
- *  steps are fetched from LDS (eight 128-bit reads) while the current 32 dependent
- *  reductions execute, so a step costs one VALU issue plus a quarter of an LDS read. */
-template <typename Reducer, typename DType, int PACKS>
+/*! \brief fold this lane's elements [begin, count) into res, in order. Element r lives at
+ *  vals[(r / 4) * GSTRIDE + r % 4]: groups of four consecutive elements are contiguous
+ *  (one 128-bit LDS read), GSTRIDE floats apart (4 = fully contiguous). The operands of
+ *  the next 32 steps are fetched from LDS (eight 128-bit reads) while the current 32
+ *  dependent reductions execute, so a step costs one VALU issue plus a quarter of an LDS
+ *  read. */
+template <typename Reducer, typename DType, int PACKS, int GSTRIDE>
 __device__ __forceinline__ void ChainLoad(expr::Pack<DType, 4> (&dst)[PACKS], const DType *src) {
 #pragma unroll
   for (int i = 0; i < PACKS; ++i) {
-    dst[i] = *reinterpret_cast<const expr::Pack<DType, 4> *>(src + 4 * i);
+    dst[i] = *reinterpret_cast<const expr::Pack<DType, 4> *>(src + GSTRIDE * i);
   }
 }
 template <typename Reducer, typename DType, int PACKS>
@@ -77,27 +81,30 @@ __device__ __forceinline__ void ChainApply(DType &res, const expr::Pack<DType, 4
   }
 }
 
-template <typename Reducer, typename DType>
+template <typename Reducer, int GSTRIDE = 4, typename DType>
 __device__ __forceinline__ void ChainFold(DType &res, const DType *vals, int begin, int count) {
   typedef expr::Pack<DType, 4> P4;
   const int kBlk = 32;
   const int kPacks = kBlk / 4;
+  const int kBlkStride = kPacks * GSTRIDE;  // floats between consecutive blocks of 32
+#define MSHADOW_CHAIN_AT(r) vals[((r) >> 2) * GSTRIDE + ((r) & 3)]
   int r = begin;
-  for (; r < count && (r & (kBlk - 1)); ++r) Reducer::Reduce(res, vals[r]);
+  for (; r < count && (r & (kBlk - 1)); ++r) Reducer::Reduce(res, MSHADOW_CHAIN_AT(r));
   if (r + kBlk <= count) {
     /* two register sets alternate: while one is being folded the other is in flight */
+    const DType *blk = vals + (r >> 2) * GSTRIDE;
     P4 a[kPacks], b[kPacks];
-    ChainLoad<Reducer, DType, kPacks>(a, vals + r);
-    for (; r + 3 * kBlk <= count; r += 2 * kBlk) {
-      ChainLoad<Reducer, DType, kPacks>(b, vals + r + kBlk);
+    ChainLoad<Reducer, DType, kPacks, GSTRIDE>(a, blk);
+    for (; r + 3 * kBlk <= count; r += 2 * kBlk, blk += 2 * kBlkStride) {
+      ChainLoad<Reducer, DType, kPacks, GSTRIDE>(b, blk + kBlkStride);
       __builtin_amdgcn_sched_barrier(0);
       ChainApply<Reducer, DType, kPacks>(res, a);
-      ChainLoad<Reducer, DType, kPacks>(a, vals + r + 2 * kBlk);
+      ChainLoad<Reducer, DType, kPacks, GSTRIDE>(a, blk + 2 * kBlkStride);
       __builtin_amdgcn_sched_barrier(0);
       ChainApply<Reducer, DType, kPacks>(res, b);
     }
     if (r + 2 * kBlk <= count) {
-      ChainLoad<Reducer, DType, kPacks>(b, vals + r + kBlk);
+      ChainLoad<Reducer, DType, kPacks, GSTRIDE>(b, blk + kBlkStride);
       __builtin_amdgcn_sched_barrier(0);
       ChainApply<Reducer, DType, kPacks>(res, a);
       ChainApply<Reducer, DType, kPacks>(res, b);
@@ -107,7 +114,8 @@ __device__ __forceinline__ void ChainFold(DType &res, const DType *vals, int beg
       r += kBlk;
     }
   }
-  for (; r < count; ++r) Reducer::Reduce(res, vals[r]);
+  for (; r < count; ++r) Reducer::Reduce(res, MSHADOW_CHAIN_AT(r));
+#undef MSHADOW_CHAIN_AT
 }
 
 /*! \brief which strip of kLowestCols columns a workgroup takes. Workgroups are dealt to
@@ -188,7 +196,7 @@ template <typename Saver, typename Reducer, typename DType, int THREADS, int SEG
           typename SPlan>
 __global__ void __launch_bounds__(THREADS)
     ReduceKeepHighDimKernel(DPlan dplan, SPlan splan, uint32_t n_out, uint32_t n_keep,
-                            uint32_t n_y, uint32_t n_x, DType scale) {
+                            uint32_t n_y, uint32_t n_x, FastDivU32 div_x, DType scale) {
   const int TL = THREADS * kRedDepth / SEGS;  // elements of each segment per stage
   const int LD = TL + 4;
   __shared__ MSHADOW_ALIGNED(16) DType tile[2][SEGS * LD];
@@ -213,7 +221,7 @@ __global__ void __launch_bounds__(THREADS)
       /* never predicated (see KeepLowest): clamp to the last valid element */         \
       n_ = n_ < n_out ? n_ : n_out - 1;                                                \
       e_ = e_ < seg_len ? e_ : seg_len - 1;                                            \
-      const uint32_t y_ = e_ / n_x;                                                    \
+      const uint32_t y_ = div_x.Div(e_);                                               \
       REGS[k] = splan.Eval((n_ * n_keep + c) * n_y + y_, e_ - y_ * n_x);               \
     }                                                                                  \
   }

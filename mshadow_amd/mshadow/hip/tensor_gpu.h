@@ -406,6 +406,38 @@ inline void MapExp(TRValue<R, gpu, dim, DType> *dst, const expr::Exp<E, DType, e
 #endif
 }
 
+namespace gpu_detail {
+/*! \brief reductions whose source is a float tensor in memory and whose reducer / saver are
+ *  the built-in ones go to the fixed-function entry points of the library, which fetch
+ *  the tensor straight into LDS; every other reduction (an expression source, another
+ *  element type, a caller-defined reducer) is compiled from the generic kernel templates */
+template <typename Saver, typename Reducer, typename R, typename E, typename DType>
+struct ReduceRoute {
+  static const bool kFixed = false;
+  template <typename... Args> static void Lowest(Args...) {}
+  template <typename... Args> static void HighDim(Args...) {}
+};
+template <typename Saver, typename Reducer, int dim>
+struct ReduceRoute<Saver, Reducer, Tensor<gpu, 1, float>, Tensor<gpu, dim, float>, float> {
+  static const bool kFixed = SaverCode<Saver>::value >= 0 && ReducerCode<Reducer>::value >= 0;
+  static void Lowest(const Tensor<gpu, 1, float> &dst, const Tensor<gpu, dim, float> &src,
+                     uint32_t rows, uint32_t cols, float scale) {
+    MSHADOW_HIP_CALL(mshadow_hip_reduce_keep_lowest_f32(
+        dst.dptr_, src.dptr_, static_cast<int>(src.stride_), static_cast<int>(rows),
+        static_cast<int>(cols), ReducerCode<Reducer>::value, SaverCode<Saver>::value, scale,
+        Stream<gpu>::GetStream(dst.stream_)));
+  }
+  static void HighDim(const Tensor<gpu, 1, float> &dst, const Tensor<gpu, dim, float> &src,
+                      uint32_t n_out, uint32_t n_keep, uint32_t n_y, uint32_t n_x, float scale) {
+    MSHADOW_HIP_CALL(mshadow_hip_reduce_keep_highdim_f32(
+        dst.dptr_, src.dptr_, static_cast<int>(src.stride_), static_cast<int>(n_out),
+        static_cast<int>(n_keep), static_cast<int>(n_y), static_cast<int>(n_x),
+        ReducerCode<Reducer>::value, SaverCode<Saver>::value, scale,
+        Stream<gpu>::GetStream(dst.stream_)));
+  }
+};
+}  // namespace gpu_detail
+
 template <typename Saver, typename Reducer, typename R, typename DType, typename E, int etype>
 inline void MapReduceKeepLowest(TRValue<R, gpu, 1, DType> *dst,
                                 const expr::Exp<E, DType, etype> &exp, DType scale) {
@@ -415,6 +447,11 @@ inline void MapReduceKeepLowest(TRValue<R, gpu, 1, DType> *dst,
   Shape<1> dshape = expr::ShapeCheck<1, R>::Check(dst->self());
   CHECK_EQ(eshape[1], dshape[0]) << "MapReduceKeepLowest::reduction dimension do not match";
   CHECK_NE(eshape[0], 0U) << "can not reduce over empty tensor";
+  typedef gpu_detail::ReduceRoute<Saver, Reducer, R, E, DType> Route;
+  if (Route::kFixed) {
+    Route::Lowest(dst->self(), exp.self(), eshape[0], eshape[1], scale);
+    return;
+  }
 #if defined(__HIPCC__)
   typedef expr::Plan<R, DType> DPlan;
   typedef expr::Plan<E, DType> SPlan;
@@ -449,6 +486,12 @@ inline void MapReduceKeepHighDim(TRValue<R, gpu, 1, DType> *dst,
   EShape eshape = expr::ShapeCheck<expr::ExpInfo<E>::kDim, E>::Check(exp.self());
   Shape<1> dshape = expr::ShapeCheck<1, R>::Check(dst->self());
   CHECK_EQ(eshape[dimkeep], dshape[0]) << "MapReduceKeepHighDim::reduction dimension do not match";
+  typedef gpu_detail::ReduceRoute<Saver, Reducer, R, E, DType> Route;
+  if (Route::kFixed) {
+    Route::HighDim(dst->self(), exp.self(), eshape.ProdShape(0, dimkeep), eshape[dimkeep],
+                   eshape.ProdShape(dimkeep + 1, EShape::kSubdim), eshape[EShape::kSubdim], scale);
+    return;
+  }
 #if defined(__HIPCC__)
   typedef expr::Plan<R, DType> DPlan;
   typedef expr::Plan<E, DType> SPlan;
@@ -457,7 +500,9 @@ inline void MapReduceKeepHighDim(TRValue<R, gpu, 1, DType> *dst,
   uint32_t n_out = eshape.ProdShape(0, dimkeep), n_keep = eshape[dimkeep];
   uint32_t n_y = eshape.ProdShape(dimkeep + 1, EShape::kSubdim), n_x = eshape[EShape::kSubdim];
   if (n_keep == 0) return;
-  void *args[] = {&dplan, &splan, &n_out, &n_keep, &n_y, &n_x, &scale};
+  CHECK_LT(static_cast<uint64_t>(n_y) * n_x, 1ull << 31) << "MapReduceKeepHighDim: inner extent too large";
+  FastDivU32 div_x(n_x > 0 ? n_x : 1);
+  void *args[] = {&dplan, &splan, &n_out, &n_keep, &n_y, &n_x, &div_x, &scale};
   void *stream = Stream<gpu>::GetStream(expr::StreamInfo<gpu, R>::Get(dst->self()));
   /* segments staged side by side = chain lanes in use (fewer, longer pieces when the
      outer extent is small); the large workgroup when each kept index has enough work */

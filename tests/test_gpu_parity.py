@@ -143,7 +143,7 @@ def test_map_shape_mismatch_is_an_error(G, stream):
 
 # ------------------------------------------------------------------ reductions
 LOWEST_SHAPES = [((16384 // 8, 4096 // 8), 0), ((1000, 37), 3), ((1, 130), 0), ((257, 16), 0),
-                 ((255, 1), 1), ((4097, 48), 0)]
+                 ((255, 1), 1), ((4097, 48), 0), ((2500, 19), 2)]
 
 
 @pytest.mark.parametrize("shape,pad", LOWEST_SHAPES)
@@ -166,7 +166,10 @@ def test_reduce_keep_lowest(G, O, stream, shape, pad, reducer, route):
 
 
 HIGH_SHAPES = [((8, 32, 56, 56), 0), ((64, 5, 7, 9), 2), ((3, 4, 5, 6), 0), ((1, 3, 2, 4), 0),
-               ((70, 3, 1, 1), 0), ((17, 2, 33, 65), 3), ((2, 2, 70, 70), 0)]
+               ((70, 3, 1, 1), 0), ((17, 2, 33, 65), 3), ((2, 2, 70, 70), 0),
+               # long enough for the direct-to-LDS kernels, one shape per segment count
+               ((70, 3, 33, 65), 3), ((5, 2, 130, 129), 0), ((2, 2, 200, 200), 0),
+               ((1, 2, 300, 300), 1)]
 
 
 @pytest.mark.parametrize("shape,pad", HIGH_SHAPES)
