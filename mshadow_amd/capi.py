@@ -62,6 +62,7 @@ HIP_SYMBOLS = {
     "mshadow_hip_peek_last_error": ([], _i),
     "mshadow_hip_suggest_grid": ([_sz, _sz, _i, C.POINTER(C.c_uint32)], _i),
     "mshadow_hip_softmax_f32": ([_p, _i, _p, _i, _i, _i, _p], _i),
+    "mshadow_hip_softmax_rowsum_f32": ([_p, _p, _i, _i, _i, _p], _i),
     "mshadow_hip_softmax_grad_f32": ([_p, _i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_hip_reduce_keep_lowest_f32": ([_p, _p, _i, _i, _i, _i, _i, _f, _p], _i),
     "mshadow_hip_reduce_keep_highdim_f32": ([_p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p], _i),
@@ -236,6 +237,10 @@ class Library:
         rows, cols = src.rows, src.cols
         self.check(self.dll.mshadow_hip_softmax_f32(dst.ptr, dst.stride, src.ptr, src.stride, rows,
                                                     cols, stream))
+
+    def softmax_rowsum(self, sums, terms, stream=None):
+        self.check(self.dll.mshadow_hip_softmax_rowsum_f32(sums.ptr, terms.ptr, terms.stride,
+                                                           terms.rows, terms.cols, stream))
 
     def softmax_grad(self, dst, src, label, stream=None):
         self.check(self.dll.mshadow_hip_softmax_grad_f32(dst.ptr, dst.stride, src.ptr, src.stride,

@@ -200,8 +200,8 @@ int mshadow_hip_softmax_f32(float *dst, int dstride, const float *src, int sstri
   const bool vec = Aligned16(dst) && Aligned16(src) && dstride % 4 == 0 && sstride % 4 == 0 &&
                    cols % 4 == 0;
 #define SOFTMAX_LAUNCH(T, S, V) \
-  hipLaunchKernelGGL((SoftmaxRowKernel<T, S, V>), dim3(rows), dim3(T), 0, s, dst, dstride, src, \
-                     sstride, cols)
+  hipLaunchKernelGGL((SoftmaxRowKernel<T, S, V, false>), dim3(rows), dim3(T), 0, s, dst, dstride, \
+                     src, sstride, cols)
   if (vec) {
     if (cols <= 1024) SOFTMAX_LAUNCH(256, 1, 4);
     else if (cols <= 2048) SOFTMAX_LAUNCH(256, 2, 4);
@@ -222,6 +222,37 @@ int mshadow_hip_softmax_f32(float *dst, int dstride, const float *src, int sstri
   }
 #undef SOFTMAX_LAUNCH
   return AfterLaunch("softmax");
+}
+
+int mshadow_hip_softmax_rowsum_f32(float *sums, const float *terms, int tstride, int rows,
+                                   int cols, void *stream) {
+  ABI_REQUIRE(rows >= 0 && cols >= 0, "negative shape");
+  if (rows == 0) return MSHADOW_HIP_OK;
+  ABI_REQUIRE(sums != NULL && (terms != NULL || cols == 0), "NULL tensor");
+  ABI_REQUIRE(tstride >= cols, "pitch smaller than the row");
+  ABI_REQUIRE(cols <= 65536, "row longer than the register-resident softmax kernels take");
+  hipStream_t s = AsStream(stream);
+  const bool vec = Aligned16(terms) && tstride % 4 == 0 && cols % 4 == 0;
+#define ROWSUM_LAUNCH(T, S, V) \
+  hipLaunchKernelGGL((SoftmaxRowKernel<T, S, V, true>), dim3(rows), dim3(T), 0, s, sums, 0, terms, \
+                     tstride, cols)
+  if (vec) {
+    if (cols <= 1024) ROWSUM_LAUNCH(256, 1, 4);
+    else if (cols <= 2048) ROWSUM_LAUNCH(256, 2, 4);
+    else if (cols <= 4096) ROWSUM_LAUNCH(256, 4, 4);
+    else if (cols <= 8192) ROWSUM_LAUNCH(256, 8, 4);
+    else if (cols <= 16384) ROWSUM_LAUNCH(512, 8, 4);
+    else if (cols <= 32768) ROWSUM_LAUNCH(512, 16, 4);
+    else ROWSUM_LAUNCH(1024, 16, 4);
+  } else {
+    ABI_REQUIRE(cols <= 32768, "unaligned rows longer than 32768 terms are not register-resident");
+    if (cols <= 1024) ROWSUM_LAUNCH(256, 4, 1);
+    else if (cols <= 4096) ROWSUM_LAUNCH(256, 16, 1);
+    else if (cols <= 16384) ROWSUM_LAUNCH(1024, 16, 1);
+    else ROWSUM_LAUNCH(1024, 32, 1);
+  }
+#undef ROWSUM_LAUNCH
+  return AfterLaunch("softmax_rowsum");
 }
 
 int mshadow_hip_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride,

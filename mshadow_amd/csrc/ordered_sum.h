@@ -94,8 +94,9 @@ OSUM_HD float LaneQuant(const float (&t)[N], const Binade &b) {
   for (int i = 0; i < N; ++i) {
     const float scaled = t[i] * b.inv_u;  /* exact: inv_u is a power of two */
     const float q = rintf(scaled);        /* round to nearest even */
-    /* |scaled - q| == 0.5 exactly when the term sits half way; NaN also lands here */
-    tie = tie || !(fabsf(scaled - q) < 0.5f);
+    /* |scaled - q| == 0.5 exactly when the term sits half way; NaN also lands here. A
+       negative term would move the sum down, which the one-sided Fits() does not watch */
+    tie = tie || !(fabsf(scaled - q) < 0.5f) || !(scaled >= 0.0f);
     sum += q;
   }
   return tie ? kReject : sum;
@@ -108,6 +109,75 @@ OSUM_HD bool Fits(const Binade &b, float q) { return b.m + q < kLimit; }
 /*! \brief S after accepting integer contributions summing to q (Fits(b, q) holds) */
 OSUM_HD float Accept(float s, const Binade &b, float q) {
   return b.usable ? (b.m + q) * b.u : s;
+}
+
+/* ---- whole-row planning -------------------------------------------------------------
+ * A row is cut into chunks (the terms one wave holds in one register slab). Cheap
+ * approximate prefix sums say, before any exact work, which chunks the running sum
+ * traverses without leaving a binade ("clean"): those are quantised against that binade
+ * by all waves at once and enter the sum as one exact integer each. Only the chunks in
+ * which a power of two is crossed ("dirty", about one per binade of the final sum) are
+ * walked in order, and inside such a chunk the same plan is made per lane: lanes that
+ * stay in one binade enter as integers, the few next to the crossing (and lanes holding
+ * a tie) are added term by term. The plan is only a plan: every clean run is verified
+ * when it is applied (FlushRun), so a wrong guess costs time, never a bit. */
+
+/*! \brief plan codes: a biased exponent e (27 <= e < 255) means clean in that binade;
+ *  kPlanTwoBinades + e: the sum starts in binade e and may cross into e + 1 (or holds a
+ *  tie): walked with both quantisations prepared; kPlanWalk: anything else */
+const int kPlanWalk = -1;
+const int kPlanTwoBinades = 256;
+
+OSUM_HD uint32_t ExponentOf(float f) { return (BitsOf(f) >> 23) & 0xffu; }
+
+/*! \brief how far the sequential sum of n non-negative terms can sit from an accurate
+ *  sum of the same terms, relative to it: every addition rounds by at most half an ulp
+ *  of the running sum (n * 2^-25 in all, and rows with many terms below half an ulp come
+ *  close to it); doubled for the approximate sums themselves */
+OSUM_HD float PlanMargin(int n) {
+  const float m = static_cast<float>(n) * 5.9604644775390625e-08f;  // n * 2^-24
+  return m < 1.52587890625e-05f ? 1.52587890625e-05f : (m > 0.25f ? 0.25f : m);
+}
+
+/*! \brief binade with biased exponent e (27 <= e < 255); m is not set */
+OSUM_HD Binade BinadeOfExponent(uint32_t e) {
+  Binade r;
+  r.usable = true;
+  r.u = FloatOf((e - 23u) << 23);
+  r.inv_u = FloatOf((277u - e) << 23);
+  r.m = 0.0f;
+  return r;
+}
+
+/*! \brief plan for a piece (a chunk, or one lane's terms) whose approximate prefix sums
+ *  before / after are st <= en: the binade it stays in, or kPlanWalk */
+OSUM_HD int PlanPiece(float st, float en, float margin) {
+  const float lo = st * (1.0f - margin);
+  const float hi = en * (1.0f + margin);
+  /* 2^-98: keeps the exponent of lo at 28 or more; comparisons are false for NaN */
+  const bool usable = lo >= 3.1554436e-30f && hi < 1.0e38f;
+  const int elo = static_cast<int>(ExponentOf(lo));
+  const int ehi = static_cast<int>(ExponentOf(hi));
+  if (!usable) return kPlanWalk;
+  if (elo == ehi) return elo;
+  return (ehi == elo + 1) ? kPlanTwoBinades + elo : kPlanWalk;
+}
+/*! \brief the same for one lane's few terms, where only "stays in a binade" is of use */
+OSUM_HD int PlanLane(float st, float en, float margin) {
+  const int c = PlanPiece(st, en, margin);
+  return c < kPlanTwoBinades ? c : kPlanWalk;
+}
+
+/*! \brief apply a run of clean pieces - integer contributions totalling `run`, quantised
+ *  against the binade with biased exponent e_run - to s. Sets *fail (and returns s
+ *  unchanged) unless s really is in that binade and stays in it. */
+OSUM_HD float FlushRun(float s, int e_run, uint32_t run, bool *fail) {
+  const Binade b = BinadeOfExponent(static_cast<uint32_t>(e_run));
+  const float m = s * b.inv_u;  /* s in the binade <=> 2^23 <= m < 2^24, and m is an integer */
+  const float r = m + static_cast<float>(run);
+  const bool ok = m >= 8388608.0f && r < kLimit && run < 16777216u;
+  if (!ok) *fail = true;
+  return ok ? r * b.u : s;
 }
 
 /*! \brief the real thing: N float additions in order */

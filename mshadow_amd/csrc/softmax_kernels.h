@@ -6,8 +6,10 @@
  * kernel, mshadow/cuda/tensor_gpu-inl.cuh:330-393, moves 5). Steps per row:
  *   1. 128-bit loads, row maximum by DPP wave reduction + one LDS exchange;
  *   2. p = exp(x - max) in registers (hardware exp2 with a compensated argument);
- *   3. the row sum in the CPU path's left-to-right order (ordered_sum.h), so that the
- *      sum is, bit for bit, what mshadow/tensor_cpu-inl.h:277-281 computes from the same p;
+ *   3. the row sum in the CPU path's left-to-right order (ordered_sum.h: planned from
+ *      approximate prefix sums, exact integer adds inside a binade, a short ordered
+ *      walk over the chunks where a power of two is crossed), so that the sum is, bit
+ *      for bit, what mshadow/tensor_cpu-inl.h:277-281 computes from the same p;
  *   4. p / sum (reciprocal and one correction step), 128-bit stores.
  * dst may alias src (every element is read before the row is written).
  * SoftmaxLongRowKernel covers rows too long for registers with the same arithmetic,
@@ -105,6 +107,465 @@ __device__ inline float BlockOrderedAdd(float s, const float (&t)[N],
   }
 }
 
+/* ---- planned row sum (registers hold the whole row) ---------------------------------
+ * Thread layout: wave w owns a contiguous W-th of the row, slab j of it is the chunk
+ * k = w * SLABS + j (64 * N consecutive terms, lane-major). See ordered_sum.h for the
+ * plan; the steps here are
+ *   A  every wave: approximate sum of each of its chunks -> LDS            (barrier)
+ *   B  every wave (redundantly): prefix over all chunks, plan per chunk
+ *   C  every wave: quantise its clean chunks, integer totals -> LDS; for its dirty
+ *      chunks a plan per lane, parked in an LDS slot with the chunk's terms  (barrier)
+ *   D  waves that own dirty chunks, in order: apply the clean run in front of each
+ *      dirty chunk, walk the chunk (runs of clean lanes as integers, the other lanes
+ *      term by term), hand the sum on through LDS                         (barrier each)
+ *   E  every wave: apply the clean run behind the last dirty chunk.
+ * Lane l keeps the chunk-table entries of chunks l * CPL .. l * CPL + CPL - 1. */
+const uint32_t kDirtyQ = 0xffffffffu;
+/*! \brief dirty chunks per row with a lane-level plan parked in LDS (a row of softmax
+ *  terms has about a dozen); further ones are resolved by wave scans */
+const int kPlanSlots = 24;
+
+/* hook for a profiling build: a translation unit may define this to record a timestamp
+   at the boundaries of the steps; it is empty in the library */
+#ifndef MSHADOW_ROWSUM_STAMP
+#define MSHADOW_ROWSUM_STAMP(step)
+#endif
+#ifndef MSHADOW_ROWSUM_NOTE
+#define MSHADOW_ROWSUM_NOTE(slot, value)
+#endif
+
+/*! \brief lane-level plan of one dirty chunk, parked in LDS between steps C and D, with
+ *  the chunk's terms (so that the walk needs nothing from the register-resident row).
+ *  General chunk: a = integer total of the clean lanes in front of the lane, b = its plan
+ *  code. Two-binade chunk: a / b = inclusive integer prefix of the lanes quantised against
+ *  the lower / upper binade (lanes holding a tie count as 0), c = tie flags. */
+template <int N>
+struct LanePlanSlot {
+  float t[kWave][N];
+  uint32_t a[kWave];
+  uint32_t b[kWave];
+  uint32_t c[kWave];
+  uint32_t total;  //!< general chunks: integer total of the clean lanes
+  int kind;        //!< plan code of the chunk (kPlanWalk or kPlanTwoBinades + e)
+};
+
+template <int W, int SLABS, int N>
+struct RowSumLds {
+  /* small workgroups share a CU with several others: fewer slots each */
+  static const int kWanted = W <= 4 ? kPlanSlots * 2 / 3 : kPlanSlots;
+  static const int kSlots = (W * SLABS < kWanted) ? W * SLABS : kWanted;
+  float approx[W * SLABS];
+  uint32_t q[W * SLABS];
+  float s;       //!< running sum handed from wave to wave
+  uint32_t ex;   //!< integer prefix (over clean chunks) already applied to s
+  int fail;      //!< a verification failed: redo the row the slow way
+  uint32_t nslots;  //!< plan slots handed out
+  float wmax[W];
+  /*! \brief per wave and slab: the plan slot of the chunk, or -1 */
+  signed char slot_of[W][SLABS];
+  LanePlanSlot<N> plan[kSlots];
+};
+
+/*! \brief plan code of a piece that stays in one binade */
+__device__ __forceinline__ bool IsClean(int code) {
+  return code >= 0 && code < ordered_sum::kPlanTwoBinades;
+}
+
+/*! \brief entry k of a table spread over lanes (CPL entries per lane); k is uniform */
+template <int CPL>
+__device__ __forceinline__ uint32_t TableAt(const uint32_t (&a)[CPL], int k) {
+  /* every slot is read from the lane first and the choice made among the scalars: a
+     choice among the per-lane registers would be turned into an indexed private array */
+  uint32_t v = mshadow::hip::ReadLaneU32(a[0], k / CPL);
+#pragma unroll
+  for (int c = 1; c < CPL; ++c) {
+    const uint32_t o = mshadow::hip::ReadLaneU32(a[c], k / CPL);
+    v = (k % CPL == c) ? o : v;
+  }
+  return v;
+}
+
+/*! \brief slab j of the register-resident row (j uniform, not a compile-time constant):
+ *  a binary tree of uniform branches, log2(SLABS) deep */
+template <int LO, int HI, int SLABS, int N>
+struct SlabPicker {
+  static __device__ __forceinline__ void Pick(float (&t)[N], const float (&v)[SLABS][N], int j) {
+    const int MID = (LO + HI) / 2;
+    if (j < MID) {
+      SlabPicker<LO, MID, SLABS, N>::Pick(t, v, j);
+    } else {
+      SlabPicker<MID, HI, SLABS, N>::Pick(t, v, j);
+    }
+  }
+};
+template <int LO, int SLABS, int N>
+struct SlabPicker<LO, LO + 1, SLABS, N> {
+  static __device__ __forceinline__ void Pick(float (&t)[N], const float (&v)[SLABS][N], int) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      t[i] = v[LO][i];
+      /* keeps the tree a tree: folded into one indexed access, the whole row would move
+         from registers to scratch memory */
+      asm volatile("" : "+v"(t[i]));
+    }
+  }
+};
+template <int SLABS, int N>
+__device__ __forceinline__ void SelectSlab(float (&t)[N], const float (&v)[SLABS][N], int j) {
+  SlabPicker<0, SLABS, SLABS, N>::Pick(t, v, j);
+}
+
+/*! \brief lane-level plan of one chunk whose approximate prefix sum in front is `start`:
+ *  *code = binade the lane's terms stay in, or kPlanWalk; *ex = integer total of the
+ *  clean lanes in front of this lane; returns the integer total of all clean lanes */
+template <int N>
+__device__ __forceinline__ uint32_t PlanLanes(const float (&t)[N], float start, float margin,
+                                              uint32_t *ex, int *code) {
+  using namespace ordered_sum;
+  float a = t[0];
+#pragma unroll
+  for (int i = 1; i < N; ++i) a += t[i];
+  const float incl = WaveInclusiveScanF32(a);
+  int c = PlanLane(start + (incl - a), start + incl, margin);
+  float q = 0.0f;
+  if (c >= 0) {
+    q = LaneQuant<N>(t, BinadeOfExponent(static_cast<uint32_t>(c)));
+    if (!(q < kLimit)) c = kPlanWalk;  // a tie (or a term the plan did not expect)
+  }
+  /* neighbouring clean lanes must agree on the binade, or the later one is walked */
+  const int before = __shfl_up(c, 1);
+  if (LaneId() > 0 && c >= 0 && before >= 0 && before != c) c = kPlanWalk;
+  const uint32_t qi = c >= 0 ? static_cast<uint32_t>(q) : 0u;
+  const uint32_t inclu = mshadow::hip::WaveInclusiveScanU32(qi);
+  *ex = inclu - qi;
+  *code = c;
+  return mshadow::hip::ReadLaneU32(inclu, kWave - 1);
+}
+
+/*! \brief s plus one chunk, given its lane-level plan: runs of clean lanes are applied as
+ *  integers (and verified), every other lane adds its terms one by one */
+template <int N>
+__device__ __forceinline__ float WalkLanes(float s, const float (&t)[N], uint32_t ex, int code,
+                                           uint32_t total, bool *fail) {
+  using namespace ordered_sum;
+  unsigned long long todo = __ballot(code < 0);
+  uint32_t done = 0u;
+  while (todo != 0ull) {
+    const int l = __ffsll(static_cast<long long>(todo)) - 1;
+    todo &= todo - 1ull;
+    const uint32_t exl = mshadow::hip::ReadLaneU32(ex, l);
+    if (exl != done) {
+      const int e = static_cast<int>(mshadow::hip::ReadLaneU32(static_cast<uint32_t>(code), l - 1));
+      s = FlushRun(s, e, exl - done, fail);
+      done = exl;
+    }
+#pragma unroll
+    for (int i = 0; i < N; ++i) s = s + ReadLaneF32(t[i], l);
+  }
+  if (total != done) {
+    const int e = static_cast<int>(mshadow::hip::ReadLaneU32(static_cast<uint32_t>(code), kWave - 1));
+    s = FlushRun(s, e, total - done, fail);
+  }
+  return s;
+}
+
+/*! \brief plan of a chunk that starts in binade elo and may end in elo + 1: every lane
+ *  quantised against both; *flags bit 0 / 1 = the lane holds a tie under the lower /
+ *  upper binade (such a lane counts as 0 in that prefix) */
+template <int N>
+__device__ __forceinline__ void PlanTwoBinades(const float (&t)[N], int elo, uint32_t *incl_lo,
+                                               uint32_t *incl_hi, uint32_t *flags) {
+  using namespace ordered_sum;
+  const float qlo = LaneQuant<N>(t, BinadeOfExponent(static_cast<uint32_t>(elo)));
+  const float qhi = LaneQuant<N>(t, BinadeOfExponent(static_cast<uint32_t>(elo + 1)));
+  const bool tlo = !(qlo < kLimit), thi = !(qhi < kLimit);
+  *incl_lo = mshadow::hip::WaveInclusiveScanU32(tlo ? 0u : static_cast<uint32_t>(qlo));
+  *incl_hi = mshadow::hip::WaveInclusiveScanU32(thi ? 0u : static_cast<uint32_t>(qhi));
+  *flags = (tlo ? 1u : 0u) | (thi ? 2u : 0u);
+}
+
+/*! \brief s plus one chunk planned by PlanTwoBinades. Each round accepts, as integers,
+ *  the lanes up to the first one that holds a tie or would carry the sum out of the
+ *  current binade, adds that lane's terms one by one, and goes on - against the upper
+ *  binade once the sum has crossed. A crossing chunk takes two rounds. */
+template <int N>
+__device__ __forceinline__ float WalkTwoBinades(float s, const float (&t)[N], int elo,
+                                                uint32_t incl_lo, uint32_t incl_hi,
+                                                uint32_t flags, bool *fail) {
+  using namespace ordered_sum;
+  using mshadow::hip::ReadLaneU32;
+  const int lane = LaneId();
+  int p = 0;        // lanes before p are in s
+  bool hi = false;  // s has crossed into the upper binade
+  while (true) {
+    Binade b = BinadeOfExponent(static_cast<uint32_t>(elo + (hi ? 1 : 0)));
+    float m = s * b.inv_u;
+    if (!hi && !(m < kLimit)) {
+      hi = true;
+      b = BinadeOfExponent(static_cast<uint32_t>(elo + 1));
+      m = s * b.inv_u;
+    }
+    if (!(m >= 8388608.0f && m < kLimit)) {  // s is in neither binade: the plan was wrong
+      *fail = true;
+      return s;
+    }
+    const uint32_t incl = hi ? incl_hi : incl_lo;
+    const bool tie = (flags & (hi ? 2u : 1u)) != 0u;
+    const uint32_t base = p > 0 ? ReadLaneU32(incl, p - 1) : 0u;
+    const uint32_t room = 16777216u - static_cast<uint32_t>(m);  // integer steps left in the binade
+    const unsigned long long events = __ballot(lane >= p && (tie || incl - base >= room));
+    if (events == 0ull) {
+      return (m + static_cast<float>(ReadLaneU32(incl, kWave - 1) - base)) * b.u;
+    }
+    const int f = __ffsll(static_cast<long long>(events)) - 1;
+    const uint32_t upto = f > 0 ? ReadLaneU32(incl, f - 1) : 0u;
+    s = (m + static_cast<float>(upto - base)) * b.u;
+#pragma unroll
+    for (int i = 0; i < N; ++i) s = s + ReadLaneF32(t[i], f);
+    p = f + 1;
+    if (p == kWave) return s;
+  }
+}
+
+template <int THREADS, int SLABS, int N>
+__device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
+                                      RowSumLds<THREADS / kWave, SLABS, N> *lds) {
+  using namespace ordered_sum;
+  using mshadow::hip::ReadLaneU32;
+  using mshadow::hip::WaveInclusiveScanU32;
+  typedef RowSumLds<THREADS / kWave, SLABS, N> Lds;
+  const int W = THREADS / kWave;
+  const int NCH = W * SLABS;
+  const int CPL = (NCH + kWave - 1) / kWave;
+  static_assert(NCH % CPL == 0 && SLABS % CPL == 0, "chunk table does not tile the lanes");
+  static_assert(SLABS <= 32, "the per-wave dirty mask has 32 bits");
+  const int wave = __builtin_amdgcn_readfirstlane(WaveId());
+  const int lane = LaneId();
+  const float margin = PlanMargin(cols);
+
+  /* A: approximate chunk sums */
+  MSHADOW_ROWSUM_STAMP(0)
+  if (threadIdx.x == 0) {
+    lds->s = 0.0f;
+    lds->ex = 0u;
+    lds->fail = 0;
+    lds->nslots = 0u;
+  }
+#pragma unroll
+  for (int j = 0; j < SLABS; ++j) {
+    float a = v[j][0];
+#pragma unroll
+    for (int i = 1; i < N; ++i) a += v[j][i];
+    a = ReadLaneF32(WaveInclusiveScanF32(a), kWave - 1);
+    if (lane == 0) lds->approx[wave * SLABS + j] = a;
+  }
+  __syncthreads();
+  MSHADOW_ROWSUM_STAMP(1)
+
+  /* B: plan per chunk, identical in every wave */
+  uint32_t code[CPL];   // int codes kept as raw bits for TableAt
+  float start[CPL];     // approximate prefix sum in front of each chunk
+  float approx_total;
+  {
+    float pre[CPL + 1];
+    pre[0] = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+      const int k = lane * CPL + c;
+      pre[c + 1] = pre[c] + (k < NCH ? lds->approx[k] : 0.0f);
+    }
+    const float incl = WaveInclusiveScanF32(pre[CPL]);
+    const float excl = incl - pre[CPL];
+    approx_total = ReadLaneF32(incl, kWave - 1);
+    int raw[CPL];
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+      start[c] = excl + pre[c];
+      raw[c] = PlanPiece(start[c], excl + pre[c + 1], margin);
+    }
+    /* neighbouring clean chunks must agree on the binade, or the later one is walked:
+       every run of clean chunks then has one scale */
+    const int before = __shfl_up(raw[CPL - 1], 1);
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+      const int prev = (c == 0) ? ((lane == 0) ? kPlanWalk : before) : raw[c - 1];
+      const bool clash = IsClean(raw[c]) && IsClean(prev) && prev != raw[c];
+      code[c] = static_cast<uint32_t>(clash ? kPlanTwoBinades + (prev < raw[c] ? prev : raw[c]) : raw[c]);
+    }
+  }
+  /* a NaN among the terms makes the sum NaN whatever the order */
+  if (approx_total != approx_total) return approx_total;
+
+  /* C: integer totals of this wave's clean chunks ... */
+  MSHADOW_ROWSUM_STAMP(2)
+  uint32_t dirty_mask = 0u;  // this wave's slabs that have to be walked
+  uint32_t tie_mask = 0u;    // of those, planned clean but found to hold a tie
+#pragma unroll
+  for (int j = 0; j < SLABS; ++j) {
+    const int k = wave * SLABS + j;
+    const int ck = static_cast<int>(ReadLaneU32(code[j % CPL], k / CPL));
+    uint32_t total = kDirtyQ;
+    if (IsClean(ck)) {
+      const Binade b = BinadeOfExponent(static_cast<uint32_t>(ck));
+      const float q = ReadLaneF32(WaveInclusiveScanF32(LaneQuant<N>(v[j], b)), kWave - 1);
+      if (q < kLimit) {
+        total = static_cast<uint32_t>(q);
+      } else {
+        tie_mask |= 1u << j;  // a tie somewhere in the chunk pushed q past 2^24
+      }
+    }
+    if (total == kDirtyQ) dirty_mask |= 1u << j;
+    if (lane == 0) {
+      lds->q[k] = total;
+      lds->slot_of[wave][j] = -1;
+    }
+  }
+  /* ... and lane plans of its dirty ones, parked in LDS slots */
+  for (uint32_t todo = dirty_mask; todo != 0u; todo &= todo - 1u) {
+    const int j = __ffs(static_cast<int>(todo)) - 1;
+    const int k = wave * SLABS + j;
+    uint32_t slot = 0u;
+    if (lane == 0) slot = atomicAdd(&lds->nslots, 1u);
+    slot = __builtin_amdgcn_readfirstlane(slot);
+    if (slot >= static_cast<uint32_t>(Lds::kSlots)) break;  // the rest is resolved by wave scans
+    int ck = static_cast<int>(TableAt<CPL>(code, k));
+    if ((tie_mask >> j) & 1u) ck = kPlanTwoBinades + ck;
+    float t[N];
+    SelectSlab<SLABS, N>(t, v, j);
+    uint32_t pa, pb, pc = 0u, tot = 0u;
+    if (ck >= kPlanTwoBinades) {
+      PlanTwoBinades<N>(t, ck - kPlanTwoBinades, &pa, &pb, &pc);
+    } else {
+      float st = start[0];
+#pragma unroll
+      for (int c = 1; c < CPL; ++c) st = (k % CPL == c) ? start[c] : st;
+      int code_l;
+      tot = PlanLanes<N>(t, ReadLaneF32(st, k / CPL), margin, &pa, &code_l);
+      pb = static_cast<uint32_t>(code_l);
+    }
+    LanePlanSlot<N> *ps = &lds->plan[slot];
+#pragma unroll
+    for (int i = 0; i < N; ++i) ps->t[lane][i] = t[i];
+    ps->a[lane] = pa;
+    ps->b[lane] = pb;
+    ps->c[lane] = pc;
+    if (lane == 0) {
+      ps->total = tot;
+      ps->kind = ck;
+      lds->slot_of[wave][j] = static_cast<signed char>(slot);
+    }
+  }
+  __syncthreads();
+  MSHADOW_ROWSUM_STAMP(3)
+
+  /* D: tables of the walk */
+  uint32_t ex[CPL];  // integer prefix over clean chunks in front of each chunk
+  uint32_t total_ex;
+  uint32_t owners = 0u;  // waves that own at least one dirty chunk
+  const int LPW = SLABS / CPL;  // table lanes per wave
+  {
+    uint32_t pre[CPL + 1];
+    pre[0] = 0u;
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+      const int k = lane * CPL + c;
+      const uint32_t q = k < NCH ? lds->q[k] : 0u;
+      if (q == kDirtyQ && IsClean(static_cast<int>(code[c]))) code[c] = static_cast<uint32_t>(kPlanWalk);
+      const bool is_dirty = k < NCH && !IsClean(static_cast<int>(code[c]));
+      pre[c + 1] = pre[c] + (is_dirty ? 0u : q);
+      const unsigned long long mask = __ballot(is_dirty);
+#pragma unroll
+      for (int w = 0; w < W; ++w) {
+        owners |= (((mask >> (w * LPW)) & ((1ull << LPW) - 1ull)) != 0ull ? 1u : 0u) << w;
+      }
+    }
+    const uint32_t incl = WaveInclusiveScanU32(pre[CPL]);
+    const uint32_t excl = incl - pre[CPL];
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) ex[c] = excl + pre[c];
+    total_ex = ReadLaneU32(incl, kWave - 1);
+  }
+  MSHADOW_ROWSUM_STAMP(4)
+  for (int w = 0; w < W; ++w) {
+    if (((owners >> w) & 1u) == 0u) continue;  // block-uniform: every wave holds the same tables
+    if (wave == w) {
+      MSHADOW_ROWSUM_STAMP(8)
+      float s = lds->s;
+      uint32_t done = lds->ex;
+      bool fail = false;
+      for (uint32_t todo = dirty_mask; todo != 0u; todo &= todo - 1u) {
+        const int j = __ffs(static_cast<int>(todo)) - 1;
+        const int k = w * SLABS + j;
+        const int slot = lds->slot_of[w][j];
+        /* the plan is fetched first: it does not depend on s */
+        float t[N];
+        uint32_t pa = 0u, pb = 0u, pc = 0u, tot = 0u;
+        int kind = kPlanWalk;
+        if (slot >= 0) {
+          const LanePlanSlot<N> *ps = &lds->plan[slot];
+#pragma unroll
+          for (int i = 0; i < N; ++i) t[i] = ps->t[lane][i];
+          pa = ps->a[lane];
+          pb = ps->b[lane];
+          pc = ps->c[lane];
+          tot = ps->total;
+          kind = ps->kind;
+        }
+        const uint32_t exk = TableAt<CPL>(ex, k);
+        if (exk != done) {
+          s = FlushRun(s, static_cast<int>(TableAt<CPL>(code, k - 1)), exk - done, &fail);
+          done = exk;
+        }
+        if (slot < 0) {
+          SelectSlab<SLABS, N>(t, v, j);
+          s = WaveResolve<N>(s, t);
+        } else if (kind >= kPlanTwoBinades) {
+          s = WalkTwoBinades<N>(s, t, kind - kPlanTwoBinades, pa, pb, pc, &fail);
+        } else {
+          s = WalkLanes<N>(s, t, pa, static_cast<int>(pb), tot, &fail);
+        }
+      }
+      if (lane == 0) {
+        lds->s = s;
+        lds->ex = done;
+        if (fail) lds->fail = 1;
+      }
+      MSHADOW_ROWSUM_STAMP(9)
+    }
+    __syncthreads();
+  }
+
+  /* E: the clean run behind the last dirty chunk */
+  MSHADOW_ROWSUM_STAMP(5)
+  float s = lds->s;
+  bool fail = lds->fail != 0;
+  if (total_ex != lds->ex) {
+    s = FlushRun(s, static_cast<int>(TableAt<CPL>(code, NCH - 1)), total_ex - lds->ex, &fail);
+  }
+  MSHADOW_ROWSUM_STAMP(6)
+  if (!fail) return s;
+  MSHADOW_ROWSUM_STAMP(7)
+
+  /* a plan did not hold (kept so that the result cannot depend on the plan): every chunk
+     is resolved in order by wave scans, wave after wave */
+  __syncthreads();
+  if (threadIdx.x == 0) lds->s = 0.0f;
+  __syncthreads();
+  for (int w = 0; w < W; ++w) {
+    if (wave == w) {
+      float r = lds->s;
+      for (int j = 0; j < SLABS; ++j) {
+        float t[N];
+        SelectSlab<SLABS, N>(t, v, j);
+        r = WaveResolve<N>(r, t);
+      }
+      if (lane == 0) lds->s = r;
+    }
+    __syncthreads();
+  }
+  return lds->s;
+}
+
 /*! \brief e^x for x <= 0 (any float accepted): 2^(x * log2 e) with the rounding error of
  *  the product carried separately, so the result stays within about 1.5 ulp for the whole
  *  range a softmax sees. The hardware exp2 does not return subnormals, so results below
@@ -134,61 +595,69 @@ __device__ __forceinline__ float DivideBy(float p, float s, float rcp) {
 }
 
 template <int THREADS>
-__device__ inline float BlockMax(float v, OrderedSumLds<THREADS / kWave> *lds) {
+__device__ inline float BlockMax(float v, float *wmax) {
   const int W = THREADS / kWave;
   v = WaveMaxF32(v);
-  if (LaneId() == 0) lds->wmax[WaveId()] = v;
+  if (LaneId() == 0) wmax[WaveId()] = v;
   __syncthreads();
-  float m = lds->wmax[0];
+  float m = wmax[0];
 #pragma unroll
   for (int w = 1; w < W; ++w) {
-    const float o = lds->wmax[w];
+    const float o = wmax[w];
     m = (m < o) ? o : m;
   }
   return m;
 }
 
 /*! \brief THREADS * SLABS * VEC >= cols. VEC == 4 needs 16-byte aligned rows and
- *  cols % 4 == 0. */
-template <int THREADS, int SLABS, int VEC>
+ *  cols % 4 == 0. Wave w holds columns [w, w + 1) * SLABS * 64 * VEC, slab j of it the
+ *  next 64 * VEC, lane l of that VEC consecutive ones: each load is one contiguous
+ *  kilobyte per wave and the order of the row is wave, slab, lane, element.
+ *  TERMS_GIVEN: src already holds the (non-negative) terms and dst[row] receives their
+ *  left-to-right sum - the row-sum stage on its own. */
+template <int THREADS, int SLABS, int VEC, bool TERMS_GIVEN>
 __global__ void __launch_bounds__(THREADS, 4)  // >= 4 waves per SIMD: two 512-thread rows per CU
     SoftmaxRowKernel(float *dst, int dstride, const float *src, int sstride, int cols) {
-  __shared__ OrderedSumLds<THREADS / kWave> lds;
-  const int tid = threadIdx.x;
+  __shared__ RowSumLds<THREADS / kWave, SLABS, VEC> lds;
+  const int wave = __builtin_amdgcn_readfirstlane(WaveId());
+  const int lane = LaneId();
   const float *in = src + static_cast<size_t>(blockIdx.x) * sstride;
   float *out = dst + static_cast<size_t>(blockIdx.x) * dstride;
   const float kNegInf = -__builtin_huge_valf();
+  const float kAbsent = TERMS_GIVEN ? 0.0f : kNegInf;
 
   float v[SLABS][VEC];
   float mx = kNegInf;
 #pragma unroll
   for (int j = 0; j < SLABS; ++j) {
-    const int base = (j * THREADS + tid) * VEC;
+    const int base = ((wave * SLABS + j) * kWave + lane) * VEC;
     if (VEC == 4) {  // cols % 4 == 0: a pack is either whole or absent
-      F4 q = {kNegInf, kNegInf, kNegInf, kNegInf};
+      F4 q = {kAbsent, kAbsent, kAbsent, kAbsent};
       if (base < cols) q = StreamLoadF4(in + base);
       v[j][0] = q.x; v[j][1 % VEC] = q.y; v[j][2 % VEC] = q.z; v[j][3 % VEC] = q.w;
     } else {
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) v[j][i] = (base + i < cols) ? in[base + i] : kNegInf;
+      for (int i = 0; i < VEC; ++i) v[j][i] = (base + i < cols) ? in[base + i] : kAbsent;
     }
+    if (!TERMS_GIVEN) {
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) mx = (mx < v[j][i]) ? v[j][i] : mx;
+      for (int i = 0; i < VEC; ++i) mx = (mx < v[j][i]) ? v[j][i] : mx;
+    }
   }
-  mx = BlockMax<THREADS>(mx, &lds);
-
+  if (!TERMS_GIVEN) {
+    mx = BlockMax<THREADS>(mx, lds.wmax);
 #pragma unroll
-  for (int j = 0; j < SLABS; ++j) {
-    const int base = (j * THREADS + tid) * VEC;
+    for (int j = 0; j < SLABS; ++j) {
+      const int base = ((wave * SLABS + j) * kWave + lane) * VEC;
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) v[j][i] = (base + i < cols) ? ExpNonPositive(v[j][i] - mx) : 0.0f;
+      for (int i = 0; i < VEC; ++i) v[j][i] = (base + i < cols) ? ExpNonPositive(v[j][i] - mx) : 0.0f;
+    }
   }
 
-  float s = 0.0f;
-  int buf = 0;
-#pragma unroll
-  for (int j = 0; j < SLABS; ++j) {
-    if (j * THREADS * VEC < cols) s = BlockOrderedAdd<THREADS, VEC>(s, v[j], &lds, &buf);
+  const float s = RowOrderedSum<THREADS, SLABS, VEC>(v, cols, &lds);
+  if (TERMS_GIVEN) {
+    if (threadIdx.x == 0) dst[blockIdx.x] = s;
+    return;
   }
 
   /* s >= 1 for finite logits (the maximum contributes exp(0)); anything else (NaN or
@@ -197,7 +666,7 @@ __global__ void __launch_bounds__(THREADS, 4)  // >= 4 waves per SIMD: two 512-t
   const float rcp = 1.0f / s;
 #pragma unroll
   for (int j = 0; j < SLABS; ++j) {
-    const int base = (j * THREADS + tid) * VEC;
+    const int base = ((wave * SLABS + j) * kWave + lane) * VEC;
     float o[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) o[i] = fast_div ? DivideBy(v[j][i], s, rcp) : v[j][i] / s;
@@ -228,7 +697,7 @@ __global__ void __launch_bounds__(THREADS)
     const float e = in[x];
     mx = (mx < e) ? e : mx;
   }
-  mx = BlockMax<THREADS>(mx, &lds);
+  mx = BlockMax<THREADS>(mx, lds.wmax);
   float s = 0.0f;
   int buf = 0;
   for (int x0 = 0; x0 < cols; x0 += THREADS) {

@@ -260,6 +260,69 @@ def test_softmax_exact_cases(G, stream):
         assert -6e-5 < seq_bias < -5e-6, seq_bias
 
 
+def _serial_row_sums(O, terms):
+    """strictly left-to-right float32 sums of each row (the oracle's keep-dimension fold)"""
+    rows, cols = terms.shape
+    want = np.empty(rows, f32)
+    O.reduce_keep_highdim(want, np.ascontiguousarray(terms).reshape(1, rows, 1, cols), SUM, SAVETO, 1.0)
+    return want
+
+
+ROWSUM_COLS = [1, 3, 64, 255, 256, 1000, 1024, 1028, 2048, 3000, 4096, 5001, 8192, 12000, 16384,
+               20001, 32000, 32768, 40000, 65536]
+
+
+@pytest.mark.parametrize("cols", ROWSUM_COLS)
+def test_softmax_rowsum_is_the_serial_sum(G, O, stream, cols):
+    """the row-sum stage of Softmax, fed with terms directly, against a serial float sum:
+    bit for bit, on terms shaped like a softmax's and on ones built to hit ties, long runs
+    of zeros, many binade crossings in one chunk and sums that end next to a power of two"""
+    rng = np.random.default_rng(1000 + cols)
+    rows = []
+    for sigma in (0.1, 1.0, 3.0, 10.0, 40.0):
+        x = rng.standard_normal(cols) * sigma
+        rows.append(np.exp(x - x.max()))
+    rows.append(rng.uniform(0, 1, cols))
+    rows.append(np.full(cols, 1.0))                               # exact integers
+    rows.append(np.ldexp(rng.integers(1, 9, cols).astype(np.float64), -3))   # multiples of 1/8: ties
+    rows.append(np.ldexp(rng.integers(0, 3, cols).astype(np.float64), -24) + (np.arange(cols) == 0))
+    z = rng.uniform(0, 1, cols)
+    z[: cols // 2] = 0.0                                          # leading zeros
+    rows.append(z)
+    rows.append(np.ldexp(1.0, rng.integers(-40, 20, cols)))       # huge dynamic range
+    rows.append(np.where(np.arange(cols) % 97 == 0, 1.0, 1e-7))   # rare large terms
+    rows.append(np.zeros(cols))
+    t = np.zeros(cols)
+    t[-1] = 3.5
+    rows.append(t)
+    rows.append(np.full(cols, 2.0 ** -130))                       # subnormal terms
+    terms = np.asarray(rows, dtype=f32)
+    want = _serial_row_sums(O, terms)
+    if cols % 4 == 0 or cols <= 32768:
+        for pad in (0, 1) if cols <= 32768 else (0,):
+            sums = G.buffer((terms.shape[0],), f32)
+            G.softmax_rowsum(sums, G.to_device(terms, pad), stream)
+            assert_bits_equal(sums.download(stream), want, f"row sum cols={cols} pad={pad}")
+
+
+def test_softmax_rowsum_specials(G, O, stream):
+    cols = 5000
+    base = np.random.default_rng(7).uniform(0, 1, cols).astype(f32)
+    rows = []
+    for pos in (0, 17, 2500, cols - 1):
+        for val in (np.inf, np.nan, -0.5, 3.0e38):
+            r = base.copy()
+            r[pos] = val
+            rows.append(r)
+    terms = np.asarray(rows, dtype=f32)
+    want = _serial_row_sums(O, terms)
+    sums = G.buffer((terms.shape[0],), f32)
+    G.softmax_rowsum(sums, G.to_device(terms), stream)
+    got = sums.download(stream)
+    same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
+    assert same.all(), (got, want)
+
+
 def test_softmax_extreme_rows(G, O, stream):
     rows = [
         np.linspace(-200, 0, 5000),          # long underflowing head (leading zeros)
