@@ -60,6 +60,17 @@ def work_elements():
 
 OPS = [k for k in algorithmic_bytes() if k != "calib_copy"]
 
+# HBM bytes per launch of each operation's kernel, measured with rocprofv3 --pmc FETCH_SIZE and
+# --pmc WRITE_SIZE (two runs of `bench.py --only <all ops>,calib_copy`), each counter scaled by
+# what it reads for the calibration copy of known size (FETCH_SIZE x 1.9986, WRITE_SIZE x 0.9992);
+# the counter table is kept under profiles/. bench.py cannot run the profiler on itself, so
+# `roofline.traffic` quotes this table.
+MEASURED_HBM_BYTES = {
+    "map_fused": 335412917, "sumall_except_dim1": 211833765, "sum_rows": 268411278,
+    "softmax": 2096329166, "softmax_grad": 2096241944, "pool_max": 518109063,
+    "unpool_max": 1134310162, "im2col_f16": 513629238, "col2im_f16": 542471701,
+}
+
 
 def make_inputs(scale=1):
     """Seeded synthetic inputs of the BASELINE shapes (scale > 1 shrinks the leading
@@ -218,7 +229,7 @@ def main():
                    "arch": props.arch.decode(), "compute_units": props.compute_units},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(dom_gbs, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
-                     "traffic": None},
+                     "traffic": MEASURED_HBM_BYTES.get(dominant) if args.scale == 1 else None},
         "per_op": per_op,
         "input_generation_s": round(gen_s, 1),
     }

@@ -83,7 +83,9 @@ float orc_half2float(uint16_t h) {
       x |= sign;
     }
   } else if (e == 31) {
-    x = sign | 0x7f800000u | (m << 13);
+    /* inf, or NaN with the payload kept and the quiet bit set: what the F16C conversion
+       the reference is built with returns for a signalling NaN (mshadow/half.h:285-296) */
+    x = sign | 0x7f800000u | (m << 13) | (m ? 0x00400000u : 0u);
   } else {
     x = sign | ((e + 112u) << 23) | (m << 13);
   }
