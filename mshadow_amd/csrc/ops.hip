@@ -182,6 +182,48 @@ int Col2Im(T *img, int istride, const T *col, int cstride, const PatchGeom &g, v
   }
   return AfterLaunch("col2im");
 }
+struct UnpoolArgs {
+  float *dst; int dstride; const float *src; int sstride; const float *pooled; int pstride;
+  const float *grad; int gstride; PoolGeom g; int prow_max; unsigned blocks; size_t lds;
+  hipStream_t s;
+};
+#define UNPOOL_ARGS(a) a.dst, a.dstride, a.src, a.sstride, a.pooled, a.pstride, a.grad, a.gstride, a.g, a.prow_max
+template <int KY, int KX, int SY, int SX, bool VEC>
+void LaunchUnpoolBlock(int reducer, const UnpoolArgs &a, const mshadow::FastDivU32 &div_bw) {
+  switch (reducer) {
+    case MSHADOW_HIP_SUM:
+      hipLaunchKernelGGL((UnpoolBlockKernel<MSHADOW_HIP_SUM, KY, KX, SY, SX, VEC>), dim3(a.blocks),
+                         dim3(kPoolBlock), a.lds, a.s, UNPOOL_ARGS(a), div_bw);
+      break;
+    case MSHADOW_HIP_MAX:
+      hipLaunchKernelGGL((UnpoolBlockKernel<MSHADOW_HIP_MAX, KY, KX, SY, SX, VEC>), dim3(a.blocks),
+                         dim3(kPoolBlock), a.lds, a.s, UNPOOL_ARGS(a), div_bw);
+      break;
+    default:
+      hipLaunchKernelGGL((UnpoolBlockKernel<MSHADOW_HIP_MIN, KY, KX, SY, SX, VEC>), dim3(a.blocks),
+                         dim3(kPoolBlock), a.lds, a.s, UNPOOL_ARGS(a), div_bw);
+      break;
+  }
+}
+void LaunchUnpoolGeneric(int reducer, const UnpoolArgs &a) {
+  switch (reducer) {
+    case MSHADOW_HIP_SUM:
+      hipLaunchKernelGGL((UnpoolKernel<MSHADOW_HIP_SUM, 0, 0, 0, 0>), dim3(a.blocks), dim3(kPoolBlock),
+                         a.lds, a.s, UNPOOL_ARGS(a));
+      break;
+    case MSHADOW_HIP_MAX:
+      hipLaunchKernelGGL((UnpoolKernel<MSHADOW_HIP_MAX, 0, 0, 0, 0>), dim3(a.blocks), dim3(kPoolBlock),
+                         a.lds, a.s, UNPOOL_ARGS(a));
+      break;
+    default:
+      hipLaunchKernelGGL((UnpoolKernel<MSHADOW_HIP_MIN, 0, 0, 0, 0>), dim3(a.blocks), dim3(kPoolBlock),
+                         a.lds, a.s, UNPOOL_ARGS(a));
+      break;
+  }
+}
+#undef UNPOOL_ARGS
+
+
 }  // namespace
 
 
@@ -467,9 +509,10 @@ int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstrid
   while (band > 8 && static_cast<long long>(planes) * ((h + band - 1) / band) < 1024) {
     band = (band + 1) / 2;
   }
-  if (band >= 1) {  // equal-sized bands
+  if (band >= 1) {  // equal-sized bands, starting at multiples of the stride
     const long long nb = (h + band - 1) / band;
     band = (h + nb - 1) / nb;
+    band = (band + sy - 1) / sy * sy;
   }
   if (band >= 1 && max_prow >= 3) {
     g.band = static_cast<int>(band);
@@ -478,29 +521,25 @@ int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstrid
     const size_t lds = static_cast<size_t>(prow_max) * row_bytes + 32;
     const long long blocks = static_cast<long long>(planes) * g.bands;
     ABI_REQUIRE(blocks < (1ll << 31), "too many workgroups");
-#define UNPOOL_TILED(KY, KX, SY, SX)                                                                   \
-  switch (reducer) {                                                                           \
-    case MSHADOW_HIP_SUM:                                                                      \
-      hipLaunchKernelGGL((UnpoolKernel<MSHADOW_HIP_SUM, KY, KX, SY, SX>),                              \
-                         dim3(static_cast<unsigned>(blocks)), dim3(kPoolBlock), lds, s, dst,   \
-                         dstride, src, sstride, pooled, pstride, grad, gstride, g, prow_max);  \
-      break;                                                                                   \
-    case MSHADOW_HIP_MAX:                                                                      \
-      hipLaunchKernelGGL((UnpoolKernel<MSHADOW_HIP_MAX, KY, KX, SY, SX>),                              \
-                         dim3(static_cast<unsigned>(blocks)), dim3(kPoolBlock), lds, s, dst,   \
-                         dstride, src, sstride, pooled, pstride, grad, gstride, g, prow_max);  \
-      break;                                                                                   \
-    default:                                                                                   \
-      hipLaunchKernelGGL((UnpoolKernel<MSHADOW_HIP_MIN, KY, KX, SY, SX>),                              \
-                         dim3(static_cast<unsigned>(blocks)), dim3(kPoolBlock), lds, s, dst,   \
-                         dstride, src, sstride, pooled, pstride, grad, gstride, g, prow_max);  \
-      break;                                                                                   \
-  }
-    if (ky == 3 && kx == 3 && sy == 2 && sx == 2) { UNPOOL_TILED(3, 3, 2, 2) }
-    else if (ky == 2 && kx == 2 && sy == 2 && sx == 2) { UNPOOL_TILED(2, 2, 2, 2) }
-    else if (ky == 3 && kx == 3 && sy == 1 && sx == 1) { UNPOOL_TILED(3, 3, 1, 1) }
-    else { UNPOOL_TILED(0, 0, 0, 0) }
-#undef UNPOOL_TILED
+    ABI_REQUIRE(lds <= 160 * 1024, "pooled rows too long for the LDS-tiled kernel");
+    const mshadow::FastDivU32 div_bw(static_cast<uint32_t>((w + sx - 1) / sx));
+    /* whole, aligned blocks of sx pixels per row: a block row is one memory access */
+    const bool vec = (sx == 2 || sx == 4) && w % sx == 0 && dstride % sx == 0 && sstride % sx == 0 &&
+                     reinterpret_cast<uintptr_t>(dst) % (sx * 4) == 0 &&
+                     reinterpret_cast<uintptr_t>(src) % (sx * 4) == 0;
+    const UnpoolArgs ua = {dst, dstride, src, sstride, pooled, pstride, grad, gstride, g, prow_max,
+                           static_cast<unsigned>(blocks), lds, s};
+    if (ky == 3 && kx == 3 && sy == 2 && sx == 2) {
+      if (vec) LaunchUnpoolBlock<3, 3, 2, 2, true>(reducer, ua, div_bw);
+      else LaunchUnpoolBlock<3, 3, 2, 2, false>(reducer, ua, div_bw);
+    } else if (ky == 2 && kx == 2 && sy == 2 && sx == 2) {
+      if (vec) LaunchUnpoolBlock<2, 2, 2, 2, true>(reducer, ua, div_bw);
+      else LaunchUnpoolBlock<2, 2, 2, 2, false>(reducer, ua, div_bw);
+    } else if (ky == 3 && kx == 3 && sy == 1 && sx == 1) {
+      LaunchUnpoolBlock<3, 3, 1, 1, false>(reducer, ua, div_bw);
+    } else {
+      LaunchUnpoolGeneric(reducer, ua);
+    }
   } else {
     const unsigned total = static_cast<unsigned>(planes) * h * w;
     unsigned grid = 0;

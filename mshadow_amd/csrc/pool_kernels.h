@@ -23,6 +23,8 @@
 
 #include <cfloat>
 
+#include <mshadow/core/fastdiv.h>
+
 #include "stream_access.h"
 
 namespace mshadow_hipk {
@@ -255,6 +257,115 @@ __global__ void __launch_bounds__(kPoolBlock)
             }
           }
           StreamStore(out + static_cast<size_t>(yr) * dstride + x, val);
+        }
+      }
+    }
+  }
+}
+
+/*! \brief unpool for a window and stride fixed at compile time, one thread per SY x SX
+ *  block of source pixels aligned to the stride. The windows that can cover a pixel of the
+ *  block at (a, b) are (a - jy, b - jx), jy < ceil(KY / SY), jx < ceil(KX / SX): the
+ *  pooled value and the gradient of each are read from LDS once per block (not once per
+ *  pixel), and which of them cover which pixel of the block - jy * SY + dy < KY - is known
+ *  to the compiler, so only existing terms are evaluated, in the reference's py, px order.
+ *  VEC: rows are made of whole blocks and are aligned, a block row moves as one access.
+ *  Same grid and LDS layout as UnpoolKernel; bands start at multiples of SY. */
+template <int REDUCER, int KY, int KX, int SY, int SX, bool VEC>
+__global__ void __launch_bounds__(kPoolBlock)
+    UnpoolBlockKernel(float *dst, int dstride, const float *src, int sstride, const float *pooled,
+                      int pstride, const float *grad, int gstride, PoolGeom g, int prow_max,
+                      mshadow::FastDivU32 div_bw) {
+  extern __shared__ float smem[];
+  typedef PoolOp<REDUCER> Op;
+  const int JY = (KY + SY - 1) / SY, JX = (KX + SX - 1) / SX;
+  const int plane = blockIdx.x / g.bands;
+  const int band = blockIdx.x - plane * g.bands;
+  const int y0 = band * g.band;
+  const int ny = min(g.band, g.h - y0);
+  const int ylast = y0 + ny - 1;
+  const int p0 = y0 < KY ? 0 : (y0 - KY + SY) / SY;
+  const int p1 = min((ylast + SY) / SY, g.ph);
+  const int np = max(p1 - p0, 0);
+  const float *pin = pooled + (static_cast<size_t>(plane) * g.ph + p0) * pstride;
+  const float *gin = grad + (static_cast<size_t>(plane) * g.ph + p0) * gstride;
+  float *sp = smem + LdsPhase(pin);
+  float *sg = smem + prow_max * g.lds_pitch + 4 + LdsPhase(gin);
+  StageRows(sp, g.lds_pitch, pin, pstride, np, g.pw);
+  StageRows(sg, g.lds_pitch, gin, gstride, np, g.pw);
+  const float *in = src + (static_cast<size_t>(plane) * g.h + y0) * sstride;
+  float *out = dst + (static_cast<size_t>(plane) * g.h + y0) * dstride;
+  const int bw = (g.w + SX - 1) / SX;
+  const int a0 = y0 / SY;
+  const unsigned nblk = static_cast<unsigned>((ny + SY - 1) / SY) * bw;
+  const int kAhead = 2;  // blocks per thread whose loads are issued before any is used
+  __syncthreads();
+  for (unsigned t0 = threadIdx.x; t0 < nblk; t0 += kPoolBlock * kAhead) {
+    float vs[kAhead][SY][SX];
+    int ar[kAhead], b[kAhead];
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      /* past the end: re-read the last block (unpredicated loads), nothing is stored */
+      const unsigned t = min(t0 + u * kPoolBlock, nblk - 1);
+      ar[u] = static_cast<int>(div_bw.Div(t));
+      b[u] = static_cast<int>(t) - ar[u] * bw;
+#pragma unroll
+      for (int dy = 0; dy < SY; ++dy) {
+        const int yr = min(ar[u] * SY + dy, ny - 1);
+        const float *row = in + static_cast<size_t>(yr) * sstride + b[u] * SX;
+        if (VEC) {
+          StreamLoadN<SX>(vs[u][dy], row);
+        } else {
+#pragma unroll
+          for (int dx = 0; dx < SX; ++dx) vs[u][dy][dx] = StreamLoad(row + min(dx, g.w - 1 - b[u] * SX));
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      if (t0 + u * kPoolBlock >= nblk) break;
+      float pv[JY][JX], gv[JY][JX];
+      bool ok[JY][JX];
+#pragma unroll
+      for (int jy = 0; jy < JY; ++jy) {
+#pragma unroll
+        for (int jx = 0; jx < JX; ++jx) {
+          const int py = a0 + ar[u] - jy, px = b[u] - jx;
+          ok[jy][jx] = py >= 0 && py < g.ph && px >= 0 && px < g.pw;
+          /* a window that does not exist reads slot 0 and is skipped by the select below */
+          const int li = ok[jy][jx] ? (py - p0) * g.lds_pitch + px : 0;
+          pv[jy][jx] = sp[li];
+          gv[jy][jx] = sg[li];
+        }
+      }
+#pragma unroll
+      for (int dy = 0; dy < SY; ++dy) {
+        const int yr = ar[u] * SY + dy;
+        float val[SX];
+#pragma unroll
+        for (int dx = 0; dx < SX; ++dx) {
+          val[dx] = 0.0f;
+#pragma unroll
+          for (int jy = JY - 1; jy >= 0; --jy) {      // py ascending
+            if (jy * SY + dy >= KY) continue;         // this window row does not reach the pixel
+#pragma unroll
+            for (int jx = JX - 1; jx >= 0; --jx) {    // px ascending
+              if (jx * SX + dx >= KX) continue;
+              const float t = val[dx] + Op::Grad(vs[u][dy][dx], pv[jy][jx]) * gv[jy][jx];
+              val[dx] = ok[jy][jx] ? t : val[dx];
+            }
+          }
+        }
+        if (yr < ny) {
+          float *orow = out + static_cast<size_t>(yr) * dstride + b[u] * SX;
+          if (VEC) {
+            StreamStoreN<SX>(orow, val);
+          } else {
+#pragma unroll
+            for (int dx = 0; dx < SX; ++dx) {
+              if (b[u] * SX + dx < g.w) StreamStore(orow + dx, val[dx]);
+            }
+          }
         }
       }
     }

@@ -14,6 +14,7 @@ namespace mshadow_hipk {
 
 typedef float F4 __attribute__((ext_vector_type(4)));
 typedef uint32_t U4 __attribute__((ext_vector_type(4)));
+typedef float F2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ F4 StreamLoadF4(const float *p) {
   return __builtin_nontemporal_load(reinterpret_cast<const F4 *>(p));
@@ -22,6 +23,22 @@ __device__ __forceinline__ void StreamStoreF4(float *p, F4 v) {
   __builtin_nontemporal_store(v, reinterpret_cast<F4 *>(p));
 }
 __device__ __forceinline__ float StreamLoad(const float *p) { return __builtin_nontemporal_load(p); }
+/*! \brief N consecutive floats (N = 2 or 4) as one access; p aligned to N * 4 bytes */
+template <int N>
+__device__ __forceinline__ void StreamLoadN(float (&v)[N], const float *p) {
+  typedef float V __attribute__((ext_vector_type(N)));
+  const V q = __builtin_nontemporal_load(reinterpret_cast<const V *>(p));
+#pragma unroll
+  for (int i = 0; i < N; ++i) v[i] = q[i];
+}
+template <int N>
+__device__ __forceinline__ void StreamStoreN(float *p, const float (&v)[N]) {
+  typedef float V __attribute__((ext_vector_type(N)));
+  V q;
+#pragma unroll
+  for (int i = 0; i < N; ++i) q[i] = v[i];
+  __builtin_nontemporal_store(q, reinterpret_cast<V *>(p));
+}
 __device__ __forceinline__ void StreamStore(float *p, float v) { __builtin_nontemporal_store(v, p); }
 __device__ __forceinline__ uint16_t StreamLoad(const uint16_t *p) {
   return __builtin_nontemporal_load(p);
