@@ -166,7 +166,12 @@ int Col2Im(T *img, int istride, const T *col, int cstride, const PatchGeom &g, v
     const size_t lds = static_cast<size_t>(taps) * t.pitch * sizeof(T);
     const long long blocks = planes * nb;
     if (blocks >= (1ll << 31)) return Fail(MSHADOW_HIP_ERR_ARGUMENT, "col2im: too many workgroups");
-    if (g.dy == 1 && g.dx == 1 && g.sy == 1 && g.sx == 1) {
+    if (sizeof(T) == 2 && g.dy == 1 && g.dx == 1 && g.sy == 1 && g.sx == 1 && g.ky == 3 && g.kx == 3) {
+      const mshadow::FastDivU32 div_wpairs(static_cast<uint32_t>((g.w + 1) / 2));
+      hipLaunchKernelGGL((Col2ImHalfPairKernel<3, 3>), dim3(static_cast<unsigned>(blocks)),
+                         dim3(kPatchBlock), lds, AsStream(stream), reinterpret_cast<uint16_t *>(img),
+                         istride, reinterpret_cast<const uint16_t *>(col), cstride, g, t, div_wpairs);
+    } else if (g.dy == 1 && g.dx == 1 && g.sy == 1 && g.sx == 1) {
       hipLaunchKernelGGL((Col2ImTiledKernel<T, EPT, true>), dim3(static_cast<unsigned>(blocks)),
                          dim3(kPatchBlock), lds, AsStream(stream), img, istride, col, cstride, g, t);
     } else {

@@ -19,6 +19,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mshadow/core/fastdiv.h>
+
 #include "stream_access.h"
 
 namespace mshadow_hipk {
@@ -213,6 +215,127 @@ __global__ void __launch_bounds__(kPatchBlock)
         }
       }
       dst[static_cast<size_t>(cyr) * istride + cx] = res;
+    }
+  }
+}
+
+/*! \brief col2im for binary16, stride 1, dilation 1 and a KY x KX window fixed at compile
+ *  time (the convolution-backward case). Same tiling as Col2ImTiledKernel, with
+ *   - the staging loads of all taps issued before any is parked in LDS (KY*KX 128-bit
+ *     loads in flight per thread);
+ *   - two adjacent pixels per thread, summed as a packed pair: adding two binary16 values
+ *     in binary16 is the same as widening both to float, adding (exactly) and rounding
+ *     back, which is what the reference's half_t operator+= does after every term
+ *     (mshadow/half.h:58-62), so one packed add per tap replaces two conversions, an add
+ *     and a rounding per pixel;
+ *   - the taps unrolled in the reference's order (py ascending = a descending, then px
+ *     ascending = b descending), a tap that does not exist for a pixel skipped by a
+ *     16-bit-wise select. */
+template <int KY, int KX>
+__global__ void __launch_bounds__(kPatchBlock)
+    Col2ImHalfPairKernel(uint16_t *img, int istride, const uint16_t *col, int cstride, PatchGeom g,
+                         PatchTile t, mshadow::FastDivU32 div_wpairs) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  typedef uint16_t T;
+  typedef _Float16 H2 __attribute__((ext_vector_type(2)));
+  const int EPT = 8;
+  const int TAPS = KY * KX;
+  T *lds = reinterpret_cast<T *>(smem_raw);
+  const int plane = blockIdx.x / t.bands;
+  const int band = blockIdx.x - plane * t.bands;
+  const int ch = plane % g.c;
+  const int n = plane / g.c;
+  const int cy0 = band * t.band;
+  const int ncy = min(t.band, g.h - cy0);
+  const int yf = cy0 + g.pad_y, yl = cy0 + ncy - 1 + g.pad_y;
+  const int p0 = yf < KY ? 0 : yf - KY + 1;
+  const int p1 = min(yl + 1, g.oh);
+  const int npy = max(p1 - p0, 0);
+  const int run = npy * g.ow;
+  const size_t j0 = (static_cast<size_t>(n) * g.oh + p0) * g.ow;
+  const T *in0 = col + static_cast<size_t>(ch * TAPS) * cstride + j0;
+  const bool vec_ok = reinterpret_cast<uintptr_t>(in0) % 16 == 0 && cstride % EPT == 0;
+  if (vec_ok) {
+    for (int e0 = threadIdx.x * EPT; e0 < run; e0 += kPatchBlock * EPT) {
+      const bool whole = e0 + EPT <= run;
+      /* unpredicated: a partial last pack is fetched from its last whole position */
+      const int ec = whole ? e0 : max(run - EPT, 0);
+      U4 q[TAPS];
+      if (run >= EPT) {
+#pragma unroll
+        for (int tap = 0; tap < TAPS; ++tap) {
+          /* only whole packs can be fetched at an aligned address */
+          q[tap] = StreamLoad16(in0 + static_cast<size_t>(tap) * cstride + (whole ? ec : (ec / EPT) * EPT));
+        }
+      }
+#pragma unroll
+      for (int tap = 0; tap < TAPS; ++tap) {
+        T *out = lds + tap * t.pitch;
+        if (whole) {
+          *reinterpret_cast<U4 *>(out + e0) = q[tap];
+        } else {
+          const T *in = in0 + static_cast<size_t>(tap) * cstride;
+          for (int e = e0; e < run; ++e) out[e] = in[e];
+        }
+      }
+    }
+  } else {
+    for (int tap = 0; tap < TAPS; ++tap) {
+      const T *in = in0 + static_cast<size_t>(tap) * cstride;
+      T *out = lds + tap * t.pitch;
+      for (int e = threadIdx.x; e < run; e += kPatchBlock) out[e] = in[e];
+    }
+  }
+  __syncthreads();
+  T *dst = img + (static_cast<size_t>(plane) * g.h + cy0) * istride;
+  const int wpairs = (g.w + 1) / 2;
+  const int npairs = ncy * wpairs;
+  const bool store32 = istride % 2 == 0 && reinterpret_cast<uintptr_t>(img) % 4 == 0;
+  for (int idx = threadIdx.x; idx < npairs; idx += kPatchBlock) {
+    const int cyr = static_cast<int>(div_wpairs.Div(static_cast<uint32_t>(idx)));
+    const int cx = (idx - cyr * wpairs) * 2;
+    const int y = cy0 + cyr + g.pad_y;
+    const int x = cx + g.pad_x;
+    const bool second = cx + 1 < g.w;
+    /* per b: where the two pixels read (clamped into the row) and which of them exist */
+    int pxc[KX][2];
+    uint32_t keep[KX];
+#pragma unroll
+    for (int b = 0; b < KX; ++b) {
+      const int px0 = x - b, px1 = x + 1 - b;
+      const bool ok0 = px0 >= 0 && px0 < g.ow;
+      const bool ok1 = second && px1 >= 0 && px1 < g.ow;
+      pxc[b][0] = min(max(px0, 0), g.ow - 1);
+      pxc[b][1] = min(max(px1, 0), g.ow - 1);
+      keep[b] = (ok0 ? 0x0000ffffu : 0u) | (ok1 ? 0xffff0000u : 0u);
+    }
+    uint32_t res = 0u;  // two binary16 zeros
+#pragma unroll
+    for (int a = KY - 1; a >= 0; --a) {
+      const int py = y - a;
+      const bool row_ok = py >= 0 && py < g.oh;
+      const int rowbase = (min(max(py, p0), max(p1 - 1, p0)) - p0) * g.ow;
+#pragma unroll
+      for (int b = KX - 1; b >= 0; --b) {
+        const T *tap = lds + (a * KX + b) * t.pitch + rowbase;
+        const uint32_t v = static_cast<uint32_t>(tap[pxc[b][0]]) |
+                           (static_cast<uint32_t>(tap[pxc[b][1]]) << 16);
+        H2 acc, term;
+        __builtin_memcpy(&acc, &res, 4);
+        __builtin_memcpy(&term, &v, 4);
+        const H2 sum = acc + term;
+        uint32_t sbits;
+        __builtin_memcpy(&sbits, &sum, 4);
+        const uint32_t m = row_ok ? keep[b] : 0u;
+        res = (sbits & m) | (res & ~m);
+      }
+    }
+    T *out = dst + static_cast<size_t>(cyr) * istride + cx;
+    if (second && store32) {
+      *reinterpret_cast<uint32_t *>(out) = res;
+    } else {
+      out[0] = static_cast<T>(res & 0xffffu);
+      if (second) out[1] = static_cast<T>(res >> 16);
     }
   }
 }
