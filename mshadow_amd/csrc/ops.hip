@@ -118,9 +118,22 @@ int Im2Col(T *col, int cstride, const T *img, int istride, const PatchGeom &g, v
     t.bands = static_cast<int>(nb);
     t.rows_max = static_cast<int>((band - 1) * g.sy + halo);
     t.pitch = g.wp;
-    const size_t lds = static_cast<size_t>(t.rows_max) * row_bytes;
     const long long blocks = planes * nb;
     if (blocks >= (1ll << 31)) return Fail(MSHADOW_HIP_ERR_ARGUMENT, "im2col: too many workgroups");
+    /* binary16, 3 taps per row, stride and dilation 1, rows of whole aligned packs */
+    const bool row3 = sizeof(T) == 2 && g.kx == 3 && g.sy == 1 && g.sx == 1 && g.dy == 1 &&
+                      g.dx == 1 && g.ow % 8 == 0 && cstride % 8 == 0 &&
+                      reinterpret_cast<uintptr_t>(col) % 16 == 0;
+    if (row3) {
+      t.pitch = (g.wp + 7) / 8 * 8;
+      const size_t lds = static_cast<size_t>(t.rows_max) * t.pitch * sizeof(T);
+      const mshadow::FastDivU32 div_ppr(static_cast<uint32_t>(g.ow / 8));
+      hipLaunchKernelGGL(Im2ColHalfRow3Kernel, dim3(static_cast<unsigned>(blocks)), dim3(kPatchBlock),
+                         lds, AsStream(stream), reinterpret_cast<uint16_t *>(col), cstride,
+                         reinterpret_cast<const uint16_t *>(img), istride, g, t, div_ppr);
+      return AfterLaunch("im2col");
+    }
+    const size_t lds = static_cast<size_t>(t.rows_max) * row_bytes;
     hipLaunchKernelGGL((Im2ColTiledKernel<T, EPT>), dim3(static_cast<unsigned>(blocks)),
                        dim3(kPatchBlock), lds, AsStream(stream), col, cstride, img, istride, g, t);
   } else {

@@ -154,6 +154,67 @@ __global__ void __launch_bounds__(kPatchBlock)
   }
 }
 
+/*! \brief im2col for binary16, stride 1, dilation 1, kx = 3 and a patch row made of whole
+ *  8-element packs (ow % 8 == 0). The three taps b = 0, 1, 2 of one (a, oy, ox..ox+7)
+ *  position read overlapping LDS elements ox..ox+9: they are fetched once as five aligned
+ *  dwords and the three 16-byte output packs are cut from them (b = 1 by a funnel shift),
+ *  so a pack costs less than one LDS read instead of eight 16-bit ones. LDS rows are
+ *  16-byte aligned (t.pitch % 8 == 0). */
+__global__ void __launch_bounds__(kPatchBlock)
+    Im2ColHalfRow3Kernel(uint16_t *col, int cstride, const uint16_t *img, int istride, PatchGeom g,
+                         PatchTile t, mshadow::FastDivU32 div_ppr) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  typedef uint16_t T;
+  T *lds = reinterpret_cast<T *>(smem_raw);
+  const int plane = blockIdx.x / t.bands;
+  const int band = blockIdx.x - plane * t.bands;
+  const int ch = plane % g.c;
+  const int n = plane / g.c;
+  const int oy0 = band * t.band;
+  const int noy = min(t.band, g.oh - oy0);
+  const int in_rows = noy + g.ky - 1;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const T *src = img + static_cast<size_t>(plane) * g.h * istride;
+  for (int r = wave; r < in_rows; r += kPatchBlock / 64) {
+    const int y = oy0 + r - g.pad_y;
+    const bool row_ok = y >= 0 && y < g.h;
+    for (int xx = lane; xx < t.pitch; xx += 64) {
+      const int x = xx - g.pad_x;
+      T v = 0;
+      if (row_ok && x >= 0 && x < g.w) v = src[static_cast<size_t>(y) * istride + x];
+      lds[r * t.pitch + xx] = v;
+    }
+  }
+  __syncthreads();
+  const int ppr = g.ow / 8;            // packs per patch row
+  const int ppt = noy * ppr;           // packs per tap of this band
+  const int items = g.ky * ppt;
+  const size_t j0 = (static_cast<size_t>(n) * g.oh + oy0) * g.ow;
+  for (int item = threadIdx.x; item < items; item += kPatchBlock) {
+    int a = 0, pk = item;
+    while (pk >= ppt) {
+      pk -= ppt;
+      ++a;
+    }
+    const int oy = static_cast<int>(div_ppr.Div(static_cast<uint32_t>(pk)));
+    const int ox = (pk - oy * ppr) * 8;
+    const uint32_t *w = reinterpret_cast<const uint32_t *>(lds + (oy + a) * t.pitch + ox);
+    const U4 w03 = *reinterpret_cast<const U4 *>(w);
+    const uint32_t w4 = w[4];
+    U4 mid;
+    mid.x = __builtin_amdgcn_alignbit(w03.y, w03.x, 16);
+    mid.y = __builtin_amdgcn_alignbit(w03.z, w03.y, 16);
+    mid.z = __builtin_amdgcn_alignbit(w03.w, w03.z, 16);
+    mid.w = __builtin_amdgcn_alignbit(w4, w03.w, 16);
+    U4 hi;
+    hi.x = w03.y; hi.y = w03.z; hi.z = w03.w; hi.w = w4;
+    T *out = col + static_cast<size_t>((ch * g.ky + a) * 3) * cstride + j0 + static_cast<size_t>(pk) * 8;
+    StreamStore16(out, w03);
+    StreamStore16(out + cstride, mid);
+    StreamStore16(out + 2 * static_cast<size_t>(cstride), hi);
+  }
+}
+
 /*! \brief FAST: stride 1 and dilation 1 in both directions (the common convolution case):
  *  every patch-range bound is then a subtraction instead of a division. */
 template <typename T, int EPT, bool FAST>
