@@ -90,16 +90,21 @@ OSUM_HD float LaneQuant(const float (&t)[N], const Binade &b) {
     return any ? kReject : 0.0f;
   }
   float sum = 0.0f;
-  bool tie = false;
+  float worst = 0.0f;    /* largest distance of a scaled term from its rounded value */
+  float least = 0.0f;    /* most negative scaled term */
   for (int i = 0; i < N; ++i) {
     const float scaled = t[i] * b.inv_u;  /* exact: inv_u is a power of two */
     const float q = rintf(scaled);        /* round to nearest even */
-    /* |scaled - q| == 0.5 exactly when the term sits half way; NaN also lands here. A
-       negative term would move the sum down, which the one-sided Fits() does not watch */
-    tie = tie || !(fabsf(scaled - q) < 0.5f) || !(scaled >= 0.0f);
+    worst = fmaxf(worst, fabsf(scaled - q));
+    least = fminf(least, scaled);
     sum += q;
   }
-  return tie ? kReject : sum;
+  /* worst == 0.5 exactly when some term sits half way between two integers. A negative
+     term would move the sum down, which the one-sided Fits() does not watch. NaN and
+     infinite terms slip through the max / min but leave `sum` NaN or infinite, which
+     no caller accepts (every acceptance is a `< kLimit` comparison). */
+  const bool bad = !(worst < 0.5f) || least < 0.0f;
+  return bad ? kReject : sum;
 }
 
 /*! \brief true if integer contributions totalling q can be added without leaving the

@@ -138,15 +138,19 @@ const int kPlanSlots = 24;
  *  the chunk's terms (so that the walk needs nothing from the register-resident row).
  *  General chunk: a = integer total of the clean lanes in front of the lane, b = its plan
  *  code. Two-binade chunk: a / b = inclusive integer prefix of the lanes quantised against
- *  the lower / upper binade (lanes holding a tie count as 0), c = tie flags. */
+ *  the lower / upper binade (lanes holding a tie count as 0). */
 template <int N>
 struct LanePlanSlot {
   float t[kWave][N];
   uint32_t a[kWave];
   uint32_t b[kWave];
-  uint32_t c[kWave];
+  unsigned long long tie_lo, tie_hi;  //!< two-binade chunks: lanes holding a tie (lower / upper binade)
   uint32_t total;  //!< general chunks: integer total of the clean lanes
   int kind;        //!< plan code of the chunk (kPlanWalk or kPlanTwoBinades + e)
+  float start;     //!< approximate prefix sum in front of the chunk
+  int chunk;       //!< index of the chunk in the row
+  uint32_t ex;     //!< integer total of the clean chunks in front of this one
+  int e_run;       //!< binade of the clean chunk just in front (if there is one)
 };
 
 template <int W, int SLABS, int N>
@@ -243,45 +247,52 @@ __device__ __forceinline__ uint32_t PlanLanes(const float (&t)[N], float start, 
 }
 
 /*! \brief s plus one chunk, given its lane-level plan: runs of clean lanes are applied as
- *  integers (and verified), every other lane adds its terms one by one */
+ *  integers (and verified), runs of other lanes add their terms one by one */
 template <int N>
 __device__ __forceinline__ float WalkLanes(float s, const float (&t)[N], uint32_t ex, int code,
                                            uint32_t total, bool *fail) {
   using namespace ordered_sum;
+  using mshadow::hip::ReadLaneU32;
   unsigned long long todo = __ballot(code < 0);
   uint32_t done = 0u;
   while (todo != 0ull) {
-    const int l = __ffsll(static_cast<long long>(todo)) - 1;
-    todo &= todo - 1ull;
-    const uint32_t exl = mshadow::hip::ReadLaneU32(ex, l);
+    const int l0 = __ffsll(static_cast<long long>(todo)) - 1;
+    const uint32_t exl = ReadLaneU32(ex, l0);
     if (exl != done) {
-      const int e = static_cast<int>(mshadow::hip::ReadLaneU32(static_cast<uint32_t>(code), l - 1));
-      s = FlushRun(s, e, exl - done, fail);
+      s = FlushRun(s, static_cast<int>(ReadLaneU32(static_cast<uint32_t>(code), l0 - 1)), exl - done, fail);
       done = exl;
     }
+    /* the lanes l0 .. l1-1 are walked: l1 = first clean lane above l0 (or 64) */
+    const unsigned long long above = ~(todo >> l0);
+    const int len = above != 0ull ? __ffsll(static_cast<long long>(above)) - 1 : kWave - l0;
+    const int l1 = l0 + len;
+    for (int l = l0; l < l1; ++l) {
 #pragma unroll
-    for (int i = 0; i < N; ++i) s = s + ReadLaneF32(t[i], l);
+      for (int i = 0; i < N; ++i) s = s + ReadLaneF32(t[i], l);
+    }
+    todo = l1 < kWave ? (todo >> l1) << l1 : 0ull;
   }
   if (total != done) {
-    const int e = static_cast<int>(mshadow::hip::ReadLaneU32(static_cast<uint32_t>(code), kWave - 1));
-    s = FlushRun(s, e, total - done, fail);
+    s = FlushRun(s, static_cast<int>(ReadLaneU32(static_cast<uint32_t>(code), kWave - 1)), total - done, fail);
   }
   return s;
 }
 
 /*! \brief plan of a chunk that starts in binade elo and may end in elo + 1: every lane
- *  quantised against both; *flags bit 0 / 1 = the lane holds a tie under the lower /
- *  upper binade (such a lane counts as 0 in that prefix) */
+ *  quantised against both; a lane holding a tie under a binade counts as 0 in that prefix
+ *  and is named in the tie mask */
 template <int N>
 __device__ __forceinline__ void PlanTwoBinades(const float (&t)[N], int elo, uint32_t *incl_lo,
-                                               uint32_t *incl_hi, uint32_t *flags) {
+                                               uint32_t *incl_hi, unsigned long long *tie_lo,
+                                               unsigned long long *tie_hi) {
   using namespace ordered_sum;
   const float qlo = LaneQuant<N>(t, BinadeOfExponent(static_cast<uint32_t>(elo)));
   const float qhi = LaneQuant<N>(t, BinadeOfExponent(static_cast<uint32_t>(elo + 1)));
   const bool tlo = !(qlo < kLimit), thi = !(qhi < kLimit);
   *incl_lo = mshadow::hip::WaveInclusiveScanU32(tlo ? 0u : static_cast<uint32_t>(qlo));
   *incl_hi = mshadow::hip::WaveInclusiveScanU32(thi ? 0u : static_cast<uint32_t>(qhi));
-  *flags = (tlo ? 1u : 0u) | (thi ? 2u : 0u);
+  *tie_lo = __ballot(tlo);
+  *tie_hi = __ballot(thi);
 }
 
 /*! \brief s plus one chunk planned by PlanTwoBinades. Each round accepts, as integers,
@@ -291,39 +302,72 @@ __device__ __forceinline__ void PlanTwoBinades(const float (&t)[N], int elo, uin
 template <int N>
 __device__ __forceinline__ float WalkTwoBinades(float s, const float (&t)[N], int elo,
                                                 uint32_t incl_lo, uint32_t incl_hi,
-                                                uint32_t flags, bool *fail) {
+                                                unsigned long long tie_lo,
+                                                unsigned long long tie_hi, bool *fail) {
   using namespace ordered_sum;
   using mshadow::hip::ReadLaneU32;
-  const int lane = LaneId();
-  int p = 0;        // lanes before p are in s
-  bool hi = false;  // s has crossed into the upper binade
+  /* The usual course in straight-line code: the lanes up to the crossing (or tie) lane f
+     as integers in the lower binade, lane f term by term, all lanes behind it as integers
+     in whichever of the two binades the sum is in then. Anything else (a second tie, a sum
+     in neither binade) takes the general rounds below from the start. */
+  {
+    const uint32_t el = static_cast<uint32_t>(elo);
+    const float m = s * FloatOf((277u - el) << 23);
+    const uint32_t room = 16777216u - static_cast<uint32_t>(m);
+    const unsigned long long ev = __ballot(incl_lo >= room) | tie_lo;
+    const bool in_lo = m >= 8388608.0f && m < kLimit;
+    if (in_lo && ev == 0ull) {
+      return (m + static_cast<float>(ReadLaneU32(incl_lo, kWave - 1))) * FloatOf((el - 23u) << 23);
+    }
+    if (in_lo) {
+      const int f = __ffsll(static_cast<long long>(ev)) - 1;
+      const uint32_t upto = f > 0 ? ReadLaneU32(incl_lo, f - 1) : 0u;
+      float s2 = (m + static_cast<float>(upto)) * FloatOf((el - 23u) << 23);
+#pragma unroll
+      for (int i = 0; i < N; ++i) s2 = s2 + ReadLaneF32(t[i], f);
+      const float mh = s2 * FloatOf((276u - el) << 23);  // in units of the upper binade
+      const bool up = mh >= 8388608.0f;
+      const float m2 = up ? mh : mh + mh;                 // exact either way
+      const uint32_t incl2 = up ? incl_hi : incl_lo;
+      const uint32_t base2 = ReadLaneU32(incl2, f);
+      const uint32_t room2 = 16777216u - static_cast<uint32_t>(m2);
+      const unsigned long long behind = f < kWave - 1 ? (~0ull << 1) << f : 0ull;
+      const unsigned long long ev2 = (__ballot(incl2 - base2 >= room2) | (up ? tie_hi : tie_lo)) & behind;
+      if (ev2 == 0ull && m2 >= 8388608.0f && m2 < kLimit) {
+        const float u2 = FloatOf((el - 23u + (up ? 1u : 0u)) << 23);
+        return (m2 + static_cast<float>(ReadLaneU32(incl2, kWave - 1) - base2)) * u2;
+      }
+    }
+  }
+  unsigned long long pending = ~0ull;  // lanes not yet in s
+  int p = 0;                           // = number of lanes in s
+  bool hi = false;                     // s has crossed into the upper binade
   while (true) {
-    Binade b = BinadeOfExponent(static_cast<uint32_t>(elo + (hi ? 1 : 0)));
-    float m = s * b.inv_u;
+    const uint32_t e = static_cast<uint32_t>(elo) + (hi ? 1u : 0u);
+    const float m = s * FloatOf((277u - e) << 23);
     if (!hi && !(m < kLimit)) {
       hi = true;
-      b = BinadeOfExponent(static_cast<uint32_t>(elo + 1));
-      m = s * b.inv_u;
+      continue;
     }
     if (!(m >= 8388608.0f && m < kLimit)) {  // s is in neither binade: the plan was wrong
       *fail = true;
       return s;
     }
+    const float u = FloatOf((e - 23u) << 23);
     const uint32_t incl = hi ? incl_hi : incl_lo;
-    const bool tie = (flags & (hi ? 2u : 1u)) != 0u;
     const uint32_t base = p > 0 ? ReadLaneU32(incl, p - 1) : 0u;
     const uint32_t room = 16777216u - static_cast<uint32_t>(m);  // integer steps left in the binade
-    const unsigned long long events = __ballot(lane >= p && (tie || incl - base >= room));
-    if (events == 0ull) {
-      return (m + static_cast<float>(ReadLaneU32(incl, kWave - 1) - base)) * b.u;
-    }
+    /* lanes already in s compare on a wrapped difference; `pending` masks them out */
+    const unsigned long long events = (__ballot(incl - base >= room) | (hi ? tie_hi : tie_lo)) & pending;
+    if (events == 0ull) return (m + static_cast<float>(ReadLaneU32(incl, kWave - 1) - base)) * u;
     const int f = __ffsll(static_cast<long long>(events)) - 1;
     const uint32_t upto = f > 0 ? ReadLaneU32(incl, f - 1) : 0u;
-    s = (m + static_cast<float>(upto - base)) * b.u;
+    s = (m + static_cast<float>(upto - base)) * u;
 #pragma unroll
     for (int i = 0; i < N; ++i) s = s + ReadLaneF32(t[i], f);
+    if (f == kWave - 1) return s;
     p = f + 1;
-    if (p == kWave) return s;
+    pending = (~0ull << 1) << f;
   }
 }
 
@@ -351,13 +395,16 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
     lds->fail = 0;
     lds->nslots = 0u;
   }
+  {
+    float part[SLABS];
 #pragma unroll
-  for (int j = 0; j < SLABS; ++j) {
-    float a = v[j][0];
+    for (int j = 0; j < SLABS; ++j) {
+      part[j] = v[j][0];
 #pragma unroll
-    for (int i = 1; i < N; ++i) a += v[j][i];
-    a = ReadLaneF32(WaveInclusiveScanF32(a), kWave - 1);
-    if (lane == 0) lds->approx[wave * SLABS + j] = a;
+      for (int i = 1; i < N; ++i) part[j] += v[j][i];
+    }
+    const float mine = mshadow::hip::WaveSumMany<SLABS>(part);  // lane l: chunk l % SLABS
+    if (lane < SLABS) lds->approx[wave * SLABS + lane] = mine;
   }
   __syncthreads();
   MSHADOW_ROWSUM_STAMP(1)
@@ -398,29 +445,38 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
 
   /* C: integer totals of this wave's clean chunks ... */
   MSHADOW_ROWSUM_STAMP(2)
-  uint32_t dirty_mask = 0u;  // this wave's slabs that have to be walked
-  uint32_t tie_mask = 0u;    // of those, planned clean but found to hold a tie
+  uint32_t dirty_mask;  // this wave's slabs that have to be walked
+  uint32_t tie_mask;    // of those, planned clean but found to hold a tie
+  {
+    float part[SLABS];
 #pragma unroll
-  for (int j = 0; j < SLABS; ++j) {
-    const int k = wave * SLABS + j;
-    const int ck = static_cast<int>(ReadLaneU32(code[j % CPL], k / CPL));
-    uint32_t total = kDirtyQ;
-    if (IsClean(ck)) {
-      const Binade b = BinadeOfExponent(static_cast<uint32_t>(ck));
-      const float q = ReadLaneF32(WaveInclusiveScanF32(LaneQuant<N>(v[j], b)), kWave - 1);
-      if (q < kLimit) {
-        total = static_cast<uint32_t>(q);
-      } else {
-        tie_mask |= 1u << j;  // a tie somewhere in the chunk pushed q past 2^24
-      }
+    for (int j = 0; j < SLABS; ++j) {
+      const int k = wave * SLABS + j;
+      const int ck = static_cast<int>(ReadLaneU32(code[j % CPL], k / CPL));
+      part[j] = 0.0f;
+      if (IsClean(ck)) part[j] = LaneQuant<N>(v[j], BinadeOfExponent(static_cast<uint32_t>(ck)));
     }
-    if (total == kDirtyQ) dirty_mask |= 1u << j;
-    if (lane == 0) {
-      lds->q[k] = total;
-      lds->slot_of[wave][j] = -1;
+    const float q = mshadow::hip::WaveSumMany<SLABS>(part);  // lane l: chunk l % SLABS
+    /* lanes 0 .. SLABS-1 file the result of "their" chunk; its plan code sits in the
+       chunk table at lane k / CPL, slot k % CPL = lane % CPL */
+    const int k = wave * SLABS + (lane % SLABS);
+    int ck = 0;
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+      const int got = __shfl(static_cast<int>(code[c]), k / CPL);
+      ck = (lane % CPL == c) ? got : ck;
     }
+    const bool clean = IsClean(ck);
+    const bool whole = clean && q < kLimit;  // a tie anywhere in the chunk pushes q past 2^24
+    if (lane < SLABS) {
+      lds->q[k] = whole ? static_cast<uint32_t>(q) : kDirtyQ;
+      lds->slot_of[wave][lane] = -1;
+    }
+    dirty_mask = static_cast<uint32_t>(__ballot(lane < SLABS && !whole));
+    tie_mask = static_cast<uint32_t>(__ballot(lane < SLABS && clean && !whole));
   }
-  /* ... and lane plans of its dirty ones, parked in LDS slots */
+  /* ... and its dirty ones handed, with their terms, to plan slots: the lane plans are
+     made by all waves together further down (the first wave of a row owns most dirty chunks) */
   for (uint32_t todo = dirty_mask; todo != 0u; todo &= todo - 1u) {
     const int j = __ffs(static_cast<int>(todo)) - 1;
     const int k = wave * SLABS + j;
@@ -428,36 +484,26 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
     if (lane == 0) slot = atomicAdd(&lds->nslots, 1u);
     slot = __builtin_amdgcn_readfirstlane(slot);
     if (slot >= static_cast<uint32_t>(Lds::kSlots)) break;  // the rest is resolved by wave scans
-    int ck = static_cast<int>(TableAt<CPL>(code, k));
-    if ((tie_mask >> j) & 1u) ck = kPlanTwoBinades + ck;
     float t[N];
     SelectSlab<SLABS, N>(t, v, j);
-    uint32_t pa, pb, pc = 0u, tot = 0u;
-    if (ck >= kPlanTwoBinades) {
-      PlanTwoBinades<N>(t, ck - kPlanTwoBinades, &pa, &pb, &pc);
-    } else {
-      float st = start[0];
-#pragma unroll
-      for (int c = 1; c < CPL; ++c) st = (k % CPL == c) ? start[c] : st;
-      int code_l;
-      tot = PlanLanes<N>(t, ReadLaneF32(st, k / CPL), margin, &pa, &code_l);
-      pb = static_cast<uint32_t>(code_l);
-    }
     LanePlanSlot<N> *ps = &lds->plan[slot];
 #pragma unroll
     for (int i = 0; i < N; ++i) ps->t[lane][i] = t[i];
-    ps->a[lane] = pa;
-    ps->b[lane] = pb;
-    ps->c[lane] = pc;
+    int ck = static_cast<int>(TableAt<CPL>(code, k));
+    if ((tie_mask >> j) & 1u) ck = kPlanTwoBinades + ck;
+    uint32_t start_bits[CPL];
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) start_bits[c] = __float_as_uint(start[c]);
+    const float st = __uint_as_float(TableAt<CPL>(start_bits, k));
     if (lane == 0) {
-      ps->total = tot;
       ps->kind = ck;
+      ps->start = st;
+      ps->chunk = k;
       lds->slot_of[wave][j] = static_cast<signed char>(slot);
     }
   }
   __syncthreads();
   MSHADOW_ROWSUM_STAMP(3)
-
   /* D: tables of the walk */
   uint32_t ex[CPL];  // integer prefix over clean chunks in front of each chunk
   uint32_t total_ex;
@@ -485,44 +531,87 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
     for (int c = 0; c < CPL; ++c) ex[c] = excl + pre[c];
     total_ex = ReadLaneU32(incl, kWave - 1);
   }
+  /* lane plans of the dirty chunks, made by all waves together */
+  {
+    const uint32_t handed = lds->nslots;
+    const int nslots = handed < static_cast<uint32_t>(Lds::kSlots) ? static_cast<int>(handed) : Lds::kSlots;
+    for (int sl = wave; sl < nslots; sl += W) {
+      LanePlanSlot<N> *ps = &lds->plan[sl];
+      float t[N];
+#pragma unroll
+      for (int i = 0; i < N; ++i) t[i] = ps->t[lane][i];
+      const int ck = ps->kind;
+      uint32_t pa, pb;
+      if (ck >= kPlanTwoBinades) {
+        unsigned long long tlo, thi;
+        PlanTwoBinades<N>(t, ck - kPlanTwoBinades, &pa, &pb, &tlo, &thi);
+        if (lane == 0) {
+          ps->tie_lo = tlo;
+          ps->tie_hi = thi;
+        }
+      } else {
+        int code_l;
+        const uint32_t tot = PlanLanes<N>(t, ps->start, margin, &pa, &code_l);
+        pb = static_cast<uint32_t>(code_l);
+        if (lane == 0) ps->total = tot;
+      }
+      ps->a[lane] = pa;
+      ps->b[lane] = pb;
+      /* what the walk needs from the chunk table, so that it reads scalars only */
+      const int k = ps->chunk;
+      const uint32_t exk = TableAt<CPL>(ex, k);
+      const uint32_t erun = k > 0 ? TableAt<CPL>(code, k - 1) : 0u;
+      if (lane == 0) {
+        ps->ex = exk;
+        ps->e_run = static_cast<int>(erun);
+      }
+    }
+  }
+
+  __syncthreads();
   MSHADOW_ROWSUM_STAMP(4)
   for (int w = 0; w < W; ++w) {
     if (((owners >> w) & 1u) == 0u) continue;  // block-uniform: every wave holds the same tables
     if (wave == w) {
       MSHADOW_ROWSUM_STAMP(8)
+      /* the walk is one chain of dependent instructions that the whole row waits for;
+         the other waves on this SIMD (another row's bulk phases) yield issue slots to it */
+      __builtin_amdgcn_s_setprio(3);
       float s = lds->s;
       uint32_t done = lds->ex;
       bool fail = false;
       for (uint32_t todo = dirty_mask; todo != 0u; todo &= todo - 1u) {
         const int j = __ffs(static_cast<int>(todo)) - 1;
-        const int k = w * SLABS + j;
         const int slot = lds->slot_of[w][j];
-        /* the plan is fetched first: it does not depend on s */
-        float t[N];
-        uint32_t pa = 0u, pb = 0u, pc = 0u, tot = 0u;
-        int kind = kPlanWalk;
         if (slot >= 0) {
+          /* everything about the chunk comes from its slot and none of it depends on s */
           const LanePlanSlot<N> *ps = &lds->plan[slot];
+          float t[N];
 #pragma unroll
           for (int i = 0; i < N; ++i) t[i] = ps->t[lane][i];
-          pa = ps->a[lane];
-          pb = ps->b[lane];
-          pc = ps->c[lane];
-          tot = ps->total;
-          kind = ps->kind;
-        }
-        const uint32_t exk = TableAt<CPL>(ex, k);
-        if (exk != done) {
-          s = FlushRun(s, static_cast<int>(TableAt<CPL>(code, k - 1)), exk - done, &fail);
-          done = exk;
-        }
-        if (slot < 0) {
+          const uint32_t pa = ps->a[lane];
+          const uint32_t pb = ps->b[lane];
+          const int kind = ps->kind;
+          const uint32_t exk = ps->ex;
+          if (exk != done) {
+            s = FlushRun(s, ps->e_run, exk - done, &fail);
+            done = exk;
+          }
+          if (kind >= kPlanTwoBinades) {
+            s = WalkTwoBinades<N>(s, t, kind - kPlanTwoBinades, pa, pb, ps->tie_lo, ps->tie_hi, &fail);
+          } else {
+            s = WalkLanes<N>(s, t, pa, static_cast<int>(pb), ps->total, &fail);
+          }
+        } else {
+          const int k = w * SLABS + j;
+          const uint32_t exk = TableAt<CPL>(ex, k);
+          if (exk != done) {
+            s = FlushRun(s, static_cast<int>(TableAt<CPL>(code, k - 1)), exk - done, &fail);
+            done = exk;
+          }
+          float t[N];
           SelectSlab<SLABS, N>(t, v, j);
           s = WaveResolve<N>(s, t);
-        } else if (kind >= kPlanTwoBinades) {
-          s = WalkTwoBinades<N>(s, t, kind - kPlanTwoBinades, pa, pb, pc, &fail);
-        } else {
-          s = WalkLanes<N>(s, t, pa, static_cast<int>(pb), tot, &fail);
         }
       }
       if (lane == 0) {
@@ -530,6 +619,7 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
         lds->ex = done;
         if (fail) lds->fail = 1;
       }
+      __builtin_amdgcn_s_setprio(0);
       MSHADOW_ROWSUM_STAMP(9)
     }
     __syncthreads();

@@ -73,6 +73,62 @@ __device__ __forceinline__ float WaveInclusiveScanF32(float v) {
 #undef MSHADOW_FSCAN_STEP
   return v;
 }
+#define MSHADOW_DPP_QUAD_PERM(a, b, c, d) ((a) | ((b) << 2) | ((c) << 4) | ((d) << 6))
+#define MSHADOW_DPP_ROW_ROR(n) (0x120 + (n))   // lane i reads lane (i + n) % 16 of its row
+
+/*! \brief value of `v` in the lane paired with this one at distance D: lane ^ D for
+ *  D = 1, 2, 8, 16, 32 and (lane + 4) % 16 within the row for D = 4 - in every case a lane
+ *  whose bit log2(D) is the opposite of this lane's, which is all WaveSumMany needs */
+template <int D>
+__device__ __forceinline__ float PairedLaneF32(float v) {
+  const uint32_t u = __float_as_uint(v);
+  if (D == 1) return __uint_as_float(DppU32<MSHADOW_DPP_QUAD_PERM(1, 0, 3, 2), 0xf>(u, u));
+  if (D == 2) return __uint_as_float(DppU32<MSHADOW_DPP_QUAD_PERM(2, 3, 0, 1), 0xf>(u, u));
+  if (D == 4) return __uint_as_float(DppU32<MSHADOW_DPP_ROW_ROR(4), 0xf>(u, u));
+  if (D == 8) return __uint_as_float(DppU32<MSHADOW_DPP_ROW_ROR(8), 0xf>(u, u));
+  return __shfl_xor(v, D);
+}
+
+/*! \brief M sums over the wave at once (M a power of two up to 32): returns, in lane l,
+ *  the sum over all 64 lanes of a[l % M]. Each of the first log2(M) steps halves the
+ *  number of values a lane carries (it keeps the values whose index has this lane's bit
+ *  and hands the others to its paired lane), so the whole thing costs about M + 2 * 6
+ *  additions instead of 6 * M. `a` is clobbered. Exact on integer-valued floats below 2^24;
+ *  on other floats the order of additions differs from a scan. */
+template <int M, int S = 0>
+struct WaveSumManyStep {
+  static __device__ __forceinline__ void Run(float (&a)[M]) {
+    const bool bit = (threadIdx.x >> S) & 1;
+    const int CNT = M >> (S + 1);
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) {
+      const float keep = bit ? a[2 * i + 1] : a[2 * i];
+      const float send = bit ? a[2 * i] : a[2 * i + 1];
+      a[i] = keep + PairedLaneF32<(1 << S)>(send);
+    }
+    WaveSumManyStep<M, ((2 << S) < M) ? S + 1 : 64>::Run(a);
+  }
+};
+template <int M>
+struct WaveSumManyStep<M, 64> {
+  static __device__ __forceinline__ void Run(float (&)[M]) {}
+};
+template <int M, int D>
+struct WaveSumRest {
+  static __device__ __forceinline__ float Run(float r) {
+    return WaveSumRest<M, D * 2>::Run(r + PairedLaneF32<D>(r));
+  }
+};
+template <int M>
+struct WaveSumRest<M, 64> {
+  static __device__ __forceinline__ float Run(float r) { return r; }
+};
+template <int M>
+__device__ __forceinline__ float WaveSumMany(float (&a)[M]) {
+  if (M > 1) WaveSumManyStep<M, (M > 1 ? 0 : 64)>::Run(a);
+  return WaveSumRest<M, M>::Run(a[0]);
+}
+
 /*! \brief sum over the 64 lanes; result in every lane (as a scalar) */
 __device__ __forceinline__ uint32_t WaveSumU32(uint32_t v) {
   return ReadLaneU32(WaveInclusiveScanU32(v), kWave - 1);
