@@ -121,6 +121,8 @@ __device__ inline float BlockOrderedAdd(float s, const float (&t)[N],
  *   E  every wave: apply the clean run behind the last dirty chunk.
  * Lane l keeps the chunk-table entries of chunks l * CPL .. l * CPL + CPL - 1. */
 const uint32_t kDirtyQ = 0xffffffffu;
+/*! \brief lanes of a row's first chunk that are added serially without a plan */
+const int kHeadLanes = 32;
 /*! \brief dirty chunks per row with a lane-level plan parked in LDS (a row of softmax
  *  terms has about a dozen); further ones are resolved by wave scans */
 const int kPlanSlots = 24;
@@ -129,9 +131,6 @@ const int kPlanSlots = 24;
    at the boundaries of the steps; it is empty in the library */
 #ifndef MSHADOW_ROWSUM_STAMP
 #define MSHADOW_ROWSUM_STAMP(step)
-#endif
-#ifndef MSHADOW_ROWSUM_NOTE
-#define MSHADOW_ROWSUM_NOTE(slot, value)
 #endif
 
 /*! \brief lane-level plan of one dirty chunk, parked in LDS between steps C and D, with
@@ -224,13 +223,16 @@ __device__ __forceinline__ void SelectSlab(float (&t)[N], const float (&v)[SLABS
  *  clean lanes in front of this lane; returns the integer total of all clean lanes */
 template <int N>
 __device__ __forceinline__ uint32_t PlanLanes(const float (&t)[N], float start, float margin,
-                                              uint32_t *ex, int *code) {
+                                              bool head, uint32_t *ex, int *code) {
   using namespace ordered_sum;
   float a = t[0];
 #pragma unroll
   for (int i = 1; i < N; ++i) a += t[i];
   const float incl = WaveInclusiveScanF32(a);
   int c = PlanLane(start + (incl - a), start + incl, margin);
+  /* the head of a row (the sum starts at zero): its first lanes cross a binade or hold a
+     tie nearly every time and are added term by term without asking */
+  if (head && LaneId() < kHeadLanes) c = kPlanWalk;
   float q = 0.0f;
   if (c >= 0) {
     q = LaneQuant<N>(t, BinadeOfExponent(static_cast<uint32_t>(c)));
@@ -246,14 +248,38 @@ __device__ __forceinline__ uint32_t PlanLanes(const float (&t)[N], float start, 
   return mshadow::hip::ReadLaneU32(inclu, kWave - 1);
 }
 
+/*! \brief s plus the terms of lanes 0 .. kHeadLanes-1 of a chunk parked in LDS (t[lane][i]),
+ *  one float add after the other. Every lane reads the same addresses (an LDS broadcast),
+ *  so the operands arrive in vector registers and the only chain is the adds themselves. */
+template <int N>
+__device__ __forceinline__ float HeadSerialAdd(float s, const float (*t)[N]) {
+  const int kBatch = 8;  // lanes whose terms are fetched before they are added
+#pragma unroll
+  for (int l0 = 0; l0 < kHeadLanes; l0 += kBatch) {
+    float r[kBatch][N];
+#pragma unroll
+    for (int l = 0; l < kBatch; ++l) {
+#pragma unroll
+      for (int i = 0; i < N; ++i) r[l][i] = t[l0 + l][i];
+    }
+#pragma unroll
+    for (int l = 0; l < kBatch; ++l) {
+#pragma unroll
+      for (int i = 0; i < N; ++i) s = s + r[l][i];
+    }
+  }
+  return s;
+}
+
 /*! \brief s plus one chunk, given its lane-level plan: runs of clean lanes are applied as
- *  integers (and verified), runs of other lanes add their terms one by one */
+ *  integers (and verified), runs of other lanes add their terms one by one. `skip` names
+ *  lanes that are in s already. */
 template <int N>
 __device__ __forceinline__ float WalkLanes(float s, const float (&t)[N], uint32_t ex, int code,
-                                           uint32_t total, bool *fail) {
+                                           uint32_t total, unsigned long long skip, bool *fail) {
   using namespace ordered_sum;
   using mshadow::hip::ReadLaneU32;
-  unsigned long long todo = __ballot(code < 0);
+  unsigned long long todo = __ballot(code < 0) & ~skip;
   uint32_t done = 0u;
   while (todo != 0ull) {
     const int l0 = __ffsll(static_cast<long long>(todo)) - 1;
@@ -551,7 +577,7 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
         }
       } else {
         int code_l;
-        const uint32_t tot = PlanLanes<N>(t, ps->start, margin, &pa, &code_l);
+        const uint32_t tot = PlanLanes<N>(t, ps->start, margin, ps->chunk == 0, &pa, &code_l);
         pb = static_cast<uint32_t>(code_l);
         if (lane == 0) ps->total = tot;
       }
@@ -599,8 +625,11 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
           }
           if (kind >= kPlanTwoBinades) {
             s = WalkTwoBinades<N>(s, t, kind - kPlanTwoBinades, pa, pb, ps->tie_lo, ps->tie_hi, &fail);
+          } else if (ps->chunk == 0) {
+            s = HeadSerialAdd<N>(s, ps->t);
+            s = WalkLanes<N>(s, t, pa, static_cast<int>(pb), ps->total, (1ull << kHeadLanes) - 1ull, &fail);
           } else {
-            s = WalkLanes<N>(s, t, pa, static_cast<int>(pb), ps->total, &fail);
+            s = WalkLanes<N>(s, t, pa, static_cast<int>(pb), ps->total, 0ull, &fail);
           }
         } else {
           const int k = w * SLABS + j;
