@@ -26,8 +26,11 @@ namespace mshadow {
 namespace hip {
 
 const int kMapBlock = 256;
-/*! \brief packs per thread; the loads of all of them are issued before the first use */
+/*! \brief packs per thread; the loads of all of them are issued before the first use.
+ *  Expressions that read several tensors take the deeper one (measured on the 4-in 1-out
+ *  map: 56 us against 59 us), a one-tensor map the shallower (more workgroups). */
 const int kPackUnroll = 4;
+const int kPackUnrollDeep = 8;
 
 template <typename Saver, typename DType, typename DPlan, typename SPlan>
 __global__ void __launch_bounds__(kMapBlock)
@@ -41,8 +44,8 @@ __global__ void __launch_bounds__(kMapBlock)
   }
 }
 
-template <typename Saver, typename DType, int N, bool kFlat, bool kStream, typename DPlan,
-          typename SPlan>
+template <typename Saver, typename DType, int N, bool kFlat, bool kStream, int kPackUnroll,
+          typename DPlan, typename SPlan>
 __global__ void __launch_bounds__(kMapBlock)
     MapPackKernel(DPlan dplan, SPlan splan, uint32_t total_packs, uint32_t packs_per_row) {
   typedef expr::Pack<DType, N> P;

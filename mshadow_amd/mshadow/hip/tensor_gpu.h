@@ -357,15 +357,18 @@ struct MapLauncher<Saver, DType, DPlan, SPlan, true> {
     }
     uint32_t ppr = cols / N;
     uint32_t total = rows * ppr;
-    const uint32_t per_block = hip::kMapBlock * hip::kPackUnroll;
+    /* a plan that carries three or more tensor leaves (pointer + pitch each) is "deep" */
+    const int kUnroll = sizeof(SPlan) >= 3 * (sizeof(void *) + sizeof(index_t))
+                            ? hip::kPackUnrollDeep : hip::kPackUnroll;
+    const uint32_t per_block = hip::kMapBlock * kUnroll;
     const uint32_t grid = (total + per_block - 1) / per_block;
     void *args[] = {&dplan, &splan, &total, &ppr};
     /* streaming (non-temporal) accesses once a tensor no longer fits the caches anyway */
     const bool stream_hint = static_cast<size_t>(rows) * cols * sizeof(DType) >= (8u << 20);
     const bool is_flat = flat || rows == 1;
 #define MSHADOW_MAP_LAUNCH(FLAT, STREAM)                                                   \
-  Launch(hip::MapPackKernel<Saver, DType, N, FLAT, STREAM, DPlan, SPlan>, grid, hip::kMapBlock, \
-         args, stream)
+  Launch(hip::MapPackKernel<Saver, DType, N, FLAT, STREAM, kUnroll, DPlan, SPlan>, grid,   \
+         hip::kMapBlock, args, stream)
     if (is_flat && stream_hint) {
       MSHADOW_MAP_LAUNCH(true, true);
     } else if (is_flat) {
