@@ -265,6 +265,114 @@ void orc_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride
   }
 }
 
+/* SoftmaxGrad with ignore_label, SmoothSoftmaxGrad with and without it,
+   mshadow/tensor_cpu-inl.h:304-362. (src - 1.0f) + alpha is evaluated left to right;
+   smooth_grad = alpha / (cols - 1) in float. */
+static inline void grad_row(float *o, long ostep, const float *s, long sstep, int cols, int k,
+                            int flags, int ignored, float alpha, float smooth_grad) {
+  for (int x = 0; x < cols; ++x) {
+    float v;
+    if ((flags & ORC_GRAD_IGNORE) && ignored) {
+      v = 0.0f;
+    } else if (x == k) {
+      v = s[x * sstep] - 1.0f;
+      if (flags & ORC_GRAD_SMOOTH) v = v + alpha;
+    } else {
+      v = s[x * sstep];
+      if (flags & ORC_GRAD_SMOOTH) v = v - smooth_grad;
+    }
+    o[x * ostep] = v;
+  }
+}
+
+void orc_softmax_grad_ex_f32(float *dst, int dstride, const float *src, int sstride,
+                             const float *label, int rows, int cols, int flags,
+                             float ignore_label, float alpha) {
+  const float smooth_grad = alpha / (float)(cols - 1);
+#pragma omp parallel for
+  for (int y = 0; y < rows; ++y) {
+    const int k = (int)label[y];
+    grad_row(dst + (int64_t)y * dstride, 1, src + (int64_t)y * sstride, 1, cols, k, flags,
+             (int)ignore_label == k, alpha, smooth_grad);
+  }
+}
+
+/* Softmax on 3-D tensors, mshadow/tensor_cpu-inl.h:474-495: over the middle dimension,
+   max by strict <, exp, sequential sum, true division */
+void orc_softmax3d_f32(float *dst, int dstride, const float *src, int sstride, int d0, int d1,
+                       int d2) {
+#pragma omp parallel for
+  for (int y = 0; y < d0; ++y) {
+    for (int n = 0; n < d2; ++n) {
+      const float *s = src + (int64_t)y * d1 * sstride + n;
+      float *o = dst + (int64_t)y * d1 * dstride + n;
+      float mmax = s[0];
+      for (int x = 1; x < d1; ++x) {
+        if (mmax < s[(int64_t)x * sstride]) mmax = s[(int64_t)x * sstride];
+      }
+      float sum = 0.0f;
+      for (int x = 0; x < d1; ++x) {
+        o[(int64_t)x * dstride] = expf(s[(int64_t)x * sstride] - mmax);
+        sum += o[(int64_t)x * dstride];
+      }
+      for (int x = 0; x < d1; ++x) o[(int64_t)x * dstride] /= sum;
+    }
+  }
+}
+
+/* the four 3-D gradient functions, mshadow/tensor_cpu-inl.h:364-462 */
+void orc_softmax3d_grad_f32(float *dst, int dstride, const float *src, int sstride,
+                            const float *label, int lstride, int d0, int d1, int d2, int flags,
+                            float ignore_label, float alpha) {
+  const float smooth_grad = alpha / (float)(d1 - 1);
+#pragma omp parallel for
+  for (int n = 0; n < d2; ++n) {
+    for (int y = 0; y < d0; ++y) {
+      const int k = (int)label[(int64_t)y * lstride + n];
+      grad_row(dst + (int64_t)y * d1 * dstride + n, dstride, src + (int64_t)y * d1 * sstride + n,
+               sstride, d1, k, flags, k == (int)ignore_label, alpha, smooth_grad);
+    }
+  }
+}
+
+static inline int index_at(const void *index, int is_int, int y) {
+  return is_int ? ((const int32_t *)index)[y] : (int)((const float *)index)[y];
+}
+
+/* AddTakeGrad, mshadow/tensor_cpu-inl.h:497-508: indices clamped into [0, K), rows added
+   one after the other in index order */
+void orc_add_take_grad_f32(float *dst, int dstride, int k_rows, const void *index,
+                           int index_is_int, int n_index, const float *src, int sstride,
+                           int cols) {
+  for (int y = 0; y < n_index; ++y) {
+    int j = index_at(index, index_is_int, y);
+    if (j <= 0) j = 0;
+    else if (j >= k_rows) j = k_rows - 1;
+    for (int x = 0; x < cols; ++x) dst[(int64_t)j * dstride + x] += src[(int64_t)y * sstride + x];
+  }
+}
+
+/* AddTakeGradLargeBatch, mshadow/tensor_cpu-inl.h:510-518 */
+void orc_add_take_grad_large_batch_f32(float *dst, int dstride, const void *sorted,
+                                       const void *index, int index_is_int, int n_index,
+                                       const float *src, int sstride, int cols) {
+  for (int y = 0; y < n_index; ++y) {
+    const int j = index_at(sorted, index_is_int, y);
+    const int i = index_at(index, index_is_int, y);
+    for (int x = 0; x < cols; ++x) dst[(int64_t)j * dstride + x] += src[(int64_t)i * sstride + x];
+  }
+}
+
+/* IndexFill, mshadow/tensor_cpu-inl.h:520-528: a later entry of the index overwrites an
+   earlier one that names the same row */
+void orc_index_fill_f32(float *dst, int dstride, const void *index, int index_is_int,
+                        int n_index, const float *src, int sstride, int cols) {
+  for (int y = 0; y < n_index; ++y) {
+    const int j = index_at(index, index_is_int, y);
+    for (int x = 0; x < cols; ++x) dst[(int64_t)j * dstride + x] = src[(int64_t)y * sstride + x];
+  }
+}
+
 /* ------------------------------------------------------------------ pool / unpool */
 
 static inline int imin(int a, int b) { return a < b ? a : b; }

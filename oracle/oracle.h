@@ -55,6 +55,30 @@ void orc_softmax_f32(float *dst, int dstride, const float *src, int sstride, int
 void orc_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride,
                           const float *label, int rows, int cols);
 
+/* The rest of the softmax family and the row scatter / gather functions
+   (mshadow/tensor_cpu-inl.h:304-528). `flags`: bit 0 = smooth (alpha used), bit 1 = the
+   ignore_label argument is used. 3-D tensors are (d0, d1, d2) with the softmax over d1
+   and a row pitch on d2; their label is (d0, d2) with pitch lstride. */
+#define ORC_GRAD_SMOOTH 1
+#define ORC_GRAD_IGNORE 2
+void orc_softmax_grad_ex_f32(float *dst, int dstride, const float *src, int sstride,
+                             const float *label, int rows, int cols, int flags,
+                             float ignore_label, float alpha);
+void orc_softmax3d_f32(float *dst, int dstride, const float *src, int sstride, int d0, int d1,
+                       int d2);
+void orc_softmax3d_grad_f32(float *dst, int dstride, const float *src, int sstride,
+                            const float *label, int lstride, int d0, int d1, int d2, int flags,
+                            float ignore_label, float alpha);
+/* index_is_int: the index array holds int32 (else float, truncated like a label) */
+void orc_add_take_grad_f32(float *dst, int dstride, int k_rows, const void *index,
+                           int index_is_int, int n_index, const float *src, int sstride,
+                           int cols);
+void orc_add_take_grad_large_batch_f32(float *dst, int dstride, const void *sorted,
+                                       const void *index, int index_is_int, int n_index,
+                                       const float *src, int sstride, int cols);
+void orc_index_fill_f32(float *dst, int dstride, const void *index, int index_is_int,
+                        int n_index, const float *src, int sstride, int cols);
+
 void orc_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes, int h, int w,
                   int ph, int pw, int ky, int kx, int sy, int sx, int reducer);
 void orc_unpool_f32(float *dst, int dstride, const float *src, int sstride, const float *pooled,

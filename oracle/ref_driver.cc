@@ -131,6 +131,78 @@ void ref_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride
   SoftmaxGrad(T2(dst, rows, cols, dstride), T2(src, rows, cols, sstride), T1(label, rows));
 }
 
+void ref_softmax_grad_ex_f32(float *dst, int dstride, const float *src, int sstride,
+                             const float *label, int rows, int cols, int flags,
+                             float ignore_label, float alpha) {
+  Tensor<cpu, 2, float> D = T2(dst, rows, cols, dstride), S = T2(src, rows, cols, sstride);
+  Tensor<cpu, 1, float> L = T1(label, rows);
+  switch (flags) {
+    case 0: SoftmaxGrad(D, S, L); break;
+    case 1: SmoothSoftmaxGrad(D, S, L, alpha); break;
+    case 2: SoftmaxGrad(D, S, L, ignore_label); break;
+    default: SmoothSoftmaxGrad(D, S, L, ignore_label, alpha); break;
+  }
+}
+
+static Tensor<cpu, 3, float> T3s(const float *p, int d0, int d1, int d2, int stride) {
+  Tensor<cpu, 3, float> t(const_cast<float *>(p), Shape3(d0, d1, d2));
+  t.stride_ = stride;
+  return t;
+}
+
+void ref_softmax3d_f32(float *dst, int dstride, const float *src, int sstride, int d0, int d1,
+                       int d2) {
+  Softmax(T3s(dst, d0, d1, d2, dstride), T3s(src, d0, d1, d2, sstride));
+}
+
+void ref_softmax3d_grad_f32(float *dst, int dstride, const float *src, int sstride,
+                            const float *label, int lstride, int d0, int d1, int d2, int flags,
+                            float ignore_label, float alpha) {
+  Tensor<cpu, 3, float> D = T3s(dst, d0, d1, d2, dstride), S = T3s(src, d0, d1, d2, sstride);
+  Tensor<cpu, 2, float> L = T2(label, d0, d2, lstride);
+  switch (flags) {
+    case 0: SoftmaxGrad(D, S, L); break;
+    case 1: SmoothSoftmaxGrad(D, S, L, alpha); break;
+    case 2: SoftmaxGrad(D, S, L, ignore_label); break;
+    default: SmoothSoftmaxGrad(D, S, L, ignore_label, alpha); break;
+  }
+}
+
+void ref_add_take_grad_f32(float *dst, int dstride, int k_rows, const void *index,
+                           int index_is_int, int n_index, const float *src, int sstride,
+                           int cols) {
+  Tensor<cpu, 2, float> D = T2(dst, k_rows, cols, dstride), S = T2(src, n_index, cols, sstride);
+  if (index_is_int) {
+    AddTakeGrad(D, Tensor<cpu, 1, int>(const_cast<int *>(static_cast<const int *>(index)), Shape1(n_index)), S);
+  } else {
+    AddTakeGrad(D, T1(static_cast<const float *>(index), n_index), S);
+  }
+}
+
+void ref_add_take_grad_large_batch_f32(float *dst, int dstride, const void *sorted,
+                                       const void *index, int index_is_int, int n_index,
+                                       const float *src, int sstride, int cols) {
+  /* the row counts of dst and src are not used by the reference beyond the indices */
+  Tensor<cpu, 2, float> D = T2(dst, 1 << 30, cols, dstride), S = T2(src, 1 << 30, cols, sstride);
+  if (index_is_int) {
+    AddTakeGradLargeBatch(D, Tensor<cpu, 1, int>(const_cast<int *>(static_cast<const int *>(sorted)), Shape1(n_index)),
+                          Tensor<cpu, 1, int>(const_cast<int *>(static_cast<const int *>(index)), Shape1(n_index)), S);
+  } else {
+    AddTakeGradLargeBatch(D, T1(static_cast<const float *>(sorted), n_index),
+                          T1(static_cast<const float *>(index), n_index), S);
+  }
+}
+
+void ref_index_fill_f32(float *dst, int dstride, const void *index, int index_is_int,
+                        int n_index, const float *src, int sstride, int cols) {
+  Tensor<cpu, 2, float> D = T2(dst, 1 << 30, cols, dstride), S = T2(src, n_index, cols, sstride);
+  if (index_is_int) {
+    IndexFill(D, Tensor<cpu, 1, int>(const_cast<int *>(static_cast<const int *>(index)), Shape1(n_index)), S);
+  } else {
+    IndexFill(D, T1(static_cast<const float *>(index), n_index), S);
+  }
+}
+
 void ref_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes, int h, int w,
                   int ph, int pw, int ky, int kx, int sy, int sx, int reducer) {
   Tensor<cpu, 3, float> S = T3(src, planes, h, w, sstride);

@@ -17,6 +17,7 @@ REF_SO = os.path.join(ROOT, "oracle", "_ref", "libmshadow_ref.so")
 
 SAVETO, PLUSTO, MINUSTO, MULTO, DIVTO = range(5)
 SUM, MAX, MIN = range(3)
+GRAD_SMOOTH, GRAD_IGNORE = 1, 2
 
 _i = C.c_int
 _f = C.c_float
@@ -76,6 +77,12 @@ class Checker:
         self._fn("reduce_keep_highdim_f32", [_p, _p, _i, _i, _i, _i, _i, _i, _i, _f])
         self._fn("softmax_f32", [_p, _i, _p, _i, _i, _i])
         self._fn("softmax_grad_f32", [_p, _i, _p, _i, _p, _i, _i])
+        self._fn("softmax_grad_ex_f32", [_p, _i, _p, _i, _p, _i, _i, _i, _f, _f])
+        self._fn("softmax3d_f32", [_p, _i, _p, _i, _i, _i, _i])
+        self._fn("softmax3d_grad_f32", [_p, _i, _p, _i, _p, _i, _i, _i, _i, _i, _f, _f])
+        self._fn("add_take_grad_f32", [_p, _i, _i, _p, _i, _i, _p, _i, _i])
+        self._fn("add_take_grad_large_batch_f32", [_p, _i, _p, _p, _i, _i, _p, _i, _i])
+        self._fn("index_fill_f32", [_p, _i, _p, _i, _i, _p, _i, _i])
         self._fn("pool_f32", [_p, _i, _p, _i] + [_i] * 10)
         self._fn("unpool_f32", [_p, _i, _p, _i, _p, _i, _p, _i] + [_i] * 10)
         for t in ("f16", "f32"):
@@ -140,6 +147,46 @@ class Checker:
         rows, cols = src.shape
         assert label.dtype == np.float32 and label.shape == (rows,)
         self._softmax_grad_f32(ptr(dst), pitch(dst), ptr(src), pitch(src), ptr(label), rows, cols)
+        return dst
+
+    def softmax_grad_ex(self, dst, src, label, flags, ignore_label=0.0, alpha=0.0):
+        rows, cols = src.shape
+        self._softmax_grad_ex_f32(ptr(dst), pitch(dst), ptr(src), pitch(src), ptr(label), rows,
+                                  cols, flags, ignore_label, alpha)
+        return dst
+
+    def softmax3d(self, dst, src):
+        d0, d1, d2 = src.shape
+        self._softmax3d_f32(ptr(dst), pitch(dst), ptr(src), pitch(src), d0, d1, d2)
+        return dst
+
+    def softmax3d_grad(self, dst, src, label, flags, ignore_label=0.0, alpha=0.0):
+        d0, d1, d2 = src.shape
+        assert label.shape == (d0, d2)
+        self._softmax3d_grad_f32(ptr(dst), pitch(dst), ptr(src), pitch(src), ptr(label),
+                                 pitch(label), d0, d1, d2, flags, ignore_label, alpha)
+        return dst
+
+    @staticmethod
+    def _is_int(index):
+        assert index.dtype in (np.int32, np.float32)
+        return 1 if index.dtype == np.int32 else 0
+
+    def add_take_grad(self, dst, index, src):
+        self._add_take_grad_f32(ptr(dst), pitch(dst), dst.shape[0], ptr(index), self._is_int(index),
+                                index.shape[0], ptr(src), pitch(src), src.shape[1])
+        return dst
+
+    def add_take_grad_large_batch(self, dst, sorted_rows, index, src):
+        assert sorted_rows.dtype == index.dtype
+        self._add_take_grad_large_batch_f32(ptr(dst), pitch(dst), ptr(sorted_rows), ptr(index),
+                                            self._is_int(index), index.shape[0], ptr(src),
+                                            pitch(src), src.shape[1])
+        return dst
+
+    def index_fill(self, dst, index, src):
+        self._index_fill_f32(ptr(dst), pitch(dst), ptr(index), self._is_int(index),
+                             index.shape[0], ptr(src), pitch(src), src.shape[1])
         return dst
 
     # -- pool / unpool: arrays are (..., H, W); leading dims are planes
