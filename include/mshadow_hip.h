@@ -142,6 +142,46 @@ int mshadow_hip_softmax_rowsum_f32(float *sums, const float *terms, int tstride,
 int mshadow_hip_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride,
                                  const float *label, int rows, int cols, void *stream);
 
+/* The gradient family in one entry: SoftmaxGrad with ignore_label and SmoothSoftmaxGrad with
+   and without it, mshadow/tensor_gpu-inl.h:176-199 -> tensor_gpu-inl.cuh:258-328, 414-477
+   (CPU definitions tensor_cpu-inl.h:304-362). flags: MSHADOW_HIP_GRAD_SMOOTH uses alpha
+   (label entry: src - 1 + alpha, others: src - alpha / (cols - 1)); MSHADOW_HIP_GRAD_IGNORE
+   zeroes the rows whose label equals ignore_label (both truncated to int). flags = 0 is
+   mshadow_hip_softmax_grad_f32. */
+#define MSHADOW_HIP_GRAD_SMOOTH 1
+#define MSHADOW_HIP_GRAD_IGNORE 2
+int mshadow_hip_softmax_grad_ex_f32(float *dst, int dstride, const float *src, int sstride,
+                                    const float *label, int rows, int cols, int flags,
+                                    float ignore_label, float alpha, void *stream);
+/* Softmax on 3-D tensors (d0, d1, d2), over the middle dimension, row pitch on d2:
+   mshadow/tensor_gpu-inl.h:163-167 -> tensor_gpu-inl.cuh:479-524 (CPU tensor_cpu-inl.h:474-495). */
+int mshadow_hip_softmax3d_f32(float *dst, int dstride, const float *src, int sstride, int d0,
+                              int d1, int d2, void *stream);
+/* SoftmaxGrad / SmoothSoftmaxGrad on 3-D tensors, label (d0, d2) with pitch lstride:
+   mshadow/tensor_gpu-inl.h:201-214 -> tensor_gpu-inl.cuh:526-597 (CPU tensor_cpu-inl.h:364-462). */
+int mshadow_hip_softmax3d_grad_f32(float *dst, int dstride, const float *src, int sstride,
+                                   const float *label, int lstride, int d0, int d1, int d2,
+                                   int flags, float ignore_label, float alpha, void *stream);
+/* AddTakeGrad(dst, index, src): dst[clamp(index[y], 0, k_rows - 1)] += src[y] for y in order
+   (mshadow/tensor_gpu-inl.h:216-222 -> tensor_gpu-inl.cuh:599-672; CPU tensor_cpu-inl.h:497-508).
+   index holds n_index entries of int32 (index_is_int != 0) or float. Rows that are named
+   several times receive their additions in index order, as on the CPU. */
+int mshadow_hip_add_take_grad_f32(float *dst, int dstride, int k_rows, const void *index,
+                                  int index_is_int, int n_index, const float *src, int sstride,
+                                  int cols, void *stream);
+/* AddTakeGradLargeBatch(dst, sorted, index, src): dst[sorted[y]] += src[index[y]] for y in
+   order (mshadow/tensor_gpu-inl.h:224-232 -> tensor_gpu-inl.cuh:674-760; CPU
+   tensor_cpu-inl.h:510-518). Needs no workspace here. */
+int mshadow_hip_add_take_grad_large_batch_f32(float *dst, int dstride, int k_rows,
+                                              const void *sorted, const void *index,
+                                              int index_is_int, int n_index, const float *src,
+                                              int sstride, int cols, void *stream);
+/* IndexFill(dst, index, src): dst[index[y]] = src[y]; the last entry naming a row counts
+   (mshadow/tensor_gpu-inl.h:234-240 -> tensor_gpu-inl.cuh:762-782; CPU tensor_cpu-inl.h:520-528). */
+int mshadow_hip_index_fill_f32(float *dst, int dstride, int k_rows, const void *index,
+                               int index_is_int, int n_index, const float *src, int sstride,
+                               int cols, void *stream);
+
 /* MapReduceKeepLowest<Saver, Reducer>(dst, src, scale): mshadow/tensor_gpu-inl.h:118-133
    -> MapRedKeepLowestKernel, tensor_gpu-inl.cuh:122-168. dst[x] <saver>= scale *
    reduce_y src[y][x], rows >= 1, reduced top to bottom like tensor_cpu-inl.h:221-227. */

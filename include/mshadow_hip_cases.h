@@ -51,6 +51,22 @@ int mshadow_case_softmax_f32(float *dst, int dstride, const float *src, int sstr
 int mshadow_case_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride,
                                   const float *label, int rows, int cols, void *stream);
 
+/* SoftmaxGrad / SmoothSoftmaxGrad with and without ignore_label, on 2-D tensors (d0 == 0:
+   rows x cols, label of `rows` floats) or 3-D tensors (d0, d1, d2; label (d0, d2) with
+   pitch lstride); flags as MSHADOW_HIP_GRAD_* */
+int mshadow_case_grad_family_f32(float *dst, int dstride, const float *src, int sstride,
+                                 const float *label, int lstride, int d0, int rows_or_d1,
+                                 int cols_or_d2, int flags, float ignore_label, float alpha,
+                                 void *stream);
+/* Softmax(dst, src) on 3-D tensors */
+int mshadow_case_softmax3d_f32(float *dst, int dstride, const float *src, int sstride, int d0,
+                               int d1, int d2, void *stream);
+/* op 0: AddTakeGrad(dst, index, src); 1: AddTakeGradLargeBatch(dst, sorted, index, src);
+   2: IndexFill(dst, index, src); int32 index vectors */
+int mshadow_case_rows_by_index_f32(int op, float *dst, int dstride, int k_rows, const int *sorted,
+                                   const int *index, int n_index, const float *src, int sstride,
+                                   int src_rows, int cols, void *stream);
+
 /* dst = pool<Reducer>(src, Shape2(ph, pw), ky, kx, sy, sx) */
 int mshadow_case_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes,
                           int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,

@@ -63,6 +63,12 @@ HIP_SYMBOLS = {
     "mshadow_hip_suggest_grid": ([_sz, _sz, _i, C.POINTER(C.c_uint32)], _i),
     "mshadow_hip_softmax_f32": ([_p, _i, _p, _i, _i, _i, _p], _i),
     "mshadow_hip_softmax_rowsum_f32": ([_p, _p, _i, _i, _i, _p], _i),
+    "mshadow_hip_softmax_grad_ex_f32": ([_p, _i, _p, _i, _p, _i, _i, _i, _f, _f, _p], _i),
+    "mshadow_hip_softmax3d_f32": ([_p, _i, _p, _i, _i, _i, _i, _p], _i),
+    "mshadow_hip_softmax3d_grad_f32": ([_p, _i, _p, _i, _p, _i, _i, _i, _i, _i, _f, _f, _p], _i),
+    "mshadow_hip_add_take_grad_f32": ([_p, _i, _i, _p, _i, _i, _p, _i, _i, _p], _i),
+    "mshadow_hip_add_take_grad_large_batch_f32": ([_p, _i, _i, _p, _p, _i, _i, _p, _i, _i, _p], _i),
+    "mshadow_hip_index_fill_f32": ([_p, _i, _i, _p, _i, _i, _p, _i, _i, _p], _i),
     "mshadow_hip_softmax_grad_f32": ([_p, _i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_hip_reduce_keep_lowest_f32": ([_p, _p, _i, _i, _i, _i, _i, _f, _p], _i),
     "mshadow_hip_reduce_keep_highdim_f32": ([_p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p], _i),
@@ -82,6 +88,9 @@ CASES_SYMBOLS = {
     "mshadow_case_reduce_keep_lowest_f32": ([_p, _p, _i, _i, _i, _i, _i, _f, _i, _p], _i),
     "mshadow_case_reduce_keep_highdim_f32": ([_p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _i, _p], _i),
     "mshadow_case_softmax_f32": ([_p, _i, _p, _i, _i, _i, _p], _i),
+    "mshadow_case_grad_family_f32": ([_p, _i, _p, _i, _p, _i, _i, _i, _i, _i, _f, _f, _p], _i),
+    "mshadow_case_softmax3d_f32": ([_p, _i, _p, _i, _i, _i, _i, _p], _i),
+    "mshadow_case_rows_by_index_f32": ([_i, _p, _i, _i, _p, _p, _i, _p, _i, _i, _i, _p], _i),
     "mshadow_case_softmax_grad_f32": ([_p, _i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_case_pool_f32": ([_p, _i, _p, _i] + [_i] * 11 + [_p], _i),
     "mshadow_case_unpool_f32": ([_p, _i, _p, _i, _p, _i, _p, _i] + [_i] * 11 + [_p], _i),
@@ -242,6 +251,42 @@ class Library:
         self.check(self.dll.mshadow_hip_softmax_rowsum_f32(sums.ptr, terms.ptr, terms.stride,
                                                            terms.rows, terms.cols, stream))
 
+    def softmax_grad_ex(self, dst, src, label, flags, ignore_label=0.0, alpha=0.0, stream=None):
+        self.check(self.dll.mshadow_hip_softmax_grad_ex_f32(
+            dst.ptr, dst.stride, src.ptr, src.stride, label.ptr, src.rows, src.cols, flags,
+            ignore_label, alpha, stream))
+
+    def softmax3d(self, dst, src, stream=None):
+        d0, d1, d2 = src.shape
+        self.check(self.dll.mshadow_hip_softmax3d_f32(dst.ptr, dst.stride, src.ptr, src.stride,
+                                                      d0, d1, d2, stream))
+
+    def softmax3d_grad(self, dst, src, label, flags, ignore_label=0.0, alpha=0.0, stream=None):
+        d0, d1, d2 = src.shape
+        self.check(self.dll.mshadow_hip_softmax3d_grad_f32(
+            dst.ptr, dst.stride, src.ptr, src.stride, label.ptr, label.stride, d0, d1, d2, flags,
+            ignore_label, alpha, stream))
+
+    @staticmethod
+    def _index_is_int(index):
+        assert index.dtype in (np.dtype(np.int32), np.dtype(np.float32))
+        return 1 if index.dtype == np.dtype(np.int32) else 0
+
+    def add_take_grad(self, dst, index, src, stream=None):
+        self.check(self.dll.mshadow_hip_add_take_grad_f32(
+            dst.ptr, dst.stride, dst.rows, index.ptr, self._index_is_int(index), index.cols,
+            src.ptr, src.stride, src.cols, stream))
+
+    def add_take_grad_large_batch(self, dst, sorted_rows, index, src, stream=None):
+        self.check(self.dll.mshadow_hip_add_take_grad_large_batch_f32(
+            dst.ptr, dst.stride, dst.rows, sorted_rows.ptr, index.ptr, self._index_is_int(index),
+            index.cols, src.ptr, src.stride, src.cols, stream))
+
+    def index_fill(self, dst, index, src, stream=None):
+        self.check(self.dll.mshadow_hip_index_fill_f32(
+            dst.ptr, dst.stride, dst.rows, index.ptr, self._index_is_int(index), index.cols,
+            src.ptr, src.stride, src.cols, stream))
+
     def softmax_grad(self, dst, src, label, stream=None):
         self.check(self.dll.mshadow_hip_softmax_grad_f32(dst.ptr, dst.stride, src.ptr, src.stride,
                                                          label.ptr, src.rows, src.cols, stream))
@@ -297,6 +342,25 @@ class Library:
     def case_map_axpb(self, dst, a, s1, s2, s3, saver=SAVETO, stream=None):
         self.check_case(self.cases.mshadow_case_map_axpb_f32(
             dst.ptr, dst.stride, a.ptr, a.stride, dst.rows, dst.cols, s1, s2, s3, saver, stream))
+
+    def case_grad_family(self, dst, src, label, flags, ignore_label=0.0, alpha=0.0, stream=None):
+        if len(src.shape) == 2:
+            d0, a, b = 0, src.rows, src.cols
+        else:
+            d0, a, b = src.shape
+        self.check_case(self.cases.mshadow_case_grad_family_f32(
+            dst.ptr, dst.stride, src.ptr, src.stride, label.ptr, label.stride, d0, a, b, flags,
+            ignore_label, alpha, stream))
+
+    def case_softmax3d(self, dst, src, stream=None):
+        d0, d1, d2 = src.shape
+        self.check_case(self.cases.mshadow_case_softmax3d_f32(dst.ptr, dst.stride, src.ptr,
+                                                              src.stride, d0, d1, d2, stream))
+
+    def case_rows_by_index(self, op, dst, sorted_rows, index, src, stream=None):
+        self.check_case(self.cases.mshadow_case_rows_by_index_f32(
+            op, dst.ptr, dst.stride, dst.rows, sorted_rows.ptr if sorted_rows is not None else None,
+            index.ptr, index.cols, src.ptr, src.stride, src.rows, src.cols, stream))
 
     def case_reduce_keep_lowest(self, dst, src, reducer=SUM, saver=SAVETO, scale=1.0, variant=0,
                                 stream=None):

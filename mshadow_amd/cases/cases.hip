@@ -168,6 +168,69 @@ int mshadow_case_softmax_grad_f32(float *dst, int dstride, const float *src, int
   CASE_END
 }
 
+/* the gradient family and the 3-D softmax through the C++ functions; flags as in
+   mshadow_hip.h (bit 0 smooth, bit 1 ignore_label); d0 == 0 selects the 2-D functions */
+int mshadow_case_grad_family_f32(float *dst, int dstride, const float *src, int sstride,
+                                 const float *label, int lstride, int d0, int rows_or_d1,
+                                 int cols_or_d2, int flags, float ignore_label, float alpha,
+                                 void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  if (d0 == 0) {
+    const int rows = rows_or_d1, cols = cols_or_d2;
+    Tensor<gpu, 2, float> D = G2(dst, rows, cols, dstride, st.get());
+    Tensor<gpu, 2, float> S = G2(src, rows, cols, sstride, st.get());
+    Tensor<gpu, 1, float> L = G1(label, rows, st.get());
+    switch (flags) {
+      case 0: SoftmaxGrad(D, S, L); break;
+      case 1: SmoothSoftmaxGrad(D, S, L, alpha); break;
+      case 2: SoftmaxGrad(D, S, L, ignore_label); break;
+      default: SmoothSoftmaxGrad(D, S, L, ignore_label, alpha); break;
+    }
+  } else {
+    const int d1 = rows_or_d1, d2 = cols_or_d2;
+    Tensor<gpu, 3, float> D = G3(dst, d0, d1, d2, dstride, st.get());
+    Tensor<gpu, 3, float> S = G3(src, d0, d1, d2, sstride, st.get());
+    Tensor<gpu, 2, float> L = G2(label, d0, d2, lstride, st.get());
+    switch (flags) {
+      case 0: SoftmaxGrad(D, S, L); break;
+      case 1: SmoothSoftmaxGrad(D, S, L, alpha); break;
+      case 2: SoftmaxGrad(D, S, L, ignore_label); break;
+      default: SmoothSoftmaxGrad(D, S, L, ignore_label, alpha); break;
+    }
+  }
+  CASE_END
+}
+
+int mshadow_case_softmax3d_f32(float *dst, int dstride, const float *src, int sstride, int d0,
+                               int d1, int d2, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Softmax(G3(dst, d0, d1, d2, dstride, st.get()), G3(src, d0, d1, d2, sstride, st.get()));
+  CASE_END
+}
+
+/* op: 0 AddTakeGrad(dst, index, src), 1 AddTakeGradLargeBatch(dst, sorted, index, src),
+   2 IndexFill(dst, index, src); int32 index vectors */
+int mshadow_case_rows_by_index_f32(int op, float *dst, int dstride, int k_rows, const int *sorted,
+                                   const int *index, int n_index, const float *src, int sstride,
+                                   int src_rows, int cols, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Tensor<gpu, 2, float> D = G2(dst, k_rows, cols, dstride, st.get());
+  Tensor<gpu, 2, float> S = G2(src, src_rows, cols, sstride, st.get());
+  Tensor<gpu, 1, int> I(const_cast<int *>(index), Shape1(n_index), st.get());
+  if (op == 0) {
+    AddTakeGrad(D, I, S);
+  } else if (op == 1) {
+    Tensor<gpu, 1, int> Srt(const_cast<int *>(sorted), Shape1(n_index), st.get());
+    AddTakeGradLargeBatch(D, Srt, I, S);
+  } else {
+    IndexFill(D, I, S);
+  }
+  CASE_END
+}
+
 int mshadow_case_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes,
                           int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,
                           int reducer, int variant, void *stream) {

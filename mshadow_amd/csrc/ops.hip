@@ -11,6 +11,7 @@
 
 #include "patch_kernels.h"
 #include "pool_kernels.h"
+#include "row_kernels.h"
 #include "softmax_kernels.h"
 
 using namespace mshadow_abi;
@@ -242,6 +243,25 @@ void LaunchUnpoolGeneric(int reducer, const UnpoolArgs &a) {
 #undef UNPOOL_ARGS
 
 
+struct GradLaunch {
+  float *dst; int dstride; const float *src; int sstride; const float *label; int cols;
+  unsigned chunks; GradParams gp; unsigned blocks; hipStream_t s;
+};
+template <bool VEC>
+void LaunchGrad(int flags, const GradLaunch &g) {
+#define GRAD2D(FLAGS)                                                                         \
+  hipLaunchKernelGGL((SoftmaxGradKernel<VEC, FLAGS>), dim3(g.blocks), dim3(kGradBlock), 0, g.s, \
+                     g.dst, g.dstride, g.src, g.sstride, g.label, g.cols, g.chunks, g.gp)
+  switch (flags) {
+    case 0: GRAD2D(0); break;
+    case 1: GRAD2D(1); break;
+    case 2: GRAD2D(2); break;
+    default: GRAD2D(3); break;
+  }
+#undef GRAD2D
+}
+
+
 }  // namespace
 
 
@@ -315,9 +335,11 @@ int mshadow_hip_softmax_rowsum_f32(float *sums, const float *terms, int tstride,
   return AfterLaunch("softmax_rowsum");
 }
 
-int mshadow_hip_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride,
-                                 const float *label, int rows, int cols, void *stream) {
+int mshadow_hip_softmax_grad_ex_f32(float *dst, int dstride, const float *src, int sstride,
+                                    const float *label, int rows, int cols, int flags,
+                                    float ignore_label, float alpha, void *stream) {
   ABI_REQUIRE(rows >= 0 && cols >= 0, "negative shape");
+  ABI_REQUIRE(flags >= 0 && flags <= 3, "unknown gradient flags");
   if (rows == 0 || cols == 0) return MSHADOW_HIP_OK;
   ABI_REQUIRE(dst != NULL && src != NULL && label != NULL, "NULL tensor");
   ABI_REQUIRE(dstride >= cols && sstride >= cols, "pitch smaller than the row");
@@ -326,16 +348,126 @@ int mshadow_hip_softmax_grad_f32(float *dst, int dstride, const float *src, int 
   const unsigned long long blocks = static_cast<unsigned long long>(rows) * chunks;
   ABI_REQUIRE(blocks < (1ull << 31), "too many workgroups");
   const bool vec = Aligned16(dst) && Aligned16(src) && dstride % 4 == 0 && sstride % 4 == 0;
-  if (vec) {
-    hipLaunchKernelGGL((SoftmaxGradKernel<true>), dim3(static_cast<unsigned>(blocks)),
-                       dim3(kGradBlock), 0, AsStream(stream), dst, dstride, src, sstride, label,
-                       cols, chunks);
-  } else {
-    hipLaunchKernelGGL((SoftmaxGradKernel<false>), dim3(static_cast<unsigned>(blocks)),
-                       dim3(kGradBlock), 0, AsStream(stream), dst, dstride, src, sstride, label,
-                       cols, chunks);
-  }
+  /* alpha / (classes - 1) with the count converted from unsigned, as the reference writes it */
+  const GradParams gp = {static_cast<int>(ignore_label), alpha,
+                         alpha / static_cast<float>(static_cast<unsigned>(cols - 1))};
+  GradLaunch gl = {dst, dstride, src, sstride, label, cols, chunks, gp,
+                   static_cast<unsigned>(blocks), AsStream(stream)};
+  if (vec) LaunchGrad<true>(flags, gl);
+  else LaunchGrad<false>(flags, gl);
   return AfterLaunch("softmax_grad");
+}
+
+int mshadow_hip_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride,
+                                 const float *label, int rows, int cols, void *stream) {
+  return mshadow_hip_softmax_grad_ex_f32(dst, dstride, src, sstride, label, rows, cols, 0, 0.0f,
+                                         0.0f, stream);
+}
+
+int mshadow_hip_softmax3d_f32(float *dst, int dstride, const float *src, int sstride, int d0,
+                              int d1, int d2, void *stream) {
+  ABI_REQUIRE(d0 >= 0 && d1 >= 0 && d2 >= 0, "negative shape");
+  if (d0 == 0 || d1 == 0 || d2 == 0) return MSHADOW_HIP_OK;
+  ABI_REQUIRE(dst != NULL && src != NULL, "NULL tensor");
+  ABI_REQUIRE(dstride >= d2 && sstride >= d2, "pitch smaller than the row");
+  ABI_REQUIRE(static_cast<long long>(d0) * d2 < (1ll << 31) &&
+                  static_cast<long long>(d0) * d1 < (1ll << 31),
+              "too large for 32-bit indices");
+  unsigned grid = 0;
+  int st = mshadow_hip_suggest_grid(static_cast<size_t>(d0) * d2, kSoftmax3dBlock, 8, &grid);
+  if (st != MSHADOW_HIP_OK) return st;
+  hipLaunchKernelGGL(Softmax3dKernel, dim3(grid), dim3(kSoftmax3dBlock), 0, AsStream(stream), dst,
+                     dstride, src, sstride, d0, d1, d2,
+                     mshadow::FastDivU32(static_cast<uint32_t>(d2)));
+  return AfterLaunch("softmax3d");
+}
+
+int mshadow_hip_softmax3d_grad_f32(float *dst, int dstride, const float *src, int sstride,
+                                   const float *label, int lstride, int d0, int d1, int d2,
+                                   int flags, float ignore_label, float alpha, void *stream) {
+  ABI_REQUIRE(d0 >= 0 && d1 >= 0 && d2 >= 0, "negative shape");
+  ABI_REQUIRE(flags >= 0 && flags <= 3, "unknown gradient flags");
+  if (d0 == 0 || d1 == 0 || d2 == 0) return MSHADOW_HIP_OK;
+  ABI_REQUIRE(dst != NULL && src != NULL && label != NULL, "NULL tensor");
+  ABI_REQUIRE(dstride >= d2 && sstride >= d2 && lstride >= d2, "pitch smaller than the row");
+  ABI_REQUIRE(static_cast<long long>(d0) * d1 * d2 < (1ll << 31), "too large for 32-bit indices");
+  unsigned grid = 0;
+  int st = mshadow_hip_suggest_grid(static_cast<size_t>(d0) * d1 * d2, kSoftmax3dBlock, 8, &grid);
+  if (st != MSHADOW_HIP_OK) return st;
+  const GradParams gp = {static_cast<int>(ignore_label), alpha,
+                         alpha / static_cast<float>(static_cast<unsigned>(d1 - 1))};
+  const mshadow::FastDivU32 div_d2(static_cast<uint32_t>(d2)), div_d1(static_cast<uint32_t>(d1));
+#define GRAD3D(FLAGS)                                                                          \
+  hipLaunchKernelGGL((Softmax3dGradKernel<FLAGS>), dim3(grid), dim3(kSoftmax3dBlock), 0,       \
+                     AsStream(stream), dst, dstride, src, sstride, label, lstride, d0, d1, d2, \
+                     div_d2, div_d1, gp)
+  switch (flags) {
+    case 0: GRAD3D(0); break;
+    case 1: GRAD3D(1); break;
+    case 2: GRAD3D(2); break;
+    default: GRAD3D(3); break;
+  }
+#undef GRAD3D
+  return AfterLaunch("softmax3d_grad");
+}
+
+static int RowOpCheck(const float *dst, int dstride, int k_rows, const void *index, int n_index,
+                      const float *src, int sstride, int cols) {
+  ABI_REQUIRE(k_rows >= 0 && n_index >= 0 && cols >= 0, "negative shape");
+  if (k_rows == 0 || n_index == 0 || cols == 0) return -1;  // nothing to do
+  ABI_REQUIRE(dst != NULL && src != NULL && index != NULL, "NULL tensor");
+  ABI_REQUIRE(dstride >= cols && sstride >= cols, "pitch smaller than the row");
+  return MSHADOW_HIP_OK;
+}
+
+int mshadow_hip_add_take_grad_f32(float *dst, int dstride, int k_rows, const void *index,
+                                  int index_is_int, int n_index, const float *src, int sstride,
+                                  int cols, void *stream) {
+  const int chk = RowOpCheck(dst, dstride, k_rows, index, n_index, src, sstride, cols);
+  if (chk != MSHADOW_HIP_OK) return chk < 0 ? MSHADOW_HIP_OK : chk;
+  const unsigned grid = (static_cast<unsigned>(k_rows) + kRowBlock / 64 - 1) / (kRowBlock / 64);
+  if (index_is_int) {
+    hipLaunchKernelGGL((AddTakeGradKernel<true, true>), dim3(grid), dim3(kRowBlock), 0,
+                       AsStream(stream), dst, dstride, k_rows, index, index, n_index, src, sstride, cols);
+  } else {
+    hipLaunchKernelGGL((AddTakeGradKernel<false, true>), dim3(grid), dim3(kRowBlock), 0,
+                       AsStream(stream), dst, dstride, k_rows, index, index, n_index, src, sstride, cols);
+  }
+  return AfterLaunch("add_take_grad");
+}
+
+int mshadow_hip_add_take_grad_large_batch_f32(float *dst, int dstride, int k_rows,
+                                              const void *sorted, const void *index,
+                                              int index_is_int, int n_index, const float *src,
+                                              int sstride, int cols, void *stream) {
+  const int chk = RowOpCheck(dst, dstride, k_rows, index, n_index, src, sstride, cols);
+  if (chk != MSHADOW_HIP_OK) return chk < 0 ? MSHADOW_HIP_OK : chk;
+  ABI_REQUIRE(sorted != NULL, "NULL tensor");
+  const unsigned grid = (static_cast<unsigned>(k_rows) + kRowBlock / 64 - 1) / (kRowBlock / 64);
+  if (index_is_int) {
+    hipLaunchKernelGGL((AddTakeGradKernel<true, false>), dim3(grid), dim3(kRowBlock), 0,
+                       AsStream(stream), dst, dstride, k_rows, sorted, index, n_index, src, sstride, cols);
+  } else {
+    hipLaunchKernelGGL((AddTakeGradKernel<false, false>), dim3(grid), dim3(kRowBlock), 0,
+                       AsStream(stream), dst, dstride, k_rows, sorted, index, n_index, src, sstride, cols);
+  }
+  return AfterLaunch("add_take_grad_large_batch");
+}
+
+int mshadow_hip_index_fill_f32(float *dst, int dstride, int k_rows, const void *index,
+                               int index_is_int, int n_index, const float *src, int sstride,
+                               int cols, void *stream) {
+  const int chk = RowOpCheck(dst, dstride, k_rows, index, n_index, src, sstride, cols);
+  if (chk != MSHADOW_HIP_OK) return chk < 0 ? MSHADOW_HIP_OK : chk;
+  const unsigned grid = (static_cast<unsigned>(k_rows) + kRowBlock / 64 - 1) / (kRowBlock / 64);
+  if (index_is_int) {
+    hipLaunchKernelGGL((IndexFillKernel<true>), dim3(grid), dim3(kRowBlock), 0, AsStream(stream),
+                       dst, dstride, k_rows, index, n_index, src, sstride, cols);
+  } else {
+    hipLaunchKernelGGL((IndexFillKernel<false>), dim3(grid), dim3(kRowBlock), 0, AsStream(stream),
+                       dst, dstride, k_rows, index, n_index, src, sstride, cols);
+  }
+  return AfterLaunch("index_fill");
 }
 
 /* ------------------------------------------------------------------ reductions */

@@ -21,6 +21,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <mshadow/core/fastdiv.h>
 #include <mshadow/hip/kernels/common.h>
 
 #include "ordered_sum.h"
@@ -832,16 +833,42 @@ __global__ void __launch_bounds__(THREADS)
 const int kGradBlock = 256;
 const int kGradPacks = 2;  // 128-bit packs per thread
 
+/*! \brief flags of the gradient family (mshadow/tensor_cpu-inl.h:287-462) */
+const int kGradSmooth = 1;  //!< SmoothSoftmaxGrad: alpha is spread over the other classes
+const int kGradIgnore = 2;  //!< rows whose label equals ignore_label get a zero gradient
+
+struct GradParams {
+  int ignore_label;   //!< static_cast<int>(ignore_label)
+  float alpha;
+  float smooth_grad;  //!< alpha / (classes - 1), computed in float like the reference
+};
+
+/*! \brief one element of the gradient; the expressions are the reference's, in its order */
+template <int FLAGS>
+__device__ __forceinline__ float GradElement(float s, bool at_label, bool ignored, const GradParams &p) {
+  float v;
+  if (at_label) {
+    v = s - 1.0f;
+    if (FLAGS & kGradSmooth) v = v + p.alpha;
+  } else {
+    v = s;
+    if (FLAGS & kGradSmooth) v = v - p.smooth_grad;
+  }
+  if ((FLAGS & kGradIgnore) && ignored) v = 0.0f;
+  return v;
+}
+
 /*! \brief grid.x = rows * chunks, a chunk being kGradBlock * kGradPacks * 4 columns.
  *  Consecutive workgroups walk along a row, so the workgroups in flight at any moment
  *  stream one contiguous region of memory. */
-template <bool VEC4>
+template <bool VEC4, int FLAGS>
 __global__ void __launch_bounds__(kGradBlock)
     SoftmaxGradKernel(float *dst, int dstride, const float *src, int sstride, const float *label,
-                      int cols, unsigned chunks) {
+                      int cols, unsigned chunks, GradParams gp) {
   const int y = blockIdx.x / chunks;
   const int chunk = blockIdx.x - y * chunks;
   const int k = static_cast<int>(label[y]);
+  const bool ignored = (FLAGS & kGradIgnore) && k == gp.ignore_label;
   const float *in = src + static_cast<size_t>(y) * sstride;
   float *out = dst + static_cast<size_t>(y) * dstride;
   const int chunk0 = chunk * (kGradBlock * kGradPacks * 4);
@@ -856,21 +883,85 @@ __global__ void __launch_bounds__(kGradBlock)
     for (int u = 0; u < kGradPacks; ++u) {
       const int x = chunk0 + (u * kGradBlock + threadIdx.x) * 4;
       if (x + 4 <= cols) {
-        if (k == x) q[u].x = q[u].x - 1.0f;
-        if (k == x + 1) q[u].y = q[u].y - 1.0f;
-        if (k == x + 2) q[u].z = q[u].z - 1.0f;
-        if (k == x + 3) q[u].w = q[u].w - 1.0f;
+        if (FLAGS == 0) {
+          if (k == x) q[u].x = q[u].x - 1.0f;
+          if (k == x + 1) q[u].y = q[u].y - 1.0f;
+          if (k == x + 2) q[u].z = q[u].z - 1.0f;
+          if (k == x + 3) q[u].w = q[u].w - 1.0f;
+        } else {
+          q[u].x = GradElement<FLAGS>(q[u].x, k == x, ignored, gp);
+          q[u].y = GradElement<FLAGS>(q[u].y, k == x + 1, ignored, gp);
+          q[u].z = GradElement<FLAGS>(q[u].z, k == x + 2, ignored, gp);
+          q[u].w = GradElement<FLAGS>(q[u].w, k == x + 3, ignored, gp);
+        }
         StreamStoreF4(out + x, q[u]);
       } else {
-        for (int i = x; i < cols; ++i) out[i] = (i == k) ? in[i] - 1.0f : in[i];
+        for (int i = x; i < cols; ++i) out[i] = GradElement<FLAGS>(in[i], i == k, ignored, gp);
       }
     }
   } else {
 #pragma unroll
     for (int u = 0; u < kGradPacks * 4; ++u) {
       const int x = chunk0 + u * kGradBlock + threadIdx.x;
-      if (x < cols) out[x] = (x == k) ? in[x] - 1.0f : in[x];
+      if (x < cols) out[x] = GradElement<FLAGS>(in[x], x == k, ignored, gp);
     }
+  }
+}
+
+/* ---- 3-D tensors (d0, d1, d2), softmax over d1, row pitch on d2 ----------------------
+ * (mshadow/tensor_cpu-inl.h:474-495; cuda/tensor_gpu-inl.cuh:479-597). One thread per
+ * (y, n) pair, n fastest: every access of a wave is one contiguous run along d2, and the
+ * max / sum over the classes is a serial loop in the thread - the reference's own order. */
+const int kSoftmax3dBlock = 256;
+
+__global__ void __launch_bounds__(kSoftmax3dBlock)
+    Softmax3dKernel(float *dst, int dstride, const float *src, int sstride, int d0, int d1, int d2,
+                    mshadow::FastDivU32 div_d2) {
+  const unsigned total = static_cast<unsigned>(d0) * d2;
+  for (unsigned i = blockIdx.x * kSoftmax3dBlock + threadIdx.x; i < total;
+       i += gridDim.x * kSoftmax3dBlock) {
+    const unsigned y = div_d2.Div(i);
+    const unsigned n = i - y * d2;
+    const float *in = src + static_cast<size_t>(y) * d1 * sstride + n;
+    float *out = dst + static_cast<size_t>(y) * d1 * dstride + n;
+    float mx = in[0];
+    for (int x = 1; x < d1; ++x) {
+      const float e = in[static_cast<size_t>(x) * sstride];
+      mx = (mx < e) ? e : mx;
+    }
+    float sum = 0.0f;
+    for (int x = 0; x < d1; ++x) {
+      const float p = ExpNonPositive(in[static_cast<size_t>(x) * sstride] - mx);
+      out[static_cast<size_t>(x) * dstride] = p;
+      sum = sum + p;
+    }
+    const bool fast_div = sum >= 1.0f && sum < 3.0e38f;
+    const float rcp = 1.0f / sum;
+    for (int x = 0; x < d1; ++x) {
+      const float p = out[static_cast<size_t>(x) * dstride];
+      out[static_cast<size_t>(x) * dstride] = fast_div ? DivideBy(p, sum, rcp) : p / sum;
+    }
+  }
+}
+
+/*! \brief gradient on 3-D tensors: label is (d0, d2) with pitch lstride; elementwise over
+ *  the (d0 * d1, d2) view */
+template <int FLAGS>
+__global__ void __launch_bounds__(kSoftmax3dBlock)
+    Softmax3dGradKernel(float *dst, int dstride, const float *src, int sstride, const float *label,
+                        int lstride, int d0, int d1, int d2, mshadow::FastDivU32 div_d2,
+                        mshadow::FastDivU32 div_d1, GradParams gp) {
+  const unsigned total = static_cast<unsigned>(d0) * d1 * d2;
+  for (unsigned i = blockIdx.x * kSoftmax3dBlock + threadIdx.x; i < total;
+       i += gridDim.x * kSoftmax3dBlock) {
+    const unsigned row = div_d2.Div(i);       // y * d1 + x
+    const unsigned n = i - row * d2;
+    const unsigned y = div_d1.Div(row);
+    const int x = static_cast<int>(row - y * d1);
+    const int k = static_cast<int>(label[static_cast<size_t>(y) * lstride + n]);
+    const float s = src[static_cast<size_t>(row) * sstride + n];
+    dst[static_cast<size_t>(row) * dstride + n] =
+        GradElement<FLAGS>(s, x == k, (FLAGS & kGradIgnore) && k == gp.ignore_label, gp);
   }
 }
 

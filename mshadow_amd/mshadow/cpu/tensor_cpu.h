@@ -236,5 +236,133 @@ inline void SoftmaxGrad(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 2, DType> &
   }
 }
 
+
+/* ---- the rest of the softmax family and the row scatter / gather functions
+ * (mshadow/tensor_cpu-inl.h:304-528 of the reference). One element of every gradient
+ * variant is GradValue(): smooth spreads alpha over the other classes, a row whose label
+ * equals ignore_label gets zeros. */
+namespace cpu_detail {
+template <typename DType>
+inline DType GradValue(DType s, bool at_label, bool smooth, float alpha, float smooth_grad) {
+  if (at_label) return smooth ? DType(s - 1.0f + alpha) : DType(s - 1.0f);
+  return smooth ? DType(s - smooth_grad) : s;
+}
+template <typename DType>
+inline void Grad2D(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 2, DType> &src,
+                   const Tensor<cpu, 1, DType> &label, bool use_ignore, int ignore, bool smooth,
+                   float alpha) {
+  const float smooth_grad = alpha / (dst.size(1) - 1);
+#pragma omp parallel for
+  for (openmp_index_t y = 0; y < dst.size(0); ++y) {
+    const int k = static_cast<int>(label[y]);
+    for (int x = 0; x < static_cast<int>(dst.size(1)); ++x) {
+      dst[y][x] = (use_ignore && ignore == k) ? DType(0.0f)
+                                              : GradValue(src[y][x], x == k, smooth, alpha, smooth_grad);
+    }
+  }
+}
+template <typename DType>
+inline void Grad3D(Tensor<cpu, 3, DType> dst, const Tensor<cpu, 3, DType> &src,
+                   const Tensor<cpu, 2, DType> &label, bool use_ignore, int ignore, bool smooth,
+                   float alpha) {
+  const float smooth_grad = alpha / (dst.size(1) - 1);
+#pragma omp parallel for
+  for (openmp_index_t n = 0; n < dst.size(2); ++n) {
+    for (index_t y = 0; y < dst.size(0); ++y) {
+      const int k = static_cast<int>(label[y][n]);
+      for (int x = 0; x < static_cast<int>(dst.size(1)); ++x) {
+        dst[y][x][n] = (use_ignore && ignore == k)
+                           ? DType(0.0f)
+                           : GradValue(src[y][x][n], x == k, smooth, alpha, smooth_grad);
+      }
+    }
+  }
+}
+}  // namespace cpu_detail
+
+template <typename DType>
+inline void SmoothSoftmaxGrad(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 2, DType> &src,
+                              const Tensor<cpu, 1, DType> &label, const float alpha) {
+  cpu_detail::Grad2D(dst, src, label, false, 0, true, alpha);
+}
+template <typename DType>
+inline void SoftmaxGrad(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 2, DType> &src,
+                        const Tensor<cpu, 1, DType> &label, const DType &ignore_label) {
+  cpu_detail::Grad2D(dst, src, label, true, static_cast<int>(ignore_label), false, 0.0f);
+}
+template <typename DType>
+inline void SmoothSoftmaxGrad(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 2, DType> &src,
+                              const Tensor<cpu, 1, DType> &label, const DType &ignore_label,
+                              const float alpha) {
+  cpu_detail::Grad2D(dst, src, label, true, static_cast<int>(ignore_label), true, alpha);
+}
+template <typename DType>
+inline void SoftmaxGrad(Tensor<cpu, 3, DType> dst, const Tensor<cpu, 3, DType> &src,
+                        const Tensor<cpu, 2, DType> &label) {
+  cpu_detail::Grad3D(dst, src, label, false, 0, false, 0.0f);
+}
+template <typename DType>
+inline void SmoothSoftmaxGrad(Tensor<cpu, 3, DType> dst, const Tensor<cpu, 3, DType> &src,
+                              const Tensor<cpu, 2, DType> &label, const float alpha) {
+  cpu_detail::Grad3D(dst, src, label, false, 0, true, alpha);
+}
+template <typename DType>
+inline void SoftmaxGrad(Tensor<cpu, 3, DType> dst, const Tensor<cpu, 3, DType> &src,
+                        const Tensor<cpu, 2, DType> &label, const DType &ignore_label) {
+  cpu_detail::Grad3D(dst, src, label, true, static_cast<int>(ignore_label), false, 0.0f);
+}
+template <typename DType>
+inline void SmoothSoftmaxGrad(Tensor<cpu, 3, DType> dst, const Tensor<cpu, 3, DType> &src,
+                              const Tensor<cpu, 2, DType> &label, const DType &ignore_label,
+                              const float alpha) {
+  cpu_detail::Grad3D(dst, src, label, true, static_cast<int>(ignore_label), true, alpha);
+}
+/*! \brief softmax over the middle dimension of (d0, d1, d2) */
+template <typename DType>
+inline void Softmax(Tensor<cpu, 3, DType> dst, const Tensor<cpu, 3, DType> &energy) {
+  CHECK_EQ(dst.shape_, energy.shape_) << "Softmax: shape mismatch";
+#pragma omp parallel for
+  for (openmp_index_t y = 0; y < dst.size(0); ++y) {
+    for (index_t n = 0; n < dst.size(2); ++n) {
+      DType mmax = energy[y][0][n];
+      for (index_t x = 1; x < dst.size(1); ++x) {
+        if (mmax < energy[y][x][n]) mmax = energy[y][x][n];
+      }
+      DType sum = DType(0.0f);
+      for (index_t x = 0; x < dst.size(1); ++x) {
+        dst[y][x][n] = std::exp(energy[y][x][n] - mmax);
+        sum += dst[y][x][n];
+      }
+      for (index_t x = 0; x < dst.size(1); ++x) dst[y][x][n] /= sum;
+    }
+  }
+}
+/*! \brief dst[clamp(index[y])] += src[y], front to back */
+template <typename IndexType, typename DType>
+inline void AddTakeGrad(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 1, IndexType> &index,
+                        const Tensor<cpu, 2, DType> &src) {
+  const int K = dst.shape_[0];
+  for (index_t y = 0; y < index.size(0); ++y) {
+    int j = index[y];
+    j = j <= 0 ? 0 : (j >= K ? K - 1 : j);
+    dst[j] += src[y];
+  }
+}
+/*! \brief dst[sorted[y]] += src[index[y]], front to back */
+template <typename IndexType, typename DType>
+inline void AddTakeGradLargeBatch(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 1, IndexType> &sorted,
+                                  const Tensor<cpu, 1, IndexType> &index,
+                                  const Tensor<cpu, 2, DType> &src) {
+  for (index_t y = 0; y < sorted.size(0); ++y) dst[sorted[y]] += src[index[y]];
+}
+/*! \brief dst[index[y]] = src[y], front to back */
+template <typename IndexType, typename DType>
+inline void IndexFill(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 1, IndexType> &index,
+                      const Tensor<cpu, 2, DType> &src) {
+  for (index_t y = 0; y < index.size(0); ++y) {
+    for (index_t j = 0; j < src.size(1); j++) dst[index[y]][j] = src[y][j];
+  }
+}
+
 }  // namespace mshadow
 #endif  // MSHADOW_CPU_TENSOR_CPU_H_

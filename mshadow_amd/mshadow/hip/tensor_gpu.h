@@ -168,6 +168,102 @@ inline void SoftmaxGrad(const Tensor<gpu, 2, DType> &dst, const Tensor<gpu, 2, D
   LOG(FATAL) << "SoftmaxGrad<gpu>: only float is provided by this backend";
 }
 
+/* ---- the rest of the softmax family and the row scatter / gather functions: float tensors,
+ * int32 or float indices, each one call into the library */
+namespace gpu_detail {
+inline void Grad2D(const Tensor<gpu, 2, float> &dst, const Tensor<gpu, 2, float> &src,
+                   const Tensor<gpu, 1, float> &label, int flags, float ignore_label, float alpha) {
+  CHECK_EQ(dst.shape_, src.shape_) << "SoftmaxGrad: shape mismatch";
+  CHECK_EQ(dst.size(0), label.size(0)) << "SoftmaxGrad: label shape mismatch";
+  MSHADOW_HIP_CALL(mshadow_hip_softmax_grad_ex_f32(
+      dst.dptr_, dst.stride_, src.dptr_, src.stride_, label.dptr_, dst.size(0), dst.size(1), flags,
+      ignore_label, alpha, Stream<gpu>::GetStream(dst.stream_)));
+}
+inline void Grad3D(const Tensor<gpu, 3, float> &dst, const Tensor<gpu, 3, float> &src,
+                   const Tensor<gpu, 2, float> &label, int flags, float ignore_label, float alpha) {
+  CHECK_EQ(dst.shape_, src.shape_) << "SoftmaxGrad: shape mismatch";
+  CHECK(dst.size(0) == label.size(0) && dst.size(2) == label.size(1))
+      << "SoftmaxGrad: label shape mismatch";
+  MSHADOW_HIP_CALL(mshadow_hip_softmax3d_grad_f32(
+      dst.dptr_, dst.stride_, src.dptr_, src.stride_, label.dptr_, label.stride_, dst.size(0),
+      dst.size(1), dst.size(2), flags, ignore_label, alpha, Stream<gpu>::GetStream(dst.stream_)));
+}
+template <typename IndexType>
+struct IndexKind;  // only int32 and float index vectors are provided
+template <>
+struct IndexKind<int> { static const int kIsInt = 1; };
+template <>
+struct IndexKind<float> { static const int kIsInt = 0; };
+}  // namespace gpu_detail
+
+inline void Softmax(Tensor<gpu, 3, float> dst, const Tensor<gpu, 3, float> &src) {
+  CHECK_EQ(dst.shape_, src.shape_) << "Softmax: shape mismatch";
+  MSHADOW_HIP_CALL(mshadow_hip_softmax3d_f32(dst.dptr_, dst.stride_, src.dptr_, src.stride_,
+                                             dst.size(0), dst.size(1), dst.size(2),
+                                             Stream<gpu>::GetStream(dst.stream_)));
+}
+inline void SmoothSoftmaxGrad(const Tensor<gpu, 2, float> &dst, const Tensor<gpu, 2, float> &src,
+                              const Tensor<gpu, 1, float> &label, const float alpha) {
+  gpu_detail::Grad2D(dst, src, label, MSHADOW_HIP_GRAD_SMOOTH, 0.0f, alpha);
+}
+inline void SoftmaxGrad(const Tensor<gpu, 2, float> &dst, const Tensor<gpu, 2, float> &src,
+                        const Tensor<gpu, 1, float> &label, const float &ignore_label) {
+  gpu_detail::Grad2D(dst, src, label, MSHADOW_HIP_GRAD_IGNORE, ignore_label, 0.0f);
+}
+inline void SmoothSoftmaxGrad(const Tensor<gpu, 2, float> &dst, const Tensor<gpu, 2, float> &src,
+                              const Tensor<gpu, 1, float> &label, const float &ignore_label,
+                              const float alpha) {
+  gpu_detail::Grad2D(dst, src, label, MSHADOW_HIP_GRAD_SMOOTH | MSHADOW_HIP_GRAD_IGNORE,
+                     ignore_label, alpha);
+}
+inline void SoftmaxGrad(const Tensor<gpu, 3, float> &dst, const Tensor<gpu, 3, float> &src,
+                        const Tensor<gpu, 2, float> &label) {
+  gpu_detail::Grad3D(dst, src, label, 0, 0.0f, 0.0f);
+}
+inline void SmoothSoftmaxGrad(const Tensor<gpu, 3, float> &dst, const Tensor<gpu, 3, float> &src,
+                              const Tensor<gpu, 2, float> &label, const float alpha) {
+  gpu_detail::Grad3D(dst, src, label, MSHADOW_HIP_GRAD_SMOOTH, 0.0f, alpha);
+}
+inline void SoftmaxGrad(const Tensor<gpu, 3, float> &dst, const Tensor<gpu, 3, float> &src,
+                        const Tensor<gpu, 2, float> &label, const float &ignore_label) {
+  gpu_detail::Grad3D(dst, src, label, MSHADOW_HIP_GRAD_IGNORE, ignore_label, 0.0f);
+}
+inline void SmoothSoftmaxGrad(const Tensor<gpu, 3, float> &dst, const Tensor<gpu, 3, float> &src,
+                              const Tensor<gpu, 2, float> &label, const float &ignore_label,
+                              const float alpha) {
+  gpu_detail::Grad3D(dst, src, label, MSHADOW_HIP_GRAD_SMOOTH | MSHADOW_HIP_GRAD_IGNORE,
+                     ignore_label, alpha);
+}
+template <typename IndexType>
+inline void AddTakeGrad(Tensor<gpu, 2, float> dst, const Tensor<gpu, 1, IndexType> &index,
+                        const Tensor<gpu, 2, float> &src) {
+  CHECK_EQ(dst.size(1), src.size(1)) << "AddTakeGrad: shape mismatch";
+  CHECK_EQ(index.size(0), src.size(0)) << "AddTakeGrad: shape mismatch";
+  MSHADOW_HIP_CALL(mshadow_hip_add_take_grad_f32(
+      dst.dptr_, dst.stride_, dst.size(0), index.dptr_, gpu_detail::IndexKind<IndexType>::kIsInt,
+      index.size(0), src.dptr_, src.stride_, src.size(1), Stream<gpu>::GetStream(dst.stream_)));
+}
+template <typename IndexType>
+inline void AddTakeGradLargeBatch(Tensor<gpu, 2, float> dst, const Tensor<gpu, 1, IndexType> &sorted,
+                                  const Tensor<gpu, 1, IndexType> &index,
+                                  const Tensor<gpu, 2, float> &src) {
+  CHECK_EQ(dst.size(1), src.size(1)) << "AddTakeGradLargeBatch: shape mismatch";
+  CHECK_EQ(sorted.size(0), index.size(0)) << "AddTakeGradLargeBatch: shape mismatch";
+  MSHADOW_HIP_CALL(mshadow_hip_add_take_grad_large_batch_f32(
+      dst.dptr_, dst.stride_, dst.size(0), sorted.dptr_, index.dptr_,
+      gpu_detail::IndexKind<IndexType>::kIsInt, index.size(0), src.dptr_, src.stride_, src.size(1),
+      Stream<gpu>::GetStream(dst.stream_)));
+}
+template <typename IndexType>
+inline void IndexFill(Tensor<gpu, 2, float> dst, const Tensor<gpu, 1, IndexType> &index,
+                      const Tensor<gpu, 2, float> &src) {
+  CHECK_EQ(dst.size(1), src.size(1)) << "IndexFill: shape mismatch";
+  CHECK_EQ(index.size(0), src.size(0)) << "IndexFill: shape mismatch";
+  MSHADOW_HIP_CALL(mshadow_hip_index_fill_f32(
+      dst.dptr_, dst.stride_, dst.size(0), index.dptr_, gpu_detail::IndexKind<IndexType>::kIsInt,
+      index.size(0), src.dptr_, src.stride_, src.size(1), Stream<gpu>::GetStream(dst.stream_)));
+}
+
 /* ------------------------------------------------------------------ expression routing */
 namespace gpu_detail {
 

@@ -91,6 +91,65 @@ template <typename DType>
 inline void SoftmaxGrad(const Tensor<gpu, 2, DType> &dst, const Tensor<gpu, 2, DType> &src,
                         const Tensor<gpu, 1, DType> &label);
 
+/*! \brief the rest of the softmax family: label smoothing (alpha), ignore_label, and
+ *  3-D tensors (d0, d1, d2) whose softmax runs over the middle dimension */
+template <typename DType>
+inline void Softmax(Tensor<cpu, 3, DType> dst, const Tensor<cpu, 3, DType> &energy);
+template <typename DType>
+inline void Softmax(Tensor<gpu, 3, DType> dst, const Tensor<gpu, 3, DType> &energy);
+#define MSHADOW_DECLARE_GRAD_FAMILY(Device, DstQual)                                              \
+  template <typename DType>                                                                       \
+  inline void SmoothSoftmaxGrad(DstQual(Device, 2) dst, const Tensor<Device, 2, DType> &src,      \
+                                const Tensor<Device, 1, DType> &label, const float alpha);        \
+  template <typename DType>                                                                       \
+  inline void SoftmaxGrad(DstQual(Device, 2) dst, const Tensor<Device, 2, DType> &src,            \
+                          const Tensor<Device, 1, DType> &label, const DType &ignore_label);      \
+  template <typename DType>                                                                       \
+  inline void SmoothSoftmaxGrad(DstQual(Device, 2) dst, const Tensor<Device, 2, DType> &src,      \
+                                const Tensor<Device, 1, DType> &label, const DType &ignore_label, \
+                                const float alpha);                                               \
+  template <typename DType>                                                                       \
+  inline void SoftmaxGrad(DstQual(Device, 3) dst, const Tensor<Device, 3, DType> &src,            \
+                          const Tensor<Device, 2, DType> &label);                                 \
+  template <typename DType>                                                                       \
+  inline void SmoothSoftmaxGrad(DstQual(Device, 3) dst, const Tensor<Device, 3, DType> &src,      \
+                                const Tensor<Device, 2, DType> &label, const float alpha);        \
+  template <typename DType>                                                                       \
+  inline void SoftmaxGrad(DstQual(Device, 3) dst, const Tensor<Device, 3, DType> &src,            \
+                          const Tensor<Device, 2, DType> &label, const DType &ignore_label);      \
+  template <typename DType>                                                                       \
+  inline void SmoothSoftmaxGrad(DstQual(Device, 3) dst, const Tensor<Device, 3, DType> &src,      \
+                                const Tensor<Device, 2, DType> &label, const DType &ignore_label, \
+                                const float alpha);
+#define MSHADOW_DST_BY_VALUE(Device, dim) Tensor<Device, dim, DType>
+#define MSHADOW_DST_BY_CREF(Device, dim) const Tensor<Device, dim, DType> &
+MSHADOW_DECLARE_GRAD_FAMILY(cpu, MSHADOW_DST_BY_VALUE)
+MSHADOW_DECLARE_GRAD_FAMILY(gpu, MSHADOW_DST_BY_CREF)
+#undef MSHADOW_DECLARE_GRAD_FAMILY
+#undef MSHADOW_DST_BY_VALUE
+#undef MSHADOW_DST_BY_CREF
+/*! \brief rows gathered / scattered by an index vector, applied front to back */
+template <typename IndexType, typename DType>
+inline void AddTakeGrad(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 1, IndexType> &index,
+                        const Tensor<cpu, 2, DType> &src);
+template <typename IndexType, typename DType>
+inline void AddTakeGrad(Tensor<gpu, 2, DType> dst, const Tensor<gpu, 1, IndexType> &index,
+                        const Tensor<gpu, 2, DType> &src);
+template <typename IndexType, typename DType>
+inline void AddTakeGradLargeBatch(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 1, IndexType> &sorted,
+                                  const Tensor<cpu, 1, IndexType> &index,
+                                  const Tensor<cpu, 2, DType> &src);
+template <typename IndexType, typename DType>
+inline void AddTakeGradLargeBatch(Tensor<gpu, 2, DType> dst, const Tensor<gpu, 1, IndexType> &sorted,
+                                  const Tensor<gpu, 1, IndexType> &index,
+                                  const Tensor<gpu, 2, DType> &src);
+template <typename IndexType, typename DType>
+inline void IndexFill(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 1, IndexType> &index,
+                      const Tensor<cpu, 2, DType> &src);
+template <typename IndexType, typename DType>
+inline void IndexFill(Tensor<gpu, 2, DType> dst, const Tensor<gpu, 1, IndexType> &index,
+                      const Tensor<gpu, 2, DType> &src);
+
 /*! \brief Saver::Save(dst(y,x), exp(y,x)) for every element */
 template <typename Saver, typename R, int dim, typename DType, typename E, int etype>
 inline void MapExp(TRValue<R, cpu, dim, DType> *dst, const expr::Exp<E, DType, etype> &exp);

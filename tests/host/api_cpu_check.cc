@@ -248,6 +248,57 @@ int main() {
     back = crop(padded, Shape2(H, W));  // centred crop undoes the symmetric pad
     EXPECT(back[1][1][4][5] == I[1][1][4][5] && back[0][0][0][0] == I[0][0][0][0]);
   }
+  // ---- the rest of the softmax family and the row scatter / gather functions
+  {
+    const int R = 7, C = 13;
+    std::vector<float> p = Rand(R * C, 20, 0, 1), lab = {0, 12, 4, 4, -2, 13, 5};
+    Tensor<cpu, 2> P(p.data(), Shape2(R, C));
+    Tensor<cpu, 1> L(lab.data(), Shape1(R));
+    for (int flags = 1; flags < 4; ++flags) {
+      std::vector<float> o1(R * C), o2(R * C);
+      Tensor<cpu, 2> O(o1.data(), Shape2(R, C));
+      if (flags == 1) SmoothSoftmaxGrad(O, P, L, 0.1f);
+      else if (flags == 2) SoftmaxGrad(O, P, L, 4.0f);
+      else SmoothSoftmaxGrad(O, P, L, 4.0f, 0.1f);
+      orc_softmax_grad_ex_f32(o2.data(), C, p.data(), C, lab.data(), R, C, flags, 4.0f, 0.1f);
+      EXPECT(SameBits(o1.data(), o2.data(), o1.size()));
+    }
+    const int D0 = 3, D1 = 6, D2 = 5;
+    std::vector<float> x = Rand(D0 * D1 * D2, 21, -6, 6), s1(x.size()), s2(x.size());
+    Tensor<cpu, 3> X(x.data(), Shape3(D0, D1, D2)), S(s1.data(), Shape3(D0, D1, D2));
+    Softmax(S, X);
+    orc_softmax3d_f32(s2.data(), D2, x.data(), D2, D0, D1, D2);
+    EXPECT(SameBits(s1.data(), s2.data(), s1.size()));
+    std::vector<float> l3 = Rand(D0 * D2, 22, 0, 5.99f);
+    Tensor<cpu, 2> L3(l3.data(), Shape2(D0, D2));
+    for (int flags = 0; flags < 4; ++flags) {
+      std::vector<float> g1(x.size()), g2(x.size());
+      Tensor<cpu, 3> Gt(g1.data(), Shape3(D0, D1, D2));
+      if (flags == 0) SoftmaxGrad(Gt, S, L3);
+      else if (flags == 1) SmoothSoftmaxGrad(Gt, S, L3, 0.2f);
+      else if (flags == 2) SoftmaxGrad(Gt, S, L3, 3.0f);
+      else SmoothSoftmaxGrad(Gt, S, L3, 3.0f, 0.2f);
+      orc_softmax3d_grad_f32(g2.data(), D2, s2.data(), D2, l3.data(), D2, D0, D1, D2, flags, 3.0f, 0.2f);
+      EXPECT(SameBits(g1.data(), g2.data(), g1.size()));
+    }
+    const int K = 5, N = 40, W = 3;
+    std::vector<float> src = Rand(N * W, 23), d1 = Rand(K * W, 24), d2 = d1;
+    std::vector<int> idx(N), srt(N), ord(N);
+    for (int i = 0; i < N; ++i) idx[i] = (i * 7) % 9 - 2;
+    Tensor<cpu, 2> Sr(src.data(), Shape2(N, W)), Dd(d1.data(), Shape2(K, W));
+    Tensor<cpu, 1, int> I(idx.data(), Shape1(N));
+    AddTakeGrad(Dd, I, Sr);
+    orc_add_take_grad_f32(d2.data(), W, K, idx.data(), 1, N, src.data(), W, W);
+    EXPECT(SameBits(d1.data(), d2.data(), d1.size()));
+    for (int i = 0; i < N; ++i) { srt[i] = i * K / N; ord[i] = (i * 17) % N; }
+    Tensor<cpu, 1, int> So(srt.data(), Shape1(N)), Or(ord.data(), Shape1(N));
+    AddTakeGradLargeBatch(Dd, So, Or, Sr);
+    orc_add_take_grad_large_batch_f32(d2.data(), W, srt.data(), ord.data(), 1, N, src.data(), W, W);
+    EXPECT(SameBits(d1.data(), d2.data(), d1.size()));
+    IndexFill(Dd, So, Sr);
+    orc_index_fill_f32(d2.data(), W, srt.data(), 1, N, src.data(), W, W);
+    EXPECT(SameBits(d1.data(), d2.data(), d1.size()));
+  }
   if (g_fail) {
     fprintf(stderr, "%d of %d checks failed\n", g_fail, g_checks);
     return 1;
