@@ -46,6 +46,11 @@ def algorithmic_bytes():
         "im2col_f16": 2 * 32 * 256 * 56 * 56 + 2 * 2304 * 100352,
         "col2im_f16": 2 * 32 * 256 * 56 * 56 + 2 * 2304 * 100352,
         "calib_copy": 2 * e * 4096 * 4096,
+        # rows next to the hot path (only with --only; never part of the step)
+        "smooth_softmax_grad_ignore": 2 * e * 8192 * 32000 + e * 8192,
+        "softmax3d": 2 * e * 256 * 21 * 16384,
+        "softmax3d_grad": 2 * e * 256 * 21 * 16384 + e * 256 * 16384,
+        "add_take_grad": e * 16384 + 3 * e * 16384 * 512,
     }
 
 
@@ -55,10 +60,13 @@ def work_elements():
         "sum_rows": 16384 * 4096, "softmax": 8192 * 32000, "softmax_grad": 8192 * 32000,
         "pool_max": 128 * 64 * 55 * 55, "unpool_max": 128 * 64 * 112 * 112,
         "im2col_f16": 2304 * 100352, "col2im_f16": 2304 * 100352, "calib_copy": 4096 * 4096,
+        "smooth_softmax_grad_ignore": 8192 * 32000, "softmax3d": 256 * 21 * 16384,
+        "softmax3d_grad": 256 * 21 * 16384, "add_take_grad": 16384 * 512,
     }
 
 
-OPS = [k for k in algorithmic_bytes() if k != "calib_copy"]
+EXTRA_OPS = ("calib_copy", "smooth_softmax_grad_ignore", "softmax3d", "softmax3d_grad", "add_take_grad")
+OPS = [k for k in algorithmic_bytes() if k not in EXTRA_OPS]
 
 # HBM bytes per launch of each operation's kernel, measured with rocprofv3 --pmc FETCH_SIZE and
 # --pmc WRITE_SIZE (two runs of `bench.py --only <all ops>,calib_copy`), each counter scaled by
@@ -140,8 +148,28 @@ def main():
     out_col = G.buffer(col_h.shape, np.uint16)
     out_img = G.buffer(img_h.shape, np.uint16)
 
+    extra = {}
+    if any(o in EXTRA_OPS[1:] for o in only):
+        rng = np.random.default_rng(13)
+        x3 = (rng.standard_normal((256, 21, 16384), dtype=f32) * f32(3))
+        extra["x3"] = G.to_device(x3)
+        extra["p3"] = G.buffer(x3.shape, f32)
+        extra["g3"] = G.buffer(x3.shape, f32)
+        extra["l3"] = G.to_device(rng.integers(0, 21, (256, 16384)).astype(f32))
+        extra["emb"] = G.to_device(np.zeros((50000, 512), f32))
+        extra["idx"] = G.to_device(rng.integers(0, 50000, 16384).astype(np.int32))
+        extra["rows"] = G.to_device(rng.standard_normal((16384, 512), dtype=f32))
+
     def run_op(name):
-        if name == "map_fused":
+        if name == "smooth_softmax_grad_ignore":
+            G.softmax_grad_ex(out_g, out_p, dev["labels"], 3, 17.0, 0.1, s)
+        elif name == "softmax3d":
+            G.softmax3d(extra["p3"], extra["x3"], s)
+        elif name == "softmax3d_grad":
+            G.softmax3d_grad(extra["g3"], extra["p3"], extra["l3"], 0, 0.0, 0.0, s)
+        elif name == "add_take_grad":
+            G.add_take_grad(extra["emb"], extra["idx"], extra["rows"], s)
+        elif name == "map_fused":
             G.case_map_fused(out_map, dev["A"], dev["B"], dev["C"], dev["D"], 0, s)
         elif name == "sumall_except_dim1":
             G.reduce_keep_highdim(out_2a, dev["X2a"], stream=s)

@@ -373,6 +373,19 @@ int mshadow_hip_softmax3d_f32(float *dst, int dstride, const float *src, int sst
   ABI_REQUIRE(static_cast<long long>(d0) * d2 < (1ll << 31) &&
                   static_cast<long long>(d0) * d1 < (1ll << 31),
               "too large for 32-bit indices");
+  const mshadow::FastDivU32 div_d2s(static_cast<uint32_t>(d2));
+  const unsigned pairs = static_cast<unsigned>(d0) * d2;
+  const unsigned one_each = (pairs + kSoftmax3dBlock - 1) / kSoftmax3dBlock;
+  if (d1 <= 8) {
+    hipLaunchKernelGGL((Softmax3dSmallKernel<8>), dim3(one_each), dim3(kSoftmax3dBlock), 0,
+                       AsStream(stream), dst, dstride, src, sstride, d0, d1, d2, div_d2s);
+    return AfterLaunch("softmax3d");
+  }
+  if (d1 <= 32) {
+    hipLaunchKernelGGL((Softmax3dSmallKernel<32>), dim3(one_each), dim3(kSoftmax3dBlock), 0,
+                       AsStream(stream), dst, dstride, src, sstride, d0, d1, d2, div_d2s);
+    return AfterLaunch("softmax3d");
+  }
   unsigned grid = 0;
   int st = mshadow_hip_suggest_grid(static_cast<size_t>(d0) * d2, kSoftmax3dBlock, 8, &grid);
   if (st != MSHADOW_HIP_OK) return st;
@@ -397,6 +410,25 @@ int mshadow_hip_softmax3d_grad_f32(float *dst, int dstride, const float *src, in
   const GradParams gp = {static_cast<int>(ignore_label), alpha,
                          alpha / static_cast<float>(static_cast<unsigned>(d1 - 1))};
   const mshadow::FastDivU32 div_d2(static_cast<uint32_t>(d2)), div_d1(static_cast<uint32_t>(d1));
+  const bool vec = d2 % 4 == 0 && dstride % 4 == 0 && sstride % 4 == 0 && lstride % 4 == 0 &&
+                   Aligned16(dst) && Aligned16(src) && Aligned16(label);
+  if (vec) {
+    const unsigned packs = static_cast<unsigned>(d0) * d1 * (d2 / 4);
+    const unsigned vgrid = (packs + kSoftmax3dBlock - 1) / kSoftmax3dBlock;
+    const mshadow::FastDivU32 div_q2(static_cast<uint32_t>(d2 / 4));
+#define GRAD3DV(FLAGS)                                                                         \
+  hipLaunchKernelGGL((Softmax3dGradVecKernel<FLAGS>), dim3(vgrid), dim3(kSoftmax3dBlock), 0,   \
+                     AsStream(stream), dst, dstride, src, sstride, label, lstride, d0, d1, d2, \
+                     div_q2, div_d1, gp)
+    switch (flags) {
+      case 0: GRAD3DV(0); break;
+      case 1: GRAD3DV(1); break;
+      case 2: GRAD3DV(2); break;
+      default: GRAD3DV(3); break;
+    }
+#undef GRAD3DV
+    return AfterLaunch("softmax3d_grad");
+  }
 #define GRAD3D(FLAGS)                                                                          \
   hipLaunchKernelGGL((Softmax3dGradKernel<FLAGS>), dim3(grid), dim3(kSoftmax3dBlock), 0,       \
                      AsStream(stream), dst, dstride, src, sstride, label, lstride, d0, d1, d2, \

@@ -944,8 +944,76 @@ __global__ void __launch_bounds__(kSoftmax3dBlock)
   }
 }
 
+/*! \brief the same for at most D1MAX classes: the column of one (y, n) pair is fetched once
+ *  (all loads in flight together), kept in registers and written once */
+template <int D1MAX>
+__global__ void __launch_bounds__(kSoftmax3dBlock)
+    Softmax3dSmallKernel(float *dst, int dstride, const float *src, int sstride, int d0, int d1,
+                         int d2, mshadow::FastDivU32 div_d2) {
+  const unsigned total = static_cast<unsigned>(d0) * d2;
+  const unsigned i = blockIdx.x * kSoftmax3dBlock + threadIdx.x;
+  if (i >= total) return;
+  const unsigned y = div_d2.Div(i);
+  const unsigned n = i - y * d2;
+  const float *in = src + static_cast<size_t>(y) * d1 * sstride + n;
+  float *out = dst + static_cast<size_t>(y) * d1 * dstride + n;
+  float v[D1MAX];
+#pragma unroll
+  for (int x = 0; x < D1MAX; ++x) {
+    /* unpredicated: classes past the end re-read the last one and are not used */
+    v[x] = StreamLoad(in + static_cast<size_t>(x < d1 ? x : d1 - 1) * sstride);
+  }
+  float mx = v[0];
+#pragma unroll
+  for (int x = 1; x < D1MAX; ++x) {
+    if (x < d1) mx = (mx < v[x]) ? v[x] : mx;
+  }
+  float sum = 0.0f;
+#pragma unroll
+  for (int x = 0; x < D1MAX; ++x) {
+    if (x < d1) {
+      v[x] = ExpNonPositive(v[x] - mx);
+      sum = sum + v[x];
+    }
+  }
+  const bool fast_div = sum >= 1.0f && sum < 3.0e38f;
+  const float rcp = 1.0f / sum;
+#pragma unroll
+  for (int x = 0; x < D1MAX; ++x) {
+    if (x < d1) {
+      StreamStore(out + static_cast<size_t>(x) * dstride, fast_div ? DivideBy(v[x], sum, rcp) : v[x] / sum);
+    }
+  }
+}
+
 /*! \brief gradient on 3-D tensors: label is (d0, d2) with pitch lstride; elementwise over
- *  the (d0 * d1, d2) view */
+ *  the (d0 * d1, d2) view, VEC consecutive n per thread (VEC = 4 needs d2 % 4 == 0 and
+ *  16-byte aligned rows) */
+template <int FLAGS>
+__global__ void __launch_bounds__(kSoftmax3dBlock)
+    Softmax3dGradVecKernel(float *dst, int dstride, const float *src, int sstride,
+                           const float *label, int lstride, int d0, int d1, int d2,
+                           mshadow::FastDivU32 div_q2, mshadow::FastDivU32 div_d1, GradParams gp) {
+  const unsigned q2 = static_cast<unsigned>(d2) / 4;  // packs per row
+  const unsigned total = static_cast<unsigned>(d0) * d1 * q2;
+  const unsigned i = blockIdx.x * kSoftmax3dBlock + threadIdx.x;
+  if (i >= total) return;
+  const unsigned row = div_q2.Div(i);
+  const unsigned n = (i - row * q2) * 4;
+  const unsigned y = div_d1.Div(row);
+  const int x = static_cast<int>(row - y * d1);
+  const F4 l = *reinterpret_cast<const F4 *>(label + static_cast<size_t>(y) * lstride + n);
+  F4 s = StreamLoadF4(src + static_cast<size_t>(row) * sstride + n);
+  const int k0 = static_cast<int>(l.x), k1 = static_cast<int>(l.y), k2 = static_cast<int>(l.z),
+            k3 = static_cast<int>(l.w);
+  s.x = GradElement<FLAGS>(s.x, x == k0, (FLAGS & kGradIgnore) && k0 == gp.ignore_label, gp);
+  s.y = GradElement<FLAGS>(s.y, x == k1, (FLAGS & kGradIgnore) && k1 == gp.ignore_label, gp);
+  s.z = GradElement<FLAGS>(s.z, x == k2, (FLAGS & kGradIgnore) && k2 == gp.ignore_label, gp);
+  s.w = GradElement<FLAGS>(s.w, x == k3, (FLAGS & kGradIgnore) && k3 == gp.ignore_label, gp);
+  StreamStoreF4(dst + static_cast<size_t>(row) * dstride + n, s);
+}
+
+/*! \brief any alignment: one element per thread-iteration */
 template <int FLAGS>
 __global__ void __launch_bounds__(kSoftmax3dBlock)
     Softmax3dGradKernel(float *dst, int dstride, const float *src, int sstride, const float *label,

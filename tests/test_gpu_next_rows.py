@@ -42,7 +42,8 @@ def test_grad_family_2d(G, O, shape, pad, flags):
         assert_bits_equal(dst.download(), want, f"grad flags={flags} {shape} {route}")
 
 
-@pytest.mark.parametrize("shape,pad", [((7, 19, 33), 0), ((3, 5, 1), 2), ((2, 1000, 70), 1), ((64, 21, 257), 0)])
+@pytest.mark.parametrize("shape,pad", [((7, 19, 33), 0), ((3, 5, 1), 2), ((2, 1000, 70), 1), ((64, 21, 257), 0),
+                                       ((4, 21, 64), 0), ((3, 40, 128), 4), ((2, 8, 12), 0)])
 def test_softmax3d_and_grads(G, O, shape, pad):
     rng = np.random.default_rng(6)
     x = (rng.standard_normal(shape) * 3).astype(f32)
