@@ -457,14 +457,21 @@ int mshadow_hip_add_take_grad_f32(float *dst, int dstride, int k_rows, const voi
                                   int cols, void *stream) {
   const int chk = RowOpCheck(dst, dstride, k_rows, index, n_index, src, sstride, cols);
   if (chk != MSHADOW_HIP_OK) return chk < 0 ? MSHADOW_HIP_OK : chk;
-  const unsigned grid = (static_cast<unsigned>(k_rows) + kRowBlock / 64 - 1) / (kRowBlock / 64);
-  if (index_is_int) {
-    hipLaunchKernelGGL((AddTakeGradKernel<true, true>), dim3(grid), dim3(kRowBlock), 0,
-                       AsStream(stream), dst, dstride, k_rows, index, index, n_index, src, sstride, cols);
+  /* one wave per destination row, or per index entry when the table has more rows */
+  const bool by_entry = n_index < k_rows;
+  const unsigned waves = static_cast<unsigned>(by_entry ? n_index : k_rows);
+  const unsigned grid = (waves + kRowBlock / 64 - 1) / (kRowBlock / 64);
+#define ROW_LAUNCH(...)                                                                    \
+  hipLaunchKernelGGL((__VA_ARGS__), dim3(grid), dim3(kRowBlock), 0, AsStream(stream), dst, dstride, \
+                     k_rows, index, index, n_index, src, sstride, cols)
+  if (by_entry) {
+    if (index_is_int) ROW_LAUNCH(AddTakeGradByEntryKernel<true, true>);
+    else ROW_LAUNCH(AddTakeGradByEntryKernel<false, true>);
   } else {
-    hipLaunchKernelGGL((AddTakeGradKernel<false, true>), dim3(grid), dim3(kRowBlock), 0,
-                       AsStream(stream), dst, dstride, k_rows, index, index, n_index, src, sstride, cols);
+    if (index_is_int) ROW_LAUNCH(AddTakeGradKernel<true, true>);
+    else ROW_LAUNCH(AddTakeGradKernel<false, true>);
   }
+#undef ROW_LAUNCH
   return AfterLaunch("add_take_grad");
 }
 
@@ -475,14 +482,20 @@ int mshadow_hip_add_take_grad_large_batch_f32(float *dst, int dstride, int k_row
   const int chk = RowOpCheck(dst, dstride, k_rows, index, n_index, src, sstride, cols);
   if (chk != MSHADOW_HIP_OK) return chk < 0 ? MSHADOW_HIP_OK : chk;
   ABI_REQUIRE(sorted != NULL, "NULL tensor");
-  const unsigned grid = (static_cast<unsigned>(k_rows) + kRowBlock / 64 - 1) / (kRowBlock / 64);
-  if (index_is_int) {
-    hipLaunchKernelGGL((AddTakeGradKernel<true, false>), dim3(grid), dim3(kRowBlock), 0,
-                       AsStream(stream), dst, dstride, k_rows, sorted, index, n_index, src, sstride, cols);
+  const bool by_entry = n_index < k_rows;
+  const unsigned waves = static_cast<unsigned>(by_entry ? n_index : k_rows);
+  const unsigned grid = (waves + kRowBlock / 64 - 1) / (kRowBlock / 64);
+#define ROW_LAUNCH(...)                                                                    \
+  hipLaunchKernelGGL((__VA_ARGS__), dim3(grid), dim3(kRowBlock), 0, AsStream(stream), dst, dstride, \
+                     k_rows, sorted, index, n_index, src, sstride, cols)
+  if (by_entry) {
+    if (index_is_int) ROW_LAUNCH(AddTakeGradByEntryKernel<true, false>);
+    else ROW_LAUNCH(AddTakeGradByEntryKernel<false, false>);
   } else {
-    hipLaunchKernelGGL((AddTakeGradKernel<false, false>), dim3(grid), dim3(kRowBlock), 0,
-                       AsStream(stream), dst, dstride, k_rows, sorted, index, n_index, src, sstride, cols);
+    if (index_is_int) ROW_LAUNCH(AddTakeGradKernel<true, false>);
+    else ROW_LAUNCH(AddTakeGradKernel<false, false>);
   }
+#undef ROW_LAUNCH
   return AfterLaunch("add_take_grad_large_batch");
 }
 
@@ -491,14 +504,20 @@ int mshadow_hip_index_fill_f32(float *dst, int dstride, int k_rows, const void *
                                int cols, void *stream) {
   const int chk = RowOpCheck(dst, dstride, k_rows, index, n_index, src, sstride, cols);
   if (chk != MSHADOW_HIP_OK) return chk < 0 ? MSHADOW_HIP_OK : chk;
-  const unsigned grid = (static_cast<unsigned>(k_rows) + kRowBlock / 64 - 1) / (kRowBlock / 64);
-  if (index_is_int) {
-    hipLaunchKernelGGL((IndexFillKernel<true>), dim3(grid), dim3(kRowBlock), 0, AsStream(stream),
-                       dst, dstride, k_rows, index, n_index, src, sstride, cols);
+  const bool by_entry = n_index < k_rows;
+  const unsigned waves = static_cast<unsigned>(by_entry ? n_index : k_rows);
+  const unsigned grid = (waves + kRowBlock / 64 - 1) / (kRowBlock / 64);
+#define ROW_LAUNCH(...)                                                                    \
+  hipLaunchKernelGGL((__VA_ARGS__), dim3(grid), dim3(kRowBlock), 0, AsStream(stream), dst, dstride, \
+                     k_rows, index, n_index, src, sstride, cols)
+  if (by_entry) {
+    if (index_is_int) ROW_LAUNCH(IndexFillByEntryKernel<true>);
+    else ROW_LAUNCH(IndexFillByEntryKernel<false>);
   } else {
-    hipLaunchKernelGGL((IndexFillKernel<false>), dim3(grid), dim3(kRowBlock), 0, AsStream(stream),
-                       dst, dstride, k_rows, index, n_index, src, sstride, cols);
+    if (index_is_int) ROW_LAUNCH(IndexFillKernel<true>);
+    else ROW_LAUNCH(IndexFillKernel<false>);
   }
+#undef ROW_LAUNCH
   return AfterLaunch("index_fill");
 }
 

@@ -61,6 +61,67 @@ __global__ void __launch_bounds__(kRowBlock)
   }
 }
 
+/*! \brief the same result with one wave per ENTRY of the index vector instead of one per
+ *  destination row, for tables with more rows than there are entries: the wave of entry y
+ *  looks for an earlier entry naming the same row and retires if there is one; the wave of
+ *  a row's first entry then applies all of that row's entries in order. Work is about
+ *  entries^2 / 64 wave-steps, independent of the number of rows. */
+template <bool IS_INT, bool CLAMP>
+__global__ void __launch_bounds__(kRowBlock)
+    AddTakeGradByEntryKernel(float *dst, int dstride, int k_rows, const void *rows_of,
+                             const void *from_of, int n_index, const float *src, int sstride,
+                             int cols) {
+  const int lane = threadIdx.x & 63;
+  const int me = blockIdx.x * (kRowBlock / 64) + (threadIdx.x >> 6);
+  if (me >= n_index) return;
+  int j = IndexAt<IS_INT>(rows_of, me);
+  if (CLAMP) j = j <= 0 ? 0 : (j >= k_rows ? k_rows - 1 : j);
+  if (j < 0 || j >= k_rows) return;
+  float *out = dst + static_cast<size_t>(j) * dstride;
+  for (int y0 = 0; y0 < n_index; y0 += 64) {
+    const int y = y0 + lane;
+    int r = -1;
+    if (y < n_index) {
+      r = IndexAt<IS_INT>(rows_of, y);
+      if (CLAMP) r = r <= 0 ? 0 : (r >= k_rows ? k_rows - 1 : r);
+    }
+    unsigned long long hits = __ballot(r == j);
+    if (y0 <= me && hits != 0ull) {
+      /* the first entry of the row, at or before mine, is in this chunk */
+      if (y0 + __ffsll(static_cast<long long>(hits)) - 1 != me) return;  // not the row's first entry
+    }
+    if (y0 + 63 < me) continue;  // still in front of my entry: nothing to apply yet
+    while (hits != 0ull) {
+      const int b = __ffsll(static_cast<long long>(hits)) - 1;
+      hits &= hits - 1ull;
+      const int from = CLAMP ? y0 + b : IndexAt<IS_INT>(from_of, y0 + b);
+      const float *in = src + static_cast<size_t>(from) * sstride;
+      for (int x = lane; x < cols; x += 64) out[x] = out[x] + in[x];
+    }
+  }
+}
+
+/*! \brief IndexFill by entry: the wave of entry y copies its row unless a later entry names
+ *  the same destination */
+template <bool IS_INT>
+__global__ void __launch_bounds__(kRowBlock)
+    IndexFillByEntryKernel(float *dst, int dstride, int k_rows, const void *index, int n_index,
+                           const float *src, int sstride, int cols) {
+  const int lane = threadIdx.x & 63;
+  const int me = blockIdx.x * (kRowBlock / 64) + (threadIdx.x >> 6);
+  if (me >= n_index) return;
+  const int j = IndexAt<IS_INT>(index, me);
+  if (j < 0 || j >= k_rows) return;
+  for (int y0 = (me / 64) * 64; y0 < n_index; y0 += 64) {
+    const int y = y0 + lane;
+    const bool later = y > me && y < n_index && IndexAt<IS_INT>(index, y) == j;
+    if (__ballot(later) != 0ull) return;
+  }
+  const float *in = src + static_cast<size_t>(me) * sstride;
+  float *out = dst + static_cast<size_t>(j) * dstride;
+  for (int x = lane; x < cols; x += 64) out[x] = in[x];
+}
+
 /*! \brief dst[index[y]] = src[y]; of several entries naming one row the last one counts */
 template <bool IS_INT>
 __global__ void __launch_bounds__(kRowBlock)
