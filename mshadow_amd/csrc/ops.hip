@@ -613,6 +613,7 @@ int mshadow_hip_reduce_keep_highdim_f32(float *dst, const float *src, int sstrid
 /* ------------------------------------------------------------------ pool / unpool */
 
 static const size_t kPoolLdsBudget = 48 * 1024;  // per workgroup: three resident per CU
+static const size_t kUnpoolLdsBudget = 16 * 1024;  // smaller bands: more workgroups in different phases per CU
 
 int mshadow_hip_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes,
                          int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,
@@ -704,7 +705,7 @@ int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstrid
   hipStream_t s = AsStream(stream);
   const size_t row_bytes = static_cast<size_t>(g.lds_pitch) * sizeof(float) * 2;  // pooled + grad
   /* source rows per band: prow_max = (band + ky - 2) / sy + 2 pooled rows must fit */
-  long long max_prow = static_cast<long long>(kPoolLdsBudget / row_bytes);
+  long long max_prow = static_cast<long long>(kUnpoolLdsBudget / row_bytes);
   long long band = (max_prow - 2) * sy - ky + 2;
   if (band > h) band = h;
   while (band > 8 && static_cast<long long>(planes) * ((h + band - 1) / band) < 1024) {

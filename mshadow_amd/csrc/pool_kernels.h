@@ -298,7 +298,7 @@ __global__ void __launch_bounds__(kPoolBlock)
   const int bw = (g.w + SX - 1) / SX;
   const int a0 = y0 / SY;
   const unsigned nblk = static_cast<unsigned>((ny + SY - 1) / SY) * bw;
-  const int kAhead = 2;  // blocks per thread whose loads are issued before any is used
+  const int kAhead = 4;  // blocks per thread whose loads are issued before any is used
   __syncthreads();
   for (unsigned t0 = threadIdx.x; t0 < nblk; t0 += kPoolBlock * kAhead) {
     float vs[kAhead][SY][SX];
