@@ -831,7 +831,7 @@ __global__ void __launch_bounds__(THREADS)
 }
 
 const int kGradBlock = 256;
-const int kGradPacks = 2;  // 128-bit packs per thread
+const int kGradPacks = 1;  // 128-bit packs per thread
 
 /*! \brief flags of the gradient family (mshadow/tensor_cpu-inl.h:287-462) */
 const int kGradSmooth = 1;  //!< SmoothSoftmaxGrad: alpha is spread over the other classes
