@@ -63,6 +63,7 @@ int DispatchReducer(int reducer, F f) {
 
 namespace {
 const size_t kPatchLdsBudget = 40 * 1024;  // per workgroup
+const size_t kIm2ColLdsBudget = 40 * 1024;  // input rows staged per workgroup
 /* reductions long enough to fill the LDS ring of the direct-to-LDS kernels (which hold
    a whole CU's LDS); shorter ones run the register-staged kernels, several per CU */
 const int kDmaMinRows = 2048;
@@ -105,7 +106,7 @@ int Im2Col(T *col, int cstride, const T *img, int istride, const PatchGeom &g, v
   const int EPT = 16 / sizeof(T);
   /* tiled: padded input rows of a band of patch rows must fit the LDS budget */
   const size_t row_bytes = static_cast<size_t>(g.wp) * sizeof(T);
-  const long long max_rows = static_cast<long long>(kPatchLdsBudget / row_bytes);
+  const long long max_rows = static_cast<long long>(kIm2ColLdsBudget / row_bytes);
   const long long halo = static_cast<long long>(g.ky - 1) * g.dy + 1;
   long long band = max_rows >= halo ? (max_rows - halo) / g.sy + 1 : 0;
   if (band > g.oh) band = g.oh;
