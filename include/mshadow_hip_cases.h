@@ -67,6 +67,12 @@ int mshadow_case_rows_by_index_f32(int op, float *dst, int dstride, int k_rows, 
                                    const int *index, int n_index, const float *src, int sstride,
                                    int src_rows, int cols, void *stream);
 
+/* broadcast<1> / repmat / reshape / swapaxis / mirror / upsampling_nearest /
+   broadcast_scalar expressions over a dense (n, c, h, w) input `a` and a vector `v`
+   (op 0..9, listed with the expression each evaluates in cases.hip) */
+int mshadow_case_shaping_f32(int op, float *out, const float *a, const float *v, int n, int c,
+                             int h, int w, void *stream);
+
 /* dst = pool<Reducer>(src, Shape2(ph, pw), ky, kx, sy, sx) */
 int mshadow_case_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes,
                           int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,

@@ -91,6 +91,7 @@ CASES_SYMBOLS = {
     "mshadow_case_grad_family_f32": ([_p, _i, _p, _i, _p, _i, _i, _i, _i, _i, _f, _f, _p], _i),
     "mshadow_case_softmax3d_f32": ([_p, _i, _p, _i, _i, _i, _i, _p], _i),
     "mshadow_case_rows_by_index_f32": ([_i, _p, _i, _i, _p, _p, _i, _p, _i, _i, _i, _p], _i),
+    "mshadow_case_shaping_f32": ([_i, _p, _p, _p, _i, _i, _i, _i, _p], _i),
     "mshadow_case_softmax_grad_f32": ([_p, _i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_case_pool_f32": ([_p, _i, _p, _i] + [_i] * 11 + [_p], _i),
     "mshadow_case_unpool_f32": ([_p, _i, _p, _i, _p, _i, _p, _i] + [_i] * 11 + [_p], _i),
@@ -361,6 +362,10 @@ class Library:
         self.check_case(self.cases.mshadow_case_rows_by_index_f32(
             op, dst.ptr, dst.stride, dst.rows, sorted_rows.ptr if sorted_rows is not None else None,
             index.ptr, index.cols, src.ptr, src.stride, src.rows, src.cols, stream))
+
+    def case_shaping(self, op, out, a, v, n, c, h, w, stream=None):
+        self.check_case(self.cases.mshadow_case_shaping_f32(op, out.ptr, a.ptr, v.ptr, n, c, h, w,
+                                                            stream))
 
     def case_reduce_keep_lowest(self, dst, src, reducer=SUM, saver=SAVETO, scale=1.0, variant=0,
                                 stream=None):

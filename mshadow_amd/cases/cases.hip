@@ -231,6 +231,57 @@ int mshadow_case_rows_by_index_f32(int op, float *dst, int dstride, int k_rows, 
   CASE_END
 }
 
+/* index-remapping extensions through the generic expression kernel; dense tensors */
+int mshadow_case_shaping_f32(int op, float *out, const float *a, const float *v, int n, int c,
+                             int h, int w, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+#define OUT4(d0, d1, d2, d3) G4(out, d0, d1, d2, d3, d3, st.get())
+#define OUT2(d0, d1) G2(out, d0, d1, d1, st.get())
+#define IN4(d0, d1, d2, d3) G4(a, d0, d1, d2, d3, d3, st.get())
+#define IN2(d0, d1) G2(a, d0, d1, d1, st.get())
+#define VEC(len) G1(v, len, st.get())
+  /* a: (n, c, h, w) contiguous input; v: c values; out: result, shape depends on op */
+  switch (op) {
+    case 0:   // bias add over channels, the convnet's `nhidden += broadcast<1>(hbias, shape)`
+      OUT4(n, c, h, w) = IN4(n, c, h, w) + broadcast<1>(VEC(c), Shape4(n, c, h, w));
+      break;
+    case 1:   // row bias, `nout += repmat(obias, batch)` on the (n*c*h, w) view with w values
+      OUT2(n * c * h, w) = IN2(n * c * h, w) + repmat(VEC(w), n * c * h);
+      break;
+    case 2:   // (c, n, h, w) -> (n, c, h, w), the convnet's conv forward epilogue
+      OUT4(c, n, h, w) = swapaxis<1, 0>(reshape(IN2(n, c * h * w), Shape4(n, c, h, w)));
+      break;
+    case 3:   // the inverse direction, chained into a 2-D result
+      OUT2(c, n * h * w) = reshape(swapaxis<1, 0>(IN4(n, c, h, w)), Shape2(c, n * h * w));
+      break;
+    case 4:   // swap the last dimension with the second
+      OUT4(n, w, h, c) = swapaxis<3, 1>(IN4(n, c, h, w));
+      break;
+    case 5:   // swap two middle dimensions
+      OUT4(n, h, c, w) = swapaxis<2, 1>(IN4(n, c, h, w));
+      break;
+    case 6:
+      OUT4(n, c, h, w) = mirror(IN4(n, c, h, w));
+      break;
+    case 7:
+      OUT4(n, c, h * 2, w * 2) = upsampling_nearest(IN4(n, c, h, w), 2);
+      break;
+    case 8:   // scalar broadcast scaled
+      OUT4(n, c, h, w) = broadcast_scalar(VEC(1), Shape4(n, c, h, w)) * IN4(n, c, h, w);
+      break;
+    default:  // reshape of a vector expression
+      OUT2(n * c, h * w) = reshape(VEC(n * c * h * w) * 2.0f, Shape2(n * c, h * w));
+      break;
+  }
+#undef OUT4
+#undef OUT2
+#undef IN4
+#undef IN2
+#undef VEC
+  CASE_END
+}
+
 int mshadow_case_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes,
                           int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,
                           int reducer, int variant, void *stream) {

@@ -5,4 +5,5 @@
 #include "./ext/reduceto1d.h"
 #include "./ext/pooling.h"
 #include "./ext/patches.h"
+#include "./ext/shaping.h"
 #endif  // MSHADOW_EXTENSION_H_

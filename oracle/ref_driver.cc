@@ -203,6 +203,55 @@ void ref_index_fill_f32(float *dst, int dstride, const void *index, int index_is
   }
 }
 
+/* index-remapping extensions (broadcast, repmat, reshape, swapaxis, mirror,
+   upsampling_nearest): the same expressions the GPU cases library evaluates */
+void ref_shaping_f32(int op, float *out, const float *a, const float *v, int n, int c, int h,
+                     int w) {
+#define OUT4(d0, d1, d2, d3) T4(out, d0, d1, d2, d3, d3)
+#define OUT2(d0, d1) T2(out, d0, d1, d1)
+#define IN4(d0, d1, d2, d3) T4(a, d0, d1, d2, d3, d3)
+#define IN2(d0, d1) T2(a, d0, d1, d1)
+#define VEC(len) T1(v, len)
+  /* a: (n, c, h, w) contiguous input; v: c values; out: result, shape depends on op */
+  switch (op) {
+    case 0:   // bias add over channels, the convnet's `nhidden += broadcast<1>(hbias, shape)`
+      OUT4(n, c, h, w) = IN4(n, c, h, w) + broadcast<1>(VEC(c), Shape4(n, c, h, w));
+      break;
+    case 1:   // row bias, `nout += repmat(obias, batch)` on the (n*c*h, w) view with w values
+      OUT2(n * c * h, w) = IN2(n * c * h, w) + repmat(VEC(w), n * c * h);
+      break;
+    case 2:   // (c, n, h, w) -> (n, c, h, w), the convnet's conv forward epilogue
+      OUT4(c, n, h, w) = swapaxis<1, 0>(reshape(IN2(n, c * h * w), Shape4(n, c, h, w)));
+      break;
+    case 3:   // the inverse direction, chained into a 2-D result
+      OUT2(c, n * h * w) = reshape(swapaxis<1, 0>(IN4(n, c, h, w)), Shape2(c, n * h * w));
+      break;
+    case 4:   // swap the last dimension with the second
+      OUT4(n, w, h, c) = swapaxis<3, 1>(IN4(n, c, h, w));
+      break;
+    case 5:   // swap two middle dimensions
+      OUT4(n, h, c, w) = swapaxis<2, 1>(IN4(n, c, h, w));
+      break;
+    case 6:
+      OUT4(n, c, h, w) = mirror(IN4(n, c, h, w));
+      break;
+    case 7:
+      OUT4(n, c, h * 2, w * 2) = upsampling_nearest(IN4(n, c, h, w), 2);
+      break;
+    case 8:   // scalar broadcast scaled
+      OUT4(n, c, h, w) = broadcast_scalar(VEC(1), Shape4(n, c, h, w)) * IN4(n, c, h, w);
+      break;
+    default:  // reshape of a vector expression
+      OUT2(n * c, h * w) = reshape(VEC(n * c * h * w) * 2.0f, Shape2(n * c, h * w));
+      break;
+  }
+#undef OUT4
+#undef OUT2
+#undef IN4
+#undef IN2
+#undef VEC
+}
+
 void ref_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes, int h, int w,
                   int ph, int pw, int ky, int kx, int sy, int sx, int reducer) {
   Tensor<cpu, 3, float> S = T3(src, planes, h, w, sstride);

@@ -83,6 +83,8 @@ class Checker:
         self._fn("add_take_grad_f32", [_p, _i, _i, _p, _i, _i, _p, _i, _i])
         self._fn("add_take_grad_large_batch_f32", [_p, _i, _p, _p, _i, _i, _p, _i, _i])
         self._fn("index_fill_f32", [_p, _i, _p, _i, _i, _p, _i, _i])
+        if self.prefix == "ref":
+            self._fn("shaping_f32", [_i, _p, _p, _p, _i, _i, _i, _i])
         self._fn("pool_f32", [_p, _i, _p, _i] + [_i] * 10)
         self._fn("unpool_f32", [_p, _i, _p, _i, _p, _i, _p, _i] + [_i] * 10)
         for t in ("f16", "f32"):
@@ -188,6 +190,11 @@ class Checker:
         self._index_fill_f32(ptr(dst), pitch(dst), ptr(index), self._is_int(index),
                              index.shape[0], ptr(src), pitch(src), src.shape[1])
         return dst
+
+    def shaping(self, op, out, a, v, n, c, h, w):
+        """reference build only: the index-remapping extension expressions"""
+        self._shaping_f32(op, ptr(out), ptr(a), ptr(v), n, c, h, w)
+        return out
 
     # -- pool / unpool: arrays are (..., H, W); leading dims are planes
     def pool(self, dst, src, ky, kx, sy, sx, reducer=MAX):

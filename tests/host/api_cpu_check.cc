@@ -299,6 +299,55 @@ int main() {
     orc_index_fill_f32(d2.data(), W, srt.data(), 1, N, src.data(), W, W);
     EXPECT(SameBits(d1.data(), d2.data(), d1.size()));
   }
+  // ---- index-remapping extensions on the CPU device, against plain index loops
+  {
+    const int n = 2, c = 3, h = 4, w = 5;
+    std::vector<float> a = Rand(n * c * h * w, 30), v = Rand(n * c * h * w, 31);
+    auto A = [&](int i, int j, int k, int l) { return a[((i * c + j) * h + k) * w + l]; };
+    Tensor<cpu, 4> In(a.data(), Shape4(n, c, h, w));
+    Tensor<cpu, 1> Vc(v.data(), Shape1(c)), Vw(v.data(), Shape1(w));
+    TensorContainer<cpu, 4> o(Shape4(n, c, h, w));
+    o = In + broadcast<1>(Vc, o.shape_);
+    bool ok = true;
+    for (int i = 0; i < n; ++i) for (int j = 0; j < c; ++j) for (int k = 0; k < h; ++k)
+      for (int l = 0; l < w; ++l) ok = ok && o[i][j][k][l] == A(i, j, k, l) + v[j];
+    EXPECT(ok);
+    TensorContainer<cpu, 2> o2(Shape2(n * c * h, w));
+    o2 = In.FlatTo2D() + repmat(Vw, n * c * h);
+    ok = true;
+    for (int r = 0; r < n * c * h; ++r) for (int l = 0; l < w; ++l) ok = ok && o2[r][l] == a[r * w + l] + v[l];
+    EXPECT(ok);
+    TensorContainer<cpu, 4> sw(Shape4(c, n, h, w));
+    sw = swapaxis<1, 0>(reshape(Tensor<cpu, 2>(a.data(), Shape2(n, c * h * w)), Shape4(n, c, h, w)));
+    ok = true;
+    for (int i = 0; i < n; ++i) for (int j = 0; j < c; ++j) for (int k = 0; k < h; ++k)
+      for (int l = 0; l < w; ++l) ok = ok && sw[j][i][k][l] == A(i, j, k, l);
+    EXPECT(ok);
+    TensorContainer<cpu, 4> s31(Shape4(n, w, h, c)), s21(Shape4(n, h, c, w)), mi(Shape4(n, c, h, w)),
+        up(Shape4(n, c, 2 * h, 2 * w));
+    s31 = swapaxis<3, 1>(In);
+    s21 = swapaxis<2, 1>(In);
+    mi = mirror(In);
+    up = upsampling_nearest(In, 2);
+    ok = true;
+    for (int i = 0; i < n; ++i) for (int j = 0; j < c; ++j) for (int k = 0; k < h; ++k)
+      for (int l = 0; l < w; ++l) {
+        ok = ok && s31[i][l][k][j] == A(i, j, k, l) && s21[i][k][j][l] == A(i, j, k, l) &&
+             mi[i][j][k][w - 1 - l] == A(i, j, k, l) && up[i][j][2 * k + 1][2 * l] == A(i, j, k, l) &&
+             up[i][j][2 * k][2 * l + 1] == A(i, j, k, l);
+      }
+    EXPECT(ok);
+    // guide/basic.cpp:127-134 of the reference: sum-pooling an upsampled tensor gives 9 x the source
+    TensorContainer<cpu, 4> pooled(Shape4(n, c, h, w)), up3(Shape4(n, c, 3 * h, 3 * w));
+    up3 = upsampling_nearest(In, 3);
+    pooled = pool<red::sum>(up3, 3, 3, 3, 3);
+    EXPECT(std::fabs(pooled[1][2][3][4] - 9.0f * A(1, 2, 3, 4)) < 1e-5f);
+    Tensor<cpu, 1> one(v.data(), Shape1(1));
+    o = broadcast_scalar(one, o.shape_) * In;
+    EXPECT(o[1][1][1][1] == v[0] * A(1, 1, 1, 1));
+    EXPECT(Throws([&] { o = In + broadcast<1>(Vw, o.shape_); }));          // length != shape[1]
+    EXPECT(Throws([&] { o2 = reshape(In, Shape2(n * c * h, w + 1)); }));    // size mismatch
+  }
   if (g_fail) {
     fprintf(stderr, "%d of %d checks failed\n", g_fail, g_checks);
     return 1;
