@@ -51,6 +51,8 @@ def algorithmic_bytes():
         "softmax3d": 2 * e * 256 * 21 * 16384,
         "softmax3d_grad": 2 * e * 256 * 21 * 16384 + e * 256 * 16384,
         "add_take_grad": e * 16384 + 3 * e * 16384 * 512,
+        "bias_add_broadcast": 2 * e * 64 * 256 * 56 * 56 + e * 256,
+        "swapaxis10_reshape": 2 * e * 64 * 256 * 56 * 56,
     }
 
 
@@ -62,10 +64,12 @@ def work_elements():
         "im2col_f16": 2304 * 100352, "col2im_f16": 2304 * 100352, "calib_copy": 4096 * 4096,
         "smooth_softmax_grad_ignore": 8192 * 32000, "softmax3d": 256 * 21 * 16384,
         "softmax3d_grad": 256 * 21 * 16384, "add_take_grad": 16384 * 512,
+        "bias_add_broadcast": 64 * 256 * 56 * 56, "swapaxis10_reshape": 64 * 256 * 56 * 56,
     }
 
 
-EXTRA_OPS = ("calib_copy", "smooth_softmax_grad_ignore", "softmax3d", "softmax3d_grad", "add_take_grad")
+EXTRA_OPS = ("calib_copy", "smooth_softmax_grad_ignore", "softmax3d", "softmax3d_grad", "add_take_grad",
+             "bias_add_broadcast", "swapaxis10_reshape")
 OPS = [k for k in algorithmic_bytes() if k not in EXTRA_OPS]
 
 # HBM bytes per launch of each operation's kernel, measured with rocprofv3 --pmc FETCH_SIZE and
@@ -160,8 +164,16 @@ def main():
         extra["idx"] = G.to_device(rng.integers(0, 50000, 16384).astype(np.int32))
         extra["rows"] = G.to_device(rng.standard_normal((16384, 512), dtype=f32))
 
+    if any(o in ("bias_add_broadcast", "swapaxis10_reshape") for o in only):
+        extra["out4"] = G.buffer(H["X2a"].shape, f32)
+        extra["bias"] = G.to_device(np.random.default_rng(14).standard_normal(51380224, dtype=f32)[:256].copy())
+
     def run_op(name):
-        if name == "smooth_softmax_grad_ignore":
+        if name == "bias_add_broadcast":
+            G.case_shaping(0, extra["out4"], dev["X2a"], extra["bias"], 64, 256, 56, 56, s)
+        elif name == "swapaxis10_reshape":
+            G.case_shaping(2, extra["out4"], dev["X2a"], extra["bias"], 64, 256, 56, 56, s)
+        elif name == "smooth_softmax_grad_ignore":
             G.softmax_grad_ex(out_g, out_p, dev["labels"], 3, 17.0, 0.1, s)
         elif name == "softmax3d":
             G.softmax3d(extra["p3"], extra["x3"], s)

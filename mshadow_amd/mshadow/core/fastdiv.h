@@ -30,6 +30,8 @@ struct FastDivU32 {
       shift = p - 32;
     }
   }
+  /*! \brief e % d */
+  MSHADOW_XINLINE uint32_t Mod(uint32_t e) const { return e - Div(e) * div; }
   MSHADOW_XINLINE uint32_t Div(uint32_t e) const {
     if (div == 1) return e;
 #if defined(__HIP_DEVICE_COMPILE__)

@@ -17,6 +17,7 @@
 #ifndef MSHADOW_EXT_SHAPING_H_
 #define MSHADOW_EXT_SHAPING_H_
 
+#include "../core/fastdiv.h"
 #include "../tensor.h"
 
 namespace mshadow {
@@ -72,12 +73,12 @@ struct Plan<Broadcast1DExp<SrcExp, DType, dimdst, dimdst_m_cast>, DType> {
       : src_(MakePlan(e.src_)), below_(e.shape_.ProdShape(dimcast + 1, dimdst - 1)),
         length_(e.shape_[dimcast]) {}
   MSHADOW_XINLINE DType Eval(index_t y, index_t) const {
-    return src_.Eval(0, (y / below_) % length_);
+    return src_.Eval(0, length_.Mod(below_.Div(y)));
   }
 
  private:
   Plan<SrcExp, DType> src_;
-  const index_t below_, length_;
+  const FastDivU32 below_, length_;
 };
 /* the broadcast dimension is the last one: its index is the column */
 template <typename SrcExp, typename DType, int dimdst>
@@ -125,12 +126,14 @@ struct Plan<ReshapeExp<SrcExp, DType, dimdst, dimsrc>, DType> {
   MSHADOW_XINLINE DType Eval(index_t y, index_t x) const {
     const index_t flat = y * ocols_ + x;  // position in row-major order, the same on both sides
     if (dimsrc == 1) return src_.Eval(0, flat);
-    return src_.Eval(flat / icols_, flat % icols_);
+    const index_t row = icols_.Div(flat);
+    return src_.Eval(row, flat - row * icols_.div);
   }
 
  private:
   Plan<SrcExp, DType> src_;
-  const index_t ocols_, icols_;
+  const index_t ocols_;
+  const FastDivU32 icols_;
 };
 
 /* ------------------------------------------------------------------ swapaxis */
@@ -169,26 +172,26 @@ struct Plan<SwapAxisExp<SrcExp, DType, dimsrc, m_a1, a2>, DType> {
   MSHADOW_XINLINE DType Eval(index_t i, index_t j) const {
     if (m_a1 == 1) {
       /* the swapped-in dimension is the column: row = (outer, P, mid), column = Q */
-      const index_t mid = i % mid_;
-      const index_t rest = i / mid_;
-      const index_t p = rest % p_;
-      const index_t outer = rest / p_;
-      return src_.Eval((outer * q_ + j) * mid_ + mid, p);
+      index_t rest = mid_.Div(i);
+      const index_t mid = i - rest * mid_.div;
+      const index_t outer = p_.Div(rest);
+      const index_t p = rest - outer * p_.div;
+      return src_.Eval((outer * q_.div + j) * mid_.div + mid, p);
     }
-    const index_t inner = i % inner_;
-    index_t rest = i / inner_;
-    const index_t q = rest % q_;
-    rest /= q_;
-    const index_t mid = rest % mid_;
-    rest /= mid_;
-    const index_t p = rest % p_;
-    const index_t outer = rest / p_;
-    return src_.Eval((((outer * q_ + q) * mid_ + mid) * p_ + p) * inner_ + inner, j);
+    index_t rest = inner_.Div(i);
+    const index_t inner = i - rest * inner_.div;
+    index_t next = q_.Div(rest);
+    const index_t q = rest - next * q_.div;
+    rest = mid_.Div(next);
+    const index_t mid = next - rest * mid_.div;
+    const index_t outer = p_.Div(rest);
+    const index_t p = rest - outer * p_.div;
+    return src_.Eval((((outer * q_.div + q) * mid_.div + mid) * p_.div + p) * inner_.div + inner, j);
   }
 
  private:
   Plan<SrcExp, DType> src_;
-  const index_t inner_, q_, mid_, p_;
+  const FastDivU32 inner_, q_, mid_, p_;
 };
 
 /* ------------------------------------------------------------------ mirror */
@@ -243,13 +246,14 @@ struct Plan<UpSamplingNearestExp<SrcExp, DType, srcdim>, DType> {
       : src_(MakePlan(e.src_)), scale_(e.scale_), out_h_(e.shape_[srcdim - 2]),
         src_h_(e.shape_[srcdim - 2] / e.scale_) {}
   MSHADOW_XINLINE DType Eval(index_t i, index_t j) const {
-    const index_t plane = i / out_h_;
-    return src_.Eval(plane * src_h_ + (i % out_h_) / scale_, j / scale_);
+    const index_t plane = out_h_.Div(i);
+    return src_.Eval(plane * src_h_ + scale_.Div(i - plane * out_h_.div), scale_.Div(j));
   }
 
  private:
   Plan<SrcExp, DType> src_;
-  const index_t scale_, out_h_, src_h_;
+  const FastDivU32 scale_, out_h_;
+  const index_t src_h_;
 };
 
 }  // namespace expr

@@ -14,11 +14,13 @@
  *                Algorithmic traffic: (leaves + 1) * sizeof(DType) bytes per element,
  *                HBM-bound (5 * 4 B for dst = A*B + 0.5f*F<sigmoid>(C) - D).
  * MapScalarKernel any plan (chainers, transposes, caller-defined plans, unaligned or
- *                ragged rows): one element per thread-iteration, grid-stride.
+ *                ragged rows): one element per thread-iteration, grid-stride; the split of
+ *                the flat index into (row, column) is a multiply-high.
  */
 #ifndef MSHADOW_HIP_KERNELS_MAP_H_
 #define MSHADOW_HIP_KERNELS_MAP_H_
 
+#include "../../core/fastdiv.h"
 #include "../../expr/plan.h"
 #include "./common.h"
 
@@ -32,15 +34,22 @@ const int kMapBlock = 256;
 const int kPackUnroll = 4;
 const int kPackUnrollDeep = 8;
 
-template <typename Saver, typename DType, typename DPlan, typename SPlan>
+/*! \brief PER consecutive elements of one row per thread-iteration (PER divides cols): the
+ *  PER evaluations are independent, so their loads are in flight together, and where a
+ *  plan reads consecutive addresses the compiler merges them into one wide load. */
+template <typename Saver, typename DType, typename DPlan, typename SPlan, int PER>
 __global__ void __launch_bounds__(kMapBlock)
-    MapScalarKernel(DPlan dplan, SPlan splan, uint32_t rows, uint32_t cols) {
+    MapScalarKernel(DPlan dplan, SPlan splan, uint32_t rows, uint32_t cols, FastDivU32 div_cols) {
   const uint32_t total = rows * cols;
-  const uint32_t step = gridDim.x * kMapBlock;
-  for (uint32_t i = blockIdx.x * kMapBlock + threadIdx.x; i < total; i += step) {
-    const uint32_t y = i / cols;
+  const uint32_t step = gridDim.x * kMapBlock * PER;
+  for (uint32_t i = (blockIdx.x * kMapBlock + threadIdx.x) * PER; i < total; i += step) {
+    const uint32_t y = div_cols.Div(i);  // a multiply-high, not a hardware division
     const uint32_t x = i - y * cols;
-    Saver::template Save<DType>(dplan.REval(y, x), splan.Eval(y, x));
+    DType v[PER];
+#pragma unroll
+    for (int k = 0; k < PER; ++k) v[k] = splan.Eval(y, x + k);
+#pragma unroll
+    for (int k = 0; k < PER; ++k) Saver::template Save<DType>(dplan.REval(y, x + k), v[k]);
   }
 }
 

@@ -432,10 +432,19 @@ struct MapLauncher {
     uint32_t rows = shape[0], cols = shape[1];
     if (rows == 0 || cols == 0) return;
     uint32_t grid = 0;
-    MSHADOW_HIP_CALL(mshadow_hip_suggest_grid(static_cast<size_t>(rows) * cols, hip::kMapBlock,
-                                              32, &grid));
-    void *args[] = {&dplan, &splan, &rows, &cols};
-    Launch(hip::MapScalarKernel<Saver, DType, DPlan, SPlan>, grid, hip::kMapBlock, args, stream);
+    CHECK_LT(static_cast<uint64_t>(rows) * cols, 1ull << 31) << "MapExp<gpu>: too many elements";
+    FastDivU32 div_cols(cols);
+    void *args[] = {&dplan, &splan, &rows, &cols, &div_cols};
+    const size_t total = static_cast<size_t>(rows) * cols;
+    if (cols % 4 == 0) {
+      MSHADOW_HIP_CALL(mshadow_hip_suggest_grid(total / 4, hip::kMapBlock, 32, &grid));
+      Launch(hip::MapScalarKernel<Saver, DType, DPlan, SPlan, 4>, grid, hip::kMapBlock, args,
+             stream);
+    } else {
+      MSHADOW_HIP_CALL(mshadow_hip_suggest_grid(total, hip::kMapBlock, 32, &grid));
+      Launch(hip::MapScalarKernel<Saver, DType, DPlan, SPlan, 1>, grid, hip::kMapBlock, args,
+             stream);
+    }
   }
 };
 template <typename Saver, typename DType, typename DPlan, typename SPlan>
