@@ -18,6 +18,7 @@
 #ifndef MSHADOW_EXT_PATCHES_H_
 #define MSHADOW_EXT_PATCHES_H_
 
+#include "../core/fastdiv.h"
 #include "../tensor.h"
 
 namespace mshadow {
@@ -58,8 +59,8 @@ struct Plan<PaddingExp<SrcExp, DType, srcdim>, DType> {
         new_height_(e.shape_[srcdim - 2]), src_height_(e.src_height_),
         src_width_(e.src_width_) {}
   MSHADOW_XINLINE DType Eval(index_t i, index_t j) const {
-    const index_t y = i % new_height_;
-    const index_t plane = i / new_height_;
+    const index_t plane = new_height_.Div(i);
+    const index_t y = i - plane * new_height_.div;
     if (y < pad_y_ || j < pad_x_) return static_cast<DType>(0);
     const index_t h = y - pad_y_;
     const index_t w = j - pad_x_;
@@ -69,7 +70,9 @@ struct Plan<PaddingExp<SrcExp, DType, srcdim>, DType> {
 
  private:
   Plan<SrcExp, DType> src_;
-  const index_t pad_y_, pad_x_, new_height_, src_height_, src_width_;
+  const index_t pad_y_, pad_x_;
+  const FastDivU32 new_height_;
+  const index_t src_height_, src_width_;
 };
 
 /* ------------------------------------------------------------------ crop */
@@ -128,14 +131,16 @@ struct Plan<CroppingExp<SrcExp, DType, srcdim>, DType> {
       : src_(MakePlan(e.src_)), off_y_(e.pad_height_), off_x_(e.pad_width_),
         new_height_(e.shape_[srcdim - 2]), src_height_(e.src_height_) {}
   MSHADOW_XINLINE DType Eval(index_t i, index_t j) const {
-    const index_t y = i % new_height_;
-    const index_t plane = i / new_height_;
+    const index_t plane = new_height_.Div(i);
+    const index_t y = i - plane * new_height_.div;
     return src_.Eval(plane * src_height_ + y + off_y_, j + off_x_);
   }
 
  private:
   Plan<SrcExp, DType> src_;
-  const index_t off_y_, off_x_, new_height_, src_height_;
+  const index_t off_y_, off_x_;
+  const FastDivU32 new_height_;
+  const index_t src_height_;
 };
 
 /* ------------------------------------------------------------------ unpack_patch2col */
@@ -187,24 +192,28 @@ struct Plan<UnpackPatchToColXExp<SrcExp, DType, srcdim>, DType> {
       : src_(MakePlan(e.img_)), ky_(e.psize_y_), kx_(e.psize_x_), sy_(e.pstride_y_),
         sx_(e.pstride_x_), dy_(e.pdilate_y_), dx_(e.pdilate_x_), ch_(e.i_channel_),
         h_(e.i_height_), w_(e.i_width_),
-        oh_((h_ - (dy_ * (ky_ - 1) + 1)) / sy_ + 1), ow_((w_ - (dx_ * (kx_ - 1) + 1)) / sx_ + 1) {}
+        oh_((h_ - (dy_ * (e.psize_y_ - 1) + 1)) / sy_ + 1),
+        ow_((w_ - (dx_ * (e.psize_x_ - 1) + 1)) / sx_ + 1) {}
   MSHADOW_XINLINE DType Eval(index_t i, index_t j) const {
     /* row i -> (channel, tap y, tap x); column j -> (image, out y, out x) */
-    const index_t tap_x = (i % kx_) * dx_;
-    const index_t i_rest = i / kx_;
-    const index_t tap_y = (i_rest % ky_) * dy_;
-    const index_t c = i_rest / ky_;
-    const index_t x = (j % ow_) * sx_ + tap_x;
-    const index_t j_rest = j / ow_;
-    const index_t y = (j_rest % oh_) * sy_ + tap_y;
-    const index_t n = j_rest / oh_;
+    const index_t i_rest = kx_.Div(i);
+    const index_t tap_x = (i - i_rest * kx_.div) * dx_;
+    const index_t c = ky_.Div(i_rest);
+    const index_t tap_y = (i_rest - c * ky_.div) * dy_;
+    const index_t j_rest = ow_.Div(j);
+    const index_t x = (j - j_rest * ow_.div) * sx_ + tap_x;
+    const index_t n = oh_.Div(j_rest);
+    const index_t y = (j_rest - n * oh_.div) * sy_ + tap_y;
     if (x < w_ && y < h_) return src_.Eval((n * ch_ + c) * h_ + y, x);
     return DType(0.0f);
   }
 
  private:
   Plan<SrcExp, DType> src_;
-  const index_t ky_, kx_, sy_, sx_, dy_, dx_, ch_, h_, w_, oh_, ow_;
+  /* members in order of initialisation; the divisors of Eval as multiply-high constants */
+  const FastDivU32 ky_, kx_;
+  const index_t sy_, sx_, dy_, dx_, ch_, h_, w_;
+  const FastDivU32 oh_, ow_;
 };
 
 /* ------------------------------------------------------------------ pack_col2patch */
@@ -259,27 +268,28 @@ struct Plan<PackColToPatchXExp<SrcExp, DType, dstdim>, DType> {
       : src_(MakePlan(e.src_)), ky_(e.psize_y_), kx_(e.psize_x_), sy_(e.pstride_y_),
         sx_(e.pstride_x_), dy_(e.pdilate_y_), dx_(e.pdilate_x_), ch_(e.shape_[dstdim - 3]),
         h_(e.shape_[dstdim - 2]),
-        oh_((e.shape_[dstdim - 2] - (dy_ * (ky_ - 1) + 1)) / sy_ + 1),
-        ow_((e.shape_[dstdim - 1] - (dx_ * (kx_ - 1) + 1)) / sx_ + 1) {}
+        oh_((e.shape_[dstdim - 2] - (dy_.div * (ky_ - 1) + 1)) / sy_.div + 1),
+        ow_((e.shape_[dstdim - 1] - (dx_.div * (kx_ - 1) + 1)) / sx_.div + 1) {}
   MSHADOW_XINLINE DType Eval(index_t i, index_t j) const {
-    const index_t y = i % h_;
-    const index_t i_rest = i / h_;
-    const index_t c = i_rest % ch_;
-    const index_t n = i_rest / ch_;
+    const index_t i_rest = h_.Div(i);
+    const index_t y = i - i_rest * h_.div;
+    const index_t n = ch_.Div(i_rest);
+    const index_t c = i_rest - n * ch_.div;
     const index_t x = j;
-    const index_t span_y = dy_ * (ky_ - 1) + 1;
-    const index_t span_x = dx_ * (kx_ - 1) + 1;
+    const index_t sy = sy_.div, sx = sx_.div, dy = dy_.div, dx = dx_.div;
+    const index_t span_y = dy * (ky_ - 1) + 1;
+    const index_t span_x = dx * (kx_ - 1) + 1;
     /* patches whose (dilated) extent reaches this pixel */
-    const index_t py0 = y < span_y ? y % dy_ : (y - span_y + sy_) / sy_;
-    const index_t px0 = x < span_x ? x % dx_ : (x - span_x + sx_) / sx_;
-    index_t py1 = (y + sy_) / sy_;
-    index_t px1 = (x + sx_) / sx_;
+    const index_t py0 = y < span_y ? dy_.Mod(y) : sy_.Div(y - span_y + sy);
+    const index_t px0 = x < span_x ? dx_.Mod(x) : sx_.Div(x - span_x + sx);
+    index_t py1 = sy_.Div(y + sy);
+    index_t px1 = sx_.Div(x + sx);
     if (py1 > oh_) py1 = oh_;
     if (px1 > ow_) px1 = ow_;
     DType res = static_cast<DType>(0);
-    for (index_t py = py0; py < py1; py += dy_) {
-      for (index_t px = px0; px < px1; px += dx_) {
-        res += src_.Eval((c * ky_ + (y - py * sy_) / dy_) * kx_ + (x - px * sx_) / dx_,
+    for (index_t py = py0; py < py1; py += dy) {
+      for (index_t px = px0; px < px1; px += dx) {
+        res += src_.Eval((c * ky_ + dy_.Div(y - py * sy)) * kx_ + dx_.Div(x - px * sx),
                          (n * oh_ + py) * ow_ + px);
       }
     }
@@ -288,7 +298,9 @@ struct Plan<PackColToPatchXExp<SrcExp, DType, dstdim>, DType> {
 
  private:
   Plan<SrcExp, DType> src_;
-  const index_t ky_, kx_, sy_, sx_, dy_, dx_, ch_, h_, oh_, ow_;
+  const index_t ky_, kx_;
+  const FastDivU32 sy_, sx_, dy_, dx_, ch_, h_;
+  const index_t oh_, ow_;
 };
 
 }  // namespace expr

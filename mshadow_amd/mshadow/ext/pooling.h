@@ -16,6 +16,7 @@
 #ifndef MSHADOW_EXT_POOLING_H_
 #define MSHADOW_EXT_POOLING_H_
 
+#include "../core/fastdiv.h"
 #include "../tensor.h"
 
 namespace mshadow {
@@ -81,8 +82,8 @@ struct Plan<PoolingExp<Reducer, SrcExp, DType, srcdim>, DType> {
       : src_(MakePlan(e.src_)), ky_(e.ksize_y_), kx_(e.ksize_x_), sy_(e.kstride_y_),
         sx_(e.kstride_x_), h_(e.src_height_), w_(e.src_width_), ph_(e.shape_[srcdim - 2]) {}
   MSHADOW_XINLINE DType Eval(index_t i, index_t j) const {
-    const index_t plane = i / ph_;
-    const index_t y0 = (i % ph_) * sy_;
+    const index_t plane = ph_.Div(i);
+    const index_t y0 = (i - plane * ph_.div) * sy_;
     const index_t x0 = j * sx_;
     const index_t y1 = (y0 + ky_ < h_) ? y0 + ky_ : h_;
     const index_t x1 = (x0 + kx_ < w_) ? x0 + kx_ : w_;
@@ -96,7 +97,8 @@ struct Plan<PoolingExp<Reducer, SrcExp, DType, srcdim>, DType> {
 
  private:
   Plan<SrcExp, DType> src_;
-  const index_t ky_, kx_, sy_, sx_, h_, w_, ph_;
+  const index_t ky_, kx_, sy_, sx_, h_, w_;
+  const FastDivU32 ph_;
 };
 
 template <typename Reducer, typename SrcExp, typename DType, int srcdim>
@@ -145,14 +147,14 @@ struct Plan<UnPoolingExp<Reducer, SrcExp, DType, srcdim>, DType> {
         pw_(e.pshape_x_), ky_(e.ksize_y_), kx_(e.ksize_x_), sy_(e.kstride_y_),
         sx_(e.kstride_x_) {}
   MSHADOW_XINLINE DType Eval(index_t i, index_t j) const {
-    const index_t y = i % h_;
-    const index_t plane = i / h_;
+    const index_t plane = h_.Div(i);
+    const index_t y = i - plane * h_.div;
     const DType vsrc = src_.Eval(i, j);
     /* first and one-past-last window index whose extent [p*s, p*s + k) contains the pixel */
-    const index_t py0 = y < ky_ ? 0 : (y - ky_ + sy_) / sy_;
-    const index_t px0 = j < kx_ ? 0 : (j - kx_ + sx_) / sx_;
-    index_t py1 = (y + sy_) / sy_;
-    index_t px1 = (j + sx_) / sx_;
+    const index_t py0 = y < ky_ ? 0 : sy_.Div(y - ky_ + sy_.div);
+    const index_t px0 = j < kx_ ? 0 : sx_.Div(j - kx_ + sx_.div);
+    index_t py1 = sy_.Div(y + sy_.div);
+    index_t px1 = sx_.Div(j + sx_.div);
     if (py1 > ph_) py1 = ph_;
     if (px1 > pw_) px1 = pw_;
     DType val = static_cast<DType>(0);
@@ -167,7 +169,9 @@ struct Plan<UnPoolingExp<Reducer, SrcExp, DType, srcdim>, DType> {
 
  private:
   Plan<SrcExp, DType> src_, pooled_, grad_;
-  const index_t h_, ph_, pw_, ky_, kx_, sy_, sx_;
+  const FastDivU32 h_;
+  const index_t ph_, pw_, ky_, kx_;
+  const FastDivU32 sy_, sx_;
 };
 
 }  // namespace expr
