@@ -73,6 +73,16 @@ int mshadow_case_rows_by_index_f32(int op, float *dst, int dstride, int k_rows, 
 int mshadow_case_shaping_f32(int op, float *out, const float *a, const float *v, int n, int c,
                              int h, int w, void *stream);
 
+/* chpool / ch_unpool, reduce_with_axis / reduce_keepdim, broadcast_with_axis /
+   broadcast_keepdim, transpose / transpose_indices, concat / slice / flip (also as the
+   target of an assignment), take / take_grad / one_hot_encode / mat_choose_row_element /
+   mat_fill_row_element / mask / range over a dense (n, ch, h, w) input `a`, operands `b`,
+   `c` and parameters p0..p2 (op 0..27, listed with the expression each evaluates in
+   cases.hip) */
+int mshadow_case_extensions_f32(int op, float *out, const float *a, const float *b, const float *c,
+                                int n, int ch, int h, int w, int p0, int p1, int p2,
+                                void *stream);
+
 /* dst = pool<Reducer>(src, Shape2(ph, pw), ky, kx, sy, sx) */
 int mshadow_case_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes,
                           int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,

@@ -92,6 +92,7 @@ CASES_SYMBOLS = {
     "mshadow_case_softmax3d_f32": ([_p, _i, _p, _i, _i, _i, _i, _p], _i),
     "mshadow_case_rows_by_index_f32": ([_i, _p, _i, _i, _p, _p, _i, _p, _i, _i, _i, _p], _i),
     "mshadow_case_shaping_f32": ([_i, _p, _p, _p, _i, _i, _i, _i, _p], _i),
+    "mshadow_case_extensions_f32": ([_i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p], _i),
     "mshadow_case_softmax_grad_f32": ([_p, _i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_case_pool_f32": ([_p, _i, _p, _i] + [_i] * 11 + [_p], _i),
     "mshadow_case_unpool_f32": ([_p, _i, _p, _i, _p, _i, _p, _i] + [_i] * 11 + [_p], _i),
@@ -366,6 +367,11 @@ class Library:
     def case_shaping(self, op, out, a, v, n, c, h, w, stream=None):
         self.check_case(self.cases.mshadow_case_shaping_f32(op, out.ptr, a.ptr, v.ptr, n, c, h, w,
                                                             stream))
+
+    def case_extensions(self, op, out, a, b, c, n, ch, h, w, p0=0, p1=0, p2=0, stream=None):
+        self.check_case(self.cases.mshadow_case_extensions_f32(
+            op, out.ptr, a.ptr, b.ptr if b is not None else None,
+            c.ptr if c is not None else None, n, ch, h, w, p0, p1, p2, stream))
 
     def case_reduce_keep_lowest(self, dst, src, reducer=SUM, saver=SAVETO, scale=1.0, variant=0,
                                 stream=None):

@@ -282,6 +282,27 @@ int mshadow_case_shaping_f32(int op, float *out, const float *a, const float *v,
   CASE_END
 }
 
+/* channel pooling, axis reductions / broadcasts, permutations, assignable views and the
+   index look-ups, through the generic expression kernel; dense tensors */
+int mshadow_case_extensions_f32(int op, float *out, const float *a, const float *b, const float *c,
+                                int n, int ch, int h, int w, int p0, int p1, int p2,
+                                void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+#define TENSOR(dim) Tensor<gpu, dim, float>
+#define V1(p, len) G1(p, len, st.get())
+#define V2(p, d0, d1) G2(p, d0, d1, d1, st.get())
+#define V3(p, d0, d1, d2) G3(p, d0, d1, d2, d2, st.get())
+#define V4(p, d0, d1, d2, d3) G4(p, d0, d1, d2, d3, d3, st.get())
+#include "./extension_cases.inc"
+#undef TENSOR
+#undef V1
+#undef V2
+#undef V3
+#undef V4
+  CASE_END
+}
+
 int mshadow_case_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes,
                           int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,
                           int reducer, int variant, void *stream) {

@@ -6,4 +6,7 @@
 #include "./ext/pooling.h"
 #include "./ext/patches.h"
 #include "./ext/shaping.h"
+#include "./ext/channels.h"
+#include "./ext/axes.h"
+#include "./ext/indexing.h"
 #endif  // MSHADOW_EXTENSION_H_

@@ -1,0 +1,2 @@
+/*! \file take_grad.h  include name kept for callers; the code lives under ../ext/ */
+#include "../extension.h"

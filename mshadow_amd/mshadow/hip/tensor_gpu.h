@@ -416,6 +416,19 @@ struct FastPath<sv::saveto, ddim, DType,
   }
 };
 
+/*! \brief the fixed-function routes write into plain tensors; an assignable view as the
+ *  target (slice, concat, flip) always takes the generic kernel */
+template <typename Saver, typename R, int dim, typename DType, typename E>
+struct FastPathFor {
+  inline static bool Run(R *, const E &) { return false; }
+};
+template <typename Saver, int dim, typename DType, typename E>
+struct FastPathFor<Saver, Tensor<gpu, dim, DType>, dim, DType, E> {
+  inline static bool Run(Tensor<gpu, dim, DType> *dst, const E &exp) {
+    return FastPath<Saver, dim, DType, E>::Run(dst, exp);
+  }
+};
+
 #if defined(__HIPCC__)
 template <typename K>
 inline void Launch(K kernel, uint32_t grid_x, uint32_t block_x, void **args, void *stream) {
@@ -499,7 +512,7 @@ inline void MapExp(TRValue<R, gpu, dim, DType> *dst, const expr::Exp<E, DType, e
   CHECK(eshape[0] == 0 || eshape == dshape)
       << "Assignment: Shape of Tensors are not consistent with target, "
       << "eshape: " << eshape << " dshape:" << dshape;
-  if (gpu_detail::FastPath<Saver, dim, DType, E>::Run(dst->ptrself(), exp.self())) return;
+  if (gpu_detail::FastPathFor<Saver, R, dim, DType, E>::Run(dst->ptrself(), exp.self())) return;
 #if defined(__HIPCC__)
   typedef expr::Plan<R, DType> DPlan;
   typedef expr::Plan<E, DType> SPlan;

@@ -252,6 +252,23 @@ void ref_shaping_f32(int op, float *out, const float *a, const float *v, int n, 
 #undef VEC
 }
 
+void ref_extensions_f32(int op, float *out, const float *a, const float *b, const float *c, int n,
+                        int ch, int h, int w, int p0, int p1, int p2) {
+#define TENSOR(dim) Tensor<cpu, dim, float>
+#define V1(p, len) T1(p, len)
+#define V2(p, d0, d1) T2(p, d0, d1, d1)
+#define V3(p, d0, d1, d2) T3(p, d0, d1, d2, d2)
+#define V4(p, d0, d1, d2, d3) T4(p, d0, d1, d2, d3, d3)
+#define MSHADOW_CASES_REFERENCE_HEADERS
+#include "../mshadow_amd/cases/extension_cases.inc"
+#undef MSHADOW_CASES_REFERENCE_HEADERS
+#undef TENSOR
+#undef V1
+#undef V2
+#undef V3
+#undef V4
+}
+
 void ref_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes, int h, int w,
                   int ph, int pw, int ky, int kx, int sy, int sx, int reducer) {
   Tensor<cpu, 3, float> S = T3(src, planes, h, w, sstride);

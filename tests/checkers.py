@@ -85,6 +85,7 @@ class Checker:
         self._fn("index_fill_f32", [_p, _i, _p, _i, _i, _p, _i, _i])
         if self.prefix == "ref":
             self._fn("shaping_f32", [_i, _p, _p, _p, _i, _i, _i, _i])
+            self._fn("extensions_f32", [_i, _p, _p, _p, _p] + [_i] * 7)
         self._fn("pool_f32", [_p, _i, _p, _i] + [_i] * 10)
         self._fn("unpool_f32", [_p, _i, _p, _i, _p, _i, _p, _i] + [_i] * 10)
         for t in ("f16", "f32"):
@@ -194,6 +195,12 @@ class Checker:
     def shaping(self, op, out, a, v, n, c, h, w):
         """reference build only: the index-remapping extension expressions"""
         self._shaping_f32(op, ptr(out), ptr(a), ptr(v), n, c, h, w)
+        return out
+
+    def extensions(self, op, out, a, b, c, n, ch, h, w, p0=0, p1=0, p2=0):
+        """reference build only: channel pooling, axis, view and index look-up expressions"""
+        self._extensions_f32(op, ptr(out), ptr(a), ptr(b) if b is not None else None,
+                             ptr(c) if c is not None else None, n, ch, h, w, p0, p1, p2)
         return out
 
     # -- pool / unpool: arrays are (..., H, W); leading dims are planes

@@ -1,0 +1,36 @@
+// The extension expressions of mshadow_amd/cases/extension_cases.inc evaluated on
+// Tensor<cpu> of this backend's headers (plain g++, no GPU): built as a small shared
+// library by tests/test_extensions.py and compared with numpy there.
+#include <mshadow/tensor.h>
+
+using namespace mshadow;
+using namespace mshadow::expr;
+
+namespace {
+template <int dim>
+Tensor<cpu, dim, float> View(const float *p, Shape<dim> shape) {
+  return Tensor<cpu, dim, float>(const_cast<float *>(p), shape);
+}
+}  // namespace
+
+extern "C" int host_extensions_f32(int op, float *out, const float *a, const float *b,
+                                   const float *c, int n, int ch, int h, int w, int p0, int p1,
+                                   int p2) {
+  try {
+#define TENSOR(dim) Tensor<cpu, dim, float>
+#define V1(p, len) View(p, Shape1(len))
+#define V2(p, d0, d1) View(p, Shape2(d0, d1))
+#define V3(p, d0, d1, d2) View(p, Shape3(d0, d1, d2))
+#define V4(p, d0, d1, d2, d3) View(p, Shape4(d0, d1, d2, d3))
+#include "../../mshadow_amd/cases/extension_cases.inc"
+#undef TENSOR
+#undef V1
+#undef V2
+#undef V3
+#undef V4
+  } catch (const std::exception &e) {
+    fprintf(stderr, "%s\n", e.what());
+    return 1;
+  }
+  return 0;
+}

@@ -1,0 +1,251 @@
+"""chpool / ch_unpool, reduce_with_axis / reduce_keepdim, broadcast_with_axis / broadcast_keepdim,
+transpose / transpose_indices, concat / slice / flip (as values and as assignment targets),
+take / take_grad / one_hot_encode / mat_choose_row_element / mat_fill_row_element / mask / range:
+the expressions of mshadow_case_extensions_f32 against plain numpy index loops, on the
+reference build (CPU, where present) and on the GPU through the generic expression kernel.
+Every result is data movement or a short fixed-order float32 chain: bit for bit."""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from checkers import have_ref
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+f32 = np.float32
+SHAPES = [(2, 6, 3, 5), (3, 5, 2, 8), (1, 7, 1, 4)]
+BIG = (8, 16, 14, 28)
+
+
+# ---- numpy statements of what each node means (mshadow/extension/*.h of the reference)
+def _chpool(a, nsize, stride, pad, reducer):
+    n, ch, h, w = a.shape
+    pc = (ch - nsize + 2 * pad + 1) // stride
+    init = f32(0) if reducer == "sum" else f32(-np.finfo(f32).max)
+    out = np.full((n, pc, h, w), init, f32)
+    for c in range(pc):
+        first = max(c * stride - pad, 0)
+        last = min(c * stride - pad + nsize, pc, ch)   # cut at the pooled channel count
+        for cc in range(first, last):
+            out[:, c] = out[:, c] + a[:, cc] if reducer == "sum" else np.maximum(out[:, c], a[:, cc])
+    return out
+
+
+def _ch_unpool(a, pooled, grad, nsize, stride, pad, reducer):
+    n, ch, h, w = a.shape
+    out = np.zeros_like(a)
+    for c in range(ch):
+        reach = nsize - pad
+        first = 0 if c < reach else (c - reach + stride) // stride
+        # cut at the source channel count (the reference stops there and can run past the
+        # pooled tensor; this backend also stops at the pooled channel count)
+        last = min((c + pad + stride) // stride, ch, pooled.shape[1])
+        for cc in range(first, last):
+            pg = np.ones_like(a[:, c]) if reducer == "sum" else (a[:, c] == pooled[:, cc]).astype(f32)
+            out[:, c] = out[:, c] + pg * grad[:, cc]
+    return out
+
+
+def _seq_reduce(a, axis, reducer):
+    moved = np.moveaxis(a, axis, 0)
+    if reducer == "sum":
+        res = np.zeros(moved.shape[1:], f32)
+        for k in range(moved.shape[0]):
+            res = res + moved[k]
+        return res
+    return moved.min(axis=0) if reducer == "min" else moved.max(axis=0)
+
+
+def _perm(p0):
+    return (p0 // 1000, p0 // 100 % 10, p0 // 10 % 10, p0 % 10)
+
+
+class Case(object):
+    """inputs, parameters and the expected output of one op on one shape"""
+
+    def __init__(self, op, shape):
+        n, ch, h, w = shape
+        rng = np.random.default_rng(1000 * op + sum(shape))
+        a = rng.standard_normal(shape).astype(f32)
+        self.op, self.shape, self.a = op, shape, a
+        self.b = self.c = None
+        self.p = (0, 0, 0)
+        rows = n * ch * h
+        if op == 0:
+            self.p = (3, 0, 0)
+            self.want = _chpool(a, 3, 1, 1, "sum")
+        elif op == 1:
+            self.p = (3, 2, 1)
+            self.want = _chpool(a, 3, 2, 1, "max")
+        elif op in (2, 3):
+            # window 5, pad 2 keeps the channel count (the only kind of window for which the
+            # reference stays inside the pooled tensor); the large shape, checked on the GPU
+            # only, uses a strided window
+            self.p = (3, 2, 1) if shape == BIG else (5, 1, 2)
+            red = "sum" if op == 2 else "max"
+            self.b = _chpool(a, *self.p, red)
+            self.c = rng.standard_normal(self.b.shape).astype(f32)
+            self.want = _ch_unpool(a, self.b, self.c, *self.p, red)
+        elif op == 4:
+            self.p = (1 + sum(shape) % 3, 0, 0)
+            self.want = _seq_reduce(a, self.p[0], "sum")
+        elif op == 5:
+            self.p = (sum(shape) % 4, 0, 0)
+            self.want = a.argmax(axis=self.p[0]).astype(f32)
+        elif op == 6:
+            self.p = ((sum(shape) + 1) % 4, 0, 0)
+            self.want = np.expand_dims(_seq_reduce(a, self.p[0], "min"), self.p[0])
+        elif op == 7:
+            self.p = ([2031, 3102, 1230][sum(shape) % 3], 0, 0)
+            self.want = a.transpose(_perm(self.p[0]))
+        elif op == 8:
+            k = ch // 2
+            self.p = (k, 0, 0)
+            two = a * f32(2)
+            self.want = np.concatenate([two[:, :k].ravel(), two[:, k:].ravel()])
+        elif op == 9:
+            self.p = (2, 0, 0)
+            self.b = rng.standard_normal((n, 2, h, w)).astype(f32)
+            self.want = np.concatenate([a, self.b], axis=1) + f32(1)
+        elif op == 10:
+            self.p = (1, ch - 1, 0)
+            self.want = a[:, 1:ch - 1]
+        elif op == 11:
+            self.p = (1, ch - 1, 0)
+            self.b = rng.standard_normal(shape).astype(f32)
+            self.c = rng.standard_normal((n, ch - 2, h, w)).astype(f32)
+            self.want = self.b.copy()
+            self.want[:, 1:ch - 1] = self.c * f32(3)
+        elif op == 12:
+            self.p = (3, 0, 0)
+            self.b = rng.standard_normal((n, ch, h, 3)).astype(f32)
+            self.want = np.concatenate([a, self.b], axis=3)
+        elif op == 13:
+            self.p = (1, w - 1, 0)
+            self.want = a[..., 1:w - 1]
+        elif op == 14:
+            self.p = (2, h - 1, 1)
+            self.want = a[:, 2:, h - 1:, 1:]
+        elif op == 15:
+            self.p = (sum(shape) % 4, 0, 0)
+            self.want = np.flip(a + f32(0.5), axis=self.p[0])
+        elif op == 16:
+            self.p = ((sum(shape) + 2) % 4, 0, 0)
+            self.want = np.flip(a, axis=self.p[0])
+        elif op == 17:
+            axis = sum(shape) % 4 - 1
+            self.p = (axis, 3, 0)
+            a3 = a.reshape(n * ch, h, w)
+            self.want = np.repeat(np.expand_dims(a3, axis + 1), 3, axis=axis + 1)
+        elif op == 18:
+            axis = sum(shape) % 4
+            self.p = (axis, 3, 0)
+            self.b = np.ascontiguousarray(np.take(a, [0], axis=axis))
+            self.want = np.repeat(self.b, 3, axis=axis)
+        elif op == 19:
+            self.p = (3, 0, 0)
+            self.want = a * (_chpool(a * a, 3, 1, 1, "sum") * f32(0.1) + f32(1))
+        elif op == 20:
+            k = 7
+            self.p = (k, 0, 0)
+            self.b = rng.integers(0, rows, k).astype(f32)
+            self.want = a.reshape(rows, w)[self.b.astype(int)]
+        elif op == 21:
+            k, dim = min(rows, 9), 4
+            self.p = (k, dim, 0)
+            self.b = rng.integers(0, dim, k).astype(f32)
+            src = a.reshape(rows, w)[:k]
+            self.want = np.zeros((dim, w), f32)
+            for i in range(k):
+                self.want[int(self.b[i])] = self.want[int(self.b[i])] + src[i]
+        elif op == 22:
+            k, choices = 6, 5
+            self.p = (k, choices, 0)
+            self.b = rng.integers(0, choices, k).astype(f32)
+            self.want = (np.arange(choices)[None, :] == self.b.astype(int)[:, None]).astype(f32)
+        elif op == 23:
+            self.b = rng.integers(0, w, rows).astype(f32)
+            self.want = a.reshape(rows, w)[np.arange(rows), self.b.astype(int)]
+        elif op == 24:
+            self.b = rng.integers(0, w, rows).astype(f32)
+            self.c = rng.standard_normal(rows).astype(f32)
+            self.want = a.reshape(rows, w).copy()
+            self.want[np.arange(rows), self.b.astype(int)] = self.c
+        elif op == 25:
+            self.b = rng.integers(0, 2, rows).astype(f32)
+            self.want = a.reshape(rows, w) * self.b[:, None]
+        elif op == 26:
+            self.p = (2, 2 + sum(shape), 3)
+            count = -(-(self.p[1] - self.p[0]) // self.p[2])
+            self.want = np.repeat(f32(self.p[0]) + np.arange(count).astype(f32) * f32(self.p[2]), 2)
+        else:
+            k = 11
+            perm = [2031, 3102, 1230][sum(shape) % 3]
+            self.p = (perm, k, 0)
+            flat = rng.integers(0, a.size, k)
+            self.b = flat.astype(f32)
+            pos = np.unravel_index(flat, shape)
+            axes = _perm(perm)
+            tshape = tuple(shape[x] for x in axes)
+            self.want = np.ravel_multi_index(tuple(pos[x] for x in axes), tshape).astype(f32)
+        self.want = np.ascontiguousarray(self.want, dtype=f32)
+
+
+N_OPS = 28
+
+
+@pytest.fixture(scope="module")
+def host_lib(tmp_path_factory):
+    """the same expressions on Tensor<cpu> of this backend's headers, compiled with g++"""
+    so = str(tmp_path_factory.mktemp("hostcases") / "libhostcases.so")
+    cmd = ["g++", "-std=c++17", "-O2", "-fopenmp", "-ffp-contract=off", "-mf16c", "-fPIC", "-shared",
+           "-DDMLC_LOG_FATAL_THROW=1", "-I", os.path.join(ROOT, "include"),
+           "-I", os.path.join(ROOT, "mshadow_amd"), "-o", so,
+           os.path.join(ROOT, "tests", "host", "ext_cpu_cases.cc")]
+    subprocess.run(cmd, check=True, capture_output=True, text=True)
+    lib = ctypes.CDLL(so)
+    fp = ctypes.c_void_p
+    lib.host_extensions_f32.argtypes = [ctypes.c_int, fp, fp, fp, fp] + [ctypes.c_int] * 7
+    return lib
+
+
+def _ptr(x):
+    return x.ctypes.data_as(ctypes.c_void_p) if x is not None else None
+
+
+@pytest.mark.parametrize("shape", SHAPES + [BIG])
+@pytest.mark.parametrize("op", range(N_OPS))
+def test_cpu_device_matches_numpy(host_lib, shape, op):
+    case = Case(op, shape)
+    out = np.full(case.want.shape, np.nan, f32)
+    rc = host_lib.host_extensions_f32(op, _ptr(out), _ptr(case.a), _ptr(case.b), _ptr(case.c),
+                                      *shape, *case.p)
+    assert rc == 0
+    assert np.array_equal(out.view(np.uint32), case.want.view(np.uint32)), (op, shape)
+
+
+@pytest.mark.skipif(not have_ref(), reason="reference build absent")
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("op", [o for o in range(N_OPS) if o != 15])
+def test_reference_build_matches_numpy(ref, shape, op):
+    case = Case(op, shape)
+    out = np.full(case.want.shape, np.nan, f32)
+    ref.extensions(op, out, case.a, case.b, case.c, *shape, *case.p)
+    assert np.array_equal(out.view(np.uint32), case.want.view(np.uint32)), (op, shape)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", SHAPES + [BIG])
+@pytest.mark.parametrize("op", range(N_OPS))
+def test_gpu_matches_numpy(shape, op):
+    import mshadow_amd
+    G = mshadow_amd.load_cases()
+    G.set_device(0)
+    case = Case(op, shape)
+    out = G.to_device(np.full(case.want.shape, np.nan, f32))
+    dev = lambda x: G.to_device(x) if x is not None else None
+    G.case_extensions(op, out, dev(case.a), dev(case.b), dev(case.c), *shape, *case.p)
+    got = out.download()
+    assert np.array_equal(got.view(np.uint32), case.want.view(np.uint32)), (op, shape)
