@@ -53,6 +53,9 @@ def algorithmic_bytes():
         "add_take_grad": e * 16384 + 3 * e * 16384 * 512,
         "bias_add_broadcast": 2 * e * 64 * 256 * 56 * 56 + e * 256,
         "swapaxis10_reshape": 2 * e * 64 * 256 * 56 * 56,
+        "lrn_scale_chpool5": 2 * e * 64 * 256 * 56 * 56,
+        "transpose_nchw_nhwc": 2 * e * 64 * 256 * 56 * 56,
+        "sort_by_key_f32": 4 * e * (1 << 24),
     }
 
 
@@ -65,11 +68,14 @@ def work_elements():
         "smooth_softmax_grad_ignore": 8192 * 32000, "softmax3d": 256 * 21 * 16384,
         "softmax3d_grad": 256 * 21 * 16384, "add_take_grad": 16384 * 512,
         "bias_add_broadcast": 64 * 256 * 56 * 56, "swapaxis10_reshape": 64 * 256 * 56 * 56,
+        "lrn_scale_chpool5": 64 * 256 * 56 * 56, "transpose_nchw_nhwc": 64 * 256 * 56 * 56,
+        "sort_by_key_f32": 1 << 24,
     }
 
 
 EXTRA_OPS = ("calib_copy", "smooth_softmax_grad_ignore", "softmax3d", "softmax3d_grad", "add_take_grad",
-             "bias_add_broadcast", "swapaxis10_reshape")
+             "bias_add_broadcast", "swapaxis10_reshape", "lrn_scale_chpool5", "transpose_nchw_nhwc",
+             "sort_by_key_f32")
 OPS = [k for k in algorithmic_bytes() if k not in EXTRA_OPS]
 
 # HBM bytes per launch of each operation's kernel, measured with rocprofv3 --pmc FETCH_SIZE and
@@ -164,7 +170,17 @@ def main():
         extra["idx"] = G.to_device(rng.integers(0, 50000, 16384).astype(np.int32))
         extra["rows"] = G.to_device(rng.standard_normal((16384, 512), dtype=f32))
 
-    if any(o in ("bias_add_broadcast", "swapaxis10_reshape") for o in only):
+    if "sort_by_key_f32" in only:
+        import ctypes
+        rng = np.random.default_rng(15)
+        extra["keys"] = G.to_device(rng.standard_normal(1 << 24, dtype=f32))
+        extra["vals"] = G.to_device(np.arange(1 << 24, dtype=np.int32))
+        need = ctypes.c_size_t(0)
+        G.check(G.dll.mshadow_hip_sort_by_key_workspace(1 << 24, ctypes.byref(need)))
+        extra["work"] = G.buffer((need.value,), np.uint8)
+        extra["work_bytes"] = need.value
+    if any(o in ("bias_add_broadcast", "swapaxis10_reshape", "lrn_scale_chpool5",
+                 "transpose_nchw_nhwc") for o in only):
         extra["out4"] = G.buffer(H["X2a"].shape, f32)
         extra["bias"] = G.to_device(np.random.default_rng(14).standard_normal(51380224, dtype=f32)[:256].copy())
 
@@ -173,6 +189,13 @@ def main():
             G.case_shaping(0, extra["out4"], dev["X2a"], extra["bias"], 64, 256, 56, 56, s)
         elif name == "swapaxis10_reshape":
             G.case_shaping(2, extra["out4"], dev["X2a"], extra["bias"], 64, 256, 56, 56, s)
+        elif name == "lrn_scale_chpool5":   # x * (chpool<sum>(x * x, 5) * 0.1 + 1)
+            G.case_extensions(19, extra["out4"], dev["X2a"], None, None, 64, 256, 56, 56, 5, 0, 0, s)
+        elif name == "transpose_nchw_nhwc":
+            G.case_extensions(7, extra["out4"], dev["X2a"], None, None, 64, 256, 56, 56, 231, 0, 0, s)
+        elif name == "sort_by_key_f32":     # 16M (float key, int value) pairs, ascending
+            G.check(G.dll.mshadow_hip_sort_by_key_32(extra["keys"].ptr, 0, extra["vals"].ptr, 1 << 24,
+                                                     1, extra["work"].ptr, extra["work_bytes"], s))
         elif name == "smooth_softmax_grad_ignore":
             G.softmax_grad_ex(out_g, out_p, dev["labels"], 3, 17.0, 0.1, s)
         elif name == "softmax3d":

@@ -182,6 +182,21 @@ int mshadow_hip_index_fill_f32(float *dst, int dstride, int k_rows, const void *
                                int index_is_int, int n_index, const float *src, int sstride,
                                int cols, void *stream);
 
+/* SortByKey(keys, values, is_ascend): stable sort of the pairs by key, in place
+   (mshadow/tensor_gpu-inl.h:231-235 -> tensor_gpu-inl.cuh:784-806, thrust::stable_sort_by_key;
+   CPU tensor_cpu-inl.h:531-559). Keys and values are 32-bit elements; key_kind says how the key
+   bits are ordered; values are moved as opaque words. Pairs of equivalent keys (+0.0f and
+   -0.0f are equivalent) keep their order in both directions. The scratch memory is the
+   caller's: `workspace` holds at least the number of bytes the first call reports for n and
+   is 256-byte aligned. VectorizedSort(values, segments) of the reference
+   (tensor_cpu-inl.h:561-566) is two of these calls. */
+#define MSHADOW_HIP_KEY_F32 0
+#define MSHADOW_HIP_KEY_I32 1
+#define MSHADOW_HIP_KEY_U32 2
+int mshadow_hip_sort_by_key_workspace(size_t n, size_t *bytes);
+int mshadow_hip_sort_by_key_32(void *keys, int key_kind, void *values, size_t n, int is_ascend,
+                               void *workspace, size_t workspace_bytes, void *stream);
+
 /* MapReduceKeepLowest<Saver, Reducer>(dst, src, scale): mshadow/tensor_gpu-inl.h:118-133
    -> MapRedKeepLowestKernel, tensor_gpu-inl.cuh:122-168. dst[x] <saver>= scale *
    reduce_y src[y][x], rows >= 1, reduced top to bottom like tensor_cpu-inl.h:221-227. */

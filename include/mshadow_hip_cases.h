@@ -73,6 +73,11 @@ int mshadow_case_rows_by_index_f32(int op, float *dst, int dstride, int k_rows, 
 int mshadow_case_shaping_f32(int op, float *out, const float *a, const float *v, int n, int c,
                              int h, int w, void *stream);
 
+/* op 0: SortByKey(keys, values, is_ascend); 1: VectorizedSort(keys, values as segment numbers).
+   key_kind 0: float keys with int values, 1: int keys with float values (int segments for op 1) */
+int mshadow_case_sort_by_key_32(int op, void *keys, int key_kind, void *values, int n,
+                                int is_ascend, void *stream);
+
 /* chpool / ch_unpool, reduce_with_axis / reduce_keepdim, broadcast_with_axis /
    broadcast_keepdim, transpose / transpose_indices, concat / slice / flip (also as the
    target of an assignment), take / take_grad / one_hot_encode / mat_choose_row_element /

@@ -17,6 +17,7 @@ CASES_SO = os.path.join(HERE, "lib", "libmshadow_cases.so")
 SAVETO, PLUSTO, MINUSTO, MULTO, DIVTO = range(5)
 SUM, MAX, MIN = range(3)
 H2D, D2H, D2D = 1, 2, 3
+KEY_F32, KEY_I32, KEY_U32 = range(3)
 
 _i, _f, _p, _sz = C.c_int, C.c_float, C.c_void_p, C.c_size_t
 
@@ -69,6 +70,8 @@ HIP_SYMBOLS = {
     "mshadow_hip_add_take_grad_f32": ([_p, _i, _i, _p, _i, _i, _p, _i, _i, _p], _i),
     "mshadow_hip_add_take_grad_large_batch_f32": ([_p, _i, _i, _p, _p, _i, _i, _p, _i, _i, _p], _i),
     "mshadow_hip_index_fill_f32": ([_p, _i, _i, _p, _i, _i, _p, _i, _i, _p], _i),
+    "mshadow_hip_sort_by_key_workspace": ([_sz, C.POINTER(_sz)], _i),
+    "mshadow_hip_sort_by_key_32": ([_p, _i, _p, _sz, _i, _p, _sz, _p], _i),
     "mshadow_hip_softmax_grad_f32": ([_p, _i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_hip_reduce_keep_lowest_f32": ([_p, _p, _i, _i, _i, _i, _i, _f, _p], _i),
     "mshadow_hip_reduce_keep_highdim_f32": ([_p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p], _i),
@@ -92,6 +95,7 @@ CASES_SYMBOLS = {
     "mshadow_case_softmax3d_f32": ([_p, _i, _p, _i, _i, _i, _i, _p], _i),
     "mshadow_case_rows_by_index_f32": ([_i, _p, _i, _i, _p, _p, _i, _p, _i, _i, _i, _p], _i),
     "mshadow_case_shaping_f32": ([_i, _p, _p, _p, _i, _i, _i, _i, _p], _i),
+    "mshadow_case_sort_by_key_32": ([_i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_case_extensions_f32": ([_i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p], _i),
     "mshadow_case_softmax_grad_f32": ([_p, _i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_case_pool_f32": ([_p, _i, _p, _i] + [_i] * 11 + [_p], _i),
@@ -289,6 +293,22 @@ class Library:
             dst.ptr, dst.stride, dst.rows, index.ptr, self._index_is_int(index), index.cols,
             src.ptr, src.stride, src.cols, stream))
 
+    @staticmethod
+    def _key_kind(buf):
+        return {"float32": KEY_F32, "int32": KEY_I32, "uint32": KEY_U32}[buf.dtype.name]
+
+    def sort_by_key(self, keys, values, is_ascend=True, stream=None):
+        """in place; the scratch buffer is allocated here and freed once the sort has finished"""
+        n = keys.cols
+        need = _sz(0)
+        self.check(self.dll.mshadow_hip_sort_by_key_workspace(n, C.byref(need)))
+        work = self.buffer((max(need.value, 1),), np.uint8)
+        self.check(self.dll.mshadow_hip_sort_by_key_32(keys.ptr, self._key_kind(keys), values.ptr, n,
+                                                       1 if is_ascend else 0, work.ptr, need.value,
+                                                       stream))
+        self.check(self.dll.mshadow_hip_stream_sync(stream))
+        return need.value
+
     def softmax_grad(self, dst, src, label, stream=None):
         self.check(self.dll.mshadow_hip_softmax_grad_f32(dst.ptr, dst.stride, src.ptr, src.stride,
                                                          label.ptr, src.rows, src.cols, stream))
@@ -367,6 +387,11 @@ class Library:
     def case_shaping(self, op, out, a, v, n, c, h, w, stream=None):
         self.check_case(self.cases.mshadow_case_shaping_f32(op, out.ptr, a.ptr, v.ptr, n, c, h, w,
                                                             stream))
+
+    def case_sort_by_key(self, op, keys, values, is_ascend=True, stream=None):
+        self.check_case(self.cases.mshadow_case_sort_by_key_32(
+            op, keys.ptr, self._key_kind(keys), values.ptr, keys.cols, 1 if is_ascend else 0,
+            stream))
 
     def case_extensions(self, op, out, a, b, c, n, ch, h, w, p0=0, p1=0, p2=0, stream=None):
         self.check_case(self.cases.mshadow_case_extensions_f32(

@@ -282,6 +282,29 @@ int mshadow_case_shaping_f32(int op, float *out, const float *a, const float *v,
   CASE_END
 }
 
+/* op 0: SortByKey(keys, values, is_ascend); op 1: VectorizedSort(keys as the values to sort,
+   values as the segment numbers). key_kind 0: float keys / int values, 1: int keys / float
+   values (for op 1 the segments are int either way) */
+int mshadow_case_sort_by_key_32(int op, void *keys, int key_kind, void *values, int n,
+                                int is_ascend, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  if (op == 0 && key_kind == 0) {
+    SortByKey(G1(static_cast<float *>(keys), n, st.get()), G1(static_cast<int *>(values), n, st.get()),
+              is_ascend != 0);
+  } else if (op == 0) {
+    SortByKey(G1(static_cast<int *>(keys), n, st.get()), G1(static_cast<float *>(values), n, st.get()),
+              is_ascend != 0);
+  } else if (key_kind == 0) {
+    VectorizedSort(G1(static_cast<float *>(keys), n, st.get()),
+                   G1(static_cast<int *>(values), n, st.get()));
+  } else {
+    VectorizedSort(G1(static_cast<int *>(keys), n, st.get()),
+                   G1(static_cast<int *>(values), n, st.get()));
+  }
+  CASE_END
+}
+
 /* channel pooling, axis reductions / broadcasts, permutations, assignable views and the
    index look-ups, through the generic expression kernel; dense tensors */
 int mshadow_case_extensions_f32(int op, float *out, const float *a, const float *b, const float *c,

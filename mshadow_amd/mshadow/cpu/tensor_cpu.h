@@ -8,6 +8,8 @@
 #ifndef MSHADOW_CPU_TENSOR_CPU_H_
 #define MSHADOW_CPU_TENSOR_CPU_H_
 
+#include <algorithm>
+#include <vector>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -362,6 +364,41 @@ inline void IndexFill(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 1, IndexType>
   for (index_t y = 0; y < index.size(0); ++y) {
     for (index_t j = 0; j < src.size(1); j++) dst[index[y]][j] = src[y][j];
   }
+}
+
+/*! \brief mshadow/tensor_cpu-inl.h:531-559 of the reference: positions are sorted stably
+ *  under keys[i1] < keys[i2] (ascending) or > (descending), then both vectors are
+ *  permuted */
+template <typename KDType, typename VDType>
+inline void SortByKey(Tensor<cpu, 1, KDType> keys, Tensor<cpu, 1, VDType> values,
+                      bool is_ascend) {
+  CHECK_EQ(keys.CheckContiguous(), true);
+  CHECK_EQ(values.CheckContiguous(), true);
+  CHECK_EQ(keys.size(0), values.size(0))
+      << "The sizes of key/value are not equal! keys_size: " << keys.size(0)
+      << "values_size: " << values.size(0);
+  const index_t n = keys.size(0);
+  std::vector<KDType> k(keys.dptr_, keys.dptr_ + n);
+  std::vector<VDType> v(values.dptr_, values.dptr_ + n);
+  std::vector<index_t> order(n);
+  for (index_t i = 0; i < n; ++i) order[i] = i;
+  if (is_ascend) {
+    std::stable_sort(order.begin(), order.end(),
+                     [&k](index_t a, index_t b) { return k[a] < k[b]; });
+  } else {
+    std::stable_sort(order.begin(), order.end(),
+                     [&k](index_t a, index_t b) { return k[a] > k[b]; });
+  }
+  for (index_t i = 0; i < n; ++i) {
+    keys[i] = k[order[i]];
+    values[i] = v[order[i]];
+  }
+}
+/*! \brief two stable sorts: by value, then by segment number (tensor_cpu-inl.h:561-566) */
+template <typename Device, typename VDType, typename SDType>
+inline void VectorizedSort(Tensor<Device, 1, VDType> values, Tensor<Device, 1, SDType> segments) {
+  SortByKey(values, segments, true);
+  SortByKey(segments, values, true);
 }
 
 }  // namespace mshadow

@@ -11,8 +11,10 @@
  * evaluate N adjacent columns at once (EvalPack<N>) from one 128-bit global load per
  * tensor leaf. A plan advertises that with `kPackable`; PackReady() checks at run
  * time that every leaf pointer and pitch is aligned for N-wide access. EvalPack's second
- * template argument asks the leaves for non-temporal (streaming) accesses. Plans without
- * these members (caller-defined ones) simply take the scalar path.
+ * template argument asks the leaves for non-temporal (streaming) accesses. Chainer plans
+ * that read their source at the column they are asked for (row remappings, windows over
+ * rows) forward packs too; they clear *flat in PackReady because they need the real row
+ * number. Plans without these members (caller-defined ones) simply take the scalar path.
  */
 #ifndef MSHADOW_EXPR_PLAN_H_
 #define MSHADOW_EXPR_PLAN_H_
@@ -278,8 +280,18 @@ class Plan<UnaryMapExp<OP, TA, DType, etype>, DType> {
 template <typename SubType, typename SrcExp, int dim, typename DType>
 struct Plan<MakeTensorExp<SubType, SrcExp, dim, DType>, DType> {
  public:
+  /*! \brief a chainer that keeps the column of its source (a remapping of rows, a window
+   *  over rows) can evaluate packs; its concrete plan says so */
+  static const bool kPackable = plan_detail::Packable<Plan<SubType, DType> >::value;
   Plan(const Plan<SubType, DType> &src) : src_(src) {}  // NOLINT(*)
   MSHADOW_XINLINE DType Eval(index_t y, index_t x) const { return src_.Eval(y, x); }
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t x) const {
+    return src_.template EvalPack<N, STREAM>(y, x);
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    return src_.PackReady(n, cols, flat);
+  }
 
  private:
   Plan<SubType, DType> src_;

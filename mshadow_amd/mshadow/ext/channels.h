@@ -78,10 +78,65 @@ struct Plan<ChannelPoolingExp<Reducer, SrcExp, DType, srcdim>, DType> {
     if (last > src_channel_) last = src_channel_;
     DType res;
     Reducer::SetInitValue(res);
-    for (index_t cc = first; cc < last; ++cc) {
-      Reducer::Reduce(res, src_.Eval((n * src_channel_ + cc) * height_.div + y, j));
+    /* four channels fetched before they are reduced, in channel order either way: the loads
+       do not wait for each other */
+    const index_t step = height_.div;
+    index_t row = (n * src_channel_ + first) * step + y;
+    index_t cc = first;
+    for (; cc + 4 <= last; cc += 4, row += 4 * step) {
+      const DType v0 = src_.Eval(row, j), v1 = src_.Eval(row + step, j),
+                  v2 = src_.Eval(row + 2 * step, j), v3 = src_.Eval(row + 3 * step, j);
+      Reducer::Reduce(res, v0);
+      Reducer::Reduce(res, v1);
+      Reducer::Reduce(res, v2);
+      Reducer::Reduce(res, v3);
+    }
+    for (; cc < last; ++cc, row += step) Reducer::Reduce(res, src_.Eval(row, j));
+    return res;
+  }
+  /* the window runs over rows of the source at the same column: N adjacent columns at once */
+  static const bool kPackable = plan_detail::Packable<Plan<SrcExp, DType> >::value;
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t i, index_t j) const {
+    const index_t plane = height_.Div(i);
+    const index_t y = i - plane * height_.div;
+    const index_t n = channel_.Div(plane);
+    const index_t c = plane - n * channel_.div;
+    const index_t first = c * stride_ < pad_ ? 0 : c * stride_ - pad_;
+    index_t last = c * stride_ - pad_ + nsize_;
+    if (last > channel_.div) last = channel_.div;
+    if (last > src_channel_) last = src_channel_;
+    Pack<DType, N> res;
+#pragma unroll
+    for (int k = 0; k < N; ++k) Reducer::SetInitValue(res.v[k]);
+    const index_t step = height_.div;
+    index_t row = (n * src_channel_ + first) * step + y;
+    index_t cc = first;
+    /* neighbouring windows read the same rows again: ordinary (cached) loads */
+    for (; cc + 4 <= last; cc += 4, row += 4 * step) {
+      const Pack<DType, N> v0 = src_.template EvalPack<N, false>(row, j),
+                           v1 = src_.template EvalPack<N, false>(row + step, j),
+                           v2 = src_.template EvalPack<N, false>(row + 2 * step, j),
+                           v3 = src_.template EvalPack<N, false>(row + 3 * step, j);
+#pragma unroll
+      for (int k = 0; k < N; ++k) {
+        Reducer::Reduce(res.v[k], v0.v[k]);
+        Reducer::Reduce(res.v[k], v1.v[k]);
+        Reducer::Reduce(res.v[k], v2.v[k]);
+        Reducer::Reduce(res.v[k], v3.v[k]);
+      }
+    }
+    for (; cc < last; ++cc, row += step) {
+      const Pack<DType, N> v = src_.template EvalPack<N, false>(row, j);
+#pragma unroll
+      for (int k = 0; k < N; ++k) Reducer::Reduce(res.v[k], v.v[k]);
     }
     return res;
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    *flat = false;
+    bool ignored = true;
+    return src_.PackReady(n, cols, &ignored);
   }
 
  private:
@@ -159,6 +214,37 @@ struct Plan<ChannelUnpoolingExp<Reducer, SrcExp, DType, srcdim>, DType> {
       val += Reducer::PartialGrad(vsrc, pooled_.Eval(row, j)) * grad_.Eval(row, j);
     }
     return val;
+  }
+  static const bool kPackable = plan_detail::Packable<Plan<SrcExp, DType> >::value;
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t i, index_t j) const {
+    const Pack<DType, N> vsrc = src_.template EvalPack<N, STREAM>(i, j);
+    const index_t plane = height_.Div(i);
+    const index_t y = i - plane * height_.div;
+    const index_t n = channel_.Div(plane);
+    const index_t c = plane - n * channel_.div;
+    const index_t reach = nsize_ - pad_;
+    const index_t first = c < reach ? 0 : stride_.Div(c - reach + stride_.div);
+    index_t last = stride_.Div(c + pad_ + stride_.div);
+    if (last > channel_.div) last = channel_.div;
+    if (last > pchannel_) last = pchannel_;
+    Pack<DType, N> val;
+#pragma unroll
+    for (int k = 0; k < N; ++k) val.v[k] = static_cast<DType>(0);
+    index_t row = (n * pchannel_ + first) * height_.div + y;
+    for (index_t cc = first; cc < last; ++cc, row += height_.div) {
+      const Pack<DType, N> p = pooled_.template EvalPack<N, false>(row, j),
+                           g = grad_.template EvalPack<N, false>(row, j);
+#pragma unroll
+      for (int k = 0; k < N; ++k) val.v[k] += Reducer::PartialGrad(vsrc.v[k], p.v[k]) * g.v[k];
+    }
+    return val;
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    *flat = false;
+    bool ignored = true;
+    return src_.PackReady(n, cols, &ignored) && pooled_.PackReady(n, cols, &ignored) &&
+           grad_.PackReady(n, cols, &ignored);
   }
 
  private:

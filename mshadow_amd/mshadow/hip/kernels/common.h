@@ -161,6 +161,16 @@ struct SaverReadsDst<sv::saveto> {
   static const bool value = false;
 };
 
+/*! \brief which piece of the work a workgroup takes. Workgroups are dealt to the 8 XCDs
+ *  round-robin, and each XCD has its own L2: handing XCD k the k-th contiguous eighth of
+ *  the pieces (when the count divides evenly) keeps neighbouring pieces - which share
+ *  cache lines, halos or, for windowed expressions, whole operands - behind one L2. */
+__device__ __forceinline__ uint32_t StripOfBlock(uint32_t block, uint32_t nblocks) {
+  const uint32_t kXcd = 8;
+  if (nblocks % kXcd != 0) return block;
+  return (block % kXcd) * (nblocks / kXcd) + block / kXcd;
+}
+
 }  // namespace hip
 }  // namespace mshadow
 #endif  // MSHADOW_HIP_KERNELS_COMMON_H_

@@ -42,7 +42,8 @@ __global__ void __launch_bounds__(kMapBlock)
     MapScalarKernel(DPlan dplan, SPlan splan, uint32_t rows, uint32_t cols, FastDivU32 div_cols) {
   const uint32_t total = rows * cols;
   const uint32_t step = gridDim.x * kMapBlock * PER;
-  for (uint32_t i = (blockIdx.x * kMapBlock + threadIdx.x) * PER; i < total; i += step) {
+  const uint32_t piece = StripOfBlock(blockIdx.x, gridDim.x);
+  for (uint32_t i = (piece * kMapBlock + threadIdx.x) * PER; i < total; i += step) {
     const uint32_t y = div_cols.Div(i);  // a multiply-high, not a hardware division
     const uint32_t x = i - y * cols;
     DType v[PER];
@@ -56,9 +57,13 @@ __global__ void __launch_bounds__(kMapBlock)
 template <typename Saver, typename DType, int N, bool kFlat, bool kStream, int kPackUnroll,
           typename DPlan, typename SPlan>
 __global__ void __launch_bounds__(kMapBlock)
-    MapPackKernel(DPlan dplan, SPlan splan, uint32_t total_packs, uint32_t packs_per_row) {
+    MapPackKernel(DPlan dplan, SPlan splan, uint32_t total_packs, uint32_t packs_per_row,
+                  FastDivU32 div_ppr) {
   typedef expr::Pack<DType, N> P;
-  const uint32_t base = blockIdx.x * (kMapBlock * kPackUnroll) + threadIdx.x;
+  /* with real row numbers in play (windows over rows re-read their neighbours' data), each
+     XCD takes a contiguous run of the workgroups */
+  const uint32_t block = kFlat ? blockIdx.x : StripOfBlock(blockIdx.x, gridDim.x);
+  const uint32_t base = block * (kMapBlock * kPackUnroll) + threadIdx.x;
   uint32_t y[kPackUnroll], x[kPackUnroll];
   P val[kPackUnroll];
 #pragma unroll
@@ -68,7 +73,7 @@ __global__ void __launch_bounds__(kMapBlock)
       y[u] = 0;
       x[u] = p * N;
     } else {
-      y[u] = p / packs_per_row;
+      y[u] = div_ppr.Div(p);
       x[u] = (p - y[u] * packs_per_row) * N;
     }
     if (p < total_packs) val[u] = splan.template EvalPack<N, kStream>(y[u], x[u]);

@@ -118,15 +118,6 @@ __device__ __forceinline__ void ChainFold(DType &res, const DType *vals, int beg
 #undef MSHADOW_CHAIN_AT
 }
 
-/*! \brief which strip of kLowestCols columns a workgroup takes. Workgroups are dealt to
- *  the 8 XCDs round-robin; neighbouring strips share 128-byte cache lines, so each XCD
- *  (one L2) is given a contiguous run of strips when the count divides evenly. */
-__device__ __forceinline__ uint32_t StripOfBlock(uint32_t block, uint32_t nblocks) {
-  const uint32_t kXcd = 8;
-  if (nblocks % kXcd != 0) return block;
-  return (block % kXcd) * (nblocks / kXcd) + block / kXcd;
-}
-
 /* ------------------------------------------------------------------ KeepLowest */
 template <typename Saver, typename Reducer, typename DType, int THREADS, typename DPlan,
           typename SPlan>

@@ -264,6 +264,44 @@ inline void IndexFill(Tensor<gpu, 2, float> dst, const Tensor<gpu, 1, IndexType>
       index.size(0), src.dptr_, src.stride_, src.size(1), Stream<gpu>::GetStream(dst.stream_)));
 }
 
+namespace gpu_detail {
+/*! \brief how the bits of a 32-bit key type are ordered (-1: no device sort for this type) */
+template <typename KDType>
+struct SortKeyKind { static const int value = -1; };
+template <>
+struct SortKeyKind<float> { static const int value = MSHADOW_HIP_KEY_F32; };
+template <>
+struct SortKeyKind<int32_t> { static const int value = MSHADOW_HIP_KEY_I32; };
+template <>
+struct SortKeyKind<uint32_t> { static const int value = MSHADOW_HIP_KEY_U32; };
+}  // namespace gpu_detail
+/*! \brief stable sort by key on the device (the reference: thrust::stable_sort_by_key,
+ *  tensor_gpu-inl.cuh:784-806, which takes its scratch memory from the runtime as this does;
+ *  half_t keys or values are as fatal here as there). Returns once the sort has finished. */
+template <typename KDType, typename VDType>
+inline void SortByKey(Tensor<gpu, 1, KDType> keys, Tensor<gpu, 1, VDType> values,
+                      bool is_ascend) {
+  CHECK_EQ(keys.CheckContiguous(), true);
+  CHECK_EQ(values.CheckContiguous(), true);
+  CHECK_EQ(keys.size(0), values.size(0))
+      << "The sizes of key/value are not equal! keys_size: " << keys.size(0)
+      << "values_size: " << values.size(0);
+  CHECK(gpu_detail::SortKeyKind<KDType>::value >= 0 && sizeof(VDType) == 4)
+      << "SortByKey<gpu>: implemented for 32-bit float / integer keys and 32-bit values";
+  const size_t n = keys.size(0);
+  if (n == 0) return;
+  void *stream = Stream<gpu>::GetStream(keys.stream_);
+  size_t bytes = 0, pitch = 0;
+  void *workspace = NULL;
+  MSHADOW_HIP_CALL(mshadow_hip_sort_by_key_workspace(n, &bytes));
+  MSHADOW_HIP_CALL(mshadow_hip_malloc_pitch(&workspace, &pitch, bytes, 1));
+  MSHADOW_HIP_CALL(mshadow_hip_sort_by_key_32(keys.dptr_, gpu_detail::SortKeyKind<KDType>::value,
+                                              values.dptr_, n, is_ascend ? 1 : 0, workspace, bytes,
+                                              stream));
+  MSHADOW_HIP_CALL(mshadow_hip_stream_sync(stream));
+  MSHADOW_HIP_CALL(mshadow_hip_free(workspace));
+}
+
 /* ------------------------------------------------------------------ expression routing */
 namespace gpu_detail {
 
@@ -480,7 +518,8 @@ struct MapLauncher<Saver, DType, DPlan, SPlan, true> {
                             ? hip::kPackUnrollDeep : hip::kPackUnroll;
     const uint32_t per_block = hip::kMapBlock * kUnroll;
     const uint32_t grid = (total + per_block - 1) / per_block;
-    void *args[] = {&dplan, &splan, &total, &ppr};
+    FastDivU32 div_ppr(ppr);
+    void *args[] = {&dplan, &splan, &total, &ppr, &div_ppr};
     /* streaming (non-temporal) accesses once a tensor no longer fits the caches anyway */
     const bool stream_hint = static_cast<size_t>(rows) * cols * sizeof(DType) >= (8u << 20);
     const bool is_flat = flat || rows == 1;

@@ -149,6 +149,18 @@ inline void IndexFill(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 1, IndexType>
 template <typename IndexType, typename DType>
 inline void IndexFill(Tensor<gpu, 2, DType> dst, const Tensor<gpu, 1, IndexType> &index,
                       const Tensor<gpu, 2, DType> &src);
+/*! \brief stable sort of the (key, value) pairs by key, in place; equivalent keys keep their
+ *  order whichever the direction */
+template <typename KDType, typename VDType>
+inline void SortByKey(Tensor<cpu, 1, KDType> keys, Tensor<cpu, 1, VDType> values,
+                      bool is_ascend = true);
+template <typename KDType, typename VDType>
+inline void SortByKey(Tensor<gpu, 1, KDType> keys, Tensor<gpu, 1, VDType> values,
+                      bool is_ascend = true);
+/*! \brief ascending sort of the values inside every segment; `segments` is a non-decreasing
+ *  vector of segment numbers such as [0, 0, 0, 1, 1, 2, 3, 3] */
+template <typename Device, typename VDType, typename SDType>
+inline void VectorizedSort(Tensor<Device, 1, VDType> values, Tensor<Device, 1, SDType> segments);
 
 /*! \brief Saver::Save(dst(y,x), exp(y,x)) for every element */
 template <typename Saver, typename R, int dim, typename DType, typename E, int etype>

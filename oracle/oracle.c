@@ -23,6 +23,7 @@
 
 #include <float.h>
 #include <math.h>
+#include <stdlib.h>
 #include <string.h>
 #ifdef _OPENMP
 #include <omp.h>
@@ -371,6 +372,54 @@ void orc_index_fill_f32(float *dst, int dstride, const void *index, int index_is
     const int j = index_at(index, index_is_int, y);
     for (int x = 0; x < cols; ++x) dst[(int64_t)j * dstride + x] = src[(int64_t)y * sstride + x];
   }
+}
+
+/* SortByKey, mshadow/tensor_cpu-inl.h:531-559: std::stable_sort of the positions under
+   keys[a] < keys[b] (ascending) or keys[a] > keys[b] (descending), then keys and values
+   permuted alike. Restated as a bottom-up merge sort, which is stable by construction: the
+   right run's element is taken only when it is strictly before the left run's. Keys are
+   compared in their own type (key_kind 0 float, 1 int32, 2 uint32), so +0.0f and -0.0f are
+   equivalent; values are 32-bit words. VectorizedSort (:561-566) is two of these. */
+static int key_before(const uint32_t *k, int key_kind, int ascend, int a, int b) {
+  if (key_kind == 0) {
+    float x, y;
+    memcpy(&x, &k[a], 4);
+    memcpy(&y, &k[b], 4);
+    return ascend ? x < y : x > y;
+  }
+  if (key_kind == 1) {
+    const int32_t x = (int32_t)k[a], y = (int32_t)k[b];
+    return ascend ? x < y : x > y;
+  }
+  return ascend ? k[a] < k[b] : k[a] > k[b];
+}
+void orc_sort_by_key_32(void *keys, int key_kind, void *values, int n, int is_ascend) {
+  if (n <= 0) return;
+  uint32_t *k = (uint32_t *)keys, *v = (uint32_t *)values;
+  int *ord = (int *)malloc(sizeof(int) * (size_t)n), *tmp = (int *)malloc(sizeof(int) * (size_t)n);
+  uint32_t *kc = (uint32_t *)malloc(4 * (size_t)n), *vc = (uint32_t *)malloc(4 * (size_t)n);
+  for (int i = 0; i < n; ++i) ord[i] = i;
+  for (int64_t width = 1; width < n; width *= 2) {
+    for (int64_t lo = 0; lo < n; lo += 2 * width) {
+      const int64_t mid = lo + width < n ? lo + width : n, hi = lo + 2 * width < n ? lo + 2 * width : n;
+      int64_t i = lo, j = mid, o = lo;
+      while (i < mid && j < hi) tmp[o++] = key_before(k, key_kind, is_ascend, ord[j], ord[i]) ? ord[j++] : ord[i++];
+      while (i < mid) tmp[o++] = ord[i++];
+      while (j < hi) tmp[o++] = ord[j++];
+    }
+    int *sw = ord; ord = tmp; tmp = sw;
+  }
+  memcpy(kc, k, 4 * (size_t)n);
+  memcpy(vc, v, 4 * (size_t)n);
+  for (int i = 0; i < n; ++i) {
+    k[i] = kc[ord[i]];
+    v[i] = vc[ord[i]];
+  }
+  free(ord); free(tmp); free(kc); free(vc);
+}
+void orc_vectorized_sort_32(void *values, int value_kind, void *segments, int n) {
+  orc_sort_by_key_32(values, value_kind, segments, n, 1);
+  orc_sort_by_key_32(segments, 1, values, n, 1);
 }
 
 /* ------------------------------------------------------------------ pool / unpool */

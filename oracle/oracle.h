@@ -79,6 +79,9 @@ void orc_add_take_grad_large_batch_f32(float *dst, int dstride, const void *sort
 void orc_index_fill_f32(float *dst, int dstride, const void *index, int index_is_int,
                         int n_index, const float *src, int sstride, int cols);
 
+void orc_sort_by_key_32(void *keys, int key_kind, void *values, int n, int is_ascend);
+void orc_vectorized_sort_32(void *values, int value_kind, void *segments, int n);
+
 void orc_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes, int h, int w,
                   int ph, int pw, int ky, int kx, int sy, int sx, int reducer);
 void orc_unpool_f32(float *dst, int dstride, const float *src, int sstride, const float *pooled,

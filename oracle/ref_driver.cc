@@ -203,6 +203,23 @@ void ref_index_fill_f32(float *dst, int dstride, const void *index, int index_is
   }
 }
 
+/* key_kind 0: float keys with int values; 1: int keys with float values (the value words are
+   only moved); uint32 keys are not a type the callers of the reference use */
+void ref_sort_by_key_32(void *keys, int key_kind, void *values, int n, int is_ascend) {
+  if (key_kind == 0) {
+    SortByKey(Tensor<cpu, 1, float>(static_cast<float *>(keys), Shape1(n)),
+              Tensor<cpu, 1, int>(static_cast<int *>(values), Shape1(n)), is_ascend != 0);
+  } else {
+    SortByKey(Tensor<cpu, 1, int>(static_cast<int *>(keys), Shape1(n)),
+              Tensor<cpu, 1, float>(static_cast<float *>(values), Shape1(n)), is_ascend != 0);
+  }
+}
+void ref_vectorized_sort_32(void *values, int value_kind, void *segments, int n) {
+  Tensor<cpu, 1, int> seg(static_cast<int *>(segments), Shape1(n));
+  if (value_kind == 0) VectorizedSort(Tensor<cpu, 1, float>(static_cast<float *>(values), Shape1(n)), seg);
+  else VectorizedSort(Tensor<cpu, 1, int>(static_cast<int *>(values), Shape1(n)), seg);
+}
+
 /* index-remapping extensions (broadcast, repmat, reshape, swapaxis, mirror,
    upsampling_nearest): the same expressions the GPU cases library evaluates */
 void ref_shaping_f32(int op, float *out, const float *a, const float *v, int n, int c, int h,

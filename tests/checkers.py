@@ -83,6 +83,8 @@ class Checker:
         self._fn("add_take_grad_f32", [_p, _i, _i, _p, _i, _i, _p, _i, _i])
         self._fn("add_take_grad_large_batch_f32", [_p, _i, _p, _p, _i, _i, _p, _i, _i])
         self._fn("index_fill_f32", [_p, _i, _p, _i, _i, _p, _i, _i])
+        self._fn("sort_by_key_32", [_p, _i, _p, _i, _i])
+        self._fn("vectorized_sort_32", [_p, _i, _p, _i])
         if self.prefix == "ref":
             self._fn("shaping_f32", [_i, _p, _p, _p, _i, _i, _i, _i])
             self._fn("extensions_f32", [_i, _p, _p, _p, _p] + [_i] * 7)
@@ -191,6 +193,20 @@ class Checker:
         self._index_fill_f32(ptr(dst), pitch(dst), ptr(index), self._is_int(index),
                              index.shape[0], ptr(src), pitch(src), src.shape[1])
         return dst
+
+    @staticmethod
+    def _key_kind(keys):
+        return {"float32": 0, "int32": 1, "uint32": 2}[keys.dtype.name]
+
+    def sort_by_key(self, keys, values, is_ascend=True):
+        """in place on two contiguous 1-D arrays of 32-bit elements"""
+        self._sort_by_key_32(ptr(keys), self._key_kind(keys), ptr(values), keys.shape[0],
+                             1 if is_ascend else 0)
+        return keys, values
+
+    def vectorized_sort(self, values, segments):
+        self._vectorized_sort_32(ptr(values), self._key_kind(values), ptr(segments), values.shape[0])
+        return values, segments
 
     def shaping(self, op, out, a, v, n, c, h, w):
         """reference build only: the index-remapping extension expressions"""

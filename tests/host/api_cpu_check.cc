@@ -299,6 +299,31 @@ int main() {
     orc_index_fill_f32(d2.data(), W, srt.data(), 1, N, src.data(), W, W);
     EXPECT(SameBits(d1.data(), d2.data(), d1.size()));
   }
+  // ---- SortByKey / VectorizedSort on the CPU device against the oracle
+  {
+    const int N = 777;
+    std::vector<float> kf(N), kf2;
+    std::vector<int> vi(N), vi2, seg(N), seg2;
+    for (int i = 0; i < N; ++i) {
+      kf[i] = static_cast<float>((i * 37) % 11 - 5) * 0.5f;
+      if (i % 13 == 0) kf[i] = -0.0f;
+      vi[i] = i;
+      seg[i] = i / 50;
+    }
+    for (int ascend = 0; ascend < 2; ++ascend) {
+      kf2 = kf; vi2 = vi;
+      std::vector<float> a = kf; std::vector<int> b = vi;
+      SortByKey(Tensor<cpu, 1, float>(a.data(), Shape1(N)), Tensor<cpu, 1, int>(b.data(), Shape1(N)),
+                ascend != 0);
+      orc_sort_by_key_32(kf2.data(), 0, vi2.data(), N, ascend);
+      EXPECT(SameBits(a.data(), kf2.data(), N) && b == vi2);
+    }
+    kf2 = kf; seg2 = seg;
+    std::vector<float> a = kf;
+    VectorizedSort(Tensor<cpu, 1, float>(a.data(), Shape1(N)), Tensor<cpu, 1, int>(seg.data(), Shape1(N)));
+    orc_vectorized_sort_32(kf2.data(), 0, seg2.data(), N);
+    EXPECT(SameBits(a.data(), kf2.data(), N) && seg == seg2);
+  }
   // ---- index-remapping extensions on the CPU device, against plain index loops
   {
     const int n = 2, c = 3, h = 4, w = 5;

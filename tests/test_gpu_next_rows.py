@@ -1,7 +1,9 @@
 """GPU parity for the rows next to the hot path - SmoothSoftmaxGrad / ignore_label gradients,
-3-D softmax and its gradients, AddTakeGrad, AddTakeGradLargeBatch, IndexFill - through the C
-ABI and through the C++ functions, against the oracle. Bit for bit everywhere except the
+3-D softmax and its gradients, AddTakeGrad, AddTakeGradLargeBatch, IndexFill, SortByKey /
+VectorizedSort - through the C ABI and through the C++ functions, against the oracle. Bit for bit everywhere except the
 3-D softmax forward (relative 1e-5: device exponential)."""
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -116,3 +118,69 @@ def test_many_duplicates_keep_index_order(G, O):
     dst = G.to_device(start)
     G.add_take_grad(dst, G.to_device(idx), G.to_device(src))
     assert_bits_equal(dst.download(), want, "ordered accumulation")
+
+
+# ---- SortByKey / VectorizedSort
+def _sort_inputs(kind, n, seed):
+    rng = np.random.default_rng(seed)
+    if kind == "f32":
+        keys = (rng.integers(-40, 41, n).astype(f32) * f32(0.25)) if n < 5000 else \
+            rng.standard_normal(n).astype(f32)
+        keys[rng.random(n) < 0.05] = f32(-0.0)
+        keys[rng.random(n) < 0.05] = f32(0.0)
+        if n > 8:
+            keys[:4] = [np.inf, -np.inf, np.finfo(f32).max, np.finfo(f32).tiny / 4]
+        values = np.arange(n, dtype=np.int32)
+    else:
+        keys = rng.integers(-50, 51, n).astype(np.int32) if n < 5000 else \
+            rng.integers(-2**31, 2**31, n, dtype=np.int64).astype(np.int32)
+        if n > 8:
+            keys[:2] = [np.iinfo(np.int32).min, np.iinfo(np.int32).max]
+        values = rng.standard_normal(n).astype(f32)
+    return keys, values
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["f32", "i32"])
+@pytest.mark.parametrize("n", [1, 2, 255, 1000, 65537, 1 << 20])
+@pytest.mark.parametrize("ascend", [True, False])
+def test_sort_by_key(G, O, kind, n, ascend):
+    keys, values = _sort_inputs(kind, n, 3 + n)
+    want_k, want_v = O.sort_by_key(keys.copy(), values.copy(), ascend)
+    for route in ("abi", "header"):
+        dk, dv = G.to_device(keys), G.to_device(values)
+        if route == "abi":
+            G.sort_by_key(dk, dv, ascend)
+        else:
+            G.case_sort_by_key(0, dk, dv, ascend)
+        assert np.array_equal(dk.download().view(np.uint32), want_k.view(np.uint32)), route
+        assert np.array_equal(dv.download().view(np.uint32), want_v.view(np.uint32)), route
+
+
+@pytest.mark.gpu
+def test_sort_by_key_unsigned_and_empty(G):
+    rng = np.random.default_rng(8)
+    keys = rng.integers(0, 2**32, 5000, dtype=np.int64).astype(np.uint32)
+    values = np.arange(5000, dtype=np.int32)
+    dk, dv = G.to_device(keys), G.to_device(values)
+    G.sort_by_key(dk, dv, False)
+    order = np.argsort(-keys.astype(np.int64), kind="stable")
+    assert np.array_equal(dk.download(), keys[order]) and np.array_equal(dv.download(), values[order])
+    need = ctypes.c_size_t(7)
+    G.check(G.dll.mshadow_hip_sort_by_key_workspace(0, ctypes.byref(need)))
+    assert need.value == 0
+    G.check(G.dll.mshadow_hip_sort_by_key_32(None, 0, None, 0, 1, None, 0, None))
+    assert G.dll.mshadow_hip_sort_by_key_32(dk.ptr, 0, dv.ptr, 5000, 1, dk.ptr, 16, None) != 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["f32", "i32"])
+def test_vectorized_sort(G, O, kind):
+    n = 30000
+    keys, _ = _sort_inputs(kind, n, 21)
+    seg = np.sort(np.random.default_rng(4).integers(0, 300, n)).astype(np.int32)
+    want_v, want_s = O.vectorized_sort(keys.copy(), seg.copy())
+    dv, ds = G.to_device(keys), G.to_device(seg)
+    G.case_sort_by_key(1, dv, ds)
+    assert np.array_equal(dv.download().view(np.uint32), want_v.view(np.uint32))
+    assert np.array_equal(ds.download(), want_s)

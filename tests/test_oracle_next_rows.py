@@ -142,3 +142,66 @@ def test_oracle_equals_reference_build(orc, ref):
         orc.index_fill(d1, inside, src)
         ref.index_fill(d2, inside, src)
         assert np.array_equal(d1.view(np.uint32), d2.view(np.uint32))
+
+
+# ---- SortByKey / VectorizedSort (mshadow/tensor_cpu-inl.h:531-566)
+def _sort_inputs(kind, n, seed):
+    rng = np.random.default_rng(seed)
+    if kind == "f32":
+        # few distinct values: long runs of equivalent keys, both zeros among them
+        keys = rng.integers(-4, 5, n).astype(f32) * f32(0.5)
+        keys[rng.random(n) < 0.1] = f32(-0.0)
+        values = np.arange(n, dtype=np.int32)
+    else:
+        keys = rng.integers(-5, 6, n).astype(np.int32)
+        keys[: n // 7] = np.iinfo(np.int32).min
+        keys[n // 7: 2 * (n // 7)] = np.iinfo(np.int32).max
+        rng.shuffle(keys)
+        values = np.arange(n, dtype=f32)
+    return keys, values
+
+
+def _stable_order(keys, ascend):
+    """positions in the order a stable sort under < (or >) leaves them: equivalent keys (which
+    includes +0.0 and -0.0) keep their original order in both directions"""
+    ranks = keys.astype(np.float64)
+    return np.argsort(ranks if ascend else -ranks, kind="stable")
+
+
+@pytest.mark.parametrize("kind", ["f32", "i32"])
+@pytest.mark.parametrize("n", [0, 1, 2, 17, 1000, 4099])
+@pytest.mark.parametrize("ascend", [True, False])
+def test_sort_by_key_is_the_stable_permutation(orc, kind, n, ascend):
+    keys, values = _sort_inputs(kind, n, 5 + n)
+    order = _stable_order(keys, ascend)
+    k, v = keys.copy(), values.copy()
+    orc.sort_by_key(k, v, ascend)
+    assert np.array_equal(k.view(np.uint32), keys[order].view(np.uint32))   # -0.0 stays -0.0
+    assert np.array_equal(v, values[order])
+
+
+def test_vectorized_sort_sorts_inside_segments(orc):
+    rng = np.random.default_rng(11)
+    seg = np.sort(rng.integers(0, 9, 500)).astype(np.int32)
+    vals = rng.standard_normal(500).astype(f32)
+    v, s = vals.copy(), seg.copy()
+    orc.vectorized_sort(v, s)
+    assert np.array_equal(s, seg)
+    for g in np.unique(seg):
+        assert np.array_equal(v[seg == g], np.sort(vals[seg == g]))
+
+
+@pytest.mark.skipif(not have_ref(), reason="reference build absent")
+@pytest.mark.parametrize("kind", ["f32", "i32"])
+@pytest.mark.parametrize("n", [1, 33, 2048, 50001])
+@pytest.mark.parametrize("ascend", [True, False])
+def test_sort_by_key_matches_reference_build(orc, ref, kind, n, ascend):
+    keys, values = _sort_inputs(kind, n, 9 + n)
+    ko, vo = orc.sort_by_key(keys.copy(), values.copy(), ascend)
+    kr, vr = ref.sort_by_key(keys.copy(), values.copy(), ascend)
+    assert np.array_equal(ko.view(np.uint32), kr.view(np.uint32))
+    assert np.array_equal(vo.view(np.uint32), vr.view(np.uint32))
+    seg = np.sort(np.random.default_rng(n).integers(0, 1 + n // 5, n)).astype(np.int32)
+    a, b = orc.vectorized_sort(keys.copy(), seg.copy())
+    c, d = ref.vectorized_sort(keys.copy(), seg.copy())
+    assert np.array_equal(a.view(np.uint32), c.view(np.uint32)) and np.array_equal(b, d)
