@@ -63,6 +63,13 @@ struct RowDigits {
     return digit;
   }
 };
+/*! \brief PackReady of a source plan for a node that needs real row numbers itself */
+template <typename P>
+inline bool SourcePackReady(const P &plan, int n, index_t cols, bool *flat) {
+  *flat = false;
+  bool ignored = true;
+  return plan.PackReady(n, cols, &ignored);
+}
 }  // namespace axes_detail
 
 /* ------------------------------------------------------------------ reduce_with_axis */
@@ -125,6 +132,43 @@ struct Plan<ReduceWithAxisExp<Reducer, SrcExp, DType, dimsrc, mask, dimdst>, DTy
       if (mask && before != res) where = k;
     }
     return mask ? static_cast<DType>(static_cast<int>(where)) : res;
+  }
+  /* when the reduced axis is not the last one, the elements along it sit in different rows of
+     the source at the same column: N adjacent columns are reduced side by side */
+  static const bool kPackable = plan_detail::Packable<Plan<SrcExp, DType> >::value;
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t i, index_t j) const {
+    const index_t flat = i * last_dst_dim_ + j;
+    const index_t outer = trailing_.Div(flat);
+    const index_t inner = flat - outer * trailing_.div;
+    index_t row = at_.last.Div(outer * size_ * trailing_.div + inner);
+    const index_t row_step = at_.last.Div(trailing_.div);
+    Pack<DType, N> res;
+    index_t where[N];
+#pragma unroll
+    for (int c = 0; c < N; ++c) {
+      Reducer::SetInitValue(res.v[c]);
+      where[c] = 0;
+    }
+    for (index_t k = 0; k < size_; ++k, row += row_step) {
+      const Pack<DType, N> v = src_.template EvalPack<N, STREAM>(row, j);
+#pragma unroll
+      for (int c = 0; c < N; ++c) {
+        const DType before = res.v[c];
+        Reducer::Reduce(res.v[c], v.v[c]);
+        if (mask && before != res.v[c]) where[c] = k;
+      }
+    }
+    if (mask) {
+#pragma unroll
+      for (int c = 0; c < N; ++c) res.v[c] = static_cast<DType>(static_cast<int>(where[c]));
+    }
+    return res;
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    const index_t last = at_.last.div;
+    return axes_detail::SourcePackReady(src_, n, cols, flat) && last_dst_dim_ == last &&
+           trailing_.div % last == 0;
   }
 
  private:
@@ -199,6 +243,21 @@ struct Plan<BroadcastWithAxisExp<SrcExp, DType, dimsrc, dimdst>, DType> {
     const index_t upper = trailing_.Div(flat);  // (outer, position on the new axis)
     const index_t inner = flat - upper * trailing_.div;
     return at_.Eval(src_, size_.Div(upper) * trailing_.div + inner);
+  }
+  /* a new axis in front of the last dimension repeats whole rows */
+  static const bool kPackable = plan_detail::Packable<Plan<SrcExp, DType> >::value;
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t i, index_t j) const {
+    const index_t flat = i * dst_last_ + j;
+    const index_t upper = trailing_.Div(flat);
+    const index_t inner = flat - upper * trailing_.div;
+    return src_.template EvalPack<N, false>(at_.last.Div(size_.Div(upper) * trailing_.div + inner),
+                                            j);
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    const index_t last = at_.last.div;
+    return axes_detail::SourcePackReady(src_, n, cols, flat) && dst_last_ == last &&
+           trailing_.div % last == 0;
   }
 
  private:
@@ -340,6 +399,18 @@ struct Plan<TransposeExExp<SrcExp, DType, dimsrc>, DType> {
 #pragma unroll
     for (int k = dimsrc - 2; k >= 0; --k) flat += digits_.Pop(k, i) * step_[k];
     return at_.Eval(src_, flat);
+  }
+  /* a permutation that leaves the last axis in place permutes rows */
+  static const bool kPackable = plan_detail::Packable<Plan<SrcExp, DType> >::value;
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t i, index_t j) const {
+    index_t flat = 0;
+#pragma unroll
+    for (int k = dimsrc - 2; k >= 0; --k) flat += digits_.Pop(k, i) * step_[k];
+    return src_.template EvalPack<N, STREAM>(at_.last.Div(flat), j);
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    return axes_detail::SourcePackReady(src_, n, cols, flat) && step_[dimsrc - 1] == 1;
   }
 
  private:
@@ -516,6 +587,26 @@ struct Plan<ConcatExp<LhsExp, RhsExp, Device, DType, srcdim, dimsrc_m_cat>, DTyp
     const index_t row = Locate(i, &second);
     return second ? src2_.REval(row, j) : src1_.REval(row, j);
   }
+  static const bool kPackable = plan_detail::Packable<Plan<LhsExp, DType> >::value &&
+                                plan_detail::Packable<Plan<RhsExp, DType> >::value;
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t i, index_t j) const {
+    bool second;
+    const index_t row = Locate(i, &second);
+    return second ? src2_.template EvalPack<N, STREAM>(row, j)
+                  : src1_.template EvalPack<N, STREAM>(row, j);
+  }
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE void StorePack(index_t i, index_t j, const Pack<DType, N> &p) {
+    bool second;
+    const index_t row = Locate(i, &second);
+    if (second) src2_.template StorePack<N, STREAM>(row, j, p);
+    else src1_.template StorePack<N, STREAM>(row, j, p);
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    return axes_detail::SourcePackReady(src1_, n, cols, flat) &&
+           axes_detail::SourcePackReady(src2_, n, cols, flat);
+  }
 
  private:
   /*! \brief which operand holds row i of the concatenation, and at which of its rows */
@@ -603,6 +694,18 @@ struct Plan<SliceExp<SrcExp, Device, DType, srcdim, dimsrc_m_slice>, DType> {
         ch_(e.shape_[dimslice]), ch_begin_(e.ch_begin_), ch_old_(e.ch_old_) {}
   MSHADOW_XINLINE DType Eval(index_t i, index_t j) const { return src_.Eval(Row(i), j); }
   MSHADOW_XINLINE DType &REval(index_t i, index_t j) { return src_.REval(Row(i), j); }
+  static const bool kPackable = plan_detail::Packable<Plan<SrcExp, DType> >::value;
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t i, index_t j) const {
+    return src_.template EvalPack<N, STREAM>(Row(i), j);
+  }
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE void StorePack(index_t i, index_t j, const Pack<DType, N> &p) {
+    src_.template StorePack<N, STREAM>(Row(i), j, p);
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    return axes_detail::SourcePackReady(src_, n, cols, flat);
+  }
 
  private:
   MSHADOW_XINLINE index_t Row(index_t i) const {
@@ -740,6 +843,20 @@ struct Plan<FlipExp<SrcExp, Device, DType, srcdim>, DType> {
       : src_(MakePlan(e.src_)), at_(e.stride_j_), trailing_(e.trailing_), stride_(e.stride_) {}
   MSHADOW_XINLINE DType Eval(index_t i, index_t j) const { return at_.Eval(src_, Mirror(i, j)); }
   MSHADOW_XINLINE DType &REval(index_t i, index_t j) { return at_.REval(src_, Mirror(i, j)); }
+  /* reversing any axis but the last reverses runs of whole rows */
+  static const bool kPackable = plan_detail::Packable<Plan<SrcExp, DType> >::value;
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t i, index_t j) const {
+    return src_.template EvalPack<N, STREAM>(at_.last.Div(Mirror(i, 0)), j);
+  }
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE void StorePack(index_t i, index_t j, const Pack<DType, N> &p) {
+    src_.template StorePack<N, STREAM>(at_.last.Div(Mirror(i, 0)), j, p);
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    return axes_detail::SourcePackReady(src_, n, cols, flat) &&
+           trailing_.div % at_.last.div == 0;
+  }
 
  private:
   MSHADOW_XINLINE index_t Mirror(index_t i, index_t j) const {

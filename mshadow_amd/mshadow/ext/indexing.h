@@ -48,6 +48,17 @@ struct Plan<TakeExp<IndexExp, SrcExp, DType>, DType> {
   MSHADOW_XINLINE DType Eval(index_t y, index_t x) const {
     return static_cast<DType>(src_.Eval(static_cast<index_t>(index_.Eval(0, y)), x));
   }
+  /* a row of the result is a row of the source */
+  static const bool kPackable = plan_detail::Packable<Plan<SrcExp, DType> >::value;
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t x) const {
+    return src_.template EvalPack<N, false>(static_cast<index_t>(index_.Eval(0, y)), x);
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    *flat = false;
+    bool ignored = true;
+    return src_.PackReady(n, cols, &ignored);
+  }
 
  private:
   Plan<IndexExp, DType> index_;
@@ -151,6 +162,20 @@ struct Plan<MaskExp<IndexExp, SrcExp, DType>, DType> {
       : index_(MakePlan(e.index_)), src_(MakePlan(e.src_)) {}
   MSHADOW_XINLINE DType Eval(index_t y, index_t x) const {
     return static_cast<DType>(src_.Eval(y, x) * index_.Eval(0, y));
+  }
+  static const bool kPackable = plan_detail::Packable<Plan<SrcExp, DType> >::value;
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t x) const {
+    Pack<DType, N> p = src_.template EvalPack<N, STREAM>(y, x);
+    const DType factor = index_.Eval(0, y);
+#pragma unroll
+    for (int k = 0; k < N; ++k) p.v[k] = static_cast<DType>(p.v[k] * factor);
+    return p;
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    *flat = false;
+    bool ignored = true;
+    return src_.PackReady(n, cols, &ignored);
   }
 
  private:

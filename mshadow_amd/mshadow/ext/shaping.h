@@ -75,6 +75,20 @@ struct Plan<Broadcast1DExp<SrcExp, DType, dimdst, dimdst_m_cast>, DType> {
   MSHADOW_XINLINE DType Eval(index_t y, index_t) const {
     return src_.Eval(0, length_.Mod(below_.Div(y)));
   }
+  /* one value for the whole row: a pack is that value N times */
+  static const bool kPackable = true;
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t) const {
+    const DType v = src_.Eval(0, length_.Mod(below_.Div(y)));
+    Pack<DType, N> p;
+#pragma unroll
+    for (int k = 0; k < N; ++k) p.v[k] = v;
+    return p;
+  }
+  inline bool PackReady(int, index_t, bool *flat) const {
+    *flat = false;
+    return true;
+  }
 
  private:
   Plan<SrcExp, DType> src_;
@@ -86,6 +100,16 @@ struct Plan<Broadcast1DExp<SrcExp, DType, dimdst, 1>, DType> {
  public:
   explicit Plan(const Broadcast1DExp<SrcExp, DType, dimdst, 1> &e) : src_(MakePlan(e.src_)) {}
   MSHADOW_XINLINE DType Eval(index_t, index_t x) const { return src_.Eval(0, x); }
+  static const bool kPackable = plan_detail::Packable<Plan<SrcExp, DType> >::value;
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t, index_t x) const {
+    return src_.template EvalPack<N, false>(0, x);  // every row reads it again: cached loads
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    *flat = false;
+    bool ignored = true;
+    return src_.PackReady(n, cols, &ignored);
+  }
 
  private:
   Plan<SrcExp, DType> src_;
@@ -95,6 +119,16 @@ struct Plan<BroadcastScalarExp<SrcExp, DType, dimdst>, DType> {
  public:
   explicit Plan(const BroadcastScalarExp<SrcExp, DType, dimdst> &e) : src_(MakePlan(e.src_)) {}
   MSHADOW_XINLINE DType Eval(index_t, index_t) const { return src_.Eval(0, 0); }
+  static const bool kPackable = true;
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t, index_t) const {
+    const DType v = src_.Eval(0, 0);
+    Pack<DType, N> p;
+#pragma unroll
+    for (int k = 0; k < N; ++k) p.v[k] = v;
+    return p;
+  }
+  inline bool PackReady(int, index_t, bool *) const { return true; }
 
  private:
   Plan<SrcExp, DType> src_;
@@ -128,6 +162,20 @@ struct Plan<ReshapeExp<SrcExp, DType, dimdst, dimsrc>, DType> {
     if (dimsrc == 1) return src_.Eval(0, flat);
     const index_t row = icols_.Div(flat);
     return src_.Eval(row, flat - row * icols_.div);
+  }
+  /* N adjacent elements stay adjacent in the source as long as N divides both row lengths */
+  static const bool kPackable = plan_detail::Packable<Plan<SrcExp, DType> >::value;
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t x) const {
+    const index_t flat = y * ocols_ + x;
+    if (dimsrc == 1) return src_.template EvalPack<N, STREAM>(0, flat);
+    const index_t row = icols_.Div(flat);
+    return src_.template EvalPack<N, STREAM>(row, flat - row * icols_.div);
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    *flat = false;
+    bool ignored = true;
+    return ocols_ % n == 0 && icols_.div % n == 0 && src_.PackReady(n, icols_.div, &ignored);
   }
 
  private:
@@ -178,6 +226,23 @@ struct Plan<SwapAxisExp<SrcExp, DType, dimsrc, m_a1, a2>, DType> {
       const index_t p = rest - outer * p_.div;
       return src_.Eval((outer * q_.div + j) * mid_.div + mid, p);
     }
+    return src_.Eval(SourceRow(i), j);
+  }
+  /* with the last dimension left alone the swap is a permutation of rows */
+  static const bool kPackable = (m_a1 != 1) && plan_detail::Packable<Plan<SrcExp, DType> >::value;
+  template <int N, bool STREAM = false>
+  MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t i, index_t j) const {
+    return src_.template EvalPack<N, STREAM>(SourceRow(i), j);
+  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const {
+    *flat = false;
+    bool ignored = true;
+    return src_.PackReady(n, cols, &ignored);
+  }
+
+ private:
+  /*! \brief row of the source that holds row i of the result (a1 is not the last dimension) */
+  MSHADOW_XINLINE index_t SourceRow(index_t i) const {
     index_t rest = inner_.Div(i);
     const index_t inner = i - rest * inner_.div;
     index_t next = q_.Div(rest);
@@ -186,10 +251,8 @@ struct Plan<SwapAxisExp<SrcExp, DType, dimsrc, m_a1, a2>, DType> {
     const index_t mid = next - rest * mid_.div;
     const index_t outer = p_.Div(rest);
     const index_t p = rest - outer * p_.div;
-    return src_.Eval((((outer * q_.div + q) * mid_.div + mid) * p_.div + p) * inner_.div + inner, j);
+    return (((outer * q_.div + q) * mid_.div + mid) * p_.div + p) * inner_.div + inner;
   }
-
- private:
   Plan<SrcExp, DType> src_;
   const FastDivU32 inner_, q_, mid_, p_;
 };
