@@ -114,12 +114,16 @@ __device__ inline float BlockOrderedAdd(float s, const float (&t)[N],
  * plan; the steps here are
  *   A  every wave: approximate sum of each of its chunks -> LDS            (barrier)
  *   B  every wave (redundantly): prefix over all chunks, plan per chunk
- *   C  every wave: quantise its clean chunks, integer totals -> LDS; for its dirty
- *      chunks a plan per lane, parked in an LDS slot with the chunk's terms  (barrier)
- *   D  waves that own dirty chunks, in order: apply the clean run in front of each
- *      dirty chunk, walk the chunk (runs of clean lanes as integers, the other lanes
- *      term by term), hand the sum on through LDS                         (barrier each)
+ *   C  every wave: quantise its clean chunks, integer totals -> LDS; its dirty chunks
+ *      are parked, with their terms, in LDS slots                          (barrier)
+ *   D  every wave: integer prefix over the clean chunks; all waves together: a plan per
+ *      lane for each parked chunk, and the order of the slots in the row   (barrier)
+ *      wave 0: for each parked chunk in row order, apply the clean run in front of it
+ *      and walk it (runs of clean lanes as integers, the other lanes term by term),
+ *      fetching the next slot meanwhile                                    (barrier)
  *   E  every wave: apply the clean run behind the last dirty chunk.
+ * A row with more dirty chunks than slots is summed by wave scans instead (as is a row
+ * whose plan fails a verification).
  * Lane l keeps the chunk-table entries of chunks l * CPL .. l * CPL + CPL - 1. */
 const uint32_t kDirtyQ = 0xffffffffu;
 /*! \brief lanes of a row's first chunk that are added serially without a plan */
@@ -165,8 +169,8 @@ struct RowSumLds {
   int fail;      //!< a verification failed: redo the row the slow way
   uint32_t nslots;  //!< plan slots handed out
   float wmax[W];
-  /*! \brief per wave and slab: the plan slot of the chunk, or -1 */
-  signed char slot_of[W][SLABS];
+  /*! \brief the plan slots in the order of their chunks in the row */
+  signed char order[kSlots];
   LanePlanSlot<N> plan[kSlots];
 };
 
@@ -254,7 +258,7 @@ __device__ __forceinline__ uint32_t PlanLanes(const float (&t)[N], float start, 
  *  so the operands arrive in vector registers and the only chain is the adds themselves. */
 template <int N>
 __device__ __forceinline__ float HeadSerialAdd(float s, const float (*t)[N]) {
-  const int kBatch = 8;  // lanes whose terms are fetched before they are added
+  const int kBatch = 4;  // lanes whose terms are fetched before they are added
 #pragma unroll
   for (int l0 = 0; l0 < kHeadLanes; l0 += kBatch) {
     float r[kBatch][N];
@@ -497,7 +501,6 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
     const bool whole = clean && q < kLimit;  // a tie anywhere in the chunk pushes q past 2^24
     if (lane < SLABS) {
       lds->q[k] = whole ? static_cast<uint32_t>(q) : kDirtyQ;
-      lds->slot_of[wave][lane] = -1;
     }
     dirty_mask = static_cast<uint32_t>(__ballot(lane < SLABS && !whole));
     tie_mask = static_cast<uint32_t>(__ballot(lane < SLABS && clean && !whole));
@@ -510,7 +513,10 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
     uint32_t slot = 0u;
     if (lane == 0) slot = atomicAdd(&lds->nslots, 1u);
     slot = __builtin_amdgcn_readfirstlane(slot);
-    if (slot >= static_cast<uint32_t>(Lds::kSlots)) break;  // the rest is resolved by wave scans
+    if (slot >= static_cast<uint32_t>(Lds::kSlots)) {  // no room: the row is redone by wave scans
+      if (lane == 0) lds->fail = 1;
+      break;
+    }
     float t[N];
     SelectSlab<SLABS, N>(t, v, j);
     LanePlanSlot<N> *ps = &lds->plan[slot];
@@ -526,7 +532,6 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
       ps->kind = ck;
       ps->start = st;
       ps->chunk = k;
-      lds->slot_of[wave][j] = static_cast<signed char>(slot);
     }
   }
   __syncthreads();
@@ -534,8 +539,6 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
   /* D: tables of the walk */
   uint32_t ex[CPL];  // integer prefix over clean chunks in front of each chunk
   uint32_t total_ex;
-  uint32_t owners = 0u;  // waves that own at least one dirty chunk
-  const int LPW = SLABS / CPL;  // table lanes per wave
   {
     uint32_t pre[CPL + 1];
     pre[0] = 0u;
@@ -546,11 +549,6 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
       if (q == kDirtyQ && IsClean(static_cast<int>(code[c]))) code[c] = static_cast<uint32_t>(kPlanWalk);
       const bool is_dirty = k < NCH && !IsClean(static_cast<int>(code[c]));
       pre[c + 1] = pre[c] + (is_dirty ? 0u : q);
-      const unsigned long long mask = __ballot(is_dirty);
-#pragma unroll
-      for (int w = 0; w < W; ++w) {
-        owners |= (((mask >> (w * LPW)) & ((1ull << LPW) - 1ull)) != 0ull ? 1u : 0u) << w;
-      }
     }
     const uint32_t incl = WaveInclusiveScanU32(pre[CPL]);
     const uint32_t excl = incl - pre[CPL];
@@ -562,6 +560,8 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
   {
     const uint32_t handed = lds->nslots;
     const int nslots = handed < static_cast<uint32_t>(Lds::kSlots) ? static_cast<int>(handed) : Lds::kSlots;
+    /* slots were handed out in no particular order: the walk takes them by chunk number */
+    const int chunk_of_lane = lane < nslots ? lds->plan[lane < Lds::kSlots ? lane : 0].chunk : 0x7fffffff;
     for (int sl = wave; sl < nslots; sl += W) {
       LanePlanSlot<N> *ps = &lds->plan[sl];
       float t[N];
@@ -588,72 +588,79 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
       const int k = ps->chunk;
       const uint32_t exk = TableAt<CPL>(ex, k);
       const uint32_t erun = k > 0 ? TableAt<CPL>(code, k - 1) : 0u;
+      const int rank = __popcll(__ballot(chunk_of_lane < k));
       if (lane == 0) {
         ps->ex = exk;
         ps->e_run = static_cast<int>(erun);
+        lds->order[rank] = static_cast<signed char>(sl);
       }
     }
   }
 
   __syncthreads();
   MSHADOW_ROWSUM_STAMP(4)
-  for (int w = 0; w < W; ++w) {
-    if (((owners >> w) & 1u) == 0u) continue;  // block-uniform: every wave holds the same tables
-    if (wave == w) {
-      MSHADOW_ROWSUM_STAMP(8)
-      /* the walk is one chain of dependent instructions that the whole row waits for;
-         the other waves on this SIMD (another row's bulk phases) yield issue slots to it */
-      __builtin_amdgcn_s_setprio(3);
-      float s = lds->s;
-      uint32_t done = lds->ex;
-      bool fail = false;
-      for (uint32_t todo = dirty_mask; todo != 0u; todo &= todo - 1u) {
-        const int j = __ffs(static_cast<int>(todo)) - 1;
-        const int slot = lds->slot_of[w][j];
-        if (slot >= 0) {
-          /* everything about the chunk comes from its slot and none of it depends on s */
-          const LanePlanSlot<N> *ps = &lds->plan[slot];
-          float t[N];
+  /* the walk: one wave takes the dirty chunks in row order; everything it needs sits in the
+     plan slots */
+  if (wave == 0 && lds->fail == 0) {
+    MSHADOW_ROWSUM_STAMP(8)
+    /* the whole row waits for this chain; the other waves on this SIMD (another row's bulk
+       phases) yield issue slots to it */
+    __builtin_amdgcn_s_setprio(3);
+    const uint32_t handed = lds->nslots;
+    const int nslots = handed < static_cast<uint32_t>(Lds::kSlots) ? static_cast<int>(handed) : Lds::kSlots;
+    const int slot_at = lane < nslots ? lds->order[lane < Lds::kSlots ? lane : 0] : 0;
+    float s = 0.0f;
+    uint32_t done = 0u;
+    bool fail = false;
+    /* the lane-wise part of the next chunk's slot is fetched while the current chunk's chain
+       of dependent instructions runs (none of it depends on the running sum) */
+    float nt[N];
+    uint32_t npa = 0u, npb = 0u;
+    const LanePlanSlot<N> *nps = &lds->plan[ReadLaneU32(static_cast<uint32_t>(slot_at), 0)];
+    if (nslots > 0) {
 #pragma unroll
-          for (int i = 0; i < N; ++i) t[i] = ps->t[lane][i];
-          const uint32_t pa = ps->a[lane];
-          const uint32_t pb = ps->b[lane];
-          const int kind = ps->kind;
-          const uint32_t exk = ps->ex;
-          if (exk != done) {
-            s = FlushRun(s, ps->e_run, exk - done, &fail);
-            done = exk;
-          }
-          if (kind >= kPlanTwoBinades) {
-            s = WalkTwoBinades<N>(s, t, kind - kPlanTwoBinades, pa, pb, ps->tie_lo, ps->tie_hi, &fail);
-          } else if (ps->chunk == 0) {
-            s = HeadSerialAdd<N>(s, ps->t);
-            s = WalkLanes<N>(s, t, pa, static_cast<int>(pb), ps->total, (1ull << kHeadLanes) - 1ull, &fail);
-          } else {
-            s = WalkLanes<N>(s, t, pa, static_cast<int>(pb), ps->total, 0ull, &fail);
-          }
-        } else {
-          const int k = w * SLABS + j;
-          const uint32_t exk = TableAt<CPL>(ex, k);
-          if (exk != done) {
-            s = FlushRun(s, static_cast<int>(TableAt<CPL>(code, k - 1)), exk - done, &fail);
-            done = exk;
-          }
-          float t[N];
-          SelectSlab<SLABS, N>(t, v, j);
-          s = WaveResolve<N>(s, t);
-        }
-      }
-      if (lane == 0) {
-        lds->s = s;
-        lds->ex = done;
-        if (fail) lds->fail = 1;
-      }
-      __builtin_amdgcn_s_setprio(0);
-      MSHADOW_ROWSUM_STAMP(9)
+      for (int e = 0; e < N; ++e) nt[e] = nps->t[lane][e];
+      npa = nps->a[lane];
+      npb = nps->b[lane];
     }
-    __syncthreads();
+    for (int i = 0; i < nslots; ++i) {
+      const LanePlanSlot<N> *ps = nps;
+      float t[N];
+#pragma unroll
+      for (int e = 0; e < N; ++e) t[e] = nt[e];
+      const uint32_t pa = npa, pb = npb;
+      const int kind = ps->kind;
+      const uint32_t exk = ps->ex;
+      const int erun = ps->e_run;
+      if (i + 1 < nslots) {
+        nps = &lds->plan[ReadLaneU32(static_cast<uint32_t>(slot_at), i + 1)];
+#pragma unroll
+        for (int e = 0; e < N; ++e) nt[e] = nps->t[lane][e];
+        npa = nps->a[lane];
+        npb = nps->b[lane];
+      }
+      if (exk != done) {
+        s = FlushRun(s, erun, exk - done, &fail);
+        done = exk;
+      }
+      if (kind >= kPlanTwoBinades) {
+        s = WalkTwoBinades<N>(s, t, kind - kPlanTwoBinades, pa, pb, ps->tie_lo, ps->tie_hi, &fail);
+      } else if (ps->chunk == 0) {
+        s = HeadSerialAdd<N>(s, ps->t);
+        s = WalkLanes<N>(s, t, pa, static_cast<int>(pb), ps->total, (1ull << kHeadLanes) - 1ull, &fail);
+      } else {
+        s = WalkLanes<N>(s, t, pa, static_cast<int>(pb), ps->total, 0ull, &fail);
+      }
+    }
+    if (lane == 0) {
+      lds->s = s;
+      lds->ex = done;
+      if (fail) lds->fail = 1;
+    }
+    __builtin_amdgcn_s_setprio(0);
+    MSHADOW_ROWSUM_STAMP(9)
   }
+  __syncthreads();
 
   /* E: the clean run behind the last dirty chunk */
   MSHADOW_ROWSUM_STAMP(5)
