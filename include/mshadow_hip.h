@@ -182,6 +182,13 @@ int mshadow_hip_index_fill_f32(float *dst, int dstride, int k_rows, const void *
                                int index_is_int, int n_index, const float *src, int sstride,
                                int cols, void *stream);
 
+/* dst = transpose(src, axes) / dst = swapaxis<a1, a2>(src) on dense tensors of 32-bit
+   elements: dst axis i is src axis axes[i]; `shape` is the source's, ndim <= 6
+   (mshadow/extension/transpose.h:24-88, swapaxis.h:20-106, evaluated there element by element
+   through the generic map kernel). dst and src must not overlap. */
+int mshadow_hip_permute_32(void *dst, const void *src, int ndim, const int *shape,
+                           const int *axes, void *stream);
+
 /* SortByKey(keys, values, is_ascend): stable sort of the pairs by key, in place
    (mshadow/tensor_gpu-inl.h:231-235 -> tensor_gpu-inl.cuh:784-806, thrust::stable_sort_by_key;
    CPU tensor_cpu-inl.h:531-559). Keys and values are 32-bit elements; key_kind says how the key

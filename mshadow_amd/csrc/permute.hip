@@ -1,0 +1,296 @@
+/*
+ * Permutation of the axes of a dense tensor of 32-bit elements: dst axis i is src axis
+ * axes[i]. This is what `dst = transpose(src, axes)` and `dst = swapaxis<a1, a2>(src)`
+ * compute (mshadow/extension/transpose.h:24-88, swapaxis.h:20-106 of the reference, which
+ * evaluate them element by element through the generic map kernel).
+ *
+ * On the host the problem is first reduced: axes of length 1 are dropped and axes that
+ * stay neighbours in the same order are merged, so NCHW -> NHWC becomes a batch of 2-D
+ * transposes (n, c, h*w) -> (n, h*w, c). Then
+ *  - if the last axis stays last, rows are permuted: one thread per 16 bytes (or per
+ *    element), the source row found by taking the destination row number apart;
+ *  - otherwise the source's last axis (extent L) lands on some other destination axis and
+ *    the destination's last axis (extent A) comes from some other source axis: the two span
+ *    a plane that is moved in 64 x 64 tiles through LDS, read along L and written along A,
+ *    so that both sides are coalesced. The remaining axes are batch indices.
+ * Pure data movement: bit-exact. HBM-bound, 2 * 4 bytes per element.
+ */
+#include <mshadow/core/fastdiv.h>
+#include <mshadow/hip/kernels/common.h>
+
+#include "./abi_common.h"
+
+using mshadow::FastDivU32;
+using mshadow_abi::AfterLaunch;
+using mshadow_abi::AsStream;
+
+namespace {
+
+const int kMaxAxes = 6;
+const int kTile = 64;
+const int kPermuteBlock = 256;
+
+/*! \brief the batch axes of the reduced problem: how to take a batch number apart and what
+ *  each digit is worth in the source and in the destination */
+struct BatchAxes {
+  int count;
+  FastDivU32 extent[kMaxAxes];
+  uint32_t src_step[kMaxAxes];
+  uint32_t dst_step[kMaxAxes];
+  __device__ __forceinline__ void Offsets(uint32_t batch, uint32_t *src_off, uint32_t *dst_off) const {
+    uint32_t s = 0, d = 0;
+    for (int k = count - 1; k >= 0; --k) {
+      const uint32_t q = extent[k].Div(batch);
+      const uint32_t digit = batch - q * extent[k].div;
+      s += digit * src_step[k];
+      d += digit * dst_step[k];
+      batch = q;
+    }
+    *src_off = s;
+    *dst_off = d;
+  }
+};
+
+/*! \brief one 64 x 64 tile of the (A, L) plane per workgroup: src[batch][a][l] at
+ *  a * src_step_a + l, dst[batch][l][a] at l * dst_step_l + a */
+__global__ void __launch_bounds__(kPermuteBlock)
+    PermuteTileKernel(uint32_t *dst, const uint32_t *src, uint32_t extent_a, uint32_t extent_l,
+                      uint32_t src_step_a, uint32_t dst_step_l, FastDivU32 tiles_a,
+                      FastDivU32 tiles_l, BatchAxes batch_axes) {
+  __shared__ uint32_t tile[kTile][kTile + 1];
+  const uint32_t block = mshadow::hip::StripOfBlock(blockIdx.x, gridDim.x);
+  const uint32_t rest = tiles_l.Div(block);
+  const uint32_t tl = block - rest * tiles_l.div;
+  const uint32_t batch = tiles_a.Div(rest);
+  const uint32_t ta = rest - batch * tiles_a.div;
+  uint32_t src_off, dst_off;
+  batch_axes.Offsets(batch, &src_off, &dst_off);
+  const uint32_t tx = threadIdx.x % kTile, ty = threadIdx.x / kTile;
+  const int kRowsPerPass = kPermuteBlock / kTile;
+  {
+    const uint32_t l = tl * kTile + tx;
+    const uint32_t *from = src + src_off + l;
+#pragma unroll
+    for (int r = 0; r < kTile; r += kRowsPerPass) {
+      const uint32_t a = ta * kTile + r + ty;
+      if (a < extent_a && l < extent_l) {
+        tile[r + ty][tx] = __builtin_nontemporal_load(from + static_cast<size_t>(a) * src_step_a);
+      }
+    }
+  }
+  __syncthreads();
+  {
+    const uint32_t a = ta * kTile + tx;
+    uint32_t *to = dst + dst_off + a;
+#pragma unroll
+    for (int r = 0; r < kTile; r += kRowsPerPass) {
+      const uint32_t l = tl * kTile + r + ty;
+      if (a < extent_a && l < extent_l) {
+        __builtin_nontemporal_store(tile[tx][r + ty], to + static_cast<size_t>(l) * dst_step_l);
+      }
+    }
+  }
+}
+
+/*! \brief the same tile with 128-bit global accesses on both sides (extents, steps and
+ *  offsets are multiples of four words, pointers 16-byte aligned). A thread moves four
+ *  adjacent words of a row; the transposition happens in the word-wise LDS accesses, whose
+ *  row pitch of 65 words spreads the 64 lanes over all banks. */
+__global__ void __launch_bounds__(kPermuteBlock)
+    PermuteTileVecKernel(uint32_t *dst, const uint32_t *src, uint32_t extent_a, uint32_t extent_l,
+                         uint32_t src_step_a, uint32_t dst_step_l, FastDivU32 tiles_a,
+                         FastDivU32 tiles_l, BatchAxes batch_axes) {
+  typedef uint32_t Vec4 __attribute__((ext_vector_type(4)));
+  __shared__ uint32_t tile[kTile][kTile + 1];
+  const uint32_t block = mshadow::hip::StripOfBlock(blockIdx.x, gridDim.x);
+  const uint32_t rest = tiles_l.Div(block);
+  const uint32_t tl = block - rest * tiles_l.div;
+  const uint32_t batch = tiles_a.Div(rest);
+  const uint32_t ta = rest - batch * tiles_a.div;
+  uint32_t src_off, dst_off;
+  batch_axes.Offsets(batch, &src_off, &dst_off);
+  const int kLanesPerRow = kTile / 4;                       // 16 threads cover a row of the tile
+  const int kRowsPerPass = kPermuteBlock / kLanesPerRow;    // 16 rows per pass
+  const uint32_t tx = (threadIdx.x % kLanesPerRow) * 4, ty = threadIdx.x / kLanesPerRow;
+  {
+    const uint32_t l = tl * kTile + tx;
+    const uint32_t *from = src + src_off + l;
+    Vec4 got[kTile / kRowsPerPass];
+#pragma unroll
+    for (int r = 0; r < kTile; r += kRowsPerPass) {
+      const uint32_t a = ta * kTile + r + ty;
+      if (a < extent_a && l < extent_l) {
+        got[r / kRowsPerPass] = __builtin_nontemporal_load(
+            reinterpret_cast<const Vec4 *>(from + static_cast<size_t>(a) * src_step_a));
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < kTile; r += kRowsPerPass) {
+      const Vec4 v = got[r / kRowsPerPass];
+      tile[r + ty][tx + 0] = v.x;
+      tile[r + ty][tx + 1] = v.y;
+      tile[r + ty][tx + 2] = v.z;
+      tile[r + ty][tx + 3] = v.w;
+    }
+  }
+  __syncthreads();
+  {
+    const uint32_t a = ta * kTile + tx;
+    uint32_t *to = dst + dst_off + a;
+#pragma unroll
+    for (int r = 0; r < kTile; r += kRowsPerPass) {
+      const uint32_t l = tl * kTile + r + ty;
+      Vec4 v;
+      v.x = tile[tx + 0][r + ty];
+      v.y = tile[tx + 1][r + ty];
+      v.z = tile[tx + 2][r + ty];
+      v.w = tile[tx + 3][r + ty];
+      if (a < extent_a && l < extent_l) {
+        __builtin_nontemporal_store(v, reinterpret_cast<Vec4 *>(to + static_cast<size_t>(l) * dst_step_l));
+      }
+    }
+  }
+}
+
+/*! \brief the last axis stays: destination row `row` is source row Offsets(row); WORDS
+ *  32-bit words per thread (4 when rows are made of whole aligned 16-byte packs) */
+template <int WORDS>
+__global__ void __launch_bounds__(kPermuteBlock)
+    PermuteRowsKernel(uint32_t *dst, const uint32_t *src, uint32_t rows, uint32_t cols,
+                      FastDivU32 packs_per_row, BatchAxes row_axes) {
+  typedef uint32_t Vec __attribute__((ext_vector_type(WORDS)));
+  const uint32_t total = rows * packs_per_row.div;
+  const uint32_t step = gridDim.x * kPermuteBlock;
+  const uint32_t block = mshadow::hip::StripOfBlock(blockIdx.x, gridDim.x);
+  for (uint32_t p = block * kPermuteBlock + threadIdx.x; p < total; p += step) {
+    const uint32_t row = packs_per_row.Div(p);
+    const uint32_t x = (p - row * packs_per_row.div) * WORDS;
+    uint32_t src_off, dst_off;
+    row_axes.Offsets(row, &src_off, &dst_off);
+    const Vec v = __builtin_nontemporal_load(reinterpret_cast<const Vec *>(src + src_off + x));
+    __builtin_nontemporal_store(v, reinterpret_cast<Vec *>(dst + static_cast<size_t>(row) * cols + x));
+  }
+}
+
+}  // namespace
+
+extern "C" int mshadow_hip_permute_32(void *dst, const void *src, int ndim, const int *shape,
+                                      const int *axes, void *stream) {
+  ABI_REQUIRE(ndim >= 1 && ndim <= kMaxAxes, "1 to 6 axes");
+  ABI_REQUIRE(shape != NULL && axes != NULL, "NULL shape or axes");
+  bool seen[kMaxAxes] = {false, false, false, false, false, false};
+  uint64_t total = 1;
+  for (int i = 0; i < ndim; ++i) {
+    ABI_REQUIRE(axes[i] >= 0 && axes[i] < ndim && !seen[axes[i]], "axes is not a permutation");
+    ABI_REQUIRE(shape[i] >= 0, "negative shape");
+    seen[axes[i]] = true;
+    total *= static_cast<uint64_t>(shape[i]);
+  }
+  if (total == 0) return MSHADOW_HIP_OK;
+  ABI_REQUIRE(total < (1ull << 31), "too many elements");
+  ABI_REQUIRE(dst != NULL && src != NULL, "NULL tensor");
+
+  /* reduce: walk the destination axes, drop extents of 1, merge an axis into the previous
+     one when the two are neighbours in the source as well */
+  uint32_t src_step_of[kMaxAxes];
+  {
+    uint32_t step = 1;
+    for (int k = ndim - 1; k >= 0; --k) {
+      src_step_of[k] = step;
+      step *= static_cast<uint32_t>(shape[k]);
+    }
+  }
+  uint32_t ext[kMaxAxes], sstep[kMaxAxes];
+  int from_axis[kMaxAxes];
+  int n = 0;
+  for (int i = 0; i < ndim; ++i) {
+    const int a = axes[i];
+    if (shape[a] == 1) continue;
+    if (n > 0 && sstep[n - 1] == src_step_of[a] * static_cast<uint32_t>(shape[a])) {
+      ext[n - 1] *= static_cast<uint32_t>(shape[a]);   // (previous, this) is one run of the source
+      sstep[n - 1] = src_step_of[a];
+      continue;
+    }
+    ext[n] = static_cast<uint32_t>(shape[a]);
+    sstep[n] = src_step_of[a];
+    from_axis[n] = a;
+    ++n;
+  }
+  (void)from_axis;
+  hipStream_t s = AsStream(stream);
+  if (n <= 1) {  // the elements keep their order
+    ABI_HIP(hipMemcpyAsync(dst, src, total * sizeof(uint32_t), hipMemcpyDeviceToDevice, s));
+    return MSHADOW_HIP_OK;
+  }
+  uint32_t dstep[kMaxAxes];
+  {
+    uint32_t step = 1;
+    for (int k = n - 1; k >= 0; --k) {
+      dstep[k] = step;
+      step *= ext[k];
+    }
+  }
+  uint32_t *d = static_cast<uint32_t *>(dst);
+  const uint32_t *sp = static_cast<const uint32_t *>(src);
+  if (sstep[n - 1] == 1) {
+    /* rows of ext[n-1] elements are permuted */
+    BatchAxes ba;
+    ba.count = n - 1;
+    uint32_t rows = 1;
+    for (int k = 0; k < n - 1; ++k) {
+      ba.extent[k] = FastDivU32(ext[k]);
+      ba.src_step[k] = sstep[k];
+      ba.dst_step[k] = dstep[k];
+      rows *= ext[k];
+    }
+    const uint32_t cols = ext[n - 1];
+    const bool wide = cols % 4 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(src) % 16 == 0;
+    const uint32_t ppr = wide ? cols / 4 : cols;
+    const uint64_t work = static_cast<uint64_t>(rows) * ppr;
+    uint64_t blocks = (work + kPermuteBlock - 1) / kPermuteBlock;
+    if (blocks > 65536) blocks = 65536;
+    if (wide) {
+      hipLaunchKernelGGL(PermuteRowsKernel<4>, dim3(static_cast<unsigned>(blocks)), dim3(kPermuteBlock),
+                         0, s, d, sp, rows, cols, FastDivU32(ppr), ba);
+    } else {
+      hipLaunchKernelGGL(PermuteRowsKernel<1>, dim3(static_cast<unsigned>(blocks)), dim3(kPermuteBlock),
+                         0, s, d, sp, rows, cols, FastDivU32(ppr), ba);
+    }
+    return AfterLaunch("permute (rows)");
+  }
+  /* the source's last axis is destination axis b; the destination's last axis is n - 1 */
+  int b = -1;
+  for (int k = 0; k < n; ++k) {
+    if (sstep[k] == 1) b = k;
+  }
+  ABI_REQUIRE(b >= 0 && b < n - 1, "internal: no unit-stride axis");
+  BatchAxes ba;
+  ba.count = 0;
+  uint64_t batches = 1;
+  for (int k = 0; k < n - 1; ++k) {
+    if (k == b) continue;
+    ba.extent[ba.count] = FastDivU32(ext[k]);
+    ba.src_step[ba.count] = sstep[k];
+    ba.dst_step[ba.count] = dstep[k];
+    ++ba.count;
+    batches *= ext[k];
+  }
+  const uint32_t extent_a = ext[n - 1], extent_l = ext[b];
+  const uint32_t ta = (extent_a + kTile - 1) / kTile, tl = (extent_l + kTile - 1) / kTile;
+  const uint64_t blocks = batches * ta * tl;
+  ABI_REQUIRE(blocks < (1ull << 31), "too many tiles");
+  bool wide = extent_a % 4 == 0 && extent_l % 4 == 0 && sstep[n - 1] % 4 == 0 && dstep[b] % 4 == 0 &&
+              reinterpret_cast<uintptr_t>(dst) % 16 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0;
+  for (int k = 0; k < ba.count; ++k) wide = wide && ba.src_step[k] % 4 == 0 && ba.dst_step[k] % 4 == 0;
+  if (wide) {
+    hipLaunchKernelGGL(PermuteTileVecKernel, dim3(static_cast<unsigned>(blocks)), dim3(kPermuteBlock),
+                       0, s, d, sp, extent_a, extent_l, sstep[n - 1], dstep[b], FastDivU32(ta),
+                       FastDivU32(tl), ba);
+  } else {
+    hipLaunchKernelGGL(PermuteTileKernel, dim3(static_cast<unsigned>(blocks)), dim3(kPermuteBlock), 0,
+                       s, d, sp, extent_a, extent_l, sstep[n - 1], dstep[b], FastDivU32(ta),
+                       FastDivU32(tl), ba);
+  }
+  return AfterLaunch("permute (tiles)");
+}

@@ -311,6 +311,14 @@ template <typename Saver, int dim, typename DType, typename E>
 struct FastPath {
   inline static bool Run(Tensor<gpu, dim, DType> *dst, const E &exp) { return false; }
 };
+/* a chainer node reaches the engine as its MakeTensorExp base: match on the concrete node */
+template <typename Saver, int dim, typename DType, typename Node, typename SrcExp>
+struct FastPath<Saver, dim, DType, expr::MakeTensorExp<Node, SrcExp, dim, DType> > {
+  inline static bool Run(Tensor<gpu, dim, DType> *dst,
+                         const expr::MakeTensorExp<Node, SrcExp, dim, DType> &exp) {
+    return FastPath<Saver, dim, DType, Node>::Run(dst, exp.real_self());
+  }
+};
 
 /* dst = pool<Reducer>(float tensor, ...) */
 template <typename Reducer, int dim>
@@ -382,12 +390,15 @@ struct HasPatchAbi<half::half_t> { static const bool value = true; };
 template <typename DType, int sdim>
 struct FastPath<sv::saveto, 2, DType,
                 expr::UnpackPatchToColXExp<
-                    expr::PaddingExp<Tensor<gpu, sdim, DType>, DType, sdim>, DType, sdim> > {
-  typedef expr::UnpackPatchToColXExp<expr::PaddingExp<Tensor<gpu, sdim, DType>, DType, sdim>,
-                                     DType, sdim> E;
+                    expr::MakeTensorExp<expr::PaddingExp<Tensor<gpu, sdim, DType>, DType, sdim>,
+                                        Tensor<gpu, sdim, DType>, sdim, DType>,
+                    DType, sdim> > {
+  typedef expr::PaddingExp<Tensor<gpu, sdim, DType>, DType, sdim> Pad;
+  typedef expr::UnpackPatchToColXExp<
+      expr::MakeTensorExp<Pad, Tensor<gpu, sdim, DType>, sdim, DType>, DType, sdim> E;
   inline static bool Run(Tensor<gpu, 2, DType> *dst, const E &e) {
     if (!HasPatchAbi<DType>::value) return false;
-    const expr::PaddingExp<Tensor<gpu, sdim, DType>, DType, sdim> &p = e.img_;
+    const Pad &p = e.img_.real_self();
     const Tensor<gpu, sdim, DType> &img = p.src_;
     MSHADOW_HIP_CALL(PatchAbi<DType>::Im2Col(
         dst->dptr_, dst->stride_, img.dptr_, img.stride_, img.shape_.ProdShape(0, sdim - 3),
@@ -415,13 +426,16 @@ struct FastPath<sv::saveto, 2, DType,
 /* img = crop(pack_col2patch(col, padded shape, ...), (h, w), py, px) */
 template <typename DType, int ddim>
 struct FastPath<sv::saveto, ddim, DType,
-                expr::CroppingExp<expr::PackColToPatchXExp<Tensor<gpu, 2, DType>, DType, ddim>,
-                                  DType, ddim> > {
+                expr::CroppingExp<
+                    expr::MakeTensorExp<expr::PackColToPatchXExp<Tensor<gpu, 2, DType>, DType, ddim>,
+                                        Tensor<gpu, 2, DType>, ddim, DType>,
+                    DType, ddim> > {
   typedef expr::PackColToPatchXExp<Tensor<gpu, 2, DType>, DType, ddim> Pack;
-  typedef expr::CroppingExp<Pack, DType, ddim> E;
+  typedef expr::CroppingExp<expr::MakeTensorExp<Pack, Tensor<gpu, 2, DType>, ddim, DType>, DType,
+                            ddim> E;
   inline static bool Run(Tensor<gpu, ddim, DType> *dst, const E &e) {
     if (!HasPatchAbi<DType>::value) return false;
-    const Pack &p = e.src_;
+    const Pack &p = e.src_.real_self();
     const index_t h = e.shape_[ddim - 2], w = e.shape_[ddim - 1];
     /* the fixed-function kernel handles symmetric padding: the crop must sit pad_y / pad_x
        inside an image that is exactly 2 * pad larger */
@@ -451,6 +465,46 @@ struct FastPath<sv::saveto, ddim, DType,
         p.pstride_y_, p.pstride_x_, p.pdilate_y_, p.pdilate_x_, 0, 0,
         Stream<gpu>::GetStream(dst->stream_)));
     return true;
+  }
+};
+
+/* dst = transpose(tensor, axes) and dst = swapaxis<a1, a2>(tensor) on dense tensors of 32-bit
+   elements: the tiled permutation of the library */
+template <typename DType, int dim>
+inline bool PermuteInto(Tensor<gpu, dim, DType> *dst, const Tensor<gpu, dim, DType> &src,
+                        const int (&axes)[dim]) {
+  if (sizeof(DType) != 4 || dim > 6 || !dst->CheckContiguous() || !src.CheckContiguous()) return false;
+  int shape[dim];
+  for (int i = 0; i < dim; ++i) shape[i] = static_cast<int>(src.shape_[i]);
+  MSHADOW_HIP_CALL(mshadow_hip_permute_32(dst->dptr_, src.dptr_, dim, shape, axes,
+                                          Stream<gpu>::GetStream(dst->stream_)));
+  return true;
+}
+template <typename DType, int dim>
+struct FastPath<sv::saveto, dim, DType, expr::TransposeExExp<Tensor<gpu, dim, DType>, DType, dim> > {
+  typedef expr::TransposeExExp<Tensor<gpu, dim, DType>, DType, dim> E;
+  inline static bool Run(Tensor<gpu, dim, DType> *dst, const E &e) {
+    int axes[dim];
+    bool seen[dim];
+    for (int i = 0; i < dim; ++i) seen[i] = false;
+    for (int i = 0; i < dim; ++i) {
+      axes[i] = static_cast<int>(e.axes_[i]);
+      if (axes[i] >= dim || seen[axes[i]]) return false;  // not a permutation: evaluated as written
+      seen[axes[i]] = true;
+    }
+    return PermuteInto(dst, e.src_, axes);
+  }
+};
+template <typename DType, int dim, int m_a1, int a2>
+struct FastPath<sv::saveto, dim, DType,
+                expr::SwapAxisExp<Tensor<gpu, dim, DType>, DType, dim, m_a1, a2> > {
+  typedef expr::SwapAxisExp<Tensor<gpu, dim, DType>, DType, dim, m_a1, a2> E;
+  inline static bool Run(Tensor<gpu, dim, DType> *dst, const E &e) {
+    int axes[dim];
+    for (int i = 0; i < dim; ++i) axes[i] = i;
+    axes[dim - m_a1] = a2;
+    axes[a2] = dim - m_a1;
+    return PermuteInto(dst, e.src_, axes);
   }
 };
 

@@ -249,3 +249,36 @@ def test_gpu_matches_numpy(shape, op):
     G.case_extensions(op, out, dev(case.a), dev(case.b), dev(case.c), *shape, *case.p)
     got = out.download()
     assert np.array_equal(got.view(np.uint32), case.want.view(np.uint32)), (op, shape)
+
+
+PERMUTE_CASES = [
+    ((5, 7), (1, 0)), ((64, 64), (1, 0)), ((65, 130), (1, 0)), ((1, 9), (1, 0)),
+    ((3, 4, 5), (2, 1, 0)), ((3, 4, 5), (1, 0, 2)), ((3, 4, 5), (0, 2, 1)), ((3, 4, 5), (2, 0, 1)),
+    ((2, 3, 4, 8), (0, 2, 3, 1)), ((2, 3, 4, 8), (0, 3, 1, 2)), ((2, 3, 4, 8), (3, 2, 1, 0)),
+    ((2, 3, 4, 8), (1, 0, 2, 3)), ((2, 3, 4, 8), (0, 1, 2, 3)), ((2, 1, 4, 1), (3, 2, 1, 0)),
+    ((4, 16, 70, 3), (0, 2, 3, 1)), ((2, 3, 2, 5, 6), (4, 0, 3, 1, 2)), ((2, 2, 3, 2, 2, 5), (5, 4, 3, 2, 1, 0)),
+    ((8, 100, 33, 9), (0, 3, 1, 2)), ((0, 4, 5), (2, 1, 0)),
+    ((2, 68, 8, 12), (0, 2, 3, 1)), ((3, 128, 200), (0, 2, 1)), ((4, 8, 16, 12), (3, 1, 2, 0)),
+    ((2, 4, 36, 4), (2, 0, 1, 3)),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape,axes", PERMUTE_CASES)
+@pytest.mark.parametrize("dtype", [np.float32, np.int32])
+def test_permute_entry_point(shape, axes, dtype):
+    """mshadow_hip_permute_32 against numpy.transpose: every element in its new place"""
+    import mshadow_amd
+    G = mshadow_amd.load_cases()
+    G.set_device(0)
+    a = np.arange(int(np.prod(shape)), dtype=np.int64).reshape(shape)
+    a = (a * 2654435761 % 2**31).astype(dtype)       # every element distinct enough to notice a mix-up
+    want = np.ascontiguousarray(a.transpose(axes))
+    if a.size == 0:   # nothing to move: the call must succeed without touching memory
+        src, out = G.buffer((1,), dtype), G.buffer((1,), dtype)
+        src.shape = shape
+        G.permute(out, src, axes)
+        return
+    out = G.to_device(np.full(want.shape, -1, dtype))
+    G.permute(out, G.to_device(a), axes)
+    assert np.array_equal(out.download(), want), (shape, axes)

@@ -47,6 +47,24 @@ def test_python_symbol_tables_match_headers():
     assert sorted(capi.CASES_SYMBOLS) == _declared("mshadow_hip_cases.h")
 
 
+def test_expression_routes_reach_the_fixed_function_entries():
+    """`dst = pool(...)`, `unpool`, `unpack_patch2col(pad(.))`, `crop(pack_col2patch(.))`,
+    `transpose` / `swapaxis` of plain tensors and the reductions are recognised at compile
+    time and handed to the library: the caller-style cases library, which only ever writes
+    expressions, must therefore import those entry points"""
+    if not os.path.exists(os.path.join(LIBDIR, "libmshadow_cases.so")):
+        _lib("libmshadow_cases.so")
+    out = subprocess.run(["nm", "-D", "--undefined-only", os.path.join(LIBDIR, "libmshadow_cases.so")],
+                         check=True, capture_output=True, text=True).stdout
+    imported = set(re.findall(r"\bU (mshadow_hip_\w+)", out))
+    wanted = {"mshadow_hip_pool_f32", "mshadow_hip_unpool_f32", "mshadow_hip_im2col_f16",
+              "mshadow_hip_im2col_f32", "mshadow_hip_col2im_f16", "mshadow_hip_col2im_f32",
+              "mshadow_hip_permute_32", "mshadow_hip_reduce_keep_lowest_f32",
+              "mshadow_hip_reduce_keep_highdim_f32", "mshadow_hip_softmax_f32",
+              "mshadow_hip_sort_by_key_32"}
+    assert wanted <= imported, sorted(wanted - imported)
+
+
 def _compile_and_run(tmp_path, source, extra):
     exe = str(tmp_path / "check")
     cmd = ["g++", "-std=c++17", "-O2", "-fopenmp", "-ffp-contract=off", "-mf16c",
