@@ -105,6 +105,11 @@ int mshadow_hip_memcpy2d_async(void *dst, size_t dpitch_bytes, const void *src,
                                size_t spitch_bytes, size_t width_bytes, size_t rows, int kind,
                                void *stream);
 int mshadow_hip_memset_async(void *dst, int byte_value, size_t bytes, void *stream);
+/* dst = scalar on a (rows, cols) view of 32-bit elements with pitch dstride (elements):
+   what `tensor = value` and NewTensor's initial value do through MapExp in the reference
+   (mshadow/tensor_gpu-inl.h:101-116 with a ScalarExp source). `bits` is the element's
+   bit pattern. A kernel, not a memset: it may be recorded into a graph. */
+int mshadow_hip_fill_32(void *dst, int dstride, int rows, int cols, uint32_t bits, void *stream);
 
 /* ------------------------------------------------------------------ 2. launch */
 

@@ -70,6 +70,7 @@ HIP_SYMBOLS = {
     "mshadow_hip_add_take_grad_f32": ([_p, _i, _i, _p, _i, _i, _p, _i, _i, _p], _i),
     "mshadow_hip_add_take_grad_large_batch_f32": ([_p, _i, _i, _p, _p, _i, _i, _p, _i, _i, _p], _i),
     "mshadow_hip_index_fill_f32": ([_p, _i, _i, _p, _i, _i, _p, _i, _i, _p], _i),
+    "mshadow_hip_fill_32": ([_p, _i, _i, _i, C.c_uint32, _p], _i),
     "mshadow_hip_permute_32": ([_p, _p, _i, C.POINTER(_i), C.POINTER(_i), _p], _i),
     "mshadow_hip_sort_by_key_workspace": ([_sz, C.POINTER(_sz)], _i),
     "mshadow_hip_sort_by_key_32": ([_p, _i, _p, _sz, _i, _p, _sz, _p], _i),
@@ -293,6 +294,11 @@ class Library:
         self.check(self.dll.mshadow_hip_index_fill_f32(
             dst.ptr, dst.stride, dst.rows, index.ptr, self._index_is_int(index), index.cols,
             src.ptr, src.stride, src.cols, stream))
+
+    def fill(self, dst, value, stream=None):
+        """every element of a buffer of 32-bit elements set to `value`"""
+        bits = int(np.array([value], dtype=dst.dtype).view(np.uint32)[0])
+        self.check(self.dll.mshadow_hip_fill_32(dst.ptr, dst.stride, dst.rows, dst.cols, bits, stream))
 
     def permute(self, dst, src, axes, stream=None):
         """dst axis i = src axis axes[i]; dense buffers of 32-bit elements"""

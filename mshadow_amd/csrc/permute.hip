@@ -14,6 +14,8 @@
  *    a plane that is moved in 64 x 64 tiles through LDS, read along L and written along A,
  *    so that both sides are coalesced. The remaining axes are batch indices.
  * Pure data movement: bit-exact. HBM-bound, 2 * 4 bytes per element.
+ *
+ * Also here: the fill of a 2-D view with one 32-bit pattern (`tensor = scalar`).
  */
 #include <mshadow/core/fastdiv.h>
 #include <mshadow/hip/kernels/common.h>
@@ -172,7 +174,50 @@ __global__ void __launch_bounds__(kPermuteBlock)
   }
 }
 
+/*! \brief every element of a pitched 2-D view set to one 32-bit pattern; WORDS words per
+ *  store (4 when rows are made of whole aligned 16-byte packs) */
+template <int WORDS>
+__global__ void __launch_bounds__(kPermuteBlock)
+    FillKernel(uint32_t *dst, uint32_t stride, uint32_t rows, uint32_t packs_per_row,
+               FastDivU32 div_ppr, uint32_t bits) {
+  typedef uint32_t Vec __attribute__((ext_vector_type(WORDS)));
+  Vec v;
+#pragma unroll
+  for (int k = 0; k < WORDS; ++k) v[k] = bits;
+  const uint32_t total = rows * packs_per_row;
+  const uint32_t step = gridDim.x * kPermuteBlock;
+  for (uint32_t i = blockIdx.x * kPermuteBlock + threadIdx.x; i < total; i += step) {
+    const uint32_t y = div_ppr.Div(i);
+    __builtin_nontemporal_store(
+        v, reinterpret_cast<Vec *>(dst + static_cast<size_t>(y) * stride + (i - y * packs_per_row) * WORDS));
+  }
+}
+
 }  // namespace
+
+extern "C" int mshadow_hip_fill_32(void *dst, int dstride, int rows, int cols, uint32_t bits,
+                                   void *stream) {
+  ABI_REQUIRE(rows >= 0 && cols >= 0, "negative shape");
+  if (rows == 0 || cols == 0) return MSHADOW_HIP_OK;
+  ABI_REQUIRE(dst != NULL, "NULL tensor");
+  ABI_REQUIRE(dstride >= cols, "pitch smaller than the row");
+  const uint64_t total = static_cast<uint64_t>(rows) * cols;
+  ABI_REQUIRE(total < (1ull << 31), "too many elements");
+  const bool wide = cols % 4 == 0 && dstride % 4 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0;
+  const uint32_t ppr = static_cast<uint32_t>(wide ? cols / 4 : cols);
+  uint64_t blocks = (static_cast<uint64_t>(rows) * ppr + kPermuteBlock - 1) / kPermuteBlock;
+  if (blocks > 65536) blocks = 65536;
+  if (wide) {
+    hipLaunchKernelGGL(FillKernel<4>, dim3(static_cast<unsigned>(blocks)), dim3(kPermuteBlock), 0,
+                       AsStream(stream), static_cast<uint32_t *>(dst), static_cast<uint32_t>(dstride),
+                       static_cast<uint32_t>(rows), ppr, FastDivU32(ppr), bits);
+  } else {
+    hipLaunchKernelGGL(FillKernel<1>, dim3(static_cast<unsigned>(blocks)), dim3(kPermuteBlock), 0,
+                       AsStream(stream), static_cast<uint32_t *>(dst), static_cast<uint32_t>(dstride),
+                       static_cast<uint32_t>(rows), ppr, FastDivU32(ppr), bits);
+  }
+  return AfterLaunch("fill");
+}
 
 extern "C" int mshadow_hip_permute_32(void *dst, const void *src, int ndim, const int *shape,
                                       const int *axes, void *stream) {

@@ -17,6 +17,8 @@
 
 #include <mshadow_hip.h>
 
+#include <cstring>
+
 #include "../tensor.h"
 #include "./stream.h"
 
@@ -468,6 +470,19 @@ struct FastPath<sv::saveto, ddim, DType,
   }
 };
 
+/* dst = scalar (also NewTensor's initial value) on tensors of 32-bit elements */
+template <int dim, typename DType>
+struct FastPath<sv::saveto, dim, DType, expr::ScalarExp<DType> > {
+  inline static bool Run(Tensor<gpu, dim, DType> *dst, const expr::ScalarExp<DType> &e) {
+    if (sizeof(DType) != 4) return false;
+    uint32_t bits = 0;
+    memcpy(&bits, &e.scalar_, sizeof(DType) == 4 ? 4 : 0);
+    const Shape<2> s2 = dst->shape_.FlatTo2D();
+    MSHADOW_HIP_CALL(mshadow_hip_fill_32(dst->dptr_, dst->stride_, s2[0], s2[1], bits,
+                                         Stream<gpu>::GetStream(dst->stream_)));
+    return true;
+  }
+};
 /* dst = transpose(tensor, axes) and dst = swapaxis<a1, a2>(tensor) on dense tensors of 32-bit
    elements: the tiled permutation of the library */
 template <typename DType, int dim>

@@ -1,0 +1,63 @@
+// A caller that is compiled by the host compiler only (no device compiler) can still use
+// everything of Tensor<gpu> that sits behind the C ABI: allocation, copies, streams and the
+// assignments that are recognised as fixed-function operations. This file is compiled and
+// linked by the CPU test suite (it proves the claim at build time) and run by a GPU test.
+#include <mshadow/tensor.h>
+
+#include <cstdio>
+#include <vector>
+
+using namespace mshadow;
+using namespace mshadow::expr;
+
+int main() {
+  InitTensorEngine<gpu>(0);
+  Stream<gpu> *s = NewStream<gpu>(0);
+  const int n = 2, c = 3, h = 9, w = 12;
+  std::vector<float> host(n * c * h * w);
+  for (size_t i = 0; i < host.size(); ++i) host[i] = static_cast<float>((i * 37) % 101) - 50.0f;
+  Tensor<cpu, 4> hx(host.data(), Shape4(n, c, h, w));
+  Tensor<gpu, 4> x = NewTensor<gpu>(Shape4(n, c, h, w), 0.0f, false, s);
+  Tensor<gpu, 4> p = NewTensor<gpu>(Shape4(n, c, 4, 5), 0.0f, false, s);
+  Tensor<gpu, 4> g = NewTensor<gpu>(Shape4(n, c, h, w), 0.0f, false, s);
+  Tensor<gpu, 4> t = NewTensor<gpu>(Shape4(n, h, w, c), 0.0f, false, s);
+  Tensor<gpu, 2> m = NewTensor<gpu>(Shape2(n * c * h, w), 0.0f, false, s);
+  Tensor<gpu, 1> v = NewTensor<gpu>(Shape1(w), 0.0f, false, s);
+  Copy(x, hx, s);
+  p = pool<red::maximum>(x, 3, 3, 2, 2);
+  g = unpool<red::maximum>(x, p, p, 3, 3, 2, 2);
+  t = transpose(x, Shape4(0, 2, 3, 1));
+  Copy(m, x.FlatTo2D(), s);
+  v = sum_rows(m);
+  Softmax(m, m);
+  // expected values on the host with the CPU device of the same headers
+  TensorContainer<cpu, 4> cp(Shape4(n, c, 4, 5)), ct(Shape4(n, h, w, c));
+  TensorContainer<cpu, 1> cv(Shape1(w));
+  cp = pool<red::maximum>(hx, 3, 3, 2, 2);
+  ct = transpose(hx, Shape4(0, 2, 3, 1));
+  cv = sum_rows(hx.FlatTo2D());
+  TensorContainer<cpu, 4> gp(Shape4(n, c, 4, 5)), gt(Shape4(n, h, w, c));
+  TensorContainer<cpu, 1> gv(Shape1(w));
+  Copy(gp, p, s);
+  Copy(gt, t, s);
+  Copy(gv, v, s);
+  s->Wait();
+  int bad_pool = 0, bad_transpose = 0, bad_sum = 0;
+  /* the containers pad their rows: compare element by element, not the raw buffers */
+  Tensor<cpu, 2> cp2 = cp.FlatTo2D(), gp2 = gp.FlatTo2D(), ct2 = ct.FlatTo2D(), gt2 = gt.FlatTo2D();
+  for (index_t y = 0; y < cp2.size(0); ++y)
+    for (index_t x = 0; x < cp2.size(1); ++x) bad_pool += cp2[y][x] != gp2[y][x];
+  for (index_t y = 0; y < ct2.size(0); ++y)
+    for (index_t x = 0; x < ct2.size(1); ++x) bad_transpose += ct2[y][x] != gt2[y][x];
+  for (index_t i = 0; i < cv.size(0); ++i) bad_sum += cv[i] != gv[i];
+  const int bad = bad_pool + bad_transpose + bad_sum;
+  FreeSpace(&x); FreeSpace(&p); FreeSpace(&g); FreeSpace(&t); FreeSpace(&m); FreeSpace(&v);
+  DeleteStream(s);
+  ShutdownTensorEngine<gpu>();
+  if (bad) {
+    printf("values that differ: pool %d, transpose %d, sum_rows %d\n", bad_pool, bad_transpose, bad_sum);
+    return 1;
+  }
+  printf("OK\n");
+  return 0;
+}

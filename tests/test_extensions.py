@@ -282,3 +282,22 @@ def test_permute_entry_point(shape, axes, dtype):
     out = G.to_device(np.full(want.shape, -1, dtype))
     G.permute(out, G.to_device(a), axes)
     assert np.array_equal(out.download(), want), (shape, axes)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape,pad", [((7, 13), 0), ((7, 13), 3), ((64, 256), 0), ((5, 8), 4), ((1, 1), 0),
+                                       ((3, 4, 5, 8), 0)])
+def test_fill_entry_point(shape, pad):
+    """mshadow_hip_fill_32 sets exactly the elements of the view; the pitch gap keeps its contents"""
+    import mshadow_amd
+    G = mshadow_amd.load_cases()
+    G.set_device(0)
+    buf = G.buffer(shape, f32, pad=pad, fill=0)
+    G.fill(buf, -1.5)
+    assert np.array_equal(buf.download(), np.full(shape, -1.5, f32))
+    if pad:
+        raw = G.buffer((buf.rows, buf.stride), f32)
+        G.check(G.dll.mshadow_hip_memcpy2d_async(raw.ptr, raw.stride * 4, buf.ptr, buf.stride * 4,
+                                                 buf.stride * 4, buf.rows, 3, None))
+        G.stream_sync(None)
+        assert np.all(raw.download()[:, buf.cols:] == 0)

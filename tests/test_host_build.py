@@ -88,3 +88,27 @@ def test_header_api_on_cpu_matches_oracle(tmp_path, orc):
     out = _compile_and_run(tmp_path, "api_cpu_check.cc",
                            [os.path.join(oracle_dir, "liboracle.so"), "-Wl,-rpath," + oracle_dir])
     assert out.startswith("OK"), out
+
+
+def _build_host_only_caller(tmp_path):
+    exe = str(tmp_path / "hostonly")
+    cmd = ["g++", "-std=c++17", "-O2", "-fopenmp", "-ffp-contract=off", "-mf16c",
+           "-I", os.path.join(ROOT, "include"), "-I", os.path.join(ROOT, "mshadow_amd"),
+           "-o", exe, os.path.join(ROOT, "tests", "host", "gpu_api_hostonly.cc"),
+           "-L" + LIBDIR, "-lmshadow_hip", "-Wl,-rpath," + LIBDIR]
+    subprocess.run(cmd, check=True, capture_output=True, text=True)
+    return exe
+
+
+def test_host_compiler_only_caller_builds(tmp_path):
+    """Tensor<gpu> code whose assignments are all fixed-function operations needs no device
+    compiler: g++ alone compiles it and links it against the library (run by a GPU test)"""
+    _lib("libmshadow_hip.so")
+    assert os.path.exists(_build_host_only_caller(tmp_path))
+
+
+@pytest.mark.gpu
+def test_host_compiler_only_caller_runs(tmp_path):
+    out = subprocess.run([_build_host_only_caller(tmp_path)], capture_output=True, text=True,
+                         timeout=300)
+    assert out.returncode == 0 and out.stdout.startswith("OK"), out.stdout[-2000:] + out.stderr[-2000:]
