@@ -80,13 +80,13 @@ OPS = [k for k in algorithmic_bytes() if k not in EXTRA_OPS]
 
 # HBM bytes per launch of each operation's kernel, measured with rocprofv3 --pmc FETCH_SIZE and
 # --pmc WRITE_SIZE (two runs of `bench.py --only <all ops>,calib_copy`), each counter scaled by
-# what it reads for the calibration copy of known size (FETCH_SIZE x 1.9978, WRITE_SIZE x 0.9993);
+# what it reads for the calibration copy of known size (FETCH_SIZE x 1.9981, WRITE_SIZE x 0.9993);
 # the counter table is kept under profiles/. bench.py cannot run the profiler on itself, so
 # `roofline.traffic` quotes this table.
 MEASURED_HBM_BYTES = {
-    "map_fused": 335404089, "sumall_except_dim1": 205361096, "sum_rows": 271005681,
-    "softmax": 2095910480, "softmax_grad": 2095875769, "pool_max": 517805036,
-    "unpool_max": 1064903488, "im2col_f16": 513830021, "col2im_f16": 543967579,
+    "map_fused": 335456759, "sumall_except_dim1": 205383085, "sum_rows": 271459999,
+    "softmax": 2096088147, "softmax_grad": 2096037454, "pool_max": 517871947,
+    "unpool_max": 1068772362, "im2col_f16": 513898202, "col2im_f16": 544026496,
 }
 
 
