@@ -317,11 +317,13 @@ int mshadow_case_extensions_f32(int op, float *out, const float *a, const float 
 #define V2(p, d0, d1) G2(p, d0, d1, d1, st.get())
 #define V3(p, d0, d1, d2) G3(p, d0, d1, d2, d2, st.get())
 #define V4(p, d0, d1, d2, d3) G4(p, d0, d1, d2, d3, d3, st.get())
+#define V4S(p, d0, d1, d2, d3, pitch) G4(p, d0, d1, d2, d3, pitch, st.get())
 #include "./extension_cases.inc"
 #undef TENSOR
 #undef V1
 #undef V2
 #undef V3
+#undef V4S
 #undef V4
   CASE_END
 }

@@ -276,6 +276,7 @@ void ref_extensions_f32(int op, float *out, const float *a, const float *b, cons
 #define V2(p, d0, d1) T2(p, d0, d1, d1)
 #define V3(p, d0, d1, d2) T3(p, d0, d1, d2, d2)
 #define V4(p, d0, d1, d2, d3) T4(p, d0, d1, d2, d3, d3)
+#define V4S(p, d0, d1, d2, d3, pitch) T4(p, d0, d1, d2, d3, pitch)
 #define MSHADOW_CASES_REFERENCE_HEADERS
 #include "../mshadow_amd/cases/extension_cases.inc"
 #undef MSHADOW_CASES_REFERENCE_HEADERS
@@ -283,6 +284,7 @@ void ref_extensions_f32(int op, float *out, const float *a, const float *b, cons
 #undef V1
 #undef V2
 #undef V3
+#undef V4S
 #undef V4
 }
 

@@ -22,11 +22,14 @@ extern "C" int host_extensions_f32(int op, float *out, const float *a, const flo
 #define V2(p, d0, d1) View(p, Shape2(d0, d1))
 #define V3(p, d0, d1, d2) View(p, Shape3(d0, d1, d2))
 #define V4(p, d0, d1, d2, d3) View(p, Shape4(d0, d1, d2, d3))
+#define V4S(p, d0, d1, d2, d3, pitch) \
+  Tensor<cpu, 4, float>(const_cast<float *>(p), Shape4(d0, d1, d2, d3), pitch, NULL)
 #include "../../mshadow_amd/cases/extension_cases.inc"
 #undef TENSOR
 #undef V1
 #undef V2
 #undef V3
+#undef V4S
 #undef V4
   } catch (const std::exception &e) {
     fprintf(stderr, "%s\n", e.what());

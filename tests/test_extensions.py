@@ -72,6 +72,7 @@ class Case(object):
         self.op, self.shape, self.a = op, shape, a
         self.b = self.c = None
         self.p = (0, 0, 0)
+        self.pitch_pad = 0   # ops 28..31: rows of `a` and of the result are this much apart more
         rows = n * ch * h
         if op == 0:
             self.p = (3, 0, 0)
@@ -180,6 +181,23 @@ class Case(object):
             self.p = (2, 2 + sum(shape), 3)
             count = -(-(self.p[1] - self.p[0]) // self.p[2])
             self.want = np.repeat(f32(self.p[0]) + np.arange(count).astype(f32) * f32(self.p[2]), 2)
+        elif op >= 28:
+            # a pitch that keeps 16-byte alignment (pack route where the row length allows it)
+            # or one that breaks it (element-wise route)
+            self.pitch_pad = 4 if sum(shape) % 2 else 1
+            if op == 28:
+                self.p = (0, 0, self.pitch_pad)
+                self.b = rng.standard_normal(ch).astype(f32)
+                self.want = a + self.b.reshape(1, ch, 1, 1)
+            elif op == 29:
+                self.p = (3, 0, self.pitch_pad)
+                self.want = _chpool(a, 3, 1, 1, "sum")
+            elif op == 30:
+                self.p = (1, ch - 1, self.pitch_pad)
+                self.want = a[:, 1:ch - 1]
+            else:
+                self.p = (0, 0, self.pitch_pad)
+                self.want = a.transpose(0, 2, 1, 3)
         else:
             k = 11
             perm = [2031, 3102, 1230][sum(shape) % 3]
@@ -193,7 +211,26 @@ class Case(object):
         self.want = np.ascontiguousarray(self.want, dtype=f32)
 
 
-N_OPS = 28
+N_OPS = 32
+
+
+def _pitched(arr, pad):
+    """the array laid out with `pad` unused elements behind every row (NaN there)"""
+    rows = arr.reshape(-1, arr.shape[-1])
+    out = np.full((rows.shape[0], rows.shape[1] + pad), np.nan, f32)
+    out[:, :rows.shape[1]] = rows
+    return out
+
+
+def _run_on_host(call, case):
+    """runs `call(out, a)` on host arrays, through pitched copies for the pitched ops"""
+    if not case.pitch_pad:
+        out = np.full(case.want.shape, np.nan, f32)
+        call(out, case.a)
+        return out
+    out = _pitched(np.full(case.want.shape, np.nan, f32), case.pitch_pad)
+    call(out, _pitched(case.a, case.pitch_pad))
+    return np.ascontiguousarray(out[:, :case.want.shape[-1]]).reshape(case.want.shape)
 
 
 @pytest.fixture(scope="module")
@@ -219,10 +256,11 @@ def _ptr(x):
 @pytest.mark.parametrize("op", range(N_OPS))
 def test_cpu_device_matches_numpy(host_lib, shape, op):
     case = Case(op, shape)
-    out = np.full(case.want.shape, np.nan, f32)
-    rc = host_lib.host_extensions_f32(op, _ptr(out), _ptr(case.a), _ptr(case.b), _ptr(case.c),
-                                      *shape, *case.p)
-    assert rc == 0
+
+    def call(out, a):
+        assert host_lib.host_extensions_f32(op, _ptr(out), _ptr(a), _ptr(case.b), _ptr(case.c),
+                                            *shape, *case.p) == 0
+    out = _run_on_host(call, case)
     assert np.array_equal(out.view(np.uint32), case.want.view(np.uint32)), (op, shape)
 
 
@@ -231,8 +269,7 @@ def test_cpu_device_matches_numpy(host_lib, shape, op):
 @pytest.mark.parametrize("op", [o for o in range(N_OPS) if o != 15])
 def test_reference_build_matches_numpy(ref, shape, op):
     case = Case(op, shape)
-    out = np.full(case.want.shape, np.nan, f32)
-    ref.extensions(op, out, case.a, case.b, case.c, *shape, *case.p)
+    out = _run_on_host(lambda o, a: ref.extensions(op, o, a, case.b, case.c, *shape, *case.p), case)
     assert np.array_equal(out.view(np.uint32), case.want.view(np.uint32)), (op, shape)
 
 
@@ -244,9 +281,10 @@ def test_gpu_matches_numpy(shape, op):
     G = mshadow_amd.load_cases()
     G.set_device(0)
     case = Case(op, shape)
-    out = G.to_device(np.full(case.want.shape, np.nan, f32))
+    out = G.to_device(np.full(case.want.shape, np.nan, f32), pad=case.pitch_pad)
     dev = lambda x: G.to_device(x) if x is not None else None
-    G.case_extensions(op, out, dev(case.a), dev(case.b), dev(case.c), *shape, *case.p)
+    G.case_extensions(op, out, G.to_device(case.a, pad=case.pitch_pad), dev(case.b), dev(case.c),
+                      *shape, *case.p)
     got = out.download()
     assert np.array_equal(got.view(np.uint32), case.want.view(np.uint32)), (op, shape)
 
