@@ -72,7 +72,6 @@ struct Plan<ChannelPoolingExp<Reducer, SrcExp, DType, srcdim>, DType> {
     const index_t n = channel_.Div(plane);
     const index_t c = plane - n * channel_.div;
     const index_t first = c * stride_ < pad_ ? 0 : c * stride_ - pad_;
-    /* modular arithmetic as in the reference: the sum is in range whenever it matters */
     index_t last = c * stride_ - pad_ + nsize_;
     if (last > channel_.div) last = channel_.div;
     if (last > src_channel_) last = src_channel_;
