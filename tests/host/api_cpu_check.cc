@@ -6,6 +6,7 @@
 // Prints "OK <n> checks"; exit status 0 on success.
 #define DMLC_LOG_FATAL_THROW 1
 #include <mshadow/tensor.h>
+#include <mshadow/io.h>
 
 #include <cstdio>
 #include <cstring>
@@ -298,6 +299,44 @@ int main() {
     IndexFill(Dd, So, Sr);
     orc_index_fill_f32(d2.data(), W, srt.data(), 1, N, src.data(), W, W);
     EXPECT(SameBits(d1.data(), d2.data(), d1.size()));
+  }
+  // ---- SaveBinary / LoadBinary: the record is the shape followed by the dense rows
+  {
+    struct MemStream : public utils::IStream {
+      std::vector<char> bytes;
+      size_t pos = 0;
+      size_t Read(void *ptr, size_t size) override {
+        const size_t n = std::min(size, bytes.size() - pos);
+        memcpy(ptr, bytes.data() + pos, n);
+        pos += n;
+        return n;
+      }
+      void Write(const void *ptr, size_t size) override {
+        const char *c = static_cast<const char *>(ptr);
+        bytes.insert(bytes.end(), c, c + size);
+      }
+    } ms;
+    TensorContainer<cpu, 3> t(Shape3(2, 3, 5));   // padded rows: the pitch is not stored
+    for (index_t i = 0; i < 2; ++i) for (index_t j = 0; j < 3; ++j) for (index_t k = 0; k < 5; ++k)
+      t[i][j][k] = static_cast<float>(100 * i + 10 * j + k);
+    SaveBinary(ms, t);
+    EXPECT(ms.bytes.size() == 3 * sizeof(index_t) + 30 * sizeof(float));
+    index_t stored[3];
+    memcpy(stored, ms.bytes.data(), sizeof(stored));
+    EXPECT(stored[0] == 2 && stored[1] == 3 && stored[2] == 5);
+    float first_row[5];
+    memcpy(first_row, ms.bytes.data() + sizeof(stored) + 5 * sizeof(float), sizeof(first_row));
+    EXPECT(first_row[0] == 10.0f && first_row[4] == 14.0f);
+    Tensor<cpu, 3> back;
+    LoadBinary(ms, &back, false);
+    bool same = back.shape_ == t.shape_;
+    for (index_t i = 0; i < 2; ++i) for (index_t j = 0; j < 3; ++j) for (index_t k = 0; k < 5; ++k)
+      same = same && back[i][j][k] == t[i][j][k];
+    EXPECT(same);
+    FreeSpace(&back);
+    ms.pos = 0;
+    TensorContainer<cpu, 3> wrong(Shape3(2, 3, 4));
+    EXPECT(Throws([&] { LoadBinary(ms, &wrong, true); }));
   }
   // ---- SortByKey / VectorizedSort on the CPU device against the oracle
   {

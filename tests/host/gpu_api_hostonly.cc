@@ -3,8 +3,10 @@
 // assignments that are recognised as fixed-function operations. This file is compiled and
 // linked by the CPU test suite (it proves the claim at build time) and run by a GPU test.
 #include <mshadow/tensor.h>
+#include <mshadow/io.h>
 
 #include <cstdio>
+#include <cstring>
 #include <vector>
 
 using namespace mshadow;
@@ -50,8 +52,35 @@ int main() {
   for (index_t y = 0; y < ct2.size(0); ++y)
     for (index_t x = 0; x < ct2.size(1); ++x) bad_transpose += ct2[y][x] != gt2[y][x];
   for (index_t i = 0; i < cv.size(0); ++i) bad_sum += cv[i] != gv[i];
-  const int bad = bad_pool + bad_transpose + bad_sum;
+  int bad = 0;
+  /* a device tensor written to a byte stream and read back into a new device tensor */
+  struct MemStream {
+    std::vector<char> bytes;
+    size_t pos = 0;
+    size_t Read(void *ptr, size_t size) {
+      const size_t k = size < bytes.size() - pos ? size : bytes.size() - pos;
+      memcpy(ptr, bytes.data() + pos, k);
+      pos += k;
+      return k;
+    }
+    void Write(const void *ptr, size_t size) {
+      const char *c = static_cast<const char *>(ptr);
+      bytes.insert(bytes.end(), c, c + size);
+    }
+  } ms;
+  SaveBinary(ms, t);
+  Tensor<gpu, 4> t2;
+  t2.set_stream(s);
+  LoadBinary(ms, &t2, false);
+  TensorContainer<cpu, 4> gt_again(Shape4(n, h, w, c));
+  Copy(gt_again, t2, s);
+  s->Wait();
+  Tensor<cpu, 2> again2 = gt_again.FlatTo2D();
+  for (index_t y = 0; y < ct2.size(0); ++y)
+    for (index_t x2 = 0; x2 < ct2.size(1); ++x2) bad_transpose += ct2[y][x2] != again2[y][x2];
+  FreeSpace(&t2);
   FreeSpace(&x); FreeSpace(&p); FreeSpace(&g); FreeSpace(&t); FreeSpace(&m); FreeSpace(&v);
+  bad = bad_pool + bad_transpose + bad_sum;
   DeleteStream(s);
   ShutdownTensorEngine<gpu>();
   if (bad) {
