@@ -187,6 +187,21 @@ int mshadow_hip_index_fill_f32(float *dst, int dstride, int k_rows, const void *
                                int index_is_int, int n_index, const float *src, int sstride,
                                int cols, void *stream);
 
+/* Random<gpu>::GetRandInt / SampleUniform / SampleGaussian (mshadow/random.h:372-568, cuRAND
+   there): Philox-4x32-10 blocks of four words; element e of a call uses block `counter + e / 4`
+   of the stream (seed, subsequence), word e % 4. The generator has no state in memory: the
+   caller advances `counter` by (elements + 3) / 4 per call. Uniform values lie strictly inside
+   (a, b) up to rounding; normal values are mu + z * sigma with z from Box-Muller. The values
+   are not cuRAND's. dstride in elements. */
+int mshadow_hip_random_u32(uint32_t *dst, size_t n, uint64_t seed, uint64_t subsequence,
+                           uint64_t counter, void *stream);
+int mshadow_hip_random_uniform_f32(float *dst, int dstride, int rows, int cols, uint64_t seed,
+                                   uint64_t subsequence, uint64_t counter, float a, float b,
+                                   void *stream);
+int mshadow_hip_random_normal_f32(float *dst, int dstride, int rows, int cols, uint64_t seed,
+                                  uint64_t subsequence, uint64_t counter, float mu, float sigma,
+                                  void *stream);
+
 /* dst = transpose(src, axes) / dst = swapaxis<a1, a2>(src) on dense tensors of 32-bit
    elements: dst axis i is src axis axes[i]; `shape` is the source's, ndim <= 6
    (mshadow/extension/transpose.h:24-88, swapaxis.h:20-106, evaluated there element by element

@@ -73,6 +73,10 @@ int mshadow_case_rows_by_index_f32(int op, float *dst, int dstride, int k_rows, 
 int mshadow_case_shaping_f32(int op, float *out, const float *a, const float *v, int n, int c,
                              int h, int w, void *stream);
 
+/* Random<gpu>(seed): op 0 SampleUniform(p0, p1) into the two halves of out in turn; 1
+   SampleGaussian(p0, p1); 2 out = uniform(Shape1(n)) * 2; 3 GetRandInt (unsigned words) */
+int mshadow_case_random_f32(int op, int seed, float *out, int n, float p0, float p1, void *stream);
+
 /* op 0: SortByKey(keys, values, is_ascend); 1: VectorizedSort(keys, values as segment numbers).
    key_kind 0: float keys with int values, 1: int keys with float values (int segments for op 1) */
 int mshadow_case_sort_by_key_32(int op, void *keys, int key_kind, void *values, int n,

@@ -1,7 +1,7 @@
 """Build recipe for the native parts (gfx950 only).
 
   libmshadow_hip.so    the C ABI device layer (csrc/runtime.hip, csrc/ops.hip, csrc/sort.hip,
-                       csrc/permute.hip)
+                       csrc/permute.hip, csrc/random.hip)
   libmshadow_cases.so  caller-style programs written against <mshadow/tensor.h>
                        (cases/cases.hip), exported as C functions for tests and bench
 
@@ -52,7 +52,7 @@ def _run(cmd, verbose):
 
 def build_hip_library(verbose=True):
     os.makedirs(LIB_DIR, exist_ok=True)
-    srcs = [os.path.join(HERE, "csrc", f) for f in ("runtime.hip", "ops.hip", "sort.hip", "permute.hip")]
+    srcs = [os.path.join(HERE, "csrc", f) for f in ("runtime.hip", "ops.hip", "sort.hip", "permute.hip", "random.hip")]
     _run([hipcc()] + COMMON + ["-o", HIP_SO] + srcs, verbose)
     return HIP_SO
 

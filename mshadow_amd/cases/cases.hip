@@ -6,6 +6,7 @@
  */
 #define DMLC_LOG_FATAL_THROW 1
 #include <mshadow/tensor.h>
+#include <mshadow/random.h>
 #include <mshadow_hip_cases.h>
 
 #include <string>
@@ -279,6 +280,30 @@ int mshadow_case_shaping_f32(int op, float *out, const float *a, const float *v,
 #undef IN4
 #undef IN2
 #undef VEC
+  CASE_END
+}
+
+/* Random<gpu>: op 0 SampleUniform(p0, p1) into the first half and then into the second half of
+   out; 1 SampleGaussian(p0, p1); 2 out = rnd.uniform(Shape1(n)) * 2; 3 GetRandInt (out holds
+   unsigned words) */
+int mshadow_case_random_f32(int op, int seed, float *out, int n, float p0, float p1, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Random<gpu, float> rnd(seed);
+  rnd.set_stream(st.get());
+  Tensor<gpu, 1, float> dst = G1(out, n, st.get());
+  if (op == 0) {
+    Tensor<gpu, 1, float> lo = dst.Slice(0, n / 2), hi = dst.Slice(n / 2, n);
+    rnd.SampleUniform(&lo, p0, p1);
+    rnd.SampleUniform(&hi, p0, p1);
+  } else if (op == 1) {
+    rnd.SampleGaussian(&dst, p0, p1);
+  } else if (op == 2) {
+    dst = rnd.uniform(Shape1(n)) * 2.0f;
+  } else {
+    rnd.GetRandInt(G1(reinterpret_cast<unsigned *>(out), n, st.get()));
+  }
+  st.get()->Wait();   // rnd's buffer is released when it goes out of scope
   CASE_END
 }
 

@@ -1,0 +1,141 @@
+/*
+ * Random numbers on the device: Philox-4x32-10, a counter-based generator (Salmon, Moraes,
+ * Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3", SC'11). Element e of a call
+ * is a pure function of (seed, subsequence, counter + e / 4, e % 4), so a launch needs no
+ * generator state in memory and any launch shape gives the same values; the caller (the
+ * Random<gpu> object) advances `counter` by the blocks a call consumed.
+ *
+ * This is the role cuRAND's default generator plays for Random<gpu> in the reference
+ * (mshadow/random.h:372-568: curandGenerate / curandGenerateUniform /
+ * curandGenerateNormal). The values are those of Philox, not of cuRAND's XORWOW: no two
+ * generator families agree, and the reference's CPU path (std::mt19937) does not agree
+ * with its own GPU path either.
+ *   uniform  u = ((x >> 8) + 0.5) * 2^-24, strictly inside (0, 1), then u * (b - a) + a
+ *   normal   Box-Muller on two uniforms: sqrt(-2 ln u1) * (cos, sin)(2 pi u2), then
+ *            mu + z * sigma
+ */
+#include <mshadow/core/fastdiv.h>
+
+#include "./abi_common.h"
+
+using mshadow::FastDivU32;
+using mshadow_abi::AfterLaunch;
+using mshadow_abi::AsStream;
+
+namespace {
+
+const int kRandomBlock = 256;
+
+struct Philox4 {
+  uint32_t w[4];
+};
+
+/*! \brief one block of four 32-bit words */
+__device__ __forceinline__ Philox4 Philox4x32_10(uint64_t seed, uint64_t subsequence,
+                                                 uint64_t counter) {
+  uint32_t c0 = static_cast<uint32_t>(counter), c1 = static_cast<uint32_t>(counter >> 32);
+  uint32_t c2 = static_cast<uint32_t>(subsequence), c3 = static_cast<uint32_t>(subsequence >> 32);
+  uint32_t k0 = static_cast<uint32_t>(seed), k1 = static_cast<uint32_t>(seed >> 32);
+#pragma unroll
+  for (int round = 0; round < 10; ++round) {
+    const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+    const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+    c0 = hi1 ^ c1 ^ k0;
+    c1 = lo1;
+    c2 = hi0 ^ c3 ^ k1;
+    c3 = lo0;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  Philox4 out = {{c0, c1, c2, c3}};
+  return out;
+}
+
+__device__ __forceinline__ float UnitOpen(uint32_t x) {
+  return (static_cast<float>(x >> 8) + 0.5f) * 5.9604644775390625e-08f;  // 2^-24
+}
+
+enum { kWords = 0, kUniform = 1, kNormal = 2 };
+
+/*! \brief element e of the dense (rows, cols) view lands at row e / cols, column e % cols of
+ *  a destination whose rows are `stride` elements apart; one thread per four elements */
+template <int KIND>
+__global__ void __launch_bounds__(kRandomBlock)
+    RandomKernel(uint32_t *dst, uint32_t stride, uint32_t total, uint32_t cols, FastDivU32 div_cols,
+                 uint64_t seed, uint64_t subsequence, uint64_t counter, float p0, float p1) {
+  const uint32_t blocks = (total + 3u) / 4u;
+  const uint32_t step = gridDim.x * kRandomBlock;
+  for (uint32_t b = blockIdx.x * kRandomBlock + threadIdx.x; b < blocks; b += step) {
+    const Philox4 r = Philox4x32_10(seed, subsequence, counter + b);
+    uint32_t out[4];
+    if (KIND == kWords) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) out[k] = r.w[k];
+    } else if (KIND == kUniform) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) out[k] = __float_as_uint(UnitOpen(r.w[k]) * (p1 - p0) + p0);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; k += 2) {
+        const float radius = __builtin_sqrtf(-2.0f * __logf(UnitOpen(r.w[k])));
+        float sn, cs;
+        __sincosf(6.283185307179586f * UnitOpen(r.w[k + 1]), &sn, &cs);
+        out[k] = __float_as_uint(p0 + radius * cs * p1);
+        out[k + 1] = __float_as_uint(p0 + radius * sn * p1);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t e = b * 4u + k;
+      if (e < total) {
+        const uint32_t y = div_cols.Div(e);
+        dst[static_cast<size_t>(y) * stride + (e - y * cols)] = out[k];
+      }
+    }
+  }
+}
+
+template <int KIND>
+int LaunchRandom(void *dst, int dstride, int rows, int cols, uint64_t seed, uint64_t subsequence,
+                 uint64_t counter, float p0, float p1, void *stream, const char *what) {
+  if (rows < 0 || cols < 0) return mshadow_abi::Fail(MSHADOW_HIP_ERR_ARGUMENT, std::string(what) + ": negative shape");
+  if (rows == 0 || cols == 0) return MSHADOW_HIP_OK;
+  if (dst == NULL) return mshadow_abi::Fail(MSHADOW_HIP_ERR_ARGUMENT, std::string(what) + ": NULL tensor");
+  if (dstride < cols) return mshadow_abi::Fail(MSHADOW_HIP_ERR_ARGUMENT, std::string(what) + ": pitch smaller than the row");
+  const uint64_t total = static_cast<uint64_t>(rows) * cols;
+  if (total >= (1ull << 31)) return mshadow_abi::Fail(MSHADOW_HIP_ERR_ARGUMENT, std::string(what) + ": too many elements");
+  uint64_t grid = ((total + 3) / 4 + kRandomBlock - 1) / kRandomBlock;
+  if (grid > 16384) grid = 16384;
+  hipLaunchKernelGGL(RandomKernel<KIND>, dim3(static_cast<unsigned>(grid)), dim3(kRandomBlock), 0,
+                     AsStream(stream), static_cast<uint32_t *>(dst), static_cast<uint32_t>(dstride),
+                     static_cast<uint32_t>(total), static_cast<uint32_t>(cols), FastDivU32(cols), seed,
+                     subsequence, counter, p0, p1);
+  return AfterLaunch(what);
+}
+
+}  // namespace
+
+extern "C" {
+
+int mshadow_hip_random_u32(uint32_t *dst, size_t n, uint64_t seed, uint64_t subsequence,
+                           uint64_t counter, void *stream) {
+  ABI_REQUIRE(n < (1ull << 31), "too many elements");
+  return LaunchRandom<kWords>(dst, static_cast<int>(n), 1, static_cast<int>(n), seed, subsequence,
+                              counter, 0.0f, 0.0f, stream, "random_u32");
+}
+
+int mshadow_hip_random_uniform_f32(float *dst, int dstride, int rows, int cols, uint64_t seed,
+                                   uint64_t subsequence, uint64_t counter, float a, float b,
+                                   void *stream) {
+  return LaunchRandom<kUniform>(dst, dstride, rows, cols, seed, subsequence, counter, a, b, stream,
+                                "random_uniform");
+}
+
+int mshadow_hip_random_normal_f32(float *dst, int dstride, int rows, int cols, uint64_t seed,
+                                  uint64_t subsequence, uint64_t counter, float mu, float sigma,
+                                  void *stream) {
+  return LaunchRandom<kNormal>(dst, dstride, rows, cols, seed, subsequence, counter, mu, sigma,
+                               stream, "random_normal");
+}
+
+}  // extern "C"

@@ -9,6 +9,7 @@
  * baseline. Signatures mirror oracle.h with the prefix ref_.
  */
 #include <mshadow/tensor.h>
+#include <mshadow/random.h>
 
 #include <omp.h>
 #include <stdint.h>
@@ -267,6 +268,10 @@ void ref_shaping_f32(int op, float *out, const float *a, const float *v, int n, 
 #undef IN4
 #undef IN2
 #undef VEC
+}
+
+void ref_random_f32(int op, int seed, float *out, int n, float p0, float p1) {
+#include "../mshadow_amd/cases/random_cases.inc"
 }
 
 void ref_extensions_f32(int op, float *out, const float *a, const float *b, const float *c, int n,

@@ -88,6 +88,7 @@ class Checker:
         if self.prefix == "ref":
             self._fn("shaping_f32", [_i, _p, _p, _p, _i, _i, _i, _i])
             self._fn("extensions_f32", [_i, _p, _p, _p, _p] + [_i] * 7)
+            self._fn("random_f32", [_i, _i, _p, _i, _f, _f])
         self._fn("pool_f32", [_p, _i, _p, _i] + [_i] * 10)
         self._fn("unpool_f32", [_p, _i, _p, _i, _p, _i, _p, _i] + [_i] * 10)
         for t in ("f16", "f32"):
@@ -211,6 +212,11 @@ class Checker:
     def shaping(self, op, out, a, v, n, c, h, w):
         """reference build only: the index-remapping extension expressions"""
         self._shaping_f32(op, ptr(out), ptr(a), ptr(v), n, c, h, w)
+        return out
+
+    def random(self, op, seed, out, p0=0.0, p1=1.0):
+        """reference build only: Random<cpu> samplers into a float vector"""
+        self._random_f32(op, seed, ptr(out), out.shape[0], p0, p1)
         return out
 
     def extensions(self, op, out, a, b, c, n, ch, h, w, p0=0, p1=0, p2=0):

@@ -2,6 +2,7 @@
 // Tensor<cpu> of this backend's headers (plain g++, no GPU): built as a small shared
 // library by tests/test_extensions.py and compared with numpy there.
 #include <mshadow/tensor.h>
+#include <mshadow/random.h>
 
 using namespace mshadow;
 using namespace mshadow::expr;
@@ -31,6 +32,16 @@ extern "C" int host_extensions_f32(int op, float *out, const float *a, const flo
 #undef V3
 #undef V4S
 #undef V4
+  } catch (const std::exception &e) {
+    fprintf(stderr, "%s\n", e.what());
+    return 1;
+  }
+  return 0;
+}
+
+extern "C" int host_random_f32(int op, int seed, float *out, int n, float p0, float p1) {
+  try {
+#include "../../mshadow_amd/cases/random_cases.inc"
   } catch (const std::exception &e) {
     fprintf(stderr, "%s\n", e.what());
     return 1;

@@ -1,0 +1,184 @@
+"""Random<cpu> and Random<gpu>.
+
+CPU: the samplers are the standard library's distributions on std::mt19937, so this backend's
+headers and the reference's, built in the same container, must draw identical values from a
+seed (checked bit for bit where the reference build is present) - plus range / moment checks
+that do not need the reference.
+
+GPU: the generator is Philox-4x32-10. Its three published known-answer vectors (Random123,
+kat_vectors: all-zero, all-one and pi-digit inputs) pin the Python model below, and the model
+pins the device words for arbitrary (seed, subsequence, counter). The uniform transform is
+checked exactly, the normal transform against the same formula in double precision (device
+log / sin / cos: relative 1e-5) and by its moments. There is no parity with the reference's
+GPU path to check: it asks cuRAND for the numbers (parity unpinned by nature)."""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from checkers import have_ref
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+f32 = np.float32
+M32 = 0xFFFFFFFF
+
+
+def philox4x32_10(seed, subsequence, counter):
+    c = [counter & M32, counter >> 32, subsequence & M32, subsequence >> 32]
+    k = [seed & M32, seed >> 32]
+    for _ in range(10):
+        p0, p1 = 0xD2511F53 * c[0], 0xCD9E8D57 * c[2]
+        c = [(p1 >> 32) ^ c[1] ^ k[0], p1 & M32, (p0 >> 32) ^ c[3] ^ k[1], p0 & M32]
+        k = [(k[0] + 0x9E3779B9) & M32, (k[1] + 0xBB67AE85) & M32]
+    return c
+
+
+KATS = [
+    (0, 0, 0, [0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8]),
+    (2**64 - 1, 2**64 - 1, 2**64 - 1, [0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd]),
+    (0x299f31d0a4093822, 0x0370734413198a2e, 0x85a308d3243f6a88,
+     [0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1]),
+]
+
+
+@pytest.mark.parametrize("seed,subsequence,counter,want", KATS)
+def test_philox_model_known_answers(seed, subsequence, counter, want):
+    assert philox4x32_10(seed, subsequence, counter) == want
+
+
+def model_words(seed, subsequence, counter, n):
+    out = []
+    for b in range((n + 3) // 4):
+        out += philox4x32_10(seed, subsequence, (counter + b) % 2**64)
+    return np.array(out[:n], dtype=np.uint32)
+
+
+def unit_open(words):
+    return ((words >> 8).astype(f32) + f32(0.5)) * f32(2.0 ** -24)
+
+
+# ---------------------------------------------------------------- CPU
+@pytest.fixture(scope="module")
+def host_lib(tmp_path_factory):
+    so = str(tmp_path_factory.mktemp("hostrandom") / "libhostcases.so")
+    cmd = ["g++", "-std=c++17", "-O2", "-fopenmp", "-ffp-contract=off", "-mf16c", "-fPIC", "-shared",
+           "-DDMLC_LOG_FATAL_THROW=1", "-I", os.path.join(ROOT, "include"),
+           "-I", os.path.join(ROOT, "mshadow_amd"), "-o", so,
+           os.path.join(ROOT, "tests", "host", "ext_cpu_cases.cc")]
+    subprocess.run(cmd, check=True, capture_output=True, text=True)
+    lib = ctypes.CDLL(so)
+    lib.host_random_f32.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_int,
+                                    ctypes.c_float, ctypes.c_float]
+    return lib
+
+
+def _host(lib, op, seed, n, p0, p1):
+    out = np.full(n, np.nan, f32)
+    assert lib.host_random_f32(op, seed, out.ctypes.data_as(ctypes.c_void_p), n, p0, p1) == 0
+    return out
+
+
+CPU_CASES = [(0, -2.0, 3.0), (1, 1.0, 0.5), (1, 1.0, 0.0), (2, 2.0, 1.5), (3, 0.7, 0.0), (4, 3.5, 0.0),
+             (5, 4.0, 0.3), (6, 2.5, 0.4), (6, 2.5, 0.0), (7, 0.0, 0.0), (8, 0.0, 1.0), (9, 0.0, 0.0)]
+
+
+@pytest.mark.skipif(not have_ref(), reason="reference build absent")
+@pytest.mark.parametrize("op,p0,p1", CPU_CASES)
+@pytest.mark.parametrize("seed", [0, 17, -5])
+def test_cpu_random_draws_what_the_reference_draws(host_lib, ref, op, p0, p1, seed):
+    n = 4000
+    mine = _host(host_lib, op, seed, n, p0, p1)
+    theirs = ref.random(op, seed, np.full(n, np.nan, f32), p0, p1)
+    assert np.array_equal(mine.view(np.uint32), theirs.view(np.uint32))
+
+
+def test_cpu_random_ranges_and_moments(host_lib):
+    n = 200000
+    u = _host(host_lib, 0, 3, n, -2.0, 3.0)
+    assert u.min() >= -2.0 and u.max() < 3.0 and abs(u.mean() - 0.5) < 0.02
+    g = _host(host_lib, 1, 3, n, 1.0, 0.5)
+    assert abs(g.mean() - 1.0) < 0.01 and abs(g.std() - 0.5) < 0.01
+    assert np.all(_host(host_lib, 1, 3, 100, 1.25, 0.0) == f32(1.25))        # sigma <= 0: the mean
+    p = _host(host_lib, 4, 3, n, 3.5, 0.0)
+    assert np.all(p == np.round(p)) and abs(p.mean() - 3.5) < 0.03
+    assert not np.array_equal(_host(host_lib, 0, 3, 100, 0.0, 1.0), _host(host_lib, 0, 4, 100, 0.0, 1.0))
+    assert np.array_equal(_host(host_lib, 0, 3, 100, 0.0, 1.0), _host(host_lib, 0, 3, 100, 0.0, 1.0))
+
+
+# ---------------------------------------------------------------- GPU
+@pytest.fixture(scope="module")
+def G():
+    import mshadow_amd
+    g = mshadow_amd.load_cases()
+    g.set_device(0)
+    return g
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed,subsequence,counter,want", KATS)
+def test_gpu_philox_known_answers(G, seed, subsequence, counter, want):
+    out = G.buffer((4,), np.uint32)
+    G.random_u32(out, seed, subsequence, counter)
+    assert list(out.download()) == want
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n", [1, 3, 4, 5, 1023, 70001])
+def test_gpu_words_follow_the_model(G, n):
+    seed, sub, ctr = 0x1234567890ABCDEF, 7, 2**64 - 3      # the counter wraps inside the call
+    out = G.buffer((n,), np.uint32)
+    G.random_u32(out, seed, sub, ctr)
+    assert np.array_equal(out.download(), model_words(seed, sub, ctr, n))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape,pad", [((1000,), 0), ((37, 29), 0), ((37, 29), 3), ((4, 5, 6), 2)])
+def test_gpu_uniform_is_the_stated_transform(G, shape, pad):
+    seed, ctr, a, b = 99, 1000, f32(-1.5), f32(2.25)
+    n = int(np.prod(shape))
+    out = G.buffer(shape, f32, pad=pad, fill=0)
+    G.random_uniform(out, seed, 0, ctr, float(a), float(b))
+    want = (unit_open(model_words(seed, 0, ctr, n)) * (b - a) + a).astype(f32)
+    got = out.download().ravel()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert got.min() > a and got.max() < b
+
+
+@pytest.mark.gpu
+def test_gpu_normal_matches_box_muller_and_its_moments(G):
+    seed, ctr, n = 5, 0, 1 << 20
+    out = G.buffer((n,), f32)
+    G.random_normal(out, seed, 0, ctr, 1.0, 2.0)
+    got = out.download().astype(np.float64)
+    u = unit_open(model_words(seed, 0, ctr, n)).astype(np.float64)
+    r = np.sqrt(-2.0 * np.log(u[0::2]))
+    z = np.empty(n)
+    z[0::2] = r * np.cos(2 * np.pi * u[1::2])
+    z[1::2] = r * np.sin(2 * np.pi * u[1::2])
+    want = 1.0 + z * 2.0
+    assert np.max(np.abs(got - want)) < 2e-4       # device log / sin / cos, values up to ~10
+    assert abs(got.mean() - 1.0) < 0.01 and abs(got.std() - 2.0) < 0.01
+    assert abs(((got - 1.0) / 2.0 > 1.96).mean() - 0.025) < 0.002
+
+
+@pytest.mark.gpu
+def test_random_gpu_object_advances_and_rewinds(G):
+    """the header class: consecutive calls continue the stream, Seed() starts it again"""
+    n, seed = 10000, 42
+    out = G.buffer((n,), f32)
+    G.case_random(0, seed, out, -1.0, 1.0)
+    got = out.download()
+    words = model_words(seed, 0, 0, 4 * ((n // 2 + 3) // 4) + n - n // 2)
+    first = unit_open(words[: n // 2]) * f32(2) + f32(-1)
+    second = unit_open(words[4 * ((n // 2 + 3) // 4):][: n - n // 2]) * f32(2) + f32(-1)
+    assert np.array_equal(got[: n // 2], first.astype(f32)) and np.array_equal(got[n // 2:], second.astype(f32))
+    G.case_random(2, seed, out)
+    assert np.array_equal(out.download(), (unit_open(model_words(seed, 0, 0, n)) * f32(2)).astype(f32))
+    ints = G.buffer((n,), np.uint32)
+    G.case_random(3, -1, ints)      # a negative seed is sign-extended to 64 bits
+    assert np.array_equal(ints.download(), model_words(2**64 - 1, 0, 0, n))
+    G.case_random(1, seed, out, 0.0, 1.0)
+    z = out.download()
+    assert abs(z.mean()) < 0.05 and abs(z.std() - 1.0) < 0.05
