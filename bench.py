@@ -9,7 +9,7 @@ timed region; every operation is queued on one stream through the C ABI (the ele
 map through the C++ expression API compiled in libmshadow_cases.so).
 
 Output: one JSON line. `value` is the whole-step effective bandwidth: algorithmic bytes
-(each tensor counted once, table in BASELINE.md) of all nine operations divided by the
+(each tensor counted once) of all nine operations divided by the
 step time. `per_op` lists each operation's own GB/s, fraction of the 8 TB/s HBM peak and
 GElem/s from HIP events recorded around it on the same stream. `roofline` describes the
 kernel that takes the largest share of the step. `cpu_baseline` times the reference CPU
@@ -33,7 +33,7 @@ f32 = np.float32
 
 
 def algorithmic_bytes():
-    """Compulsory traffic per operation: every tensor once."""
+    """Compulsory traffic per operation: every tensor read or written once."""
     e = 4
     return {
         "map_fused": 5 * e * 4096 * 4096,
