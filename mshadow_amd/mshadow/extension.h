@@ -9,4 +9,5 @@
 #include "./ext/channels.h"
 #include "./ext/axes.h"
 #include "./ext/indexing.h"
+#include "./ext/complex.h"
 #endif  // MSHADOW_EXTENSION_H_

@@ -181,6 +181,36 @@ class Case(object):
             self.p = (2, 2 + sum(shape), 3)
             count = -(-(self.p[1] - self.p[0]) // self.p[2])
             self.want = np.repeat(f32(self.p[0]) + np.arange(count).astype(f32) * f32(self.p[2]), 2)
+        elif op >= 32:
+            # complex numbers as (real, imaginary) pairs along the last dimension
+            if w % 2:
+                pytest.skip("complex operands need an even last dimension")
+            a2 = a.reshape(rows, w)
+            self.b = rng.standard_normal((rows, w)).astype(f32)
+            self.c = rng.standard_normal((rows, w // 2)).astype(f32)
+            ar, ai, br, bi, cr = a2[:, 0::2], a2[:, 1::2], self.b[:, 0::2], self.b[:, 1::2], self.c
+            zero = np.zeros_like(cr)
+
+            def pairs(re, im):
+                out = np.empty((rows, 2 * re.shape[1]), f32)
+                out[:, 0::2], out[:, 1::2] = re, im
+                return out
+
+            def mul(xr, xi, yr, yi):
+                return pairs(xr * yr - xi * yi, xr * yi + yr * xi)
+
+            def div(xr, xi, yr, yi):
+                den = yr * yr + yi * yi
+                return pairs((xr * yr + xi * yi) / den, (yr * xi - xr * yi) / den)
+
+            self.want = {
+                32: lambda: mul(ar, ai, br, bi), 33: lambda: mul(ar, ai, cr, zero),
+                34: lambda: mul(cr, zero, ar, ai), 35: lambda: div(ar, ai, br, bi),
+                36: lambda: div(ar, ai, cr, zero), 37: lambda: div(cr, zero, ar, ai),
+                38: lambda: pairs(ar, -ai), 39: lambda: pairs(ai, ar),
+                40: lambda: pairs(a2, np.zeros_like(a2)), 41: lambda: ar,
+                42: lambda: ar * ar + ai * ai, 43: lambda: ar + ai,
+            }[op]()
         elif op >= 28:
             # a pitch that keeps 16-byte alignment (pack route where the row length allows it)
             # or one that breaks it (element-wise route)
@@ -211,7 +241,7 @@ class Case(object):
         self.want = np.ascontiguousarray(self.want, dtype=f32)
 
 
-N_OPS = 32
+N_OPS = 44
 
 
 def _pitched(arr, pad):
