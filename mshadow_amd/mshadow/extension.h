@@ -10,4 +10,5 @@
 #include "./ext/axes.h"
 #include "./ext/indexing.h"
 #include "./ext/complex.h"
+#include "./ext/implicit_gemm.h"
 #endif  // MSHADOW_EXTENSION_H_

@@ -181,6 +181,20 @@ class Case(object):
             self.p = (2, 2 + sum(shape), 3)
             count = -(-(self.p[1] - self.p[0]) // self.p[2])
             self.want = np.repeat(f32(self.p[0]) + np.arange(count).astype(f32) * f32(self.p[2]), 2)
+        elif op == 44:
+            # four running sums over the multiple-of-4 prefix, folded (s0 + s2) + (s1 + s3), then
+            # the tail one by one
+            k = h * w
+            self.b = rng.standard_normal((k, w)).astype(f32)
+            lhs, rhs = a.reshape(n * ch, k), self.b * f32(0.5)
+            part = np.zeros((4, n * ch, w), f32)
+            whole = k // 4 * 4
+            for i in range(whole):
+                part[i % 4] = part[i % 4] + lhs[:, i:i + 1] * rhs[i:i + 1, :]
+            res = (part[0] + part[2]) + (part[1] + part[3])
+            for i in range(whole, k):
+                res = res + lhs[:, i:i + 1] * rhs[i:i + 1, :]
+            self.want = res
         elif op >= 32:
             # complex numbers as (real, imaginary) pairs along the last dimension
             if w % 2:
@@ -241,7 +255,7 @@ class Case(object):
         self.want = np.ascontiguousarray(self.want, dtype=f32)
 
 
-N_OPS = 44
+N_OPS = 45
 
 
 def _pitched(arr, pad):
