@@ -266,6 +266,33 @@ void LaunchGrad(int flags, const GradLaunch &g) {
 }  // namespace
 
 
+/* about as many workgroups as the machine holds at once (two of these per CU), each owning a
+   run of destination rows and scanning the index vector once */
+template <bool CLAMP>
+static int LaunchAddTakeGrad(float *dst, int dstride, int k_rows, const void *rows_of,
+                             const void *from_of, int index_is_int, int n_index, const float *src,
+                             int sstride, int cols, void *stream, const char *what) {
+  const int kWavesPerBlock = kTakeBlock / 64;
+  const int rows_per_block_wanted = (k_rows + 511) / 512;
+  const int rows_per_wave = (rows_per_block_wanted + kWavesPerBlock - 1) / kWavesPerBlock;
+  const int rows_per_block = rows_per_wave * kWavesPerBlock;
+  const unsigned grid = static_cast<unsigned>((k_rows + rows_per_block - 1) / rows_per_block);
+  const bool vec = Aligned16(dst) && Aligned16(src) && dstride % 4 == 0 && sstride % 4 == 0 &&
+                   cols % 4 == 0;
+  hipStream_t s = AsStream(stream);
+#define TAKE_LAUNCH(INT, VEC)                                                                   \
+  hipLaunchKernelGGL((AddTakeGradBlockKernel<INT, CLAMP, VEC>), dim3(grid), dim3(kTakeBlock), 0, s, \
+                     dst, dstride, k_rows, rows_per_wave, rows_of, from_of, n_index, src, sstride, \
+                     cols)
+  if (index_is_int) {
+    if (vec) TAKE_LAUNCH(true, true); else TAKE_LAUNCH(true, false);
+  } else {
+    if (vec) TAKE_LAUNCH(false, true); else TAKE_LAUNCH(false, false);
+  }
+#undef TAKE_LAUNCH
+  return AfterLaunch(what);
+}
+
 extern "C" {
 
 /* ------------------------------------------------------------------ softmax */
@@ -458,22 +485,8 @@ int mshadow_hip_add_take_grad_f32(float *dst, int dstride, int k_rows, const voi
                                   int cols, void *stream) {
   const int chk = RowOpCheck(dst, dstride, k_rows, index, n_index, src, sstride, cols);
   if (chk != MSHADOW_HIP_OK) return chk < 0 ? MSHADOW_HIP_OK : chk;
-  /* one wave per destination row, or per index entry when the table has more rows */
-  const bool by_entry = n_index < k_rows;
-  const unsigned waves = static_cast<unsigned>(by_entry ? n_index : k_rows);
-  const unsigned grid = (waves + kRowBlock / 64 - 1) / (kRowBlock / 64);
-#define ROW_LAUNCH(...)                                                                    \
-  hipLaunchKernelGGL((__VA_ARGS__), dim3(grid), dim3(kRowBlock), 0, AsStream(stream), dst, dstride, \
-                     k_rows, index, index, n_index, src, sstride, cols)
-  if (by_entry) {
-    if (index_is_int) ROW_LAUNCH(AddTakeGradByEntryKernel<true, true>);
-    else ROW_LAUNCH(AddTakeGradByEntryKernel<false, true>);
-  } else {
-    if (index_is_int) ROW_LAUNCH(AddTakeGradKernel<true, true>);
-    else ROW_LAUNCH(AddTakeGradKernel<false, true>);
-  }
-#undef ROW_LAUNCH
-  return AfterLaunch("add_take_grad");
+  return LaunchAddTakeGrad<true>(dst, dstride, k_rows, index, index, index_is_int, n_index, src,
+                                 sstride, cols, stream, "add_take_grad");
 }
 
 int mshadow_hip_add_take_grad_large_batch_f32(float *dst, int dstride, int k_rows,
@@ -483,21 +496,8 @@ int mshadow_hip_add_take_grad_large_batch_f32(float *dst, int dstride, int k_row
   const int chk = RowOpCheck(dst, dstride, k_rows, index, n_index, src, sstride, cols);
   if (chk != MSHADOW_HIP_OK) return chk < 0 ? MSHADOW_HIP_OK : chk;
   ABI_REQUIRE(sorted != NULL, "NULL tensor");
-  const bool by_entry = n_index < k_rows;
-  const unsigned waves = static_cast<unsigned>(by_entry ? n_index : k_rows);
-  const unsigned grid = (waves + kRowBlock / 64 - 1) / (kRowBlock / 64);
-#define ROW_LAUNCH(...)                                                                    \
-  hipLaunchKernelGGL((__VA_ARGS__), dim3(grid), dim3(kRowBlock), 0, AsStream(stream), dst, dstride, \
-                     k_rows, sorted, index, n_index, src, sstride, cols)
-  if (by_entry) {
-    if (index_is_int) ROW_LAUNCH(AddTakeGradByEntryKernel<true, false>);
-    else ROW_LAUNCH(AddTakeGradByEntryKernel<false, false>);
-  } else {
-    if (index_is_int) ROW_LAUNCH(AddTakeGradKernel<true, false>);
-    else ROW_LAUNCH(AddTakeGradKernel<false, false>);
-  }
-#undef ROW_LAUNCH
-  return AfterLaunch("add_take_grad_large_batch");
+  return LaunchAddTakeGrad<false>(dst, dstride, k_rows, sorted, index, index_is_int, n_index, src,
+                                  sstride, cols, stream, "add_take_grad_large_batch");
 }
 
 int mshadow_hip_index_fill_f32(float *dst, int dstride, int k_rows, const void *index,
