@@ -268,8 +268,8 @@ void LaunchGrad(int flags, const GradLaunch &g) {
 
 /* about as many workgroups as the machine holds at once (two of these per CU), each owning a
    run of destination rows and scanning the index vector once */
-template <bool CLAMP>
-static int LaunchAddTakeGrad(float *dst, int dstride, int k_rows, const void *rows_of,
+template <int OP>
+static int LaunchRowsByIndex(float *dst, int dstride, int k_rows, const void *rows_of,
                              const void *from_of, int index_is_int, int n_index, const float *src,
                              int sstride, int cols, void *stream, const char *what) {
   const int kWavesPerBlock = kTakeBlock / 64;
@@ -280,16 +280,15 @@ static int LaunchAddTakeGrad(float *dst, int dstride, int k_rows, const void *ro
   const bool vec = Aligned16(dst) && Aligned16(src) && dstride % 4 == 0 && sstride % 4 == 0 &&
                    cols % 4 == 0;
   hipStream_t s = AsStream(stream);
-#define TAKE_LAUNCH(INT, VEC)                                                                   \
-  hipLaunchKernelGGL((AddTakeGradBlockKernel<INT, CLAMP, VEC>), dim3(grid), dim3(kTakeBlock), 0, s, \
-                     dst, dstride, k_rows, rows_per_wave, rows_of, from_of, n_index, src, sstride, \
-                     cols)
+#define ROWS_LAUNCH(INT, VEC)                                                                 \
+  hipLaunchKernelGGL((RowsByIndexKernel<INT, OP, VEC>), dim3(grid), dim3(kTakeBlock), 0, s, dst,  \
+                     dstride, k_rows, rows_per_wave, rows_of, from_of, n_index, src, sstride, cols)
   if (index_is_int) {
-    if (vec) TAKE_LAUNCH(true, true); else TAKE_LAUNCH(true, false);
+    if (vec) ROWS_LAUNCH(true, true); else ROWS_LAUNCH(true, false);
   } else {
-    if (vec) TAKE_LAUNCH(false, true); else TAKE_LAUNCH(false, false);
+    if (vec) ROWS_LAUNCH(false, true); else ROWS_LAUNCH(false, false);
   }
-#undef TAKE_LAUNCH
+#undef ROWS_LAUNCH
   return AfterLaunch(what);
 }
 
@@ -485,8 +484,8 @@ int mshadow_hip_add_take_grad_f32(float *dst, int dstride, int k_rows, const voi
                                   int cols, void *stream) {
   const int chk = RowOpCheck(dst, dstride, k_rows, index, n_index, src, sstride, cols);
   if (chk != MSHADOW_HIP_OK) return chk < 0 ? MSHADOW_HIP_OK : chk;
-  return LaunchAddTakeGrad<true>(dst, dstride, k_rows, index, index, index_is_int, n_index, src,
-                                 sstride, cols, stream, "add_take_grad");
+  return LaunchRowsByIndex<kTakeGrad>(dst, dstride, k_rows, index, index, index_is_int, n_index,
+                                      src, sstride, cols, stream, "add_take_grad");
 }
 
 int mshadow_hip_add_take_grad_large_batch_f32(float *dst, int dstride, int k_rows,
@@ -496,8 +495,9 @@ int mshadow_hip_add_take_grad_large_batch_f32(float *dst, int dstride, int k_row
   const int chk = RowOpCheck(dst, dstride, k_rows, index, n_index, src, sstride, cols);
   if (chk != MSHADOW_HIP_OK) return chk < 0 ? MSHADOW_HIP_OK : chk;
   ABI_REQUIRE(sorted != NULL, "NULL tensor");
-  return LaunchAddTakeGrad<false>(dst, dstride, k_rows, sorted, index, index_is_int, n_index, src,
-                                  sstride, cols, stream, "add_take_grad_large_batch");
+  return LaunchRowsByIndex<kTakeGradSorted>(dst, dstride, k_rows, sorted, index, index_is_int,
+                                            n_index, src, sstride, cols, stream,
+                                            "add_take_grad_large_batch");
 }
 
 int mshadow_hip_index_fill_f32(float *dst, int dstride, int k_rows, const void *index,
@@ -505,21 +505,8 @@ int mshadow_hip_index_fill_f32(float *dst, int dstride, int k_rows, const void *
                                int cols, void *stream) {
   const int chk = RowOpCheck(dst, dstride, k_rows, index, n_index, src, sstride, cols);
   if (chk != MSHADOW_HIP_OK) return chk < 0 ? MSHADOW_HIP_OK : chk;
-  const bool by_entry = n_index < k_rows;
-  const unsigned waves = static_cast<unsigned>(by_entry ? n_index : k_rows);
-  const unsigned grid = (waves + kRowBlock / 64 - 1) / (kRowBlock / 64);
-#define ROW_LAUNCH(...)                                                                    \
-  hipLaunchKernelGGL((__VA_ARGS__), dim3(grid), dim3(kRowBlock), 0, AsStream(stream), dst, dstride, \
-                     k_rows, index, n_index, src, sstride, cols)
-  if (by_entry) {
-    if (index_is_int) ROW_LAUNCH(IndexFillByEntryKernel<true>);
-    else ROW_LAUNCH(IndexFillByEntryKernel<false>);
-  } else {
-    if (index_is_int) ROW_LAUNCH(IndexFillKernel<true>);
-    else ROW_LAUNCH(IndexFillKernel<false>);
-  }
-#undef ROW_LAUNCH
-  return AfterLaunch("index_fill");
+  return LaunchRowsByIndex<kFill>(dst, dstride, k_rows, index, index, index_is_int, n_index, src,
+                                  sstride, cols, stream, "index_fill");
 }
 
 /* ------------------------------------------------------------------ reductions */

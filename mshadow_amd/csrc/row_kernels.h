@@ -8,9 +8,8 @@
  * and, for IndexFill, keeps the LAST source row written to it. To reproduce that without
  * a sort or a workspace, every destination row has one owner wave that applies the entries
  * naming it in index order, the lanes spread over the columns; nothing else touches the row,
- * so there is no atomic and no race. AddTakeGrad shares one scan of the index vector among
- * the sixteen waves of a workgroup (AddTakeGradBlockKernel); IndexFill, which only needs the
- * last entry of a row, scans per row or per entry.
+ * so there is no atomic and no race. The sixteen waves of a workgroup share one scan of the
+ * index vector (RowsByIndexKernel).
  */
 #ifndef MSHADOW_AMD_CSRC_ROW_KERNELS_H_
 #define MSHADOW_AMD_CSRC_ROW_KERNELS_H_
@@ -22,7 +21,6 @@
 
 namespace mshadow_hipk {
 
-const int kRowBlock = 256;  // four destination rows per workgroup
 
 /*! \brief entry y of an index vector stored as int32 or as float (truncated like a label) */
 template <bool IS_INT>
@@ -33,10 +31,16 @@ __device__ __forceinline__ int IndexAt(const void *index, int y) {
 
 const int kTakeBlock = 1024;  // sixteen waves share one scan of the index vector
 
-/*! \brief dst[row(y)] += src[from(y)] for y = 0 .. n_index-1 in order.
- *  CLAMP: row(y) = index[y] clamped into [0, k_rows) and from(y) = y    (AddTakeGrad);
- *  else:  row(y) = sorted[y] and from(y) = index[y]                   (AddTakeGradLargeBatch,
- *  which therefore also gives the reference's result when `sorted` is not sorted).
+/*! \brief what the three functions do to a destination row for entry y, front to back */
+enum RowOp {
+  kTakeGrad = 0,       //!< dst[clamp(index[y])] += src[y]                      (AddTakeGrad)
+  kTakeGradSorted = 1, //!< dst[sorted[y]] += src[index[y]], rows outside the table skipped
+                       //!< (AddTakeGradLargeBatch; also right when `sorted` is not sorted)
+  kFill = 2            //!< dst[index[y]] = src[y], rows outside the table skipped: of several
+                       //!< entries naming one row the last one counts          (IndexFill)
+};
+
+/*! \brief the row operation OP for y = 0 .. n_index-1 in order.
  *  a workgroup owns 16 * rows_per_wave consecutive destination rows and scans the index
  *  vector once, 1024 entries at a time. The entries of a chunk that fall into its rows are
  *  compacted, in index order, into a list in LDS (a ballot per wave and a prefix over the
@@ -45,12 +49,14 @@ const int kTakeBlock = 1024;  // sixteen waves share one scan of the index vecto
  *  chunks follow each other, so every row receives its additions in index order - with no
  *  atomic, no sort and no workspace. Scan work is (rows / rows per workgroup) * entries / 64
  *  wave-steps. VEC4: rows are whole aligned 16-byte packs. */
-template <bool IS_INT, bool CLAMP, bool VEC4>
+template <bool IS_INT, int OP, bool VEC4>
 __global__ void __launch_bounds__(kTakeBlock)
-    AddTakeGradBlockKernel(float *dst, int dstride, int k_rows, int rows_per_wave,
+    RowsByIndexKernel(float *dst, int dstride, int k_rows, int rows_per_wave,
                            const void *rows_of, const void *from_of, int n_index, const float *src,
                            int sstride, int cols) {
   typedef float F4 __attribute__((ext_vector_type(4)));
+  const bool CLAMP = OP == kTakeGrad;
+  const bool FROM_ENTRY = OP != kTakeGradSorted;
   const int W = kTakeBlock / 64;
   __shared__ int list_y[2][kTakeBlock];
   __shared__ int list_r[2][kTakeBlock];
@@ -99,7 +105,7 @@ __global__ void __launch_bounds__(kTakeBlock)
         mine &= mine - 1ull;
         const int row = __shfl(er, b);
         const int entry = __shfl(ey, b);
-        const int from = CLAMP ? entry : IndexAt<IS_INT>(from_of, entry);
+        const int from = FROM_ENTRY ? entry : IndexAt<IS_INT>(from_of, entry);
         const float *in = src + static_cast<size_t>(from) * sstride;
         float *out = dst + static_cast<size_t>(row) * dstride;
         if (VEC4) {
@@ -111,64 +117,22 @@ __global__ void __launch_bounds__(kTakeBlock)
             for (int k = 0; k < 4; ++k) {
               const int x = x0 + k * 256;
               if (x < cols) {
-                a[k] = *reinterpret_cast<const F4 *>(out + x);
+                if (OP != kFill) a[k] = *reinterpret_cast<const F4 *>(out + x);
                 c[k] = __builtin_nontemporal_load(reinterpret_cast<const F4 *>(in + x));
               }
             }
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
               const int x = x0 + k * 256;
-              if (x < cols) *reinterpret_cast<F4 *>(out + x) = a[k] + c[k];
+              if (x < cols) *reinterpret_cast<F4 *>(out + x) = OP == kFill ? c[k] : a[k] + c[k];
             }
           }
         } else {
-          for (int x = lane; x < cols; x += 64) out[x] = out[x] + in[x];
+          for (int x = lane; x < cols; x += 64) out[x] = OP == kFill ? in[x] : out[x] + in[x];
         }
       }
     }
   }
-}
-
-/*! \brief IndexFill by entry: the wave of entry y copies its row unless a later entry names
- *  the same destination */
-template <bool IS_INT>
-__global__ void __launch_bounds__(kRowBlock)
-    IndexFillByEntryKernel(float *dst, int dstride, int k_rows, const void *index, int n_index,
-                           const float *src, int sstride, int cols) {
-  const int lane = threadIdx.x & 63;
-  const int me = blockIdx.x * (kRowBlock / 64) + (threadIdx.x >> 6);
-  if (me >= n_index) return;
-  const int j = IndexAt<IS_INT>(index, me);
-  if (j < 0 || j >= k_rows) return;
-  for (int y0 = (me / 64) * 64; y0 < n_index; y0 += 64) {
-    const int y = y0 + lane;
-    const bool later = y > me && y < n_index && IndexAt<IS_INT>(index, y) == j;
-    if (__ballot(later) != 0ull) return;
-  }
-  const float *in = src + static_cast<size_t>(me) * sstride;
-  float *out = dst + static_cast<size_t>(j) * dstride;
-  for (int x = lane; x < cols; x += 64) out[x] = in[x];
-}
-
-/*! \brief dst[index[y]] = src[y]; of several entries naming one row the last one counts */
-template <bool IS_INT>
-__global__ void __launch_bounds__(kRowBlock)
-    IndexFillKernel(float *dst, int dstride, int k_rows, const void *index, int n_index,
-                    const float *src, int sstride, int cols) {
-  const int lane = threadIdx.x & 63;
-  const int j = blockIdx.x * (kRowBlock / 64) + (threadIdx.x >> 6);
-  if (j >= k_rows) return;
-  int last = -1;
-  for (int y0 = 0; y0 < n_index; y0 += 64) {
-    const int y = y0 + lane;
-    const bool hit = y < n_index && IndexAt<IS_INT>(index, y) == j;
-    const unsigned long long hits = __ballot(hit);
-    if (hits != 0ull) last = y0 + 63 - __clzll(static_cast<long long>(hits));
-  }
-  if (last < 0) return;
-  const float *in = src + static_cast<size_t>(last) * sstride;
-  float *out = dst + static_cast<size_t>(j) * dstride;
-  for (int x = lane; x < cols; x += 64) out[x] = in[x];
 }
 
 }  // namespace mshadow_hipk
