@@ -189,7 +189,7 @@ def main():
             G.case_shaping(0, extra["out4"], dev["X2a"], extra["bias"], 64, 256, 56, 56, s)
         elif name == "swapaxis10_reshape":
             G.case_shaping(2, extra["out4"], dev["X2a"], extra["bias"], 64, 256, 56, 56, s)
-        elif name == "lrn_scale_chpool5":   # x * (chpool<sum>(x * x, 5) * 0.1 + 1)
+        elif name == "lrn_scale_chpool5":   # x * (chpool<sum>(F<square>(x), 5) * 0.1 + 1)
             G.case_extensions(19, extra["out4"], dev["X2a"], None, None, 64, 256, 56, 56, 5, 0, 0, s)
         elif name == "transpose_nchw_nhwc":
             G.case_extensions(7, extra["out4"], dev["X2a"], None, None, 64, 256, 56, 56, 231, 0, 0, s)

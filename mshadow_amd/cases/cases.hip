@@ -330,6 +330,11 @@ int mshadow_case_sort_by_key_32(int op, void *keys, int key_kind, void *values, 
   CASE_END
 }
 
+/* caller-side functor of the extension cases (local response normalisation squares its input) */
+struct square_of {
+  MSHADOW_XINLINE static float Map(float a) { return a * a; }
+};
+
 /* channel pooling, axis reductions / broadcasts, permutations, assignable views and the
    index look-ups, through the generic expression kernel; dense tensors */
 int mshadow_case_extensions_f32(int op, float *out, const float *a, const float *b, const float *c,

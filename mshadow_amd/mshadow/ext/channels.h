@@ -105,6 +105,10 @@ struct Plan<ChannelPoolingExp<Reducer, SrcExp, DType, srcdim>, DType> {
     index_t last = c * stride_ - pad_ + nsize_;
     if (last > channel_.div) last = channel_.div;
     if (last > src_channel_) last = src_channel_;
+    /* the usual window sizes as straight-line code: all fetches of a window (and of the other
+       packs the calling thread evaluates) are in flight together */
+    if (nsize_ == 5) return FixedWindow<5, N>(n, c, y, j, last);
+    if (nsize_ == 3) return FixedWindow<3, N>(n, c, y, j, last);
     Pack<DType, N> res;
 #pragma unroll
     for (int k = 0; k < N; ++k) Reducer::SetInitValue(res.v[k]);
@@ -139,6 +143,37 @@ struct Plan<ChannelPoolingExp<Reducer, SrcExp, DType, srcdim>, DType> {
   }
 
  private:
+  /*! \brief a window of K channels starting at c * stride - pad and ending before `last`:
+   *  every position is fetched (a position outside the window re-reads the pooled channel's
+   *  own row index clamped into the source, and is not reduced), then reduced in channel order */
+  template <int K, int N>
+  MSHADOW_XINLINE Pack<DType, N> FixedWindow(index_t n, index_t c, index_t y, index_t j,
+                                             index_t last) const {
+    const index_t step = height_.div;
+    const index_t start = c * stride_ - pad_;  // may be negative: those positions are skipped
+    Pack<DType, N> v[K];
+    bool inside[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const index_t cc = start + k;
+      inside[k] = cc >= 0 && cc < last;
+      const index_t safe = inside[k] ? cc : 0;
+      v[k] = src_.template EvalPack<N, false>((n * src_channel_ + safe) * step + y, j);
+    }
+    Pack<DType, N> res;
+#pragma unroll
+    for (int e = 0; e < N; ++e) Reducer::SetInitValue(res.v[e]);
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+#pragma unroll
+      for (int e = 0; e < N; ++e) {
+        DType with = res.v[e];
+        Reducer::Reduce(with, v[k].v[e]);
+        res.v[e] = inside[k] ? with : res.v[e];
+      }
+    }
+    return res;
+  }
   Plan<SrcExp, DType> src_;
   const FastDivU32 channel_, height_;
   const index_t nsize_, stride_, pad_, src_channel_;

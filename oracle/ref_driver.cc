@@ -274,6 +274,11 @@ void ref_random_f32(int op, int seed, float *out, int n, float p0, float p1) {
 #include "../mshadow_amd/cases/random_cases.inc"
 }
 
+/* caller-side functor of the extension cases (local response normalisation squares its input) */
+struct square_of {
+  MSHADOW_XINLINE static float Map(float a) { return a * a; }
+};
+
 void ref_extensions_f32(int op, float *out, const float *a, const float *b, const float *c, int n,
                         int ch, int h, int w, int p0, int p1, int p2) {
 #define TENSOR(dim) Tensor<cpu, dim, float>

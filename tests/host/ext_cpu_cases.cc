@@ -14,6 +14,11 @@ Tensor<cpu, dim, float> View(const float *p, Shape<dim> shape) {
 }
 }  // namespace
 
+/* caller-side functor of the extension cases (local response normalisation squares its input) */
+struct square_of {
+  MSHADOW_XINLINE static float Map(float a) { return a * a; }
+};
+
 extern "C" int host_extensions_f32(int op, float *out, const float *a, const float *b,
                                    const float *c, int n, int ch, int h, int w, int p0, int p1,
                                    int p2) {
