@@ -92,6 +92,11 @@ int mshadow_case_extensions_f32(int op, float *out, const float *a, const float 
                                 int n, int ch, int h, int w, int p0, int p1, int p2,
                                 void *stream);
 
+/* dst <saver>= scale * dot(a[.T()], b[.T()]) for matrices and vectors, VectorDot, BatchGEMM and
+   batch_dot over dense operands (op 0..16, listed with shapes in cases/dot_cases.inc) */
+int mshadow_case_dot_f32(int op, float *out, const float *a, const float *b, int m, int k, int n,
+                         int batch, void *stream);
+
 /* dst = pool<Reducer>(src, Shape2(ph, pw), ky, kx, sy, sx) */
 int mshadow_case_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes,
                           int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,

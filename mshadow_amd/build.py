@@ -52,8 +52,9 @@ def _run(cmd, verbose):
 
 def build_hip_library(verbose=True):
     os.makedirs(LIB_DIR, exist_ok=True)
-    srcs = [os.path.join(HERE, "csrc", f) for f in ("runtime.hip", "ops.hip", "sort.hip", "permute.hip", "random.hip")]
-    _run([hipcc()] + COMMON + ["-o", HIP_SO] + srcs, verbose)
+    srcs = [os.path.join(HERE, "csrc", f) for f in ("runtime.hip", "ops.hip", "sort.hip", "permute.hip", "random.hip", "blas.hip")]
+    # -ldl: blas.hip opens rocBLAS at run time, on the first matrix product
+    _run([hipcc()] + COMMON + ["-o", HIP_SO] + srcs + ["-ldl"], verbose)
     return HIP_SO
 
 

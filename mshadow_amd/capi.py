@@ -18,8 +18,10 @@ SAVETO, PLUSTO, MINUSTO, MULTO, DIVTO = range(5)
 SUM, MAX, MIN = range(3)
 H2D, D2H, D2D = 1, 2, 3
 KEY_F32, KEY_I32, KEY_U32 = range(3)
+BLAS_F32, BLAS_F64, BLAS_F16 = range(3)
 
 _i, _f, _p, _sz = C.c_int, C.c_float, C.c_void_p, C.c_size_t
+_d, _ll = C.c_double, C.c_longlong
 
 
 class HipError(RuntimeError):
@@ -33,7 +35,7 @@ class Props(C.Structure):
                 ("lds_bytes_per_block", _sz), ("total_global_mem", _sz)]
 
 
-# name -> argtypes, for every symbol include/mshadow_hip.h declares
+# name -> argtypes, for every symbol include/mshadow_hip.h and include/mshadow_hip_blas.h declare
 HIP_SYMBOLS = {
     "mshadow_hip_last_error": ([], C.c_char_p),
     "mshadow_hip_abi_version": ([], _i),
@@ -86,6 +88,10 @@ HIP_SYMBOLS = {
     "mshadow_hip_im2col_f32": ([_p, _i, _p, _i] + [_i] * 12 + [_p], _i),
     "mshadow_hip_col2im_f16": ([_p, _i, _p, _i] + [_i] * 12 + [_p], _i),
     "mshadow_hip_col2im_f32": ([_p, _i, _p, _i] + [_i] * 12 + [_p], _i),
+    "mshadow_hip_blas_gemm": ([_i, _i, _i, _i, _i, _i, _d, _p, _i, _ll, _p, _i, _ll, _d, _p, _i, _ll, _i, _p], _i),
+    "mshadow_hip_blas_gemv": ([_i, _i, _i, _i, _d, _p, _i, _ll, _p, _i, _ll, _d, _p, _i, _ll, _i, _p], _i),
+    "mshadow_hip_blas_ger": ([_i, _i, _i, _d, _p, _i, _ll, _p, _i, _ll, _p, _i, _ll, _i, _p], _i),
+    "mshadow_hip_blas_dot": ([_i, _i, _p, _i, _p, _i, _p, _p], _i),
 }
 
 CASES_SYMBOLS = {
@@ -103,6 +109,7 @@ CASES_SYMBOLS = {
     "mshadow_case_random_f32": ([_i, _i, _p, _i, _f, _f, _p], _i),
     "mshadow_case_sort_by_key_32": ([_i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_case_extensions_f32": ([_i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p], _i),
+    "mshadow_case_dot_f32": ([_i, _p, _p, _p, _i, _i, _i, _i, _p], _i),
     "mshadow_case_softmax_grad_f32": ([_p, _i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_case_pool_f32": ([_p, _i, _p, _i] + [_i] * 11 + [_p], _i),
     "mshadow_case_unpool_f32": ([_p, _i, _p, _i, _p, _i, _p, _i] + [_i] * 11 + [_p], _i),
@@ -417,6 +424,29 @@ class Library:
         self.check_case(self.cases.mshadow_case_shaping_f32(op, out.ptr, a.ptr, v.ptr, n, c, h, w,
                                                             stream))
 
+    # column-major BLAS entry points (include/mshadow_hip_blas.h); operands are DeviceBuffers
+    def blas_gemm(self, dtype, transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc,
+                  batch=1, strides=(0, 0, 0), stream=None):
+        self.check(self.dll.mshadow_hip_blas_gemm(dtype, int(transa), int(transb), m, n, k, alpha,
+                                                  A.ptr, lda, strides[0], B.ptr, ldb, strides[1],
+                                                  beta, Cm.ptr, ldc, strides[2], batch, stream))
+
+    def blas_gemv(self, dtype, trans, m, n, alpha, A, lda, x, incx, beta, y, incy, batch=1,
+                  strides=(0, 0, 0), stream=None):
+        self.check(self.dll.mshadow_hip_blas_gemv(dtype, int(trans), m, n, alpha, A.ptr, lda,
+                                                  strides[0], x.ptr, incx, strides[1], beta,
+                                                  y.ptr, incy, strides[2], batch, stream))
+
+    def blas_ger(self, dtype, m, n, alpha, x, incx, y, incy, A, lda, batch=1, strides=(0, 0, 0),
+                 stream=None):
+        self.check(self.dll.mshadow_hip_blas_ger(dtype, m, n, alpha, x.ptr, incx, strides[0],
+                                                 y.ptr, incy, strides[1], A.ptr, lda, strides[2],
+                                                 batch, stream))
+
+    def blas_dot(self, dtype, n, x, incx, y, incy, result, stream=None):
+        self.check(self.dll.mshadow_hip_blas_dot(dtype, n, x.ptr, incx, y.ptr, incy, result.ptr,
+                                                 stream))
+
     def case_random(self, op, seed, out, p0=0.0, p1=1.0, stream=None):
         self.check_case(self.cases.mshadow_case_random_f32(op, seed, out.ptr, out.cols, p0, p1, stream))
 
@@ -424,6 +454,9 @@ class Library:
         self.check_case(self.cases.mshadow_case_sort_by_key_32(
             op, keys.ptr, self._key_kind(keys), values.ptr, keys.cols, 1 if is_ascend else 0,
             stream))
+
+    def case_dot(self, op, out, a, b, m, k, n, batch=1, stream=None):
+        self.check_case(self.cases.mshadow_case_dot_f32(op, out.ptr, a.ptr, b.ptr, m, k, n, batch, stream))
 
     def case_extensions(self, op, out, a, b, c, n, ch, h, w, p0=0, p1=0, p2=0, stream=None):
         self.check_case(self.cases.mshadow_case_extensions_f32(

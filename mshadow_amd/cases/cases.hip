@@ -358,6 +358,30 @@ int mshadow_case_extensions_f32(int op, float *out, const float *a, const float 
   CASE_END
 }
 
+/* matrix products through the expression engine, VectorDot and BatchGEMM; dense operands
+   (shapes per op in dot_cases.inc) */
+int mshadow_case_dot_f32(int op, float *out, const float *a, const float *b, int m, int k, int n,
+                         int batch, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+#define XPU gpu
+#define STREAM st.get()
+#define TENSOR(dim) Tensor<gpu, dim, float>
+#define V1(p, len) G1(p, len, st.get())
+#define V2(p, d0, d1) G2(p, d0, d1, d1, st.get())
+#define V2S(p, d0, d1, pitch) G2(p, d0, d1, pitch, st.get())
+#define V3(p, d0, d1, d2) G3(p, d0, d1, d2, d2, st.get())
+#include "./dot_cases.inc"
+#undef XPU
+#undef STREAM
+#undef TENSOR
+#undef V1
+#undef V2
+#undef V2S
+#undef V3
+  CASE_END
+}
+
 int mshadow_case_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes,
                           int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,
                           int reducer, int variant, void *stream) {

@@ -2,8 +2,8 @@
  * ExpEngine: where `dst <saver>= expression` lands. Mapper, chainer and rvalue
  * trees go to MapExp on the destination's device; complex trees (reduce-to-1D, dot)
  * go to an ExpComplexEngine specialisation. Contract:
- * mshadow/expr_engine-inl.h:436-479 of the reference. The dot engine (BLAS) is not
- * part of this backend, so DotExp has no ExpComplexEngine here.
+ * mshadow/expr_engine-inl.h:436-479 of the reference. The specialisation for DotExp
+ * is in dot_engine.h, the one for reduce-to-1D in ext/reduceto1d.h.
  */
 #ifndef MSHADOW_EXPR_ENGINE_H_
 #define MSHADOW_EXPR_ENGINE_H_

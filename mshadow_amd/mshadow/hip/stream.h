@@ -3,8 +3,9 @@
  *
  * Stream<gpu> keeps the members callers touch in the reference
  * (mshadow/stream_gpu-inl.h:18-180): stream_, dev_id, Wait(), CheckIdle(),
- * GetStream(); the BLAS / solver / DNN handle members exist but are inert because
- * this backend has no BLAS engine. A NULL stream is fatal when MSHADOW_FORCE_STREAM
+ * GetStream(); the BLAS / solver / DNN handle members exist but are inert: the library
+ * behind the C ABI keeps its own rocBLAS handle per thread and device and binds it to the
+ * stream of each call, and there is no solver or DNN engine. A NULL stream is fatal when MSHADOW_FORCE_STREAM
  * is on, and otherwise means the device's default stream (:79-88).
  */
 #ifndef MSHADOW_HIP_STREAM_H_
@@ -83,7 +84,8 @@ struct Stream<gpu> {
     }
     return stream->stream_;
   }
-  /* no BLAS / solver / DNN engine in this backend: creation is accepted and ignored */
+  /* handles are owned by the library (BLAS) or do not exist (solver, DNN): creation is
+     accepted and ignored */
   inline void CreateBlasHandle() {}
   inline void DestroyBlasHandle() {}
   inline void CreateSolverHandle() {}

@@ -38,11 +38,13 @@ inline void ShutdownTensorEngine(void);
 template <typename Device>
 inline void SetDevice(int devid);
 /*! \brief create a computation stream; the two flags ask for BLAS / DNN handles, which
- *  this backend does not provide (they are accepted and ignored) */
+ *  callers do not hold here (they are accepted and ignored) */
 template <typename Device>
 inline Stream<Device> *NewStream(bool create_blas_handle, bool create_dnn_handle, int dev_id = -1);
+/*! \brief the default of dev_id is an addition: guide/basic_stream.cu of the reference calls
+ *  NewStream<gpu>() with no argument, which its own header (tensor.h:658-661) does not accept */
 template <typename Device>
-inline Stream<Device> *NewStream(int dev_id) {
+inline Stream<Device> *NewStream(int dev_id = -1) {
   return NewStream<Device>(true, false, dev_id);
 }
 template <typename Device>
@@ -162,6 +164,16 @@ inline void SortByKey(Tensor<gpu, 1, KDType> keys, Tensor<gpu, 1, VDType> values
 template <typename Device, typename VDType, typename SDType>
 inline void VectorizedSort(Tensor<Device, 1, VDType> values, Tensor<Device, 1, SDType> segments);
 
+/*! \brief dst[0] = sum_i lhs[i] * rhs[i]; dst is a vector of length one on the same device */
+template <typename Device, typename DType>
+inline void VectorDot(Tensor<Device, 1, DType> dst, const Tensor<Device, 1, DType> &lhs,
+                      const Tensor<Device, 1, DType> &rhs);
+/*! \brief dst[b] = alpha * op(lhs[b]) op(rhs[b]) + beta * dst[b] for every matrix b of the batch */
+template <bool transpose_left, bool transpose_right, typename Device, typename DType>
+inline void BatchGEMM(Tensor<Device, 3, DType> dst, const Tensor<Device, 3, DType> &lhs,
+                      const Tensor<Device, 3, DType> &rhs, DType alpha, DType beta,
+                      Tensor<Device, 1, DType *> workspace);
+
 /*! \brief Saver::Save(dst(y,x), exp(y,x)) for every element */
 template <typename Saver, typename R, int dim, typename DType, typename E, int etype>
 inline void MapExp(TRValue<R, cpu, dim, DType> *dst, const expr::Exp<E, DType, etype> &exp);
@@ -191,6 +203,9 @@ inline void MapReduceKeepHighDim(TRValue<R, gpu, 1, DType> *dst,
 #include "./expr/scalar_ops.h"
 #include "./cpu/tensor_cpu.h"
 #include "./hip/tensor_gpu.h"
+#include "./dot_engine.h"
+#include "./io.h"
 #include "./tensor_container.h"
+#include "./random.h"
 
 #endif  // MSHADOW_TENSOR_H_

@@ -1,0 +1,5 @@
+/*! \file tensor_gpu-inl.h  public include name kept for callers; everything comes with tensor.h */
+#ifndef MSHADOW_TENSOR_GPU_INL_H_
+#define MSHADOW_TENSOR_GPU_INL_H_
+#include "./tensor.h"
+#endif  // MSHADOW_TENSOR_GPU_INL_H_

@@ -298,6 +298,21 @@ void ref_extensions_f32(int op, float *out, const float *a, const float *b, cons
 #undef V4
 }
 
+/* the three matrix products the reference can evaluate without an external BLAS (its
+   stand-alone build sends them to implicit_dot, dot_engine-inl.h:853-863); every other form
+   of the product cases needs CBLAS or MKL there and is checked against float64 instead */
+void ref_dot_f32(int op, float *out, const float *a, const float *b, int m, int k, int n) {
+  const int batch = 1;
+  (void)batch;
+#define TENSOR(dim) Tensor<cpu, dim, float>
+#define V2(p, d0, d1) T2(p, d0, d1, d1)
+#define MSHADOW_CASES_REFERENCE_HEADERS
+#include "../mshadow_amd/cases/dot_cases.inc"
+#undef MSHADOW_CASES_REFERENCE_HEADERS
+#undef TENSOR
+#undef V2
+}
+
 void ref_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes, int h, int w,
                   int ph, int pw, int ky, int kx, int sy, int sx, int reducer) {
   Tensor<cpu, 3, float> S = T3(src, planes, h, w, sstride);

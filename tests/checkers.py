@@ -89,6 +89,7 @@ class Checker:
             self._fn("shaping_f32", [_i, _p, _p, _p, _i, _i, _i, _i])
             self._fn("extensions_f32", [_i, _p, _p, _p, _p] + [_i] * 7)
             self._fn("random_f32", [_i, _i, _p, _i, _f, _f])
+            self._fn("dot_f32", [_i, _p, _p, _p, _i, _i, _i])
         self._fn("pool_f32", [_p, _i, _p, _i] + [_i] * 10)
         self._fn("unpool_f32", [_p, _i, _p, _i, _p, _i, _p, _i] + [_i] * 10)
         for t in ("f16", "f32"):
@@ -217,6 +218,12 @@ class Checker:
     def random(self, op, seed, out, p0=0.0, p1=1.0):
         """reference build only: Random<cpu> samplers into a float vector"""
         self._random_f32(op, seed, ptr(out), out.shape[0], p0, p1)
+        return out
+
+    def dot(self, op, out, a, b, m, k, n):
+        """reference build only: the matrix products it evaluates without an external BLAS
+        (op 0..2 of the product cases)"""
+        self._dot_f32(op, ptr(out), ptr(a), ptr(b), m, k, n)
         return out
 
     def extensions(self, op, out, a, b, c, n, ch, h, w, p0=0, p1=0, p2=0):

@@ -4,6 +4,8 @@
 #include <mshadow/tensor.h>
 #include <mshadow/random.h>
 
+#include "../../mshadow_amd/cases/portable_math.h"
+
 using namespace mshadow;
 using namespace mshadow::expr;
 
@@ -13,6 +15,11 @@ Tensor<cpu, dim, float> View(const float *p, Shape<dim> shape) {
   return Tensor<cpu, dim, float>(const_cast<float *>(p), shape);
 }
 }  // namespace
+
+/* caller-side functor of the product cases, same arithmetic as the device build */
+struct sigmoid {
+  MSHADOW_XINLINE static float Map(float a) { return pmath_sigmoid(a); }
+};
 
 /* caller-side functor of the extension cases (local response normalisation squares its input) */
 struct square_of {
@@ -47,6 +54,32 @@ extern "C" int host_extensions_f32(int op, float *out, const float *a, const flo
 extern "C" int host_random_f32(int op, int seed, float *out, int n, float p0, float p1) {
   try {
 #include "../../mshadow_amd/cases/random_cases.inc"
+  } catch (const std::exception &e) {
+    fprintf(stderr, "%s\n", e.what());
+    return 1;
+  }
+  return 0;
+}
+
+extern "C" int host_dot_f32(int op, float *out, const float *a, const float *b, int m, int k,
+                            int n, int batch) {
+  try {
+#define XPU cpu
+#define STREAM static_cast<Stream<cpu> *>(NULL)
+#define TENSOR(dim) Tensor<cpu, dim, float>
+#define V1(p, len) View(p, Shape1(len))
+#define V2(p, d0, d1) View(p, Shape2(d0, d1))
+#define V2S(p, d0, d1, pitch) \
+  Tensor<cpu, 2, float>(const_cast<float *>(p), Shape2(d0, d1), pitch, NULL)
+#define V3(p, d0, d1, d2) View(p, Shape3(d0, d1, d2))
+#include "../../mshadow_amd/cases/dot_cases.inc"
+#undef XPU
+#undef STREAM
+#undef TENSOR
+#undef V1
+#undef V2
+#undef V2S
+#undef V3
   } catch (const std::exception &e) {
     fprintf(stderr, "%s\n", e.what());
     return 1;

@@ -29,10 +29,11 @@ def _lib(name):
 
 
 @pytest.mark.parametrize("header,libname", [("mshadow_hip.h", "libmshadow_hip.so"),
+                                            ("mshadow_hip_blas.h", "libmshadow_hip.so"),
                                             ("mshadow_hip_cases.h", "libmshadow_cases.so")])
 def test_every_declared_symbol_is_exported(header, libname):
     names = _declared(header)
-    assert len(names) >= 10
+    assert len(names) >= (4 if "blas" in header else 10)
     if libname == "libmshadow_cases.so":
         _lib("libmshadow_hip.so")
     lib = _lib(libname)
@@ -43,7 +44,8 @@ def test_every_declared_symbol_is_exported(header, libname):
 def test_python_symbol_tables_match_headers():
     from mshadow_amd import capi
 
-    assert sorted(capi.HIP_SYMBOLS) == _declared("mshadow_hip.h")
+    assert sorted(capi.HIP_SYMBOLS) == sorted(_declared("mshadow_hip.h") +
+                                              _declared("mshadow_hip_blas.h"))
     assert sorted(capi.CASES_SYMBOLS) == _declared("mshadow_hip_cases.h")
 
 
@@ -61,7 +63,8 @@ def test_expression_routes_reach_the_fixed_function_entries():
               "mshadow_hip_im2col_f32", "mshadow_hip_col2im_f16", "mshadow_hip_col2im_f32",
               "mshadow_hip_permute_32", "mshadow_hip_reduce_keep_lowest_f32",
               "mshadow_hip_reduce_keep_highdim_f32", "mshadow_hip_softmax_f32",
-              "mshadow_hip_sort_by_key_32"}
+              "mshadow_hip_sort_by_key_32", "mshadow_hip_blas_gemm", "mshadow_hip_blas_gemv",
+              "mshadow_hip_blas_ger", "mshadow_hip_blas_dot"}
     assert wanted <= imported, sorted(wanted - imported)
 
 
