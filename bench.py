@@ -56,6 +56,8 @@ def algorithmic_bytes():
         "lrn_scale_chpool5": 2 * e * 64 * 256 * 56 * 56,
         "transpose_nchw_nhwc": 2 * e * 64 * 256 * 56 * 56,
         "sort_by_key_f32": 4 * e * (1 << 24),
+        "dot_f32_4096": 3 * e * 4096 * 4096,
+        "dot_f16_8192": 3 * 2 * 8192 * 8192,
     }
 
 
@@ -69,13 +71,18 @@ def work_elements():
         "softmax3d_grad": 256 * 21 * 16384, "add_take_grad": 16384 * 512,
         "bias_add_broadcast": 64 * 256 * 56 * 56, "swapaxis10_reshape": 64 * 256 * 56 * 56,
         "lrn_scale_chpool5": 64 * 256 * 56 * 56, "transpose_nchw_nhwc": 64 * 256 * 56 * 56,
-        "sort_by_key_f32": 1 << 24,
+        "sort_by_key_f32": 1 << 24, "dot_f32_4096": 4096 * 4096, "dot_f16_8192": 8192 * 8192,
     }
+
+
+# multiply-adds count two: the plain library products (rocBLAS), priced against the dense
+# matrix-core peaks (fp32 157.3 TFLOP/s, fp16 2500 TFLOP/s)
+PRODUCT_FLOPS = {"dot_f32_4096": (2 * 4096 ** 3, 157.3), "dot_f16_8192": (2 * 8192 ** 3, 2500.0)}
 
 
 EXTRA_OPS = ("calib_copy", "smooth_softmax_grad_ignore", "softmax3d", "softmax3d_grad", "add_take_grad",
              "bias_add_broadcast", "swapaxis10_reshape", "lrn_scale_chpool5", "transpose_nchw_nhwc",
-             "sort_by_key_f32")
+             "sort_by_key_f32", "dot_f32_4096", "dot_f16_8192")
 OPS = [k for k in algorithmic_bytes() if k not in EXTRA_OPS]
 
 # HBM bytes per launch of each operation's kernel, measured with rocprofv3 --pmc FETCH_SIZE and
@@ -184,8 +191,22 @@ def main():
         extra["out4"] = G.buffer(H["X2a"].shape, f32)
         extra["bias"] = G.to_device(np.random.default_rng(14).standard_normal(51380224, dtype=f32)[:256].copy())
 
+    if "dot_f32_4096" in only:   # dst = dot(A, B.T()) through the expression engine
+        extra["mm_out"] = G.buffer((4096, 4096), f32)
+    if "dot_f16_8192" in only:
+        from mshadow_amd import capi
+        h = np.random.default_rng(16).standard_normal(8192 * 8192, dtype=f32).astype(np.float16)
+        extra["ha"], extra["hb"] = G.to_device(h), G.to_device(h[::-1].copy())
+        extra["hc"] = G.buffer((8192 * 8192,), np.float16)
+        extra["f16"] = capi.BLAS_F16
+
     def run_op(name):
-        if name == "bias_add_broadcast":
+        if name == "dot_f32_4096":
+            G.case_dot(1, extra["mm_out"], dev["A"], dev["B"], 4096, 4096, 4096, 1, s)
+        elif name == "dot_f16_8192":
+            G.blas_gemm(extra["f16"], 1, 0, 8192, 8192, 8192, 1.0, extra["ha"], 8192, extra["hb"], 8192,
+                        0.0, extra["hc"], 8192, stream=s)
+        elif name == "bias_add_broadcast":
             G.case_shaping(0, extra["out4"], dev["X2a"], extra["bias"], 64, 256, 56, 56, s)
         elif name == "swapaxis10_reshape":
             G.case_shaping(2, extra["out4"], dev["X2a"], extra["bias"], 64, 256, 56, 56, s)
@@ -261,6 +282,10 @@ def main():
         per_op.append({"op": name, "ms": round(float(ms.mean()), 4), "ms_min": round(float(ms.min()), 4),
                        "GBps": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
                        "GElemps": round(elems[name] * scale_fix / (ms.mean() * 1e-3) / 1e9, 2)})
+        if name in PRODUCT_FLOPS:
+            flops, peak = PRODUCT_FLOPS[name]
+            per_op[-1]["TFLOPps"] = round(flops / (ms.mean() * 1e-3) / 1e12, 1)
+            per_op[-1]["frac_of_mfma_peak"] = round(per_op[-1]["TFLOPps"] / peak, 4)
     step_ms = wall / args.steps * 1e3
     total_bytes = sum(abytes[n] for n in only) * scale_fix
     value = total_bytes / (step_ms * 1e-3) / 1e9

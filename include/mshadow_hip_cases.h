@@ -97,6 +97,14 @@ int mshadow_case_extensions_f32(int op, float *out, const float *a, const float 
 int mshadow_case_dot_f32(int op, float *out, const float *a, const float *b, int m, int k, int n,
                          int batch, void *stream);
 
+/* a two-layer perceptron trained for `steps` full-batch updates on the device
+   (cases/two_layer_net.h): x (batch, n_in), label (batch), w1 (n_in, n_hidden) and w2
+   (n_hidden, n_out) in / out, probs (batch, n_out) out. Unlike the other cases every pointer
+   is HOST memory: the program moves its data itself, and returns when the device is done */
+int mshadow_case_two_layer_net_f32(int steps, float eta, float decay, int batch, int n_in,
+                                   int n_hidden, int n_out, const float *x, const float *label,
+                                   float *w1, float *w2, float *probs, void *stream);
+
 /* dst = pool<Reducer>(src, Shape2(ph, pw), ky, kx, sy, sx) */
 int mshadow_case_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes,
                           int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,

@@ -12,6 +12,7 @@
 #include <string>
 
 #include "portable_math.h"
+#include "two_layer_net.h"
 
 using namespace mshadow;
 using namespace mshadow::expr;
@@ -379,6 +380,22 @@ int mshadow_case_dot_f32(int op, float *out, const float *a, const float *b, int
 #undef V2
 #undef V2S
 #undef V3
+  CASE_END
+}
+
+/* two_layer_net::Train on the device; every pointer is HOST memory (the program copies) */
+int mshadow_case_two_layer_net_f32(int steps, float eta, float decay, int batch, int n_in,
+                                   int n_hidden, int n_out, const float *x, const float *label,
+                                   float *w1, float *w2, float *probs, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  two_layer_net::Train<gpu>(
+      st.get(), steps, eta, decay,
+      Tensor<cpu, 2, float>(const_cast<float *>(x), Shape2(batch, n_in)),
+      Tensor<cpu, 1, float>(const_cast<float *>(label), Shape1(batch)),
+      Tensor<cpu, 2, float>(w1, Shape2(n_in, n_hidden)),
+      Tensor<cpu, 2, float>(w2, Shape2(n_hidden, n_out)),
+      Tensor<cpu, 2, float>(probs, Shape2(batch, n_out)));
   CASE_END
 }
 

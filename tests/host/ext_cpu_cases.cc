@@ -5,6 +5,7 @@
 #include <mshadow/random.h>
 
 #include "../../mshadow_amd/cases/portable_math.h"
+#include "../../mshadow_amd/cases/two_layer_net.h"
 
 using namespace mshadow;
 using namespace mshadow::expr;
@@ -80,6 +81,20 @@ extern "C" int host_dot_f32(int op, float *out, const float *a, const float *b, 
 #undef V2
 #undef V2S
 #undef V3
+  } catch (const std::exception &e) {
+    fprintf(stderr, "%s\n", e.what());
+    return 1;
+  }
+  return 0;
+}
+
+extern "C" int host_two_layer_net_f32(int steps, float eta, float decay, int batch, int n_in,
+                                      int n_hidden, int n_out, const float *x, const float *label,
+                                      float *w1, float *w2, float *probs) {
+  try {
+    two_layer_net::Train<cpu>(NULL, steps, eta, decay, View(x, Shape2(batch, n_in)),
+                              View(label, Shape1(batch)), View(w1, Shape2(n_in, n_hidden)),
+                              View(w2, Shape2(n_hidden, n_out)), View(probs, Shape2(batch, n_out)));
   } catch (const std::exception &e) {
     fprintf(stderr, "%s\n", e.what());
     return 1;

@@ -138,6 +138,66 @@ def test_products_of_the_compiled_reference(ref, host_lib, op, dims):
     close(mine, out.astype(np.float64).reshape(want.shape), f"host vs reference op {op} {dims}")
 
 
+# ----------------------------------------------------------------- a whole caller program
+def two_layer_model(steps, eta, decay, x, label, w1, w2):
+    """cases/two_layer_net.h in float64"""
+    x, w1, w2 = x.astype(np.float64), w1.astype(np.float64), w2.astype(np.float64)
+    batch = x.shape[0]
+    b1, b2 = np.zeros(w1.shape[1]), np.zeros(w2.shape[1])
+    onehot = np.zeros((batch, w2.shape[1]))
+    onehot[np.arange(batch), label.astype(int)] = 1
+    losses = []
+    for _ in range(steps):
+        act = sigmoid(x @ w1 + b1)
+        z = act @ w2 + b2
+        e = np.exp(z - z.max(axis=1, keepdims=True))
+        p = e / e.sum(axis=1, keepdims=True)
+        losses.append(float(-np.log(p[np.arange(batch), label.astype(int)]).mean()))
+        g = (p - onehot) / batch
+        gb2, gw2 = g.sum(axis=0), act.T @ g
+        ga = act * (1 - act) * (g @ w2.T)
+        gb1, gw1 = ga.sum(axis=0), x.T @ ga
+        w1 -= eta * (decay * w1 + gw1)
+        w2 -= eta * (decay * w2 + gw2)
+        b1 -= eta * gb1
+        b2 -= eta * gb2
+    return w1, w2, p, losses
+
+
+def two_layer_problem():
+    rng = np.random.default_rng(21)
+    batch, n_in, n_hidden, n_out = 96, 50, 40, 10
+    centres = rng.standard_normal((n_out, n_in))
+    label = rng.integers(0, n_out, batch)
+    x = (centres[label] + 0.3 * rng.standard_normal((batch, n_in))).astype(f32)
+    w1 = (0.1 * rng.standard_normal((n_in, n_hidden))).astype(f32)
+    w2 = (0.1 * rng.standard_normal((n_hidden, n_out))).astype(f32)
+    return x, label.astype(f32), w1, w2
+
+
+def check_two_layer(run, what):
+    steps, eta, decay = 30, 0.8, 1e-5
+    x, label, w1, w2 = two_layer_problem()
+    mw1, mw2, mp, losses = two_layer_model(steps, eta, decay, x, label, w1, w2)
+    assert losses[-1] < 0.5 * losses[0], "the model problem does not train"
+    probs = np.full(mp.shape, np.nan, f32)
+    run(steps, eta, decay, x, label, w1, w2, probs)
+    close(w1, mw1, what + " w1", 1e-4)
+    close(w2, mw2, what + " w2", 1e-4)
+    close(probs, mp, what + " probabilities", 1e-4)
+
+
+def test_two_layer_net_on_the_host(host_lib):
+    fl, ip = ctypes.c_float, ctypes.c_int
+    host_lib.host_two_layer_net_f32.argtypes = [ip, fl, fl, ip, ip, ip, ip] + [ctypes.c_void_p] * 5
+
+    def run(steps, eta, decay, x, label, w1, w2, probs):
+        assert host_lib.host_two_layer_net_f32(steps, eta, decay, x.shape[0], x.shape[1], w1.shape[1],
+                                               w2.shape[1], _ptr(x), _ptr(label), _ptr(w1), _ptr(w2),
+                                               _ptr(probs)) == 0
+    check_two_layer(run, "host")
+
+
 # ----------------------------------------------------------------- the reference's own programs, host
 def _run(name, *args):
     exe = os.path.join(DROPIN, name)
@@ -201,9 +261,12 @@ def test_unknown_case_is_an_error_on_the_device_too(G):
         G.case_dot(99, buf, buf, buf, 1, 1, 1)
 
 
-def _colmajor(x):
-    """bytes of a matrix in column-major order, as a flat array"""
-    return np.ascontiguousarray(x.T).reshape(-1)
+@pytest.mark.gpu
+def test_two_layer_net_on_the_device(G):
+    """Copy in, 30 updates of dot / repmat / F<> / Softmax / SoftmaxGrad / sum_rows / scaled
+    saves on one stream, Copy out: the float64 model's weights and probabilities to 1e-4"""
+    s = G.stream_create()
+    check_two_layer(lambda *a: G.case_two_layer_net(*a, stream=s), "device")
 
 
 @pytest.mark.gpu

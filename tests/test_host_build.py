@@ -68,6 +68,46 @@ def test_expression_routes_reach_the_fixed_function_entries():
     assert wanted <= imported, sorted(wanted - imported)
 
 
+def _symbols(path):
+    out = subprocess.run(["readelf", "-Ws", "--wide", path], check=True, capture_output=True, text=True).stdout
+    return [line.split()[-1] for line in out.splitlines() if " FUNC " in line or " OBJECT " in line]
+
+
+@pytest.mark.parametrize("libname", ["libmshadow_hip.so", "libmshadow_cases.so"])
+def test_host_and_device_halves_of_a_library_come_from_the_same_sources(libname, tmp_path):
+    """hipcc compiles a file twice, once per side; a source edited between the two passes
+    leaves launch stubs in the host code whose kernels are not in the gfx950 code object, and
+    the first such launch ends the process. Every stub must find its kernel."""
+    bundler = "/opt/rocm/llvm/bin/clang-offload-bundler"
+    if not os.path.exists(bundler):
+        pytest.skip("clang-offload-bundler not installed")
+    _lib(libname)
+    so = os.path.join(LIBDIR, libname)
+    fat = str(tmp_path / "fat.bin")
+    subprocess.run(["objcopy", "-O", "binary", "--only-section=.hip_fatbin", so, fat], check=True)
+    # one bundle per source file of the library, back to back in the section
+    magic = b"__CLANG_OFFLOAD_BUNDLE__"
+    blob = open(fat, "rb").read()
+    starts = [m.start() for m in re.finditer(re.escape(magic), blob)]
+    assert starts, "no device code in " + libname
+    kernels = set()
+    for i, at in enumerate(starts):
+        part, dev = str(tmp_path / f"bundle{i}.bin"), str(tmp_path / f"dev{i}.co")
+        with open(part, "wb") as f:
+            f.write(blob[at:starts[i + 1] if i + 1 < len(starts) else len(blob)])
+        subprocess.run([bundler, "--unbundle", "--type=o", f"--input={part}", f"--output={dev}",
+                        "--targets=hipv4-amdgcn-amd-amdhsa--gfx950"], check=True)
+        kernels.update(_symbols(dev))
+
+    def kernel_of(stub):
+        # <len>__device_stub__<name> -> <len - 15><name>
+        return re.sub(r"(\d+)__device_stub__", lambda m: str(int(m.group(1)) - 15), stub, count=1)
+    stubs = [n for n in _symbols(so) if "__device_stub__" in n]
+    assert len(stubs) > 100
+    missing = [n for n in stubs if kernel_of(n) not in kernels]
+    assert not missing, (len(missing), missing[:3])
+
+
 def _compile_and_run(tmp_path, source, extra):
     exe = str(tmp_path / "check")
     cmd = ["g++", "-std=c++17", "-O2", "-fopenmp", "-ffp-contract=off", "-mf16c",
