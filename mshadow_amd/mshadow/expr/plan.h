@@ -169,6 +169,19 @@ class Plan<ScalarExp<DType>, DType> {
   DType scalar_;
 };
 
+/*! \brief rows of one plane of the destination when somewhere in the plan a window runs
+ *  over neighbouring planes (channel pooling), 0 otherwise: the launcher then hands each
+ *  thread packs of adjacent planes, so that a window's fetches are mostly repeats of the
+ *  thread's own. Plans say so with a PlaneRows() member; any plan may go without. */
+template <typename P>
+inline auto PlaneRowsOf(const P &plan, int) -> decltype(plan.PlaneRows()) {
+  return plan.PlaneRows();
+}
+template <typename P>
+inline index_t PlaneRowsOf(const P &, long) {
+  return 0;
+}
+
 /* ---- interior nodes ---- */
 template <typename DstDType, typename SrcDType, typename EType, int etype>
 class Plan<TypecastExp<DstDType, SrcDType, EType, etype>, DstDType> {
@@ -192,7 +205,44 @@ struct Packable {
   static long Test(...);  // NOLINT(*)
   static const bool value = sizeof(Test<P>(0)) == sizeof(char);
 };
+/*! \brief P::kPlaneWindow if the plan type declares it, false otherwise: somewhere in the
+ *  plan a window runs over neighbouring planes, and the plan has EvalPackRun */
+template <typename P>
+struct PlaneWindow {
+  template <typename Q>
+  static char Test(int (*)[Q::kPlaneWindow ? 1 : -1]);
+  template <typename Q>
+  static long Test(...);  // NOLINT(*)
+  static const bool value = sizeof(Test<P>(0)) == sizeof(char);
+};
+template <bool kWindow>
+struct RunOf {
+  template <int N, bool STREAM, int K, typename P, typename DType>
+  MSHADOW_XINLINE static void Eval(const P &plan, index_t y0, index_t dy, index_t x,
+                                   Pack<DType, N> *out) {
+#pragma unroll
+    for (int u = 0; u < K; ++u) out[u] = plan.template EvalPack<N, STREAM>(y0 + u * dy, x);
+  }
+};
+template <>
+struct RunOf<true> {
+  template <int N, bool STREAM, int K, typename P, typename DType>
+  MSHADOW_XINLINE static void Eval(const P &plan, index_t y0, index_t dy, index_t x,
+                                   Pack<DType, N> *out) {
+    plan.template EvalPackRun<N, STREAM, K>(y0, dy, x, out);
+  }
+};
 }  // namespace plan_detail
+
+/*! \brief out[u] = plan.EvalPack(y0 + u * dy, x) for u < K: the same place of K planes that
+ *  are dy rows apart. A plan with a window over planes shares the fetches of overlapping
+ *  windows (its EvalPackRun); every other plan evaluates the K packs one by one. */
+template <int N, bool STREAM, int K, typename P, typename DType>
+MSHADOW_XINLINE void EvalPackRun(const P &plan, index_t y0, index_t dy, index_t x,
+                                 Pack<DType, N> *out) {
+  plan_detail::RunOf<plan_detail::PlaneWindow<P>::value>::template Eval<N, STREAM, K>(plan, y0, dy,
+                                                                                      x, out);
+}
 
 template <typename OP, typename TA, typename TB, typename TC, int etype, typename DType>
 class Plan<TernaryMapExp<OP, TA, TB, TC, DType, etype>, DType> {
@@ -248,6 +298,23 @@ class Plan<BinaryMapExp<OP, TA, TB, DType, etype>, DType> {
   inline bool PackReady(int n, index_t cols, bool *flat) const {
     return lhs_.PackReady(n, cols, flat) && rhs_.PackReady(n, cols, flat);
   }
+  inline index_t PlaneRows() const {
+    const index_t l = PlaneRowsOf(lhs_, 0);
+    return l != 0 ? l : PlaneRowsOf(rhs_, 0);
+  }
+  static const bool kPlaneWindow = plan_detail::PlaneWindow<Plan<TA, DType> >::value ||
+                                   plan_detail::PlaneWindow<Plan<TB, DType> >::value;
+  template <int N, bool STREAM, int K>
+  MSHADOW_XINLINE void EvalPackRun(index_t y0, index_t dy, index_t x, Pack<DType, N> *out) const {
+    Pack<DType, N> a[K], b[K];
+    expr::EvalPackRun<N, STREAM, K>(lhs_, y0, dy, x, a);
+    expr::EvalPackRun<N, STREAM, K>(rhs_, y0, dy, x, b);
+#pragma unroll
+    for (int u = 0; u < K; ++u) {
+#pragma unroll
+      for (int i = 0; i < N; ++i) out[u].v[i] = OP::Map(a[u].v[i], b[u].v[i]);
+    }
+  }
 
  private:
   Plan<TA, DType> lhs_;
@@ -271,6 +338,17 @@ class Plan<UnaryMapExp<OP, TA, DType, etype>, DType> {
   inline bool PackReady(int n, index_t cols, bool *flat) const {
     return src_.PackReady(n, cols, flat);
   }
+  inline index_t PlaneRows() const { return PlaneRowsOf(src_, 0); }
+  static const bool kPlaneWindow = plan_detail::PlaneWindow<Plan<TA, DType> >::value;
+  template <int N, bool STREAM, int K>
+  MSHADOW_XINLINE void EvalPackRun(index_t y0, index_t dy, index_t x, Pack<DType, N> *out) const {
+    expr::EvalPackRun<N, STREAM, K>(src_, y0, dy, x, out);
+#pragma unroll
+    for (int u = 0; u < K; ++u) {
+#pragma unroll
+      for (int i = 0; i < N; ++i) out[u].v[i] = OP::Map(out[u].v[i]);
+    }
+  }
 
  private:
   Plan<TA, DType> src_;
@@ -291,6 +369,12 @@ struct Plan<MakeTensorExp<SubType, SrcExp, dim, DType>, DType> {
   }
   inline bool PackReady(int n, index_t cols, bool *flat) const {
     return src_.PackReady(n, cols, flat);
+  }
+  inline index_t PlaneRows() const { return PlaneRowsOf(src_, 0); }
+  static const bool kPlaneWindow = plan_detail::PlaneWindow<Plan<SubType, DType> >::value;
+  template <int N, bool STREAM, int K>
+  MSHADOW_XINLINE void EvalPackRun(index_t y0, index_t dy, index_t x, Pack<DType, N> *out) const {
+    expr::EvalPackRun<N, STREAM, K>(src_, y0, dy, x, out);
   }
 
  private:

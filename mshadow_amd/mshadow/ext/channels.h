@@ -141,8 +141,58 @@ struct Plan<ChannelPoolingExp<Reducer, SrcExp, DType, srcdim>, DType> {
     bool ignored = true;
     return src_.PackReady(n, cols, &ignored);
   }
+  /*! \brief windows of neighbouring pooled channels overlap in all but `stride` planes */
+  inline index_t PlaneRows() const { return nsize_ > stride_ ? height_.div : 0; }
+  static const bool kPlaneWindow = kPackable;
+  /*! \brief the same place (y, j) of K planes dy rows apart, starting at row i0. When these
+   *  are K consecutive pooled channels of one image with windows one channel apart, the
+   *  K + nsize - 1 source channels under them are fetched once and every window is reduced
+   *  from registers, in channel order as always. */
+  template <int N, bool STREAM, int K>
+  MSHADOW_XINLINE void EvalPackRun(index_t i0, index_t dy, index_t j, Pack<DType, N> *out) const {
+    const index_t plane = height_.Div(i0);
+    const index_t y = i0 - plane * height_.div;
+    const index_t n = channel_.Div(plane);
+    const index_t c0 = plane - n * channel_.div;
+    if (dy == height_.div && stride_ == 1 && c0 + K <= channel_.div) {
+      if (nsize_ == 5) return SharedWindows<5, N, K>(n, c0, y, j, out);
+      if (nsize_ == 3) return SharedWindows<3, N, K>(n, c0, y, j, out);
+    }
+#pragma unroll
+    for (int u = 0; u < K; ++u) out[u] = this->template EvalPack<N, STREAM>(i0 + u * dy, j);
+  }
 
  private:
+  template <int W, int N, int K>
+  MSHADOW_XINLINE void SharedWindows(index_t n, index_t c0, index_t y, index_t j,
+                                     Pack<DType, N> *out) const {
+    const index_t step = height_.div;
+    const index_t start = c0 - pad_;  // may be negative: those positions are skipped
+    const index_t limit = channel_.div < src_channel_ ? channel_.div : src_channel_;
+    Pack<DType, N> v[K + W - 1];
+    bool inside[K + W - 1];
+#pragma unroll
+    for (int k = 0; k < K + W - 1; ++k) {
+      const index_t cc = start + k;
+      inside[k] = cc >= 0 && cc < limit;
+      const index_t safe = inside[k] ? cc : 0;
+      v[k] = src_.template EvalPack<N, false>((n * src_channel_ + safe) * step + y, j);
+    }
+#pragma unroll
+    for (int u = 0; u < K; ++u) {
+#pragma unroll
+      for (int e = 0; e < N; ++e) Reducer::SetInitValue(out[u].v[e]);
+#pragma unroll
+      for (int k = 0; k < W; ++k) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) {
+          DType with = out[u].v[e];
+          Reducer::Reduce(with, v[u + k].v[e]);
+          out[u].v[e] = inside[u + k] ? with : out[u].v[e];
+        }
+      }
+    }
+  }
   /*! \brief a window of K channels starting at c * stride - pad and ending before `last`:
    *  every position is fetched (a position outside the window re-reads the pooled channel's
    *  own row index clamped into the source, and is not reduced), then reduced in channel order */

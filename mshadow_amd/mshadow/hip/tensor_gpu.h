@@ -567,6 +567,35 @@ struct MapLauncher {
     }
   }
 };
+/*! \brief plans with a window over neighbouring planes (channel pooling) walk the planes
+ *  kUnroll at a time when the rows divide into planes; false = not launched */
+template <typename Saver, typename DType, int N, int kUnroll, typename DPlan, typename SPlan,
+          bool kWindow>
+struct PlanesLauncher {
+  inline static bool Run(DPlan, SPlan, uint32_t, uint32_t, bool, void *) { return false; }
+};
+template <typename Saver, typename DType, int N, int kUnroll, typename DPlan, typename SPlan>
+struct PlanesLauncher<Saver, DType, N, kUnroll, DPlan, SPlan, true> {
+  inline static bool Run(DPlan dplan, SPlan splan, uint32_t rows, uint32_t ppr, bool stream_hint,
+                         void *stream) {
+    uint32_t plane_rows = static_cast<uint32_t>(splan.PlaneRows());
+    if (plane_rows == 0 || rows % plane_rows != 0 || rows / plane_rows < 2) return false;
+    const uint32_t planes = rows / plane_rows, plane_packs = plane_rows * ppr;
+    const uint32_t places = (planes + kUnroll - 1) / kUnroll * plane_packs;
+    const uint32_t grid = (places + hip::kMapBlock - 1) / hip::kMapBlock;
+    uint32_t total = rows * ppr;
+    FastDivU32 div_ppr(ppr), div_plane_packs(plane_packs);
+    void *args[] = {&dplan, &splan, &total, &ppr, &div_ppr, &plane_rows, &div_plane_packs};
+    if (stream_hint) {
+      Launch(hip::MapPackPlanesKernel<Saver, DType, N, true, kUnroll, DPlan, SPlan>, grid,
+             hip::kMapBlock, args, stream);
+    } else {
+      Launch(hip::MapPackPlanesKernel<Saver, DType, N, false, kUnroll, DPlan, SPlan>, grid,
+             hip::kMapBlock, args, stream);
+    }
+    return true;
+  }
+};
 template <typename Saver, typename DType, typename DPlan, typename SPlan>
 struct MapLauncher<Saver, DType, DPlan, SPlan, true> {
   inline static void Run(DPlan dplan, SPlan splan, Shape<2> shape, void *stream) {
@@ -592,6 +621,12 @@ struct MapLauncher<Saver, DType, DPlan, SPlan, true> {
     /* streaming (non-temporal) accesses once a tensor no longer fits the caches anyway */
     const bool stream_hint = static_cast<size_t>(rows) * cols * sizeof(DType) >= (8u << 20);
     const bool is_flat = flat || rows == 1;
+    if (!is_flat &&
+        PlanesLauncher<Saver, DType, N, kUnroll, DPlan, SPlan,
+                       expr::plan_detail::PlaneWindow<SPlan>::value>::Run(dplan, splan, rows, ppr,
+                                                                          stream_hint, stream)) {
+      return;
+    }
 #define MSHADOW_MAP_LAUNCH(FLAT, STREAM)                                                   \
   Launch(hip::MapPackKernel<Saver, DType, N, FLAT, STREAM, kUnroll, DPlan, SPlan>, grid,   \
          hip::kMapBlock, args, stream)

@@ -333,6 +333,46 @@ def test_gpu_matches_numpy(shape, op):
     assert np.array_equal(got.view(np.uint32), case.want.view(np.uint32)), (op, shape)
 
 
+# channel windows where a thread of the plane-walking kernel evaluates 8 adjacent planes at once:
+# channel counts above, at and below 8, not multiples of 8 (a group of planes that crosses into
+# the next image, a short last group), windows of 3 and 5 (fetches shared in registers) and 7
+WINDOW_SHAPES = [(3, 20, 4, 8), (2, 16, 5, 12), (1, 9, 2, 4), (2, 8, 3, 4), (5, 3, 2, 4), (1, 64, 7, 28),
+                 (2, 24, 1, 4), (3, 11, 3, 5)]
+
+
+# the nodes refuse a window wider than the channel count, like the reference (channel_pool.h:39)
+WINDOW_CASES = [(shape, nsize) for shape in WINDOW_SHAPES for nsize in (3, 5, 7) if nsize <= shape[1]]
+
+
+def _window_case(shape, nsize, op):
+    rng = np.random.default_rng(nsize * 100 + op + sum(shape))
+    a = rng.standard_normal(shape).astype(f32)
+    pooled = _chpool(a if op == 0 else a * a, nsize, 1, nsize // 2, "sum")
+    return a, pooled if op == 0 else a * (pooled * f32(0.1) + f32(1))
+
+
+@pytest.mark.parametrize("shape,nsize", WINDOW_CASES)
+@pytest.mark.parametrize("op", [0, 19])
+def test_channel_windows_on_host_tensors(host_lib, shape, nsize, op):
+    a, want = _window_case(shape, nsize, op)
+    out = np.full(want.shape, np.nan, f32)
+    assert host_lib.host_extensions_f32(op, _ptr(out), _ptr(a), None, None, *shape, nsize, 0, 0) == 0
+    assert np.array_equal(out.view(np.uint32), want.view(np.uint32)), (op, shape, nsize)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape,nsize", WINDOW_CASES)
+@pytest.mark.parametrize("op", [0, 19])
+def test_channel_windows_across_groups_of_planes(shape, nsize, op):
+    import mshadow_amd
+    G = mshadow_amd.load_cases()
+    G.set_device(0)
+    a, want = _window_case(shape, nsize, op)
+    out = G.to_device(np.full(want.shape, np.nan, f32))
+    G.case_extensions(op, out, G.to_device(a), None, None, *shape, nsize, 0, 0)
+    assert np.array_equal(out.download().view(np.uint32), want.view(np.uint32)), (op, shape, nsize)
+
+
 PERMUTE_CASES = [
     ((5, 7), (1, 0)), ((64, 64), (1, 0)), ((65, 130), (1, 0)), ((1, 9), (1, 0)),
     ((3, 4, 5), (2, 1, 0)), ((3, 4, 5), (1, 0, 2)), ((3, 4, 5), (0, 2, 1)), ((3, 4, 5), (2, 0, 1)),
