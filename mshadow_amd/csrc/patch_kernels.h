@@ -73,15 +73,27 @@ struct PatchTile {
   int pitch;      // im2col: LDS elements per staged input row; col2im: per staged tap
 };
 
+/*! \brief which (image, channel, band) a workgroup works on: bands fastest, then images, then
+ *  channels. A row of the column matrix holds one tap of one channel for all images one after
+ *  the other, so workgroups that run at the same time write (or read) neighbouring stretches
+ *  of the same few rows instead of one stretch in each of thousands of rows; measured on the
+ *  (32,256,56,56) binary16 case, channels fastest against images fastest: im2col 99 -> 91 us. */
+__device__ __forceinline__ void PlaneOfBlock(const PatchGeom &g, const PatchTile &t, int *n, int *ch,
+                                             int *band) {
+  const int seq = blockIdx.x / t.bands;
+  *band = blockIdx.x - seq * t.bands;
+  *ch = seq / g.n;
+  *n = seq - *ch * g.n;
+}
+
 template <typename T, int EPT>
 __global__ void __launch_bounds__(kPatchBlock)
     Im2ColTiledKernel(T *col, int cstride, const T *img, int istride, PatchGeom g, PatchTile t) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   T *lds = reinterpret_cast<T *>(smem_raw);
-  const int plane = blockIdx.x / t.bands;      // n * c + ch
-  const int band = blockIdx.x - plane * t.bands;
-  const int ch = plane % g.c;
-  const int n = plane / g.c;
+  int n, ch, band;
+  PlaneOfBlock(g, t, &n, &ch, &band);
+  const int plane = n * g.c + ch;
   const int oy0 = band * t.band;
   const int noy = min(t.band, g.oh - oy0);
   const int iy0 = oy0 * g.sy;                  // first padded input row of the band
@@ -166,10 +178,9 @@ __global__ void __launch_bounds__(kPatchBlock)
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   typedef uint16_t T;
   T *lds = reinterpret_cast<T *>(smem_raw);
-  const int plane = blockIdx.x / t.bands;
-  const int band = blockIdx.x - plane * t.bands;
-  const int ch = plane % g.c;
-  const int n = plane / g.c;
+  int n, ch, band;
+  PlaneOfBlock(g, t, &n, &ch, &band);
+  const int plane = n * g.c + ch;
   const int oy0 = band * t.band;
   const int noy = min(t.band, g.oh - oy0);
   const int in_rows = noy + g.ky - 1;
@@ -225,10 +236,9 @@ __global__ void __launch_bounds__(kPatchBlock)
   if (FAST) {
     g.sy = g.sx = g.dy = g.dx = 1;
   }
-  const int plane = blockIdx.x / t.bands;
-  const int band = blockIdx.x - plane * t.bands;
-  const int ch = plane % g.c;
-  const int n = plane / g.c;
+  int n, ch, band;
+  PlaneOfBlock(g, t, &n, &ch, &band);
+  const int plane = n * g.c + ch;
   const int cy0 = band * t.band;
   const int ncy = min(t.band, g.h - cy0);
   const int span_y = g.dy * (g.ky - 1) + 1;
@@ -302,10 +312,9 @@ __global__ void __launch_bounds__(kPatchBlock)
   const int EPT = 8;
   const int TAPS = KY * KX;
   T *lds = reinterpret_cast<T *>(smem_raw);
-  const int plane = blockIdx.x / t.bands;
-  const int band = blockIdx.x - plane * t.bands;
-  const int ch = plane % g.c;
-  const int n = plane / g.c;
+  int n, ch, band;
+  PlaneOfBlock(g, t, &n, &ch, &band);
+  const int plane = n * g.c + ch;
   const int cy0 = band * t.band;
   const int ncy = min(t.band, g.h - cy0);
   const int yf = cy0 + g.pad_y, yl = cy0 + ncy - 1 + g.pad_y;
