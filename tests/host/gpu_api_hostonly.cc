@@ -79,12 +79,43 @@ int main() {
   for (index_t y = 0; y < ct2.size(0); ++y)
     for (index_t x2 = 0; x2 < ct2.size(1); ++x2) bad_transpose += ct2[y][x2] != again2[y][x2];
   FreeSpace(&t2);
+  /* matrix products are library calls behind the ABI: (3x5 of i+j) x (4x5 of i-j)^T, and the
+     scalar product of two of the rows, in small integers (exact in float) */
+  int bad_dot = 0;
+  {
+    TensorContainer<cpu, 2> ha(Shape2(3, 5)), hb(Shape2(4, 5)), hc(Shape2(3, 4));
+    TensorContainer<cpu, 1> hd(Shape1(1));
+    for (index_t i = 0; i < 3; ++i) for (index_t j = 0; j < 5; ++j) ha[i][j] = static_cast<float>(i + j);
+    for (index_t i = 0; i < 4; ++i) for (index_t j = 0; j < 5; ++j) hb[i][j] = static_cast<float>(i) - j;
+    TensorContainer<gpu, 2> da(ha.shape_), db(hb.shape_), dc(hc.shape_);
+    TensorContainer<gpu, 1> dd(Shape1(1));
+    da.set_stream(s), db.set_stream(s), dc.set_stream(s), dd.set_stream(s);
+    Copy(da, ha, s);
+    Copy(db, hb, s);
+    dc = 1.0f;
+    dc += 2.0f * dot(da, db.T());
+    VectorDot(dd, da[2], db[3]);
+    Copy(hc, dc, s);
+    Copy(hd, dd, s);
+    s->Wait();
+    float vd = 0.0f;
+    for (index_t j = 0; j < 5; ++j) vd += ha[2][j] * hb[3][j];
+    bad_dot += hd[0] != vd;
+    for (index_t i = 0; i < 3; ++i) {
+      for (index_t k = 0; k < 4; ++k) {
+        float want = 0.0f;
+        for (index_t j = 0; j < 5; ++j) want += ha[i][j] * hb[k][j];
+        bad_dot += hc[i][k] != 1.0f + 2.0f * want;
+      }
+    }
+  }
   FreeSpace(&x); FreeSpace(&p); FreeSpace(&g); FreeSpace(&t); FreeSpace(&m); FreeSpace(&v);
-  bad = bad_pool + bad_transpose + bad_sum;
+  bad = bad_pool + bad_transpose + bad_sum + bad_dot;
   DeleteStream(s);
   ShutdownTensorEngine<gpu>();
   if (bad) {
-    printf("values that differ: pool %d, transpose %d, sum_rows %d\n", bad_pool, bad_transpose, bad_sum);
+    printf("values that differ: pool %d, transpose %d, sum_rows %d, dot %d\n", bad_pool, bad_transpose,
+           bad_sum, bad_dot);
     return 1;
   }
   printf("OK\n");
