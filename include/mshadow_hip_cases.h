@@ -97,6 +97,9 @@ int mshadow_case_extensions_f32(int op, float *out, const float *a, const float 
 int mshadow_case_dot_f32(int op, float *out, const float *a, const float *b, int m, int k, int n,
                          int batch, void *stream);
 
+/* out = x * x + x over a Tensor<gpu, 1, half2_t> of n_pairs elements (2 * n_pairs binary16 values) */
+int mshadow_case_half2_map(uint16_t *out, const uint16_t *x, int n_pairs, void *stream);
+
 /* a two-layer perceptron trained for `steps` full-batch updates on the device
    (cases/two_layer_net.h): x (batch, n_in), label (batch), w1 (n_in, n_hidden) and w2
    (n_hidden, n_out) in / out, probs (batch, n_out) out. Unlike the other cases every pointer

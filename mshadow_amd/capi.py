@@ -110,6 +110,7 @@ CASES_SYMBOLS = {
     "mshadow_case_sort_by_key_32": ([_i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_case_extensions_f32": ([_i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p], _i),
     "mshadow_case_dot_f32": ([_i, _p, _p, _p, _i, _i, _i, _i, _p], _i),
+    "mshadow_case_half2_map": ([_p, _p, _i, _p], _i),
     "mshadow_case_two_layer_net_f32": ([_i, _f, _f, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p], _i),
     "mshadow_case_softmax_grad_f32": ([_p, _i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_case_pool_f32": ([_p, _i, _p, _i] + [_i] * 11 + [_p], _i),
@@ -458,6 +459,9 @@ class Library:
 
     def case_dot(self, op, out, a, b, m, k, n, batch=1, stream=None):
         self.check_case(self.cases.mshadow_case_dot_f32(op, out.ptr, a.ptr, b.ptr, m, k, n, batch, stream))
+
+    def case_half2_map(self, out, x, stream=None):
+        self.check_case(self.cases.mshadow_case_half2_map(out.ptr, x.ptr, x.cols // 2, stream))
 
     def case_two_layer_net(self, steps, eta, decay, x, label, w1, w2, probs, stream=None):
         """host numpy arrays (float32, contiguous); w1 and w2 are updated in place"""

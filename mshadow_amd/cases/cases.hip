@@ -383,6 +383,17 @@ int mshadow_case_dot_f32(int op, float *out, const float *a, const float *b, int
   CASE_END
 }
 
+/* out = x * x + x over n pairs of binary16 values taken as half2_t elements */
+int mshadow_case_half2_map(uint16_t *out, const uint16_t *x, int n_pairs, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  typedef half::half2_t H2;
+  Tensor<gpu, 1, H2> X = G1(reinterpret_cast<const H2 *>(x), n_pairs, st.get());
+  Tensor<gpu, 1, H2> O = G1(reinterpret_cast<const H2 *>(out), n_pairs, st.get());
+  O = X * X + X;
+  CASE_END
+}
+
 /* two_layer_net::Train on the device; every pointer is HOST memory (the program copies) */
 int mshadow_case_two_layer_net_f32(int steps, float eta, float decay, int batch, int n_in,
                                    int n_hidden, int n_out, const float *x, const float *label,

@@ -16,6 +16,7 @@
 
 #include "./core/config.h"
 #include "./half.h"
+#include "./half2.h"
 #include "./logging.h"
 
 namespace mshadow {
@@ -52,6 +53,12 @@ MSHADOW_DECLARE_DATATYPE(int8_t, kInt8)
 MSHADOW_DECLARE_DATATYPE(int32_t, kInt32)
 MSHADOW_DECLARE_DATATYPE(int64_t, kInt64)
 #undef MSHADOW_DECLARE_DATATYPE
+/*! \brief two binary16 lanes per element (mshadow/base.h:361-365) */
+template <>
+struct DataType<half::half2_t> {
+  static const int kFlag = kFloat16;
+  static const int kLanes = 2;
+};
 /*! \brief type enum value for default real type */
 const int default_type_flag = DataType<default_real_t>::kFlag;
 
@@ -102,6 +109,19 @@ const int default_layout_5d = kNCDHW;
     MSHADOW_SWITCH_CASE_(mshadow::kInt64, int64_t, DType, __VA_ARGS__)             \
     MSHADOW_SWITCH_END_(type)                                                      \
   }
+/*! \brief MSHADOW_TYPE_SWITCH without int8, with binary16 taken two lanes at a time
+ *  (mshadow/base.h:919-959) */
+#define MSHADOW_TYPE_SWITCH_WITH_HALF2(type, DType, ...)                            \
+  switch (type) {                                                                   \
+    MSHADOW_SWITCH_CASE_(mshadow::kFloat32, float, DType, __VA_ARGS__)              \
+    MSHADOW_SWITCH_CASE_(mshadow::kFloat64, double, DType, __VA_ARGS__)             \
+    MSHADOW_SWITCH_CASE_(mshadow::kFloat16, mshadow::half::half2_t, DType, __VA_ARGS__) \
+    MSHADOW_SWITCH_CASE_(mshadow::kUint8, uint8_t, DType, __VA_ARGS__)              \
+    MSHADOW_SWITCH_CASE_(mshadow::kInt32, int32_t, DType, __VA_ARGS__)              \
+    MSHADOW_SWITCH_CASE_(mshadow::kInt64, int64_t, DType, __VA_ARGS__)              \
+    MSHADOW_SWITCH_END_(type)                                                       \
+  }
+
 #define MSHADOW_SGL_DBL_TYPE_SWITCH(type, DType, ...)                   \
   switch (type) {                                                       \
     MSHADOW_SWITCH_CASE_(mshadow::kFloat32, float, DType, __VA_ARGS__)  \

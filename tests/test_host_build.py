@@ -133,6 +133,28 @@ def test_header_api_on_cpu_matches_oracle(tmp_path, orc):
     assert out.startswith("OK"), out
 
 
+def test_half2_on_host_tensors(tmp_path):
+    _lib("libmshadow_hip.so")
+    out = _compile_and_run(tmp_path, "half2_check.cc",
+                           ["-L" + LIBDIR, "-lmshadow_hip", "-Wl,-rpath," + LIBDIR])
+    assert out.startswith("OK"), out
+
+
+@pytest.mark.gpu
+def test_half2_map_on_the_device():
+    """x * x + x over half2_t elements: each lane is half_t arithmetic, rounded after the
+    product and after the sum, which numpy's float16 does too"""
+    import numpy as np
+    import mshadow_amd
+    G = mshadow_amd.load_cases()
+    G.set_device(0)
+    x = np.random.default_rng(8).uniform(-4, 4, 4096 + 6).astype(np.float16)
+    want = (x * x).astype(np.float16) + x
+    out = G.buffer(x.shape, np.uint16)
+    G.case_half2_map(out, G.to_device(x.view(np.uint16)))
+    assert np.array_equal(out.download(), want.astype(np.float16).view(np.uint16))
+
+
 def _build_host_only_caller(tmp_path):
     exe = str(tmp_path / "hostonly")
     cmd = ["g++", "-std=c++17", "-O2", "-fopenmp", "-ffp-contract=off", "-mf16c",
