@@ -141,6 +141,41 @@ const int default_layout_5d = kNCDHW;
       break;                                                                           \
     MSHADOW_SWITCH_END_(type)                                                          \
   }
+/*! \brief floating-point types only, with a second name for the type sums are kept in:
+ *  float for binary16 (mshadow/base.h:1013-1055) */
+#define MSHADOW_REAL_TYPE_SWITCH_EX(type, DType, DLargeType, ...)                           \
+  switch (type) {                                                                           \
+    case mshadow::kFloat32: {                                                               \
+      typedef float DType;                                                                  \
+      typedef float DLargeType;                                                             \
+      { __VA_ARGS__ }                                                                       \
+    } break;                                                                                \
+    case mshadow::kFloat64: {                                                               \
+      typedef double DType;                                                                 \
+      typedef double DLargeType;                                                            \
+      { __VA_ARGS__ }                                                                       \
+    } break;                                                                                \
+    case mshadow::kFloat16: {                                                               \
+      typedef mshadow::half::half_t DType;                                                  \
+      typedef float DLargeType;                                                             \
+      { __VA_ARGS__ }                                                                       \
+    } break;                                                                                \
+    case mshadow::kUint8:                                                                   \
+      LOG(FATAL) << "This operation only support floating point types not uint8";           \
+      break;                                                                                \
+    case mshadow::kInt8:                                                                    \
+      LOG(FATAL) << "This operation only support floating point types not int8";            \
+      break;                                                                                \
+    case mshadow::kInt32:                                                                   \
+      LOG(FATAL) << "This operation only support floating point types, not int32";          \
+      break;                                                                                \
+    case mshadow::kInt64:                                                                   \
+      LOG(FATAL) << "This operation only support floating point types, not int64";          \
+      break;                                                                                \
+    default:                                                                                \
+      LOG(FATAL) << "Unknown type enum " << type;                                           \
+  }
+
 #define MSHADOW_IDX_TYPE_SWITCH(type, DType, ...)                         \
   switch (type) {                                                         \
     MSHADOW_SWITCH_CASE_(mshadow::kInt32, int32_t, DType, __VA_ARGS__)    \

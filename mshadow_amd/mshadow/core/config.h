@@ -4,8 +4,9 @@
  * The macro names callers may set are the reference's (mshadow/base.h:49-158,
  * :192-224): MSHADOW_ALLOC_PAD, MSHADOW_MIN_PAD_RATIO, MSHADOW_FORCE_STREAM,
  * MSHADOW_INT64_TENSOR_SIZE, MSHADOW_DEFAULT_DTYPE. There is one GPU target, so no
- * backend-selection switches exist: a translation unit built by hipcc sees device
- * code, one built by a host compiler sees the host-side API only.
+ * backend-selection switch changes anything here (the reference's are defined for callers
+ * that test them): a translation unit built by hipcc sees device code, one built by a host
+ * compiler sees the host-side API only.
  */
 #ifndef MSHADOW_CORE_CONFIG_H_
 #define MSHADOW_CORE_CONFIG_H_
@@ -28,6 +29,51 @@
 
 /*! \brief the GPU device of this build; kept for callers that test it */
 #define MSHADOW_USE_HIP 1
+
+/* The switches of the reference's base.h (:49-158, :226-231) that callers test with #if. This
+   backend reads none of them; the values say what a caller finds here: Tensor<gpu> exists
+   (MSHADOW_USE_CUDA is the reference's name for that and is 1 there by default too), matrix
+   products need no external host BLAS, and there is no cuDNN, cuSOLVER, NVML or glog. */
+#ifndef MSHADOW_USE_CUDA
+#define MSHADOW_USE_CUDA 1
+#endif
+#ifndef MSHADOW_USE_CUDNN
+#define MSHADOW_USE_CUDNN 0
+#endif
+#ifndef MSHADOW_USE_CUSOLVER
+#define MSHADOW_USE_CUSOLVER 0
+#endif
+#ifndef MSHADOW_USE_CBLAS
+#define MSHADOW_USE_CBLAS 0
+#endif
+#ifndef MSHADOW_USE_MKL
+#define MSHADOW_USE_MKL 0
+#endif
+#ifndef MSHADOW_STAND_ALONE
+#define MSHADOW_STAND_ALONE 0
+#endif
+#ifndef MSHADOW_OLD_CUDA
+#define MSHADOW_OLD_CUDA 0
+#endif
+#ifndef MSHADOW_IN_CXX11
+#define MSHADOW_IN_CXX11 1
+#endif
+#ifndef MSHADOW_USE_SSE
+#define MSHADOW_USE_SSE 0
+#endif
+#ifndef MSHADOW_USE_F16C
+#if defined(__F16C__) && !defined(__HIP_DEVICE_COMPILE__)
+#define MSHADOW_USE_F16C 1  /* half.h converts with the host's F16C instructions */
+#else
+#define MSHADOW_USE_F16C 0
+#endif
+#endif
+#ifndef MSHADOW_USE_NVML
+#define MSHADOW_USE_NVML 0
+#endif
+#ifndef MSHADOW_USE_GLOG
+#define MSHADOW_USE_GLOG 0
+#endif
 
 #ifdef MSHADOW_XINLINE
 #error "MSHADOW_XINLINE must not be defined"

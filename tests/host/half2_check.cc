@@ -19,6 +19,12 @@ int main() {
   int lanes = 0;
   MSHADOW_TYPE_SWITCH_WITH_HALF2(kFloat16, DType, { lanes = DataType<DType>::kLanes; });
   bad += lanes != 2;
+  int large_bytes = 0;
+  MSHADOW_REAL_TYPE_SWITCH_EX(kFloat16, DType, DLarge, { large_bytes = sizeof(DType) * 10 + sizeof(DLarge); });
+  bad += large_bytes != 24;
+#if !MSHADOW_USE_CUDA || MSHADOW_USE_CUDNN || MSHADOW_USE_CBLAS
+  bad += 1;  // the switches callers test: Tensor<gpu> exists, no cuDNN, no external host BLAS
+#endif
 #ifdef __HIPCC__
   Stream<gpu> *s = NewStream<gpu>();
   TensorContainer<gpu, 2, h2> gx(Shape2(3, 4)), gy(Shape2(3, 4));
