@@ -56,6 +56,9 @@ def algorithmic_bytes():
         "lrn_scale_chpool5": 2 * e * 64 * 256 * 56 * 56,
         "transpose_nchw_nhwc": 2 * e * 64 * 256 * 56 * 56,
         "sort_by_key_f32": 4 * e * (1 << 24),
+        # what plain streaming reaches on this machine: a copy and a fill of 8192x32000 floats
+        "ceiling_copy": 2 * e * 8192 * 32000,
+        "ceiling_fill": e * 8192 * 32000,
         "dot_f32_4096": 3 * e * 4096 * 4096,
         "dot_f16_8192": 3 * 2 * 8192 * 8192,
     }
@@ -72,6 +75,7 @@ def work_elements():
         "bias_add_broadcast": 64 * 256 * 56 * 56, "swapaxis10_reshape": 64 * 256 * 56 * 56,
         "lrn_scale_chpool5": 64 * 256 * 56 * 56, "transpose_nchw_nhwc": 64 * 256 * 56 * 56,
         "sort_by_key_f32": 1 << 24, "dot_f32_4096": 4096 * 4096, "dot_f16_8192": 8192 * 8192,
+        "ceiling_copy": 8192 * 32000, "ceiling_fill": 8192 * 32000,
     }
 
 
@@ -82,7 +86,7 @@ PRODUCT_FLOPS = {"dot_f32_4096": (2 * 4096 ** 3, 157.3), "dot_f16_8192": (2 * 81
 
 EXTRA_OPS = ("calib_copy", "smooth_softmax_grad_ignore", "softmax3d", "softmax3d_grad", "add_take_grad",
              "bias_add_broadcast", "swapaxis10_reshape", "lrn_scale_chpool5", "transpose_nchw_nhwc",
-             "sort_by_key_f32", "dot_f32_4096", "dot_f16_8192")
+             "sort_by_key_f32", "dot_f32_4096", "dot_f16_8192", "ceiling_copy", "ceiling_fill")
 OPS = [k for k in algorithmic_bytes() if k not in EXTRA_OPS]
 
 # HBM bytes per launch of each operation's kernel, measured with rocprofv3 --pmc FETCH_SIZE and
@@ -201,7 +205,11 @@ def main():
         extra["f16"] = capi.BLAS_F16
 
     def run_op(name):
-        if name == "dot_f32_4096":
+        if name == "ceiling_copy":     # dst = (src + 0) / 1 + 0 through the expression kernel
+            G.case_map_axpb(out_g, dev["L"], 0.0, 1.0, 0.0, 0, s)
+        elif name == "ceiling_fill":   # dst = scalar
+            G.fill(out_g, 1.0, s)
+        elif name == "dot_f32_4096":
             G.case_dot(1, extra["mm_out"], dev["A"], dev["B"], 4096, 4096, 4096, 1, s)
         elif name == "dot_f16_8192":
             G.blas_gemm(extra["f16"], 1, 0, 8192, 8192, 8192, 1.0, extra["ha"], 8192, extra["hb"], 8192,
