@@ -17,6 +17,9 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 f32 = np.float32
 SHAPES = [(2, 6, 3, 5), (3, 5, 2, 8), (1, 7, 1, 4)]
 BIG = (8, 16, 14, 28)
+# rows of whole 128-bit packs with channel counts around the 8 planes a thread of the
+# plane-walking kernel takes, and an odd height: the pack-evaluating paths of every node
+PACKED = [(2, 12, 5, 12), (4, 9, 7, 16), (1, 33, 2, 4), (3, 8, 4, 20)]
 
 
 # ---- numpy statements of what each node means (mshadow/extension/*.h of the reference)
@@ -296,7 +299,7 @@ def _ptr(x):
     return x.ctypes.data_as(ctypes.c_void_p) if x is not None else None
 
 
-@pytest.mark.parametrize("shape", SHAPES + [BIG])
+@pytest.mark.parametrize("shape", SHAPES + [BIG] + PACKED)
 @pytest.mark.parametrize("op", range(N_OPS))
 def test_cpu_device_matches_numpy(host_lib, shape, op):
     case = Case(op, shape)
@@ -318,7 +321,7 @@ def test_reference_build_matches_numpy(ref, shape, op):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("shape", SHAPES + [BIG])
+@pytest.mark.parametrize("shape", SHAPES + [BIG] + PACKED)
 @pytest.mark.parametrize("op", range(N_OPS))
 def test_gpu_matches_numpy(shape, op):
     import mshadow_amd
