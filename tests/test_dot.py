@@ -364,6 +364,10 @@ def test_abi_rejects_what_would_read_out_of_bounds(G):
         G.blas_ger(capi.BLAS_F32, 2, 2, 1.0, buf, 0, buf, 1, buf, 2)
     # empty problems are accepted and do nothing
     G.blas_gemm(capi.BLAS_F32, 0, 0, 0, 8, 8, 1.0, buf, 1, buf, 8, 0.0, buf, 1)
+    # an empty inner dimension leaves beta * C, as BLAS defines it
+    c = G.to_device(np.arange(6, dtype=f32))
+    G.blas_gemm(capi.BLAS_F32, 0, 0, 2, 3, 0, 1.0, buf, 2, buf, 1, 0.5, c, 2)
+    assert np.array_equal(c.download(), np.arange(6, dtype=f32) * f32(0.5))
 
 
 # ----------------------------------------------------------------- the reference's own programs, device
