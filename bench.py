@@ -57,6 +57,8 @@ def algorithmic_bytes():
         "transpose_nchw_nhwc": 2 * e * 64 * 256 * 56 * 56,
         "sort_by_key_f32": 4 * e * (1 << 24),
         # what plain streaming reaches on this machine: a copy and a fill of 8192x32000 floats
+        "random_uniform": e * 8192 * 32000,
+        "random_normal": e * 8192 * 32000,
         "ceiling_copy": 2 * e * 8192 * 32000,
         "ceiling_fill": e * 8192 * 32000,
         "dot_f32_4096": 3 * e * 4096 * 4096,
@@ -76,6 +78,7 @@ def work_elements():
         "lrn_scale_chpool5": 64 * 256 * 56 * 56, "transpose_nchw_nhwc": 64 * 256 * 56 * 56,
         "sort_by_key_f32": 1 << 24, "dot_f32_4096": 4096 * 4096, "dot_f16_8192": 8192 * 8192,
         "ceiling_copy": 8192 * 32000, "ceiling_fill": 8192 * 32000,
+        "random_uniform": 8192 * 32000, "random_normal": 8192 * 32000,
     }
 
 
@@ -86,7 +89,8 @@ PRODUCT_FLOPS = {"dot_f32_4096": (2 * 4096 ** 3, 157.3), "dot_f16_8192": (2 * 81
 
 EXTRA_OPS = ("calib_copy", "smooth_softmax_grad_ignore", "softmax3d", "softmax3d_grad", "add_take_grad",
              "bias_add_broadcast", "swapaxis10_reshape", "lrn_scale_chpool5", "transpose_nchw_nhwc",
-             "sort_by_key_f32", "dot_f32_4096", "dot_f16_8192", "ceiling_copy", "ceiling_fill")
+             "sort_by_key_f32", "dot_f32_4096", "dot_f16_8192", "ceiling_copy", "ceiling_fill",
+             "random_uniform", "random_normal")
 OPS = [k for k in algorithmic_bytes() if k not in EXTRA_OPS]
 
 # HBM bytes per launch of each operation's kernel, measured with rocprofv3 --pmc FETCH_SIZE and
@@ -207,6 +211,10 @@ def main():
     def run_op(name):
         if name == "ceiling_copy":     # dst = (src + 0) / 1 + 0 through the expression kernel
             G.case_map_axpb(out_g, dev["L"], 0.0, 1.0, 0.0, 0, s)
+        elif name == "random_uniform":  # Random<gpu>::SampleUniform over 8192x32000 floats
+            G.random_uniform(out_g, 7, 0, 0, -1.0, 1.0, s)
+        elif name == "random_normal":   # Random<gpu>::SampleGaussian
+            G.random_normal(out_g, 7, 0, 0, 0.0, 1.0, s)
         elif name == "ceiling_fill":   # dst = scalar
             G.fill(out_g, 1.0, s)
         elif name == "dot_f32_4096":

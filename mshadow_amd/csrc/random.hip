@@ -59,7 +59,9 @@ enum { kWords = 0, kUniform = 1, kNormal = 2 };
 
 /*! \brief element e of the dense (rows, cols) view lands at row e / cols, column e % cols of
  *  a destination whose rows are `stride` elements apart; one thread per four elements */
-template <int KIND>
+/*! \brief PACKS: rows are whole aligned groups of four, so a thread's four values are
+ *  neighbours in one row and leave as one 128-bit streaming store */
+template <int KIND, bool PACKS>
 __global__ void __launch_bounds__(kRandomBlock)
     RandomKernel(uint32_t *dst, uint32_t stride, uint32_t total, uint32_t cols, FastDivU32 div_cols,
                  uint64_t seed, uint64_t subsequence, uint64_t counter, float p0, float p1) {
@@ -84,6 +86,16 @@ __global__ void __launch_bounds__(kRandomBlock)
         out[k + 1] = __float_as_uint(p0 + radius * sn * p1);
       }
     }
+    if (PACKS) {
+      const uint32_t e = b * 4u;
+      const uint32_t y = div_cols.Div(e);
+      typedef uint32_t V4 __attribute__((ext_vector_type(4)));
+      V4 v;
+      v.x = out[0], v.y = out[1], v.z = out[2], v.w = out[3];
+      __builtin_nontemporal_store(
+          v, reinterpret_cast<V4 *>(dst + static_cast<size_t>(y) * stride + (e - y * cols)));
+      continue;
+    }
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const uint32_t e = b * 4u + k;
@@ -106,10 +118,19 @@ int LaunchRandom(void *dst, int dstride, int rows, int cols, uint64_t seed, uint
   if (total >= (1ull << 31)) return mshadow_abi::Fail(MSHADOW_HIP_ERR_ARGUMENT, std::string(what) + ": too many elements");
   uint64_t grid = ((total + 3) / 4 + kRandomBlock - 1) / kRandomBlock;
   if (grid > 16384) grid = 16384;
-  hipLaunchKernelGGL(RandomKernel<KIND>, dim3(static_cast<unsigned>(grid)), dim3(kRandomBlock), 0,
-                     AsStream(stream), static_cast<uint32_t *>(dst), static_cast<uint32_t>(dstride),
-                     static_cast<uint32_t>(total), static_cast<uint32_t>(cols), FastDivU32(cols), seed,
-                     subsequence, counter, p0, p1);
+  const bool packs = cols % 4 == 0 && dstride % 4 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0;
+#define MSHADOW_RANDOM_LAUNCH(PACKS)                                                              \
+  hipLaunchKernelGGL((RandomKernel<KIND, PACKS>), dim3(static_cast<unsigned>(grid)),              \
+                     dim3(kRandomBlock), 0, AsStream(stream), static_cast<uint32_t *>(dst),       \
+                     static_cast<uint32_t>(dstride), static_cast<uint32_t>(total),                \
+                     static_cast<uint32_t>(cols), FastDivU32(cols), seed, subsequence, counter,   \
+                     p0, p1)
+  if (packs) {
+    MSHADOW_RANDOM_LAUNCH(true);
+  } else {
+    MSHADOW_RANDOM_LAUNCH(false);
+  }
+#undef MSHADOW_RANDOM_LAUNCH
   return AfterLaunch(what);
 }
 
