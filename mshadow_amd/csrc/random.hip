@@ -79,9 +79,13 @@ __global__ void __launch_bounds__(kRandomBlock)
     } else {
 #pragma unroll
       for (int k = 0; k < 4; k += 2) {
-        const float radius = __builtin_sqrtf(-2.0f * __logf(UnitOpen(r.w[k])));
-        float sn, cs;
-        __sincosf(6.283185307179586f * UnitOpen(r.w[k + 1]), &sn, &cs);
+        /* Box-Muller on the hardware's own functions: the arguments lie in [2^-25, 1), so
+           none of the range handling of the library versions is needed. log2 -> ln by a
+           factor; sine and cosine take their argument in revolutions */
+        const float u = UnitOpen(r.w[k]), turn = UnitOpen(r.w[k + 1]);
+        const float radius =
+            __builtin_amdgcn_sqrtf(-1.3862943611198906f * __builtin_amdgcn_logf(u));  // -2 ln 2
+        const float sn = __builtin_amdgcn_sinf(turn), cs = __builtin_amdgcn_cosf(turn);
         out[k] = __float_as_uint(p0 + radius * cs * p1);
         out[k + 1] = __float_as_uint(p0 + radius * sn * p1);
       }
