@@ -292,6 +292,28 @@ static int LaunchRowsByIndex(float *dst, int dstride, int k_rows, const void *ro
   return AfterLaunch(what);
 }
 
+namespace {
+/*! \brief rows of at most 256 columns: one thread per row up to 32 columns, one wave per row
+ *  above (1, 2 or 4 columns per lane) */
+template <bool TERMS_GIVEN>
+void LaunchShortSoftmax(float *dst, int dstride, const float *src, int sstride, int rows, int cols,
+                        hipStream_t s) {
+  if (cols <= 32) {
+    hipLaunchKernelGGL((SoftmaxThreadRowKernel<32, TERMS_GIVEN>), dim3((rows + 255) / 256), dim3(256),
+                       0, s, dst, dstride, src, sstride, rows, cols);
+  } else if (cols <= 64) {
+    hipLaunchKernelGGL((SoftmaxWaveRowKernel<1, TERMS_GIVEN>), dim3((rows + 3) / 4), dim3(256), 0, s,
+                       dst, dstride, src, sstride, rows, cols);
+  } else if (cols <= 128) {
+    hipLaunchKernelGGL((SoftmaxWaveRowKernel<2, TERMS_GIVEN>), dim3((rows + 3) / 4), dim3(256), 0, s,
+                       dst, dstride, src, sstride, rows, cols);
+  } else {
+    hipLaunchKernelGGL((SoftmaxWaveRowKernel<4, TERMS_GIVEN>), dim3((rows + 3) / 4), dim3(256), 0, s,
+                       dst, dstride, src, sstride, rows, cols);
+  }
+}
+}  // namespace
+
 extern "C" {
 
 /* ------------------------------------------------------------------ softmax */
@@ -303,6 +325,10 @@ int mshadow_hip_softmax_f32(float *dst, int dstride, const float *src, int sstri
   ABI_REQUIRE(dst != NULL && src != NULL, "NULL tensor");
   ABI_REQUIRE(dstride >= cols && sstride >= cols, "pitch smaller than the row");
   hipStream_t s = AsStream(stream);
+  if (cols <= 256) {  // short rows: a thread or a wave per row instead of a workgroup
+    LaunchShortSoftmax<false>(dst, dstride, src, sstride, rows, cols, s);
+    return AfterLaunch("softmax");
+  }
   /* 128-bit path: aligned rows made of whole packs */
   const bool vec = Aligned16(dst) && Aligned16(src) && dstride % 4 == 0 && sstride % 4 == 0 &&
                    cols % 4 == 0;
@@ -339,6 +365,10 @@ int mshadow_hip_softmax_rowsum_f32(float *sums, const float *terms, int tstride,
   ABI_REQUIRE(tstride >= cols, "pitch smaller than the row");
   ABI_REQUIRE(cols <= 65536, "row longer than the register-resident softmax kernels take");
   hipStream_t s = AsStream(stream);
+  if (cols <= 256) {
+    LaunchShortSoftmax<true>(sums, 0, terms, tstride, rows, cols, s);
+    return AfterLaunch("softmax_rowsum");
+  }
   const bool vec = Aligned16(terms) && tstride % 4 == 0 && cols % 4 == 0;
 #define ROWSUM_LAUNCH(T, S, V) \
   hipLaunchKernelGGL((SoftmaxRowKernel<T, S, V, true>), dim3(rows), dim3(T), 0, s, sums, 0, terms, \

@@ -810,6 +810,88 @@ __global__ void __launch_bounds__(THREADS, 4)  // >= 4 waves per SIMD: two 512-t
   }
 }
 
+/* ---- short rows -----------------------------------------------------------------------
+ * A workgroup per row wastes the machine on the rows classifiers usually have (tens to a few
+ * hundred classes). Same arithmetic as SoftmaxRowKernel, other ownership: */
+
+/*! \brief one thread per row, cols <= CMAX: the row sits in the thread's registers and its
+ *  sum is the serial loop itself. A wave reads 64 neighbouring rows, so the cache lines it
+ *  touches are used whole. */
+template <int CMAX, bool TERMS_GIVEN>
+__global__ void __launch_bounds__(256)
+    SoftmaxThreadRowKernel(float *dst, int dstride, const float *src, int sstride, int rows,
+                           int cols) {
+  const int row = blockIdx.x * 256 + threadIdx.x;
+  if (row >= rows) return;
+  const float *in = src + static_cast<size_t>(row) * sstride;
+  const float kNegInf = -__builtin_huge_valf();
+  float v[CMAX];
+  float mx = kNegInf;
+#pragma unroll
+  for (int i = 0; i < CMAX; ++i) {
+    v[i] = (i < cols) ? in[i] : (TERMS_GIVEN ? 0.0f : kNegInf);
+    mx = (mx < v[i]) ? v[i] : mx;
+  }
+  if (!TERMS_GIVEN) {
+#pragma unroll
+    for (int i = 0; i < CMAX; ++i) v[i] = (i < cols) ? ExpNonPositive(v[i] - mx) : 0.0f;
+  }
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < CMAX; ++i) {
+    if (i < cols) s = s + v[i];
+  }
+  if (TERMS_GIVEN) {
+    dst[row] = s;
+    return;
+  }
+  float *out = dst + static_cast<size_t>(row) * dstride;
+  const bool fast_div = s >= 1.0f && s < 3.0e38f;
+  const float rcp = 1.0f / s;
+#pragma unroll
+  for (int i = 0; i < CMAX; ++i) {
+    if (i < cols) out[i] = fast_div ? DivideBy(v[i], s, rcp) : v[i] / s;
+  }
+}
+
+/*! \brief one wave per row, cols <= 64 * N: lane l holds the N consecutive columns from
+ *  l * N, the sum is resolved in lane order by wave scans (WaveResolve), four rows per
+ *  workgroup and nothing shared between them */
+template <int N, bool TERMS_GIVEN>
+__global__ void __launch_bounds__(256)
+    SoftmaxWaveRowKernel(float *dst, int dstride, const float *src, int sstride, int rows,
+                         int cols) {
+  const int row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(WaveId());
+  if (row >= rows) return;
+  const int base = LaneId() * N;
+  const float *in = src + static_cast<size_t>(row) * sstride;
+  const float kNegInf = -__builtin_huge_valf();
+  float v[N];
+  float mx = kNegInf;
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    v[i] = (base + i < cols) ? in[base + i] : (TERMS_GIVEN ? 0.0f : kNegInf);
+    mx = (mx < v[i]) ? v[i] : mx;
+  }
+  if (!TERMS_GIVEN) {
+    mx = WaveMaxF32(mx);
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = (base + i < cols) ? ExpNonPositive(v[i] - mx) : 0.0f;
+  }
+  const float s = WaveResolve<N>(0.0f, v);
+  if (TERMS_GIVEN) {
+    if (LaneId() == 0) dst[row] = s;
+    return;
+  }
+  float *out = dst + static_cast<size_t>(row) * dstride;
+  const bool fast_div = s >= 1.0f && s < 3.0e38f;
+  const float rcp = 1.0f / s;
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    if (base + i < cols) out[base + i] = fast_div ? DivideBy(v[i], s, rcp) : v[i] / s;
+  }
+}
+
 /*! \brief any row length: three passes, exp(x - max) parked in dst between them */
 template <int THREADS>
 __global__ void __launch_bounds__(THREADS)

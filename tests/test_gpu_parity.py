@@ -207,7 +207,10 @@ def test_reduce_reference_known_answers(G, stream):
 # ------------------------------------------------------------------ softmax
 SOFTMAX_SHAPES = [((64, 32000), 0), ((5, 1000), 0), ((5, 1001), 0), ((3, 7), 1), ((9, 2048), 4),
                   ((4, 8192), 0), ((3, 16384), 0), ((2, 40000), 0), ((2, 70001), 0), ((7, 1), 0),
-                  ((3, 5000), 3), ((2, 20000), 1)]
+                  ((3, 5000), 3), ((2, 20000), 1),
+                  # short rows: one thread per row up to 32 columns, one wave per row up to 256
+                  ((1000, 10), 0), ((300, 32), 0), ((77, 33), 2), ((130, 64), 0), ((50, 65), 1),
+                  ((41, 128), 0), ((19, 200), 3), ((64, 256), 0), ((9, 257), 0), ((5, 2), 0)]
 
 
 def _softmax_check(got, want, src):
@@ -268,7 +271,7 @@ def _serial_row_sums(O, terms):
     return want
 
 
-ROWSUM_COLS = [1, 3, 64, 255, 256, 1000, 1024, 1028, 2048, 3000, 4096, 5001, 8192, 12000, 16384,
+ROWSUM_COLS = [1, 3, 10, 31, 32, 33, 64, 65, 128, 129, 255, 256, 257, 1000, 1024, 1028, 2048, 3000, 4096, 5001, 8192, 12000, 16384,
                20001, 32000, 32768, 40000, 65536]
 
 
