@@ -51,6 +51,21 @@ int mshadow_case_softmax_f32(float *dst, int dstride, const float *src, int sstr
 int mshadow_case_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride,
                                   const float *label, int rows, int cols, void *stream);
 
+/* The same four on half_t tensors, passed as their 16-bit patterns (scale too), and Softmax on
+   double tensors: the element-type-generic paths of the header API */
+int mshadow_case_reduce_keep_lowest_f16(uint16_t *dst, const uint16_t *src, int sstride, int rows,
+                                        int cols, int reducer, int saver, uint16_t scale,
+                                        int variant, void *stream);
+int mshadow_case_reduce_keep_highdim_f16(uint16_t *dst, const uint16_t *src, int sstride, int n,
+                                         int c, int y, int x, int reducer, int saver,
+                                         uint16_t scale, int variant, void *stream);
+int mshadow_case_softmax_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride,
+                             int rows, int cols, void *stream);
+int mshadow_case_softmax_grad_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride,
+                                  const uint16_t *label, int rows, int cols, void *stream);
+int mshadow_case_softmax_f64(double *dst, int dstride, const double *src, int sstride, int rows,
+                             int cols, void *stream);
+
 /* SoftmaxGrad / SmoothSoftmaxGrad with and without ignore_label, on 2-D tensors (d0 == 0:
    rows x cols, label of `rows` floats) or 3-D tensors (d0, d1, d2; label (d0, d2) with
    pitch lstride); flags as MSHADOW_HIP_GRAD_* */

@@ -102,6 +102,11 @@ CASES_SYMBOLS = {
     "mshadow_case_reduce_keep_lowest_f32": ([_p, _p, _i, _i, _i, _i, _i, _f, _i, _p], _i),
     "mshadow_case_reduce_keep_highdim_f32": ([_p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _i, _p], _i),
     "mshadow_case_softmax_f32": ([_p, _i, _p, _i, _i, _i, _p], _i),
+    "mshadow_case_reduce_keep_lowest_f16": ([_p, _p, _i, _i, _i, _i, _i, C.c_uint16, _i, _p], _i),
+    "mshadow_case_reduce_keep_highdim_f16": ([_p, _p, _i, _i, _i, _i, _i, _i, _i, C.c_uint16, _i, _p], _i),
+    "mshadow_case_softmax_f16": ([_p, _i, _p, _i, _i, _i, _p], _i),
+    "mshadow_case_softmax_grad_f16": ([_p, _i, _p, _i, _p, _i, _i, _p], _i),
+    "mshadow_case_softmax_f64": ([_p, _i, _p, _i, _i, _i, _p], _i),
     "mshadow_case_grad_family_f32": ([_p, _i, _p, _i, _p, _i, _i, _i, _i, _i, _f, _f, _p], _i),
     "mshadow_case_softmax3d_f32": ([_p, _i, _p, _i, _i, _i, _i, _p], _i),
     "mshadow_case_rows_by_index_f32": ([_i, _p, _i, _i, _p, _p, _i, _p, _i, _i, _i, _p], _i),
@@ -477,23 +482,31 @@ class Library:
 
     def case_reduce_keep_lowest(self, dst, src, reducer=SUM, saver=SAVETO, scale=1.0, variant=0,
                                 stream=None):
-        self.check_case(self.cases.mshadow_case_reduce_keep_lowest_f32(
-            dst.ptr, src.ptr, src.stride, src.rows, src.cols, reducer, saver, scale, variant,
-            stream))
+        """float tensors, or half_t tensors as uint16 buffers (scale then is the half's bits)"""
+        fn = (self.cases.mshadow_case_reduce_keep_lowest_f16 if src.dtype == np.uint16
+              else self.cases.mshadow_case_reduce_keep_lowest_f32)
+        self.check_case(fn(dst.ptr, src.ptr, src.stride, src.rows, src.cols, reducer, saver, scale,
+                           variant, stream))
 
     def case_reduce_keep_highdim(self, dst, src, reducer=SUM, saver=SAVETO, scale=1.0, variant=0,
                                  stream=None):
         n, c, y, x = src.shape
-        self.check_case(self.cases.mshadow_case_reduce_keep_highdim_f32(
-            dst.ptr, src.ptr, src.stride, n, c, y, x, reducer, saver, scale, variant, stream))
+        fn = (self.cases.mshadow_case_reduce_keep_highdim_f16 if src.dtype == np.uint16
+              else self.cases.mshadow_case_reduce_keep_highdim_f32)
+        self.check_case(fn(dst.ptr, src.ptr, src.stride, n, c, y, x, reducer, saver, scale,
+                           variant, stream))
 
     def case_softmax(self, dst, src, stream=None):
-        self.check_case(self.cases.mshadow_case_softmax_f32(dst.ptr, dst.stride, src.ptr,
-                                                            src.stride, src.rows, src.cols, stream))
+        fn = {"float32": self.cases.mshadow_case_softmax_f32,
+              "uint16": self.cases.mshadow_case_softmax_f16,
+              "float64": self.cases.mshadow_case_softmax_f64}[src.dtype.name]
+        self.check_case(fn(dst.ptr, dst.stride, src.ptr, src.stride, src.rows, src.cols, stream))
 
     def case_softmax_grad(self, dst, src, label, stream=None):
-        self.check_case(self.cases.mshadow_case_softmax_grad_f32(
-            dst.ptr, dst.stride, src.ptr, src.stride, label.ptr, src.rows, src.cols, stream))
+        fn = (self.cases.mshadow_case_softmax_grad_f16 if src.dtype == np.uint16
+              else self.cases.mshadow_case_softmax_grad_f32)
+        self.check_case(fn(dst.ptr, dst.stride, src.ptr, src.stride, label.ptr, src.rows, src.cols,
+                           stream))
 
     def case_pool(self, dst, src, ky, kx, sy, sx, reducer=MAX, variant=0, stream=None):
         h, w = src.shape[-2:]

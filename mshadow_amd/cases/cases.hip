@@ -64,17 +64,21 @@ void Assign(Dst dst, const E &e, int saver) {
   }
 }
 
-template <typename Reducer, typename Src>
-void ReduceInto(Tensor<gpu, 1, float> dst, const Src &src, int saver, float scale) {
+template <typename Reducer, typename DType, typename Src>
+void ReduceInto(Tensor<gpu, 1, DType> dst, const Src &src, int saver, DType scale) {
   Assign(dst, scale * reduce_except_dim<1, Reducer>(src), saver);
 }
-template <typename Src>
-void ReduceDispatch(Tensor<gpu, 1, float> dst, const Src &src, int reducer, int saver,
-                    float scale) {
+template <typename DType, typename Src>
+void ReduceDispatch(Tensor<gpu, 1, DType> dst, const Src &src, int reducer, int saver,
+                    DType scale) {
   if (reducer == 0) ReduceInto<red::sum>(dst, src, saver, scale);
   else if (reducer == 1) ReduceInto<red::maximum>(dst, src, saver, scale);
   else ReduceInto<red::minimum>(dst, src, saver, scale);
 }
+
+typedef half::half_t HalfT;
+inline const HalfT *H(const uint16_t *p) { return reinterpret_cast<const HalfT *>(p); }
+inline HalfT *H(uint16_t *p) { return reinterpret_cast<HalfT *>(p); }
 
 }  // namespace
 
@@ -167,6 +171,59 @@ int mshadow_case_softmax_grad_f32(float *dst, int dstride, const float *src, int
   BorrowedStream st(stream);
   SoftmaxGrad(G2(dst, rows, cols, dstride, st.get()), G2(src, rows, cols, sstride, st.get()),
               G1(label, rows, st.get()));
+  CASE_END
+}
+
+/* the reductions and the softmax pair on half_t tensors (16-bit patterns; scale is a half_t) */
+int mshadow_case_reduce_keep_lowest_f16(uint16_t *dst, const uint16_t *src, int sstride, int rows,
+                                        int cols, int reducer, int saver, uint16_t scale,
+                                        int variant, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Tensor<gpu, 2, HalfT> S = G2(H(src), rows, cols, sstride, st.get());
+  Tensor<gpu, 1, HalfT> o = G1(H(dst), cols, st.get());
+  const HalfT sc = HalfT::Binary(scale);
+  if (variant == 0) ReduceDispatch(o, S, reducer, saver, sc);
+  else ReduceDispatch(o, F<op::identity>(S), reducer, saver, sc);
+  CASE_END
+}
+
+int mshadow_case_reduce_keep_highdim_f16(uint16_t *dst, const uint16_t *src, int sstride, int n,
+                                         int c, int y, int x, int reducer, int saver,
+                                         uint16_t scale, int variant, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Tensor<gpu, 4, HalfT> S = G4(H(src), n, c, y, x, sstride, st.get());
+  Tensor<gpu, 1, HalfT> o = G1(H(dst), c, st.get());
+  const HalfT sc = HalfT::Binary(scale);
+  if (variant == 0) ReduceDispatch(o, S, reducer, saver, sc);
+  else ReduceDispatch(o, F<op::identity>(S), reducer, saver, sc);
+  CASE_END
+}
+
+int mshadow_case_softmax_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride,
+                             int rows, int cols, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Softmax(G2(H(dst), rows, cols, dstride, st.get()), G2(H(src), rows, cols, sstride, st.get()));
+  CASE_END
+}
+
+int mshadow_case_softmax_grad_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride,
+                                  const uint16_t *label, int rows, int cols, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  SoftmaxGrad(G2(H(dst), rows, cols, dstride, st.get()), G2(H(src), rows, cols, sstride, st.get()),
+              G1(H(label), rows, st.get()));
+  CASE_END
+}
+
+/* Softmax(dst, src) on double tensors */
+int mshadow_case_softmax_f64(double *dst, int dstride, const double *src, int sstride, int rows,
+                             int cols, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Softmax(G2(dst, rows, cols, dstride, st.get()), G2(src, rows, cols, sstride, st.get()));
   CASE_END
 }
 

@@ -25,6 +25,7 @@
 #if defined(__HIPCC__)
 #include "./kernels/map.h"
 #include "./kernels/reduce.h"
+#include "./kernels/softmax_any.h"
 #endif
 
 namespace mshadow {
@@ -158,16 +159,49 @@ inline void SoftmaxGrad(const Tensor<gpu, 2, float> &dst, const Tensor<gpu, 2, f
                                                 label.dptr_, dst.size(0), dst.size(1),
                                                 Stream<gpu>::GetStream(dst.stream_)));
 }
-/* the templates declared in tensor.h forward to the float implementations above; other
-   element types have no fixed-function softmax in this backend */
+/* other element types (half_t, double): kernel templates in the element type's own
+   arithmetic, instantiated in the calling translation unit (kernels/softmax_any.h) */
 template <typename DType>
 inline void Softmax(Tensor<gpu, 2, DType> dst, const Tensor<gpu, 2, DType> &src) {
-  LOG(FATAL) << "Softmax<gpu>: only float is provided by this backend";
+  CHECK_EQ(dst.shape_, src.shape_) << "Softmax: shape mismatch";
+#if defined(__HIPCC__)
+  uint32_t rows = dst.size(0), cols = dst.size(1);
+  if (rows == 0 || cols == 0) return;
+  DType *d = dst.dptr_;
+  const DType *s = src.dptr_;
+  uint32_t dstride = dst.stride_, sstride = src.stride_;
+  void *args[] = {&d, &dstride, &s, &sstride, &rows, &cols};
+  const uint32_t grid[3] = {(rows + hip::kAnyRowsPerBlock - 1) / hip::kAnyRowsPerBlock, 1, 1};
+  const uint32_t block[3] = {static_cast<uint32_t>(hip::kAnyBlock), 1, 1};
+  MSHADOW_HIP_CALL(mshadow_hip_launch(reinterpret_cast<const void *>(hip::SoftmaxAnyKernel<DType>),
+                                      grid, block, args, 0, Stream<gpu>::GetStream(dst.stream_)));
+#else
+  LOG(FATAL) << "Softmax<gpu> of this element type: compile the calling translation unit with hipcc";
+#endif
 }
 template <typename DType>
 inline void SoftmaxGrad(const Tensor<gpu, 2, DType> &dst, const Tensor<gpu, 2, DType> &src,
                         const Tensor<gpu, 1, DType> &label) {
-  LOG(FATAL) << "SoftmaxGrad<gpu>: only float is provided by this backend";
+  CHECK_EQ(dst.shape_, src.shape_) << "SoftmaxGrad: shape mismatch";
+  CHECK_EQ(dst.size(0), label.size(0)) << "SoftmaxGrad: label shape mismatch";
+#if defined(__HIPCC__)
+  uint32_t rows = dst.size(0), cols = dst.size(1);
+  if (rows == 0 || cols == 0) return;
+  DType *d = dst.dptr_;
+  const DType *s = src.dptr_;
+  const DType *l = label.dptr_;
+  uint32_t dstride = dst.stride_, sstride = src.stride_;
+  void *args[] = {&d, &dstride, &s, &sstride, &l, &cols};
+  /* rows on the grid's x axis (up to 2^31 - 1), a row's columns over a few workgroups */
+  uint32_t per_row = (cols + hip::kAnyBlock * 8 - 1) / (hip::kAnyBlock * 8);
+  if (per_row > 64) per_row = 64;
+  const uint32_t grid[3] = {rows, per_row, 1};
+  const uint32_t block[3] = {static_cast<uint32_t>(hip::kAnyBlock), 1, 1};
+  MSHADOW_HIP_CALL(mshadow_hip_launch(reinterpret_cast<const void *>(hip::SoftmaxGradAnyKernel<DType>),
+                                      grid, block, args, 0, Stream<gpu>::GetStream(dst.stream_)));
+#else
+  LOG(FATAL) << "SoftmaxGrad<gpu> of this element type: compile the calling translation unit with hipcc";
+#endif
 }
 
 /* ---- the rest of the softmax family and the row scatter / gather functions: float tensors,

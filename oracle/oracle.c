@@ -266,6 +266,106 @@ void orc_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride
   }
 }
 
+/* ---- the same functions on half_t tensors (16-bit storage). Every half_t operator widens
+   to float, computes, and rounds back to 16 bits (mshadow/half.h:45-66), so each step of
+   an accumulation rounds: a sum of ones stops growing at 2048. Comparisons are made on the
+   widened values (:341-348). */
+static inline uint16_t half_of(float v) { return orc_float2half(v); }
+static inline float wide(uint16_t h) { return orc_half2float(h); }
+
+static inline void save_f16(uint16_t *dst, uint16_t v, int saver) {
+  switch (saver) {
+    case ORC_SAVETO: *dst = v; break;
+    case ORC_PLUSTO: *dst = half_of(wide(*dst) + wide(v)); break;
+    case ORC_MINUSTO: *dst = half_of(wide(*dst) - wide(v)); break;
+    case ORC_MULTO: *dst = half_of(wide(*dst) * wide(v)); break;
+    default: *dst = half_of(wide(*dst) / wide(v)); break;
+  }
+}
+
+/* red::sum / maximum / minimum on half_t (mshadow/base.h:692-697, :751-761, :807-817:
+   std::max(dst, src) returns src only when dst < src, std::min only when src < dst) */
+static inline void reduce_f16(uint16_t *dst, uint16_t src, int reducer) {
+  switch (reducer) {
+    case ORC_SUM: *dst = half_add(*dst, src); break;
+    case ORC_MAX: *dst = (wide(*dst) < wide(src)) ? src : *dst; break;
+    default: *dst = (wide(src) < wide(*dst)) ? src : *dst; break;
+  }
+}
+
+/* mshadow/base.h:716-719 (0), :798-801 (MSHADOW_HALF_MIN = 0xFBFF), :862-865
+   (MSHADOW_HALF_MAX = 0x7BFF) */
+static inline uint16_t init_f16(int reducer) {
+  switch (reducer) {
+    case ORC_SUM: return 0;
+    case ORC_MAX: return 0xFBFFu;
+    default: return 0x7BFFu;
+  }
+}
+
+/* MapReduceKeepLowest on half_t, mshadow/tensor_cpu-inl.h:203-228 */
+void orc_reduce_keep_lowest_f16(uint16_t *dst, const uint16_t *src, int sstride, int rows,
+                                int cols, int reducer, int saver, uint16_t scale) {
+#pragma omp parallel for
+  for (int x = 0; x < cols; ++x) {
+    uint16_t res = src[x];
+    for (int y = 1; y < rows; ++y) reduce_f16(&res, src[(int64_t)y * sstride + x], reducer);
+    save_f16(&dst[x], half_of(wide(res) * wide(scale)), saver);
+  }
+}
+
+/* MapReduceKeepHighDim on half_t, mshadow/tensor_cpu-inl.h:230-268 */
+void orc_reduce_keep_highdim_f16(uint16_t *dst, const uint16_t *src, int sstride, int n, int c,
+                                 int y, int x, int reducer, int saver, uint16_t scale) {
+#pragma omp parallel for
+  for (int ci = 0; ci < c; ++ci) {
+    uint16_t res = init_f16(reducer);
+    for (int ni = 0; ni < n; ++ni) {
+      uint16_t tres = init_f16(reducer);
+      for (int yi = 0; yi < y; ++yi) {
+        const uint16_t *row = src + (int64_t)((ni * c + ci) * y + yi) * sstride;
+        for (int xi = 0; xi < x; ++xi) reduce_f16(&tres, row[xi], reducer);
+      }
+      reduce_f16(&res, tres, reducer);
+    }
+    save_f16(&dst[ci], half_of(wide(res) * wide(scale)), saver);
+  }
+}
+
+/* Softmax on half_t, mshadow/tensor_cpu-inl.h:270-285: energy[x] - mmax is a half_t
+   (rounded), std::exp takes it as a float and its result is rounded into dst[x]; the sum
+   is a half_t that rounds after every add; dst[x] /= sum is a float division rounded. */
+void orc_softmax_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride, int rows,
+                     int cols) {
+#pragma omp parallel for
+  for (int y = 0; y < rows; ++y) {
+    const uint16_t *e = src + (int64_t)y * sstride;
+    uint16_t *o = dst + (int64_t)y * dstride;
+    uint16_t mmax = e[0];
+    for (int x = 1; x < cols; ++x) {
+      if (wide(mmax) < wide(e[x])) mmax = e[x];
+    }
+    uint16_t sum = half_of(0.0f);
+    for (int x = 0; x < cols; ++x) {
+      o[x] = half_of(expf(wide(half_of(wide(e[x]) - wide(mmax)))));
+      sum = half_add(sum, o[x]);
+    }
+    for (int x = 0; x < cols; ++x) o[x] = half_of(wide(o[x]) / wide(sum));
+  }
+}
+
+/* SoftmaxGrad on half_t, mshadow/tensor_cpu-inl.h:287-302 */
+void orc_softmax_grad_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride,
+                          const uint16_t *label, int rows, int cols) {
+#pragma omp parallel for
+  for (int y = 0; y < rows; ++y) {
+    const int k = (int)wide(label[y]);
+    const uint16_t *s = src + (int64_t)y * sstride;
+    uint16_t *o = dst + (int64_t)y * dstride;
+    for (int x = 0; x < cols; ++x) o[x] = (x == k) ? half_of(wide(s[x]) - 1.0f) : s[x];
+  }
+}
+
 /* SoftmaxGrad with ignore_label, SmoothSoftmaxGrad with and without it,
    mshadow/tensor_cpu-inl.h:304-362. (src - 1.0f) + alpha is evaluated left to right;
    smooth_grad = alpha / (cols - 1) in float. */

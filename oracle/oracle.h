@@ -55,6 +55,17 @@ void orc_softmax_f32(float *dst, int dstride, const float *src, int sstride, int
 void orc_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride,
                           const float *label, int rows, int cols);
 
+/* The reductions and the softmax pair on half_t tensors (16-bit storage; every operation
+   rounds to 16 bits, so accumulations round after each step). `scale` is a half_t too. */
+void orc_reduce_keep_lowest_f16(uint16_t *dst, const uint16_t *src, int sstride, int rows,
+                                int cols, int reducer, int saver, uint16_t scale);
+void orc_reduce_keep_highdim_f16(uint16_t *dst, const uint16_t *src, int sstride, int n, int c,
+                                 int y, int x, int reducer, int saver, uint16_t scale);
+void orc_softmax_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride, int rows,
+                     int cols);
+void orc_softmax_grad_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride,
+                          const uint16_t *label, int rows, int cols);
+
 /* The rest of the softmax family and the row scatter / gather functions
    (mshadow/tensor_cpu-inl.h:304-528). `flags`: bit 0 = smooth (alpha used), bit 1 = the
    ignore_label argument is used. 3-D tensors are (d0, d1, d2) with the softmax over d1

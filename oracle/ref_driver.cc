@@ -65,6 +65,21 @@ void ReduceHigh(Tensor<cpu, 1, float> dst, const Src &src, int saver, float scal
   }
 }
 
+typedef half::half_t HalfT;
+const HalfT *H(const uint16_t *p) { return reinterpret_cast<const HalfT *>(p); }
+HalfT *H(uint16_t *p) { return reinterpret_cast<HalfT *>(p); }
+
+template <typename Reducer, typename Src>
+void ReduceHighHalf(Tensor<cpu, 1, HalfT> dst, const Src &src, int saver, HalfT scale) {
+  switch (saver) {
+    case 0: dst = scale * reduce_except_dim<1, Reducer>(src); break;
+    case 1: dst += scale * reduce_except_dim<1, Reducer>(src); break;
+    case 2: dst -= scale * reduce_except_dim<1, Reducer>(src); break;
+    case 3: dst *= scale * reduce_except_dim<1, Reducer>(src); break;
+    default: dst /= scale * reduce_except_dim<1, Reducer>(src); break;
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -130,6 +145,38 @@ void ref_softmax_f32(float *dst, int dstride, const float *src, int sstride, int
 void ref_softmax_grad_f32(float *dst, int dstride, const float *src, int sstride,
                           const float *label, int rows, int cols) {
   SoftmaxGrad(T2(dst, rows, cols, dstride), T2(src, rows, cols, sstride), T1(label, rows));
+}
+
+/* the same on half_t tensors */
+void ref_reduce_keep_lowest_f16(uint16_t *dst, const uint16_t *src, int sstride, int rows,
+                                int cols, int reducer, int saver, uint16_t scale) {
+  Tensor<cpu, 2, HalfT> S = T2(H(src), rows, cols, sstride);
+  Tensor<cpu, 1, HalfT> o = T1(H(dst), cols);
+  const HalfT sc = HalfT::Binary(scale);
+  if (reducer == 0) ReduceHighHalf<red::sum>(o, S, saver, sc);
+  else if (reducer == 1) ReduceHighHalf<red::maximum>(o, S, saver, sc);
+  else ReduceHighHalf<red::minimum>(o, S, saver, sc);
+}
+
+void ref_reduce_keep_highdim_f16(uint16_t *dst, const uint16_t *src, int sstride, int n, int c,
+                                 int y, int x, int reducer, int saver, uint16_t scale) {
+  Tensor<cpu, 4, HalfT> S = T4(H(src), n, c, y, x, sstride);
+  Tensor<cpu, 1, HalfT> o = T1(H(dst), c);
+  const HalfT sc = HalfT::Binary(scale);
+  if (reducer == 0) ReduceHighHalf<red::sum>(o, S, saver, sc);
+  else if (reducer == 1) ReduceHighHalf<red::maximum>(o, S, saver, sc);
+  else ReduceHighHalf<red::minimum>(o, S, saver, sc);
+}
+
+void ref_softmax_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride, int rows,
+                     int cols) {
+  Softmax(T2(H(dst), rows, cols, dstride), T2(H(src), rows, cols, sstride));
+}
+
+void ref_softmax_grad_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride,
+                          const uint16_t *label, int rows, int cols) {
+  SoftmaxGrad(T2(H(dst), rows, cols, dstride), T2(H(src), rows, cols, sstride),
+              T1(H(label), rows));
 }
 
 void ref_softmax_grad_ex_f32(float *dst, int dstride, const float *src, int sstride,

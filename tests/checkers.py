@@ -77,6 +77,11 @@ class Checker:
         self._fn("reduce_keep_highdim_f32", [_p, _p, _i, _i, _i, _i, _i, _i, _i, _f])
         self._fn("softmax_f32", [_p, _i, _p, _i, _i, _i])
         self._fn("softmax_grad_f32", [_p, _i, _p, _i, _p, _i, _i])
+        _h = C.c_uint16
+        self._fn("reduce_keep_lowest_f16", [_p, _p, _i, _i, _i, _i, _i, _h])
+        self._fn("reduce_keep_highdim_f16", [_p, _p, _i, _i, _i, _i, _i, _i, _i, _h])
+        self._fn("softmax_f16", [_p, _i, _p, _i, _i, _i])
+        self._fn("softmax_grad_f16", [_p, _i, _p, _i, _p, _i, _i])
         self._fn("softmax_grad_ex_f32", [_p, _i, _p, _i, _p, _i, _i, _i, _f, _f])
         self._fn("softmax3d_f32", [_p, _i, _p, _i, _i, _i, _i])
         self._fn("softmax3d_grad_f32", [_p, _i, _p, _i, _p, _i, _i, _i, _i, _i, _f, _f])
@@ -133,6 +138,10 @@ class Checker:
     def reduce_keep_lowest(self, dst, src, reducer=SUM, saver=SAVETO, scale=1.0):
         rows, cols = int(np.prod(src.shape[:-1])), src.shape[-1]
         assert dst.shape == (cols,)
+        if src.dtype == np.uint16:  # half_t tensors as their 16-bit patterns; scale is rounded to half
+            self._reduce_keep_lowest_f16(ptr(dst), ptr(src), pitch(src), rows, cols, reducer, saver,
+                                         int(self.float2half(np.array([scale], np.float32))[0]))
+            return dst
         self._reduce_keep_lowest_f32(ptr(dst), ptr(src), pitch(src), rows, cols, reducer, saver,
                                      scale)
         return dst
@@ -140,6 +149,10 @@ class Checker:
     def reduce_keep_highdim(self, dst, src, reducer=SUM, saver=SAVETO, scale=1.0):
         n, c, y, x = src.shape
         assert dst.shape == (c,)
+        if src.dtype == np.uint16:
+            self._reduce_keep_highdim_f16(ptr(dst), ptr(src), pitch(src), n, c, y, x, reducer,
+                                          saver, int(self.float2half(np.array([scale], np.float32))[0]))
+            return dst
         self._reduce_keep_highdim_f32(ptr(dst), ptr(src), pitch(src), n, c, y, x, reducer, saver,
                                       scale)
         return dst
@@ -147,11 +160,18 @@ class Checker:
     # -- softmax
     def softmax(self, dst, src):
         rows, cols = src.shape
+        if src.dtype == np.uint16:
+            self._softmax_f16(ptr(dst), pitch(dst), ptr(src), pitch(src), rows, cols)
+            return dst
         self._softmax_f32(ptr(dst), pitch(dst), ptr(src), pitch(src), rows, cols)
         return dst
 
     def softmax_grad(self, dst, src, label):
         rows, cols = src.shape
+        if src.dtype == np.uint16:
+            assert label.dtype == np.uint16 and label.shape == (rows,)
+            self._softmax_grad_f16(ptr(dst), pitch(dst), ptr(src), pitch(src), ptr(label), rows, cols)
+            return dst
         assert label.dtype == np.float32 and label.shape == (rows,)
         self._softmax_grad_f32(ptr(dst), pitch(dst), ptr(src), pitch(src), ptr(label), rows, cols)
         return dst

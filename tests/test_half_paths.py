@@ -1,0 +1,218 @@
+"""Reductions and the softmax pair on half_t tensors: the oracle against the compiled reference
+and against what 16-bit arithmetic fixes in closed form (CPU), and the HIP path against the
+oracle (GPU).
+
+half_t rounds after every operation (mshadow/half.h:45-66), so these functions are sensitive
+to the order of the additions in a way the float ones are not: a sum of ones stops at 2048
+(2048 + 1 is a tie that rounds to even), which no tree sum reproduces. Bars: bit-exact for the
+reductions and the softmax gradient; Softmax forward within the task's relative 2e-3 for
+half_t (observed: the only differences come from expf and are single roundings).
+"""
+import numpy as np
+import pytest
+
+from checkers import DIVTO, MAX, MIN, MINUSTO, MULTO, PLUSTO, SAVETO, SUM, Checker, have_ref
+
+f32 = np.float32
+
+
+def halves(orc, seed, shape, sigma=1.0):
+    rng = np.random.default_rng(seed)
+    return orc.float2half((rng.standard_normal(shape) * sigma).astype(f32))
+
+
+# ------------------------------------------------------------------ CPU: oracle pinned
+def test_half_sum_saturates_at_2048(orc):
+    ones = orc.float2half(np.ones((5000, 3), f32))
+    out = np.zeros(3, np.uint16)
+    orc.reduce_keep_lowest(out, ones)
+    assert orc.half2float(out).tolist() == [2048.0] * 3
+    # order matters: 2048 first absorbs every later 1; the ones first reach 2050
+    col = np.ones((3, 1), f32)
+    col[0, 0] = 2048.0
+    out1 = np.zeros(1, np.uint16)
+    orc.reduce_keep_lowest(out1, orc.float2half(col))
+    orc_rev = np.zeros(1, np.uint16)
+    orc.reduce_keep_lowest(orc_rev, orc.float2half(col[::-1].copy()))
+    assert orc.half2float(out1)[0] == 2048.0 and orc.half2float(orc_rev)[0] == 2050.0
+
+
+def test_half_highdim_two_level_order(orc):
+    # per kept index: inner sums over (y, x) per n, merged in n order. 3000 ones per n would
+    # saturate a single running sum at 2048; two levels give 2 * 2048 = 4096
+    src = orc.float2half(np.ones((2, 2, 30, 100), f32))
+    out = np.zeros(2, np.uint16)
+    orc.reduce_keep_highdim(out, src)
+    assert orc.half2float(out).tolist() == [4096.0, 4096.0]
+    orc.reduce_keep_highdim(out, src, reducer=MAX, scale=0.5)
+    assert orc.half2float(out).tolist() == [0.5, 0.5]
+
+
+def test_half_softmax_known_answers(orc):
+    # n equal logits: every term is exactly 1; the half sum is n up to 2048 and stays there
+    for n, denom in ((8, 8.0), (2048, 2048.0), (4096, 2048.0), (10000, 2048.0)):
+        x = orc.float2half(np.full((2, n), 0.25, f32))
+        p = np.empty_like(x)
+        orc.softmax(p, x)
+        assert np.all(orc.half2float(p) == f32(1.0 / denom)), n
+    # gradient: half(p - 1) at static_cast<int>(label) (9.7 -> 9), a copy elsewhere and for
+    # labels outside the row; multiples of 1/16 keep p - 1 exact
+    p = orc.float2half((np.arange(40, dtype=f32) / 16).reshape(4, 10))
+    lab = orc.float2half(np.array([3.0, 9.7, -1.0, 10.0], f32))
+    g = np.empty_like(p)
+    orc.softmax_grad(g, p, lab)
+    d = orc.half2float(g) - orc.half2float(p)
+    want = np.zeros((4, 10), f32)
+    want[0, 3] = want[1, 9] = -1.0
+    assert np.array_equal(d, want)
+    # and a value where p - 1 has to round to 11 bits: 0.0769 - 1 = -0.9231 -> -0.92285
+    q = orc.float2half(np.array([[0.0769]], f32))
+    orc.softmax_grad(g[:1, :1], q, orc.float2half(np.zeros(1, f32)))
+    assert g[0, 0] == orc.float2half(orc.half2float(q) - f32(1.0))[0, 0]
+
+
+@pytest.mark.skipif(not have_ref(), reason="reference build absent")
+@pytest.mark.parametrize("shape", [(1, 1), (7, 5), (300, 33), (5000, 4), (64, 1000)])
+def test_half_oracle_equals_reference(orc, ref, shape):
+    x = halves(orc, 7, shape, 3.0)
+    a, b = np.empty_like(x), np.empty_like(x)
+    orc.softmax(a, x)
+    ref.softmax(b, x)
+    assert np.array_equal(a, b)
+    lab = orc.float2half(np.random.default_rng(8).integers(-1, shape[1] + 1, shape[0]).astype(f32))
+    ga, gb = np.empty_like(x), np.empty_like(x)
+    orc.softmax_grad(ga, a, lab)
+    ref.softmax_grad(gb, a, lab)
+    assert np.array_equal(ga, gb)
+    for reducer in (SUM, MAX, MIN):
+        for saver, scale in ((SAVETO, 1.0), (PLUSTO, 0.5), (MINUSTO, 3.0), (MULTO, 0.25), (DIVTO, 2.0)):
+            oa = halves(orc, 9, (shape[1],))
+            ob = oa.copy()
+            orc.reduce_keep_lowest(oa, x, reducer, saver, scale)
+            ref.reduce_keep_lowest(ob, x, reducer, saver, scale)
+            assert np.array_equal(oa, ob), (reducer, saver)
+
+
+@pytest.mark.skipif(not have_ref(), reason="reference build absent")
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1), (3, 5, 7, 9), (20, 4, 30, 31)])
+def test_half_highdim_oracle_equals_reference(orc, ref, shape):
+    x = halves(orc, 11, shape)
+    for reducer in (SUM, MAX, MIN):
+        for saver, scale in ((SAVETO, 1.0), (PLUSTO, 0.5)):
+            oa = halves(orc, 12, (shape[1],))
+            ob = oa.copy()
+            orc.reduce_keep_highdim(oa, x, reducer, saver, scale)
+            ref.reduce_keep_highdim(ob, x, reducer, saver, scale)
+            assert np.array_equal(oa, ob), (reducer, saver)
+
+
+# ------------------------------------------------------------------ GPU parity
+@pytest.fixture(scope="module")
+def G():
+    import mshadow_amd
+    g = mshadow_amd.load_cases()
+    assert g.device_count() >= 1, "no GPU visible"
+    g.set_device(0)
+    return g
+
+
+@pytest.fixture(scope="module")
+def stream(G):
+    s = G.stream_create()
+    yield s
+    G.stream_destroy(s)
+
+
+def _bits(orc, scale):
+    return int(orc.float2half(np.array([scale], f32))[0])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape,pad", [((1, 1), 0), ((5000, 3), 0), ((300, 33), 5), ((4096, 130), 0),
+                                       ((17, 1000), 2)])
+def test_gpu_half_reduce_keep_lowest(G, orc, stream, shape, pad):
+    x = halves(orc, 21, shape)
+    if shape == (5000, 3):
+        x = orc.float2half(np.ones(shape, f32))       # saturates at 2048 only in row order
+    src = G.to_device(x, pad)
+    for variant in (0, 1):
+        for reducer in (SUM, MAX, MIN):
+            for saver, scale in ((SAVETO, 1.0), (PLUSTO, 0.5), (DIVTO, 2.0)):
+                init = halves(orc, 22, (shape[1],))
+                want = init.copy()
+                orc.reduce_keep_lowest(want, x, reducer, saver, scale)
+                dst = G.to_device(init)
+                G.case_reduce_keep_lowest(dst, src, reducer, saver, _bits(orc, scale), variant, stream)
+                got = dst.download(stream)
+                assert np.array_equal(got, want), (variant, reducer, saver)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape,pad", [((1, 1, 1, 1), 0), ((3, 5, 7, 9), 3), ((2, 2, 30, 100), 0),
+                                       ((20, 6, 28, 28), 0)])
+def test_gpu_half_reduce_keep_highdim(G, orc, stream, shape, pad):
+    x = halves(orc, 31, shape)
+    if shape == (2, 2, 30, 100):
+        x = orc.float2half(np.ones(shape, f32))       # 4096 only with the two-level order
+    src = G.to_device(x, pad)
+    for variant in (0, 1):
+        for reducer in (SUM, MAX, MIN):
+            for saver, scale in ((SAVETO, 1.0), (MINUSTO, 0.5)):
+                init = halves(orc, 32, (shape[1],))
+                want = init.copy()
+                orc.reduce_keep_highdim(want, x, reducer, saver, scale)
+                dst = G.to_device(init)
+                G.case_reduce_keep_highdim(dst, src, reducer, saver, _bits(orc, scale), variant, stream)
+                assert np.array_equal(dst.download(stream), want), (variant, reducer, saver)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape,pad", [((1, 1), 0), ((7, 5), 0), ((9, 513), 3), ((64, 1000), 0),
+                                       ((5, 4096), 0), ((3, 32000), 0), ((130, 77), 1)])
+def test_gpu_half_softmax(G, orc, stream, shape, pad):
+    x = halves(orc, 41, shape, 3.0)
+    if shape == (5, 4096):
+        x = orc.float2half(np.full(shape, 0.25, f32))  # 1/2048 each: the sum saturates
+    want = np.empty_like(x)
+    orc.softmax(want, x)
+    src = G.to_device(x, pad)
+    dst = G.buffer(shape, np.uint16, pad)
+    G.case_softmax(dst, src, stream)
+    got = dst.download(stream)
+    w, g = orc.half2float(want).astype(np.float64), orc.half2float(got).astype(np.float64)
+    differ = int(np.count_nonzero(got != want))
+    # relative 2e-3 for values above the smallest normal half (one subnormal ulp below it)
+    tol = np.maximum(2e-3 * np.abs(w), 2.0 ** -24)
+    assert np.all(np.abs(g - w) <= tol), np.max(np.abs(g - w) / np.maximum(np.abs(w), 2.0 ** -14))
+    if shape == (5, 4096):
+        assert differ == 0 and np.all(g == 1.0 / 2048)
+    print(f"half softmax {shape}: {differ} of {got.size} outputs differ from the CPU path")
+    # in place
+    G.case_softmax(src, src, stream)
+    assert np.array_equal(src.download(stream), got)
+    # gradient: bit-exact, labels inside, on the edge and outside the row
+    lab = orc.float2half(np.random.default_rng(42).integers(-1, shape[1] + 1, shape[0]).astype(f32))
+    gw = np.empty_like(got)
+    orc.softmax_grad(gw, got, lab)
+    gd = G.buffer(shape, np.uint16, pad)
+    G.case_softmax_grad(gd, src, G.to_device(lab), stream)
+    assert np.array_equal(gd.download(stream), gw)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(1, 1), (33, 1000), (4, 20000)])
+def test_gpu_double_softmax(G, stream, shape):
+    """Softmax on double tensors: the same left-to-right sum in double, against numpy's
+    float64 evaluation of the same steps (parity unpinned at the ulp level: the device and
+    the host exponential are different libraries)"""
+    rng = np.random.default_rng(51)
+    x = rng.standard_normal(shape) * 3.0
+    t = np.exp(x - x.max(axis=1, keepdims=True))
+    s = np.zeros(shape[0])
+    for j in range(shape[1]):
+        s = s + t[:, j]
+    want = t / s[:, None]
+    dst = G.buffer(shape, np.float64)
+    G.case_softmax(dst, G.to_device(x), stream)
+    got = dst.download(stream)
+    assert np.all(np.abs(got - want) <= 1e-13 * want + 1e-300)
