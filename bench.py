@@ -63,6 +63,11 @@ def algorithmic_bytes():
         "ceiling_fill": e * 8192 * 32000,
         "dot_f32_4096": 3 * e * 4096 * 4096,
         "dot_f16_8192": 3 * 2 * 8192 * 8192,
+        # the same shapes on half_t tensors through the element-type-generic header paths
+        "softmax_f16": 2 * 2 * 8192 * 32000,
+        "softmax_grad_f16": 2 * 2 * 8192 * 32000 + 2 * 8192,
+        "sum_rows_f16": 2 * 16384 * 4096 + 2 * 4096,
+        "sumall_except_dim1_f16": 2 * 64 * 256 * 56 * 56 + 2 * 256,
     }
 
 
@@ -79,6 +84,8 @@ def work_elements():
         "sort_by_key_f32": 1 << 24, "dot_f32_4096": 4096 * 4096, "dot_f16_8192": 8192 * 8192,
         "ceiling_copy": 8192 * 32000, "ceiling_fill": 8192 * 32000,
         "random_uniform": 8192 * 32000, "random_normal": 8192 * 32000,
+        "softmax_f16": 8192 * 32000, "softmax_grad_f16": 8192 * 32000,
+        "sum_rows_f16": 16384 * 4096, "sumall_except_dim1_f16": 64 * 256 * 56 * 56,
     }
 
 
@@ -90,7 +97,8 @@ PRODUCT_FLOPS = {"dot_f32_4096": (2 * 4096 ** 3, 157.3), "dot_f16_8192": (2 * 81
 EXTRA_OPS = ("calib_copy", "smooth_softmax_grad_ignore", "softmax3d", "softmax3d_grad", "add_take_grad",
              "bias_add_broadcast", "swapaxis10_reshape", "lrn_scale_chpool5", "transpose_nchw_nhwc",
              "sort_by_key_f32", "dot_f32_4096", "dot_f16_8192", "ceiling_copy", "ceiling_fill",
-             "random_uniform", "random_normal")
+             "random_uniform", "random_normal", "softmax_f16", "softmax_grad_f16", "sum_rows_f16",
+             "sumall_except_dim1_f16")
 OPS = [k for k in algorithmic_bytes() if k not in EXTRA_OPS]
 
 # HBM bytes per launch of each operation's kernel, measured with rocprofv3 --pmc FETCH_SIZE and
@@ -199,6 +207,18 @@ def main():
         extra["out4"] = G.buffer(H["X2a"].shape, f32)
         extra["bias"] = G.to_device(np.random.default_rng(14).standard_normal(51380224, dtype=f32)[:256].copy())
 
+    if any(o.endswith("_f16") and o not in OPS for o in only):
+        extra["hL"] = G.to_device(orc.float2half(H["L"]))
+        extra["hP"] = G.buffer(H["L"].shape, np.uint16)
+        extra["hG"] = G.buffer(H["L"].shape, np.uint16)
+        # labels a half can hold exactly (integers up to 2048)
+        extra["hlab"] = G.to_device(orc.float2half(np.minimum(H["labels"], f32(2048))))
+        extra["hM"] = G.to_device(orc.float2half(H["M2b"]))
+        extra["hX"] = G.to_device(orc.float2half(H["X2a"]))
+        extra["h2b"] = G.buffer((4096,), np.uint16)
+        extra["h2a"] = G.buffer((256,), np.uint16)
+        G.case_softmax(extra["hP"], extra["hL"], s)
+
     if "dot_f32_4096" in only:   # dst = dot(A, B.T()) through the expression engine
         extra["mm_out"] = G.buffer((4096, 4096), f32)
     if "dot_f16_8192" in only:
@@ -217,6 +237,14 @@ def main():
             G.random_normal(out_g, 7, 0, 0, 0.0, 1.0, s)
         elif name == "ceiling_fill":   # dst = scalar
             G.fill(out_g, 1.0, s)
+        elif name == "softmax_f16":     # Softmax(Tensor<gpu,2,half_t>, ...)
+            G.case_softmax(extra["hP"], extra["hL"], s)
+        elif name == "softmax_grad_f16":
+            G.case_softmax_grad(extra["hG"], extra["hP"], extra["hlab"], s)
+        elif name == "sum_rows_f16":    # half_t one is 0x3C00
+            G.case_reduce_keep_lowest(extra["h2b"], extra["hM"], 0, 0, 0x3C00, 0, s)
+        elif name == "sumall_except_dim1_f16":
+            G.case_reduce_keep_highdim(extra["h2a"], extra["hX"], 0, 0, 0x3C00, 0, s)
         elif name == "dot_f32_4096":
             G.case_dot(1, extra["mm_out"], dev["A"], dev["B"], 4096, 4096, 4096, 1, s)
         elif name == "dot_f16_8192":

@@ -161,6 +161,17 @@ inline void SoftmaxGrad(const Tensor<gpu, 2, float> &dst, const Tensor<gpu, 2, f
 }
 /* other element types (half_t, double): kernel templates in the element type's own
    arithmetic, instantiated in the calling translation unit (kernels/softmax_any.h) */
+namespace gpu_detail {
+/*! \brief rows of whole packs that all start 16-byte aligned: 128-bit accesses */
+template <typename DType>
+inline bool AnyPackable(const DType *a, uint32_t astride, const DType *b, uint32_t bstride,
+                        uint32_t cols, int pack) {
+  const size_t addr = reinterpret_cast<size_t>(a) | reinterpret_cast<size_t>(b) |
+                      (static_cast<size_t>(astride) * sizeof(DType)) |
+                      (static_cast<size_t>(bstride) * sizeof(DType));
+  return addr % 16 == 0 && cols % pack == 0;
+}
+}  // namespace gpu_detail
 template <typename DType>
 inline void Softmax(Tensor<gpu, 2, DType> dst, const Tensor<gpu, 2, DType> &src) {
   CHECK_EQ(dst.shape_, src.shape_) << "Softmax: shape mismatch";
@@ -171,10 +182,14 @@ inline void Softmax(Tensor<gpu, 2, DType> dst, const Tensor<gpu, 2, DType> &src)
   const DType *s = src.dptr_;
   uint32_t dstride = dst.stride_, sstride = src.stride_;
   void *args[] = {&d, &dstride, &s, &sstride, &rows, &cols};
-  const uint32_t grid[3] = {(rows + hip::kAnyRowsPerBlock - 1) / hip::kAnyRowsPerBlock, 1, 1};
+  const uint32_t grid[3] = {(rows + hip::kAnyRows - 1) / hip::kAnyRows, 1, 1};
   const uint32_t block[3] = {static_cast<uint32_t>(hip::kAnyBlock), 1, 1};
-  MSHADOW_HIP_CALL(mshadow_hip_launch(reinterpret_cast<const void *>(hip::SoftmaxAnyKernel<DType>),
-                                      grid, block, args, 0, Stream<gpu>::GetStream(dst.stream_)));
+  const bool vec = gpu_detail::AnyPackable(s, sstride, const_cast<const DType *>(d), dstride, cols,
+                                           hip::kAnyTile);
+  const void *kernel = vec ? reinterpret_cast<const void *>(hip::SoftmaxAnyKernel<DType, true>)
+                           : reinterpret_cast<const void *>(hip::SoftmaxAnyKernel<DType, false>);
+  MSHADOW_HIP_CALL(mshadow_hip_launch(kernel, grid, block, args, 0,
+                                      Stream<gpu>::GetStream(dst.stream_)));
 #else
   LOG(FATAL) << "Softmax<gpu> of this element type: compile the calling translation unit with hipcc";
 #endif
@@ -192,13 +207,18 @@ inline void SoftmaxGrad(const Tensor<gpu, 2, DType> &dst, const Tensor<gpu, 2, D
   const DType *l = label.dptr_;
   uint32_t dstride = dst.stride_, sstride = src.stride_;
   void *args[] = {&d, &dstride, &s, &sstride, &l, &cols};
-  /* rows on the grid's x axis (up to 2^31 - 1), a row's columns over a few workgroups */
-  uint32_t per_row = (cols + hip::kAnyBlock * 8 - 1) / (hip::kAnyBlock * 8);
+  /* rows on the grid's x axis (up to 2^31 - 1), a row's packs over a few workgroups */
+  const uint32_t per_block = hip::kAnyBlock * hip::kAnyTile;
+  uint32_t per_row = (cols + per_block - 1) / per_block;
   if (per_row > 64) per_row = 64;
   const uint32_t grid[3] = {rows, per_row, 1};
   const uint32_t block[3] = {static_cast<uint32_t>(hip::kAnyBlock), 1, 1};
-  MSHADOW_HIP_CALL(mshadow_hip_launch(reinterpret_cast<const void *>(hip::SoftmaxGradAnyKernel<DType>),
-                                      grid, block, args, 0, Stream<gpu>::GetStream(dst.stream_)));
+  const bool vec = gpu_detail::AnyPackable(s, sstride, const_cast<const DType *>(d), dstride, cols,
+                                           hip::kAnyTile);
+  const void *kernel = vec ? reinterpret_cast<const void *>(hip::SoftmaxGradAnyKernel<DType, true>)
+                           : reinterpret_cast<const void *>(hip::SoftmaxGradAnyKernel<DType, false>);
+  MSHADOW_HIP_CALL(mshadow_hip_launch(kernel, grid, block, args, 0,
+                                      Stream<gpu>::GetStream(dst.stream_)));
 #else
   LOG(FATAL) << "SoftmaxGrad<gpu> of this element type: compile the calling translation unit with hipcc";
 #endif
