@@ -63,6 +63,13 @@ int mshadow_case_softmax_f16(uint16_t *dst, int dstride, const uint16_t *src, in
                              int rows, int cols, void *stream);
 int mshadow_case_softmax_grad_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride,
                                   const uint16_t *label, int rows, int cols, void *stream);
+/* dst <saver>= a * b + c, and dst = pool<Reducer>(src, (ph, pw), ky, kx, sy, sx), on half_t tensors */
+int mshadow_case_map_muladd_f16(uint16_t *dst, int dstride, const uint16_t *a, int astride,
+                                const uint16_t *b, int bstride, const uint16_t *c, int cstride,
+                                int rows, int cols, int saver, void *stream);
+int mshadow_case_pool_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride, int planes,
+                          int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,
+                          int reducer, void *stream);
 int mshadow_case_softmax_f64(double *dst, int dstride, const double *src, int sstride, int rows,
                              int cols, void *stream);
 

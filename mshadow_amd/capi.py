@@ -107,6 +107,8 @@ CASES_SYMBOLS = {
     "mshadow_case_softmax_f16": ([_p, _i, _p, _i, _i, _i, _p], _i),
     "mshadow_case_softmax_grad_f16": ([_p, _i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_case_softmax_f64": ([_p, _i, _p, _i, _i, _i, _p], _i),
+    "mshadow_case_map_muladd_f16": ([_p, _i, _p, _i, _p, _i, _p, _i, _i, _i, _i, _p], _i),
+    "mshadow_case_pool_f16": ([_p, _i, _p, _i] + [_i] * 10 + [_p], _i),
     "mshadow_case_grad_family_f32": ([_p, _i, _p, _i, _p, _i, _i, _i, _i, _i, _f, _f, _p], _i),
     "mshadow_case_softmax3d_f32": ([_p, _i, _p, _i, _i, _i, _i, _p], _i),
     "mshadow_case_rows_by_index_f32": ([_i, _p, _i, _i, _p, _p, _i, _p, _i, _i, _i, _p], _i),
@@ -508,10 +510,20 @@ class Library:
         self.check_case(fn(dst.ptr, dst.stride, src.ptr, src.stride, label.ptr, src.rows, src.cols,
                            stream))
 
+    def case_map_muladd_f16(self, dst, a, b, c, saver=SAVETO, stream=None):
+        self.check_case(self.cases.mshadow_case_map_muladd_f16(
+            dst.ptr, dst.stride, a.ptr, a.stride, b.ptr, b.stride, c.ptr, c.stride, dst.rows,
+            dst.cols, saver, stream))
+
     def case_pool(self, dst, src, ky, kx, sy, sx, reducer=MAX, variant=0, stream=None):
         h, w = src.shape[-2:]
         ph, pw = dst.shape[-2:]
         planes = int(np.prod(src.shape[:-2]))
+        if src.dtype == np.uint16:   # half_t tensors: the generic expression kernel
+            self.check_case(self.cases.mshadow_case_pool_f16(
+                dst.ptr, dst.stride, src.ptr, src.stride, planes, h, w, ph, pw, ky, kx, sy, sx,
+                reducer, stream))
+            return
         self.check_case(self.cases.mshadow_case_pool_f32(
             dst.ptr, dst.stride, src.ptr, src.stride, planes, h, w, ph, pw, ky, kx, sy, sx,
             reducer, variant, stream))

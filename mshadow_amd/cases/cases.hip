@@ -218,6 +218,33 @@ int mshadow_case_softmax_grad_f16(uint16_t *dst, int dstride, const uint16_t *sr
   CASE_END
 }
 
+/* dst <saver>= a * b + c and pool<Reducer> on half_t tensors (the generic expression kernels) */
+int mshadow_case_map_muladd_f16(uint16_t *dst, int dstride, const uint16_t *a, int astride,
+                                const uint16_t *b, int bstride, const uint16_t *c, int cstride,
+                                int rows, int cols, int saver, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Tensor<gpu, 2, HalfT> A = G2(H(a), rows, cols, astride, st.get()),
+                        B = G2(H(b), rows, cols, bstride, st.get()),
+                        C = G2(H(c), rows, cols, cstride, st.get());
+  Assign(G2(H(dst), rows, cols, dstride, st.get()), A * B + C, saver);
+  CASE_END
+}
+
+int mshadow_case_pool_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride, int planes,
+                          int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,
+                          int reducer, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Tensor<gpu, 3, HalfT> S = G3(H(src), planes, h, w, sstride, st.get());
+  Tensor<gpu, 3, HalfT> o = G3(H(dst), planes, ph, pw, dstride, st.get());
+  const Shape<2> ps = Shape2(ph, pw);
+  if (reducer == 0) o = pool<red::sum>(S, ps, ky, kx, sy, sx);
+  else if (reducer == 1) o = pool<red::maximum>(S, ps, ky, kx, sy, sx);
+  else o = pool<red::minimum>(S, ps, ky, kx, sy, sx);
+  CASE_END
+}
+
 /* Softmax(dst, src) on double tensors */
 int mshadow_case_softmax_f64(double *dst, int dstride, const double *src, int sstride, int rows,
                              int cols, void *stream) {

@@ -303,6 +303,21 @@ static inline uint16_t init_f16(int reducer) {
   }
 }
 
+/* dst <saver>= a * b + c on half_t tensors: the product is a half_t (rounded) before the
+   sum is taken (mshadow/half.h:45-66, expression.h:353-374) */
+void orc_map_muladd_f16(uint16_t *dst, int dstride, const uint16_t *a, int astride,
+                        const uint16_t *b, int bstride, const uint16_t *c, int cstride, int rows,
+                        int cols, int saver) {
+#pragma omp parallel for
+  for (int y = 0; y < rows; ++y) {
+    for (int x = 0; x < cols; ++x) {
+      const uint16_t ab = half_of(wide(a[(int64_t)y * astride + x]) * wide(b[(int64_t)y * bstride + x]));
+      const uint16_t v = half_of(wide(ab) + wide(c[(int64_t)y * cstride + x]));
+      save_f16(&dst[(int64_t)y * dstride + x], v, saver);
+    }
+  }
+}
+
 /* MapReduceKeepLowest on half_t, mshadow/tensor_cpu-inl.h:203-228 */
 void orc_reduce_keep_lowest_f16(uint16_t *dst, const uint16_t *src, int sstride, int rows,
                                 int cols, int reducer, int saver, uint16_t scale) {
@@ -544,6 +559,30 @@ void orc_pool_f32(float *dst, int dstride, const float *src, int sstride, int pl
       for (int y = y_start; y < y_end; ++y) {
         for (int x = x_start; x < x_end; ++x) {
           reduce_f32(&res, src[(int64_t)(c * h + y) * sstride + x], reducer);
+        }
+      }
+      dst[(int64_t)i * dstride + j] = res;
+    }
+  }
+}
+
+/* the same on half_t tensors: red::sum rounds to 16 bits after every add */
+void orc_pool_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride, int planes, int h,
+                  int w, int ph, int pw, int ky, int kx, int sy, int sx, int reducer) {
+  const int out_rows = planes * ph;
+#pragma omp parallel for
+  for (int i = 0; i < out_rows; ++i) {
+    const int py = i % ph;
+    const int c = i / ph;
+    const int y_start = py * sy;
+    const int y_end = imin(y_start + ky, h);
+    for (int j = 0; j < pw; ++j) {
+      const int x_start = j * sx;
+      const int x_end = imin(x_start + kx, w);
+      uint16_t res = init_f16(reducer);
+      for (int y = y_start; y < y_end; ++y) {
+        for (int x = x_start; x < x_end; ++x) {
+          reduce_f16(&res, src[(int64_t)(c * h + y) * sstride + x], reducer);
         }
       }
       dst[(int64_t)i * dstride + j] = res;

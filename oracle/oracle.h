@@ -61,6 +61,11 @@ void orc_reduce_keep_lowest_f16(uint16_t *dst, const uint16_t *src, int sstride,
                                 int cols, int reducer, int saver, uint16_t scale);
 void orc_reduce_keep_highdim_f16(uint16_t *dst, const uint16_t *src, int sstride, int n, int c,
                                  int y, int x, int reducer, int saver, uint16_t scale);
+void orc_map_muladd_f16(uint16_t *dst, int dstride, const uint16_t *a, int astride,
+                        const uint16_t *b, int bstride, const uint16_t *c, int cstride, int rows,
+                        int cols, int saver);
+void orc_pool_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride, int planes, int h,
+                  int w, int ph, int pw, int ky, int kx, int sy, int sx, int reducer);
 void orc_softmax_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride, int rows,
                      int cols);
 void orc_softmax_grad_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride,

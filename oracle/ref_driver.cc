@@ -168,6 +168,23 @@ void ref_reduce_keep_highdim_f16(uint16_t *dst, const uint16_t *src, int sstride
   else ReduceHighHalf<red::minimum>(o, S, saver, sc);
 }
 
+void ref_map_muladd_f16(uint16_t *dst, int dstride, const uint16_t *a, int astride,
+                        const uint16_t *b, int bstride, const uint16_t *c, int cstride, int rows,
+                        int cols, int saver) {
+  Tensor<cpu, 2, HalfT> A = T2(H(a), rows, cols, astride), B = T2(H(b), rows, cols, bstride),
+                        C = T2(H(c), rows, cols, cstride);
+  Assign(T2(H(dst), rows, cols, dstride), A * B + C, saver);
+}
+
+void ref_pool_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride, int planes, int h,
+                  int w, int ph, int pw, int ky, int kx, int sy, int sx, int reducer) {
+  Tensor<cpu, 3, HalfT> S = T3(H(src), planes, h, w, sstride);
+  Tensor<cpu, 3, HalfT> o = T3(H(dst), planes, ph, pw, dstride);
+  if (reducer == 0) o = pool<red::sum>(S, Shape2(ph, pw), ky, kx, sy, sx);
+  else if (reducer == 1) o = pool<red::maximum>(S, Shape2(ph, pw), ky, kx, sy, sx);
+  else o = pool<red::minimum>(S, Shape2(ph, pw), ky, kx, sy, sx);
+}
+
 void ref_softmax_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride, int rows,
                      int cols) {
   Softmax(T2(H(dst), rows, cols, dstride), T2(H(src), rows, cols, sstride));

@@ -80,6 +80,8 @@ class Checker:
         _h = C.c_uint16
         self._fn("reduce_keep_lowest_f16", [_p, _p, _i, _i, _i, _i, _i, _h])
         self._fn("reduce_keep_highdim_f16", [_p, _p, _i, _i, _i, _i, _i, _i, _i, _h])
+        self._fn("map_muladd_f16", [_p, _i, _p, _i, _p, _i, _p, _i, _i, _i, _i])
+        self._fn("pool_f16", [_p, _i, _p, _i] + [_i] * 10)
         self._fn("softmax_f16", [_p, _i, _p, _i, _i, _i])
         self._fn("softmax_grad_f16", [_p, _i, _p, _i, _p, _i, _i])
         self._fn("softmax_grad_ex_f32", [_p, _i, _p, _i, _p, _i, _i, _i, _f, _f])
@@ -253,10 +255,20 @@ class Checker:
         return out
 
     # -- pool / unpool: arrays are (..., H, W); leading dims are planes
+    def map_muladd_f16(self, dst, a, b, c, saver=SAVETO):
+        rows, cols = int(np.prod(dst.shape[:-1])), dst.shape[-1]
+        self._map_muladd_f16(ptr(dst), pitch(dst), ptr(a), pitch(a), ptr(b), pitch(b), ptr(c),
+                             pitch(c), rows, cols, saver)
+        return dst
+
     def pool(self, dst, src, ky, kx, sy, sx, reducer=MAX):
         h, w = src.shape[-2:]
         ph, pw = dst.shape[-2:]
         planes = int(np.prod(src.shape[:-2]))
+        if src.dtype == np.uint16:
+            self._pool_f16(ptr(dst), pitch(dst), ptr(src), pitch(src), planes, h, w, ph, pw, ky,
+                           kx, sy, sx, reducer)
+            return dst
         self._pool_f32(ptr(dst), pitch(dst), ptr(src), pitch(src), planes, h, w, ph, pw, ky, kx,
                        sy, sx, reducer)
         return dst

@@ -106,6 +106,42 @@ def test_half_highdim_oracle_equals_reference(orc, ref, shape):
             assert np.array_equal(oa, ob), (reducer, saver)
 
 
+def test_half_map_and_pool_known_answers(orc):
+    # a * b rounds before + c: 1.001 * 1.001 = 1.00195 in 16 bits, where the exact product
+    # 1.0019541 + 2^-11 * 0.9 would round the sum differently
+    a = orc.float2half(np.full((2, 3), 1.0009765625, f32))          # 1 + 2^-10
+    c = orc.float2half(np.full((2, 3), 0.00048828125, f32))         # 2^-11
+    out = np.empty_like(a)
+    orc.map_muladd_f16(out, a, a, c)
+    prod = orc.float2half(orc.half2float(a) * orc.half2float(a))     # 1 + 2^-9 (the 2^-20 is lost)
+    assert np.all(orc.half2float(prod) == f32(1.001953125))
+    assert np.array_equal(out, orc.float2half(orc.half2float(prod) + orc.half2float(c)))
+    # pool<sum> of a 50 x 50 window of ones: the running 16-bit sum stops at 2048
+    img = orc.float2half(np.ones((1, 50, 50), f32))
+    o = np.empty((1, 1, 1), np.uint16)
+    orc.pool(o, img, 50, 50, 1, 1, reducer=SUM)
+    assert orc.half2float(o)[0, 0, 0] == 2048.0
+
+
+@pytest.mark.skipif(not have_ref(), reason="reference build absent")
+def test_half_map_and_pool_oracle_equals_reference(orc, ref):
+    a, b, c = (halves(orc, 70 + i, (37, 53), 2.0) for i in range(3))
+    for saver in (SAVETO, PLUSTO, MINUSTO, MULTO, DIVTO):
+        oa = halves(orc, 73, (37, 53))
+        ob = oa.copy()
+        orc.map_muladd_f16(oa, a, b, c, saver)
+        ref.map_muladd_f16(ob, a, b, c, saver)
+        assert np.array_equal(oa, ob), saver
+    img = halves(orc, 74, (3, 4, 23, 29))
+    for reducer in (SUM, MAX, MIN):
+        for (ky, kx, sy, sx) in ((3, 3, 2, 2), (2, 5, 1, 3)):
+            shape = (3, 4, (23 - ky) // sy + 1, (29 - kx) // sx + 1)
+            pa, pb = np.empty(shape, np.uint16), np.empty(shape, np.uint16)
+            orc.pool(pa, img, ky, kx, sy, sx, reducer)
+            ref.pool(pb, img, ky, kx, sy, sx, reducer)
+            assert np.array_equal(pa, pb), (reducer, ky, kx)
+
+
 # ------------------------------------------------------------------ GPU parity
 @pytest.fixture(scope="module")
 def G():
@@ -216,3 +252,35 @@ def test_gpu_double_softmax(G, stream, shape):
     G.case_softmax(dst, G.to_device(x), stream)
     got = dst.download(stream)
     assert np.all(np.abs(got - want) <= 1e-13 * want + 1e-300)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape,pad", [((1, 1), 0), ((37, 53), 3), ((256, 1024), 0), ((33, 4096), 0)])
+def test_gpu_half_map(G, orc, stream, shape, pad):
+    """dst <saver>= a * b + c on half_t tensors through the generic expression kernels, bit-exact"""
+    a, b, c = (halves(orc, 80 + i, shape, 2.0) for i in range(3))
+    da, db, dc = (G.to_device(t, pad) for t in (a, b, c))
+    for saver in (SAVETO, PLUSTO, MINUSTO, MULTO, DIVTO):
+        init = halves(orc, 83, shape)
+        want = init.copy()
+        orc.map_muladd_f16(want, a, b, c, saver)
+        dst = G.to_device(init, pad)
+        G.case_map_muladd_f16(dst, da, db, dc, saver, stream)
+        assert np.array_equal(dst.download(stream), want), saver
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("window", [(3, 3, 2, 2), (2, 5, 1, 3), (50, 50, 1, 1)])
+def test_gpu_half_pool(G, orc, stream, window):
+    ky, kx, sy, sx = window
+    img = halves(orc, 90, (3, 4, 56, 61))
+    if window == (50, 50, 1, 1):
+        img = orc.float2half(np.ones((3, 4, 56, 61), f32))   # sums stop at 2048 in window order
+    shape = (3, 4, (56 - ky) // sy + 1, (61 - kx) // sx + 1)
+    src = G.to_device(img)
+    for reducer in (SUM, MAX, MIN):
+        want = np.empty(shape, np.uint16)
+        orc.pool(want, img, ky, kx, sy, sx, reducer)
+        dst = G.buffer(shape, np.uint16)
+        G.case_pool(dst, src, ky, kx, sy, sx, reducer, 0, stream)
+        assert np.array_equal(dst.download(stream), want), reducer
