@@ -7,18 +7,20 @@
  * terms (4096 equal logits give 1/2048 each, not 1/4096), and only the left-to-right order
  * reproduces it.
  *
- * A workgroup of 256 threads takes kAnyRows = 8 rows, 32 threads per row, each thread a pack
- * of kAnyTile = 8 consecutive elements per step (one 128-bit access for half_t when rows are
- * aligned whole packs). The maximum is a reduction over the 32 threads (exact in any order).
- * The rows then pass in tiles of 256 columns: every thread computes its pack of terms (the
- * next tile's logits are already on their way), stores it to dst and parks it in LDS; eight
- * lanes of one wave then each add one row's 256 terms to that row's running sum, term by
- * term. A wave instruction costs the same for one active lane as for sixty-four, so the
- * chains of the eight rows share their instructions. A last pass divides the stored terms.
- * Measured for 8192 x 32000 half_t: 712 us; making the terms a second time from the logits
- * instead of storing them and reading them back 783 us; four or sixteen rows per workgroup
- * 843 and 824 us. A thread only ever reads back and writes the elements it handled itself,
- * so in-place calls (dst == src) are safe.
+ * A workgroup of 256 threads takes kAnyRows = 8 rows, 32 threads per row, each thread four
+ * packs of kAnyTile = 8 consecutive elements per step (128-bit accesses for half_t when rows are
+ * aligned whole packs; a row is visited in contiguous stretches of 1024 elements). The maximum
+ * is a reduction over the row's 32 threads (exact in any order). The rows then pass in tiles
+ * of 1024 columns: every thread computes its packs of terms (the next tile's logits are
+ * already on their way), stores them to dst and parks them in LDS; eight lanes of one wave
+ * then each add one row's 1024 terms to that row's running sum, term by term, four packs
+ * being added while the next four come from LDS. A wave instruction costs the same for one
+ * active lane as for sixty-four, so the chains of the eight rows share their instructions
+ * (one wave per row: 1457 us for 8192 x 32000 half_t; this kernel: 692 us; four or
+ * sixteen rows per workgroup were slower, as was making the terms a second time from the
+ * logits instead of storing them and reading them back). A last pass divides the stored
+ * terms. A thread only ever reads back and writes the elements it handled itself, so
+ * in-place calls (dst == src) are safe.
  *
  * The float versions are the fixed-function kernels of the library (csrc/softmax_kernels.h).
  */
@@ -37,7 +39,12 @@ const int kAnyRows = 8;
 /*! \brief consecutive elements of one thread per step */
 const int kAnyTile = 8;
 const int kAnyThreadsPerRow = kAnyBlock / kAnyRows;
-const int kAnyTileCols = kAnyThreadsPerRow * kAnyTile;
+/*! \brief packs of one thread per step: a row is visited in stretches of
+ *  kAnyBatch * kAnyThreadsPerRow packs (2 KB of half_t), pack q of thread p being pack
+ *  q * kAnyThreadsPerRow + p of the stretch, so that a wave's accesses stay contiguous */
+const int kAnyBatch = 4;
+const int kAnyStepCols = kAnyThreadsPerRow * kAnyTile;
+const int kAnyTileCols = kAnyBatch * kAnyStepCols;
 /*! \brief row pitch of the LDS tile: one pack more than it holds, so that the eight chain
  *  lanes read from different banks */
 const int kAnyPitch = kAnyTileCols + kAnyTile;
@@ -122,13 +129,25 @@ __global__ void __launch_bounds__(kAnyBlock)
   const DType first = e[0];
   Wide m = static_cast<Wide>(first);
   if (live) {
-    for (uint32_t x = p * kAnyTile; x < cols; x += kAnyTileCols) {
-      AnyPack<DType> in;
-      LoadAnyPack<DType, VEC>(&in, e, x, cols, first);
+    for (uint32_t x0 = 0; x0 < cols; x0 += kAnyTileCols) {
+      AnyPack<DType> in[kAnyBatch];
 #pragma unroll
-      for (int i = 0; i < kAnyTile; ++i) {
-        const Wide v = static_cast<Wide>(in.v[i]);
-        m = (m < v) ? v : m;
+      for (int q = 0; q < kAnyBatch; ++q) {
+        const uint32_t x = x0 + (q * kAnyThreadsPerRow + p) * kAnyTile;
+        if (x < cols) {
+          LoadAnyPack<DType, VEC>(&in[q], e, x, cols, first);
+        } else {
+#pragma unroll
+          for (int i = 0; i < kAnyTile; ++i) in[q].v[i] = first;
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < kAnyBatch; ++q) {
+#pragma unroll
+        for (int i = 0; i < kAnyTile; ++i) {
+          const Wide v = static_cast<Wide>(in[q].v[i]);
+          m = (m < v) ? v : m;
+        }
       }
     }
   }
@@ -147,21 +166,30 @@ __global__ void __launch_bounds__(kAnyBlock)
   const bool chain_slot = (threadIdx.x >> 6) == chain_wave && c < static_cast<uint32_t>(kAnyRows);
   const bool chain_lane = chain_slot && blockIdx.x * kAnyRows + c < rows;
   DType sum = DType(0.0f);
-  /* the pack of the next tile is fetched before this tile's terms are computed and summed */
-  AnyPack<DType> in;
-  bool have = live && p * kAnyTile < cols;
-  if (have) LoadAnyPack<DType, VEC>(&in, e, p * kAnyTile, cols, mmax);
-  for (uint32_t x0 = 0; x0 < cols; x0 += kAnyTileCols) {
-    const uint32_t x = x0 + p * kAnyTile;
-    AnyPack<DType> next = in;
-    const bool have_next = live && x + kAnyTileCols < cols;
-    if (have_next) LoadAnyPack<DType, VEC>(&next, e, x + kAnyTileCols, cols, mmax);
-    if (have) {
-      AnyPack<DType> t;
+  /* the packs of the next tile are fetched before this tile's terms are computed and summed */
+  AnyPack<DType> in[kAnyBatch];
 #pragma unroll
-      for (int i = 0; i < kAnyTile; ++i) t.v[i] = DType(SoftmaxExp(in.v[i] - mmax));
-      StoreAnyPack<DType, VEC>(o, x, cols, t);
-      tile_packs[r][p] = t;
+  for (int q = 0; q < kAnyBatch; ++q) {
+    const uint32_t x = (q * kAnyThreadsPerRow + p) * kAnyTile;
+    if (live && x < cols) LoadAnyPack<DType, VEC>(&in[q], e, x, cols, mmax);
+  }
+  for (uint32_t x0 = 0; x0 < cols; x0 += kAnyTileCols) {
+    AnyPack<DType> next[kAnyBatch];
+#pragma unroll
+    for (int q = 0; q < kAnyBatch; ++q) {
+      const uint32_t x = x0 + kAnyTileCols + (q * kAnyThreadsPerRow + p) * kAnyTile;
+      if (live && x < cols) LoadAnyPack<DType, VEC>(&next[q], e, x, cols, mmax);
+    }
+#pragma unroll
+    for (int q = 0; q < kAnyBatch; ++q) {
+      const uint32_t x = x0 + (q * kAnyThreadsPerRow + p) * kAnyTile;
+      if (live && x < cols) {
+        AnyPack<DType> t;
+#pragma unroll
+        for (int i = 0; i < kAnyTile; ++i) t.v[i] = DType(SoftmaxExp(in[q].v[i] - mmax));
+        StoreAnyPack<DType, VEC>(o, x, cols, t);
+        tile_packs[r][q * kAnyThreadsPerRow + p] = t;
+      }
     }
     __syncthreads();
     if (chain_lane) {
@@ -170,8 +198,7 @@ __global__ void __launch_bounds__(kAnyBlock)
       const uint32_t full = n / kAnyTile;  // whole packs
       uint32_t k = 0;
       if (full >= 4) {
-        /* four packs are added while the next four are on their way from LDS: the adds of
-           a group take longer than an LDS read */
+        /* four packs are added while the next four are on their way from LDS */
         AnyPack<DType> a[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) a[q] = mine[q];
@@ -179,7 +206,6 @@ __global__ void __launch_bounds__(kAnyBlock)
           AnyPack<DType> b[4];
 #pragma unroll
           for (int q = 0; q < 4; ++q) b[q] = mine[k + 4 + q];
-          __builtin_amdgcn_sched_barrier(0);  // the reads are issued before the adds, not among them
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
 #pragma unroll
@@ -202,12 +228,15 @@ __global__ void __launch_bounds__(kAnyBlock)
       }
       if (k * kAnyTile < n) {
         const AnyPack<DType> t = mine[k];
-        for (uint32_t i = 0; k * kAnyTile + i < n; ++i) ChainAdd(sum, t.v[i]);
+#pragma unroll
+        for (int i = 0; i < kAnyTile; ++i) {  // unrolled: a run-time index would put t in scratch memory
+          if (k * kAnyTile + i < n) ChainAdd(sum, t.v[i]);
+        }
       }
     }
     __syncthreads();
-    in = next;
-    have = have_next;
+#pragma unroll
+    for (int q = 0; q < kAnyBatch; ++q) in[q] = next[q];
   }
   if (chain_slot) sums[c] = sum;
   __syncthreads();
@@ -215,12 +244,22 @@ __global__ void __launch_bounds__(kAnyBlock)
 
   /* every thread reads back only what it stored itself */
   if (live) {
-    for (uint32_t x = p * kAnyTile; x < cols; x += kAnyTileCols) {
-      AnyPack<DType> t;
-      LoadAnyPack<DType, VEC>(&t, o, x, cols, sum);
+    for (uint32_t x0 = 0; x0 < cols; x0 += kAnyTileCols) {
+      AnyPack<DType> t[kAnyBatch];
 #pragma unroll
-      for (int i = 0; i < kAnyTile; ++i) t.v[i] /= sum;
-      StoreAnyPack<DType, VEC>(o, x, cols, t);
+      for (int q = 0; q < kAnyBatch; ++q) {
+        const uint32_t x = x0 + (q * kAnyThreadsPerRow + p) * kAnyTile;
+        if (x < cols) LoadAnyPack<DType, VEC>(&t[q], o, x, cols, sum);
+      }
+#pragma unroll
+      for (int q = 0; q < kAnyBatch; ++q) {
+        const uint32_t x = x0 + (q * kAnyThreadsPerRow + p) * kAnyTile;
+        if (x < cols) {
+#pragma unroll
+          for (int i = 0; i < kAnyTile; ++i) t[q].v[i] /= sum;
+          StoreAnyPack<DType, VEC>(o, x, cols, t[q]);
+        }
+      }
     }
   }
 }
