@@ -14,13 +14,15 @@
  * of 1024 columns: every thread computes its packs of terms (the next tile's logits are
  * already on their way), stores them to dst and parks them in LDS; eight lanes of one wave
  * then each add one row's 1024 terms to that row's running sum, term by term, four packs
- * being added while the next four come from LDS. A wave instruction costs the same for one
- * active lane as for sixty-four, so the chains of the eight rows share their instructions
- * (one wave per row: 1457 us for 8192 x 32000 half_t; this kernel: 692 us; four or
- * sixteen rows per workgroup were slower, as was making the terms a second time from the
- * logits instead of storing them and reading them back). A last pass divides the stored
- * terms. A thread only ever reads back and writes the elements it handled itself, so
- * in-place calls (dst == src) are safe.
+ * being added while the next four come from LDS, and while the other waves make the next
+ * tile in the second LDS buffer. A wave instruction costs the same for one active lane as
+ * for sixty-four, so the chains of the eight rows share their instructions (one wave per
+ * row: 1457 us for 8192 x 32000 half_t; this kernel: 670 us, of which the five passes over
+ * memory - logits twice, terms written, read back and written again - would take about 440
+ * at the rate of a plain copy; four or sixteen rows per workgroup were slower, as was making
+ * the terms a second time from the logits instead of storing them and reading them back).
+ * A last pass divides the stored terms. A thread only ever reads back and writes the
+ * elements it handled itself, so in-place calls (dst == src) are safe.
  *
  * The float versions are the fixed-function kernels of the library (csrc/softmax_kernels.h).
  */
@@ -115,7 +117,7 @@ __global__ void __launch_bounds__(kAnyBlock)
     SoftmaxAnyKernel(DType *dst, uint32_t dstride, const DType *src, uint32_t sstride,
                      uint32_t rows, uint32_t cols) {
   typedef typename WideOf<DType>::Type Wide;
-  __shared__ AnyPack<DType> tile_packs[kAnyRows][kAnyPitch / kAnyTile];
+  __shared__ AnyPack<DType> tile_packs[2][kAnyRows][kAnyPitch / kAnyTile];
   __shared__ DType sums[kAnyRows];
   const uint32_t r = threadIdx.x / kAnyThreadsPerRow;
   const uint32_t p = threadIdx.x % kAnyThreadsPerRow;
@@ -173,28 +175,38 @@ __global__ void __launch_bounds__(kAnyBlock)
     const uint32_t x = (q * kAnyThreadsPerRow + p) * kAnyTile;
     if (live && x < cols) LoadAnyPack<DType, VEC>(&in[q], e, x, cols, mmax);
   }
-  for (uint32_t x0 = 0; x0 < cols; x0 += kAnyTileCols) {
-    AnyPack<DType> next[kAnyBatch];
+  /* Tile i's terms are added while tile i + 1 is being made: in step i every thread makes its
+     packs of tile i (LDS buffer i & 1), then the chain lanes add tile i - 1 from the other
+     buffer, then all meet. One step more than there are tiles adds the last one. A buffer is
+     written again two steps after it was written, one barrier after it was last read. */
+  const uint32_t ntiles = (cols + kAnyTileCols - 1) / kAnyTileCols;
+  for (uint32_t step = 0; step <= ntiles; ++step) {
+    const uint32_t x0 = step * kAnyTileCols;
+    if (step < ntiles) {
+      AnyPack<DType> next[kAnyBatch];
 #pragma unroll
-    for (int q = 0; q < kAnyBatch; ++q) {
-      const uint32_t x = x0 + kAnyTileCols + (q * kAnyThreadsPerRow + p) * kAnyTile;
-      if (live && x < cols) LoadAnyPack<DType, VEC>(&next[q], e, x, cols, mmax);
-    }
-#pragma unroll
-    for (int q = 0; q < kAnyBatch; ++q) {
-      const uint32_t x = x0 + (q * kAnyThreadsPerRow + p) * kAnyTile;
-      if (live && x < cols) {
-        AnyPack<DType> t;
-#pragma unroll
-        for (int i = 0; i < kAnyTile; ++i) t.v[i] = DType(SoftmaxExp(in[q].v[i] - mmax));
-        StoreAnyPack<DType, VEC>(o, x, cols, t);
-        tile_packs[r][q * kAnyThreadsPerRow + p] = t;
+      for (int q = 0; q < kAnyBatch; ++q) {
+        const uint32_t x = x0 + kAnyTileCols + (q * kAnyThreadsPerRow + p) * kAnyTile;
+        if (live && x < cols) LoadAnyPack<DType, VEC>(&next[q], e, x, cols, mmax);
       }
+#pragma unroll
+      for (int q = 0; q < kAnyBatch; ++q) {
+        const uint32_t x = x0 + (q * kAnyThreadsPerRow + p) * kAnyTile;
+        if (live && x < cols) {
+          AnyPack<DType> t;
+#pragma unroll
+          for (int i = 0; i < kAnyTile; ++i) t.v[i] = DType(SoftmaxExp(in[q].v[i] - mmax));
+          StoreAnyPack<DType, VEC>(o, x, cols, t);
+          tile_packs[step & 1u][r][q * kAnyThreadsPerRow + p] = t;
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < kAnyBatch; ++q) in[q] = next[q];
     }
-    __syncthreads();
-    if (chain_lane) {
-      const uint32_t n = cols - x0 < static_cast<uint32_t>(kAnyTileCols) ? cols - x0 : kAnyTileCols;
-      const AnyPack<DType> *mine = tile_packs[c];
+    if (chain_lane && step > 0) {
+      const uint32_t done = x0 - kAnyTileCols;  // first column of the tile being added
+      const uint32_t n = cols - done < static_cast<uint32_t>(kAnyTileCols) ? cols - done : kAnyTileCols;
+      const AnyPack<DType> *mine = tile_packs[(step - 1u) & 1u][c];
       const uint32_t full = n / kAnyTile;  // whole packs
       uint32_t k = 0;
       if (full >= 4) {
@@ -235,8 +247,6 @@ __global__ void __launch_bounds__(kAnyBlock)
       }
     }
     __syncthreads();
-#pragma unroll
-    for (int q = 0; q < kAnyBatch; ++q) in[q] = next[q];
   }
   if (chain_slot) sums[c] = sum;
   __syncthreads();
