@@ -284,3 +284,35 @@ def test_gpu_half_pool(G, orc, stream, window):
         dst = G.buffer(shape, np.uint16)
         G.case_pool(dst, src, ky, kx, sy, sx, reducer, 0, stream)
         assert np.array_equal(dst.download(stream), want), reducer
+
+
+@pytest.mark.gpu
+def test_gpu_half_softmax_full_size(G, orc, stream):
+    """8192 x 32000 half_t logits N(0, 3): forward within relative 2e-3 of the CPU path (the
+    differences counted and printed; none observed), the gradient bit for bit, and the
+    size-independent property that the gradient differs from the probabilities at the label
+    of each row and nowhere else"""
+    rows, cols = 8192, 32000
+    x = orc.float2half(np.random.default_rng(7).standard_normal((rows, cols), dtype=f32) * f32(3))
+    want = np.empty_like(x)
+    orc.softmax(want, x)
+    src = G.to_device(x)
+    dst = G.buffer(x.shape, np.uint16)
+    G.case_softmax(dst, src, stream)
+    got = dst.download(stream)
+    differ = got != want
+    print(f"half softmax {x.shape}: {int(differ.sum())} of {got.size} outputs differ from the CPU path")
+    if differ.any():
+        w = orc.half2float(want[differ]).astype(np.float64)
+        g = orc.half2float(got[differ]).astype(np.float64)
+        assert np.all(np.abs(g - w) <= np.maximum(2e-3 * np.abs(w), 2.0 ** -24))
+    lab = orc.float2half(np.random.default_rng(8).integers(0, 2049, rows).astype(f32))
+    gd = G.buffer(x.shape, np.uint16)
+    G.case_softmax_grad(gd, dst, G.to_device(lab), stream)
+    grad = gd.download(stream)
+    gw = np.empty_like(got)
+    orc.softmax_grad(gw, got, lab)
+    assert np.array_equal(grad, gw)
+    changed = np.argwhere(grad != got)
+    assert np.array_equal(changed[:, 0], np.arange(rows))
+    assert np.array_equal(changed[:, 1], orc.half2float(lab).astype(np.int64))
