@@ -70,6 +70,10 @@ int mshadow_case_map_muladd_f16(uint16_t *dst, int dstride, const uint16_t *a, i
 int mshadow_case_pool_f16(uint16_t *dst, int dstride, const uint16_t *src, int sstride, int planes,
                           int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,
                           int reducer, void *stream);
+/* dst = scale * reduce_except_dim<1, Reducer>(src) on double tensors: n == 0 takes src as y rows of
+   x columns and keeps the columns (sum_rows), otherwise src is (n, c, y, x) and c is kept */
+int mshadow_case_reduce_f64(double *dst, const double *src, int sstride, int n, int c, int y, int x,
+                            int reducer, double scale, void *stream);
 int mshadow_case_softmax_f64(double *dst, int dstride, const double *src, int sstride, int rows,
                              int cols, void *stream);
 

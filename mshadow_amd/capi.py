@@ -107,6 +107,7 @@ CASES_SYMBOLS = {
     "mshadow_case_softmax_f16": ([_p, _i, _p, _i, _i, _i, _p], _i),
     "mshadow_case_softmax_grad_f16": ([_p, _i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_case_softmax_f64": ([_p, _i, _p, _i, _i, _i, _p], _i),
+    "mshadow_case_reduce_f64": ([_p, _p, _i, _i, _i, _i, _i, _i, C.c_double, _p], _i),
     "mshadow_case_map_muladd_f16": ([_p, _i, _p, _i, _p, _i, _p, _i, _i, _i, _i, _p], _i),
     "mshadow_case_pool_f16": ([_p, _i, _p, _i] + [_i] * 10 + [_p], _i),
     "mshadow_case_grad_family_f32": ([_p, _i, _p, _i, _p, _i, _i, _i, _i, _i, _f, _f, _p], _i),
@@ -509,6 +510,15 @@ class Library:
               else self.cases.mshadow_case_softmax_grad_f32)
         self.check_case(fn(dst.ptr, dst.stride, src.ptr, src.stride, label.ptr, src.rows, src.cols,
                            stream))
+
+    def case_reduce_f64(self, dst, src, reducer=SUM, scale=1.0, stream=None):
+        """double tensors: a 2-D src keeps its columns, a 4-D src (n, c, y, x) keeps c"""
+        if len(src.shape) == 2:
+            n, c, (y, x) = 0, 0, src.shape
+        else:
+            n, c, y, x = src.shape
+        self.check_case(self.cases.mshadow_case_reduce_f64(dst.ptr, src.ptr, src.stride, n, c, y, x,
+                                                           reducer, scale, stream))
 
     def case_map_muladd_f16(self, dst, a, b, c, saver=SAVETO, stream=None):
         self.check_case(self.cases.mshadow_case_map_muladd_f16(

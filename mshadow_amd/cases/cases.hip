@@ -245,6 +245,22 @@ int mshadow_case_pool_f16(uint16_t *dst, int dstride, const uint16_t *src, int s
   CASE_END
 }
 
+/* dst = scale * reduce_except_dim<1, Reducer>(src) on double tensors: 2-D (n == 0: rows x cols =
+   c x x... see the arguments) or 4-D (n, c, y, x) */
+int mshadow_case_reduce_f64(double *dst, const double *src, int sstride, int n, int c, int y, int x,
+                            int reducer, double scale, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  if (n == 0) {  // 2-D: y rows, x columns, keeps the columns
+    Tensor<gpu, 2, double> S = G2(src, y, x, sstride, st.get());
+    ReduceDispatch(G1(dst, x, st.get()), S, reducer, 0, scale);
+  } else {
+    Tensor<gpu, 4, double> S = G4(src, n, c, y, x, sstride, st.get());
+    ReduceDispatch(G1(dst, c, st.get()), S, reducer, 0, scale);
+  }
+  CASE_END
+}
+
 /* Softmax(dst, src) on double tensors */
 int mshadow_case_softmax_f64(double *dst, int dstride, const double *src, int sstride, int rows,
                              int cols, void *stream) {

@@ -41,6 +41,13 @@ const int kLowestCols = 16;
  *  used when the reduction is long enough to fill its pipeline */
 const int kRedBlockSmall = 256;
 const int kRedBlockLarge = 1024;
+/*! \brief the large workgroup for element type DType: its two staging tiles hold
+ *  2 * THREADS * kRedDepth elements, which for 8-byte types fits the 160 KB of LDS only with
+ *  the small workgroup */
+template <typename DType>
+struct RedBlockLargeFor {
+  static const int value = sizeof(DType) <= 4 ? kRedBlockLarge : kRedBlockSmall;
+};
 
 /*! \brief value of v in lane `lane` for any small trivially copyable type */
 template <typename DType>

@@ -781,9 +781,9 @@ inline void MapReduceKeepLowest(TRValue<R, gpu, 1, DType> *dst,
   void *stream = Stream<gpu>::GetStream(expr::StreamInfo<gpu, R>::Get(dst->self()));
   const uint32_t strips = (cols + hip::kLowestCols - 1) / hip::kLowestCols;
   if (rows >= 4096) {
-    gpu_detail::Launch(hip::ReduceKeepLowestKernel<Saver, Reducer, DType, hip::kRedBlockLarge,
+    gpu_detail::Launch(hip::ReduceKeepLowestKernel<Saver, Reducer, DType, hip::RedBlockLargeFor<DType>::value,
                                                    DPlan, SPlan>,
-                       strips, hip::kRedBlockLarge, args, stream);
+                       strips, hip::RedBlockLargeFor<DType>::value, args, stream);
   } else {
     gpu_detail::Launch(hip::ReduceKeepLowestKernel<Saver, Reducer, DType, hip::kRedBlockSmall,
                                                    DPlan, SPlan>,
@@ -827,9 +827,9 @@ inline void MapReduceKeepHighDim(TRValue<R, gpu, 1, DType> *dst,
   const bool large = static_cast<uint64_t>(n_out) * n_y * n_x >= (1u << 18);
 #define MSHADOW_HIGHDIM_LAUNCH(SEGS)                                                          \
   if (large) {                                                                                \
-    gpu_detail::Launch(hip::ReduceKeepHighDimKernel<Saver, Reducer, DType, hip::kRedBlockLarge, \
+    gpu_detail::Launch(hip::ReduceKeepHighDimKernel<Saver, Reducer, DType, hip::RedBlockLargeFor<DType>::value, \
                                                     SEGS, DPlan, SPlan>,                      \
-                       n_keep, hip::kRedBlockLarge, args, stream);                            \
+                       n_keep, hip::RedBlockLargeFor<DType>::value, args, stream);                            \
   } else {                                                                                    \
     gpu_detail::Launch(hip::ReduceKeepHighDimKernel<Saver, Reducer, DType, hip::kRedBlockSmall, \
                                                     SEGS, DPlan, SPlan>,                      \

@@ -316,3 +316,27 @@ def test_gpu_half_softmax_full_size(G, orc, stream):
     changed = np.argwhere(grad != got)
     assert np.array_equal(changed[:, 0], np.arange(rows))
     assert np.array_equal(changed[:, 1], orc.half2float(lab).astype(np.int64))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(1, 1), (5000, 7), (300, 130), (3, 5, 7, 9), (20, 6, 28, 28)])
+def test_gpu_double_reductions(G, stream, shape):
+    """sum_rows / sumall_except_dim<1> (and max, min) on double tensors through the generic
+    reduction kernels, bit for bit against the CPU path's order restated with numpy's
+    sequential float64 accumulate (mshadow/tensor_cpu-inl.h:203-268)"""
+    x = np.random.default_rng(61).standard_normal(shape)
+    src = G.to_device(x)
+    if len(shape) == 2:
+        want = {SUM: np.add.accumulate(x, axis=0)[-1], MAX: x.max(axis=0), MIN: x.min(axis=0)}
+        keep = shape[1]
+    else:
+        n, c, h, w = shape
+        inner = np.add.accumulate(x.transpose(1, 0, 2, 3).reshape(c, n, h * w), axis=2)[:, :, -1]
+        want = {SUM: np.add.accumulate(inner, axis=1)[:, -1], MAX: x.max(axis=(0, 2, 3)),
+                MIN: x.min(axis=(0, 2, 3))}
+        keep = c
+    for reducer in (SUM, MAX, MIN):
+        dst = G.buffer((keep,), np.float64)
+        G.case_reduce_f64(dst, src, reducer, 0.5, stream)
+        got = dst.download(stream)
+        assert np.array_equal(got, want[reducer] * 0.5), reducer
