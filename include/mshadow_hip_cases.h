@@ -74,6 +74,11 @@ int mshadow_case_pool_f16(uint16_t *dst, int dstride, const uint16_t *src, int s
    x columns and keeps the columns (sum_rows), otherwise src is (n, c, y, x) and c is kept */
 int mshadow_case_reduce_f64(double *dst, const double *src, int sstride, int n, int c, int y, int x,
                             int reducer, double scale, void *stream);
+/* op 0: dst = a * b + c; op 1: dst = pad(crop(a, (rows - 2, cols - 2)), 1); dense rows x cols tensors of
+   the element type named by the mshadow::TypeFlag code (float32 0, float64 1, float16 2, uint8 3,
+   int32 4, int8 5, int64 6), dispatched with MSHADOW_TYPE_SWITCH */
+int mshadow_case_map_any(int op, int type_flag, void *dst, const void *a, const void *b,
+                         const void *c, int rows, int cols, void *stream);
 int mshadow_case_softmax_f64(double *dst, int dstride, const double *src, int sstride, int rows,
                              int cols, void *stream);
 

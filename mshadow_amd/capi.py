@@ -107,6 +107,7 @@ CASES_SYMBOLS = {
     "mshadow_case_softmax_f16": ([_p, _i, _p, _i, _i, _i, _p], _i),
     "mshadow_case_softmax_grad_f16": ([_p, _i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_case_softmax_f64": ([_p, _i, _p, _i, _i, _i, _p], _i),
+    "mshadow_case_map_any": ([_i, _i, _p, _p, _p, _p, _i, _i, _p], _i),
     "mshadow_case_reduce_f64": ([_p, _p, _i, _i, _i, _i, _i, _i, C.c_double, _p], _i),
     "mshadow_case_map_muladd_f16": ([_p, _i, _p, _i, _p, _i, _p, _i, _i, _i, _i, _p], _i),
     "mshadow_case_pool_f16": ([_p, _i, _p, _i] + [_i] * 10 + [_p], _i),
@@ -519,6 +520,11 @@ class Library:
             n, c, y, x = src.shape
         self.check_case(self.cases.mshadow_case_reduce_f64(dst.ptr, src.ptr, src.stride, n, c, y, x,
                                                            reducer, scale, stream))
+
+    def case_map_any(self, op, type_flag, dst, a, b, c, stream=None):
+        """dense 2-D buffers of the element type the mshadow::TypeFlag code names"""
+        self.check_case(self.cases.mshadow_case_map_any(op, type_flag, dst.ptr, a.ptr, b.ptr, c.ptr,
+                                                        dst.rows, dst.cols, stream))
 
     def case_map_muladd_f16(self, dst, a, b, c, saver=SAVETO, stream=None):
         self.check_case(self.cases.mshadow_case_map_muladd_f16(

@@ -261,6 +261,27 @@ int mshadow_case_reduce_f64(double *dst, const double *src, int sstride, int n, 
   CASE_END
 }
 
+/* dst = a * b + c on tensors of any element type of the type switch (mshadow::TypeFlag codes),
+   and dst = pad(crop(a, (rows - 2, cols - 2)), 1) when op == 1: the generic expression kernels
+   instantiated through MSHADOW_TYPE_SWITCH for every type it knows */
+int mshadow_case_map_any(int op, int type_flag, void *dst, const void *a, const void *b,
+                         const void *c, int rows, int cols, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  MSHADOW_TYPE_SWITCH(type_flag, DType, {
+    Tensor<gpu, 2, DType> A = G2(static_cast<const DType *>(a), rows, cols, cols, st.get()),
+                          B = G2(static_cast<const DType *>(b), rows, cols, cols, st.get()),
+                          C = G2(static_cast<const DType *>(c), rows, cols, cols, st.get()),
+                          D = G2(static_cast<const DType *>(dst), rows, cols, cols, st.get());
+    if (op == 0) {
+      D = A * B + C;
+    } else {
+      D = pad(crop(A, Shape2(rows - 2, cols - 2)), 1);
+    }
+  });
+  CASE_END
+}
+
 /* Softmax(dst, src) on double tensors */
 int mshadow_case_softmax_f64(double *dst, int dstride, const double *src, int sstride, int rows,
                              int cols, void *stream) {

@@ -340,3 +340,37 @@ def test_gpu_double_reductions(G, stream, shape):
         G.case_reduce_f64(dst, src, reducer, 0.5, stream)
         got = dst.download(stream)
         assert np.array_equal(got, want[reducer] * 0.5), reducer
+
+
+# mshadow::TypeFlag codes (mshadow/base.h:306-316) and what numpy calls the type
+TYPE_FLAGS = [(0, np.float32), (1, np.float64), (2, np.float16), (3, np.uint8), (4, np.int32),
+              (5, np.int8), (6, np.int64)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("flag,dtype", TYPE_FLAGS)
+@pytest.mark.parametrize("shape", [(1, 3), (37, 53), (64, 1024)])
+def test_gpu_map_every_element_type(G, stream, flag, dtype, shape):
+    """dst = a * b + c and dst = pad(crop(a, ...), 1) for every element type of
+    MSHADOW_TYPE_SWITCH through the generic expression kernels, bit for bit against numpy
+    (integer types wrap modulo their width on the store, as the C++ conversion does; float16
+    rounds the product before the sum, as half_t does)"""
+    rng = np.random.default_rng(100 + flag)
+    if np.issubdtype(dtype, np.floating):
+        a, b, c = (rng.standard_normal(shape).astype(dtype) for _ in range(3))
+        want = (a * b).astype(dtype) + c
+    else:
+        a, b, c = (rng.integers(-50 if np.issubdtype(dtype, np.signedinteger) else 0, 50, shape)
+                   .astype(dtype) for _ in range(3))
+        wide = a.astype(np.int64) * b.astype(np.int64) + c.astype(np.int64)
+        want = wide.astype(dtype)      # modulo 2^bits, like the conversion on the store
+    da, db, dc = (G.to_device(t) for t in (a, b, c))
+    dst = G.buffer(shape, dtype)
+    G.case_map_any(0, flag, dst, da, db, dc, stream)
+    got = dst.download(stream)
+    assert np.array_equal(got.view(np.uint8), np.ascontiguousarray(want).view(np.uint8))
+    if shape[0] > 2:
+        G.case_map_any(1, flag, dst, da, db, dc, stream)
+        want = np.zeros(shape, dtype)
+        want[1:-1, 1:-1] = a[1:-1, 1:-1]
+        assert np.array_equal(dst.download(stream), want)
