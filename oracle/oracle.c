@@ -16,6 +16,12 @@
  *   patch2col      test/unpack.cu:29-59 closed form; index-valued images
  *   col2patch      coverage counts 4/6/9; adjoint identity with patch2col
  *   half           exhaustive round trip; F16C agreement where the host has it
+ *   *_f16          (map a*b+c, reductions, pool, softmax pair on half_t) what 16-bit rounding
+ *                  after every operation fixes: a sum of ones stops at 2048; 2048+1+1 = 2048
+ *                  but 1+1+2048 = 2050; two inner sums of 3000 ones merge to 4096; n equal
+ *                  logits give 1/min(n, 2048); (1+2^-10)^2 rounds to 1+2^-9 before the sum.
+ *                  The softmax's exponentials again come from libm expf (unpinned at the
+ *                  ulp level, though a 16-bit result rarely shows a last-bit difference)
  * and, where /root/reference is present, bit-for-bit agreement with the reference's
  * own headers compiled into oracle/_ref (see oracle/Makefile).
  */
