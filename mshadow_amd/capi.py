@@ -79,6 +79,7 @@ HIP_SYMBOLS = {
     "mshadow_hip_permute_32": ([_p, _p, _i, C.POINTER(_i), C.POINTER(_i), _p], _i),
     "mshadow_hip_sort_by_key_workspace": ([_sz, C.POINTER(_sz)], _i),
     "mshadow_hip_sort_by_key_32": ([_p, _i, _p, _sz, _i, _p, _sz, _p], _i),
+    "mshadow_hip_sort_by_key_32_noalloc": ([_p, _i, _p, _sz, _i, _p], _i),
     "mshadow_hip_softmax_grad_f32": ([_p, _i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_hip_reduce_keep_lowest_f32": ([_p, _p, _i, _i, _i, _i, _i, _f, _p], _i),
     "mshadow_hip_reduce_keep_highdim_f32": ([_p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p], _i),
@@ -355,6 +356,12 @@ class Library:
                                                        stream))
         self.check(self.dll.mshadow_hip_stream_sync(stream))
         return need.value
+
+    def sort_by_key_noalloc(self, keys, values, is_ascend=True, stream=None):
+        """in place, at most SORT_NOALLOC_MAX pairs; the scratch memory is the library's own"""
+        self.check(self.dll.mshadow_hip_sort_by_key_32_noalloc(
+            keys.ptr, self._key_kind(keys), values.ptr, keys.cols, 1 if is_ascend else 0, stream))
+        self.check(self.dll.mshadow_hip_stream_sync(stream))
 
     def softmax_grad(self, dst, src, label, stream=None):
         self.check(self.dll.mshadow_hip_softmax_grad_f32(dst.ptr, dst.stride, src.ptr, src.stride,
