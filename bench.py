@@ -147,7 +147,8 @@ def main():
     ap.add_argument("--scale", type=int, default=1, help="shrink leading dims (functional runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-reps", type=int, default=3)
-    ap.add_argument("--only", default="", help="comma list of ops to run (profiling aid)")
+    ap.add_argument("--only", default="", help="comma list of ops to run (profiling aid); "
+                    "softmax_phases and ceiling_chain run the probes of libmshadow_probe.so instead")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; every operation of the path runs at its "
@@ -159,6 +160,8 @@ def main():
     if G.device_count() < 1:
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
     G.set_device(0)
+    if args.only in ("softmax_phases", "ceiling_chain"):
+        return run_probe(G, args.only)
     props = G.props(0)
     orc = Checker("orc")
     only = [o for o in args.only.split(",") if o] or OPS
@@ -367,6 +370,44 @@ def main():
     }
     if cpu is not None:
         out["cpu_baseline"] = {k: v for k, v in cpu.items() if k != "per_op_ms"}
+    print(json.dumps(out))
+
+
+def run_probe(G, which):
+    """`--only softmax_phases`: where a row of the 8192 x 32000 softmax spends its time (time
+    stamps taken inside an instrumented build of the library's kernel). `--only ceiling_chain`:
+    the cost of one dependent float add for a single wave, alone on the chip and with every CU
+    busy - the floor of any kernel that must add in the reference's order, sum_rows first of
+    all (16384 dependent adds per column). Prints one JSON line."""
+    import mshadow_amd
+    P = mshadow_amd.load_probe()
+    s = G.stream_create()
+    cus = G.props(0).compute_units
+    if which == "ceiling_chain":
+        out = {"probe": "ceiling_chain", "unit": "ns per dependent float32 add, one wave",
+               "compute_units": cus, "modes": {}}
+        for mode in ("register", "lds", "lanes"):
+            out["modes"][mode] = {f"{wg} workgroups": round(P.add_chain_ns(mode, wg, s), 3)
+                                  for wg in (1, cus, 4 * cus)}
+        lds = out["modes"]["lds"]
+        out["sum_rows_floor_us"] = {k: round(16384 * v * 1e-3, 1) for k, v in lds.items()}
+    else:
+        L = np.random.default_rng(7).standard_normal((8192, 32000), dtype=f32) * f32(3)
+        src, dst = G.to_device(L), G.buffer(L.shape, f32)
+        steps, resident, kernel, fallback = P.softmax_phases(dst, src, s)
+        G.softmax(dst, src, s)   # the library's own kernel beside it, by HIP events
+        ev = [G.event_create() for _ in range(2)]
+        G.event_record(ev[0], s)
+        for _ in range(10):
+            G.softmax(dst, src, s)
+        G.event_record(ev[1], s)
+        G.stream_sync(s)
+        out = {"probe": "softmax_phases", "shape": [8192, 32000],
+               "unit": "us, mean over rows, since the previous step (thread 0 of the row)",
+               "steps": {k: round(v, 2) for k, v in steps.items()},
+               "row_resident_us": round(resident, 2), "instrumented_kernel_us": round(kernel, 1),
+               "library_kernel_us": round(G.elapsed_ms(ev[0], ev[1]) * 100.0, 1),
+               "rows_in_flight": 2 * cus, "fallback_rows": fallback}
     print(json.dumps(out))
 
 

@@ -7,8 +7,8 @@ drive them; it contains no compute path and no fallback: if the library is missi
 no GPU is present, calls raise.
 """
 from .capi import (  # noqa: F401
-    CASES_SO, HIP_SO, DeviceBuffer, HipError, Library, cases, lib, load_cases, load_lib,
+    CASES_SO, HIP_SO, DeviceBuffer, HipError, Library, cases, lib, load_cases, load_lib, load_probe,
 )
 
-__all__ = ["lib", "cases", "load_lib", "load_cases", "Library", "DeviceBuffer", "HipError",
+__all__ = ["lib", "cases", "load_lib", "load_cases", "load_probe", "Library", "DeviceBuffer", "HipError",
            "HIP_SO", "CASES_SO"]

@@ -4,6 +4,7 @@
                        csrc/permute.hip, csrc/random.hip)
   libmshadow_cases.so  caller-style programs written against <mshadow/tensor.h>
                        (cases/cases.hip), exported as C functions for tests and bench
+  libmshadow_probe.so  measurement aids of bench.py (csrc/probe.hip); nothing depends on it
 
 Both are built in-tree under mshadow_amd/lib/ with hipcc, which cross-compiles without a
 GPU. Flags that matter for results:
@@ -20,6 +21,7 @@ ROOT = os.path.dirname(HERE)
 LIB_DIR = os.path.join(HERE, "lib")
 HIP_SO = os.path.join(LIB_DIR, "libmshadow_hip.so")
 CASES_SO = os.path.join(LIB_DIR, "libmshadow_cases.so")
+PROBE_SO = os.path.join(LIB_DIR, "libmshadow_probe.so")
 
 ARCH = "gfx950"
 COMMON = [
@@ -66,9 +68,18 @@ def build_cases_library(verbose=True):
     return CASES_SO
 
 
+def build_probe_library(verbose=True):
+    """measurement aids for bench.py: instrumented copies of library kernels, micro-benchmarks"""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    src = os.path.join(HERE, "csrc", "probe.hip")
+    _run([hipcc()] + COMMON + ["-o", PROBE_SO, src], verbose)
+    return PROBE_SO
+
+
 def build_all(verbose=True):
     build_hip_library(verbose)
     build_cases_library(verbose)
+    build_probe_library(verbose)
 
 
 if __name__ == "__main__":

@@ -586,6 +586,51 @@ class Library:
         return out, stride.value
 
 
+class Probe:
+    """libmshadow_probe.so: measurement aids of bench.py (include/mshadow_hip_probe.h)"""
+    STAMPS = 16
+    STAMP_ORDER = (10, 11, 12, 13, 1, 2, 3, 4, 5, 14)
+    STAMP_NAMES = ("entry", "row loaded, thread maxima", "row maximum (barrier)", "exp",
+                   "chunk sums and maxima exchanged (barrier)", "chunk plan",
+                   "chunks quantised, lists written (barrier)", "chain: tables (wave 0)",
+                   "chain done (barrier)", "divided and stored (stores completed)")
+    CHAIN_MODES = {"register": 0, "lds": 1, "lanes": 2}
+
+    def __init__(self):
+        path = os.path.join(os.path.dirname(HIP_SO), "libmshadow_probe.so")
+        if not os.path.exists(path):
+            raise HipError(f"{path} is not built (python -m mshadow_amd.build)")
+        self.dll = C.CDLL(path)
+        self.dll.mshadow_probe_last_error.restype = C.c_char_p
+        self.dll.mshadow_probe_add_chain.argtypes = [_i, _i, C.POINTER(C.c_double), _p]
+        self.dll.mshadow_probe_softmax_phases.argtypes = [
+            _p, _i, _p, _i, _i, _i, C.POINTER(C.c_double), C.POINTER(C.c_double),
+            C.POINTER(C.c_double), C.POINTER(_i), _p]
+
+    def _check(self, status):
+        if status != 0:
+            raise HipError(self.dll.mshadow_probe_last_error().decode(errors="replace"))
+
+    def add_chain_ns(self, mode, workgroups, stream=None):
+        ns = C.c_double(0)
+        self._check(self.dll.mshadow_probe_add_chain(self.CHAIN_MODES[mode], workgroups, C.byref(ns), stream))
+        return ns.value
+
+    def softmax_phases(self, dst, src, stream=None):
+        """-> ({step name: mean us since the previous step}, resident us, kernel us, fallback rows)"""
+        mean = (C.c_double * self.STAMPS)()
+        resident, kernel, fallback = C.c_double(0), C.c_double(0), _i(0)
+        self._check(self.dll.mshadow_probe_softmax_phases(
+            dst.ptr, dst.stride, src.ptr, src.stride, src.rows, src.cols, mean, C.byref(resident),
+            C.byref(kernel), C.byref(fallback), stream))
+        steps = {f"{idx} {name}": mean[idx] for idx, name in zip(self.STAMP_ORDER, self.STAMP_NAMES)}
+        return steps, resident.value, kernel.value, fallback.value
+
+
+def load_probe():
+    return Probe()
+
+
 _lib = None
 _cases = None
 

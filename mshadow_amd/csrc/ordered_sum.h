@@ -192,5 +192,71 @@ OSUM_HD float TrueAdd(float s, const float (&t)[N]) {
   return s;
 }
 
+/* ---- the row as a list of addends -------------------------------------------------------
+ * The planned row sum of softmax_kernels.h turns a row into a short ordered list of float
+ * addends whose plain serial sum IS the left-to-right sum of all terms: a lane (N consecutive
+ * terms) whose running sum provably stays in one binade joins a run of such lanes, and the
+ * run enters the list as ONE addend, its integer total times the binade's ulp; any other lane
+ * (next to a power of two, or holding a tie) enters with its N terms themselves. Adding a
+ * run's addend is exact when the sum is in the run's binade before and after it, which is
+ * checked on the sums actually obtained (RunHolds): a wrong plan is noticed, never used. */
+
+/*! \brief quantisation of one lane's N non-negative terms against the binade with biased
+ *  exponent e (0 = the subnormal range, where sums are exact): two accumulators start at
+ *  the bottom of the binade, one ulp apart, and take the terms by ordinary float additions.
+ *  While both stay in the binade each addition moves them by rne(t / ulp) ulps; a term that
+ *  lies half way between two multiples of the ulp moves the even one down and the odd one
+ *  up, so the accumulators end one ulp apart exactly when no term was a tie. */
+struct LaneQuantum {
+  uint32_t q;  //!< sum of rne(t / ulp) over the lane's terms
+  bool ok;     //!< no tie, no NaN, and the lane alone does not leave the binade
+};
+template <int N>
+OSUM_HD LaneQuantum LaneDualQuant(const float (&t)[N], uint32_t e) {
+  const uint32_t base = e << 23;
+  float lo = FloatOf(base), hi = FloatOf(base + 1u);
+  for (int i = 0; i < N; ++i) {
+    lo = lo + t[i];
+    hi = hi + t[i];
+  }
+  const uint32_t blo = BitsOf(lo), bhi = BitsOf(hi);
+  LaneQuantum r;
+  r.ok = (bhi - blo == 1u) && blo >= base && bhi < base + (1u << 23);
+  r.q = blo - base;
+  return r;
+}
+
+/*! \brief bounds on the sequential sum from an accurate sum `approx` of the same terms:
+ *  every addition rounds by at most half an ulp, so after n terms the sequential sum sits
+ *  within n * 2^-24 of it (relative); sums of softmax terms stay well inside a quarter of
+ *  that below and almost nothing above. The bounds only steer the plan. */
+OSUM_HD float PlanLowBound(float approx, float terms_in_front) {
+  return approx * (1.0f - (terms_in_front * 1.4901161193847656e-08f + 8.0e-6f));  // n * 2^-26
+}
+OSUM_HD float PlanHighBound(float approx) { return approx * (1.0f + 8.0e-6f); }
+
+/*! \brief the binade a piece stays in if the sum is at least `low` in front of it and at
+ *  most `high` behind it; -1 if those lie in different binades (or are not finite) */
+OSUM_HD int PlanBinade(float low, float high) {
+  const uint32_t blo = BitsOf(low), bhi = BitsOf(high);
+  const uint32_t elo = (blo >> 23) & 0xffu, ehi = (bhi >> 23) & 0xffu;
+  const bool ok = elo == ehi && ehi < 255u && ((blo | bhi) >> 31) == 0u;
+  return ok ? static_cast<int>(elo) : -1;
+}
+
+/*! \brief the addend of a run with integer total r in binade e. A total that cannot fit
+ *  (the sum itself takes at least 2^23 ulps) becomes an addend that carries any sum out
+ *  of the binade, so that RunHolds fails. */
+OSUM_HD float RunAddend(uint32_t e, uint32_t r) {
+  const uint32_t base = e << 23;
+  return r < (1u << 23) ? FloatOf(base + r) - FloatOf(base) : FloatOf(base + (1u << 23));
+}
+
+/*! \brief was adding a run of binade e exact? (the sum before and after lies in it) */
+OSUM_HD bool RunHolds(float before, float after, uint32_t e) {
+  const uint32_t bb = BitsOf(before), ba = BitsOf(after);
+  return (bb >> 23) == e && (ba >> 23) == e;  // sign bits are part of the comparison
+}
+
 }  // namespace ordered_sum
 #endif  // MSHADOW_AMD_CSRC_ORDERED_SUM_H_

@@ -1,0 +1,213 @@
+/*
+ * libmshadow_probe - measurement aids for the benchmark harness; no part of the device
+ * layer (nothing in libmshadow_hip.so or the headers depends on it).
+ *
+ *   mshadow_probe_softmax_phases   the register-resident softmax kernel of the library,
+ *       compiled here with its time-stamp hook switched on: per row, when each step of the
+ *       kernel was reached (100 MHz counter), reduced on the host to mean times per step
+ *   mshadow_probe_add_chain        what one dependent float add costs a single wave, with
+ *       operands from registers, from LDS (as the column reduction feeds its chain) and
+ *       along the lanes (as the softmax row sum adds its list), at a given number of
+ *       workgroups, so that the figure can be taken with the whole chip busy
+ */
+#include <hip/hip_runtime.h>
+#include <mshadow_hip.h>
+#include <mshadow_hip_probe.h>
+
+#include <algorithm>
+#include <functional>
+#include <string>
+#include <vector>
+
+namespace {
+__device__ long long *g_stamps;  //!< [rows][kStampSlots], set before each probe launch
+const int kStampSlots = MSHADOW_PROBE_STAMPS;
+}  // namespace
+
+#define MSHADOW_ROWSUM_STAMP(step)                                                          \
+  {                                                                                         \
+    __builtin_amdgcn_sched_barrier(0);                                                      \
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");                             \
+    if (threadIdx.x == 0) {                                                                 \
+      g_stamps[static_cast<size_t>(blockIdx.x) * kStampSlots + (step)] = wall_clock64();    \
+    }                                                                                       \
+    __builtin_amdgcn_sched_barrier(0);                                                      \
+  }
+
+/* The instrumented kernels are other functions than the library's: in their own namespace,
+   or the loader would bind this file's launches to the library's copies of the same names. */
+#define mshadow_hipk mshadow_hipk_probe
+#include "softmax_kernels.h"
+
+#include <mshadow/hip/kernels/reduce.h>
+
+#include "abi_common.h"
+
+namespace mshadow_abi {
+std::string &LastError() {
+  static thread_local std::string text;
+  return text;
+}
+}  // namespace mshadow_abi
+
+using mshadow_abi::AfterLaunch;
+using mshadow_abi::AsStream;
+
+namespace {
+
+/*! \brief `iters` rounds of 32 dependent adds whose operand is a register */
+__global__ void __launch_bounds__(64) RegisterChainKernel(float *out, float a, int iters) {
+  float s = threadIdx.x;
+  float addend = a;
+  asm volatile("" : "+v"(addend));  // a vector register, as the operand of a real chain is
+  for (int i = 0; i < iters; ++i) {
+#pragma unroll
+    for (int k = 0; k < 32; ++k) {
+      s = s + addend;
+      asm volatile("" : "+v"(s));
+    }
+  }
+  out[blockIdx.x * 64 + threadIdx.x] = s;
+}
+
+/*! \brief the chain of the column reduction: 16 lanes fold `count` floats each from LDS,
+ *  four per 128-bit read, the next 32 operands fetched while 32 adds execute */
+__global__ void __launch_bounds__(64) LdsChainKernel(float *out, int iters, int count) {
+  __shared__ float buf[16 * 1028];
+  for (int i = threadIdx.x; i < 16 * 1028; i += 64) buf[i] = i * 1e-3f;
+  __syncthreads();
+  float s = 0.0f;
+  if (threadIdx.x < 16) {
+    for (int i = 0; i < iters; ++i) {
+      mshadow::hip::ChainFold<mshadow::red::sum, 4>(s, buf + threadIdx.x * 1028, 0, count);
+      asm volatile("" : "+v"(s));
+    }
+  }
+  out[blockIdx.x * 64 + threadIdx.x] = s;
+}
+
+/*! \brief the chain of the softmax row sum: a sum handed from lane to lane */
+__global__ void __launch_bounds__(64) SystolicChainKernel(float *out, float a, int iters) {
+  float s = threadIdx.x;
+  float addend = a;
+  asm volatile("" : "+v"(addend));
+  for (int i = 0; i < iters; ++i) {
+#pragma unroll
+    for (int k = 0; k < 32; ++k) mshadow_hipk::SystolicStep(&s, addend);
+  }
+  out[blockIdx.x * 64 + threadIdx.x] = s;
+}
+
+int TimeKernel(hipStream_t s, float *ms, const std::function<void()> &launch) {
+  hipEvent_t a, b;
+  ABI_HIP(hipEventCreate(&a));
+  ABI_HIP(hipEventCreate(&b));
+  launch();  // warm-up
+  ABI_HIP(hipStreamSynchronize(s));
+  ABI_HIP(hipEventRecord(a, s));
+  launch();
+  ABI_HIP(hipEventRecord(b, s));
+  ABI_HIP(hipEventSynchronize(b));
+  ABI_HIP(hipEventElapsedTime(ms, a, b));
+  ABI_HIP(hipEventDestroy(a));
+  ABI_HIP(hipEventDestroy(b));
+  return AfterLaunch("probe kernel");
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *mshadow_probe_last_error(void) { return mshadow_abi::LastError().c_str(); }
+
+int mshadow_probe_add_chain(int mode, int workgroups, double *ns_per_add, void *stream) {
+  ABI_REQUIRE(ns_per_add != NULL && workgroups >= 1 && workgroups <= 65536, "bad argument");
+  hipStream_t s = AsStream(stream);
+  float *out = NULL;
+  ABI_HIP(hipMalloc(&out, static_cast<size_t>(workgroups) * 64 * sizeof(float)));
+  float ms = 0.0f;
+  int st;
+  double adds;
+  if (mode == MSHADOW_PROBE_CHAIN_REGISTER) {
+    const int iters = 4096;
+    adds = 32.0 * iters;
+    st = TimeKernel(s, &ms, [&] {
+      hipLaunchKernelGGL(RegisterChainKernel, dim3(workgroups), dim3(64), 0, s, out, 1.5f, iters);
+    });
+  } else if (mode == MSHADOW_PROBE_CHAIN_LDS) {
+    const int iters = 128, count = 1024;
+    adds = static_cast<double>(iters) * count;
+    st = TimeKernel(s, &ms, [&] {
+      hipLaunchKernelGGL(LdsChainKernel, dim3(workgroups), dim3(64), 0, s, out, iters, count);
+    });
+  } else if (mode == MSHADOW_PROBE_CHAIN_LANES) {
+    const int iters = 4096;
+    adds = 32.0 * iters;
+    st = TimeKernel(s, &ms, [&] {
+      hipLaunchKernelGGL(SystolicChainKernel, dim3(workgroups), dim3(64), 0, s, out, 1.5f, iters);
+    });
+  } else {
+    (void)hipFree(out);
+    ABI_REQUIRE(false, "unknown mode");
+  }
+  (void)hipFree(out);
+  if (st != MSHADOW_HIP_OK) return st;
+  *ns_per_add = static_cast<double>(ms) * 1e6 / adds;
+  return MSHADOW_HIP_OK;
+}
+
+int mshadow_probe_softmax_phases(float *dst, int dstride, const float *src, int sstride, int rows,
+                                 int cols, double *mean_us, double *resident_us,
+                                 double *kernel_us, int *fallback_rows, void *stream) {
+  ABI_REQUIRE(rows >= 1 && cols > 16384 && cols <= 32768 && cols % 4 == 0 && sstride % 4 == 0 &&
+                  dstride % 4 == 0, "the probe covers the 512-thread, 16-slab kernel: 16384 < cols <= 32768, rows of whole packs");
+  ABI_REQUIRE(mean_us != NULL && resident_us != NULL && kernel_us != NULL && fallback_rows != NULL,
+              "NULL result");
+  hipStream_t s = AsStream(stream);
+  long long *stamps = NULL;
+  const size_t n = static_cast<size_t>(rows) * kStampSlots;
+  ABI_HIP(hipMalloc(&stamps, n * sizeof(long long)));
+  ABI_HIP(hipMemsetAsync(stamps, 0, n * sizeof(long long), s));
+  ABI_HIP(hipMemcpyToSymbolAsync(HIP_SYMBOL(g_stamps), &stamps, sizeof(stamps), 0,
+                                 hipMemcpyHostToDevice, s));
+  float ms = 0.0f;
+  const int st = TimeKernel(s, &ms, [&] {
+    hipLaunchKernelGGL((mshadow_hipk::SoftmaxRowKernel<512, 16, 4, false>), dim3(rows), dim3(512), 0,
+                       s, dst, dstride, src, sstride, cols);
+  });
+  if (st != MSHADOW_HIP_OK) {
+    (void)hipFree(stamps);
+    return st;
+  }
+  *kernel_us = ms * 1e3;
+  std::vector<long long> h(n);
+  ABI_HIP(hipMemcpy(h.data(), stamps, n * sizeof(long long), hipMemcpyDeviceToHost));
+  ABI_HIP(hipFree(stamps));
+  /* the steps a row passed through, in the order of the kernel; a step a row did not
+     reach (the fall-back) has no stamp and is left out of that row's chain of intervals */
+  static const int order[] = MSHADOW_PROBE_STAMP_ORDER;
+  const int norder = static_cast<int>(sizeof(order) / sizeof(order[0]));
+  std::vector<double> sum(kStampSlots, 0.0);
+  std::vector<long> cnt(kStampSlots, 0);
+  double resident = 0.0;
+  *fallback_rows = 0;
+  for (int r = 0; r < rows; ++r) {
+    const long long *t = &h[static_cast<size_t>(r) * kStampSlots];
+    if (t[MSHADOW_PROBE_STAMP_FALLBACK] != 0) ++*fallback_rows;
+    long long prev = t[order[0]];
+    for (int i = 1; i < norder; ++i) {
+      const long long now = t[order[i]];
+      if (now == 0) continue;
+      sum[order[i]] += static_cast<double>(now - prev);
+      ++cnt[order[i]];
+      prev = now;
+    }
+    resident += static_cast<double>(prev - t[order[0]]);
+  }
+  for (int i = 0; i < kStampSlots; ++i) mean_us[i] = cnt[i] ? sum[i] / cnt[i] / 100.0 : -1.0;
+  mean_us[order[0]] = 0.0;
+  *resident_us = resident / rows / 100.0;
+  return MSHADOW_HIP_OK;
+}
+
+}  // extern "C"

@@ -109,28 +109,23 @@ __device__ inline float BlockOrderedAdd(float s, const float (&t)[N],
 }
 
 /* ---- planned row sum (registers hold the whole row) ---------------------------------
- * Thread layout: wave w owns a contiguous W-th of the row, slab j of it is the chunk
- * k = w * SLABS + j (64 * N consecutive terms, lane-major). See ordered_sum.h for the
- * plan; the steps here are
- *   A  every wave: approximate sum of each of its chunks -> LDS            (barrier)
- *   B  every wave (redundantly): prefix over all chunks, plan per chunk
- *   C  every wave: quantise its clean chunks, integer totals -> LDS; its dirty chunks
- *      are parked, with their terms, in LDS slots                          (barrier)
- *   D  every wave: integer prefix over the clean chunks; all waves together: a plan per
- *      lane for each parked chunk, and the order of the slots in the row   (barrier)
- *      wave 0: for each parked chunk in row order, apply the clean run in front of it
- *      and walk it (runs of clean lanes as integers, the other lanes term by term),
- *      fetching the next slot meanwhile                                    (barrier)
- *   E  every wave: apply the clean run behind the last dirty chunk.
- * A row with more dirty chunks than slots is summed by wave scans instead (as is a row
- * whose plan fails a verification).
+ * Thread layout: chunk k of the row (64 * N consecutive terms, lane-major) is slab k / W of
+ * wave k % W, so the W waves walk the row side by side and the chunks next to the row's
+ * binade crossings are spread over the waves. ordered_sum.h describes the plan; the steps are
+ *   A  every wave: approximate sum and largest term of each of its chunks -> LDS   (barrier)
+ *   B  every wave (redundantly): prefix over all chunks, a binade per chunk where certain
+ *   C  every wave: its certain chunks quantised against their binade, integer totals -> LDS;
+ *      each of its other chunks planned lane by lane and written to LDS as a short list
+ *      of addends (a run of certain lanes = one addend, any other lane = its terms) (barrier)
+ *   D  wave 0: the chain - for each listed chunk in row order, the run of certain chunks in
+ *      front of it (one addend) and its list, summed serially and every run verified (barrier)
+ * A row whose plan fails a verification, or that has more listed chunks than slots, is summed
+ * by wave scans instead, chunk after chunk.
  * Lane l keeps the chunk-table entries of chunks l * CPL .. l * CPL + CPL - 1. */
-const uint32_t kDirtyQ = 0xffffffffu;
-/*! \brief lanes of a row's first chunk that are added serially without a plan */
-const int kHeadLanes = 32;
-/*! \brief dirty chunks per row with a lane-level plan parked in LDS (a row of softmax
- *  terms has about a dozen); further ones are resolved by wave scans */
+/*! \brief chunks per row that can hand a list of addends to the chain (a row of softmax
+ *  terms has about a dozen) */
 const int kPlanSlots = 24;
+const uint32_t kListedBit = 0x80000000u;
 
 /* hook for a profiling build: a translation unit may define this to record a timestamp
    at the boundaries of the steps; it is empty in the library */
@@ -138,46 +133,33 @@ const int kPlanSlots = 24;
 #define MSHADOW_ROWSUM_STAMP(step)
 #endif
 
-/*! \brief lane-level plan of one dirty chunk, parked in LDS between steps C and D, with
- *  the chunk's terms (so that the walk needs nothing from the register-resident row).
- *  General chunk: a = integer total of the clean lanes in front of the lane, b = its plan
- *  code. Two-binade chunk: a / b = inclusive integer prefix of the lanes quantised against
- *  the lower / upper binade (lanes holding a tie count as 0). */
+/*! \brief the addends of one listed chunk, in row order: at most one per term. check[i] is
+ *  1 + the binade the sum must be in before and after addend i (a run), or 0 (a term). */
 template <int N>
-struct LanePlanSlot {
-  float t[kWave][N];
-  uint32_t a[kWave];
-  uint32_t b[kWave];
-  unsigned long long tie_lo, tie_hi;  //!< two-binade chunks: lanes holding a tie (lower / upper binade)
-  uint32_t total;  //!< general chunks: integer total of the clean lanes
-  int kind;        //!< plan code of the chunk (kPlanWalk or kPlanTwoBinades + e)
-  float start;     //!< approximate prefix sum in front of the chunk
-  int chunk;       //!< index of the chunk in the row
-  uint32_t ex;     //!< integer total of the clean chunks in front of this one
-  int e_run;       //!< binade of the clean chunk just in front (if there is one)
+struct AddendList {
+  float addend[kWave * N];
+  unsigned char check[kWave * N];
 };
 
 template <int W, int SLABS, int N>
 struct RowSumLds {
+  static const int kChunks = W * SLABS;
   /* small workgroups share a CU with several others: fewer slots each */
   static const int kWanted = W <= 4 ? kPlanSlots * 2 / 3 : kPlanSlots;
-  static const int kSlots = (W * SLABS < kWanted) ? W * SLABS : kWanted;
-  float approx[W * SLABS];
-  uint32_t q[W * SLABS];
-  float s;       //!< running sum handed from wave to wave
-  uint32_t ex;   //!< integer prefix (over clean chunks) already applied to s
-  int fail;      //!< a verification failed: redo the row the slow way
-  uint32_t nslots;  //!< plan slots handed out
+  static const int kSlots = (kChunks < kWanted) ? kChunks : kWanted;
+  float approx[kChunks];
+  float cmax[kChunks];
+  /*! \brief certain chunk: its integer total; listed chunk: kListedBit | addends << 8 | slot */
+  uint32_t q[kChunks];
+  float s;          //!< the row's sum, from the chain to everybody
+  int fail;         //!< the plan did not hold: redo the row the slow way
+  uint32_t nslots;  //!< lists handed out
   float wmax[W];
-  /*! \brief the plan slots in the order of their chunks in the row */
-  signed char order[kSlots];
-  LanePlanSlot<N> plan[kSlots];
+  /*! \brief the chain's work list: per listed chunk its q entry, the integer total of the
+   *  certain chunks in front of it and the binade of the chunk just in front (+1; 0: listed) */
+  uint32_t item_q[kSlots], item_ex[kSlots], item_run[kSlots];
+  AddendList<N> list[kSlots];
 };
-
-/*! \brief plan code of a piece that stays in one binade */
-__device__ __forceinline__ bool IsClean(int code) {
-  return code >= 0 && code < ordered_sum::kPlanTwoBinades;
-}
 
 /*! \brief entry k of a table spread over lanes (CPL entries per lane); k is uniform */
 template <int CPL>
@@ -223,186 +205,43 @@ __device__ __forceinline__ void SelectSlab(float (&t)[N], const float (&v)[SLABS
   SlabPicker<0, SLABS, SLABS, N>::Pick(t, v, j);
 }
 
-/*! \brief lane-level plan of one chunk whose approximate prefix sum in front is `start`:
- *  *code = binade the lane's terms stay in, or kPlanWalk; *ex = integer total of the
- *  clean lanes in front of this lane; returns the integer total of all clean lanes */
-template <int N>
-__device__ __forceinline__ uint32_t PlanLanes(const float (&t)[N], float start, float margin,
-                                              bool head, uint32_t *ex, int *code) {
+/*! \brief value of v in the lane below (lane 0 receives `first`) */
+__device__ __forceinline__ uint32_t FromLaneBelowU32(uint32_t v, uint32_t first) {
+  /* DPP wave_shr:1; a lane without a source keeps the first operand */
+  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(static_cast<int>(first), static_cast<int>(v),
+                                                           0x138, 0xf, 0xf, false));
+}
+
+/*! \brief one step of the serial sum that runs along the lanes of a wave: lane l takes
+ *  the sum of lane l - 1 and adds its own addend; lane 0 has no lane below it and keeps its
+ *  value. After k steps lanes 0 .. k hold the sums after their addends, for good (a lane's
+ *  value depends only on the settled lane below it), so surplus steps change nothing. One
+ *  VALU instruction on the dependent path; the idle cycles in front of it are what the
+ *  hardware asks for between writing a register and reading it through DPP. */
+__device__ __forceinline__ void SystolicStep(float *sum, float addend) {
+  asm volatile("s_nop 1\n\tv_add_f32_dpp %0, %0, %1 wave_shr:1 row_mask:0xf bank_mask:0xf"
+               : "+v"(*sum)
+               : "v"(addend));
+}
+
+/*! \brief s plus up to 64 addends, lane l holding addend l (`count` of them, zeros behind),
+ *  one float add after the other; check = 1 + binade for a run (0 for a term). Clears *ok
+ *  if a run was added while the sum was not in its binade. */
+__device__ __forceinline__ float ChainBlock(float s, float addend, uint32_t check, int count,
+                                            bool *ok) {
   using namespace ordered_sum;
-  float a = t[0];
+  float sum = s + addend;  // right in lane 0, the start of the systolic sum
+  for (int done = 1; done < count; done += 8) {
 #pragma unroll
-  for (int i = 1; i < N; ++i) a += t[i];
-  const float incl = WaveInclusiveScanF32(a);
-  int c = PlanLane(start + (incl - a), start + incl, margin);
-  /* the head of a row (the sum starts at zero): its first lanes cross a binade or hold a
-     tie nearly every time and are added term by term without asking */
-  if (head && LaneId() < kHeadLanes) c = kPlanWalk;
-  float q = 0.0f;
-  if (c >= 0) {
-    q = LaneQuant<N>(t, BinadeOfExponent(static_cast<uint32_t>(c)));
-    if (!(q < kLimit)) c = kPlanWalk;  // a tie (or a term the plan did not expect)
+    for (int u = 0; u < 8; ++u) SystolicStep(&sum, addend);
   }
-  /* neighbouring clean lanes must agree on the binade, or the later one is walked */
-  const int before = __shfl_up(c, 1);
-  if (LaneId() > 0 && c >= 0 && before >= 0 && before != c) c = kPlanWalk;
-  const uint32_t qi = c >= 0 ? static_cast<uint32_t>(q) : 0u;
-  const uint32_t inclu = mshadow::hip::WaveInclusiveScanU32(qi);
-  *ex = inclu - qi;
-  *code = c;
-  return mshadow::hip::ReadLaneU32(inclu, kWave - 1);
+  const float before = __uint_as_float(FromLaneBelowU32(__float_as_uint(sum), __float_as_uint(s)));
+  const bool held = check == 0u || RunHolds(before, sum, check - 1u);
+  if (__ballot(!held && LaneId() < count) != 0ull) *ok = false;
+  return ReadLaneF32(sum, count - 1);
 }
 
-/*! \brief s plus the terms of lanes 0 .. kHeadLanes-1 of a chunk parked in LDS (t[lane][i]),
- *  one float add after the other. Every lane reads the same addresses (an LDS broadcast),
- *  so the operands arrive in vector registers and the only chain is the adds themselves. */
-template <int N>
-__device__ __forceinline__ float HeadSerialAdd(float s, const float (*t)[N]) {
-  const int kBatch = 4;  // lanes whose terms are fetched before they are added
-#pragma unroll
-  for (int l0 = 0; l0 < kHeadLanes; l0 += kBatch) {
-    float r[kBatch][N];
-#pragma unroll
-    for (int l = 0; l < kBatch; ++l) {
-#pragma unroll
-      for (int i = 0; i < N; ++i) r[l][i] = t[l0 + l][i];
-    }
-#pragma unroll
-    for (int l = 0; l < kBatch; ++l) {
-#pragma unroll
-      for (int i = 0; i < N; ++i) s = s + r[l][i];
-    }
-  }
-  return s;
-}
-
-/*! \brief s plus one chunk, given its lane-level plan: runs of clean lanes are applied as
- *  integers (and verified), runs of other lanes add their terms one by one. `skip` names
- *  lanes that are in s already. */
-template <int N>
-__device__ __forceinline__ float WalkLanes(float s, const float (&t)[N], uint32_t ex, int code,
-                                           uint32_t total, unsigned long long skip, bool *fail) {
-  using namespace ordered_sum;
-  using mshadow::hip::ReadLaneU32;
-  unsigned long long todo = __ballot(code < 0) & ~skip;
-  uint32_t done = 0u;
-  while (todo != 0ull) {
-    const int l0 = __ffsll(static_cast<long long>(todo)) - 1;
-    const uint32_t exl = ReadLaneU32(ex, l0);
-    if (exl != done) {
-      s = FlushRun(s, static_cast<int>(ReadLaneU32(static_cast<uint32_t>(code), l0 - 1)), exl - done, fail);
-      done = exl;
-    }
-    /* the lanes l0 .. l1-1 are walked: l1 = first clean lane above l0 (or 64) */
-    const unsigned long long above = ~(todo >> l0);
-    const int len = above != 0ull ? __ffsll(static_cast<long long>(above)) - 1 : kWave - l0;
-    const int l1 = l0 + len;
-    for (int l = l0; l < l1; ++l) {
-#pragma unroll
-      for (int i = 0; i < N; ++i) s = s + ReadLaneF32(t[i], l);
-    }
-    todo = l1 < kWave ? (todo >> l1) << l1 : 0ull;
-  }
-  if (total != done) {
-    s = FlushRun(s, static_cast<int>(ReadLaneU32(static_cast<uint32_t>(code), kWave - 1)), total - done, fail);
-  }
-  return s;
-}
-
-/*! \brief plan of a chunk that starts in binade elo and may end in elo + 1: every lane
- *  quantised against both; a lane holding a tie under a binade counts as 0 in that prefix
- *  and is named in the tie mask */
-template <int N>
-__device__ __forceinline__ void PlanTwoBinades(const float (&t)[N], int elo, uint32_t *incl_lo,
-                                               uint32_t *incl_hi, unsigned long long *tie_lo,
-                                               unsigned long long *tie_hi) {
-  using namespace ordered_sum;
-  const float qlo = LaneQuant<N>(t, BinadeOfExponent(static_cast<uint32_t>(elo)));
-  const float qhi = LaneQuant<N>(t, BinadeOfExponent(static_cast<uint32_t>(elo + 1)));
-  const bool tlo = !(qlo < kLimit), thi = !(qhi < kLimit);
-  *incl_lo = mshadow::hip::WaveInclusiveScanU32(tlo ? 0u : static_cast<uint32_t>(qlo));
-  *incl_hi = mshadow::hip::WaveInclusiveScanU32(thi ? 0u : static_cast<uint32_t>(qhi));
-  *tie_lo = __ballot(tlo);
-  *tie_hi = __ballot(thi);
-}
-
-/*! \brief s plus one chunk planned by PlanTwoBinades. Each round accepts, as integers,
- *  the lanes up to the first one that holds a tie or would carry the sum out of the
- *  current binade, adds that lane's terms one by one, and goes on - against the upper
- *  binade once the sum has crossed. A crossing chunk takes two rounds. */
-template <int N>
-__device__ __forceinline__ float WalkTwoBinades(float s, const float (&t)[N], int elo,
-                                                uint32_t incl_lo, uint32_t incl_hi,
-                                                unsigned long long tie_lo,
-                                                unsigned long long tie_hi, bool *fail) {
-  using namespace ordered_sum;
-  using mshadow::hip::ReadLaneU32;
-  /* The usual course in straight-line code: the lanes up to the crossing (or tie) lane f
-     as integers in the lower binade, lane f term by term, all lanes behind it as integers
-     in whichever of the two binades the sum is in then. Anything else (a second tie, a sum
-     in neither binade) takes the general rounds below from the start. */
-  {
-    const uint32_t el = static_cast<uint32_t>(elo);
-    const float m = s * FloatOf((277u - el) << 23);
-    const uint32_t room = 16777216u - static_cast<uint32_t>(m);
-    const unsigned long long ev = __ballot(incl_lo >= room) | tie_lo;
-    const bool in_lo = m >= 8388608.0f && m < kLimit;
-    if (in_lo && ev == 0ull) {
-      return (m + static_cast<float>(ReadLaneU32(incl_lo, kWave - 1))) * FloatOf((el - 23u) << 23);
-    }
-    if (in_lo) {
-      const int f = __ffsll(static_cast<long long>(ev)) - 1;
-      const uint32_t upto = f > 0 ? ReadLaneU32(incl_lo, f - 1) : 0u;
-      float s2 = (m + static_cast<float>(upto)) * FloatOf((el - 23u) << 23);
-#pragma unroll
-      for (int i = 0; i < N; ++i) s2 = s2 + ReadLaneF32(t[i], f);
-      const float mh = s2 * FloatOf((276u - el) << 23);  // in units of the upper binade
-      const bool up = mh >= 8388608.0f;
-      const float m2 = up ? mh : mh + mh;                 // exact either way
-      const uint32_t incl2 = up ? incl_hi : incl_lo;
-      const uint32_t base2 = ReadLaneU32(incl2, f);
-      const uint32_t room2 = 16777216u - static_cast<uint32_t>(m2);
-      const unsigned long long behind = f < kWave - 1 ? (~0ull << 1) << f : 0ull;
-      const unsigned long long ev2 = (__ballot(incl2 - base2 >= room2) | (up ? tie_hi : tie_lo)) & behind;
-      if (ev2 == 0ull && m2 >= 8388608.0f && m2 < kLimit) {
-        const float u2 = FloatOf((el - 23u + (up ? 1u : 0u)) << 23);
-        return (m2 + static_cast<float>(ReadLaneU32(incl2, kWave - 1) - base2)) * u2;
-      }
-    }
-  }
-  unsigned long long pending = ~0ull;  // lanes not yet in s
-  int p = 0;                           // = number of lanes in s
-  bool hi = false;                     // s has crossed into the upper binade
-  while (true) {
-    const uint32_t e = static_cast<uint32_t>(elo) + (hi ? 1u : 0u);
-    const float m = s * FloatOf((277u - e) << 23);
-    if (!hi && !(m < kLimit)) {
-      hi = true;
-      continue;
-    }
-    if (!(m >= 8388608.0f && m < kLimit)) {  // s is in neither binade: the plan was wrong
-      *fail = true;
-      return s;
-    }
-    const float u = FloatOf((e - 23u) << 23);
-    const uint32_t incl = hi ? incl_hi : incl_lo;
-    const uint32_t base = p > 0 ? ReadLaneU32(incl, p - 1) : 0u;
-    const uint32_t room = 16777216u - static_cast<uint32_t>(m);  // integer steps left in the binade
-    /* lanes already in s compare on a wrapped difference; `pending` masks them out */
-    const unsigned long long events = (__ballot(incl - base >= room) | (hi ? tie_hi : tie_lo)) & pending;
-    if (events == 0ull) return (m + static_cast<float>(ReadLaneU32(incl, kWave - 1) - base)) * u;
-    const int f = __ffsll(static_cast<long long>(events)) - 1;
-    const uint32_t upto = f > 0 ? ReadLaneU32(incl, f - 1) : 0u;
-    s = (m + static_cast<float>(upto - base)) * u;
-#pragma unroll
-    for (int i = 0; i < N; ++i) s = s + ReadLaneF32(t[i], f);
-    if (f == kWave - 1) return s;
-    p = f + 1;
-    pending = (~0ull << 1) << f;
-  }
-}
-
-template <int THREADS, int SLABS, int N>
+template <int THREADS, int SLABS, int N, bool CHECK_SIGN>
 __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
                                       RowSumLds<THREADS / kWave, SLABS, N> *lds) {
   using namespace ordered_sum;
@@ -412,20 +251,20 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
   const int W = THREADS / kWave;
   const int NCH = W * SLABS;
   const int CPL = (NCH + kWave - 1) / kWave;
-  static_assert(NCH % CPL == 0 && SLABS % CPL == 0, "chunk table does not tile the lanes");
-  static_assert(SLABS <= 32, "the per-wave dirty mask has 32 bits");
+  static_assert(NCH % CPL == 0, "chunk table does not tile the lanes");
+  static_assert(SLABS <= 32, "the per-wave masks have 32 bits");
+  static_assert(kWave * N <= 256, "a list's length must fit the bits it is filed in");
   const int wave = __builtin_amdgcn_readfirstlane(WaveId());
   const int lane = LaneId();
-  const float margin = PlanMargin(cols);
 
-  /* A: approximate chunk sums */
+  /* A: approximate sum and largest term of every chunk */
   MSHADOW_ROWSUM_STAMP(0)
   if (threadIdx.x == 0) {
     lds->s = 0.0f;
-    lds->ex = 0u;
     lds->fail = 0;
     lds->nslots = 0u;
   }
+  if (CHECK_SIGN) __syncthreads();  // the sign check below may set `fail`
   {
     float part[SLABS];
 #pragma unroll
@@ -434,82 +273,109 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
 #pragma unroll
       for (int i = 1; i < N; ++i) part[j] += v[j][i];
     }
-    const float mine = mshadow::hip::WaveSumMany<SLABS>(part);  // lane l: chunk l % SLABS
-    if (lane < SLABS) lds->approx[wave * SLABS + lane] = mine;
+    const float mine = mshadow::hip::WaveSumMany<SLABS>(part);  // lane l: slab l % SLABS
+    if (lane < SLABS) lds->approx[lane * W + wave] = mine;
+    asm volatile("" ::: "memory");  // the two tables one after the other: fewer registers live
+    float least = 0.0f;
+#pragma unroll
+    for (int j = 0; j < SLABS; ++j) {
+      part[j] = v[j][0];
+#pragma unroll
+      for (int i = 1; i < N; ++i) part[j] = (part[j] < v[j][i]) ? v[j][i] : part[j];
+      if (CHECK_SIGN) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) least = (v[j][i] < least) ? v[j][i] : least;
+      }
+    }
+    const float most = mshadow::hip::WaveReduceMany<mshadow::hip::WaveOpMax, float, SLABS>(part);
+    if (lane < SLABS) lds->cmax[lane * W + wave] = most;
+    /* the plan is made for non-negative terms */
+    if (CHECK_SIGN && __ballot(least < 0.0f) != 0ull && lane == 0) lds->fail = 1;
   }
   __syncthreads();
   MSHADOW_ROWSUM_STAMP(1)
 
   /* B: plan per chunk, identical in every wave */
-  uint32_t code[CPL];   // int codes kept as raw bits for TableAt
-  float start[CPL];     // approximate prefix sum in front of each chunk
-  float approx_total;
+  uint32_t code[CPL];     // 1 + binade of a certain chunk, 0: to be listed
+  uint32_t start[CPL];    // approximate prefix sum in front of each chunk (float bits)
+  uint32_t lowb[CPL];     // what the sum is at least in front of each chunk (float bits)
   {
-    float pre[CPL + 1];
+    float pre[CPL + 1], seen[CPL + 1];
     pre[0] = 0.0f;
+    seen[0] = 0.0f;
 #pragma unroll
     for (int c = 0; c < CPL; ++c) {
       const int k = lane * CPL + c;
       pre[c + 1] = pre[c] + (k < NCH ? lds->approx[k] : 0.0f);
+      const float m = k < NCH ? lds->cmax[k] : 0.0f;
+      seen[c + 1] = (seen[c] < m) ? m : seen[c];
     }
     const float incl = WaveInclusiveScanF32(pre[CPL]);
     const float excl = incl - pre[CPL];
-    approx_total = ReadLaneF32(incl, kWave - 1);
+    const float approx_total = ReadLaneF32(incl, kWave - 1);
+    /* a NaN among the terms makes the sum NaN whatever the order */
+    if (approx_total != approx_total) return approx_total;
+    const float seen_incl = mshadow::hip::WaveInclusiveScanMaxF32(seen[CPL]);
+    const float seen_excl = __uint_as_float(FromLaneBelowU32(__float_as_uint(seen_incl), 0u));
+    /* the sum never decreases and is never below a term already added: the lower bound of
+       a chunk is the largest over its own estimate and everything in front of it */
+    float low[CPL];
+    float low_run = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+      const int k = lane * CPL + c;
+      const float st = excl + pre[c];
+      float lo = PlanLowBound(st, static_cast<float>(k) * static_cast<float>(kWave * N));
+      const float sm = (seen_excl < seen[c]) ? seen[c] : seen_excl;
+      lo = (lo < sm) ? sm : lo;
+      low_run = (low_run < lo) ? lo : low_run;
+      low[c] = low_run;
+      start[c] = __float_as_uint(st);
+    }
+    const float low_incl = mshadow::hip::WaveInclusiveScanMaxF32(low[CPL - 1]);
+    const float low_excl = __uint_as_float(FromLaneBelowU32(__float_as_uint(low_incl), 0u));
     int raw[CPL];
 #pragma unroll
     for (int c = 0; c < CPL; ++c) {
-      start[c] = excl + pre[c];
-      raw[c] = PlanPiece(start[c], excl + pre[c + 1], margin);
+      const float lo = (low[c] < low_excl) ? low_excl : low[c];
+      lowb[c] = __float_as_uint(lo);
+      raw[c] = PlanBinade(lo, PlanHighBound(excl + pre[c + 1]));
     }
-    /* neighbouring clean chunks must agree on the binade, or the later one is walked:
-       every run of clean chunks then has one scale */
-    const int before = __shfl_up(raw[CPL - 1], 1);
+    /* neighbouring certain chunks must agree on the binade, or the later one is listed:
+       every run of certain chunks then has one scale */
+    const int before = static_cast<int>(FromLaneBelowU32(static_cast<uint32_t>(raw[CPL - 1]),
+                                                         static_cast<uint32_t>(-1)));
 #pragma unroll
     for (int c = 0; c < CPL; ++c) {
-      const int prev = (c == 0) ? ((lane == 0) ? kPlanWalk : before) : raw[c - 1];
-      const bool clash = IsClean(raw[c]) && IsClean(prev) && prev != raw[c];
-      code[c] = static_cast<uint32_t>(clash ? kPlanTwoBinades + (prev < raw[c] ? prev : raw[c]) : raw[c]);
+      const int prev = (c == 0) ? before : raw[c - 1];
+      const bool clash = raw[c] >= 0 && prev >= 0 && prev != raw[c];
+      code[c] = (raw[c] < 0 || clash) ? 0u : static_cast<uint32_t>(raw[c]) + 1u;
     }
   }
-  /* a NaN among the terms makes the sum NaN whatever the order */
-  if (approx_total != approx_total) return approx_total;
 
-  /* C: integer totals of this wave's clean chunks ... */
+  /* C: integer totals of this wave's certain chunks ... */
   MSHADOW_ROWSUM_STAMP(2)
-  uint32_t dirty_mask;  // this wave's slabs that have to be walked
-  uint32_t tie_mask;    // of those, planned clean but found to hold a tie
+  uint32_t listed = 0u;  // this wave's slabs that go to the chain as lists
   {
-    float part[SLABS];
+    uint32_t part[SLABS];
 #pragma unroll
     for (int j = 0; j < SLABS; ++j) {
-      const int k = wave * SLABS + j;
-      const int ck = static_cast<int>(ReadLaneU32(code[j % CPL], k / CPL));
-      part[j] = 0.0f;
-      if (IsClean(ck)) part[j] = LaneQuant<N>(v[j], BinadeOfExponent(static_cast<uint32_t>(ck)));
+      const uint32_t ck = TableAt<CPL>(code, j * W + wave);
+      const LaneQuantum lq = LaneDualQuant<N>(v[j], ck != 0u ? ck - 1u : 1u);
+      part[j] = lq.q;
+      if (ck == 0u || __ballot(!lq.ok) != 0ull) listed |= 1u << j;
     }
-    const float q = mshadow::hip::WaveSumMany<SLABS>(part);  // lane l: chunk l % SLABS
-    /* lanes 0 .. SLABS-1 file the result of "their" chunk; its plan code sits in the
-       chunk table at lane k / CPL, slot k % CPL = lane % CPL */
-    const int k = wave * SLABS + (lane % SLABS);
-    int ck = 0;
-#pragma unroll
-    for (int c = 0; c < CPL; ++c) {
-      const int got = __shfl(static_cast<int>(code[c]), k / CPL);
-      ck = (lane % CPL == c) ? got : ck;
+    const uint32_t total = mshadow::hip::WaveReduceMany<mshadow::hip::WaveOpSum, uint32_t, SLABS>(part);
+    /* lanes 0 .. SLABS-1 file the result of "their" chunk; a total that cannot fit a binade
+       is cut so that sums of totals stay inside 32 bits (the run it joins fails its check) */
+    if (lane < SLABS && ((listed >> lane) & 1u) == 0u) {
+      lds->q[lane * W + wave] = total < (1u << 24) ? total : (1u << 24);
     }
-    const bool clean = IsClean(ck);
-    const bool whole = clean && q < kLimit;  // a tie anywhere in the chunk pushes q past 2^24
-    if (lane < SLABS) {
-      lds->q[k] = whole ? static_cast<uint32_t>(q) : kDirtyQ;
-    }
-    dirty_mask = static_cast<uint32_t>(__ballot(lane < SLABS && !whole));
-    tie_mask = static_cast<uint32_t>(__ballot(lane < SLABS && clean && !whole));
   }
-  /* ... and its dirty ones handed, with their terms, to plan slots: the lane plans are
-     made by all waves together further down (the first wave of a row owns most dirty chunks) */
-  for (uint32_t todo = dirty_mask; todo != 0u; todo &= todo - 1u) {
+  /* ... and a list of addends for each of the others */
+  for (uint32_t todo = listed; todo != 0u; todo &= todo - 1u) {
     const int j = __ffs(static_cast<int>(todo)) - 1;
-    const int k = wave * SLABS + j;
+    const int k = j * W + wave;
     uint32_t slot = 0u;
     if (lane == 0) slot = atomicAdd(&lds->nslots, 1u);
     slot = __builtin_amdgcn_readfirstlane(slot);
@@ -519,198 +385,220 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
     }
     float t[N];
     SelectSlab<SLABS, N>(t, v, j);
-    LanePlanSlot<N> *ps = &lds->plan[slot];
+    const float st = __uint_as_float(TableAt<CPL>(start, k));
+    const float lb = __uint_as_float(TableAt<CPL>(lowb, k));
+    /* the lane's own bounds: approximate prefix sums inside the chunk, largest term so far */
+    float a = t[0], m = t[0];
 #pragma unroll
-    for (int i = 0; i < N; ++i) ps->t[lane][i] = t[i];
-    int ck = static_cast<int>(TableAt<CPL>(code, k));
-    if ((tie_mask >> j) & 1u) ck = kPlanTwoBinades + ck;
-    uint32_t start_bits[CPL];
-#pragma unroll
-    for (int c = 0; c < CPL; ++c) start_bits[c] = __float_as_uint(start[c]);
-    const float st = __uint_as_float(TableAt<CPL>(start_bits, k));
-    if (lane == 0) {
-      ps->kind = ck;
-      ps->start = st;
-      ps->chunk = k;
+    for (int i = 1; i < N; ++i) {
+      a += t[i];
+      m = (m < t[i]) ? t[i] : m;
     }
+    const float incl = WaveInclusiveScanF32(a);
+    const float seen_incl = mshadow::hip::WaveInclusiveScanMaxF32(m);
+    const float seen = __uint_as_float(FromLaneBelowU32(__float_as_uint(seen_incl), 0u));
+    float lo = PlanLowBound(st + (incl - a), static_cast<float>(k * kWave + lane) * static_cast<float>(N));
+    lo = (lo < seen) ? seen : lo;
+    lo = (lo < lb) ? lb : lo;
+    int c = PlanBinade(lo, PlanHighBound(st + incl));
+    const LaneQuantum lq = LaneDualQuant<N>(t, c >= 0 ? static_cast<uint32_t>(c) : 1u);
+    if (!lq.ok) c = -1;
+    /* runs: maximal stretches of certain lanes with one binade; the first lane of a run
+       files the run's addend, any other lane of it files nothing */
+    const int below = static_cast<int>(FromLaneBelowU32(static_cast<uint32_t>(c), static_cast<uint32_t>(-1)));
+    const bool term_lane = c < 0;
+    const bool head = c >= 0 && below != c;
+    const uint32_t qi = term_lane ? 0u : lq.q;
+    const uint32_t q_incl = WaveInclusiveScanU32(qi);
+    const unsigned long long edges = __ballot(term_lane || head);
+    const unsigned long long above = (edges >> lane) >> 1;
+    const int next_edge = above != 0ull ? lane + __ffsll(static_cast<long long>(above)) : kWave;
+    const uint32_t q_end = static_cast<uint32_t>(__shfl(static_cast<int>(q_incl), next_edge - 1));
+    const uint32_t n_mine = term_lane ? static_cast<uint32_t>(N) : (head ? 1u : 0u);
+    const uint32_t n_incl = WaveInclusiveScanU32(n_mine);
+    const uint32_t at = n_incl - n_mine;
+    AddendList<N> *out = &lds->list[slot];
+    if (term_lane) {
+#pragma unroll
+      for (int i = 0; i < N; ++i) {
+        out->addend[at + i] = t[i];
+        out->check[at + i] = 0;
+      }
+    } else if (head) {
+      out->addend[at] = RunAddend(static_cast<uint32_t>(c), q_end - (q_incl - qi));
+      out->check[at] = static_cast<unsigned char>(c + 1);
+    }
+    if (lane == kWave - 1) lds->q[k] = kListedBit | (n_incl << 8) | slot;
   }
   __syncthreads();
   MSHADOW_ROWSUM_STAMP(3)
-  /* D: tables of the walk */
-  uint32_t ex[CPL];  // integer prefix over clean chunks in front of each chunk
-  uint32_t total_ex;
-  {
-    uint32_t pre[CPL + 1];
-    pre[0] = 0u;
-#pragma unroll
-    for (int c = 0; c < CPL; ++c) {
-      const int k = lane * CPL + c;
-      const uint32_t q = k < NCH ? lds->q[k] : 0u;
-      if (q == kDirtyQ && IsClean(static_cast<int>(code[c]))) code[c] = static_cast<uint32_t>(kPlanWalk);
-      const bool is_dirty = k < NCH && !IsClean(static_cast<int>(code[c]));
-      pre[c + 1] = pre[c] + (is_dirty ? 0u : q);
-    }
-    const uint32_t incl = WaveInclusiveScanU32(pre[CPL]);
-    const uint32_t excl = incl - pre[CPL];
-#pragma unroll
-    for (int c = 0; c < CPL; ++c) ex[c] = excl + pre[c];
-    total_ex = ReadLaneU32(incl, kWave - 1);
-  }
-  /* lane plans of the dirty chunks, made by all waves together */
-  {
-    const uint32_t handed = lds->nslots;
-    const int nslots = handed < static_cast<uint32_t>(Lds::kSlots) ? static_cast<int>(handed) : Lds::kSlots;
-    /* slots were handed out in no particular order: the walk takes them by chunk number */
-    const int chunk_of_lane = lane < nslots ? lds->plan[lane < Lds::kSlots ? lane : 0].chunk : 0x7fffffff;
-    for (int sl = wave; sl < nslots; sl += W) {
-      LanePlanSlot<N> *ps = &lds->plan[sl];
-      float t[N];
-#pragma unroll
-      for (int i = 0; i < N; ++i) t[i] = ps->t[lane][i];
-      const int ck = ps->kind;
-      uint32_t pa, pb;
-      if (ck >= kPlanTwoBinades) {
-        unsigned long long tlo, thi;
-        PlanTwoBinades<N>(t, ck - kPlanTwoBinades, &pa, &pb, &tlo, &thi);
-        if (lane == 0) {
-          ps->tie_lo = tlo;
-          ps->tie_hi = thi;
-        }
-      } else {
-        int code_l;
-        const uint32_t tot = PlanLanes<N>(t, ps->start, margin, ps->chunk == 0, &pa, &code_l);
-        pb = static_cast<uint32_t>(code_l);
-        if (lane == 0) ps->total = tot;
-      }
-      ps->a[lane] = pa;
-      ps->b[lane] = pb;
-      /* what the walk needs from the chunk table, so that it reads scalars only */
-      const int k = ps->chunk;
-      const uint32_t exk = TableAt<CPL>(ex, k);
-      const uint32_t erun = k > 0 ? TableAt<CPL>(code, k - 1) : 0u;
-      const int rank = __popcll(__ballot(chunk_of_lane < k));
-      if (lane == 0) {
-        ps->ex = exk;
-        ps->e_run = static_cast<int>(erun);
-        lds->order[rank] = static_cast<signed char>(sl);
-      }
-    }
-  }
 
-  __syncthreads();
-  MSHADOW_ROWSUM_STAMP(4)
-  /* the walk: one wave takes the dirty chunks in row order; everything it needs sits in the
-     plan slots */
+  /* D: the chain, in one wave */
   if (wave == 0 && lds->fail == 0) {
-    MSHADOW_ROWSUM_STAMP(8)
     /* the whole row waits for this chain; the other waves on this SIMD (another row's bulk
        phases) yield issue slots to it */
     __builtin_amdgcn_s_setprio(3);
-    const uint32_t handed = lds->nslots;
-    const int nslots = handed < static_cast<uint32_t>(Lds::kSlots) ? static_cast<int>(handed) : Lds::kSlots;
-    const int slot_at = lane < nslots ? lds->order[lane < Lds::kSlots ? lane : 0] : 0;
+    /* integer prefix over the certain chunks, and the listed chunks in row order */
+    uint32_t ex[CPL];
+    uint32_t qk[CPL];
+    uint32_t total_ex, nitems;
+    {
+      uint32_t pre[CPL + 1], cnt[CPL + 1];
+      pre[0] = 0u;
+      cnt[0] = 0u;
+#pragma unroll
+      for (int c = 0; c < CPL; ++c) {
+        qk[c] = lane * CPL + c < NCH ? lds->q[lane * CPL + c] : 0u;
+        const bool is_listed = (qk[c] & kListedBit) != 0u;
+        if (is_listed) code[c] = 0u;  // planned certain, found to hold a tie
+        pre[c + 1] = pre[c] + (is_listed ? 0u : qk[c]);
+        cnt[c + 1] = cnt[c] + (is_listed ? 1u : 0u);
+      }
+      const uint32_t incl = WaveInclusiveScanU32(pre[CPL]);
+      const uint32_t cincl = WaveInclusiveScanU32(cnt[CPL]);
+      total_ex = ReadLaneU32(incl, kWave - 1);
+      nitems = ReadLaneU32(cincl, kWave - 1);
+      const uint32_t before = FromLaneBelowU32(code[CPL - 1], 0u);
+#pragma unroll
+      for (int c = 0; c < CPL; ++c) {
+        ex[c] = incl - pre[CPL] + pre[c];
+        if ((qk[c] & kListedBit) != 0u) {
+          const uint32_t rank = cincl - cnt[CPL] + cnt[c];
+          lds->item_q[rank] = qk[c];
+          lds->item_ex[rank] = ex[c];
+          lds->item_run[rank] = (c == 0) ? before : code[c - 1];
+        }
+      }
+    }
+    MSHADOW_ROWSUM_STAMP(4)
+    const bool mine = lane < static_cast<int>(nitems);
+    const uint32_t it_q = mine ? lds->item_q[lane] : 0u;
+    const uint32_t it_ex = mine ? lds->item_ex[lane] : 0u;
+    const uint32_t it_run = mine ? lds->item_run[lane] : 0u;
     float s = 0.0f;
     uint32_t done = 0u;
-    bool fail = false;
-    /* the lane-wise part of the next chunk's slot is fetched while the current chunk's chain
-       of dependent instructions runs (none of it depends on the running sum) */
-    float nt[N];
-    uint32_t npa = 0u, npb = 0u;
-    const LanePlanSlot<N> *nps = &lds->plan[ReadLaneU32(static_cast<uint32_t>(slot_at), 0)];
-    if (nslots > 0) {
-#pragma unroll
-      for (int e = 0; e < N; ++e) nt[e] = nps->t[lane][e];
-      npa = nps->a[lane];
-      npb = nps->b[lane];
+    bool ok = true;
+    /* the first block of the next item is fetched while the current item's chain runs */
+    float na = 0.0f;
+    uint32_t nc = 0u;
+    if (nitems > 0u) {
+      const uint32_t q0 = ReadLaneU32(it_q, 0);
+      const AddendList<N> *l0 = &lds->list[q0 & 0xffu];
+      const int n0 = static_cast<int>((q0 >> 8) & 0x1ffu);
+      if (lane >= 1 && lane <= n0) {
+        na = l0->addend[lane - 1];
+        nc = l0->check[lane - 1];
+      }
     }
-    for (int i = 0; i < nslots; ++i) {
-      const LanePlanSlot<N> *ps = nps;
-      float t[N];
-#pragma unroll
-      for (int e = 0; e < N; ++e) t[e] = nt[e];
-      const uint32_t pa = npa, pb = npb;
-      const int kind = ps->kind;
-      const uint32_t exk = ps->ex;
-      const int erun = ps->e_run;
-      if (i + 1 < nslots) {
-        nps = &lds->plan[ReadLaneU32(static_cast<uint32_t>(slot_at), i + 1)];
-#pragma unroll
-        for (int e = 0; e < N; ++e) nt[e] = nps->t[lane][e];
-        npa = nps->a[lane];
-        npb = nps->b[lane];
+    for (uint32_t i = 0; i < nitems; ++i) {
+      const uint32_t q = ReadLaneU32(it_q, static_cast<int>(i));
+      const uint32_t exk = ReadLaneU32(it_ex, static_cast<int>(i));
+      const uint32_t run = ReadLaneU32(it_run, static_cast<int>(i));
+      const AddendList<N> *li = &lds->list[q & 0xffu];
+      const int n = static_cast<int>((q >> 8) & 0x1ffu);
+      float a = na;
+      uint32_t chk = nc;
+      /* position 0 of the item: the run of certain chunks in front of the listed chunk */
+      if (lane == 0) {
+        a = run != 0u ? RunAddend(run - 1u, exk - done) : 0.0f;
+        chk = run;
       }
-      if (exk != done) {
-        s = FlushRun(s, erun, exk - done, &fail);
-        done = exk;
+      done = exk;
+      na = 0.0f;
+      nc = 0u;
+      if (i + 1u < nitems) {
+        const uint32_t q1 = ReadLaneU32(it_q, static_cast<int>(i + 1u));
+        const AddendList<N> *l1 = &lds->list[q1 & 0xffu];
+        const int n1 = static_cast<int>((q1 >> 8) & 0x1ffu);
+        if (lane >= 1 && lane <= n1) {
+          na = l1->addend[lane - 1];
+          nc = l1->check[lane - 1];
+        }
       }
-      if (kind >= kPlanTwoBinades) {
-        s = WalkTwoBinades<N>(s, t, kind - kPlanTwoBinades, pa, pb, ps->tie_lo, ps->tie_hi, &fail);
-      } else if (ps->chunk == 0) {
-        s = HeadSerialAdd<N>(s, ps->t);
-        s = WalkLanes<N>(s, t, pa, static_cast<int>(pb), ps->total, (1ull << kHeadLanes) - 1ull, &fail);
-      } else {
-        s = WalkLanes<N>(s, t, pa, static_cast<int>(pb), ps->total, 0ull, &fail);
+      const int first = n + 1 < kWave ? n + 1 : kWave;
+      s = ChainBlock(s, a, chk, first, &ok);
+      for (int g0 = kWave; g0 < n + 1; g0 += kWave) {  // lists longer than a wave
+        const int left = n + 1 - g0;
+        const int cnt = left < kWave ? left : kWave;
+        float a2 = 0.0f;
+        uint32_t c2 = 0u;
+        if (lane < cnt) {
+          a2 = li->addend[g0 + lane - 1];
+          c2 = li->check[g0 + lane - 1];
+        }
+        s = ChainBlock(s, a2, c2, cnt, &ok);
+      }
+    }
+    /* the run of certain chunks behind the last listed one */
+    {
+      const uint32_t run = TableAt<CPL>(code, NCH - 1);
+      if (run != 0u) {
+        const float before = s;
+        s = s + RunAddend(run - 1u, total_ex - done);
+        ok = ok && RunHolds(before, s, run - 1u);
       }
     }
     if (lane == 0) {
       lds->s = s;
-      lds->ex = done;
-      if (fail) lds->fail = 1;
+      if (!ok) lds->fail = 1;
     }
     __builtin_amdgcn_s_setprio(0);
-    MSHADOW_ROWSUM_STAMP(9)
   }
   __syncthreads();
-
-  /* E: the clean run behind the last dirty chunk */
   MSHADOW_ROWSUM_STAMP(5)
-  float s = lds->s;
-  bool fail = lds->fail != 0;
-  if (total_ex != lds->ex) {
-    s = FlushRun(s, static_cast<int>(TableAt<CPL>(code, NCH - 1)), total_ex - lds->ex, &fail);
-  }
-  MSHADOW_ROWSUM_STAMP(6)
-  if (!fail) return s;
+  if (lds->fail == 0) return lds->s;
   MSHADOW_ROWSUM_STAMP(7)
 
-  /* a plan did not hold (kept so that the result cannot depend on the plan): every chunk
-     is resolved in order by wave scans, wave after wave */
+  /* the plan did not hold (kept so that the result cannot depend on the plan): every chunk
+     is resolved in row order by wave scans, wave after wave */
   __syncthreads();
   if (threadIdx.x == 0) lds->s = 0.0f;
   __syncthreads();
-  for (int w = 0; w < W; ++w) {
-    if (wave == w) {
-      float r = lds->s;
-      for (int j = 0; j < SLABS; ++j) {
-        float t[N];
-        SelectSlab<SLABS, N>(t, v, j);
-        r = WaveResolve<N>(r, t);
+  for (int j = 0; j < SLABS; ++j) {
+    float t[N];
+    SelectSlab<SLABS, N>(t, v, j);
+    for (int w = 0; w < W; ++w) {
+      if (wave == w) {
+        const float r = WaveResolve<N>(lds->s, t);
+        if (lane == 0) lds->s = r;
       }
-      if (lane == 0) lds->s = r;
+      __syncthreads();
     }
-    __syncthreads();
   }
   return lds->s;
 }
 
-/*! \brief e^x for x <= 0 (any float accepted): 2^(x * log2 e) with the rounding error of
- *  the product carried separately, so the result stays within about 1.5 ulp for the whole
- *  range a softmax sees. The hardware exp2 does not return subnormals, so results below
- *  2^-126 are computed 64 binades up and scaled back. */
+/*! \brief the larger of two / three floats, a NaN operand ignored (one instruction; the
+ *  source-level forms compile to a compare and a select, or to extra canonicalising ops) */
+__device__ __forceinline__ float MaxNum(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ float MaxNum3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
+/*! \brief e^x for x <= 0 (any float accepted; -inf gives 0, NaN gives NaN), straight-line:
+ *  h = 2^(x * log2(e) / 2) from the hardware exp2, with the rounding error of the product
+ *  carried separately, then e^x = h * h * 2^r. The hardware exp2 does not return subnormals;
+ *  h is a normal number whenever e^x is not zero, and the product h * h rounds correctly into
+ *  the subnormal range. The result stays within about 3 ulp for the whole range a softmax
+ *  sees. */
 __device__ __forceinline__ float ExpNonPositive(float x) {
-  const float kLog2eHi = 1.44269502162933349609375f;
-  const float kLog2eLo = 1.925963033500011079013347625732421875e-08f;
-  const float t = x * kLog2eHi;
-  float r = __builtin_fmaf(x, kLog2eHi, -t);   // exact rounding error of the product
-  r = __builtin_fmaf(x, kLog2eLo, r);
-  if (__builtin_expect(!(t >= -125.0f), 0)) {   // subnormal / zero result, -inf, NaN
-    if (t < -151.0f) return 0.0f;               // below half of the smallest subnormal
-    const float e = __builtin_amdgcn_exp2f(t + 64.0f);
-    const float v = __builtin_fmaf(e, r * 0.693147182464599609375f, e);
-    return v * 5.42101086242752217003726400434970855712890625e-20f;  // 2^-64
-  }
-  const float e = __builtin_amdgcn_exp2f(t);
-  return __builtin_fmaf(e, r * 0.693147182464599609375f, e);  // e * 2^r, |r| << 1
+  const float kHalfLog2eHi = 0.5f * 1.44269502162933349609375f;
+  const float kHalfLog2eLo = 0.5f * 1.925963033500011079013347625732421875e-08f;
+  const float t = x * kHalfLog2eHi;
+  float r = __builtin_fmaf(x, kHalfLog2eHi, -t);   // exact rounding error of the product
+  r = __builtin_fmaf(x, kHalfLog2eLo, r);
+  const float h = __builtin_amdgcn_exp2f(t);
+  /* 2^(2 r) - 1 = r * 2 ln 2, |r| << 1. For x = -inf the error term is inf - inf: the NaN
+     is dropped here (h is 0 then), while a NaN x still arrives through h. */
+  const float c = MaxNum(r * 1.38629436111989061883f, -1.0f);
+  const float e = h * h;
+  return __builtin_fmaf(e, c, e);
 }
 
 /*! \brief p / s given rcp = 1 / s: one Newton correction on the quotient. The result is
@@ -737,51 +625,89 @@ __device__ inline float BlockMax(float v, float *wmax) {
 }
 
 /*! \brief THREADS * SLABS * VEC >= cols. VEC == 4 needs 16-byte aligned rows and
- *  cols % 4 == 0. Wave w holds columns [w, w + 1) * SLABS * 64 * VEC, slab j of it the
- *  next 64 * VEC, lane l of that VEC consecutive ones: each load is one contiguous
- *  kilobyte per wave and the order of the row is wave, slab, lane, element.
+ *  cols % 4 == 0. Slab j of wave w holds the 64 * VEC columns from (j * W + w) * 64 * VEC,
+ *  lane l of that VEC consecutive ones: each load is one contiguous kilobyte per wave, the
+ *  W waves together stream one contiguous stretch per slab, and the order of the row is
+ *  slab, wave, lane, element.
  *  TERMS_GIVEN: src already holds the (non-negative) terms and dst[row] receives their
  *  left-to-right sum - the row-sum stage on its own. */
 template <int THREADS, int SLABS, int VEC, bool TERMS_GIVEN>
 __global__ void __launch_bounds__(THREADS, 4)  // >= 4 waves per SIMD: two 512-thread rows per CU
     SoftmaxRowKernel(float *dst, int dstride, const float *src, int sstride, int cols) {
   __shared__ RowSumLds<THREADS / kWave, SLABS, VEC> lds;
+  const int W = THREADS / kWave;
+  const int kChunk = kWave * VEC;  // columns of one chunk
   const int wave = __builtin_amdgcn_readfirstlane(WaveId());
-  const int lane = LaneId();
+  const uint32_t lane_col = LaneId() * VEC;
   const float *in = src + static_cast<size_t>(blockIdx.x) * sstride;
   float *out = dst + static_cast<size_t>(blockIdx.x) * dstride;
   const float kNegInf = -__builtin_huge_valf();
+  /* columns past the end of the row: -inf logits (their terms are exactly 0), zero terms */
   const float kAbsent = TERMS_GIVEN ? 0.0f : kNegInf;
 
+  MSHADOW_ROWSUM_STAMP(10)
+  /* chunk k = j * W + wave starts at column k * kChunk; whether it lies wholly inside the
+     row is the same for all lanes, so the common case carries no per-lane guards */
   float v[SLABS][VEC];
-  float mx = kNegInf;
 #pragma unroll
   for (int j = 0; j < SLABS; ++j) {
-    const int base = ((wave * SLABS + j) * kWave + lane) * VEC;
-    if (VEC == 4) {  // cols % 4 == 0: a pack is either whole or absent
-      F4 q = {kAbsent, kAbsent, kAbsent, kAbsent};
-      if (base < cols) q = StreamLoadF4(in + base);
-      v[j][0] = q.x; v[j][1 % VEC] = q.y; v[j][2 % VEC] = q.z; v[j][3 % VEC] = q.w;
+    const int c0 = (j * W + wave) * kChunk;
+    const float *at = in + c0;  // uniform
+    if (c0 + kChunk <= cols) {
+      if (VEC == 4) {
+        const F4 q = StreamLoadF4(at + lane_col);
+        v[j][0] = q.x; v[j][1 % VEC] = q.y; v[j][2 % VEC] = q.z; v[j][3 % VEC] = q.w;
+      } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[j][i] = at[lane_col + i];
+      }
     } else {
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) v[j][i] = (base + i < cols) ? in[base + i] : kAbsent;
-    }
-    if (!TERMS_GIVEN) {
+      for (int i = 0; i < VEC; ++i) v[j][i] = kAbsent;
+      if (VEC == 4) {  // cols % 4 == 0: a pack is either whole or absent
+        if (c0 + static_cast<int>(lane_col) < cols) {
+          const F4 q = StreamLoadF4(at + lane_col);
+          v[j][0] = q.x; v[j][1 % VEC] = q.y; v[j][2 % VEC] = q.z; v[j][3 % VEC] = q.w;
+        }
+      } else {
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) mx = (mx < v[j][i]) ? v[j][i] : mx;
+        for (int i = 0; i < VEC; ++i) {
+          if (c0 + static_cast<int>(lane_col) + i < cols) v[j][i] = at[lane_col + i];
+        }
+      }
     }
   }
   if (!TERMS_GIVEN) {
-    mx = BlockMax<THREADS>(mx, lds.wmax);
+    float mx = kNegInf;
 #pragma unroll
     for (int j = 0; j < SLABS; ++j) {
-      const int base = ((wave * SLABS + j) * kWave + lane) * VEC;
+      if (VEC == 4) {
+        mx = MaxNum3(mx, v[j][0], v[j][1 % VEC]);
+        mx = MaxNum3(mx, v[j][2 % VEC], v[j][3 % VEC]);
+      } else {
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) v[j][i] = (base + i < cols) ? ExpNonPositive(v[j][i] - mx) : 0.0f;
+        for (int i = 0; i < VEC; ++i) mx = MaxNum(mx, v[j][i]);
+      }
     }
+    MSHADOW_ROWSUM_STAMP(11)
+    mx = BlockMax<THREADS>(mx, lds.wmax);
+    MSHADOW_ROWSUM_STAMP(12)
+#pragma unroll
+    for (int j = 0; j < SLABS; ++j) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) v[j][i] = ExpNonPositive(v[j][i] - mx);
+      /* one slab at a time: scheduled freely, the sixty-four independent chains would all
+         be in flight at once and spill. The empty statement consumes this slab's results
+         and hands out the next slab's inputs, so neither side can move across it. */
+      if (j + 1 < SLABS) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) asm volatile("" : "+v"(v[j + 1][i]) : "v"(v[j][i]));
+      }
+    }
+    MSHADOW_ROWSUM_STAMP(13)
   }
 
-  const float s = RowOrderedSum<THREADS, SLABS, VEC>(v, cols, &lds);
+  const float s = RowOrderedSum<THREADS, SLABS, VEC, TERMS_GIVEN>(v, cols, &lds);
   if (TERMS_GIVEN) {
     if (threadIdx.x == 0) dst[blockIdx.x] = s;
     return;
@@ -791,23 +717,36 @@ __global__ void __launch_bounds__(THREADS, 4)  // >= 4 waves per SIMD: two 512-t
      infinite logits) takes the plain division so that specials propagate as on the CPU */
   const bool fast_div = s >= 1.0f && s < 3.0e38f;
   const float rcp = 1.0f / s;
+  if (!fast_div) {
+#pragma unroll
+    for (int j = 0; j < SLABS; ++j) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) v[j][i] = v[j][i] / s;
+    }
+  }
 #pragma unroll
   for (int j = 0; j < SLABS; ++j) {
-    const int base = ((wave * SLABS + j) * kWave + lane) * VEC;
+    const int c0 = (j * W + wave) * kChunk;
+    float *at = out + c0;
     float o[VEC];
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) o[i] = fast_div ? DivideBy(v[j][i], s, rcp) : v[j][i] / s;
+    for (int i = 0; i < VEC; ++i) o[i] = fast_div ? DivideBy(v[j][i], s, rcp) : v[j][i];
     if (VEC == 4) {
       F4 q;
       q.x = o[0]; q.y = o[1 % VEC]; q.z = o[2 % VEC]; q.w = o[3 % VEC];
-      if (base < cols) StreamStoreF4(out + base, q);
+      if (c0 + kChunk <= cols) {
+        StreamStoreF4(at + lane_col, q);
+      } else if (c0 + static_cast<int>(lane_col) < cols) {
+        StreamStoreF4(at + lane_col, q);
+      }
     } else {
 #pragma unroll
       for (int i = 0; i < VEC; ++i) {
-        if (base + i < cols) out[base + i] = o[i];
+        if (c0 + static_cast<int>(lane_col) + i < cols) at[lane_col + i] = o[i];
       }
     }
   }
+  MSHADOW_ROWSUM_STAMP(14)
 }
 
 /* ---- short rows -----------------------------------------------------------------------

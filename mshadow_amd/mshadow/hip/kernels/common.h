@@ -78,55 +78,95 @@ __device__ __forceinline__ float WaveInclusiveScanF32(float v) {
 
 /*! \brief value of `v` in the lane paired with this one at distance D: lane ^ D for
  *  D = 1, 2, 8, 16, 32 and (lane + 4) % 16 within the row for D = 4 - in every case a lane
- *  whose bit log2(D) is the opposite of this lane's, which is all WaveSumMany needs */
+ *  whose bit log2(D) is the opposite of this lane's, which is all WaveReduceMany needs */
+template <int D>
+__device__ __forceinline__ uint32_t PairedLaneU32(uint32_t u) {
+  if (D == 1) return DppU32<MSHADOW_DPP_QUAD_PERM(1, 0, 3, 2), 0xf>(u, u);
+  if (D == 2) return DppU32<MSHADOW_DPP_QUAD_PERM(2, 3, 0, 1), 0xf>(u, u);
+  if (D == 4) return DppU32<MSHADOW_DPP_ROW_ROR(4), 0xf>(u, u);
+  if (D == 8) return DppU32<MSHADOW_DPP_ROW_ROR(8), 0xf>(u, u);
+  return static_cast<uint32_t>(__shfl_xor(static_cast<int>(u), D));
+}
 template <int D>
 __device__ __forceinline__ float PairedLaneF32(float v) {
-  const uint32_t u = __float_as_uint(v);
-  if (D == 1) return __uint_as_float(DppU32<MSHADOW_DPP_QUAD_PERM(1, 0, 3, 2), 0xf>(u, u));
-  if (D == 2) return __uint_as_float(DppU32<MSHADOW_DPP_QUAD_PERM(2, 3, 0, 1), 0xf>(u, u));
-  if (D == 4) return __uint_as_float(DppU32<MSHADOW_DPP_ROW_ROR(4), 0xf>(u, u));
-  if (D == 8) return __uint_as_float(DppU32<MSHADOW_DPP_ROW_ROR(8), 0xf>(u, u));
-  return __shfl_xor(v, D);
+  return __uint_as_float(PairedLaneU32<D>(__float_as_uint(v)));
 }
+template <int D>
+__device__ __forceinline__ uint32_t PairedLane(uint32_t v) { return PairedLaneU32<D>(v); }
+template <int D>
+__device__ __forceinline__ float PairedLane(float v) { return PairedLaneF32<D>(v); }
 
-/*! \brief M sums over the wave at once (M a power of two up to 32): returns, in lane l,
- *  the sum over all 64 lanes of a[l % M]. Each of the first log2(M) steps halves the
- *  number of values a lane carries (it keeps the values whose index has this lane's bit
+/*! \brief the combining steps WaveReduceMany can be asked for */
+struct WaveOpSum {
+  template <typename T>
+  static __device__ __forceinline__ T Do(T a, T b) { return a + b; }
+};
+struct WaveOpMax {  // operator< semantics, like red::maximum
+  template <typename T>
+  static __device__ __forceinline__ T Do(T a, T b) { return (a < b) ? b : a; }
+};
+
+/*! \brief M reductions over the wave at once (M a power of two up to 32): returns, in lane
+ *  l, the reduction over all 64 lanes of a[l % M]. Each of the first log2(M) steps halves
+ *  the number of values a lane carries (it keeps the values whose index has this lane's bit
  *  and hands the others to its paired lane), so the whole thing costs about M + 2 * 6
- *  additions instead of 6 * M. `a` is clobbered. Exact on integer-valued floats below 2^24;
- *  on other floats the order of additions differs from a scan. */
-template <int M, int S = 0>
-struct WaveSumManyStep {
-  static __device__ __forceinline__ void Run(float (&a)[M]) {
+ *  combining steps instead of 6 * M. `a` is clobbered. Sums are exact on integers and on
+ *  integer-valued floats below 2^24; on other floats the order of additions differs from
+ *  a scan. */
+template <typename Op, typename T, int M, int S = 0>
+struct WaveReduceManyStep {
+  static __device__ __forceinline__ void Run(T (&a)[M]) {
     const bool bit = (threadIdx.x >> S) & 1;
     const int CNT = M >> (S + 1);
 #pragma unroll
     for (int i = 0; i < CNT; ++i) {
-      const float keep = bit ? a[2 * i + 1] : a[2 * i];
-      const float send = bit ? a[2 * i] : a[2 * i + 1];
-      a[i] = keep + PairedLaneF32<(1 << S)>(send);
+      const T keep = bit ? a[2 * i + 1] : a[2 * i];
+      const T send = bit ? a[2 * i] : a[2 * i + 1];
+      a[i] = Op::Do(keep, PairedLane<(1 << S)>(send));
     }
-    WaveSumManyStep<M, ((2 << S) < M) ? S + 1 : 64>::Run(a);
+    WaveReduceManyStep<Op, T, M, ((2 << S) < M) ? S + 1 : 64>::Run(a);
   }
 };
-template <int M>
-struct WaveSumManyStep<M, 64> {
-  static __device__ __forceinline__ void Run(float (&)[M]) {}
+template <typename Op, typename T, int M>
+struct WaveReduceManyStep<Op, T, M, 64> {
+  static __device__ __forceinline__ void Run(T (&)[M]) {}
 };
-template <int M, int D>
-struct WaveSumRest {
-  static __device__ __forceinline__ float Run(float r) {
-    return WaveSumRest<M, D * 2>::Run(r + PairedLaneF32<D>(r));
+template <typename Op, typename T, int M, int D>
+struct WaveReduceRest {
+  static __device__ __forceinline__ T Run(T r) {
+    return WaveReduceRest<Op, T, M, D * 2>::Run(Op::Do(r, PairedLane<D>(r)));
   }
 };
-template <int M>
-struct WaveSumRest<M, 64> {
-  static __device__ __forceinline__ float Run(float r) { return r; }
+template <typename Op, typename T, int M>
+struct WaveReduceRest<Op, T, M, 64> {
+  static __device__ __forceinline__ T Run(T r) { return r; }
 };
+template <typename Op, typename T, int M>
+__device__ __forceinline__ T WaveReduceMany(T (&a)[M]) {
+  if (M > 1) WaveReduceManyStep<Op, T, M, (M > 1 ? 0 : 64)>::Run(a);
+  return WaveReduceRest<Op, T, M, M>::Run(a[0]);
+}
 template <int M>
 __device__ __forceinline__ float WaveSumMany(float (&a)[M]) {
-  if (M > 1) WaveSumManyStep<M, (M > 1 ? 0 : 64)>::Run(a);
-  return WaveSumRest<M, M>::Run(a[0]);
+  return WaveReduceMany<WaveOpSum, float, M>(a);
+}
+
+/*! \brief inclusive prefix maximum over lanes 0..63 of non-negative floats (a lane with
+ *  no source in a step sees 0, which is the identity for them) */
+__device__ __forceinline__ float WaveInclusiveScanMaxF32(float v) {
+#define MSHADOW_MSCAN_STEP(CTRL, MASK)                                      \
+  {                                                                         \
+    const float o = __uint_as_float(DppU32<CTRL, MASK>(0u, __float_as_uint(v))); \
+    v = (v < o) ? o : v;                                                    \
+  }
+  MSHADOW_MSCAN_STEP(MSHADOW_DPP_ROW_SHR(1), 0xf)
+  MSHADOW_MSCAN_STEP(MSHADOW_DPP_ROW_SHR(2), 0xf)
+  MSHADOW_MSCAN_STEP(MSHADOW_DPP_ROW_SHR(4), 0xf)
+  MSHADOW_MSCAN_STEP(MSHADOW_DPP_ROW_SHR(8), 0xf)
+  MSHADOW_MSCAN_STEP(MSHADOW_DPP_ROW_BCAST15, 0xa)
+  MSHADOW_MSCAN_STEP(MSHADOW_DPP_ROW_BCAST31, 0xc)
+#undef MSHADOW_MSCAN_STEP
+  return v;
 }
 
 /*! \brief sum over the 64 lanes; result in every lane (as a scalar) */
