@@ -36,8 +36,8 @@ int mshadow_probe_add_chain(int mode, int workgroups, double *ns_per_add, void *
 #define MSHADOW_PROBE_STAMP_NAMES                                                        \
   {"10 entry", "11 row loaded, thread maxima", "12 row maximum (barrier)", "13 exp",      \
    "1 chunk sums and maxima exchanged (barrier)", "2 chunk plan", \
-   "3 chunks quantised, lists written (barrier)", "4 chain: tables (wave 0)",           \
-   "5 chain done (barrier)", "14 divided and stored (stores completed)"}
+   "3 chunks quantised, lists written (barrier)", "4 row's list of addends assembled (barrier)",           \
+   "5 chain (wave 0; barrier)", "14 divided and stored (stores completed)"}
 int mshadow_probe_softmax_phases(float *dst, int dstride, const float *src, int sstride, int rows,
                                  int cols, double *mean_us, double *resident_us,
                                  double *kernel_us, int *fallback_rows, void *stream);

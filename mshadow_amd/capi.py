@@ -592,8 +592,8 @@ class Probe:
     STAMP_ORDER = (10, 11, 12, 13, 1, 2, 3, 4, 5, 14)
     STAMP_NAMES = ("entry", "row loaded, thread maxima", "row maximum (barrier)", "exp",
                    "chunk sums and maxima exchanged (barrier)", "chunk plan",
-                   "chunks quantised, lists written (barrier)", "chain: tables (wave 0)",
-                   "chain done (barrier)", "divided and stored (stores completed)")
+                   "chunks quantised, lists written (barrier)", "row's list of addends assembled (barrier)",
+                   "chain (wave 0; barrier)", "divided and stored (stores completed)")
     CHAIN_MODES = {"register": 0, "lds": 1, "lanes": 2}
 
     def __init__(self):

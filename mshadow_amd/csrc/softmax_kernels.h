@@ -36,6 +36,19 @@ using mshadow::hip::WaveId;
 using mshadow::hip::WaveInclusiveScanF32;
 using mshadow::hip::WaveMaxF32;
 
+/*! \brief the larger of two / three floats, a NaN operand ignored (one instruction; the
+ *  source-level forms compile to a compare and a select, or to extra canonicalising ops) */
+__device__ __forceinline__ float MaxNum(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ float MaxNum3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
 /*! \brief LDS scratch of the ordered sum: two alternating sets of per-wave totals and
  *  the hand-over slot for the running sum */
 template <int WAVES>
@@ -117,8 +130,10 @@ __device__ inline float BlockOrderedAdd(float s, const float (&t)[N],
  *   C  every wave: its certain chunks quantised against their binade, integer totals -> LDS;
  *      each of its other chunks planned lane by lane and written to LDS as a short list
  *      of addends (a run of certain lanes = one addend, any other lane = its terms) (barrier)
- *   D  wave 0: the chain - for each listed chunk in row order, the run of certain chunks in
- *      front of it (one addend) and its list, summed serially and every run verified (barrier)
+ *   D  every wave (redundantly): integer prefix over the certain chunks, the place of every
+ *      list in the row's list of addends; the lists are copied there, each by one wave, with
+ *      the run of certain chunks in front of each listed chunk as one more addend  (barrier)
+ *   E  wave 0: the chain - the row's addends summed serially, every run verified  (barrier)
  * A row whose plan fails a verification, or that has more listed chunks than slots, is summed
  * by wave scans instead, chunk after chunk.
  * Lane l keeps the chunk-table entries of chunks l * CPL .. l * CPL + CPL - 1. */
@@ -155,9 +170,13 @@ struct RowSumLds {
   int fail;         //!< the plan did not hold: redo the row the slow way
   uint32_t nslots;  //!< lists handed out
   float wmax[W];
-  /*! \brief the chain's work list: per listed chunk its q entry, the integer total of the
-   *  certain chunks in front of it and the binade of the chunk just in front (+1; 0: listed) */
-  uint32_t item_q[kSlots], item_ex[kSlots], item_run[kSlots];
+  /*! \brief the row's addends in row order, as the chain takes them: for each listed chunk
+   *  the run of certain chunks in front of it (one addend) and then its own list, and
+   *  at the end the run behind the last listed chunk */
+  static const int kRowAddends = 512;
+  float row_addend[kRowAddends];
+  unsigned char row_check[kRowAddends];
+  uint32_t row_count;
   AddendList<N> list[kSlots];
 };
 
@@ -225,10 +244,10 @@ __device__ __forceinline__ void SystolicStep(float *sum, float addend) {
 }
 
 /*! \brief s plus up to 64 addends, lane l holding addend l (`count` of them, zeros behind),
- *  one float add after the other; check = 1 + binade for a run (0 for a term). Clears *ok
- *  if a run was added while the sum was not in its binade. */
+ *  one float add after the other; check = 1 + binade for a run (0 for a term). A lane whose
+ *  run was added while the sum was not in its binade sets its *bad. */
 __device__ __forceinline__ float ChainBlock(float s, float addend, uint32_t check, int count,
-                                            bool *ok) {
+                                            bool *bad) {
   using namespace ordered_sum;
   float sum = s + addend;  // right in lane 0, the start of the systolic sum
   for (int done = 1; done < count; done += 8) {
@@ -236,8 +255,7 @@ __device__ __forceinline__ float ChainBlock(float s, float addend, uint32_t chec
     for (int u = 0; u < 8; ++u) SystolicStep(&sum, addend);
   }
   const float before = __uint_as_float(FromLaneBelowU32(__float_as_uint(sum), __float_as_uint(s)));
-  const bool held = check == 0u || RunHolds(before, sum, check - 1u);
-  if (__ballot(!held && LaneId() < count) != 0ull) *ok = false;
+  *bad = *bad || (check != 0u && !RunHolds(before, sum, check - 1u));
   return ReadLaneF32(sum, count - 1);
 }
 
@@ -265,32 +283,41 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
     lds->nslots = 0u;
   }
   if (CHECK_SIGN) __syncthreads();  // the sign check below may set `fail`
-  {
-    float part[SLABS];
+  /* the wave-wide reductions take the slabs in groups of at most sixteen (registers) */
+  const int GRP = SLABS < 16 ? SLABS : 16;
 #pragma unroll
-    for (int j = 0; j < SLABS; ++j) {
-      part[j] = v[j][0];
+  for (int g = 0; g < SLABS; g += GRP) {
+    float part[GRP];
 #pragma unroll
-      for (int i = 1; i < N; ++i) part[j] += v[j][i];
+    for (int j = 0; j < GRP; ++j) {
+      part[j] = v[g + j][0];
+#pragma unroll
+      for (int i = 1; i < N; ++i) part[j] += v[g + j][i];
     }
-    const float mine = mshadow::hip::WaveSumMany<SLABS>(part);  // lane l: slab l % SLABS
-    if (lane < SLABS) lds->approx[lane * W + wave] = mine;
+    const float mine = mshadow::hip::WaveSumMany<GRP>(part);  // lane l: slab g + l % GRP
+    if (lane < GRP) lds->approx[(g + lane) * W + wave] = mine;
     asm volatile("" ::: "memory");  // the two tables one after the other: fewer registers live
+#pragma unroll
+    for (int j = 0; j < GRP; ++j) {
+      if (N == 4) {
+        part[j] = MaxNum(MaxNum3(v[g + j][0], v[g + j][1 % N], v[g + j][2 % N]), v[g + j][3 % N]);
+      } else {
+        part[j] = v[g + j][0];
+#pragma unroll
+        for (int i = 1; i < N; ++i) part[j] = MaxNum(part[j], v[g + j][i]);
+      }
+    }
+    const float most = mshadow::hip::WaveReduceMany<mshadow::hip::WaveOpMax, float, GRP>(part);
+    if (lane < GRP) lds->cmax[(g + lane) * W + wave] = most;
+  }
+  if (CHECK_SIGN) {  // the plan is made for non-negative terms
     float least = 0.0f;
 #pragma unroll
     for (int j = 0; j < SLABS; ++j) {
-      part[j] = v[j][0];
 #pragma unroll
-      for (int i = 1; i < N; ++i) part[j] = (part[j] < v[j][i]) ? v[j][i] : part[j];
-      if (CHECK_SIGN) {
-#pragma unroll
-        for (int i = 0; i < N; ++i) least = (v[j][i] < least) ? v[j][i] : least;
-      }
+      for (int i = 0; i < N; ++i) least = (v[j][i] < least) ? v[j][i] : least;
     }
-    const float most = mshadow::hip::WaveReduceMany<mshadow::hip::WaveOpMax, float, SLABS>(part);
-    if (lane < SLABS) lds->cmax[lane * W + wave] = most;
-    /* the plan is made for non-negative terms */
-    if (CHECK_SIGN && __ballot(least < 0.0f) != 0ull && lane == 0) lds->fail = 1;
+    if (__ballot(least < 0.0f) != 0ull && lane == 0) lds->fail = 1;
   }
   __syncthreads();
   MSHADOW_ROWSUM_STAMP(1)
@@ -352,33 +379,53 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
       code[c] = (raw[c] < 0 || clash) ? 0u : static_cast<uint32_t>(raw[c]) + 1u;
     }
   }
+  /* the chunks to be listed get their slots in row order, known to every wave alike; a
+     chunk that turns out to hold a tie asks for one of the slots behind those */
+  uint32_t slot_of[CPL];
+  uint32_t planned;
+  {
+    uint32_t cnt[CPL + 1];
+    cnt[0] = 0u;
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) cnt[c + 1] = cnt[c] + ((code[c] == 0u && lane * CPL + c < NCH) ? 1u : 0u);
+    const uint32_t incl = WaveInclusiveScanU32(cnt[CPL]);
+    planned = ReadLaneU32(incl, kWave - 1);
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) slot_of[c] = incl - cnt[CPL] + cnt[c];
+  }
 
   /* C: integer totals of this wave's certain chunks ... */
   MSHADOW_ROWSUM_STAMP(2)
   uint32_t listed = 0u;  // this wave's slabs that go to the chain as lists
-  {
-    uint32_t part[SLABS];
 #pragma unroll
-    for (int j = 0; j < SLABS; ++j) {
-      const uint32_t ck = TableAt<CPL>(code, j * W + wave);
-      const LaneQuantum lq = LaneDualQuant<N>(v[j], ck != 0u ? ck - 1u : 1u);
+  for (int g = 0; g < SLABS; g += GRP) {
+    uint32_t part[GRP];
+#pragma unroll
+    for (int j = 0; j < GRP; ++j) {
+      const uint32_t ck = TableAt<CPL>(code, (g + j) * W + wave);
+      const LaneQuantum lq = LaneDualQuant<N>(v[g + j], ck != 0u ? ck - 1u : 1u);
       part[j] = lq.q;
-      if (ck == 0u || __ballot(!lq.ok) != 0ull) listed |= 1u << j;
+      if (ck == 0u || __ballot(!lq.ok) != 0ull) listed |= 1u << (g + j);
     }
-    const uint32_t total = mshadow::hip::WaveReduceMany<mshadow::hip::WaveOpSum, uint32_t, SLABS>(part);
-    /* lanes 0 .. SLABS-1 file the result of "their" chunk; a total that cannot fit a binade
+    const uint32_t total = mshadow::hip::WaveReduceMany<mshadow::hip::WaveOpSum, uint32_t, GRP>(part);
+    /* lanes 0 .. GRP-1 file the result of "their" chunk; a total that cannot fit a binade
        is cut so that sums of totals stay inside 32 bits (the run it joins fails its check) */
-    if (lane < SLABS && ((listed >> lane) & 1u) == 0u) {
-      lds->q[lane * W + wave] = total < (1u << 24) ? total : (1u << 24);
+    if (lane < GRP && ((listed >> (g + lane)) & 1u) == 0u) {
+      lds->q[(g + lane) * W + wave] = total < (1u << 24) ? total : (1u << 24);
     }
   }
   /* ... and a list of addends for each of the others */
   for (uint32_t todo = listed; todo != 0u; todo &= todo - 1u) {
     const int j = __ffs(static_cast<int>(todo)) - 1;
     const int k = j * W + wave;
-    uint32_t slot = 0u;
-    if (lane == 0) slot = atomicAdd(&lds->nslots, 1u);
-    slot = __builtin_amdgcn_readfirstlane(slot);
+    uint32_t slot;
+    if (TableAt<CPL>(code, k) == 0u) {
+      slot = TableAt<CPL>(slot_of, k);
+    } else {
+      slot = 0u;
+      if (lane == 0) slot = planned + atomicAdd(&lds->nslots, 1u);
+      slot = __builtin_amdgcn_readfirstlane(slot);
+    }
     if (slot >= static_cast<uint32_t>(Lds::kSlots)) {  // no room: the row is redone by wave scans
       if (lane == 0) lds->fail = 1;
       break;
@@ -433,114 +480,113 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
   __syncthreads();
   MSHADOW_ROWSUM_STAMP(3)
 
-  /* D: the chain, in one wave */
+  /* D: the row's list of addends. Lane-parallel and the same in every wave: the listed
+     chunks in row order, for each the addend of the run of certain chunks in front of it
+     (their integer totals since the previous listed chunk, which share one binade) and the
+     place of its list in the row's list; wave r % W then copies the list of listed chunk r. */
+  if (lds->fail == 0) {
+    uint32_t qk[CPL], pre[CPL + 1], cnt[CPL + 1], len[CPL + 1];
+    pre[0] = 0u;
+    cnt[0] = 0u;
+    len[0] = 0u;
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+      qk[c] = lane * CPL + c < NCH ? lds->q[lane * CPL + c] : 0u;
+      const bool is_listed = (qk[c] & kListedBit) != 0u;
+      if (is_listed) code[c] = 0u;  // planned certain, found to hold a tie
+      pre[c + 1] = pre[c] + (is_listed ? 0u : qk[c]);
+      cnt[c + 1] = cnt[c] + (is_listed ? 1u : 0u);
+      len[c + 1] = len[c] + (is_listed ? ((qk[c] >> 8) & 0x1ffu) + 1u : 0u);
+    }
+    const uint32_t incl = WaveInclusiveScanU32(pre[CPL]);
+    const uint32_t cincl = WaveInclusiveScanU32(cnt[CPL]);
+    const uint32_t lincl = WaveInclusiveScanU32(len[CPL]);
+    const uint32_t total_ex = ReadLaneU32(incl, kWave - 1);
+    const uint32_t total_len = ReadLaneU32(lincl, kWave - 1) + 1u;  // + the run at the end
+    /* ex = integer total of the certain chunks in front of a chunk; it never decreases,
+       so its value at the previous listed chunk is a running maximum */
+    uint32_t own_last = 0u;
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+      if ((qk[c] & kListedBit) != 0u) own_last = incl - pre[CPL] + pre[c];
+    }
+    const uint32_t last_incl = mshadow::hip::WaveInclusiveScanMaxU32(own_last);
+    const uint32_t last_ex = ReadLaneU32(last_incl, kWave - 1);
+    uint32_t prev_ex = FromLaneBelowU32(last_incl, 0u);
+    const uint32_t code_below = FromLaneBelowU32(code[CPL - 1], 0u);
+    if (total_len > static_cast<uint32_t>(Lds::kRowAddends)) {
+      if (threadIdx.x == 0) lds->fail = 1;
+    } else {
+#pragma unroll
+      for (int c = 0; c < CPL; ++c) {
+        const bool is_listed = (qk[c] & kListedBit) != 0u;
+        const uint32_t ex = incl - pre[CPL] + pre[c];
+        const uint32_t run = (c == 0) ? code_below : code[c - 1];
+        const uint32_t rank = cincl - cnt[CPL] + cnt[c];
+        const uint32_t at = lincl - len[CPL] + len[c];
+        const float front = run != 0u ? RunAddend(run != 0u ? run - 1u : 0u, ex - prev_ex) : 0.0f;
+        if (is_listed) prev_ex = ex;
+        for (unsigned long long todo = __ballot(is_listed && rank % W == static_cast<uint32_t>(wave));
+             todo != 0ull; todo &= todo - 1ull) {
+          const int l = __ffsll(static_cast<long long>(todo)) - 1;
+          const uint32_t q = ReadLaneU32(qk[c], l);
+          const uint32_t to = ReadLaneU32(at, l);
+          const float a0 = ReadLaneF32(front, l);
+          const uint32_t c0 = ReadLaneU32(run, l);
+          const AddendList<N> *from = &lds->list[q & 0xffu];
+          const int n = static_cast<int>((q >> 8) & 0x1ffu);
+          for (int g = lane; g < n; g += kWave) {
+            lds->row_addend[to + 1u + g] = from->addend[g];
+            lds->row_check[to + 1u + g] = from->check[g];
+          }
+          if (lane == 0) {
+            lds->row_addend[to] = a0;
+            lds->row_check[to] = static_cast<unsigned char>(c0);
+          }
+        }
+      }
+      if (threadIdx.x == 0) {  // the run of certain chunks behind the last listed one
+        const uint32_t run = TableAt<CPL>(code, NCH - 1);
+        lds->row_addend[total_len - 1u] = run != 0u ? RunAddend(run - 1u, total_ex - last_ex) : 0.0f;
+        lds->row_check[total_len - 1u] = static_cast<unsigned char>(run);
+        lds->row_count = total_len;
+      }
+    }
+  }
+  __syncthreads();
+  MSHADOW_ROWSUM_STAMP(4)
+
+  /* E: the chain, in one wave */
   if (wave == 0 && lds->fail == 0) {
     /* the whole row waits for this chain; the other waves on this SIMD (another row's bulk
        phases) yield issue slots to it */
     __builtin_amdgcn_s_setprio(3);
-    /* integer prefix over the certain chunks, and the listed chunks in row order */
-    uint32_t ex[CPL];
-    uint32_t qk[CPL];
-    uint32_t total_ex, nitems;
-    {
-      uint32_t pre[CPL + 1], cnt[CPL + 1];
-      pre[0] = 0u;
-      cnt[0] = 0u;
-#pragma unroll
-      for (int c = 0; c < CPL; ++c) {
-        qk[c] = lane * CPL + c < NCH ? lds->q[lane * CPL + c] : 0u;
-        const bool is_listed = (qk[c] & kListedBit) != 0u;
-        if (is_listed) code[c] = 0u;  // planned certain, found to hold a tie
-        pre[c + 1] = pre[c] + (is_listed ? 0u : qk[c]);
-        cnt[c + 1] = cnt[c] + (is_listed ? 1u : 0u);
-      }
-      const uint32_t incl = WaveInclusiveScanU32(pre[CPL]);
-      const uint32_t cincl = WaveInclusiveScanU32(cnt[CPL]);
-      total_ex = ReadLaneU32(incl, kWave - 1);
-      nitems = ReadLaneU32(cincl, kWave - 1);
-      const uint32_t before = FromLaneBelowU32(code[CPL - 1], 0u);
-#pragma unroll
-      for (int c = 0; c < CPL; ++c) {
-        ex[c] = incl - pre[CPL] + pre[c];
-        if ((qk[c] & kListedBit) != 0u) {
-          const uint32_t rank = cincl - cnt[CPL] + cnt[c];
-          lds->item_q[rank] = qk[c];
-          lds->item_ex[rank] = ex[c];
-          lds->item_run[rank] = (c == 0) ? before : code[c - 1];
-        }
-      }
-    }
-    MSHADOW_ROWSUM_STAMP(4)
-    const bool mine = lane < static_cast<int>(nitems);
-    const uint32_t it_q = mine ? lds->item_q[lane] : 0u;
-    const uint32_t it_ex = mine ? lds->item_ex[lane] : 0u;
-    const uint32_t it_run = mine ? lds->item_run[lane] : 0u;
+    const int count = static_cast<int>(lds->row_count);
     float s = 0.0f;
-    uint32_t done = 0u;
-    bool ok = true;
-    /* the first block of the next item is fetched while the current item's chain runs */
+    bool bad = false;
+    /* the next block is fetched while the current one is summed */
     float na = 0.0f;
     uint32_t nc = 0u;
-    if (nitems > 0u) {
-      const uint32_t q0 = ReadLaneU32(it_q, 0);
-      const AddendList<N> *l0 = &lds->list[q0 & 0xffu];
-      const int n0 = static_cast<int>((q0 >> 8) & 0x1ffu);
-      if (lane >= 1 && lane <= n0) {
-        na = l0->addend[lane - 1];
-        nc = l0->check[lane - 1];
-      }
+    if (lane < count) {
+      na = lds->row_addend[lane];
+      nc = lds->row_check[lane];
     }
-    for (uint32_t i = 0; i < nitems; ++i) {
-      const uint32_t q = ReadLaneU32(it_q, static_cast<int>(i));
-      const uint32_t exk = ReadLaneU32(it_ex, static_cast<int>(i));
-      const uint32_t run = ReadLaneU32(it_run, static_cast<int>(i));
-      const AddendList<N> *li = &lds->list[q & 0xffu];
-      const int n = static_cast<int>((q >> 8) & 0x1ffu);
-      float a = na;
-      uint32_t chk = nc;
-      /* position 0 of the item: the run of certain chunks in front of the listed chunk */
-      if (lane == 0) {
-        a = run != 0u ? RunAddend(run - 1u, exk - done) : 0.0f;
-        chk = run;
-      }
-      done = exk;
+    for (int g0 = 0; g0 < count; g0 += kWave) {
+      const float a = na;
+      const uint32_t chk = nc;
       na = 0.0f;
       nc = 0u;
-      if (i + 1u < nitems) {
-        const uint32_t q1 = ReadLaneU32(it_q, static_cast<int>(i + 1u));
-        const AddendList<N> *l1 = &lds->list[q1 & 0xffu];
-        const int n1 = static_cast<int>((q1 >> 8) & 0x1ffu);
-        if (lane >= 1 && lane <= n1) {
-          na = l1->addend[lane - 1];
-          nc = l1->check[lane - 1];
-        }
+      if (g0 + kWave + lane < count) {
+        na = lds->row_addend[g0 + kWave + lane];
+        nc = lds->row_check[g0 + kWave + lane];
       }
-      const int first = n + 1 < kWave ? n + 1 : kWave;
-      s = ChainBlock(s, a, chk, first, &ok);
-      for (int g0 = kWave; g0 < n + 1; g0 += kWave) {  // lists longer than a wave
-        const int left = n + 1 - g0;
-        const int cnt = left < kWave ? left : kWave;
-        float a2 = 0.0f;
-        uint32_t c2 = 0u;
-        if (lane < cnt) {
-          a2 = li->addend[g0 + lane - 1];
-          c2 = li->check[g0 + lane - 1];
-        }
-        s = ChainBlock(s, a2, c2, cnt, &ok);
-      }
+      const int left = count - g0;
+      s = ChainBlock(s, a, chk, left < kWave ? left : kWave, &bad);
     }
-    /* the run of certain chunks behind the last listed one */
-    {
-      const uint32_t run = TableAt<CPL>(code, NCH - 1);
-      if (run != 0u) {
-        const float before = s;
-        s = s + RunAddend(run - 1u, total_ex - done);
-        ok = ok && RunHolds(before, s, run - 1u);
-      }
-    }
+    const bool failed = __ballot(bad) != 0ull;
     if (lane == 0) {
       lds->s = s;
-      if (!ok) lds->fail = 1;
+      if (failed) lds->fail = 1;
     }
     __builtin_amdgcn_s_setprio(0);
   }
@@ -566,19 +612,6 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
     }
   }
   return lds->s;
-}
-
-/*! \brief the larger of two / three floats, a NaN operand ignored (one instruction; the
- *  source-level forms compile to a compare and a select, or to extra canonicalising ops) */
-__device__ __forceinline__ float MaxNum(float a, float b) {
-  float r;
-  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-  return r;
-}
-__device__ __forceinline__ float MaxNum3(float a, float b, float c) {
-  float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
 }
 
 /*! \brief e^x for x <= 0 (any float accepted; -inf gives 0, NaN gives NaN), straight-line:

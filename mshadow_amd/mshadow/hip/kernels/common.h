@@ -60,6 +60,22 @@ __device__ __forceinline__ uint32_t WaveInclusiveScanU32(uint32_t v) {
   v += DppU32<MSHADOW_DPP_ROW_BCAST31, 0xc>(0u, v);
   return v;
 }
+/*! \brief inclusive prefix maximum of unsigned integers over lanes 0..63 */
+__device__ __forceinline__ uint32_t WaveInclusiveScanMaxU32(uint32_t v) {
+#define MSHADOW_UMSCAN_STEP(CTRL, MASK)            \
+  {                                                \
+    const uint32_t o = DppU32<CTRL, MASK>(0u, v);  \
+    v = (v < o) ? o : v;                           \
+  }
+  MSHADOW_UMSCAN_STEP(MSHADOW_DPP_ROW_SHR(1), 0xf)
+  MSHADOW_UMSCAN_STEP(MSHADOW_DPP_ROW_SHR(2), 0xf)
+  MSHADOW_UMSCAN_STEP(MSHADOW_DPP_ROW_SHR(4), 0xf)
+  MSHADOW_UMSCAN_STEP(MSHADOW_DPP_ROW_SHR(8), 0xf)
+  MSHADOW_UMSCAN_STEP(MSHADOW_DPP_ROW_BCAST15, 0xa)
+  MSHADOW_UMSCAN_STEP(MSHADOW_DPP_ROW_BCAST31, 0xc)
+#undef MSHADOW_UMSCAN_STEP
+  return v;
+}
 /*! \brief the same for floats (used on integer-valued floats, where it is exact below 2^24) */
 __device__ __forceinline__ float WaveInclusiveScanF32(float v) {
 #define MSHADOW_FSCAN_STEP(CTRL, MASK) \
@@ -104,6 +120,12 @@ struct WaveOpSum {
 struct WaveOpMax {  // operator< semantics, like red::maximum
   template <typename T>
   static __device__ __forceinline__ T Do(T a, T b) { return (a < b) ? b : a; }
+  /* floats: one instruction (a NaN operand is ignored) instead of a compare and a select */
+  static __device__ __forceinline__ float Do(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+  }
 };
 
 /*! \brief M reductions over the wave at once (M a power of two up to 32): returns, in lane
