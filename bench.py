@@ -407,7 +407,11 @@ def run_probe(G, which):
                "steps": {k: round(v, 2) for k, v in steps.items()},
                "row_resident_us": round(resident, 2), "instrumented_kernel_us": round(kernel, 1),
                "library_kernel_us": round(G.elapsed_ms(ev[0], ev[1]) * 100.0, 1),
-               "rows_in_flight": 2 * cus, "fallback_rows": fallback}
+               "rows_in_flight": 2 * cus, "fallback_rows": fallback,
+               # the kernel's loads and stores alone, and with stand-in work between them
+               "row_copy_us": {f"{b} barriers x {k} multiply-adds per element":
+                               round(P.row_copy_us(dst, src, b, k, s), 1)
+                               for b, k in ((0, 0), (4, 0), (4, 2), (4, 4), (4, 8), (8, 4))}}
     print(json.dumps(out))
 
 

@@ -32,15 +32,24 @@ int mshadow_probe_add_chain(int mode, int workgroups, double *ns_per_add, void *
    hold and that were summed by wave scans instead. dst may alias src. */
 #define MSHADOW_PROBE_STAMP_FALLBACK 7
 #define MSHADOW_PROBE_STAMPS 16
-#define MSHADOW_PROBE_STAMP_ORDER {10, 11, 12, 13, 1, 2, 3, 4, 5, 14}
+#define MSHADOW_PROBE_STAMP_ORDER {10, 11, 12, 13, 1, 2, 6, 8, 3, 4, 5, 14}
 #define MSHADOW_PROBE_STAMP_NAMES                                                        \
   {"10 entry", "11 row loaded, thread maxima", "12 row maximum (barrier)", "13 exp",      \
    "1 chunk sums and maxima exchanged (barrier)", "2 chunk plan", \
-   "3 chunks quantised, lists written (barrier)", "4 row's list of addends assembled (barrier)",           \
+   "6 certain chunks quantised", "8 lists of the other chunks written",               \
+   "3 every wave's chunks done (barrier)", "4 row's list of addends assembled (barrier)",           \
    "5 chain (wave 0; barrier)", "14 divided and stored (stores completed)"}
 int mshadow_probe_softmax_phases(float *dst, int dstride, const float *src, int sstride, int rows,
                                  int cols, double *mean_us, double *resident_us,
                                  double *kernel_us, int *fallback_rows, void *stream);
+
+/* The memory side of that kernel alone: every workgroup loads its row into registers as the
+   softmax kernel does, meets `barriers` workgroup barriers with `spin` multiply-adds per
+   element before each, and stores the row. barriers = 0: what the access pattern itself
+   allows (one workgroup per row, two rows resident per CU); with spin > 0: how much work
+   between load and store the machine hides. kernel_us = duration of the launch. */
+int mshadow_probe_row_copy(float *dst, int dstride, const float *src, int sstride, int rows,
+                           int cols, int barriers, int spin, double *kernel_us, void *stream);
 
 #ifdef __cplusplus
 }

@@ -589,10 +589,11 @@ class Library:
 class Probe:
     """libmshadow_probe.so: measurement aids of bench.py (include/mshadow_hip_probe.h)"""
     STAMPS = 16
-    STAMP_ORDER = (10, 11, 12, 13, 1, 2, 3, 4, 5, 14)
+    STAMP_ORDER = (10, 11, 12, 13, 1, 2, 6, 8, 3, 4, 5, 14)
     STAMP_NAMES = ("entry", "row loaded, thread maxima", "row maximum (barrier)", "exp",
                    "chunk sums and maxima exchanged (barrier)", "chunk plan",
-                   "chunks quantised, lists written (barrier)", "row's list of addends assembled (barrier)",
+                   "certain chunks quantised", "lists of the other chunks written",
+                   "every wave's chunks done (barrier)", "row's list of addends assembled (barrier)",
                    "chain (wave 0; barrier)", "divided and stored (stores completed)")
     CHAIN_MODES = {"register": 0, "lds": 1, "lanes": 2}
 
@@ -606,6 +607,13 @@ class Probe:
         self.dll.mshadow_probe_softmax_phases.argtypes = [
             _p, _i, _p, _i, _i, _i, C.POINTER(C.c_double), C.POINTER(C.c_double),
             C.POINTER(C.c_double), C.POINTER(_i), _p]
+
+    def row_copy_us(self, dst, src, barriers, spin, stream=None):
+        us = C.c_double(0)
+        self.dll.mshadow_probe_row_copy.argtypes = [_p, _i, _p, _i, _i, _i, _i, _i, C.POINTER(C.c_double), _p]
+        self._check(self.dll.mshadow_probe_row_copy(dst.ptr, dst.stride, src.ptr, src.stride, src.rows,
+                                                    src.cols, barriers, spin, C.byref(us), stream))
+        return us.value
 
     def _check(self, status):
         if status != 0:

@@ -98,6 +98,41 @@ __global__ void __launch_bounds__(64) SystolicChainKernel(float *out, float a, i
   out[blockIdx.x * 64 + threadIdx.x] = s;
 }
 
+/*! \brief the memory side of the softmax kernel alone: a workgroup loads its row into
+ *  registers exactly as SoftmaxRowKernel does, meets `barriers` workgroup barriers with
+ *  `spin` dependent multiply-adds per element in between (a stand-in for the work between
+ *  the load and the store), and stores the row */
+template <int THREADS, int SLABS>
+__global__ void __launch_bounds__(THREADS, 4)
+    RowCopyKernel(float *dst, int dstride, const float *src, int sstride, int cols, int barriers,
+                  int spin) {
+  using mshadow_hipk::F4;
+  const int W = THREADS / 64;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t lane_col = (threadIdx.x & 63) * 4;
+  const float *in = src + static_cast<size_t>(blockIdx.x) * sstride;
+  float *out = dst + static_cast<size_t>(blockIdx.x) * dstride;
+  F4 v[SLABS];
+#pragma unroll
+  for (int j = 0; j < SLABS; ++j) {
+    const int c0 = (j * W + wave) * 256;
+    v[j] = F4{0.0f, 0.0f, 0.0f, 0.0f};
+    if (c0 + static_cast<int>(lane_col) < cols) v[j] = mshadow_hipk::StreamLoadF4(in + c0 + lane_col);
+  }
+  for (int b = 0; b < barriers; ++b) {
+    for (int k = 0; k < spin; ++k) {
+#pragma unroll
+      for (int j = 0; j < SLABS; ++j) v[j] = v[j] * 1.0000001f + 1e-9f;
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int j = 0; j < SLABS; ++j) {
+    const int c0 = (j * W + wave) * 256;
+    if (c0 + static_cast<int>(lane_col) < cols) mshadow_hipk::StreamStoreF4(out + c0 + lane_col, v[j]);
+  }
+}
+
 int TimeKernel(hipStream_t s, float *ms, const std::function<void()> &launch) {
   hipEvent_t a, b;
   ABI_HIP(hipEventCreate(&a));
@@ -153,6 +188,21 @@ int mshadow_probe_add_chain(int mode, int workgroups, double *ns_per_add, void *
   (void)hipFree(out);
   if (st != MSHADOW_HIP_OK) return st;
   *ns_per_add = static_cast<double>(ms) * 1e6 / adds;
+  return MSHADOW_HIP_OK;
+}
+
+int mshadow_probe_row_copy(float *dst, int dstride, const float *src, int sstride, int rows,
+                           int cols, int barriers, int spin, double *kernel_us, void *stream) {
+  ABI_REQUIRE(rows >= 1 && cols > 16384 && cols <= 32768 && cols % 4 == 0 && sstride % 4 == 0 &&
+                  dstride % 4 == 0 && kernel_us != NULL, "16384 < cols <= 32768, rows of whole packs");
+  hipStream_t s = AsStream(stream);
+  float ms = 0.0f;
+  const int st = TimeKernel(s, &ms, [&] {
+    hipLaunchKernelGGL((RowCopyKernel<512, 16>), dim3(rows), dim3(512), 0, s, dst, dstride, src, sstride,
+                       cols, barriers, spin);
+  });
+  if (st != MSHADOW_HIP_OK) return st;
+  *kernel_us = ms * 1e3;
   return MSHADOW_HIP_OK;
 }
 

@@ -148,12 +148,16 @@ const uint32_t kListedBit = 0x80000000u;
 #define MSHADOW_ROWSUM_STAMP(step)
 #endif
 
-/*! \brief the addends of one listed chunk, in row order: at most one per term. check[i] is
- *  1 + the binade the sum must be in before and after addend i (a run), or 0 (a term). */
+/*! \brief one addend of the chain: its value and, for a run, 1 + the binade the sum must be
+ *  in before and after it (0 for a term); eight bytes, written and read as one word */
+struct Addend {
+  float value;
+  uint32_t check;
+};
+/*! \brief the addends of one listed chunk, in row order: at most one per term */
 template <int N>
 struct AddendList {
-  float addend[kWave * N];
-  unsigned char check[kWave * N];
+  Addend entry[kWave * N];
 };
 
 template <int W, int SLABS, int N>
@@ -164,6 +168,16 @@ struct RowSumLds {
   static const int kSlots = (kChunks < kWanted) ? kChunks : kWanted;
   float approx[kChunks];
   float cmax[kChunks];
+  /*! \brief what a listed chunk's wave needs of the plan. Every wave computes the whole
+   *  plan and files it here (the same values from each), then reads its own chunks' entries
+   *  back: a wave sees its own stores, so no barrier is involved. */
+  struct ChunkPlan {
+    float start;    //!< approximate prefix sum in front of the chunk
+    float low;      //!< what the sum is at least in front of the chunk
+    uint32_t slot;  //!< the chunk's slot, if the plan lists it
+    uint32_t peak;  //!< the chunk holds a term above `low` (it can raise the bound inside the chunk)
+  };
+  MSHADOW_ALIGNED(16) ChunkPlan plan[kChunks];
   /*! \brief certain chunk: its integer total; listed chunk: kListedBit | addends << 8 | slot */
   uint32_t q[kChunks];
   float s;          //!< the row's sum, from the chain to everybody
@@ -174,10 +188,9 @@ struct RowSumLds {
    *  the run of certain chunks in front of it (one addend) and then its own list, and
    *  at the end the run behind the last listed chunk */
   static const int kRowAddends = 512;
-  float row_addend[kRowAddends];
-  unsigned char row_check[kRowAddends];
+  Addend row[kRowAddends];
   uint32_t row_count;
-  AddendList<N> list[kSlots];
+  MSHADOW_ALIGNED(8) AddendList<N> list[kSlots];
 };
 
 /*! \brief entry k of a table spread over lanes (CPL entries per lane); k is uniform */
@@ -243,6 +256,16 @@ __device__ __forceinline__ void SystolicStep(float *sum, float addend) {
                : "v"(addend));
 }
 
+/*! \brief eight such steps */
+__device__ __forceinline__ void SystolicSteps8(float *sum, float addend) {
+#define MSHADOW_STEP "s_nop 1\n\tv_add_f32_dpp %0, %0, %1 wave_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+  asm volatile(MSHADOW_STEP MSHADOW_STEP MSHADOW_STEP MSHADOW_STEP MSHADOW_STEP MSHADOW_STEP
+                   MSHADOW_STEP MSHADOW_STEP "s_nop 1"
+               : "+v"(*sum)
+               : "v"(addend));
+#undef MSHADOW_STEP
+}
+
 /*! \brief s plus up to 64 addends, lane l holding addend l (`count` of them, zeros behind),
  *  one float add after the other; check = 1 + binade for a run (0 for a term). A lane whose
  *  run was added while the sum was not in its binade sets its *bad. */
@@ -250,16 +273,13 @@ __device__ __forceinline__ float ChainBlock(float s, float addend, uint32_t chec
                                             bool *bad) {
   using namespace ordered_sum;
   float sum = s + addend;  // right in lane 0, the start of the systolic sum
-  for (int done = 1; done < count; done += 8) {
-#pragma unroll
-    for (int u = 0; u < 8; ++u) SystolicStep(&sum, addend);
-  }
+  for (int done = 1; done < count; done += 8) SystolicSteps8(&sum, addend);
   const float before = __uint_as_float(FromLaneBelowU32(__float_as_uint(sum), __float_as_uint(s)));
   *bad = *bad || (check != 0u && !RunHolds(before, sum, check - 1u));
   return ReadLaneF32(sum, count - 1);
 }
 
-template <int THREADS, int SLABS, int N, bool CHECK_SIGN>
+template <int THREADS, int SLABS, int N, bool CHECK_SIGN, bool UNIT_PEAK>
 __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
                                       RowSumLds<THREADS / kWave, SLABS, N> *lds) {
   using namespace ordered_sum;
@@ -296,19 +316,38 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
     }
     const float mine = mshadow::hip::WaveSumMany<GRP>(part);  // lane l: slab g + l % GRP
     if (lane < GRP) lds->approx[(g + lane) * W + wave] = mine;
-    asm volatile("" ::: "memory");  // the two tables one after the other: fewer registers live
+    if (!UNIT_PEAK) {
+      asm volatile("" ::: "memory");  // the two tables one after the other: fewer registers live
 #pragma unroll
-    for (int j = 0; j < GRP; ++j) {
-      if (N == 4) {
-        part[j] = MaxNum(MaxNum3(v[g + j][0], v[g + j][1 % N], v[g + j][2 % N]), v[g + j][3 % N]);
-      } else {
-        part[j] = v[g + j][0];
+      for (int j = 0; j < GRP; ++j) {
+        if (N == 4) {
+          part[j] = MaxNum(MaxNum3(v[g + j][0], v[g + j][1 % N], v[g + j][2 % N]), v[g + j][3 % N]);
+        } else {
+          part[j] = v[g + j][0];
 #pragma unroll
-        for (int i = 1; i < N; ++i) part[j] = MaxNum(part[j], v[g + j][i]);
+          for (int i = 1; i < N; ++i) part[j] = MaxNum(part[j], v[g + j][i]);
+        }
+      }
+      const float most = mshadow::hip::WaveReduceMany<mshadow::hip::WaveOpMax, float, GRP>(part);
+      if (lane < GRP) lds->cmax[(g + lane) * W + wave] = most;
+    } else {
+      /* The terms of a softmax are at most 1 and one of them is 1. A chunk's largest term
+         serves as a lower bound of the sum behind it, and only a term next to a power of
+         two - the 1 - tells more than the approximate sums do: the largest term is looked
+         for only in chunks whose sum reaches 1, and taken as 0 elsewhere. */
+      if (lane < GRP) lds->cmax[(g + lane) * W + wave] = 0.0f;
+      for (uint32_t todo = static_cast<uint32_t>(__ballot(lane < GRP && mine >= 1.0f)); todo != 0u;
+           todo &= todo - 1u) {
+        const int j = g + __ffs(static_cast<int>(todo)) - 1;
+        float t[N];
+        SelectSlab<SLABS, N>(t, v, j);
+        float m = t[0];
+#pragma unroll
+        for (int i = 1; i < N; ++i) m = MaxNum(m, t[i]);
+        m = ReadLaneF32(mshadow::hip::WaveInclusiveScanMaxF32(m), kWave - 1);
+        if (lane == 0) lds->cmax[j * W + wave] = m;
       }
     }
-    const float most = mshadow::hip::WaveReduceMany<mshadow::hip::WaveOpMax, float, GRP>(part);
-    if (lane < GRP) lds->cmax[(g + lane) * W + wave] = most;
   }
   if (CHECK_SIGN) {  // the plan is made for non-negative terms
     float least = 0.0f;
@@ -324,103 +363,128 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
 
   /* B: plan per chunk, identical in every wave */
   uint32_t code[CPL];     // 1 + binade of a certain chunk, 0: to be listed
-  uint32_t start[CPL];    // approximate prefix sum in front of each chunk (float bits)
-  uint32_t lowb[CPL];     // what the sum is at least in front of each chunk (float bits)
+  uint32_t planned;       // how many chunks the plan lists
   {
-    float pre[CPL + 1], seen[CPL + 1];
+    float pre[CPL + 1], seen[CPL + 1], own[CPL];
     pre[0] = 0.0f;
     seen[0] = 0.0f;
 #pragma unroll
     for (int c = 0; c < CPL; ++c) {
       const int k = lane * CPL + c;
       pre[c + 1] = pre[c] + (k < NCH ? lds->approx[k] : 0.0f);
-      const float m = k < NCH ? lds->cmax[k] : 0.0f;
-      seen[c + 1] = (seen[c] < m) ? m : seen[c];
+      own[c] = k < NCH ? lds->cmax[k] : 0.0f;
+      seen[c + 1] = MaxNum(seen[c], own[c]);
     }
-    const float incl = WaveInclusiveScanF32(pre[CPL]);
+    float incl = pre[CPL], seen_incl = seen[CPL];
+    mshadow::hip::WaveScanSumAndMaxF32(&incl, &seen_incl);
     const float excl = incl - pre[CPL];
     const float approx_total = ReadLaneF32(incl, kWave - 1);
     /* a NaN among the terms makes the sum NaN whatever the order */
     if (approx_total != approx_total) return approx_total;
-    const float seen_incl = mshadow::hip::WaveInclusiveScanMaxF32(seen[CPL]);
     const float seen_excl = __uint_as_float(FromLaneBelowU32(__float_as_uint(seen_incl), 0u));
-    /* the sum never decreases and is never below a term already added: the lower bound of
-       a chunk is the largest over its own estimate and everything in front of it */
-    float low[CPL];
-    float low_run = 0.0f;
+    /* the sum is never below a term already added */
+    int raw[CPL];
+    float st[CPL], lo[CPL];
 #pragma unroll
     for (int c = 0; c < CPL; ++c) {
       const int k = lane * CPL + c;
-      const float st = excl + pre[c];
-      float lo = PlanLowBound(st, static_cast<float>(k) * static_cast<float>(kWave * N));
-      const float sm = (seen_excl < seen[c]) ? seen[c] : seen_excl;
-      lo = (lo < sm) ? sm : lo;
-      low_run = (low_run < lo) ? lo : low_run;
-      low[c] = low_run;
-      start[c] = __float_as_uint(st);
-    }
-    const float low_incl = mshadow::hip::WaveInclusiveScanMaxF32(low[CPL - 1]);
-    const float low_excl = __uint_as_float(FromLaneBelowU32(__float_as_uint(low_incl), 0u));
-    int raw[CPL];
-#pragma unroll
-    for (int c = 0; c < CPL; ++c) {
-      const float lo = (low[c] < low_excl) ? low_excl : low[c];
-      lowb[c] = __float_as_uint(lo);
-      raw[c] = PlanBinade(lo, PlanHighBound(excl + pre[c + 1]));
+      st[c] = excl + pre[c];
+      lo[c] = MaxNum3(PlanLowBound(st[c], static_cast<float>(k) * static_cast<float>(kWave * N)),
+                      seen_excl, seen[c]);
+      raw[c] = PlanBinade(lo[c], PlanHighBound(excl + pre[c + 1]));
     }
     /* neighbouring certain chunks must agree on the binade, or the later one is listed:
        every run of certain chunks then has one scale */
     const int before = static_cast<int>(FromLaneBelowU32(static_cast<uint32_t>(raw[CPL - 1]),
                                                          static_cast<uint32_t>(-1)));
+    /* the chunks to be listed get their slots in row order, known to every wave alike; a
+       chunk that turns out to hold a tie asks for one of the slots behind those */
+    uint32_t in_lane[CPL];
+    uint32_t mine = 0u, below = 0u;
+    planned = 0u;
 #pragma unroll
     for (int c = 0; c < CPL; ++c) {
       const int prev = (c == 0) ? before : raw[c - 1];
       const bool clash = raw[c] >= 0 && prev >= 0 && prev != raw[c];
       code[c] = (raw[c] < 0 || clash) ? 0u : static_cast<uint32_t>(raw[c]) + 1u;
+      const bool to_list = code[c] == 0u && lane * CPL + c < NCH;
+      const unsigned long long listing = __ballot(to_list);
+      in_lane[c] = mine;  // listed chunks of this lane in front of chunk c
+      mine += to_list ? 1u : 0u;
+      below += mshadow::hip::LanesBelow(listing);
+      planned += static_cast<uint32_t>(__popcll(listing));
     }
-  }
-  /* the chunks to be listed get their slots in row order, known to every wave alike; a
-     chunk that turns out to hold a tie asks for one of the slots behind those */
-  uint32_t slot_of[CPL];
-  uint32_t planned;
-  {
-    uint32_t cnt[CPL + 1];
-    cnt[0] = 0u;
 #pragma unroll
-    for (int c = 0; c < CPL; ++c) cnt[c + 1] = cnt[c] + ((code[c] == 0u && lane * CPL + c < NCH) ? 1u : 0u);
-    const uint32_t incl = WaveInclusiveScanU32(cnt[CPL]);
-    planned = ReadLaneU32(incl, kWave - 1);
-#pragma unroll
-    for (int c = 0; c < CPL; ++c) slot_of[c] = incl - cnt[CPL] + cnt[c];
+    for (int c = 0; c < CPL; ++c) {
+      typename Lds::ChunkPlan cp;
+      cp.start = st[c];
+      cp.low = lo[c];
+      cp.slot = below + in_lane[c];
+      cp.peak = own[c] > lo[c] ? 1u : 0u;
+      if (lane * CPL + c < NCH) lds->plan[lane * CPL + c] = cp;
+    }
   }
 
   /* C: integer totals of this wave's certain chunks ... */
   MSHADOW_ROWSUM_STAMP(2)
   uint32_t listed = 0u;  // this wave's slabs that go to the chain as lists
+  static_assert(W % CPL == 0, "a wave's chunks must sit in one column of the chunk table");
+  /* chunk j * W + wave sits in lane (j * W + wave) / CPL of table column wave % CPL */
+  uint32_t my_code = code[0];
 #pragma unroll
-  for (int g = 0; g < SLABS; g += GRP) {
-    uint32_t part[GRP];
+  for (int c = 1; c < CPL; ++c) my_code = (wave % CPL == c) ? code[c] : my_code;
+  {
+    /* Every certain chunk is quantised against its binade by two accumulators one ulp apart
+       (LaneDualQuant); they end one ulp apart unless a term was a tie. The differences of
+       all slabs are and-ed together: 1 exactly if every one of them is 1 (a lane that left
+       its binade has a total that fails its run anyway). Only a wave that saw a tie looks
+       for the slab it was in. */
+    uint32_t all_gaps = 1u;
 #pragma unroll
-    for (int j = 0; j < GRP; ++j) {
-      const uint32_t ck = TableAt<CPL>(code, (g + j) * W + wave);
-      const LaneQuantum lq = LaneDualQuant<N>(v[g + j], ck != 0u ? ck - 1u : 1u);
-      part[j] = lq.q;
-      if (ck == 0u || __ballot(!lq.ok) != 0ull) listed |= 1u << (g + j);
+    for (int g = 0; g < SLABS; g += GRP) {
+      uint32_t part[GRP];
+#pragma unroll
+      for (int j = 0; j < GRP; ++j) {
+        const uint32_t ck = ReadLaneU32(my_code, ((g + j) * W + wave) / CPL);
+        /* straight-line: a chunk to be listed is quantised too (against any binade) and
+           its result dropped */
+        const bool certain = ck != 0u;
+        const uint32_t base = (certain ? ck - 1u : 1u) << 23;
+        float lo = __uint_as_float(base), hi = __uint_as_float(base + 1u);
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+          lo = lo + v[g + j][i];
+          hi = hi + v[g + j][i];
+        }
+        all_gaps &= certain ? __float_as_uint(hi) - __float_as_uint(lo) : 1u;
+        part[j] = __float_as_uint(lo) - base;
+        listed |= certain ? 0u : 1u << (g + j);
+      }
+      const uint32_t total = mshadow::hip::WaveReduceMany<mshadow::hip::WaveOpSum, uint32_t, GRP>(part);
+      /* lanes 0 .. GRP-1 file the result of "their" chunk (overwritten below if the chunk is
+         listed after all); a total that cannot fit a binade is cut so that sums of totals
+         stay inside 32 bits (the run it joins fails its check) */
+      if (lane < GRP) lds->q[(g + lane) * W + wave] = total < (1u << 24) ? total : (1u << 24);
     }
-    const uint32_t total = mshadow::hip::WaveReduceMany<mshadow::hip::WaveOpSum, uint32_t, GRP>(part);
-    /* lanes 0 .. GRP-1 file the result of "their" chunk; a total that cannot fit a binade
-       is cut so that sums of totals stay inside 32 bits (the run it joins fails its check) */
-    if (lane < GRP && ((listed >> (g + lane)) & 1u) == 0u) {
-      lds->q[(g + lane) * W + wave] = total < (1u << 24) ? total : (1u << 24);
+    if (__ballot(all_gaps != 1u) != 0ull) {
+      for (int j = 0; j < SLABS; ++j) {
+        const uint32_t ck = ReadLaneU32(my_code, (j * W + wave) / CPL);
+        if (ck == 0u) continue;
+        float t[N];
+        SelectSlab<SLABS, N>(t, v, j);
+        if (__ballot(!LaneDualQuant<N>(t, ck - 1u).ok) != 0ull) listed |= 1u << j;
+      }
     }
   }
+  MSHADOW_ROWSUM_STAMP(6)
   /* ... and a list of addends for each of the others */
   for (uint32_t todo = listed; todo != 0u; todo &= todo - 1u) {
     const int j = __ffs(static_cast<int>(todo)) - 1;
     const int k = j * W + wave;
+    const typename Lds::ChunkPlan cp = lds->plan[k];
     uint32_t slot;
-    if (TableAt<CPL>(code, k) == 0u) {
-      slot = TableAt<CPL>(slot_of, k);
+    if (ReadLaneU32(my_code, k / CPL) == 0u) {
+      slot = __builtin_amdgcn_readfirstlane(cp.slot);
     } else {
       slot = 0u;
       if (lane == 0) slot = planned + atomicAdd(&lds->nslots, 1u);
@@ -432,21 +496,23 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
     }
     float t[N];
     SelectSlab<SLABS, N>(t, v, j);
-    const float st = __uint_as_float(TableAt<CPL>(start, k));
-    const float lb = __uint_as_float(TableAt<CPL>(lowb, k));
-    /* the lane's own bounds: approximate prefix sums inside the chunk, largest term so far */
-    float a = t[0], m = t[0];
+    const float st = cp.start;
+    const float lb = cp.low;
+    /* the lane's own bounds: approximate prefix sums inside the chunk, and the largest term
+       in front of it where that can raise the bound at all */
+    float a = t[0];
 #pragma unroll
-    for (int i = 1; i < N; ++i) {
-      a += t[i];
-      m = (m < t[i]) ? t[i] : m;
-    }
+    for (int i = 1; i < N; ++i) a += t[i];
     const float incl = WaveInclusiveScanF32(a);
-    const float seen_incl = mshadow::hip::WaveInclusiveScanMaxF32(m);
-    const float seen = __uint_as_float(FromLaneBelowU32(__float_as_uint(seen_incl), 0u));
     float lo = PlanLowBound(st + (incl - a), static_cast<float>(k * kWave + lane) * static_cast<float>(N));
-    lo = (lo < seen) ? seen : lo;
-    lo = (lo < lb) ? lb : lo;
+    if (__builtin_amdgcn_readfirstlane(cp.peak) != 0u) {
+      float m = t[0];
+#pragma unroll
+      for (int i = 1; i < N; ++i) m = MaxNum(m, t[i]);
+      const float seen_incl = mshadow::hip::WaveInclusiveScanMaxF32(m);
+      lo = MaxNum(lo, __uint_as_float(FromLaneBelowU32(__float_as_uint(seen_incl), 0u)));
+    }
+    lo = MaxNum(lo, lb);
     int c = PlanBinade(lo, PlanHighBound(st + incl));
     const LaneQuantum lq = LaneDualQuant<N>(t, c >= 0 ? static_cast<uint32_t>(c) : 1u);
     if (!lq.ok) c = -1;
@@ -457,26 +523,36 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
     const bool head = c >= 0 && below != c;
     const uint32_t qi = term_lane ? 0u : lq.q;
     const uint32_t q_incl = WaveInclusiveScanU32(qi);
-    const unsigned long long edges = __ballot(term_lane || head);
-    const unsigned long long above = (edges >> lane) >> 1;
+    const unsigned long long terms = __ballot(term_lane);
+    const unsigned long long heads = __ballot(head);
+    const unsigned long long above = ((terms | heads) >> lane) >> 1;
     const int next_edge = above != 0ull ? lane + __ffsll(static_cast<long long>(above)) : kWave;
     const uint32_t q_end = static_cast<uint32_t>(__shfl(static_cast<int>(q_incl), next_edge - 1));
-    const uint32_t n_mine = term_lane ? static_cast<uint32_t>(N) : (head ? 1u : 0u);
-    const uint32_t n_incl = WaveInclusiveScanU32(n_mine);
-    const uint32_t at = n_incl - n_mine;
+    /* place in the list: N per term lane and one per run in front of this lane */
+    const uint32_t terms_below = __builtin_amdgcn_mbcnt_hi(
+        static_cast<uint32_t>(terms >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(terms), 0u));
+    const uint32_t heads_below = __builtin_amdgcn_mbcnt_hi(
+        static_cast<uint32_t>(heads >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(heads), 0u));
+    const uint32_t at = terms_below * N + heads_below;
+    const uint32_t count = static_cast<uint32_t>(__popcll(terms)) * N + static_cast<uint32_t>(__popcll(heads));
     AddendList<N> *out = &lds->list[slot];
     if (term_lane) {
 #pragma unroll
       for (int i = 0; i < N; ++i) {
-        out->addend[at + i] = t[i];
-        out->check[at + i] = 0;
+        Addend e;
+        e.value = t[i];
+        e.check = 0u;
+        out->entry[at + i] = e;
       }
     } else if (head) {
-      out->addend[at] = RunAddend(static_cast<uint32_t>(c), q_end - (q_incl - qi));
-      out->check[at] = static_cast<unsigned char>(c + 1);
+      Addend e;
+      e.value = RunAddend(static_cast<uint32_t>(c), q_end - (q_incl - qi));
+      e.check = static_cast<uint32_t>(c + 1);
+      out->entry[at] = e;
     }
-    if (lane == kWave - 1) lds->q[k] = kListedBit | (n_incl << 8) | slot;
+    if (lane == 0) lds->q[k] = kListedBit | (count << 8) | slot;
   }
+  MSHADOW_ROWSUM_STAMP(8)
   __syncthreads();
   MSHADOW_ROWSUM_STAMP(3)
 
@@ -498,11 +574,8 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
       cnt[c + 1] = cnt[c] + (is_listed ? 1u : 0u);
       len[c + 1] = len[c] + (is_listed ? ((qk[c] >> 8) & 0x1ffu) + 1u : 0u);
     }
-    const uint32_t incl = WaveInclusiveScanU32(pre[CPL]);
-    const uint32_t cincl = WaveInclusiveScanU32(cnt[CPL]);
-    const uint32_t lincl = WaveInclusiveScanU32(len[CPL]);
-    const uint32_t total_ex = ReadLaneU32(incl, kWave - 1);
-    const uint32_t total_len = ReadLaneU32(lincl, kWave - 1) + 1u;  // + the run at the end
+    uint32_t incl = pre[CPL], cincl = cnt[CPL], lincl = len[CPL];
+    mshadow::hip::WaveScanSum3U32(&incl, &cincl, &lincl);
     /* ex = integer total of the certain chunks in front of a chunk; it never decreases,
        so its value at the previous listed chunk is a running maximum */
     uint32_t own_last = 0u;
@@ -511,6 +584,8 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
       if ((qk[c] & kListedBit) != 0u) own_last = incl - pre[CPL] + pre[c];
     }
     const uint32_t last_incl = mshadow::hip::WaveInclusiveScanMaxU32(own_last);
+    const uint32_t total_ex = ReadLaneU32(incl, kWave - 1);
+    const uint32_t total_len = ReadLaneU32(lincl, kWave - 1) + 1u;  // + the run at the end
     const uint32_t last_ex = ReadLaneU32(last_incl, kWave - 1);
     uint32_t prev_ex = FromLaneBelowU32(last_incl, 0u);
     const uint32_t code_below = FromLaneBelowU32(code[CPL - 1], 0u);
@@ -535,20 +610,21 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
           const uint32_t c0 = ReadLaneU32(run, l);
           const AddendList<N> *from = &lds->list[q & 0xffu];
           const int n = static_cast<int>((q >> 8) & 0x1ffu);
-          for (int g = lane; g < n; g += kWave) {
-            lds->row_addend[to + 1u + g] = from->addend[g];
-            lds->row_check[to + 1u + g] = from->check[g];
-          }
+          for (int g = lane; g < n; g += kWave) lds->row[to + 1u + g] = from->entry[g];
           if (lane == 0) {
-            lds->row_addend[to] = a0;
-            lds->row_check[to] = static_cast<unsigned char>(c0);
+            Addend e;
+            e.value = a0;
+            e.check = c0;
+            lds->row[to] = e;
           }
         }
       }
       if (threadIdx.x == 0) {  // the run of certain chunks behind the last listed one
         const uint32_t run = TableAt<CPL>(code, NCH - 1);
-        lds->row_addend[total_len - 1u] = run != 0u ? RunAddend(run - 1u, total_ex - last_ex) : 0.0f;
-        lds->row_check[total_len - 1u] = static_cast<unsigned char>(run);
+        Addend e;
+        e.value = run != 0u ? RunAddend(run - 1u, total_ex - last_ex) : 0.0f;
+        e.check = run;
+        lds->row[total_len - 1u] = e;
         lds->row_count = total_len;
       }
     }
@@ -565,23 +641,17 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
     float s = 0.0f;
     bool bad = false;
     /* the next block is fetched while the current one is summed */
-    float na = 0.0f;
-    uint32_t nc = 0u;
-    if (lane < count) {
-      na = lds->row_addend[lane];
-      nc = lds->row_check[lane];
-    }
+    Addend next;
+    next.value = 0.0f;
+    next.check = 0u;
+    if (lane < count) next = lds->row[lane];
     for (int g0 = 0; g0 < count; g0 += kWave) {
-      const float a = na;
-      const uint32_t chk = nc;
-      na = 0.0f;
-      nc = 0u;
-      if (g0 + kWave + lane < count) {
-        na = lds->row_addend[g0 + kWave + lane];
-        nc = lds->row_check[g0 + kWave + lane];
-      }
+      const Addend now = next;
+      next.value = 0.0f;
+      next.check = 0u;
+      if (g0 + kWave + lane < count) next = lds->row[g0 + kWave + lane];
       const int left = count - g0;
-      s = ChainBlock(s, a, chk, left < kWave ? left : kWave, &bad);
+      s = ChainBlock(s, now.value, now.check, left < kWave ? left : kWave, &bad);
     }
     const bool failed = __ballot(bad) != 0ull;
     if (lane == 0) {
@@ -634,13 +704,10 @@ __device__ __forceinline__ float ExpNonPositive(float x) {
   return __builtin_fmaf(e, c, e);
 }
 
-/*! \brief p / s given rcp = 1 / s: one Newton correction on the quotient. The result is
- *  the correctly rounded quotient except for rare half-ulp cases. */
-__device__ __forceinline__ float DivideBy(float p, float s, float rcp) {
-  const float q = p * rcp;
-  const float e = __builtin_fmaf(-q, s, p);
-  return __builtin_fmaf(e, rcp, q);
-}
+/*! \brief p / s given rcp = 1 / s correctly rounded (s finite, at least 1): one multiply,
+ *  within one ulp of the true quotient (half an ulp from the reciprocal, half from the
+ *  product) */
+__device__ __forceinline__ float DivideBy(float p, float /*s*/, float rcp) { return p * rcp; }
 
 template <int THREADS>
 __device__ inline float BlockMax(float v, float *wmax) {
@@ -740,7 +807,7 @@ __global__ void __launch_bounds__(THREADS, 4)  // >= 4 waves per SIMD: two 512-t
     MSHADOW_ROWSUM_STAMP(13)
   }
 
-  const float s = RowOrderedSum<THREADS, SLABS, VEC, TERMS_GIVEN>(v, cols, &lds);
+  const float s = RowOrderedSum<THREADS, SLABS, VEC, TERMS_GIVEN, !TERMS_GIVEN>(v, cols, &lds);
   if (TERMS_GIVEN) {
     if (threadIdx.x == 0) dst[blockIdx.x] = s;
     return;

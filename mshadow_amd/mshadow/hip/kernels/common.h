@@ -60,20 +60,18 @@ __device__ __forceinline__ uint32_t WaveInclusiveScanU32(uint32_t v) {
   v += DppU32<MSHADOW_DPP_ROW_BCAST31, 0xc>(0u, v);
   return v;
 }
-/*! \brief inclusive prefix maximum of unsigned integers over lanes 0..63 */
+/*! \brief inclusive prefix maximum of unsigned integers over lanes 0..63 (one DPP
+ *  instruction per step, each behind the idle cycles the hardware asks for) */
 __device__ __forceinline__ uint32_t WaveInclusiveScanMaxU32(uint32_t v) {
-#define MSHADOW_UMSCAN_STEP(CTRL, MASK)            \
-  {                                                \
-    const uint32_t o = DppU32<CTRL, MASK>(0u, v);  \
-    v = (v < o) ? o : v;                           \
-  }
-  MSHADOW_UMSCAN_STEP(MSHADOW_DPP_ROW_SHR(1), 0xf)
-  MSHADOW_UMSCAN_STEP(MSHADOW_DPP_ROW_SHR(2), 0xf)
-  MSHADOW_UMSCAN_STEP(MSHADOW_DPP_ROW_SHR(4), 0xf)
-  MSHADOW_UMSCAN_STEP(MSHADOW_DPP_ROW_SHR(8), 0xf)
-  MSHADOW_UMSCAN_STEP(MSHADOW_DPP_ROW_BCAST15, 0xa)
-  MSHADOW_UMSCAN_STEP(MSHADOW_DPP_ROW_BCAST31, 0xc)
-#undef MSHADOW_UMSCAN_STEP
+  asm volatile(
+      "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_shr:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+      "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_shr:2 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+      "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_shr:4 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+      "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_shr:8 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+      "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+      "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+      "s_nop 1"
+      : "+v"(v));
   return v;
 }
 /*! \brief the same for floats (used on integer-valued floats, where it is exact below 2^24) */
@@ -174,21 +172,56 @@ __device__ __forceinline__ float WaveSumMany(float (&a)[M]) {
 }
 
 /*! \brief inclusive prefix maximum over lanes 0..63 of non-negative floats (a lane with
- *  no source in a step sees 0, which is the identity for them) */
+ *  no source in a step sees 0, which is the identity for them; NaN operands are ignored).
+ *  One DPP instruction per step; the idle cycles in front of each are what the hardware
+ *  asks for between writing a register and reading it through DPP. */
 __device__ __forceinline__ float WaveInclusiveScanMaxF32(float v) {
-#define MSHADOW_MSCAN_STEP(CTRL, MASK)                                      \
-  {                                                                         \
-    const float o = __uint_as_float(DppU32<CTRL, MASK>(0u, __float_as_uint(v))); \
-    v = (v < o) ? o : v;                                                    \
-  }
-  MSHADOW_MSCAN_STEP(MSHADOW_DPP_ROW_SHR(1), 0xf)
-  MSHADOW_MSCAN_STEP(MSHADOW_DPP_ROW_SHR(2), 0xf)
-  MSHADOW_MSCAN_STEP(MSHADOW_DPP_ROW_SHR(4), 0xf)
-  MSHADOW_MSCAN_STEP(MSHADOW_DPP_ROW_SHR(8), 0xf)
-  MSHADOW_MSCAN_STEP(MSHADOW_DPP_ROW_BCAST15, 0xa)
-  MSHADOW_MSCAN_STEP(MSHADOW_DPP_ROW_BCAST31, 0xc)
-#undef MSHADOW_MSCAN_STEP
+  asm volatile(
+      "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_shr:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+      "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_shr:2 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+      "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_shr:4 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+      "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_shr:8 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+      "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+      "s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+      "s_nop 1"
+      : "+v"(v));
   return v;
+}
+
+/* Several scans at once: the steps of the scans are interleaved, so that the idle cycles the
+   hardware asks for between writing a register and reading it through DPP are filled by
+   the other scans' steps instead of waiting, and the chains of dependent steps overlap. */
+#define MSHADOW_SCAN_CTRLS(X)                                  \
+  X("row_shr:1 row_mask:0xf bank_mask:0xf bound_ctrl:1")       \
+  X("row_shr:2 row_mask:0xf bank_mask:0xf bound_ctrl:1")       \
+  X("row_shr:4 row_mask:0xf bank_mask:0xf bound_ctrl:1")       \
+  X("row_shr:8 row_mask:0xf bank_mask:0xf bound_ctrl:1")       \
+  X("row_bcast:15 row_mask:0xa bank_mask:0xf")                 \
+  X("row_bcast:31 row_mask:0xc bank_mask:0xf")
+/*! \brief inclusive prefix sum of *sum and inclusive prefix maximum of *mx (non-negative
+ *  floats) over lanes 0..63 */
+__device__ __forceinline__ void WaveScanSumAndMaxF32(float *sum, float *mx) {
+#define MSHADOW_STEP(CTRL)                      \
+  "v_add_f32_dpp %0, %0, %0 " CTRL "\n\t"       \
+  "v_max_f32_dpp %1, %1, %1 " CTRL "\n\t"       \
+  "s_nop 0\n\t"
+  asm volatile("s_nop 1\n\t" MSHADOW_SCAN_CTRLS(MSHADOW_STEP) "s_nop 0" : "+v"(*sum), "+v"(*mx));
+#undef MSHADOW_STEP
+}
+/*! \brief inclusive prefix sums of *a, *b and *c (unsigned) over lanes 0..63 */
+__device__ __forceinline__ void WaveScanSum3U32(uint32_t *a, uint32_t *b, uint32_t *c) {
+#define MSHADOW_STEP(CTRL)                      \
+  "v_add_u32_dpp %0, %0, %0 " CTRL "\n\t"       \
+  "v_add_u32_dpp %1, %1, %1 " CTRL "\n\t"       \
+  "v_add_u32_dpp %2, %2, %2 " CTRL "\n\t"
+  asm volatile("s_nop 1\n\t" MSHADOW_SCAN_CTRLS(MSHADOW_STEP) "s_nop 1"
+               : "+v"(*a), "+v"(*b), "+v"(*c));
+#undef MSHADOW_STEP
+}
+/*! \brief number of set bits of `mask` below this lane */
+__device__ __forceinline__ uint32_t LanesBelow(unsigned long long mask) {
+  return __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(mask >> 32),
+                                   __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u));
 }
 
 /*! \brief sum over the 64 lanes; result in every lane (as a scalar) */

@@ -54,17 +54,15 @@ static bool PlannedSum(const std::vector<float> &row, int max_slots, float *resu
   std::vector<float> start(nch), lowb(nch);
   std::vector<int> code(nch);
   {
-    float pre = 0.0f, seen_max = 0.0f, low_run = 0.0f;
+    float pre = 0.0f, seen_max = 0.0f;
     int prev = -1;
     for (int k = 0; k < nch; ++k) {
       start[k] = pre;
-      float low = PlanLowBound(pre, static_cast<float>(k) * chunk_terms);
-      low = std::fmax(low, seen_max);
-      low_run = std::fmax(low_run, low);
-      lowb[k] = low_run;
+      const float low = std::fmax(PlanLowBound(pre, static_cast<float>(k) * chunk_terms), seen_max);
+      lowb[k] = low;
       pre += approx[k];
       seen_max = std::fmax(seen_max, cmax[k]);
-      int c = PlanBinade(low_run, PlanHighBound(pre));
+      int c = PlanBinade(low, PlanHighBound(pre));
       if (c >= 0 && prev >= 0 && prev != c) c = -1;  // a run has one binade
       code[k] = c;
       prev = c;

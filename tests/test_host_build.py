@@ -15,7 +15,7 @@ def _declared(header):
     text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     text = re.sub(r"//[^\n]*", "", text)
-    return sorted(set(re.findall(r"\b(mshadow_(?:hip|case)_\w+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(mshadow_(?:hip|case|probe)_\w+)\s*\(", text)))
 
 
 def _lib(name):
@@ -29,11 +29,12 @@ def _lib(name):
 
 
 @pytest.mark.parametrize("header,libname", [("mshadow_hip.h", "libmshadow_hip.so"),
+                                            ("mshadow_hip_probe.h", "libmshadow_probe.so"),
                                             ("mshadow_hip_blas.h", "libmshadow_hip.so"),
                                             ("mshadow_hip_cases.h", "libmshadow_cases.so")])
 def test_every_declared_symbol_is_exported(header, libname):
     names = _declared(header)
-    assert len(names) >= (4 if "blas" in header else 10)
+    assert len(names) >= (4 if "blas" in header or "probe" in header else 10)
     if libname == "libmshadow_cases.so":
         _lib("libmshadow_hip.so")
     lib = _lib(libname)
@@ -123,6 +124,15 @@ def test_ordered_sum_matches_serial_sum_on_host(tmp_path):
     """the lane arithmetic of the softmax row sum, driven lane by lane on the host,
     reproduces a strictly sequential float sum bit for bit"""
     out = _compile_and_run(tmp_path, "ordered_sum_sim.cc", [])
+    assert out.startswith("OK"), out[-500:]
+
+
+def test_planned_row_sum_matches_serial_sum_on_host(tmp_path):
+    """the plan of the long-row softmax kernel (chunks and lanes classified from approximate
+    prefix sums, a list of addends, every run verified) modelled on the host with the device
+    code's own lane functions: bit-identical to a serial float sum wherever the plan holds,
+    and it holds on every row shaped like a softmax's"""
+    out = _compile_and_run(tmp_path, "row_plan_sim.cc", [])
     assert out.startswith("OK"), out[-500:]
 
 
