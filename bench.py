@@ -101,16 +101,40 @@ EXTRA_OPS = ("calib_copy", "smooth_softmax_grad_ignore", "softmax3d", "softmax3d
              "sumall_except_dim1_f16")
 OPS = [k for k in algorithmic_bytes() if k not in EXTRA_OPS]
 
-# HBM bytes per launch of each operation's kernel, measured with rocprofv3 --pmc FETCH_SIZE and
-# --pmc WRITE_SIZE (two runs of `bench.py --only <all ops>,calib_copy`), each counter scaled by
-# what it reads for the calibration copy of known size (FETCH_SIZE x 1.9981, WRITE_SIZE x 0.9993);
-# the counter table is kept under profiles/. bench.py cannot run the profiler on itself, so
-# `roofline.traffic` quotes this table.
-MEASURED_HBM_BYTES = {
-    "map_fused": 335408137, "sumall_except_dim1": 205348938, "sum_rows": 272288862,
-    "softmax": 2096030462, "softmax_grad": 2095964771, "pool_max": 518051515,
-    "unpool_max": 1068693813, "im2col_f16": 513762151, "col2im_f16": 543883139,
+# HBM bytes per launch of each operation's kernel come from the committed counter summary
+# (two `rocprofv3 --pmc` runs of this script, FETCH_SIZE then WRITE_SIZE, each counter scaled by
+# what it reads for the calibration copy of known size; the command is in the file). bench.py
+# cannot run the profiler on itself, so `roofline.traffic` is read from that file at run time.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "hotpath_step_all_kernels_hbm_traffic.md")
+TRAFFIC_ROW_OF_OP = {
+    "map_fused": "map_fused", "sumall_except_dim1": "ReduceKeepHighDimDmaKernel",
+    "sum_rows": "ReduceKeepLowestDmaKernel", "softmax": "SoftmaxRowKernel",
+    "softmax_grad": "SoftmaxGradKernel", "pool_max": "PoolKernel", "unpool_max": "UnpoolBlockKernel",
+    "im2col_f16": "Im2ColHalfRow3Kernel", "col2im_f16": "Col2ImHalfPairKernel",
 }
+
+
+def measured_hbm_bytes(op):
+    """bytes one launch of `op`'s kernel moved to and from HBM according to the counter summary
+    under profiles/ (columns "HBM read MiB" and "HBM written MiB"), or None"""
+    row = TRAFFIC_ROW_OF_OP.get(op)
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            lines = [l for l in f if l.startswith("|")]
+    except OSError:
+        return None
+    if row is None or not lines:
+        return None
+    head = [c.strip() for c in lines[0].strip().strip("|").split("|")]
+    try:
+        rd, wr = head.index("HBM read MiB"), head.index("HBM written MiB")
+    except ValueError:
+        return None
+    for l in lines[2:]:
+        cells = [c.strip() for c in l.strip().strip("|").split("|")]
+        if cells and cells[0] == row:
+            return int(round((float(cells[rd]) + float(cells[wr])) * (1 << 20)))
+    return None
 
 
 def make_inputs(scale=1):
@@ -131,11 +155,17 @@ def make_inputs(scale=1):
     return d
 
 
-def half_inputs(orc, scale=1):
+def to_half_bits(a):
+    """binary16 bit patterns of a float32 array, rounded to nearest even (numpy.float16 rounds
+    exactly as half_t's conversion does)"""
+    return np.ascontiguousarray(a, dtype=f32).astype(np.float16).view(np.uint16)
+
+
+def half_inputs(scale=1):
     s = scale
-    img = orc.float2half(np.random.default_rng(11).uniform(-1, 1, (32 // s, 256, 56, 56)).astype(f32))
+    img = to_half_bits(np.random.default_rng(11).uniform(-1, 1, (32 // s, 256, 56, 56)).astype(f32))
     colshape = (2304, (32 // s) * 56 * 56)
-    col = orc.float2half(np.random.default_rng(12).standard_normal(colshape, dtype=f32))
+    col = to_half_bits(np.random.default_rng(12).standard_normal(colshape, dtype=f32))
     return img, col
 
 
@@ -155,7 +185,6 @@ def main():
                  "full shape on one MI355X and nothing is sharded (--gpus must be 1)")
 
     import mshadow_amd
-    from checkers import Checker, have_ref
     G = mshadow_amd.load_cases()
     if G.device_count() < 1:
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
@@ -163,12 +192,11 @@ def main():
     if args.only in ("softmax_phases", "ceiling_chain"):
         return run_probe(G, args.only)
     props = G.props(0)
-    orc = Checker("orc")
     only = [o for o in args.only.split(",") if o] or OPS
 
     t0 = time.time()
     H = make_inputs(args.scale)
-    img_h, col_h = half_inputs(orc, args.scale)
+    img_h, col_h = half_inputs(args.scale)
     gen_s = time.time() - t0
 
     s = G.stream_create()
@@ -211,13 +239,13 @@ def main():
         extra["bias"] = G.to_device(np.random.default_rng(14).standard_normal(51380224, dtype=f32)[:256].copy())
 
     if any(o.endswith("_f16") and o not in OPS for o in only):
-        extra["hL"] = G.to_device(orc.float2half(H["L"]))
+        extra["hL"] = G.to_device(to_half_bits(H["L"]))
         extra["hP"] = G.buffer(H["L"].shape, np.uint16)
         extra["hG"] = G.buffer(H["L"].shape, np.uint16)
         # labels a half can hold exactly (integers up to 2048)
-        extra["hlab"] = G.to_device(orc.float2half(np.minimum(H["labels"], f32(2048))))
-        extra["hM"] = G.to_device(orc.float2half(H["M2b"]))
-        extra["hX"] = G.to_device(orc.float2half(H["X2a"]))
+        extra["hlab"] = G.to_device(to_half_bits(np.minimum(H["labels"], f32(2048))))
+        extra["hM"] = G.to_device(to_half_bits(H["M2b"]))
+        extra["hX"] = G.to_device(to_half_bits(H["X2a"]))
         extra["h2b"] = G.buffer((4096,), np.uint16)
         extra["h2a"] = G.buffer((256,), np.uint16)
         G.case_softmax(extra["hP"], extra["hL"], s)
@@ -341,8 +369,7 @@ def main():
 
     cpu = None
     if not args.no_cpu:
-        cpu = cpu_baseline(orc, have_ref, Checker, H, img_h, col_h, only, abytes, scale_fix,
-                           args.cpu_reps)
+        cpu = cpu_baseline(H, img_h, col_h, only, abytes, scale_fix, args.cpu_reps)
         for row in per_op:
             c = cpu["per_op_ms"].get(row["op"])
             if c:
@@ -364,7 +391,8 @@ def main():
                    "arch": props.arch.decode(), "compute_units": props.compute_units},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(dom_gbs, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_HBM_BYTES.get(dominant) if args.scale == 1 else None},
+                     "traffic": measured_hbm_bytes(dominant) if args.scale == 1 else None,
+                     "traffic_source": os.path.relpath(TRAFFIC_PROFILE, ROOT)},
         "per_op": per_op,
         "input_generation_s": round(gen_s, 1),
     }
@@ -415,12 +443,14 @@ def run_probe(G, which):
     print(json.dumps(out))
 
 
-def cpu_baseline(orc, have_ref, Checker, H, img_h, col_h, only, abytes, scale_fix, reps):
+def cpu_baseline(H, img_h, col_h, only, abytes, scale_fix, reps):
     """The same nine operations on the host: the reference's own headers where the
     reference-built library is present ("reference"), the C restatement otherwise
-    ("port"). One warm-up pass, then `reps` timed passes over the full inputs."""
+    ("port"). One warm-up pass, then `reps` timed passes over the full inputs. The only part
+    of this script that loads anything from oracle/."""
+    from checkers import Checker, have_ref
     kind = "reference" if have_ref() else "port"
-    cpu = Checker("ref") if kind == "reference" else orc
+    cpu = Checker("ref" if kind == "reference" else "orc")
     o_map = np.empty_like(H["A"])
     o_2a, o_2b = np.empty(256, f32), np.empty(4096, f32)
     o_p, o_g = np.empty_like(H["L"]), np.empty_like(H["L"])

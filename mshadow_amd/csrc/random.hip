@@ -10,7 +10,7 @@
  * curandGenerateNormal). The values are those of Philox, not of cuRAND's XORWOW: no two
  * generator families agree, and the reference's CPU path (std::mt19937) does not agree
  * with its own GPU path either.
- *   uniform  u = ((x >> 8) + 0.5) * 2^-24, strictly inside (0, 1), then u * (b - a) + a
+ *   uniform  u = ((x >> 9) + 0.5) * 2^-23, strictly inside (0, 1), then u * (b - a) + a
  *   normal   Box-Muller on two uniforms: sqrt(-2 ln u1) * (cos, sin)(2 pi u2), then
  *            mu + z * sigma
  */
@@ -55,8 +55,11 @@ __device__ __forceinline__ Philox4 Philox4x32_10(uint64_t seed, uint64_t subsequ
   return out;
 }
 
+/*! \brief the top 23 bits of a word as a point strictly inside (0, 1): (n + 1/2) / 2^23 with
+ *  n < 2^23, which is exact in float32 (2n + 1 has 24 bits), so the smallest value is 2^-24
+ *  and the largest 1 - 2^-24; one bit more and n + 1/2 would round, up to 1 for the largest n */
 __device__ __forceinline__ float UnitOpen(uint32_t x) {
-  return (static_cast<float>(x >> 8) + 0.5f) * 5.9604644775390625e-08f;  // 2^-24
+  return (static_cast<float>(x >> 9) + 0.5f) * 1.1920928955078125e-07f;  // 2^-23
 }
 
 enum { kWords = 0, kUniform = 1, kNormal = 2 };
@@ -83,7 +86,7 @@ __global__ void __launch_bounds__(kRandomBlock)
     } else {
 #pragma unroll
       for (int k = 0; k < 4; k += 2) {
-        /* Box-Muller on the hardware's own functions: the arguments lie in [2^-25, 1), so
+        /* Box-Muller on the hardware's own functions: the arguments lie in [2^-24, 1), so
            none of the range handling of the library versions is needed. log2 -> ln by a
            factor; sine and cosine take their argument in revolutions */
         const float u = UnitOpen(r.w[k]), turn = UnitOpen(r.w[k + 1]);

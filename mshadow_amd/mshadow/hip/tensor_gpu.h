@@ -656,6 +656,8 @@ struct MapLauncher<Saver, DType, DPlan, SPlan, true> {
     const int N = 16 / sizeof(DType);
     uint32_t rows = shape[0], cols = shape[1];
     if (rows == 0 || cols == 0) return;
+    /* pack counts, flat offsets and the multiply-high divisions of the kernels are 32-bit */
+    CHECK_LT(static_cast<uint64_t>(rows) * cols, 1ull << 31) << "MapExp<gpu>: too many elements";
     bool flat = true;
     const bool aligned = cols % N == 0 && dplan.PackReady(N, cols, &flat) &&
                          splan.PackReady(N, cols, &flat);

@@ -337,6 +337,47 @@ int main() {
     ms.pos = 0;
     TensorContainer<cpu, 3> wrong(Shape3(2, 3, 4));
     EXPECT(Throws([&] { LoadBinary(ms, &wrong, true); }));
+    // the container's own members: the same record, and LoadBinary takes the stored shape
+    decltype(ms) cs;
+    t.SaveBinary(cs);
+    EXPECT(cs.bytes == ms.bytes);
+    TensorContainer<cpu, 3> other(Shape3(1, 1, 2), 7.0f);
+    other.LoadBinary(cs);
+    same = other.shape_ == t.shape_;
+    for (index_t i = 0; i < 2; ++i) for (index_t j = 0; j < 3; ++j) for (index_t k = 0; k < 5; ++k)
+      same = same && other[i][j][k] == t[i][j][k];
+    EXPECT(same);
+    TensorContainer<cpu, 3> dense(false);   // into an empty, unpadded container
+    cs.pos = 0;
+    dense.LoadBinary(cs);
+    EXPECT(dense.shape_ == t.shape_ && dense.stride_ == 5 && dense[1][2][4] == 124.0f);
+  }
+  // ---- TensorContainer: the view moves inside the block, a larger shape takes a new block
+  {
+    TensorContainer<cpu, 2> c(Shape2(8, 10), 1.0f);
+    float *block = c.dptr_;
+    const index_t pitch = c.stride_;
+    EXPECT(pitch >= 10);
+    c.Resize(Shape2(3, 7));                       // fits: same memory, padded pitch kept
+    EXPECT(c.dptr_ == block && c.stride_ == pitch && c.size(0) == 3 && c.size(1) == 7);
+    c.Resize(Shape2(8, 10));
+    EXPECT(c.dptr_ == block);
+    c.Resize(Shape2(9, 10), 4.0f);                // one row too many: a new block, filled
+    EXPECT(c.size(0) == 9 && c[8][9] == 4.0f);
+    TensorContainer<cpu, 2> d(false);
+    EXPECT(d.dptr_ == NULL && d.shape_[0] == 0);
+    d.Resize(Shape2(4, 6), 2.0f);
+    EXPECT(d.stride_ == 6);
+    d.Resize(Shape2(4, 3));                       // dense rows follow the shape
+    EXPECT(d.stride_ == 3);
+    TensorContainer<cpu, 2> e(c);                 // copies the elements
+    EXPECT(e.dptr_ != c.dptr_ && e[8][9] == 4.0f);
+    e = 5.0f;
+    d = e;                                        // takes shape, padding choice and elements
+    EXPECT(d.shape_ == e.shape_ && d[0][0] == 5.0f && c[0][0] == 4.0f);
+    d.Release();
+    EXPECT(d.dptr_ == NULL && d.shape_[0] == 0);
+    d.Release();
   }
   // ---- SortByKey / VectorizedSort on the CPU device against the oracle
   {

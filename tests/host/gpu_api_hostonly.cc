@@ -79,6 +79,21 @@ int main() {
   for (index_t y = 0; y < ct2.size(0); ++y)
     for (index_t x2 = 0; x2 < ct2.size(1); ++x2) bad_transpose += ct2[y][x2] != again2[y][x2];
   FreeSpace(&t2);
+  /* the members of a device container: the same record; LoadBinary takes the stored shape */
+  {
+    decltype(ms) cs;
+    TensorContainer<gpu, 4> dev(t.shape_), dev2(Shape4(1, 1, 1, 2));
+    dev.set_stream(s), dev2.set_stream(s);
+    Copy(dev, t, s);
+    dev.SaveBinary(cs);
+    bad_transpose += cs.bytes != ms.bytes;
+    dev2.LoadBinary(cs);
+    bad_transpose += !(dev2.shape_ == t.shape_);
+    Copy(gt_again, dev2, s);
+    s->Wait();
+    for (index_t y = 0; y < ct2.size(0); ++y)
+      for (index_t x2 = 0; x2 < ct2.size(1); ++x2) bad_transpose += ct2[y][x2] != again2[y][x2];
+  }
   /* matrix products are library calls behind the ABI: (3x5 of i+j) x (4x5 of i-j)^T, and the
      scalar product of two of the rows, in small integers (exact in float) */
   int bad_dot = 0;

@@ -56,7 +56,21 @@ def model_words(seed, subsequence, counter, n):
 
 
 def unit_open(words):
-    return ((words >> 8).astype(f32) + f32(0.5)) * f32(2.0 ** -24)
+    return ((words >> 9).astype(f32) + f32(0.5)) * f32(2.0 ** -23)
+
+
+def test_unit_interval_transform_stays_strictly_inside():
+    """the word -> (0, 1) transform of Random<gpu>: every word, the extreme ones included, lands
+    strictly between 0 and 1 (with 24 bits instead of 23 the largest word would round to 1)"""
+    w = np.array([0, 1, 0x1FF, 0x200, 0x7FFFFFFF, 0x80000000, 0xFFFFFDFF, 0xFFFFFE00, 0xFFFFFFFF], np.uint32)
+    u = unit_open(w)
+    assert u.dtype == f32 and u.min() == f32(2.0 ** -24) and u.max() == f32(1.0) - f32(2.0 ** -24)
+    assert np.all(u > 0) and np.all(u < 1)
+    # exact: (2n + 1) / 2^24 in float64 equals the float32 result for every n at the ends
+    n = (w >> 9).astype(np.float64)
+    assert np.array_equal(u.astype(np.float64), (2 * n + 1) / 2.0 ** 24)
+    old = ((w >> 8).astype(f32) + f32(0.5)) * f32(2.0 ** -24)
+    assert old.max() == f32(1.0)        # what this replaces
 
 
 # ---------------------------------------------------------------- CPU
