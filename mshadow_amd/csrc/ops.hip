@@ -160,6 +160,25 @@ int Col2Im(T *img, int istride, const T *col, int cstride, const PatchGeom &g, v
     return Fail(MSHADOW_HIP_ERR_ARGUMENT, "col2im: pitch smaller than the row");
   }
   const int EPT = 16 / sizeof(T);
+  /* the convolution-backward case on rows of whole aligned packs: nine shifted streams */
+  if (sizeof(T) == 2 && g.ky == 3 && g.kx == 3 && g.sy == 1 && g.sx == 1 && g.dy == 1 && g.dx == 1 &&
+      g.pad_y == 1 && g.pad_x == 1 && g.w % 8 == 0 && g.w <= 512 && istride % 8 == 0 &&
+      cstride % 8 == 0 && Aligned16(img) && Aligned16(col) && total < (1ll << 31) &&
+      static_cast<long long>(g.c) * 9 * cstride < (1ll << 40)) {
+    RowsGeom rg;
+    rg.total_rows = static_cast<uint32_t>(static_cast<long long>(g.n) * g.c * g.h);
+    rg.groups = static_cast<uint32_t>(g.w / 8);
+    rg.rows_per_wave = 64u / rg.groups;
+    rg.div_groups = mshadow::FastDivU32(rg.groups);
+    rg.div_h = mshadow::FastDivU32(static_cast<uint32_t>(g.h));
+    rg.div_c = mshadow::FastDivU32(static_cast<uint32_t>(g.c));
+    const uint32_t waves = (rg.total_rows + rg.rows_per_wave - 1) / rg.rows_per_wave;
+    const uint32_t blocks = (waves + kPatchBlock / 64 - 1) / (kPatchBlock / 64);
+    hipLaunchKernelGGL(Col2ImHalfRows3x3Kernel, dim3(blocks), dim3(kPatchBlock), 0, AsStream(stream),
+                       reinterpret_cast<uint16_t *>(img), istride,
+                       reinterpret_cast<const uint16_t *>(col), cstride, g, rg);
+    return AfterLaunch("col2im");
+  }
   /* tiled: per tap, the patch rows a band of image rows touches; all taps must fit */
   const long long taps = static_cast<long long>(g.ky) * g.kx;
   const size_t prow_bytes = static_cast<size_t>(taps) * g.ow * sizeof(T);
@@ -721,6 +740,27 @@ int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstrid
               "too large for 32-bit indices");
   PoolGeom g = {h, w, ph, pw, ky, kx, sy, sx, 0, 0, pw};
   hipStream_t s = AsStream(stream);
+  /* 3 x 3 windows with stride 2 on rows of whole aligned packs: no staging */
+  if (ky == 3 && kx == 3 && sy == 2 && sx == 2 && h % 2 == 0 && w % 4 == 0 && w <= 256 && ph >= 1 &&
+      pw >= 1 && dstride % 4 == 0 && sstride % 4 == 0 && Aligned16(dst) && Aligned16(src)) {
+    UnpoolRowsGeom rg;
+    rg.half_h = static_cast<uint32_t>(h / 2);
+    rg.total_rows = static_cast<uint32_t>(planes) * rg.half_h;
+    rg.groups = static_cast<uint32_t>(w / 4);
+    rg.rows_per_wave = 64u / rg.groups;
+    rg.div_groups = mshadow::FastDivU32(rg.groups);
+    rg.div_half_h = mshadow::FastDivU32(rg.half_h);
+    const uint32_t waves = (rg.total_rows + rg.rows_per_wave - 1) / rg.rows_per_wave;
+    const uint32_t blocks = (waves + kPoolBlock / 64 - 1) / (kPoolBlock / 64);
+#define UNPOOL_ROWS(R)                                                                         \
+  hipLaunchKernelGGL((UnpoolRows3x3s2Kernel<R>), dim3(blocks), dim3(kPoolBlock), 0, s, dst, dstride, \
+                     src, sstride, pooled, pstride, grad, gstride, g, rg)
+    if (reducer == MSHADOW_HIP_SUM) UNPOOL_ROWS(MSHADOW_HIP_SUM);
+    else if (reducer == MSHADOW_HIP_MAX) UNPOOL_ROWS(MSHADOW_HIP_MAX);
+    else UNPOOL_ROWS(MSHADOW_HIP_MIN);
+#undef UNPOOL_ROWS
+    return AfterLaunch("unpool");
+  }
   const size_t row_bytes = static_cast<size_t>(g.lds_pitch) * sizeof(float) * 2;  // pooled + grad
   /* source rows per band: prow_max = (band + ky - 2) / sy + 2 pooled rows must fit */
   long long max_prow = static_cast<long long>(kUnpoolLdsBudget / row_bytes);

@@ -410,6 +410,115 @@ __global__ void __launch_bounds__(kPatchBlock)
   }
 }
 
+/*! \brief geometry of Col2ImHalfRows3x3Kernel: rows of all image planes are numbered
+ *  plane * h + y; a wave takes `rows_per_wave` consecutive ones, `groups` lanes per row
+ *  (numbered channel by channel instead, all images of a channel together, the kernel took
+ *  98 us instead of 91) */
+struct RowsGeom {
+  uint32_t total_rows;     //!< n * c * h
+  uint32_t groups;         //!< w / 8
+  uint32_t rows_per_wave;  //!< 64 / groups
+  mshadow::FastDivU32 div_groups, div_h, div_c;
+};
+
+/*! \brief col2im for binary16, a 3 x 3 window, stride 1, dilation 1 and one pixel of padding
+ *  (so the patch grid has the image's own height and width), w a multiple of 8, rows of
+ *  whole aligned packs - the convolution-backward case - with no staging at all.
+ *
+ *  Every element of the column matrix belongs to exactly one pixel, and for a fixed tap
+ *  (a, b) the matrix row IS an image-shaped array, shifted by (1 - a, 1 - b): the result is
+ *  the sum of nine shifted streams. A thread owns 8 adjacent pixels of one image row and
+ *  fetches, for each tap, the aligned pack of the tap's stream at its own place; the streams
+ *  shifted by one pixel (b = 0, 2) are completed with the one missing element from the
+ *  neighbouring lane, which holds the next / previous pack of the same stream (a wave takes
+ *  whole rows, so the neighbour is always in the wave). Nothing is staged, no barrier: every
+ *  wave is loads -> adds -> one store, and the loads of a wave are whole contiguous aligned
+ *  runs of each stream.
+ *
+ *  The terms are added in the reference's order (py ascending = a descending, then px
+ *  ascending = b descending, mshadow/extension/pack_col2patch.h:118-144) as packed binary16
+ *  pairs: a binary16 add rounds after every term exactly as half_t's operator+= does. */
+__global__ void __launch_bounds__(kPatchBlock)
+    Col2ImHalfRows3x3Kernel(uint16_t *img, int istride, const uint16_t *col, int cstride, PatchGeom g,
+                            RowsGeom rg) {
+  typedef _Float16 H2 __attribute__((ext_vector_type(2)));
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = blockIdx.x * (kPatchBlock / 64) + (threadIdx.x >> 6);
+  const uint32_t row_in_wave = rg.div_groups.Div(lane);
+  const uint32_t group = lane - row_in_wave * rg.groups;
+  const uint32_t row = wave * rg.rows_per_wave + row_in_wave;
+  const bool live = row_in_wave < rg.rows_per_wave && row < rg.total_rows;
+  /* lanes that own no pixels follow a neighbour's addresses: they only ever hand their
+     (unused) pack to lanes that mask it */
+  const uint32_t rowc = live ? row : rg.total_rows - 1u;
+  const uint32_t plane = rg.div_h.Div(rowc);
+  const int y = static_cast<int>(rowc - plane * g.h);
+  const uint32_t n = rg.div_c.Div(plane);
+  const uint32_t ch = plane - n * g.c;
+  const int x0 = static_cast<int>(group * 8u);
+  /* the stream of tap (a, b) at this thread's place: row py = y + 1 - a of the patch grid */
+  const uint16_t *tap0 = col + static_cast<size_t>(ch) * 9u * cstride +
+                         (static_cast<size_t>(n) * g.h) * g.w + x0;
+  U4 q[9];
+#pragma unroll
+  for (int a = 0; a < 3; ++a) {
+    const int py = min(max(y + 1 - a, 0), g.h - 1);  // clamped; an absent row is skipped below
+#pragma unroll
+    for (int b = 0; b < 3; ++b) {
+      q[a * 3 + b] = StreamLoad16(tap0 + static_cast<size_t>(a * 3 + b) * cstride +
+                                  static_cast<size_t>(py) * g.w);
+    }
+  }
+  /* the pixel left of the row (b = 2 at x = 0) and right of it (b = 0 at x = w - 1) do not exist */
+  const uint32_t keep_first = group == 0u ? 0xffff0000u : 0xffffffffu;
+  const uint32_t keep_last = group + 1u == rg.groups ? 0x0000ffffu : 0xffffffffu;
+  uint32_t res[4] = {0u, 0u, 0u, 0u};  // eight binary16 zeros
+#define MSHADOW_COL2IM_ADD(d, term, keep)                         \
+  {                                                               \
+    H2 acc_, term_;                                               \
+    const uint32_t t_ = (term);                                   \
+    __builtin_memcpy(&acc_, &res[d], 4);                          \
+    __builtin_memcpy(&term_, &t_, 4);                             \
+    const H2 sum_ = acc_ + term_;                                 \
+    uint32_t s_;                                                  \
+    __builtin_memcpy(&s_, &sum_, 4);                              \
+    res[d] = ((keep) == 0xffffffffu) ? s_ : ((s_ & (keep)) | (res[d] & ~(keep))); \
+  }
+#pragma unroll
+  for (int a = 2; a >= 0; --a) {
+    const int py = y + 1 - a;
+    /* the neighbours' packs are fetched by every lane (DPP needs the whole wave) */
+    const U4 c2 = q[a * 3 + 2], c1 = q[a * 3 + 1], c0 = q[a * 3 + 0];
+    const uint32_t prev_last = static_cast<uint32_t>(
+        __builtin_amdgcn_update_dpp(0, static_cast<int>(c2.w), 0x138, 0xf, 0xf, false));  // wave_shr:1
+    const uint32_t next_first = static_cast<uint32_t>(
+        __builtin_amdgcn_update_dpp(0, static_cast<int>(c0.x), 0x130, 0xf, 0xf, false));  // wave_shl:1
+    if (py >= 0 && py < g.h) {
+      /* b = 2: pixels x - 1 */
+      MSHADOW_COL2IM_ADD(0, __builtin_amdgcn_alignbit(c2.x, prev_last, 16), keep_first)
+      MSHADOW_COL2IM_ADD(1, __builtin_amdgcn_alignbit(c2.y, c2.x, 16), 0xffffffffu)
+      MSHADOW_COL2IM_ADD(2, __builtin_amdgcn_alignbit(c2.z, c2.y, 16), 0xffffffffu)
+      MSHADOW_COL2IM_ADD(3, __builtin_amdgcn_alignbit(c2.w, c2.z, 16), 0xffffffffu)
+      /* b = 1: the pixels themselves */
+      MSHADOW_COL2IM_ADD(0, c1.x, 0xffffffffu)
+      MSHADOW_COL2IM_ADD(1, c1.y, 0xffffffffu)
+      MSHADOW_COL2IM_ADD(2, c1.z, 0xffffffffu)
+      MSHADOW_COL2IM_ADD(3, c1.w, 0xffffffffu)
+      /* b = 0: pixels x + 1 */
+      MSHADOW_COL2IM_ADD(0, __builtin_amdgcn_alignbit(c0.y, c0.x, 16), 0xffffffffu)
+      MSHADOW_COL2IM_ADD(1, __builtin_amdgcn_alignbit(c0.z, c0.y, 16), 0xffffffffu)
+      MSHADOW_COL2IM_ADD(2, __builtin_amdgcn_alignbit(c0.w, c0.z, 16), 0xffffffffu)
+      MSHADOW_COL2IM_ADD(3, __builtin_amdgcn_alignbit(next_first, c0.w, 16), keep_last)
+    }
+  }
+#undef MSHADOW_COL2IM_ADD
+  if (live) {
+    U4 out;
+    out.x = res[0], out.y = res[1], out.z = res[2], out.w = res[3];
+    StreamStore16(img + static_cast<size_t>(row) * istride + x0, out);
+  }
+}
+
 /*! \brief EPT consecutive column-matrix elements per thread; grid.x = rows of the column
  *  matrix (c, a, b) times `chunks` pieces of kPatchBlock * EPT columns each. */
 template <typename T, int EPT>

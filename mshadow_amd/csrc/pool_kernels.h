@@ -372,6 +372,97 @@ __global__ void __launch_bounds__(kPoolBlock)
   }
 }
 
+/*! \brief geometry of UnpoolRows3x3s2Kernel: the pairs of source rows (2a, 2a + 1) of all
+ *  planes are numbered plane * (h / 2) + a; a wave takes `rows_per_wave` consecutive ones,
+ *  `groups` = w / 4 lanes each */
+struct UnpoolRowsGeom {
+  uint32_t total_rows, groups, rows_per_wave, half_h;
+  mshadow::FastDivU32 div_groups, div_half_h;
+};
+
+/*! \brief unpool for a 3 x 3 window with stride 2 on rows of whole aligned packs (h even,
+ *  w a multiple of 4), with no staging: a thread owns two adjacent 2 x 2 blocks of source
+ *  pixels - four pixels of row 2a and the four below them. The windows that can cover them
+ *  are rows a - 1 and a of the pooled grid, columns 2t - 1, 2t, 2t + 1: the thread fetches
+ *  columns 2t and 2t + 1 of both rows (pooled value and gradient) and takes column 2t - 1
+ *  from the neighbouring lane, which fetched it as its own 2t' + 1 (a wave takes whole rows).
+ *  Source and result move as 128-bit accesses; nothing is staged and there is no barrier.
+ *  Terms in the reference's order (py, then px ascending; mshadow/extension/
+ *  spatial_unpool.h:102-125), a multiply and an add each. */
+template <int REDUCER>
+__global__ void __launch_bounds__(kPoolBlock)
+    UnpoolRows3x3s2Kernel(float *dst, int dstride, const float *src, int sstride, const float *pooled,
+                          int pstride, const float *grad, int gstride, PoolGeom g, UnpoolRowsGeom rg) {
+  typedef PoolOp<REDUCER> Op;
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = blockIdx.x * (kPoolBlock / 64) + (threadIdx.x >> 6);
+  const uint32_t row_in_wave = rg.div_groups.Div(lane);
+  const uint32_t t = lane - row_in_wave * rg.groups;
+  const uint32_t brow = wave * rg.rows_per_wave + row_in_wave;
+  const bool live = row_in_wave < rg.rows_per_wave && brow < rg.total_rows;
+  const uint32_t browc = live ? brow : rg.total_rows - 1u;
+  const uint32_t plane = rg.div_half_h.Div(browc);
+  const int a = static_cast<int>(browc - plane * rg.half_h);
+  const float *in = src + (static_cast<size_t>(plane) * g.h + 2 * a) * sstride + 4u * t;
+  const F4 top = StreamLoadF4(in), bottom = StreamLoadF4(in + sstride);
+  /* [jy][c]: pooled row a - jy, column 2t - 1 + c */
+  float pv[2][3], gv[2][3];
+  bool ok[2][3];
+#pragma unroll
+  for (int jy = 0; jy < 2; ++jy) {
+    const int py = a - jy;
+    const bool row_ok = py >= 0 && py < g.ph;
+    const size_t prow = static_cast<size_t>(plane) * g.ph + (row_ok ? py : 0);
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int px = static_cast<int>(2u * t) + e;
+      const bool col_ok = px < g.pw;
+      /* a window that does not exist re-reads an existing one and is skipped below */
+      const int pxc = col_ok ? px : 0;
+      pv[jy][e + 1] = pooled[prow * pstride + pxc];
+      gv[jy][e + 1] = grad[prow * gstride + pxc];
+      ok[jy][e + 1] = row_ok && col_ok;
+    }
+    /* column 2t - 1 is the neighbour's 2t' + 1 (every lane takes part in the exchange) */
+    pv[jy][0] = __uint_as_float(static_cast<uint32_t>(__builtin_amdgcn_update_dpp(
+        0, static_cast<int>(__float_as_uint(pv[jy][2])), 0x138, 0xf, 0xf, false)));
+    gv[jy][0] = __uint_as_float(static_cast<uint32_t>(__builtin_amdgcn_update_dpp(
+        0, static_cast<int>(__float_as_uint(gv[jy][2])), 0x138, 0xf, 0xf, false)));
+    ok[jy][0] = row_ok && t > 0u && static_cast<int>(2u * t) - 1 < g.pw;
+  }
+  if (!live) return;
+  const float vtop[4] = {top.x, top.y, top.z, top.w};
+  const float vbot[4] = {bottom.x, bottom.y, bottom.z, bottom.w};
+  float otop[4], obot[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    /* pixel 4t + i lies in block 2t + i / 2 at dx = i % 2: windows at columns c0 .. c1 */
+    const int c1 = 1 + i / 2;
+    const int c0 = (i % 2 == 0) ? c1 - 1 : c1;
+    float vt = 0.0f, vb = 0.0f;
+#pragma unroll
+    for (int jy = 1; jy >= 0; --jy) {  // py ascending; the row below (dy = 1) is covered by py = a only
+#pragma unroll
+      for (int c = c0; c <= c1; ++c) {  // px ascending
+        const float tt = vt + Op::Grad(vtop[i], pv[jy][c]) * gv[jy][c];
+        vt = ok[jy][c] ? tt : vt;
+        if (jy == 0) {
+          const float tb = vb + Op::Grad(vbot[i], pv[jy][c]) * gv[jy][c];
+          vb = ok[jy][c] ? tb : vb;
+        }
+      }
+    }
+    otop[i] = vt;
+    obot[i] = vb;
+  }
+  float *out = dst + (static_cast<size_t>(plane) * g.h + 2 * a) * dstride + 4u * t;
+  F4 q;
+  q.x = otop[0], q.y = otop[1], q.z = otop[2], q.w = otop[3];
+  StreamStoreF4(out, q);
+  q.x = obot[0], q.y = obot[1], q.z = obot[2], q.w = obot[3];
+  StreamStoreF4(out + dstride, q);
+}
+
 /*! \brief unpool without staging */
 template <int REDUCER>
 __global__ void __launch_bounds__(kPoolBlock)
