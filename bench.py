@@ -178,7 +178,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-reps", type=int, default=3)
     ap.add_argument("--only", default="", help="comma list of ops to run (profiling aid); "
-                    "softmax_phases and ceiling_chain run the probes of libmshadow_probe.so instead")
+                    "softmax_phases, ceiling_chain and ceiling_lds_loads run the probes of "
+                    "libmshadow_probe.so instead")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; every operation of the path runs at its "
@@ -189,7 +190,7 @@ def main():
     if G.device_count() < 1:
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
     G.set_device(0)
-    if args.only in ("softmax_phases", "ceiling_chain"):
+    if args.only in ("softmax_phases", "ceiling_chain", "ceiling_lds_loads"):
         return run_probe(G, args.only)
     props = G.props(0)
     only = [o for o in args.only.split(",") if o] or OPS
@@ -200,17 +201,24 @@ def main():
     gen_s = time.time() - t0
 
     s = G.stream_create()
-    dev = {k: G.to_device(v) for k, v in H.items()}
-    dimg, dcol_in = G.to_device(img_h), G.to_device(col_h)
-    out_map = G.buffer(H["A"].shape, f32)
-    out_2a = G.buffer((256,), f32)
-    out_2b = G.buffer((4096,), f32)
-    out_p = G.buffer(H["L"].shape, f32)
-    out_g = G.buffer(H["L"].shape, f32)
-    out_pool = G.buffer(H["G4"].shape, f32)
-    out_unpool = G.buffer(H["X4"].shape, f32)
-    out_col = G.buffer(col_h.shape, np.uint16)
-    out_img = G.buffer(img_h.shape, np.uint16)
+    def buffer_set():
+        """inputs on the device and outputs of their own: one complete set of operands"""
+        b = {"dev": {k: G.to_device(v) for k, v in H.items()},
+             "dimg": G.to_device(img_h), "dcol_in": G.to_device(col_h),
+             "out_map": G.buffer(H["A"].shape, f32), "out_2a": G.buffer((256,), f32),
+             "out_2b": G.buffer((4096,), f32), "out_p": G.buffer(H["L"].shape, f32),
+             "out_g": G.buffer(H["L"].shape, f32), "out_pool": G.buffer(H["G4"].shape, f32),
+             "out_unpool": G.buffer(H["X4"].shape, f32), "out_col": G.buffer(col_h.shape, np.uint16),
+             "out_img": G.buffer(img_h.shape, np.uint16)}
+        # softmax_grad / unpool consume the outputs of softmax / pool: make them valid first
+        G.softmax(b["out_p"], b["dev"]["L"], s)
+        G.pool(b["out_pool"], b["dev"]["X4"], 3, 3, 2, 2, stream=s)
+        return b
+
+    sets = [buffer_set()]
+    cur = dict(sets[0])     # the set run_op works on
+    dev = cur["dev"]
+    out_map, out_g, out_p = cur["out_map"], cur["out_g"], cur["out_p"]
 
     extra = {}
     if any(o in EXTRA_OPS[1:] for o in only):
@@ -301,31 +309,28 @@ def main():
         elif name == "add_take_grad":
             G.add_take_grad(extra["emb"], extra["idx"], extra["rows"], s)
         elif name == "map_fused":
-            G.case_map_fused(out_map, dev["A"], dev["B"], dev["C"], dev["D"], 0, s)
+            G.case_map_fused(cur["out_map"], cur["dev"]["A"], cur["dev"]["B"], cur["dev"]["C"], cur["dev"]["D"], 0, s)
         elif name == "sumall_except_dim1":
-            G.reduce_keep_highdim(out_2a, dev["X2a"], stream=s)
+            G.reduce_keep_highdim(cur["out_2a"], cur["dev"]["X2a"], stream=s)
         elif name == "sum_rows":
-            G.reduce_keep_lowest(out_2b, dev["M2b"], stream=s)
+            G.reduce_keep_lowest(cur["out_2b"], cur["dev"]["M2b"], stream=s)
         elif name == "softmax":
-            G.softmax(out_p, dev["L"], s)
+            G.softmax(cur["out_p"], cur["dev"]["L"], s)
         elif name == "softmax_grad":
-            G.softmax_grad(out_g, out_p, dev["labels"], s)
+            G.softmax_grad(cur["out_g"], cur["out_p"], cur["dev"]["labels"], s)
         elif name == "pool_max":
-            G.pool(out_pool, dev["X4"], 3, 3, 2, 2, stream=s)
+            G.pool(cur["out_pool"], cur["dev"]["X4"], 3, 3, 2, 2, stream=s)
         elif name == "unpool_max":
-            G.unpool(out_unpool, dev["X4"], out_pool, dev["G4"], 3, 3, 2, 2, stream=s)
+            G.unpool(cur["out_unpool"], cur["dev"]["X4"], cur["out_pool"], cur["dev"]["G4"], 3, 3, 2, 2, stream=s)
         elif name == "im2col_f16":
-            G.im2col(out_col, dimg, 3, 3, 1, 1, 1, 1, 1, 1, s)
+            G.im2col(cur["out_col"], cur["dimg"], 3, 3, 1, 1, 1, 1, 1, 1, s)
         elif name == "col2im_f16":
-            G.col2im(out_img, dcol_in, 3, 3, 1, 1, 1, 1, 1, 1, s)
+            G.col2im(cur["out_img"], cur["dcol_in"], 3, 3, 1, 1, 1, 1, 1, 1, s)
         elif name == "calib_copy":
             # one read and one write of 4096x4096 floats: the known-size kernel that the
             # HBM traffic counters are scaled by (only with --only, never part of a step)
             G.case_map_axpb(out_map, dev["A"], 0.0, 1.0, 0.0, 0, s)
 
-    # softmax_grad / unpool consume the outputs of softmax / pool: make them valid first
-    G.softmax(out_p, dev["L"], s)
-    G.pool(out_pool, dev["X4"], 3, 3, 2, 2, stream=s)
     for _ in range(args.warmup):
         for name in only:
             run_op(name)
@@ -345,6 +350,30 @@ def main():
     G.device_sync()
     wall = time.perf_counter() - wall0
 
+    # A second figure per operation: the same launch repeated back to back, so that no gap
+    # between launches is inside the interval, over three complete sets of operands in turn
+    # (3 x 205 MB and more: nothing is found in the 256 MB memory-side cache from the
+    # launch before). "ms" above is the operation's interval inside the step, gap included.
+    b2b_ms = {}
+    if args.scale == 1 and all(o in OPS for o in only):
+        while len(sets) < 3:
+            sets.append(buffer_set())
+        G.stream_sync(s)
+        reps = 12
+        for name in only:
+            ev = [G.event_create(), G.event_create()]
+            for r in range(3):
+                cur.update(sets[r])
+                run_op(name)
+            G.event_record(ev[0], s)
+            for r in range(reps):
+                cur.update(sets[r % 3])
+                run_op(name)
+            G.event_record(ev[1], s)
+            G.stream_sync(s)
+            b2b_ms[name] = G.elapsed_ms(ev[0], ev[1]) / reps
+        cur.update(sets[0])
+
     abytes = algorithmic_bytes()
     elems = work_elements()
     scale_fix = 1.0 / args.scale
@@ -357,6 +386,10 @@ def main():
         per_op.append({"op": name, "ms": round(float(ms.mean()), 4), "ms_min": round(float(ms.min()), 4),
                        "GBps": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
                        "GElemps": round(elems[name] * scale_fix / (ms.mean() * 1e-3) / 1e9, 2)})
+        if name in b2b_ms:
+            per_op[-1]["ms_back_to_back"] = round(b2b_ms[name], 4)
+            per_op[-1]["frac_of_hbm_peak_back_to_back"] = round(
+                abytes[name] / (b2b_ms[name] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
         if name in PRODUCT_FLOPS:
             flops, peak = PRODUCT_FLOPS[name]
             per_op[-1]["TFLOPps"] = round(flops / (ms.mean() * 1e-3) / 1e12, 1)
@@ -406,7 +439,10 @@ def run_probe(G, which):
     stamps taken inside an instrumented build of the library's kernel). `--only ceiling_chain`:
     the cost of one dependent float add for a single wave, alone on the chip and with every CU
     busy - the floor of any kernel that must add in the reference's order, sum_rows first of
-    all (16384 dependent adds per column). Prints one JSON line."""
+    all (16384 dependent adds per column). `--only ceiling_lds_loads`: how fast the loads from
+    global memory straight into LDS, which feed the reduction kernels, run with nothing
+    consuming the data - per access pattern, bytes per lane and waves per workgroup.
+    Prints one JSON line."""
     import mshadow_amd
     P = mshadow_amd.load_probe()
     s = G.stream_create()
@@ -419,6 +455,20 @@ def run_probe(G, which):
                                   for wg in (1, cus, 4 * cus)}
         lds = out["modes"]["lds"]
         out["sum_rows_floor_us"] = {k: round(16384 * v * 1e-3, 1) for k, v in lds.items()}
+    elif which == "ceiling_lds_loads":
+        src = G.to_device(np.ones((16384, 4096), f32))
+        mb = 16384 * 4096 * 4 / 1e6
+        out = {"probe": "ceiling_lds_loads", "matrix": [16384, 4096], "unit": "us to read the matrix once "
+               "(GB/s)", "patterns": {}}
+        names = {0: "contiguous pieces, 1024 workgroups",
+                 -1: "64 segments side by side per workgroup, 256 workgroups"}
+        names.update({c: f"{c} columns of every row per workgroup" for c in (16, 32, 64)})
+        for strip in (0, -1, 16, 32, 64):
+            for width in (4, 16):
+                for waves in (4, 8, 16) if width == 4 else (2, 4, 8):
+                    us = min(P.dma_rate_us(src, strip, width, waves, s) for _ in range(3))
+                    out["patterns"][f"{names[strip]}; {width} bytes per lane; {waves} waves"] = \
+                        [round(us, 1), round(mb / us * 1e3)]
     else:
         L = np.random.default_rng(7).standard_normal((8192, 32000), dtype=f32) * f32(3)
         src, dst = G.to_device(L), G.buffer(L.shape, f32)

@@ -51,6 +51,20 @@ int mshadow_probe_softmax_phases(float *dst, int dstride, const float *src, int 
 int mshadow_probe_row_copy(float *dst, int dstride, const float *src, int sstride, int rows,
                            int cols, int barriers, int spin, double *kernel_us, void *stream);
 
+/* Rate of loads from global memory straight into LDS (the loads of the reduction kernels),
+   with nothing consuming the data: `waves` waves per workgroup keep 32..48 loads of `width`
+   bytes per lane (4 or 16) outstanding each. strip = 0: the matrix is read as one buffer,
+   1024 workgroups take a contiguous piece each and an instruction fetches 64 * width
+   consecutive bytes; strip = 16, 32 or 64: a workgroup reads that many columns of every
+   row, as a reduction over the rows does, cols / strip workgroups, neighbouring strips
+   behind the same L2; strip = -1: the matrix is read as 64 x 256 segments, 256 workgroups
+   take 64 segments each (every 256th) and read them side by side, one instruction's worth
+   (64 * width bytes) of each in turn, as a reduction that keeps the second of four
+   dimensions does. kernel_us = duration of the
+   launch that reads rows x cols floats once. */
+int mshadow_probe_dma_rate(const float *src, int sstride, int rows, int cols, int strip, int width,
+                           int waves, double *kernel_us, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -133,6 +133,77 @@ __global__ void __launch_bounds__(THREADS, 4)
   }
 }
 
+
+/* Rate of loads from global memory straight into LDS, nothing else: `blockDim.x / 64` waves
+   per workgroup issue them in batches of 16 and keep up to 48 outstanding. WIDTH bytes per
+   lane (4 or 16). STRIP == 0: a workgroup reads a contiguous piece of the buffer, an
+   instruction 64 * WIDTH consecutive bytes. STRIP > 0: the buffer is a matrix of `rows` x
+   `cols` floats, a workgroup reads STRIP columns of every row (what a reduction over the
+   rows does), an instruction as many rows as its 64 lanes cover. STRIP == -1: the buffer
+   is 64 x gridDim.x segments of equal length, workgroup c reads segments c, c + gridDim.x,
+   ... side by side, one instruction's worth of each in turn (what a reduction that keeps
+   the second of four dimensions does). */
+template <int WIDTH, int STRIP>
+__global__ void __launch_bounds__(1024) DmaRateKernel(const float *src, uint32_t stride, uint32_t rows,
+                                                      uint32_t cols) {
+  const int kRegion = 16 * 64 * WIDTH;   // bytes of LDS a wave cycles through
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t nwave = blockDim.x >> 6;
+  const uint32_t lane = threadIdx.x & 63;
+  unsigned char *mine = lds + wave * kRegion;
+  const int kFloats = WIDTH / 4;
+  uint32_t ninstr;
+  const float *base;
+  size_t step;   // floats between this wave's consecutive instructions
+  if (STRIP == 0) {
+    const size_t total = static_cast<size_t>(rows) * stride;
+    const size_t piece = total / gridDim.x / (64 * kFloats) * (64 * kFloats);
+    ninstr = static_cast<uint32_t>(piece / (64 * kFloats)) / nwave;
+    base = src + piece * blockIdx.x + (static_cast<size_t>(wave) * 64 + lane) * kFloats;
+    step = static_cast<size_t>(nwave) * 64 * kFloats;
+  } else if (STRIP == -1) {
+    ninstr = 0;
+    base = src;
+    step = 0;
+  } else {
+    const int kLanesPerRow = STRIP / kFloats;
+    const int kRowsPerInstr = 64 / kLanesPerRow;
+    ninstr = rows / kRowsPerInstr / nwave;
+    base = src + static_cast<size_t>(wave * kRowsPerInstr + lane / kLanesPerRow) * stride +
+           mshadow::hip::StripOfBlock(blockIdx.x, gridDim.x) * STRIP + (lane % kLanesPerRow) * kFloats;
+    step = static_cast<size_t>(nwave) * kRowsPerInstr * stride;
+  }
+  uint32_t seg_len = 0;
+  if (STRIP == -1) {
+    seg_len = static_cast<uint32_t>(static_cast<size_t>(rows) * stride / 64 / gridDim.x);
+    ninstr = 64 * (seg_len / (64 * kFloats)) / nwave;
+    base = src + static_cast<size_t>(blockIdx.x) * seg_len + lane * kFloats;
+  }
+  (void)cols;
+  for (uint32_t i = 0; i + 16 <= ninstr; i += 16) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      size_t at = (i + q) * step;
+      if (STRIP == -1) {
+        const uint32_t t = (i + q) * nwave + wave;
+        at = static_cast<size_t>(t % 64) * gridDim.x * seg_len + static_cast<size_t>(t / 64) * 64 * kFloats;
+      }
+      const __attribute__((address_space(1))) void *from =
+          (const __attribute__((address_space(1))) void *)(base + at);
+      __attribute__((address_space(3))) void *to =
+          (__attribute__((address_space(3))) void *)(mine + q * 64 * WIDTH);
+      if (WIDTH == 4) {
+        __builtin_amdgcn_global_load_lds(from, to, 4, 0, 2);
+      } else {
+        __builtin_amdgcn_global_load_lds(from, to, 16, 0, 2);
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 int TimeKernel(hipStream_t s, float *ms, const std::function<void()> &launch) {
   hipEvent_t a, b;
   ABI_HIP(hipEventCreate(&a));
@@ -257,6 +328,48 @@ int mshadow_probe_softmax_phases(float *dst, int dstride, const float *src, int 
   for (int i = 0; i < kStampSlots; ++i) mean_us[i] = cnt[i] ? sum[i] / cnt[i] / 100.0 : -1.0;
   mean_us[order[0]] = 0.0;
   *resident_us = resident / rows / 100.0;
+  return MSHADOW_HIP_OK;
+}
+
+int mshadow_probe_dma_rate(const float *src, int sstride, int rows, int cols, int strip, int width,
+                           int waves, double *kernel_us, void *stream) {
+  ABI_REQUIRE(src != NULL && kernel_us != NULL && rows >= 1024 && cols >= 64 && sstride >= cols,
+              "a matrix of at least 1024 x 64");
+  ABI_REQUIRE(waves >= 1 && waves <= 16, "1..16 waves");
+  ABI_REQUIRE((width == 4 || width == 16) &&
+                  (strip == -1 || strip == 0 || strip == 16 || strip == 32 || strip == 64),
+              "width 4 or 16 bytes, strip -1, 0, 16, 32 or 64");
+  ABI_REQUIRE(cols % 64 == 0 && sstride % 4 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0,
+              "rows of whole strips, 16-byte aligned");
+  hipStream_t s = AsStream(stream);
+  const unsigned grid = strip == 0 ? 1024u : strip == -1 ? 256u : static_cast<unsigned>(cols / strip);
+  const size_t lds = static_cast<size_t>(waves) * 16 * 64 * width;
+  ABI_REQUIRE(lds <= 160 * 1024, "too many waves for the LDS");
+  float ms = 0.0f;
+  int st;
+#define PROBE_DMA(W, S)                                                                       \
+  {                                                                                           \
+    ABI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&DmaRateKernel<W, S>),         \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));     \
+    st = TimeKernel(s, &ms, [&] {                                                             \
+      hipLaunchKernelGGL((DmaRateKernel<W, S>), dim3(grid), dim3(waves * 64), lds, s, src,    \
+                         static_cast<uint32_t>(sstride), static_cast<uint32_t>(rows),         \
+                         static_cast<uint32_t>(cols));                                        \
+    });                                                                                       \
+  }
+  if (width == 4 && strip == -1) PROBE_DMA(4, -1)
+  else if (width == 16 && strip == -1) PROBE_DMA(16, -1)
+  else if (width == 4 && strip == 0) PROBE_DMA(4, 0)
+  else if (width == 16 && strip == 0) PROBE_DMA(16, 0)
+  else if (width == 4 && strip == 16) PROBE_DMA(4, 16)
+  else if (width == 16 && strip == 16) PROBE_DMA(16, 16)
+  else if (width == 4 && strip == 32) PROBE_DMA(4, 32)
+  else if (width == 16 && strip == 32) PROBE_DMA(16, 32)
+  else if (width == 4 && strip == 64) PROBE_DMA(4, 64)
+  else PROBE_DMA(16, 64)
+#undef PROBE_DMA
+  if (st != MSHADOW_HIP_OK) return st;
+  *kernel_us = ms * 1e3;
   return MSHADOW_HIP_OK;
 }
 
