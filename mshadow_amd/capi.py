@@ -115,6 +115,9 @@ CASES_SYMBOLS = {
     "mshadow_case_grad_family_f32": ([_p, _i, _p, _i, _p, _i, _i, _i, _i, _i, _f, _f, _p], _i),
     "mshadow_case_softmax3d_f32": ([_p, _i, _p, _i, _i, _i, _i, _p], _i),
     "mshadow_case_rows_by_index_f32": ([_i, _p, _i, _i, _p, _p, _i, _p, _i, _i, _i, _p], _i),
+    "mshadow_case_grad_family_any": ([_i, _p, _i, _p, _i, _p, _i, _i, _i, _i, _i, C.c_double, _f, _p], _i),
+    "mshadow_case_softmax3d_any": ([_i, _p, _i, _p, _i, _i, _i, _i, _p], _i),
+    "mshadow_case_rows_by_index_any": ([_i, _i, _i, _p, _i, _i, _p, _p, _i, _p, _i, _i, _i, _p], _i),
     "mshadow_case_shaping_f32": ([_i, _p, _p, _p, _i, _i, _i, _i, _p], _i),
     "mshadow_case_random_f32": ([_i, _i, _p, _i, _f, _f, _p], _i),
     "mshadow_case_sort_by_key_32": ([_i, _p, _i, _p, _i, _i, _p], _i),
@@ -437,6 +440,31 @@ class Library:
         self.check_case(self.cases.mshadow_case_rows_by_index_f32(
             op, dst.ptr, dst.stride, dst.rows, sorted_rows.ptr if sorted_rows is not None else None,
             index.ptr, index.cols, src.ptr, src.stride, src.rows, src.cols, stream))
+
+    # mshadow::TypeFlag codes of the element types the cases take (binary16 travels as float16)
+    TYPE_FLAG = {"float32": 0, "float64": 1, "float16": 2, "int32": 4, "int64": 6}
+
+    def case_grad_family_any(self, dst, src, label, flags, ignore_label=0.0, alpha=0.0, stream=None):
+        """the four gradients on float / double / half_t tensors (2-D or 3-D by src's shape)"""
+        if len(src.shape) == 2:
+            d0, a, b = 0, src.rows, src.cols
+        else:
+            d0, a, b = src.shape
+        self.check_case(self.cases.mshadow_case_grad_family_any(
+            self.TYPE_FLAG[src.dtype.name], dst.ptr, dst.stride, src.ptr, src.stride, label.ptr,
+            label.stride, d0, a, b, flags, ignore_label, alpha, stream))
+
+    def case_softmax3d_any(self, dst, src, stream=None):
+        d0, d1, d2 = src.shape
+        self.check_case(self.cases.mshadow_case_softmax3d_any(
+            self.TYPE_FLAG[src.dtype.name], dst.ptr, dst.stride, src.ptr, src.stride, d0, d1, d2, stream))
+
+    def case_rows_by_index_any(self, op, dst, sorted_rows, index, src, stream=None):
+        """op 0 AddTakeGrad, 1 AddTakeGradLargeBatch, 2 IndexFill for any table / index type"""
+        self.check_case(self.cases.mshadow_case_rows_by_index_any(
+            op, self.TYPE_FLAG[dst.dtype.name], self.TYPE_FLAG[index.dtype.name], dst.ptr, dst.stride,
+            dst.rows, sorted_rows.ptr if sorted_rows is not None else None, index.ptr, index.cols,
+            src.ptr, src.stride, src.rows, src.cols, stream))
 
     def case_shaping(self, op, out, a, v, n, c, h, w, stream=None):
         self.check_case(self.cases.mshadow_case_shaping_f32(op, out.ptr, a.ptr, v.ptr, n, c, h, w,

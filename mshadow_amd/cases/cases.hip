@@ -80,6 +80,73 @@ typedef half::half_t HalfT;
 inline const HalfT *H(const uint16_t *p) { return reinterpret_cast<const HalfT *>(p); }
 inline HalfT *H(uint16_t *p) { return reinterpret_cast<HalfT *>(p); }
 
+/* the gradient family and the row scatter functions for one element type (see the entry
+   points mshadow_case_grad_family_any / mshadow_case_rows_by_index_any) */
+template <typename DType>
+void GradFamilyOf(void *dst, int dstride, const void *src, int sstride, const void *label,
+                  int lstride, int d0, int rows_or_d1, int cols_or_d2, int flags,
+                  double ignore_label, float alpha, Stream<gpu> *st) {
+  const DType *s = static_cast<const DType *>(src), *l = static_cast<const DType *>(label);
+  DType *d = static_cast<DType *>(dst);
+  const DType ignore = DType(static_cast<float>(ignore_label));
+  if (d0 == 0) {
+    const int rows = rows_or_d1, cols = cols_or_d2;
+    Tensor<gpu, 2, DType> D = G2(d, rows, cols, dstride, st), S = G2(s, rows, cols, sstride, st);
+    Tensor<gpu, 1, DType> L = G1(l, rows, st);
+    switch (flags) {
+      case 0: SoftmaxGrad(D, S, L); break;
+      case 1: SmoothSoftmaxGrad(D, S, L, alpha); break;
+      case 2: SoftmaxGrad(D, S, L, ignore); break;
+      default: SmoothSoftmaxGrad(D, S, L, ignore, alpha); break;
+    }
+  } else {
+    const int d1 = rows_or_d1, d2 = cols_or_d2;
+    Tensor<gpu, 3, DType> D = G3(d, d0, d1, d2, dstride, st), S = G3(s, d0, d1, d2, sstride, st);
+    Tensor<gpu, 2, DType> L = G2(l, d0, d2, lstride, st);
+    switch (flags) {
+      case 0: SoftmaxGrad(D, S, L); break;
+      case 1: SmoothSoftmaxGrad(D, S, L, alpha); break;
+      case 2: SoftmaxGrad(D, S, L, ignore); break;
+      default: SmoothSoftmaxGrad(D, S, L, ignore, alpha); break;
+    }
+  }
+}
+template <typename IndexType, typename DType>
+void RowsByIndexOf(int op, void *dst, int dstride, int k_rows, const void *sorted, const void *index,
+                   int n_index, const void *src, int sstride, int src_rows, int cols,
+                   Stream<gpu> *st) {
+  Tensor<gpu, 2, DType> D = G2(static_cast<const DType *>(dst), k_rows, cols, dstride, st);
+  Tensor<gpu, 2, DType> S = G2(static_cast<const DType *>(src), src_rows, cols, sstride, st);
+  Tensor<gpu, 1, IndexType> I = G1(static_cast<const IndexType *>(index), n_index, st);
+  if (op == 0) {
+    AddTakeGrad(D, I, S);
+  } else if (op == 1) {
+    AddTakeGradLargeBatch(D, G1(static_cast<const IndexType *>(sorted), n_index, st), I, S);
+  } else {
+    IndexFill(D, I, S);
+  }
+}
+template <typename DType>
+void RowsByIndexOfIndex(int index_flag, int op, void *dst, int dstride, int k_rows, const void *sorted,
+                        const void *index, int n_index, const void *src, int sstride, int src_rows,
+                        int cols, Stream<gpu> *st) {
+  switch (index_flag) {
+    case kFloat32:
+      RowsByIndexOf<float, DType>(op, dst, dstride, k_rows, sorted, index, n_index, src, sstride, src_rows, cols, st);
+      break;
+    case kFloat16:
+      RowsByIndexOf<HalfT, DType>(op, dst, dstride, k_rows, sorted, index, n_index, src, sstride, src_rows, cols, st);
+      break;
+    case kInt32:
+      RowsByIndexOf<int, DType>(op, dst, dstride, k_rows, sorted, index, n_index, src, sstride, src_rows, cols, st);
+      break;
+    case kInt64:
+      RowsByIndexOf<int64_t, DType>(op, dst, dstride, k_rows, sorted, index, n_index, src, sstride, src_rows, cols, st);
+      break;
+    default:
+      LOG(FATAL) << "index type " << index_flag << " is not among the cases";
+  }
+}
 }  // namespace
 
 #define CASE_BEGIN try {
@@ -351,6 +418,47 @@ int mshadow_case_rows_by_index_f32(int op, float *dst, int dstride, int k_rows, 
   } else {
     IndexFill(D, I, S);
   }
+  CASE_END
+}
+
+/* the same families on tensors of another element type: type_flag 0 float, 1 double, 2 half_t
+   (mshadow::TypeFlag codes). ignore_label is handed over as a double and converted to the
+   element type, which is what a caller holding a DType would pass. */
+int mshadow_case_grad_family_any(int type_flag, void *dst, int dstride, const void *src, int sstride,
+                                 const void *label, int lstride, int d0, int rows_or_d1,
+                                 int cols_or_d2, int flags, double ignore_label, float alpha,
+                                 void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  MSHADOW_REAL_TYPE_SWITCH(type_flag, DType, {
+    GradFamilyOf<DType>(dst, dstride, src, sstride, label, lstride, d0, rows_or_d1, cols_or_d2, flags,
+                        ignore_label, alpha, st.get());
+  });
+  CASE_END
+}
+
+int mshadow_case_softmax3d_any(int type_flag, void *dst, int dstride, const void *src, int sstride,
+                               int d0, int d1, int d2, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  MSHADOW_REAL_TYPE_SWITCH(type_flag, DType, {
+    Softmax(G3(static_cast<const DType *>(dst), d0, d1, d2, dstride, st.get()),
+            G3(static_cast<const DType *>(src), d0, d1, d2, sstride, st.get()));
+  });
+  CASE_END
+}
+
+/* op as for mshadow_case_rows_by_index_f32; index_flag: 0 float, 2 half_t, 4 int32, 6 int64 */
+int mshadow_case_rows_by_index_any(int op, int type_flag, int index_flag, void *dst, int dstride,
+                                   int k_rows, const void *sorted, const void *index, int n_index,
+                                   const void *src, int sstride, int src_rows, int cols,
+                                   void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  MSHADOW_REAL_TYPE_SWITCH(type_flag, DType, {
+    RowsByIndexOfIndex<DType>(index_flag, op, dst, dstride, k_rows, sorted, index, n_index, src,
+                              sstride, src_rows, cols, st.get());
+  });
   CASE_END
 }
 

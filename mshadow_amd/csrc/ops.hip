@@ -285,27 +285,24 @@ void LaunchGrad(int flags, const GradLaunch &g) {
 }  // namespace
 
 
-/* about as many workgroups as the machine holds at once (two of these per CU), each owning a
-   run of destination rows and scanning the index vector once */
 template <int OP>
 static int LaunchRowsByIndex(float *dst, int dstride, int k_rows, const void *rows_of,
                              const void *from_of, int index_is_int, int n_index, const float *src,
                              int sstride, int cols, void *stream, const char *what) {
-  const int kWavesPerBlock = kTakeBlock / 64;
-  const int rows_per_block_wanted = (k_rows + 511) / 512;
-  const int rows_per_wave = (rows_per_block_wanted + kWavesPerBlock - 1) / kWavesPerBlock;
-  const int rows_per_block = rows_per_wave * kWavesPerBlock;
-  const unsigned grid = static_cast<unsigned>((k_rows + rows_per_block - 1) / rows_per_block);
+  unsigned grid = 0;
+  int rows_per_wave = 0;
+  mshadow::hip::RowsByIndexGrid(k_rows, &grid, &rows_per_wave);
   const bool vec = Aligned16(dst) && Aligned16(src) && dstride % 4 == 0 && sstride % 4 == 0 &&
                    cols % 4 == 0;
   hipStream_t s = AsStream(stream);
-#define ROWS_LAUNCH(INT, VEC)                                                                 \
-  hipLaunchKernelGGL((RowsByIndexKernel<INT, OP, VEC>), dim3(grid), dim3(kTakeBlock), 0, s, dst,  \
-                     dstride, k_rows, rows_per_wave, rows_of, from_of, n_index, src, sstride, cols)
+#define ROWS_LAUNCH(ITYPE, VEC)                                                               \
+  hipLaunchKernelGGL((RowsByIndexKernel<ITYPE, float, OP, VEC>), dim3(grid), dim3(kTakeBlock), 0, \
+                     s, dst, dstride, k_rows, rows_per_wave, static_cast<const ITYPE *>(rows_of), \
+                     static_cast<const ITYPE *>(from_of), n_index, src, sstride, cols)
   if (index_is_int) {
-    if (vec) ROWS_LAUNCH(true, true); else ROWS_LAUNCH(true, false);
+    if (vec) ROWS_LAUNCH(int32_t, true); else ROWS_LAUNCH(int32_t, false);
   } else {
-    if (vec) ROWS_LAUNCH(false, true); else ROWS_LAUNCH(false, false);
+    if (vec) ROWS_LAUNCH(float, true); else ROWS_LAUNCH(float, false);
   }
 #undef ROWS_LAUNCH
   return AfterLaunch(what);

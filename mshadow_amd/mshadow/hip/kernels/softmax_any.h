@@ -274,15 +274,38 @@ __global__ void __launch_bounds__(kAnyBlock)
   }
 }
 
-/*! \brief dst = src with 1 subtracted at column static_cast<int>(label[row]); a label
- *  outside the row leaves a copy. blockIdx.x = row, blockIdx.y = stretch of columns; a
+/*! \brief which gradient: bit 0 label smoothing, bit 1 an ignored label (the values of
+ *  MSHADOW_HIP_GRAD_SMOOTH / MSHADOW_HIP_GRAD_IGNORE) */
+const int kAnyGradSmooth = 1;
+const int kAnyGradIgnore = 2;
+
+/*! \brief one element of SoftmaxGrad / SmoothSoftmaxGrad (mshadow/tensor_cpu-inl.h:286-455)
+ *  with the host's expressions in the host's types: `p - 1.0f + alpha` and `p - smooth`
+ *  round after every operation for half_t (its operators return half_t), are double
+ *  arithmetic for double, and `smooth` = alpha / (classes - 1) is a float for every type */
+template <typename DType, int FLAGS>
+__device__ __forceinline__ DType GradElement(const DType &p, bool at_label, bool ignored,
+                                             float alpha, float smooth) {
+  if ((FLAGS & kAnyGradIgnore) && ignored) return DType(0.0f);
+  if (FLAGS & kAnyGradSmooth) {
+    if (at_label) return DType(p - 1.0f + alpha);
+    return DType(p - smooth);
+  }
+  if (at_label) return DType(p - 1.0f);
+  return p;
+}
+
+/*! \brief dst = the gradient FLAGS selects for probabilities src and labels label; a label
+ *  outside the row marks no column. blockIdx.x = row, blockIdx.y = stretch of columns; a
  *  thread moves packs of kAnyTile elements. VEC as for SoftmaxAnyKernel. */
-template <typename DType, bool VEC>
+template <typename DType, bool VEC, int FLAGS>
 __global__ void __launch_bounds__(kAnyBlock)
     SoftmaxGradAnyKernel(DType *dst, uint32_t dstride, const DType *src, uint32_t sstride,
-                         const DType *label, uint32_t cols) {
+                         const DType *label, uint32_t cols, int ignore_k, float alpha,
+                         float smooth) {
   const uint32_t row = blockIdx.x;
   const int k = LabelIndex(label[row]);
+  const bool ignored = (FLAGS & kAnyGradIgnore) && k == ignore_k;
   const DType *s = src + static_cast<size_t>(row) * sstride;
   DType *o = dst + static_cast<size_t>(row) * dstride;
   const uint32_t step = gridDim.y * kAnyBlock * kAnyTile;
@@ -290,13 +313,72 @@ __global__ void __launch_bounds__(kAnyBlock)
     AnyPack<DType> v;
     LoadAnyPack<DType, VEC>(&v, s, x, cols, DType(0.0f));
     const uint32_t off = static_cast<uint32_t>(k) - x;  // wraps for k < x
-    if (k >= 0 && off < static_cast<uint32_t>(kAnyTile)) {
+    const bool label_here = k >= 0 && off < static_cast<uint32_t>(kAnyTile);
+    if (FLAGS != 0 || label_here) {
 #pragma unroll
       for (int i = 0; i < kAnyTile; ++i) {
-        if (static_cast<uint32_t>(i) == off) v.v[i] = v.v[i] - 1.0f;
+        v.v[i] = GradElement<DType, FLAGS>(v.v[i], label_here && static_cast<uint32_t>(i) == off,
+                                           ignored, alpha, smooth);
       }
     }
     StoreAnyPack<DType, VEC>(o, x, cols, v);
+  }
+}
+
+/* ---- tensors of three dimensions (d0, d1, d2): the softmax runs over the middle one
+ * (mshadow/tensor_cpu-inl.h:466-488). Element (y, x, n) is at (y * d1 + x) * stride + n. */
+const int kAny3dBlock = 256;
+
+/*! \brief one thread per (y, n), neighbouring threads neighbouring n (coalesced): the
+ *  thread walks x three times, exactly as the host loop does - maximum, terms stored and
+ *  summed left to right in DType, quotients. In place (dst == src) is safe: a thread reads
+ *  and writes its own column only. */
+template <typename DType>
+__global__ void __launch_bounds__(kAny3dBlock)
+    Softmax3dAnyKernel(DType *dst, uint32_t dstride, const DType *src, uint32_t sstride,
+                       uint32_t d0, uint32_t d1, uint32_t d2) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * kAny3dBlock + threadIdx.x;
+  if (idx >= static_cast<size_t>(d0) * d2) return;
+  const uint32_t y = static_cast<uint32_t>(idx / d2);
+  const uint32_t n = static_cast<uint32_t>(idx - static_cast<size_t>(y) * d2);
+  const DType *s = src + static_cast<size_t>(y) * d1 * sstride + n;
+  DType *o = dst + static_cast<size_t>(y) * d1 * dstride + n;
+  DType mmax = s[0];
+  for (uint32_t x = 1; x < d1; ++x) {
+    const DType e = s[static_cast<size_t>(x) * sstride];
+    if (mmax < e) mmax = e;
+  }
+  DType sum = DType(0.0f);
+  for (uint32_t x = 0; x < d1; ++x) {
+    const DType t = DType(SoftmaxExp(DType(s[static_cast<size_t>(x) * sstride] - mmax)));
+    o[static_cast<size_t>(x) * dstride] = t;
+    ChainAdd(sum, t);
+  }
+  for (uint32_t x = 0; x < d1; ++x) {
+    DType t = o[static_cast<size_t>(x) * dstride];
+    t /= sum;
+    o[static_cast<size_t>(x) * dstride] = t;
+  }
+}
+
+/*! \brief one thread per element; label (y, n) at y * lstride + n */
+template <typename DType, int FLAGS>
+__global__ void __launch_bounds__(kAny3dBlock)
+    SoftmaxGrad3dAnyKernel(DType *dst, uint32_t dstride, const DType *src, uint32_t sstride,
+                           const DType *label, uint32_t lstride, uint32_t d0, uint32_t d1,
+                           uint32_t d2, int ignore_k, float alpha, float smooth) {
+  const size_t total = static_cast<size_t>(d0) * d1 * d2;
+  for (size_t idx = static_cast<size_t>(blockIdx.x) * kAny3dBlock + threadIdx.x; idx < total;
+       idx += static_cast<size_t>(gridDim.x) * kAny3dBlock) {
+    const size_t row = idx / d2;  // y * d1 + x
+    const uint32_t n = static_cast<uint32_t>(idx - row * d2);
+    const uint32_t y = static_cast<uint32_t>(row / d1);
+    const uint32_t x = static_cast<uint32_t>(row - static_cast<size_t>(y) * d1);
+    const int k = LabelIndex(label[static_cast<size_t>(y) * lstride + n]);
+    const bool ignored = (FLAGS & kAnyGradIgnore) && k == ignore_k;
+    dst[row * dstride + n] = GradElement<DType, FLAGS>(src[row * sstride + n],
+                                                       static_cast<int>(x) == k, ignored, alpha,
+                                                       smooth);
   }
 }
 

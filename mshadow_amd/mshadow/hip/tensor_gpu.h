@@ -25,6 +25,7 @@
 #if defined(__HIPCC__)
 #include "./kernels/map.h"
 #include "./kernels/reduce.h"
+#include "./kernels/rows_by_index.h"
 #include "./kernels/softmax_any.h"
 #endif
 
@@ -194,9 +195,21 @@ inline void Softmax(Tensor<gpu, 2, DType> dst, const Tensor<gpu, 2, DType> &src)
   LOG(FATAL) << "Softmax<gpu> of this element type: compile the calling translation unit with hipcc";
 #endif
 }
+namespace gpu_detail {
+/*! \brief static_cast<int>(label) as the host makes it (half_t goes through float) */
+inline int LabelAsInt(half::half_t v) { return static_cast<int>(static_cast<float>(v)); }
 template <typename DType>
-inline void SoftmaxGrad(const Tensor<gpu, 2, DType> &dst, const Tensor<gpu, 2, DType> &src,
-                        const Tensor<gpu, 1, DType> &label) {
+inline int LabelAsInt(DType v) { return static_cast<int>(v); }
+/*! \brief alpha / (classes - 1), the count converted from unsigned as the host writes it
+ *  (mshadow/tensor_cpu-inl.h:308) - a float whatever the element type */
+inline float SmoothShare(float alpha, index_t classes) {
+  return alpha / static_cast<float>(classes - 1);
+}
+
+/*! \brief the 2-D gradients of any element type: flags as MSHADOW_HIP_GRAD_* */
+template <typename DType>
+inline void AnyGrad2D(const Tensor<gpu, 2, DType> &dst, const Tensor<gpu, 2, DType> &src,
+                      const Tensor<gpu, 1, DType> &label, int flags, int ignore_k, float alpha) {
   CHECK_EQ(dst.shape_, src.shape_) << "SoftmaxGrad: shape mismatch";
   CHECK_EQ(dst.size(0), label.size(0)) << "SoftmaxGrad: label shape mismatch";
 #if defined(__HIPCC__)
@@ -206,17 +219,27 @@ inline void SoftmaxGrad(const Tensor<gpu, 2, DType> &dst, const Tensor<gpu, 2, D
   const DType *s = src.dptr_;
   const DType *l = label.dptr_;
   uint32_t dstride = dst.stride_, sstride = src.stride_;
-  void *args[] = {&d, &dstride, &s, &sstride, &l, &cols};
+  float smooth = SmoothShare(alpha, dst.size(1));
+  void *args[] = {&d, &dstride, &s, &sstride, &l, &cols, &ignore_k, &alpha, &smooth};
   /* rows on the grid's x axis (up to 2^31 - 1), a row's packs over a few workgroups */
   const uint32_t per_block = hip::kAnyBlock * hip::kAnyTile;
   uint32_t per_row = (cols + per_block - 1) / per_block;
   if (per_row > 64) per_row = 64;
   const uint32_t grid[3] = {rows, per_row, 1};
   const uint32_t block[3] = {static_cast<uint32_t>(hip::kAnyBlock), 1, 1};
-  const bool vec = gpu_detail::AnyPackable(s, sstride, const_cast<const DType *>(d), dstride, cols,
-                                           hip::kAnyTile);
-  const void *kernel = vec ? reinterpret_cast<const void *>(hip::SoftmaxGradAnyKernel<DType, true>)
-                           : reinterpret_cast<const void *>(hip::SoftmaxGradAnyKernel<DType, false>);
+  const bool vec = AnyPackable(s, sstride, const_cast<const DType *>(d), dstride, cols,
+                               hip::kAnyTile);
+  const void *kernel = NULL;
+#define MSHADOW_ANY_GRAD(FLAGS)                                                              \
+  kernel = vec ? reinterpret_cast<const void *>(hip::SoftmaxGradAnyKernel<DType, true, FLAGS>) \
+               : reinterpret_cast<const void *>(hip::SoftmaxGradAnyKernel<DType, false, FLAGS>)
+  switch (flags) {
+    case 0: MSHADOW_ANY_GRAD(0); break;
+    case 1: MSHADOW_ANY_GRAD(1); break;
+    case 2: MSHADOW_ANY_GRAD(2); break;
+    default: MSHADOW_ANY_GRAD(3); break;
+  }
+#undef MSHADOW_ANY_GRAD
   MSHADOW_HIP_CALL(mshadow_hip_launch(kernel, grid, block, args, 0,
                                       Stream<gpu>::GetStream(dst.stream_)));
 #else
@@ -224,8 +247,202 @@ inline void SoftmaxGrad(const Tensor<gpu, 2, DType> &dst, const Tensor<gpu, 2, D
 #endif
 }
 
-/* ---- the rest of the softmax family and the row scatter / gather functions: float tensors,
- * int32 or float indices, each one call into the library */
+/*! \brief the 3-D gradients of any element type */
+template <typename DType>
+inline void AnyGrad3D(const Tensor<gpu, 3, DType> &dst, const Tensor<gpu, 3, DType> &src,
+                      const Tensor<gpu, 2, DType> &label, int flags, int ignore_k, float alpha) {
+  CHECK_EQ(dst.shape_, src.shape_) << "SoftmaxGrad: shape mismatch";
+  CHECK(dst.size(0) == label.size(0) && dst.size(2) == label.size(1))
+      << "SoftmaxGrad: label shape mismatch";
+#if defined(__HIPCC__)
+  uint32_t d0 = dst.size(0), d1 = dst.size(1), d2 = dst.size(2);
+  if (d0 == 0 || d1 == 0 || d2 == 0) return;
+  DType *d = dst.dptr_;
+  const DType *s = src.dptr_;
+  const DType *l = label.dptr_;
+  uint32_t dstride = dst.stride_, sstride = src.stride_, lstride = label.stride_;
+  float smooth = SmoothShare(alpha, dst.size(1));
+  void *args[] = {&d, &dstride, &s, &sstride, &l, &lstride, &d0, &d1, &d2, &ignore_k, &alpha, &smooth};
+  const size_t total = static_cast<size_t>(d0) * d1 * d2;
+  size_t blocks = (total + hip::kAny3dBlock - 1) / hip::kAny3dBlock;
+  if (blocks > (1u << 20)) blocks = 1u << 20;  // the kernel strides over what is left
+  const uint32_t grid[3] = {static_cast<uint32_t>(blocks), 1, 1};
+  const uint32_t block[3] = {static_cast<uint32_t>(hip::kAny3dBlock), 1, 1};
+  const void *kernel = NULL;
+  switch (flags) {
+    case 0: kernel = reinterpret_cast<const void *>(hip::SoftmaxGrad3dAnyKernel<DType, 0>); break;
+    case 1: kernel = reinterpret_cast<const void *>(hip::SoftmaxGrad3dAnyKernel<DType, 1>); break;
+    case 2: kernel = reinterpret_cast<const void *>(hip::SoftmaxGrad3dAnyKernel<DType, 2>); break;
+    default: kernel = reinterpret_cast<const void *>(hip::SoftmaxGrad3dAnyKernel<DType, 3>); break;
+  }
+  MSHADOW_HIP_CALL(mshadow_hip_launch(kernel, grid, block, args, 0,
+                                      Stream<gpu>::GetStream(dst.stream_)));
+#else
+  LOG(FATAL) << "SoftmaxGrad<gpu> of this element type: compile the calling translation unit with hipcc";
+#endif
+}
+
+/*! \brief AddTakeGrad (OP 0) / AddTakeGradLargeBatch (1) / IndexFill (2) of any element and
+ *  index type: the kernel of mshadow/hip/kernels/rows_by_index.h compiled with the caller */
+template <int OP, typename IndexType, typename DType>
+inline void AnyRowsByIndex(Tensor<gpu, 2, DType> dst, const Tensor<gpu, 1, IndexType> &rows_of,
+                           const Tensor<gpu, 1, IndexType> &from_of,
+                           const Tensor<gpu, 2, DType> &src) {
+#if defined(__HIPCC__)
+  int k_rows = dst.size(0), n_index = from_of.size(0), cols = dst.size(1);
+  if (k_rows == 0 || n_index == 0 || cols == 0) return;
+  CHECK_LT(static_cast<uint64_t>(k_rows) + 1024u * 16u, 1ull << 31) << "table too tall";
+  DType *d = dst.dptr_;
+  const DType *s = src.dptr_;
+  const IndexType *r = rows_of.dptr_;
+  const IndexType *f = from_of.dptr_;
+  int dstride = dst.stride_, sstride = src.stride_, rows_per_wave = 0;
+  unsigned blocks = 0;
+  hip::RowsByIndexGrid(k_rows, &blocks, &rows_per_wave);
+  void *args[] = {&d, &dstride, &k_rows, &rows_per_wave, &r, &f, &n_index, &s, &sstride, &cols};
+  const uint32_t grid[3] = {blocks, 1, 1};
+  const uint32_t block[3] = {static_cast<uint32_t>(hip::kTakeBlock), 1, 1};
+  MSHADOW_HIP_CALL(mshadow_hip_launch(
+      reinterpret_cast<const void *>(hip::RowsByIndexKernel<IndexType, DType, OP, false>), grid,
+      block, args, 0, Stream<gpu>::GetStream(dst.stream_)));
+#else
+  LOG(FATAL) << "row scatter of this element type: compile the calling translation unit with hipcc";
+#endif
+}
+/*! \brief which implementation a row scatter takes: float tables with int32 or float index
+ *  vectors call the library's fixed-function kernels, everything else the template above */
+template <typename IndexType, typename DType>
+struct RowsByIndexRoute {
+  inline static void Run(int op, Tensor<gpu, 2, DType> dst, const Tensor<gpu, 1, IndexType> &rows_of,
+                         const Tensor<gpu, 1, IndexType> &from_of, const Tensor<gpu, 2, DType> &src) {
+    if (op == 0) AnyRowsByIndex<0>(dst, rows_of, from_of, src);
+    else if (op == 1) AnyRowsByIndex<1>(dst, rows_of, from_of, src);
+    else AnyRowsByIndex<2>(dst, rows_of, from_of, src);
+  }
+};
+template <typename IndexType, int IS_INT>
+struct RowsByIndexLibrary {
+  inline static void Run(int op, Tensor<gpu, 2, float> dst, const Tensor<gpu, 1, IndexType> &rows_of,
+                         const Tensor<gpu, 1, IndexType> &from_of, const Tensor<gpu, 2, float> &src) {
+    void *stream = Stream<gpu>::GetStream(dst.stream_);
+    if (op == 0) {
+      MSHADOW_HIP_CALL(mshadow_hip_add_take_grad_f32(dst.dptr_, dst.stride_, dst.size(0), from_of.dptr_,
+                                                     IS_INT, from_of.size(0), src.dptr_, src.stride_,
+                                                     src.size(1), stream));
+    } else if (op == 1) {
+      MSHADOW_HIP_CALL(mshadow_hip_add_take_grad_large_batch_f32(
+          dst.dptr_, dst.stride_, dst.size(0), rows_of.dptr_, from_of.dptr_, IS_INT, from_of.size(0),
+          src.dptr_, src.stride_, src.size(1), stream));
+    } else {
+      MSHADOW_HIP_CALL(mshadow_hip_index_fill_f32(dst.dptr_, dst.stride_, dst.size(0), from_of.dptr_,
+                                                  IS_INT, from_of.size(0), src.dptr_, src.stride_,
+                                                  src.size(1), stream));
+    }
+  }
+};
+template <>
+struct RowsByIndexRoute<int, float> : public RowsByIndexLibrary<int, 1> {};
+template <>
+struct RowsByIndexRoute<float, float> : public RowsByIndexLibrary<float, 0> {};
+}  // namespace gpu_detail
+
+/* ---- the softmax family for any element type (mshadow/tensor_gpu-inl.h:157-215): kernels in
+ * the element type's own arithmetic, compiled with the caller. Float tensors take the
+ * non-template overloads further down, which call the library. */
+template <typename DType>
+inline void SoftmaxGrad(const Tensor<gpu, 2, DType> &dst, const Tensor<gpu, 2, DType> &src,
+                        const Tensor<gpu, 1, DType> &label) {
+  gpu_detail::AnyGrad2D(dst, src, label, 0, 0, 0.0f);
+}
+template <typename DType>
+inline void SmoothSoftmaxGrad(const Tensor<gpu, 2, DType> &dst, const Tensor<gpu, 2, DType> &src,
+                              const Tensor<gpu, 1, DType> &label, const float alpha) {
+  gpu_detail::AnyGrad2D(dst, src, label, MSHADOW_HIP_GRAD_SMOOTH, 0, alpha);
+}
+template <typename DType>
+inline void SoftmaxGrad(const Tensor<gpu, 2, DType> &dst, const Tensor<gpu, 2, DType> &src,
+                        const Tensor<gpu, 1, DType> &label, const DType &ignore_label) {
+  gpu_detail::AnyGrad2D(dst, src, label, MSHADOW_HIP_GRAD_IGNORE,
+                        gpu_detail::LabelAsInt(ignore_label), 0.0f);
+}
+template <typename DType>
+inline void SmoothSoftmaxGrad(const Tensor<gpu, 2, DType> &dst, const Tensor<gpu, 2, DType> &src,
+                              const Tensor<gpu, 1, DType> &label, const DType &ignore_label,
+                              const float alpha) {
+  gpu_detail::AnyGrad2D(dst, src, label, MSHADOW_HIP_GRAD_SMOOTH | MSHADOW_HIP_GRAD_IGNORE,
+                        gpu_detail::LabelAsInt(ignore_label), alpha);
+}
+template <typename DType>
+inline void Softmax(Tensor<gpu, 3, DType> dst, const Tensor<gpu, 3, DType> &src) {
+  CHECK_EQ(dst.shape_, src.shape_) << "Softmax: shape mismatch";
+#if defined(__HIPCC__)
+  uint32_t d0 = dst.size(0), d1 = dst.size(1), d2 = dst.size(2);
+  if (d0 == 0 || d1 == 0 || d2 == 0) return;
+  DType *d = dst.dptr_;
+  const DType *s = src.dptr_;
+  uint32_t dstride = dst.stride_, sstride = src.stride_;
+  void *args[] = {&d, &dstride, &s, &sstride, &d0, &d1, &d2};
+  const size_t columns = static_cast<size_t>(d0) * d2;
+  CHECK_LT(columns, (1ull << 31) * hip::kAny3dBlock) << "Softmax: too many columns";
+  const uint32_t grid[3] = {static_cast<uint32_t>((columns + hip::kAny3dBlock - 1) / hip::kAny3dBlock), 1, 1};
+  const uint32_t block[3] = {static_cast<uint32_t>(hip::kAny3dBlock), 1, 1};
+  MSHADOW_HIP_CALL(mshadow_hip_launch(reinterpret_cast<const void *>(hip::Softmax3dAnyKernel<DType>),
+                                      grid, block, args, 0, Stream<gpu>::GetStream(dst.stream_)));
+#else
+  LOG(FATAL) << "Softmax<gpu> of this element type: compile the calling translation unit with hipcc";
+#endif
+}
+template <typename DType>
+inline void SoftmaxGrad(const Tensor<gpu, 3, DType> &dst, const Tensor<gpu, 3, DType> &src,
+                        const Tensor<gpu, 2, DType> &label) {
+  gpu_detail::AnyGrad3D(dst, src, label, 0, 0, 0.0f);
+}
+template <typename DType>
+inline void SmoothSoftmaxGrad(const Tensor<gpu, 3, DType> &dst, const Tensor<gpu, 3, DType> &src,
+                              const Tensor<gpu, 2, DType> &label, const float alpha) {
+  gpu_detail::AnyGrad3D(dst, src, label, MSHADOW_HIP_GRAD_SMOOTH, 0, alpha);
+}
+template <typename DType>
+inline void SoftmaxGrad(const Tensor<gpu, 3, DType> &dst, const Tensor<gpu, 3, DType> &src,
+                        const Tensor<gpu, 2, DType> &label, const DType &ignore_label) {
+  gpu_detail::AnyGrad3D(dst, src, label, MSHADOW_HIP_GRAD_IGNORE,
+                        gpu_detail::LabelAsInt(ignore_label), 0.0f);
+}
+template <typename DType>
+inline void SmoothSoftmaxGrad(const Tensor<gpu, 3, DType> &dst, const Tensor<gpu, 3, DType> &src,
+                              const Tensor<gpu, 2, DType> &label, const DType &ignore_label,
+                              const float alpha) {
+  gpu_detail::AnyGrad3D(dst, src, label, MSHADOW_HIP_GRAD_SMOOTH | MSHADOW_HIP_GRAD_IGNORE,
+                        gpu_detail::LabelAsInt(ignore_label), alpha);
+}
+/* ---- the row scatter / gather functions for any element and index type
+ * (mshadow/tensor_gpu-inl.h:217-240); float tensors with int32 or float indices take the
+ * overloads further down */
+template <typename IndexType, typename DType>
+inline void AddTakeGrad(Tensor<gpu, 2, DType> dst, const Tensor<gpu, 1, IndexType> &index,
+                        const Tensor<gpu, 2, DType> &src) {
+  CHECK_EQ(dst.size(1), src.size(1)) << "AddTakeGrad: shape mismatch";
+  CHECK_EQ(index.size(0), src.size(0)) << "AddTakeGrad: shape mismatch";
+  gpu_detail::RowsByIndexRoute<IndexType, DType>::Run(0, dst, index, index, src);
+}
+template <typename IndexType, typename DType>
+inline void AddTakeGradLargeBatch(Tensor<gpu, 2, DType> dst, const Tensor<gpu, 1, IndexType> &sorted,
+                                  const Tensor<gpu, 1, IndexType> &index,
+                                  const Tensor<gpu, 2, DType> &src) {
+  CHECK_EQ(dst.size(1), src.size(1)) << "AddTakeGradLargeBatch: shape mismatch";
+  CHECK_EQ(sorted.size(0), index.size(0)) << "AddTakeGradLargeBatch: shape mismatch";
+  gpu_detail::RowsByIndexRoute<IndexType, DType>::Run(1, dst, sorted, index, src);
+}
+template <typename IndexType, typename DType>
+inline void IndexFill(Tensor<gpu, 2, DType> dst, const Tensor<gpu, 1, IndexType> &index,
+                      const Tensor<gpu, 2, DType> &src) {
+  CHECK_EQ(dst.size(1), src.size(1)) << "IndexFill: shape mismatch";
+  CHECK_EQ(index.size(0), src.size(0)) << "IndexFill: shape mismatch";
+  gpu_detail::RowsByIndexRoute<IndexType, DType>::Run(2, dst, index, index, src);
+}
+
+/* ---- the softmax family for float tensors: non-template overloads, each one call into the
+ * library's fixed-function kernels */
 namespace gpu_detail {
 inline void Grad2D(const Tensor<gpu, 2, float> &dst, const Tensor<gpu, 2, float> &src,
                    const Tensor<gpu, 1, float> &label, int flags, float ignore_label, float alpha) {
@@ -244,12 +461,6 @@ inline void Grad3D(const Tensor<gpu, 3, float> &dst, const Tensor<gpu, 3, float>
       dst.dptr_, dst.stride_, src.dptr_, src.stride_, label.dptr_, label.stride_, dst.size(0),
       dst.size(1), dst.size(2), flags, ignore_label, alpha, Stream<gpu>::GetStream(dst.stream_)));
 }
-template <typename IndexType>
-struct IndexKind;  // only int32 and float index vectors are provided
-template <>
-struct IndexKind<int> { static const int kIsInt = 1; };
-template <>
-struct IndexKind<float> { static const int kIsInt = 0; };
 }  // namespace gpu_detail
 
 inline void Softmax(Tensor<gpu, 3, float> dst, const Tensor<gpu, 3, float> &src) {
@@ -290,36 +501,6 @@ inline void SmoothSoftmaxGrad(const Tensor<gpu, 3, float> &dst, const Tensor<gpu
   gpu_detail::Grad3D(dst, src, label, MSHADOW_HIP_GRAD_SMOOTH | MSHADOW_HIP_GRAD_IGNORE,
                      ignore_label, alpha);
 }
-template <typename IndexType>
-inline void AddTakeGrad(Tensor<gpu, 2, float> dst, const Tensor<gpu, 1, IndexType> &index,
-                        const Tensor<gpu, 2, float> &src) {
-  CHECK_EQ(dst.size(1), src.size(1)) << "AddTakeGrad: shape mismatch";
-  CHECK_EQ(index.size(0), src.size(0)) << "AddTakeGrad: shape mismatch";
-  MSHADOW_HIP_CALL(mshadow_hip_add_take_grad_f32(
-      dst.dptr_, dst.stride_, dst.size(0), index.dptr_, gpu_detail::IndexKind<IndexType>::kIsInt,
-      index.size(0), src.dptr_, src.stride_, src.size(1), Stream<gpu>::GetStream(dst.stream_)));
-}
-template <typename IndexType>
-inline void AddTakeGradLargeBatch(Tensor<gpu, 2, float> dst, const Tensor<gpu, 1, IndexType> &sorted,
-                                  const Tensor<gpu, 1, IndexType> &index,
-                                  const Tensor<gpu, 2, float> &src) {
-  CHECK_EQ(dst.size(1), src.size(1)) << "AddTakeGradLargeBatch: shape mismatch";
-  CHECK_EQ(sorted.size(0), index.size(0)) << "AddTakeGradLargeBatch: shape mismatch";
-  MSHADOW_HIP_CALL(mshadow_hip_add_take_grad_large_batch_f32(
-      dst.dptr_, dst.stride_, dst.size(0), sorted.dptr_, index.dptr_,
-      gpu_detail::IndexKind<IndexType>::kIsInt, index.size(0), src.dptr_, src.stride_, src.size(1),
-      Stream<gpu>::GetStream(dst.stream_)));
-}
-template <typename IndexType>
-inline void IndexFill(Tensor<gpu, 2, float> dst, const Tensor<gpu, 1, IndexType> &index,
-                      const Tensor<gpu, 2, float> &src) {
-  CHECK_EQ(dst.size(1), src.size(1)) << "IndexFill: shape mismatch";
-  CHECK_EQ(index.size(0), src.size(0)) << "IndexFill: shape mismatch";
-  MSHADOW_HIP_CALL(mshadow_hip_index_fill_f32(
-      dst.dptr_, dst.stride_, dst.size(0), index.dptr_, gpu_detail::IndexKind<IndexType>::kIsInt,
-      index.size(0), src.dptr_, src.stride_, src.size(1), Stream<gpu>::GetStream(dst.stream_)));
-}
-
 namespace gpu_detail {
 /*! \brief how the bits of a 32-bit key type are ordered (-1: no device sort for this type) */
 template <typename KDType>

@@ -495,6 +495,176 @@ void orc_index_fill_f32(float *dst, int dstride, const void *index, int index_is
   }
 }
 
+/* ---- the gradient family, the 3-D softmax and the row scatter functions on tensors of another
+   element type: type_flag 0 float, 1 double, 2 half_t (mshadow/base.h:305-313 TypeFlag codes).
+   The host templates (mshadow/tensor_cpu-inl.h:286-528) are written once for every DType; what
+   differs is where a value is rounded. double: `src - 1.0f + alpha` and `src - smooth_grad`
+   promote the float operands, smooth_grad itself stays a float quotient. half_t: every operator
+   returns a half_t (mshadow/half.h:45-56), so `src - 1.0f` rounds to 16 bits before `+ alpha`
+   rounds again; a row addition is one float add rounded to 16 bits. Labels, ignore_label and
+   index entries reach `int` through the type's conversion (half_t: through float). */
+#define ORC_T_F32 0
+#define ORC_T_F64 1
+#define ORC_T_F16 2
+#define ORC_T_I32 4
+#define ORC_T_I64 6
+
+static inline int int_of_entry(const void *v, int type_flag, int64_t i) {
+  switch (type_flag) {
+    case ORC_T_F32: return (int)((const float *)v)[i];
+    case ORC_T_F64: return (int)((const double *)v)[i];
+    case ORC_T_F16: return (int)wide(((const uint16_t *)v)[i]);
+    case ORC_T_I32: return ((const int32_t *)v)[i];
+    default: return (int)((const int64_t *)v)[i];
+  }
+}
+
+static inline double grad_f64(double p, int at_label, int flags, int ignored, float alpha,
+                              float smooth_grad) {
+  if ((flags & ORC_GRAD_IGNORE) && ignored) return 0.0;
+  if (at_label) {
+    double v = p - 1.0f;
+    if (flags & ORC_GRAD_SMOOTH) v = v + alpha;
+    return v;
+  }
+  return (flags & ORC_GRAD_SMOOTH) ? p - smooth_grad : p;
+}
+static inline uint16_t grad_f16(uint16_t p, int at_label, int flags, int ignored, float alpha,
+                                float smooth_grad) {
+  if ((flags & ORC_GRAD_IGNORE) && ignored) return half_of(0.0f);
+  if (at_label) {
+    uint16_t v = half_of(wide(p) - 1.0f);
+    if (flags & ORC_GRAD_SMOOTH) v = half_of(wide(v) + alpha);
+    return v;
+  }
+  return (flags & ORC_GRAD_SMOOTH) ? half_of(wide(p) - smooth_grad) : p;
+}
+static inline float grad_f32(float p, int at_label, int flags, int ignored, float alpha,
+                             float smooth_grad) {
+  if ((flags & ORC_GRAD_IGNORE) && ignored) return 0.0f;
+  if (at_label) {
+    float v = p - 1.0f;
+    if (flags & ORC_GRAD_SMOOTH) v = v + alpha;
+    return v;
+  }
+  return (flags & ORC_GRAD_SMOOTH) ? p - smooth_grad : p;
+}
+
+/* d0 == 0: the 2-D functions on rows_or_d1 x cols_or_d2 (label: one per row); otherwise the 3-D
+   ones on (d0, d1, d2) with labels (d0, d2) of pitch lstride */
+void orc_grad_family_any(int type_flag, void *dst, int dstride, const void *src, int sstride,
+                         const void *label, int lstride, int d0, int rows_or_d1, int cols_or_d2,
+                         int flags, double ignore_label, float alpha) {
+  const int two_d = d0 == 0;
+  const int outer = two_d ? rows_or_d1 : d0;
+  const int classes = two_d ? cols_or_d2 : rows_or_d1;
+  const int inner = two_d ? 1 : cols_or_d2;
+  const float smooth_grad = alpha / (float)(unsigned)(classes - 1);
+  int ignore_k;
+  if (type_flag == ORC_T_F16) ignore_k = (int)wide(half_of((float)ignore_label));
+  else if (type_flag == ORC_T_F64) ignore_k = (int)(double)(float)ignore_label;
+  else ignore_k = (int)(float)ignore_label;
+#pragma omp parallel for
+  for (int y = 0; y < outer; ++y) {
+    for (int n = 0; n < inner; ++n) {
+      const int64_t lab_at = two_d ? y : (int64_t)y * lstride + n;
+      const int k = int_of_entry(label, type_flag, lab_at);
+      const int ignored = k == ignore_k;
+      for (int x = 0; x < classes; ++x) {
+        const int64_t so = two_d ? (int64_t)y * sstride + x : ((int64_t)y * classes + x) * sstride + n;
+        const int64_t dof = two_d ? (int64_t)y * dstride + x : ((int64_t)y * classes + x) * dstride + n;
+        if (type_flag == ORC_T_F16) {
+          ((uint16_t *)dst)[dof] = grad_f16(((const uint16_t *)src)[so], x == k, flags, ignored, alpha, smooth_grad);
+        } else if (type_flag == ORC_T_F64) {
+          ((double *)dst)[dof] = grad_f64(((const double *)src)[so], x == k, flags, ignored, alpha, smooth_grad);
+        } else {
+          ((float *)dst)[dof] = grad_f32(((const float *)src)[so], x == k, flags, ignored, alpha, smooth_grad);
+        }
+      }
+    }
+  }
+}
+
+/* Softmax on 3-D tensors of another element type, mshadow/tensor_cpu-inl.h:466-488 */
+void orc_softmax3d_any(int type_flag, void *dst, int dstride, const void *src, int sstride, int d0,
+                       int d1, int d2) {
+  if (type_flag == ORC_T_F32) {
+    orc_softmax3d_f32((float *)dst, dstride, (const float *)src, sstride, d0, d1, d2);
+    return;
+  }
+#pragma omp parallel for
+  for (int y = 0; y < d0; ++y) {
+    for (int n = 0; n < d2; ++n) {
+      if (type_flag == ORC_T_F64) {
+        const double *s = (const double *)src + (int64_t)y * d1 * sstride + n;
+        double *o = (double *)dst + (int64_t)y * d1 * dstride + n;
+        double mmax = s[0];
+        for (int x = 1; x < d1; ++x) {
+          if (mmax < s[(int64_t)x * sstride]) mmax = s[(int64_t)x * sstride];
+        }
+        double sum = 0.0;
+        for (int x = 0; x < d1; ++x) {
+          o[(int64_t)x * dstride] = exp(s[(int64_t)x * sstride] - mmax);
+          sum += o[(int64_t)x * dstride];
+        }
+        for (int x = 0; x < d1; ++x) o[(int64_t)x * dstride] /= sum;
+      } else {
+        const uint16_t *s = (const uint16_t *)src + (int64_t)y * d1 * sstride + n;
+        uint16_t *o = (uint16_t *)dst + (int64_t)y * d1 * dstride + n;
+        uint16_t mmax = s[0];
+        for (int x = 1; x < d1; ++x) {
+          if (wide(mmax) < wide(s[(int64_t)x * sstride])) mmax = s[(int64_t)x * sstride];
+        }
+        uint16_t sum = half_of(0.0f);
+        for (int x = 0; x < d1; ++x) {
+          const uint16_t t = half_of(expf(wide(half_of(wide(s[(int64_t)x * sstride]) - wide(mmax)))));
+          o[(int64_t)x * dstride] = t;
+          sum = half_add(sum, t);
+        }
+        for (int x = 0; x < d1; ++x) {
+          o[(int64_t)x * dstride] = half_of(wide(o[(int64_t)x * dstride]) / wide(sum));
+        }
+      }
+    }
+  }
+}
+
+/* op 0 AddTakeGrad, 1 AddTakeGradLargeBatch, 2 IndexFill (mshadow/tensor_cpu-inl.h:497-528) for
+   tables of type_flag elements and index vectors of index_flag entries */
+void orc_rows_by_index_any(int op, int type_flag, int index_flag, void *dst, int dstride, int k_rows,
+                           const void *sorted, const void *index, int n_index, const void *src,
+                           int sstride, int cols) {
+  for (int y = 0; y < n_index; ++y) {
+    int j, from = y;
+    if (op == 0) {
+      j = int_of_entry(index, index_flag, y);
+      if (j <= 0) j = 0;
+      else if (j >= k_rows) j = k_rows - 1;
+    } else if (op == 1) {
+      j = int_of_entry(sorted, index_flag, y);
+      from = int_of_entry(index, index_flag, y);
+    } else {
+      j = int_of_entry(index, index_flag, y);
+    }
+    for (int x = 0; x < cols; ++x) {
+      const int64_t d = (int64_t)j * dstride + x, s = (int64_t)from * sstride + x;
+      if (type_flag == ORC_T_F16) {
+        uint16_t *D = (uint16_t *)dst;
+        const uint16_t v = ((const uint16_t *)src)[s];
+        D[d] = op == 2 ? v : half_of(wide(D[d]) + wide(v));
+      } else if (type_flag == ORC_T_F64) {
+        double *D = (double *)dst;
+        const double v = ((const double *)src)[s];
+        D[d] = op == 2 ? v : D[d] + v;
+      } else {
+        float *D = (float *)dst;
+        const float v = ((const float *)src)[s];
+        D[d] = op == 2 ? v : D[d] + v;
+      }
+    }
+  }
+}
+
 /* SortByKey, mshadow/tensor_cpu-inl.h:531-559: std::stable_sort of the positions under
    keys[a] < keys[b] (ascending) or keys[a] > keys[b] (descending), then keys and values
    permuted alike. Restated as a bottom-up merge sort, which is stable by construction: the

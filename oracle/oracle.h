@@ -95,6 +95,17 @@ void orc_add_take_grad_large_batch_f32(float *dst, int dstride, const void *sort
 void orc_index_fill_f32(float *dst, int dstride, const void *index, int index_is_int,
                         int n_index, const float *src, int sstride, int cols);
 
+/* the same families for another element type (type_flag 0 float, 1 double, 2 half_t) and, for the
+   row functions, another index type (index_flag 0 float, 2 half_t, 4 int32, 6 int64) */
+void orc_grad_family_any(int type_flag, void *dst, int dstride, const void *src, int sstride,
+                         const void *label, int lstride, int d0, int rows_or_d1, int cols_or_d2,
+                         int flags, double ignore_label, float alpha);
+void orc_softmax3d_any(int type_flag, void *dst, int dstride, const void *src, int sstride, int d0,
+                       int d1, int d2);
+void orc_rows_by_index_any(int op, int type_flag, int index_flag, void *dst, int dstride, int k_rows,
+                           const void *sorted, const void *index, int n_index, const void *src,
+                           int sstride, int cols);
+
 void orc_sort_by_key_32(void *keys, int key_kind, void *values, int n, int is_ascend);
 void orc_vectorized_sort_32(void *values, int value_kind, void *segments, int n);
 

@@ -80,6 +80,71 @@ void ReduceHighHalf(Tensor<cpu, 1, HalfT> dst, const Src &src, int saver, HalfT 
   }
 }
 
+/* the gradient family and the row scatter functions of the reference for one element type */
+template <typename T>
+Tensor<cpu, 3, T> T3p(const T *p, int d0, int d1, int d2, int stride) {
+  Tensor<cpu, 3, T> t(const_cast<T *>(p), Shape3(d0, d1, d2));
+  t.stride_ = stride;
+  return t;
+}
+template <typename DType>
+void RefGradFamily(void *dst, int dstride, const void *src, int sstride, const void *label,
+                   int lstride, int d0, int rows_or_d1, int cols_or_d2, int flags,
+                   double ignore_label, float alpha) {
+  const DType *s = static_cast<const DType *>(src), *l = static_cast<const DType *>(label);
+  DType *d = static_cast<DType *>(dst);
+  const DType ignore = DType(static_cast<float>(ignore_label));
+  if (d0 == 0) {
+    const int rows = rows_or_d1, cols = cols_or_d2;
+    Tensor<cpu, 2, DType> D = T2(d, rows, cols, dstride), S = T2(s, rows, cols, sstride);
+    Tensor<cpu, 1, DType> L = T1(l, rows);
+    switch (flags) {
+      case 0: SoftmaxGrad(D, S, L); break;
+      case 1: SmoothSoftmaxGrad(D, S, L, alpha); break;
+      case 2: SoftmaxGrad(D, S, L, ignore); break;
+      default: SmoothSoftmaxGrad(D, S, L, ignore, alpha); break;
+    }
+  } else {
+    const int d1 = rows_or_d1, d2 = cols_or_d2;
+    Tensor<cpu, 3, DType> D = T3p(d, d0, d1, d2, dstride), S = T3p(s, d0, d1, d2, sstride);
+    Tensor<cpu, 2, DType> L = T2(l, d0, d2, lstride);
+    switch (flags) {
+      case 0: SoftmaxGrad(D, S, L); break;
+      case 1: SmoothSoftmaxGrad(D, S, L, alpha); break;
+      case 2: SoftmaxGrad(D, S, L, ignore); break;
+      default: SmoothSoftmaxGrad(D, S, L, ignore, alpha); break;
+    }
+  }
+}
+template <typename IndexType, typename DType>
+void RefRowsByIndex(int op, void *dst, int dstride, int k_rows, const void *sorted, const void *index,
+                    int n_index, const void *src, int sstride, int cols) {
+  /* the row count of src is not used by the reference beyond the indices */
+  Tensor<cpu, 2, DType> D = T2(static_cast<const DType *>(dst), k_rows, cols, dstride);
+  Tensor<cpu, 2, DType> S = T2(static_cast<const DType *>(src), 1 << 30, cols, sstride);
+  Tensor<cpu, 1, IndexType> I = T1(static_cast<const IndexType *>(index), n_index);
+  if (op == 0) {
+    S.shape_[0] = n_index;
+    AddTakeGrad(D, I, S);
+  } else if (op == 1) {
+    AddTakeGradLargeBatch(D, T1(static_cast<const IndexType *>(sorted), n_index), I, S);
+  } else {
+    S.shape_[0] = n_index;
+    IndexFill(D, I, S);
+  }
+}
+template <typename DType>
+void RefRowsByIndexOfIndex(int index_flag, int op, void *dst, int dstride, int k_rows,
+                           const void *sorted, const void *index, int n_index, const void *src,
+                           int sstride, int cols) {
+  switch (index_flag) {
+    case kFloat32: RefRowsByIndex<float, DType>(op, dst, dstride, k_rows, sorted, index, n_index, src, sstride, cols); break;
+    case kFloat16: RefRowsByIndex<HalfT, DType>(op, dst, dstride, k_rows, sorted, index, n_index, src, sstride, cols); break;
+    case kInt32: RefRowsByIndex<int, DType>(op, dst, dstride, k_rows, sorted, index, n_index, src, sstride, cols); break;
+    default: RefRowsByIndex<int64_t, DType>(op, dst, dstride, k_rows, sorted, index, n_index, src, sstride, cols); break;
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -266,6 +331,32 @@ void ref_index_fill_f32(float *dst, int dstride, const void *index, int index_is
   } else {
     IndexFill(D, T1(static_cast<const float *>(index), n_index), S);
   }
+}
+
+void ref_grad_family_any(int type_flag, void *dst, int dstride, const void *src, int sstride,
+                         const void *label, int lstride, int d0, int rows_or_d1, int cols_or_d2,
+                         int flags, double ignore_label, float alpha) {
+  MSHADOW_REAL_TYPE_SWITCH(type_flag, DType, {
+    RefGradFamily<DType>(dst, dstride, src, sstride, label, lstride, d0, rows_or_d1, cols_or_d2,
+                         flags, ignore_label, alpha);
+  });
+}
+
+void ref_softmax3d_any(int type_flag, void *dst, int dstride, const void *src, int sstride, int d0,
+                       int d1, int d2) {
+  MSHADOW_REAL_TYPE_SWITCH(type_flag, DType, {
+    Softmax(T3p(static_cast<const DType *>(dst), d0, d1, d2, dstride),
+            T3p(static_cast<const DType *>(src), d0, d1, d2, sstride));
+  });
+}
+
+void ref_rows_by_index_any(int op, int type_flag, int index_flag, void *dst, int dstride, int k_rows,
+                           const void *sorted, const void *index, int n_index, const void *src,
+                           int sstride, int cols) {
+  MSHADOW_REAL_TYPE_SWITCH(type_flag, DType, {
+    RefRowsByIndexOfIndex<DType>(index_flag, op, dst, dstride, k_rows, sorted, index, n_index, src,
+                                 sstride, cols);
+  });
 }
 
 /* key_kind 0: float keys with int values; 1: int keys with float values (the value words are

@@ -90,6 +90,9 @@ class Checker:
         self._fn("add_take_grad_f32", [_p, _i, _i, _p, _i, _i, _p, _i, _i])
         self._fn("add_take_grad_large_batch_f32", [_p, _i, _p, _p, _i, _i, _p, _i, _i])
         self._fn("index_fill_f32", [_p, _i, _p, _i, _i, _p, _i, _i])
+        self._fn("grad_family_any", [_i, _p, _i, _p, _i, _p, _i, _i, _i, _i, _i, C.c_double, _f])
+        self._fn("softmax3d_any", [_i, _p, _i, _p, _i, _i, _i, _i])
+        self._fn("rows_by_index_any", [_i, _i, _i, _p, _i, _i, _p, _p, _i, _p, _i, _i])
         self._fn("sort_by_key_32", [_p, _i, _p, _i, _i])
         self._fn("vectorized_sort_32", [_p, _i, _p, _i])
         if self.prefix == "ref":
@@ -216,6 +219,34 @@ class Checker:
     def index_fill(self, dst, index, src):
         self._index_fill_f32(ptr(dst), pitch(dst), ptr(index), self._is_int(index),
                              index.shape[0], ptr(src), pitch(src), src.shape[1])
+        return dst
+
+    TYPE_FLAG = {"float32": 0, "float64": 1, "float16": 2, "int32": 4, "int64": 6}
+
+    def grad_family_any(self, dst, src, label, flags, ignore_label=0.0, alpha=0.0):
+        """SoftmaxGrad / SmoothSoftmaxGrad (with or without ignore_label) on float32, float64
+        or float16 (= half_t) arrays; 2-D or 3-D by src's shape"""
+        if src.ndim == 2:
+            d0, a, b = 0, src.shape[0], src.shape[1]
+            lpitch = label.shape[0]
+        else:
+            d0, a, b = src.shape
+            lpitch = pitch(label)
+        self._grad_family_any(self.TYPE_FLAG[src.dtype.name], ptr(dst), pitch(dst), ptr(src),
+                              pitch(src), ptr(label), lpitch, d0, a, b, flags, ignore_label, alpha)
+        return dst
+
+    def softmax3d_any(self, dst, src):
+        d0, d1, d2 = src.shape
+        self._softmax3d_any(self.TYPE_FLAG[src.dtype.name], ptr(dst), pitch(dst), ptr(src),
+                            pitch(src), d0, d1, d2)
+        return dst
+
+    def rows_by_index_any(self, op, dst, sorted_rows, index, src):
+        self._rows_by_index_any(op, self.TYPE_FLAG[dst.dtype.name], self.TYPE_FLAG[index.dtype.name],
+                                ptr(dst), pitch(dst), dst.shape[0],
+                                ptr(sorted_rows) if sorted_rows is not None else None, ptr(index),
+                                index.shape[0], ptr(src), pitch(src), src.shape[1])
         return dst
 
     @staticmethod
