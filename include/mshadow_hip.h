@@ -201,6 +201,17 @@ int mshadow_hip_random_uniform_f32(float *dst, int dstride, int rows, int cols, 
 int mshadow_hip_random_normal_f32(float *dst, int dstride, int rows, int cols, uint64_t seed,
                                   uint64_t subsequence, uint64_t counter, float mu, float sigma,
                                   void *stream);
+/* The same for Random<gpu, double> (mshadow/random.h:486-514: curandGenerateUniformDouble /
+   curandGenerateNormalDouble there). A value takes two words, 52 bits of them: element e of a
+   call uses block `counter + e / 2`, words 2 (e % 2) and 2 (e % 2) + 1; the caller advances
+   `counter` by (elements + 1) / 2 per call. Box-Muller runs in double on the block's two
+   uniforms. */
+int mshadow_hip_random_uniform_f64(double *dst, int dstride, int rows, int cols, uint64_t seed,
+                                   uint64_t subsequence, uint64_t counter, double a, double b,
+                                   void *stream);
+int mshadow_hip_random_normal_f64(double *dst, int dstride, int rows, int cols, uint64_t seed,
+                                  uint64_t subsequence, uint64_t counter, double mu, double sigma,
+                                  void *stream);
 
 /* dst = transpose(src, axes) / dst = swapaxis<a1, a2>(src) on dense tensors of 32-bit
    elements: dst axis i is src axis axes[i]; `shape` is the source's, ndim <= 6

@@ -97,6 +97,20 @@ int mshadow_case_softmax3d_f32(float *dst, int dstride, const float *src, int ss
 int mshadow_case_rows_by_index_f32(int op, float *dst, int dstride, int k_rows, const int *sorted,
                                    const int *index, int n_index, const float *src, int sstride,
                                    int src_rows, int cols, void *stream);
+/* the gradient family (d0 == 0: 2-D), the 3-D Softmax and the row functions on tensors of
+   another element type: type_flag 0 float, 1 double, 2 half_t (mshadow::TypeFlag codes);
+   index_flag 0 float, 2 half_t, 4 int32, 6 int64. ignore_label is converted to the element
+   type before the call, as a caller holding a DType would pass it. */
+int mshadow_case_grad_family_any(int type_flag, void *dst, int dstride, const void *src, int sstride,
+                                 const void *label, int lstride, int d0, int rows_or_d1,
+                                 int cols_or_d2, int flags, double ignore_label, float alpha,
+                                 void *stream);
+int mshadow_case_softmax3d_any(int type_flag, void *dst, int dstride, const void *src, int sstride,
+                               int d0, int d1, int d2, void *stream);
+int mshadow_case_rows_by_index_any(int op, int type_flag, int index_flag, void *dst, int dstride,
+                                   int k_rows, const void *sorted, const void *index, int n_index,
+                                   const void *src, int sstride, int src_rows, int cols,
+                                   void *stream);
 
 /* broadcast<1> / repmat / reshape / swapaxis / mirror / upsampling_nearest /
    broadcast_scalar expressions over a dense (n, c, h, w) input `a` and a vector `v`
@@ -107,6 +121,8 @@ int mshadow_case_shaping_f32(int op, float *out, const float *a, const float *v,
 /* Random<gpu>(seed): op 0 SampleUniform(p0, p1) into the two halves of out in turn; 1
    SampleGaussian(p0, p1); 2 out = uniform(Shape1(n)) * 2; 3 GetRandInt (unsigned words) */
 int mshadow_case_random_f32(int op, int seed, float *out, int n, float p0, float p1, void *stream);
+/* Random<gpu, double>(seed): ops 0-2 as above */
+int mshadow_case_random_f64(int op, int seed, double *out, int n, double p0, double p1, void *stream);
 
 /* op 0: SortByKey(keys, values, is_ascend); 1: VectorizedSort(keys, values as segment numbers).
    key_kind 0: float keys with int values, 1: int keys with float values (int segments for op 1) */

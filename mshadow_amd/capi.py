@@ -75,6 +75,8 @@ HIP_SYMBOLS = {
     "mshadow_hip_random_u32": ([_p, _sz, C.c_uint64, C.c_uint64, C.c_uint64, _p], _i),
     "mshadow_hip_random_uniform_f32": ([_p, _i, _i, _i, C.c_uint64, C.c_uint64, C.c_uint64, _f, _f, _p], _i),
     "mshadow_hip_random_normal_f32": ([_p, _i, _i, _i, C.c_uint64, C.c_uint64, C.c_uint64, _f, _f, _p], _i),
+    "mshadow_hip_random_uniform_f64": ([_p, _i, _i, _i, C.c_uint64, C.c_uint64, C.c_uint64, C.c_double, C.c_double, _p], _i),
+    "mshadow_hip_random_normal_f64": ([_p, _i, _i, _i, C.c_uint64, C.c_uint64, C.c_uint64, C.c_double, C.c_double, _p], _i),
     "mshadow_hip_fill_32": ([_p, _i, _i, _i, C.c_uint32, _p], _i),
     "mshadow_hip_permute_32": ([_p, _p, _i, C.POINTER(_i), C.POINTER(_i), _p], _i),
     "mshadow_hip_sort_by_key_workspace": ([_sz, C.POINTER(_sz)], _i),
@@ -120,6 +122,7 @@ CASES_SYMBOLS = {
     "mshadow_case_rows_by_index_any": ([_i, _i, _i, _p, _i, _i, _p, _p, _i, _p, _i, _i, _i, _p], _i),
     "mshadow_case_shaping_f32": ([_i, _p, _p, _p, _i, _i, _i, _i, _p], _i),
     "mshadow_case_random_f32": ([_i, _i, _p, _i, _f, _f, _p], _i),
+    "mshadow_case_random_f64": ([_i, _i, _p, _i, C.c_double, C.c_double, _p], _i),
     "mshadow_case_sort_by_key_32": ([_i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_case_extensions_f32": ([_i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p], _i),
     "mshadow_case_dot_f32": ([_i, _p, _p, _p, _i, _i, _i, _i, _p], _i),
@@ -325,12 +328,15 @@ class Library:
         self.check(self.dll.mshadow_hip_random_u32(dst.ptr, dst.cols, seed, subsequence, counter, stream))
 
     def random_uniform(self, dst, seed, subsequence=0, counter=0, a=0.0, b=1.0, stream=None):
-        self.check(self.dll.mshadow_hip_random_uniform_f32(dst.ptr, dst.stride, dst.rows, dst.cols, seed,
-                                                           subsequence, counter, a, b, stream))
+        """float32 or float64 buffers (the _f32 / _f64 entry point by the buffer's type)"""
+        fn = (self.dll.mshadow_hip_random_uniform_f64 if dst.dtype == np.float64
+              else self.dll.mshadow_hip_random_uniform_f32)
+        self.check(fn(dst.ptr, dst.stride, dst.rows, dst.cols, seed, subsequence, counter, a, b, stream))
 
     def random_normal(self, dst, seed, subsequence=0, counter=0, mu=0.0, sigma=1.0, stream=None):
-        self.check(self.dll.mshadow_hip_random_normal_f32(dst.ptr, dst.stride, dst.rows, dst.cols, seed,
-                                                          subsequence, counter, mu, sigma, stream))
+        fn = (self.dll.mshadow_hip_random_normal_f64 if dst.dtype == np.float64
+              else self.dll.mshadow_hip_random_normal_f32)
+        self.check(fn(dst.ptr, dst.stride, dst.rows, dst.cols, seed, subsequence, counter, mu, sigma, stream))
 
     def fill(self, dst, value, stream=None):
         """every element of a buffer of 32-bit elements set to `value`"""
@@ -494,7 +500,9 @@ class Library:
                                                  stream))
 
     def case_random(self, op, seed, out, p0=0.0, p1=1.0, stream=None):
-        self.check_case(self.cases.mshadow_case_random_f32(op, seed, out.ptr, out.cols, p0, p1, stream))
+        fn = (self.cases.mshadow_case_random_f64 if out.dtype == np.float64
+              else self.cases.mshadow_case_random_f32)
+        self.check_case(fn(op, seed, out.ptr, out.cols, p0, p1, stream))
 
     def case_sort_by_key(self, op, keys, values, is_ascend=True, stream=None):
         self.check_case(self.cases.mshadow_case_sort_by_key_32(

@@ -537,6 +537,26 @@ int mshadow_case_random_f32(int op, int seed, float *out, int n, float p0, float
   CASE_END
 }
 
+/* the same through Random<gpu, double> (ops 0-2) */
+int mshadow_case_random_f64(int op, int seed, double *out, int n, double p0, double p1, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Random<gpu, double> rnd(seed);
+  rnd.set_stream(st.get());
+  Tensor<gpu, 1, double> dst = G1(out, n, st.get());
+  if (op == 0) {
+    Tensor<gpu, 1, double> lo = dst.Slice(0, n / 2), hi = dst.Slice(n / 2, n);
+    rnd.SampleUniform(&lo, p0, p1);
+    rnd.SampleUniform(&hi, p0, p1);
+  } else if (op == 1) {
+    rnd.SampleGaussian(&dst, p0, p1);
+  } else {
+    dst = rnd.uniform(Shape1(n)) * 2.0;
+  }
+  st.get()->Wait();
+  CASE_END
+}
+
 /* op 0: SortByKey(keys, values, is_ascend); op 1: VectorizedSort(keys as the values to sort,
    values as the segment numbers). key_kind 0: float keys / int values, 1: int keys / float
    values (for op 1 the segments are int either way) */

@@ -13,6 +13,12 @@
  *   uniform  u = ((x >> 9) + 0.5) * 2^-23, strictly inside (0, 1), then u * (b - a) + a
  *   normal   Box-Muller on two uniforms: sqrt(-2 ln u1) * (cos, sin)(2 pi u2), then
  *            mu + z * sigma
+ * Double tensors (Random<gpu, double>, mshadow/random.h:486-514 of the reference:
+ * curandGenerateUniformDouble / curandGenerateNormalDouble) take two words per value:
+ *   uniform  n = word0 * 2^20 + (word1 >> 12) (52 bits), u = (n + 0.5) * 2^-52, strictly
+ *            inside (0, 1) and exact (2n + 1 has 53 bits); element e of a call comes from
+ *            block counter + e / 2, words 2 (e % 2) and 2 (e % 2) + 1
+ *   normal   the same Box-Muller in double on the block's two uniforms, a pair per block
  */
 #include <mshadow/core/fastdiv.h>
 
@@ -118,6 +124,83 @@ __global__ void __launch_bounds__(kRandomBlock)
   }
 }
 
+/*! \brief 52 bits of two words as a point strictly inside (0, 1): (n + 1/2) / 2^52 */
+__device__ __forceinline__ double UnitOpenDouble(uint32_t hi, uint32_t lo) {
+  const uint64_t n = (static_cast<uint64_t>(hi) << 20) | (lo >> 12);
+  return (static_cast<double>(n) + 0.5) * 2.220446049250313e-16;  // 2^-52
+}
+
+/*! \brief double values: a Philox block makes two of them; one thread per block. PAIRS: rows
+ *  are whole aligned pairs, which leave as one 128-bit streaming store */
+template <int KIND, bool PAIRS>
+__global__ void __launch_bounds__(kRandomBlock)
+    RandomDoubleKernel(double *dst, uint32_t stride, uint32_t total, uint32_t cols,
+                       FastDivU32 div_cols, uint64_t seed, uint64_t subsequence, uint64_t counter,
+                       double p0, double p1) {
+  const uint32_t blocks = (total + 1u) / 2u;
+  const uint32_t step = gridDim.x * kRandomBlock;
+  for (uint32_t b = blockIdx.x * kRandomBlock + threadIdx.x; b < blocks; b += step) {
+    const Philox4 r = Philox4x32_10(seed, subsequence, counter + b);
+    const double u0 = UnitOpenDouble(r.w[0], r.w[1]), u1 = UnitOpenDouble(r.w[2], r.w[3]);
+    double out[2];
+    if (KIND == kUniform) {
+      out[0] = u0 * (p1 - p0) + p0;
+      out[1] = u1 * (p1 - p0) + p0;
+    } else {
+      const double radius = sqrt(-2.0 * log(u0));
+      double sn, cs;
+      sincospi(2.0 * u1, &sn, &cs);
+      out[0] = p0 + radius * cs * p1;
+      out[1] = p0 + radius * sn * p1;
+    }
+    if (PAIRS) {
+      const uint32_t e = b * 2u;
+      const uint32_t y = div_cols.Div(e);
+      typedef double V2 __attribute__((ext_vector_type(2)));
+      V2 v;
+      v.x = out[0], v.y = out[1];
+      __builtin_nontemporal_store(
+          v, reinterpret_cast<V2 *>(dst + static_cast<size_t>(y) * stride + (e - y * cols)));
+      continue;
+    }
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const uint32_t e = b * 2u + k;
+      if (e < total) {
+        const uint32_t y = div_cols.Div(e);
+        dst[static_cast<size_t>(y) * stride + (e - y * cols)] = out[k];
+      }
+    }
+  }
+}
+
+template <int KIND>
+int LaunchRandomDouble(double *dst, int dstride, int rows, int cols, uint64_t seed,
+                       uint64_t subsequence, uint64_t counter, double p0, double p1, void *stream,
+                       const char *what) {
+  if (rows < 0 || cols < 0) return mshadow_abi::Fail(MSHADOW_HIP_ERR_ARGUMENT, std::string(what) + ": negative shape");
+  if (rows == 0 || cols == 0) return MSHADOW_HIP_OK;
+  if (dst == NULL) return mshadow_abi::Fail(MSHADOW_HIP_ERR_ARGUMENT, std::string(what) + ": NULL tensor");
+  if (dstride < cols) return mshadow_abi::Fail(MSHADOW_HIP_ERR_ARGUMENT, std::string(what) + ": pitch smaller than the row");
+  const uint64_t total = static_cast<uint64_t>(rows) * cols;
+  if (total >= (1ull << 31)) return mshadow_abi::Fail(MSHADOW_HIP_ERR_ARGUMENT, std::string(what) + ": too many elements");
+  uint64_t grid = ((total + 1) / 2 + kRandomBlock - 1) / kRandomBlock;
+  if (grid > 16384) grid = 16384;
+  const bool pairs = cols % 2 == 0 && dstride % 2 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0;
+#define MSHADOW_RANDOM_LAUNCH(PAIRS)                                                              \
+  hipLaunchKernelGGL((RandomDoubleKernel<KIND, PAIRS>), dim3(static_cast<unsigned>(grid)),        \
+                     dim3(kRandomBlock), 0, AsStream(stream), dst, static_cast<uint32_t>(dstride), \
+                     static_cast<uint32_t>(total), static_cast<uint32_t>(cols), FastDivU32(cols), \
+                     seed, subsequence, counter, p0, p1)
+  if (pairs) {
+    MSHADOW_RANDOM_LAUNCH(true);
+  } else {
+    MSHADOW_RANDOM_LAUNCH(false);
+  }
+#undef MSHADOW_RANDOM_LAUNCH
+  return AfterLaunch(what);
+}
+
 template <int KIND>
 int LaunchRandom(void *dst, int dstride, int rows, int cols, uint64_t seed, uint64_t subsequence,
                  uint64_t counter, float p0, float p1, void *stream, const char *what) {
@@ -168,6 +251,20 @@ int mshadow_hip_random_normal_f32(float *dst, int dstride, int rows, int cols, u
                                   void *stream) {
   return LaunchRandom<kNormal>(dst, dstride, rows, cols, seed, subsequence, counter, mu, sigma,
                                stream, "random_normal");
+}
+
+int mshadow_hip_random_uniform_f64(double *dst, int dstride, int rows, int cols, uint64_t seed,
+                                   uint64_t subsequence, uint64_t counter, double a, double b,
+                                   void *stream) {
+  return LaunchRandomDouble<kUniform>(dst, dstride, rows, cols, seed, subsequence, counter, a, b,
+                                      stream, "random_uniform_f64");
+}
+
+int mshadow_hip_random_normal_f64(double *dst, int dstride, int rows, int cols, uint64_t seed,
+                                  uint64_t subsequence, uint64_t counter, double mu, double sigma,
+                                  void *stream) {
+  return LaunchRandomDouble<kNormal>(dst, dstride, rows, cols, seed, subsequence, counter, mu, sigma,
+                                     stream, "random_normal_f64");
 }
 
 }  // extern "C"

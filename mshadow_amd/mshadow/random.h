@@ -158,23 +158,17 @@ class Random<gpu, DType> {
   }
   inline void GetRandInt(const Tensor<gpu, 1, unsigned> &dst) {
     MSHADOW_HIP_CALL(mshadow_hip_random_u32(dst.dptr_, dst.size(0), seed_, 0, counter_, Raw()));
-    Advance(dst.size(0));
+    Advance((static_cast<size_t>(dst.size(0)) + 3) / 4);
   }
   template <int dim>
   inline void SampleUniform(Tensor<gpu, dim, DType> *dst, DType a = 0.0f, DType b = 1.0f) {
-    RequireFloat();
     const Shape<2> s = dst->shape_.FlatTo2D();
-    MSHADOW_HIP_CALL(mshadow_hip_random_uniform_f32(dst->dptr_, dst->stride_, s[0], s[1], seed_, 0,
-                                                    counter_, a, b, Raw()));
-    Advance(dst->shape_.Size());
+    Advance(Draw(0, dst->dptr_, dst->stride_, s[0], s[1], a, b));
   }
   template <int dim>
   inline void SampleGaussian(Tensor<gpu, dim, DType> *dst, DType mu = 0.0f, DType sigma = 1.0f) {
-    RequireFloat();
     const Shape<2> s = dst->shape_.FlatTo2D();
-    MSHADOW_HIP_CALL(mshadow_hip_random_normal_f32(dst->dptr_, dst->stride_, s[0], s[1], seed_, 0,
-                                                   counter_, mu, sigma, Raw()));
-    Advance(dst->shape_.Size());
+    Advance(Draw(1, dst->dptr_, dst->stride_, s[0], s[1], mu, sigma));
   }
   /*! \brief normal values of the given shape, valid until the next call */
   template <int dim>
@@ -195,10 +189,34 @@ class Random<gpu, DType> {
 
  private:
   inline void *Raw() { return Stream<gpu>::GetStream(stream_); }
-  inline void Advance(size_t elements) { counter_ += (elements + 3) / 4; }
-  inline static void RequireFloat() {
-    CHECK((std::is_same<DType, float>::value)) << "Random<gpu>: float tensors only";
+  inline void Advance(size_t blocks) { counter_ += blocks; }
+  /*! \brief kind 0 uniform (p0, p1), 1 normal (mean p0, deviation p1); returns the generator
+   *  blocks the call consumed: four floats or two doubles come out of one */
+  inline size_t Draw(int kind, float *dst, index_t stride, index_t rows, index_t cols, float p0,
+                     float p1) {
+    if (kind == 0) {
+      MSHADOW_HIP_CALL(mshadow_hip_random_uniform_f32(dst, stride, rows, cols, seed_, 0, counter_,
+                                                      p0, p1, Raw()));
+    } else {
+      MSHADOW_HIP_CALL(mshadow_hip_random_normal_f32(dst, stride, rows, cols, seed_, 0, counter_,
+                                                     p0, p1, Raw()));
+    }
+    return (static_cast<size_t>(rows) * cols + 3) / 4;
   }
+  inline size_t Draw(int kind, double *dst, index_t stride, index_t rows, index_t cols, double p0,
+                     double p1) {
+    if (kind == 0) {
+      MSHADOW_HIP_CALL(mshadow_hip_random_uniform_f64(dst, stride, rows, cols, seed_, 0, counter_,
+                                                      p0, p1, Raw()));
+    } else {
+      MSHADOW_HIP_CALL(mshadow_hip_random_normal_f64(dst, stride, rows, cols, seed_, 0, counter_,
+                                                     p0, p1, Raw()));
+    }
+    return (static_cast<size_t>(rows) * cols + 1) / 2;
+  }
+  static_assert(std::is_same<DType, float>::value || std::is_same<DType, double>::value,
+                "Random<gpu, DType>: float and double, the types the reference's generator "
+                "library serves (mshadow/random.h:486-514)");
   Stream<gpu> *stream_;
   uint64_t seed_;
   uint64_t counter_;

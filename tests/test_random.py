@@ -73,6 +73,25 @@ def test_unit_interval_transform_stays_strictly_inside():
     assert old.max() == f32(1.0)        # what this replaces
 
 
+def unit_open_double(words):
+    """two words per value: 52 bits, (n + 1/2) / 2^52 - exact in float64 (2n + 1 has 53 bits)"""
+    w = words.astype(np.uint64)
+    n = (w[0::2] << np.uint64(20)) | (w[1::2] >> np.uint64(12))
+    return (n.astype(np.float64) + 0.5) * 2.0 ** -52
+
+
+def test_double_unit_interval_transform_is_exact_and_strictly_inside():
+    w = np.array([0, 0, 0, 0xFFF, 0, 0x1000, 0xFFFFFFFF, 0xFFFFFFFF, 0x80000000, 0], np.uint32)
+    u = unit_open_double(w)
+    assert u[0] == 2.0 ** -53 and u[1] == 2.0 ** -53 and u[2] == 1.5 * 2.0 ** -52
+    assert u[3] == 1.0 - 2.0 ** -53 and u[4] == 0.5 + 2.0 ** -53
+    assert np.all(u > 0) and np.all(u < 1)
+    # exactness: the same values from integers
+    from fractions import Fraction
+    n = [(int(w[2 * i]) << 20) | (int(w[2 * i + 1]) >> 12) for i in range(5)]
+    assert [Fraction(float(x)) for x in u] == [Fraction(2 * k + 1, 2 ** 53) for k in n]
+
+
 # ---------------------------------------------------------------- CPU
 @pytest.fixture(scope="module")
 def host_lib(tmp_path_factory):
@@ -193,6 +212,59 @@ def test_random_gpu_object_advances_and_rewinds(G):
     ints = G.buffer((n,), np.uint32)
     G.case_random(3, -1, ints)      # a negative seed is sign-extended to 64 bits
     assert np.array_equal(ints.download(), model_words(2**64 - 1, 0, 0, n))
+    G.case_random(1, seed, out, 0.0, 1.0)
+    z = out.download()
+    assert abs(z.mean()) < 0.05 and abs(z.std() - 1.0) < 0.05
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape,pad", [((1000,), 0), ((37, 29), 0), ((37, 29), 3), ((37, 30), 0), ((4, 5, 6), 2)])
+def test_gpu_double_uniform_is_the_stated_transform(G, shape, pad):
+    seed, ctr, a, b = 99, 2**64 - 2, -1.5, 2.25         # the counter wraps inside the call
+    n = int(np.prod(shape))
+    out = G.buffer(shape, np.float64, pad=pad, fill=0)
+    G.random_uniform(out, seed, 3, ctr, a, b)
+    want = unit_open_double(model_words(seed, 3, ctr, 2 * n + 2))[:n] * (b - a) + a
+    got = out.download().ravel()
+    assert np.array_equal(got.view(np.uint64), want.view(np.uint64))
+    assert got.min() > a and got.max() < b
+
+
+@pytest.mark.gpu
+def test_gpu_double_normal_matches_box_muller_and_its_moments(G):
+    seed, ctr, n = 5, 0, 1 << 20
+    out = G.buffer((n,), np.float64)
+    G.random_normal(out, seed, 0, ctr, 1.0, 2.0)
+    got = out.download()
+    u = unit_open_double(model_words(seed, 0, ctr, 2 * n))
+    r = np.sqrt(-2.0 * np.log(u[0::2]))
+    z = np.empty(n)
+    z[0::2] = r * np.cos(2 * np.pi * u[1::2])
+    z[1::2] = r * np.sin(2 * np.pi * u[1::2])
+    want = 1.0 + z * 2.0
+    # double library functions on both sides; cos / sin near their zeros lose relative, not
+    # absolute, accuracy
+    assert np.max(np.abs(got - want)) < 1e-13
+    assert abs(got.mean() - 1.0) < 0.01 and abs(got.std() - 2.0) < 0.01
+    assert abs(((got - 1.0) / 2.0 > 1.96).mean() - 0.025) < 0.002
+
+
+@pytest.mark.gpu
+def test_random_gpu_double_object_advances_and_rewinds(G):
+    """Random<gpu, double>: two values per generator block; consecutive calls continue the
+    stream, the expression form starts from the object's seed"""
+    n, seed = 10001, 42
+    out = G.buffer((n,), np.float64)
+    G.case_random(0, seed, out, -1.0, 1.0)
+    got = out.download()
+    h = n // 2
+    blocks_first = (h + 1) // 2
+    words = model_words(seed, 0, 0, 4 * blocks_first + 2 * (n - h) + 2)
+    first = unit_open_double(words[: 4 * blocks_first])[:h] * 2.0 - 1.0
+    second = unit_open_double(words[4 * blocks_first:])[: n - h] * 2.0 - 1.0
+    assert np.array_equal(got[:h], first) and np.array_equal(got[h:], second)
+    G.case_random(2, seed, out)
+    assert np.array_equal(out.download(), unit_open_double(model_words(seed, 0, 0, 2 * n + 2))[:n] * 2.0)
     G.case_random(1, seed, out, 0.0, 1.0)
     z = out.download()
     assert abs(z.mean()) < 0.05 and abs(z.std() - 1.0) < 0.05
