@@ -128,6 +128,10 @@ int mshadow_case_random_f64(int op, int seed, double *out, int n, double p0, dou
    key_kind 0: float keys with int values, 1: int keys with float values (int segments for op 1) */
 int mshadow_case_sort_by_key_32(int op, void *keys, int key_kind, void *values, int n,
                                 int is_ascend, void *stream);
+/* SortByKey for keys and values of any type of the type switch (mshadow::TypeFlag codes:
+   0 float, 1 double, 2 half_t, 3 uint8, 4 int32, 5 int8, 6 int64) */
+int mshadow_case_sort_by_key_any(int key_flag, int value_flag, void *keys, void *values, int n,
+                                 int is_ascend, void *stream);
 
 /* chpool / ch_unpool, reduce_with_axis / reduce_keepdim, broadcast_with_axis /
    broadcast_keepdim, transpose / transpose_indices, concat / slice / flip (also as the

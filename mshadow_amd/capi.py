@@ -122,6 +122,7 @@ CASES_SYMBOLS = {
     "mshadow_case_rows_by_index_any": ([_i, _i, _i, _p, _i, _i, _p, _p, _i, _p, _i, _i, _i, _p], _i),
     "mshadow_case_shaping_f32": ([_i, _p, _p, _p, _i, _i, _i, _i, _p], _i),
     "mshadow_case_random_f32": ([_i, _i, _p, _i, _f, _f, _p], _i),
+    "mshadow_case_sort_by_key_any": ([_i, _i, _p, _p, _i, _i, _p], _i),
     "mshadow_case_random_f64": ([_i, _i, _p, _i, C.c_double, C.c_double, _p], _i),
     "mshadow_case_sort_by_key_32": ([_i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_case_extensions_f32": ([_i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p], _i),
@@ -471,6 +472,13 @@ class Library:
             op, self.TYPE_FLAG[dst.dtype.name], self.TYPE_FLAG[index.dtype.name], dst.ptr, dst.stride,
             dst.rows, sorted_rows.ptr if sorted_rows is not None else None, index.ptr, index.cols,
             src.ptr, src.stride, src.rows, src.cols, stream))
+
+    def case_sort_by_key_any(self, keys, values, is_ascend=True, stream=None):
+        """SortByKey on buffers of any element type of the type switch"""
+        flag = dict(self.TYPE_FLAG, uint8=3, int8=5)
+        self.check_case(self.cases.mshadow_case_sort_by_key_any(
+            flag[keys.dtype.name], flag[values.dtype.name], keys.ptr, values.ptr, keys.cols,
+            1 if is_ascend else 0, stream))
 
     def case_shaping(self, op, out, a, v, n, c, h, w, stream=None):
         self.check_case(self.cases.mshadow_case_shaping_f32(op, out.ptr, a.ptr, v.ptr, n, c, h, w,

@@ -580,6 +580,21 @@ int mshadow_case_sort_by_key_32(int op, void *keys, int key_kind, void *values, 
   CASE_END
 }
 
+/* SortByKey(keys, values, is_ascend) for keys and values of any type of the type switch
+   (mshadow::TypeFlag codes: 0 float, 1 double, 2 half_t, 3 uint8, 4 int32, 5 int8, 6 int64) */
+int mshadow_case_sort_by_key_any(int key_flag, int value_flag, void *keys, void *values, int n,
+                                 int is_ascend, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  MSHADOW_TYPE_SWITCH(key_flag, KDType, {
+    MSHADOW_TYPE_SWITCH(value_flag, VDType, {
+      SortByKey(G1(static_cast<KDType *>(keys), n, st.get()),
+                G1(static_cast<VDType *>(values), n, st.get()), is_ascend != 0);
+    });
+  });
+  CASE_END
+}
+
 /* caller-side functor of the extension cases (local response normalisation squares its input) */
 struct square_of {
   MSHADOW_XINLINE static float Map(float a) { return a * a; }

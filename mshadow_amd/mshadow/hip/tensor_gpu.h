@@ -27,6 +27,7 @@
 #include "./kernels/reduce.h"
 #include "./kernels/rows_by_index.h"
 #include "./kernels/softmax_any.h"
+#include "./kernels/sort_any.h"
 #endif
 
 namespace mshadow {
@@ -511,10 +512,118 @@ template <>
 struct SortKeyKind<int32_t> { static const int value = MSHADOW_HIP_KEY_I32; };
 template <>
 struct SortKeyKind<uint32_t> { static const int value = MSHADOW_HIP_KEY_U32; };
+/*! \brief the device sort for key / value types the library's 32-bit entry point does not
+ *  take: through a permutation, one stable 32-bit pass per key word (kernels/sort_any.h) */
+template <typename KDType, typename VDType>
+inline void SortByKeyThroughPermutation(Tensor<gpu, 1, KDType> keys, Tensor<gpu, 1, VDType> values,
+                                        bool is_ascend) {
+#if defined(__HIPCC__)
+  const size_t n = keys.size(0);
+  CHECK_LT(n, 1ull << 31) << "SortByKey: too many elements";
+  void *stream = Stream<gpu>::GetStream(keys.stream_);
+  size_t sort_bytes = 0, pitch = 0;
+  MSHADOW_HIP_CALL(mshadow_hip_sort_by_key_workspace(n, &sort_bytes));
+  /* words | permutation | copy of the keys | copy of the values | the sort's scratch, each
+     part starting on a multiple of 256 bytes */
+  const size_t part = 256;
+  const size_t words_at = 0;
+  const size_t perm_at = words_at + (n * 4 + part - 1) / part * part;
+  const size_t keys_at = perm_at + (n * 4 + part - 1) / part * part;
+  const size_t vals_at = keys_at + (n * sizeof(KDType) + part - 1) / part * part;
+  const size_t sort_at = vals_at + (n * sizeof(VDType) + part - 1) / part * part;
+  void *block = NULL;
+  MSHADOW_HIP_CALL(mshadow_hip_malloc_pitch(&block, &pitch, sort_at + sort_bytes, 1));
+  char *base = static_cast<char *>(block);
+  uint32_t *words = reinterpret_cast<uint32_t *>(base + words_at);
+  uint32_t *perm = reinterpret_cast<uint32_t *>(base + perm_at);
+  KDType *keys_copy = reinterpret_cast<KDType *>(base + keys_at);
+  VDType *vals_copy = reinterpret_cast<VDType *>(base + vals_at);
+  uint32_t count = static_cast<uint32_t>(n);
+  uint32_t blocks = (count + hip::kSortAnyBlock - 1) / hip::kSortAnyBlock;
+  if (blocks > 65536u) blocks = 65536u;
+  const uint32_t grid[3] = {blocks, 1, 1};
+  const uint32_t block_dim[3] = {static_cast<uint32_t>(hip::kSortAnyBlock), 1, 1};
+  const KDType *key_src = keys.dptr_;
+  const uint32_t *no_perm = NULL;
+  const uint32_t *cur_perm = perm;
+  {  // low word of every key, and the identity permutation
+    void *args[] = {&words, &perm, &key_src, &no_perm, &count};
+    MSHADOW_HIP_CALL(mshadow_hip_launch(
+        reinterpret_cast<const void *>(hip::SortKeyWordKernel<KDType, false>), grid, block_dim, args,
+        0, stream));
+  }
+  MSHADOW_HIP_CALL(mshadow_hip_sort_by_key_32(words, MSHADOW_HIP_KEY_U32, perm, n, is_ascend ? 1 : 0,
+                                              base + sort_at, sort_bytes, stream));
+  if (sizeof(KDType) > 4) {  // then, stably, by the high word of the keys in their new order
+    void *args[] = {&words, &perm, &key_src, &cur_perm, &count};
+    MSHADOW_HIP_CALL(mshadow_hip_launch(
+        reinterpret_cast<const void *>(hip::SortKeyWordKernel<KDType, true>), grid, block_dim, args, 0,
+        stream));
+    MSHADOW_HIP_CALL(mshadow_hip_sort_by_key_32(words, MSHADOW_HIP_KEY_U32, perm, n,
+                                                is_ascend ? 1 : 0, base + sort_at, sort_bytes,
+                                                stream));
+  }
+  MSHADOW_HIP_CALL(mshadow_hip_memcpy2d_async(keys_copy, n * sizeof(KDType), keys.dptr_,
+                                              n * sizeof(KDType), n * sizeof(KDType), 1,
+                                              MSHADOW_HIP_D2D, stream));
+  MSHADOW_HIP_CALL(mshadow_hip_memcpy2d_async(vals_copy, n * sizeof(VDType), values.dptr_,
+                                              n * sizeof(VDType), n * sizeof(VDType), 1,
+                                              MSHADOW_HIP_D2D, stream));
+  {
+    KDType *out = keys.dptr_;
+    const KDType *in = keys_copy;
+    void *args[] = {&out, &in, &cur_perm, &count};
+    MSHADOW_HIP_CALL(mshadow_hip_launch(reinterpret_cast<const void *>(hip::SortGatherKernel<KDType>),
+                                        grid, block_dim, args, 0, stream));
+  }
+  {
+    VDType *out = values.dptr_;
+    const VDType *in = vals_copy;
+    void *args[] = {&out, &in, &cur_perm, &count};
+    MSHADOW_HIP_CALL(mshadow_hip_launch(reinterpret_cast<const void *>(hip::SortGatherKernel<VDType>),
+                                        grid, block_dim, args, 0, stream));
+  }
+  MSHADOW_HIP_CALL(mshadow_hip_stream_sync(stream));
+  MSHADOW_HIP_CALL(mshadow_hip_free(block));
+#else
+  LOG(FATAL) << "SortByKey<gpu> of these element types: compile the calling translation unit with hipcc";
+#endif
+}
+/*! \brief 32-bit float / integer keys with 32-bit values go to the library as they are */
+template <typename KDType, typename VDType,
+          bool DIRECT = (SortKeyKind<KDType>::value >= 0 && sizeof(VDType) == 4)>
+struct SortRoute {
+  inline static void Run(Tensor<gpu, 1, KDType> keys, Tensor<gpu, 1, VDType> values, bool is_ascend) {
+    SortByKeyThroughPermutation(keys, values, is_ascend);
+  }
+};
+template <typename KDType, typename VDType>
+struct SortRoute<KDType, VDType, true> {
+  inline static void Run(Tensor<gpu, 1, KDType> keys, Tensor<gpu, 1, VDType> values, bool is_ascend) {
+    const size_t n = keys.size(0);
+    void *stream = Stream<gpu>::GetStream(keys.stream_);
+    size_t bytes = 0, pitch = 0;
+    void *workspace = NULL;
+    MSHADOW_HIP_CALL(mshadow_hip_sort_by_key_workspace(n, &bytes));
+    MSHADOW_HIP_CALL(mshadow_hip_malloc_pitch(&workspace, &pitch, bytes, 1));
+    MSHADOW_HIP_CALL(mshadow_hip_sort_by_key_32(keys.dptr_, SortKeyKind<KDType>::value, values.dptr_, n,
+                                                is_ascend ? 1 : 0, workspace, bytes, stream));
+    MSHADOW_HIP_CALL(mshadow_hip_stream_sync(stream));
+    MSHADOW_HIP_CALL(mshadow_hip_free(workspace));
+  }
+};
+template <typename VDType>
+struct SortRoute<half::half_t, VDType, false> {
+  inline static void Run(Tensor<gpu, 1, half::half_t>, Tensor<gpu, 1, VDType>, bool) {
+    LOG(FATAL) << "SortByKey is not supported for half_t keys";   // as in the reference
+  }
+};
 }  // namespace gpu_detail
 /*! \brief stable sort by key on the device (the reference: thrust::stable_sort_by_key,
  *  tensor_gpu-inl.cuh:784-806, which takes its scratch memory from the runtime as this does;
- *  half_t keys or values are as fatal here as there). Returns once the sort has finished. */
+ *  half_t keys are as fatal here as there). Keys of any integer or floating type with any
+ *  value type; 32-bit keys with 32-bit values are sorted in place by the library, everything
+ *  else through a permutation. Returns once the sort has finished. */
 template <typename KDType, typename VDType>
 inline void SortByKey(Tensor<gpu, 1, KDType> keys, Tensor<gpu, 1, VDType> values,
                       bool is_ascend) {
@@ -523,20 +632,8 @@ inline void SortByKey(Tensor<gpu, 1, KDType> keys, Tensor<gpu, 1, VDType> values
   CHECK_EQ(keys.size(0), values.size(0))
       << "The sizes of key/value are not equal! keys_size: " << keys.size(0)
       << "values_size: " << values.size(0);
-  CHECK(gpu_detail::SortKeyKind<KDType>::value >= 0 && sizeof(VDType) == 4)
-      << "SortByKey<gpu>: implemented for 32-bit float / integer keys and 32-bit values";
-  const size_t n = keys.size(0);
-  if (n == 0) return;
-  void *stream = Stream<gpu>::GetStream(keys.stream_);
-  size_t bytes = 0, pitch = 0;
-  void *workspace = NULL;
-  MSHADOW_HIP_CALL(mshadow_hip_sort_by_key_workspace(n, &bytes));
-  MSHADOW_HIP_CALL(mshadow_hip_malloc_pitch(&workspace, &pitch, bytes, 1));
-  MSHADOW_HIP_CALL(mshadow_hip_sort_by_key_32(keys.dptr_, gpu_detail::SortKeyKind<KDType>::value,
-                                              values.dptr_, n, is_ascend ? 1 : 0, workspace, bytes,
-                                              stream));
-  MSHADOW_HIP_CALL(mshadow_hip_stream_sync(stream));
-  MSHADOW_HIP_CALL(mshadow_hip_free(workspace));
+  if (keys.size(0) == 0) return;
+  gpu_detail::SortRoute<KDType, VDType>::Run(keys, values, is_ascend);
 }
 
 /* ------------------------------------------------------------------ expression routing */

@@ -370,6 +370,16 @@ void ref_sort_by_key_32(void *keys, int key_kind, void *values, int n, int is_as
               Tensor<cpu, 1, float>(static_cast<float *>(values), Shape1(n)), is_ascend != 0);
   }
 }
+/* the reference's SortByKey<cpu> for any key / value type of its type switch */
+void ref_sort_by_key_any(int key_flag, int value_flag, void *keys, void *values, int n,
+                         int is_ascend) {
+  MSHADOW_TYPE_SWITCH(key_flag, KDType, {
+    MSHADOW_TYPE_SWITCH(value_flag, VDType, {
+      SortByKey(Tensor<cpu, 1, KDType>(static_cast<KDType *>(keys), Shape1(n)),
+                Tensor<cpu, 1, VDType>(static_cast<VDType *>(values), Shape1(n)), is_ascend != 0);
+    });
+  });
+}
 void ref_vectorized_sort_32(void *values, int value_kind, void *segments, int n) {
   Tensor<cpu, 1, int> seg(static_cast<int *>(segments), Shape1(n));
   if (value_kind == 0) VectorizedSort(Tensor<cpu, 1, float>(static_cast<float *>(values), Shape1(n)), seg);

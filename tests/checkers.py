@@ -96,6 +96,7 @@ class Checker:
         self._fn("sort_by_key_32", [_p, _i, _p, _i, _i])
         self._fn("vectorized_sort_32", [_p, _i, _p, _i])
         if self.prefix == "ref":
+            self._fn("sort_by_key_any", [_i, _i, _p, _p, _i, _i])
             self._fn("shaping_f32", [_i, _p, _p, _p, _i, _i, _i, _i])
             self._fn("extensions_f32", [_i, _p, _p, _p, _p] + [_i] * 7)
             self._fn("random_f32", [_i, _i, _p, _i, _f, _f])
@@ -252,6 +253,13 @@ class Checker:
     @staticmethod
     def _key_kind(keys):
         return {"float32": 0, "int32": 1, "uint32": 2}[keys.dtype.name]
+
+    def sort_by_key_any(self, keys, values, is_ascend=True):
+        """the reference's SortByKey<cpu> on arrays of any type of its type switch (ref only)"""
+        flag = dict(self.TYPE_FLAG, uint8=3, int8=5)
+        self._sort_by_key_any(flag[keys.dtype.name], flag[values.dtype.name], ptr(keys), ptr(values),
+                              keys.shape[0], 1 if is_ascend else 0)
+        return keys, values
 
     def sort_by_key(self, keys, values, is_ascend=True):
         """in place on two contiguous 1-D arrays of 32-bit elements"""

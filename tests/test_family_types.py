@@ -288,3 +288,65 @@ def test_gpu_rows_by_index(G, orc, stream, dtype, itype, op):
                                  G.to_device(index), G.to_device(src, pad), stream)
         got = d.download(stream)
         assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (k_rows, n_index, cols)
+
+
+# ------------------------------------------------------------------ SortByKey, any types
+def stable_order(keys, ascend):
+    """positions in the order std::stable_sort gives under `<` (ascending) or `>` (descending):
+    by key, equal keys (-0.0 and +0.0 are equal) in their original order"""
+    _, rank = np.unique(keys, return_inverse=True)
+    return np.lexsort((np.arange(keys.shape[0]), rank if ascend else -rank))
+
+
+def sort_case(seed, ktype, vtype, n):
+    rng = np.random.default_rng(seed)
+    if np.issubdtype(ktype, np.floating):
+        keys = np.round(rng.standard_normal(n) * 4, 1).astype(ktype)    # many repeated keys
+        keys[rng.integers(0, n, max(n // 50, 1))] = -0.0
+        keys[rng.integers(0, n, max(n // 50, 1))] = 0.0
+        if n > 10:
+            keys[:4] = [np.inf, -np.inf, np.finfo(ktype).max, np.finfo(ktype).tiny]
+    else:
+        info = np.iinfo(ktype)
+        keys = rng.integers(max(info.min, -300), min(info.max, 300), n, endpoint=True).astype(ktype)
+        if n > 10:
+            keys[:2] = [info.min, info.max]
+    wrap = {1: 251, 2: 2039}.get(np.dtype(vtype).itemsize, n + 1)   # values the narrow types hold exactly
+    values = (np.arange(n) % wrap).astype(vtype)
+    return keys, values
+
+
+SORT_TYPES = [(f64, np.int32), (np.int64, f32), (f64, f64), (np.int64, np.uint8), (np.uint8, np.int64),
+              (np.int8, f32), (f32, f64), (np.int32, f16), (f32, np.int32)]
+
+
+@pytest.mark.skipif(not have_ref(), reason="reference build absent")
+@pytest.mark.parametrize("ktype,vtype", SORT_TYPES)
+@pytest.mark.parametrize("ascend", [True, False])
+def test_stable_order_model_is_what_the_reference_sorts(ref, ktype, vtype, ascend):
+    keys, values = sort_case(61, ktype, vtype, 3000)
+    order = stable_order(keys, ascend)
+    k, v = ref.sort_by_key_any(keys.copy(), values.copy(), ascend)
+    assert np.array_equal(k.view(np.uint8), keys[order].view(np.uint8))
+    assert np.array_equal(v.view(np.uint8), values[order].view(np.uint8))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("ktype,vtype", SORT_TYPES)
+@pytest.mark.parametrize("ascend", [True, False])
+@pytest.mark.parametrize("n", [1, 2, 777, 100000])
+def test_gpu_sort_by_key_any_types(G, stream, ktype, vtype, ascend, n):
+    keys, values = sort_case(62 + n, ktype, vtype, n)
+    order = stable_order(keys, ascend)
+    dk, dv = G.to_device(keys), G.to_device(values)
+    G.case_sort_by_key_any(dk, dv, ascend, stream)
+    assert np.array_equal(dk.download(stream).view(np.uint8), keys[order].view(np.uint8))
+    assert np.array_equal(dv.download(stream).view(np.uint8), values[order].view(np.uint8))
+
+
+@pytest.mark.gpu
+def test_gpu_sort_by_half_keys_is_refused_like_the_reference(G, stream):
+    from mshadow_amd.capi import HipError
+    dk, dv = G.to_device(np.ones(8, f16)), G.to_device(np.arange(8, dtype=np.int32))
+    with pytest.raises(HipError, match="half_t"):
+        G.case_sort_by_key_any(dk, dv, True, stream)
