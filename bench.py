@@ -109,8 +109,8 @@ TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "hotpath_step_all_kernels_hbm_t
 TRAFFIC_ROW_OF_OP = {
     "map_fused": "map_fused", "sumall_except_dim1": "ReduceKeepHighDimDmaKernel",
     "sum_rows": "ReduceKeepLowestDmaKernel", "softmax": "SoftmaxRowKernel",
-    "softmax_grad": "SoftmaxGradKernel", "pool_max": "PoolKernel", "unpool_max": "UnpoolBlockKernel",
-    "im2col_f16": "Im2ColHalfRow3Kernel", "col2im_f16": "Col2ImHalfPairKernel",
+    "softmax_grad": "SoftmaxGradKernel", "pool_max": "PoolKernel", "unpool_max": "UnpoolRows3x3s2Kernel",
+    "im2col_f16": "Im2ColHalfRow3Kernel", "col2im_f16": "Col2ImHalfRows3x3Kernel",
 }
 
 
@@ -176,7 +176,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--scale", type=int, default=1, help="shrink leading dims (functional runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-reps", type=int, default=3)
+    ap.add_argument("--cpu-reps", type=int, default=30)
     ap.add_argument("--only", default="", help="comma list of ops to run (profiling aid); "
                     "softmax_phases, ceiling_chain and ceiling_lds_loads run the probes of "
                     "libmshadow_probe.so instead")
@@ -450,11 +450,13 @@ def run_probe(G, which):
     if which == "ceiling_chain":
         out = {"probe": "ceiling_chain", "unit": "ns per dependent float32 add, one wave",
                "compute_units": cus, "modes": {}}
-        for mode in ("register", "lds", "lanes"):
+        for mode in ("register", "register_f16", "lds", "lanes"):
             out["modes"][mode] = {f"{wg} workgroups": round(P.add_chain_ns(mode, wg, s), 3)
                                   for wg in (1, cus, 4 * cus)}
         lds = out["modes"]["lds"]
         out["sum_rows_floor_us"] = {k: round(16384 * v * 1e-3, 1) for k, v in lds.items()}
+        out["sum_rows_f16_floor_us"] = {k: round(16384 * v * 1e-3, 1)
+                                        for k, v in out["modes"]["register_f16"].items()}
     elif which == "ceiling_lds_loads":
         src = G.to_device(np.ones((16384, 4096), f32))
         mb = 16384 * 4096 * 4 / 1e6

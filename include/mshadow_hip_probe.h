@@ -21,6 +21,7 @@ const char *mshadow_probe_last_error(void);
                                           128-bit LDS reads fetched 32 adds ahead */
 #define MSHADOW_PROBE_CHAIN_LANES 2    /* the softmax row sum's chain: the sum handed to the
                                           next lane by a DPP add */
+#define MSHADOW_PROBE_CHAIN_REGISTER_F16 3 /* s = s + a on binary16 values (a half_t sum) */
 int mshadow_probe_add_chain(int mode, int workgroups, double *ns_per_add, void *stream);
 
 /* The softmax kernel for rows of 16385..32768 columns (one 512-thread workgroup per row, the

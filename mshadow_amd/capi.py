@@ -639,7 +639,7 @@ class Probe:
                    "certain chunks quantised", "lists of the other chunks written",
                    "every wave's chunks done (barrier)", "row's list of addends assembled (barrier)",
                    "chain (wave 0; barrier)", "divided and stored (stores completed)")
-    CHAIN_MODES = {"register": 0, "lds": 1, "lanes": 2}
+    CHAIN_MODES = {"register": 0, "lds": 1, "lanes": 2, "register_f16": 3}
 
     def __init__(self):
         path = os.path.join(os.path.dirname(HIP_SO), "libmshadow_probe.so")

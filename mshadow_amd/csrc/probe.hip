@@ -70,6 +70,22 @@ __global__ void __launch_bounds__(64) RegisterChainKernel(float *out, float a, i
   out[blockIdx.x * 64 + threadIdx.x] = s;
 }
 
+/*! \brief the same with binary16 values: one 16-bit add per step, which is what a half_t
+ *  `sum += term` amounts to (widen, add in float, round back: one rounding of the exact sum) */
+__global__ void __launch_bounds__(64) RegisterChainHalfKernel(float *out, float a, int iters) {
+  _Float16 s = static_cast<_Float16>(static_cast<float>(threadIdx.x));
+  _Float16 addend = static_cast<_Float16>(a);
+  asm volatile("" : "+v"(addend));
+  for (int i = 0; i < iters; ++i) {
+#pragma unroll
+    for (int k = 0; k < 32; ++k) {
+      s = s + addend;
+      asm volatile("" : "+v"(s));
+    }
+  }
+  out[blockIdx.x * 64 + threadIdx.x] = static_cast<float>(s);
+}
+
 /*! \brief the chain of the column reduction: 16 lanes fold `count` floats each from LDS,
  *  four per 128-bit read, the next 32 operands fetched while 32 adds execute */
 __global__ void __launch_bounds__(64) LdsChainKernel(float *out, int iters, int count) {
@@ -239,6 +255,12 @@ int mshadow_probe_add_chain(int mode, int workgroups, double *ns_per_add, void *
     adds = 32.0 * iters;
     st = TimeKernel(s, &ms, [&] {
       hipLaunchKernelGGL(RegisterChainKernel, dim3(workgroups), dim3(64), 0, s, out, 1.5f, iters);
+    });
+  } else if (mode == MSHADOW_PROBE_CHAIN_REGISTER_F16) {
+    const int iters = 4096;
+    adds = 32.0 * iters;
+    st = TimeKernel(s, &ms, [&] {
+      hipLaunchKernelGGL(RegisterChainHalfKernel, dim3(workgroups), dim3(64), 0, s, out, 0.25f, iters);
     });
   } else if (mode == MSHADOW_PROBE_CHAIN_LDS) {
     const int iters = 128, count = 1024;
