@@ -624,7 +624,7 @@ int mshadow_hip_reduce_keep_highdim_f32(float *dst, const float *src, int sstrid
                      static_cast<uint32_t>(x), div_x, scale)
 #define HIGHDIM_LAUNCH(SEGS)                                                                   \
   if (large)                                                                                   \
-    hipLaunchKernelGGL((mshadow::hip::ReduceKeepHighDimDmaKernel<S, R, SEGS>), dim3(c),        \
+    hipLaunchKernelGGL((mshadow::hip::ReduceKeepHighDimDmaKernel<S, R, float, SEGS>), dim3(c),        \
                        dim3(mshadow::hip::kDmaThreads), 0, s, dst, src,                        \
                        static_cast<uint32_t>(sstride), static_cast<uint32_t>(n),               \
                        static_cast<uint32_t>(c), static_cast<uint32_t>(y),                     \

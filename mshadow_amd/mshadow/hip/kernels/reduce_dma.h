@@ -57,8 +57,9 @@ typedef DmaRing<8, 4096> HighDimRing;
 /*! \brief cache policy of the loads: non-temporal (the data passes through once; measured
  *  38 us against 43 us for the (64,256,56,56) reduction) */
 const int kDmaCachePolicy = 2;
-/*! \brief lane l of the wave fetches *gsrc_of_lane into lds_wave_base[l] */
-__device__ __forceinline__ void LoadDwordToLds(const float *gsrc_of_lane, float *lds_wave_base) {
+/*! \brief lane l of the wave fetches the 4 bytes at gsrc_of_lane into the l-th dword behind
+ *  lds_wave_base */
+__device__ __forceinline__ void LoadDwordToLds(const void *gsrc_of_lane, void *lds_wave_base) {
   __builtin_amdgcn_global_load_lds(
       (const __attribute__((address_space(1))) void *)gsrc_of_lane,
       (__attribute__((address_space(3))) void *)lds_wave_base, 4, 0, kDmaCachePolicy);
@@ -144,16 +145,22 @@ __global__ void __launch_bounds__(kDmaThreads)
  * segments (n values) side by side in a slot, TL = 4096 / SEGS elements of each per
  * stage, one chain lane per segment. One load instruction fetches 64 consecutive
  * elements of one segment into their place in the slot. */
-template <typename Saver, typename Reducer, int SEGS>
+/* The element type is float or a 16-bit type: a load moves a dword per lane, i.e. one float or
+ * two neighbouring 16-bit elements, which must then lie in one row of the source (n_x and the
+ * pitch even, the base 4-byte aligned: the launcher's business). */
+template <typename Saver, typename Reducer, typename DType, int SEGS>
 __global__ void __launch_bounds__(kDmaThreads)
-    ReduceKeepHighDimDmaKernel(float *dst, const float *src, uint32_t stride, uint32_t n_out,
+    ReduceKeepHighDimDmaKernel(DType *dst, const DType *src, uint32_t stride, uint32_t n_out,
                                uint32_t n_keep, uint32_t n_y, uint32_t n_x, FastDivU32 div_x,
-                               float scale) {
+                               DType scale) {
   typedef HighDimRing Ring;
   const int kDmaSlots = Ring::kSlots, kDmaAhead = Ring::kAhead, kDmaPerWave = Ring::kPerWave;
-  const int TL = Ring::kElems / SEGS;
-  const int LD = TL + 4;  // chain lanes read 16-byte words LD floats apart: no bank conflicts
-  __shared__ MSHADOW_ALIGNED(16) float ring[Ring::kSlots][SEGS * LD];
+  const int EPD = 4 / sizeof(DType);       // elements per dword
+  const int TL = Ring::kElems * EPD / SEGS;
+  const int LD = TL + 16 / sizeof(DType);  // chain lanes read words LD elements apart: no bank conflicts
+  static_assert(sizeof(DType) == 4 || sizeof(DType) == 2, "a dword holds one or two elements");
+  static_assert(TL % (kWave * EPD) == 0, "an instruction stays inside one segment");
+  __shared__ MSHADOW_ALIGNED(16) DType ring[Ring::kSlots][SEGS * LD];
 
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t lane = threadIdx.x & (kWave - 1);
@@ -169,15 +176,15 @@ __global__ void __launch_bounds__(kDmaThreads)
     uint32_t g = 0, sg = 0;  // group and stage within it of the stage being loaded
     for (uint32_t i = 0; i < nstep; ++i) {
       if (i < nstage) {
-        float *slot = ring[i % kDmaSlots];
+        DType *slot = ring[i % kDmaSlots];
 #pragma unroll
         for (int q = 0; q < kDmaPerWave; ++q) {
-          const uint32_t f0 = (q * kDmaLoaders + lw) * kWave;  // first element of this instruction
+          const uint32_t f0 = (q * kDmaLoaders + lw) * kWave * EPD;  // first element of this instruction
           const uint32_t seg = f0 / TL, off = f0 % TL;
           uint32_t n = g * SEGS + seg;
-          uint32_t e = sg * TL + off + lane;
+          uint32_t e = sg * TL + off + lane * EPD;
           n = n < n_out ? n : n_out - 1;  // clamped, never consumed
-          e = e < seg_len ? e : seg_len - 1;
+          e = e < seg_len ? e : seg_len - EPD;
           const uint32_t y = div_x.Div(e);
           const size_t row = static_cast<size_t>(n * n_keep + c) * n_y + y;
           LoadDwordToLds(src + row * stride + (e - y * n_x), slot + seg * LD + off);
@@ -193,7 +200,7 @@ __global__ void __launch_bounds__(kDmaThreads)
       BareBarrier();
     }
   } else {
-    float res, tres;
+    DType res, tres;
     Reducer::SetInitValue(res);
     Reducer::SetInitValue(tres);
     uint32_t g = 0, sg = 0;  // of the stage being folded
@@ -201,7 +208,7 @@ __global__ void __launch_bounds__(kDmaThreads)
       BareBarrier();
       if (i < static_cast<uint32_t>(kDmaAhead)) continue;
       const uint32_t st = i - kDmaAhead;
-      const float *slot = ring[st % kDmaSlots];
+      const DType *slot = ring[st % kDmaSlots];
       const uint32_t e0 = sg * TL;
       const uint32_t live = (n_out - g * SEGS < (uint32_t)SEGS) ? n_out - g * SEGS : SEGS;
       if (lane < live) {
@@ -211,7 +218,7 @@ __global__ void __launch_bounds__(kDmaThreads)
       if (++sg == stages_per_group) {
         /* the group's inner results are final: merge them in n order, then restart */
         for (uint32_t k = 0; k < live; ++k) {
-          const float v = ReadLaneF32(tres, static_cast<int>(k));
+          const DType v = WaveBroadcast(tres, static_cast<int>(k));
           Reducer::Reduce(res, v);
         }
         Reducer::SetInitValue(tres);
@@ -219,7 +226,7 @@ __global__ void __launch_bounds__(kDmaThreads)
         ++g;
       }
     }
-    if (lane == 0) Saver::template Save<float>(dst[c], res * scale);
+    if (lane == 0) Saver::template Save<DType>(dst[c], res * scale);
   }
 }
 

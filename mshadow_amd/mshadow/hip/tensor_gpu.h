@@ -25,6 +25,7 @@
 #if defined(__HIPCC__)
 #include "./kernels/map.h"
 #include "./kernels/reduce.h"
+#include "./kernels/reduce_dma.h"
 #include "./kernels/rows_by_index.h"
 #include "./kernels/softmax_any.h"
 #include "./kernels/sort_any.h"
@@ -1034,6 +1035,43 @@ struct ReduceRoute<Saver, Reducer, Tensor<gpu, 1, float>, Tensor<gpu, dim, float
         Stream<gpu>::GetStream(dst.stream_)));
   }
 };
+#if defined(__HIPCC__)
+/*! \brief sumall_except_dim of a half_t tensor in memory: the LDS-ring kernel of the float path
+ *  (kernels/reduce_dma.h) instantiated for 16-bit elements, a load bringing two neighbouring
+ *  elements of a row. Run() returns false when the shape does not allow that (odd row length or
+ *  pitch, unaligned base, little work per kept index) and the generic kernel has to do it. */
+template <typename Saver, typename Reducer, typename R, typename E>
+struct HalfRingRoute {
+  template <typename... Args> static bool HighDim(Args...) { return false; }
+};
+template <typename Saver, typename Reducer, int dim>
+struct HalfRingRoute<Saver, Reducer, Tensor<gpu, 1, half::half_t>, Tensor<gpu, dim, half::half_t> > {
+  static bool HighDim(const Tensor<gpu, 1, half::half_t> &dst, const Tensor<gpu, dim, half::half_t> &src,
+                      uint32_t n_out, uint32_t n_keep, uint32_t n_y, uint32_t n_x,
+                      half::half_t scale) {
+    const uint64_t per_kept = static_cast<uint64_t>(n_out) * n_y * n_x;
+    if (n_x % 2 != 0 || src.stride_ % 2 != 0 || reinterpret_cast<uintptr_t>(src.dptr_) % 4 != 0 ||
+        per_kept < (1u << 16) || static_cast<uint64_t>(n_y) * n_x >= (1ull << 31)) {
+      return false;
+    }
+    half::half_t *d = dst.dptr_;
+    const half::half_t *s = src.dptr_;
+    uint32_t stride = src.stride_;
+    FastDivU32 div_x(n_x);
+    void *args[] = {&d, &s, &stride, &n_out, &n_keep, &n_y, &n_x, &div_x, &scale};
+    void *stream = Stream<gpu>::GetStream(dst.stream_);
+#define MSHADOW_HALF_RING(SEGS)                                                                  \
+    Launch(hip::ReduceKeepHighDimDmaKernel<Saver, Reducer, half::half_t, SEGS>, n_keep,         \
+           hip::kDmaThreads, args, stream)
+    if (n_out > 16) MSHADOW_HALF_RING(64);
+    else if (n_out > 4) MSHADOW_HALF_RING(16);
+    else if (n_out > 1) MSHADOW_HALF_RING(4);
+    else MSHADOW_HALF_RING(1);
+#undef MSHADOW_HALF_RING
+    return true;
+  }
+};
+#endif  // __HIPCC__
 }  // namespace gpu_detail
 
 template <typename Saver, typename Reducer, typename R, typename DType, typename E, int etype>
@@ -1098,6 +1136,11 @@ inline void MapReduceKeepHighDim(TRValue<R, gpu, 1, DType> *dst,
   uint32_t n_out = eshape.ProdShape(0, dimkeep), n_keep = eshape[dimkeep];
   uint32_t n_y = eshape.ProdShape(dimkeep + 1, EShape::kSubdim), n_x = eshape[EShape::kSubdim];
   if (n_keep == 0) return;
+  if (n_out > 0 && n_y > 0 && n_x > 0 &&
+      gpu_detail::HalfRingRoute<Saver, Reducer, R, E>::HighDim(dst->self(), exp.self(), n_out, n_keep,
+                                                               n_y, n_x, scale)) {
+    return;
+  }
   CHECK_LT(static_cast<uint64_t>(n_y) * n_x, 1ull << 31) << "MapReduceKeepHighDim: inner extent too large";
   FastDivU32 div_x(n_x > 0 ? n_x : 1);
   void *args[] = {&dplan, &splan, &n_out, &n_keep, &n_y, &n_x, &div_x, &scale};

@@ -185,7 +185,13 @@ def test_gpu_half_reduce_keep_lowest(G, orc, stream, shape, pad):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("shape,pad", [((1, 1, 1, 1), 0), ((3, 5, 7, 9), 3), ((2, 2, 30, 100), 0),
-                                       ((20, 6, 28, 28), 0)])
+                                       ((20, 6, 28, 28), 0),
+                                       # enough work per kept index for the LDS-ring kernel: 64, 16, 4
+                                       # and 1 segments side by side, ragged last stages, an even pad
+                                       # (taken) and an odd one (falls back to the generic kernel)
+                                       ((64, 5, 56, 56), 0), ((70, 3, 33, 30), 2), ((6, 3, 150, 100), 0),
+                                       ((3, 2, 301, 128), 6), ((1, 2, 700, 100), 0), ((20, 3, 60, 62), 3),
+                                       ((33, 2, 40, 51), 1)])
 def test_gpu_half_reduce_keep_highdim(G, orc, stream, shape, pad):
     x = halves(orc, 31, shape)
     if shape == (2, 2, 30, 100):
