@@ -107,32 +107,45 @@ inline Tensor<Device, dim, DType> NewTensor(const Shape<dim> &shape, DType initv
   return obj;
 }
 
+/*! \brief element-for-element copy between two host tensors of one shape (either may be
+ *  pitched): one block when both are dense, otherwise row by row */
 template <int dim, typename DType>
-inline void Copy(Tensor<cpu, dim, DType> _dst, const Tensor<cpu, dim, DType> &_src,
+inline void Copy(Tensor<cpu, dim, DType> to, const Tensor<cpu, dim, DType> &from,
                  Stream<cpu> *stream) {
-  CHECK_EQ(_dst.shape_, _src.shape_)
-      << "Copy:shape mismatch:" << _dst.shape_ << " vs " << _src.shape_;
-  if (_dst.CheckContiguous() && _src.CheckContiguous()) {
-    memcpy(_dst.dptr_, _src.dptr_, sizeof(DType) * _dst.shape_.Size());
+  CHECK_EQ(to.shape_, from.shape_) << "Copy:shape mismatch:" << to.shape_ << " vs " << from.shape_;
+  const Shape<2> flat = to.shape_.FlatTo2D();
+  const size_t row_bytes = sizeof(DType) * flat[1];
+  if (to.stride_ == flat[1] && from.stride_ == flat[1]) {
+    memcpy(to.dptr_, from.dptr_, row_bytes * flat[0]);
     return;
   }
-  Tensor<cpu, 2, DType> dst = _dst.FlatTo2D();
-  Tensor<cpu, 2, DType> src = _src.FlatTo2D();
-  for (index_t y = 0; y < dst.size(0); ++y) {
-    memcpy(dst[y].dptr_, src[y].dptr_, sizeof(DType) * dst.size(1));
+  for (index_t r = 0; r < flat[0]; ++r) {
+    memcpy(to.dptr_ + static_cast<size_t>(r) * to.stride_,
+           from.dptr_ + static_cast<size_t>(r) * from.stride_, row_bytes);
   }
 }
+
+namespace cpu_detail {
+/*! \brief destination and source plans of one assignment or reduction, with the checked
+ *  (rows, columns) extent of the source */
+template <typename R, typename E, typename DType>
+struct PlanPair {
+  expr::Plan<R, DType> out;
+  expr::Plan<E, DType> in;
+  PlanPair(const R &dst, const E &src) : out(expr::MakePlan(dst)), in(expr::MakePlan(src)) {}
+};
+}  // namespace cpu_detail
 
 /*! \brief the host evaluation loop: rows in parallel, columns in order */
 template <typename Saver, typename R, int dim, typename DType, typename E>
 inline void MapPlan(TRValue<R, cpu, dim, DType> *dst, const expr::Plan<E, DType> &plan) {
-  Shape<2> shape = expr::ShapeCheck<dim, R>::Check(dst->self()).FlatTo2D();
-  expr::Plan<R, DType> dplan = expr::MakePlan(dst->self());
+  const Shape<2> extent = expr::ShapeCheck<dim, R>::Check(dst->self()).FlatTo2D();
+  expr::Plan<R, DType> target = expr::MakePlan(dst->self());
+  const openmp_index_t rows = extent[0];
+  const index_t cols = extent[1];
 #pragma omp parallel for
-  for (openmp_index_t y = 0; y < shape[0]; ++y) {
-    for (index_t x = 0; x < shape[1]; ++x) {
-      Saver::template Save<DType>(dplan.REval(y, x), plan.Eval(y, x));
-    }
+  for (openmp_index_t r = 0; r < rows; ++r) {
+    for (index_t c = 0; c < cols; ++c) Saver::template Save<DType>(target.REval(r, c), plan.Eval(r, c));
   }
 }
 
@@ -140,104 +153,110 @@ template <typename Saver, typename R, int dim, typename DType, typename E, int e
 inline void MapExp(TRValue<R, cpu, dim, DType> *dst, const expr::Exp<E, DType, etype> &exp) {
   expr::TypeCheckPass<expr::TypeCheck<cpu, dim, DType, E>::kMapPass>::
       Error_All_Tensor_in_Exp_Must_Have_Same_Type();
-  Shape<dim> eshape = expr::ShapeCheck<dim, E>::Check(exp.self());
-  Shape<dim> dshape = expr::ShapeCheck<dim, R>::Check(dst->self());
-  CHECK(eshape[0] == 0 || eshape == dshape)
+  const Shape<dim> want = expr::ShapeCheck<dim, R>::Check(dst->self());
+  const Shape<dim> have = expr::ShapeCheck<dim, E>::Check(exp.self());
+  /* a shape whose first extent is 0 is a scalar-like expression that fits any target */
+  CHECK(have[0] == 0 || have == want)
       << "Assignment: Shape of Tensors are not consistent with target, "
-      << "eshape: " << eshape << " dshape:" << dshape;
+      << "eshape: " << have << " dshape:" << want;
   MapPlan<Saver>(dst, expr::MakePlan(exp.self()));
 }
 
+/*! \brief dst[x] <saver>= scale * reduce over y of exp(y, x): every column is one serial chain
+ *  that starts from the element of row 0 (not from the reducer's initial value) and takes
+ *  the rows in order; columns run in parallel */
 template <typename Saver, typename Reducer, typename R, typename DType, typename E, int etype>
 inline void MapReduceKeepLowest(TRValue<R, cpu, 1, DType> *dst,
                                 const expr::Exp<E, DType, etype> &exp, DType scale) {
   expr::TypeCheckPass<expr::TypeCheck<cpu, 1, DType, E>::kRedPass>::
       Error_TypeCheck_Not_Pass_For_Reduce_Exp();
-  Shape<2> eshape = expr::ShapeCheck<expr::ExpInfo<E>::kDim, E>::Check(exp.self()).FlatTo2D();
-  Shape<1> dshape = expr::ShapeCheck<1, R>::Check(dst->self());
-  CHECK_EQ(eshape[1], dshape[0]) << "MapReduceKeepLowest::reduction dimension do not match";
-  CHECK_NE(eshape[0], 0U) << "can not reduce over empty tensor";
-  expr::Plan<R, DType> dplan = expr::MakePlan(dst->self());
-  expr::Plan<E, DType> splan = expr::MakePlan(exp.self());
+  const Shape<2> extent = expr::ShapeCheck<expr::ExpInfo<E>::kDim, E>::Check(exp.self()).FlatTo2D();
+  const Shape<1> target = expr::ShapeCheck<1, R>::Check(dst->self());
+  CHECK_EQ(extent[1], target[0]) << "MapReduceKeepLowest::reduction dimension do not match";
+  CHECK_NE(extent[0], 0U) << "can not reduce over empty tensor";
+  cpu_detail::PlanPair<R, E, DType> plans(dst->self(), exp.self());
+  const openmp_index_t cols = extent[1];
+  const index_t rows = extent[0];
 #pragma omp parallel for
-  for (openmp_index_t x = 0; x < eshape[1]; ++x) {
-    DType res = splan.Eval(0, x);
-    for (index_t y = 1; y < eshape[0]; ++y) Reducer::Reduce(res, splan.Eval(y, x));
-    Saver::template Save<DType>(dplan.REval(0, x), res * scale);
+  for (openmp_index_t c = 0; c < cols; ++c) {
+    DType acc = plans.in.Eval(0, c);
+    for (index_t r = 1; r < rows; ++r) Reducer::Reduce(acc, plans.in.Eval(r, c));
+    Saver::template Save<DType>(plans.out.REval(0, c), acc * scale);
   }
 }
 
+/*! \brief dst[c] <saver>= scale * reduce of exp over every axis but `dimkeep`. The source is
+ *  viewed as (before, kept, rows behind, last axis); for a kept index the elements behind each
+ *  `before` index are reduced first, in memory order, into a partial result that starts from
+ *  the reducer's initial value, and the partial results are then reduced in `before` order -
+ *  two levels, which a floating-point sum can tell from one */
 template <typename Saver, typename Reducer, int dimkeep, typename R, typename DType, typename E,
           int etype>
 inline void MapReduceKeepHighDim(TRValue<R, cpu, 1, DType> *dst,
                                  const expr::Exp<E, DType, etype> &exp, DType scale) {
   expr::TypeCheckPass<expr::TypeCheck<cpu, dimkeep, DType, E>::kRedPass>::
       Error_TypeCheck_Not_Pass_For_Reduce_Exp();
-  typedef Shape<expr::ExpInfo<E>::kDim> EShape;
-  EShape eshape = expr::ShapeCheck<expr::ExpInfo<E>::kDim, E>::Check(exp.self());
-  Shape<1> dshape = expr::ShapeCheck<1, R>::Check(dst->self());
-  CHECK_EQ(eshape[dimkeep], dshape[0]) << "MapReduceKeepHighDim::reduction dimension do not match";
-  /* (outer, kept, inner rows, last dim) */
-  const index_t n_out = eshape.ProdShape(0, dimkeep);
-  const index_t n_keep = eshape[dimkeep];
-  const index_t n_y = eshape.ProdShape(dimkeep + 1, EShape::kSubdim);
-  const index_t n_x = eshape[EShape::kSubdim];
-  expr::Plan<R, DType> dplan = expr::MakePlan(dst->self());
-  expr::Plan<E, DType> splan = expr::MakePlan(exp.self());
+  typedef Shape<expr::ExpInfo<E>::kDim> SourceShape;
+  const SourceShape extent = expr::ShapeCheck<expr::ExpInfo<E>::kDim, E>::Check(exp.self());
+  const Shape<1> target = expr::ShapeCheck<1, R>::Check(dst->self());
+  CHECK_EQ(extent[dimkeep], target[0]) << "MapReduceKeepHighDim::reduction dimension do not match";
+  const index_t before = extent.ProdShape(0, dimkeep);
+  const openmp_index_t kept = extent[dimkeep];
+  const index_t rows_behind = extent.ProdShape(dimkeep + 1, SourceShape::kSubdim);
+  const index_t last = extent[SourceShape::kSubdim];
+  cpu_detail::PlanPair<R, E, DType> plans(dst->self(), exp.self());
 #pragma omp parallel for
-  for (openmp_index_t c = 0; c < n_keep; ++c) {
-    DType res;
-    Reducer::SetInitValue(res);
-    for (index_t n = 0; n < n_out; ++n) {
-      DType tres;
-      Reducer::SetInitValue(tres);
-      for (index_t y = 0; y < n_y; ++y) {
-        for (index_t x = 0; x < n_x; ++x) {
-          Reducer::Reduce(tres, splan.Eval((n * n_keep + c) * n_y + y, x));
-        }
+  for (openmp_index_t c = 0; c < kept; ++c) {
+    DType total;
+    Reducer::SetInitValue(total);
+    for (index_t b = 0; b < before; ++b) {
+      DType partial;
+      Reducer::SetInitValue(partial);
+      const index_t first_row = (b * static_cast<index_t>(kept) + static_cast<index_t>(c)) * rows_behind;
+      for (index_t r = first_row; r < first_row + rows_behind; ++r) {
+        for (index_t x = 0; x < last; ++x) Reducer::Reduce(partial, plans.in.Eval(r, x));
       }
-      Reducer::Reduce(res, tres);
+      Reducer::Reduce(total, partial);
     }
-    Saver::template Save<DType>(dplan.REval(0, c), DType(res * scale));
+    Saver::template Save<DType>(plans.out.REval(0, c), DType(total * scale));
   }
 }
 
-/*! \brief one row: max, exp(x - max) summed left to right, then divide */
+namespace cpu_detail {
+/*! \brief softmax of `count` elements `step` apart, in the element type's own arithmetic:
+ *  the largest element by strict <, exp(x - largest) stored and summed left to right, every
+ *  stored term divided by the sum. The 1-D, 2-D and 3-D functions are this on different
+ *  strides (mshadow/tensor_cpu-inl.h:270-285, 466-488). */
+template <typename DType>
+inline void SoftmaxStrided(DType *out, size_t out_step, const DType *in, size_t in_step,
+                           index_t count) {
+  DType largest = in[0];
+  for (index_t i = 1; i < count; ++i) {
+    if (largest < in[i * in_step]) largest = in[i * in_step];
+  }
+  DType denominator = DType(0.0f);
+  for (index_t i = 0; i < count; ++i) {
+    out[i * out_step] = std::exp(in[i * in_step] - largest);
+    denominator += out[i * out_step];
+  }
+  for (index_t i = 0; i < count; ++i) out[i * out_step] /= denominator;
+}
+}  // namespace cpu_detail
+
 template <typename DType>
 inline void Softmax(Tensor<cpu, 1, DType> dst, const Tensor<cpu, 1, DType> &energy) {
-  DType mmax = energy[0];
-  for (index_t x = 1; x < dst.size(0); ++x) {
-    if (mmax < energy[x]) mmax = energy[x];
-  }
-  DType sum = DType(0.0f);
-  for (index_t x = 0; x < dst.size(0); ++x) {
-    dst[x] = std::exp(energy[x] - mmax);
-    sum += dst[x];
-  }
-  for (index_t x = 0; x < dst.size(0); ++x) dst[x] /= sum;
+  cpu_detail::SoftmaxStrided(dst.dptr_, 1, energy.dptr_, 1, dst.size(0));
 }
 template <typename DType>
 inline void Softmax(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 2, DType> &energy) {
   CHECK_EQ(dst.shape_, energy.shape_) << "Softmax: shape mismatch";
+  const openmp_index_t rows = dst.size(0);
 #pragma omp parallel for
-  for (openmp_index_t y = 0; y < dst.size(0); ++y) Softmax(dst[y], energy[y]);
-}
-template <typename DType>
-inline void SoftmaxGrad(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 2, DType> &src,
-                        const Tensor<cpu, 1, DType> &label) {
-#pragma omp parallel for
-  for (openmp_index_t y = 0; y < dst.size(0); ++y) {
-    const index_t k = static_cast<int>(label[y]);
-    for (index_t x = 0; x < dst.size(1); ++x) {
-      if (x == k) {
-        dst[y][k] = src[y][k] - 1.0f;
-      } else {
-        dst[y][x] = src[y][x];
-      }
-    }
+  for (openmp_index_t r = 0; r < rows; ++r) {
+    cpu_detail::SoftmaxStrided(dst.dptr_ + static_cast<size_t>(r) * dst.stride_, 1,
+                               energy.dptr_ + static_cast<size_t>(r) * energy.stride_, 1, dst.size(1));
   }
 }
-
 
 /* ---- the rest of the softmax family and the row scatter / gather functions
  * (mshadow/tensor_cpu-inl.h:304-528 of the reference). One element of every gradient
@@ -283,6 +302,11 @@ inline void Grad3D(Tensor<cpu, 3, DType> dst, const Tensor<cpu, 3, DType> &src,
 }  // namespace cpu_detail
 
 template <typename DType>
+inline void SoftmaxGrad(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 2, DType> &src,
+                        const Tensor<cpu, 1, DType> &label) {
+  cpu_detail::Grad2D(dst, src, label, false, 0, false, 0.0f);
+}
+template <typename DType>
 inline void SmoothSoftmaxGrad(Tensor<cpu, 2, DType> dst, const Tensor<cpu, 2, DType> &src,
                               const Tensor<cpu, 1, DType> &label, const float alpha) {
   cpu_detail::Grad2D(dst, src, label, false, 0, true, alpha);
@@ -319,23 +343,19 @@ inline void SmoothSoftmaxGrad(Tensor<cpu, 3, DType> dst, const Tensor<cpu, 3, DT
                               const float alpha) {
   cpu_detail::Grad3D(dst, src, label, true, static_cast<int>(ignore_label), true, alpha);
 }
-/*! \brief softmax over the middle dimension of (d0, d1, d2) */
+/*! \brief softmax over the middle dimension of (d0, d1, d2): element (y, x, n) is
+ *  (y * d1 + x) * stride + n, so a column (y, n) is d1 elements one pitch apart */
 template <typename DType>
 inline void Softmax(Tensor<cpu, 3, DType> dst, const Tensor<cpu, 3, DType> &energy) {
   CHECK_EQ(dst.shape_, energy.shape_) << "Softmax: shape mismatch";
+  const openmp_index_t outer = dst.size(0);
+  const index_t classes = dst.size(1), inner = dst.size(2);
 #pragma omp parallel for
-  for (openmp_index_t y = 0; y < dst.size(0); ++y) {
-    for (index_t n = 0; n < dst.size(2); ++n) {
-      DType mmax = energy[y][0][n];
-      for (index_t x = 1; x < dst.size(1); ++x) {
-        if (mmax < energy[y][x][n]) mmax = energy[y][x][n];
-      }
-      DType sum = DType(0.0f);
-      for (index_t x = 0; x < dst.size(1); ++x) {
-        dst[y][x][n] = std::exp(energy[y][x][n] - mmax);
-        sum += dst[y][x][n];
-      }
-      for (index_t x = 0; x < dst.size(1); ++x) dst[y][x][n] /= sum;
+  for (openmp_index_t y = 0; y < outer; ++y) {
+    DType *out = dst.dptr_ + static_cast<size_t>(y) * classes * dst.stride_;
+    const DType *in = energy.dptr_ + static_cast<size_t>(y) * classes * energy.stride_;
+    for (index_t n = 0; n < inner; ++n) {
+      cpu_detail::SoftmaxStrided(out + n, dst.stride_, in + n, energy.stride_, classes);
     }
   }
 }
