@@ -24,41 +24,58 @@ struct ReduceTo1DExp
   ReduceTo1DExp(const SrcExp &src, DType scale) : src_(src), scale_(scale) {}
 };
 
-template <int dimkeep, typename SrcExp, typename DType, int etype>
-inline ReduceTo1DExp<SrcExp, DType, red::sum, ExpInfo<SrcExp>::kDim - dimkeep> sumall_except_dim(
-    const Exp<SrcExp, DType, etype> &exp) {
-  return ReduceTo1DExp<SrcExp, DType, red::sum, ExpInfo<SrcExp>::kDim - dimkeep>(exp.self(),
-                                                                                  DType(1));
-}
+namespace reduce_detail {
+/*! \brief the node type for keeping dimension `dimkeep` (counted from the front) of SrcExp */
+template <int dimkeep, typename Reducer, typename SrcExp, typename DType>
+struct NodeFor {
+  typedef ReduceTo1DExp<SrcExp, DType, Reducer, ExpInfo<SrcExp>::kDim - dimkeep> Type;
+  inline static Type Make(const SrcExp &src) { return Type(src, DType(1)); }
+};
+/*! \brief which device function evaluates the node: the kept dimension is the last one
+ *  (every output is a chain over the rows) or any other (two-level reduction) */
+template <bool kKeepsLast>
+struct Evaluate {
+  template <typename SV, typename Reducer, int dimkeep, typename Dst, typename SrcExp, typename DType>
+  inline static void Run(Dst *dst, const SrcExp &src, DType scale) {
+    MapReduceKeepHighDim<SV, Reducer, dimkeep>(dst, src, scale);
+  }
+};
+template <>
+struct Evaluate<true> {
+  template <typename SV, typename Reducer, int dimkeep, typename Dst, typename SrcExp, typename DType>
+  inline static void Run(Dst *dst, const SrcExp &src, DType scale) {
+    MapReduceKeepLowest<SV, Reducer>(dst, src, scale);
+  }
+};
+}  // namespace reduce_detail
+
 template <int dimkeep, typename Reducer, typename SrcExp, typename DType, int etype>
-inline ReduceTo1DExp<SrcExp, DType, Reducer, ExpInfo<SrcExp>::kDim - dimkeep> reduce_except_dim(
+inline typename reduce_detail::NodeFor<dimkeep, Reducer, SrcExp, DType>::Type reduce_except_dim(
     const Exp<SrcExp, DType, etype> &exp) {
-  return ReduceTo1DExp<SrcExp, DType, Reducer, ExpInfo<SrcExp>::kDim - dimkeep>(exp.self(),
-                                                                                 DType(1));
+  return reduce_detail::NodeFor<dimkeep, Reducer, SrcExp, DType>::Make(exp.self());
 }
+template <int dimkeep, typename SrcExp, typename DType, int etype>
+inline typename reduce_detail::NodeFor<dimkeep, red::sum, SrcExp, DType>::Type sumall_except_dim(
+    const Exp<SrcExp, DType, etype> &exp) {
+  return reduce_except_dim<dimkeep, red::sum>(exp);
+}
+/*! \brief column sums of a matrix */
 template <typename SrcExp, typename DType, int etype>
 inline ReduceTo1DExp<SrcExp, DType, red::sum, 1> sum_rows(const Exp<SrcExp, DType, etype> &exp) {
   TypeCheckPass<ExpInfo<SrcExp>::kDim == 2>::Error_Expression_Does_Not_Meet_Dimension_Req();
   return sumall_except_dim<1>(exp);
 }
 
+/*! \brief dst [sv] node: one engine for every kept dimension */
 template <typename SV, typename Device, typename DType, typename SrcExp, typename Reducer,
           int m_dimkeep>
 struct ExpComplexEngine<SV, Tensor<Device, 1, DType>,
                         ReduceTo1DExp<SrcExp, DType, Reducer, m_dimkeep>, DType> {
-  static const int dimkeep = ExpInfo<SrcExp>::kDim - m_dimkeep;
   inline static void Eval(Tensor<Device, 1, DType> *dst,
                           const ReduceTo1DExp<SrcExp, DType, Reducer, m_dimkeep> &exp) {
-    TypeCheckPass<m_dimkeep != 1>::Error_Expression_Does_Not_Meet_Dimension_Req();
-    MapReduceKeepHighDim<SV, Reducer, dimkeep>(dst, exp.src_, exp.scale_);
-  }
-};
-template <typename SV, typename Device, typename DType, typename SrcExp, typename Reducer>
-struct ExpComplexEngine<SV, Tensor<Device, 1, DType>, ReduceTo1DExp<SrcExp, DType, Reducer, 1>,
-                        DType> {
-  inline static void Eval(Tensor<Device, 1, DType> *dst,
-                          const ReduceTo1DExp<SrcExp, DType, Reducer, 1> &exp) {
-    MapReduceKeepLowest<SV, Reducer>(dst, exp.src_, exp.scale_);
+    reduce_detail::Evaluate<m_dimkeep == 1>::template Run<SV, Reducer,
+                                                          ExpInfo<SrcExp>::kDim - m_dimkeep>(
+        dst, exp.src_, exp.scale_);
   }
 };
 
