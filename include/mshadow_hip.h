@@ -108,7 +108,9 @@ int mshadow_hip_memset_async(void *dst, int byte_value, size_t bytes, void *stre
 /* dst = scalar on a (rows, cols) view of 32-bit elements with pitch dstride (elements):
    what `tensor = value` and NewTensor's initial value do through MapExp in the reference
    (mshadow/tensor_gpu-inl.h:101-116 with a ScalarExp source). `bits` is the element's
-   bit pattern. A kernel, not a memset: it may be recorded into a graph. */
+   bit pattern. A kernel, not a memset: it may be recorded into a graph. No limit on the
+   element count short of `int` rows and columns (runs of rows of less than 2^31 elements
+   each are launched one after the other). */
 int mshadow_hip_fill_32(void *dst, int dstride, int rows, int cols, uint32_t bits, void *stream);
 
 /* ------------------------------------------------------------------ 2. launch */

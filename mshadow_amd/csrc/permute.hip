@@ -17,6 +17,8 @@
  *
  * Also here: the fill of a 2-D view with one 32-bit pattern (`tensor = scalar`).
  */
+#include <algorithm>
+
 #include <mshadow/core/fastdiv.h>
 #include <mshadow/hip/kernels/common.h>
 
@@ -201,20 +203,25 @@ extern "C" int mshadow_hip_fill_32(void *dst, int dstride, int rows, int cols, u
   if (rows == 0 || cols == 0) return MSHADOW_HIP_OK;
   ABI_REQUIRE(dst != NULL, "NULL tensor");
   ABI_REQUIRE(dstride >= cols, "pitch smaller than the row");
-  const uint64_t total = static_cast<uint64_t>(rows) * cols;
-  ABI_REQUIRE(total < (1ull << 31), "too many elements");
   const bool wide = cols % 4 == 0 && dstride % 4 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0;
   const uint32_t ppr = static_cast<uint32_t>(wide ? cols / 4 : cols);
-  uint64_t blocks = (static_cast<uint64_t>(rows) * ppr + kPermuteBlock - 1) / kPermuteBlock;
-  if (blocks > 65536) blocks = 65536;
-  if (wide) {
-    hipLaunchKernelGGL(FillKernel<4>, dim3(static_cast<unsigned>(blocks)), dim3(kPermuteBlock), 0,
-                       AsStream(stream), static_cast<uint32_t *>(dst), static_cast<uint32_t>(dstride),
-                       static_cast<uint32_t>(rows), ppr, FastDivU32(ppr), bits);
-  } else {
-    hipLaunchKernelGGL(FillKernel<1>, dim3(static_cast<unsigned>(blocks)), dim3(kPermuteBlock), 0,
-                       AsStream(stream), static_cast<uint32_t *>(dst), static_cast<uint32_t>(dstride),
-                       static_cast<uint32_t>(rows), ppr, FastDivU32(ppr), bits);
+  /* the kernel counts packs in 32 bits: a tensor of 2^31 elements or more (it fits this
+     device many times over) is filled in runs of whole rows */
+  const int rows_per_launch = static_cast<int>(std::max<uint64_t>(1, ((1ull << 31) - 1) / ppr));
+  for (int row0 = 0; row0 < rows; row0 += rows_per_launch) {
+    const int nrows = std::min(rows_per_launch, rows - row0);
+    uint32_t *first = static_cast<uint32_t *>(dst) + static_cast<size_t>(row0) * dstride;
+    uint64_t blocks = (static_cast<uint64_t>(nrows) * ppr + kPermuteBlock - 1) / kPermuteBlock;
+    if (blocks > 65536) blocks = 65536;
+    if (wide) {
+      hipLaunchKernelGGL(FillKernel<4>, dim3(static_cast<unsigned>(blocks)), dim3(kPermuteBlock), 0,
+                         AsStream(stream), first, static_cast<uint32_t>(dstride),
+                         static_cast<uint32_t>(nrows), ppr, FastDivU32(ppr), bits);
+    } else {
+      hipLaunchKernelGGL(FillKernel<1>, dim3(static_cast<unsigned>(blocks)), dim3(kPermuteBlock), 0,
+                         AsStream(stream), first, static_cast<uint32_t>(dstride),
+                         static_cast<uint32_t>(nrows), ppr, FastDivU32(ppr), bits);
+    }
   }
   return AfterLaunch("fill");
 }

@@ -487,3 +487,25 @@ def test_im2col_reference_known_answer(G, stream):
             for oy in range(2):
                 for ox in range(2):
                     assert got[ky * 3 + kx, oy * 2 + ox] == img[0, 0, 2 * oy + ky, 2 * ox + kx]
+
+
+@pytest.mark.gpu
+def test_fill_of_more_than_2_to_the_31_elements(G, stream):
+    """`tensor = scalar` on 8.6 GB: the entry point launches runs of whole rows; the first and
+    last rows, the rows on either side of a run boundary and a guard row behind the tensor
+    are read back"""
+    rows, cols = (1 << 15) + 3, (1 << 16) + 1      # odd rows: one element per store, 32767 rows per run
+    buf = G.buffer((rows + 1, cols), np.float32)
+    G.fill(buf, 0.0, stream)            # the whole allocation, guard row included
+    bits = int(np.array([2.5], np.float32).view(np.uint32)[0])
+    G.check(G.dll.mshadow_hip_fill_32(buf.ptr, cols, rows, cols, bits, stream))
+    per_run = ((1 << 31) - 1) // cols
+    assert 1 < per_run < rows
+    from mshadow_amd.capi import D2H
+    for r, want in ((0, 2.5), (1, 2.5), (per_run - 1, 2.5), (per_run, 2.5), (rows - 1, 2.5), (rows, 0.0)):
+        out = np.empty(cols, np.float32)
+        G.check(G.dll.mshadow_hip_memcpy2d_async(out.ctypes.data, cols * 4, buf.ptr + r * cols * 4, cols * 4,
+                                                 cols * 4, 1, D2H, stream))
+        G.stream_sync(stream)
+        assert np.all(out == np.float32(want)), r
+    buf.free()
