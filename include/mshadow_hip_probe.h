@@ -53,8 +53,8 @@ int mshadow_probe_row_copy(float *dst, int dstride, const float *src, int sstrid
                            int cols, int barriers, int spin, double *kernel_us, void *stream);
 
 /* Rate of loads from global memory straight into LDS (the loads of the reduction kernels),
-   with nothing consuming the data: `waves` waves per workgroup keep 32..48 loads of `width`
-   bytes per lane (4 or 16) outstanding each. strip = 0: the matrix is read as one buffer,
+   with nothing consuming the data: `waves` waves per workgroup keep window .. window + 16
+   loads (window = 16 or 32) of `width` bytes per lane (4 or 16) outstanding each. strip = 0: the matrix is read as one buffer,
    1024 workgroups take a contiguous piece each and an instruction fetches 64 * width
    consecutive bytes; strip = 16, 32 or 64: a workgroup reads that many columns of every
    row, as a reduction over the rows does, cols / strip workgroups, neighbouring strips
@@ -64,7 +64,7 @@ int mshadow_probe_row_copy(float *dst, int dstride, const float *src, int sstrid
    dimensions does. kernel_us = duration of the
    launch that reads rows x cols floats once. */
 int mshadow_probe_dma_rate(const float *src, int sstride, int rows, int cols, int strip, int width,
-                           int waves, double *kernel_us, void *stream);
+                           int waves, int window, double *kernel_us, void *stream);
 
 #ifdef __cplusplus
 }

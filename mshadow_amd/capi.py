@@ -659,12 +659,12 @@ class Probe:
                                                     src.cols, barriers, spin, C.byref(us), stream))
         return us.value
 
-    def dma_rate_us(self, src, strip, width, waves, stream=None):
+    def dma_rate_us(self, src, strip, width, waves, stream=None, window=32):
         """time to read `src` once by loads into LDS (strip 0/16/32 columns, width 4/16 bytes)"""
         us = C.c_double(0)
-        self.dll.mshadow_probe_dma_rate.argtypes = [_p, _i, _i, _i, _i, _i, _i, C.POINTER(C.c_double), _p]
+        self.dll.mshadow_probe_dma_rate.argtypes = [_p, _i, _i, _i, _i, _i, _i, _i, C.POINTER(C.c_double), _p]
         self._check(self.dll.mshadow_probe_dma_rate(src.ptr, src.stride, src.rows, src.cols, strip, width,
-                                                    waves, C.byref(us), stream))
+                                                    waves, window, C.byref(us), stream))
         return us.value
 
     def _check(self, status):

@@ -151,7 +151,8 @@ __global__ void __launch_bounds__(THREADS, 4)
 
 
 /* Rate of loads from global memory straight into LDS, nothing else: `blockDim.x / 64` waves
-   per workgroup issue them in batches of 16 and keep up to 48 outstanding. WIDTH bytes per
+   per workgroup issue them in batches of 16 and wait until `window` (16 or 32) are left
+   outstanding, so that window .. window + 16 are in flight per wave. WIDTH bytes per
    lane (4 or 16). STRIP == 0: a workgroup reads a contiguous piece of the buffer, an
    instruction 64 * WIDTH consecutive bytes. STRIP > 0: the buffer is a matrix of `rows` x
    `cols` floats, a workgroup reads STRIP columns of every row (what a reduction over the
@@ -161,7 +162,7 @@ __global__ void __launch_bounds__(THREADS, 4)
    the second of four dimensions does). */
 template <int WIDTH, int STRIP>
 __global__ void __launch_bounds__(1024) DmaRateKernel(const float *src, uint32_t stride, uint32_t rows,
-                                                      uint32_t cols) {
+                                                      uint32_t cols, int window) {
   const int kRegion = 16 * 64 * WIDTH;   // bytes of LDS a wave cycles through
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -215,7 +216,11 @@ __global__ void __launch_bounds__(1024) DmaRateKernel(const float *src, uint32_t
         __builtin_amdgcn_global_load_lds(from, to, 16, 0, 2);
       }
     }
-    asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
+    if (window == 16) {
+      asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
+    }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
@@ -354,10 +359,11 @@ int mshadow_probe_softmax_phases(float *dst, int dstride, const float *src, int 
 }
 
 int mshadow_probe_dma_rate(const float *src, int sstride, int rows, int cols, int strip, int width,
-                           int waves, double *kernel_us, void *stream) {
+                           int waves, int window, double *kernel_us, void *stream) {
   ABI_REQUIRE(src != NULL && kernel_us != NULL && rows >= 1024 && cols >= 64 && sstride >= cols,
               "a matrix of at least 1024 x 64");
   ABI_REQUIRE(waves >= 1 && waves <= 16, "1..16 waves");
+  ABI_REQUIRE(window == 16 || window == 32, "16 or 32 loads left outstanding");
   ABI_REQUIRE((width == 4 || width == 16) &&
                   (strip == -1 || strip == 0 || strip == 16 || strip == 32 || strip == 64),
               "width 4 or 16 bytes, strip -1, 0, 16, 32 or 64");
@@ -376,7 +382,7 @@ int mshadow_probe_dma_rate(const float *src, int sstride, int rows, int cols, in
     st = TimeKernel(s, &ms, [&] {                                                             \
       hipLaunchKernelGGL((DmaRateKernel<W, S>), dim3(grid), dim3(waves * 64), lds, s, src,    \
                          static_cast<uint32_t>(sstride), static_cast<uint32_t>(rows),         \
-                         static_cast<uint32_t>(cols));                                        \
+                         static_cast<uint32_t>(cols), window);                                \
     });                                                                                       \
   }
   if (width == 4 && strip == -1) PROBE_DMA(4, -1)
