@@ -9,10 +9,13 @@ timed region; every operation is queued on one stream through the C ABI (the ele
 map through the C++ expression API compiled in libmshadow_cases.so).
 
 Output: one JSON line. `value` is the whole-step effective bandwidth: algorithmic bytes
-(each tensor counted once) of all nine operations divided by the
-step time. `per_op` lists each operation's own GB/s, fraction of the 8 TB/s HBM peak and
-GElem/s from HIP events recorded around it on the same stream. `roofline` describes the
-kernel that takes the largest share of the step. `cpu_baseline` times the reference CPU
+(each tensor counted once) of all nine operations divided by the step time of the timed
+region - exactly K steps between two synchronizations, with HIP events only around the
+dominant operation (`roofline`: the kernel that takes the largest share of the step, timed
+live inside the timed region). `per_op` lists each operation's own figures from a pass of
+the same K steps made just before, with an event after every launch (`ms`: the interval
+inside a step, a few microseconds of launch gap included) and from launches repeated back to
+back over rotating operand sets (`ms_back_to_back`). `cpu_baseline` times the reference CPU
 path (oracle/_ref, the reference's own headers) or, where that library is absent, the C
 restatement, on the host cores of the same machine over the same inputs.
 """
@@ -337,10 +340,12 @@ def main():
     G.stream_sync(s)
     G.device_sync()
 
+    # Per-operation pass (not the timed region): the same K steps with an event after every
+    # launch, which gives every operation's interval and names the dominant one. An event
+    # between two launches costs the step about 3 us each, so the timed region below keeps
+    # only the two around the dominant operation.
     nev = len(only) + 1
     events = [[G.event_create() for _ in range(nev)] for _ in range(args.steps)]
-    G.device_sync()
-    wall0 = time.perf_counter()
     for k in range(args.steps):
         G.event_record(events[k][0], s)
         for i, name in enumerate(only):
@@ -348,7 +353,26 @@ def main():
             G.event_record(events[k][i + 1], s)
     G.stream_sync(s)
     G.device_sync()
+    pass_ms = {name: np.array([G.elapsed_ms(events[k][i], events[k][i + 1]) for k in range(args.steps)])
+               for i, name in enumerate(only)}
+    dominant = max(pass_ms, key=lambda n: pass_ms[n].mean())
+
+    # The timed region: exactly K steps, synchronized on both sides
+    dom_events = [(G.event_create(), G.event_create()) for _ in range(args.steps)]
+    G.device_sync()
+    wall0 = time.perf_counter()
+    for k in range(args.steps):
+        for name in only:
+            if name == dominant:
+                G.event_record(dom_events[k][0], s)
+                run_op(name)
+                G.event_record(dom_events[k][1], s)
+            else:
+                run_op(name)
+    G.stream_sync(s)
+    G.device_sync()
     wall = time.perf_counter() - wall0
+    dom_ms = float(np.mean([G.elapsed_ms(a, b) for a, b in dom_events]))
 
     # A second figure per operation: the same launch repeated back to back, so that no gap
     # between launches is inside the interval, over three complete sets of operands in turn
@@ -380,7 +404,7 @@ def main():
     per_op = []
     op_ms = {}
     for i, name in enumerate(only):
-        ms = np.array([G.elapsed_ms(events[k][i], events[k][i + 1]) for k in range(args.steps)])
+        ms = pass_ms[name]
         op_ms[name] = float(ms.mean())
         gbs = abytes[name] * scale_fix / (ms.mean() * 1e-3) / 1e9
         per_op.append({"op": name, "ms": round(float(ms.mean()), 4), "ms_min": round(float(ms.min()), 4),
@@ -397,8 +421,7 @@ def main():
     step_ms = wall / args.steps * 1e3
     total_bytes = sum(abytes[n] for n in only) * scale_fix
     value = total_bytes / (step_ms * 1e-3) / 1e9
-    dominant = max(op_ms, key=op_ms.get)
-    dom_gbs = abytes[dominant] * scale_fix / (op_ms[dominant] * 1e-3) / 1e9
+    dom_gbs = abytes[dominant] * scale_fix / (dom_ms * 1e-3) / 1e9
 
     cpu = None
     if not args.no_cpu:
