@@ -325,6 +325,28 @@ def test_gpu_half_softmax_full_size(G, orc, stream):
 
 
 @pytest.mark.gpu
+def test_gpu_half_reductions_full_size(G, orc, stream):
+    """the two reductions on half_t at the BASELINE shapes, bit for bit against the CPU path (the
+    compiled reference where it is present): sumall_except_dim<1> over (64,256,56,56) through the
+    LDS-ring kernel, sum_rows over 16384 x 4096 through the generic one"""
+    chk = Checker("ref") if have_ref() else orc
+    x4 = halves(orc, 71, (64, 256, 56, 56))
+    src4 = G.to_device(x4)
+    for reducer in (SUM, MAX):
+        want = np.zeros(256, np.uint16)
+        chk.reduce_keep_highdim(want, x4, reducer, SAVETO, 1.0)
+        dst = G.buffer((256,), np.uint16)
+        G.case_reduce_keep_highdim(dst, src4, reducer, SAVETO, _bits(orc, 1.0), 0, stream)
+        assert np.array_equal(dst.download(stream), want), reducer
+    m = halves(orc, 72, (16384, 4096))
+    want = np.zeros(4096, np.uint16)
+    chk.reduce_keep_lowest(want, m, SUM, SAVETO, 1.0)
+    dst = G.buffer((4096,), np.uint16)
+    G.case_reduce_keep_lowest(dst, G.to_device(m), SUM, SAVETO, _bits(orc, 1.0), 0, stream)
+    assert np.array_equal(dst.download(stream), want)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("shape", [(1, 1), (5000, 7), (300, 130), (3, 5, 7, 9), (20, 6, 28, 28)])
 def test_gpu_double_reductions(G, stream, shape):
     """sum_rows / sumall_except_dim<1> (and max, min) on double tensors through the generic
