@@ -514,7 +514,8 @@ def run_probe(G, which):
                # the kernel's loads and stores alone, and with stand-in work between them
                "row_copy_us": {f"{b} barriers x {k} multiply-adds per element":
                                round(P.row_copy_us(dst, src, b, k, s), 1)
-                               for b, k in ((0, 0), (4, 0), (4, 2), (4, 4), (4, 8), (8, 4))}}
+                               for b, k in ((0, 0), (4, 0), (4, 2), (4, 4), (4, 8), (8, 4))},
+               "row_copy_one_row_per_cu_us": round(min(P.row_copy_us(dst, src, 0, 0, s, 1) for _ in range(3)), 1)}
     print(json.dumps(out))
 
 

@@ -48,9 +48,11 @@ int mshadow_probe_softmax_phases(float *dst, int dstride, const float *src, int 
    softmax kernel does, meets `barriers` workgroup barriers with `spin` multiply-adds per
    element before each, and stores the row. barriers = 0: what the access pattern itself
    allows (one workgroup per row, two rows resident per CU); with spin > 0: how much work
-   between load and store the machine hides. kernel_us = duration of the launch. */
+   between load and store the machine hides. resident = 2: two rows per CU as in the softmax
+   kernel; 1: one (a second workgroup is kept off the CU). kernel_us = duration of the launch. */
 int mshadow_probe_row_copy(float *dst, int dstride, const float *src, int sstride, int rows,
-                           int cols, int barriers, int spin, double *kernel_us, void *stream);
+                           int cols, int barriers, int spin, int resident, double *kernel_us,
+                           void *stream);
 
 /* Rate of loads from global memory straight into LDS (the loads of the reduction kernels),
    with nothing consuming the data: `waves` waves per workgroup keep window .. window + 16

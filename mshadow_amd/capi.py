@@ -652,11 +652,11 @@ class Probe:
             _p, _i, _p, _i, _i, _i, C.POINTER(C.c_double), C.POINTER(C.c_double),
             C.POINTER(C.c_double), C.POINTER(_i), _p]
 
-    def row_copy_us(self, dst, src, barriers, spin, stream=None):
+    def row_copy_us(self, dst, src, barriers, spin, stream=None, resident=2):
         us = C.c_double(0)
-        self.dll.mshadow_probe_row_copy.argtypes = [_p, _i, _p, _i, _i, _i, _i, _i, C.POINTER(C.c_double), _p]
+        self.dll.mshadow_probe_row_copy.argtypes = [_p, _i, _p, _i, _i, _i, _i, _i, _i, C.POINTER(C.c_double), _p]
         self._check(self.dll.mshadow_probe_row_copy(dst.ptr, dst.stride, src.ptr, src.stride, src.rows,
-                                                    src.cols, barriers, spin, C.byref(us), stream))
+                                                    src.cols, barriers, spin, resident, C.byref(us), stream))
         return us.value
 
     def dma_rate_us(self, src, strip, width, waves, stream=None, window=32):

@@ -290,14 +290,17 @@ int mshadow_probe_add_chain(int mode, int workgroups, double *ns_per_add, void *
 }
 
 int mshadow_probe_row_copy(float *dst, int dstride, const float *src, int sstride, int rows,
-                           int cols, int barriers, int spin, double *kernel_us, void *stream) {
+                           int cols, int barriers, int spin, int resident, double *kernel_us,
+                           void *stream) {
+  ABI_REQUIRE(resident == 1 || resident == 2, "one or two rows resident per CU");
   ABI_REQUIRE(rows >= 1 && cols > 16384 && cols <= 32768 && cols % 4 == 0 && sstride % 4 == 0 &&
                   dstride % 4 == 0 && kernel_us != NULL, "16384 < cols <= 32768, rows of whole packs");
   hipStream_t s = AsStream(stream);
   float ms = 0.0f;
   const int st = TimeKernel(s, &ms, [&] {
-    hipLaunchKernelGGL((RowCopyKernel<512, 16>), dim3(rows), dim3(512), 0, s, dst, dstride, src, sstride,
-                       cols, barriers, spin);
+    /* one row per CU: dynamic LDS the kernel never touches keeps a second workgroup off the CU */
+    hipLaunchKernelGGL((RowCopyKernel<512, 16>), dim3(rows), dim3(512), resident == 1 ? 90000 : 0, s, dst,
+                       dstride, src, sstride, cols, barriers, spin);
   });
   if (st != MSHADOW_HIP_OK) return st;
   *kernel_us = ms * 1e3;
