@@ -165,10 +165,14 @@ def _bits(orc, scale):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("shape,pad", [((1, 1), 0), ((5000, 3), 0), ((300, 33), 5), ((4096, 130), 0),
-                                       ((17, 1000), 2)])
+                                       ((17, 1000), 2),
+                                       # long columns: several stages of the large workgroup, a ragged last
+                                       # stage, fewer columns than a strip, even and odd pitches
+                                       ((2048, 2), 0), ((5000, 64), 2), ((6001, 36), 0), ((3000, 100), 3),
+                                       ((5000, 4), 0)])
 def test_gpu_half_reduce_keep_lowest(G, orc, stream, shape, pad):
     x = halves(orc, 21, shape)
-    if shape == (5000, 3):
+    if shape in ((5000, 3), (5000, 4)):
         x = orc.float2half(np.ones(shape, f32))       # saturates at 2048 only in row order
     src = G.to_device(x, pad)
     for variant in (0, 1):
