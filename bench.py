@@ -64,6 +64,11 @@ def algorithmic_bytes():
         "random_normal": e * 8192 * 32000,
         "ceiling_copy": 2 * e * 8192 * 32000,
         "ceiling_fill": e * 8192 * 32000,
+        # Copy(Tensor<gpu>, Tensor<gpu>): dense rows; rows of 32000 floats at a pitch of 32064; rows
+        # of 31990 floats at a pitch of 32000 (what AllocSpace gives them with padding on)
+        "copy_d2d": 2 * e * 8192 * 32000,
+        "copy_d2d_pitched": 2 * e * 8192 * 32000,
+        "copy_d2d_ragged": 2 * e * 8192 * 31990,
         "dot_f32_4096": 3 * e * 4096 * 4096,
         "dot_f16_8192": 3 * 2 * 8192 * 8192,
         # the same shapes on half_t tensors through the element-type-generic header paths
@@ -86,6 +91,7 @@ def work_elements():
         "lrn_scale_chpool5": 64 * 256 * 56 * 56, "transpose_nchw_nhwc": 64 * 256 * 56 * 56,
         "sort_by_key_f32": 1 << 24, "dot_f32_4096": 4096 * 4096, "dot_f16_8192": 8192 * 8192,
         "ceiling_copy": 8192 * 32000, "ceiling_fill": 8192 * 32000,
+        "copy_d2d": 8192 * 32000, "copy_d2d_pitched": 8192 * 32000, "copy_d2d_ragged": 8192 * 31990,
         "random_uniform": 8192 * 32000, "random_normal": 8192 * 32000,
         "softmax_f16": 8192 * 32000, "softmax_grad_f16": 8192 * 32000,
         "sum_rows_f16": 16384 * 4096, "sumall_except_dim1_f16": 64 * 256 * 56 * 56,
@@ -101,7 +107,7 @@ EXTRA_OPS = ("calib_copy", "smooth_softmax_grad_ignore", "softmax3d", "softmax3d
              "bias_add_broadcast", "swapaxis10_reshape", "lrn_scale_chpool5", "transpose_nchw_nhwc",
              "sort_by_key_f32", "dot_f32_4096", "dot_f16_8192", "ceiling_copy", "ceiling_fill",
              "random_uniform", "random_normal", "softmax_f16", "softmax_grad_f16", "sum_rows_f16",
-             "sumall_except_dim1_f16")
+             "sumall_except_dim1_f16", "copy_d2d", "copy_d2d_pitched", "copy_d2d_ragged")
 OPS = [k for k in algorithmic_bytes() if k not in EXTRA_OPS]
 
 # HBM bytes per launch of each operation's kernel come from the committed counter summary
@@ -183,6 +189,8 @@ def main():
     ap.add_argument("--only", default="", help="comma list of ops to run (profiling aid); "
                     "softmax_phases, ceiling_chain and ceiling_lds_loads run the probes of "
                     "libmshadow_probe.so instead")
+    ap.add_argument("--pattern", default="", help="with --only ceiling_lds_loads: one pattern "
+                    "'strip:width:waves' instead of the whole table (for a counter run)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; every operation of the path runs at its "
@@ -193,8 +201,9 @@ def main():
     if G.device_count() < 1:
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
     G.set_device(0)
-    if args.only in ("softmax_phases", "ceiling_chain", "ceiling_lds_loads"):
-        return run_probe(G, args.only)
+    if args.only in ("softmax_phases", "ceiling_chain", "ceiling_lds_loads", "ceiling_seg_loads",
+                     "softmax_prefetch_copy", "highdim_split_configs"):
+        return run_probe(G, args.only, args.pattern)
     props = G.props(0)
     only = [o for o in args.only.split(",") if o] or OPS
 
@@ -261,6 +270,9 @@ def main():
         extra["h2a"] = G.buffer((256,), np.uint16)
         G.case_softmax(extra["hP"], extra["hL"], s)
 
+    if any(o.startswith("copy_d2d_") for o in only):
+        extra["pitched_src"] = G.buffer(H["L"].shape, f32, pad=64)
+        extra["pitched_dst"] = G.buffer(H["L"].shape, f32, pad=64)
     if "dot_f32_4096" in only:   # dst = dot(A, B.T()) through the expression engine
         extra["mm_out"] = G.buffer((4096, 4096), f32)
     if "dot_f16_8192" in only:
@@ -273,6 +285,12 @@ def main():
     def run_op(name):
         if name == "ceiling_copy":     # dst = (src + 0) / 1 + 0 through the expression kernel
             G.case_map_axpb(out_g, dev["L"], 0.0, 1.0, 0.0, 0, s)
+        elif name == "copy_d2d":
+            G.case_copy_d2d(out_g, dev["L"], s)
+        elif name == "copy_d2d_pitched":
+            G.case_copy_d2d(extra["pitched_dst"], extra["pitched_src"], s)
+        elif name == "copy_d2d_ragged":
+            G.case_copy_d2d(out_g, dev["L"], s, cols=31990)
         elif name == "random_uniform":  # Random<gpu>::SampleUniform over 8192x32000 floats
             G.random_uniform(out_g, 7, 0, 0, -1.0, 1.0, s)
         elif name == "random_normal":   # Random<gpu>::SampleGaussian
@@ -457,7 +475,7 @@ def main():
     print(json.dumps(out))
 
 
-def run_probe(G, which):
+def run_probe(G, which, pattern=""):
     """`--only softmax_phases`: where a row of the 8192 x 32000 softmax spends its time (time
     stamps taken inside an instrumented build of the library's kernel). `--only ceiling_chain`:
     the cost of one dependent float add for a single wave, alone on the chip and with every CU
@@ -488,12 +506,68 @@ def run_probe(G, which):
         names = {0: "contiguous pieces, 1024 workgroups",
                  -1: "64 segments side by side per workgroup, 256 workgroups"}
         names.update({c: f"{c} columns of every row per workgroup" for c in (16, 32, 64)})
-        for strip in (0, -1, 16, 32, 64):
-            for width in (4, 16):
-                for waves in (4, 8, 16) if width == 4 else (2, 4, 8):
+        table = [(strip, width, waves) for strip in (0, -1, 16, 32, 64) for width in (4, 16)
+                 for waves in ((4, 8, 16) if width == 4 else (2, 4, 8))]
+        if pattern:
+            table = [tuple(int(v) for v in pattern.split(":"))]
+        for strip, width, waves in table:
+            if True:
+                if True:
                     us = min(P.dma_rate_us(src, strip, width, waves, s) for _ in range(3))
                     out["patterns"][f"{names[strip]}; {width} bytes per lane; {waves} waves"] = \
                         [round(us, 1), round(mb / us * 1e3)]
+    elif which == "ceiling_seg_loads":
+        # segments of 3136 floats one after the other as in a (n,c,56,56) tensor; 270 MB, more
+        # than the memory-side cache holds, so that a launch finds nothing from the one before
+        nseg = 21504
+        src = G.to_device(np.ones((nseg, 3136), f32))
+        mb = nseg * 3136 * 4 / 1e6
+        out = {"probe": "ceiling_seg_loads", "segments": [nseg, 3136],
+               "unit": "us to read the segments once (GB/s of what was read)", "patterns": {}}
+        for segs in (64, 32, 16, 8):
+            for width, waves, piece in ((4, 8, 1), (4, 16, 1), (4, 8, 7), (4, 4, 1), (16, 4, 1), (16, 8, 1),
+                                        (16, 8, 4), (16, 4, 4)):
+                per_seg = 3136 // (16 * width)
+                read = per_seg // piece * piece * 16 * width / 3136.0
+                us = min(P.seg_rate_us(src, 3136, nseg, segs, width, waves, piece, s) for _ in range(3))
+                out["patterns"][f"{segs} segments per workgroup ({nseg // segs} workgroups); {width} bytes per lane; "
+                                f"{waves} waves; pieces of {piece * 64 * width} bytes"] = \
+                    [round(us, 1), round(mb * read / us * 1e3)]
+    elif which == "highdim_split_configs":
+        out = {"probe": "highdim_split_configs", "unit": "us per launch (cold memory-side cache)", "shapes": {}}
+        names = {-1: "one workgroup per kept index", 0: "64 segments, 8 loader waves, 8 slots, 4 bytes per lane",
+                 1: "32, 8, 8, 4", 2: "16, 8, 4, 16", 3: "32, 8, 4, 16", 4: "16, 4, 8, 4", 5: "32, 8, 6, 4",
+                 6: "64, 8, 6, 4", 7: "32, 4, 8, 4", 8: "16, 8, 8, 4"}
+        for shape in ((64, 256, 56, 56), (64, 64, 112, 112), (256, 16, 112, 112), (64, 1024, 28, 28)):
+            x = np.random.default_rng(5).standard_normal(shape, dtype=f32)
+            a, b = G.to_device(x), G.to_device(x)
+            dst = G.buffer((shape[1],), f32)
+            res = {}
+            want = None
+            for cfg in sorted(names):
+                us = min(P.highdim_split_us(dst, a, b, cfg, s) for _ in range(3))
+                got = dst.download(s)
+                want = got if want is None else want
+                res[names[cfg]] = [round(us, 1), bool(np.array_equal(got.view(np.uint32), want.view(np.uint32)))]
+            out["shapes"]["x".join(map(str, shape))] = res
+    elif which == "softmax_prefetch_copy":
+        L = np.random.default_rng(7).standard_normal((8192, 32000), dtype=f32) * f32(3)
+        src, dst = G.to_device(L), G.buffer(L.shape, f32)
+        out = {"probe": "softmax_prefetch_copy", "shape": [8192, 32000], "unit": "us per copy of the matrix",
+               "row_copy_two_rows_per_cu": round(min(P.row_copy_us(dst, src, 0, 0, s) for _ in range(3)), 1),
+               "variants": {}}
+        for threads, pre, wgs in ((1024, 8, cus), (1024, 4, cus), (512, 8, 2 * cus), (512, 4, 2 * cus),
+                                  (512, 16, cus), (512, 4, 3 * cus)):
+            for barriers, spin in ((0, 0), (4, 4), (8, 8), (8, 16)):
+                us = min(P.row_copy_prefetch_us(dst, src, threads, pre, barriers, spin, wgs, s) for _ in range(3))
+                out["variants"][f"{threads} threads, {pre} KB per wave ahead in LDS, {wgs} workgroups; "
+                                f"{barriers} barriers x {spin} multiply-adds"] = round(us, 1)
+        G.fill(dst, 0.0, s)
+        P.row_copy_prefetch_us(dst, src, 1024, 8, 2, 0, cus, s)
+        ok = np.array_equal(dst.download(s), L)
+        G.fill(dst, 0.0, s)
+        P.row_copy_prefetch_us(dst, src, 512, 8, 2, 0, 2 * cus, s)
+        out["copy_is_exact"] = bool(ok and np.array_equal(dst.download(s), L))
     else:
         L = np.random.default_rng(7).standard_normal((8192, 32000), dtype=f32) * f32(3)
         src, dst = G.to_device(L), G.buffer(L.shape, f32)

@@ -100,7 +100,10 @@ int mshadow_hip_free(void *ptr);
 int mshadow_hip_malloc_host(void **host_ptr, size_t bytes);
 int mshadow_hip_free_host(void *host_ptr);
 /* Copy cpu<->gpu, gpu<->gpu: mshadow/tensor_gpu-inl.h:57-92 (cudaMemcpy2DAsync).
-   Pitches and width in BYTES here, like the runtime call it replaces. */
+   Pitches and width in BYTES here, like the runtime call it replaces. Device to device the
+   copy is a kernel of this library (streaming 128-bit or 32-bit accesses, any number of
+   bytes) when addresses, width and pitches are multiples of 4 bytes, the runtime's copy
+   otherwise; the two views must not overlap. */
 int mshadow_hip_memcpy2d_async(void *dst, size_t dpitch_bytes, const void *src,
                                size_t spitch_bytes, size_t width_bytes, size_t rows, int kind,
                                void *stream);
@@ -112,6 +115,11 @@ int mshadow_hip_memset_async(void *dst, int byte_value, size_t bytes, void *stre
    element count short of `int` rows and columns (runs of rows of less than 2^31 elements
    each are launched one after the other). */
 int mshadow_hip_fill_32(void *dst, int dstride, int rows, int cols, uint32_t bits, void *stream);
+/* The runs of whole rows mshadow_hip_fill_32 launches for a (rows, cols) view (wide != 0: rows
+   of 128-bit packs): first row and row count of up to max_runs runs into runs[2 i], runs[2 i + 1];
+   returns their number. Host arithmetic only - no launch, no device - so that the splitting can
+   be checked for shapes too large to allocate. No counterpart in the reference. */
+int mshadow_hip_fill_32_runs(int rows, int cols, int wide, int64_t *runs, int max_runs);
 
 /* ------------------------------------------------------------------ 2. launch */
 
@@ -260,6 +268,18 @@ int mshadow_hip_reduce_keep_lowest_f32(float *dst, const float *src, int sstride
 int mshadow_hip_reduce_keep_highdim_f32(float *dst, const float *src, int sstride, int n, int c,
                                         int y, int x, int reducer, int saver, float scale,
                                         void *stream);
+/* Scratch memory for a reduction kernel that spreads the inner (n, c) chains of
+   MapReduceKeepHighDim over more workgroups than there are kept indices (the reference's
+   kernel, tensor_gpu-inl.cuh:170-215, runs one block per kept index and needs none): `words`
+   32-bit words for the inner results and a block of counters that are zero between launches
+   (what the kernel template expects: mshadow/hip/kernels/reduce_dma.h), both inside
+   a device array that is part of the library (nothing is allocated). One slot per stream and
+   GPU, returned again on every call with that stream until mshadow_hip_stream_destroy; launches
+   that use it must be queued on that stream. *partial == NULL: none to be had (more words than
+   a slot holds, or every slot of the GPU taken) - the caller then runs a kernel that needs
+   none. Called by mshadow_hip_reduce_keep_highdim_f32 itself and by the header API for the
+   element types whose kernels are instantiated with the caller. */
+int mshadow_hip_reduce_scratch(void *stream, size_t words, uint32_t **partial, uint32_t **counter);
 
 /* dst = pool<Reducer>(src, Shape2(ph, pw), ky, kx, sy, sx): the MapPlanKernel launch of
    tensor_gpu-inl.cuh:67-120 with Plan<PoolingExp>::Eval (extension/spatial_pool.h:125-142)

@@ -185,6 +185,30 @@ int mshadow_case_col2im_f32(float *img, int istride, const float *col, int cstri
                             int h, int w, int ky, int kx, int sy, int sx, int dy, int dx,
                             int pad_y, int pad_x, int variant, void *stream);
 
+/* A convolutional network as one caller program (cases/conv_net.h; the network of the
+   reference's guide/neuralnet/convnet.cu:81-122 with today's signatures): `steps` rounds of
+   forward, backward and update on one batch, on one stream. geometry = {batch, in_channels,
+   in_size, channels, ksize, kstride, pad, psize, num_out}. Every pointer is host memory:
+   images (batch, in_channels, in_size, in_size), labels (batch, class numbers as floats),
+   fixed_grad NULL or (batch, num_out) to enter the backward pass instead of probs -
+   onehot(label), kernel (channels, in_channels * ksize^2) and weight (flat, num_out) in and
+   out, keep NULL or an array of host pointers (NULL each) that receive the tensors of the
+   last round in the order of conv_net::Kept. */
+int mshadow_case_conv_net_f32(const int *geometry, int steps, float eta, float decay,
+                              const float *images, const float *labels, const float *fixed_grad,
+                              float *kernel, float *weight, float *const *keep, void *stream);
+/* The convolution of that network and the gradient of its input alone, on float (half == 0)
+   or binary16 tensors: image -> pad -> unpack_patch2col -> product -> swapaxis(reshape), and
+   grad_out -> reshape(swapaxis) -> product -> pack_col2patch -> crop. Host memory. */
+int mshadow_case_conv_pair(int half, const int *geometry, const void *image, const void *kernel,
+                           const void *grad_out, void *col_forward, void *out, void *col_backward,
+                           void *image_grad, void *stream);
+
+/* Copy(Tensor<gpu,2,float> dst, Tensor<gpu,2,float> src, stream): device to device, either
+   side possibly pitched */
+int mshadow_case_copy_d2d_f32(float *dst, int dstride, const float *src, int sstride, int rows,
+                              int cols, void *stream);
+
 /* InitTensorEngine / NewStream / TensorContainer<gpu> / Copy (host -> device -> device ->
    host) / DeleteStream on host buffers of rows x cols floats; *device_stride receives the
    pitch AllocSpace chose with pad on or off. */

@@ -78,6 +78,8 @@ HIP_SYMBOLS = {
     "mshadow_hip_random_uniform_f64": ([_p, _i, _i, _i, C.c_uint64, C.c_uint64, C.c_uint64, C.c_double, C.c_double, _p], _i),
     "mshadow_hip_random_normal_f64": ([_p, _i, _i, _i, C.c_uint64, C.c_uint64, C.c_uint64, C.c_double, C.c_double, _p], _i),
     "mshadow_hip_fill_32": ([_p, _i, _i, _i, C.c_uint32, _p], _i),
+    "mshadow_hip_fill_32_runs": ([_i, _i, _i, C.POINTER(C.c_int64), _i], _i),
+    "mshadow_hip_reduce_scratch": ([_p, C.c_size_t, C.POINTER(_p), C.POINTER(_p)], _i),
     "mshadow_hip_permute_32": ([_p, _p, _i, C.POINTER(_i), C.POINTER(_i), _p], _i),
     "mshadow_hip_sort_by_key_workspace": ([_sz, C.POINTER(_sz)], _i),
     "mshadow_hip_sort_by_key_32": ([_p, _i, _p, _sz, _i, _p, _sz, _p], _i),
@@ -137,6 +139,9 @@ CASES_SYMBOLS = {
     "mshadow_case_col2im_f16": ([_p, _i, _p, _i] + [_i] * 13 + [_p], _i),
     "mshadow_case_col2im_f32": ([_p, _i, _p, _i] + [_i] * 13 + [_p], _i),
     "mshadow_case_copy_roundtrip_f32": ([_p, _p, _i, _i, _i, C.POINTER(_i)], _i),
+    "mshadow_case_copy_d2d_f32": ([_p, _i, _p, _i, _i, _i, _p], _i),
+    "mshadow_case_conv_net_f32": ([_p, _i, _f, _f, _p, _p, _p, _p, _p, _p, _p], _i),
+    "mshadow_case_conv_pair": ([_i, _p, _p, _p, _p, _p, _p, _p, _p, _p], _i),
 }
 
 
@@ -425,6 +430,11 @@ class Library:
         self.check_case(self.cases.mshadow_case_map_scalar_f32(dst.ptr, dst.stride, dst.rows,
                                                                dst.cols, scalar, saver, stream))
 
+    def case_copy_d2d(self, dst, src, stream=None, cols=None):
+        """Copy(dst, src, stream) on device tensors; `cols` narrows both to their first columns"""
+        self.check_case(self.cases.mshadow_case_copy_d2d_f32(
+            dst.ptr, dst.stride, src.ptr, src.stride, dst.rows, dst.cols if cols is None else cols, stream))
+
     def case_map_axpb(self, dst, a, s1, s2, s3, saver=SAVETO, stream=None):
         self.check_case(self.cases.mshadow_case_map_axpb_f32(
             dst.ptr, dst.stride, a.ptr, a.stride, dst.rows, dst.cols, s1, s2, s3, saver, stream))
@@ -631,7 +641,7 @@ class Library:
 
 
 class Probe:
-    """libmshadow_probe.so: measurement aids of bench.py (include/mshadow_hip_probe.h)"""
+    """libmshadow_probe.so: measurement aids of bench.py (csrc/mshadow_hip_probe.h)"""
     STAMPS = 16
     STAMP_ORDER = (10, 11, 12, 13, 1, 2, 6, 8, 3, 4, 5, 14)
     STAMP_NAMES = ("entry", "row loaded, thread maxima", "row maximum (barrier)", "exp",
@@ -657,6 +667,31 @@ class Probe:
         self.dll.mshadow_probe_row_copy.argtypes = [_p, _i, _p, _i, _i, _i, _i, _i, _i, C.POINTER(C.c_double), _p]
         self._check(self.dll.mshadow_probe_row_copy(dst.ptr, dst.stride, src.ptr, src.stride, src.rows,
                                                     src.cols, barriers, spin, resident, C.byref(us), stream))
+        return us.value
+
+    def row_copy_prefetch_us(self, dst, src, threads, prefetch_slabs, barriers, spin, workgroups, stream=None):
+        us = C.c_double(0)
+        self.dll.mshadow_probe_row_copy_prefetch.argtypes = [_p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _i,
+                                                             C.POINTER(C.c_double), _p]
+        self._check(self.dll.mshadow_probe_row_copy_prefetch(
+            dst.ptr, dst.stride, src.ptr, src.stride, src.rows, src.cols, threads, prefetch_slabs,
+            barriers, spin, workgroups, C.byref(us), stream))
+        return us.value
+
+    def seg_rate_us(self, src, seg_len, nseg, segs, width, waves, piece_instr, stream=None):
+        us = C.c_double(0)
+        self.dll.mshadow_probe_seg_rate.argtypes = [_p, C.c_size_t, _i, _i, _i, _i, _i, _i,
+                                                    C.POINTER(C.c_double), _p]
+        self._check(self.dll.mshadow_probe_seg_rate(src.ptr, src.rows * src.stride, seg_len, nseg, segs,
+                                                    width, waves, piece_instr, C.byref(us), stream))
+        return us.value
+
+    def highdim_split_us(self, dst, warm, src, config, stream=None):
+        n, c, y, x = src.shape
+        us = C.c_double(0)
+        self.dll.mshadow_probe_highdim_split.argtypes = [_p, _p, _p, _i, _i, _i, _i, _i, C.POINTER(C.c_double), _p]
+        self._check(self.dll.mshadow_probe_highdim_split(dst.ptr, warm.ptr, src.ptr, n, c, y, x, config,
+                                                         C.byref(us), stream))
         return us.value
 
     def dma_rate_us(self, src, strip, width, waves, stream=None, window=32):

@@ -13,6 +13,7 @@
 
 #include "portable_math.h"
 #include "two_layer_net.h"
+#include "conv_net.h"
 
 using namespace mshadow;
 using namespace mshadow::expr;
@@ -674,6 +675,40 @@ int mshadow_case_two_layer_net_f32(int steps, float eta, float decay, int batch,
   CASE_END
 }
 
+/* conv_net::Train on the device; every pointer is HOST memory (the program copies) */
+int mshadow_case_conv_net_f32(const int *geometry, int steps, float eta, float decay,
+                              const float *images, const float *labels, const float *fixed_grad,
+                              float *kernel, float *weight, float *const *keep, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  const conv_net::Geometry g = {geometry[0], geometry[1], geometry[2], geometry[3], geometry[4],
+                                geometry[5], geometry[6], geometry[7], geometry[8]};
+  conv_net::Train<gpu>(st.get(), g, steps, eta, decay, images, labels, fixed_grad, kernel, weight, keep);
+  CASE_END
+}
+
+/* conv_net::ConvPair on the device for float (half == 0) or binary16 elements; HOST memory */
+int mshadow_case_conv_pair(int half, const int *geometry, const void *image, const void *kernel,
+                           const void *grad_out, void *col_forward, void *out, void *col_backward,
+                           void *image_grad, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  const conv_net::Geometry g = {geometry[0], geometry[1], geometry[2], geometry[3], geometry[4],
+                                geometry[5], geometry[6], geometry[7], geometry[8]};
+  if (half) {
+    conv_net::ConvPair<gpu, HalfT>(st.get(), g, static_cast<const HalfT *>(image),
+                                   static_cast<const HalfT *>(kernel), static_cast<const HalfT *>(grad_out),
+                                   static_cast<HalfT *>(col_forward), static_cast<HalfT *>(out),
+                                   static_cast<HalfT *>(col_backward), static_cast<HalfT *>(image_grad));
+  } else {
+    conv_net::ConvPair<gpu, float>(st.get(), g, static_cast<const float *>(image),
+                                   static_cast<const float *>(kernel), static_cast<const float *>(grad_out),
+                                   static_cast<float *>(col_forward), static_cast<float *>(out),
+                                   static_cast<float *>(col_backward), static_cast<float *>(image_grad));
+  }
+  CASE_END
+}
+
 int mshadow_case_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes,
                           int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,
                           int reducer, int variant, void *stream) {
@@ -760,6 +795,14 @@ CASE_IM2COL(mshadow_case_im2col_f32, float, float)
   }
 CASE_COL2IM(mshadow_case_col2im_f16, uint16_t, half::half_t)
 CASE_COL2IM(mshadow_case_col2im_f32, float, float)
+
+int mshadow_case_copy_d2d_f32(float *dst, int dstride, const float *src, int sstride, int rows,
+                              int cols, void *stream) {
+  CASE_BEGIN
+  BorrowedStream st(stream);
+  Copy(G2(dst, rows, cols, dstride, st.get()), G2(src, rows, cols, sstride, st.get()), st.get());
+  CASE_END
+}
 
 int mshadow_case_copy_roundtrip_f32(float *host_out, const float *host_in, int rows, int cols,
                                     int pad, int *device_stride) {

@@ -33,6 +33,16 @@ inline hipStream_t AsStream(void *s) { return reinterpret_cast<hipStream_t>(s); 
    (mshadow/cuda/tensor_gpu-inl.cuh:16-21); hipGetLastError also clears the sticky code */
 inline int AfterLaunch(const char *what) { return FromHip(hipGetLastError(), what); }
 
+/* compute units of the calling thread's device (looked up once per thread) */
+int ComputeUnits();
+
+/* device-to-device copy of a pitched view by the library's own kernel; false: not covered */
+bool CopyRowsOnDevice(void *dst, size_t dpitch_bytes, const void *src, size_t spitch_bytes,
+                      size_t width_bytes, size_t rows, hipStream_t s);
+
+/* a stream is going away: whatever scratch memory of the library it was given is free again */
+void ReleaseReduceScratch(void *stream);
+
 }  // namespace mshadow_abi
 
 #define ABI_HIP(call)                                              \

@@ -1,6 +1,6 @@
 /*
  * libmshadow_probe - measurement aids used by bench.py (`--only softmax_phases`,
- * `--only ceiling_chain`). They have no counterpart in the reference and are no part of
+ * `--only ceiling_chain`, ...). They have no counterpart in the reference and are no part of
  * the device layer: libmshadow_hip.so and the mshadow headers do not depend on them.
  * Same conventions as mshadow_hip.h: 0 on success, text from mshadow_probe_last_error().
  */
@@ -53,6 +53,32 @@ int mshadow_probe_softmax_phases(float *dst, int dstride, const float *src, int 
 int mshadow_probe_row_copy(float *dst, int dstride, const float *src, int sstride, int rows,
                            int cols, int barriers, int spin, int resident, double *kernel_us,
                            void *stream);
+
+/* The row copy as persistent workgroups fed from their own next row: `workgroups` workgroups
+   of `threads` threads (1024: one per CU, 512: two) take rows in turn; while a row is in
+   registers (stand-in work as above, then its stores) the first `prefetch_slabs` kilobytes per
+   wave of the workgroup's next row are loaded straight into LDS, the rest when the row's turn
+   comes. 28672 < cols <= 32768. */
+int mshadow_probe_row_copy_prefetch(float *dst, int dstride, const float *src, int sstride, int rows,
+                                    int cols, int threads, int prefetch_slabs, int barriers, int spin,
+                                    int workgroups, double *kernel_us, void *stream);
+
+/* Rate of loads into LDS when workgroup b reads segments b * segs .. b * segs + segs - 1 of
+   `seg_len` floats each (they lie one after the other in memory) side by side, `piece_instr`
+   instructions (64 * width bytes each) of one segment, then of the next: nseg / segs
+   workgroups of `waves` waves. The part of a segment that does not fill a round of pieces is
+   not read. */
+int mshadow_probe_seg_rate(const float *src, size_t floats, int seg_len, int nseg, int segs, int width,
+                           int waves, int piece_instr, double *kernel_us, void *stream);
+
+/* sumall_except_dim<1> over a dense (n, c, y, x) float tensor with the inner chains dealt out
+   in groups of segments (kernels/reduce_dma.h), for a choice of segments per workgroup, loader
+   waves, ring slots and bytes per lane and load: config 0..8 = (64,8,8,4) (32,8,8,4) (16,8,4,16)
+   (32,8,4,16) (16,4,8,4) (32,8,6,4) (64,8,6,4) (32,4,8,4) (16,8,8,4); config -1 = one workgroup
+   per kept index. The timed launch reads `src`
+   after a launch on `warm` (another tensor of the shape). kernel_us = its duration. */
+int mshadow_probe_highdim_split(float *dst, const float *warm, const float *src, int n, int c, int y,
+                                int x, int config, double *kernel_us, void *stream);
 
 /* Rate of loads from global memory straight into LDS (the loads of the reduction kernels),
    with nothing consuming the data: `waves` waves per workgroup keep window .. window + 16

@@ -6,6 +6,8 @@
  */
 #include "abi_common.h"
 
+#include <mutex>
+
 #include <mshadow/hip/kernels/reduce.h>
 #include <mshadow/hip/kernels/reduce_dma.h>
 
@@ -330,6 +332,80 @@ void LaunchShortSoftmax(float *dst, int dstride, const float *src, int sstride, 
 }
 }  // namespace
 
+/* Scratch memory of the split KeepHighDim reduction (kernels/reduce_dma.h): the inner results of
+   a launch and the counter that tells the last workgroup. It is part of the library's image
+   - a file-scope device array, one copy per GPU, nothing is allocated at run time - and is
+   handed out per stream: launches on one stream run one after the other, so a stream's slot is
+   never in use twice; a ninth stream on one GPU, or a launch with more inner results than a
+   slot holds, gets none and its reduction runs the one-workgroup-per-kept-index kernel. */
+namespace {
+const int kReduceScratchSlots = 8;
+const size_t kReduceScratchWords = 1u << 16;
+const int kReduceScratchDevices = 16;
+struct ReduceScratchSlot {
+  uint32_t partial[kReduceScratchWords];
+  uint32_t counter[mshadow::hip::kSplitCounterWords];  // zero between launches
+};
+static __device__ __align__(256) ReduceScratchSlot g_reduce_scratch[kReduceScratchSlots];
+
+struct ReduceScratchTable {
+  std::mutex mu;
+  ReduceScratchSlot *base[kReduceScratchDevices];
+  bool used[kReduceScratchDevices][kReduceScratchSlots];
+  void *owner[kReduceScratchDevices][kReduceScratchSlots];
+};
+ReduceScratchTable &ScratchTable() {
+  static ReduceScratchTable t = {};
+  return t;
+}
+}  // namespace
+
+namespace mshadow_abi {
+void ReleaseReduceScratch(void *stream) {
+  ReduceScratchTable &t = ScratchTable();
+  std::lock_guard<std::mutex> lock(t.mu);
+  for (int d = 0; d < kReduceScratchDevices; ++d) {
+    for (int i = 0; i < kReduceScratchSlots; ++i) {
+      if (t.used[d][i] && t.owner[d][i] == stream) t.used[d][i] = false;
+    }
+  }
+}
+}  // namespace mshadow_abi
+
+extern "C" int mshadow_hip_reduce_scratch(void *stream, size_t words, uint32_t **partial,
+                                          uint32_t **counter) {
+  ABI_REQUIRE(partial != NULL && counter != NULL, "NULL result");
+  *partial = NULL;
+  *counter = NULL;
+  if (words > kReduceScratchWords) return MSHADOW_HIP_OK;
+  int dev = 0;
+  ABI_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kReduceScratchDevices) return MSHADOW_HIP_OK;
+  ReduceScratchTable &t = ScratchTable();
+  std::lock_guard<std::mutex> lock(t.mu);
+  if (t.base[dev] == NULL) {
+    /* the array's name is a host-side stand-in; this is its address on the current device */
+    void *p = NULL;
+    ABI_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(g_reduce_scratch)));
+    t.base[dev] = static_cast<ReduceScratchSlot *>(p);
+  }
+  int slot = -1;
+  for (int i = 0; i < kReduceScratchSlots && slot < 0; ++i) {
+    if (t.used[dev][i] && t.owner[dev][i] == stream) slot = i;
+  }
+  for (int i = 0; i < kReduceScratchSlots && slot < 0; ++i) {
+    if (!t.used[dev][i]) {
+      t.used[dev][i] = true;
+      t.owner[dev][i] = stream;
+      slot = i;
+    }
+  }
+  if (slot < 0) return MSHADOW_HIP_OK;
+  *partial = t.base[dev][slot].partial;
+  *counter = t.base[dev][slot].counter;
+  return MSHADOW_HIP_OK;
+}
+
 extern "C" {
 
 /* ------------------------------------------------------------------ softmax */
@@ -612,6 +688,27 @@ int mshadow_hip_reduce_keep_highdim_f32(float *dst, const float *src, int sstrid
   RawPlan2D<const float> sp = {src, sstride};
   const mshadow::FastDivU32 div_x(static_cast<uint32_t>(x > 0 ? x : 1));
   hipStream_t s = AsStream(stream);
+  /* The split kernel walks dense rows as one row per segment. It needs scratch memory for
+     n * c inner results. */
+  int v_y = y, v_x = x, v_stride = sstride;
+  if (sstride == x) {
+    v_x = v_stride = y * x;
+    v_y = 1;
+  }
+  uint32_t *split_partial = NULL, *split_counter = NULL;
+  /* With a kept index for (nearly) every CU the one-workgroup-per-kept-index kernel fills the
+     chip and ends without a merge; with fewer the inner chains are dealt out by segments:
+     16 per workgroup and a kilobyte of each per load where rows are whole 16-byte packs, else
+     32 per workgroup and 256 bytes of each. */
+  const bool few_kept = static_cast<long long>(c) * 4 < 3ll * mshadow_abi::ComputeUnits();
+  const bool whole_packs = v_x % 4 == 0 && v_stride % 4 == 0 && Aligned16(src);
+  if (few_kept && static_cast<long long>(n) * y * x >= kDmaMinPerKept &&
+      static_cast<long long>(n) * c < (1ll << 31)) {
+    const int sc = mshadow_hip_reduce_scratch(stream, static_cast<size_t>(n) * c, &split_partial,
+                                              &split_counter);
+    if (sc != MSHADOW_HIP_OK) return sc;
+  }
+  const mshadow::FastDivU32 v_div_x(static_cast<uint32_t>(v_x > 0 ? v_x : 1));
   int st = DispatchReducer(reducer, [&](auto red) {
     return DispatchSaver(saver, [&](auto sv) {
       typedef decltype(red) R;
@@ -631,6 +728,22 @@ int mshadow_hip_reduce_keep_highdim_f32(float *dst, const float *src, int sstrid
                        static_cast<uint32_t>(x), div_x, scale);                                \
   else HIGHDIM_LAUNCH_T(mshadow::hip::kRedBlockSmall, SEGS)
       const bool large = static_cast<long long>(n) * y * x >= kDmaMinPerKept;
+      if (large && split_partial != NULL) {
+#define HIGHDIM_SPLIT(RING)                                                                    \
+  hipLaunchKernelGGL((mshadow::hip::ReduceKeepHighDimSplitKernel<S, R, float, RING>),          \
+                     dim3((static_cast<unsigned>(n) * c + RING::kSegs - 1) / RING::kSegs),      \
+                     dim3(RING::kThreads), 0, s, dst, src, static_cast<uint32_t>(v_stride),    \
+                     static_cast<uint32_t>(n), static_cast<uint32_t>(c),                       \
+                     static_cast<uint32_t>(v_y), static_cast<uint32_t>(v_x), v_div_x, scale,   \
+                     split_partial, split_counter)
+        if (whole_packs) {
+          HIGHDIM_SPLIT(mshadow::hip::HighDimSplitRingPacks);
+        } else {
+          HIGHDIM_SPLIT(mshadow::hip::HighDimSplitRing);
+        }
+#undef HIGHDIM_SPLIT
+        return MSHADOW_HIP_OK;
+      }
       if (n > 16) { HIGHDIM_LAUNCH(64); }
       else if (n > 4) { HIGHDIM_LAUNCH(16); }
       else if (n > 1) { HIGHDIM_LAUNCH(4); }

@@ -12,7 +12,7 @@
  */
 #include <hip/hip_runtime.h>
 #include <mshadow_hip.h>
-#include <mshadow_hip_probe.h>
+#include "mshadow_hip_probe.h"
 
 #include <algorithm>
 #include <functional>
@@ -40,6 +40,13 @@ const int kStampSlots = MSHADOW_PROBE_STAMPS;
 #include "softmax_kernels.h"
 
 #include <mshadow/hip/kernels/reduce.h>
+#define ReduceKeepHighDimSplitKernel ReduceKeepHighDimSplitProbeKernel
+#define ReduceKeepHighDimDmaKernel ReduceKeepHighDimDmaProbeKernel
+#define ReduceKeepLowestDmaKernel ReduceKeepLowestDmaProbeKernel
+#include <mshadow/hip/kernels/reduce_dma.h>
+#undef ReduceKeepHighDimSplitKernel
+#undef ReduceKeepHighDimDmaKernel
+#undef ReduceKeepLowestDmaKernel
 
 #include "abi_common.h"
 
@@ -149,6 +156,112 @@ __global__ void __launch_bounds__(THREADS, 4)
   }
 }
 
+
+/*! \brief the row copy as a persistent workgroup that is fed from its own next row: while a
+ *  row sits in registers (stand-in work, then its stores), the first PRE slabs of the
+ *  workgroup's next row are already on their way into LDS by loads that bypass the registers;
+ *  the rest of a row (SLABS - PRE slabs) is loaded into registers when the row's turn comes.
+ *  A wave reads back from LDS exactly the bytes its own loads delivered, so the hand-over
+ *  needs a wait on the wave's own counter and no barrier. The counter retires loads and
+ *  stores in issue order: the wait leaves the stores of the row before and the direct
+ *  loads of this row outstanding (at most the last slab of either is skipped by a wave). */
+template <int THREADS, int SLABS, int PRE>
+__global__ void __launch_bounds__(THREADS)
+    RowCopyPrefetchKernel(float *dst, int dstride, const float *src, int sstride, int rows, int cols,
+                          int barriers, int spin) {
+  using mshadow_hipk::F4;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const int W = THREADS / 64;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int lane_col = lane * 4;
+  unsigned char *mine = lds + static_cast<size_t>(wave) * PRE * 1024;
+  auto prefetch = [&](int row) {
+    const float *in = src + static_cast<size_t>(row) * sstride;
+#pragma unroll
+    for (int j = 0; j < PRE; ++j) {
+      int col = (j * W + wave) * 256 + lane_col;
+      col = col < cols ? col : cols - 4;  // clamped, never consumed
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(in + col),
+                                       (__attribute__((address_space(3))) void *)(mine + j * 1024), 16, 0,
+                                       2);
+    }
+  };
+  int row = blockIdx.x;
+  if (row < rows) prefetch(row);
+  for (; row < rows; row += gridDim.x) {
+    const float *in = src + static_cast<size_t>(row) * sstride;
+    float *out = dst + static_cast<size_t>(row) * dstride;
+    F4 v[SLABS];
+#pragma unroll
+    for (int j = PRE; j < SLABS; ++j) {
+      const int c0 = (j * W + wave) * 256;
+      v[j] = F4{0.0f, 0.0f, 0.0f, 0.0f};
+      if (c0 + lane_col < cols) v[j] = mshadow_hipk::StreamLoadF4(in + c0 + lane_col);
+    }
+    const int kLater = (SLABS - 1) + (PRE < SLABS ? SLABS - PRE - 1 : 0);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLater) : "memory");
+#pragma unroll
+    for (int j = 0; j < PRE; ++j) v[j] = *reinterpret_cast<const F4 *>(mine + j * 1024 + lane * 16);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (row + static_cast<int>(gridDim.x) < rows) prefetch(row + gridDim.x);
+    for (int b = 0; b < barriers; ++b) {
+      for (int k = 0; k < spin; ++k) {
+#pragma unroll
+        for (int j = 0; j < SLABS; ++j) v[j] = v[j] * 1.0000001f + 1e-9f;
+      }
+      asm volatile("s_barrier" ::: "memory");
+    }
+#pragma unroll
+    for (int j = 0; j < SLABS; ++j) {
+      const int c0 = (j * W + wave) * 256;
+      if (c0 + lane_col < cols) mshadow_hipk::StreamStoreF4(out + c0 + lane_col, v[j]);
+    }
+  }
+}
+
+/* Rate of loads into LDS when a workgroup reads `segs` neighbouring segments of `seg_len`
+   floats side by side (64 * WIDTH bytes of each in turn), workgroup b taking segments
+   b * segs .. b * segs + segs - 1: the pattern of a reduction whose inner chains run one per
+   lane over segments that lie one after the other in memory. */
+template <int WIDTH>
+__global__ void __launch_bounds__(1024) SegRateKernel(const float *src, uint32_t seg_len, uint32_t segs,
+                                                      uint32_t piece_instr) {
+  const int kRegion = 16 * 64 * WIDTH;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t nwave = blockDim.x >> 6;
+  const uint32_t lane = threadIdx.x & 63;
+  unsigned char *mine = lds + wave * kRegion;
+  const int kFloats = WIDTH / 4;
+  const uint32_t per_seg = seg_len / (64 * kFloats);          // instructions per segment
+  const uint32_t turns = per_seg / piece_instr;               // rounds over the segments
+  const uint32_t ninstr = segs * turns * piece_instr / nwave;  // per wave
+  const float *base = src + static_cast<size_t>(blockIdx.x) * segs * seg_len + lane * kFloats;
+  for (uint32_t i = 0; i + 16 <= ninstr; i += 16) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      const uint32_t t = (i + q) * nwave + wave;
+      /* t counts instructions in the order (turn, segment, instruction of the piece) */
+      const uint32_t in_piece = t % piece_instr;
+      const uint32_t u = t / piece_instr;
+      const uint32_t seg = u % segs, turn = u / segs;
+      const size_t at = static_cast<size_t>(seg) * seg_len +
+                        static_cast<size_t>(turn * piece_instr + in_piece) * 64 * kFloats;
+      const __attribute__((address_space(1))) void *from =
+          (const __attribute__((address_space(1))) void *)(base + at);
+      __attribute__((address_space(3))) void *to =
+          (__attribute__((address_space(3))) void *)(mine + q * 64 * WIDTH);
+      if (WIDTH == 4) {
+        __builtin_amdgcn_global_load_lds(from, to, 4, 0, 2);
+      } else {
+        __builtin_amdgcn_global_load_lds(from, to, 16, 0, 2);
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
 
 /* Rate of loads from global memory straight into LDS, nothing else: `blockDim.x / 64` waves
    per workgroup issue them in batches of 16 and wait until `window` (16 or 32) are left
@@ -305,6 +418,128 @@ int mshadow_probe_row_copy(float *dst, int dstride, const float *src, int sstrid
   if (st != MSHADOW_HIP_OK) return st;
   *kernel_us = ms * 1e3;
   return MSHADOW_HIP_OK;
+}
+
+int mshadow_probe_row_copy_prefetch(float *dst, int dstride, const float *src, int sstride, int rows,
+                                    int cols, int threads, int prefetch_slabs, int barriers, int spin,
+                                    int workgroups, double *kernel_us, void *stream) {
+  ABI_REQUIRE(rows >= 1 && cols > 28672 && cols <= 32768 && cols % 4 == 0 && sstride % 4 == 0 &&
+                  dstride % 4 == 0 && kernel_us != NULL, "28672 < cols <= 32768, rows of whole packs");
+  ABI_REQUIRE(workgroups >= 1 && workgroups <= rows, "1..rows workgroups");
+  ABI_REQUIRE(reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0,
+              "16-byte aligned");
+  hipStream_t s = AsStream(stream);
+  float ms = 0.0f;
+  int st = MSHADOW_HIP_ERR_ARGUMENT;
+#define PROBE_PREFETCH(T, SL, PRE)                                                                  \
+  if (threads == T && prefetch_slabs == PRE) {                                                      \
+    const size_t lds = static_cast<size_t>(T) / 64 * PRE * 1024;                                    \
+    ABI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&RowCopyPrefetchKernel<T, SL, PRE>), \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));           \
+    st = TimeKernel(s, &ms, [&] {                                                                   \
+      hipLaunchKernelGGL((RowCopyPrefetchKernel<T, SL, PRE>), dim3(workgroups), dim3(T), lds, s, dst, \
+                         dstride, src, sstride, rows, cols, barriers, spin);                        \
+    });                                                                                             \
+  }
+  PROBE_PREFETCH(1024, 8, 8)
+  PROBE_PREFETCH(1024, 8, 4)
+  PROBE_PREFETCH(512, 16, 8)
+  PROBE_PREFETCH(512, 16, 4)
+  PROBE_PREFETCH(512, 16, 16)
+#undef PROBE_PREFETCH
+  ABI_REQUIRE(st != MSHADOW_HIP_ERR_ARGUMENT, "threads / prefetch_slabs: 1024 with 8 or 4, 512 with 16, 8 or 4");
+  if (st != MSHADOW_HIP_OK) return st;
+  *kernel_us = ms * 1e3;
+  return MSHADOW_HIP_OK;
+}
+
+int mshadow_probe_seg_rate(const float *src, size_t floats, int seg_len, int nseg, int segs, int width,
+                           int waves, int piece_instr, double *kernel_us, void *stream) {
+  ABI_REQUIRE(src != NULL && kernel_us != NULL && seg_len >= 64 && nseg >= 1 && segs >= 1, "bad argument");
+  ABI_REQUIRE(static_cast<size_t>(seg_len) * nseg <= floats && nseg % segs == 0, "segments beyond the buffer");
+  ABI_REQUIRE((width == 4 || width == 16) && waves >= 1 && waves <= 16 && piece_instr >= 1, "bad argument");
+  ABI_REQUIRE(seg_len % 4 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0, "16-byte aligned segments");
+  hipStream_t s = AsStream(stream);
+  const size_t lds = static_cast<size_t>(waves) * 16 * 64 * width;
+  float ms = 0.0f;
+  int st;
+  if (width == 4) {
+    st = TimeKernel(s, &ms, [&] {
+      hipLaunchKernelGGL((SegRateKernel<4>), dim3(nseg / segs), dim3(waves * 64), lds, s, src,
+                         static_cast<uint32_t>(seg_len), static_cast<uint32_t>(segs),
+                         static_cast<uint32_t>(piece_instr));
+    });
+  } else {
+    ABI_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&SegRateKernel<16>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    st = TimeKernel(s, &ms, [&] {
+      hipLaunchKernelGGL((SegRateKernel<16>), dim3(nseg / segs), dim3(waves * 64), lds, s, src,
+                         static_cast<uint32_t>(seg_len), static_cast<uint32_t>(segs),
+                         static_cast<uint32_t>(piece_instr));
+    });
+  }
+  if (st != MSHADOW_HIP_OK) return st;
+  *kernel_us = ms * 1e3;
+  return MSHADOW_HIP_OK;
+}
+
+int mshadow_probe_highdim_split(float *dst, const float *warm, const float *src, int n, int c, int y,
+                                int x, int config, double *kernel_us, void *stream) {
+  using namespace mshadow::hip;
+  ABI_REQUIRE(dst != NULL && warm != NULL && src != NULL && kernel_us != NULL, "NULL argument");
+  ABI_REQUIRE(n >= 1 && c >= 1 && (static_cast<long long>(y) * x) % 4 == 0 && y * x >= 4, "segments of whole packs");
+  hipStream_t s = AsStream(stream);
+  uint32_t *scratch = NULL;
+  const size_t words = static_cast<size_t>(n) * c;
+  ABI_HIP(hipMalloc(&scratch, (words + kSplitCounterWords) * 4));
+  ABI_HIP(hipMemsetAsync(scratch, 0, (words + kSplitCounterWords) * 4, s));
+  uint32_t *counter = scratch + words;
+  const uint32_t seg = static_cast<uint32_t>(y) * x;
+  const mshadow::FastDivU32 div_seg(seg), div_x(static_cast<uint32_t>(x));
+  hipEvent_t a, b;
+  ABI_HIP(hipEventCreate(&a));
+  ABI_HIP(hipEventCreate(&b));
+  typedef mshadow::sv::saveto SV;
+  typedef mshadow::red::sum RD;
+  auto launch = [&](const float *from) {
+#define PROBE_SPLIT(ID, SEGS, LOADERS, SLOTS, W)                                                    \
+  if (config == ID) {                                                                               \
+    typedef SplitRing<SEGS, LOADERS, SLOTS, W> Ring;                                                \
+    hipLaunchKernelGGL((ReduceKeepHighDimSplitProbeKernel<SV, RD, float, Ring>),                    \
+                       dim3((n * c + SEGS - 1) / SEGS), dim3(Ring::kThreads), 0, s, dst, from, seg, \
+                       static_cast<uint32_t>(n), static_cast<uint32_t>(c), 1u, seg, div_seg, 1.0f,  \
+                       scratch, counter);                                                           \
+  }
+    PROBE_SPLIT(0, 64, 8, 8, 4)
+    PROBE_SPLIT(1, 32, 8, 8, 4)
+    PROBE_SPLIT(2, 16, 8, 4, 16)
+    PROBE_SPLIT(3, 32, 8, 4, 16)
+    PROBE_SPLIT(4, 16, 4, 8, 4)
+    PROBE_SPLIT(5, 32, 8, 6, 4)
+    PROBE_SPLIT(6, 64, 8, 6, 4)
+    PROBE_SPLIT(7, 32, 4, 8, 4)
+    PROBE_SPLIT(8, 16, 8, 8, 4)
+#undef PROBE_SPLIT
+    if (config < 0) {
+      hipLaunchKernelGGL((ReduceKeepHighDimDmaProbeKernel<SV, RD, float, 64>), dim3(c), dim3(kDmaThreads), 0,
+                         s, dst, from, static_cast<uint32_t>(x), static_cast<uint32_t>(n),
+                         static_cast<uint32_t>(c), static_cast<uint32_t>(y), static_cast<uint32_t>(x),
+                         div_x, 1.0f);
+    }
+  };
+  launch(src);
+  launch(warm);   // what the timed launch reads is no longer in the memory-side cache
+  ABI_HIP(hipEventRecord(a, s));
+  launch(src);
+  ABI_HIP(hipEventRecord(b, s));
+  ABI_HIP(hipEventSynchronize(b));
+  float ms = 0.0f;
+  ABI_HIP(hipEventElapsedTime(&ms, a, b));
+  ABI_HIP(hipEventDestroy(a));
+  ABI_HIP(hipEventDestroy(b));
+  ABI_HIP(hipFree(scratch));
+  *kernel_us = ms * 1e3;
+  return AfterLaunch("probe kernel");
 }
 
 int mshadow_probe_softmax_phases(float *dst, int dstride, const float *src, int sstride, int rows,

@@ -1,6 +1,7 @@
 /*
  * C ABI, groups 1 and 2: device / stream / event / memory / copy and the generic
- * kernel launch. Thin, stateless wrappers over the HIP runtime; see
+ * kernel launch. Thin, stateless wrappers over the HIP runtime (copies between device
+ * tensors run a kernel of the library where alignment allows); see
  * include/mshadow_hip.h for the contract of each entry point.
  */
 #include "abi_common.h"
@@ -11,6 +12,23 @@ namespace mshadow_abi {
 std::string &LastError() {
   static thread_local std::string msg;
   return msg;
+}
+}  // namespace mshadow_abi
+
+namespace mshadow_abi {
+int ComputeUnits() {
+  static thread_local int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) {
+      cus = p.multiProcessorCount;
+    } else {
+      (void)hipGetLastError();
+      cus = 256;  // MI355X
+    }
+  }
+  return cus;
 }
 }  // namespace mshadow_abi
 
@@ -73,6 +91,7 @@ int mshadow_hip_stream_create(void **stream) {
 }
 int mshadow_hip_stream_destroy(void *stream) {
   if (stream == NULL) return MSHADOW_HIP_OK;
+  ReleaseReduceScratch(stream);
   ABI_HIP(hipStreamDestroy(AsStream(stream)));
   return MSHADOW_HIP_OK;
 }
@@ -165,6 +184,10 @@ int mshadow_hip_memcpy2d_async(void *dst, size_t dpitch_bytes, const void *src,
   if (width_bytes == 0 || rows == 0) return MSHADOW_HIP_OK;
   ABI_REQUIRE(dst != NULL && src != NULL, "NULL buffer");
   ABI_REQUIRE(dpitch_bytes >= width_bytes && spitch_bytes >= width_bytes, "pitch < width");
+  if (kind == MSHADOW_HIP_D2D &&
+      CopyRowsOnDevice(dst, dpitch_bytes, src, spitch_bytes, width_bytes, rows, AsStream(stream))) {
+    return AfterLaunch("copy");
+  }
   if (dpitch_bytes == width_bytes && spitch_bytes == width_bytes) {
     ABI_HIP(hipMemcpyAsync(dst, src, width_bytes * rows, k, AsStream(stream)));
   } else {
@@ -195,17 +218,7 @@ int mshadow_hip_peek_last_error(void) { return FromHip(hipPeekAtLastError(), "pe
 int mshadow_hip_suggest_grid(size_t work_items, size_t items_per_block, int max_waves,
                              uint32_t *grid_x) {
   ABI_REQUIRE(grid_x != NULL && items_per_block > 0, "bad argument");
-  static thread_local int cus = 0;
-  if (cus == 0) {
-    int dev = 0;
-    hipDeviceProp_t p;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) {
-      cus = p.multiProcessorCount;
-    } else {
-      (void)hipGetLastError();
-      cus = 256;  // MI355X
-    }
-  }
+  const int cus = ComputeUnits();
   size_t blocks = (work_items + items_per_block - 1) / items_per_block;
   if (blocks == 0) blocks = 1;
   /* a 256-thread block holds 4 waves; 8 such blocks fill a CU's 32 wave slots */

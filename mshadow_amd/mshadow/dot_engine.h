@@ -253,6 +253,35 @@ struct DotEngine {
                           const Tensor<Device, rdim, DType> &rhs, DType scale);
 };
 
+/*! \brief The reference built without an external BLAS (MSHADOW_STAND_ALONE, which is what this
+ *  device is compared with) evaluates dst = dot(A, B), dot(A, B.T()) and dot(A.T(), B) on the
+ *  host through implicit_dot (dot_engine-inl.h:853-863): four partial sums per element, folded
+ *  (s0 + s2) + (s1 + s3). The host device takes the same route for those three forms, so its
+ *  products agree with that build bit for bit; every other form (a scale, a saver other than
+ *  `=`, both operands transposed) runs the plain loops of BLASEngine<cpu>. */
+template <typename SV, typename xpu, bool transpose_left, bool transpose_right, typename DType>
+struct HostProduct {
+  inline static bool Run(Tensor<xpu, 2, DType> *, const Tensor<xpu, 2, DType> &,
+                         const Tensor<xpu, 2, DType> &, DType) {
+    return false;
+  }
+};
+template <bool transpose_left, bool transpose_right, typename DType>
+struct HostProduct<sv::saveto, cpu, transpose_left, transpose_right, DType> {
+  inline static bool Run(Tensor<cpu, 2, DType> *dst, const Tensor<cpu, 2, DType> &lhs,
+                         const Tensor<cpu, 2, DType> &rhs, DType scale) {
+    if (!(scale == DType(1.0f)) || (transpose_left && transpose_right)) return false;
+    if (transpose_left) {
+      *dst = expr::implicit_dot(lhs.T(), rhs);
+    } else if (transpose_right) {
+      *dst = expr::implicit_dot(lhs, rhs.T());
+    } else {
+      *dst = expr::implicit_dot(lhs, rhs);
+    }
+    return true;
+  }
+};
+
 inline Shape<2> GetShape(const Shape<2> &shape, bool transpose) {
   return transpose ? Shape2(shape[1], shape[0]) : shape;
 }
@@ -264,6 +293,7 @@ struct DotEngine<SV, xpu, 2, 2, 2, transpose_left, transpose_right, DType> {
   inline static void Eval(Tensor<xpu, 2, DType> *p_dst, const Tensor<xpu, 2, DType> &lhs,
                           const Tensor<xpu, 2, DType> &rhs, DType scale) {
     Tensor<xpu, 2, DType> &dst = *p_dst;
+    if (HostProduct<SV, xpu, transpose_left, transpose_right, DType>::Run(p_dst, lhs, rhs, scale)) return;
     BLASEngine<xpu, DType>::SetStream(dst.stream_);
     Shape<2> sleft = GetShape(lhs.shape_, transpose_left);
     Shape<2> sright = GetShape(rhs.shape_, transpose_right);

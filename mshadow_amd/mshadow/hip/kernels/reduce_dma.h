@@ -230,6 +230,197 @@ __global__ void __launch_bounds__(kDmaThreads)
   }
 }
 
+/* ------------------------------------------------------------------ KeepHighDim, split over n
+ * The reference's order has two levels (mshadow/tensor_cpu-inl.h:230-268): an inner chain
+ * per (n, c) segment, then a chain over n of the inner results. Only the second is tied to
+ * the kept index c; the inner chains are independent of one another, so they are dealt out in
+ * the order the segments lie in memory, SEGS neighbouring segments per workgroup (one chain
+ * lane each), however few kept indices there are. The inner results go to a scratch array
+ * `partial` of n_out * n_keep words; the workgroup that finishes last (counters in the
+ * scratch memory, kSplitCounterWords words at `counter`, tell it so) folds them per kept index
+ * in n order and saves the result; the counters are zero again when the launch ends. Launches that share a scratch array must not
+ * overlap: the library hands one out per stream.
+ *
+ * A stage is one load instruction per segment: 64 lanes x 4 or 16 bytes of consecutive
+ * elements, which land in LDS as they lie in memory, so a chain lane reads its operands four
+ * at a time. 16-byte loads need rows of whole 16-byte packs (n_x, pitch, base); 4-byte loads
+ * of 16-bit elements rows of whole pairs. */
+template <int SEGS_, int LOADERS_, int SLOTS_, int WBYTES_>
+struct SplitRing {
+  static const int kSegs = SEGS_;
+  static const int kLoaders = LOADERS_;
+  static const int kSlots = SLOTS_;
+  /*! \brief bytes a lane loads at a time: 4, or 16 where rows are whole 16-byte packs */
+  static const int kLaneBytes = WBYTES_;
+  static const int kAhead = SLOTS_ - 2;
+  static const int kPerWave = SEGS_ / LOADERS_;
+  static const int kThreads = (LOADERS_ + 1) * kWave;
+  static_assert(SEGS_ % LOADERS_ == 0 && SEGS_ <= kWave, "one chain lane per segment");
+  static_assert(kAhead >= 1 && kAhead * kPerWave < 64, "the wait-by-count immediate has 6 bits");
+  static_assert(WBYTES_ == 4 || WBYTES_ == 16, "load width");
+};
+/*! \brief the configurations the library launches (measured on MI355X, sum over
+ *  (64,64,112,112) / (256,16,112,112) floats: 54 / 71 us and 68 / 87 us, against 103 / 388 us
+ *  with one workgroup per kept index): rows of whole 16-byte packs - 16 segments per
+ *  workgroup, a kilobyte of each per stage; any rows - 32 segments, 256 bytes of each. */
+typedef SplitRing<16, 8, 4, 16> HighDimSplitRingPacks;
+typedef SplitRing<32, 8, 8, 4> HighDimSplitRing;
+
+template <int BYTES>
+__device__ __forceinline__ void LoadLaneToLds(const void *gsrc_of_lane, void *lds_wave_base) {
+  const __attribute__((address_space(1))) void *from =
+      (const __attribute__((address_space(1))) void *)gsrc_of_lane;
+  __attribute__((address_space(3))) void *to = (__attribute__((address_space(3))) void *)lds_wave_base;
+  if (BYTES == 16) {
+    __builtin_amdgcn_global_load_lds(from, to, 16, 0, kDmaCachePolicy);
+  } else {
+    __builtin_amdgcn_global_load_lds(from, to, 4, 0, kDmaCachePolicy);
+  }
+}
+
+/*! \brief the counters of the split reduction: a root and kSplitLeaves leaves, each in a cache
+ *  line of its own (kSplitCounterStride words apart), all zero between launches */
+const int kSplitLeaves = 64;
+const int kSplitCounterStride = 32;
+const int kSplitCounterWords = (1 + kSplitLeaves) * kSplitCounterStride;
+
+/*! \brief words of scratch memory a launch needs for its inner results */
+inline size_t SplitPartialWords(uint32_t n_out, uint32_t n_keep) {
+  return static_cast<size_t>(n_out) * n_keep;
+}
+
+template <typename Saver, typename Reducer, typename DType, typename Ring>
+__global__ void __launch_bounds__(Ring::kThreads)
+    ReduceKeepHighDimSplitKernel(DType *dst, const DType *src, uint32_t stride, uint32_t n_out,
+                                 uint32_t n_keep, uint32_t n_y, uint32_t n_x, FastDivU32 div_x,
+                                 DType scale, uint32_t *partial, uint32_t *counter) {
+  const int SEGS = Ring::kSegs, kSlots = Ring::kSlots, kAhead = Ring::kAhead, kPerWave = Ring::kPerWave;
+  const int EPL = Ring::kLaneBytes / sizeof(DType);  // elements per lane and load
+  const int TL = kWave * EPL;          // elements of a segment per stage
+  const int LD = TL + 16 / sizeof(DType);  // chain lanes read words LD elements apart: no bank conflicts
+  static_assert(sizeof(DType) == 4 || sizeof(DType) == 2, "a word of scratch memory holds a result");
+  __shared__ MSHADOW_ALIGNED(16) DType ring[kSlots][SEGS * LD];
+  __shared__ uint32_t i_am_last;
+
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t nseg = n_out * n_keep;
+  const uint32_t s0 = blockIdx.x * SEGS;
+  const uint32_t live = (nseg - s0 < static_cast<uint32_t>(SEGS)) ? nseg - s0 : SEGS;
+  const uint32_t seg_len = n_y * n_x;
+  const uint32_t nstage = (seg_len + TL - 1) / TL;
+  const uint32_t nstep = nstage == 0 ? 0 : nstage + kAhead;
+
+  if (wave != 0) {
+    const uint32_t lw = wave - 1;
+    for (uint32_t i = 0; i < nstep; ++i) {
+      if (i < nstage) {
+        DType *slot = ring[i % kSlots];
+        uint32_t e = i * TL + lane * EPL;
+        e = e < seg_len ? e : seg_len - EPL;  // clamped, never consumed
+        const uint32_t y = div_x.Div(e);
+        const size_t in_seg = static_cast<size_t>(y) * stride + (e - y * n_x);
+#pragma unroll
+        for (int q = 0; q < kPerWave; ++q) {
+          const uint32_t seg = q * Ring::kLoaders + lw;
+          const uint32_t sg = s0 + seg < nseg ? s0 + seg : nseg - 1;  // clamped likewise
+          LoadLaneToLds<Ring::kLaneBytes>(src + static_cast<size_t>(sg) * n_y * stride + in_seg,
+                                          slot + seg * LD);
+        }
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAhead * kPerWave) : "memory");
+      } else {
+        WaitAllLanded();
+      }
+      BareBarrier();
+    }
+  } else {
+    DType tres;
+    Reducer::SetInitValue(tres);
+    for (uint32_t i = 0; i < nstep; ++i) {
+      BareBarrier();
+      if (i < static_cast<uint32_t>(kAhead)) continue;
+      const uint32_t st = i - kAhead;
+      const uint32_t e0 = st * TL;
+      if (lane < live) {
+        const int count = (seg_len - e0 < (uint32_t)TL) ? static_cast<int>(seg_len - e0) : TL;
+        ChainFold<Reducer>(tres, ring[st % kSlots] + lane * LD, 0, count);
+      }
+    }
+    if (lane < live) {
+      uint32_t bits = 0;
+      __builtin_memcpy(&bits, static_cast<const void *>(&tres), sizeof(DType));
+      __hip_atomic_store(partial + s0 + lane, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    /* The inner results must have reached the memory side before a counter moves. They are
+       written through by device-scope stores, whose completion is what the wait below waits
+       for; a release fence would do, but it also writes back this L2's every dirty line,
+       once per workgroup. The last workgroup reads them with device-scope loads.
+       Counting is in two levels, because increments of one address are served one after the
+       other (about 40 ns each, which a thousand workgroups finishing together would wait
+       for): workgroup b counts on leaf b % kSplitLeaves, and whoever completes a leaf counts
+       on the root; whoever completes the root is last. A completed counter is cleared by the
+       workgroup that completed it. */
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (lane == 0) {
+      const uint32_t leaf = blockIdx.x % kSplitLeaves;
+      const uint32_t in_leaf = (gridDim.x - leaf + kSplitLeaves - 1) / kSplitLeaves;
+      const uint32_t leaves = gridDim.x < static_cast<uint32_t>(kSplitLeaves) ? gridDim.x : kSplitLeaves;
+      uint32_t *leaf_counter = counter + (1 + leaf) * kSplitCounterStride;
+      uint32_t last = 0u;
+      if (__hip_atomic_fetch_add(leaf_counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+          in_leaf - 1u) {
+        __hip_atomic_store(leaf_counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (__hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+            leaves - 1u) {
+          last = 1u;
+        }
+      }
+      i_am_last = last;
+    }
+  }
+  __syncthreads();
+  if (i_am_last == 0u) return;
+  /* The merge: dst[c] = fold over n of the inner results, in n order. The results come in by
+     device-scope loads, a tile of kMergeCols kept indices x as many n as the ring's memory
+     holds at a time, all of a tile's loads in flight together (one after the other they would
+     cost a trip to memory each); then thread c folds its column of the tile from LDS. */
+  const int kMergeCols = 256;
+  static_assert(Ring::kThreads >= kMergeCols, "a thread per kept index of a tile");
+  uint32_t *tile = reinterpret_cast<uint32_t *>(&ring[0][0]);
+  const uint32_t tile_words = sizeof(ring) / sizeof(uint32_t);
+  const uint32_t tile_n = tile_words / kMergeCols;
+  for (uint32_t c0 = 0; c0 < n_keep; c0 += kMergeCols) {
+    const uint32_t c = c0 + threadIdx.x;
+    DType res;
+    Reducer::SetInitValue(res);
+    for (uint32_t n0 = 0; n0 < n_out; n0 += tile_n) {
+      const uint32_t nn = (n_out - n0 < tile_n) ? n_out - n0 : tile_n;
+      for (uint32_t i = threadIdx.x; i < nn * kMergeCols; i += Ring::kThreads) {
+        const uint32_t cc = c0 + i % kMergeCols;
+        if (cc < n_keep) {
+          tile[i] = __hip_atomic_load(partial + static_cast<size_t>(n0 + i / kMergeCols) * n_keep + cc,
+                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+      __syncthreads();
+      if (threadIdx.x < static_cast<uint32_t>(kMergeCols) && c < n_keep) {
+        for (uint32_t n = 0; n < nn; ++n) {
+          const uint32_t bits = tile[n * kMergeCols + threadIdx.x];
+          DType v;
+          __builtin_memcpy(static_cast<void *>(&v), &bits, sizeof(DType));
+          Reducer::Reduce(res, v);
+        }
+      }
+      __syncthreads();
+    }
+    if (threadIdx.x < static_cast<uint32_t>(kMergeCols) && c < n_keep) {
+      Saver::template Save<DType>(dst[c], res * scale);
+    }
+  }
+  if (threadIdx.x == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 }  // namespace hip
 }  // namespace mshadow
 #endif  // MSHADOW_HIP_KERNELS_REDUCE_DMA_H_

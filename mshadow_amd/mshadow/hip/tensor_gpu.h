@@ -1057,9 +1057,43 @@ struct HalfRingRoute<Saver, Reducer, Tensor<gpu, 1, half::half_t>, Tensor<gpu, d
     half::half_t *d = dst.dptr_;
     const half::half_t *s = src.dptr_;
     uint32_t stride = src.stride_;
+    void *stream = Stream<gpu>::GetStream(dst.stream_);
+    /* the inner chains spread over as many workgroups as there are groups of segments, where
+       rows are whole 16-byte packs (dense rows are walked as one row per segment) and the
+       library has scratch memory for the inner results of this stream */
+    {
+      uint32_t v_y = n_y, v_x = n_x, v_stride = stride;
+      if (stride == n_x) {
+        v_x = v_stride = n_y * n_x;
+        v_y = 1;
+      }
+      uint32_t *partial = NULL, *counter = NULL;
+      /* fewer kept indices than CUs (the chip's 256: the one-workgroup-per-kept-index kernel
+         below would leave some idle): the inner chains are dealt out by segments */
+      const bool few_kept = n_keep < 192u;
+      const bool packs = v_x % 8 == 0 && v_stride % 8 == 0 && reinterpret_cast<uintptr_t>(s) % 16 == 0;
+      if (few_kept && static_cast<uint64_t>(n_out) * n_keep < (1ull << 31)) {
+        MSHADOW_HIP_CALL(mshadow_hip_reduce_scratch(stream, static_cast<size_t>(n_out) * n_keep,
+                                                    &partial, &counter));
+      }
+      if (partial != NULL) {
+        FastDivU32 v_div_x(v_x);
+        void *sargs[] = {&d, &s, &v_stride, &n_out, &n_keep, &v_y, &v_x, &v_div_x, &scale, &partial,
+                         &counter};
+        if (packs) {
+          typedef hip::HighDimSplitRingPacks Ring;
+          Launch(hip::ReduceKeepHighDimSplitKernel<Saver, Reducer, half::half_t, Ring>,
+                 (n_out * n_keep + Ring::kSegs - 1) / Ring::kSegs, Ring::kThreads, sargs, stream);
+        } else {
+          typedef hip::HighDimSplitRing Ring;
+          Launch(hip::ReduceKeepHighDimSplitKernel<Saver, Reducer, half::half_t, Ring>,
+                 (n_out * n_keep + Ring::kSegs - 1) / Ring::kSegs, Ring::kThreads, sargs, stream);
+        }
+        return true;
+      }
+    }
     FastDivU32 div_x(n_x);
     void *args[] = {&d, &s, &stride, &n_out, &n_keep, &n_y, &n_x, &div_x, &scale};
-    void *stream = Stream<gpu>::GetStream(dst.stream_);
 #define MSHADOW_HALF_RING(SEGS)                                                                  \
     Launch(hip::ReduceKeepHighDimDmaKernel<Saver, Reducer, half::half_t, SEGS>, n_keep,         \
            hip::kDmaThreads, args, stream)

@@ -214,9 +214,16 @@ class Random<gpu, DType> {
     }
     return (static_cast<size_t>(rows) * cols + 1) / 2;
   }
-  static_assert(std::is_same<DType, float>::value || std::is_same<DType, double>::value,
-                "Random<gpu, DType>: float and double, the types the reference's generator "
-                "library serves (mshadow/random.h:486-514)");
+  /*! \brief any other element type: the class itself instantiates (an operator templated over
+   *  DType may hold a Random<gpu, DType> it never samples from), sampling does not compile,
+   *  as with the float* / double* overloads of mshadow/random.h:486-514 */
+  template <typename T>
+  inline size_t Draw(int, T *, index_t, index_t, index_t, T, T) {
+    static_assert(std::is_same<T, float>::value || std::is_same<T, double>::value,
+                  "Random<gpu, DType> samples float and double, the types the reference's "
+                  "generator library serves (mshadow/random.h:486-514)");
+    return 0;
+  }
   Stream<gpu> *stream_;
   uint64_t seed_;
   uint64_t counter_;

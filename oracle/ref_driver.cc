@@ -15,6 +15,8 @@
 #include <stdint.h>
 
 #include "../mshadow_amd/cases/portable_math.h"
+/* a caller program written against <mshadow/tensor.h>: here that is the reference's */
+#include "../mshadow_amd/cases/conv_net.h"
 
 using namespace mshadow;
 using namespace mshadow::expr;
@@ -523,5 +525,32 @@ REF_IM2COL(ref_im2col_f32, float, float)
   }
 REF_COL2IM(ref_col2im_f16, uint16_t, half::half_t)
 REF_COL2IM(ref_col2im_f32, float, float)
+
+/* the convolutional network of cases/conv_net.h on the reference's CPU device (its stand-alone
+   build evaluates the three forms of dot the program uses through implicit_dot) */
+void ref_conv_net_f32(const int *v, int steps, float eta, float decay, const float *images,
+                      const float *labels, const float *fixed_grad, float *kernel, float *weight,
+                      float *const *keep) {
+  const conv_net::Geometry g = {v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8]};
+  conv_net::Train<cpu>(NULL, g, steps, eta, decay, images, labels, fixed_grad, kernel, weight, keep);
+}
+
+void ref_conv_pair(int half, const int *v, const void *image, const void *kernel,
+                   const void *grad_out, void *col_forward, void *out, void *col_backward,
+                   void *image_grad) {
+  typedef half::half_t H;
+  const conv_net::Geometry g = {v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8]};
+  if (half) {
+    conv_net::ConvPair<cpu, H>(NULL, g, static_cast<const H *>(image), static_cast<const H *>(kernel),
+                               static_cast<const H *>(grad_out), static_cast<H *>(col_forward),
+                               static_cast<H *>(out), static_cast<H *>(col_backward),
+                               static_cast<H *>(image_grad));
+  } else {
+    conv_net::ConvPair<cpu, float>(NULL, g, static_cast<const float *>(image),
+                                   static_cast<const float *>(kernel), static_cast<const float *>(grad_out),
+                                   static_cast<float *>(col_forward), static_cast<float *>(out),
+                                   static_cast<float *>(col_backward), static_cast<float *>(image_grad));
+  }
+}
 
 }  // extern "C"

@@ -6,6 +6,7 @@
 
 #include "../../mshadow_amd/cases/portable_math.h"
 #include "../../mshadow_amd/cases/two_layer_net.h"
+#include "../../mshadow_amd/cases/conv_net.h"
 
 using namespace mshadow;
 using namespace mshadow::expr;
@@ -95,6 +96,47 @@ extern "C" int host_two_layer_net_f32(int steps, float eta, float decay, int bat
     two_layer_net::Train<cpu>(NULL, steps, eta, decay, View(x, Shape2(batch, n_in)),
                               View(label, Shape1(batch)), View(w1, Shape2(n_in, n_hidden)),
                               View(w2, Shape2(n_hidden, n_out)), View(probs, Shape2(batch, n_out)));
+  } catch (const std::exception &e) {
+    fprintf(stderr, "%s\n", e.what());
+    return 1;
+  }
+  return 0;
+}
+
+static conv_net::Geometry GeometryOf(const int *v) {
+  const conv_net::Geometry g = {v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8]};
+  return g;
+}
+
+extern "C" int host_conv_net_f32(const int *geometry, int steps, float eta, float decay,
+                                 const float *images, const float *labels, const float *fixed_grad,
+                                 float *kernel, float *weight, float *const *keep) {
+  try {
+    conv_net::Train<cpu>(NULL, GeometryOf(geometry), steps, eta, decay, images, labels, fixed_grad,
+                         kernel, weight, keep);
+  } catch (const std::exception &e) {
+    fprintf(stderr, "%s\n", e.what());
+    return 1;
+  }
+  return 0;
+}
+
+extern "C" int host_conv_pair(int half, const int *geometry, const void *image, const void *kernel,
+                              const void *grad_out, void *col_forward, void *out, void *col_backward,
+                              void *image_grad) {
+  typedef half::half_t H;
+  try {
+    if (half) {
+      conv_net::ConvPair<cpu, H>(NULL, GeometryOf(geometry), static_cast<const H *>(image),
+                                 static_cast<const H *>(kernel), static_cast<const H *>(grad_out),
+                                 static_cast<H *>(col_forward), static_cast<H *>(out),
+                                 static_cast<H *>(col_backward), static_cast<H *>(image_grad));
+    } else {
+      conv_net::ConvPair<cpu, float>(NULL, GeometryOf(geometry), static_cast<const float *>(image),
+                                     static_cast<const float *>(kernel), static_cast<const float *>(grad_out),
+                                     static_cast<float *>(col_forward), static_cast<float *>(out),
+                                     static_cast<float *>(col_backward), static_cast<float *>(image_grad));
+    }
   } catch (const std::exception &e) {
     fprintf(stderr, "%s\n", e.what());
     return 1;

@@ -4,6 +4,7 @@
 // linked by the CPU test suite (it proves the claim at build time) and run by a GPU test.
 #include <mshadow/tensor.h>
 #include <mshadow/io.h>
+#include <mshadow/random.h>
 
 #include <cstdio>
 #include <cstring>
@@ -11,6 +12,17 @@
 
 using namespace mshadow;
 using namespace mshadow::expr;
+
+// An operator templated over its element type may hold a generator it never samples from:
+// the class instantiates for every DType (sampling anything but float and double does not
+// compile, as with the reference's float* / double* generator calls).
+template <typename DType>
+struct HoldsAGenerator {
+  Random<gpu, DType> *rnd;
+  size_t Footprint() const { return sizeof(Random<gpu, DType>); }
+};
+template struct HoldsAGenerator<half::half_t>;
+template struct HoldsAGenerator<int>;
 
 int main() {
   InitTensorEngine<gpu>(0);

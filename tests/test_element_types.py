@@ -195,7 +195,10 @@ def test_gpu_half_reduce_keep_lowest(G, orc, stream, shape, pad):
                                        # (taken) and an odd one (falls back to the generic kernel)
                                        ((64, 5, 56, 56), 0), ((70, 3, 33, 30), 2), ((6, 3, 150, 100), 0),
                                        ((3, 2, 301, 128), 6), ((1, 2, 700, 100), 0), ((20, 3, 60, 62), 3),
-                                       ((33, 2, 40, 51), 1)])
+                                       ((33, 2, 40, 51), 1),
+                                       # pitched rows of whole 16-byte packs: the inner chains in
+                                       # groups of 16 segments, as for the dense shapes above
+                                       ((36, 5, 40, 48), 8)])
 def test_gpu_half_reduce_keep_highdim(G, orc, stream, shape, pad):
     x = halves(orc, 31, shape)
     if shape == (2, 2, 30, 100):

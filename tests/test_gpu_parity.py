@@ -80,6 +80,42 @@ def test_copy_roundtrip_and_pitch(G, shape, pad):
         assert stride == shape[1]
 
 
+@pytest.mark.parametrize("rows,width,dpitch,spitch,doff,soff", [
+    (7, 220, 220, 224, 0, 0),          # 4-byte units, different pitches
+    (33, 256, 512, 272, 0, 0),         # whole 16-byte packs, pitched on both sides
+    (21, 1000, 1016, 1008, 8, 0),      # 8-byte units
+    (5, 4000, 4000, 4000, 0, 0),       # dense: one run
+    (1, 4004, 4004, 4004, 0, 0),       # a single row keeps its width, whatever the pitch says
+    (3, 1001, 1008, 1003, 0, 0),       # an odd number of bytes: the runtime's copy
+    (9, 64, 96, 80, 2, 6),             # addresses that are no multiple of 4: the runtime's copy
+    (700, 128000, 128000, 128256, 0, 0),
+    (650, 127960, 128000, 128000, 0, 0)])
+def test_device_to_device_copy_of_pitched_views(G, stream, rows, width, dpitch, spitch, doff, soff):
+    """mshadow_hip_memcpy2d_async device to device: exactly the bytes of the view arrive, the
+    gaps between rows and around the view keep their contents"""
+    from mshadow_amd.capi import D2D
+    rng = np.random.default_rng(rows * 31 + width)
+    src_host = rng.integers(0, 256, rows * spitch + 64, dtype=np.uint8)
+    dst_host = rng.integers(0, 256, rows * dpitch + 64, dtype=np.uint8)
+    src, dst = G.to_device(src_host), G.to_device(dst_host)
+    G.check(G.dll.mshadow_hip_memcpy2d_async(dst.ptr + doff, dpitch, src.ptr + soff, spitch, width, rows,
+                                             D2D, stream))
+    want = dst_host.copy()
+    for y in range(rows):
+        want[doff + y * dpitch: doff + y * dpitch + width] = src_host[soff + y * spitch: soff + y * spitch + width]
+    assert np.array_equal(dst.download(stream), want)
+
+
+def test_copy_between_device_tensors_through_the_header_api(G, stream):
+    """Copy(Tensor<gpu>, Tensor<gpu>, stream) with either side pitched"""
+    a = uniform(3, (37, 300))
+    for spad, dpad in ((0, 0), (4, 0), (0, 12), (5, 3)):
+        src = G.to_device(a, spad)
+        dst = G.to_device(np.zeros_like(a), dpad)
+        G.case_copy_d2d(dst, src, stream)
+        assert_bits_equal(dst.download(stream), a, f"Copy pads {spad} {dpad}")
+
+
 # ------------------------------------------------------------------ elementwise map
 MAP_SHAPES = [((4096 // 8, 4096 // 8), 0), ((257, 515), 0), ((257, 516), 4), ((33, 7), 1),
               ((1, 1), 0), ((5, 1024), 0), ((129, 260), 12)]
@@ -169,7 +205,14 @@ HIGH_SHAPES = [((8, 32, 56, 56), 0), ((64, 5, 7, 9), 2), ((3, 4, 5, 6), 0), ((1,
                ((70, 3, 1, 1), 0), ((17, 2, 33, 65), 3), ((2, 2, 70, 70), 0),
                # long enough for the direct-to-LDS kernels, one shape per segment count
                ((70, 3, 33, 65), 3), ((5, 2, 130, 129), 0), ((2, 2, 200, 200), 0),
-               ((1, 2, 300, 300), 1)]
+               ((1, 2, 300, 300), 1),
+               # rows of whole 16-byte packs: the inner chains are dealt out in groups of 16
+               # segments (dense; pitched; more groups than kept indices; a last group that is
+               # not full; segments of one pack; more inner results than the scratch memory holds)
+               ((64, 7, 32, 36), 0), ((33, 5, 40, 52), 4), ((300, 1, 16, 16), 0),
+               ((20000, 3, 1, 4), 0), ((70000, 1, 1, 4), 0), ((9, 40, 90, 100), 0),
+               # a kept index for every CU: one workgroup each, no merge
+               ((40, 200, 41, 40), 0)]
 
 
 @pytest.mark.parametrize("shape,pad", HIGH_SHAPES)
@@ -189,6 +232,26 @@ def test_reduce_keep_highdim(G, O, stream, shape, pad, reducer, route):
             G.case_reduce_keep_highdim(dst, src, reducer, saver, scale,
                                        1 if route == "expr_generic" else 0, stream)
         assert_bits_equal(dst.download(stream), want, f"keep_highdim {shape} {route}")
+
+
+def test_reduce_keep_highdim_on_more_streams_than_scratch_slots(G, O):
+    """every stream gets the same result, whether it was given scratch memory for the inner
+    results (the first eight of a GPU) or runs the kernel that needs none; a slot is free again
+    once its stream is destroyed"""
+    shape = (40, 6, 48, 64)
+    x = normal(52, shape)
+    want = np.empty(shape[1], f32)
+    O.reduce_keep_highdim(want, x, SUM, SAVETO, 1.0)
+    src = G.to_device(x)
+    for _ in range(2):
+        streams = [G.stream_create() for _ in range(11)]
+        outs = [G.buffer((shape[1],), f32) for _ in streams]
+        for st, dst in zip(streams, outs):
+            G.reduce_keep_highdim(dst, src, SUM, SAVETO, 1.0, st)
+            G.reduce_keep_highdim(dst, src, SUM, SAVETO, 1.0, st)   # the counter is zero again
+        for st, dst in zip(streams, outs):
+            assert_bits_equal(dst.download(st), want, "keep_highdim, many streams")
+            G.stream_destroy(st)
 
 
 def test_reduce_reference_known_answers(G, stream):
