@@ -103,6 +103,15 @@ def work_elements():
 PRODUCT_FLOPS = {"dot_f32_4096": (2 * 4096 ** 3, 157.3), "dot_f16_8192": (2 * 8192 ** 3, 2500.0)}
 
 
+# What a kernel that adds in the reference's order can reach at all: sum_rows is one chain of
+# 16384 dependent adds per column, 3.9 ns each with every CU busy (bench.py --only ceiling_chain)
+# = 64 us, and its loads - 64 bytes of every row per CU, half a cache line per request, at most
+# about 128 requests in flight per CU - take 68 us alone (--only ceiling_lds_loads).
+ORDER_FAITHFUL = {
+    "sum_rows": {"order_faithful_ceiling": 0.52,
+                 "ceiling_from": "16384 dependent adds per column x 3.9 ns = 64 us; column-strip loads alone 68 us"},
+}
+
 EXTRA_OPS = ("calib_copy", "smooth_softmax_grad_ignore", "softmax3d", "softmax3d_grad", "add_take_grad",
              "bias_add_broadcast", "swapaxis10_reshape", "lrn_scale_chpool5", "transpose_nchw_nhwc",
              "sort_by_key_f32", "dot_f32_4096", "dot_f16_8192", "ceiling_copy", "ceiling_fill",
@@ -227,10 +236,20 @@ def main():
         G.pool(b["out_pool"], b["dev"]["X4"], 3, 3, 2, 2, stream=s)
         return b
 
-    sets = [buffer_set()]
+    # Three complete sets of operands, taken in turn step by step, so that no launch finds its
+    # input in the 256 MB memory-side cache from the launch before. unpool and softmax_grad read
+    # what pool and softmax wrote - from the NEXT set (written two steps ago, same values), not
+    # from the launch that has just finished.
+    rotate = args.scale == 1 and all(o in OPS for o in only)
+    sets = [buffer_set() for _ in range(3 if rotate else 1)]
     cur = dict(sets[0])     # the set run_op works on
+    nxt = dict(sets[1 % len(sets)])   # where unpool / softmax_grad take their producer's output
     dev = cur["dev"]
     out_map, out_g, out_p = cur["out_map"], cur["out_g"], cur["out_p"]
+
+    def use_set(k):
+        cur.update(sets[k % len(sets)])
+        nxt.update(sets[(k + 1) % len(sets)])
 
     extra = {}
     if any(o in EXTRA_OPS[1:] for o in only):
@@ -338,11 +357,11 @@ def main():
         elif name == "softmax":
             G.softmax(cur["out_p"], cur["dev"]["L"], s)
         elif name == "softmax_grad":
-            G.softmax_grad(cur["out_g"], cur["out_p"], cur["dev"]["labels"], s)
+            G.softmax_grad(cur["out_g"], nxt["out_p"], cur["dev"]["labels"], s)
         elif name == "pool_max":
             G.pool(cur["out_pool"], cur["dev"]["X4"], 3, 3, 2, 2, stream=s)
         elif name == "unpool_max":
-            G.unpool(cur["out_unpool"], cur["dev"]["X4"], cur["out_pool"], cur["dev"]["G4"], 3, 3, 2, 2, stream=s)
+            G.unpool(cur["out_unpool"], cur["dev"]["X4"], nxt["out_pool"], cur["dev"]["G4"], 3, 3, 2, 2, stream=s)
         elif name == "im2col_f16":
             G.im2col(cur["out_col"], cur["dimg"], 3, 3, 1, 1, 1, 1, 1, 1, s)
         elif name == "col2im_f16":
@@ -352,7 +371,8 @@ def main():
             # HBM traffic counters are scaled by (only with --only, never part of a step)
             G.case_map_axpb(out_map, dev["A"], 0.0, 1.0, 0.0, 0, s)
 
-    for _ in range(args.warmup):
+    for k in range(args.warmup):
+        use_set(k)
         for name in only:
             run_op(name)
     G.stream_sync(s)
@@ -365,6 +385,7 @@ def main():
     nev = len(only) + 1
     events = [[G.event_create() for _ in range(nev)] for _ in range(args.steps)]
     for k in range(args.steps):
+        use_set(k)
         G.event_record(events[k][0], s)
         for i, name in enumerate(only):
             run_op(name)
@@ -380,6 +401,7 @@ def main():
     G.device_sync()
     wall0 = time.perf_counter()
     for k in range(args.steps):
+        use_set(k)
         for name in only:
             if name == dominant:
                 G.event_record(dom_events[k][0], s)
@@ -397,24 +419,22 @@ def main():
     # (3 x 205 MB and more: nothing is found in the 256 MB memory-side cache from the
     # launch before). "ms" above is the operation's interval inside the step, gap included.
     b2b_ms = {}
-    if args.scale == 1 and all(o in OPS for o in only):
-        while len(sets) < 3:
-            sets.append(buffer_set())
+    if rotate:
         G.stream_sync(s)
         reps = 12
         for name in only:
             ev = [G.event_create(), G.event_create()]
             for r in range(3):
-                cur.update(sets[r])
+                use_set(r)
                 run_op(name)
             G.event_record(ev[0], s)
             for r in range(reps):
-                cur.update(sets[r % 3])
+                use_set(r)
                 run_op(name)
             G.event_record(ev[1], s)
             G.stream_sync(s)
             b2b_ms[name] = G.elapsed_ms(ev[0], ev[1]) / reps
-        cur.update(sets[0])
+        use_set(0)
 
     abytes = algorithmic_bytes()
     elems = work_elements()
@@ -432,6 +452,8 @@ def main():
             per_op[-1]["ms_back_to_back"] = round(b2b_ms[name], 4)
             per_op[-1]["frac_of_hbm_peak_back_to_back"] = round(
                 abytes[name] / (b2b_ms[name] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+        if name in ORDER_FAITHFUL:
+            per_op[-1].update(ORDER_FAITHFUL[name])
         if name in PRODUCT_FLOPS:
             flops, peak = PRODUCT_FLOPS[name]
             per_op[-1]["TFLOPps"] = round(flops / (ms.mean() * 1e-3) / 1e12, 1)
@@ -590,6 +612,11 @@ def run_probe(G, which, pattern=""):
                                round(P.row_copy_us(dst, src, b, k, s), 1)
                                for b, k in ((0, 0), (4, 0), (4, 2), (4, 4), (4, 8), (8, 4))},
                "row_copy_one_row_per_cu_us": round(min(P.row_copy_us(dst, src, 0, 0, s, 1) for _ in range(3)), 1)}
+        # how long the steps take when a row has its CU to itself, on 8 and on 16 waves
+        for variant, name in ((1, "one_row_per_cu_512_threads"), (2, "one_row_per_cu_1024_threads")):
+            st, res, ker, fb = P.softmax_phases(dst, src, s, variant)
+            out[name] = {"steps": {k: round(v, 2) for k, v in st.items()}, "row_resident_us": round(res, 2),
+                         "kernel_us": round(ker, 1), "fallback_rows": fb}
     print(json.dumps(out))
 
 

@@ -659,7 +659,7 @@ class Probe:
         self.dll.mshadow_probe_last_error.restype = C.c_char_p
         self.dll.mshadow_probe_add_chain.argtypes = [_i, _i, C.POINTER(C.c_double), _p]
         self.dll.mshadow_probe_softmax_phases.argtypes = [
-            _p, _i, _p, _i, _i, _i, C.POINTER(C.c_double), C.POINTER(C.c_double),
+            _p, _i, _p, _i, _i, _i, _i, C.POINTER(C.c_double), C.POINTER(C.c_double),
             C.POINTER(C.c_double), C.POINTER(_i), _p]
 
     def row_copy_us(self, dst, src, barriers, spin, stream=None, resident=2):
@@ -711,12 +711,12 @@ class Probe:
         self._check(self.dll.mshadow_probe_add_chain(self.CHAIN_MODES[mode], workgroups, C.byref(ns), stream))
         return ns.value
 
-    def softmax_phases(self, dst, src, stream=None):
+    def softmax_phases(self, dst, src, stream=None, variant=0):
         """-> ({step name: mean us since the previous step}, resident us, kernel us, fallback rows)"""
         mean = (C.c_double * self.STAMPS)()
         resident, kernel, fallback = C.c_double(0), C.c_double(0), _i(0)
         self._check(self.dll.mshadow_probe_softmax_phases(
-            dst.ptr, dst.stride, src.ptr, src.stride, src.rows, src.cols, mean, C.byref(resident),
+            dst.ptr, dst.stride, src.ptr, src.stride, src.rows, src.cols, variant, mean, C.byref(resident),
             C.byref(kernel), C.byref(fallback), stream))
         steps = {f"{idx} {name}": mean[idx] for idx, name in zip(self.STAMP_ORDER, self.STAMP_NAMES)}
         return steps, resident.value, kernel.value, fallback.value

@@ -30,7 +30,9 @@ int mshadow_probe_add_chain(int mode, int workgroups, double *ns_per_add, void *
    mean_us[i] = mean over rows of the time from the previous step of the list to step i
    (-1: no row reached it); resident_us = mean time from entry to the last step;
    kernel_us = duration of the launch by HIP events; fallback_rows = rows whose plan did not
-   hold and that were summed by wave scans instead. dst may alias src. */
+   hold and that were summed by wave scans instead. dst may alias src. variant 0: the kernel as
+   the library launches it (two rows resident per CU); 1: the same with one row per CU; 2: one
+   row per CU on 1024 threads - how long a row's steps take when the row has the CU to itself. */
 #define MSHADOW_PROBE_STAMP_FALLBACK 7
 #define MSHADOW_PROBE_STAMPS 16
 #define MSHADOW_PROBE_STAMP_ORDER {10, 11, 12, 13, 1, 2, 6, 8, 3, 4, 5, 14}
@@ -41,7 +43,7 @@ int mshadow_probe_add_chain(int mode, int workgroups, double *ns_per_add, void *
    "3 every wave's chunks done (barrier)", "4 row's list of addends assembled (barrier)",           \
    "5 chain (wave 0; barrier)", "14 divided and stored (stores completed)"}
 int mshadow_probe_softmax_phases(float *dst, int dstride, const float *src, int sstride, int rows,
-                                 int cols, double *mean_us, double *resident_us,
+                                 int cols, int variant, double *mean_us, double *resident_us,
                                  double *kernel_us, int *fallback_rows, void *stream);
 
 /* The memory side of that kernel alone: every workgroup loads its row into registers as the

@@ -682,7 +682,12 @@ int mshadow_hip_reduce_keep_highdim_f32(float *dst, const float *src, int sstrid
   ABI_REQUIRE(dst != NULL, "NULL tensor");
   ABI_REQUIRE(src != NULL || static_cast<long long>(n) * y * x == 0, "NULL tensor");
   ABI_REQUIRE(sstride >= x, "pitch smaller than the row");
-  ABI_REQUIRE(static_cast<long long>(n) * c * y < (1ll << 31), "too many rows for 32-bit indices");
+  /* the kernels that stream a tensor from memory compute row numbers in 64 bits; the
+     register-staged ones for short reductions (fewer than 2^16 values per kept index) in 32 */
+  ABI_REQUIRE(static_cast<long long>(n) * c < (1ll << 31), "too many (n, c) segments for 32-bit indices");
+  ABI_REQUIRE(static_cast<long long>(n) * c * y < (1ll << 31) ||
+                  static_cast<long long>(n) * y * x >= kDmaMinPerKept,
+              "too many rows for 32-bit indices");
   ABI_REQUIRE(static_cast<long long>(y) * x < (1ll << 31), "inner extent too large for 32-bit indices");
   RawPlan1D<float> d = {dst};
   RawPlan2D<const float> sp = {src, sstride};

@@ -164,7 +164,8 @@ __global__ void __launch_bounds__(THREADS, 4)
  *  A wave reads back from LDS exactly the bytes its own loads delivered, so the hand-over
  *  needs a wait on the wave's own counter and no barrier. The counter retires loads and
  *  stores in issue order: the wait leaves the stores of the row before and the direct
- *  loads of this row outstanding (at most the last slab of either is skipped by a wave). */
+ *  loads of this row outstanding (at most the last slab of either is skipped by a wave);
+ *  in front of a workgroup's first row there are no stores to leave. */
 template <int THREADS, int SLABS, int PRE>
 __global__ void __launch_bounds__(THREADS)
     RowCopyPrefetchKernel(float *dst, int dstride, const float *src, int sstride, int rows, int cols,
@@ -199,8 +200,15 @@ __global__ void __launch_bounds__(THREADS)
       v[j] = F4{0.0f, 0.0f, 0.0f, 0.0f};
       if (c0 + lane_col < cols) v[j] = mshadow_hipk::StreamLoadF4(in + c0 + lane_col);
     }
-    const int kLater = (SLABS - 1) + (PRE < SLABS ? SLABS - PRE - 1 : 0);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLater) : "memory");
+    /* operations issued behind this row's loads into LDS, at least: its own direct loads and,
+       from the second row on, the stores of the row before */
+    const int kDirect = PRE < SLABS ? SLABS - PRE - 1 : 0;
+    const int kLater = (SLABS - 1) + kDirect;
+    if (row == static_cast<int>(blockIdx.x)) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDirect) : "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLater) : "memory");
+    }
 #pragma unroll
     for (int j = 0; j < PRE; ++j) v[j] = *reinterpret_cast<const F4 *>(mine + j * 1024 + lane * 16);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -543,8 +551,9 @@ int mshadow_probe_highdim_split(float *dst, const float *warm, const float *src,
 }
 
 int mshadow_probe_softmax_phases(float *dst, int dstride, const float *src, int sstride, int rows,
-                                 int cols, double *mean_us, double *resident_us,
+                                 int cols, int variant, double *mean_us, double *resident_us,
                                  double *kernel_us, int *fallback_rows, void *stream) {
+  ABI_REQUIRE(variant >= 0 && variant <= 2, "variant 0, 1 or 2");
   ABI_REQUIRE(rows >= 1 && cols > 16384 && cols <= 32768 && cols % 4 == 0 && sstride % 4 == 0 &&
                   dstride % 4 == 0, "the probe covers the 512-thread, 16-slab kernel: 16384 < cols <= 32768, rows of whole packs");
   ABI_REQUIRE(mean_us != NULL && resident_us != NULL && kernel_us != NULL && fallback_rows != NULL,
@@ -558,8 +567,16 @@ int mshadow_probe_softmax_phases(float *dst, int dstride, const float *src, int 
                                  hipMemcpyHostToDevice, s));
   float ms = 0.0f;
   const int st = TimeKernel(s, &ms, [&] {
-    hipLaunchKernelGGL((mshadow_hipk::SoftmaxRowKernel<512, 16, 4, false>), dim3(rows), dim3(512), 0,
-                       s, dst, dstride, src, sstride, cols);
+    if (variant == 0) {
+      hipLaunchKernelGGL((mshadow_hipk::SoftmaxRowKernel<512, 16, 4, false>), dim3(rows), dim3(512), 0,
+                         s, dst, dstride, src, sstride, cols);
+    } else if (variant == 1) {  // one row per CU: LDS the kernel never touches keeps a second one off
+      hipLaunchKernelGGL((mshadow_hipk::SoftmaxRowKernel<512, 16, 4, false>), dim3(rows), dim3(512),
+                         90000, s, dst, dstride, src, sstride, cols);
+    } else {  // one row per CU, on sixteen waves
+      hipLaunchKernelGGL((mshadow_hipk::SoftmaxRowKernel<1024, 8, 4, false>), dim3(rows), dim3(1024),
+                         90000, s, dst, dstride, src, sstride, cols);
+    }
   });
   if (st != MSHADOW_HIP_OK) {
     (void)hipFree(stamps);

@@ -105,15 +105,17 @@ class Plan<Tensor<Device, dim, DType>, DType> {
  public:
   static const bool kPackable = true;
   explicit Plan(const Tensor<Device, dim, DType> &t) : dptr_(t.dptr_), stride_(t.stride_) {}
-  MSHADOW_XINLINE DType &REval(index_t y, index_t x) { return dptr_[y * stride_ + x]; }
-  MSHADOW_XINLINE const DType &Eval(index_t y, index_t x) const { return dptr_[y * stride_ + x]; }
+  /* offsets in 64 bits whatever index_t is: a tensor whose dimensions each fit index_t may
+     still hold 2^31 elements or more (65536 x 32768 floats are 8 GiB of a 288 GB device) */
+  MSHADOW_XINLINE DType &REval(index_t y, index_t x) { return dptr_[At(y, x)]; }
+  MSHADOW_XINLINE const DType &Eval(index_t y, index_t x) const { return dptr_[At(y, x)]; }
   template <int N, bool STREAM = false>
   MSHADOW_XINLINE Pack<DType, N> EvalPack(index_t y, index_t x) const {
-    return plan_detail::LoadPack<DType, N, STREAM>(dptr_ + y * stride_ + x);
+    return plan_detail::LoadPack<DType, N, STREAM>(dptr_ + At(y, x));
   }
   template <int N, bool STREAM = false>
   MSHADOW_XINLINE void StorePack(index_t y, index_t x, const Pack<DType, N> &p) {
-    plan_detail::StorePackTo<DType, N, STREAM>(dptr_ + y * stride_ + x, p);
+    plan_detail::StorePackTo<DType, N, STREAM>(dptr_ + At(y, x), p);
   }
   /*! \brief host check: pointer and pitch allow n-wide access; *flat stays true only
    *  while rows are dense (pitch == cols) so that the 2-D view can be walked linearly */
@@ -123,6 +125,9 @@ class Plan<Tensor<Device, dim, DType>, DType> {
   }
 
  private:
+  MSHADOW_XINLINE int64_t At(index_t y, index_t x) const {
+    return static_cast<int64_t>(y) * stride_ + x;
+  }
   DType *dptr_;
   index_t stride_;
 };

@@ -39,13 +39,17 @@ const int kPackUnrollDeep = 8;
  *  plan reads consecutive addresses the compiler merges them into one wide load. */
 template <typename Saver, typename DType, typename DPlan, typename SPlan, int PER>
 __global__ void __launch_bounds__(kMapBlock)
-    MapScalarKernel(DPlan dplan, SPlan splan, uint32_t rows, uint32_t cols, FastDivU32 div_cols) {
+    MapScalarKernel(DPlan dplan, SPlan splan, uint32_t rows, uint32_t cols, FastDivU32 div_cols,
+                    uint32_t row0) {
+  /* one launch covers `rows` rows from row0 on, fewer than 2^31 elements; a larger view is
+     covered by several launches */
   const uint32_t total = rows * cols;
   const uint32_t step = gridDim.x * kMapBlock * PER;
   const uint32_t piece = StripOfBlock(blockIdx.x, gridDim.x);
   for (uint32_t i = (piece * kMapBlock + threadIdx.x) * PER; i < total; i += step) {
-    const uint32_t y = div_cols.Div(i);  // a multiply-high, not a hardware division
-    const uint32_t x = i - y * cols;
+    const uint32_t yr = div_cols.Div(i);  // a multiply-high, not a hardware division
+    const uint32_t x = i - yr * cols;
+    const uint32_t y = yr + row0;
     DType v[PER];
 #pragma unroll
     for (int k = 0; k < PER; ++k) v[k] = splan.Eval(y, x + k);
@@ -73,7 +77,7 @@ template <typename Saver, typename DType, int N, bool kFlat, bool kStream, int k
           typename DPlan, typename SPlan>
 __global__ void __launch_bounds__(kMapBlock)
     MapPackKernel(DPlan dplan, SPlan splan, uint32_t total_packs, uint32_t packs_per_row,
-                  FastDivU32 div_ppr) {
+                  FastDivU32 div_ppr, uint32_t row0) {
   typedef expr::Pack<DType, N> P;
   /* with real row numbers in play (windows over rows re-read their neighbours' data), each
      XCD takes a contiguous run of the workgroups */
@@ -88,8 +92,9 @@ __global__ void __launch_bounds__(kMapBlock)
       y[u] = 0;
       x[u] = p * N;
     } else {
-      y[u] = div_ppr.Div(p);
-      x[u] = (p - y[u] * packs_per_row) * N;
+      const uint32_t yr = div_ppr.Div(p);
+      x[u] = (p - yr * packs_per_row) * N;
+      y[u] = yr + row0;  // the launch covers whole rows from row0 on, fewer than 2^31 packs
     }
     if (p < total_packs) val[u] = splan.template EvalPack<N, kStream>(y[u], x[u]);
   }

@@ -175,6 +175,30 @@ inline bool AnyPackable(const DType *a, uint32_t astride, const DType *b, uint32
   return addr % 16 == 0 && cols % pack == 0;
 }
 }  // namespace gpu_detail
+namespace gpu_detail {
+#if defined(__HIPCC__)
+/*! \brief long half_t rows: one workgroup per row, the row kept in registers; false = not
+ *  this shape or element type */
+template <typename DType>
+inline bool SoftmaxLongRows(DType *, uint32_t, const DType *, uint32_t, uint32_t, uint32_t, bool, void *) {
+  return false;
+}
+inline bool SoftmaxLongRows(half::half_t *d, uint32_t dstride, const half::half_t *s, uint32_t sstride,
+                            uint32_t rows, uint32_t cols, bool vec, void *stream) {
+  if (cols < static_cast<uint32_t>(hip::kHalfRowMinCols) ||
+      cols > static_cast<uint32_t>(hip::kHalfRowMaxCols)) {
+    return false;
+  }
+  void *args[] = {&d, &dstride, &s, &sstride, &cols};
+  const uint32_t grid[3] = {rows, 1, 1};
+  const uint32_t block[3] = {static_cast<uint32_t>(hip::kHalfRowBlock), 1, 1};
+  const void *kernel = vec ? reinterpret_cast<const void *>(hip::SoftmaxHalfRowKernel<true>)
+                           : reinterpret_cast<const void *>(hip::SoftmaxHalfRowKernel<false>);
+  MSHADOW_HIP_CALL(mshadow_hip_launch(kernel, grid, block, args, 0, stream));
+  return true;
+}
+#endif
+}  // namespace gpu_detail
 template <typename DType>
 inline void Softmax(Tensor<gpu, 2, DType> dst, const Tensor<gpu, 2, DType> &src) {
   CHECK_EQ(dst.shape_, src.shape_) << "Softmax: shape mismatch";
@@ -184,6 +208,12 @@ inline void Softmax(Tensor<gpu, 2, DType> dst, const Tensor<gpu, 2, DType> &src)
   DType *d = dst.dptr_;
   const DType *s = src.dptr_;
   uint32_t dstride = dst.stride_, sstride = src.stride_;
+  if (gpu_detail::SoftmaxLongRows(d, dstride, s, sstride, rows, cols,
+                                  gpu_detail::AnyPackable(s, sstride, const_cast<const DType *>(d),
+                                                          dstride, cols, hip::kAnyTile),
+                                  Stream<gpu>::GetStream(dst.stream_))) {
+    return;
+  }
   void *args[] = {&d, &dstride, &s, &sstride, &rows, &cols};
   const uint32_t grid[3] = {(rows + hip::kAnyRows - 1) / hip::kAnyRows, 1, 1};
   const uint32_t block[3] = {static_cast<uint32_t>(hip::kAnyBlock), 1, 1};
@@ -869,6 +899,15 @@ struct FastPathFor<Saver, Tensor<gpu, dim, DType>, dim, DType, E> {
   }
 };
 
+/*! \brief whole rows of `units` units (elements or packs) a launch of a map kernel covers:
+ *  its counters are 32-bit, so fewer than 2^31 units (a margin of one workgroup's reach
+ *  keeps the index of the last, partly idle, workgroup inside 32 bits) */
+inline uint32_t RowsPerLaunch(uint32_t units) {
+  const uint64_t limit = (1ull << 31) - (1u << 16);
+  const uint64_t rows = limit / (units ? units : 1);
+  return rows < 1 ? 1u : static_cast<uint32_t>(rows > 0xffffffffull ? 0xffffffffull : rows);
+}
+
 #if defined(__HIPCC__)
 template <typename K>
 inline void Launch(K kernel, uint32_t grid_x, uint32_t block_x, void **args, void *stream) {
@@ -882,21 +921,27 @@ inline void Launch(K kernel, uint32_t grid_x, uint32_t block_x, void **args, voi
 template <typename Saver, typename DType, typename DPlan, typename SPlan, bool kPackable>
 struct MapLauncher {
   inline static void Run(DPlan dplan, SPlan splan, Shape<2> shape, void *stream) {
-    uint32_t rows = shape[0], cols = shape[1];
-    if (rows == 0 || cols == 0) return;
-    uint32_t grid = 0;
-    CHECK_LT(static_cast<uint64_t>(rows) * cols, 1ull << 31) << "MapExp<gpu>: too many elements";
+    const uint32_t all_rows = shape[0];
+    uint32_t cols = shape[1];
+    if (all_rows == 0 || cols == 0) return;
     FastDivU32 div_cols(cols);
-    void *args[] = {&dplan, &splan, &rows, &cols, &div_cols};
-    const size_t total = static_cast<size_t>(rows) * cols;
-    if (cols % 4 == 0) {
-      MSHADOW_HIP_CALL(mshadow_hip_suggest_grid(total / 4, hip::kMapBlock, 32, &grid));
-      Launch(hip::MapScalarKernel<Saver, DType, DPlan, SPlan, 4>, grid, hip::kMapBlock, args,
-             stream);
-    } else {
-      MSHADOW_HIP_CALL(mshadow_hip_suggest_grid(total, hip::kMapBlock, 32, &grid));
-      Launch(hip::MapScalarKernel<Saver, DType, DPlan, SPlan, 1>, grid, hip::kMapBlock, args,
-             stream);
+    /* the kernels count elements in 32 bits: a view of 2^31 elements or more is evaluated in
+       runs of whole rows */
+    const uint32_t run_rows = RowsPerLaunch(cols);
+    for (uint32_t row0 = 0; row0 < all_rows; row0 += run_rows) {
+      uint32_t rows = all_rows - row0 < run_rows ? all_rows - row0 : run_rows;
+      uint32_t first = row0, grid = 0;
+      void *args[] = {&dplan, &splan, &rows, &cols, &div_cols, &first};
+      const size_t total = static_cast<size_t>(rows) * cols;
+      if (cols % 4 == 0) {
+        MSHADOW_HIP_CALL(mshadow_hip_suggest_grid(total / 4, hip::kMapBlock, 32, &grid));
+        Launch(hip::MapScalarKernel<Saver, DType, DPlan, SPlan, 4>, grid, hip::kMapBlock, args,
+               stream);
+      } else {
+        MSHADOW_HIP_CALL(mshadow_hip_suggest_grid(total, hip::kMapBlock, 32, &grid));
+        Launch(hip::MapScalarKernel<Saver, DType, DPlan, SPlan, 1>, grid, hip::kMapBlock, args,
+               stream);
+      }
     }
   }
 };
@@ -935,8 +980,6 @@ struct MapLauncher<Saver, DType, DPlan, SPlan, true> {
     const int N = 16 / sizeof(DType);
     uint32_t rows = shape[0], cols = shape[1];
     if (rows == 0 || cols == 0) return;
-    /* pack counts, flat offsets and the multiply-high divisions of the kernels are 32-bit */
-    CHECK_LT(static_cast<uint64_t>(rows) * cols, 1ull << 31) << "MapExp<gpu>: too many elements";
     bool flat = true;
     const bool aligned = cols % N == 0 && dplan.PackReady(N, cols, &flat) &&
                          splan.PackReady(N, cols, &flat);
@@ -945,36 +988,44 @@ struct MapLauncher<Saver, DType, DPlan, SPlan, true> {
       return;
     }
     uint32_t ppr = cols / N;
-    uint32_t total = rows * ppr;
     /* a plan that carries three or more tensor leaves (pointer + pitch each) is "deep" */
     const int kUnroll = sizeof(SPlan) >= 3 * (sizeof(void *) + sizeof(index_t))
                             ? hip::kPackUnrollDeep : hip::kPackUnroll;
     const uint32_t per_block = hip::kMapBlock * kUnroll;
-    const uint32_t grid = (total + per_block - 1) / per_block;
     FastDivU32 div_ppr(ppr);
-    void *args[] = {&dplan, &splan, &total, &ppr, &div_ppr};
     /* streaming (non-temporal) accesses once a tensor no longer fits the caches anyway */
     const bool stream_hint = static_cast<size_t>(rows) * cols * sizeof(DType) >= (8u << 20);
-    const bool is_flat = flat || rows == 1;
-    if (!is_flat &&
+    /* The kernels count packs in 32 bits, and a plan takes its column as an index_t - in a
+       flat run the column is the element's offset in the whole view: a view of 2^31 ELEMENTS
+       or more is evaluated in runs of whole rows (and then never as one flat run). */
+    const uint32_t run_rows = RowsPerLaunch(cols);
+    const bool one_run = rows <= run_rows;
+    const bool is_flat = one_run && (flat || rows == 1);
+    if (one_run && !is_flat &&
         PlanesLauncher<Saver, DType, N, kUnroll, DPlan, SPlan,
                        expr::plan_detail::PlaneWindow<SPlan>::value>::Run(dplan, splan, rows, ppr,
                                                                           stream_hint, stream)) {
       return;
     }
+    for (uint32_t row0 = 0; row0 < rows; row0 += run_rows) {
+      uint32_t first = row0;
+      uint32_t total = (rows - row0 < run_rows ? rows - row0 : run_rows) * ppr;
+      const uint32_t grid = (total + per_block - 1) / per_block;
+      void *args[] = {&dplan, &splan, &total, &ppr, &div_ppr, &first};
 #define MSHADOW_MAP_LAUNCH(FLAT, STREAM)                                                   \
   Launch(hip::MapPackKernel<Saver, DType, N, FLAT, STREAM, kUnroll, DPlan, SPlan>, grid,   \
          hip::kMapBlock, args, stream)
-    if (is_flat && stream_hint) {
-      MSHADOW_MAP_LAUNCH(true, true);
-    } else if (is_flat) {
-      MSHADOW_MAP_LAUNCH(true, false);
-    } else if (stream_hint) {
-      MSHADOW_MAP_LAUNCH(false, true);
-    } else {
-      MSHADOW_MAP_LAUNCH(false, false);
-    }
+      if (is_flat && stream_hint) {
+        MSHADOW_MAP_LAUNCH(true, true);
+      } else if (is_flat) {
+        MSHADOW_MAP_LAUNCH(true, false);
+      } else if (stream_hint) {
+        MSHADOW_MAP_LAUNCH(false, true);
+      } else {
+        MSHADOW_MAP_LAUNCH(false, false);
+      }
 #undef MSHADOW_MAP_LAUNCH
+    }
   }
 };
 #endif  // __HIPCC__

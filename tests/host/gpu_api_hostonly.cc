@@ -24,7 +24,25 @@ struct HoldsAGenerator {
 template struct HoldsAGenerator<half::half_t>;
 template struct HoldsAGenerator<int>;
 
+// The map kernels count in 32 bits; a larger view is evaluated in runs of whole rows. Nothing
+// in that split may narrow: for any row length the run stays below 2^31 units with room for
+// the last workgroup's reach, and covers at least one row.
+static bool RunsOfRowsFit() {
+  const uint32_t lengths[] = {1u, 3u, 4096u, 32768u, 65535u, (1u << 30) + 5u, 0x7fffffffu};
+  for (uint32_t units : lengths) {
+    const uint64_t rows = gpu_detail::RowsPerLaunch(units);
+    if (rows < 1) return false;
+    if (rows > 1 && rows * units + (1u << 16) > (1ull << 31)) return false;
+    if ((rows + 1) * units + (1u << 16) <= (1ull << 31) && rows != 0xffffffffull) return false;  // not the largest run
+  }
+  return true;
+}
+
 int main() {
+  if (!RunsOfRowsFit()) {
+    std::printf("FAIL runs of rows\n");
+    return 1;
+  }
   InitTensorEngine<gpu>(0);
   Stream<gpu> *s = NewStream<gpu>(0);
   const int n = 2, c = 3, h = 9, w = 12;

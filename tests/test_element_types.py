@@ -300,6 +300,54 @@ def test_gpu_half_pool(G, orc, stream, window):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("shape,pad,kind", [
+    ((3, 32000), 0, "equal"),        # every term counts until the sum stops: too many for the list
+    ((4, 31999), 1, "normal"),       # ragged rows, odd pitch
+    ((6, 4100), 4, "normal"),        # just above the shortest row this kernel takes
+    ((5, 8192), 8, "normal"),        # pitched rows of whole packs
+    ((2, 32768), 0, "normal"),       # the longest row it takes
+    ((2, 32769), 0, "normal"),       # one more: several rows per workgroup again
+    ((3, 20000), 0, "ascending"),    # the largest term comes last: the bound stays low
+    ((3, 20000), 0, "descending"),   # ... comes first
+    ((3, 24000), 0, "spike"),        # one class far above the others
+    ((2, 16000), 0, "tiny")])        # terms that are all subnormal or zero but one
+def test_gpu_half_softmax_long_rows(G, orc, stream, shape, pad, kind):
+    """rows of 4096 .. 32768 half_t are kept on chip and their sum is built from the terms that
+    can still change it (mshadow/hip/kernels/half_prune.h): bit-identical to the CPU path's
+    term-by-term sum whatever the row looks like"""
+    rng = np.random.default_rng(hash(kind) % 1000 + shape[1])
+    x = rng.standard_normal(shape, dtype=f32) * f32(3)
+    if kind == "equal":
+        x[:] = f32(0.25)
+    elif kind == "ascending":
+        x = np.sort(x, axis=1)
+    elif kind == "descending":
+        x = -np.sort(-x, axis=1)
+    elif kind == "spike":
+        x[np.arange(shape[0]), rng.integers(0, shape[1], shape[0])] += f32(30)
+    elif kind == "tiny":
+        x = x - f32(14)
+        x[:, 5000] = f32(3)
+    x = orc.float2half(x)
+    want = np.empty_like(x)
+    orc.softmax(want, x)
+    src = G.to_device(x, pad)
+    dst = G.buffer(shape, np.uint16, pad)
+    G.case_softmax(dst, src, stream)
+    got = dst.download(stream)
+    differ = int(np.count_nonzero(got != want))
+    w, g = orc.half2float(want).astype(np.float64), orc.half2float(got).astype(np.float64)
+    tol = np.maximum(2e-3 * np.abs(w), 2.0 ** -24)
+    assert np.all(np.abs(g - w) <= tol), (kind, differ)
+    if kind == "equal":
+        assert differ == 0 and np.all(g == 1.0 / 2048)
+    print(f"half softmax {shape} {kind}: {differ} of {got.size} outputs differ from the CPU path")
+    # the sum itself, free of the exponential: the library's terms, summed by the CPU path's loop
+    G.case_softmax(src, src, stream)   # in place
+    assert np.array_equal(src.download(stream), got)
+
+
+@pytest.mark.gpu
 def test_gpu_half_softmax_full_size(G, orc, stream):
     """8192 x 32000 half_t logits N(0, 3): forward within relative 2e-3 of the CPU path (the
     differences counted and printed; none observed), the gradient bit for bit, and the

@@ -169,3 +169,24 @@ def test_im2col_col2im_full(G, O, stream):
     ky = np.minimum(np.arange(h) + 1, 2) + np.minimum(h - 1 - np.arange(h), 1)
     kx = np.minimum(np.arange(w) + 1, 2) + np.minimum(w - 1 - np.arange(w), 1)
     assert np.array_equal(cnt, np.broadcast_to((ky[:, None] * kx[None, :]).astype(f32), cnt.shape))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("type_flag,dtype", [(3, np.uint8), (5, np.int8)])
+def test_map_over_more_than_2_to_the_31_elements(G, stream, type_flag, dtype):
+    """dst = a * b + c on 2^31 + 4096 one-byte elements (mshadow::kUint8 / kInt8): more than
+    the 32-bit counters of one launch cover, so the view is evaluated in runs of rows and the
+    leaves address it in 64 bits; checked against numpy's wrapping arithmetic"""
+    rows, cols = 524289, 4096
+    assert rows * cols == 2 ** 31 + 4096
+    rng = np.random.default_rng(77)
+    hosts = [rng.integers(0, 256, (rows, cols), dtype=np.uint8).view(dtype) for _ in range(3)]
+    dev = [G.to_device(h, stream=stream) for h in hosts]
+    dst = G.buffer((rows, cols), dtype)
+    G.case_map_any(0, type_flag, dst, dev[0], dev[1], dev[2], stream)
+    got = dst.download(stream)
+    want = hosts[0] * hosts[1]
+    want += hosts[2]
+    assert np.array_equal(got, want)
+    for d in dev + [dst]:
+        d.free()

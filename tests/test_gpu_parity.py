@@ -326,18 +326,6 @@ def test_softmax_exact_cases(G, stream):
         assert -6e-5 < seq_bias < -5e-6, seq_bias
 
 
-def test_map_refuses_more_elements_than_32_bit_indexing_covers(G):
-    """the elementwise kernels index with 32 bits; a 65536 x 65536 view (2^32 elements) must be
-    refused before anything is launched - on the pack path as on the scalar one - and not wrap
-    around (nothing is allocated for this: the check comes first)"""
-    tiny = G.buffer((4, 4), f32)
-    for cols in (65536, 65537):      # rows of whole packs / ragged rows
-        rc = G.cases.mshadow_case_map_axpb_f32(tiny.ptr, cols, tiny.ptr, cols, 65536, cols,
-                                               0.0, 1.0, 0.0, 0, None)
-        assert rc != 0
-        assert b"too many elements" in G.cases.mshadow_case_last_error()
-
-
 def _serial_row_sums(O, terms):
     """strictly left-to-right float32 sums of each row (the oracle's keep-dimension fold)"""
     rows, cols = terms.shape

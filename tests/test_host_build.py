@@ -45,6 +45,27 @@ def test_every_declared_symbol_is_exported(header, libname):
     assert not missing, missing
 
 
+def test_fill_runs_of_rows_do_not_overflow():
+    """tensor = scalar on 2^31 elements or more is launched in runs of whole rows; the run
+    boundaries are host arithmetic and are checked here for shapes too large to allocate
+    (INT_MAX rows of three elements: the row counter must not wrap)"""
+    lib = _lib("libmshadow_hip.so")
+    fn = lib.mshadow_hip_fill_32_runs
+    fn.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_int64), ctypes.c_int]
+    for rows, cols, wide in ((2 ** 31 - 1, 3, 0), (2 ** 31 - 1, 2, 0), (2 ** 31 - 1, 8, 1), (70000, 65536, 1),
+                             (5, 7, 0), (1, 2 ** 31 - 1, 0)):
+        runs = (ctypes.c_int64 * 64)()
+        n = fn(rows, cols, wide, runs, 32)
+        assert 1 <= n <= 32, (rows, cols, n)
+        units = cols // 4 if wide else cols
+        at = 0
+        for i in range(n):
+            first, count = runs[2 * i], runs[2 * i + 1]
+            assert first == at and count >= 1 and count * units < 2 ** 31, (rows, cols, i, first, count)
+            at += count
+        assert at == rows
+
+
 def test_python_symbol_tables_match_headers():
     from mshadow_amd import capi
 
@@ -149,6 +170,16 @@ def test_signed_column_sums_leave_most_of_the_chain(tmp_path):
     assert out.startswith("OK"), out[-500:]
     shares = {int(g): float(v) for g, v in re.findall(r"grain (\d+): ([0-9.]+)", out)}
     assert 0.10 < shares[1] < 0.18 and 0.18 < shares[4] < 0.30 and shares[64] > 0.6, shares
+
+
+def test_half_sum_pruning_rule_is_exhaustively_sound(tmp_path):
+    """the binary16 softmax row sum leaves out the terms below half an ulp of a lower bound of
+    the running sum: for every pair of a finite non-negative binary16 sum and term the rule
+    drops, half_t's `sum += term` indeed returns the sum unchanged (all 10^9 pairs)"""
+    out = _compile_and_run(tmp_path, "half_prune_check.cc", [])
+    assert out.startswith("OK"), out[-500:]
+    dropped, kept_noops = (int(v) for v in out.split()[1:3])
+    assert dropped > 10 ** 8 and kept_noops < 10 ** 5   # sound, and nearly tight (ties stay in)
 
 
 def test_header_api_on_cpu_matches_oracle(tmp_path, orc):
