@@ -244,10 +244,13 @@ int mshadow_hip_permute_32(void *dst, const void *src, int ndim, const int *shap
 int mshadow_hip_sort_by_key_workspace(size_t n, size_t *bytes);
 int mshadow_hip_sort_by_key_32(void *keys, int key_kind, void *values, size_t n, int is_ascend,
                                void *workspace, size_t workspace_bytes, void *stream);
-/* The same sort for callers that cannot allocate device memory (code under graph capture,
-   serving loops, harnesses that forbid it). It has no counterpart in the reference. The
-   scratch memory is an array inside the library, one copy per GPU (about 40 MiB, held from
-   the library's load until the process ends); the call itself allocates and frees nothing.
+/* The same sort for callers that cannot allocate device memory (serving loops, harnesses
+   that forbid it). It has no counterpart in the reference. The scratch memory is an array
+   inside the library, one copy per GPU (about 40 MiB, held from the library's load until the
+   process ends); the call itself allocates and frees nothing. Where the array lives on a GPU
+   is looked up when mshadow_hip_set_device selects that GPU (else on the first call there);
+   a call then consists of a host-side size query and three kernel launches. It has not been
+   exercised under graph capture.
    At most MSHADOW_HIP_SORT_NOALLOC_MAX pairs; more is an argument error. Every call on a GPU
    uses that GPU's one array: calls that overlap in time on the same GPU (different streams
    or host threads) race on it and must be ordered by the caller. */

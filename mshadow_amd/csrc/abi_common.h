@@ -33,6 +33,10 @@ inline hipStream_t AsStream(void *s) { return reinterpret_cast<hipStream_t>(s); 
    (mshadow/cuda/tensor_gpu-inl.cuh:16-21); hipGetLastError also clears the sticky code */
 inline int AfterLaunch(const char *what) { return FromHip(hipGetLastError(), what); }
 
+/* looks up, once per device, where the scratch array of the sort that allocates nothing lives
+   on the current device (csrc/sort.hip) */
+void ResolveSortScratch();
+
 /* compute units of the calling thread's device (looked up once per thread) */
 int ComputeUnits();
 

@@ -52,6 +52,7 @@ int mshadow_hip_device_count(int *count) {
 }
 int mshadow_hip_set_device(int device) {
   ABI_HIP(hipSetDevice(device));
+  ResolveSortScratch();
   return MSHADOW_HIP_OK;
 }
 int mshadow_hip_get_device(int *device) {

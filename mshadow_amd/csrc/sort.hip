@@ -154,6 +154,16 @@ int ScratchOfCurrentDevice(char **ptr) {
 
 }  // namespace
 
+namespace mshadow_abi {
+/* called when a device is selected (mshadow_hip_set_device): the runtime's lookup of the
+   scratch array on that device - loading the code object there, if need be - happens then and
+   not inside the first sort */
+void ResolveSortScratch() {
+  char *unused = NULL;
+  if (ScratchOfCurrentDevice(&unused) != MSHADOW_HIP_OK) (void)hipGetLastError();
+}
+}  // namespace mshadow_abi
+
 extern "C" {
 
 int mshadow_hip_sort_by_key_workspace(size_t n, size_t *bytes) {

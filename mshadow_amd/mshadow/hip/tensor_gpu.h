@@ -543,6 +543,28 @@ template <>
 struct SortKeyKind<int32_t> { static const int value = MSHADOW_HIP_KEY_I32; };
 template <>
 struct SortKeyKind<uint32_t> { static const int value = MSHADOW_HIP_KEY_U32; };
+/*! \brief device memory that is given back when its owner goes out of scope - also when a
+ *  failed call between allocation and release throws (DMLC_LOG_FATAL_THROW builds) */
+struct ScopedDeviceBlock {
+  void *ptr;
+  ScopedDeviceBlock() : ptr(NULL) {}
+  ~ScopedDeviceBlock() {
+    if (ptr != NULL) (void)mshadow_hip_free(ptr);
+  }
+  inline void Allocate(size_t bytes) {
+    size_t pitch = 0;
+    MSHADOW_HIP_CALL(mshadow_hip_malloc_pitch(&ptr, &pitch, bytes, 1));
+  }
+  inline void Release() {
+    void *p = ptr;
+    ptr = NULL;
+    MSHADOW_HIP_CALL(mshadow_hip_free(p));
+  }
+
+ private:
+  ScopedDeviceBlock(const ScopedDeviceBlock &);
+  ScopedDeviceBlock &operator=(const ScopedDeviceBlock &);
+};
 /*! \brief the device sort for key / value types the library's 32-bit entry point does not
  *  take: through a permutation, one stable 32-bit pass per key word (kernels/sort_any.h) */
 template <typename KDType, typename VDType>
@@ -552,7 +574,7 @@ inline void SortByKeyThroughPermutation(Tensor<gpu, 1, KDType> keys, Tensor<gpu,
   const size_t n = keys.size(0);
   CHECK_LT(n, 1ull << 31) << "SortByKey: too many elements";
   void *stream = Stream<gpu>::GetStream(keys.stream_);
-  size_t sort_bytes = 0, pitch = 0;
+  size_t sort_bytes = 0;
   MSHADOW_HIP_CALL(mshadow_hip_sort_by_key_workspace(n, &sort_bytes));
   /* words | permutation | copy of the keys | copy of the values | the sort's scratch, each
      part starting on a multiple of 256 bytes */
@@ -562,9 +584,9 @@ inline void SortByKeyThroughPermutation(Tensor<gpu, 1, KDType> keys, Tensor<gpu,
   const size_t keys_at = perm_at + (n * 4 + part - 1) / part * part;
   const size_t vals_at = keys_at + (n * sizeof(KDType) + part - 1) / part * part;
   const size_t sort_at = vals_at + (n * sizeof(VDType) + part - 1) / part * part;
-  void *block = NULL;
-  MSHADOW_HIP_CALL(mshadow_hip_malloc_pitch(&block, &pitch, sort_at + sort_bytes, 1));
-  char *base = static_cast<char *>(block);
+  ScopedDeviceBlock block;
+  block.Allocate(sort_at + sort_bytes);
+  char *base = static_cast<char *>(block.ptr);
   uint32_t *words = reinterpret_cast<uint32_t *>(base + words_at);
   uint32_t *perm = reinterpret_cast<uint32_t *>(base + perm_at);
   KDType *keys_copy = reinterpret_cast<KDType *>(base + keys_at);
@@ -615,7 +637,7 @@ inline void SortByKeyThroughPermutation(Tensor<gpu, 1, KDType> keys, Tensor<gpu,
                                         grid, block_dim, args, 0, stream));
   }
   MSHADOW_HIP_CALL(mshadow_hip_stream_sync(stream));
-  MSHADOW_HIP_CALL(mshadow_hip_free(block));
+  block.Release();
 #else
   LOG(FATAL) << "SortByKey<gpu> of these element types: compile the calling translation unit with hipcc";
 #endif
@@ -633,14 +655,14 @@ struct SortRoute<KDType, VDType, true> {
   inline static void Run(Tensor<gpu, 1, KDType> keys, Tensor<gpu, 1, VDType> values, bool is_ascend) {
     const size_t n = keys.size(0);
     void *stream = Stream<gpu>::GetStream(keys.stream_);
-    size_t bytes = 0, pitch = 0;
-    void *workspace = NULL;
+    size_t bytes = 0;
+    ScopedDeviceBlock workspace;
     MSHADOW_HIP_CALL(mshadow_hip_sort_by_key_workspace(n, &bytes));
-    MSHADOW_HIP_CALL(mshadow_hip_malloc_pitch(&workspace, &pitch, bytes, 1));
+    workspace.Allocate(bytes);
     MSHADOW_HIP_CALL(mshadow_hip_sort_by_key_32(keys.dptr_, SortKeyKind<KDType>::value, values.dptr_, n,
-                                                is_ascend ? 1 : 0, workspace, bytes, stream));
+                                                is_ascend ? 1 : 0, workspace.ptr, bytes, stream));
     MSHADOW_HIP_CALL(mshadow_hip_stream_sync(stream));
-    MSHADOW_HIP_CALL(mshadow_hip_free(workspace));
+    workspace.Release();
   }
 };
 template <typename VDType>
