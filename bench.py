@@ -76,6 +76,9 @@ def algorithmic_bytes():
         "softmax_grad_f16": 2 * 2 * 8192 * 32000 + 2 * 8192,
         "sum_rows_f16": 2 * 16384 * 4096 + 2 * 4096,
         "sumall_except_dim1_f16": 2 * 64 * 256 * 56 * 56 + 2 * 256,
+        # sumall_except_dim<1> where few indices are kept: (64,64,112,112) and (256,16,112,112)
+        "sumall_except_dim1_64_kept": e * 64 * 64 * 112 * 112 + e * 64,
+        "sumall_except_dim1_16_kept": e * 256 * 16 * 112 * 112 + e * 16,
     }
 
 
@@ -95,6 +98,7 @@ def work_elements():
         "random_uniform": 8192 * 32000, "random_normal": 8192 * 32000,
         "softmax_f16": 8192 * 32000, "softmax_grad_f16": 8192 * 32000,
         "sum_rows_f16": 16384 * 4096, "sumall_except_dim1_f16": 64 * 256 * 56 * 56,
+        "sumall_except_dim1_64_kept": 64 * 64 * 112 * 112, "sumall_except_dim1_16_kept": 256 * 16 * 112 * 112,
     }
 
 
@@ -116,7 +120,8 @@ EXTRA_OPS = ("calib_copy", "smooth_softmax_grad_ignore", "softmax3d", "softmax3d
              "bias_add_broadcast", "swapaxis10_reshape", "lrn_scale_chpool5", "transpose_nchw_nhwc",
              "sort_by_key_f32", "dot_f32_4096", "dot_f16_8192", "ceiling_copy", "ceiling_fill",
              "random_uniform", "random_normal", "softmax_f16", "softmax_grad_f16", "sum_rows_f16",
-             "sumall_except_dim1_f16", "copy_d2d", "copy_d2d_pitched", "copy_d2d_ragged")
+             "sumall_except_dim1_f16", "copy_d2d", "copy_d2d_pitched", "copy_d2d_ragged",
+             "sumall_except_dim1_64_kept", "sumall_except_dim1_16_kept")
 OPS = [k for k in algorithmic_bytes() if k not in EXTRA_OPS]
 
 # HBM bytes per launch of each operation's kernel come from the committed counter summary
@@ -194,6 +199,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--scale", type=int, default=1, help="shrink leading dims (functional runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--sets", type=int, default=3, help="complete operand sets the steps take in turn "
+                    "(1 = every step on the same buffers; the default keeps a launch from finding "
+                    "its operands in the memory-side cache)")
     ap.add_argument("--cpu-reps", type=int, default=30)
     ap.add_argument("--only", default="", help="comma list of ops to run (profiling aid); "
                     "softmax_phases, ceiling_chain and ceiling_lds_loads run the probes of "
@@ -241,7 +249,7 @@ def main():
     # what pool and softmax wrote - from the NEXT set (written two steps ago, same values), not
     # from the launch that has just finished.
     rotate = args.scale == 1 and all(o in OPS for o in only)
-    sets = [buffer_set() for _ in range(3 if rotate else 1)]
+    sets = [buffer_set() for _ in range(max(1, args.sets) if rotate else 1)]
     cur = dict(sets[0])     # the set run_op works on
     nxt = dict(sets[1 % len(sets)])   # where unpool / softmax_grad take their producer's output
     dev = cur["dev"]
@@ -324,6 +332,12 @@ def main():
             G.case_reduce_keep_lowest(extra["h2b"], extra["hM"], 0, 0, 0x3C00, 0, s)
         elif name == "sumall_except_dim1_f16":
             G.case_reduce_keep_highdim(extra["h2a"], extra["hX"], 0, 0, 0x3C00, 0, s)
+        elif name == "sumall_except_dim1_64_kept":   # the floats of X2a read as (64,64,112,112)
+            G.check(G.dll.mshadow_hip_reduce_keep_highdim_f32(
+                cur["out_2a"].ptr, cur["dev"]["X2a"].ptr, 112, 64, 64, 112, 112, 0, 0, 1.0, s))
+        elif name == "sumall_except_dim1_16_kept":   # ... and as (256,16,112,112)
+            G.check(G.dll.mshadow_hip_reduce_keep_highdim_f32(
+                cur["out_2a"].ptr, cur["dev"]["X2a"].ptr, 112, 256, 16, 112, 112, 0, 0, 1.0, s))
         elif name == "dot_f32_4096":
             G.case_dot(1, extra["mm_out"], dev["A"], dev["B"], 4096, 4096, 4096, 1, s)
         elif name == "dot_f16_8192":

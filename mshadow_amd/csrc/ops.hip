@@ -132,9 +132,20 @@ int Im2Col(T *col, int cstride, const T *img, int istride, const PatchGeom &g, v
       t.pitch = (g.wp + 7) / 8 * 8;
       const size_t lds = static_cast<size_t>(t.rows_max) * t.pitch * sizeof(T);
       const mshadow::FastDivU32 div_ppr(static_cast<uint32_t>(g.ow / 8));
-      hipLaunchKernelGGL(Im2ColHalfRow3Kernel, dim3(static_cast<unsigned>(blocks)), dim3(kPatchBlock),
-                         lds, AsStream(stream), reinterpret_cast<uint16_t *>(col), cstride,
-                         reinterpret_cast<const uint16_t *>(img), istride, g, t, div_ppr);
+      /* rows without padding between them and made of whole aligned packs: staged by packs */
+      const bool dense = istride == g.w && g.w % 8 == 0 && reinterpret_cast<uintptr_t>(img) % 16 == 0;
+      const mshadow::FastDivU32 div_w(static_cast<uint32_t>(g.w));
+      if (dense) {
+        hipLaunchKernelGGL(Im2ColHalfRow3Kernel<true>, dim3(static_cast<unsigned>(blocks)),
+                           dim3(kPatchBlock), lds, AsStream(stream), reinterpret_cast<uint16_t *>(col),
+                           cstride, reinterpret_cast<const uint16_t *>(img), istride, g, t, div_ppr,
+                           div_w);
+      } else {
+        hipLaunchKernelGGL(Im2ColHalfRow3Kernel<false>, dim3(static_cast<unsigned>(blocks)),
+                           dim3(kPatchBlock), lds, AsStream(stream), reinterpret_cast<uint16_t *>(col),
+                           cstride, reinterpret_cast<const uint16_t *>(img), istride, g, t, div_ppr,
+                           div_w);
+      }
       return AfterLaunch("im2col");
     }
     const size_t lds = static_cast<size_t>(t.rows_max) * row_bytes;

@@ -490,6 +490,10 @@ CONV = [  # n, c, h, w, ky, kx, sy, sx, dy, dx, py, px
     (3, 5, 19, 23, 5, 3, 2, 1, 1, 1, 2, 1), (2, 3, 19, 23, 3, 3, 1, 1, 2, 2, 2, 2),
     (2, 3, 9, 8, 2, 3, 1, 2, 2, 2, 1, 0), (1, 1, 6, 6, 3, 3, 2, 2, 1, 1, 0, 0),
     (2, 4, 7, 7, 1, 1, 1, 1, 1, 1, 0, 0), (1, 2, 30, 31, 7, 7, 3, 3, 1, 1, 3, 3),
+    # dense rows of whole packs, staged pack by pack: many small planes; 5 taps down; planes
+    # cut into several bands of rows
+    (40, 64, 16, 16, 3, 3, 1, 1, 1, 1, 1, 1), (3, 700, 8, 24, 5, 3, 1, 1, 1, 1, 2, 1),
+    (1, 2, 300, 128, 3, 3, 1, 1, 1, 1, 1, 1), (2, 1, 181, 264, 4, 3, 1, 1, 1, 1, 2, 1),
 ]
 
 
