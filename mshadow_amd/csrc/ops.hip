@@ -132,9 +132,26 @@ int Im2Col(T *col, int cstride, const T *img, int istride, const PatchGeom &g, v
       t.pitch = (g.wp + 7) / 8 * 8;
       const size_t lds = static_cast<size_t>(t.rows_max) * t.pitch * sizeof(T);
       const mshadow::FastDivU32 div_ppr(static_cast<uint32_t>(g.ow / 8));
-      /* rows without padding between them and made of whole aligned packs: staged by packs */
+      /* rows without padding between them and made of whole aligned packs: fetched by packs -
+         straight into the taps where the image is padded by one column, else staged */
       const bool dense = istride == g.w && g.w % 8 == 0 && reinterpret_cast<uintptr_t>(img) % 16 == 0;
       const mshadow::FastDivU32 div_w(static_cast<uint32_t>(g.w));
+      if (dense && g.pad_x == 1 && g.ow == g.w) {
+        const uint32_t places = static_cast<uint32_t>(cols / 8);
+        const uint32_t per_block = kPatchBlock * kIm2ColDirectPer;
+        const uint32_t chunks = (places + per_block - 1) / per_block;
+        const long long pieces = (static_cast<long long>(g.c) * chunks + 7) / 8 * 8;
+        const long long direct_blocks = pieces * g.ky;
+        if (direct_blocks < (1ll << 31)) {
+          hipLaunchKernelGGL(Im2ColHalfRow3DirectKernel<kIm2ColDirectPer>,
+                             dim3(static_cast<unsigned>(direct_blocks)), dim3(kPatchBlock), 0,
+                             AsStream(stream), reinterpret_cast<uint16_t *>(col), cstride,
+                             reinterpret_cast<const uint16_t *>(img), g, div_ppr,
+                             mshadow::FastDivU32(static_cast<uint32_t>(g.oh)), chunks,
+                             mshadow::FastDivU32(chunks));
+          return AfterLaunch("im2col");
+        }
+      }
       if (dense) {
         hipLaunchKernelGGL(Im2ColHalfRow3Kernel<true>, dim3(static_cast<unsigned>(blocks)),
                            dim3(kPatchBlock), lds, AsStream(stream), reinterpret_cast<uint16_t *>(col),

@@ -257,6 +257,77 @@ __global__ void __launch_bounds__(kPatchBlock)
   }
 }
 
+/*! \brief The same copy with no staging at all, for dense images padded by one column on each
+ *  side (ow == w): a thread makes the three packs (b = 0, 1, 2) of one place (a, oy, ox..ox+7)
+ *  of one channel from the aligned pack of image row oy + a - pad_y at ox and the element on
+ *  either side of it, and stores them. A workgroup is 256 consecutive places of one (channel,
+ *  a) pair - the three rows of the column matrix are contiguous over images and patch rows -
+ *  and ends after its three stores per thread, so the machine sees many small independent
+ *  pieces, the form in which plain copies and fills run fastest here. The image is read
+ *  ky times, the repeats from L2. MI355X, (32,256,56,56), pad 1: 92-94 us with the image
+ *  coming from HBM and 78 us with the image in the memory-side cache, against 100-103 us
+ *  and 86 us for the staged kernel above; two or four places per thread (PER) are slower
+ *  (111 / 115 us), as is one thread storing all nine packs that one image pack feeds (125 us). */
+const int kIm2ColDirectPer = 1;
+template <int PER>
+__global__ void __launch_bounds__(kPatchBlock)
+    Im2ColHalfRow3DirectKernel(uint16_t *col, int cstride, const uint16_t *img, PatchGeom g,
+                               mshadow::FastDivU32 div_ppr, mshadow::FastDivU32 div_oh,
+                               uint32_t chunks, mshadow::FastDivU32 div_chunks) {
+  typedef uint16_t T;
+  /* Workgroups are dealt to the XCDs in turn, eight at a time. The ky workgroups that read
+     the same piece of the image (one per tap row a) get numbers 8 apart: they run on one XCD
+     at about the same time, and its L2 fetches that piece once.
+     blockIdx = ((piece / 8) * ky + a) * 8 + piece % 8, piece = ch * chunks + chunk */
+  const uint32_t lane8 = blockIdx.x & 7u;
+  const uint32_t turn = blockIdx.x >> 3;
+  const uint32_t group = turn / static_cast<uint32_t>(g.ky);
+  const int a = static_cast<int>(turn - group * g.ky);
+  const uint32_t piece = group * 8 + lane8;
+  const uint32_t ch = div_chunks.Div(piece);
+  if (ch >= static_cast<uint32_t>(g.c)) return;
+  const uint32_t chunk = piece - ch * chunks;
+  const uint32_t row3 = ch * g.ky + a;
+  const uint32_t ppr = static_cast<uint32_t>(g.ow) / 8;
+  const uint32_t places = static_cast<uint32_t>(g.n) * g.oh * ppr;
+  U4 w03[PER], mid[PER], hi[PER];
+#pragma unroll
+  for (int u = 0; u < PER; ++u) {
+    const uint32_t pk = (chunk * PER + u) * kPatchBlock + threadIdx.x;
+    w03[u] = mid[u] = hi[u] = U4{0u, 0u, 0u, 0u};
+    if (pk >= places) continue;
+    const uint32_t line = div_ppr.Div(pk);             // n * oh + oy
+    const int ox = static_cast<int>(pk - line * ppr) * 8;
+    const uint32_t n = div_oh.Div(line);
+    const int oy = static_cast<int>(line - n * g.oh);
+    const int y = oy + a - g.pad_y;
+    if (y >= 0 && y < g.h) {
+      const T *in = img + (static_cast<size_t>(n * g.c + ch) * g.h + y) * g.w + ox;
+      const U4 m = *reinterpret_cast<const U4 *>(in);
+      const uint32_t before = ox > 0 ? in[-1] : 0u;
+      const uint32_t after = ox + 8 < g.w ? in[8] : 0u;
+      mid[u] = m;
+      w03[u].x = (m.x << 16) | before;
+      w03[u].y = __builtin_amdgcn_alignbit(m.y, m.x, 16);
+      w03[u].z = __builtin_amdgcn_alignbit(m.z, m.y, 16);
+      w03[u].w = __builtin_amdgcn_alignbit(m.w, m.z, 16);
+      hi[u].x = w03[u].y;
+      hi[u].y = w03[u].z;
+      hi[u].z = w03[u].w;
+      hi[u].w = (after << 16) | (m.w >> 16);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < PER; ++u) {
+    const uint32_t pk = (chunk * PER + u) * kPatchBlock + threadIdx.x;
+    if (pk >= places) continue;
+    T *out = col + static_cast<size_t>(row3 * 3) * cstride + static_cast<size_t>(pk) * 8;
+    StreamStore16(out, w03[u]);
+    StreamStore16(out + cstride, mid[u]);
+    StreamStore16(out + 2 * static_cast<size_t>(cstride), hi[u]);
+  }
+}
+
 /*! \brief FAST: stride 1 and dilation 1 in both directions (the common convolution case):
  *  every patch-range bound is then a subtraction instead of a division. */
 template <typename T, int EPT, bool FAST>

@@ -226,13 +226,20 @@ __global__ void __launch_bounds__(kPermuteBlock)
   }
 }
 
-const int kCopyUnroll = 4;
-const uint32_t kCopyMaxUnits = (1u << 31) - kPermuteBlock * kCopyUnroll;  // per launch
+/* 16 bytes per thread, whatever the unit: 8192x32000 floats by 16-byte units in 321 us with one
+   unit per thread, 345 us with four, 500 us with eight (MI355X) */
+template <typename T>
+struct CopyUnroll {
+  static const int value = sizeof(T) >= 16 ? 1 : 16 / sizeof(T);
+};
+const int kCopyMaxUnroll = 4;
+const uint32_t kCopyMaxUnits = (1u << 31) - kPermuteBlock * kCopyMaxUnroll;  // per launch
 
 template <typename T>
 void LaunchCopyRows(void *dst, size_t dpitch_bytes, const void *src, size_t spitch_bytes,
                     size_t width_bytes, size_t rows, hipStream_t s) {
   const size_t unit = sizeof(T);
+  const int kCopyUnroll = CopyUnroll<T>::value;
   const bool dense = rows == 1 || (dpitch_bytes == width_bytes && spitch_bytes == width_bytes);
   size_t per_row = width_bytes / unit;
   if (dense) {  // one run of rows * width bytes, cut into launches the 32-bit counters cover
@@ -269,7 +276,7 @@ namespace mshadow_abi {
    - both addresses, the width and (with more than one row) both pitches - is a multiple of 4
    bytes; false: not covered, the caller uses the runtime's copy. The runtime's own 2-D copy
    reaches 0.73 of the HBM peak on rows of a kilobyte multiple and 0.36 on rows of 127,960
-   bytes at a pitch of 128,000; this kernel 0.74 on either (8192 rows, MI355X). */
+   bytes at a pitch of 128,000; this kernel 0.79-0.81 and 0.71 (8192 rows, MI355X). */
 bool CopyRowsOnDevice(void *dst, size_t dpitch_bytes, const void *src, size_t spitch_bytes,
                       size_t width_bytes, size_t rows, hipStream_t s) {
   size_t all = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src) | width_bytes;
@@ -328,7 +335,7 @@ extern "C" int mshadow_hip_fill_32(void *dst, int dstride, int rows, int cols, u
     const int64_t nrows = std::min<int64_t>(rows_per_launch, rows - row0);
     uint32_t *first = static_cast<uint32_t *>(dst) + static_cast<size_t>(row0) * dstride;
     uint64_t blocks = (static_cast<uint64_t>(nrows) * ppr + kPermuteBlock - 1) / kPermuteBlock;
-    if (blocks > 65536) blocks = 65536;
+    if (blocks > (1u << 20)) blocks = 1u << 20;
     if (wide) {
       hipLaunchKernelGGL(FillKernel<4>, dim3(static_cast<unsigned>(blocks)), dim3(kPermuteBlock), 0,
                          AsStream(stream), first, static_cast<uint32_t>(dstride),
@@ -417,7 +424,7 @@ extern "C" int mshadow_hip_permute_32(void *dst, const void *src, int ndim, cons
     const uint32_t ppr = wide ? cols / 4 : cols;
     const uint64_t work = static_cast<uint64_t>(rows) * ppr;
     uint64_t blocks = (work + kPermuteBlock - 1) / kPermuteBlock;
-    if (blocks > 65536) blocks = 65536;
+    if (blocks > (1u << 20)) blocks = 1u << 20;
     if (wide) {
       hipLaunchKernelGGL(PermuteRowsKernel<4>, dim3(static_cast<unsigned>(blocks)), dim3(kPermuteBlock),
                          0, s, d, sp, rows, cols, FastDivU32(ppr), ba);

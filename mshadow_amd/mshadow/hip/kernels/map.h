@@ -29,10 +29,13 @@ namespace hip {
 
 const int kMapBlock = 256;
 /*! \brief packs per thread; the loads of all of them are issued before the first use.
- *  Expressions that read several tensors take the deeper one (measured on the 4-in 1-out
- *  map: 56 us against 59 us), a one-tensor map the shallower (more workgroups). */
-const int kPackUnroll = 4;
-const int kPackUnrollDeep = 8;
+ *  One pack per thread and many small workgroups serve a one- or two-tensor map best
+ *  (MI355X: dst = src over 8192x32000 floats 337 us against 353 us with four packs;
+ *  dst = x + broadcast<1>(bias) over (64,256,56,56) 70 us against 80 us); an expression
+ *  that reads three tensors or more takes four (the 4-in 1-out map: 57 us, 58-59 us
+ *  with two or eight). */
+const int kPackUnroll = 1;
+const int kPackUnrollDeep = 4;
 
 /*! \brief PER consecutive elements of one row per thread-iteration (PER divides cols): the
  *  PER evaluations are independent, so their loads are in flight together, and where a
