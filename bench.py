@@ -133,7 +133,7 @@ TRAFFIC_ROW_OF_OP = {
     "map_fused": "map_fused", "sumall_except_dim1": "ReduceKeepHighDimDmaKernel",
     "sum_rows": "ReduceKeepLowestDmaKernel", "softmax": "SoftmaxRowKernel",
     "softmax_grad": "SoftmaxGradKernel", "pool_max": "PoolKernel", "unpool_max": "UnpoolRows3x3s2Kernel",
-    "im2col_f16": "Im2ColHalfRow3Kernel", "col2im_f16": "Col2ImHalfRows3x3Kernel",
+    "im2col_f16": "Im2ColHalfRow3DirectKernel", "col2im_f16": "Col2ImHalfRows3x3Kernel",
 }
 
 
@@ -203,6 +203,9 @@ def main():
                     "(1 = every step on the same buffers; the default keeps a launch from finding "
                     "its operands in the memory-side cache)")
     ap.add_argument("--cpu-reps", type=int, default=30)
+    ap.add_argument("--hold", default="", help="comma list of operands that stay those of the first "
+                    "set while the others rotate (profiling aid): dimg, out_col, out_unpool, dev.X4, "
+                    "dev.G4, ... and nxt for the producer outputs unpool / softmax_grad read")
     ap.add_argument("--only", default="", help="comma list of ops to run (profiling aid); "
                     "softmax_phases, ceiling_chain and ceiling_lds_loads run the probes of "
                     "libmshadow_probe.so instead")
@@ -255,9 +258,20 @@ def main():
     dev = cur["dev"]
     out_map, out_g, out_p = cur["out_map"], cur["out_g"], cur["out_p"]
 
+    hold = [x for x in args.hold.split(",") if x]
+
     def use_set(k):
         cur.update(sets[k % len(sets)])
         nxt.update(sets[(k + 1) % len(sets)])
+        if any(x.startswith("dev.") for x in hold):
+            cur["dev"] = dict(cur["dev"])
+        for x in hold:
+            if x == "nxt":
+                nxt.update(sets[0])
+            elif x.startswith("dev."):
+                cur["dev"][x[4:]] = sets[0]["dev"][x[4:]]
+            else:
+                cur[x] = sets[0][x]
 
     extra = {}
     if any(o in EXTRA_OPS[1:] for o in only):
@@ -627,7 +641,9 @@ def run_probe(G, which, pattern=""):
                                for b, k in ((0, 0), (4, 0), (4, 2), (4, 4), (4, 8), (8, 4))},
                "row_copy_one_row_per_cu_us": round(min(P.row_copy_us(dst, src, 0, 0, s, 1) for _ in range(3)), 1)}
         # how long the steps take when a row has its CU to itself, on 8 and on 16 waves
-        for variant, name in ((1, "one_row_per_cu_512_threads"), (2, "one_row_per_cu_1024_threads")):
+        # ... and with three rows per CU on four waves each (128 floats of the row per thread)
+        for variant, name in ((1, "one_row_per_cu_512_threads"), (2, "one_row_per_cu_1024_threads"),
+                              (3, "three_rows_per_cu_256_threads")):
             st, res, ker, fb = P.softmax_phases(dst, src, s, variant)
             out[name] = {"steps": {k: round(v, 2) for k, v in st.items()}, "row_resident_us": round(res, 2),
                          "kernel_us": round(ker, 1), "fallback_rows": fb}

@@ -553,7 +553,7 @@ int mshadow_probe_highdim_split(float *dst, const float *warm, const float *src,
 int mshadow_probe_softmax_phases(float *dst, int dstride, const float *src, int sstride, int rows,
                                  int cols, int variant, double *mean_us, double *resident_us,
                                  double *kernel_us, int *fallback_rows, void *stream) {
-  ABI_REQUIRE(variant >= 0 && variant <= 2, "variant 0, 1 or 2");
+  ABI_REQUIRE(variant >= 0 && variant <= 3, "variant 0 to 3");
   ABI_REQUIRE(rows >= 1 && cols > 16384 && cols <= 32768 && cols % 4 == 0 && sstride % 4 == 0 &&
                   dstride % 4 == 0, "the probe covers the 512-thread, 16-slab kernel: 16384 < cols <= 32768, rows of whole packs");
   ABI_REQUIRE(mean_us != NULL && resident_us != NULL && kernel_us != NULL && fallback_rows != NULL,
@@ -573,9 +573,12 @@ int mshadow_probe_softmax_phases(float *dst, int dstride, const float *src, int 
     } else if (variant == 1) {  // one row per CU: LDS the kernel never touches keeps a second one off
       hipLaunchKernelGGL((mshadow_hipk::SoftmaxRowKernel<512, 16, 4, false>), dim3(rows), dim3(512),
                          90000, s, dst, dstride, src, sstride, cols);
-    } else {  // one row per CU, on sixteen waves
+    } else if (variant == 2) {  // one row per CU, on sixteen waves
       hipLaunchKernelGGL((mshadow_hipk::SoftmaxRowKernel<1024, 8, 4, false>), dim3(rows), dim3(1024),
                          90000, s, dst, dstride, src, sstride, cols);
+    } else {  // three rows per CU, four waves each (a wave per SIMD, 168 registers)
+      hipLaunchKernelGGL((mshadow_hipk::SoftmaxRowKernel<256, 32, 4, false, 3>), dim3(rows), dim3(256),
+                         0, s, dst, dstride, src, sstride, cols);
     }
   });
   if (st != MSHADOW_HIP_OK) {

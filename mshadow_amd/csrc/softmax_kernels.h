@@ -731,8 +731,8 @@ __device__ inline float BlockMax(float v, float *wmax) {
  *  slab, wave, lane, element.
  *  TERMS_GIVEN: src already holds the (non-negative) terms and dst[row] receives their
  *  left-to-right sum - the row-sum stage on its own. */
-template <int THREADS, int SLABS, int VEC, bool TERMS_GIVEN>
-__global__ void __launch_bounds__(THREADS, 4)  // >= 4 waves per SIMD: two 512-thread rows per CU
+template <int THREADS, int SLABS, int VEC, bool TERMS_GIVEN, int MIN_WAVES = 4>
+__global__ void __launch_bounds__(THREADS, MIN_WAVES)  // 4 waves per SIMD: two 512-thread rows per CU
     SoftmaxRowKernel(float *dst, int dstride, const float *src, int sstride, int cols) {
   __shared__ RowSumLds<THREADS / kWave, SLABS, VEC> lds;
   const int W = THREADS / kWave;
