@@ -133,7 +133,7 @@ TRAFFIC_ROW_OF_OP = {
     "map_fused": "map_fused", "sumall_except_dim1": "ReduceKeepHighDimDmaKernel",
     "sum_rows": "ReduceKeepLowestDmaKernel", "softmax": "SoftmaxRowKernel",
     "softmax_grad": "SoftmaxGradKernel", "pool_max": "PoolKernel", "unpool_max": "UnpoolRows3x3s2Kernel",
-    "im2col_f16": "Im2ColHalfRow3DirectKernel", "col2im_f16": "Col2ImHalfRows3x3Kernel",
+    "im2col_f16": "Im2ColRow3DirectKernel", "col2im_f16": "Col2ImHalfRows3x3Kernel",
 }
 
 
@@ -224,6 +224,8 @@ def main():
     if args.only in ("softmax_phases", "ceiling_chain", "ceiling_lds_loads", "ceiling_seg_loads",
                      "softmax_prefetch_copy", "highdim_split_configs"):
         return run_probe(G, args.only, args.pattern)
+    if args.only == "neighbour_shapes":
+        return neighbour_shapes(G)
     props = G.props(0)
     only = [o for o in args.only.split(",") if o] or OPS
 
@@ -523,6 +525,85 @@ def main():
     if cpu is not None:
         out["cpu_baseline"] = {k: v for k, v in cpu.items() if k != "per_op_ms"}
     print(json.dumps(out))
+
+
+def neighbour_shapes(G):
+    """`--only neighbour_shapes`: the fixed-function operations on shapes next to the BASELINE
+    ones (other windows, strides, paddings, plane sizes, row lengths, float images), each
+    launched 10 times on the same buffers after 2 warm-up launches - small operands stay in the
+    caches, so these are upper figures. Prints one JSON line: op, shape, us, GB/s over the
+    algorithmic bytes, fraction of the HBM peak."""
+    s = G.stream_create()
+    rng = np.random.default_rng(3)
+    rows_out = []
+
+    def timeit(fn, reps=10):
+        for _ in range(2):
+            fn()
+        G.stream_sync(s)
+        a, b = G.event_create(), G.event_create()
+        G.event_record(a, s)
+        for _ in range(reps):
+            fn()
+        G.event_record(b, s)
+        G.event_sync(b)
+        return G.elapsed_ms(a, b) / reps * 1e3
+
+    def report(op, shape, nbytes, us):
+        rows_out.append({"op": op, "shape": shape, "us": round(us, 1), "GBps": round(nbytes / us / 1e3),
+                         "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 3)})
+
+    def big(shape):
+        return rng.standard_normal(int(np.prod(shape)), dtype=f32).reshape(shape)
+
+    for shape, k, st in (((128, 64, 112, 112), 2, 2), ((128, 64, 112, 112), 3, 2), ((128, 64, 112, 112), 3, 1),
+                         ((64, 96, 55, 55), 3, 2), ((256, 256, 13, 13), 3, 2), ((32, 64, 224, 224), 2, 2),
+                         ((128, 256, 28, 28), 2, 2)):
+        n, c, h, w = shape
+        ph, pw = (h - k) // st + 1, (w - k) // st + 1
+        x = big(shape)
+        dx, out = G.to_device(x), G.buffer((n, c, ph, pw), f32)
+        report("pool max", f"{shape} k{k} s{st}", x.nbytes + out.nbytes,
+               timeit(lambda: G.pool(out, dx, k, k, st, st, stream=s)))
+        gr, up = G.to_device(big((n, c, ph, pw))), G.buffer(shape, f32)
+        report("unpool max", f"{shape} k{k} s{st}", 2 * x.nbytes + 2 * out.nbytes,
+               timeit(lambda: G.unpool(up, dx, out, gr, k, k, st, st, stream=s)))
+        del dx, out, gr, up
+    for shape, k, st, pad, dt in (((32, 256, 56, 56), 3, 1, 1, f32), ((32, 256, 56, 56), 3, 1, 1, np.uint16),
+                                  ((32, 64, 112, 112), 3, 1, 1, np.uint16), ((32, 256, 56, 56), 1, 1, 0, np.uint16),
+                                  ((32, 3, 224, 224), 7, 2, 3, f32), ((32, 128, 28, 28), 5, 1, 2, np.uint16),
+                                  ((32, 256, 56, 56), 3, 2, 1, np.uint16), ((32, 256, 56, 56), 3, 1, 0, np.uint16)):
+        n, c, h, w = shape
+        oh, ow = (h + 2 * pad - k) // st + 1, (w + 2 * pad - k) // st + 1
+        img = big(shape) if dt == f32 else big(shape).astype(np.float16).view(np.uint16)
+        dimg, dcol = G.to_device(img), G.buffer((c * k * k, n * oh * ow), dt)
+        tag = f"{shape} k{k} s{st} p{pad} {'f32' if dt == f32 else 'f16'}"
+        report("im2col", tag, img.nbytes + dcol.nbytes,
+               timeit(lambda: G.im2col(dcol, dimg, k, k, st, st, 1, 1, pad, pad, s)))
+        back = G.buffer(shape, dt)
+        report("col2im", tag, img.nbytes + dcol.nbytes,
+               timeit(lambda: G.col2im(back, dcol, k, k, st, st, 1, 1, pad, pad, s)))
+        del dimg, dcol, back
+    for shape in ((64, 256, 56, 56), (128, 64, 112, 112), (32, 512, 28, 28), (256, 1000, 1, 1), (64, 2048, 7, 7),
+                  (8, 256, 200, 200)):
+        x = big(shape)
+        dx, out = G.to_device(x), G.buffer((shape[1],), f32)
+        report("sumall_except_dim<1>", str(shape), x.nbytes, timeit(lambda: G.reduce_keep_highdim(out, dx, stream=s)))
+        del dx, out
+    for shape in ((16384, 4096), (256, 1000), (4096, 4096), (65536, 1024), (1024, 65536), (100000, 100), (128, 1 << 20)):
+        x = big(shape)
+        dx, out = G.to_device(x), G.buffer((shape[1],), f32)
+        report("sum_rows", str(shape), x.nbytes, timeit(lambda: G.reduce_keep_lowest(out, dx, stream=s)))
+        del dx, out
+    for shape in ((8192, 32000), (65536, 1000), (128, 1000), (4096, 4096), (2048, 50257), (16, 250000), (512, 128000)):
+        x = big(shape) * f32(3)
+        dx, out = G.to_device(x), G.buffer(shape, f32)
+        report("softmax", str(shape), 2 * x.nbytes, timeit(lambda: G.softmax(out, dx, s)))
+        lab, g = G.to_device(rng.integers(0, shape[1], shape[0]).astype(f32)), G.buffer(shape, f32)
+        report("softmax_grad", str(shape), 2 * x.nbytes, timeit(lambda: G.softmax_grad(g, out, lab, s)))
+        del dx, out, lab, g
+    print(json.dumps({"probe": "neighbour_shapes", "unit": "us per launch, 10 launches on the same buffers",
+                      "rows": rows_out}))
 
 
 def run_probe(G, which, pattern=""):

@@ -106,6 +106,43 @@ int Im2Col(T *col, int cstride, const T *img, int istride, const PatchGeom &g, v
     return Fail(MSHADOW_HIP_ERR_ARGUMENT, "im2col: pitch smaller than the row");
   }
   const int EPT = 16 / sizeof(T);
+  const bool unit_steps = g.sy == 1 && g.sx == 1 && g.dy == 1 && g.dx == 1;
+  /* the binary16 3-tap kernel without staging (below) serves this case better */
+  const bool three_taps_direct = unit_steps && g.kx == 3 && g.pad_x == 1 && g.ow == g.w &&
+                                 g.w % EPT == 0 && istride == g.w && cstride % EPT == 0 &&
+                                 Aligned16(col) && Aligned16(img) && cols < (1ll << 31);
+  if (three_taps_direct) {
+    const uint32_t places = static_cast<uint32_t>(cols / EPT);
+    const uint32_t per_block = kPatchBlock * kIm2ColDirectPer;
+    const uint32_t chunks = (places + per_block - 1) / per_block;
+    const long long pieces = (static_cast<long long>(g.c) * chunks + 7) / 8 * 8;
+    const long long direct_blocks = pieces * g.ky;
+    if (direct_blocks < (1ll << 31)) {
+      hipLaunchKernelGGL((Im2ColRow3DirectKernel<T, kIm2ColDirectPer>),
+                         dim3(static_cast<unsigned>(direct_blocks)), dim3(kPatchBlock), 0,
+                         AsStream(stream), col, cstride, img, g,
+                         mshadow::FastDivU32(static_cast<uint32_t>(g.ow / EPT)),
+                         mshadow::FastDivU32(static_cast<uint32_t>(g.oh)), chunks,
+                         mshadow::FastDivU32(chunks));
+      return AfterLaunch("im2col");
+    }
+  }
+  /* stride 1, dilation 1, patch rows of a pack or more: pack by pack, no staging */
+  if (unit_steps && g.ow >= EPT) {
+    const long long ppr = (g.ow + EPT - 1) / EPT;
+    const long long places = static_cast<long long>(g.n) * g.oh * ppr;
+    const uint32_t chunks = static_cast<uint32_t>((places + kPatchBlock - 1) / kPatchBlock);
+    const long long pieces = (static_cast<long long>(g.c) * chunks + 7) / 8 * 8;
+    const long long blocks = pieces * g.ky * g.kx;
+    if (places + kPatchBlock < (1ll << 31) && blocks < (1ll << 31)) {
+      hipLaunchKernelGGL((Im2ColDirectS1Kernel<T>), dim3(static_cast<unsigned>(blocks)),
+                         dim3(kPatchBlock), 0, AsStream(stream), col, cstride, img, istride, g,
+                         mshadow::FastDivU32(static_cast<uint32_t>(ppr)),
+                         mshadow::FastDivU32(static_cast<uint32_t>(g.oh)), chunks,
+                         mshadow::FastDivU32(chunks), static_cast<uint32_t>(places));
+      return AfterLaunch("im2col");
+    }
+  }
   /* tiled: padded input rows of a band of patch rows must fit the LDS budget */
   const size_t row_bytes = static_cast<size_t>(g.wp) * sizeof(T);
   const long long max_rows = static_cast<long long>(kIm2ColLdsBudget / row_bytes);
@@ -136,22 +173,6 @@ int Im2Col(T *col, int cstride, const T *img, int istride, const PatchGeom &g, v
          straight into the taps where the image is padded by one column, else staged */
       const bool dense = istride == g.w && g.w % 8 == 0 && reinterpret_cast<uintptr_t>(img) % 16 == 0;
       const mshadow::FastDivU32 div_w(static_cast<uint32_t>(g.w));
-      if (dense && g.pad_x == 1 && g.ow == g.w) {
-        const uint32_t places = static_cast<uint32_t>(cols / 8);
-        const uint32_t per_block = kPatchBlock * kIm2ColDirectPer;
-        const uint32_t chunks = (places + per_block - 1) / per_block;
-        const long long pieces = (static_cast<long long>(g.c) * chunks + 7) / 8 * 8;
-        const long long direct_blocks = pieces * g.ky;
-        if (direct_blocks < (1ll << 31)) {
-          hipLaunchKernelGGL(Im2ColHalfRow3DirectKernel<kIm2ColDirectPer>,
-                             dim3(static_cast<unsigned>(direct_blocks)), dim3(kPatchBlock), 0,
-                             AsStream(stream), reinterpret_cast<uint16_t *>(col), cstride,
-                             reinterpret_cast<const uint16_t *>(img), g, div_ppr,
-                             mshadow::FastDivU32(static_cast<uint32_t>(g.oh)), chunks,
-                             mshadow::FastDivU32(chunks));
-          return AfterLaunch("im2col");
-        }
-      }
       if (dense) {
         hipLaunchKernelGGL(Im2ColHalfRow3Kernel<true>, dim3(static_cast<unsigned>(blocks)),
                            dim3(kPatchBlock), lds, AsStream(stream), reinterpret_cast<uint16_t *>(col),
@@ -208,6 +229,19 @@ int Col2Im(T *img, int istride, const T *col, int cstride, const PatchGeom &g, v
                        reinterpret_cast<uint16_t *>(img), istride,
                        reinterpret_cast<const uint16_t *>(col), cstride, g, rg);
     return AfterLaunch("col2im");
+  }
+  /* stride 1, dilation 1, image rows of a pack or more: pack by pack, no staging */
+  if (g.sy == 1 && g.sx == 1 && g.dy == 1 && g.dx == 1 && g.w >= EPT) {
+    const long long wpk = (g.w + EPT - 1) / EPT;
+    const long long packs = static_cast<long long>(g.n) * g.c * g.h * wpk;
+    if (packs + kPatchBlock < (1ll << 31) && cols < (1ll << 31)) {
+      const unsigned blocks = static_cast<unsigned>((packs + kPatchBlock - 1) / kPatchBlock);
+      hipLaunchKernelGGL((Col2ImDirectS1Kernel<T>), dim3(blocks), dim3(kPatchBlock), 0, AsStream(stream),
+                         img, istride, col, cstride, g, mshadow::FastDivU32(static_cast<uint32_t>(wpk)),
+                         mshadow::FastDivU32(static_cast<uint32_t>(g.h)),
+                         mshadow::FastDivU32(static_cast<uint32_t>(g.c)), static_cast<uint32_t>(packs));
+      return AfterLaunch("col2im");
+    }
   }
   /* tiled: per tap, the patch rows a band of image rows touches; all taps must fit */
   const long long taps = static_cast<long long>(g.ky) * g.kx;
@@ -449,30 +483,20 @@ int mshadow_hip_softmax_f32(float *dst, int dstride, const float *src, int sstri
     LaunchShortSoftmax<false>(dst, dstride, src, sstride, rows, cols, s);
     return AfterLaunch("softmax");
   }
-  /* 128-bit path: aligned rows made of whole packs */
-  const bool vec = Aligned16(dst) && Aligned16(src) && dstride % 4 == 0 && sstride % 4 == 0 &&
-                   cols % 4 == 0;
+  /* 16-byte packs wherever the rows start and whatever their length (the accesses need no
+     alignment; a row's last, partial pack goes element by element) */
 #define SOFTMAX_LAUNCH(T, S, V) \
   hipLaunchKernelGGL((SoftmaxRowKernel<T, S, V, false>), dim3(rows), dim3(T), 0, s, dst, dstride, \
                      src, sstride, cols)
-  if (vec) {
-    if (cols <= 1024) SOFTMAX_LAUNCH(256, 1, 4);
-    else if (cols <= 2048) SOFTMAX_LAUNCH(256, 2, 4);
-    else if (cols <= 4096) SOFTMAX_LAUNCH(256, 4, 4);
-    else if (cols <= 8192) SOFTMAX_LAUNCH(256, 8, 4);
-    else if (cols <= 16384) SOFTMAX_LAUNCH(512, 8, 4);
-    else if (cols <= 32768) SOFTMAX_LAUNCH(512, 16, 4);
-    else if (cols <= 65536) SOFTMAX_LAUNCH(1024, 16, 4);
-    else hipLaunchKernelGGL((SoftmaxLongRowKernel<1024>), dim3(rows), dim3(1024), 0, s, dst,
-                            dstride, src, sstride, cols);
-  } else {
-    if (cols <= 1024) SOFTMAX_LAUNCH(256, 4, 1);
-    else if (cols <= 4096) SOFTMAX_LAUNCH(256, 16, 1);
-    else if (cols <= 16384) SOFTMAX_LAUNCH(1024, 16, 1);
-    else if (cols <= 32768) SOFTMAX_LAUNCH(1024, 32, 1);
-    else hipLaunchKernelGGL((SoftmaxLongRowKernel<1024>), dim3(rows), dim3(1024), 0, s, dst,
-                            dstride, src, sstride, cols);
-  }
+  if (cols <= 1024) SOFTMAX_LAUNCH(256, 1, 4);
+  else if (cols <= 2048) SOFTMAX_LAUNCH(256, 2, 4);
+  else if (cols <= 4096) SOFTMAX_LAUNCH(256, 4, 4);
+  else if (cols <= 8192) SOFTMAX_LAUNCH(256, 8, 4);
+  else if (cols <= 16384) SOFTMAX_LAUNCH(512, 8, 4);
+  else if (cols <= 32768) SOFTMAX_LAUNCH(512, 16, 4);
+  else if (cols <= 65536) SOFTMAX_LAUNCH(1024, 16, 4);
+  else hipLaunchKernelGGL((SoftmaxLongRowKernel<1024>), dim3(rows), dim3(1024), 0, s, dst,
+                          dstride, src, sstride, cols);
 #undef SOFTMAX_LAUNCH
   return AfterLaunch("softmax");
 }
@@ -524,14 +548,12 @@ int mshadow_hip_softmax_grad_ex_f32(float *dst, int dstride, const float *src, i
   const unsigned chunks = (cols + per_block - 1) / per_block;
   const unsigned long long blocks = static_cast<unsigned long long>(rows) * chunks;
   ABI_REQUIRE(blocks < (1ull << 31), "too many workgroups");
-  const bool vec = Aligned16(dst) && Aligned16(src) && dstride % 4 == 0 && sstride % 4 == 0;
   /* alpha / (classes - 1) with the count converted from unsigned, as the reference writes it */
   const GradParams gp = {static_cast<int>(ignore_label), alpha,
                          alpha / static_cast<float>(static_cast<unsigned>(cols - 1))};
   GradLaunch gl = {dst, dstride, src, sstride, label, cols, chunks, gp,
                    static_cast<unsigned>(blocks), AsStream(stream)};
-  if (vec) LaunchGrad<true>(flags, gl);
-  else LaunchGrad<false>(flags, gl);
+  LaunchGrad<true>(flags, gl);   // 16-byte packs wherever the rows start (no alignment needed)
   return AfterLaunch("softmax_grad");
 }
 
@@ -769,7 +791,9 @@ int mshadow_hip_reduce_keep_highdim_f32(float *dst, const float *src, int sstrid
                      static_cast<uint32_t>(n), static_cast<uint32_t>(c),                       \
                      static_cast<uint32_t>(v_y), static_cast<uint32_t>(v_x), v_div_x, scale,   \
                      split_partial, split_counter)
-        if (whole_packs) {
+        if (whole_packs && static_cast<long long>(n) * c > 16ll * mshadow_abi::ComputeUnits()) {
+          HIGHDIM_SPLIT(mshadow::hip::HighDimSplitRingPacksWide);
+        } else if (whole_packs) {
           HIGHDIM_SPLIT(mshadow::hip::HighDimSplitRingPacks);
         } else {
           HIGHDIM_SPLIT(mshadow::hip::HighDimSplitRing);
@@ -829,6 +853,40 @@ int mshadow_hip_pool_f32(float *dst, int dstride, const float *src, int sstride,
     case MSHADOW_HIP_SUM: hipLaunchKernelGGL((KERNEL<MSHADOW_HIP_SUM>), __VA_ARGS__); break;    \
     case MSHADOW_HIP_MAX: hipLaunchKernelGGL((KERNEL<MSHADOW_HIP_MAX>), __VA_ARGS__); break;    \
     default: hipLaunchKernelGGL((KERNEL<MSHADOW_HIP_MIN>), __VA_ARGS__); break;                 \
+  }
+  /* small planes: several whole planes per workgroup, about 24 KB of them */
+  const long long plane_bytes = static_cast<long long>(h) * row_bytes;
+  if (plane_bytes * 2 <= 24 * 1024 && planes >= 2) {
+    long long per_block = (24 * 1024) / plane_bytes;
+    /* ... but no fewer workgroups than keep every CU busy four times over */
+    while (per_block > 1 && (planes + per_block - 1) / per_block < 4ll * mshadow_abi::ComputeUnits()) {
+      per_block = (per_block + 1) / 2;
+    }
+    if (per_block >= 2) {
+      const size_t lds = static_cast<size_t>(per_block) * plane_bytes + 16;
+      const unsigned blocks = static_cast<unsigned>((planes + per_block - 1) / per_block);
+      const mshadow::FastDivU32 div_ph(static_cast<uint32_t>(ph));
+#define POOL_PLANES(KY, KX)                                                                     \
+  switch (reducer) {                                                                           \
+    case MSHADOW_HIP_SUM:                                                                      \
+      hipLaunchKernelGGL((PoolPlanesKernel<MSHADOW_HIP_SUM, KY, KX>), dim3(blocks), dim3(kPoolBlock), \
+                         lds, s, dst, dstride, src, sstride, g, planes, static_cast<int>(per_block), div_ph); \
+      break;                                                                                   \
+    case MSHADOW_HIP_MAX:                                                                      \
+      hipLaunchKernelGGL((PoolPlanesKernel<MSHADOW_HIP_MAX, KY, KX>), dim3(blocks), dim3(kPoolBlock), \
+                         lds, s, dst, dstride, src, sstride, g, planes, static_cast<int>(per_block), div_ph); \
+      break;                                                                                   \
+    default:                                                                                   \
+      hipLaunchKernelGGL((PoolPlanesKernel<MSHADOW_HIP_MIN, KY, KX>), dim3(blocks), dim3(kPoolBlock), \
+                         lds, s, dst, dstride, src, sstride, g, planes, static_cast<int>(per_block), div_ph); \
+      break;                                                                                   \
+  }
+      if (ky == 3 && kx == 3) { POOL_PLANES(3, 3) }
+      else if (ky == 2 && kx == 2) { POOL_PLANES(2, 2) }
+      else { POOL_PLANES(0, 0) }
+#undef POOL_PLANES
+      return AfterLaunch("pool");
+    }
   }
   if (band >= 1) {
     g.band = static_cast<int>(band);
@@ -903,6 +961,47 @@ int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstrid
     else UNPOOL_ROWS(MSHADOW_HIP_MIN);
 #undef UNPOOL_ROWS
     return AfterLaunch("unpool");
+  }
+  /* small planes: several whole planes per workgroup (about 24 KB of pooled values and gradients) */
+  {
+    const long long plane_bytes = static_cast<long long>(ph) * g.lds_pitch * sizeof(float) * 2;
+    const long long src_plane_bytes = static_cast<long long>(h) * w * sizeof(float);
+    if (plane_bytes > 0 && plane_bytes * 2 <= 24 * 1024 && src_plane_bytes <= 4 * 1024 && planes >= 2) {
+      long long per_block = (24 * 1024) / plane_bytes;
+      while (per_block > 1 &&
+             (planes + per_block - 1) / per_block < 4ll * mshadow_abi::ComputeUnits()) {
+        per_block = (per_block + 1) / 2;
+      }
+      if (per_block >= 2) {
+        const size_t lds = static_cast<size_t>(per_block) * plane_bytes + 32;
+        const unsigned blocks = static_cast<unsigned>((planes + per_block - 1) / per_block);
+        const mshadow::FastDivU32 div_h(static_cast<uint32_t>(h));
+#define UNPOOL_PLANES(KY, KX, SY, SX)                                                          \
+  switch (reducer) {                                                                           \
+    case MSHADOW_HIP_SUM:                                                                      \
+      hipLaunchKernelGGL((UnpoolPlanesKernel<MSHADOW_HIP_SUM, KY, KX, SY, SX>), dim3(blocks),   \
+                         dim3(kPoolBlock), lds, s, dst, dstride, src, sstride, pooled, pstride, \
+                         grad, gstride, g, planes, static_cast<int>(per_block), div_h);        \
+      break;                                                                                   \
+    case MSHADOW_HIP_MAX:                                                                      \
+      hipLaunchKernelGGL((UnpoolPlanesKernel<MSHADOW_HIP_MAX, KY, KX, SY, SX>), dim3(blocks),   \
+                         dim3(kPoolBlock), lds, s, dst, dstride, src, sstride, pooled, pstride, \
+                         grad, gstride, g, planes, static_cast<int>(per_block), div_h);        \
+      break;                                                                                   \
+    default:                                                                                   \
+      hipLaunchKernelGGL((UnpoolPlanesKernel<MSHADOW_HIP_MIN, KY, KX, SY, SX>), dim3(blocks),   \
+                         dim3(kPoolBlock), lds, s, dst, dstride, src, sstride, pooled, pstride, \
+                         grad, gstride, g, planes, static_cast<int>(per_block), div_h);        \
+      break;                                                                                   \
+  }
+        if (ky == 3 && kx == 3 && sy == 2 && sx == 2) { UNPOOL_PLANES(3, 3, 2, 2) }
+        else if (ky == 2 && kx == 2 && sy == 2 && sx == 2) { UNPOOL_PLANES(2, 2, 2, 2) }
+        else if (ky == 3 && kx == 3 && sy == 1 && sx == 1) { UNPOOL_PLANES(3, 3, 1, 1) }
+        else { UNPOOL_PLANES(0, 0, 0, 0) }
+#undef UNPOOL_PLANES
+        return AfterLaunch("unpool");
+      }
+    }
   }
   const size_t row_bytes = static_cast<size_t>(g.lds_pitch) * sizeof(float) * 2;  // pooled + grad
   /* source rows per band: prow_max = (band + ky - 2) / sy + 2 pooled rows must fit */

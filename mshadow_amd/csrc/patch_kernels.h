@@ -257,10 +257,10 @@ __global__ void __launch_bounds__(kPatchBlock)
   }
 }
 
-/*! \brief The same copy with no staging at all, for dense images padded by one column on each
- *  side (ow == w): a thread makes the three packs (b = 0, 1, 2) of one place (a, oy, ox..ox+7)
- *  of one channel from the aligned pack of image row oy + a - pad_y at ox and the element on
- *  either side of it, and stores them. A workgroup is 256 consecutive places of one (channel,
+/*! \brief The same copy with no staging at all, for dense images (binary16 or float) padded by one
+ *  column on each side (ow == w): a thread makes the three packs (b = 0, 1, 2) of one place
+ *  (a, oy, a pack of columns) of one channel from the aligned pack of image row oy + a - pad_y
+ *  and the element on either side of it, and stores them. A workgroup is 256 consecutive places of one (channel,
  *  a) pair - the three rows of the column matrix are contiguous over images and patch rows -
  *  and ends after its three stores per thread, so the machine sees many small independent
  *  pieces, the form in which plain copies and fills run fastest here. The image is read
@@ -269,12 +269,12 @@ __global__ void __launch_bounds__(kPatchBlock)
  *  and 86 us for the staged kernel above; two or four places per thread (PER) are slower
  *  (111 / 115 us), as is one thread storing all nine packs that one image pack feeds (125 us). */
 const int kIm2ColDirectPer = 1;
-template <int PER>
+template <typename T, int PER>
 __global__ void __launch_bounds__(kPatchBlock)
-    Im2ColHalfRow3DirectKernel(uint16_t *col, int cstride, const uint16_t *img, PatchGeom g,
-                               mshadow::FastDivU32 div_ppr, mshadow::FastDivU32 div_oh,
-                               uint32_t chunks, mshadow::FastDivU32 div_chunks) {
-  typedef uint16_t T;
+    Im2ColRow3DirectKernel(T *col, int cstride, const T *img, PatchGeom g,
+                           mshadow::FastDivU32 div_ppr, mshadow::FastDivU32 div_oh,
+                           uint32_t chunks, mshadow::FastDivU32 div_chunks) {
+  const int EPT = 16 / sizeof(T);
   /* Workgroups are dealt to the XCDs in turn, eight at a time. The ky workgroups that read
      the same piece of the image (one per tap row a) get numbers 8 apart: they run on one XCD
      at about the same time, and its L2 fetches that piece once.
@@ -288,7 +288,7 @@ __global__ void __launch_bounds__(kPatchBlock)
   if (ch >= static_cast<uint32_t>(g.c)) return;
   const uint32_t chunk = piece - ch * chunks;
   const uint32_t row3 = ch * g.ky + a;
-  const uint32_t ppr = static_cast<uint32_t>(g.ow) / 8;
+  const uint32_t ppr = static_cast<uint32_t>(g.ow) / EPT;
   const uint32_t places = static_cast<uint32_t>(g.n) * g.oh * ppr;
   U4 w03[PER], mid[PER], hi[PER];
 #pragma unroll
@@ -297,35 +297,240 @@ __global__ void __launch_bounds__(kPatchBlock)
     w03[u] = mid[u] = hi[u] = U4{0u, 0u, 0u, 0u};
     if (pk >= places) continue;
     const uint32_t line = div_ppr.Div(pk);             // n * oh + oy
-    const int ox = static_cast<int>(pk - line * ppr) * 8;
+    const int ox = static_cast<int>(pk - line * ppr) * EPT;
     const uint32_t n = div_oh.Div(line);
     const int oy = static_cast<int>(line - n * g.oh);
     const int y = oy + a - g.pad_y;
     if (y >= 0 && y < g.h) {
       const T *in = img + (static_cast<size_t>(n * g.c + ch) * g.h + y) * g.w + ox;
       const U4 m = *reinterpret_cast<const U4 *>(in);
-      const uint32_t before = ox > 0 ? in[-1] : 0u;
-      const uint32_t after = ox + 8 < g.w ? in[8] : 0u;
+      uint32_t before = 0u, after = 0u;                // the element on either side, zero-extended
+      if (ox > 0) __builtin_memcpy(&before, in - 1, sizeof(T));
+      if (ox + EPT < g.w) __builtin_memcpy(&after, in + EPT, sizeof(T));
       mid[u] = m;
-      w03[u].x = (m.x << 16) | before;
-      w03[u].y = __builtin_amdgcn_alignbit(m.y, m.x, 16);
-      w03[u].z = __builtin_amdgcn_alignbit(m.z, m.y, 16);
-      w03[u].w = __builtin_amdgcn_alignbit(m.w, m.z, 16);
-      hi[u].x = w03[u].y;
-      hi[u].y = w03[u].z;
-      hi[u].z = w03[u].w;
-      hi[u].w = (after << 16) | (m.w >> 16);
+      if (sizeof(T) == 2) {
+        w03[u].x = (m.x << 16) | before;
+        w03[u].y = __builtin_amdgcn_alignbit(m.y, m.x, 16);
+        w03[u].z = __builtin_amdgcn_alignbit(m.z, m.y, 16);
+        w03[u].w = __builtin_amdgcn_alignbit(m.w, m.z, 16);
+        hi[u].x = w03[u].y;
+        hi[u].y = w03[u].z;
+        hi[u].z = w03[u].w;
+        hi[u].w = (after << 16) | (m.w >> 16);
+      } else {
+        w03[u] = U4{before, m.x, m.y, m.z};
+        hi[u] = U4{m.y, m.z, m.w, after};
+      }
     }
   }
 #pragma unroll
   for (int u = 0; u < PER; ++u) {
     const uint32_t pk = (chunk * PER + u) * kPatchBlock + threadIdx.x;
     if (pk >= places) continue;
-    T *out = col + static_cast<size_t>(row3 * 3) * cstride + static_cast<size_t>(pk) * 8;
+    T *out = col + static_cast<size_t>(row3 * 3) * cstride + static_cast<size_t>(pk) * EPT;
     StreamStore16(out, w03[u]);
     StreamStore16(out + cstride, mid[u]);
     StreamStore16(out + 2 * static_cast<size_t>(cstride), hi[u]);
   }
+}
+
+/* ------------------------------------------------------- stride 1, dilation 1, any window
+ * With stride and dilation 1 the row (channel, a, b) of the column matrix is, image by image,
+ * the image itself shifted by (a - pad_y, b - pad_x) and cut to the patch grid: a run of a
+ * patch row is a run of an image row. So both directions can work pack by pack with no
+ * staging: one side of a pack is aligned (the side that is stored), the other is fetched
+ * wherever it lies - 16-byte global loads need no alignment on this machine. Very many small
+ * workgroups that end after a handful of accesses each. */
+
+/*! \brief 16 bytes from an address aligned only to the element */
+template <typename T>
+__device__ __forceinline__ U4 LoadPackAnywhere(const T *p) {
+  typedef U4 Loose __attribute__((aligned(2)));   // the narrowest element type here
+  return *reinterpret_cast<const Loose *>(p);
+}
+
+/*! \brief element e of a pack of EPT elements of type T, and its replacement */
+template <typename T>
+__device__ __forceinline__ T PackElement(const U4 &q, int e) {
+  const int per = 4 / sizeof(T);   // elements per dword
+  const uint32_t w = q[e / per];
+  T v;
+  if (sizeof(T) == 4) {
+    __builtin_memcpy(&v, &w, sizeof(T));
+  } else {
+    const uint16_t h = static_cast<uint16_t>(w >> (16 * (e % per)));
+    __builtin_memcpy(&v, &h, sizeof(T));
+  }
+  return v;
+}
+template <typename T>
+__device__ __forceinline__ void SetPackElement(U4 *q, int e, T v) {
+  const int per = 4 / sizeof(T);
+  if (sizeof(T) == 4) {
+    uint32_t w;
+    __builtin_memcpy(&w, &v, 4);
+    (*q)[e / per] = w;
+  } else {
+    uint16_t h;
+    __builtin_memcpy(&h, &v, 2);
+    const int sh = 16 * (e % per);
+    (*q)[e / per] = ((*q)[e / per] & ~(0xffffu << sh)) | (static_cast<uint32_t>(h) << sh);
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ void StorePackAnywhere(T *p, const U4 &q) {
+  typedef U4 Loose __attribute__((aligned(2)));
+  __builtin_nontemporal_store(q, reinterpret_cast<Loose *>(p));
+}
+
+/*! \brief the pack with every element outside [lo, hi) cleared */
+template <typename T>
+__device__ __forceinline__ U4 KeepElements(U4 q, int lo, int hi) {
+  const int per = 4 / sizeof(T);
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    uint32_t m = 0u;
+#pragma unroll
+    for (int k = 0; k < per; ++k) {
+      const int e = d * per + k;
+      if (e >= lo && e < hi) m |= (sizeof(T) == 4 ? 0xffffffffu : 0xffffu << (16 * k));
+    }
+    q[d] &= m;
+  }
+  return q;
+}
+
+/*! \brief EPT consecutive elements from p, of which only [lo, hi) are wanted (the others come
+ *  back as zero): one 16-byte load where all 16 bytes lie inside [first, last), else element
+ *  by element */
+template <typename T>
+__device__ __forceinline__ U4 LoadPackInside(const T *p, int lo, int hi, const T *first, const T *last) {
+  const int EPT = 16 / sizeof(T);
+  if (p >= first && p + EPT <= last) return KeepElements<T>(LoadPackAnywhere(p), lo, hi);
+  U4 q = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    if (e >= lo && e < hi) SetPackElement(&q, e, p[e]);
+  }
+  return q;
+}
+
+/*! \brief im2col, stride 1, dilation 1, patch rows of at least one pack: a thread makes one pack
+ *  of one patch row of one row of the column matrix. The last pack of a patch row that is not
+ *  whole packs is moved back to end with the row (it overlaps its neighbour, both write the
+ *  same values), so no pack ever straddles two rows. grid: the taps of one piece of a channel 8
+ *  workgroups apart, as in Im2ColRow3DirectKernel. */
+template <typename T>
+__global__ void __launch_bounds__(kPatchBlock)
+    Im2ColDirectS1Kernel(T *col, int cstride, const T *img, int istride, PatchGeom g,
+                         mshadow::FastDivU32 div_ppr, mshadow::FastDivU32 div_oh, uint32_t chunks,
+                         mshadow::FastDivU32 div_chunks, uint32_t places) {
+  const int EPT = 16 / sizeof(T);
+  const uint32_t taps = static_cast<uint32_t>(g.ky * g.kx);
+  const uint32_t lane8 = blockIdx.x & 7u;
+  const uint32_t turn = blockIdx.x >> 3;
+  const uint32_t group = turn / taps;
+  const uint32_t tap = turn - group * taps;
+  const uint32_t piece = group * 8 + lane8;
+  const uint32_t ch = div_chunks.Div(piece);
+  if (ch >= static_cast<uint32_t>(g.c)) return;
+  const uint32_t chunk = piece - ch * chunks;
+  const int a = static_cast<int>(tap) / g.kx;
+  const int b = static_cast<int>(tap) - a * g.kx;
+  const uint32_t pk = chunk * kPatchBlock + threadIdx.x;   // place: (n * oh + oy) * ppr + p
+  if (pk >= places) return;
+  const uint32_t line = div_ppr.Div(pk);
+  const int ox = min(static_cast<int>(pk - line * div_ppr.div) * EPT, g.ow - EPT);
+  const uint32_t n = div_oh.Div(line);
+  const int oy = static_cast<int>(line - n * g.oh);
+  const int y = oy + a - g.pad_y;
+  const int xs = ox + b - g.pad_x;
+  U4 q = {0u, 0u, 0u, 0u};
+  if (y >= 0 && y < g.h) {
+    const T *row = img + (static_cast<size_t>(n * g.c + ch) * g.h + y) * istride;
+    const T *last = img + (static_cast<size_t>(g.n) * g.c * g.h - 1) * istride + g.w;
+    q = LoadPackInside<T>(row + xs, max(0, -xs), min(EPT, g.w - xs), img, last);
+  }
+  StorePackAnywhere(col + static_cast<size_t>(ch * taps + tap) * cstride +
+                        static_cast<size_t>(line) * g.ow + ox, q);
+}
+
+/*! \brief one pack plus another, element by element, rounded after every add as the element
+ *  type's own += does (binary16: a packed half add is exactly that); elements whose bit in
+ *  `keep` is clear stay as they are */
+template <typename T>
+__device__ __forceinline__ void AddPackWhere(U4 *acc, const U4 &term, uint32_t keep) {
+  const int EPT = 16 / sizeof(T);
+  if (sizeof(T) == 4) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float x, y;
+      const uint32_t xa = (*acc)[e], ya = term[e];
+      __builtin_memcpy(&x, &xa, 4);
+      __builtin_memcpy(&y, &ya, 4);
+      const float r = x + y;
+      uint32_t w;
+      __builtin_memcpy(&w, &r, 4);
+      if (keep & (1u << e)) (*acc)[e] = w;
+    }
+  } else {
+    typedef _Float16 H2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      H2 x, y;
+      const uint32_t xa = (*acc)[d], ya = term[d];
+      __builtin_memcpy(&x, &xa, 4);
+      __builtin_memcpy(&y, &ya, 4);
+      const H2 r = x + y;
+      uint32_t w;
+      __builtin_memcpy(&w, &r, 4);
+      const uint32_t m = ((keep >> (2 * d)) & 1u ? 0x0000ffffu : 0u) |
+                         ((keep >> (2 * d + 1)) & 1u ? 0xffff0000u : 0u);
+      (*acc)[d] = (w & m) | ((*acc)[d] & ~m);
+    }
+  }
+  (void)EPT;
+}
+
+/*! \brief col2im, stride 1, dilation 1, image rows of at least one pack: a thread sums one pack of
+ *  an image row (the last pack of a row that is not whole packs moved back to end with the
+ *  row, as above) from the ky * kx rows of the column matrix that cover it, terms in the
+ *  reference's order (py ascending, then px ascending:
+ *  mshadow/extension/pack_col2patch.h:118-144). */
+template <typename T>
+__global__ void __launch_bounds__(kPatchBlock)
+    Col2ImDirectS1Kernel(T *img, int istride, const T *col, int cstride, PatchGeom g,
+                         mshadow::FastDivU32 div_wpk, mshadow::FastDivU32 div_h,
+                         mshadow::FastDivU32 div_c, uint32_t total_packs) {
+  const int EPT = 16 / sizeof(T);
+  const uint32_t pk = blockIdx.x * kPatchBlock + threadIdx.x;
+  if (pk >= total_packs) return;
+  const uint32_t rowi = div_wpk.Div(pk);             // (n * c + ch) * h + y
+  const int x0 = min(static_cast<int>(pk - rowi * div_wpk.div) * EPT, g.w - EPT);
+  const uint32_t plane = div_h.Div(rowi);
+  const int y = static_cast<int>(rowi - plane * g.h);
+  const uint32_t n = div_c.Div(plane);
+  const uint32_t ch = plane - n * g.c;
+  const uint32_t taps = static_cast<uint32_t>(g.ky * g.kx);
+  const size_t cols = static_cast<size_t>(g.n) * g.oh * g.ow;
+  const T *last = col + (static_cast<size_t>(g.c) * taps - 1) * cstride + cols;
+  const T *base = col + static_cast<size_t>(ch) * taps * cstride + static_cast<size_t>(n) * g.oh * g.ow;
+  U4 acc = {0u, 0u, 0u, 0u};
+  for (int a = g.ky - 1; a >= 0; --a) {
+    const int py = y + g.pad_y - a;
+    if (py < 0 || py >= g.oh) continue;
+    for (int b = g.kx - 1; b >= 0; --b) {
+      const int px0 = x0 + g.pad_x - b;              // patch column of the pack's first pixel
+      const int lo = max(0, -px0), hi = min(EPT, g.ow - px0);   // elements [lo, hi) have a patch
+      if (lo >= hi) continue;
+      const T *at = base + static_cast<size_t>(a * g.kx + b) * cstride + static_cast<size_t>(py) * g.ow;
+      const U4 term = LoadPackInside<T>(at + px0, lo, hi, col, last);
+      const uint32_t keep = ((1u << hi) - 1u) & ~((1u << lo) - 1u);
+      AddPackWhere<T>(&acc, term, keep);
+    }
+  }
+  StorePackAnywhere(img + static_cast<size_t>(rowi) * istride + x0, acc);
 }
 
 /*! \brief FAST: stride 1 and dilation 1 in both directions (the common convolution case):

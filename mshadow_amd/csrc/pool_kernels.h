@@ -154,6 +154,61 @@ __global__ void __launch_bounds__(kPoolBlock)
   }
 }
 
+/*! \brief The same for small planes: a workgroup takes `per_block` whole consecutive planes (they
+ *  are consecutive rows of the tensor's 2-D view, so their rows stage as one band) and computes
+ *  all their windows; with one small plane per workgroup the launch of the workgroups is what
+ *  takes the time ((256,256,13,13), 3x3 stride 2: 91 us for 54 MB). grid.x = ceil(planes /
+ *  per_block); dynamic LDS: per_block * h * lds_pitch + 4 floats. */
+template <int REDUCER, int KY, int KX>
+__global__ void __launch_bounds__(kPoolBlock)
+    PoolPlanesKernel(float *dst, int dstride, const float *src, int sstride, PoolGeom g, int planes,
+                     int per_block, mshadow::FastDivU32 div_ph) {
+  extern __shared__ float smem[];
+  typedef PoolOp<REDUCER> Op;
+  const int ky = KY > 0 ? KY : g.ky;
+  const int kx = KX > 0 ? KX : g.kx;
+  const int plane0 = blockIdx.x * per_block;
+  const int np = min(per_block, planes - plane0);
+  const float *in = src + static_cast<size_t>(plane0) * g.h * sstride;
+  float *tile = smem + LdsPhase(in);
+  StageRows(tile, g.lds_pitch, in, sstride, np * g.h, g.w);
+  __syncthreads();
+  float *out = dst + static_cast<size_t>(plane0) * g.ph * dstride;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  /* a wave takes `rpw` output rows at a time, pw lanes each (64 / pw of them, at least one) */
+  const int rpw = g.pw >= 64 ? 1 : 64 / g.pw;
+  const int sub = rpw == 1 ? 0 : lane / g.pw;
+  const int px0 = rpw == 1 ? lane : lane - sub * g.pw;
+  const int rows_out = np * g.ph;
+  for (int r0 = wave * rpw; r0 < rows_out; r0 += kPoolWaves * rpw) {
+    const int r = r0 + sub;
+    if (sub >= rpw || r >= rows_out) continue;
+    const int p = static_cast<int>(div_ph.Div(static_cast<uint32_t>(r)));
+    const int py = r - p * g.ph;
+    const int ys = p * g.h + py * g.sy;
+    const int ye = min(ys + ky, (p + 1) * g.h);
+    for (int px = px0; px < g.pw; px += (rpw == 1 ? 64 : g.pw)) {
+      const int xs = px * g.sx;
+      const int xe = min(xs + kx, g.w);
+      float res = Op::Init();
+      if (KY > 0 && KX > 0 && ye - ys == KY && xe - xs == KX) {
+#pragma unroll
+        for (int y = 0; y < (KY > 0 ? KY : 1); ++y) {
+#pragma unroll
+          for (int x = 0; x < (KX > 0 ? KX : 1); ++x) {
+            res = Op::Reduce(res, tile[(ys + y) * g.lds_pitch + xs + x]);
+          }
+        }
+      } else {
+        for (int y = ys; y < ye; ++y) {
+          for (int x = xs; x < xe; ++x) res = Op::Reduce(res, tile[y * g.lds_pitch + x]);
+        }
+      }
+      StreamStore(out + static_cast<size_t>(r) * dstride + px, res);
+    }
+  }
+}
+
 /*! \brief no staging: used when even one band of rows does not fit in LDS */
 template <int REDUCER>
 __global__ void __launch_bounds__(kPoolBlock)
@@ -259,6 +314,79 @@ __global__ void __launch_bounds__(kPoolBlock)
           StreamStore(out + static_cast<size_t>(yr) * dstride + x, val);
         }
       }
+    }
+  }
+}
+
+/*! \brief unpool for small planes: a workgroup takes `per_block` whole consecutive planes, stages
+ *  their pooled values and gradients (per_block * ph rows each) and computes every source pixel
+ *  of those planes; a wave takes 64 / w source rows at a time when rows are short. Terms in
+ *  the reference's order (py, then px ascending; mshadow/extension/spatial_unpool.h:102-125), a
+ *  multiply and an add each. grid.x = ceil(planes / per_block); dynamic LDS: two arrays of
+ *  per_block * ph * lds_pitch + 4 floats. */
+template <int REDUCER, int KY, int KX, int SY, int SX>
+__global__ void __launch_bounds__(kPoolBlock)
+    UnpoolPlanesKernel(float *dst, int dstride, const float *src, int sstride, const float *pooled,
+                       int pstride, const float *grad, int gstride, PoolGeom g, int planes,
+                       int per_block, mshadow::FastDivU32 div_h) {
+  extern __shared__ float smem[];
+  typedef PoolOp<REDUCER> Op;
+  const bool kFixed = KY > 0 && KX > 0 && SY > 0 && SX > 0;
+  if (kFixed) {   // window and stride known to the compiler: the range divisions become shifts
+    g.ky = KY; g.kx = KX; g.sy = SY; g.sx = SX;
+  }
+  const int kCandY = kFixed ? (KY + SY - 1) / (SY > 0 ? SY : 1) : 1;
+  const int kCandX = kFixed ? (KX + SX - 1) / (SX > 0 ? SX : 1) : 1;
+  const int plane0 = blockIdx.x * per_block;
+  const int np = min(per_block, planes - plane0);
+  const float *pin = pooled + static_cast<size_t>(plane0) * g.ph * pstride;
+  const float *gin = grad + static_cast<size_t>(plane0) * g.ph * gstride;
+  float *sp = smem + LdsPhase(pin);
+  float *sg = smem + per_block * g.ph * g.lds_pitch + 4 + LdsPhase(gin);
+  StageRows(sp, g.lds_pitch, pin, pstride, np * g.ph, g.pw);
+  StageRows(sg, g.lds_pitch, gin, gstride, np * g.ph, g.pw);
+  __syncthreads();
+  const float *in = src + static_cast<size_t>(plane0) * g.h * sstride;
+  float *out = dst + static_cast<size_t>(plane0) * g.h * dstride;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int rpw = g.w >= 64 ? 1 : 64 / g.w;
+  const int sub = rpw == 1 ? 0 : lane / g.w;
+  const int x0 = rpw == 1 ? lane : lane - sub * g.w;
+  const int rows = np * g.h;
+  for (int r0 = wave * rpw; r0 < rows; r0 += kPoolWaves * rpw) {
+    const int r = r0 + sub;
+    if (sub >= rpw || r >= rows) continue;
+    const int p = static_cast<int>(div_h.Div(static_cast<uint32_t>(r)));
+    const int y = r - p * g.h;
+    const int py_min = y < g.ky ? 0 : (y - g.ky + g.sy) / g.sy;
+    const int py_max = min((y + g.sy) / g.sy, g.ph);
+    for (int x = x0; x < g.w; x += (rpw == 1 ? 64 : g.w)) {
+      const float vs = StreamLoad(in + static_cast<size_t>(r) * sstride + x);
+      const int px_min = x < g.kx ? 0 : (x - g.kx + g.sx) / g.sx;
+      const int px_max = min((x + g.sx) / g.sx, g.pw);
+      float val = 0.0f;
+      if (kFixed) {
+#pragma unroll
+        for (int iy = 0; iy < kCandY; ++iy) {
+          const int py = py_min + iy;
+#pragma unroll
+          for (int ix = 0; ix < kCandX; ++ix) {
+            const int px = px_min + ix;
+            const bool live = py < py_max && px < px_max;
+            const int li = live ? (p * g.ph + py) * g.lds_pitch + px : 0;
+            const float t = val + Op::Grad(vs, sp[li]) * sg[li];
+            val = live ? t : val;
+          }
+        }
+      } else {
+        for (int py = py_min; py < py_max; ++py) {
+          for (int px = px_min; px < px_max; ++px) {
+            const int li = (p * g.ph + py) * g.lds_pitch + px;
+            val = val + Op::Grad(vs, sp[li]) * sg[li];
+          }
+        }
+      }
+      StreamStore(out + static_cast<size_t>(r) * dstride + x, val);
     }
   }
 }

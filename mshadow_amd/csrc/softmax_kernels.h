@@ -724,8 +724,8 @@ __device__ inline float BlockMax(float v, float *wmax) {
   return m;
 }
 
-/*! \brief THREADS * SLABS * VEC >= cols. VEC == 4 needs 16-byte aligned rows and
- *  cols % 4 == 0. Slab j of wave w holds the 64 * VEC columns from (j * W + w) * 64 * VEC,
+/*! \brief THREADS * SLABS * VEC >= cols. VEC == 4 moves 16-byte packs wherever the rows
+ *  start and whatever their length (the last, partial pack of a row element by element). Slab j of wave w holds the 64 * VEC columns from (j * W + w) * 64 * VEC,
  *  lane l of that VEC consecutive ones: each load is one contiguous kilobyte per wave, the
  *  W waves together stream one contiguous stretch per slab, and the order of the row is
  *  slab, wave, lane, element.
@@ -755,7 +755,7 @@ __global__ void __launch_bounds__(THREADS, MIN_WAVES)  // 4 waves per SIMD: two 
     const float *at = in + c0;  // uniform
     if (c0 + kChunk <= cols) {
       if (VEC == 4) {
-        const F4 q = StreamLoadF4(at + lane_col);
+        const F4 q = StreamLoadF4Anywhere(at + lane_col);
         v[j][0] = q.x; v[j][1 % VEC] = q.y; v[j][2 % VEC] = q.z; v[j][3 % VEC] = q.w;
       } else {
 #pragma unroll
@@ -764,10 +764,15 @@ __global__ void __launch_bounds__(THREADS, MIN_WAVES)  // 4 waves per SIMD: two 
     } else {
 #pragma unroll
       for (int i = 0; i < VEC; ++i) v[j][i] = kAbsent;
-      if (VEC == 4) {  // cols % 4 == 0: a pack is either whole or absent
-        if (c0 + static_cast<int>(lane_col) < cols) {
-          const F4 q = StreamLoadF4(at + lane_col);
+      if (VEC == 4) {  // whole packs as packs, the one the row ends in element by element
+        if (c0 + static_cast<int>(lane_col) + VEC <= cols) {
+          const F4 q = StreamLoadF4Anywhere(at + lane_col);
           v[j][0] = q.x; v[j][1 % VEC] = q.y; v[j][2 % VEC] = q.z; v[j][3 % VEC] = q.w;
+        } else {
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) {
+            if (c0 + static_cast<int>(lane_col) + i < cols) v[j][i] = at[lane_col + i];
+          }
         }
       } else {
 #pragma unroll
@@ -834,10 +839,13 @@ __global__ void __launch_bounds__(THREADS, MIN_WAVES)  // 4 waves per SIMD: two 
     if (VEC == 4) {
       F4 q;
       q.x = o[0]; q.y = o[1 % VEC]; q.z = o[2 % VEC]; q.w = o[3 % VEC];
-      if (c0 + kChunk <= cols) {
-        StreamStoreF4(at + lane_col, q);
-      } else if (c0 + static_cast<int>(lane_col) < cols) {
-        StreamStoreF4(at + lane_col, q);
+      if (c0 + kChunk <= cols || c0 + static_cast<int>(lane_col) + VEC <= cols) {
+        StreamStoreF4Anywhere(at + lane_col, q);
+      } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          if (c0 + static_cast<int>(lane_col) + i < cols) at[lane_col + i] = o[i];
+        }
       }
     } else {
 #pragma unroll
@@ -1005,7 +1013,7 @@ __global__ void __launch_bounds__(kGradBlock)
 #pragma unroll
     for (int u = 0; u < kGradPacks; ++u) {
       const int x = chunk0 + (u * kGradBlock + threadIdx.x) * 4;
-      if (x + 4 <= cols) q[u] = StreamLoadF4(in + x);
+      if (x + 4 <= cols) q[u] = StreamLoadF4Anywhere(in + x);
     }
 #pragma unroll
     for (int u = 0; u < kGradPacks; ++u) {
@@ -1022,7 +1030,7 @@ __global__ void __launch_bounds__(kGradBlock)
           q[u].z = GradElement<FLAGS>(q[u].z, k == x + 2, ignored, gp);
           q[u].w = GradElement<FLAGS>(q[u].w, k == x + 3, ignored, gp);
         }
-        StreamStoreF4(out + x, q[u]);
+        StreamStoreF4Anywhere(out + x, q[u]);
       } else {
         for (int i = x; i < cols; ++i) out[i] = GradElement<FLAGS>(in[i], i == k, ignored, gp);
       }

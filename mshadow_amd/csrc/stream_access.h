@@ -22,6 +22,15 @@ __device__ __forceinline__ F4 StreamLoadF4(const float *p) {
 __device__ __forceinline__ void StreamStoreF4(float *p, F4 v) {
   __builtin_nontemporal_store(v, reinterpret_cast<F4 *>(p));
 }
+/*! \brief the same at any float boundary: 16-byte global accesses need no 16-byte alignment
+ *  on this machine (they cost a little more where they straddle a cache line) */
+typedef F4 F4Loose __attribute__((aligned(4)));
+__device__ __forceinline__ F4 StreamLoadF4Anywhere(const float *p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const F4Loose *>(p));
+}
+__device__ __forceinline__ void StreamStoreF4Anywhere(float *p, F4 v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<F4Loose *>(p));
+}
 __device__ __forceinline__ float StreamLoad(const float *p) { return __builtin_nontemporal_load(p); }
 /*! \brief N consecutive floats (N = 2 or 4) as one access; p aligned to N * 4 bytes */
 template <int N>

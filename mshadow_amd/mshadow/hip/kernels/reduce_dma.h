@@ -264,6 +264,10 @@ struct SplitRing {
  *  with one workgroup per kept index): rows of whole 16-byte packs - 16 segments per
  *  workgroup, a kilobyte of each per stage; any rows - 32 segments, 256 bytes of each. */
 typedef SplitRing<16, 8, 4, 16> HighDimSplitRingPacks;
+/*! \brief ... and with more segments than 16 per CU: 32 per workgroup, one workgroup per CU
+ *  (two workgroups of 16 on a CU ask for more than the CU's loads deliver: (128,64,112,112)
+ *  took 105 us) */
+typedef SplitRing<32, 8, 4, 16> HighDimSplitRingPacksWide;
 typedef SplitRing<32, 8, 8, 4> HighDimSplitRing;
 
 template <int BYTES>
@@ -311,8 +315,12 @@ __global__ void __launch_bounds__(Ring::kThreads)
   const uint32_t nstage = (seg_len + TL - 1) / TL;
   const uint32_t nstep = nstage == 0 ? 0 : nstage + kAhead;
 
-  if (wave != 0) {
-    const uint32_t lw = wave - 1;
+  /* Which wave runs the chains: two workgroups share a CU where the ring is half the LDS, and
+     two chain waves on one SIMD take turns (measured: 11.4 ns per add against 5.6 ns). The
+     workgroups that meet on a CU differ in the lowest bit of their number or in bit 8. */
+  const uint32_t chain_wave = (blockIdx.x ^ (blockIdx.x >> 8)) & 1u;
+  if (wave != chain_wave) {
+    const uint32_t lw = wave < chain_wave ? wave : wave - 1;
     for (uint32_t i = 0; i < nstep; ++i) {
       if (i < nstage) {
         DType *slot = ring[i % kSlots];

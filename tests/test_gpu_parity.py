@@ -271,6 +271,8 @@ def test_reduce_reference_known_answers(G, stream):
 SOFTMAX_SHAPES = [((64, 32000), 0), ((5, 1000), 0), ((5, 1001), 0), ((3, 7), 1), ((9, 2048), 4),
                   ((4, 8192), 0), ((3, 16384), 0), ((2, 40000), 0), ((2, 70001), 0), ((7, 1), 0),
                   ((3, 5000), 3), ((2, 20000), 1),
+                  # rows that neither start at multiples of 16 bytes nor are whole packs
+                  ((3, 50257), 0), ((2, 33333), 1), ((2, 65535), 0), ((6, 4097), 2), ((5, 1023), 0),
                   # short rows: one thread per row up to 32 columns, one wave per row up to 256
                   ((1000, 10), 0), ((300, 32), 0), ((77, 33), 2), ((130, 64), 0), ((50, 65), 1),
                   ((41, 128), 0), ((19, 200), 3), ((64, 256), 0), ((9, 257), 0), ((5, 2), 0)]
@@ -432,6 +434,9 @@ POOL_CASES = [  # planes, h, w, ky, kx, sy, sx, pad
     (16, 112, 112, 3, 3, 2, 2, 0), (6, 37, 41, 3, 3, 2, 2, 2), (6, 37, 41, 2, 2, 2, 2, 0),
     (3, 9, 11, 3, 2, 1, 3, 1), (2, 30, 30, 5, 5, 3, 2, 0), (4, 6, 6, 1, 1, 1, 1, 0),
     (2, 7, 300, 7, 3, 1, 2, 0), (1, 3, 20000, 2, 2, 1, 2, 0),
+    # many small planes: several per workgroup, the last workgroup with fewer
+    (4096, 9, 9, 3, 3, 2, 2, 0), (2560, 13, 13, 3, 3, 2, 2, 1), (2500, 7, 10, 2, 2, 2, 2, 0),
+    (3001, 12, 70, 3, 2, 1, 2, 2),
 ]
 
 
@@ -494,6 +499,10 @@ CONV = [  # n, c, h, w, ky, kx, sy, sx, dy, dx, py, px
     # cut into several bands of rows
     (40, 64, 16, 16, 3, 3, 1, 1, 1, 1, 1, 1), (3, 700, 8, 24, 5, 3, 1, 1, 1, 1, 2, 1),
     (1, 2, 300, 128, 3, 3, 1, 1, 1, 1, 1, 1), (2, 1, 181, 264, 4, 3, 1, 1, 1, 1, 2, 1),
+    # stride 1 with patch rows that are not whole packs, no padding, wide windows, odd sizes
+    (2, 5, 54, 54, 3, 3, 1, 1, 1, 1, 0, 0), (3, 4, 28, 28, 5, 5, 1, 1, 1, 1, 2, 2),
+    (8, 3, 13, 17, 3, 5, 1, 1, 1, 1, 0, 2), (8, 2, 9, 9, 7, 7, 1, 1, 1, 1, 3, 3),
+    (16, 6, 10, 12, 1, 1, 1, 1, 1, 1, 0, 0), (8, 2, 6, 40, 2, 4, 1, 1, 1, 1, 1, 3),
 ]
 
 
