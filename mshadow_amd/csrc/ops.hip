@@ -127,7 +127,9 @@ int Im2Col(T *col, int cstride, const T *img, int istride, const PatchGeom &g, v
       return AfterLaunch("im2col");
     }
   }
-  /* stride 1, dilation 1, patch rows of a pack or more: pack by pack, no staging */
+  /* stride 1, dilation 1, patch rows of a pack or more: pack by pack, no staging. (With a stride
+     the elements of a pack lie apart in the image; fetched one by one, 3x3 stride 2 on
+     (32,256,56,56) took 115 us against 64 us for the staged kernel below.) */
   if (unit_steps && g.ow >= EPT) {
     const long long ppr = (g.ow + EPT - 1) / EPT;
     const long long places = static_cast<long long>(g.n) * g.oh * ppr;
@@ -238,6 +240,23 @@ int Col2Im(T *img, int istride, const T *col, int cstride, const PatchGeom &g, v
       const unsigned blocks = static_cast<unsigned>((packs + kPatchBlock - 1) / kPatchBlock);
       hipLaunchKernelGGL((Col2ImDirectS1Kernel<T>), dim3(blocks), dim3(kPatchBlock), 0, AsStream(stream),
                          img, istride, col, cstride, g, mshadow::FastDivU32(static_cast<uint32_t>(wpk)),
+                         mshadow::FastDivU32(static_cast<uint32_t>(g.h)),
+                         mshadow::FastDivU32(static_cast<uint32_t>(g.c)), static_cast<uint32_t>(packs));
+      return AfterLaunch("col2im");
+    }
+  }
+  /* strides above 1, image rows of a pack or more: a pixel has few patches, gathered directly */
+  if ((g.sy > 1 || g.sx > 1) && g.w >= EPT) {
+    const long long wpk = (g.w + EPT - 1) / EPT;
+    const long long packs = static_cast<long long>(g.n) * g.c * g.h * wpk;
+    if (packs + kPatchBlock < (1ll << 31) && cols < (1ll << 31)) {
+      const unsigned blocks = static_cast<unsigned>((packs + kPatchBlock - 1) / kPatchBlock);
+      const PatchDivs dv = {mshadow::FastDivU32(static_cast<uint32_t>(g.sy)),
+                            mshadow::FastDivU32(static_cast<uint32_t>(g.sx)),
+                            mshadow::FastDivU32(static_cast<uint32_t>(g.dy)),
+                            mshadow::FastDivU32(static_cast<uint32_t>(g.dx))};
+      hipLaunchKernelGGL((Col2ImGatherKernel<T>), dim3(blocks), dim3(kPatchBlock), 0, AsStream(stream),
+                         img, istride, col, cstride, g, dv, mshadow::FastDivU32(static_cast<uint32_t>(wpk)),
                          mshadow::FastDivU32(static_cast<uint32_t>(g.h)),
                          mshadow::FastDivU32(static_cast<uint32_t>(g.c)), static_cast<uint32_t>(packs));
       return AfterLaunch("col2im");
@@ -488,6 +507,19 @@ int mshadow_hip_softmax_f32(float *dst, int dstride, const float *src, int sstri
 #define SOFTMAX_LAUNCH(T, S, V) \
   hipLaunchKernelGGL((SoftmaxRowKernel<T, S, V, false>), dim3(rows), dim3(T), 0, s, dst, dstride, \
                      src, sstride, cols)
+#define SOFTMAX_WAVE(SLABS) \
+  hipLaunchKernelGGL((SoftmaxWaveSlabsKernel<SLABS, false>), dim3((rows + 3) / 4), dim3(256), 0, s, dst, \
+                     dstride, src, sstride, rows, cols)
+  /* many rows of up to 2048 columns: a wave per row (65536 rows of 300 / 1000 / 2000 columns:
+     71 / 109 / 122 us against 163 / 193 / 139 us with a workgroup per row; from 4096 columns on,
+     or with few rows, the workgroup per row is faster) */
+  if (cols <= 2048 && rows >= 8 * mshadow_abi::ComputeUnits()) {
+    if (cols <= 512) SOFTMAX_WAVE(2);
+    else if (cols <= 1024) SOFTMAX_WAVE(4);
+    else SOFTMAX_WAVE(8);
+    return AfterLaunch("softmax");
+  }
+#undef SOFTMAX_WAVE
   if (cols <= 1024) SOFTMAX_LAUNCH(256, 1, 4);
   else if (cols <= 2048) SOFTMAX_LAUNCH(256, 2, 4);
   else if (cols <= 4096) SOFTMAX_LAUNCH(256, 4, 4);
@@ -511,6 +543,16 @@ int mshadow_hip_softmax_rowsum_f32(float *sums, const float *terms, int tstride,
   hipStream_t s = AsStream(stream);
   if (cols <= 256) {
     LaunchShortSoftmax<true>(sums, 0, terms, tstride, rows, cols, s);
+    return AfterLaunch("softmax_rowsum");
+  }
+  if (cols <= 2048 && rows >= 8 * mshadow_abi::ComputeUnits()) {  // as in mshadow_hip_softmax_f32
+#define ROWSUM_WAVE(SLABS) \
+  hipLaunchKernelGGL((SoftmaxWaveSlabsKernel<SLABS, true>), dim3((rows + 3) / 4), dim3(256), 0, s, sums, 0, \
+                     terms, tstride, rows, cols)
+    if (cols <= 512) ROWSUM_WAVE(2);
+    else if (cols <= 1024) ROWSUM_WAVE(4);
+    else ROWSUM_WAVE(8);
+#undef ROWSUM_WAVE
     return AfterLaunch("softmax_rowsum");
   }
   const bool vec = Aligned16(terms) && tstride % 4 == 0 && cols % 4 == 0;
@@ -961,6 +1003,22 @@ int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstrid
     else UNPOOL_ROWS(MSHADOW_HIP_MIN);
 #undef UNPOOL_ROWS
     return AfterLaunch("unpool");
+  }
+  /* small planes under a stride of 2 or more (a pixel has few windows): no staging. Measured on
+     (128,256,28,28), 2x2 stride 2: 56 us against 96 us for the kernels below; on large planes or
+     with stride 1 the staged kernels are faster. */
+  if (static_cast<long long>(h) * w * sizeof(float) <= 4 * 1024 && sy >= 2 && sx >= 2 && w >= 4) {
+    const long long wpk = (w + 3) / 4;
+    const long long packs = static_cast<long long>(planes) * h * wpk;
+    if (packs + kPoolBlock < (1ll << 31)) {
+      const unsigned blocks = static_cast<unsigned>((packs + kPoolBlock - 1) / kPoolBlock);
+      POOL_SWITCH(UnpoolGatherKernel, dim3(blocks), dim3(kPoolBlock), 0, s, dst, dstride, src, sstride,
+                  pooled, pstride, grad, gstride, g, mshadow::FastDivU32(static_cast<uint32_t>(sy)),
+                  mshadow::FastDivU32(static_cast<uint32_t>(sx)),
+                  mshadow::FastDivU32(static_cast<uint32_t>(wpk)),
+                  mshadow::FastDivU32(static_cast<uint32_t>(h)), static_cast<uint32_t>(packs))
+      return AfterLaunch("unpool");
+    }
   }
   /* small planes: several whole planes per workgroup (about 24 KB of pooled values and gradients) */
   {

@@ -882,6 +882,55 @@ __global__ void __launch_bounds__(kPatchBlock)
   }
 }
 
+/*! \brief the divisions by stride and dilation that col2im's patch ranges need, as multiplications */
+struct PatchDivs {
+  mshadow::FastDivU32 sy, sx, dy, dx;
+};
+
+/*! \brief col2im for any stride and dilation, no staging: a thread sums one pack of an image row
+ *  (the last pack of a row moved back to end with the row), pixel by pixel over the patches
+ *  that cover it, exactly the loops of mshadow/extension/pack_col2patch.h:118-144 with the
+ *  divisions done by multiplication; the terms come by element-sized loads, which neighbouring
+ *  lanes and pixels share cache lines for. For strides above 1, where a pixel has few patches. */
+template <typename T>
+__global__ void __launch_bounds__(kPatchBlock)
+    Col2ImGatherKernel(T *img, int istride, const T *col, int cstride, PatchGeom g, PatchDivs dv,
+                       mshadow::FastDivU32 div_wpk, mshadow::FastDivU32 div_h,
+                       mshadow::FastDivU32 div_c, uint32_t total_packs) {
+  const int EPT = 16 / sizeof(T);
+  const uint32_t pk = blockIdx.x * kPatchBlock + threadIdx.x;
+  if (pk >= total_packs) return;
+  const uint32_t rowi = div_wpk.Div(pk);             // (n * c + ch) * h + cy
+  const int x0 = min(static_cast<int>(pk - rowi * div_wpk.div) * EPT, g.w - EPT);
+  const uint32_t plane = div_h.Div(rowi);
+  const int cy = static_cast<int>(rowi - plane * g.h);
+  const uint32_t n = div_c.Div(plane);
+  const uint32_t ch = plane - n * g.c;
+  const int span_y = g.dy * (g.ky - 1) + 1;
+  const int span_x = g.dx * (g.kx - 1) + 1;
+  const int y = cy + g.pad_y;                        // position in the padded image
+  const int py_min = y < span_y ? static_cast<int>(dv.dy.Mod(y)) : static_cast<int>(dv.sy.Div(y - span_y + g.sy));
+  const int py_max = min(static_cast<int>(dv.sy.Div(y + g.sy)), g.oh);
+  const T *base = col + static_cast<size_t>(ch) * g.ky * g.kx * cstride + static_cast<size_t>(n) * g.oh * g.ow;
+  U4 acc = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const int x = x0 + e + g.pad_x;
+    const int px_min = x < span_x ? static_cast<int>(dv.dx.Mod(x)) : static_cast<int>(dv.sx.Div(x - span_x + g.sx));
+    const int px_max = min(static_cast<int>(dv.sx.Div(x + g.sx)), g.ow);
+    T res = Acc<T>::Zero();
+    for (int py = py_min; py < py_max; py += g.dy) {
+      const int a = static_cast<int>(dv.dy.Div(y - py * g.sy));
+      for (int px = px_min; px < px_max; px += g.dx) {
+        const int b = static_cast<int>(dv.dx.Div(x - px * g.sx));
+        res = Acc<T>::Add(res, base[static_cast<size_t>(a * g.kx + b) * cstride + py * g.ow + px]);
+      }
+    }
+    SetPackElement(&acc, e, res);
+  }
+  StorePackAnywhere(img + static_cast<size_t>(rowi) * istride + x0, acc);
+}
+
 /*! \brief one image pixel per thread; consecutive threads take consecutive x so that,
  *  for a fixed patch offset, their column-matrix reads are consecutive too */
 template <typename T>

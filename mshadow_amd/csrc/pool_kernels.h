@@ -318,6 +318,48 @@ __global__ void __launch_bounds__(kPoolBlock)
   }
 }
 
+/*! \brief unpool with no staging, any window and stride, rows of four pixels or more: a thread
+ *  takes four neighbouring source pixels (one 16-byte access each way, at any alignment; the
+ *  last pack of a row moved back to end with the row) and, pixel by pixel, the windows that
+ *  cover it in the reference's order (py, then px ascending;
+ *  mshadow/extension/spatial_unpool.h:102-125), their pooled values and gradients by
+ *  element-sized loads that neighbouring pixels and lanes share cache lines for. */
+template <int REDUCER>
+__global__ void __launch_bounds__(kPoolBlock)
+    UnpoolGatherKernel(float *dst, int dstride, const float *src, int sstride, const float *pooled,
+                       int pstride, const float *grad, int gstride, PoolGeom g,
+                       mshadow::FastDivU32 div_sy, mshadow::FastDivU32 div_sx,
+                       mshadow::FastDivU32 div_wpk, mshadow::FastDivU32 div_h, uint32_t total_packs) {
+  typedef PoolOp<REDUCER> Op;
+  const uint32_t pk = blockIdx.x * kPoolBlock + threadIdx.x;
+  if (pk >= total_packs) return;
+  const uint32_t r = div_wpk.Div(pk);                // plane * h + y
+  const int x0 = min(static_cast<int>(pk - r * div_wpk.div) * 4, g.w - 4);
+  const uint32_t plane = div_h.Div(r);
+  const int y = static_cast<int>(r - plane * g.h);
+  const F4 vs = StreamLoadF4Anywhere(src + static_cast<size_t>(r) * sstride + x0);
+  const int py_min = y < g.ky ? 0 : static_cast<int>(div_sy.Div(y - g.ky + g.sy));
+  const int py_max = min(static_cast<int>(div_sy.Div(y + g.sy)), g.ph);
+  const float *prow = pooled + static_cast<size_t>(plane) * g.ph * pstride;
+  const float *grow = grad + static_cast<size_t>(plane) * g.ph * gstride;
+  F4 out;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int x = x0 + e;
+    const int px_min = x < g.kx ? 0 : static_cast<int>(div_sx.Div(x - g.kx + g.sx));
+    const int px_max = min(static_cast<int>(div_sx.Div(x + g.sx)), g.pw);
+    float val = 0.0f;
+    for (int py = py_min; py < py_max; ++py) {
+      for (int px = px_min; px < px_max; ++px) {
+        val = val + Op::Grad(vs[e], prow[static_cast<size_t>(py) * pstride + px]) *
+                        grow[static_cast<size_t>(py) * gstride + px];
+      }
+    }
+    out[e] = val;
+  }
+  StreamStoreF4Anywhere(dst + static_cast<size_t>(r) * dstride + x0, out);
+}
+
 /*! \brief unpool for small planes: a workgroup takes `per_block` whole consecutive planes, stages
  *  their pooled values and gradients (per_block * ph rows each) and computes every source pixel
  *  of those planes; a wave takes 64 / w source rows at a time when rows are short. Terms in

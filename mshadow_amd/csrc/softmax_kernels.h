@@ -939,6 +939,76 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+/*! \brief one wave per row, cols <= 256 * SLABS: slab k is the 256 columns from 256 * k, lane l
+ *  holds the four from 256 * k + 4 * l (every load and store of the wave is one contiguous
+ *  kilobyte), and the sum is resolved slab after slab, in lane order within a slab
+ *  (WaveResolve) - the row's own order. Four rows per workgroup, nothing shared between them,
+ *  no barrier: for rows of a few hundred to a few thousand columns, where a workgroup per row
+ *  spends its time in the barriers of the long-row plan (65536 x 1000: 194 us). */
+template <int SLABS, bool TERMS_GIVEN>
+__global__ void __launch_bounds__(256)
+    SoftmaxWaveSlabsKernel(float *dst, int dstride, const float *src, int sstride, int rows,
+                           int cols) {
+  const int row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(WaveId());
+  if (row >= rows) return;
+  const int lane_col = LaneId() * 4;
+  const float *in = src + static_cast<size_t>(row) * sstride;
+  const float kNegInf = -__builtin_huge_valf();
+  const float kAbsent = TERMS_GIVEN ? 0.0f : kNegInf;
+  float v[SLABS][4];
+  float mx = kNegInf;
+#pragma unroll
+  for (int k = 0; k < SLABS; ++k) {
+    const int c = k * 256 + lane_col;
+    if (c + 4 <= cols) {
+      const F4 q = StreamLoadF4Anywhere(in + c);
+      v[k][0] = q.x; v[k][1] = q.y; v[k][2] = q.z; v[k][3] = q.w;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[k][i] = (c + i < cols) ? in[c + i] : kAbsent;
+    }
+    mx = MaxNum3(mx, v[k][0], v[k][1]);
+    mx = MaxNum3(mx, v[k][2], v[k][3]);
+  }
+  if (!TERMS_GIVEN) {
+    mx = WaveMaxF32(mx);
+#pragma unroll
+    for (int k = 0; k < SLABS; ++k) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[k][i] = ExpNonPositive(v[k][i] - mx);
+    }
+  }
+  float s = 0.0f;
+#pragma unroll
+  for (int k = 0; k < SLABS; ++k) {
+    if (k * 256 < cols) s = WaveResolve<4>(s, v[k]);
+  }
+  if (TERMS_GIVEN) {
+    if (LaneId() == 0) dst[row] = s;
+    return;
+  }
+  float *out = dst + static_cast<size_t>(row) * dstride;
+  const bool fast_div = s >= 1.0f && s < 3.0e38f;
+  const float rcp = 1.0f / s;
+#pragma unroll
+  for (int k = 0; k < SLABS; ++k) {
+    const int c = k * 256 + lane_col;
+    float o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = fast_div ? DivideBy(v[k][i], s, rcp) : v[k][i] / s;
+    if (c + 4 <= cols) {
+      F4 q;
+      q.x = o[0]; q.y = o[1]; q.z = o[2]; q.w = o[3];
+      StreamStoreF4Anywhere(out + c, q);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (c + i < cols) out[c + i] = o[i];
+      }
+    }
+  }
+}
+
 /*! \brief any row length: three passes, exp(x - max) parked in dst between them */
 template <int THREADS>
 __global__ void __launch_bounds__(THREADS)

@@ -273,6 +273,8 @@ SOFTMAX_SHAPES = [((64, 32000), 0), ((5, 1000), 0), ((5, 1001), 0), ((3, 7), 1),
                   ((3, 5000), 3), ((2, 20000), 1),
                   # rows that neither start at multiples of 16 bytes nor are whole packs
                   ((3, 50257), 0), ((2, 33333), 1), ((2, 65535), 0), ((6, 4097), 2), ((5, 1023), 0),
+                  # many rows of a few hundred to 2048 columns: a wave per row, slab after slab
+                  ((2100, 300), 0), ((2049, 777), 3), ((2050, 1024), 0), ((2048, 2047), 1), ((4100, 513), 0),
                   # short rows: one thread per row up to 32 columns, one wave per row up to 256
                   ((1000, 10), 0), ((300, 32), 0), ((77, 33), 2), ((130, 64), 0), ((50, 65), 1),
                   ((41, 128), 0), ((19, 200), 3), ((64, 256), 0), ((9, 257), 0), ((5, 2), 0)]
@@ -336,7 +338,7 @@ def _serial_row_sums(O, terms):
     return want
 
 
-ROWSUM_COLS = [1, 3, 10, 31, 32, 33, 64, 65, 128, 129, 255, 256, 257, 1000, 1024, 1028, 2048, 3000, 4096, 5001, 8192, 12000, 16384,
+ROWSUM_COLS = [1, 3, 10, 31, 32, 33, 64, 65, 128, 129, 255, 256, 257, 300, 513, 777, 1000, 1024, 1028, 2048, 3000, 4096, 5001, 8192, 12000, 16384,
                20001, 32000, 32768, 40000, 65536]
 
 
@@ -371,6 +373,12 @@ def test_softmax_rowsum_is_the_serial_sum(G, O, stream, cols):
             sums = G.buffer((terms.shape[0],), f32)
             G.softmax_rowsum(sums, G.to_device(terms, pad), stream)
             assert_bits_equal(sums.download(stream), want, f"row sum cols={cols} pad={pad}")
+    if 256 < cols <= 2048:
+        # with thousands of rows these lengths take the kernel with a wave per row
+        many = np.tile(terms, (150, 1))
+        sums = G.buffer((many.shape[0],), f32)
+        G.softmax_rowsum(sums, G.to_device(many, 1), stream)
+        assert_bits_equal(sums.download(stream), np.tile(want, 150), f"row sum cols={cols}, a wave per row")
 
 
 def test_softmax_rowsum_specials(G, O, stream):
@@ -503,6 +511,10 @@ CONV = [  # n, c, h, w, ky, kx, sy, sx, dy, dx, py, px
     (2, 5, 54, 54, 3, 3, 1, 1, 1, 1, 0, 0), (3, 4, 28, 28, 5, 5, 1, 1, 1, 1, 2, 2),
     (8, 3, 13, 17, 3, 5, 1, 1, 1, 1, 0, 2), (8, 2, 9, 9, 7, 7, 1, 1, 1, 1, 3, 3),
     (16, 6, 10, 12, 1, 1, 1, 1, 1, 1, 0, 0), (8, 2, 6, 40, 2, 4, 1, 1, 1, 1, 1, 3),
+    # strides and dilations on rows of a pack or more
+    (4, 6, 56, 56, 3, 3, 2, 2, 1, 1, 1, 1), (2, 3, 64, 70, 7, 7, 2, 2, 1, 1, 3, 3),
+    (3, 2, 40, 44, 3, 3, 1, 1, 2, 2, 2, 2), (2, 2, 45, 50, 3, 5, 3, 2, 2, 1, 1, 2),
+    (2, 3, 33, 47, 11, 11, 4, 4, 1, 1, 0, 0),
 ]
 
 
