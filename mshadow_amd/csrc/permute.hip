@@ -228,6 +228,25 @@ __global__ void __launch_bounds__(kPermuteBlock)
 
 /* 16 bytes per thread, whatever the unit: 8192x32000 floats by 16-byte units in 321 us with one
    unit per thread, 345 us with four, 500 us with eight (MI355X) */
+/*! \brief rows whose width, pitches or addresses are multiples of 4 but not of 16 bytes: still
+ *  16 bytes per thread - such accesses need no alignment here -, the last pack of a row moved
+ *  back so that it ends with the row (it overlaps its neighbour; both store the same bytes).
+ *  Rows of 16 bytes or more. 8192 rows of 127,960 bytes at a pitch of 128,000: 0.80 of the HBM
+XX
+__global__ void __launch_bounds__(kPermuteBlock)
+    CopyRowsAnywhereKernel(char *dst, size_t dpitch, const char *src, size_t spitch, uint32_t total,
+                           uint32_t packs_per_row, uint32_t width, FastDivU32 div_ppr) {
+  typedef uint32_t Vec4 __attribute__((ext_vector_type(4)));
+  typedef Vec4 Loose __attribute__((aligned(4)));
+  const uint32_t p = blockIdx.x * kPermuteBlock + threadIdx.x;
+  if (p >= total) return;
+  const uint32_t y = div_ppr.Div(p);
+  uint32_t x = (p - y * packs_per_row) * 16u;
+  x = x + 16u <= width ? x : width - 16u;
+  const Vec4 v = __builtin_nontemporal_load(reinterpret_cast<const Loose *>(src + static_cast<size_t>(y) * spitch + x));
+  __builtin_nontemporal_store(v, reinterpret_cast<Loose *>(dst + static_cast<size_t>(y) * dpitch + x));
+}
+
 template <typename T>
 struct CopyUnroll {
   static const int value = sizeof(T) >= 16 ? 1 : 16 / sizeof(T);
@@ -284,9 +303,17 @@ bool CopyRowsOnDevice(void *dst, size_t dpitch_bytes, const void *src, size_t sp
   if (all % 16 == 0) {
     typedef uint32_t Vec __attribute__((ext_vector_type(4)));
     LaunchCopyRows<Vec>(dst, dpitch_bytes, src, spitch_bytes, width_bytes, rows, s);
-  } else if (all % 8 == 0) {
-    typedef uint32_t Vec2 __attribute__((ext_vector_type(2)));
-    LaunchCopyRows<Vec2>(dst, dpitch_bytes, src, spitch_bytes, width_bytes, rows, s);
+  } else if (all % 4 == 0 && width_bytes >= 16 && width_bytes < (1ull << 32)) {
+    const uint32_t ppr = static_cast<uint32_t>((width_bytes + 15) / 16);
+    const size_t rows_per_launch = std::max<size_t>(1, kCopyMaxUnits / ppr);
+    for (size_t y0 = 0; y0 < rows; y0 += rows_per_launch) {
+      const size_t nrows = std::min(rows_per_launch, rows - y0);
+      const uint32_t n = static_cast<uint32_t>(nrows * ppr);
+      hipLaunchKernelGGL(CopyRowsAnywhereKernel, dim3((n + kPermuteBlock - 1) / kPermuteBlock),
+                         dim3(kPermuteBlock), 0, s, static_cast<char *>(dst) + y0 * dpitch_bytes,
+                         dpitch_bytes, static_cast<const char *>(src) + y0 * spitch_bytes, spitch_bytes, n,
+                         ppr, static_cast<uint32_t>(width_bytes), FastDivU32(ppr));
+    }
   } else if (all % 4 == 0) {
     LaunchCopyRows<uint32_t>(dst, dpitch_bytes, src, spitch_bytes, width_bytes, rows, s);
   } else {

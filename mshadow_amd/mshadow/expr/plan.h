@@ -56,31 +56,42 @@ struct RawVec<1> {
 };
 /*! \brief load / store one Pack. STREAM marks the access non-temporal: the data passes
  *  through once and should not displace other lines in the caches (device code only). */
+/* On the device a pack is moved as one access wherever it lies: the address needs the
+   element's alignment only (16-byte global accesses need no 16-byte alignment on gfx950; where
+   the address happens to be aligned the instruction is the same one). */
 template <typename DType, int N, bool STREAM>
 MSHADOW_XINLINE Pack<DType, N> LoadPack(const DType *p) {
 #if defined(__HIP_DEVICE_COMPILE__)
+  typedef typename RawVec<sizeof(DType) * N>::type Raw;
+  typedef Raw Loose __attribute__((aligned(1)));
+  Raw raw;
   if (STREAM) {
-    typedef typename RawVec<sizeof(DType) * N>::type Raw;
-    const Raw raw = __builtin_nontemporal_load(reinterpret_cast<const Raw *>(p));
-    Pack<DType, N> out;
-    __builtin_memcpy(&out, &raw, sizeof(out));
-    return out;
+    raw = __builtin_nontemporal_load(reinterpret_cast<const Loose *>(p));
+  } else {
+    raw = *reinterpret_cast<const Loose *>(p);
   }
-#endif
+  Pack<DType, N> out;
+  __builtin_memcpy(&out, &raw, sizeof(out));
+  return out;
+#else
   return *reinterpret_cast<const Pack<DType, N> *>(p);
+#endif
 }
 template <typename DType, int N, bool STREAM>
 MSHADOW_XINLINE void StorePackTo(DType *p, const Pack<DType, N> &v) {
 #if defined(__HIP_DEVICE_COMPILE__)
+  typedef typename RawVec<sizeof(DType) * N>::type Raw;
+  typedef Raw Loose __attribute__((aligned(1)));
+  Raw raw;
+  __builtin_memcpy(&raw, &v, sizeof(raw));
   if (STREAM) {
-    typedef typename RawVec<sizeof(DType) * N>::type Raw;
-    Raw raw;
-    __builtin_memcpy(&raw, &v, sizeof(raw));
-    __builtin_nontemporal_store(raw, reinterpret_cast<Raw *>(p));
-    return;
+    __builtin_nontemporal_store(raw, reinterpret_cast<Loose *>(p));
+  } else {
+    *reinterpret_cast<Loose *>(p) = raw;
   }
-#endif
+#else
   *reinterpret_cast<Pack<DType, N> *>(p) = v;
+#endif
 }
 }  // namespace plan_detail
 
@@ -104,6 +115,7 @@ template <typename Device, int dim, typename DType>
 class Plan<Tensor<Device, dim, DType>, DType> {
  public:
   static const bool kPackable = true;
+  static const bool kRaggedRows = true;
   explicit Plan(const Tensor<Device, dim, DType> &t) : dptr_(t.dptr_), stride_(t.stride_) {}
   /* offsets in 64 bits whatever index_t is: a tensor whose dimensions each fit index_t may
      still hold 2^31 elements or more (65536 x 32768 floats are 8 GiB of a 288 GB device) */
@@ -121,7 +133,7 @@ class Plan<Tensor<Device, dim, DType>, DType> {
    *  while rows are dense (pitch == cols) so that the 2-D view can be walked linearly */
   inline bool PackReady(int n, index_t cols, bool *flat) const {
     if (stride_ != cols) *flat = false;
-    return reinterpret_cast<uintptr_t>(dptr_) % (sizeof(DType) * n) == 0 && stride_ % n == 0;
+    return true;  // a pack is fetched wherever it lies
   }
 
  private:
@@ -136,6 +148,7 @@ template <typename Device, typename DType>
 class Plan<Tensor<Device, 1, DType>, DType> {
  public:
   static const bool kPackable = true;
+  static const bool kRaggedRows = true;
   explicit Plan(const Tensor<Device, 1, DType> &t) : dptr_(t.dptr_) {}
   MSHADOW_XINLINE DType &REval(index_t y, index_t x) { return dptr_[x]; }
   MSHADOW_XINLINE const DType &Eval(index_t y, index_t x) const { return dptr_[x]; }
@@ -147,9 +160,7 @@ class Plan<Tensor<Device, 1, DType>, DType> {
   MSHADOW_XINLINE void StorePack(index_t y, index_t x, const Pack<DType, N> &p) {
     plan_detail::StorePackTo<DType, N, STREAM>(dptr_ + x, p);
   }
-  inline bool PackReady(int n, index_t cols, bool *flat) const {
-    return reinterpret_cast<uintptr_t>(dptr_) % (sizeof(DType) * n) == 0;
-  }
+  inline bool PackReady(int n, index_t cols, bool *flat) const { return true; }
 
  private:
   DType *dptr_;
@@ -159,6 +170,7 @@ template <typename DType>
 class Plan<ScalarExp<DType>, DType> {
  public:
   static const bool kPackable = true;
+  static const bool kRaggedRows = true;
   explicit Plan(DType scalar) : scalar_(scalar) {}
   MSHADOW_XINLINE DType Eval(index_t y, index_t x) const { return scalar_; }
   template <int N, bool STREAM = false>
@@ -210,6 +222,17 @@ struct Packable {
   static long Test(...);  // NOLINT(*)
   static const bool value = sizeof(Test<P>(0)) == sizeof(char);
 };
+/*! \brief P::kRaggedRows if the plan type declares it, false otherwise: the plan is made of
+ *  tensors, scalars and elementwise functions only, so it evaluates a pack at any column of
+ *  any row (rows need not be whole packs, nor start at multiples of 16 bytes) */
+template <typename P>
+struct RaggedRows {
+  template <typename Q>
+  static char Test(int (*)[Q::kRaggedRows ? 1 : -1]);
+  template <typename Q>
+  static long Test(...);  // NOLINT(*)
+  static const bool value = sizeof(Test<P>(0)) == sizeof(char);
+};
 /*! \brief P::kPlaneWindow if the plan type declares it, false otherwise: somewhere in the
  *  plan a window runs over neighbouring planes, and the plan has EvalPackRun */
 template <typename P>
@@ -255,6 +278,9 @@ class Plan<TernaryMapExp<OP, TA, TB, TC, DType, etype>, DType> {
   static const bool kPackable = plan_detail::Packable<Plan<TA, DType> >::value &&
                                 plan_detail::Packable<Plan<TB, DType> >::value &&
                                 plan_detail::Packable<Plan<TC, DType> >::value;
+  static const bool kRaggedRows = plan_detail::RaggedRows<Plan<TA, DType> >::value &&
+                                  plan_detail::RaggedRows<Plan<TB, DType> >::value &&
+                                  plan_detail::RaggedRows<Plan<TC, DType> >::value;
   explicit Plan(const Plan<TA, DType> &item1, const Plan<TB, DType> &item2,
                 const Plan<TC, DType> &item3)
       : item1_(item1), item2_(item2), item3_(item3) {}
@@ -287,6 +313,8 @@ class Plan<BinaryMapExp<OP, TA, TB, DType, etype>, DType> {
  public:
   static const bool kPackable = plan_detail::Packable<Plan<TA, DType> >::value &&
                                 plan_detail::Packable<Plan<TB, DType> >::value;
+  static const bool kRaggedRows = plan_detail::RaggedRows<Plan<TA, DType> >::value &&
+                                  plan_detail::RaggedRows<Plan<TB, DType> >::value;
   explicit Plan(const Plan<TA, DType> &lhs, const Plan<TB, DType> &rhs) : lhs_(lhs), rhs_(rhs) {}
   MSHADOW_XINLINE DType Eval(index_t y, index_t x) const {
     return OP::Map(lhs_.Eval(y, x), rhs_.Eval(y, x));
@@ -330,6 +358,7 @@ template <typename OP, typename TA, int etype, typename DType>
 class Plan<UnaryMapExp<OP, TA, DType, etype>, DType> {
  public:
   static const bool kPackable = plan_detail::Packable<Plan<TA, DType> >::value;
+  static const bool kRaggedRows = plan_detail::RaggedRows<Plan<TA, DType> >::value;
   explicit Plan(const Plan<TA, DType> &src) : src_(src) {}
   MSHADOW_XINLINE DType Eval(index_t y, index_t x) const { return OP::Map(src_.Eval(y, x)); }
   template <int N, bool STREAM = false>

@@ -4,9 +4,11 @@
  * MapPlanLargeKernel of the reference (mshadow/cuda/tensor_gpu-inl.cuh:67-120), which
  * handle one element per thread with a division per element and 4-byte accesses.
  *
- * MapPackKernel  every leaf is a tensor or scalar and all pointers / pitches are
- *                16-byte aligned: each thread moves kPackUnroll packs of N = 16 /
- *                sizeof(DType) elements with one 128-bit global access per leaf. When
+ * MapPackKernel  every leaf evaluates packs: each thread moves kPackUnroll packs of N = 16 /
+ *                sizeof(DType) elements with one 128-bit global access per leaf, wherever the
+ *                pack lies (no alignment is needed). Plans of tensors, scalars and elementwise
+ *                functions also take rows that are not whole packs (the last pack of a row
+ *                element by element); other packable plans need cols % N == 0. When
  *                all rows are dense the 2-D view is walked linearly and no division
  *                is executed at all; otherwise there is one per pack. Large tensors are
  *                moved with non-temporal accesses (measured on MI355X: 6.3 TB/s against
@@ -76,11 +78,14 @@ __device__ __forceinline__ void SavePack(DPlan &dplan, uint32_t y, uint32_t x,
   }
 }
 
+/*! \brief row_elems: elements of a row (of the whole run when kFlat). Where it is not a multiple
+ *  of N the last pack of a row (of the run) is partial and is evaluated element by element;
+ *  only plans of tensors, scalars and elementwise functions are launched that way. */
 template <typename Saver, typename DType, int N, bool kFlat, bool kStream, int kPackUnroll,
           typename DPlan, typename SPlan>
 __global__ void __launch_bounds__(kMapBlock)
     MapPackKernel(DPlan dplan, SPlan splan, uint32_t total_packs, uint32_t packs_per_row,
-                  FastDivU32 div_ppr, uint32_t row0) {
+                  FastDivU32 div_ppr, uint32_t row0, uint32_t row_elems) {
   typedef expr::Pack<DType, N> P;
   /* with real row numbers in play (windows over rows re-read their neighbours' data), each
      XCD takes a contiguous run of the workgroups */
@@ -99,12 +104,30 @@ __global__ void __launch_bounds__(kMapBlock)
       x[u] = (p - yr * packs_per_row) * N;
       y[u] = yr + row0;  // the launch covers whole rows from row0 on, fewer than 2^31 packs
     }
-    if (p < total_packs) val[u] = splan.template EvalPack<N, kStream>(y[u], x[u]);
+    if (p < total_packs) {
+      if (x[u] + N <= row_elems) {
+        val[u] = splan.template EvalPack<N, kStream>(y[u], x[u]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+          if (x[u] + i < row_elems) val[u].v[i] = splan.Eval(y[u], x[u] + i);
+        }
+      }
+    }
   }
 #pragma unroll
   for (int u = 0; u < kPackUnroll; ++u) {
     const uint32_t p = base + u * kMapBlock;
-    if (p < total_packs) SavePack<Saver, DType, N, kStream>(dplan, y[u], x[u], val[u]);
+    if (p < total_packs) {
+      if (x[u] + N <= row_elems) {
+        SavePack<Saver, DType, N, kStream>(dplan, y[u], x[u], val[u]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+          if (x[u] + i < row_elems) Saver::template Save<DType>(dplan.REval(y[u], x[u] + i), val[u].v[i]);
+        }
+      }
+    }
   }
 }
 

@@ -1003,13 +1003,16 @@ struct MapLauncher<Saver, DType, DPlan, SPlan, true> {
     uint32_t rows = shape[0], cols = shape[1];
     if (rows == 0 || cols == 0) return;
     bool flat = true;
-    const bool aligned = cols % N == 0 && dplan.PackReady(N, cols, &flat) &&
-                         splan.PackReady(N, cols, &flat);
+    /* rows that are not whole packs: only for plans that evaluate a pack at any column */
+    const bool ragged_ok = expr::plan_detail::RaggedRows<DPlan>::value &&
+                           expr::plan_detail::RaggedRows<SPlan>::value;
+    const bool aligned = (cols % N == 0 || (ragged_ok && cols >= static_cast<uint32_t>(N))) &&
+                         dplan.PackReady(N, cols, &flat) && splan.PackReady(N, cols, &flat);
     if (!aligned) {
       MapLauncher<Saver, DType, DPlan, SPlan, false>::Run(dplan, splan, shape, stream);
       return;
     }
-    uint32_t ppr = cols / N;
+    uint32_t ppr = (cols + N - 1) / N;
     /* a plan that carries three or more tensor leaves (pointer + pitch each) is "deep" */
     const int kUnroll = sizeof(SPlan) >= 3 * (sizeof(void *) + sizeof(index_t))
                             ? hip::kPackUnrollDeep : hip::kPackUnroll;
@@ -1023,7 +1026,7 @@ struct MapLauncher<Saver, DType, DPlan, SPlan, true> {
     const uint32_t run_rows = RowsPerLaunch(cols);
     const bool one_run = rows <= run_rows;
     const bool is_flat = one_run && (flat || rows == 1);
-    if (one_run && !is_flat &&
+    if (one_run && !is_flat && cols % N == 0 &&
         PlanesLauncher<Saver, DType, N, kUnroll, DPlan, SPlan,
                        expr::plan_detail::PlaneWindow<SPlan>::value>::Run(dplan, splan, rows, ppr,
                                                                           stream_hint, stream)) {
@@ -1031,9 +1034,12 @@ struct MapLauncher<Saver, DType, DPlan, SPlan, true> {
     }
     for (uint32_t row0 = 0; row0 < rows; row0 += run_rows) {
       uint32_t first = row0;
-      uint32_t total = (rows - row0 < run_rows ? rows - row0 : run_rows) * ppr;
+      const uint32_t nrows = rows - row0 < run_rows ? rows - row0 : run_rows;
+      /* a flat run is one long row: only its very last pack can be partial */
+      uint32_t row_elems = is_flat ? nrows * cols : cols;
+      uint32_t total = is_flat ? (row_elems + N - 1) / N : nrows * ppr;
       const uint32_t grid = (total + per_block - 1) / per_block;
-      void *args[] = {&dplan, &splan, &total, &ppr, &div_ppr, &first};
+      void *args[] = {&dplan, &splan, &total, &ppr, &div_ppr, &first, &row_elems};
 #define MSHADOW_MAP_LAUNCH(FLAT, STREAM)                                                   \
   Launch(hip::MapPackKernel<Saver, DType, N, FLAT, STREAM, kUnroll, DPlan, SPlan>, grid,   \
          hip::kMapBlock, args, stream)
