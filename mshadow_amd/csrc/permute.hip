@@ -231,8 +231,8 @@ __global__ void __launch_bounds__(kPermuteBlock)
 /*! \brief rows whose width, pitches or addresses are multiples of 4 but not of 16 bytes: still
  *  16 bytes per thread - such accesses need no alignment here -, the last pack of a row moved
  *  back so that it ends with the row (it overlaps its neighbour; both store the same bytes).
- *  Rows of 16 bytes or more. 8192 rows of 127,960 bytes at a pitch of 128,000: 0.80 of the HBM
-XX
+ *  Rows of 16 bytes or more. 8192 rows of 127,960 bytes at a pitch of 128,000: 0.78 of the HBM
+ *  peak against 0.75 by 8-byte units. */
 __global__ void __launch_bounds__(kPermuteBlock)
     CopyRowsAnywhereKernel(char *dst, size_t dpitch, const char *src, size_t spitch, uint32_t total,
                            uint32_t packs_per_row, uint32_t width, FastDivU32 div_ppr) {
