@@ -163,31 +163,6 @@ int Im2Col(T *col, int cstride, const T *img, int istride, const PatchGeom &g, v
     t.pitch = g.wp;
     const long long blocks = planes * nb;
     if (blocks >= (1ll << 31)) return Fail(MSHADOW_HIP_ERR_ARGUMENT, "im2col: too many workgroups");
-    /* binary16, 3 taps per row, stride and dilation 1, rows of whole aligned packs */
-    const bool row3 = sizeof(T) == 2 && g.kx == 3 && g.sy == 1 && g.sx == 1 && g.dy == 1 &&
-                      g.dx == 1 && g.ow % 8 == 0 && cstride % 8 == 0 &&
-                      reinterpret_cast<uintptr_t>(col) % 16 == 0;
-    if (row3) {
-      t.pitch = (g.wp + 7) / 8 * 8;
-      const size_t lds = static_cast<size_t>(t.rows_max) * t.pitch * sizeof(T);
-      const mshadow::FastDivU32 div_ppr(static_cast<uint32_t>(g.ow / 8));
-      /* rows without padding between them and made of whole aligned packs: fetched by packs -
-         straight into the taps where the image is padded by one column, else staged */
-      const bool dense = istride == g.w && g.w % 8 == 0 && reinterpret_cast<uintptr_t>(img) % 16 == 0;
-      const mshadow::FastDivU32 div_w(static_cast<uint32_t>(g.w));
-      if (dense) {
-        hipLaunchKernelGGL(Im2ColHalfRow3Kernel<true>, dim3(static_cast<unsigned>(blocks)),
-                           dim3(kPatchBlock), lds, AsStream(stream), reinterpret_cast<uint16_t *>(col),
-                           cstride, reinterpret_cast<const uint16_t *>(img), istride, g, t, div_ppr,
-                           div_w);
-      } else {
-        hipLaunchKernelGGL(Im2ColHalfRow3Kernel<false>, dim3(static_cast<unsigned>(blocks)),
-                           dim3(kPatchBlock), lds, AsStream(stream), reinterpret_cast<uint16_t *>(col),
-                           cstride, reinterpret_cast<const uint16_t *>(img), istride, g, t, div_ppr,
-                           div_w);
-      }
-      return AfterLaunch("im2col");
-    }
     const size_t lds = static_cast<size_t>(t.rows_max) * row_bytes;
     hipLaunchKernelGGL((Im2ColTiledKernel<T, EPT>), dim3(static_cast<unsigned>(blocks)),
                        dim3(kPatchBlock), lds, AsStream(stream), col, cstride, img, istride, g, t);
@@ -283,12 +258,7 @@ int Col2Im(T *img, int istride, const T *col, int cstride, const PatchGeom &g, v
     const size_t lds = static_cast<size_t>(taps) * t.pitch * sizeof(T);
     const long long blocks = planes * nb;
     if (blocks >= (1ll << 31)) return Fail(MSHADOW_HIP_ERR_ARGUMENT, "col2im: too many workgroups");
-    if (sizeof(T) == 2 && g.dy == 1 && g.dx == 1 && g.sy == 1 && g.sx == 1 && g.ky == 3 && g.kx == 3) {
-      const mshadow::FastDivU32 div_wpairs(static_cast<uint32_t>((g.w + 1) / 2));
-      hipLaunchKernelGGL((Col2ImHalfPairKernel<3, 3>), dim3(static_cast<unsigned>(blocks)),
-                         dim3(kPatchBlock), lds, AsStream(stream), reinterpret_cast<uint16_t *>(img),
-                         istride, reinterpret_cast<const uint16_t *>(col), cstride, g, t, div_wpairs);
-    } else if (g.dy == 1 && g.dx == 1 && g.sy == 1 && g.sx == 1) {
+    if (g.dy == 1 && g.dx == 1 && g.sy == 1 && g.sx == 1) {
       hipLaunchKernelGGL((Col2ImTiledKernel<T, EPT, true>), dim3(static_cast<unsigned>(blocks)),
                          dim3(kPatchBlock), lds, AsStream(stream), img, istride, col, cstride, g, t);
     } else {

@@ -166,99 +166,8 @@ __global__ void __launch_bounds__(kPatchBlock)
   }
 }
 
-/*! \brief im2col for binary16, stride 1, dilation 1, kx = 3 and a patch row made of whole
- *  8-element packs (ow % 8 == 0). The three taps b = 0, 1, 2 of one (a, oy, ox..ox+7)
- *  position read overlapping LDS elements ox..ox+9: they are fetched once as five aligned
- *  dwords and the three 16-byte output packs are cut from them (b = 1 by a funnel shift),
- *  so a pack costs less than one LDS read instead of eight 16-bit ones. LDS rows are
- *  16-byte aligned (t.pitch % 8 == 0).
- *  DENSE: the image rows lie in memory without padding between them and are whole 16-byte
- *  packs (w % 8 == 0, istride == w, aligned base): the band's rows are one contiguous run
- *  and are fetched as 16-byte packs instead of element by element. With the image coming
- *  from HBM (not found in the memory-side cache) that is 98 us against 115 us on the
- *  (32,256,56,56) case; with the image in that cache both forms take 84-87 us. The loads
- *  keep the default cache policy: as streaming loads they never find the image in the
- *  memory-side cache (101-105 us either way). */
-template <bool DENSE>
-__global__ void __launch_bounds__(kPatchBlock)
-    Im2ColHalfRow3Kernel(uint16_t *col, int cstride, const uint16_t *img, int istride, PatchGeom g,
-                         PatchTile t, mshadow::FastDivU32 div_ppr, mshadow::FastDivU32 div_w) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  typedef uint16_t T;
-  T *lds = reinterpret_cast<T *>(smem_raw);
-  int n, ch, band;
-  PlaneOfBlock(g, t, &n, &ch, &band);
-  const int plane = n * g.c + ch;
-  const int oy0 = band * t.band;
-  const int noy = min(t.band, g.oh - oy0);
-  const int in_rows = noy + g.ky - 1;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const T *src = img + static_cast<size_t>(plane) * g.h * istride;
-  if (DENSE) {
-    for (int i = threadIdx.x; i < in_rows * t.pitch / 2; i += kPatchBlock) {
-      reinterpret_cast<uint32_t *>(lds)[i] = 0u;
-    }
-    __syncthreads();
-    const int top = oy0 - g.pad_y;                   // image row of the first staged row
-    const int ylo = max(top, 0), yhi = min(top + in_rows, g.h);
-    const int npk = (yhi - ylo) * (g.w / 8);
-    const U4 *packs = reinterpret_cast<const U4 *>(src + static_cast<size_t>(ylo) * g.w);
-    for (int pk = threadIdx.x; pk < npk; pk += kPatchBlock) {
-      const U4 q = packs[pk];
-      const int e0 = pk * 8;
-      const int yy = static_cast<int>(div_w.Div(static_cast<uint32_t>(e0)));
-      const int x = e0 - yy * g.w;
-      T *to = lds + (ylo + yy - top) * t.pitch + g.pad_x + x;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        to[2 * e] = static_cast<T>(q[e] & 0xffffu);
-        to[2 * e + 1] = static_cast<T>(q[e] >> 16);
-      }
-    }
-  } else {
-    for (int r = wave; r < in_rows; r += kPatchBlock / 64) {
-      const int y = oy0 + r - g.pad_y;
-      const bool row_ok = y >= 0 && y < g.h;
-      for (int xx = lane; xx < t.pitch; xx += 64) {
-        const int x = xx - g.pad_x;
-        T v = 0;
-        if (row_ok && x >= 0 && x < g.w) v = src[static_cast<size_t>(y) * istride + x];
-        lds[r * t.pitch + xx] = v;
-      }
-    }
-  }
-  __syncthreads();
-  const int ppr = g.ow / 8;            // packs per patch row
-  const int ppt = noy * ppr;           // packs per tap of this band
-  const int items = g.ky * ppt;
-  const size_t j0 = (static_cast<size_t>(n) * g.oh + oy0) * g.ow;
-  for (int item = threadIdx.x; item < items; item += kPatchBlock) {
-    int a = 0, pk = item;
-    while (pk >= ppt) {
-      pk -= ppt;
-      ++a;
-    }
-    const int oy = static_cast<int>(div_ppr.Div(static_cast<uint32_t>(pk)));
-    const int ox = (pk - oy * ppr) * 8;
-    const uint32_t *w = reinterpret_cast<const uint32_t *>(lds + (oy + a) * t.pitch + ox);
-    const U4 w03 = *reinterpret_cast<const U4 *>(w);
-    const uint32_t w4 = w[4];
-    U4 mid;
-    mid.x = __builtin_amdgcn_alignbit(w03.y, w03.x, 16);
-    mid.y = __builtin_amdgcn_alignbit(w03.z, w03.y, 16);
-    mid.z = __builtin_amdgcn_alignbit(w03.w, w03.z, 16);
-    mid.w = __builtin_amdgcn_alignbit(w4, w03.w, 16);
-    U4 hi;
-    hi.x = w03.y; hi.y = w03.z; hi.z = w03.w; hi.w = w4;
-    T *out = col + static_cast<size_t>((ch * g.ky + a) * 3) * cstride + j0 + static_cast<size_t>(pk) * 8;
-    StreamStore16(out, w03);
-    StreamStore16(out + cstride, mid);
-    StreamStore16(out + 2 * static_cast<size_t>(cstride), hi);
-  }
-}
-
-/*! \brief The same copy with no staging at all, for dense images (binary16 or float) padded by one
- *  column on each side (ow == w): a thread makes the three packs (b = 0, 1, 2) of one place
+/*! \brief im2col with no staging at all, for three taps per row, stride 1, dilation 1 and dense
+ *  images (binary16 or float) padded by one column on each side (ow == w): a thread makes the three packs (b = 0, 1, 2) of one place
  *  (a, oy, a pack of columns) of one channel from the aligned pack of image row oy + a - pad_y
  *  and the element on either side of it, and stores them. A workgroup is 256 consecutive places of one (channel,
  *  a) pair - the three rows of the column matrix are contiguous over images and patch rows -
@@ -266,7 +175,7 @@ __global__ void __launch_bounds__(kPatchBlock)
  *  pieces, the form in which plain copies and fills run fastest here. The image is read
  *  ky times, the repeats from L2. MI355X, (32,256,56,56), pad 1: 92-94 us with the image
  *  coming from HBM and 78 us with the image in the memory-side cache, against 100-103 us
- *  and 86 us for the staged kernel above; two or four places per thread (PER) are slower
+ *  and 86 us for a kernel that staged a plane's rows in LDS; two or four places per thread (PER) are slower
  *  (111 / 115 us), as is one thread storing all nine packs that one image pack feeds (125 us). */
 const int kIm2ColDirectPer = 1;
 template <typename T, int PER>
@@ -593,126 +502,6 @@ __global__ void __launch_bounds__(kPatchBlock)
         }
       }
       dst[static_cast<size_t>(cyr) * istride + cx] = res;
-    }
-  }
-}
-
-/*! \brief col2im for binary16, stride 1, dilation 1 and a KY x KX window fixed at compile
- *  time (the convolution-backward case). Same tiling as Col2ImTiledKernel, with
- *   - the staging loads of all taps issued before any is parked in LDS (KY*KX 128-bit
- *     loads in flight per thread);
- *   - two adjacent pixels per thread, summed as a packed pair: adding two binary16 values
- *     in binary16 is the same as widening both to float, adding (exactly) and rounding
- *     back, which is what the reference's half_t operator+= does after every term
- *     (mshadow/half.h:58-62), so one packed add per tap replaces two conversions, an add
- *     and a rounding per pixel;
- *   - the taps unrolled in the reference's order (py ascending = a descending, then px
- *     ascending = b descending), a tap that does not exist for a pixel skipped by a
- *     16-bit-wise select. */
-template <int KY, int KX>
-__global__ void __launch_bounds__(kPatchBlock)
-    Col2ImHalfPairKernel(uint16_t *img, int istride, const uint16_t *col, int cstride, PatchGeom g,
-                         PatchTile t, mshadow::FastDivU32 div_wpairs) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  typedef uint16_t T;
-  typedef _Float16 H2 __attribute__((ext_vector_type(2)));
-  const int EPT = 8;
-  const int TAPS = KY * KX;
-  T *lds = reinterpret_cast<T *>(smem_raw);
-  int n, ch, band;
-  PlaneOfBlock(g, t, &n, &ch, &band);
-  const int plane = n * g.c + ch;
-  const int cy0 = band * t.band;
-  const int ncy = min(t.band, g.h - cy0);
-  const int yf = cy0 + g.pad_y, yl = cy0 + ncy - 1 + g.pad_y;
-  const int p0 = yf < KY ? 0 : yf - KY + 1;
-  const int p1 = min(yl + 1, g.oh);
-  const int npy = max(p1 - p0, 0);
-  const int run = npy * g.ow;
-  const size_t j0 = (static_cast<size_t>(n) * g.oh + p0) * g.ow;
-  const T *in0 = col + static_cast<size_t>(ch * TAPS) * cstride + j0;
-  const bool vec_ok = reinterpret_cast<uintptr_t>(in0) % 16 == 0 && cstride % EPT == 0;
-  if (vec_ok) {
-    for (int e0 = threadIdx.x * EPT; e0 < run; e0 += kPatchBlock * EPT) {
-      const bool whole = e0 + EPT <= run;
-      /* unpredicated: a partial last pack is fetched from its last whole position */
-      const int ec = whole ? e0 : max(run - EPT, 0);
-      U4 q[TAPS];
-      if (run >= EPT) {
-#pragma unroll
-        for (int tap = 0; tap < TAPS; ++tap) {
-          /* only whole packs can be fetched at an aligned address */
-          q[tap] = StreamLoad16(in0 + static_cast<size_t>(tap) * cstride + (whole ? ec : (ec / EPT) * EPT));
-        }
-      }
-#pragma unroll
-      for (int tap = 0; tap < TAPS; ++tap) {
-        T *out = lds + tap * t.pitch;
-        if (whole) {
-          *reinterpret_cast<U4 *>(out + e0) = q[tap];
-        } else {
-          const T *in = in0 + static_cast<size_t>(tap) * cstride;
-          for (int e = e0; e < run; ++e) out[e] = in[e];
-        }
-      }
-    }
-  } else {
-    for (int tap = 0; tap < TAPS; ++tap) {
-      const T *in = in0 + static_cast<size_t>(tap) * cstride;
-      T *out = lds + tap * t.pitch;
-      for (int e = threadIdx.x; e < run; e += kPatchBlock) out[e] = in[e];
-    }
-  }
-  __syncthreads();
-  T *dst = img + (static_cast<size_t>(plane) * g.h + cy0) * istride;
-  const int wpairs = (g.w + 1) / 2;
-  const int npairs = ncy * wpairs;
-  const bool store32 = istride % 2 == 0 && reinterpret_cast<uintptr_t>(img) % 4 == 0;
-  for (int idx = threadIdx.x; idx < npairs; idx += kPatchBlock) {
-    const int cyr = static_cast<int>(div_wpairs.Div(static_cast<uint32_t>(idx)));
-    const int cx = (idx - cyr * wpairs) * 2;
-    const int y = cy0 + cyr + g.pad_y;
-    const int x = cx + g.pad_x;
-    const bool second = cx + 1 < g.w;
-    /* per b: where the two pixels read (clamped into the row) and which of them exist */
-    int pxc[KX][2];
-    uint32_t keep[KX];
-#pragma unroll
-    for (int b = 0; b < KX; ++b) {
-      const int px0 = x - b, px1 = x + 1 - b;
-      const bool ok0 = px0 >= 0 && px0 < g.ow;
-      const bool ok1 = second && px1 >= 0 && px1 < g.ow;
-      pxc[b][0] = min(max(px0, 0), g.ow - 1);
-      pxc[b][1] = min(max(px1, 0), g.ow - 1);
-      keep[b] = (ok0 ? 0x0000ffffu : 0u) | (ok1 ? 0xffff0000u : 0u);
-    }
-    uint32_t res = 0u;  // two binary16 zeros
-#pragma unroll
-    for (int a = KY - 1; a >= 0; --a) {
-      const int py = y - a;
-      const bool row_ok = py >= 0 && py < g.oh;
-      const int rowbase = (min(max(py, p0), max(p1 - 1, p0)) - p0) * g.ow;
-#pragma unroll
-      for (int b = KX - 1; b >= 0; --b) {
-        const T *tap = lds + (a * KX + b) * t.pitch + rowbase;
-        const uint32_t v = static_cast<uint32_t>(tap[pxc[b][0]]) |
-                           (static_cast<uint32_t>(tap[pxc[b][1]]) << 16);
-        H2 acc, term;
-        __builtin_memcpy(&acc, &res, 4);
-        __builtin_memcpy(&term, &v, 4);
-        const H2 sum = acc + term;
-        uint32_t sbits;
-        __builtin_memcpy(&sbits, &sum, 4);
-        const uint32_t m = row_ok ? keep[b] : 0u;
-        res = (sbits & m) | (res & ~m);
-      }
-    }
-    T *out = dst + static_cast<size_t>(cyr) * istride + cx;
-    if (second && store32) {
-      *reinterpret_cast<uint32_t *>(out) = res;
-    } else {
-      out[0] = static_cast<T>(res & 0xffffu);
-      if (second) out[1] = static_cast<T>(res >> 16);
     }
   }
 }
