@@ -15,7 +15,8 @@ dominant operation (`roofline`: the kernel that takes the largest share of the s
 live inside the timed region). `per_op` lists each operation's own figures from a pass of
 the same K steps made just before, with an event after every launch (`ms`: the interval
 inside a step, a few microseconds of launch gap included) and from launches repeated back to
-back over rotating operand sets (`ms_back_to_back`). `cpu_baseline` times the reference CPU
+back over rotating operand sets (`ms_back_to_back`). `ms_per_step_graph_replay` is the step
+recorded once into a HIP graph and replayed. `cpu_baseline` times the reference CPU
 path (oracle/_ref, the reference's own headers) or, where that library is absent, the C
 restatement, on the host cores of the same machine over the same inputs.
 """
@@ -466,6 +467,32 @@ def main():
             b2b_ms[name] = G.elapsed_ms(ev[0], ev[1]) / reps
         use_set(0)
 
+    # A third figure for the step: the same launches recorded once into a HIP graph (one step per
+    # operand set) and replayed - what a caller that replays a fixed sequence pays per step.
+    graph_ms = None
+    if rotate and all(o in OPS for o in only):
+        try:
+            G.graph_begin(s)
+            for k in range(len(sets)):
+                use_set(k)
+                for name in only:
+                    run_op(name)
+            graph = G.graph_end(s)
+            replays = max(1, (args.steps + len(sets) - 1) // len(sets))
+            G.graph_launch(graph, s)          # warm-up
+            G.stream_sync(s)
+            gev = [G.event_create(), G.event_create()]
+            G.event_record(gev[0], s)
+            for _ in range(replays):
+                G.graph_launch(graph, s)
+            G.event_record(gev[1], s)
+            G.stream_sync(s)
+            graph_ms = G.elapsed_ms(gev[0], gev[1]) / (replays * len(sets))
+            G.graph_destroy(graph)
+        except Exception as e:  # noqa: BLE001 - the figure is an extra; the line must still come out
+            print(f"bench.py: graph replay skipped: {e}", file=sys.stderr)
+        use_set(0)
+
     abytes = algorithmic_bytes()
     elems = work_elements()
     scale_fix = 1.0 / args.scale
@@ -522,6 +549,8 @@ def main():
         "per_op": per_op,
         "input_generation_s": round(gen_s, 1),
     }
+    if graph_ms is not None:
+        out["ms_per_step_graph_replay"] = round(graph_ms, 4)
     if cpu is not None:
         out["cpu_baseline"] = {k: v for k, v in cpu.items() if k != "per_op_ms"}
     print(json.dumps(out))

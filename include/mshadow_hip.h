@@ -91,6 +91,19 @@ int mshadow_hip_event_record(void *event, void *stream);
 int mshadow_hip_event_sync(void *event);
 int mshadow_hip_event_elapsed_ms(void *start, void *stop, float *ms);
 
+/* A sequence of launches recorded once and replayed (the reference has nothing of the kind: it
+   launches kernel by kernel). Everything queued on `stream` between begin and end - launches of
+   this library and of kernels compiled with the caller alike - is recorded instead of run;
+   end hands back an executable graph that mshadow_hip_graph_launch queues on any stream of the
+   same device as often as wanted, with the pointers and shapes of the recording. While a stream
+   records, only launches and copies between device buffers may be queued on it: no allocation,
+   no synchronisation, no copy from or to pageable host memory, and none of the entry points
+   that allocate or wait (the sort entries, mshadow_hip_blas_*). `stream` must not be NULL. */
+int mshadow_hip_graph_begin(void *stream);
+int mshadow_hip_graph_end(void *stream, void **graph);
+int mshadow_hip_graph_launch(void *graph, void *stream);
+int mshadow_hip_graph_destroy(void *graph);
+
 /* AllocSpace / FreeSpace<gpu>: mshadow/tensor_gpu-inl.h:37-56 (cudaMallocPitch,
    cudaFree). pitch_bytes is a multiple of 256 when rows > 1. */
 int mshadow_hip_malloc_pitch(void **ptr, size_t *pitch_bytes, size_t width_bytes, size_t rows);

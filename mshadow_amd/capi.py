@@ -84,6 +84,10 @@ HIP_SYMBOLS = {
     "mshadow_hip_sort_by_key_workspace": ([_sz, C.POINTER(_sz)], _i),
     "mshadow_hip_sort_by_key_32": ([_p, _i, _p, _sz, _i, _p, _sz, _p], _i),
     "mshadow_hip_sort_by_key_32_noalloc": ([_p, _i, _p, _sz, _i, _p], _i),
+    "mshadow_hip_graph_begin": ([_p], _i),
+    "mshadow_hip_graph_end": ([_p, C.POINTER(C.c_void_p)], _i),
+    "mshadow_hip_graph_launch": ([_p, _p], _i),
+    "mshadow_hip_graph_destroy": ([_p], _i),
     "mshadow_hip_softmax_grad_f32": ([_p, _i, _p, _i, _p, _i, _i, _p], _i),
     "mshadow_hip_reduce_keep_lowest_f32": ([_p, _p, _i, _i, _i, _i, _i, _f, _p], _i),
     "mshadow_hip_reduce_keep_highdim_f32": ([_p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p], _i),
@@ -258,6 +262,21 @@ class Library:
 
     def device_sync(self):
         self.check(self.dll.mshadow_hip_device_sync())
+
+    # -- a sequence of launches recorded once and replayed
+    def graph_begin(self, stream):
+        self.check(self.dll.mshadow_hip_graph_begin(stream))
+
+    def graph_end(self, stream):
+        g = C.c_void_p()
+        self.check(self.dll.mshadow_hip_graph_end(stream, C.byref(g)))
+        return g
+
+    def graph_launch(self, graph, stream=None):
+        self.check(self.dll.mshadow_hip_graph_launch(graph, stream))
+
+    def graph_destroy(self, graph):
+        self.check(self.dll.mshadow_hip_graph_destroy(graph))
 
     def event_create(self):
         e = _p()

@@ -46,6 +46,9 @@ bool CopyRowsOnDevice(void *dst, size_t dpitch_bytes, const void *src, size_t sp
 
 /* a stream is going away: whatever scratch memory of the library it was given is free again */
 void ReleaseReduceScratch(void *stream);
+/* looks up, once per device, where the scratch slots of the split reductions live on the current
+   device (csrc/ops.hip) */
+void ResolveReduceScratch();
 
 }  // namespace mshadow_abi
 

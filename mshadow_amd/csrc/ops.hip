@@ -421,6 +421,25 @@ void ReleaseReduceScratch(void *stream) {
     }
   }
 }
+/* called when a device is selected: where the scratch array lives on that device is looked up
+   then, not inside the first reduction that wants a slot (which may be being recorded) */
+void ResolveReduceScratch() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kReduceScratchDevices) {
+    (void)hipGetLastError();
+    return;
+  }
+  ReduceScratchTable &t = ScratchTable();
+  std::lock_guard<std::mutex> lock(t.mu);
+  if (t.base[dev] == NULL) {
+    void *p = NULL;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_reduce_scratch)) == hipSuccess) {
+      t.base[dev] = static_cast<ReduceScratchSlot *>(p);
+    } else {
+      (void)hipGetLastError();
+    }
+  }
+}
 }  // namespace mshadow_abi
 
 extern "C" int mshadow_hip_reduce_scratch(void *stream, size_t words, uint32_t **partial,

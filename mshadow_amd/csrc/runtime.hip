@@ -53,6 +53,7 @@ int mshadow_hip_device_count(int *count) {
 int mshadow_hip_set_device(int device) {
   ABI_HIP(hipSetDevice(device));
   ResolveSortScratch();
+  ResolveReduceScratch();
   return MSHADOW_HIP_OK;
 }
 int mshadow_hip_get_device(int *device) {
@@ -110,6 +111,38 @@ int mshadow_hip_stream_query(void *stream, int *idle) {
   }
   *idle = 1;
   return FromHip(e, "hipStreamQuery");
+}
+
+int mshadow_hip_graph_begin(void *stream) {
+  ABI_REQUIRE(stream != NULL, "the default stream cannot record");
+  ABI_HIP(hipStreamBeginCapture(AsStream(stream), hipStreamCaptureModeThreadLocal));
+  return MSHADOW_HIP_OK;
+}
+
+int mshadow_hip_graph_end(void *stream, void **graph) {
+  ABI_REQUIRE(stream != NULL && graph != NULL, "NULL stream or result");
+  *graph = NULL;
+  hipGraph_t recorded = NULL;
+  ABI_HIP(hipStreamEndCapture(AsStream(stream), &recorded));
+  ABI_REQUIRE(recorded != NULL, "nothing was recorded");
+  hipGraphExec_t exec = NULL;
+  const hipError_t e = hipGraphInstantiate(&exec, recorded, NULL, NULL, 0);
+  (void)hipGraphDestroy(recorded);
+  ABI_HIP(e);
+  *graph = exec;
+  return MSHADOW_HIP_OK;
+}
+
+int mshadow_hip_graph_launch(void *graph, void *stream) {
+  ABI_REQUIRE(graph != NULL, "NULL graph");
+  ABI_HIP(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), AsStream(stream)));
+  return MSHADOW_HIP_OK;
+}
+
+int mshadow_hip_graph_destroy(void *graph) {
+  if (graph == NULL) return MSHADOW_HIP_OK;
+  ABI_HIP(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)));
+  return MSHADOW_HIP_OK;
 }
 
 int mshadow_hip_event_create(void **event) {
