@@ -993,6 +993,18 @@ int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstrid
 #undef UNPOOL_ROWS
     return AfterLaunch("unpool");
   }
+  /* 2 x 2 windows, stride 2: a pixel has one window at most; four pixels and two windows per thread */
+  if (ky == 2 && kx == 2 && sy == 2 && sx == 2 && w >= 4) {
+    const long long wpk = (w + 3) / 4;
+    const long long packs = static_cast<long long>(planes) * h * wpk;
+    if (packs + kPoolBlock < (1ll << 31)) {
+      const unsigned blocks = static_cast<unsigned>((packs + kPoolBlock - 1) / kPoolBlock);
+      POOL_SWITCH(Unpool2x2s2Kernel, dim3(blocks), dim3(kPoolBlock), 0, s, dst, dstride, src, sstride,
+                  pooled, pstride, grad, gstride, g, mshadow::FastDivU32(static_cast<uint32_t>(wpk)),
+                  mshadow::FastDivU32(static_cast<uint32_t>(h)), static_cast<uint32_t>(packs))
+      return AfterLaunch("unpool");
+    }
+  }
   /* small planes under a stride of 2 or more (a pixel has few windows): no staging. Measured on
      (128,256,28,28), 2x2 stride 2: 56 us against 96 us for the kernels below; on large planes or
      with stride 1 the staged kernels are faster. */

@@ -360,6 +360,68 @@ __global__ void __launch_bounds__(kPoolBlock)
   StreamStoreF4Anywhere(dst + static_cast<size_t>(r) * dstride + x0, out);
 }
 
+/*! \brief unpool for 2 x 2 windows with stride 2 - windows that do not overlap, so a source
+ *  pixel has at most one - with no staging: a thread takes four neighbouring source pixels of
+ *  one row (one 16-byte access each way, any alignment), which lie under two neighbouring windows of one pooled row, and fetches the
+ *  pooled values and gradients of those two as one 8-byte access each. The single term is
+ *  added to zero as the reference's loop does (mshadow/extension/spatial_unpool.h:102-125). */
+template <int REDUCER>
+__global__ void __launch_bounds__(kPoolBlock)
+    Unpool2x2s2Kernel(float *dst, int dstride, const float *src, int sstride, const float *pooled,
+                      int pstride, const float *grad, int gstride, PoolGeom g,
+                      mshadow::FastDivU32 div_wpk, mshadow::FastDivU32 div_h, uint32_t total_packs) {
+  typedef PoolOp<REDUCER> Op;
+  typedef F2 F2Loose __attribute__((aligned(4)));
+  const uint32_t pk = blockIdx.x * kPoolBlock + threadIdx.x;
+  if (pk >= total_packs) return;
+  const uint32_t r = div_wpk.Div(pk);                // plane * h + y
+  int x0 = static_cast<int>(pk - r * div_wpk.div) * 4;
+  /* the last pack of a row of even width is moved back to end with the row (it still starts a
+     window); of an odd width it is partial */
+  if (x0 + 4 > g.w && (g.w & 1) == 0) x0 = g.w - 4;
+  const uint32_t plane = div_h.Div(r);
+  const int y = static_cast<int>(r - plane * g.h);
+  const int py = y >> 1, px = x0 >> 1;
+  const float *in = src + static_cast<size_t>(r) * sstride + x0;
+  float *out = dst + static_cast<size_t>(r) * dstride + x0;
+  const int live = min(4, g.w - x0);                 // 4, or 3 when the width is odd
+  float vs[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (live == 4) {
+    const F4 q = StreamLoadF4Anywhere(in);
+    vs[0] = q.x; vs[1] = q.y; vs[2] = q.z; vs[3] = q.w;
+  } else {
+    for (int e = 0; e < live; ++e) vs[e] = in[e];
+  }
+  float pv[2] = {0.0f, 0.0f}, gv[2] = {0.0f, 0.0f};
+  const bool row_ok = py < g.ph;
+  if (row_ok) {
+    const float *prow = pooled + (static_cast<size_t>(plane) * g.ph + py) * pstride + px;
+    const float *grow = grad + (static_cast<size_t>(plane) * g.ph + py) * gstride + px;
+    if (px + 2 <= g.pw) {
+      const F2 a = *reinterpret_cast<const F2Loose *>(prow);
+      const F2 b = *reinterpret_cast<const F2Loose *>(grow);
+      pv[0] = a.x; pv[1] = a.y; gv[0] = b.x; gv[1] = b.y;
+    } else if (px < g.pw) {
+      pv[0] = prow[0];
+      gv[0] = grow[0];
+    }
+  }
+  float o[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const bool has = row_ok && px + (e >> 1) < g.pw;
+    const float t = 0.0f + Op::Grad(vs[e], pv[e >> 1]) * gv[e >> 1];
+    o[e] = has ? t : 0.0f;
+  }
+  if (live == 4) {
+    F4 q;
+    q.x = o[0]; q.y = o[1]; q.z = o[2]; q.w = o[3];
+    StreamStoreF4Anywhere(out, q);
+  } else {
+    for (int e = 0; e < live; ++e) out[e] = o[e];
+  }
+}
+
 /*! \brief unpool for small planes: a workgroup takes `per_block` whole consecutive planes, stages
  *  their pooled values and gradients (per_block * ph rows each) and computes every source pixel
  *  of those planes; a wave takes 64 / w source rows at a time when rows are short. Terms in

@@ -445,6 +445,9 @@ POOL_CASES = [  # planes, h, w, ky, kx, sy, sx, pad
     # many small planes: several per workgroup, the last workgroup with fewer
     (4096, 9, 9, 3, 3, 2, 2, 0), (2560, 13, 13, 3, 3, 2, 2, 1), (2500, 7, 10, 2, 2, 2, 2, 0),
     (3001, 12, 70, 3, 2, 1, 2, 2),
+    # 2 x 2 stride 2 on even and odd sizes, narrow and wide rows
+    (5, 40, 44, 2, 2, 2, 2, 3), (7, 41, 43, 2, 2, 2, 2, 0), (3, 9, 6, 2, 2, 2, 2, 1), (2, 8, 5, 2, 2, 2, 2, 0),
+    (2, 6, 258, 2, 2, 2, 2, 0),
 ]
 
 
