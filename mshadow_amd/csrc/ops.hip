@@ -972,21 +972,32 @@ int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstrid
               "too large for 32-bit indices");
   PoolGeom g = {h, w, ph, pw, ky, kx, sy, sx, 0, 0, pw};
   hipStream_t s = AsStream(stream);
-  /* 3 x 3 windows with stride 2 on rows of whole aligned packs: no staging */
-  if (ky == 3 && kx == 3 && sy == 2 && sx == 2 && h % 2 == 0 && w % 4 == 0 && w <= 256 && ph >= 1 &&
-      pw >= 1 && dstride % 4 == 0 && sstride % 4 == 0 && Aligned16(dst) && Aligned16(src)) {
+  /* 3 x 3 windows with stride 2 on rows of up to 256 pixels: no staging. Even heights and rows of
+     whole aligned packs take the plain form, everything else the one that moves packs anywhere */
+  if (ky == 3 && kx == 3 && sy == 2 && sx == 2 && w <= 256 && ph >= 1 && pw >= 1) {
+    const bool whole = h % 2 == 0 && w % 4 == 0 && dstride % 4 == 0 && sstride % 4 == 0 &&
+                       Aligned16(dst) && Aligned16(src);
     UnpoolRowsGeom rg;
-    rg.half_h = static_cast<uint32_t>(h / 2);
+    rg.half_h = static_cast<uint32_t>((h + 1) / 2);
     rg.total_rows = static_cast<uint32_t>(planes) * rg.half_h;
-    rg.groups = static_cast<uint32_t>(w / 4);
+    rg.groups = static_cast<uint32_t>((w + 3) / 4);
     rg.rows_per_wave = 64u / rg.groups;
     rg.div_groups = mshadow::FastDivU32(rg.groups);
     rg.div_half_h = mshadow::FastDivU32(rg.half_h);
+    rg.pooled_floats = (static_cast<size_t>(planes) * ph - 1) * pstride + pw;
+    rg.grad_floats = (static_cast<size_t>(planes) * ph - 1) * gstride + pw;
     const uint32_t waves = (rg.total_rows + rg.rows_per_wave - 1) / rg.rows_per_wave;
     const uint32_t blocks = (waves + kPoolBlock / 64 - 1) / (kPoolBlock / 64);
-#define UNPOOL_ROWS(R)                                                                         \
-  hipLaunchKernelGGL((UnpoolRows3x3s2Kernel<R>), dim3(blocks), dim3(kPoolBlock), 0, s, dst, dstride, \
-                     src, sstride, pooled, pstride, grad, gstride, g, rg)
+#define UNPOOL_ROWS(R)                                                                          \
+  do {                                                                                          \
+    if (whole) {                                                                                \
+      hipLaunchKernelGGL((UnpoolRows3x3s2Kernel<R, false>), dim3(blocks), dim3(kPoolBlock), 0, s, dst, \
+                         dstride, src, sstride, pooled, pstride, grad, gstride, g, rg);         \
+    } else {                                                                                    \
+      hipLaunchKernelGGL((UnpoolRows3x3s2Kernel<R, true>), dim3(blocks), dim3(kPoolBlock), 0, s, dst, \
+                         dstride, src, sstride, pooled, pstride, grad, gstride, g, rg);         \
+    }                                                                                           \
+  } while (0)
     if (reducer == MSHADOW_HIP_SUM) UNPOOL_ROWS(MSHADOW_HIP_SUM);
     else if (reducer == MSHADOW_HIP_MAX) UNPOOL_ROWS(MSHADOW_HIP_MAX);
     else UNPOOL_ROWS(MSHADOW_HIP_MIN);

@@ -360,6 +360,9 @@ __global__ void __launch_bounds__(kPoolBlock)
   StreamStoreF4Anywhere(dst + static_cast<size_t>(r) * dstride + x0, out);
 }
 
+/*! \brief two floats fetched as one 8-byte access at any 4-byte boundary */
+typedef F2 F2Loose __attribute__((aligned(4)));
+
 /*! \brief unpool for 2 x 2 windows with stride 2 - windows that do not overlap, so a source
  *  pixel has at most one - with no staging: a thread takes four neighbouring source pixels of
  *  one row (one 16-byte access each way, any alignment), which lie under two neighbouring windows of one pooled row, and fetches the
@@ -371,7 +374,6 @@ __global__ void __launch_bounds__(kPoolBlock)
                       int pstride, const float *grad, int gstride, PoolGeom g,
                       mshadow::FastDivU32 div_wpk, mshadow::FastDivU32 div_h, uint32_t total_packs) {
   typedef PoolOp<REDUCER> Op;
-  typedef F2 F2Loose __attribute__((aligned(4)));
   const uint32_t pk = blockIdx.x * kPoolBlock + threadIdx.x;
   if (pk >= total_packs) return;
   const uint32_t r = div_wpk.Div(pk);                // plane * h + y
@@ -609,19 +611,22 @@ __global__ void __launch_bounds__(kPoolBlock)
  *  `groups` = w / 4 lanes each */
 struct UnpoolRowsGeom {
   uint32_t total_rows, groups, rows_per_wave, half_h;
+  size_t pooled_floats, grad_floats;   // extent of the two pooled-size arrays, last row unpadded
   mshadow::FastDivU32 div_groups, div_half_h;
 };
 
-/*! \brief unpool for a 3 x 3 window with stride 2 on rows of whole aligned packs (h even,
- *  w a multiple of 4), with no staging: a thread owns two adjacent 2 x 2 blocks of source
- *  pixels - four pixels of row 2a and the four below them. The windows that can cover them
+/*! \brief unpool for a 3 x 3 window with stride 2 on rows of up to 256 pixels, with no staging:
+ *  a thread owns two adjacent 2 x 2 blocks of source pixels - four pixels of row 2a and the four
+ *  below them. RAGGED = false: h even, w a multiple of 4, rows of whole aligned packs. RAGGED =
+ *  true: any h and w at any alignment - the last pair of rows of an odd height has no lower row,
+ *  the last pack of a row that is not whole packs moves element by element. The windows that can cover them
  *  are rows a - 1 and a of the pooled grid, columns 2t - 1, 2t, 2t + 1: the thread fetches
  *  columns 2t and 2t + 1 of both rows (pooled value and gradient) and takes column 2t - 1
  *  from the neighbouring lane, which fetched it as its own 2t' + 1 (a wave takes whole rows).
  *  Source and result move as 128-bit accesses; nothing is staged and there is no barrier.
  *  Terms in the reference's order (py, then px ascending; mshadow/extension/
  *  spatial_unpool.h:102-125), a multiply and an add each. */
-template <int REDUCER>
+template <int REDUCER, bool RAGGED>
 __global__ void __launch_bounds__(kPoolBlock)
     UnpoolRows3x3s2Kernel(float *dst, int dstride, const float *src, int sstride, const float *pooled,
                           int pstride, const float *grad, int gstride, PoolGeom g, UnpoolRowsGeom rg) {
@@ -636,7 +641,26 @@ __global__ void __launch_bounds__(kPoolBlock)
   const uint32_t plane = rg.div_half_h.Div(browc);
   const int a = static_cast<int>(browc - plane * rg.half_h);
   const float *in = src + (static_cast<size_t>(plane) * g.h + 2 * a) * sstride + 4u * t;
-  const F4 top = StreamLoadF4(in), bottom = StreamLoadF4(in + sstride);
+  const int live_px = RAGGED ? min(4, g.w - static_cast<int>(4u * t)) : 4;
+  const bool has_bottom = !RAGGED || 2 * a + 1 < g.h;
+  F4 top, bottom;
+  if (!RAGGED) {
+    top = StreamLoadF4(in), bottom = StreamLoadF4(in + sstride);
+  } else {
+    top = bottom = F4{0.0f, 0.0f, 0.0f, 0.0f};
+    if (live_px == 4) {
+      top = StreamLoadF4Anywhere(in);
+      if (has_bottom) bottom = StreamLoadF4Anywhere(in + sstride);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 3; ++i) {
+        if (i < live_px) {
+          top[i] = StreamLoad(in + i);
+          if (has_bottom) bottom[i] = StreamLoad(in + sstride + i);
+        }
+      }
+    }
+  }
   /* [jy][c]: pooled row a - jy, column 2t - 1 + c */
   float pv[2][3], gv[2][3];
   bool ok[2][3];
@@ -645,16 +669,34 @@ __global__ void __launch_bounds__(kPoolBlock)
     const int py = a - jy;
     const bool row_ok = py >= 0 && py < g.ph;
     const size_t prow = static_cast<size_t>(plane) * g.ph + (row_ok ? py : 0);
-#pragma unroll
-    for (int e = 0; e < 2; ++e) {
-      const int px = static_cast<int>(2u * t) + e;
-      const bool col_ok = px < g.pw;
-      /* a window that does not exist re-reads an existing one and is skipped below */
-      const int pxc = col_ok ? px : 0;
-      pv[jy][e + 1] = pooled[prow * pstride + pxc];
-      gv[jy][e + 1] = grad[prow * gstride + pxc];
-      ok[jy][e + 1] = row_ok && col_ok;
+    /* columns 2t and 2t + 1 as one 8-byte access per array; a window that does not exist reads
+       an existing float (the next row's first at most) and is skipped below. Only the last
+       floats of the two arrays have nothing behind them: there the columns come one by one */
+    const int px = static_cast<int>(2u * t);
+    const int pxc = px < g.pw ? px : 0;
+    const size_t poff = prow * pstride + pxc, goff = prow * gstride + pxc;
+    /* pooled row a - 1 is row a' of the pair above, which the lanes `groups` below hold when
+       that pair is in this wave and plane */
+    const bool from_above = jy == 1 && row_in_wave > 0u && a > 0 && live;
+    if (from_above) {
+      pv[jy][1] = pv[jy][2] = gv[jy][1] = gv[jy][2] = 0.0f;
+    } else if (poff + 2 <= rg.pooled_floats && goff + 2 <= rg.grad_floats) {
+      const F2 pp = *reinterpret_cast<const F2Loose *>(pooled + poff);
+      const F2 gg = *reinterpret_cast<const F2Loose *>(grad + goff);
+      pv[jy][1] = pp.x, pv[jy][2] = pp.y;
+      gv[jy][1] = gg.x, gv[jy][2] = gg.y;
+    } else {
+      pv[jy][1] = pv[jy][2] = pooled[poff];
+      gv[jy][1] = gv[jy][2] = grad[goff];
     }
+    if (jy == 1) {
+      const int from = from_above ? static_cast<int>(lane - rg.groups) : static_cast<int>(lane);
+      const float p1 = __shfl(pv[0][1], from), p2 = __shfl(pv[0][2], from);
+      const float g1 = __shfl(gv[0][1], from), g2 = __shfl(gv[0][2], from);
+      if (from_above) pv[1][1] = p1, pv[1][2] = p2, gv[1][1] = g1, gv[1][2] = g2;
+    }
+    ok[jy][1] = row_ok && px < g.pw;
+    ok[jy][2] = row_ok && px + 1 < g.pw;
     /* column 2t - 1 is the neighbour's 2t' + 1 (every lane takes part in the exchange) */
     pv[jy][0] = __uint_as_float(static_cast<uint32_t>(__builtin_amdgcn_update_dpp(
         0, static_cast<int>(__float_as_uint(pv[jy][2])), 0x138, 0xf, 0xf, false)));
@@ -689,10 +731,25 @@ __global__ void __launch_bounds__(kPoolBlock)
   }
   float *out = dst + (static_cast<size_t>(plane) * g.h + 2 * a) * dstride + 4u * t;
   F4 q;
-  q.x = otop[0], q.y = otop[1], q.z = otop[2], q.w = otop[3];
-  StreamStoreF4(out, q);
-  q.x = obot[0], q.y = obot[1], q.z = obot[2], q.w = obot[3];
-  StreamStoreF4(out + dstride, q);
+  if (!RAGGED) {
+    q.x = otop[0], q.y = otop[1], q.z = otop[2], q.w = otop[3];
+    StreamStoreF4(out, q);
+    q.x = obot[0], q.y = obot[1], q.z = obot[2], q.w = obot[3];
+    StreamStoreF4(out + dstride, q);
+  } else if (live_px == 4) {
+    q.x = otop[0], q.y = otop[1], q.z = otop[2], q.w = otop[3];
+    StreamStoreF4Anywhere(out, q);
+    q.x = obot[0], q.y = obot[1], q.z = obot[2], q.w = obot[3];
+    if (has_bottom) StreamStoreF4Anywhere(out + dstride, q);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+      if (i < live_px) {
+        StreamStore(out + i, otop[i]);
+        if (has_bottom) StreamStore(out + dstride + i, obot[i]);
+      }
+    }
+  }
 }
 
 /*! \brief unpool without staging */

@@ -448,6 +448,9 @@ POOL_CASES = [  # planes, h, w, ky, kx, sy, sx, pad
     # 2 x 2 stride 2 on even and odd sizes, narrow and wide rows
     (5, 40, 44, 2, 2, 2, 2, 3), (7, 41, 43, 2, 2, 2, 2, 0), (3, 9, 6, 2, 2, 2, 2, 1), (2, 8, 5, 2, 2, 2, 2, 0),
     (2, 6, 258, 2, 2, 2, 2, 0),
+    # 3 x 3 stride 2 on odd heights, rows that are not whole packs, pitches, one to 64 packs per row
+    (96, 55, 55, 3, 3, 2, 2, 0), (40, 27, 27, 3, 3, 2, 2, 3), (5, 8, 5, 3, 3, 2, 2, 0), (3, 7, 256, 3, 3, 2, 2, 0),
+    (3, 6, 254, 3, 3, 2, 2, 1), (70, 3, 3, 3, 3, 2, 2, 0), (9, 14, 18, 3, 3, 2, 2, 2), (4, 5, 260, 3, 3, 2, 2, 0),
 ]
 
 
@@ -483,6 +486,27 @@ def test_pool_unpool(G, O, stream, case, reducer, variant):
         u2 = G.buffer((planes, h, w), f32)
         G.unpool(u2, dsrc, dpool, dgrad, ky, kx, sy, sx, reducer, stream)
         assert_bits_equal(u2.download(stream), wantu, "unpool abi")
+
+
+@pytest.mark.parametrize("shape", [(3, 9, 12, 3, 4), (3, 9, 12, 4, 5), (2, 10, 16, 2, 7), (2, 11, 13, 5, 3),
+                                   (4, 8, 8, 3, 3), (5, 6, 10, 2, 4)])
+@pytest.mark.parametrize("reducer", [MAX, SUM])
+def test_unpool_given_pooled_shape(G, O, stream, shape, reducer):
+    """unpool with a pooled grid the caller names (smaller than the natural one): only its windows count"""
+    planes, h, w, ph, pw = shape
+    for ky, kx, sy, sx in ((3, 3, 2, 2), (2, 2, 2, 2)):
+        if (ph - 1) * sy + ky > h or (pw - 1) * sx + kx > w:
+            continue
+        rng = np.random.default_rng(500 + h * w + ph)
+        src = rng.integers(-8, 9, (planes, h, w)).astype(f32) / f32(8)
+        pooled = np.empty((planes, ph, pw), f32)
+        O.pool(pooled, src, ky, kx, sy, sx, reducer)
+        grad = normal(73, (planes, ph, pw))
+        want = np.empty((planes, h, w), f32)
+        O.unpool(want, src, pooled, grad, ky, kx, sy, sx, reducer)
+        out = G.buffer((planes, h, w), f32)
+        G.unpool(out, G.to_device(src), G.to_device(pooled), G.to_device(grad), ky, kx, sy, sx, reducer, stream)
+        assert_bits_equal(out.download(stream), want, f"unpool {shape} k{ky} s{sy}")
 
 
 def test_pool_reference_known_answers(G, stream):
