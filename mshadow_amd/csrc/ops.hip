@@ -850,6 +850,23 @@ int mshadow_hip_reduce_keep_highdim_f32(float *dst, const float *src, int sstrid
 static const size_t kPoolLdsBudget = 48 * 1024;  // per workgroup: three resident per CU
 static const size_t kUnpoolLdsBudget = 16 * 1024;  // smaller bands: more workgroups in different phases per CU
 
+/*! \brief strips of the stride-1 unpool kernel over `rows` rows of `w` columns per plane:
+ *  sixteen rows a strip, fewer while that leaves the machine short of waves */
+static SlideGeom MakeSlideGeom(int planes, int rows, int w) {
+  SlideGeom sg;
+  sg.groups = static_cast<uint32_t>((w + 3) / 4);
+  sg.strips_per_wave = 64u / sg.groups;
+  uint32_t r = 16;
+  const long long want = 16ll * mshadow_abi::ComputeUnits();  // waves
+  while (r > 2 && static_cast<long long>(planes) * ((rows + r - 1) / r) / sg.strips_per_wave < want) r /= 2;
+  sg.strip_rows = r;
+  sg.strips_per_plane = static_cast<uint32_t>((rows + r - 1) / r);
+  sg.total_strips = static_cast<uint32_t>(planes) * sg.strips_per_plane;
+  sg.div_groups = mshadow::FastDivU32(sg.groups);
+  sg.div_spp = mshadow::FastDivU32(sg.strips_per_plane);
+  return sg;
+}
+
 int mshadow_hip_pool_f32(float *dst, int dstride, const float *src, int sstride, int planes,
                          int h, int w, int ph, int pw, int ky, int kx, int sy, int sx,
                          int reducer, void *stream) {
@@ -1002,6 +1019,33 @@ int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstrid
     else if (reducer == MSHADOW_HIP_MAX) UNPOOL_ROWS(MSHADOW_HIP_MAX);
     else UNPOOL_ROWS(MSHADOW_HIP_MIN);
 #undef UNPOOL_ROWS
+    return AfterLaunch("unpool");
+  }
+  /* 2 x 2 and 3 x 3 windows with stride 1 on planes of 64 to 256 pixels a side: no staging, the
+     pooled rows over the current source row in registers ((128,64,112,112): 368 us against 513 us
+     for the kernels below; on planes of 57 x 57 the two are level, below that the staged ones win) */
+  if (ky == kx && (ky == 2 || ky == 3) && sy == 1 && sx == 1 && w >= 64 && w <= 256 && h >= 64 && ph >= 1 && pw >= 1 &&
+      static_cast<long long>(planes) * ph * pw >= 4 && static_cast<long long>(planes) * ((h + 1) / 2) < (1ll << 31)) {
+    SlideGeom sg = MakeSlideGeom(planes, h, w);
+    sg.src_floats = (static_cast<size_t>(planes) * h - 1) * sstride + w;
+    sg.pooled_floats = (static_cast<size_t>(planes) * ph - 1) * pstride + pw;
+    sg.grad_floats = (static_cast<size_t>(planes) * ph - 1) * gstride + pw;
+    const uint32_t waves = (sg.total_strips + sg.strips_per_wave - 1) / sg.strips_per_wave;
+    const uint32_t blocks = (waves + kPoolBlock / 64 - 1) / (kPoolBlock / 64);
+#define UNPOOL_SLIDE(R)                                                                        \
+  do {                                                                                         \
+    if (ky == 2) {                                                                             \
+      hipLaunchKernelGGL((UnpoolSlideS1Kernel<R, 2, 4>), dim3(blocks), dim3(kPoolBlock), 0, s, dst, dstride, \
+                         src, sstride, pooled, pstride, grad, gstride, g, sg);                 \
+    } else {                                                                                   \
+      hipLaunchKernelGGL((UnpoolSlideS1Kernel<R, 3, 3>), dim3(blocks), dim3(kPoolBlock), 0, s, dst, dstride, \
+                         src, sstride, pooled, pstride, grad, gstride, g, sg);                 \
+    }                                                                                          \
+  } while (0)
+    if (reducer == MSHADOW_HIP_SUM) UNPOOL_SLIDE(MSHADOW_HIP_SUM);
+    else if (reducer == MSHADOW_HIP_MAX) UNPOOL_SLIDE(MSHADOW_HIP_MAX);
+    else UNPOOL_SLIDE(MSHADOW_HIP_MIN);
+#undef UNPOOL_SLIDE
     return AfterLaunch("unpool");
   }
   /* 2 x 2 windows, stride 2: a pixel has one window at most; four pixels and two windows per thread */

@@ -752,6 +752,181 @@ __global__ void __launch_bounds__(kPoolBlock)
   }
 }
 
+/*! \brief geometry of the stride-1 kernels below: a plane is cut into strips of `strip_rows`
+ *  rows; a strip is `groups` = ceil(w / 4) lanes wide and a wave takes `strips_per_wave`
+ *  consecutive strips (plane after plane), whole rows each */
+struct SlideGeom {
+  uint32_t groups, strips_per_wave, strip_rows, strips_per_plane, total_strips;
+  mshadow::FastDivU32 div_groups, div_spp;
+  size_t src_floats, pooled_floats, grad_floats;  //!< extent of each input, last row unpadded (4 or more)
+};
+
+/*! \brief the four floats at `p` as one 16-byte access at any alignment, with no branch around
+ *  the load (a loop that keeps several rows on their way needs every path to issue the same
+ *  loads, or the compiler waits for all of them at every use). Where `ok` is false the pack is
+ *  fetched from `base` instead and means nothing. Only the last pack of a tensor's last row can
+ *  reach past the tensor's end (`end`: one past its last float): it is fetched from end - 4 and
+ *  its elements are moved into place, zeros behind them. Floats past the end of a ROW are the
+ *  next row's and are the caller's to ignore or mask. */
+__device__ __forceinline__ F4 LoadPackFree(const float *base, const float *p, const float *end, bool ok) {
+  const float *last = end - 4;
+  const bool moved = ok && p > last;
+  const float *at = ok ? (moved ? last : p) : base;
+  F4 q = StreamLoadF4Anywhere(at);
+  if (__any(moved)) {  // one wave of the grid at most
+    const int sh = moved ? static_cast<int>(p - last) : 0;
+    F4 b, c;
+    b[0] = (sh & 1) ? q[1] : q[0];
+    b[1] = (sh & 1) ? q[2] : q[1];
+    b[2] = (sh & 1) ? q[3] : q[2];
+    b[3] = (sh & 1) ? 0.0f : q[3];
+    c[0] = (sh & 2) ? b[2] : b[0];
+    c[1] = (sh & 2) ? b[3] : b[1];
+    c[2] = (sh & 2) ? 0.0f : b[2];
+    c[3] = (sh & 2) ? 0.0f : b[3];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) q[e] = sh >= 4 ? 0.0f : c[e];
+  }
+  return q;
+}
+/*! \brief q with zeros in the columns from n on (and everywhere unless ok) */
+__device__ __forceinline__ F4 KeepColumns(F4 q, int x0, int n, bool ok) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) q[e] = (ok && x0 + e < n) ? q[e] : 0.0f;
+  return q;
+}
+
+/*! \brief value of v in the lane below; lane 0 receives 0 */
+__device__ __forceinline__ float FromLaneBelow(float v) {
+  return __uint_as_float(static_cast<uint32_t>(
+      __builtin_amdgcn_update_dpp(0, static_cast<int>(__float_as_uint(v)), 0x138, 0xf, 0xf, false)));
+}
+
+/*! \brief unpool for K x K windows with stride 1 (K = 2, 3) on rows of up to 256 pixels, with no
+ *  staging. A pixel lies under up to K * K windows, so a thread that took its pooled values from
+ *  memory pixel by pixel would fetch every one of them K * K times. Here a thread owns four
+ *  adjacent pixels and walks down a strip of rows with the K pooled rows that cover the current
+ *  source row in registers: per source row it fetches one pack of the source, one of the pooled
+ *  values and one of the gradients (the new pooled row; the K - 1 columns to the left of its own
+ *  four come from the neighbouring lane, which holds them as its own), computes its four pixels
+ *  from the K x (K + 3) windows it holds, and stores one pack. Every byte is fetched once apart
+ *  from the K - 1 pooled rows on top of a strip; DEPTH rows are on their way while one is
+ *  computed. The loop is unrolled DEPTH times (a multiple of K), so the K window rows are a ring
+ *  of registers with fixed places: pooled row py sits in ring row (py - y0) mod K.
+ *
+ *  The kernel is bound by its arithmetic (K * K terms per pixel), so a term is three
+ *  instructions: the reference adds PartialGrad(src, pooled) * grad, a product that is grad
+ *  where the two are equal and 0 * grad where not (a zero with grad's sign, NaN for an infinite
+ *  grad); Z = 0 * grad is made once per gradient fetched and the term is picked from (grad, Z).
+ *  Windows that do not exist (outside the pooled grid) are held as gradient 0: their term is
+ *  +0, and adding a zero never changes the sum, which starts at +0 and so is never -0. The terms
+ *  are added in the reference's order (py, then px ascending; mshadow/extension/
+ *  spatial_unpool.h:102-125). */
+template <int REDUCER, int K, int DEPTH>
+__global__ void __launch_bounds__(kPoolBlock)
+    UnpoolSlideS1Kernel(float *dst, int dstride, const float *src, int sstride, const float *pooled,
+                        int pstride, const float *grad, int gstride, PoolGeom g, SlideGeom sg) {
+  static_assert(DEPTH % K == 0, "the ring of window rows must close within one unrolled turn");
+  const int WIN = K + 3;  // window columns x0 - (K - 1) .. x0 + 3
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = blockIdx.x * (kPoolBlock / 64) + (threadIdx.x >> 6);
+  const uint32_t sub = sg.div_groups.Div(lane);
+  const uint32_t t = lane - sub * sg.groups;
+  const uint32_t strip = wave * sg.strips_per_wave + sub;
+  const bool live = sub < sg.strips_per_wave && strip < sg.total_strips;
+  const uint32_t stripc = live ? strip : sg.total_strips - 1u;
+  const uint32_t plane = sg.div_spp.Div(stripc);
+  const int y0 = static_cast<int>((stripc - plane * sg.strips_per_plane) * sg.strip_rows);
+  const int x0 = static_cast<int>(4u * t);
+  const float *pbase = pooled + static_cast<size_t>(plane) * g.ph * pstride;
+  const float *gbase = grad + static_cast<size_t>(plane) * g.ph * gstride;
+  const float *sbase = src + static_cast<size_t>(plane) * g.h * sstride;
+  float *dbase = dst + static_cast<size_t>(plane) * g.h * dstride;
+  const float *send = src + sg.src_floats, *pend = pooled + sg.pooled_floats, *gend = grad + sg.grad_floats;
+  float P[K][WIN], G[K][WIN], Z[K][WIN];
+  /* a pooled row takes its place in the ring (every lane of the wave takes part) */
+#define MSHADOW_SLIDE_PUT(SLOT, pq, gq)                                     \
+  {                                                                         \
+    _Pragma("unroll") for (int e = 0; e < 4; ++e) {                         \
+      P[SLOT][K - 1 + e] = (pq)[e];                                         \
+      G[SLOT][K - 1 + e] = (gq)[e];                                         \
+    }                                                                       \
+    _Pragma("unroll") for (int i = 0; i + 1 < K; ++i) {                     \
+      const float pl = FromLaneBelow(P[SLOT][4 + i]);                       \
+      const float gl = FromLaneBelow(G[SLOT][4 + i]);                       \
+      P[SLOT][i] = pl;                                                      \
+      G[SLOT][i] = t == 0u ? 0.0f : gl;                                     \
+    }                                                                       \
+    _Pragma("unroll") for (int i = 0; i < WIN; ++i) Z[SLOT][i] = 0.0f * G[SLOT][i]; \
+  }
+  /* the K - 1 pooled rows above the strip's first source row: row y0 - k in ring row K - k */
+#pragma unroll
+  for (int k = K - 1; k >= 1; --k) {
+    const int py = y0 - k;
+    const bool ok = live && py >= 0 && py < g.ph;
+    const F4 pq = LoadPackFree(pbase, pbase + static_cast<ptrdiff_t>(py) * pstride + x0, pend, ok);
+    const F4 gq = KeepColumns(LoadPackFree(gbase, gbase + static_cast<ptrdiff_t>(py) * gstride + x0, gend, ok),
+                              x0, g.pw, ok);
+    MSHADOW_SLIDE_PUT(K - k, pq, gq)
+  }
+  const int rows = static_cast<int>(sg.strip_rows);  // the same for every lane of the wave
+  F4 sq[DEPTH], pq[DEPTH], gq[DEPTH];
+  bool okq[DEPTH];
+#pragma unroll
+  for (int u = 0; u < DEPTH; ++u) {
+    const int y = y0 + u;
+    okq[u] = live && u < rows && y < g.h;
+    const bool pok = okq[u] && y < g.ph;
+    sq[u] = LoadPackFree(sbase, sbase + static_cast<size_t>(y) * sstride + x0, send, okq[u]);
+    pq[u] = LoadPackFree(pbase, pbase + static_cast<size_t>(y) * pstride + x0, pend, pok);
+    gq[u] = KeepColumns(LoadPackFree(gbase, gbase + static_cast<size_t>(y) * gstride + x0, gend, pok), x0, g.pw, pok);
+  }
+  for (int r0 = 0; r0 < rows; r0 += DEPTH) {
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) {
+      const int r = r0 + u;
+      if (r >= rows) break;  // the same for every lane
+      const int y = y0 + r;
+      const F4 cur = sq[u];
+      const bool cur_ok = okq[u];
+      MSHADOW_SLIDE_PUT(u % K, pq[u], gq[u])
+      const int yn = y + DEPTH;
+      okq[u] = live && r + DEPTH < rows && yn < g.h;
+      const bool pok = okq[u] && yn < g.ph;
+      sq[u] = LoadPackFree(sbase, sbase + static_cast<size_t>(yn) * sstride + x0, send, okq[u]);
+      pq[u] = LoadPackFree(pbase, pbase + static_cast<size_t>(yn) * pstride + x0, pend, pok);
+      gq[u] = KeepColumns(LoadPackFree(gbase, gbase + static_cast<size_t>(yn) * gstride + x0, gend, pok), x0, g.pw, pok);
+      F4 out;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float val = 0.0f;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {      // py = y - (K - 1) + k, in ring row (u + 1 + k) % K
+          const int slot = (u + 1 + k) % K;
+#pragma unroll
+          for (int j = 0; j < K; ++j) {    // px = x - (K - 1) + j
+            const bool hit = REDUCER == MSHADOW_HIP_SUM || cur[e] == P[slot][e + j];
+            val = val + (hit ? G[slot][e + j] : Z[slot][e + j]);
+          }
+        }
+        out[e] = val;
+      }
+      if (cur_ok) {
+        float *orow = dbase + static_cast<size_t>(y) * dstride + x0;
+        if (x0 + 4 <= g.w) {
+          StreamStoreF4Anywhere(orow, out);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 3; ++e) {
+            if (x0 + e < g.w) StreamStore(orow + e, out[e]);
+          }
+        }
+      }
+    }
+  }
+#undef MSHADOW_SLIDE_PUT
+}
+
 /*! \brief unpool without staging */
 template <int REDUCER>
 __global__ void __launch_bounds__(kPoolBlock)

@@ -451,6 +451,12 @@ POOL_CASES = [  # planes, h, w, ky, kx, sy, sx, pad
     # 3 x 3 stride 2 on odd heights, rows that are not whole packs, pitches, one to 64 packs per row
     (96, 55, 55, 3, 3, 2, 2, 0), (40, 27, 27, 3, 3, 2, 2, 3), (5, 8, 5, 3, 3, 2, 2, 0), (3, 7, 256, 3, 3, 2, 2, 0),
     (3, 6, 254, 3, 3, 2, 2, 1), (70, 3, 3, 3, 3, 2, 2, 0), (9, 14, 18, 3, 3, 2, 2, 2), (4, 5, 260, 3, 3, 2, 2, 0),
+    # stride 1, 3 x 3 and 2 x 2. Planes of 64 to 256 pixels a side: strips of rows (16 to 64 packs per row, planes
+    # that end inside a strip, rows that end inside a pack, pitches); smaller and wider ones: the staged kernels
+    (16, 112, 112, 3, 3, 1, 1, 0), (6, 70, 67, 3, 3, 1, 1, 2), (3, 65, 256, 3, 3, 1, 1, 0), (4, 80, 130, 2, 2, 1, 1, 0),
+    (2, 64, 64, 2, 2, 1, 1, 3), (700, 64, 66, 3, 3, 1, 1, 1), (5, 97, 201, 3, 3, 1, 1, 0),
+    (6, 37, 41, 3, 3, 1, 1, 2), (5, 20, 256, 3, 3, 1, 1, 0), (7, 9, 4, 3, 3, 1, 1, 0), (3, 5, 7, 2, 2, 1, 1, 1),
+    (2560, 13, 13, 3, 3, 1, 1, 0), (3, 66, 260, 3, 3, 1, 1, 0), (300, 28, 28, 3, 3, 1, 1, 3),
 ]
 
 
@@ -489,12 +495,12 @@ def test_pool_unpool(G, O, stream, case, reducer, variant):
 
 
 @pytest.mark.parametrize("shape", [(3, 9, 12, 3, 4), (3, 9, 12, 4, 5), (2, 10, 16, 2, 7), (2, 11, 13, 5, 3),
-                                   (4, 8, 8, 3, 3), (5, 6, 10, 2, 4)])
+                                   (4, 8, 8, 3, 3), (5, 6, 10, 2, 4), (2, 70, 72, 60, 66), (3, 64, 100, 31, 97)])
 @pytest.mark.parametrize("reducer", [MAX, SUM])
 def test_unpool_given_pooled_shape(G, O, stream, shape, reducer):
     """unpool with a pooled grid the caller names (smaller than the natural one): only its windows count"""
     planes, h, w, ph, pw = shape
-    for ky, kx, sy, sx in ((3, 3, 2, 2), (2, 2, 2, 2)):
+    for ky, kx, sy, sx in ((3, 3, 2, 2), (2, 2, 2, 2), (3, 3, 1, 1), (2, 2, 1, 1)):
         if (ph - 1) * sy + ky > h or (pw - 1) * sx + kx > w:
             continue
         rng = np.random.default_rng(500 + h * w + ph)
