@@ -891,9 +891,16 @@ int mshadow_hip_pool_f32(float *dst, int dstride, const float *src, int sstride,
   while (band > 8 && static_cast<long long>(planes) * ((ph + band - 1) / band) < 1024) {
     band = (band + 1) / 2;
   }
-  if (band >= 1) {  // equal-sized bands; about 24 KB of LDS each keeps several resident per CU
+  if (band >= 1) {
+    /* equal-sized bands of about 20 KB of input rows (but four output rows or more): seven or
+       eight workgroups then share a CU, and while some wait at their barrier others load.
+       (32,64,224,224) 2x2 stride 2: 80 us against 102 us with bands of 41 KB; 14 KB and less
+       lose again to the rows that neighbouring bands both read. */
     long long nb = (ph + band - 1) / band;
-    if (band * static_cast<long long>(sy) * row_bytes > 24 * 1024 && nb < 2 && ph >= 16) nb = 2;
+    const long long target = 20 * 1024;
+    const long long want = (static_cast<long long>(ph) * sy * row_bytes + target - 1) / target;
+    if (want > nb) nb = want;
+    if (nb > ph / 4 && ph >= 4) nb = ph / 4;
     band = (ph + nb - 1) / nb;
   }
 #define POOL_SWITCH(KERNEL, ...)                                                               \
