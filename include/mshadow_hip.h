@@ -160,7 +160,7 @@ int mshadow_hip_softmax_f32(float *dst, int dstride, const float *src, int sstri
 /* The row-sum stage of Softmax on its own: sums[r] = the float32 sum of the cols
    non-negative terms of row r added left to right into one accumulator, exactly as the
    loop at mshadow/tensor_cpu-inl.h:277-281 accumulates exp(energy - max). Runs the same
-   device code as mshadow_hip_softmax_f32 (rows of up to 65536 terms) and exists so that
+   device code as mshadow_hip_softmax_f32 (rows of any length) and exists so that
    this stage can be compared bit for bit with a serial sum, which the full operation
    does not allow because the device exponential differs from libm's. */
 int mshadow_hip_softmax_rowsum_f32(float *sums, const float *terms, int tstride, int rows,

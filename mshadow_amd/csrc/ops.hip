@@ -518,8 +518,16 @@ int mshadow_hip_softmax_f32(float *dst, int dstride, const float *src, int sstri
   else if (cols <= 16384) SOFTMAX_LAUNCH(512, 8, 4);
   else if (cols <= 32768) SOFTMAX_LAUNCH(512, 16, 4);
   else if (cols <= 65536) SOFTMAX_LAUNCH(1024, 16, 4);
-  else hipLaunchKernelGGL((SoftmaxLongRowKernel<1024>), dim3(rows), dim3(1024), 0, s, dst,
-                          dstride, src, sstride, cols);
+  /* longer rows: stretches of 32768 columns on 512 threads, two rows to a CU ((512,128000): 221 us
+     against 271 us with stretches of 65536 on 1024 threads; up to 65536 columns the single pass
+     above is faster than stretches, 265 against 432 us on (2048,50257)) */
+  else if (rows > mshadow_abi::ComputeUnits()) {
+    hipLaunchKernelGGL((SoftmaxStretchRowKernel<512, 16, false, 4>), dim3(rows), dim3(512), 0, s, dst,
+                       dstride, src, sstride, cols);
+  } else {
+    hipLaunchKernelGGL((SoftmaxStretchRowKernel<512, 16, false, 2>), dim3(rows), dim3(512), 0, s, dst,
+                       dstride, src, sstride, cols);
+  }
 #undef SOFTMAX_LAUNCH
   return AfterLaunch("softmax");
 }
@@ -530,7 +538,6 @@ int mshadow_hip_softmax_rowsum_f32(float *sums, const float *terms, int tstride,
   if (rows == 0) return MSHADOW_HIP_OK;
   ABI_REQUIRE(sums != NULL && (terms != NULL || cols == 0), "NULL tensor");
   ABI_REQUIRE(tstride >= cols, "pitch smaller than the row");
-  ABI_REQUIRE(cols <= 65536, "row longer than the register-resident softmax kernels take");
   hipStream_t s = AsStream(stream);
   if (cols <= 256) {
     LaunchShortSoftmax<true>(sums, 0, terms, tstride, rows, cols, s);
@@ -547,6 +554,12 @@ int mshadow_hip_softmax_rowsum_f32(float *sums, const float *terms, int tstride,
     return AfterLaunch("softmax_rowsum");
   }
   const bool vec = Aligned16(terms) && tstride % 4 == 0 && cols % 4 == 0;
+  /* rows longer than a workgroup's registers hold: stretch by stretch, at any alignment */
+  if (cols > 65536 || (!vec && cols > 32768)) {
+    hipLaunchKernelGGL((SoftmaxStretchRowKernel<512, 16, true, 2>), dim3(rows), dim3(512), 0, s, sums, 0,
+                       terms, tstride, cols);
+    return AfterLaunch("softmax_rowsum");
+  }
 #define ROWSUM_LAUNCH(T, S, V) \
   hipLaunchKernelGGL((SoftmaxRowKernel<T, S, V, true>), dim3(rows), dim3(T), 0, s, sums, 0, terms, \
                      tstride, cols)
@@ -559,7 +572,6 @@ int mshadow_hip_softmax_rowsum_f32(float *sums, const float *terms, int tstride,
     else if (cols <= 32768) ROWSUM_LAUNCH(512, 16, 4);
     else ROWSUM_LAUNCH(1024, 16, 4);
   } else {
-    ABI_REQUIRE(cols <= 32768, "unaligned rows longer than 32768 terms are not register-resident");
     if (cols <= 1024) ROWSUM_LAUNCH(256, 4, 1);
     else if (cols <= 4096) ROWSUM_LAUNCH(256, 16, 1);
     else if (cols <= 16384) ROWSUM_LAUNCH(1024, 16, 1);

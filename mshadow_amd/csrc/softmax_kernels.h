@@ -12,8 +12,8 @@
  *      for bit, what mshadow/tensor_cpu-inl.h:277-281 computes from the same p;
  *   4. p / sum (reciprocal and one correction step), 128-bit stores.
  * dst may alias src (every element is read before the row is written).
- * SoftmaxLongRowKernel covers rows too long for registers with the same arithmetic,
- * staging p through dst. SoftmaxGradKernel is a 128-bit copy with one element per row
+ * SoftmaxStretchRowKernel covers rows too long for registers with the same arithmetic,
+ * stretch by stretch. SoftmaxGradKernel is a 128-bit copy with one element per row
  * decremented (mshadow/tensor_cpu-inl.h:287-302).
  */
 #ifndef MSHADOW_AMD_CSRC_SOFTMAX_KERNELS_H_
@@ -49,15 +49,6 @@ __device__ __forceinline__ float MaxNum3(float a, float b, float c) {
   return r;
 }
 
-/*! \brief LDS scratch of the ordered sum: two alternating sets of per-wave totals and
- *  the hand-over slot for the running sum */
-template <int WAVES>
-struct OrderedSumLds {
-  float q[2][WAVES];
-  float s;
-  float wmax[WAVES];
-};
-
 /*! \brief one wave adds its 64 * N terms (lane order, then element order) to s exactly
  *  as a serial loop would; called only for the wave in which a chunk was rejected */
 template <int N>
@@ -82,45 +73,6 @@ __device__ inline float WaveResolve(float s, const float (&t)[N]) {
   }
 }
 
-/*! \brief block-wide: add one slab (THREADS * N consecutive terms, thread-major) to s.
- *  s is uniform over the block on entry and on exit. `buf` alternates the LDS slot. */
-template <int THREADS, int N>
-__device__ inline float BlockOrderedAdd(float s, const float (&t)[N],
-                                        OrderedSumLds<THREADS / kWave> *lds, int *buf) {
-  using namespace ordered_sum;
-  const int W = THREADS / kWave;
-  const int wave = WaveId();
-  const int lane = LaneId();
-  int pos = 0;  // waves before pos are already in s
-  while (true) {
-    const Binade b = BinadeOf(s);
-    if (wave >= pos) {
-      const float q = ReadLaneF32(WaveInclusiveScanF32(LaneQuant<N>(t, b)), kWave - 1);
-      if (lane == 0) lds->q[*buf][wave] = q;
-    }
-    __syncthreads();
-    /* the per-wave totals are scanned across lanes (lane w holds wave w's total): the
-       first wave whose inclusive prefix leaves the binade is the one to resolve */
-    const float qv = (lane < W && lane >= pos) ? lds->q[*buf][lane] : 0.0f;
-    const float incl = WaveInclusiveScanF32(qv);
-    const bool over = lane < W && lane >= pos && !Fits(b, incl);
-    const unsigned long long mask = __ballot(over);
-    const int failw = mask ? __ffsll(mask) - 1 : W;
-    const float acc = failw > 0 ? ReadLaneF32(incl, failw - 1) : 0.0f;
-    *buf ^= 1;
-    s = Accept(s, b, acc);
-    if (failw == W) return s;
-    if (wave == failw) {
-      const float r = WaveResolve<N>(s, t);
-      if (lane == 0) lds->s = r;
-    }
-    __syncthreads();
-    s = lds->s;
-    pos = failw + 1;
-    if (pos == W) return s;
-  }
-}
-
 /* ---- planned row sum (registers hold the whole row) ---------------------------------
  * Thread layout: chunk k of the row (64 * N consecutive terms, lane-major) is slab k / W of
  * wave k % W, so the W waves walk the row side by side and the chunks next to the row's
@@ -135,7 +87,9 @@ __device__ inline float BlockOrderedAdd(float s, const float (&t)[N],
  *      the run of certain chunks in front of each listed chunk as one more addend  (barrier)
  *   E  wave 0: the chain - the row's addends summed serially, every run verified  (barrier)
  * A row whose plan fails a verification, or that has more listed chunks than slots, is summed
- * by wave scans instead, chunk after chunk.
+ * by wave scans instead, chunk after chunk. The sum may start from s0 instead of zero (a row
+ * longer than the registers hold is summed stretch by stretch): s0 then stands in front of the
+ * approximate prefix sums and is where the chain begins.
  * Lane l keeps the chunk-table entries of chunks l * CPL .. l * CPL + CPL - 1. */
 /*! \brief chunks per row that can hand a list of addends to the chain (a row of softmax
  *  terms has about a dozen) */
@@ -281,7 +235,7 @@ __device__ __forceinline__ float ChainBlock(float s, float addend, uint32_t chec
 
 template <int THREADS, int SLABS, int N, bool CHECK_SIGN, bool UNIT_PEAK>
 __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
-                                      RowSumLds<THREADS / kWave, SLABS, N> *lds) {
+                                      RowSumLds<THREADS / kWave, SLABS, N> *lds, float s0 = 0.0f) {
   using namespace ordered_sum;
   using mshadow::hip::ReadLaneU32;
   using mshadow::hip::WaveInclusiveScanU32;
@@ -380,7 +334,7 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
     const float excl = incl - pre[CPL];
     const float approx_total = ReadLaneF32(incl, kWave - 1);
     /* a NaN among the terms makes the sum NaN whatever the order */
-    if (approx_total != approx_total) return approx_total;
+    if (approx_total != approx_total || s0 != s0) return s0 + approx_total;
     const float seen_excl = __uint_as_float(FromLaneBelowU32(__float_as_uint(seen_incl), 0u));
     /* the sum is never below a term already added */
     int raw[CPL];
@@ -388,10 +342,11 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
 #pragma unroll
     for (int c = 0; c < CPL; ++c) {
       const int k = lane * CPL + c;
-      st[c] = excl + pre[c];
-      lo[c] = MaxNum3(PlanLowBound(st[c], static_cast<float>(k) * static_cast<float>(kWave * N)),
-                      seen_excl, seen[c]);
-      raw[c] = PlanBinade(lo[c], PlanHighBound(excl + pre[c + 1]));
+      st[c] = s0 + (excl + pre[c]);
+      /* s0, the sum in front of these terms, is itself a sum the row has reached */
+      lo[c] = MaxNum(MaxNum3(PlanLowBound(st[c], static_cast<float>(k) * static_cast<float>(kWave * N)),
+                             seen_excl, seen[c]), s0);
+      raw[c] = PlanBinade(lo[c], PlanHighBound(s0 + (excl + pre[c + 1])));
     }
     /* neighbouring certain chunks must agree on the binade, or the later one is listed:
        every run of certain chunks then has one scale */
@@ -638,7 +593,7 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
        phases) yield issue slots to it */
     __builtin_amdgcn_s_setprio(3);
     const int count = static_cast<int>(lds->row_count);
-    float s = 0.0f;
+    float s = s0;
     bool bad = false;
     /* the next block is fetched while the current one is summed */
     Addend next;
@@ -668,7 +623,7 @@ __device__ inline float RowOrderedSum(const float (&v)[SLABS][N], int cols,
   /* the plan did not hold (kept so that the result cannot depend on the plan): every chunk
      is resolved in row order by wave scans, wave after wave */
   __syncthreads();
-  if (threadIdx.x == 0) lds->s = 0.0f;
+  if (threadIdx.x == 0) lds->s = s0;
   __syncthreads();
   for (int j = 0; j < SLABS; ++j) {
     float t[N];
@@ -857,6 +812,116 @@ __global__ void __launch_bounds__(THREADS, MIN_WAVES)  // 4 waves per SIMD: two 
   MSHADOW_ROWSUM_STAMP(14)
 }
 
+/*! \brief SLABS packs per thread of the stretch of a row that begins at `in` and has `left`
+ *  columns to the end of the row, in the layout of SoftmaxRowKernel (slab j of wave w holds
+ *  the 256 columns from (j * W + w) * 256): 16-byte accesses wherever the stretch starts, the
+ *  pack the row ends in element by element, `absent` behind the end */
+template <int THREADS, int SLABS>
+__device__ __forceinline__ void LoadStretch(float (&v)[SLABS][4], const float *in, int left, float absent) {
+  const int W = THREADS / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(WaveId());
+  const int lane_col = LaneId() * 4;
+#pragma unroll
+  for (int j = 0; j < SLABS; ++j) {
+    const int c0 = (j * W + wave) * 256;  // uniform
+    const float *at = in + c0 + lane_col;
+    if (c0 + 256 <= left || c0 + lane_col + 4 <= left) {
+      const F4 q = StreamLoadF4Anywhere(at);
+      v[j][0] = q.x; v[j][1] = q.y; v[j][2] = q.z; v[j][3] = q.w;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[j][i] = (c0 + lane_col + i < left) ? at[i] : absent;
+    }
+  }
+}
+
+/*! \brief rows longer than one workgroup's registers hold (more than THREADS * SLABS * 4
+ *  columns), any length: one workgroup per row takes the row stretch by stretch, three times -
+ *  the maximum; the terms exp(x - max) of each stretch and their sum, which RowOrderedSum
+ *  continues from the sum of the stretches in front (so the row's sum is the left-to-right sum
+ *  of mshadow/tensor_cpu-inl.h:277-281 as in the kernel above); the terms once more (the same
+ *  instructions on the same logits give the same terms), divided and stored. src is read three
+ *  times, the second and third time mostly from the caches, dst written once; dst may alias src
+ *  (a thread reads a pack for the last time before it writes it).
+ *  TERMS_GIVEN: src already holds the (non-negative) terms and dst[row] receives their
+ *  left-to-right sum - the row-sum stage on its own, one pass.
+ *  MIN_WAVES (per SIMD): 4 fits two 512-thread rows on a CU at the price of a few registers kept
+ *  in scratch memory - faster when there are more rows than CUs ((512,128000): 204 against
+ *  224 us), slower when there are not ((16,250000): 129 against 113 us), where 2 is used. */
+template <int THREADS, int SLABS, bool TERMS_GIVEN, int MIN_WAVES>
+__global__ void __launch_bounds__(THREADS, MIN_WAVES)
+    SoftmaxStretchRowKernel(float *dst, int dstride, const float *src, int sstride, int cols) {
+  __shared__ RowSumLds<THREADS / kWave, SLABS, 4> lds;
+  const int W = THREADS / kWave;
+  const int kStretch = THREADS * SLABS * 4;
+  const int wave = __builtin_amdgcn_readfirstlane(WaveId());
+  const int lane_col = LaneId() * 4;
+  const float *in = src + static_cast<size_t>(blockIdx.x) * sstride;
+  float *out = dst + static_cast<size_t>(blockIdx.x) * dstride;
+  const float kNegInf = -__builtin_huge_valf();
+  float v[SLABS][4];
+  float mx = kNegInf;
+  if (!TERMS_GIVEN) {
+    for (int t0 = 0; t0 < cols; t0 += kStretch) {
+      LoadStretch<THREADS, SLABS>(v, in + t0, cols - t0, kNegInf);
+#pragma unroll
+      for (int j = 0; j < SLABS; ++j) {
+        mx = MaxNum3(mx, v[j][0], v[j][1]);
+        mx = MaxNum3(mx, v[j][2], v[j][3]);
+      }
+    }
+    mx = BlockMax<THREADS>(mx, lds.wmax);
+  }
+  float s = 0.0f;
+  for (int t0 = 0; t0 < cols; t0 += kStretch) {
+    LoadStretch<THREADS, SLABS>(v, in + t0, cols - t0, TERMS_GIVEN ? 0.0f : kNegInf);
+    if (!TERMS_GIVEN) {
+#pragma unroll
+      for (int j = 0; j < SLABS; ++j) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[j][i] = ExpNonPositive(v[j][i] - mx);
+        if (j + 1 < SLABS) {  // one slab at a time, as in SoftmaxRowKernel
+#pragma unroll
+          for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(v[j + 1][i]) : "v"(v[j][i]));
+        }
+      }
+    }
+    __syncthreads();  // everybody has read the sum the stretch in front left in LDS
+    s = RowOrderedSum<THREADS, SLABS, 4, TERMS_GIVEN, !TERMS_GIVEN>(v, cols - t0, &lds, s);
+  }
+  if (TERMS_GIVEN) {
+    if (threadIdx.x == 0) dst[blockIdx.x] = s;
+    return;
+  }
+  const bool fast_div = s >= 1.0f && s < 3.0e38f;
+  const float rcp = 1.0f / s;
+  for (int t0 = 0; t0 < cols; t0 += kStretch) {
+    const int left = cols - t0;
+    LoadStretch<THREADS, SLABS>(v, in + t0, left, kNegInf);
+#pragma unroll
+    for (int j = 0; j < SLABS; ++j) {
+      const int c0 = (j * W + wave) * 256;
+      float o[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = ExpNonPositive(v[j][i] - mx);
+        o[i] = fast_div ? DivideBy(p, s, rcp) : p / s;
+      }
+      float *at = out + t0 + c0 + lane_col;
+      if (c0 + 256 <= left || c0 + lane_col + 4 <= left) {
+        F4 q;
+        q.x = o[0]; q.y = o[1]; q.z = o[2]; q.w = o[3];
+        StreamStoreF4Anywhere(at, q);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (c0 + lane_col + i < left) at[i] = o[i];
+        }
+      }
+    }
+  }
+}
+
 /* ---- short rows -----------------------------------------------------------------------
  * A workgroup per row wastes the machine on the rows classifiers usually have (tens to a few
  * hundred classes). Same arithmetic as SoftmaxRowKernel, other ownership: */
@@ -1007,33 +1072,6 @@ __global__ void __launch_bounds__(256)
       }
     }
   }
-}
-
-/*! \brief any row length: three passes, exp(x - max) parked in dst between them */
-template <int THREADS>
-__global__ void __launch_bounds__(THREADS)
-    SoftmaxLongRowKernel(float *dst, int dstride, const float *src, int sstride, int cols) {
-  __shared__ OrderedSumLds<THREADS / kWave> lds;
-  const int tid = threadIdx.x;
-  const float *in = src + static_cast<size_t>(blockIdx.x) * sstride;
-  float *out = dst + static_cast<size_t>(blockIdx.x) * dstride;
-  const float kNegInf = -__builtin_huge_valf();
-  float mx = kNegInf;
-  for (int x = tid; x < cols; x += THREADS) {
-    const float e = in[x];
-    mx = (mx < e) ? e : mx;
-  }
-  mx = BlockMax<THREADS>(mx, lds.wmax);
-  float s = 0.0f;
-  int buf = 0;
-  for (int x0 = 0; x0 < cols; x0 += THREADS) {
-    const int x = x0 + tid;
-    float p[1];
-    p[0] = (x < cols) ? ExpNonPositive(in[x] - mx) : 0.0f;
-    if (x < cols) out[x] = p[0];
-    s = BlockOrderedAdd<THREADS, 1>(s, p, &lds, &buf);
-  }
-  for (int x = tid; x < cols; x += THREADS) out[x] = out[x] / s;
 }
 
 const int kGradBlock = 256;

@@ -273,6 +273,9 @@ SOFTMAX_SHAPES = [((64, 32000), 0), ((5, 1000), 0), ((5, 1001), 0), ((3, 7), 1),
                   ((3, 5000), 3), ((2, 20000), 1),
                   # rows that neither start at multiples of 16 bytes nor are whole packs
                   ((3, 50257), 0), ((2, 33333), 1), ((2, 65535), 0), ((6, 4097), 2), ((5, 1023), 0),
+                  # rows longer than a workgroup's registers hold: stretch by stretch (two, four and five stretches,
+                  # a last stretch of one column, of one pack, pitched rows)
+                  ((3, 128000), 0), ((2, 200001), 1), ((1, 262149), 0), ((2, 65537), 3), ((2, 65540), 0), ((2, 131072), 2),
                   # many rows of a few hundred to 2048 columns: a wave per row, slab after slab
                   ((2100, 300), 0), ((2049, 777), 3), ((2050, 1024), 0), ((2048, 2047), 1), ((4100, 513), 0),
                   # short rows: one thread per row up to 32 columns, one wave per row up to 256
@@ -339,7 +342,9 @@ def _serial_row_sums(O, terms):
 
 
 ROWSUM_COLS = [1, 3, 10, 31, 32, 33, 64, 65, 128, 129, 255, 256, 257, 300, 513, 777, 1000, 1024, 1028, 2048, 3000, 4096, 5001, 8192, 12000, 16384,
-               20001, 32000, 32768, 40000, 65536]
+               20001, 32000, 32768, 40000, 65536,
+               # longer than a workgroup's registers hold: summed stretch by stretch, each from the sum in front
+               65537, 70001, 131072, 131075, 200001, 262149]
 
 
 @pytest.mark.parametrize("cols", ROWSUM_COLS)
@@ -368,11 +373,10 @@ def test_softmax_rowsum_is_the_serial_sum(G, O, stream, cols):
     rows.append(np.full(cols, 2.0 ** -130))                       # subnormal terms
     terms = np.asarray(rows, dtype=f32)
     want = _serial_row_sums(O, terms)
-    if cols % 4 == 0 or cols <= 32768:
-        for pad in (0, 1) if cols <= 32768 else (0,):
-            sums = G.buffer((terms.shape[0],), f32)
-            G.softmax_rowsum(sums, G.to_device(terms, pad), stream)
-            assert_bits_equal(sums.download(stream), want, f"row sum cols={cols} pad={pad}")
+    for pad in (0, 1):
+        sums = G.buffer((terms.shape[0],), f32)
+        G.softmax_rowsum(sums, G.to_device(terms, pad), stream)
+        assert_bits_equal(sums.download(stream), want, f"row sum cols={cols} pad={pad}")
     if 256 < cols <= 2048:
         # with thousands of rows these lengths take the kernel with a wave per row
         many = np.tile(terms, (150, 1))
