@@ -6,6 +6,7 @@
  */
 #include "abi_common.h"
 
+#include <climits>
 #include <mutex>
 
 #include <mshadow/hip/kernels/reduce.h>
@@ -521,7 +522,9 @@ int mshadow_hip_softmax_f32(float *dst, int dstride, const float *src, int sstri
   /* longer rows: stretches of 32768 columns on 512 threads, two rows to a CU ((512,128000): 221 us
      against 271 us with stretches of 65536 on 1024 threads; up to 65536 columns the single pass
      above is faster than stretches, 265 against 432 us on (2048,50257)) */
-  else if (rows > mshadow_abi::ComputeUnits()) {
+  else if (cols > INT_MAX - 32768) {
+    return Fail(MSHADOW_HIP_ERR_ARGUMENT, "softmax: row too long for 32-bit column counts");
+  } else if (rows > mshadow_abi::ComputeUnits()) {
     hipLaunchKernelGGL((SoftmaxStretchRowKernel<512, 16, false, 4>), dim3(rows), dim3(512), 0, s, dst,
                        dstride, src, sstride, cols);
   } else {
@@ -556,6 +559,7 @@ int mshadow_hip_softmax_rowsum_f32(float *sums, const float *terms, int tstride,
   const bool vec = Aligned16(terms) && tstride % 4 == 0 && cols % 4 == 0;
   /* rows longer than a workgroup's registers hold: stretch by stretch, at any alignment */
   if (cols > 65536 || (!vec && cols > 32768)) {
+    ABI_REQUIRE(cols <= INT_MAX - 32768, "row too long for 32-bit column counts");
     hipLaunchKernelGGL((SoftmaxStretchRowKernel<512, 16, true, 2>), dim3(rows), dim3(512), 0, s, sums, 0,
                        terms, tstride, cols);
     return AfterLaunch("softmax_rowsum");
