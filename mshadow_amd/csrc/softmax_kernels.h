@@ -102,6 +102,7 @@ const uint32_t kListedBit = 0x80000000u;
 #define MSHADOW_ROWSUM_STAMP(step)
 #endif
 
+
 /*! \brief one addend of the chain: its value and, for a run, 1 + the binade the sum must be
  *  in before and after it (0 for a term); eight bytes, written and read as one word */
 struct Addend {
@@ -141,7 +142,11 @@ struct RowSumLds {
   /*! \brief the row's addends in row order, as the chain takes them: for each listed chunk
    *  the run of certain chunks in front of it (one addend) and then its own list, and
    *  at the end the run behind the last listed chunk */
-  static const int kRowAddends = 512;
+  /* 512 hold nearly every row; a row whose sum ends just above a power of two has every chunk
+     behind the crossing listed lane by lane (the bounds cannot tell on which side the sum is)
+     and takes 900-1100, so workgroups of eight waves and more, two to a CU, have room for 2048:
+     the chain over them is a few microseconds, the fall-back 45 */
+  static const int kRowAddends = W <= 4 ? 512 : 2048;
   Addend row[kRowAddends];
   uint32_t row_count;
   MSHADOW_ALIGNED(8) AddendList<N> list[kSlots];
