@@ -424,6 +424,42 @@ def test_softmax_extreme_rows(G, O, stream):
         assert np.all(np.abs(got[~big].astype(np.float64) - want[~big]) <= 1e-35)
 
 
+def test_softmax_long_rows_extremes_and_specials(G, O, stream):
+    """rows taken stretch by stretch: the maximum in the last stretch, a long underflowing head, one
+    class far above the rest in a middle stretch; a NaN or an infinite logit makes the row NaN as on
+    the CPU, wherever it sits"""
+    n = 150000
+    rng = np.random.default_rng(77)
+    base = (rng.standard_normal(n) * 3).astype(f32)
+    rows = [np.linspace(-300, 0, n), np.linspace(0, -300, n), np.r_[np.full(n - 1, -5.0), 40.0], base.copy(), base.copy()]
+    rows[3][70000] = 60.0
+    rows[4][140000] = 25.0
+    x = np.asarray(rows, dtype=f32)
+    want = np.empty_like(x)
+    O.softmax(want, x)
+    dst = G.buffer(x.shape, f32)
+    G.softmax(dst, G.to_device(x), stream)
+    got = dst.download(stream)
+    rel = np.abs(got.astype(np.float64) - want) / np.maximum(want, np.finfo(f32).tiny)
+    assert rel.max() <= 1e-5, rel.max()
+    for pos in (5, 40000, 100000, n - 1):
+        for val in (np.nan, np.inf):
+            y = base.copy()[None, :]
+            y[0, pos] = val
+            O.softmax(want[:1], y)
+            G.softmax(dst, G.to_device(np.repeat(y, 5, 0)), stream)
+            got = dst.download(stream)
+            assert np.isnan(want[0]).all() and np.isnan(got).all(), (pos, val)
+    y = base.copy()[None, :]
+    y[0, 90000] = -np.inf            # a class that cannot occur: its probability is 0, the rest as usual
+    O.softmax(want[:1], y)
+    G.softmax(dst, G.to_device(np.repeat(y, 5, 0)), stream)
+    got = dst.download(stream)
+    assert got[2, 90000] == 0.0 and want[0, 90000] == 0.0
+    rel = np.abs(got[2].astype(np.float64) - want[0]) / np.maximum(want[0], np.finfo(f32).tiny)
+    assert rel.max() <= 1e-5
+
+
 @pytest.mark.parametrize("shape,pad", [((64, 32000), 0), ((9, 1001), 0), ((9, 1000), 4),
                                        ((5, 7), 1), ((3, 20000), 0)])
 def test_softmax_grad(G, O, stream, shape, pad):
