@@ -403,6 +403,27 @@ def test_softmax_rowsum_specials(G, O, stream):
     assert same.all(), (got, want)
 
 
+def test_softmax_rowsum_specials_in_long_rows(G, O, stream):
+    """rows summed stretch by stretch: a negative, infinite, huge or NaN term in any stretch gives what
+    the serial loop gives (the plan is for non-negative terms; anything else is summed by wave scans,
+    from the sum of the stretches in front)"""
+    cols = 100003
+    base = np.random.default_rng(8).uniform(0, 1, cols).astype(f32)
+    rows = []
+    for pos in (3, 32767, 32768, 70000, cols - 1):
+        for val in (np.inf, np.nan, -0.5, 3.0e38):
+            r = base.copy()
+            r[pos] = val
+            rows.append(r)
+    terms = np.asarray(rows, dtype=f32)
+    want = _serial_row_sums(O, terms)
+    sums = G.buffer((terms.shape[0],), f32)
+    G.softmax_rowsum(sums, G.to_device(terms), stream)
+    got = sums.download(stream)
+    same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
+    assert same.all(), (got, want)
+
+
 def test_softmax_extreme_rows(G, O, stream):
     rows = [
         np.linspace(-200, 0, 5000),          # long underflowing head (leading zeros)
