@@ -365,6 +365,54 @@ __global__ void __launch_bounds__(kPatchBlock)
                         static_cast<size_t>(line) * g.ow + ox, q);
 }
 
+/*! \brief im2col with a step of two pixels between patches in a row (any step between rows, any
+ *  dilation), patch rows of at least one pack: as Im2ColDirectS1Kernel, but the EPT pixels of a
+ *  pack lie two apart in the image: the thread fetches the two packs that hold them and keeps
+ *  every second element. */
+template <typename T>
+__global__ void __launch_bounds__(kPatchBlock)
+    Im2ColDirectS2Kernel(T *col, int cstride, const T *img, int istride, PatchGeom g,
+                         mshadow::FastDivU32 div_ppr, mshadow::FastDivU32 div_oh, uint32_t chunks,
+                         mshadow::FastDivU32 div_chunks, uint32_t places) {
+  const int EPT = 16 / sizeof(T);
+  const uint32_t taps = static_cast<uint32_t>(g.ky * g.kx);
+  const uint32_t lane8 = blockIdx.x & 7u;
+  const uint32_t turn = blockIdx.x >> 3;
+  const uint32_t group = turn / taps;
+  const uint32_t tap = turn - group * taps;
+  const uint32_t piece = group * 8 + lane8;
+  const uint32_t ch = div_chunks.Div(piece);
+  if (ch >= static_cast<uint32_t>(g.c)) return;
+  const uint32_t chunk = piece - ch * chunks;
+  const int a = static_cast<int>(tap) / g.kx;
+  const int b = static_cast<int>(tap) - a * g.kx;
+  const uint32_t pk = chunk * kPatchBlock + threadIdx.x;   // place: (n * oh + oy) * ppr + p
+  if (pk >= places) return;
+  const uint32_t line = div_ppr.Div(pk);
+  const int ox = min(static_cast<int>(pk - line * div_ppr.div) * EPT, g.ow - EPT);
+  const uint32_t n = div_oh.Div(line);
+  const int oy = static_cast<int>(line - n * g.oh);
+  const int y = oy * g.sy + a * g.dy - g.pad_y;
+  const int xs = ox * 2 + b * g.dx - g.pad_x;
+  U4 q = {0u, 0u, 0u, 0u};
+  if (y >= 0 && y < g.h) {
+    const T *row = img + (static_cast<size_t>(n * g.c + ch) * g.h + y) * istride;
+    const T *last = img + (static_cast<size_t>(g.n) * g.c * g.h - 1) * istride + g.w;
+    const U4 lo = LoadPackInside<T>(row + xs, max(0, -xs), min(EPT, g.w - xs), img, last);
+    const U4 hi = LoadPackInside<T>(row + xs + EPT, max(0, -xs - EPT), min(EPT, g.w - xs - EPT), img, last);
+    if (sizeof(T) == 4) {
+      q[0] = lo[0], q[1] = lo[2], q[2] = hi[0], q[3] = hi[2];
+    } else {
+      q[0] = __builtin_amdgcn_perm(lo[1], lo[0], 0x05040100u);
+      q[1] = __builtin_amdgcn_perm(lo[3], lo[2], 0x05040100u);
+      q[2] = __builtin_amdgcn_perm(hi[1], hi[0], 0x05040100u);
+      q[3] = __builtin_amdgcn_perm(hi[3], hi[2], 0x05040100u);
+    }
+  }
+  StorePackAnywhere(col + static_cast<size_t>(ch * taps + tap) * cstride +
+                        static_cast<size_t>(line) * g.ow + ox, q);
+}
+
 /*! \brief one pack plus another, element by element, rounded after every add as the element
  *  type's own += does (binary16: a packed half add is exactly that); elements whose bit in
  *  `keep` is clear stay as they are */

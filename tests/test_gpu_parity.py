@@ -608,6 +608,8 @@ CONV = [  # n, c, h, w, ky, kx, sy, sx, dy, dx, py, px
     # strides and dilations on rows of a pack or more
     (4, 6, 56, 56, 3, 3, 2, 2, 1, 1, 1, 1), (2, 3, 64, 70, 7, 7, 2, 2, 1, 1, 3, 3),
     (3, 2, 40, 44, 3, 3, 1, 1, 2, 2, 2, 2), (2, 2, 45, 50, 3, 5, 3, 2, 2, 1, 1, 2),
+    # a step of two between patches in a row: dilated taps, rows of odd length, no padding, padding wider than a pack
+    (2, 3, 50, 61, 3, 3, 1, 2, 1, 2, 1, 2), (3, 2, 33, 35, 1, 1, 2, 2, 1, 1, 0, 0), (2, 2, 30, 47, 5, 5, 2, 2, 1, 1, 0, 9),
     (2, 3, 33, 47, 11, 11, 4, 4, 1, 1, 0, 0),
 ]
 
