@@ -587,7 +587,7 @@ def neighbour_shapes(G):
 
     for shape, k, st in (((128, 64, 112, 112), 2, 2), ((128, 64, 112, 112), 3, 2), ((128, 64, 112, 112), 3, 1),
                          ((64, 96, 55, 55), 3, 2), ((256, 256, 13, 13), 3, 2), ((32, 64, 224, 224), 2, 2),
-                         ((128, 256, 28, 28), 2, 2)):
+                         ((128, 256, 28, 28), 2, 2), ((32, 64, 224, 224), 5, 1)):
         n, c, h, w = shape
         ph, pw = (h - k) // st + 1, (w - k) // st + 1
         x = big(shape)

@@ -983,6 +983,41 @@ int mshadow_hip_pool_f32(float *dst, int dstride, const float *src, int sstride,
     const size_t lds = (static_cast<size_t>(g.band - 1) * sy + ky) * row_bytes + 16;
     const long long blocks = static_cast<long long>(planes) * g.bands;
     ABI_REQUIRE(blocks < (1ll << 31), "too many workgroups");
+    /* windows that move by one element: a thread walks down an output column, KX reads of LDS an
+       output. The band's rows are cut into `nruns` runs so that the columns of all runs fill the
+       workgroup's threads in as few, as short rounds as can be. */
+    if (sy == 1 && sx == 1 && ky == kx && (ky == 2 || ky == 3 || ky == 5) && ph <= h - ky + 1 &&
+        pw <= w - kx + 1) {
+      int nruns = 1, run_len = g.band;
+      long long best = -1;
+      for (int n = 1; n <= g.band; ++n) {
+        const int rl = (g.band + n - 1) / n;
+        const long long rounds = (static_cast<long long>(n) * pw + kPoolBlock - 1) / kPoolBlock;
+        const long long cost = rounds * (rl + ky - 1);
+        if (best < 0 || cost < best) { best = cost; nruns = n; run_len = rl; }
+      }
+      const mshadow::FastDivU32 div_pw(static_cast<uint32_t>(pw));
+#define POOL_COLUMNS(K)                                                                        \
+  switch (reducer) {                                                                           \
+    case MSHADOW_HIP_SUM:                                                                      \
+      hipLaunchKernelGGL((PoolColumnsS1Kernel<MSHADOW_HIP_SUM, K, K>), dim3(static_cast<unsigned>(blocks)), \
+                         dim3(kPoolBlock), lds, s, dst, dstride, src, sstride, g, nruns, run_len, div_pw); \
+      break;                                                                                   \
+    case MSHADOW_HIP_MAX:                                                                      \
+      hipLaunchKernelGGL((PoolColumnsS1Kernel<MSHADOW_HIP_MAX, K, K>), dim3(static_cast<unsigned>(blocks)), \
+                         dim3(kPoolBlock), lds, s, dst, dstride, src, sstride, g, nruns, run_len, div_pw); \
+      break;                                                                                   \
+    default:                                                                                   \
+      hipLaunchKernelGGL((PoolColumnsS1Kernel<MSHADOW_HIP_MIN, K, K>), dim3(static_cast<unsigned>(blocks)), \
+                         dim3(kPoolBlock), lds, s, dst, dstride, src, sstride, g, nruns, run_len, div_pw); \
+      break;                                                                                   \
+  }
+      if (ky == 2) { POOL_COLUMNS(2) }
+      else if (ky == 3) { POOL_COLUMNS(3) }
+      else { POOL_COLUMNS(5) }
+#undef POOL_COLUMNS
+      return AfterLaunch("pool");
+    }
 #define POOL_TILED(KY, KX)                                                                     \
   switch (reducer) {                                                                           \
     case MSHADOW_HIP_SUM:                                                                      \

@@ -67,17 +67,28 @@ __device__ __forceinline__ int LdsPhase(const float *g) {
   return static_cast<int>((reinterpret_cast<uintptr_t>(g) >> 2) & 3);
 }
 
+__device__ __forceinline__ uint32_t IsNegZero(float v) {
+  return __float_as_uint(v) == 0x80000000u ? 1u : 0u;
+}
+
 /*! \brief copy `nrows` rows of `width` floats (global pitch gpitch) into LDS (pitch
  *  lpitch); `lds` already includes the phase shift of LdsPhase(g). When both pitches equal
  *  the width the band is one contiguous run and moves as 128-bit packs, eight loads in
- *  flight per thread; otherwise one wave takes one row at a time. */
+ *  flight per thread; otherwise one wave takes one row at a time. With WATCH, *neg_zero becomes
+ *  non-zero if this thread staged a -0.0f. */
+template <bool WATCH = false>
 __device__ __forceinline__ void StageRows(float *lds, int lpitch, const float *g, int gpitch,
-                                          int nrows, int width) {
+                                          int nrows, int width, uint32_t *neg_zero = nullptr) {
+  uint32_t seen = 0u;
   if (gpitch == width && lpitch == width) {
     const int total = nrows * width;
     const int lead = (4 - LdsPhase(g)) & 3;
     const int head = lead < total ? lead : total;
-    if (static_cast<int>(threadIdx.x) < head) lds[threadIdx.x] = g[threadIdx.x];
+    if (static_cast<int>(threadIdx.x) < head) {
+      const float v = g[threadIdx.x];
+      lds[threadIdx.x] = v;
+      if (WATCH) seen |= IsNegZero(v);
+    }
     const int nvec = (total - head) / 4;
     const float *gv = g + head;
     F4 *lv = reinterpret_cast<F4 *>(lds + head);
@@ -93,17 +104,68 @@ __device__ __forceinline__ void StageRows(float *lds, int lpitch, const float *g
       for (int u = 0; u < kUnroll; ++u) {
         const int v = v0 + u * kPoolBlock;
         if (v < nvec) lv[v] = q[u];
+        if (WATCH) seen |= IsNegZero(q[u].x) | IsNegZero(q[u].y) | IsNegZero(q[u].z) | IsNegZero(q[u].w);
       }
     }
     const int tail = head + 4 * nvec + threadIdx.x;
-    if (tail < total) lds[tail] = g[tail];
+    if (tail < total) {
+      const float v = g[tail];
+      lds[tail] = v;
+      if (WATCH) seen |= IsNegZero(v);
+    }
   } else {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     for (int r = wave; r < nrows; r += kPoolWaves) {
       const float *row = g + static_cast<size_t>(r) * gpitch;
-      for (int c = lane; c < width; c += 64) lds[r * lpitch + c] = row[c];
+      for (int c = lane; c < width; c += 64) {
+        const float v = row[c];
+        lds[r * lpitch + c] = v;
+        if (WATCH) seen |= IsNegZero(v);
+      }
     }
   }
+  if (WATCH) *neg_zero = seen;
+}
+
+/*! \brief max / min of two floats in one instruction. It gives the reference's `(d < s) ? s : d`
+ *  / `(s < d) ? s : d` whenever d is not NaN (the running result of a window never is: both forms
+ *  pass over a NaN operand) and no -0.0f is about: the comparison keeps the zero it already has,
+ *  the instruction takes +0 over -0 (max) or -0 over +0 (min) whichever came first. */
+__device__ __forceinline__ float FastMax(float d, float s) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(d), "v"(s));
+  return r;
+}
+__device__ __forceinline__ float FastMin(float d, float s) {
+  float r;
+  asm("v_min_f32 %0, %1, %2" : "=v"(r) : "v"(d), "v"(s));
+  return r;
+}
+
+/*! \brief a whole KY x KX window at `win` (row pitch `pitch`) of a staged band, reduced in the
+ *  reference's order; by_comparison = false takes the one-instruction forms (the staged values
+ *  then hold no -0.0f) */
+template <int REDUCER, int KY, int KX>
+__device__ __forceinline__ float ReduceWholeWindow(const float *win, int pitch, bool by_comparison) {
+  typedef PoolOp<REDUCER> Op;
+  float res = Op::Init();
+  if (REDUCER != MSHADOW_HIP_SUM && !by_comparison) {
+#pragma unroll
+    for (int y = 0; y < KY; ++y) {
+#pragma unroll
+      for (int x = 0; x < KX; ++x) {
+        const float v = win[y * pitch + x];
+        res = REDUCER == MSHADOW_HIP_MAX ? FastMax(res, v) : FastMin(res, v);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int y = 0; y < KY; ++y) {
+#pragma unroll
+      for (int x = 0; x < KX; ++x) res = Op::Reduce(res, win[y * pitch + x]);
+    }
+  }
+  return res;
 }
 
 /*! \brief grid.x = planes * bands. Dynamic LDS: in_rows * lds_pitch + 4 floats, where
@@ -125,8 +187,10 @@ __global__ void __launch_bounds__(kPoolBlock)
   const int nrows = max(y1 - y0, 0);
   const float *in = src + (static_cast<size_t>(plane) * g.h + y0) * sstride;
   float *tile = smem + LdsPhase(in);
-  StageRows(tile, g.lds_pitch, in, sstride, nrows, g.w);
-  __syncthreads();
+  /* max and min go by single instructions unless the band holds a -0.0f */
+  uint32_t neg_zero = 0u;
+  StageRows<REDUCER != MSHADOW_HIP_SUM>(tile, g.lds_pitch, in, sstride, nrows, g.w, &neg_zero);
+  const bool by_comparison = __syncthreads_or(static_cast<int>(neg_zero)) != 0;
   float *out = dst + (static_cast<size_t>(plane) * g.ph + py0) * dstride;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   for (int py = wave; py < npy; py += kPoolWaves) {
@@ -137,13 +201,8 @@ __global__ void __launch_bounds__(kPoolBlock)
       const int xe = min(xs + kx, g.w);
       float res = Op::Init();
       if (KY > 0 && KX > 0 && ye - ys == KY && xe - xs == KX) {
-#pragma unroll
-        for (int y = 0; y < (KY > 0 ? KY : 1); ++y) {
-#pragma unroll
-          for (int x = 0; x < (KX > 0 ? KX : 1); ++x) {
-            res = Op::Reduce(res, tile[(ys + y) * g.lds_pitch + xs + x]);
-          }
-        }
+        res = ReduceWholeWindow<REDUCER, (KY > 0 ? KY : 1), (KX > 0 ? KX : 1)>(
+            tile + ys * g.lds_pitch + xs, g.lds_pitch, by_comparison);
       } else {
         for (int y = ys; y < ye; ++y) {
           for (int x = xs; x < xe; ++x) res = Op::Reduce(res, tile[y * g.lds_pitch + x]);
@@ -152,6 +211,84 @@ __global__ void __launch_bounds__(kPoolBlock)
       StreamStore(out + static_cast<size_t>(py) * dstride + px, res);
     }
   }
+}
+
+/*! \brief the windows of one staged band when they move by one element (sy == sx == 1, all of
+ *  them whole): a thread walks down ONE output column over `run_len` output rows and keeps the
+ *  last KY rows of its KX window columns in registers, so that an output costs KX reads of LDS
+ *  instead of KY * KX. The `nruns` runs of the band times its pw columns are dealt over the
+ *  threads; lanes of a wave sit in neighbouring columns. The order of the reduction inside a
+ *  window is the reference's (rows outermost). */
+template <int REDUCER, int KY, int KX>
+__device__ __forceinline__ void ColumnsS1Band(float *out, int dstride, const float *tile, int pitch, int npy,
+                                              int pw, int nruns, int run_len, mshadow::FastDivU32 div_pw,
+                                              bool by_comparison) {
+  typedef PoolOp<REDUCER> Op;
+  const uint32_t items = static_cast<uint32_t>(nruns) * pw;
+  for (uint32_t it = threadIdx.x; it < items; it += kPoolBlock) {
+    const uint32_t run = div_pw.Div(it);
+    const int px = static_cast<int>(it - run * pw);
+    const int r0 = static_cast<int>(run) * run_len;
+    const int nr = min(run_len, npy - r0);
+    if (nr <= 0) continue;
+    const float *col = tile + r0 * pitch + px;
+    float *o = out + static_cast<size_t>(r0) * dstride + px;
+    float ring[KY][KX];  // input row t of the run sits in slot t % KY
+#pragma unroll
+    for (int y = 0; y < KY - 1; ++y) {
+#pragma unroll
+      for (int x = 0; x < KX; ++x) ring[y][x] = col[y * pitch + x];
+    }
+    for (int r = 0; r < nr; r += KY) {
+#pragma unroll
+      for (int j = 0; j < KY; ++j) {
+        if (r + j < nr) {
+#pragma unroll
+          for (int x = 0; x < KX; ++x) ring[(j + KY - 1) % KY][x] = col[(r + j + KY - 1) * pitch + x];
+          float res = Op::Init();
+          if (REDUCER != MSHADOW_HIP_SUM && !by_comparison) {
+#pragma unroll
+            for (int y = 0; y < KY; ++y) {
+#pragma unroll
+              for (int x = 0; x < KX; ++x) {
+                const float v = ring[(j + y) % KY][x];
+                res = REDUCER == MSHADOW_HIP_MAX ? FastMax(res, v) : FastMin(res, v);
+              }
+            }
+          } else {
+#pragma unroll
+            for (int y = 0; y < KY; ++y) {
+#pragma unroll
+              for (int x = 0; x < KX; ++x) res = Op::Reduce(res, ring[(j + y) % KY][x]);
+            }
+          }
+          StreamStore(o + static_cast<size_t>(r + j) * dstride, res);
+        }
+      }
+    }
+  }
+}
+
+/*! \brief stride-1 pooling, one band of one plane per workgroup, staged as in PoolKernel.
+ *  grid.x = planes * bands. */
+template <int REDUCER, int KY, int KX>
+__global__ void __launch_bounds__(kPoolBlock)
+    PoolColumnsS1Kernel(float *dst, int dstride, const float *src, int sstride, PoolGeom g, int nruns,
+                        int run_len, mshadow::FastDivU32 div_pw) {
+  extern __shared__ float smem[];
+  const int plane = blockIdx.x / g.bands;
+  const int band = blockIdx.x - plane * g.bands;
+  const int py0 = band * g.band;
+  const int npy = min(g.band, g.ph - py0);
+  const int nrows = npy + KY - 1;
+  const float *in = src + (static_cast<size_t>(plane) * g.h + py0) * sstride;
+  float *tile = smem + LdsPhase(in);
+  uint32_t neg_zero = 0u;
+  StageRows<REDUCER != MSHADOW_HIP_SUM>(tile, g.lds_pitch, in, sstride, nrows, g.w, &neg_zero);
+  const bool by_comparison = __syncthreads_or(static_cast<int>(neg_zero)) != 0;
+  float *out = dst + (static_cast<size_t>(plane) * g.ph + py0) * dstride;
+  ColumnsS1Band<REDUCER, KY, KX>(out, dstride, tile, g.lds_pitch, npy, g.pw, nruns, run_len, div_pw,
+                                 by_comparison);
 }
 
 /*! \brief The same for small planes: a workgroup takes `per_block` whole consecutive planes (they
@@ -171,8 +308,9 @@ __global__ void __launch_bounds__(kPoolBlock)
   const int np = min(per_block, planes - plane0);
   const float *in = src + static_cast<size_t>(plane0) * g.h * sstride;
   float *tile = smem + LdsPhase(in);
-  StageRows(tile, g.lds_pitch, in, sstride, np * g.h, g.w);
-  __syncthreads();
+  uint32_t neg_zero = 0u;
+  StageRows<REDUCER != MSHADOW_HIP_SUM>(tile, g.lds_pitch, in, sstride, np * g.h, g.w, &neg_zero);
+  const bool by_comparison = __syncthreads_or(static_cast<int>(neg_zero)) != 0;
   float *out = dst + static_cast<size_t>(plane0) * g.ph * dstride;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   /* a wave takes `rpw` output rows at a time, pw lanes each (64 / pw of them, at least one) */
@@ -192,13 +330,8 @@ __global__ void __launch_bounds__(kPoolBlock)
       const int xe = min(xs + kx, g.w);
       float res = Op::Init();
       if (KY > 0 && KX > 0 && ye - ys == KY && xe - xs == KX) {
-#pragma unroll
-        for (int y = 0; y < (KY > 0 ? KY : 1); ++y) {
-#pragma unroll
-          for (int x = 0; x < (KX > 0 ? KX : 1); ++x) {
-            res = Op::Reduce(res, tile[(ys + y) * g.lds_pitch + xs + x]);
-          }
-        }
+        res = ReduceWholeWindow<REDUCER, (KY > 0 ? KY : 1), (KX > 0 ? KX : 1)>(
+            tile + ys * g.lds_pitch + xs, g.lds_pitch, by_comparison);
       } else {
         for (int y = ys; y < ye; ++y) {
           for (int x = xs; x < xe; ++x) res = Op::Reduce(res, tile[y * g.lds_pitch + x]);

@@ -518,6 +518,10 @@ POOL_CASES = [  # planes, h, w, ky, kx, sy, sx, pad
     (2, 64, 64, 2, 2, 1, 1, 3), (700, 64, 66, 3, 3, 1, 1, 1), (5, 97, 201, 3, 3, 1, 1, 0),
     (6, 37, 41, 3, 3, 1, 1, 2), (5, 20, 256, 3, 3, 1, 1, 0), (7, 9, 4, 3, 3, 1, 1, 0), (3, 5, 7, 2, 2, 1, 1, 1),
     (2560, 13, 13, 3, 3, 1, 1, 0), (3, 66, 260, 3, 3, 1, 1, 0), (300, 28, 28, 3, 3, 1, 1, 3),
+    # stride 1 in the pooling kernels that walk down output columns: rows of whole packs (four columns a thread,
+    # dense and pitched by a multiple of four) and others, 5 x 5, bands that end early, fewer than 16 outputs a row
+    (4, 64, 112, 5, 5, 1, 1, 0), (3, 40, 130, 5, 5, 1, 1, 1), (2, 131, 64, 3, 3, 1, 1, 4), (5, 57, 57, 3, 3, 1, 1, 0),
+    (3, 50, 20, 5, 5, 1, 1, 0), (2, 300, 16, 2, 2, 1, 1, 0), (2, 47, 1024, 3, 3, 1, 1, 0), (3, 33, 68, 2, 2, 1, 1, 8),
 ]
 
 
@@ -553,6 +557,25 @@ def test_pool_unpool(G, O, stream, case, reducer, variant):
         u2 = G.buffer((planes, h, w), f32)
         G.unpool(u2, dsrc, dpool, dgrad, ky, kx, sy, sx, reducer, stream)
         assert_bits_equal(u2.download(stream), wantu, "unpool abi")
+
+
+@pytest.mark.parametrize("case", [(4100, 56, 60, 3), (2100, 64, 64, 2), (2300, 41, 100, 5)])
+@pytest.mark.parametrize("reducer", [MAX, MIN, SUM])
+def test_pool_stride1_many_planes_zero_signs(G, O, stream, case, reducer):
+    """stride-1 pooling over thousands of dense planes of one band each; some planes hold zeros of both
+    signs, where max and min go by the reference's comparison, the others do not"""
+    planes, h, w, k = case
+    rng = np.random.default_rng(planes + k)
+    src = rng.integers(-5, 6, (planes, h, w)).astype(f32) / f32(4)
+    some = src[::7]
+    some[rng.random(some.shape) < 0.05] = f32(-0.0)
+    src[::7] = some
+    ph, pw = h - k + 1, w - k + 1
+    want = np.empty((planes, ph, pw), f32)
+    O.pool(want, src, k, k, 1, 1, reducer)
+    dpool = G.buffer((planes, ph, pw), f32)
+    G.pool(dpool, G.to_device(src), k, k, 1, 1, reducer, stream)
+    assert_bits_equal(dpool.download(stream), want, f"pool {case}")
 
 
 @pytest.mark.parametrize("shape", [(3, 9, 12, 3, 4), (3, 9, 12, 4, 5), (2, 10, 16, 2, 7), (2, 11, 13, 5, 3),
