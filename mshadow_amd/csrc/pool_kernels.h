@@ -262,7 +262,10 @@ __device__ __forceinline__ void ColumnsS1Band(float *out, int dstride, const flo
               for (int x = 0; x < KX; ++x) res = Op::Reduce(res, ring[(j + y) % KY][x]);
             }
           }
-          StreamStore(o + static_cast<size_t>(r + j) * dstride, res);
+          /* an ordinary store: output rows are as many bytes as input rows here and seldom end on
+             a cache line, and the lines two rows share leave L2 whole this way ((128,64,112,112)
+             3x3: 151 us against 162 us with streaming stores) */
+          o[static_cast<size_t>(r + j) * dstride] = res;
         }
       }
     }
