@@ -578,6 +578,39 @@ def test_pool_stride1_many_planes_zero_signs(G, O, stream, case, reducer):
     assert_bits_equal(dpool.download(stream), want, f"pool {case}")
 
 
+@pytest.mark.parametrize("case", [(40, 70, 66, 3, 2), (40, 70, 66, 3, 1), (30, 65, 130, 2, 1), (30, 64, 64, 5, 1),
+                                  (900, 13, 13, 3, 2), (900, 13, 13, 3, 1), (24, 50, 52, 2, 2), (6, 40, 45, 4, 3)])
+@pytest.mark.parametrize("reducer", [MAX, MIN, SUM])
+def test_pool_special_values(G, O, stream, case, reducer):
+    """NaN, infinities, the largest finite values and subnormals as window members in every staged pool
+    kernel, in planes with zeros of both signs (max and min by the reference's comparison) and in planes
+    with none (by single instructions): both pass over a NaN and agree bit for bit"""
+    planes, h, w, k, st = case
+    rng = np.random.default_rng(planes + 10 * k + st)
+    src = rng.integers(-3, 4, (planes, h, w)).astype(f32) / f32(2)
+    src[src == 0] = f32(0.25)
+    specials = np.array([np.nan, np.inf, -np.inf, 3.4028235e38, -3.4028235e38, 1e-45, -1e-45], f32)
+    where = rng.random(src.shape) < 0.3
+    src[where] = specials[rng.integers(0, specials.size, int(where.sum()))]
+    src[0, :4, :] = np.nan      # windows of NaN only
+    zeros = src[1::2]           # every second plane: zeros of both signs too
+    zw = rng.random(zeros.shape) < 0.2
+    zeros[zw] = np.where(rng.random(int(zw.sum())) < 0.5, f32(-0.0), f32(0.0))
+    src[1::2] = zeros
+    ph, pw = (h - k) // st + 1, (w - k) // st + 1
+    want = np.empty((planes, ph, pw), f32)
+    O.pool(want, src, k, k, st, st, reducer)
+    dpool = G.buffer((planes, ph, pw), f32)
+    G.pool(dpool, G.to_device(src), k, k, st, st, reducer, stream)
+    got = dpool.download(stream)
+    if reducer == SUM:  # a NaN sum is a NaN on both sides; its sign and payload are the adder's own
+        assert np.array_equal(np.isnan(got), np.isnan(want)), f"pool {case}: NaN in other places"
+        got, want = np.where(np.isnan(got), f32(0), got), np.where(np.isnan(want), f32(0), want)
+    else:
+        assert not np.isnan(want).any()
+    assert_bits_equal(got, want, f"pool {case}")
+
+
 @pytest.mark.parametrize("shape", [(3, 9, 12, 3, 4), (3, 9, 12, 4, 5), (2, 10, 16, 2, 7), (2, 11, 13, 5, 3),
                                    (4, 8, 8, 3, 3), (5, 6, 10, 2, 4), (2, 70, 72, 60, 66), (3, 64, 100, 31, 97)])
 @pytest.mark.parametrize("reducer", [MAX, SUM])

@@ -155,6 +155,26 @@ def test_pool_unpool(orc, ref, cfg, reducer):
     assert same(u1, u2)
 
 
+@pytest.mark.parametrize("cfg", [(3, 3, 2, 2), (2, 2, 1, 1), (3, 3, 1, 1)])
+@pytest.mark.parametrize("reducer", [MAX, MIN, SUM])
+def test_pool_special_values(orc, ref, cfg, reducer):
+    """NaN, infinities, zeros of both signs and the largest finite values as window members: std::max /
+    std::min pass over a NaN and keep the first of two equal zeros"""
+    ky, kx, sy, sx = cfg
+    rng = np.random.default_rng(90 + ky + sy + reducer)
+    src = (rng.integers(-3, 4, (5, 21, 23)).astype(f32) / 2)
+    flat = src.reshape(-1)
+    specials = np.array([np.nan, np.inf, -np.inf, -0.0, 0.0, 3.4028235e38, -3.4028235e38, 1e-45, -1e-45], f32)
+    where = rng.random(flat.size) < 0.3
+    flat[where] = specials[rng.integers(0, specials.size, int(where.sum()))]
+    flat[:60] = np.nan  # windows of NaN only
+    ph, pw = (21 - ky) // sy + 1, (23 - kx) // sx + 1
+    p1, p2 = np.empty((5, ph, pw), f32), np.empty((5, ph, pw), f32)
+    orc.pool(p1, src, ky, kx, sy, sx, reducer)
+    ref.pool(p2, src, ky, kx, sy, sx, reducer)
+    assert same(p1, p2)
+
+
 CONV = [(3, 3, 1, 1, 1, 1, 1, 1), (3, 3, 2, 2, 1, 1, 0, 0), (5, 3, 2, 1, 1, 1, 2, 1),
         (3, 3, 1, 1, 2, 2, 2, 2), (2, 3, 1, 2, 2, 2, 1, 0), (3, 3, 2, 2, 2, 1, 2, 2),
         (1, 1, 1, 1, 1, 1, 0, 0), (7, 7, 3, 3, 1, 1, 3, 3)]
