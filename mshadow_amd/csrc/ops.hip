@@ -249,6 +249,35 @@ int Col2Im(T *img, int istride, const T *col, int cstride, const PatchGeom &g, v
                             mshadow::FastDivU32(static_cast<uint32_t>(g.sx)),
                             mshadow::FastDivU32(static_cast<uint32_t>(g.dy)),
                             mshadow::FastDivU32(static_cast<uint32_t>(g.dx))};
+      /* dilation 1 and few patches over a pixel: every load of a thread under way at once */
+      const int over_y = (g.ky + g.sy - 1) / g.sy, over_x = (g.kx + g.sx - 1) / g.sx;
+      const int over = over_y > over_x ? over_y : over_x;
+      if (g.dy == 1 && g.dx == 1 && over <= 4) {
+#define COL2IM_FLAT(TY, TX)                                                                                  \
+  hipLaunchKernelGGL((Col2ImGatherFlatKernel<T, TY, TX>), dim3(blocks), dim3(kPatchBlock), 0, AsStream(stream), \
+                     img, istride, col, cstride, g, dv, mshadow::FastDivU32(static_cast<uint32_t>(wpk)),       \
+                     mshadow::FastDivU32(static_cast<uint32_t>(g.h)),                                          \
+                     mshadow::FastDivU32(static_cast<uint32_t>(g.c)), static_cast<uint32_t>(packs))
+        /* a step of two along x: the patches of every second pixel are neighbours in the matrix */
+        if (g.sx == 2 && g.ow >= EPT / 2 && over >= 2) {
+#define COL2IM_S2(TY, TX)                                                                                    \
+  hipLaunchKernelGGL((Col2ImGatherS2Kernel<T, TY, TX>), dim3(blocks), dim3(kPatchBlock), 0, AsStream(stream), \
+                     img, istride, col, cstride, g, dv, mshadow::FastDivU32(static_cast<uint32_t>(wpk)),       \
+                     mshadow::FastDivU32(static_cast<uint32_t>(g.h)),                                          \
+                     mshadow::FastDivU32(static_cast<uint32_t>(g.c)), static_cast<uint32_t>(packs))
+          if (over == 2) COL2IM_S2(2, 2);
+          else if (over == 3) COL2IM_S2(3, 3);
+          else COL2IM_S2(4, 4);
+#undef COL2IM_S2
+          return AfterLaunch("col2im");
+        }
+        if (over <= 1) COL2IM_FLAT(1, 1);
+        else if (over == 2) COL2IM_FLAT(2, 2);
+        else if (over == 3) COL2IM_FLAT(3, 3);
+        else COL2IM_FLAT(4, 4);
+#undef COL2IM_FLAT
+        return AfterLaunch("col2im");
+      }
       hipLaunchKernelGGL((Col2ImGatherKernel<T>), dim3(blocks), dim3(kPatchBlock), 0, AsStream(stream),
                          img, istride, col, cstride, g, dv, mshadow::FastDivU32(static_cast<uint32_t>(wpk)),
                          mshadow::FastDivU32(static_cast<uint32_t>(g.h)),

@@ -768,6 +768,144 @@ __global__ void __launch_bounds__(kPatchBlock)
   StorePackAnywhere(img + static_cast<size_t>(rowi) * istride + x0, acc);
 }
 
+/*! \brief Col2ImGatherKernel for dilation 1 and at most TY x TX patches over a pixel (TY >=
+ *  ceil(ky / sy), TX >= ceil(kx / sx)): the same terms in the same order, but all of a thread's
+ *  loads are issued before the first add. The loops of the general kernel have bounds that
+ *  differ from pixel to pixel, so its loads wait for one another, 18 round trips to memory a
+ *  thread for 3x3 windows with stride 2; here the patches a pixel lacks are loaded from a valid
+ *  address all the same and enter the sum as +0, which changes no bit of it (a sum that starts
+ *  at +0 is never -0). */
+template <typename T, int TY, int TX>
+__global__ void __launch_bounds__(kPatchBlock)
+    Col2ImGatherFlatKernel(T *img, int istride, const T *col, int cstride, PatchGeom g, PatchDivs dv,
+                           mshadow::FastDivU32 div_wpk, mshadow::FastDivU32 div_h,
+                           mshadow::FastDivU32 div_c, uint32_t total_packs) {
+  const int EPT = 16 / sizeof(T);
+  const uint32_t pk = blockIdx.x * kPatchBlock + threadIdx.x;
+  if (pk >= total_packs) return;
+  const uint32_t rowi = div_wpk.Div(pk);             // (n * c + ch) * h + cy
+  const int x0 = min(static_cast<int>(pk - rowi * div_wpk.div) * EPT, g.w - EPT);
+  const uint32_t plane = div_h.Div(rowi);
+  const int cy = static_cast<int>(rowi - plane * g.h);
+  const uint32_t n = div_c.Div(plane);
+  const uint32_t ch = plane - n * g.c;
+  const int y = cy + g.pad_y;                        // position in the padded image
+  const int py_min = y < g.ky ? 0 : static_cast<int>(dv.sy.Div(y - g.ky + g.sy));
+  const int py_max = min(static_cast<int>(dv.sy.Div(y + g.sy)), g.oh);
+  const T *base = col + static_cast<size_t>(ch) * g.ky * g.kx * cstride + static_cast<size_t>(n) * g.oh * g.ow;
+  T term[EPT][TY][TX];
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const int x = x0 + e + g.pad_x;
+    const int px_min = x < g.kx ? 0 : static_cast<int>(dv.sx.Div(x - g.kx + g.sx));
+    const int px_max = min(static_cast<int>(dv.sx.Div(x + g.sx)), g.ow);
+#pragma unroll
+    for (int i = 0; i < TY; ++i) {
+      const int py = py_min + i;
+      const int a = y - py * g.sy;
+#pragma unroll
+      for (int j = 0; j < TX; ++j) {
+        const int px = px_min + j;
+        const int b = x - px * g.sx;
+        const bool there = py < py_max && px < px_max;
+        const size_t at = there ? static_cast<size_t>(a * g.kx + b) * cstride + py * g.ow + px : 0;
+        const T v = base[at];
+        term[e][i][j] = there ? v : Acc<T>::Zero();
+      }
+    }
+  }
+  U4 acc = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    T res = Acc<T>::Zero();
+#pragma unroll
+    for (int i = 0; i < TY; ++i) {
+#pragma unroll
+      for (int j = 0; j < TX; ++j) res = Acc<T>::Add(res, term[e][i][j]);
+    }
+    SetPackElement(&acc, e, res);
+  }
+  StorePackAnywhere(img + static_cast<size_t>(rowi) * istride + x0, acc);
+}
+
+/*! \brief eight bytes of the column matrix at any element border */
+typedef uint64_t U64Loose __attribute__((aligned(2)));
+
+/*! \brief element k (of sizeof(T) bytes) of eight bytes */
+template <typename T>
+__device__ __forceinline__ T ElementOf64(uint64_t q, int k) {
+  const uint32_t w = static_cast<uint32_t>(q >> (8 * sizeof(T) * k));
+  T v;
+  __builtin_memcpy(&v, &w, sizeof(T));
+  return v;
+}
+
+/*! \brief Col2ImGatherFlatKernel for a step of two between patches along x (sx == 2, dilation 1,
+ *  ow >= 8 / sizeof(T)): the pixels of one parity among a thread's pack take, for their j-th patch,
+ *  NEIGHBOURING elements of one row of the column matrix (tap column b = x - 2 * px is the same
+ *  for all of them), so they come as one 8-byte load instead of one load each: a quarter (half,
+ *  for floats) of the requests. A pixel's patches are counted from floor((x - kx) / 2) + 1 also
+ *  where that is negative; patches left of 0 or right of ow - 1 are shifted out of the 8 bytes
+ *  (the load itself is moved inside the row) and enter the sum as +0, in their place in the
+ *  ascending order of px. TY >= ceil(ky / sy), TX >= ceil(kx / 2). */
+template <typename T, int TY, int TX>
+__global__ void __launch_bounds__(kPatchBlock)
+    Col2ImGatherS2Kernel(T *img, int istride, const T *col, int cstride, PatchGeom g, PatchDivs dv,
+                         mshadow::FastDivU32 div_wpk, mshadow::FastDivU32 div_h,
+                         mshadow::FastDivU32 div_c, uint32_t total_packs) {
+  const int EPT = 16 / sizeof(T);
+  const int PAIR = EPT / 2;                // pixels of one parity
+  const int EB = 8 * sizeof(T);
+  const uint32_t pk = blockIdx.x * kPatchBlock + threadIdx.x;
+  if (pk >= total_packs) return;
+  const uint32_t rowi = div_wpk.Div(pk);             // (n * c + ch) * h + cy
+  const int x0 = min(static_cast<int>(pk - rowi * div_wpk.div) * EPT, g.w - EPT);
+  const uint32_t plane = div_h.Div(rowi);
+  const int cy = static_cast<int>(rowi - plane * g.h);
+  const uint32_t n = div_c.Div(plane);
+  const uint32_t ch = plane - n * g.c;
+  const int y = cy + g.pad_y;                        // position in the padded image
+  const int py_min = y < g.ky ? 0 : static_cast<int>(dv.sy.Div(y - g.ky + g.sy));
+  const int py_max = min(static_cast<int>(dv.sy.Div(y + g.sy)), g.oh);
+  const T *base = col + static_cast<size_t>(ch) * g.ky * g.kx * cstride + static_cast<size_t>(n) * g.oh * g.ow;
+  uint64_t pack[2][TY][TX];
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const int x = x0 + p + g.pad_x;                  // first pixel of this parity
+    const int px_lo = ((x - g.kx) >> 1) + 1;         // floor((x - kx) / 2) + 1, may be negative
+#pragma unroll
+    for (int j = 0; j < TX; ++j) {
+      const int first = px_lo + j;                   // patch of the first pixel; + k for the k-th
+      const int b = x - 2 * first;                   // < kx by construction
+      const int inside = min(max(first, 0), g.ow - PAIR);
+      const int moved = first - inside;
+      const int shift = (moved < 0 ? -moved : moved) * EB;
+#pragma unroll
+      for (int i = 0; i < TY; ++i) {
+        const int py = py_min + i;
+        const int a = y - py * g.sy;
+        const bool there = py < py_max && b >= 0 && shift < 64;
+        const size_t at = there ? static_cast<size_t>(a * g.kx + b) * cstride + py * g.ow + inside : 0;
+        const uint64_t q = *reinterpret_cast<const U64Loose *>(base + at);
+        const uint64_t r = moved < 0 ? q << (shift & 63) : q >> (shift & 63);
+        pack[p][i][j] = there ? r : 0ull;
+      }
+    }
+  }
+  U4 acc = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    T res = Acc<T>::Zero();
+#pragma unroll
+    for (int i = 0; i < TY; ++i) {
+#pragma unroll
+      for (int j = 0; j < TX; ++j) res = Acc<T>::Add(res, ElementOf64<T>(pack[e & 1][i][j], e >> 1));
+    }
+    SetPackElement(&acc, e, res);
+  }
+  StorePackAnywhere(img + static_cast<size_t>(rowi) * istride + x0, acc);
+}
+
 /*! \brief one image pixel per thread; consecutive threads take consecutive x so that,
  *  for a fixed patch offset, their column-matrix reads are consecutive too */
 template <typename T>

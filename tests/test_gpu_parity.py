@@ -667,6 +667,14 @@ CONV = [  # n, c, h, w, ky, kx, sy, sx, dy, dx, py, px
     # a step of two between patches in a row: dilated taps, rows of odd length, no padding, padding wider than a pack
     (2, 3, 50, 61, 3, 3, 1, 2, 1, 2, 1, 2), (3, 2, 33, 35, 1, 1, 2, 2, 1, 1, 0, 0), (2, 2, 30, 47, 5, 5, 2, 2, 1, 1, 0, 9),
     (2, 3, 33, 47, 11, 11, 4, 4, 1, 1, 0, 0),
+    # col2im with a step of two along x, the patches of every second pixel from one 8-byte load: windows of even
+    # and odd width from 3 to 8, rows of odd length (the last pack moved back starts at an odd pixel), the patch
+    # grid as narrow as one load, other steps along y, padding wider than the window; 9 wide: the general kernel.
+    # Steps of 3: every load issued before the first add, 1 to 4 patches over a pixel in each direction
+    (2, 3, 40, 64, 7, 7, 2, 2, 1, 1, 3, 3), (2, 2, 31, 45, 4, 4, 2, 2, 1, 1, 1, 1), (3, 2, 20, 37, 8, 8, 2, 2, 1, 1, 4, 4),
+    (2, 2, 19, 11, 3, 3, 2, 2, 1, 1, 0, 0), (2, 2, 16, 8, 3, 3, 2, 2, 1, 1, 0, 0), (2, 3, 33, 52, 5, 5, 3, 2, 1, 1, 2, 2),
+    (2, 2, 26, 38, 3, 6, 1, 2, 1, 1, 1, 7), (1, 2, 30, 41, 9, 9, 2, 2, 1, 1, 4, 4), (2, 2, 28, 28, 2, 2, 2, 2, 1, 1, 0, 0),
+    (2, 3, 34, 40, 3, 3, 3, 3, 1, 1, 1, 1), (2, 2, 35, 43, 7, 5, 3, 3, 1, 1, 3, 2), (1, 2, 40, 48, 11, 11, 3, 3, 1, 1, 5, 5),
 ]
 
 
