@@ -1129,7 +1129,7 @@ int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstrid
   /* 2 x 2 and 3 x 3 windows with stride 1 on planes of 64 to 256 pixels a side: no staging, the
      pooled rows over the current source row in registers ((128,64,112,112): 368 us against 513 us
      for the kernels below; on planes of 57 x 57 the two are level, below that the staged ones win) */
-  if (ky == kx && (ky == 2 || ky == 3) && sy == 1 && sx == 1 && w >= 64 && w <= 256 && h >= 64 && ph >= 1 && pw >= 1 &&
+  if (ky == kx && (ky == 2 || ky == 3 || ky == 5) && sy == 1 && sx == 1 && w >= 64 && w <= 256 && h >= 64 && ph >= 1 && pw >= 1 &&
       static_cast<long long>(planes) * ph * pw >= 4 && static_cast<long long>(planes) * ((h + 1) / 2) < (1ll << 31)) {
     SlideGeom sg = MakeSlideGeom(planes, h, w);
     sg.src_floats = (static_cast<size_t>(planes) * h - 1) * sstride + w;
@@ -1142,8 +1142,11 @@ int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstrid
     if (ky == 2) {                                                                             \
       hipLaunchKernelGGL((UnpoolSlideS1Kernel<R, 2, 4>), dim3(blocks), dim3(kPoolBlock), 0, s, dst, dstride, \
                          src, sstride, pooled, pstride, grad, gstride, g, sg);                 \
-    } else {                                                                                   \
+    } else if (ky == 3) {                                                                      \
       hipLaunchKernelGGL((UnpoolSlideS1Kernel<R, 3, 3>), dim3(blocks), dim3(kPoolBlock), 0, s, dst, dstride, \
+                         src, sstride, pooled, pstride, grad, gstride, g, sg);                 \
+    } else {                                                                                   \
+      hipLaunchKernelGGL((UnpoolSlideS1Kernel<R, 5, 5>), dim3(blocks), dim3(kPoolBlock), 0, s, dst, dstride, \
                          src, sstride, pooled, pstride, grad, gstride, g, sg);                 \
     }                                                                                          \
   } while (0)

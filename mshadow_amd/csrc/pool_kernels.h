@@ -953,7 +953,9 @@ __device__ __forceinline__ float FromLaneBelow(float v) {
  *  The kernel is bound by its arithmetic (K * K terms per pixel), so a term is three
  *  instructions: the reference adds PartialGrad(src, pooled) * grad, a product that is grad
  *  where the two are equal and 0 * grad where not (a zero with grad's sign, NaN for an infinite
- *  grad); Z = 0 * grad is made once per gradient fetched and the term is picked from (grad, Z).
+ *  grad); Z = 0 * grad is made once per gradient fetched and the term is picked from (grad, Z)
+ *  (for K = 5 the product is made per term instead: a third array of 40 registers would leave
+ *  one wave per SIMD).
  *  Windows that do not exist (outside the pooled grid) are held as gradient 0: their term is
  *  +0, and adding a zero never changes the sum, which starts at +0 and so is never -0. The terms
  *  are added in the reference's order (py, then px ascending; mshadow/extension/
@@ -993,7 +995,9 @@ __global__ void __launch_bounds__(kPoolBlock)
       P[SLOT][i] = pl;                                                      \
       G[SLOT][i] = t == 0u ? 0.0f : gl;                                     \
     }                                                                       \
-    _Pragma("unroll") for (int i = 0; i < WIN; ++i) Z[SLOT][i] = 0.0f * G[SLOT][i]; \
+    if (K <= 3) {                                                           \
+      _Pragma("unroll") for (int i = 0; i < WIN; ++i) Z[SLOT][i] = 0.0f * G[SLOT][i]; \
+    }                                                                       \
   }
   /* the K - 1 pooled rows above the strip's first source row: row y0 - k in ring row K - k */
 #pragma unroll
@@ -1042,7 +1046,7 @@ __global__ void __launch_bounds__(kPoolBlock)
 #pragma unroll
           for (int j = 0; j < K; ++j) {    // px = x - (K - 1) + j
             const bool hit = REDUCER == MSHADOW_HIP_SUM || cur[e] == P[slot][e + j];
-            val = val + (hit ? G[slot][e + j] : Z[slot][e + j]);
+            val = val + (hit ? G[slot][e + j] : (K <= 3 ? Z[slot][e + j] : 0.0f * G[slot][e + j]));
           }
         }
         out[e] = val;
