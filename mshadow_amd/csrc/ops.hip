@@ -130,6 +130,36 @@ int Im2Col(T *col, int cstride, const T *img, int istride, const PatchGeom &g, v
       return AfterLaunch("im2col");
     }
   }
+  /* 3, 5 or 7 taps a row next to one another, a step of one or two between patches, patch rows of
+     a pack or more: all taps of a tap row from one fetch of the image under them (3x3 stride 2 on
+     (32,256,56,56) binary16: 27 us against 41 us with a fetch per tap; 5x5 stride 1 on (32,128,28,28):
+     29 against 40 us. Three taps with a step of one keep a fetch per tap: 96 against 100 us on
+     (32,256,56,56) without padding) */
+  if (g.dx == 1 && (g.sx == 2 || (g.sx == 1 && g.kx >= 5)) && (g.kx == 3 || g.kx == 5 || g.kx == 7) && g.ow >= EPT) {
+    const long long ppr = (g.ow + EPT - 1) / EPT;
+    const long long places = static_cast<long long>(g.n) * g.oh * ppr;
+    const uint32_t chunks = static_cast<uint32_t>((places + kPatchBlock - 1) / kPatchBlock);
+    const long long pieces = (static_cast<long long>(g.c) * chunks + 7) / 8 * 8;
+    const long long blocks = pieces * g.ky;
+    if (places + kPatchBlock < (1ll << 31) && blocks < (1ll << 31)) {
+#define IM2COL_ROW_TAPS(KX, SX)                                                                       \
+  hipLaunchKernelGGL((Im2ColRowTapsKernel<T, KX, SX>), dim3(static_cast<unsigned>(blocks)),           \
+                     dim3(kPatchBlock), 0, AsStream(stream), col, cstride, img, istride, g,           \
+                     mshadow::FastDivU32(static_cast<uint32_t>(ppr)),                                 \
+                     mshadow::FastDivU32(static_cast<uint32_t>(g.oh)), chunks,                        \
+                     mshadow::FastDivU32(chunks), static_cast<uint32_t>(places))
+      if (g.sx == 1) {
+        if (g.kx == 5) IM2COL_ROW_TAPS(5, 1);
+        else IM2COL_ROW_TAPS(7, 1);
+      } else {
+        if (g.kx == 3) IM2COL_ROW_TAPS(3, 2);
+        else if (g.kx == 5) IM2COL_ROW_TAPS(5, 2);
+        else IM2COL_ROW_TAPS(7, 2);
+      }
+#undef IM2COL_ROW_TAPS
+      return AfterLaunch("im2col");
+    }
+  }
   /* stride 1, dilation 1, patch rows of a pack or more: pack by pack, no staging */
   if (unit_steps && g.ow >= EPT) {
     const long long ppr = (g.ow + EPT - 1) / EPT;

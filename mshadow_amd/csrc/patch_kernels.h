@@ -413,6 +413,92 @@ __global__ void __launch_bounds__(kPatchBlock)
                         static_cast<size_t>(line) * g.ow + ox, q);
 }
 
+/*! \brief LoadPackInside with the one 16-byte load outside any branch (a load inside a branch
+ *  makes the compiler wait for every load under way before it): the address is moved into
+ *  [first, last - EPT] for the load, and only a wave that holds a moved pack - at the first or
+ *  the last row of the whole tensor - fetches that pack again element by element. `wanted` false:
+ *  nothing is wanted, zeros come back. */
+template <typename T>
+__device__ __forceinline__ U4 LoadPackInsideFree(const T *p, int lo, int hi, const T *first, const T *last,
+                                                 bool wanted) {
+  const int EPT = 16 / sizeof(T);
+  const bool moved = wanted && (p < first || p + EPT > last);
+  const T *at = !wanted ? first : (p < first ? first : (p + EPT > last ? last - EPT : p));
+  U4 q = LoadPackAnywhere(at);
+  if (__any(moved)) {
+    U4 r = {0u, 0u, 0u, 0u};
+    if (moved) {
+#pragma unroll
+      for (int e = 0; e < EPT; ++e) {
+        if (e >= lo && e < hi) SetPackElement(&r, e, p[e]);
+      }
+    }
+    if (moved) q = r;
+  }
+  return KeepElements<T>(q, wanted ? lo : 0, wanted ? hi : 0);
+}
+
+/*! \brief im2col with a step of SX = 1 or 2 between patches in a row and dilation 1 along the
+ *  row, for KX taps a row (3, 5 or 7): a thread makes the packs of ALL KX taps of one tap row
+ *  at one place from the SX * (EPT - 1) + KX neighbouring image elements under them, fetched
+ *  once as two to four packs (Im2ColDirectS1Kernel fetches a pack per tap, Im2ColDirectS2Kernel
+ *  two: the image then crosses from L2 to the CUs KX or 2 * KX times per tap row). Tap b's pack
+ *  is every SX-th element from the b-th on. The tap rows of one piece of a channel are numbered
+ *  8 workgroups apart, as in Im2ColRow3DirectKernel. */
+template <typename T, int KX, int SX>
+__global__ void __launch_bounds__(kPatchBlock)
+    Im2ColRowTapsKernel(T *col, int cstride, const T *img, int istride, PatchGeom g,
+                        mshadow::FastDivU32 div_ppr, mshadow::FastDivU32 div_oh, uint32_t chunks,
+                        mshadow::FastDivU32 div_chunks, uint32_t places) {
+  const int EPT = 16 / sizeof(T);
+  const int NPACK = (SX * (EPT - 1) + KX + EPT - 1) / EPT;
+  const uint32_t rows = static_cast<uint32_t>(g.ky);
+  const uint32_t lane8 = blockIdx.x & 7u;
+  const uint32_t turn = blockIdx.x >> 3;
+  const uint32_t group = turn / rows;
+  const int a = static_cast<int>(turn - group * rows);
+  const uint32_t piece = group * 8 + lane8;
+  const uint32_t ch = div_chunks.Div(piece);
+  if (ch >= static_cast<uint32_t>(g.c)) return;
+  const uint32_t chunk = piece - ch * chunks;
+  const uint32_t pk = chunk * kPatchBlock + threadIdx.x;   // place: (n * oh + oy) * ppr + p
+  if (pk >= places) return;
+  const uint32_t line = div_ppr.Div(pk);
+  const int ox = min(static_cast<int>(pk - line * div_ppr.div) * EPT, g.ow - EPT);
+  const uint32_t n = div_oh.Div(line);
+  const int oy = static_cast<int>(line - n * g.oh);
+  const int y = oy * g.sy + a * g.dy - g.pad_y;
+  const int xs = ox * SX - g.pad_x;
+  const bool wanted = y >= 0 && y < g.h;
+  const T *row = img + (static_cast<size_t>(n * g.c + ch) * g.h + (wanted ? y : 0)) * istride;
+  const T *last = img + (static_cast<size_t>(g.n) * g.c * g.h - 1) * istride + g.w;
+  uint32_t R[NPACK * 4];
+#pragma unroll
+  for (int k = 0; k < NPACK; ++k) {
+    const int at = xs + k * EPT;
+    const U4 q = LoadPackInsideFree<T>(row + at, max(0, -at), min(EPT, g.w - at), img, last, wanted);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) R[4 * k + d] = q[d];
+  }
+  T *out = col + static_cast<size_t>(ch * rows * KX + a * KX) * cstride + static_cast<size_t>(line) * g.ow + ox;
+#pragma unroll
+  for (int b = 0; b < KX; ++b) {
+    U4 q;
+    if (sizeof(T) == 4) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) q[e] = R[SX * e + b];
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int i0 = SX * 2 * r + b, i1 = i0 + SX;   // the two elements of this register
+        const uint32_t lo = (i0 & 1) ? 0x0302u : 0x0100u, hi = (i1 & 1) ? 0x0706u : 0x0504u;
+        q[r] = __builtin_amdgcn_perm(R[i1 >> 1], R[i0 >> 1], (hi << 16) | lo);
+      }
+    }
+    StorePackAnywhere(out + static_cast<size_t>(b) * cstride, q);
+  }
+}
+
 /*! \brief one pack plus another, element by element, rounded after every add as the element
  *  type's own += does (binary16: a packed half add is exactly that); elements whose bit in
  *  `keep` is clear stay as they are */

@@ -675,6 +675,10 @@ CONV = [  # n, c, h, w, ky, kx, sy, sx, dy, dx, py, px
     (2, 2, 19, 11, 3, 3, 2, 2, 1, 1, 0, 0), (2, 2, 16, 8, 3, 3, 2, 2, 1, 1, 0, 0), (2, 3, 33, 52, 5, 5, 3, 2, 1, 1, 2, 2),
     (2, 2, 26, 38, 3, 6, 1, 2, 1, 1, 1, 7), (1, 2, 30, 41, 9, 9, 2, 2, 1, 1, 4, 4), (2, 2, 28, 28, 2, 2, 2, 2, 1, 1, 0, 0),
     (2, 3, 34, 40, 3, 3, 3, 3, 1, 1, 1, 1), (2, 2, 35, 43, 7, 5, 3, 3, 1, 1, 3, 2), (1, 2, 40, 48, 11, 11, 3, 3, 1, 1, 5, 5),
+    # im2col with all taps of a tap row from one fetch (3, 5, 7 taps with a step of two; 5, 7 with a step of one):
+    # dilated tap rows, steps between rows, padding wider than a pack, odd widths, the patch row as short as one pack
+    (2, 3, 30, 33, 3, 5, 2, 1, 2, 1, 2, 2), (2, 2, 24, 40, 5, 7, 1, 1, 1, 1, 0, 3), (1, 3, 21, 29, 2, 7, 3, 2, 1, 1, 1, 9),
+    (2, 2, 17, 19, 3, 5, 1, 2, 1, 1, 0, 0), (2, 2, 12, 12, 5, 5, 1, 1, 1, 1, 0, 0), (2, 2, 18, 21, 1, 3, 2, 2, 1, 1, 0, 10),
 ]
 
 
