@@ -1126,7 +1126,8 @@ int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstrid
   hipStream_t s = AsStream(stream);
   /* 3 x 3 windows with stride 2 on rows of up to 256 pixels: no staging. Even heights and rows of
      whole aligned packs take the plain form, everything else the one that moves packs anywhere */
-  if (ky == 3 && kx == 3 && sy == 2 && sx == 2 && w <= 256 && ph >= 1 && pw >= 1) {
+  if (ky == 3 && kx == 3 && sy == 2 && sx == 2 && w <= 256 && ph >= 1 && pw >= 1 &&
+      static_cast<long long>(planes) * ph * pw >= 2) {
     const bool whole = h % 2 == 0 && w % 4 == 0 && dstride % 4 == 0 && sstride % 4 == 0 &&
                        Aligned16(dst) && Aligned16(src);
     UnpoolRowsGeom rg;
@@ -1138,6 +1139,7 @@ int mshadow_hip_unpool_f32(float *dst, int dstride, const float *src, int sstrid
     rg.div_half_h = mshadow::FastDivU32(rg.half_h);
     rg.pooled_floats = (static_cast<size_t>(planes) * ph - 1) * pstride + pw;
     rg.grad_floats = (static_cast<size_t>(planes) * ph - 1) * gstride + pw;
+    rg.src_floats = (static_cast<size_t>(planes) * h - 1) * sstride + w;
     const uint32_t waves = (rg.total_rows + rg.rows_per_wave - 1) / rg.rows_per_wave;
     const uint32_t blocks = (waves + kPoolBlock / 64 - 1) / (kPoolBlock / 64);
 #define UNPOOL_ROWS(R)                                                                          \

@@ -748,14 +748,22 @@ __global__ void __launch_bounds__(kPoolBlock)
 struct UnpoolRowsGeom {
   uint32_t total_rows, groups, rows_per_wave, half_h;
   size_t pooled_floats, grad_floats;   // extent of the two pooled-size arrays, last row unpadded
+  size_t src_floats;                   // extent of the source, last row unpadded
   mshadow::FastDivU32 div_groups, div_half_h;
 };
+
+__device__ __forceinline__ F4 LoadPackFree(const float *base, const float *p, const float *end, bool ok);
 
 /*! \brief unpool for a 3 x 3 window with stride 2 on rows of up to 256 pixels, with no staging:
  *  a thread owns two adjacent 2 x 2 blocks of source pixels - four pixels of row 2a and the four
  *  below them. RAGGED = false: h even, w a multiple of 4, rows of whole aligned packs. RAGGED =
  *  true: any h and w at any alignment - the last pair of rows of an odd height has no lower row,
- *  the last pack of a row that is not whole packs moves element by element. The windows that can cover them
+ *  the last pack of a row that is not whole packs is fetched whole (what lies behind the row is
+ *  the next row's and is not stored) and stored element by element; every load of this form sits
+ *  outside any branch and is issued before the first value is used, so a thread waits for memory
+ *  once ((64,96,55,55): 52 -> 48 us; with loads inside the branches of the two cases the
+ *  compiler waits for all loads under way at each). What this form still pays against the other
+ *  (33 us on 56 x 56) are 16-byte accesses at 4-byte borders. The windows that can cover them
  *  are rows a - 1 and a of the pooled grid, columns 2t - 1, 2t, 2t + 1: the thread fetches
  *  columns 2t and 2t + 1 of both rows (pooled value and gradient) and takes column 2t - 1
  *  from the neighbouring lane, which fetched it as its own 2t' + 1 (a wave takes whole rows).
@@ -783,23 +791,32 @@ __global__ void __launch_bounds__(kPoolBlock)
   if (!RAGGED) {
     top = StreamLoadF4(in), bottom = StreamLoadF4(in + sstride);
   } else {
-    top = bottom = F4{0.0f, 0.0f, 0.0f, 0.0f};
-    if (live_px == 4) {
-      top = StreamLoadF4Anywhere(in);
-      if (has_bottom) bottom = StreamLoadF4Anywhere(in + sstride);
-    } else {
-#pragma unroll
-      for (int i = 0; i < 3; ++i) {
-        if (i < live_px) {
-          top[i] = StreamLoad(in + i);
-          if (has_bottom) bottom[i] = StreamLoad(in + sstride + i);
-        }
-      }
-    }
+    const float *send = src + rg.src_floats;
+    top = LoadPackFree(src, in, send, true);
+    bottom = LoadPackFree(src, in + sstride, send, has_bottom);
   }
   /* [jy][c]: pooled row a - jy, column 2t - 1 + c */
   float pv[2][3], gv[2][3];
   bool ok[2][3];
+  if (RAGGED) {
+    /* both pooled rows of both arrays requested at once: columns 2t and 2t + 1 as one 8-byte
+       access; only the last float of an array has nothing behind it, and is fetched as the
+       second of the pair before it */
+#pragma unroll
+    for (int jy = 0; jy < 2; ++jy) {
+      const int py = a - jy;
+      const bool row_ok = py >= 0 && py < g.ph;
+      const size_t prow = static_cast<size_t>(plane) * g.ph + (row_ok ? py : 0);
+      const int px = static_cast<int>(2u * t);
+      const int pxc = px < g.pw ? px : 0;
+      const size_t poff = prow * pstride + pxc, goff = prow * gstride + pxc;
+      const bool ptail = poff + 2 > rg.pooled_floats, gtail = goff + 2 > rg.grad_floats;
+      const F2 pp = *reinterpret_cast<const F2Loose *>(pooled + poff - (ptail ? 1 : 0));
+      const F2 gg = *reinterpret_cast<const F2Loose *>(grad + goff - (gtail ? 1 : 0));
+      pv[jy][1] = ptail ? pp.y : pp.x, pv[jy][2] = pp.y;
+      gv[jy][1] = gtail ? gg.y : gg.x, gv[jy][2] = gg.y;
+    }
+  }
 #pragma unroll
   for (int jy = 0; jy < 2; ++jy) {
     const int py = a - jy;
@@ -813,8 +830,10 @@ __global__ void __launch_bounds__(kPoolBlock)
     const size_t poff = prow * pstride + pxc, goff = prow * gstride + pxc;
     /* pooled row a - 1 is row a' of the pair above, which the lanes `groups` below hold when
        that pair is in this wave and plane */
-    const bool from_above = jy == 1 && row_in_wave > 0u && a > 0 && live;
-    if (from_above) {
+    const bool from_above = !RAGGED && jy == 1 && row_in_wave > 0u && a > 0 && live;
+    if (RAGGED) {
+      /* fetched above */
+    } else if (from_above) {
       pv[jy][1] = pv[jy][2] = gv[jy][1] = gv[jy][2] = 0.0f;
     } else if (poff + 2 <= rg.pooled_floats && goff + 2 <= rg.grad_floats) {
       const F2 pp = *reinterpret_cast<const F2Loose *>(pooled + poff);
@@ -825,7 +844,7 @@ __global__ void __launch_bounds__(kPoolBlock)
       pv[jy][1] = pv[jy][2] = pooled[poff];
       gv[jy][1] = gv[jy][2] = grad[goff];
     }
-    if (jy == 1) {
+    if (jy == 1 && !RAGGED) {
       const int from = from_above ? static_cast<int>(lane - rg.groups) : static_cast<int>(lane);
       const float p1 = __shfl(pv[0][1], from), p2 = __shfl(pv[0][2], from);
       const float g1 = __shfl(gv[0][1], from), g2 = __shfl(gv[0][2], from);
