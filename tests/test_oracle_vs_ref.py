@@ -205,7 +205,7 @@ def test_im2col_col2im(orc, ref, cfg, dtype):
 
 
 def test_col2im_half_config_like(orc, ref):
-    # the survey's check: (2,16,56,56) k3 s1 pad1 in half, N(0,1) columns
+    # the convolution shape of the benchmark in small: (2,16,56,56) k3 s1 pad1 in half, N(0,1) columns
     rng = np.random.default_rng(70)
     n, c, h, w = 2, 16, 56, 56
     shape = Checker.col_shape(n, c, h, w, 3, 3, 1, 1, 1, 1, 1, 1)
