@@ -223,7 +223,7 @@ def main():
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
     G.set_device(0)
     if args.only in ("softmax_phases", "ceiling_chain", "ceiling_lds_loads", "ceiling_seg_loads",
-                     "softmax_prefetch_copy", "highdim_split_configs"):
+                     "softmax_prefetch_copy", "highdim_split_configs", "staying_waves_copy"):
         return run_probe(G, args.only, args.pattern)
     if args.only == "neighbour_shapes":
         return neighbour_shapes(G)
@@ -710,6 +710,23 @@ def run_probe(G, which, pattern=""):
                 want = got if want is None else want
                 res[names[cfg]] = [round(us, 1), bool(np.array_equal(got.view(np.uint32), want.view(np.uint32)))]
             out["shapes"]["x".join(map(str, shape))] = res
+    elif which == "staying_waves_copy":
+        # 1 GiB copied by waves that stay until it is done: each wave on a contiguous run of its own
+        # (as many sequential streams as waves) against the waves side by side on one moving region
+        floats = 1 << 28
+        src, dst = G.buffer((8192, 32768), f32), G.buffer((8192, 32768), f32)
+        G.fill(src, 1.0, s)
+        out = {"probe": "staying_waves_copy", "bytes_read": floats * 4, "bytes_written": floats * 4,
+               "unit": "us per copy; fraction of the HBM peak", "variants": {}}
+        for per_cu in (1, 2, 4, 8):
+            wgs = per_cu * cus
+            for own_run, name in ((1, "own contiguous run per wave"), (0, "waves side by side")):
+                us = min(P.stream_copy_us(dst, src, floats, wgs, own_run, s) for _ in range(3))
+                out["variants"][f"{wgs} workgroups of 4 waves, {name}"] = [
+                    round(us, 1), round(2 * floats * 4 / us / 1e3 / HBM_PEAK_GBS, 3)]
+        # and by 65536 workgroups that move 16 KB each and end
+        out["short_lived_workgroups_us"] = round(min(P.stream_copy_us(dst, src, floats, floats // (4 * 256 * 4), 1, s)
+                                                     for _ in range(3)), 1)
     elif which == "softmax_prefetch_copy":
         L = np.random.default_rng(7).standard_normal((8192, 32000), dtype=f32) * f32(3)
         src, dst = G.to_device(L), G.buffer(L.shape, f32)

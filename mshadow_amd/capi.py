@@ -688,6 +688,13 @@ class Probe:
                                                     src.cols, barriers, spin, resident, C.byref(us), stream))
         return us.value
 
+    def stream_copy_us(self, dst, src, floats, workgroups, own_run, stream=None):
+        us = C.c_double(0)
+        self.dll.mshadow_probe_stream_copy.argtypes = [_p, _p, C.c_size_t, _i, _i, C.POINTER(C.c_double), _p]
+        self._check(self.dll.mshadow_probe_stream_copy(dst.ptr, src.ptr, floats, workgroups, int(own_run),
+                                                       C.byref(us), stream))
+        return us.value
+
     def row_copy_prefetch_us(self, dst, src, threads, prefetch_slabs, barriers, spin, workgroups, stream=None):
         us = C.c_double(0)
         self.dll.mshadow_probe_row_copy_prefetch.argtypes = [_p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _i,

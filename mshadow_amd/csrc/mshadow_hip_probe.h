@@ -65,6 +65,14 @@ int mshadow_probe_row_copy_prefetch(float *dst, int dstride, const float *src, i
                                     int cols, int threads, int prefetch_slabs, int barriers, int spin,
                                     int workgroups, double *kernel_us, void *stream);
 
+/* A copy of `floats` floats by `workgroups` workgroups of four waves that stay until it is done
+   (floats a multiple of workgroups x 16 KB), each wave moving 1 KB pieces, four on their way.
+   own_run = 1: a wave's pieces are one contiguous run - the resident waves are as many separate
+   sequential streams; 0: piece i of wave w is piece i * waves + w - the resident waves work side
+   by side on one region that moves through memory. kernel_us = duration of the launch. */
+int mshadow_probe_stream_copy(float *dst, const float *src, size_t floats, int workgroups, int own_run,
+                              double *kernel_us, void *stream);
+
 /* Rate of loads into LDS when workgroup b reads segments b * segs .. b * segs + segs - 1 of
    `seg_len` floats each (they lie one after the other in memory) side by side, `piece_instr`
    instructions (64 * width bytes each) of one segment, then of the next: nseg / segs

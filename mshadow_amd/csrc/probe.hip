@@ -346,6 +346,34 @@ __global__ void __launch_bounds__(1024) DmaRateKernel(const float *src, uint32_t
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+/*! \brief a copy by waves that stay: every wave moves `per_wave` pieces of 1 KB (64 lanes x 16
+ *  bytes), DEPTH of them on their way at a time. OWN_RUN: the pieces of a wave are one
+ *  contiguous run of memory, so the waves resident at any moment read and write as many
+ *  separate sequential streams; otherwise piece i of wave w is piece i * waves + w, so that at
+ *  any moment the resident waves work side by side on one region. */
+template <bool OWN_RUN, int DEPTH>
+__global__ void __launch_bounds__(256) StreamCopyKernel(float *dst, const float *src, uint32_t per_wave) {
+  using mshadow_hipk::F4;
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = blockIdx.x * 4u + (threadIdx.x >> 6);
+  const uint32_t waves = gridDim.x * 4u;
+  for (uint32_t i = 0; i < per_wave; i += DEPTH) {
+    F4 q[DEPTH];
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) {
+      const size_t piece = OWN_RUN ? static_cast<size_t>(wave) * per_wave + i + u
+                                   : static_cast<size_t>(i + u) * waves + wave;
+      q[u] = mshadow_hipk::StreamLoadF4(src + piece * 256u + lane * 4u);
+    }
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) {
+      const size_t piece = OWN_RUN ? static_cast<size_t>(wave) * per_wave + i + u
+                                   : static_cast<size_t>(i + u) * waves + wave;
+      mshadow_hipk::StreamStoreF4(dst + piece * 256u + lane * 4u, q[u]);
+    }
+  }
+}
+
 int TimeKernel(hipStream_t s, float *ms, const std::function<void()> &launch) {
   hipEvent_t a, b;
   ABI_HIP(hipEventCreate(&a));
@@ -654,6 +682,28 @@ int mshadow_probe_dma_rate(const float *src, int sstride, int rows, int cols, in
   else if (width == 4 && strip == 64) PROBE_DMA(4, 64)
   else PROBE_DMA(16, 64)
 #undef PROBE_DMA
+  if (st != MSHADOW_HIP_OK) return st;
+  *kernel_us = ms * 1e3;
+  return MSHADOW_HIP_OK;
+}
+
+int mshadow_probe_stream_copy(float *dst, const float *src, size_t floats, int workgroups, int own_run,
+                              double *kernel_us, void *stream) {
+  ABI_REQUIRE(dst != NULL && src != NULL && kernel_us != NULL && workgroups >= 1, "bad argument");
+  const size_t waves = static_cast<size_t>(workgroups) * 4;
+  const int kDepth = 4;
+  ABI_REQUIRE(floats % (waves * 256 * kDepth) == 0 && floats / (waves * 256) < (1ull << 31),
+              "floats must be a multiple of workgroups x 4 KB x 4");
+  const uint32_t per_wave = static_cast<uint32_t>(floats / (waves * 256));
+  hipStream_t s = AsStream(stream);
+  float ms = 0.0f;
+  const int st = TimeKernel(s, &ms, [&] {
+    if (own_run) {
+      hipLaunchKernelGGL((StreamCopyKernel<true, kDepth>), dim3(workgroups), dim3(256), 0, s, dst, src, per_wave);
+    } else {
+      hipLaunchKernelGGL((StreamCopyKernel<false, kDepth>), dim3(workgroups), dim3(256), 0, s, dst, src, per_wave);
+    }
+  });
   if (st != MSHADOW_HIP_OK) return st;
   *kernel_us = ms * 1e3;
   return MSHADOW_HIP_OK;
