@@ -577,13 +577,22 @@ int mshadow_hip_softmax_f32(float *dst, int dstride, const float *src, int sstri
 #define SOFTMAX_WAVE(SLABS) \
   hipLaunchKernelGGL((SoftmaxWaveSlabsKernel<SLABS, false>), dim3((rows + 3) / 4), dim3(256), 0, s, dst, \
                      dstride, src, sstride, rows, cols)
-  /* many rows of up to 2048 columns: a wave per row (65536 rows of 300 / 1000 / 2000 columns:
-     71 / 109 / 122 us against 163 / 193 / 139 us with a workgroup per row; from 4096 columns on,
-     or with few rows, the workgroup per row is faster) */
-  if (cols <= 2048 && rows >= 8 * mshadow_abi::ComputeUnits()) {
+  /* many rows of up to 3072 columns: a wave per row (65536 rows of 300 / 1000 / 2000 columns:
+     71 / 109 / 122 us against 163 / 193 / 139 us with a workgroup per row; 16384 rows of 2304 /
+     3000 columns: 80 / 98 us against 120 / 133 us; at 4096 columns, 64 of them a lane, the wave
+     takes 176 us against 127 us, and with few rows the workgroup per row is faster) */
+  if (cols <= 3072 && rows >= 8 * mshadow_abi::ComputeUnits()) {
     if (cols <= 512) SOFTMAX_WAVE(2);
     else if (cols <= 1024) SOFTMAX_WAVE(4);
-    else SOFTMAX_WAVE(8);
+    else if (cols <= 2048) SOFTMAX_WAVE(8);
+    else SOFTMAX_WAVE(12);
+    return AfterLaunch("softmax");
+  }
+  /* many rows of 8193 to 16384 columns: four waves a row with 64 columns a thread, eight rows to a
+     CU instead of four ((4096,10000): 82 against 104 us, (8192,12288): 153 against 196 us; with
+     2048 rows the eight waves a row below finish them sooner, 57 against 70 us) */
+  if (cols > 8192 && cols <= 16384 && rows >= 16 * mshadow_abi::ComputeUnits()) {
+    SOFTMAX_LAUNCH(256, 16, 4);
     return AfterLaunch("softmax");
   }
 #undef SOFTMAX_WAVE
@@ -621,13 +630,14 @@ int mshadow_hip_softmax_rowsum_f32(float *sums, const float *terms, int tstride,
     LaunchShortSoftmax<true>(sums, 0, terms, tstride, rows, cols, s);
     return AfterLaunch("softmax_rowsum");
   }
-  if (cols <= 2048 && rows >= 8 * mshadow_abi::ComputeUnits()) {  // as in mshadow_hip_softmax_f32
+  if (cols <= 3072 && rows >= 8 * mshadow_abi::ComputeUnits()) {  // as in mshadow_hip_softmax_f32
 #define ROWSUM_WAVE(SLABS) \
   hipLaunchKernelGGL((SoftmaxWaveSlabsKernel<SLABS, true>), dim3((rows + 3) / 4), dim3(256), 0, s, sums, 0, \
                      terms, tstride, rows, cols)
     if (cols <= 512) ROWSUM_WAVE(2);
     else if (cols <= 1024) ROWSUM_WAVE(4);
-    else ROWSUM_WAVE(8);
+    else if (cols <= 2048) ROWSUM_WAVE(8);
+    else ROWSUM_WAVE(12);
 #undef ROWSUM_WAVE
     return AfterLaunch("softmax_rowsum");
   }
@@ -643,7 +653,8 @@ int mshadow_hip_softmax_rowsum_f32(float *sums, const float *terms, int tstride,
   hipLaunchKernelGGL((SoftmaxRowKernel<T, S, V, true>), dim3(rows), dim3(T), 0, s, sums, 0, terms, \
                      tstride, cols)
   if (vec) {
-    if (cols <= 1024) ROWSUM_LAUNCH(256, 1, 4);
+    if (cols > 8192 && cols <= 16384 && rows >= 16 * mshadow_abi::ComputeUnits()) ROWSUM_LAUNCH(256, 16, 4);  // as above
+    else if (cols <= 1024) ROWSUM_LAUNCH(256, 1, 4);
     else if (cols <= 2048) ROWSUM_LAUNCH(256, 2, 4);
     else if (cols <= 4096) ROWSUM_LAUNCH(256, 4, 4);
     else if (cols <= 8192) ROWSUM_LAUNCH(256, 8, 4);

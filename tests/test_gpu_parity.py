@@ -278,6 +278,8 @@ SOFTMAX_SHAPES = [((64, 32000), 0), ((5, 1000), 0), ((5, 1001), 0), ((3, 7), 1),
                   ((3, 128000), 0), ((2, 200001), 1), ((1, 262149), 0), ((2, 65537), 3), ((2, 65540), 0), ((2, 131072), 2),
                   # many rows of a few hundred to 2048 columns: a wave per row, slab after slab
                   ((2100, 300), 0), ((2049, 777), 3), ((2050, 1024), 0), ((2048, 2047), 1), ((4100, 513), 0),
+                  # ... up to 3072 columns; many rows of 8193 to 16384 columns: four waves a row
+                  ((2100, 2304), 0), ((2050, 3072), 1), ((2049, 2999), 0), ((4100, 8200), 0), ((4096, 12001), 0),
                   # short rows: one thread per row up to 32 columns, one wave per row up to 256
                   ((1000, 10), 0), ((300, 32), 0), ((77, 33), 2), ((130, 64), 0), ((50, 65), 1),
                   ((41, 128), 0), ((19, 200), 3), ((64, 256), 0), ((9, 257), 0), ((5, 2), 0)]
@@ -341,7 +343,8 @@ def _serial_row_sums(O, terms):
     return want
 
 
-ROWSUM_COLS = [1, 3, 10, 31, 32, 33, 64, 65, 128, 129, 255, 256, 257, 300, 513, 777, 1000, 1024, 1028, 2048, 3000, 4096, 5001, 8192, 12000, 16384,
+ROWSUM_COLS = [1, 3, 10, 31, 32, 33, 64, 65, 128, 129, 255, 256, 257, 300, 513, 777, 1000, 1024, 1028, 2048, 2049, 2304, 3000,
+               3072, 3073, 4096, 5001, 8192, 8196, 12000, 16384,
                20001, 32000, 32768, 40000, 65536,
                # longer than a workgroup's registers hold: summed stretch by stretch, each from the sum in front
                65537, 70001, 131072, 131075, 200001, 262149]
@@ -377,12 +380,18 @@ def test_softmax_rowsum_is_the_serial_sum(G, O, stream, cols):
         sums = G.buffer((terms.shape[0],), f32)
         G.softmax_rowsum(sums, G.to_device(terms, pad), stream)
         assert_bits_equal(sums.download(stream), want, f"row sum cols={cols} pad={pad}")
-    if 256 < cols <= 2048:
+    if 256 < cols <= 3072:
         # with thousands of rows these lengths take the kernel with a wave per row
         many = np.tile(terms, (150, 1))
         sums = G.buffer((many.shape[0],), f32)
         G.softmax_rowsum(sums, G.to_device(many, 1), stream)
         assert_bits_equal(sums.download(stream), np.tile(want, 150), f"row sum cols={cols}, a wave per row")
+    if 8192 < cols <= 16384 and cols % 4 == 0:
+        # and these, as whole packs, the workgroup of four waves with 64 columns a thread
+        many = np.tile(terms, (260, 1))
+        sums = G.buffer((many.shape[0],), f32)
+        G.softmax_rowsum(sums, G.to_device(many), stream)
+        assert_bits_equal(sums.download(stream), np.tile(want, 260), f"row sum cols={cols}, four waves a row")
 
 
 def test_softmax_rowsum_specials(G, O, stream):
