@@ -130,12 +130,13 @@ int Im2Col(T *col, int cstride, const T *img, int istride, const PatchGeom &g, v
       return AfterLaunch("im2col");
     }
   }
-  /* 3, 5 or 7 taps a row next to one another, a step of one or two between patches, patch rows of
+  /* 3, 5 or 7 taps a row next to one another (4 with a step of two), a step of one or two between patches, patch rows of
      a pack or more: all taps of a tap row from one fetch of the image under them (3x3 stride 2 on
      (32,256,56,56) binary16: 27 us against 41 us with a fetch per tap; 5x5 stride 1 on (32,128,28,28):
      29 against 40 us. Three taps with a step of one keep a fetch per tap: 96 against 100 us on
      (32,256,56,56) without padding) */
-  if (g.dx == 1 && (g.sx == 2 || (g.sx == 1 && g.kx >= 5)) && (g.kx == 3 || g.kx == 5 || g.kx == 7) && g.ow >= EPT) {
+  if (g.dx == 1 && (g.sx == 2 || (g.sx == 1 && g.kx >= 5)) &&
+      (g.kx == 3 || g.kx == 5 || g.kx == 7 || (g.kx == 4 && g.sx == 2)) && g.ow >= EPT) {
     const long long ppr = (g.ow + EPT - 1) / EPT;
     const long long places = static_cast<long long>(g.n) * g.oh * ppr;
     const uint32_t chunks = static_cast<uint32_t>((places + kPatchBlock - 1) / kPatchBlock);
@@ -153,6 +154,7 @@ int Im2Col(T *col, int cstride, const T *img, int istride, const PatchGeom &g, v
         else IM2COL_ROW_TAPS(7, 1);
       } else {
         if (g.kx == 3) IM2COL_ROW_TAPS(3, 2);
+        else if (g.kx == 4) IM2COL_ROW_TAPS(4, 2);
         else if (g.kx == 5) IM2COL_ROW_TAPS(5, 2);
         else IM2COL_ROW_TAPS(7, 2);
       }

@@ -439,7 +439,7 @@ __device__ __forceinline__ U4 LoadPackInsideFree(const T *p, int lo, int hi, con
 }
 
 /*! \brief im2col with a step of SX = 1 or 2 between patches in a row and dilation 1 along the
- *  row, for KX taps a row (3, 5 or 7): a thread makes the packs of ALL KX taps of one tap row
+ *  row, for KX taps a row (3, 4, 5 or 7): a thread makes the packs of ALL KX taps of one tap row
  *  at one place from the SX * (EPT - 1) + KX neighbouring image elements under them, fetched
  *  once as two to four packs (Im2ColDirectS1Kernel fetches a pack per tap, Im2ColDirectS2Kernel
  *  two: the image then crosses from L2 to the CUs KX or 2 * KX times per tap row). Tap b's pack

@@ -688,6 +688,7 @@ CONV = [  # n, c, h, w, ky, kx, sy, sx, dy, dx, py, px
     # dilated tap rows, steps between rows, padding wider than a pack, odd widths, the patch row as short as one pack
     (2, 3, 30, 33, 3, 5, 2, 1, 2, 1, 2, 2), (2, 2, 24, 40, 5, 7, 1, 1, 1, 1, 0, 3), (1, 3, 21, 29, 2, 7, 3, 2, 1, 1, 1, 9),
     (2, 2, 17, 19, 3, 5, 1, 2, 1, 1, 0, 0), (2, 2, 12, 12, 5, 5, 1, 1, 1, 1, 0, 0), (2, 2, 18, 21, 1, 3, 2, 2, 1, 1, 0, 10),
+    (2, 3, 32, 32, 4, 4, 2, 2, 1, 1, 1, 1), (3, 2, 21, 35, 4, 4, 2, 2, 1, 1, 0, 2),
 ]
 
 
