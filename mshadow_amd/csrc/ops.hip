@@ -450,14 +450,14 @@ void LaunchShortSoftmax(float *dst, int dstride, const float *src, int sstride, 
   if (cols <= 32) {
     hipLaunchKernelGGL((SoftmaxThreadRowKernel<32, TERMS_GIVEN>), dim3((rows + 255) / 256), dim3(256),
                        0, s, dst, dstride, src, sstride, rows, cols);
-  } else if (cols <= 64) {
-    hipLaunchKernelGGL((SoftmaxWaveRowKernel<1, TERMS_GIVEN>), dim3((rows + 3) / 4), dim3(256), 0, s,
+  } else if (cols <= 64) {   // four rows to a wave
+    hipLaunchKernelGGL((SoftmaxPartWaveKernel<16, 4, TERMS_GIVEN>), dim3((rows + 15) / 16), dim3(256), 0, s,
                        dst, dstride, src, sstride, rows, cols);
   } else if (cols <= 128) {
-    hipLaunchKernelGGL((SoftmaxWaveRowKernel<2, TERMS_GIVEN>), dim3((rows + 3) / 4), dim3(256), 0, s,
+    hipLaunchKernelGGL((SoftmaxPartWaveKernel<16, 8, TERMS_GIVEN>), dim3((rows + 15) / 16), dim3(256), 0, s,
                        dst, dstride, src, sstride, rows, cols);
-  } else {
-    hipLaunchKernelGGL((SoftmaxWaveRowKernel<4, TERMS_GIVEN>), dim3((rows + 3) / 4), dim3(256), 0, s,
+  } else {                   // two rows to a wave
+    hipLaunchKernelGGL((SoftmaxPartWaveKernel<32, 8, TERMS_GIVEN>), dim3((rows + 7) / 8), dim3(256), 0, s,
                        dst, dstride, src, sstride, rows, cols);
   }
 }

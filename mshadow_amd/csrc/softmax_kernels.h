@@ -971,41 +971,125 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-/*! \brief one wave per row, cols <= 64 * N: lane l holds the N consecutive columns from
- *  l * N, the sum is resolved in lane order by wave scans (WaveResolve), four rows per
- *  workgroup and nothing shared between them */
-template <int N, bool TERMS_GIVEN>
+/*! \brief WaveResolve for four or two rows side by side in one wave, one to each group of LANES =
+ *  16 (a DPP row) or 32 lanes: every group adds its LANES * N terms (lane order, then element
+ *  order) to its own s exactly as a serial loop would. The scans stop at the groups' borders; a
+ *  group that is done idles while the others finish. Every lane of the wave must call it. */
+template <int LANES, int N>
+__device__ inline float PartWaveResolve(float s, const float (&t)[N]) {
+  using namespace ordered_sum;
+  static_assert(LANES == 16 || LANES == 32, "a quarter or a half of a wave");
+  const int lane = LaneId();
+  const int l = lane & (LANES - 1), first_lane = lane & ~(LANES - 1);
+  int start = 0;
+  bool done = false;
+  while (true) {
+    const Binade b = BinadeOf(s);
+    const bool active = !done && l >= start;
+    float incl = active ? LaneQuant<N>(t, b) : 0.0f;
+#define MSHADOW_ROWSCAN_STEP(SH) \
+    incl += __uint_as_float(mshadow::hip::DppU32<MSHADOW_DPP_ROW_SHR(SH), 0xf>(0u, __float_as_uint(incl)));
+    MSHADOW_ROWSCAN_STEP(1)
+    MSHADOW_ROWSCAN_STEP(2)
+    MSHADOW_ROWSCAN_STEP(4)
+    MSHADOW_ROWSCAN_STEP(8)
+#undef MSHADOW_ROWSCAN_STEP
+    if (LANES == 32) {  // lane 15 of rows 0 and 2 to every lane of rows 1 and 3
+      incl += __uint_as_float(mshadow::hip::DppU32<MSHADOW_DPP_ROW_BCAST15, 0xa>(0u, __float_as_uint(incl)));
+    }
+    const bool fail = active && !Fits(b, incl);
+    const unsigned long long mask = __ballot(fail);
+    const uint32_t mine = static_cast<uint32_t>(mask >> first_lane) & (LANES == 32 ? 0xffffffffu : 0xffffu);
+    const int first = mine ? __ffs(static_cast<int>(mine)) - 1 : LANES;
+    /* what the lanes in front of `first` add is exact (their inclusive prefix is) */
+    const float upto = __shfl(incl, first_lane + (first > 0 ? first - 1 : 0));
+    const float s1 = Accept(s, b, first > 0 ? upto : 0.0f);
+    /* lane `first` does real float adds; every lane computes, one result is taken */
+    const float s2 = __shfl(TrueAdd<N>(s1, t), first_lane + (first < LANES ? first : LANES - 1));
+    if (!done) {
+      s = first < LANES ? s2 : s1;
+      start = first + 1;
+      done = start >= LANES;
+    }
+    if (__all(done)) return s;
+  }
+}
+
+/*! \brief four or two rows per wave, LANES = 16 or 32 lanes each, cols <= LANES * N: lane l of a
+ *  row's group holds the N consecutive columns from l * N. The wave-wide steps of a row - the
+ *  maximum, the scans of the ordered sum - cost the same instructions whether a wave holds one
+ *  short row or four, and rows of up to 256 columns by the hundred thousand are bound by
+ *  exactly those. 256 / LANES rows per workgroup, nothing shared between them, no barrier. */
+template <int LANES, int N, bool TERMS_GIVEN>
 __global__ void __launch_bounds__(256)
-    SoftmaxWaveRowKernel(float *dst, int dstride, const float *src, int sstride, int rows,
-                         int cols) {
-  const int row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(WaveId());
-  if (row >= rows) return;
-  const int base = LaneId() * N;
-  const float *in = src + static_cast<size_t>(row) * sstride;
+    SoftmaxPartWaveKernel(float *dst, int dstride, const float *src, int sstride, int rows, int cols) {
+  const int row = blockIdx.x * (256 / LANES) + static_cast<int>(threadIdx.x) / LANES;
+  const bool there = row < rows;
+  const int rowc = there ? row : rows - 1;   // every lane takes part in the wave-wide steps
+  const int lane = LaneId();
+  const int base = (lane & (LANES - 1)) * N;
+  const float *in = src + static_cast<size_t>(rowc) * sstride;
   const float kNegInf = -__builtin_huge_valf();
+  const float kAbsent = TERMS_GIVEN ? 0.0f : kNegInf;
   float v[N];
-  float mx = kNegInf;
 #pragma unroll
-  for (int i = 0; i < N; ++i) {
-    v[i] = (base + i < cols) ? in[base + i] : (TERMS_GIVEN ? 0.0f : kNegInf);
-    mx = (mx < v[i]) ? v[i] : mx;
+  for (int p = 0; p < N; p += 4) {
+    if (base + p + 4 <= cols) {
+      const F4 q = StreamLoadF4Anywhere(in + base + p);
+      v[p] = q.x; v[p + 1] = q.y; v[p + 2] = q.z; v[p + 3] = q.w;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[p + i] = (base + p + i < cols) ? in[base + p + i] : kAbsent;
+    }
   }
   if (!TERMS_GIVEN) {
-    mx = WaveMaxF32(mx);
+    float mx = kNegInf;
+#pragma unroll
+    for (int i = 0; i < N; ++i) mx = (mx < v[i]) ? v[i] : mx;
+#define MSHADOW_ROWMAX_STEP(SH)                                                                   \
+    {                                                                                             \
+      const float o = __uint_as_float(mshadow::hip::DppU32<MSHADOW_DPP_ROW_SHR(SH), 0xf>(         \
+          __float_as_uint(mx), __float_as_uint(mx)));                                             \
+      mx = (mx < o) ? o : mx;                                                                     \
+    }
+    MSHADOW_ROWMAX_STEP(1)
+    MSHADOW_ROWMAX_STEP(2)
+    MSHADOW_ROWMAX_STEP(4)
+    MSHADOW_ROWMAX_STEP(8)
+#undef MSHADOW_ROWMAX_STEP
+    if (LANES == 32) {
+      const float o = __uint_as_float(mshadow::hip::DppU32<MSHADOW_DPP_ROW_BCAST15, 0xa>(
+          __float_as_uint(mx), __float_as_uint(mx)));
+      mx = (mx < o) ? o : mx;
+    }
+    mx = __shfl(mx, lane | (LANES - 1));   // the group's last lane holds the maximum of all its lanes
 #pragma unroll
     for (int i = 0; i < N; ++i) v[i] = (base + i < cols) ? ExpNonPositive(v[i] - mx) : 0.0f;
   }
-  const float s = WaveResolve<N>(0.0f, v);
+  const float s = PartWaveResolve<LANES, N>(0.0f, v);
+  if (!there) return;
   if (TERMS_GIVEN) {
-    if (LaneId() == 0) dst[row] = s;
+    if ((lane & (LANES - 1)) == 0) dst[row] = s;
     return;
   }
   float *out = dst + static_cast<size_t>(row) * dstride;
   const bool fast_div = s >= 1.0f && s < 3.0e38f;
   const float rcp = 1.0f / s;
 #pragma unroll
-  for (int i = 0; i < N; ++i) {
-    if (base + i < cols) out[base + i] = fast_div ? DivideBy(v[i], s, rcp) : v[i] / s;
+  for (int p = 0; p < N; p += 4) {
+    float o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = fast_div ? DivideBy(v[p + i], s, rcp) : v[p + i] / s;
+    if (base + p + 4 <= cols) {
+      F4 q;
+      q.x = o[0]; q.y = o[1]; q.z = o[2]; q.w = o[3];
+      StreamStoreF4Anywhere(out + base + p, q);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (base + p + i < cols) out[base + p + i] = o[i];
+      }
+    }
   }
 }
 

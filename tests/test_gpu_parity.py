@@ -282,7 +282,10 @@ SOFTMAX_SHAPES = [((64, 32000), 0), ((5, 1000), 0), ((5, 1001), 0), ((3, 7), 1),
                   ((2100, 2304), 0), ((2050, 3072), 1), ((2049, 2999), 0), ((4100, 8200), 0), ((4096, 12001), 0),
                   # short rows: one thread per row up to 32 columns, one wave per row up to 256
                   ((1000, 10), 0), ((300, 32), 0), ((77, 33), 2), ((130, 64), 0), ((50, 65), 1),
-                  ((41, 128), 0), ((19, 200), 3), ((64, 256), 0), ((9, 257), 0), ((5, 2), 0)]
+                  ((41, 128), 0), ((19, 200), 3), ((64, 256), 0), ((9, 257), 0), ((5, 2), 0),
+                  # ... four rows to a wave (33 to 128 columns) and two (129 to 256), thousands of them, pitched rows,
+                  # row counts that leave the last wave partly empty
+                  ((5003, 100), 1), ((3001, 250), 0), ((4099, 48), 3), ((2050, 129), 2), ((1, 256), 0), ((3, 40), 0)]
 
 
 def _softmax_check(got, want, src):
