@@ -624,7 +624,7 @@ def neighbour_shapes(G):
         dx, out = G.to_device(x), G.buffer((shape[1],), f32)
         report("sum_rows", str(shape), x.nbytes, timeit(lambda: G.reduce_keep_lowest(out, dx, stream=s)))
         del dx, out
-    for shape in ((8192, 32000), (65536, 1000), (128, 1000), (4096, 4096), (16384, 2304), (8192, 12288), (2048, 50257), (16, 250000), (512, 128000)):
+    for shape in ((8192, 32000), (65536, 1000), (128, 1000), (4096, 4096), (131072, 256), (16384, 2304), (8192, 12288), (2048, 50257), (16, 250000), (512, 128000)):
         x = big(shape) * f32(3)
         dx, out = G.to_device(x), G.buffer(shape, f32)
         report("softmax", str(shape), 2 * x.nbytes, timeit(lambda: G.softmax(out, dx, s)))
