@@ -688,6 +688,23 @@ int mshadow_hip_softmax_grad_ex_f32(float *dst, int dstride, const float *src, i
   /* alpha / (classes - 1) with the count converted from unsigned, as the reference writes it */
   const GradParams gp = {static_cast<int>(ignore_label), alpha,
                          alpha / static_cast<float>(static_cast<unsigned>(cols - 1))};
+  if (cols <= 512) {  // short rows: several to a workgroup, a pack a thread
+    const int ppr = (cols + 3) / 4;
+    const int rows_per_block = kGradBlock / ppr;
+    const unsigned grid = static_cast<unsigned>((rows + rows_per_block - 1) / rows_per_block);
+    const mshadow::FastDivU32 div_ppr(static_cast<uint32_t>(ppr));
+#define GRAD_SHORT(FLAGS)                                                                            \
+  hipLaunchKernelGGL((SoftmaxGradShortRowsKernel<FLAGS>), dim3(grid), dim3(kGradBlock), 0, AsStream(stream), \
+                     dst, dstride, src, sstride, label, rows, cols, rows_per_block, div_ppr, gp)
+    switch (flags) {
+      case 0: GRAD_SHORT(0); break;
+      case 1: GRAD_SHORT(1); break;
+      case 2: GRAD_SHORT(2); break;
+      default: GRAD_SHORT(3); break;
+    }
+#undef GRAD_SHORT
+    return AfterLaunch("softmax_grad");
+  }
   GradLaunch gl = {dst, dstride, src, sstride, label, cols, chunks, gp,
                    static_cast<unsigned>(blocks), AsStream(stream)};
   LaunchGrad<true>(flags, gl);   // 16-byte packs wherever the rows start (no alignment needed)

@@ -1241,6 +1241,34 @@ __global__ void __launch_bounds__(kGradBlock)
   }
 }
 
+/*! \brief the same for rows of up to 512 columns, where a workgroup per row leaves most of its
+ *  threads idle: a workgroup takes kGradBlock / ppr consecutive rows, ppr = ceil(cols / 4) packs
+ *  each (`div_ppr` divides by it), a thread one pack. grid.x = ceil(rows / rows_per_block). */
+template <int FLAGS>
+__global__ void __launch_bounds__(kGradBlock)
+    SoftmaxGradShortRowsKernel(float *dst, int dstride, const float *src, int sstride, const float *label,
+                               int rows, int cols, int rows_per_block, mshadow::FastDivU32 div_ppr,
+                               GradParams gp) {
+  const uint32_t r = div_ppr.Div(threadIdx.x);
+  const int y = blockIdx.x * rows_per_block + static_cast<int>(r);
+  if (static_cast<int>(r) >= rows_per_block || y >= rows) return;
+  const int x = static_cast<int>(threadIdx.x - r * div_ppr.div) * 4;
+  const int k = static_cast<int>(label[y]);
+  const bool ignored = (FLAGS & kGradIgnore) && k == gp.ignore_label;
+  const float *in = src + static_cast<size_t>(y) * sstride;
+  float *out = dst + static_cast<size_t>(y) * dstride;
+  if (x + 4 <= cols) {
+    F4 q = StreamLoadF4Anywhere(in + x);
+    q.x = GradElement<FLAGS>(q.x, k == x, ignored, gp);
+    q.y = GradElement<FLAGS>(q.y, k == x + 1, ignored, gp);
+    q.z = GradElement<FLAGS>(q.z, k == x + 2, ignored, gp);
+    q.w = GradElement<FLAGS>(q.w, k == x + 3, ignored, gp);
+    StreamStoreF4Anywhere(out + x, q);
+  } else {
+    for (int i = x; i < cols; ++i) out[i] = GradElement<FLAGS>(in[i], i == k, ignored, gp);
+  }
+}
+
 /* ---- 3-D tensors (d0, d1, d2), softmax over d1, row pitch on d2 ----------------------
  * (mshadow/tensor_cpu-inl.h:474-495; cuda/tensor_gpu-inl.cuh:479-597). One thread per
  * (y, n) pair, n fastest: every access of a wave is one contiguous run along d2, and the
